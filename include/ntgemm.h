@@ -1,0 +1,170 @@
+/*
+ * ntgemm.h -- C ABI of the MI355X (gfx950) backend for NeuroTensor's dense matmult path.
+ *
+ * The library behind this header replaces the reference's static library `nt_matmult`
+ * (CMakeLists.txt:88-90, cmake/matmult_sources.cmake:3-21), whose only exports are the
+ * per-dtype instantiations of
+ *
+ *   nt::functional::cpu::nt_matmult<T>        nt/functional/cpu/matmult/nt_matmult.h:6-7
+ *   nt::functional::cpu::nt_matmult_batch<T>  nt/functional/cpu/matmult/nt_matmult.h:9-10
+ *
+ * and offers, for callers that keep their tensors in device memory, the fused forms the
+ * layers above need (bias-initialised GEMM for cpu::linear, im2col + GEMM for conv2d).
+ *
+ * Conventions (identical to the reference, nt_matmult.hpp:238-292, 370-394):
+ *   - all matrices are dense row-major; sizes are LOGICAL (after the transpose flags):
+ *     a_rows = m, a_cols = b_rows = k, b_cols = n;
+ *   - transpose_a != 0 means A is STORED [k, m]; transpose_b != 0 means B is STORED [n, k];
+ *   - the GEMM ACCUMULATES: C[m, n] += op(A) . op(B); the caller initialises C;
+ *   - A and B are read-only and may alias each other; C must not alias an input.
+ *
+ * Every entry point returns 0 (NTG_OK) or a non-zero ntg_status and never throws;
+ * ntg_last_error() returns a thread-local description of the last failure.
+ * Host-pointer entry points are synchronous (results are in C on return) and thread-safe.
+ * Device-pointer entry points (suffix _dev) enqueue on the given HIP stream and return.
+ */
+#ifndef NTGEMM_H
+#define NTGEMM_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Values equal nt::DType (nt/dtype/DType_enum.h:14-20, expanded from
+ * nt/dtype/compatible/DTypeDeclareMacros.h:5-33) so a caller can pass
+ * static_cast<int>(tensor.dtype()).  BFLOAT16 and UINT64 are extensions: the reference
+ * has no BFloat16 DType (nt/types/bfloat16.h:4-5) and instantiates uint64_t only at the
+ * kernel level (nt_matmult_uint64.cpp). Complex and 128-bit types are not supported. */
+typedef enum ntg_dtype {
+    NTG_FLOAT16 = 0,
+    NTG_FLOAT32 = 1,
+    NTG_FLOAT64 = 2,
+    NTG_INT8 = 7,
+    NTG_INT16 = 8,
+    NTG_INT32 = 9,
+    NTG_INT64 = 10,
+    NTG_UINT8 = 12,
+    NTG_UINT16 = 13,
+    NTG_UINT32 = 14,
+    NTG_BFLOAT16 = 100,
+    NTG_UINT64 = 101
+} ntg_dtype;
+
+typedef enum ntg_status {
+    NTG_OK = 0,
+    NTG_ERR_INVALID_ARGUMENT = 1,
+    NTG_ERR_UNSUPPORTED_DTYPE = 2,
+    NTG_ERR_DEVICE = 3,          /* a HIP call failed; see ntg_last_error() */
+    NTG_ERR_OUT_OF_MEMORY = 4,
+    NTG_ERR_NO_DEVICE = 5
+} ntg_status;
+
+/* what the GEMM does with the incoming C */
+typedef enum ntg_c_mode {
+    NTG_C_OVERWRITE = 0,   /* C  = op(A).op(B); legal replacement of "zeros then accumulate"
+                              (matmult_cpu.cpp:110, :707) */
+    NTG_C_ACCUMULATE = 1,  /* C += op(A).op(B); the nt_matmult contract */
+    NTG_C_BIAS = 2         /* C  = bias (+) op(A).op(B); cpu::linear's "clone the expanded
+                              bias, then accumulate" (matmult_cpu.cpp:1637-1647) in one pass */
+} ntg_c_mode;
+
+const char* ntg_last_error(void);
+int ntg_version(void);
+int64_t ntg_dtype_size(int dtype);          /* bytes per element, 0 if unsupported */
+int ntg_device_count(void);                 /* gfx950 devices visible to HIP */
+
+/* ------------------------------------------------------------------------------------ */
+/* Host-pointer entry points: the drop-in seam.                                           */
+/* ------------------------------------------------------------------------------------ */
+
+/* Replaces nt::functional::cpu::nt_matmult<T> (nt_matmult.h:6-7; nt_matmult.hpp:370-378).
+ * Same argument list with the dtype made explicit; a_cols must equal b_rows. */
+int ntg_matmult(int dtype, const void* A, const void* B, void* C,
+                int64_t a_rows, int64_t a_cols, int64_t b_rows, int64_t b_cols,
+                int transpose_a, int transpose_b);
+
+/* Replaces nt::functional::cpu::nt_matmult_batch<T> (nt_matmult.h:9-10;
+ * nt_matmult.hpp:386-394, 228-235).  A/B/C are arrays of `batches` host pointers; all
+ * items share one shape and one flag pair; A/B entries may repeat (that is how the
+ * dispatcher broadcasts, matmult_cpu.cpp:883) and each distinct matrix is uploaded once. */
+int ntg_matmult_batch(int dtype, const void* const* A, const void* const* B, void* const* C,
+                      int64_t batches, int64_t a_rows, int64_t a_cols, int64_t b_rows, int64_t b_cols,
+                      int transpose_a, int transpose_b);
+
+/* Replaces the 2-D body of nt::functional::cpu::linear (matmult_cpu.cpp:1624-1647):
+ * Y[m, n] = broadcast(bias) + op(X) . op(W).  bias is [bias_rows, bias_cols] with
+ * bias_rows in {1, m} and bias_cols in {1, n}. */
+int ntg_linear(int dtype, const void* X, const void* W, const void* bias, void* Y,
+               int64_t m, int64_t k, int64_t n, int transpose_x, int transpose_w,
+               int64_t bias_rows, int64_t bias_cols);
+
+/* Replaces nt::functional::cpu::unfold2d_ with transpose_out = true
+ * (nt/functional/cpu/unfold2d.cpp:219-235, im2col_cpu :12-112):
+ * col[batch, channels*k_r*k_c, Ho*Wo] is fully written (zeros in the padding). */
+int ntg_unfold2d(int dtype, const void* image, void* col,
+                 int64_t batch, int64_t channels, int64_t height, int64_t width,
+                 int64_t k_r, int64_t k_c, int64_t s_r, int64_t s_c,
+                 int64_t p_r, int64_t p_c, int64_t d_r, int64_t d_c);
+
+/* Replaces the groups == 1 and groups > 1 bodies of nt::functional::conv2d
+ * (nt/functional/tensor_files/conv.cpp:69-119): out[batch, out_channels, Ho, Wo].
+ * kernel is [out_channels, channels/groups, k_r, k_c]. */
+int ntg_conv2d(int dtype, const void* image, const void* kernel, void* out,
+               int64_t batch, int64_t channels, int64_t height, int64_t width,
+               int64_t out_channels, int64_t k_r, int64_t k_c,
+               int64_t s_r, int64_t s_c, int64_t p_r, int64_t p_c, int64_t d_r, int64_t d_c,
+               int64_t groups);
+
+/* ------------------------------------------------------------------------------------ */
+/* Device-pointer entry points (buffers already in HBM; asynchronous on `stream`).        */
+/* `stream` is a hipStream_t passed as void*; NULL is the default stream.                 */
+/* ------------------------------------------------------------------------------------ */
+
+typedef struct ntg_gemm_desc {
+    int32_t dtype;              /* ntg_dtype */
+    int32_t transpose_a;
+    int32_t transpose_b;
+    int32_t c_mode;             /* ntg_c_mode */
+    int64_t m, k, n;            /* logical sizes */
+    int64_t lda, ldb, ldc;      /* row length of the STORED matrices in elements; 0 = dense */
+    int64_t batches;            /* >= 1 */
+    int64_t stride_a, stride_b, stride_c;   /* elements between items; 0 on A/B = broadcast */
+    const void* bias;           /* device pointer, NTG_C_BIAS only */
+    int64_t bias_batch_stride, bias_row_stride, bias_col_stride;   /* elements; 0 = broadcast */
+} ntg_gemm_desc;
+
+/* nt_matmult<T> on device buffers: C += op(A).op(B), dense leading dimensions. */
+int ntg_matmult_dev(int dtype, const void* dA, const void* dB, void* dC,
+                    int64_t m, int64_t k, int64_t n, int transpose_a, int transpose_b, void* stream);
+
+/* General strided/broadcast batch; what functional::matmult's N-D x K-D paths
+ * (matmult_cpu.cpp:863-1005) lower to when the views are affine. */
+int ntg_gemm_dev(const ntg_gemm_desc* desc, const void* dA, const void* dB, void* dC, void* stream);
+
+/* nt_matmult_batch<T> with the pointer tables themselves in device memory. */
+int ntg_gemm_ptrs_dev(const ntg_gemm_desc* desc, const void* const* dA, const void* const* dB,
+                      void* const* dC, void* stream);
+
+int ntg_unfold2d_dev(int dtype, const void* image, void* col,
+                     int64_t batch, int64_t channels, int64_t height, int64_t width,
+                     int64_t k_r, int64_t k_c, int64_t s_r, int64_t s_c,
+                     int64_t p_r, int64_t p_c, int64_t d_r, int64_t d_c, void* stream);
+
+/* bytes of device workspace ntg_conv2d_dev needs (the im2col buffer). */
+int64_t ntg_conv2d_workspace_bytes(int dtype, int64_t batch, int64_t channels, int64_t height, int64_t width,
+                                   int64_t k_r, int64_t k_c, int64_t s_r, int64_t s_c,
+                                   int64_t p_r, int64_t p_c, int64_t d_r, int64_t d_c);
+
+int ntg_conv2d_dev(int dtype, const void* image, const void* kernel, void* out,
+                   void* workspace, int64_t workspace_bytes,
+                   int64_t batch, int64_t channels, int64_t height, int64_t width,
+                   int64_t out_channels, int64_t k_r, int64_t k_c,
+                   int64_t s_r, int64_t s_c, int64_t p_r, int64_t p_c, int64_t d_r, int64_t d_c,
+                   int64_t groups, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* NTGEMM_H */

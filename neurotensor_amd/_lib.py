@@ -1,0 +1,87 @@
+"""ctypes binding of libntgemm.so (the C ABI declared in include/ntgemm.h).
+
+There is no fallback: if the HIP library has not been built, loading raises.
+"""
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libntgemm.so")
+
+# ntg_dtype (== nt::DType values; BF16/U64 are extensions)
+FLOAT16, FLOAT32, FLOAT64 = 0, 1, 2
+INT8, INT16, INT32, INT64 = 7, 8, 9, 10
+UINT8, UINT16, UINT32 = 12, 13, 14
+BFLOAT16, UINT64 = 100, 101
+
+C_OVERWRITE, C_ACCUMULATE, C_BIAS = 0, 1, 2
+
+STATUS_NAMES = {0: "NTG_OK", 1: "NTG_ERR_INVALID_ARGUMENT", 2: "NTG_ERR_UNSUPPORTED_DTYPE",
+                3: "NTG_ERR_DEVICE", 4: "NTG_ERR_OUT_OF_MEMORY", 5: "NTG_ERR_NO_DEVICE"}
+
+
+class GemmDesc(ctypes.Structure):
+    _fields_ = [
+        ("dtype", ctypes.c_int32), ("transpose_a", ctypes.c_int32), ("transpose_b", ctypes.c_int32), ("c_mode", ctypes.c_int32),
+        ("m", ctypes.c_int64), ("k", ctypes.c_int64), ("n", ctypes.c_int64),
+        ("lda", ctypes.c_int64), ("ldb", ctypes.c_int64), ("ldc", ctypes.c_int64),
+        ("batches", ctypes.c_int64),
+        ("stride_a", ctypes.c_int64), ("stride_b", ctypes.c_int64), ("stride_c", ctypes.c_int64),
+        ("bias", ctypes.c_void_p),
+        ("bias_batch_stride", ctypes.c_int64), ("bias_row_stride", ctypes.c_int64), ("bias_col_stride", ctypes.c_int64),
+    ]
+
+
+class NtgError(RuntimeError):
+    """Raised when an entry point of libntgemm.so returns a non-zero ntg_status."""
+
+    def __init__(self, status, message):
+        super().__init__(f"{STATUS_NAMES.get(status, status)}: {message}")
+        self.status = status
+
+
+# every symbol include/ntgemm.h declares, with its ctypes signature
+_i64, _vp, _ci = ctypes.c_int64, ctypes.c_void_p, ctypes.c_int
+_pp = ctypes.POINTER(ctypes.c_void_p)
+SIGNATURES = {
+    "ntg_last_error": (ctypes.c_char_p, []),
+    "ntg_version": (_ci, []),
+    "ntg_dtype_size": (_i64, [_ci]),
+    "ntg_device_count": (_ci, []),
+    "ntg_matmult": (_ci, [_ci, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _ci, _ci]),
+    "ntg_matmult_batch": (_ci, [_ci, _pp, _pp, _pp, _i64, _i64, _i64, _i64, _i64, _ci, _ci]),
+    "ntg_linear": (_ci, [_ci, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _ci, _ci, _i64, _i64]),
+    "ntg_unfold2d": (_ci, [_ci, _vp, _vp] + [_i64] * 12),
+    "ntg_conv2d": (_ci, [_ci, _vp, _vp, _vp] + [_i64] * 14),
+    "ntg_matmult_dev": (_ci, [_ci, _vp, _vp, _vp, _i64, _i64, _i64, _ci, _ci, _vp]),
+    "ntg_gemm_dev": (_ci, [ctypes.POINTER(GemmDesc), _vp, _vp, _vp, _vp]),
+    "ntg_gemm_ptrs_dev": (_ci, [ctypes.POINTER(GemmDesc), _vp, _vp, _vp, _vp]),
+    "ntg_unfold2d_dev": (_ci, [_ci, _vp, _vp] + [_i64] * 12 + [_vp]),
+    "ntg_conv2d_workspace_bytes": (_i64, [_ci] + [_i64] * 12),
+    "ntg_conv2d_dev": (_ci, [_ci, _vp, _vp, _vp, _vp, _i64] + [_i64] * 14 + [_vp]),
+}
+
+_lib = None
+
+
+def load():
+    """Load libntgemm.so once; raise if it is missing (no CPU fallback exists)."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(
+            f"{LIB_PATH} is missing: the HIP extension is not built. "
+            "Run `python -c 'import __graft_entry__ as g; g.build()'` (or `make -C neurotensor_amd/csrc`).")
+    lib = ctypes.CDLL(LIB_PATH)
+    for name, (res, args) in SIGNATURES.items():
+        fn = getattr(lib, name)          # AttributeError if the symbol is not exported
+        fn.restype = res
+        fn.argtypes = args
+    _lib = lib
+    return lib
+
+
+def check(status):
+    if status != 0:
+        raise NtgError(status, load().ntg_last_error().decode("utf-8", "replace"))

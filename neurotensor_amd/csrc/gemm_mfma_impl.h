@@ -1,0 +1,392 @@
+// LDS-tiled MFMA GEMM for gfx950:  C (+)= op(A) . op(B)   (row-major, dense)
+//
+// Replaces the packed SIMD path of the reference, pack_multiply_directly_var_threaded
+// (nt/functional/cpu/matmult/nt_matmult.hpp:124-225) and its micro kernel
+// (nt_matmult_simde.hpp:301-350), for Float32, Float64, Float16 and BFloat16.
+//
+// One workgroup = 4 wavefronts in a 2x2 grid; each wavefront owns WBM x WBN MFMA blocks
+// (32x32 for fp32/fp16/bf16, 16x16 for fp64) of a BM x BN tile of C and walks K in steps
+// of BK through double-buffered LDS.  transpose_a / transpose_b, leading dimensions,
+// batch strides (0 = broadcast) and pointer-table batches are absorbed by the loaders:
+// nothing is copied or re-laid-out in global memory.
+//
+// LDS layouts ("vec" = 16 bytes):
+//   K-major  [tile row][BK/VE vecs + 1 pad vec]   for operands stored K-contiguous; a lane
+//            reads one vec = VE consecutive k of its row.  The odd row stride makes the
+//            16 rows read together fall into 16 different 16-byte bank groups.
+//   MN-major [k row][tile rows]                    fp32/fp64 operands stored MN-contiguous;
+//            a lane reads WB consecutive rows at one k, so MFMA block b of the wavefront
+//            covers tile rows  lane_row*WB + b  (interleaved) and no transposition exists.
+//   16-bit operands stored MN-contiguous are transposed in registers (8x8 sub-blocks,
+//   v_perm_b32) on their way into the K-major layout, because an MFMA lane needs 8
+//   consecutive k packed in 4 registers.
+#pragma once
+#include "ntg_common.h"
+
+namespace ntg {
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef double doublex4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 halfx8 __attribute__((ext_vector_type(8)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+template <int DT> struct Elem;
+
+template <> struct Elem<DT_F32> {
+    using T = float; using AccS = float; using AccV = floatx16;
+    static constexpr int R = 32, G = 2, VE = 4, ACCN = 16;
+    static __device__ __forceinline__ void mma(AccV& c, float a, float b) { c = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0); }
+};
+template <> struct Elem<DT_F64> {
+    using T = double; using AccS = double; using AccV = doublex4;
+    static constexpr int R = 16, G = 4, VE = 2, ACCN = 4;
+    static __device__ __forceinline__ void mma(AccV& c, double a, double b) { c = __builtin_amdgcn_mfma_f64_16x16x4f64(a, b, c, 0, 0, 0); }
+};
+template <> struct Elem<DT_F16> {
+    using T = _Float16; using AccS = float; using AccV = floatx16;
+    static constexpr int R = 32, G = 2, VE = 8, ACCN = 16;
+    static __device__ __forceinline__ void mma(AccV& c, u32x4 a, u32x4 b) {
+        c = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(halfx8, a), __builtin_bit_cast(halfx8, b), c, 0, 0, 0);
+    }
+};
+template <> struct Elem<DT_BF16> {
+    using T = __bf16; using AccS = float; using AccV = floatx16;
+    static constexpr int R = 32, G = 2, VE = 8, ACCN = 16;
+    static __device__ __forceinline__ void mma(AccV& c, u32x4 a, u32x4 b) {
+        c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+    }
+};
+
+// row of the R x R result block held in accumulator register r of `lane`
+template <int R> __device__ __forceinline__ int acc_row(int r, int lane);
+template <> __device__ __forceinline__ int acc_row<32>(int r, int lane) { return 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3); }
+template <> __device__ __forceinline__ int acc_row<16>(int r, int lane) { return 4 * r + (lane >> 4); }
+
+template <class T, int VE, bool ALIGNED>
+__device__ __forceinline__ u32x4 ldvec(const T* src, bool outer_ok, int c0, int cmax, bool vec_ok) {
+    if constexpr (ALIGNED) {
+        return *reinterpret_cast<const u32x4*>(src);
+    } else {
+        u32x4 r = {0u, 0u, 0u, 0u};
+        if (outer_ok) {
+            if (vec_ok && c0 + VE <= cmax) {
+                r = *reinterpret_cast<const u32x4*>(src);
+            } else {
+                T tmp[VE];
+#pragma unroll
+                for (int e = 0; e < VE; ++e) tmp[e] = (c0 + e < cmax) ? src[e] : (T)0.0f;
+                __builtin_memcpy(&r, tmp, 16);
+            }
+        }
+        return r;
+    }
+}
+
+// One operand's BMN x BK tile: global -> registers -> LDS.
+//   KC: stored K-contiguous in global memory (A without transpose_a, B with transpose_b)
+//   KM: K-major LDS layout
+template <int DT, bool KC, bool KM, int TMN, int BK, bool ALIGNED>
+struct TileLoader {
+    using T = typename Elem<DT>::T;
+    static constexpr int VE = Elem<DT>::VE;
+    static constexpr int KV = BK / VE;
+    static constexpr int S = KV + 1;
+    static constexpr int MV = TMN / VE;
+    static constexpr int LDS_BYTES = KM ? TMN * S * 16 : BK * MV * 16;
+    static constexpr bool TRANSPOSE = (!KC && KM);
+    static constexpr int KG = BK / 8;
+    static constexpr int NSB = KG * (TMN / 8);
+    static constexpr int NQ = (NSB + 255) / 256;
+    static constexpr int NV = TRANSPOSE ? 8 * NQ : (TMN * BK / VE) / 256;
+    static_assert(TRANSPOSE ? (VE == 8) : ((TMN * BK / VE) % 256 == 0), "tile does not split over 256 threads");
+    static_assert(KM || !KC, "K-contiguous operands always use the K-major layout");
+
+    u32x4 v[NV];
+
+    __device__ __forceinline__ void load(const T* base, int64_t ld, int mn0, int k0, int MN, int K, bool vec_ok, int tid) {
+        if constexpr (!TRANSPOSE && KC) {
+#pragma unroll
+            for (int p = 0; p < NV; ++p) {
+                const int vi = tid + p * 256;
+                const int row = vi / KV, kv = vi % KV;
+                const int mn = mn0 + row, k = k0 + kv * VE;
+                v[p] = ldvec<T, VE, ALIGNED>(base + (int64_t)mn * ld + k, mn < MN, k, K, vec_ok);
+            }
+        } else if constexpr (!TRANSPOSE) {
+#pragma unroll
+            for (int p = 0; p < NV; ++p) {
+                const int vi = tid + p * 256;
+                const int kr = vi / MV, mv = vi % MV;
+                const int k = k0 + kr, mn = mn0 + mv * VE;
+                v[p] = ldvec<T, VE, ALIGNED>(base + (int64_t)k * ld + mn, k < K, mn, MN, vec_ok);
+            }
+        } else {
+#pragma unroll
+            for (int q = 0; q < NQ; ++q) {
+                const int sb = tid + q * 256;
+                if (NSB % 256 == 0 || sb < NSB) {
+                    const int kg = sb % KG, mv = sb / KG;
+                    const int mn = mn0 + mv * 8;
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) {
+                        const int k = k0 + kg * 8 + i;
+                        v[q * 8 + i] = ldvec<T, VE, ALIGNED>(base + (int64_t)k * ld + mn, k < K, mn, MN, vec_ok);
+                    }
+                }
+            }
+        }
+    }
+
+    __device__ __forceinline__ void store(char* lds, int tid) const {
+        if constexpr (!TRANSPOSE && KC) {
+#pragma unroll
+            for (int p = 0; p < NV; ++p) {
+                const int vi = tid + p * 256;
+                const int row = vi / KV, kv = vi % KV;
+                *reinterpret_cast<u32x4*>(lds + (row * S + kv) * 16) = v[p];
+            }
+        } else if constexpr (!TRANSPOSE) {
+#pragma unroll
+            for (int p = 0; p < NV; ++p) {
+                const int vi = tid + p * 256;
+                *reinterpret_cast<u32x4*>(lds + vi * 16) = v[p];
+            }
+        } else {
+#pragma unroll
+            for (int q = 0; q < NQ; ++q) {
+                const int sb = tid + q * 256;
+                if (NSB % 256 == 0 || sb < NSB) {
+                    const int kg = sb % KG, mv = sb / KG;
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) {
+                        // output vec j = tile row mv*8+j, k = kg*8 .. kg*8+7:
+                        // dword d packs element j of source vecs 2d and 2d+1
+                        u32x4 o;
+#pragma unroll
+                        for (int d = 0; d < 4; ++d) {
+                            const uint32_t lo = v[q * 8 + 2 * d][j >> 1];
+                            const uint32_t hi = v[q * 8 + 2 * d + 1][j >> 1];
+                            o[d] = (j & 1) ? __builtin_amdgcn_perm(hi, lo, 0x07060302u)
+                                           : __builtin_amdgcn_perm(hi, lo, 0x05040100u);
+                        }
+                        *reinterpret_cast<u32x4*>(lds + ((mv * 8 + j) * S + kg) * 16) = o;
+                    }
+                }
+            }
+        }
+    }
+};
+
+template <int DT, bool TA, bool TB, int WBM, int WBN, int BK>
+struct GemmShape {
+    using E = Elem<DT>;
+    using T = typename E::T;
+    static constexpr bool IS16 = sizeof(T) == 2;
+    static constexpr bool A_KC = !TA, B_KC = TB;
+    static constexpr bool A_KM = IS16 || A_KC, B_KM = IS16 || B_KC;
+    static constexpr int BM = 2 * WBM * E::R, BN = 2 * WBN * E::R;
+    static constexpr int LDS_A = TileLoader<DT, A_KC, A_KM, BM, BK, true>::LDS_BYTES;
+    static constexpr int LDS_B = TileLoader<DT, B_KC, B_KM, BN, BK, true>::LDS_BYTES;
+    static constexpr int STAGE = LDS_A + LDS_B;
+    static constexpr int LDS_TOTAL = 2 * STAGE;
+    static constexpr int GROUP_M = (1024 / BM) > 0 ? (1024 / BM) : 1;
+};
+
+template <int DT, bool TA, bool TB, int WBM, int WBN, int BK, bool ALIGNED>
+__global__ void __launch_bounds__(256) gemm_mfma_kernel(const GemmParams p) {
+    using SH = GemmShape<DT, TA, TB, WBM, WBN, BK>;
+    using E = Elem<DT>;
+    using T = typename E::T;
+    using AccS = typename E::AccS;
+    using AccV = typename E::AccV;
+    constexpr int R = E::R, G = E::G, VE = E::VE;
+    constexpr bool IS16 = SH::IS16;
+    constexpr bool A_KM = SH::A_KM, B_KM = SH::B_KM;
+    constexpr int BM = SH::BM, BN = SH::BN;
+    using LA = TileLoader<DT, SH::A_KC, A_KM, BM, BK, ALIGNED>;
+    using LB = TileLoader<DT, SH::B_KC, B_KM, BN, BK, ALIGNED>;
+    constexpr int SA = LA::S, SB = LB::S;
+
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int lr = lane % R, lg = lane / R;
+
+    const int lid = xcd_contiguous_id(blockIdx.x, gridDim.x);
+    const int tiles = p.tiles_m * p.tiles_n;
+    const int b = lid / tiles;
+    int tm, tn;
+    tile_coords(lid - b * tiles, p.tiles_m, p.tiles_n, SH::GROUP_M, tm, tn);
+    const int m0 = tm * BM, n0 = tn * BN;
+
+    const T* A = p.Aptr ? static_cast<const T*>(p.Aptr[b]) : static_cast<const T*>(p.A) + (int64_t)b * p.sA;
+    const T* B = p.Bptr ? static_cast<const T*>(p.Bptr[b]) : static_cast<const T*>(p.B) + (int64_t)b * p.sB;
+    T* C = p.Cptr ? static_cast<T*>(p.Cptr[b]) : static_cast<T*>(p.C) + (int64_t)b * p.sC;
+    const bool vecA = p.vecA_ok && ((reinterpret_cast<uintptr_t>(A) & 15) == 0);
+    const bool vecB = p.vecB_ok && ((reinterpret_cast<uintptr_t>(B) & 15) == 0);
+
+    AccV acc[WBM][WBN];
+#pragma unroll
+    for (int i = 0; i < WBM; ++i)
+#pragma unroll
+        for (int j = 0; j < WBN; ++j)
+#pragma unroll
+            for (int r = 0; r < E::ACCN; ++r) acc[i][j][r] = (AccS)0;
+
+    LA la;
+    LB lb;
+    const int KT = (p.K + BK - 1) / BK;
+
+    la.load(A, p.lda, m0, 0, p.M, p.K, vecA, tid);
+    lb.load(B, p.ldb, n0, 0, p.N, p.K, vecB, tid);
+    la.store(smem, tid);
+    lb.store(smem + SH::LDS_A, tid);
+    __syncthreads();
+
+    for (int kt = 0; kt < KT; ++kt) {
+        const char* sA = smem + (kt & 1) * SH::STAGE;
+        const char* sB = sA + SH::LDS_A;
+        const bool more = (kt + 1 < KT);
+        if (more) {
+            la.load(A, p.lda, m0, (kt + 1) * BK, p.M, p.K, vecA, tid);
+            lb.load(B, p.ldb, n0, (kt + 1) * BK, p.N, p.K, vecB, tid);
+        }
+
+        if constexpr (IS16) {
+            constexpr int KQ = BK / 16;
+#pragma unroll
+            for (int kq = 0; kq < KQ; ++kq) {
+                u32x4 af[WBM], bf[WBN];
+#pragma unroll
+                for (int i = 0; i < WBM; ++i)
+                    af[i] = *reinterpret_cast<const u32x4*>(sA + (((wm * WBM + i) * R + lr) * SA + kq * G + lg) * 16);
+#pragma unroll
+                for (int j = 0; j < WBN; ++j)
+                    bf[j] = *reinterpret_cast<const u32x4*>(sB + (((wn * WBN + j) * R + lr) * SB + kq * G + lg) * 16);
+#pragma unroll
+                for (int i = 0; i < WBM; ++i)
+#pragma unroll
+                    for (int j = 0; j < WBN; ++j) E::mma(acc[i][j], af[i], bf[j]);
+            }
+        } else {
+            constexpr int KQ = BK / (G * VE);
+            typedef T TVA __attribute__((ext_vector_type(WBM)));
+            typedef T TVB __attribute__((ext_vector_type(WBN)));
+            typedef T TVE __attribute__((ext_vector_type(VE)));
+#pragma unroll
+            for (int kq = 0; kq < KQ; ++kq) {
+                T af[WBM][VE], bf[WBN][VE];
+                if constexpr (A_KM) {
+#pragma unroll
+                    for (int i = 0; i < WBM; ++i) {
+                        const TVE t = *reinterpret_cast<const TVE*>(sA + (((wm * WBM + i) * R + lr) * SA + kq * G + lg) * 16);
+#pragma unroll
+                        for (int e = 0; e < VE; ++e) af[i][e] = t[e];
+                    }
+                } else {
+#pragma unroll
+                    for (int e = 0; e < VE; ++e) {
+                        const int krow = (kq * G + lg) * VE + e;
+                        const TVA t = *reinterpret_cast<const TVA*>(sA + ((int)sizeof(T)) * (krow * BM + (wm * R + lr) * WBM));
+#pragma unroll
+                        for (int i = 0; i < WBM; ++i) af[i][e] = t[i];
+                    }
+                }
+                if constexpr (B_KM) {
+#pragma unroll
+                    for (int j = 0; j < WBN; ++j) {
+                        const TVE t = *reinterpret_cast<const TVE*>(sB + (((wn * WBN + j) * R + lr) * SB + kq * G + lg) * 16);
+#pragma unroll
+                        for (int e = 0; e < VE; ++e) bf[j][e] = t[e];
+                    }
+                } else {
+#pragma unroll
+                    for (int e = 0; e < VE; ++e) {
+                        const int krow = (kq * G + lg) * VE + e;
+                        const TVB t = *reinterpret_cast<const TVB*>(sB + ((int)sizeof(T)) * (krow * BN + (wn * R + lr) * WBN));
+#pragma unroll
+                        for (int j = 0; j < WBN; ++j) bf[j][e] = t[j];
+                    }
+                }
+#pragma unroll
+                for (int e = 0; e < VE; ++e)
+#pragma unroll
+                    for (int i = 0; i < WBM; ++i)
+#pragma unroll
+                        for (int j = 0; j < WBN; ++j) E::mma(acc[i][j], af[i][e], bf[j][e]);
+            }
+        }
+
+        if (more) {
+            char* dA = smem + ((kt + 1) & 1) * SH::STAGE;
+            la.store(dA, tid);
+            lb.store(dA + SH::LDS_A, tid);
+        }
+        __syncthreads();
+    }
+
+    // epilogue: every lane owns ACCN elements per block; C0 comes from C (accumulate),
+    // from the broadcast bias (linear) or is zero (overwrite)
+    const int cmode = p.cmode;
+    const T* bias = static_cast<const T*>(p.bias);
+#pragma unroll
+    for (int i = 0; i < WBM; ++i) {
+#pragma unroll
+        for (int j = 0; j < WBN; ++j) {
+            const int n = n0 + (B_KM ? (wn * WBN + j) * R + lr : (wn * R + lr) * WBN + j);
+#pragma unroll
+            for (int r = 0; r < E::ACCN; ++r) {
+                const int lrow = acc_row<R>(r, lane);
+                const int m = m0 + (A_KM ? (wm * WBM + i) * R + lrow : (wm * R + lrow) * WBM + i);
+                if (ALIGNED || (m < p.M && n < p.N)) {
+                    T* cp = C + (int64_t)m * p.ldc + n;
+                    AccS val = acc[i][j][r];
+                    if (cmode == C_ACCUMULATE) val += (AccS)(*cp);
+                    else if (cmode == C_BIAS) val += (AccS)bias[(int64_t)b * p.bias_bs + (int64_t)m * p.bias_rs + (int64_t)n * p.bias_cs];
+                    *cp = (T)val;
+                }
+            }
+        }
+    }
+}
+
+template <int DT, bool TA, bool TB, int WBM, int WBN, int BK>
+static hipError_t launch_cfg(const GemmParams& pin, hipStream_t s) {
+    using SH = GemmShape<DT, TA, TB, WBM, WBN, BK>;
+    GemmParams p = pin;
+    p.tiles_m = (p.M + SH::BM - 1) / SH::BM;
+    p.tiles_n = (p.N + SH::BN - 1) / SH::BN;
+    const int64_t blocks = (int64_t)p.tiles_m * p.tiles_n * p.batch;
+    if (blocks <= 0) return hipSuccess;
+    if (blocks > 0x7fffffffLL) return hipErrorInvalidValue;
+    constexpr int VE = Elem<DT>::VE;
+    const bool aligned = (p.M % SH::BM == 0) && (p.N % SH::BN == 0) && (p.K % BK == 0) &&
+                         p.vecA_ok && p.vecB_ok && !p.Aptr && !p.Bptr &&
+                         ((reinterpret_cast<uintptr_t>(p.A) & 15) == 0) && ((reinterpret_cast<uintptr_t>(p.B) & 15) == 0) &&
+                         (p.sA % VE == 0) && (p.sB % VE == 0);
+    // tiles above 64 KiB of LDS need the opt-in once per kernel
+    if (aligned) {
+        auto k = gemm_mfma_kernel<DT, TA, TB, WBM, WBN, BK, true>;
+        static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(k), hipFuncAttributeMaxDynamicSharedMemorySize, SH::LDS_TOTAL);
+        if (attr != hipSuccess) return attr;
+        hipLaunchKernelGGL(k, dim3((unsigned)blocks), dim3(256), SH::LDS_TOTAL, s, p);
+    } else {
+        auto k = gemm_mfma_kernel<DT, TA, TB, WBM, WBN, BK, false>;
+        static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(k), hipFuncAttributeMaxDynamicSharedMemorySize, SH::LDS_TOTAL);
+        if (attr != hipSuccess) return attr;
+        hipLaunchKernelGGL(k, dim3((unsigned)blocks), dim3(256), SH::LDS_TOTAL, s, p);
+    }
+    return hipGetLastError();
+}
+
+template <int DT, int WBM, int WBN, int BK>
+static hipError_t launch_trans(bool ta, bool tb, const GemmParams& p, hipStream_t s) {
+    if (ta) return tb ? launch_cfg<DT, true, true, WBM, WBN, BK>(p, s) : launch_cfg<DT, true, false, WBM, WBN, BK>(p, s);
+    return tb ? launch_cfg<DT, false, true, WBM, WBN, BK>(p, s) : launch_cfg<DT, false, false, WBM, WBN, BK>(p, s);
+}
+
+}  // namespace ntg

@@ -1,0 +1,84 @@
+// Shared declarations of the gfx950 matmult backend (device + host side).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace ntg {
+
+// numeric values follow nt::DType (nt/dtype/DType_enum.h:14-20); BF16/U64 are extensions
+enum DType : int {
+    DT_F16 = 0, DT_F32 = 1, DT_F64 = 2,
+    DT_I8 = 7, DT_I16 = 8, DT_I32 = 9, DT_I64 = 10,
+    DT_U8 = 12, DT_U16 = 13, DT_U32 = 14,
+    DT_BF16 = 100, DT_U64 = 101
+};
+
+// how the kernel treats the incoming C
+enum CMode : int {
+    C_OVERWRITE = 0,   // C  = op(A).op(B)          (caller knows C would be zeros)
+    C_ACCUMULATE = 1,  // C += op(A).op(B)          (contract of nt_matmult, nt_matmult.hpp:370-378)
+    C_BIAS = 2         // C  = bias (+) op(A).op(B) (cpu::linear, matmult_cpu.cpp:1637-1647)
+};
+
+struct GemmParams {
+    const void* A;
+    const void* B;
+    void* C;
+    // pointer tables in device memory (nt_matmult_batch's A[]/B[]/C[]); null => strided addressing
+    const void* const* Aptr;
+    const void* const* Bptr;
+    void* const* Cptr;
+    // C_BIAS: C0(b,i,j) = bias[b*bias_bs + i*bias_rs + j*bias_cs]
+    const void* bias;
+    int64_t bias_bs, bias_rs, bias_cs;
+    int64_t lda, ldb, ldc;   // row length of the stored matrices, in elements
+    int64_t sA, sB, sC;      // batch strides in elements, 0 = the same matrix for every item
+    int M, N, K, batch;      // logical sizes (after the transpose flags)
+    int cmode;
+    int tiles_m, tiles_n;
+    int vecA_ok, vecB_ok;    // 16-byte vector loads are legal for every row of A / B
+};
+
+static inline int64_t elem_size(int dt) {
+    switch (dt) {
+    case DT_I8: case DT_U8: return 1;
+    case DT_F16: case DT_BF16: case DT_I16: case DT_U16: return 2;
+    case DT_F32: case DT_I32: case DT_U32: return 4;
+    case DT_F64: case DT_I64: case DT_U64: return 8;
+    default: return 0;
+    }
+}
+
+// launchers implemented in the .hip files; all return a hipError_t
+hipError_t launch_gemm_mfma(int dtype, bool ta, bool tb, const GemmParams& p, hipStream_t s);
+hipError_t launch_gemm_valu(int dtype, bool ta, bool tb, const GemmParams& p, hipStream_t s);
+hipError_t launch_gemm_skinny(int dtype, bool ta, bool tb, const GemmParams& p, hipStream_t s, bool* handled);
+hipError_t launch_unfold2d(int64_t elem_size, const void* im, void* col,
+                           int64_t batch, int64_t channels, int64_t height, int64_t width,
+                           int64_t k_r, int64_t k_c, int64_t s_r, int64_t s_c,
+                           int64_t p_r, int64_t p_c, int64_t d_r, int64_t d_c, hipStream_t s);
+
+#ifdef __HIPCC__
+// Workgroup ids are dealt round-robin to the 8 XCDs; make the ids that land on one
+// XCD (its own L2) a contiguous range of logical tile ids.
+__device__ __forceinline__ int xcd_contiguous_id(int bid, int nb) {
+    const int NX = 8;
+    const int base = nb / NX, rem = nb % NX;
+    const int x = bid % NX, q = bid / NX;
+    return x * base + (x < rem ? x : rem) + q;
+}
+
+// logical id -> (tile_m, tile_n): column-major inside groups of GROUP_M tile rows,
+// so a contiguous id range covers a compact rectangle of C.
+__device__ __forceinline__ void tile_coords(int t, int tiles_m, int tiles_n, int GROUP_M, int& tm, int& tn) {
+    const int group_size = GROUP_M * tiles_n;
+    const int g = t / group_size;
+    const int first_m = g * GROUP_M;
+    const int gm = (tiles_m - first_m < GROUP_M) ? tiles_m - first_m : GROUP_M;
+    const int r = t - g * group_size;
+    tm = first_m + r % gm;
+    tn = r / gm;
+}
+#endif
+
+}  // namespace ntg

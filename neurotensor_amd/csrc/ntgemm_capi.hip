@@ -1,0 +1,408 @@
+// C ABI of the gfx950 matmult backend (declared in include/ntgemm.h): argument checks,
+// dtype dispatch, host<->device staging for the host-pointer entry points, and the
+// conv2d lowering.  No entry point throws; failures are reported as ntg_status plus a
+// thread-local message.
+#include "../../include/ntgemm.h"
+#include "ntg_common.h"
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <map>
+#include <string>
+#include <vector>
+
+namespace ntg {
+hipError_t launch_gemm_mfma_f32(bool ta, bool tb, const GemmParams& p, hipStream_t s);
+hipError_t launch_gemm_mfma_f64(bool ta, bool tb, const GemmParams& p, hipStream_t s);
+hipError_t launch_gemm_mfma_f16(bool ta, bool tb, const GemmParams& p, hipStream_t s);
+hipError_t launch_gemm_mfma_bf16(bool ta, bool tb, const GemmParams& p, hipStream_t s);
+hipError_t launch_gemm_skinny(int dtype, bool ta, bool tb, const GemmParams& p, hipStream_t s, bool* handled);
+}  // namespace ntg
+
+namespace {
+
+thread_local std::string g_last_error;
+
+int fail(int status, const char* fmt, ...) {
+    char buf[512];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof buf, fmt, ap);
+    va_end(ap);
+    g_last_error = buf;
+    return status;
+}
+
+int hip_fail(hipError_t e, const char* what) {
+    if (e == hipErrorOutOfMemory) return fail(NTG_ERR_OUT_OF_MEMORY, "%s: %s", what, hipGetErrorString(e));
+    if (e == hipErrorNoDevice || e == hipErrorInvalidDevice) return fail(NTG_ERR_NO_DEVICE, "%s: %s", what, hipGetErrorString(e));
+    return fail(NTG_ERR_DEVICE, "%s: %s", what, hipGetErrorString(e));
+}
+
+#define HIP_TRY(expr)                                   \
+    do {                                                \
+        hipError_t e__ = (expr);                        \
+        if (e__ != hipSuccess) return hip_fail(e__, #expr); \
+    } while (0)
+
+struct DeviceMem {
+    void* p = nullptr;
+    ~DeviceMem() { if (p) (void)hipFree(p); }
+    hipError_t alloc(size_t bytes) { return hipMalloc(&p, bytes ? bytes : 1); }
+    char* at(size_t off) const { return static_cast<char*>(p) + off; }
+};
+
+inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+bool is_int_dtype(int dt) {
+    switch (dt) {
+    case ntg::DT_I8: case ntg::DT_I16: case ntg::DT_I32: case ntg::DT_I64:
+    case ntg::DT_U8: case ntg::DT_U16: case ntg::DT_U32: case ntg::DT_U64: return true;
+    default: return false;
+    }
+}
+
+// Fills the derived fields and launches the kernel family for the dtype.
+int run_gemm(ntg::GemmParams p, int dtype, bool ta, bool tb, hipStream_t s) {
+    const int64_t es = ntg::elem_size(dtype);
+    if (es == 0) return fail(NTG_ERR_UNSUPPORTED_DTYPE, "dtype %d is not supported by the gfx950 matmult backend", dtype);
+    if (p.M == 0 || p.N == 0 || p.batch == 0) return NTG_OK;
+    const int64_t ve = 16 / es;
+    p.vecA_ok = (p.lda % ve == 0) && (p.Aptr || p.sA % ve == 0);
+    p.vecB_ok = (p.ldb % ve == 0) && (p.Bptr || p.sB % ve == 0);
+    hipError_t e;
+    if (is_int_dtype(dtype)) {
+        e = ntg::launch_gemm_valu(dtype, ta, tb, p, s);
+    } else {
+        bool handled = false;
+        e = ntg::launch_gemm_skinny(dtype, ta, tb, p, s, &handled);
+        if (e != hipSuccess) return hip_fail(e, "skinny gemm launch");
+        if (handled) return NTG_OK;
+        switch (dtype) {
+        case ntg::DT_F32: e = ntg::launch_gemm_mfma_f32(ta, tb, p, s); break;
+        case ntg::DT_F64: e = ntg::launch_gemm_mfma_f64(ta, tb, p, s); break;
+        case ntg::DT_F16: e = ntg::launch_gemm_mfma_f16(ta, tb, p, s); break;
+        case ntg::DT_BF16: e = ntg::launch_gemm_mfma_bf16(ta, tb, p, s); break;
+        default: return fail(NTG_ERR_UNSUPPORTED_DTYPE, "dtype %d is not supported", dtype);
+        }
+    }
+    if (e != hipSuccess) return hip_fail(e, "gemm launch");
+    return NTG_OK;
+}
+
+int check_sizes(int64_t m, int64_t k, int64_t n, int64_t batches) {
+    if (m < 0 || k < 0 || n < 0 || batches < 0) return fail(NTG_ERR_INVALID_ARGUMENT, "negative size (m=%lld k=%lld n=%lld batches=%lld)", (long long)m, (long long)k, (long long)n, (long long)batches);
+    if (m > 0x7fffffffLL || k > 0x7fffffffLL || n > 0x7fffffffLL || batches > 0x7fffffffLL)
+        return fail(NTG_ERR_INVALID_ARGUMENT, "a size exceeds 2^31-1");
+    return NTG_OK;
+}
+
+int desc_to_params(const ntg_gemm_desc* d, ntg::GemmParams& p) {
+    if (!d) return fail(NTG_ERR_INVALID_ARGUMENT, "null descriptor");
+    if (ntg::elem_size(d->dtype) == 0) return fail(NTG_ERR_UNSUPPORTED_DTYPE, "dtype %d is not supported", d->dtype);
+    int rc = check_sizes(d->m, d->k, d->n, d->batches);
+    if (rc) return rc;
+    if (d->c_mode < 0 || d->c_mode > 2) return fail(NTG_ERR_INVALID_ARGUMENT, "c_mode %d is not one of overwrite/accumulate/bias", d->c_mode);
+    std::memset(&p, 0, sizeof p);
+    p.M = (int)d->m; p.K = (int)d->k; p.N = (int)d->n; p.batch = (int)d->batches;
+    p.lda = d->lda ? d->lda : (d->transpose_a ? d->m : d->k);
+    p.ldb = d->ldb ? d->ldb : (d->transpose_b ? d->k : d->n);
+    p.ldc = d->ldc ? d->ldc : d->n;
+    if (p.lda < (d->transpose_a ? d->m : d->k) || p.ldb < (d->transpose_b ? d->k : d->n) || p.ldc < d->n)
+        return fail(NTG_ERR_INVALID_ARGUMENT, "leading dimension smaller than the stored row length");
+    p.sA = d->stride_a; p.sB = d->stride_b; p.sC = d->stride_c;
+    p.cmode = d->c_mode;
+    p.bias = d->bias;
+    p.bias_bs = d->bias_batch_stride; p.bias_rs = d->bias_row_stride; p.bias_cs = d->bias_col_stride;
+    if (p.cmode == NTG_C_BIAS && !p.bias) return fail(NTG_ERR_INVALID_ARGUMENT, "c_mode is bias but bias is null");
+    return NTG_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* ntg_last_error(void) { return g_last_error.c_str(); }
+int ntg_version(void) { return 100; }
+int64_t ntg_dtype_size(int dtype) { return ntg::elem_size(dtype); }
+
+int ntg_device_count(void) {
+    int n = 0;
+    if (hipGetDeviceCount(&n) != hipSuccess) return 0;
+    return n;
+}
+
+int ntg_gemm_dev(const ntg_gemm_desc* d, const void* dA, const void* dB, void* dC, void* stream) {
+    ntg::GemmParams p;
+    int rc = desc_to_params(d, p);
+    if (rc) return rc;
+    if (p.M == 0 || p.N == 0 || p.batch == 0) return NTG_OK;
+    if (!dA || !dB || !dC) return fail(NTG_ERR_INVALID_ARGUMENT, "null matrix pointer");
+    if (p.batch > 1 && p.sC == 0) return fail(NTG_ERR_INVALID_ARGUMENT, "stride_c must be non-zero for a batch (outputs may not alias)");
+    p.A = dA; p.B = dB; p.C = dC;
+    return run_gemm(p, d->dtype, d->transpose_a != 0, d->transpose_b != 0, static_cast<hipStream_t>(stream));
+}
+
+int ntg_gemm_ptrs_dev(const ntg_gemm_desc* d, const void* const* dA, const void* const* dB, void* const* dC, void* stream) {
+    ntg::GemmParams p;
+    int rc = desc_to_params(d, p);
+    if (rc) return rc;
+    if (p.M == 0 || p.N == 0 || p.batch == 0) return NTG_OK;
+    if (!dA || !dB || !dC) return fail(NTG_ERR_INVALID_ARGUMENT, "null pointer table");
+    p.Aptr = dA; p.Bptr = dB; p.Cptr = dC;
+    return run_gemm(p, d->dtype, d->transpose_a != 0, d->transpose_b != 0, static_cast<hipStream_t>(stream));
+}
+
+int ntg_matmult_dev(int dtype, const void* dA, const void* dB, void* dC, int64_t m, int64_t k, int64_t n,
+                    int transpose_a, int transpose_b, void* stream) {
+    ntg_gemm_desc d;
+    std::memset(&d, 0, sizeof d);
+    d.dtype = dtype; d.transpose_a = transpose_a; d.transpose_b = transpose_b; d.c_mode = NTG_C_ACCUMULATE;
+    d.m = m; d.k = k; d.n = n; d.batches = 1;
+    return ntg_gemm_dev(&d, dA, dB, dC, stream);
+}
+
+int ntg_matmult(int dtype, const void* A, const void* B, void* C,
+                int64_t a_rows, int64_t a_cols, int64_t b_rows, int64_t b_cols,
+                int transpose_a, int transpose_b) {
+    const void* As[1] = {A};
+    const void* Bs[1] = {B};
+    void* Cs[1] = {C};
+    return ntg_matmult_batch(dtype, As, Bs, Cs, 1, a_rows, a_cols, b_rows, b_cols, transpose_a, transpose_b);
+}
+
+int ntg_matmult_batch(int dtype, const void* const* A, const void* const* B, void* const* C,
+                      int64_t batches, int64_t a_rows, int64_t a_cols, int64_t b_rows, int64_t b_cols,
+                      int transpose_a, int transpose_b) {
+    const int64_t es = ntg::elem_size(dtype);
+    if (es == 0) return fail(NTG_ERR_UNSUPPORTED_DTYPE, "dtype %d is not supported by the gfx950 matmult backend", dtype);
+    if (a_cols != b_rows) return fail(NTG_ERR_INVALID_ARGUMENT, "inner sizes differ: a_cols=%lld b_rows=%lld", (long long)a_cols, (long long)b_rows);
+    const int64_t m = a_rows, k = a_cols, n = b_cols;
+    int rc = check_sizes(m, k, n, batches);
+    if (rc) return rc;
+    if (batches == 0 || m == 0 || n == 0 || k == 0) return NTG_OK;   // C += empty sum
+    if (!A || !B || !C) return fail(NTG_ERR_INVALID_ARGUMENT, "null pointer array");
+    for (int64_t i = 0; i < batches; ++i)
+        if (!A[i] || !B[i] || !C[i]) return fail(NTG_ERR_INVALID_ARGUMENT, "null matrix pointer in item %lld", (long long)i);
+
+    const size_t a_bytes = (size_t)(m * k * es), b_bytes = (size_t)(k * n * es), c_bytes = (size_t)(m * n * es);
+    // every distinct input matrix gets one slot in a single device arena
+    std::map<const void*, size_t> slotA, slotB;
+    size_t off = 0;
+    for (int64_t i = 0; i < batches; ++i)
+        if (slotA.emplace(A[i], off).second) off += align_up(a_bytes, 256);
+    for (int64_t i = 0; i < batches; ++i)
+        if (slotB.emplace(B[i], off).second) off += align_up(b_bytes, 256);
+    const size_t c_off = off;
+    off += align_up(c_bytes, 256) * (size_t)batches;
+    const size_t tab_off = off;
+    off += 3 * sizeof(void*) * (size_t)batches;
+
+    DeviceMem mem;
+    HIP_TRY(mem.alloc(off));
+    for (auto& kv : slotA) HIP_TRY(hipMemcpy(mem.at(kv.second), kv.first, a_bytes, hipMemcpyHostToDevice));
+    for (auto& kv : slotB) HIP_TRY(hipMemcpy(mem.at(kv.second), kv.first, b_bytes, hipMemcpyHostToDevice));
+    std::vector<void*> tab(3 * (size_t)batches);
+    for (int64_t i = 0; i < batches; ++i) {
+        for (int64_t j = 0; j < i; ++j)
+            if (C[j] == C[i]) return fail(NTG_ERR_INVALID_ARGUMENT, "output pointers of items %lld and %lld alias", (long long)j, (long long)i);
+        char* dc = mem.at(c_off + (size_t)i * align_up(c_bytes, 256));
+        HIP_TRY(hipMemcpy(dc, C[i], c_bytes, hipMemcpyHostToDevice));   // accumulate contract: C is an input too
+        tab[(size_t)i] = mem.at(slotA[A[i]]);
+        tab[(size_t)(batches + i)] = mem.at(slotB[B[i]]);
+        tab[(size_t)(2 * batches + i)] = dc;
+    }
+    HIP_TRY(hipMemcpy(mem.at(tab_off), tab.data(), tab.size() * sizeof(void*), hipMemcpyHostToDevice));
+
+    ntg_gemm_desc d;
+    std::memset(&d, 0, sizeof d);
+    d.dtype = dtype; d.transpose_a = transpose_a; d.transpose_b = transpose_b; d.c_mode = NTG_C_ACCUMULATE;
+    d.m = m; d.k = k; d.n = n; d.batches = batches;
+    void** dtab = reinterpret_cast<void**>(mem.at(tab_off));
+    if (batches == 1) {
+        rc = ntg_gemm_dev(&d, tab[0], tab[1], tab[2], nullptr);
+    } else {
+        rc = ntg_gemm_ptrs_dev(&d, dtab, dtab + batches, dtab + 2 * batches, nullptr);
+    }
+    if (rc) return rc;
+    HIP_TRY(hipStreamSynchronize(nullptr));
+    for (int64_t i = 0; i < batches; ++i)
+        HIP_TRY(hipMemcpy(C[i], tab[(size_t)(2 * batches + i)], c_bytes, hipMemcpyDeviceToHost));
+    return NTG_OK;
+}
+
+int ntg_linear(int dtype, const void* X, const void* W, const void* bias, void* Y,
+               int64_t m, int64_t k, int64_t n, int transpose_x, int transpose_w,
+               int64_t bias_rows, int64_t bias_cols) {
+    const int64_t es = ntg::elem_size(dtype);
+    if (es == 0) return fail(NTG_ERR_UNSUPPORTED_DTYPE, "dtype %d is not supported by the gfx950 matmult backend", dtype);
+    int rc = check_sizes(m, k, n, 1);
+    if (rc) return rc;
+    if ((bias_rows != 1 && bias_rows != m) || (bias_cols != 1 && bias_cols != n))
+        return fail(NTG_ERR_INVALID_ARGUMENT, "bias shape [%lld, %lld] does not broadcast to [%lld, %lld]",
+                    (long long)bias_rows, (long long)bias_cols, (long long)m, (long long)n);
+    if (m == 0 || n == 0) return NTG_OK;
+    if (!X || !W || !bias || !Y) return fail(NTG_ERR_INVALID_ARGUMENT, "null pointer");
+    const size_t x_bytes = (size_t)(m * k * es), w_bytes = (size_t)(k * n * es), y_bytes = (size_t)(m * n * es);
+    const size_t bias_bytes = (size_t)(bias_rows * bias_cols * es);
+    DeviceMem mem;
+    const size_t ox = 0, ow = align_up(x_bytes, 256), ob = ow + align_up(w_bytes, 256), oy = ob + align_up(bias_bytes, 256);
+    HIP_TRY(mem.alloc(oy + y_bytes));
+    if (x_bytes) HIP_TRY(hipMemcpy(mem.at(ox), X, x_bytes, hipMemcpyHostToDevice));
+    if (w_bytes) HIP_TRY(hipMemcpy(mem.at(ow), W, w_bytes, hipMemcpyHostToDevice));
+    HIP_TRY(hipMemcpy(mem.at(ob), bias, bias_bytes, hipMemcpyHostToDevice));
+    ntg_gemm_desc d;
+    std::memset(&d, 0, sizeof d);
+    d.dtype = dtype; d.transpose_a = transpose_x; d.transpose_b = transpose_w; d.c_mode = NTG_C_BIAS;
+    d.m = m; d.k = k; d.n = n; d.batches = 1;
+    d.bias = mem.at(ob);
+    d.bias_row_stride = (bias_rows == 1) ? 0 : bias_cols;
+    d.bias_col_stride = (bias_cols == 1) ? 0 : 1;
+    rc = ntg_gemm_dev(&d, mem.at(ox), mem.at(ow), mem.at(oy), nullptr);
+    if (rc) return rc;
+    HIP_TRY(hipStreamSynchronize(nullptr));
+    HIP_TRY(hipMemcpy(Y, mem.at(oy), y_bytes, hipMemcpyDeviceToHost));
+    return NTG_OK;
+}
+
+static int unfold_out(int64_t height, int64_t width, int64_t k_r, int64_t k_c, int64_t s_r, int64_t s_c,
+                      int64_t p_r, int64_t p_c, int64_t d_r, int64_t d_c, int64_t& Ho, int64_t& Wo) {
+    if (k_r < 1 || k_c < 1 || s_r < 1 || s_c < 1 || d_r < 1 || d_c < 1 || p_r < 0 || p_c < 0)
+        return fail(NTG_ERR_INVALID_ARGUMENT, "kernel/stride/dilation must be >= 1 and padding >= 0");
+    Ho = (height + 2 * p_r - d_r * (k_r - 1) - 1) / s_r + 1;
+    Wo = (width + 2 * p_c - d_c * (k_c - 1) - 1) / s_c + 1;
+    if (height + 2 * p_r - d_r * (k_r - 1) - 1 < 0 || width + 2 * p_c - d_c * (k_c - 1) - 1 < 0 || Ho <= 0 || Wo <= 0)
+        return fail(NTG_ERR_INVALID_ARGUMENT, "the array of sliding blocks would be empty (Ho=%lld, Wo=%lld)", (long long)Ho, (long long)Wo);
+    return NTG_OK;
+}
+
+int ntg_unfold2d_dev(int dtype, const void* image, void* col,
+                     int64_t batch, int64_t channels, int64_t height, int64_t width,
+                     int64_t k_r, int64_t k_c, int64_t s_r, int64_t s_c,
+                     int64_t p_r, int64_t p_c, int64_t d_r, int64_t d_c, void* stream) {
+    const int64_t es = ntg::elem_size(dtype);
+    if (es == 0) return fail(NTG_ERR_UNSUPPORTED_DTYPE, "dtype %d is not supported", dtype);
+    if (batch < 0 || channels < 0 || height < 0 || width < 0) return fail(NTG_ERR_INVALID_ARGUMENT, "negative size");
+    int64_t Ho, Wo;
+    int rc = unfold_out(height, width, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c, Ho, Wo);
+    if (rc) return rc;
+    if (batch == 0 || channels == 0) return NTG_OK;
+    if (!image || !col) return fail(NTG_ERR_INVALID_ARGUMENT, "null pointer");
+    hipError_t e = ntg::launch_unfold2d(es, image, col, batch, channels, height, width, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c,
+                                        static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return hip_fail(e, "unfold2d launch");
+    return NTG_OK;
+}
+
+int ntg_unfold2d(int dtype, const void* image, void* col,
+                 int64_t batch, int64_t channels, int64_t height, int64_t width,
+                 int64_t k_r, int64_t k_c, int64_t s_r, int64_t s_c,
+                 int64_t p_r, int64_t p_c, int64_t d_r, int64_t d_c) {
+    const int64_t es = ntg::elem_size(dtype);
+    if (es == 0) return fail(NTG_ERR_UNSUPPORTED_DTYPE, "dtype %d is not supported", dtype);
+    int64_t Ho, Wo;
+    int rc = unfold_out(height, width, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c, Ho, Wo);
+    if (rc) return rc;
+    if (batch <= 0 || channels <= 0) return batch < 0 || channels < 0 ? fail(NTG_ERR_INVALID_ARGUMENT, "negative size") : NTG_OK;
+    if (!image || !col) return fail(NTG_ERR_INVALID_ARGUMENT, "null pointer");
+    const size_t im_bytes = (size_t)(batch * channels * height * width * es);
+    const size_t col_bytes = (size_t)(batch * channels * k_r * k_c * Ho * Wo * es);
+    DeviceMem mem;
+    const size_t oc = align_up(im_bytes, 256);
+    HIP_TRY(mem.alloc(oc + col_bytes));
+    HIP_TRY(hipMemcpy(mem.at(0), image, im_bytes, hipMemcpyHostToDevice));
+    rc = ntg_unfold2d_dev(dtype, mem.at(0), mem.at(oc), batch, channels, height, width, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c, nullptr);
+    if (rc) return rc;
+    HIP_TRY(hipStreamSynchronize(nullptr));
+    HIP_TRY(hipMemcpy(col, mem.at(oc), col_bytes, hipMemcpyDeviceToHost));
+    return NTG_OK;
+}
+
+int64_t ntg_conv2d_workspace_bytes(int dtype, int64_t batch, int64_t channels, int64_t height, int64_t width,
+                                   int64_t k_r, int64_t k_c, int64_t s_r, int64_t s_c,
+                                   int64_t p_r, int64_t p_c, int64_t d_r, int64_t d_c) {
+    const int64_t es = ntg::elem_size(dtype);
+    int64_t Ho, Wo;
+    if (es == 0 || unfold_out(height, width, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c, Ho, Wo)) return -1;
+    return batch * channels * k_r * k_c * Ho * Wo * es;
+}
+
+int ntg_conv2d_dev(int dtype, const void* image, const void* kernel, void* out,
+                   void* workspace, int64_t workspace_bytes,
+                   int64_t batch, int64_t channels, int64_t height, int64_t width,
+                   int64_t out_channels, int64_t k_r, int64_t k_c,
+                   int64_t s_r, int64_t s_c, int64_t p_r, int64_t p_c, int64_t d_r, int64_t d_c,
+                   int64_t groups, void* stream) {
+    const int64_t es = ntg::elem_size(dtype);
+    if (es == 0) return fail(NTG_ERR_UNSUPPORTED_DTYPE, "dtype %d is not supported", dtype);
+    if (batch < 0 || channels < 0 || out_channels < 0 || height < 0 || width < 0) return fail(NTG_ERR_INVALID_ARGUMENT, "negative size");
+    if (groups < 1) return fail(NTG_ERR_INVALID_ARGUMENT, "groups must be >= 1");
+    // conv.cpp:97-98
+    if (channels % groups != 0) return fail(NTG_ERR_INVALID_ARGUMENT, "image channels (%lld) not divisible by groups (%lld)", (long long)channels, (long long)groups);
+    if (out_channels % groups != 0) return fail(NTG_ERR_INVALID_ARGUMENT, "out channels (%lld) not divisible by groups (%lld)", (long long)out_channels, (long long)groups);
+    int64_t Ho, Wo;
+    int rc = unfold_out(height, width, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c, Ho, Wo);
+    if (rc) return rc;
+    if (batch == 0 || out_channels == 0) return NTG_OK;
+    if (!image || !kernel || !out) return fail(NTG_ERR_INVALID_ARGUMENT, "null pointer");
+    const int64_t need = batch * channels * k_r * k_c * Ho * Wo * es;
+    if (need > 0 && (!workspace || workspace_bytes < need))
+        return fail(NTG_ERR_INVALID_ARGUMENT, "workspace of %lld bytes needed, %lld given", (long long)need, (long long)workspace_bytes);
+    rc = ntg_unfold2d_dev(dtype, image, workspace, batch, channels, height, width, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c, stream);
+    if (rc) return rc;
+    // Per image b and group g:  out_b[g*og:(g+1)*og, L] = W_g[og, add] . col_b[g*add:(g+1)*add, L].
+    // The reference forms (col_b^T . W_g^T) and swaps rows/columns afterwards (conv.cpp:94);
+    // each output element is the same ascending-k sum of the same products.
+    const int64_t L = Ho * Wo, ckk = channels * k_r * k_c;
+    const int64_t add = (channels / groups) * k_r * k_c, og = out_channels / groups;
+    for (int64_t g = 0; g < groups; ++g) {
+        ntg_gemm_desc d;
+        std::memset(&d, 0, sizeof d);
+        d.dtype = dtype; d.c_mode = NTG_C_OVERWRITE;
+        d.m = og; d.k = add; d.n = L;
+        d.lda = add; d.ldb = L; d.ldc = L;
+        d.batches = batch;
+        d.stride_a = 0; d.stride_b = ckk * L; d.stride_c = out_channels * L;
+        rc = ntg_gemm_dev(&d, static_cast<const char*>(kernel) + g * og * add * es,
+                          static_cast<const char*>(workspace) + g * add * L * es,
+                          static_cast<char*>(out) + g * og * L * es, stream);
+        if (rc) return rc;
+    }
+    return NTG_OK;
+}
+
+int ntg_conv2d(int dtype, const void* image, const void* kernel, void* out,
+               int64_t batch, int64_t channels, int64_t height, int64_t width,
+               int64_t out_channels, int64_t k_r, int64_t k_c,
+               int64_t s_r, int64_t s_c, int64_t p_r, int64_t p_c, int64_t d_r, int64_t d_c,
+               int64_t groups) {
+    const int64_t es = ntg::elem_size(dtype);
+    if (es == 0) return fail(NTG_ERR_UNSUPPORTED_DTYPE, "dtype %d is not supported", dtype);
+    if (batch < 0 || channels < 0 || out_channels < 0 || height < 0 || width < 0) return fail(NTG_ERR_INVALID_ARGUMENT, "negative size");
+    if (groups < 1 || channels % groups != 0 || out_channels % groups != 0)
+        return fail(NTG_ERR_INVALID_ARGUMENT, "channels (%lld) and out channels (%lld) must be divisible by groups (%lld)",
+                    (long long)channels, (long long)out_channels, (long long)groups);
+    int64_t Ho, Wo;
+    int rc = unfold_out(height, width, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c, Ho, Wo);
+    if (rc) return rc;
+    if (batch == 0 || out_channels == 0) return NTG_OK;
+    if (!image || !kernel || !out) return fail(NTG_ERR_INVALID_ARGUMENT, "null pointer");
+    const size_t im_bytes = (size_t)(batch * channels * height * width * es);
+    const size_t k_bytes = (size_t)(out_channels * (channels / groups) * k_r * k_c * es);
+    const size_t o_bytes = (size_t)(batch * out_channels * Ho * Wo * es);
+    const int64_t ws = ntg_conv2d_workspace_bytes(dtype, batch, channels, height, width, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c);
+    DeviceMem mem;
+    const size_t ok_ = align_up(im_bytes, 256), oo = ok_ + align_up(k_bytes, 256), ow = oo + align_up(o_bytes, 256);
+    HIP_TRY(mem.alloc(ow + (size_t)ws));
+    if (im_bytes) HIP_TRY(hipMemcpy(mem.at(0), image, im_bytes, hipMemcpyHostToDevice));
+    if (k_bytes) HIP_TRY(hipMemcpy(mem.at(ok_), kernel, k_bytes, hipMemcpyHostToDevice));
+    rc = ntg_conv2d_dev(dtype, mem.at(0), mem.at(ok_), mem.at(oo), mem.at(ow), ws, batch, channels, height, width,
+                        out_channels, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c, groups, nullptr);
+    if (rc) return rc;
+    HIP_TRY(hipStreamSynchronize(nullptr));
+    HIP_TRY(hipMemcpy(out, mem.at(oo), o_bytes, hipMemcpyDeviceToHost));
+    return NTG_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,64 @@
+// im2col on the GPU: col[b, c*kh*kw + i*kw + j, h*Wo + w] = im[b, c, h*s_r - p_r + i*d_r, w*s_c - p_c + j*d_c]
+// (zero where the tap falls in the padding).  Same layout as the reference's im2col_cpu
+// (nt/functional/cpu/unfold2d.cpp:12-112) behind functional::unfold2d(..., transpose_out=true)
+// (nt/functional/tensor_files/colim_transform.cpp:565-588).  Pure data movement, HBM bound:
+// one lane per output element, the fast index runs along Wo so stores are coalesced and,
+// for stride 1, so are the loads.
+#include "ntg_common.h"
+
+namespace ntg {
+
+struct UnfoldParams {
+    int64_t batch, channels, height, width;
+    int64_t k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c;
+    int64_t Ho, Wo, ccol, total;
+};
+
+template <class T>
+__global__ void __launch_bounds__(256) unfold2d_kernel(const T* __restrict__ im, T* __restrict__ col, const UnfoldParams u) {
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < u.total; idx += stride) {
+        const int64_t w = idx % u.Wo;
+        int64_t t = idx / u.Wo;
+        const int64_t h = t % u.Ho;
+        t /= u.Ho;
+        const int64_t c = t % u.ccol;
+        const int64_t b = t / u.ccol;
+        const int64_t j = c % u.k_c;
+        const int64_t i = (c / u.k_c) % u.k_r;
+        const int64_t c_im = c / (u.k_r * u.k_c);
+        const int64_t hp = h * u.s_r - u.p_r + i * u.d_r;
+        const int64_t wp = w * u.s_c - u.p_c + j * u.d_c;
+        T v = 0;
+        if (hp >= 0 && hp < u.height && wp >= 0 && wp < u.width)
+            v = im[((b * u.channels + c_im) * u.height + hp) * u.width + wp];
+        col[idx] = v;
+    }
+}
+
+hipError_t launch_unfold2d(int64_t es, const void* im, void* col,
+                           int64_t batch, int64_t channels, int64_t height, int64_t width,
+                           int64_t k_r, int64_t k_c, int64_t s_r, int64_t s_c,
+                           int64_t p_r, int64_t p_c, int64_t d_r, int64_t d_c, hipStream_t s) {
+    UnfoldParams u;
+    u.batch = batch; u.channels = channels; u.height = height; u.width = width;
+    u.k_r = k_r; u.k_c = k_c; u.s_r = s_r; u.s_c = s_c; u.p_r = p_r; u.p_c = p_c; u.d_r = d_r; u.d_c = d_c;
+    u.Ho = (height + 2 * p_r - d_r * (k_r - 1) - 1) / s_r + 1;
+    u.Wo = (width + 2 * p_c - d_c * (k_c - 1) - 1) / s_c + 1;
+    if (u.Ho <= 0 || u.Wo <= 0) return hipErrorInvalidValue;
+    u.ccol = channels * k_r * k_c;
+    u.total = batch * u.ccol * u.Ho * u.Wo;
+    if (u.total == 0) return hipSuccess;
+    int64_t blocks = (u.total + 255) / 256;
+    if (blocks > 256 * 64) blocks = 256 * 64;   // grid-stride beyond 64 workgroups per CU
+    switch (es) {
+    case 1: hipLaunchKernelGGL(unfold2d_kernel<uint8_t>, dim3((unsigned)blocks), dim3(256), 0, s, (const uint8_t*)im, (uint8_t*)col, u); break;
+    case 2: hipLaunchKernelGGL(unfold2d_kernel<uint16_t>, dim3((unsigned)blocks), dim3(256), 0, s, (const uint16_t*)im, (uint16_t*)col, u); break;
+    case 4: hipLaunchKernelGGL(unfold2d_kernel<uint32_t>, dim3((unsigned)blocks), dim3(256), 0, s, (const uint32_t*)im, (uint32_t*)col, u); break;
+    case 8: hipLaunchKernelGGL(unfold2d_kernel<uint64_t>, dim3((unsigned)blocks), dim3(256), 0, s, (const uint64_t*)im, (uint64_t*)col, u); break;
+    default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+
+}  // namespace ntg

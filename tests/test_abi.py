@@ -1,0 +1,78 @@
+"""CPU-side checks of the drop-in boundary: libntgemm.so loads, exports every symbol
+include/ntgemm.h declares, and rejects bad arguments before touching a device."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+from neurotensor_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "ntgemm.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(ntg_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_symbols_all_exported_and_bound():
+    lib = _lib.load()
+    names = declared_symbols()
+    assert len(names) >= 14
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in ntgemm.h but not exported"
+        assert n in _lib.SIGNATURES, f"{n} has no ctypes signature"
+    assert set(_lib.SIGNATURES) == set(names)
+
+
+def test_dtype_sizes_follow_nt_dtype_values():
+    lib = _lib.load()
+    sizes = {_lib.FLOAT16: 2, _lib.FLOAT32: 4, _lib.FLOAT64: 8, _lib.INT8: 1, _lib.INT16: 2, _lib.INT32: 4,
+             _lib.INT64: 8, _lib.UINT8: 1, _lib.UINT16: 2, _lib.UINT32: 4, _lib.BFLOAT16: 2, _lib.UINT64: 8}
+    for dt, sz in sizes.items():
+        assert lib.ntg_dtype_size(dt) == sz
+    # Float128=3, complex 4..6, int128=11, uint128=15, Bool=16, TensorObj=17 are not served
+    for dt in (3, 4, 5, 6, 11, 15, 16, 17, 55):
+        assert lib.ntg_dtype_size(dt) == 0
+    assert lib.ntg_version() >= 100
+
+
+def test_desc_struct_layout():
+    assert ctypes.sizeof(_lib.GemmDesc) == 16 + 8 * 3 + 8 * 3 + 8 + 8 * 3 + 8 + 8 * 3
+
+
+def test_argument_errors_do_not_need_a_device():
+    lib = _lib.load()
+    a = np.zeros((4, 4), np.float32)
+    p = a.ctypes.data_as(ctypes.c_void_p)
+    # inner sizes differ
+    rc = lib.ntg_matmult(_lib.FLOAT32, p, p, p, 4, 4, 3, 4, 0, 0)
+    assert rc == 1 and b"inner sizes" in lib.ntg_last_error()
+    # unsupported dtype (Complex64 = 5)
+    rc = lib.ntg_matmult(5, p, p, p, 4, 4, 4, 4, 0, 0)
+    assert rc == 2
+    # negative size
+    rc = lib.ntg_matmult(_lib.FLOAT32, p, p, p, -1, 4, 4, 4, 0, 0)
+    assert rc == 1
+    # empty product is a no-op
+    assert lib.ntg_matmult(_lib.FLOAT32, p, p, p, 0, 4, 4, 4, 0, 0) == 0
+    # bias that does not broadcast
+    rc = lib.ntg_linear(_lib.FLOAT32, p, p, p, p, 4, 4, 4, 0, 0, 2, 4)
+    assert rc == 1 and b"bias" in lib.ntg_last_error()
+    # empty sliding-block array
+    rc = lib.ntg_unfold2d(_lib.FLOAT32, p, p, 1, 1, 2, 2, 5, 5, 1, 1, 0, 0, 1, 1)
+    assert rc == 1
+    assert lib.ntg_conv2d_workspace_bytes(_lib.FLOAT32, 1, 3, 8, 8, 3, 3, 1, 1, 1, 1, 1, 1) == 27 * 64 * 4
+    d = _lib.GemmDesc()
+    d.dtype, d.m, d.k, d.n, d.batches, d.c_mode = _lib.FLOAT32, 4, 4, 4, 1, 7
+    assert lib.ntg_gemm_dev(ctypes.byref(d), p, p, p, None) == 1
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "libntgemm.so"))
+    with pytest.raises(RuntimeError, match="not built"):
+        _lib.load()

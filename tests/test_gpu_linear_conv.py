@@ -1,0 +1,196 @@
+"""GPU parity of the layers above the GEMM: linear (bias-initialised GEMM + gradient GEMMs),
+unfold2d and conv2d, against the reference's golden vectors and the CPU oracle."""
+import ctypes
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from neurotensor_amd import _lib
+from neurotensor_amd import functional as F
+from util import HALF_REL, float_tol, from_torch, randn, to_f64, to_torch
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def setup_module(module):
+    assert torch.cuda.is_available(), "GPU tests need a visible MI355X"
+    _lib.load()
+
+
+def load(golden_dir, name):
+    return np.load(os.path.join(golden_dir, name + ".npy"), allow_pickle=False)
+
+
+def nt_allclose(a, b, rtol=1e-5, atol=1e-6):
+    return bool(np.all(np.abs(a - b) <= atol + rtol * np.abs(b)))
+
+
+def dev(x):
+    return torch.from_numpy(np.ascontiguousarray(x)).to(DEV)
+
+
+def linear_backward_gpu(x, w, grad, ta, tb):
+    """The gradient GEMMs of TensorGrad linear (nn/functional/matmult.cpp:253-275), flags only."""
+    dx = F.matmult(w, grad, None, tb, True) if ta else F.matmult(grad, w, None, False, not tb)
+    dw = F.matmult(grad, x, None, True, ta) if tb else F.matmult(x, grad, None, not ta, False)
+    return dx, dw
+
+
+def test_linear_golden_grads(golden_dir):
+    """tests/src/linear_autograd_test.cpp:126-148 replayed on the GPU path."""
+    x, w, b, g = (load(golden_dir, "linear_" + n) for n in ("input", "weight", "bias", "grad"))
+    out = F.linear(dev(x), dev(w), dev(b), False, True)
+    assert tuple(out.shape) == (3, 4, 3)
+    assert np.allclose(out.cpu().numpy(), oracle.linear(x, w, b, False, True), rtol=1e-5, atol=1e-6)
+    dx, dw = linear_backward_gpu(dev(x), dev(w), dev(g), False, True)
+    dw = dw.sum(0)                                   # accumulate_gradient's broadcast reduction
+    db = dev(g).reshape(-1, 3).sum(0)
+    assert nt_allclose(dx.cpu().numpy(), load(golden_dir, "linear_xgrad"))
+    assert nt_allclose(dw.cpu().numpy(), load(golden_dir, "linear_wgrad"))
+    assert nt_allclose(db.cpu().numpy(), load(golden_dir, "linear_bgrad"))
+
+
+def test_linear_host_entry_and_bias_shapes():
+    rng = np.random.default_rng(700)
+    m, k, n = 45, 70, 33
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    w = rng.standard_normal((n, k)).astype(np.float32)       # transpose_w
+    lib = _lib.load()
+    p = lambda a: a.ctypes.data_as(ctypes.c_void_p)
+    for br, bc in [(1, n), (m, 1), (m, n), (1, 1)]:
+        bias = rng.standard_normal((br, bc)).astype(np.float32)
+        y = np.full((m, n), np.nan, np.float32)
+        _lib.check(lib.ntg_linear(_lib.FLOAT32, p(x), p(w), p(bias), p(y), m, k, n, 0, 1, br, bc))
+        ref = oracle.linear(x, w, bias, False, True)
+        assert np.abs(y - ref).max() <= float_tol(k, x, w) + 1e-6
+        yd = F.linear(dev(x), dev(w), dev(bias), False, True)
+        assert np.array_equal(yd.cpu().numpy(), y)
+    with pytest.raises(ValueError):
+        F.linear(dev(x), dev(w), dev(np.zeros((2, n), np.float32)), False, True)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, "bf16"], ids=["fp32", "bf16"])
+def test_config4_linear_training_step(dtype):
+    """X[8192,4096], W[11008,4096] (transpose_b), b zeros; Y = X.W^T + b, dX = dY.W, dW = dY^T.X."""
+    M, K, N = 8192, 4096, 11008
+    bf = dtype == "bf16"
+    rng = np.random.default_rng(1006)
+    x = randn(rng, (M, K), dtype)
+    w = randn(rng, (N, K), dtype, 0.02)
+    gy = randn(rng, (M, N), dtype)
+    bias = np.zeros((N,), np.uint16 if bf else np.float32)
+    tx, tw, tg, tb_ = (to_torch(v, DEV, bf) for v in (x, w, gy, bias))
+    y = F.linear(tx, tw, tb_, False, True)
+    dx, dw = linear_backward_gpu(tx, tw, tg, False, True)
+    torch.cuda.synchronize()
+    assert tuple(y.shape) == (M, N) and tuple(dx.shape) == (M, K) and tuple(dw.shape) == (N, K)
+    code = oracle.BF16 if bf else oracle.F32
+    rows = np.r_[0:24, 5000:5024]
+    cols = np.r_[0:24, 11000:11008]
+
+    def check(got_t, A, B, ta, tb, r, c, kk):
+        Al = A.T if ta else A
+        Bl = B.T if tb else B
+        sa, sb = np.ascontiguousarray(Al[r, :]), np.ascontiguousarray(Bl[:, c])
+        ref = oracle.matmult2d(sa, sb, dt=code)
+        got = from_torch(got_t[r][:, c].contiguous())
+        if bf:
+            rr, gg = to_f64(ref, True), to_f64(got, True)
+            assert np.abs(rr - gg).max() / np.abs(rr).max() <= HALF_REL
+        else:
+            assert np.abs(ref - got).max() <= float_tol(kk, sa, sb)
+
+    check(y, x, w, False, True, rows, cols, K)                    # Y  = X . W^T
+    check(dx, gy, w, False, False, rows, np.r_[0:24, 4072:4096], N)   # dX = dY . W
+    check(dw, gy, x, True, False, np.r_[0:24, 10984:11008], np.r_[0:24, 4072:4096], M)   # dW = dY^T . X
+    # whole-matrix cross-check with an independent GEMM
+    if not bf:
+        ref = torch.matmul(tx.double(), tw.double().t())
+        assert (y.double() - ref).abs().max().item() <= 1e-5 * K * tx.abs().max().item() * tw.abs().max().item()
+    else:
+        ref = torch.matmul(tx.float(), tw.float().t())
+        assert ((y.float() - ref).abs().max() / ref.abs().max()).item() <= HALF_REL
+
+
+def test_unfold_golden_and_random(golden_dir):
+    x = load(golden_dir, "unfold_input")
+    exp = load(golden_dir, "unfold_output")
+    col = F.unfold2d(dev(x), (3, 2), dilation=(1, 2), padding=1, stride=(2, 2))
+    assert np.array_equal(col.cpu().numpy(), exp)
+    rng = np.random.default_rng(800)
+    for dtype in (np.float32, np.float64, np.float16, np.int32):
+        xi = (rng.standard_normal((3, 5, 13, 17)) * 10).astype(dtype)
+        for k, d, p, s in [((3, 3), 1, 1, 1), ((2, 4), (2, 1), (0, 3), (1, 2)), ((1, 1), 1, 0, 3), ((5, 5), 1, 2, 2)]:
+            got = F.unfold2d(dev(xi), k, dilation=d, padding=p, stride=s).cpu().numpy()
+            assert np.array_equal(got, oracle.unfold2d(xi, k, dilation=d, padding=p, stride=s))
+    # host entry point
+    lib = _lib.load()
+    xi = rng.standard_normal((2, 3, 9, 8)).astype(np.float32)
+    col = np.full((2, 27, 72), np.nan, np.float32)
+    _lib.check(lib.ntg_unfold2d(_lib.FLOAT32, xi.ctypes.data_as(ctypes.c_void_p), col.ctypes.data_as(ctypes.c_void_p),
+                                2, 3, 9, 8, 3, 3, 1, 1, 1, 1, 1, 1))
+    assert np.array_equal(col, oracle.unfold2d(xi, 3, padding=1))
+    with pytest.raises(ValueError):
+        F.unfold2d(dev(xi), 20)
+
+
+CONV_CASES = [("", 1, 1), ("_batched", 1, 1), ("_grouped", 0, 2), ("_grouped_batched", 0, 2)]
+
+
+@pytest.mark.parametrize("sfx,pad,groups", CONV_CASES)
+def test_conv2d_golden(golden_dir, sfx, pad, groups):
+    """tests/src/conv_autograd_test.cpp:250-371 forward outputs on the GPU path."""
+    x = load(golden_dir, "conv2d_input" + sfx)
+    w = load(golden_dir, "conv2d_weight" + sfx)
+    exp = load(golden_dir, "conv2d_output" + sfx)
+    out = F.conv2d(dev(x), dev(w), stride=1, padding=pad, dilation=1, groups=groups).cpu().numpy()
+    assert out.shape == exp.shape
+    assert np.abs(out - exp).max() <= 1e-4
+    assert np.abs(out - oracle.conv2d(x, w, 1, pad, 1, groups)).max() <= 1e-5
+    # host entry point
+    lib = _lib.load()
+    B, C, H, W = x.shape
+    O, _, kh, kw = w.shape
+    y = np.full(exp.shape, np.nan, np.float32)
+    p = lambda a: np.ascontiguousarray(a).ctypes.data_as(ctypes.c_void_p)
+    _lib.check(lib.ntg_conv2d(_lib.FLOAT32, p(x), p(w), y.ctypes.data_as(ctypes.c_void_p), B, C, H, W, O, kh, kw,
+                              1, 1, pad, pad, 1, 1, groups))
+    assert np.array_equal(y, out)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64, np.float16, np.int32])
+def test_conv2d_random_vs_oracle(dtype):
+    rng = np.random.default_rng(900)
+    x = (rng.standard_normal((3, 6, 14, 11)) * (4 if dtype == np.int32 else 1)).astype(dtype)
+    w = (rng.standard_normal((8, 3, 3, 2)) * (4 if dtype == np.int32 else 1)).astype(dtype)
+    out = F.conv2d(dev(x), dev(w), stride=(2, 1), padding=(1, 2), dilation=(1, 2), groups=2).cpu().numpy()
+    ref = oracle.conv2d(x, w, (2, 1), (1, 2), (1, 2), 2)
+    if dtype == np.int32:
+        assert np.array_equal(out, ref)
+    elif dtype == np.float16:
+        assert np.abs(out.astype(np.float64) - ref.astype(np.float64)).max() <= HALF_REL * np.abs(ref.astype(np.float64)).max()
+    else:
+        assert np.abs(out - ref).max() <= 1e-5 * 18 * np.abs(x).max() * np.abs(w).max()
+    with pytest.raises(ValueError):
+        F.conv2d(dev(x), dev(w), groups=4)
+
+
+def test_config5a_conv2d_resnet_block():
+    """image [64,256,56,56], weight [256,256,3,3], stride 1, pad 1 (GEMM M=200704, K=2304, N=256)."""
+    rng = np.random.default_rng(1007)
+    x = rng.standard_normal((64, 256, 56, 56)).astype(np.float32)
+    w = (rng.standard_normal((256, 256, 3, 3)) / np.sqrt(2304.0)).astype(np.float32)
+    tx, tw = dev(x), dev(w)
+    out = F.conv2d(tx, tw, stride=1, padding=1)
+    torch.cuda.synchronize()
+    assert tuple(out.shape) == (64, 256, 56, 56)
+    tol = float_tol(2304, x, w)
+    for b in (0, 63):                                            # two whole images through the oracle
+        ref = oracle.conv2d(x[b:b + 1], w, 1, 1, 1, 1, kind="tiled")
+        assert np.abs(out[b:b + 1].cpu().numpy() - ref).max() <= tol
+    ref_all = torch.nn.functional.conv2d(tx.double(), tw.double(), padding=1)
+    assert (out.double() - ref_all).abs().max().item() <= tol

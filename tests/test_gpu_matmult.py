@@ -1,0 +1,327 @@
+"""GPU parity of the matmult path against the CPU oracle, through the C ABI.
+
+Integer dtypes must be bit-exact; fp32/fp64 within max|d| <= 1e-5*K*max|A|*max|B|;
+fp16/bf16 within 2e-2 of max|C_ref| (fp32 accumulate on the GPU; the fp16 oracle rounds
+to half every 16 k like the reference's AVX2 build, the bf16 oracle is this build's own
+definition -- "parity unpinned" by the reference, which has no BFloat16 DType).
+"""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from neurotensor_amd import _lib
+from neurotensor_amd import functional as F
+from util import HALF_REL, float_tol, from_torch, randn, to_f64, to_torch
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+TRANS = [(False, False), (False, True), (True, False), (True, True)]
+FLOATS = [np.float32, np.float64, np.float16, "bf16"]
+INTS = [np.int8, np.int16, np.int32, np.int64, np.uint8, np.uint16, np.uint32, np.uint64]
+
+
+def setup_module(module):
+    assert torch.cuda.is_available(), "GPU tests need a visible MI355X"
+    _lib.load()
+
+
+def code_of(dtype):
+    return oracle.BF16 if dtype == "bf16" else oracle._NP_TO_DT[np.dtype(dtype)]
+
+
+def make_inputs(rng, m, k, n, dtype, ta, tb, scale=1.0, int_range=None):
+    if dtype in FLOATS or dtype == "bf16":
+        a = randn(rng, (m, k), dtype, scale)
+        b = randn(rng, (k, n), dtype, scale)
+        c0 = randn(rng, (m, n), dtype, scale)
+    else:
+        info = np.iinfo(dtype)
+        lo, hi = int_range if int_range else (info.min, info.max)
+        a = rng.integers(lo, hi, (m, k), dtype=dtype, endpoint=True)
+        b = rng.integers(lo, hi, (k, n), dtype=dtype, endpoint=True)
+        c0 = rng.integers(lo, hi, (m, n), dtype=dtype, endpoint=True)
+    sa = np.ascontiguousarray(a.T) if ta else a
+    sb = np.ascontiguousarray(b.T) if tb else b
+    return a, b, sa, sb, c0
+
+
+def assert_close(got, ref, a, b, k, dtype, what=""):
+    bf = dtype == "bf16"
+    if dtype in (np.float32, np.float64):
+        tol = float_tol(k, a, b)
+        err = np.abs(got.astype(np.float64) - ref.astype(np.float64)).max(initial=0.0)
+        assert err <= tol, f"{what}: max|d|={err} > {tol}"
+    elif dtype in (np.float16, "bf16"):
+        g, r = to_f64(got, bf), to_f64(ref, bf)
+        scale = max(np.abs(r).max(initial=0.0), 1e-30)
+        err = np.abs(g - r).max(initial=0.0) / scale
+        assert err <= HALF_REL, f"{what}: rel err {err} > {HALF_REL}"
+    else:
+        assert got.tobytes() == ref.tobytes(), f"{what}: integer result not bit-exact"
+
+
+def host_matmult(sa, sb, c, m, k, n, ta, tb, dt):
+    lib = _lib.load()
+    p = lambda x: x.ctypes.data_as(ctypes.c_void_p)
+    _lib.check(lib.ntg_matmult(dt, p(sa), p(sb), p(c), m, k, k, n, int(ta), int(tb)))
+    return c
+
+
+def dev_matmult(sa, sb, c0, m, k, n, ta, tb, dtype, mode=_lib.C_ACCUMULATE):
+    bf = dtype == "bf16"
+    ta_, tb_ = to_torch(sa, DEV, bf), to_torch(sb, DEV, bf)
+    tc = to_torch(c0.copy(), DEV, bf)
+    lib = _lib.load()
+    d = _lib.GemmDesc()
+    d.dtype = code_of(dtype)
+    d.transpose_a, d.transpose_b, d.c_mode = int(ta), int(tb), mode
+    d.m, d.k, d.n, d.batches = m, k, n, 1
+    _lib.check(lib.ntg_gemm_dev(ctypes.byref(d), ta_.data_ptr(), tb_.data_ptr(), tc.data_ptr(),
+                                ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)))
+    torch.cuda.synchronize()
+    return from_torch(tc)
+
+
+@pytest.mark.parametrize("dtype", FLOATS + INTS, ids=lambda d: d if isinstance(d, str) else np.dtype(d).name)
+@pytest.mark.parametrize("ta,tb", TRANS)
+def test_host_entry_point_every_dtype(dtype, ta, tb):
+    """ntg_matmult == nt_matmult<T>: host pointers, C += op(A).op(B), ragged sizes."""
+    rng = np.random.default_rng(100)
+    m, k, n = 37, 53, 29
+    a, b, sa, sb, c0 = make_inputs(rng, m, k, n, dtype, ta, tb)
+    dt = code_of(dtype)
+    ref = oracle.matmult2d(sa, sb, c0.copy(), ta, tb, dt=dt)
+    got = host_matmult(sa, sb, c0.copy(), m, k, n, ta, tb, dt)
+    af = to_f64(a, dtype == "bf16") if dtype in FLOATS else a
+    bfm = to_f64(b, dtype == "bf16") if dtype in FLOATS else b
+    assert_close(got, ref, af, bfm, k, dtype, f"host {dtype} ta={ta} tb={tb}")
+
+
+SHAPES = [(1, 1, 1), (1, 64, 1), (5, 1, 7), (33, 70, 65), (64, 64, 64), (128, 128, 128), (129, 131, 127),
+          (256, 64, 256), (300, 200, 500), (17, 1000, 19), (512, 96, 384), (100, 333, 40)]
+
+
+@pytest.mark.parametrize("dtype", FLOATS, ids=lambda d: d if isinstance(d, str) else np.dtype(d).name)
+@pytest.mark.parametrize("shape", SHAPES, ids=lambda s: "x".join(map(str, s)))
+def test_device_entry_point_shapes(dtype, shape):
+    """Edge and ragged sizes on device buffers, all four flag pairs, accumulate into C0 != 0."""
+    m, k, n = shape
+    rng = np.random.default_rng(200 + m + k + n)
+    for ta, tb in TRANS:
+        a, b, sa, sb, c0 = make_inputs(rng, m, k, n, dtype, ta, tb)
+        ref = oracle.matmult2d(sa, sb, c0.copy(), ta, tb, dt=code_of(dtype))
+        got = dev_matmult(sa, sb, c0, m, k, n, ta, tb, dtype)
+        bf = dtype == "bf16"
+        assert_close(got, ref, to_f64(a, bf), to_f64(b, bf), k, dtype, f"dev {dtype} {shape} ta={ta} tb={tb}")
+
+
+@pytest.mark.parametrize("dtype", [np.int32, np.int64, np.int8, np.int16])
+@pytest.mark.parametrize("shape", [(1, 1, 1), (65, 130, 67), (128, 64, 128), (200, 17, 3)])
+def test_device_integers_bit_exact(dtype, shape):
+    m, k, n = shape
+    rng = np.random.default_rng(300 + m)
+    for ta, tb in TRANS:
+        a, b, sa, sb, c0 = make_inputs(rng, m, k, n, dtype, ta, tb)
+        ref = oracle.matmult2d(sa, sb, c0.copy(), ta, tb)
+        got = dev_matmult(sa, sb, c0, m, k, n, ta, tb, dtype)
+        assert got.tobytes() == ref.tobytes()
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16, "bf16", np.float64])
+def test_c_modes(dtype):
+    """overwrite ignores the incoming C (even NaN); accumulate adds to it."""
+    rng = np.random.default_rng(400)
+    m, k, n = 70, 90, 50
+    a, b, sa, sb, c0 = make_inputs(rng, m, k, n, dtype, False, False)
+    zeros = np.zeros_like(c0)
+    ref0 = oracle.matmult2d(sa, sb, zeros.copy(), dt=code_of(dtype))
+    junk = c0.copy()
+    if dtype == "bf16":
+        junk[:] = 0x7FC0
+    else:
+        junk[:] = np.nan
+    got = dev_matmult(sa, sb, junk, m, k, n, False, False, dtype, mode=_lib.C_OVERWRITE)
+    bf = dtype == "bf16"
+    assert_close(got, ref0, to_f64(a, bf), to_f64(b, bf), k, dtype, "overwrite")
+
+
+def test_host_batch_with_repeated_pointers():
+    """nt_matmult_batch: uniform shape, entries of A/B may repeat (broadcast by handle)."""
+    rng = np.random.default_rng(500)
+    m, k, n = 40, 33, 21
+    As = [rng.standard_normal((m, k)).astype(np.float32) for _ in range(3)]
+    Bsh = rng.standard_normal((n, k)).astype(np.float32)          # stored [n,k] -> transpose_b
+    Alist = [As[0], As[1], As[2], As[0], As[1]]
+    Blist = [Bsh] * 5
+    C0 = [rng.standard_normal((m, n)).astype(np.float32) for _ in range(5)]
+    ref = [c.copy() for c in C0]
+    oracle.matmult_batch_ptrs(Alist, Blist, ref, False, True)
+    got = [c.copy() for c in C0]
+    arr = ctypes.c_void_p * 5
+    lib = _lib.load()
+    _lib.check(lib.ntg_matmult_batch(_lib.FLOAT32, arr(*[x.ctypes.data for x in Alist]), arr(*[x.ctypes.data for x in Blist]),
+                                     arr(*[x.ctypes.data for x in got]), 5, m, k, k, n, 0, 1))
+    for g, r, a_ in zip(got, ref, Alist):
+        assert np.abs(g - r).max() <= float_tol(k, a_, Bsh)
+    # same pointers -> bit-identical results (the reference's batched == per-item invariant)
+    assert got[0].tobytes() != got[3].tobytes() or np.array_equal(C0[0], C0[3])
+    single = host_matmult(As[0], Bsh, C0[0].copy(), m, k, n, False, True, _lib.FLOAT32)
+    assert single.tobytes() == got[0].tobytes()
+
+
+def test_functional_batch_rules_and_views():
+    """N-D x K-D: trailing batch dims must match; lower-rank operand is reused; a transposed
+    view is consumed by flipping the flag (no copy); results equal the oracle's."""
+    rng = np.random.default_rng(600)
+    a = rng.standard_normal((2, 3, 10, 7)).astype(np.float32)
+    b = rng.standard_normal((3, 7, 6)).astype(np.float32)
+    ta_, tb_ = torch.from_numpy(a).to(DEV), torch.from_numpy(b).to(DEV)
+    out = F.matmult(ta_, tb_)
+    ref = oracle.matmult(a, b)
+    assert tuple(out.shape) == ref.shape
+    assert np.abs(out.cpu().numpy() - ref).max() <= float_tol(7, a, b)
+    # single-matrix B broadcasts with stride 0
+    b2 = rng.standard_normal((7, 5)).astype(np.float32)
+    out2 = F.matmult(ta_, torch.from_numpy(b2).to(DEV))
+    assert np.abs(out2.cpu().numpy() - oracle.matmult(a, b2)).max() <= float_tol(7, a, b2)
+    # lower-rank A with both flags
+    a3 = rng.standard_normal((7, 10)).astype(np.float32)
+    b3 = rng.standard_normal((4, 6, 7)).astype(np.float32)
+    out3 = F.matmult(torch.from_numpy(a3).to(DEV), torch.from_numpy(b3).to(DEV), None, True, True)
+    assert np.abs(out3.cpu().numpy() - oracle.matmult(a3, b3, None, True, True)).max() <= float_tol(7, a3, b3)
+    # transposed view == explicit flag
+    v = tb_.transpose(-1, -2)                       # shape (3, 6, 7), non-contiguous
+    out4 = F.matmult(ta_, v, None, False, True)
+    assert torch.equal(out4, out)
+    # out= accumulates
+    acc = out.clone()
+    F.matmult(ta_, tb_, acc)
+    assert torch.allclose(acc, 2 * out, rtol=1e-6, atol=1e-6)
+    with pytest.raises(ValueError):
+        F.matmult(ta_, torch.from_numpy(np.zeros((2, 7, 6), np.float32)).to(DEV))   # batch dims do not line up
+    with pytest.raises(ValueError):
+        F.matmult(ta_, tb_, None, True, False)                                       # inner sizes differ
+    with pytest.raises(ValueError):
+        F.matmult(ta_, tb_.double())                                                 # dtype mismatch
+
+
+# ---------------------------------------------------------------------------------------
+# BASELINE configurations
+# ---------------------------------------------------------------------------------------
+
+def test_config1_fp32_512_cube():
+    rng = np.random.default_rng(1001)
+    a = rng.standard_normal((512, 512)).astype(np.float32)
+    b = rng.standard_normal((512, 512)).astype(np.float32)
+    ref = oracle.matmult2d(a, b)
+    got = dev_matmult(a, b, np.zeros((512, 512), np.float32), 512, 512, 512, False, False, np.float32)
+    err = np.abs(got - ref).max()
+    assert err <= float_tol(512, a, b)
+    # far inside the stated bound in practice: a few ulps of sqrt(K)
+    assert err <= 1e-3
+    host = host_matmult(a, b, np.zeros((512, 512), np.float32), 512, 512, 512, False, False, _lib.FLOAT32)
+    assert host.tobytes() == got.tobytes()
+
+
+def test_config2_batched_fp32_and_transpose_b():
+    rng = np.random.default_rng(1002)
+    a = rng.standard_normal((32, 1024, 768)).astype(np.float32)
+    b = rng.standard_normal((32, 768, 1024)).astype(np.float32)
+    bt = np.ascontiguousarray(b.transpose(0, 2, 1))                 # stored [32,1024,768]
+    ta_, tb_, tbt = (torch.from_numpy(x).to(DEV) for x in (a, b, bt))
+    out_a = F.matmult(ta_, tb_)
+    out_b = F.matmult(ta_, tbt, None, False, True)
+    tol = float_tol(768, a, b)
+    assert (out_a - out_b).abs().max().item() <= tol
+    ref64 = torch.bmm(ta_.double(), tb_.double())
+    assert (out_a.double() - ref64).abs().max().item() <= tol
+    # oracle on a few whole items (the tiled restatement is bit-equal to the closed form)
+    got = out_a.cpu().numpy()
+    for i in (0, 13, 31):
+        ref = oracle.matmult2d(a[i], b[i], kind="tiled")
+        assert np.abs(got[i] - ref).max() <= tol
+        ref_t = oracle.matmult2d(a[i], bt[i], tb=True, kind="tiled")
+        assert ref_t.tobytes() == ref.tobytes()
+
+
+def test_config2_int32_bit_exact():
+    rng = np.random.default_rng(1003)
+    a = rng.integers(-8, 9, (8, 1024, 1024)).astype(np.int32)
+    b = rng.integers(-8, 9, (8, 1024, 1024)).astype(np.int32)
+    out = F.matmult(torch.from_numpy(a).to(DEV), torch.from_numpy(b).to(DEV)).cpu().numpy()
+    for i in range(8):
+        ref = oracle.matmult2d(a[i], b[i], kind="tiled")
+        assert out[i].tobytes() == ref.tobytes()
+
+
+def _sampled_oracle_check(a_np, b_np, got_t, ta, tb, dtype, rows, cols, k):
+    """Oracle parity on a sub-block of a large product: op(A)[rows,:] . op(B)[:,cols]."""
+    bf = dtype == "bf16"
+    A = a_np.T if ta else a_np
+    B = b_np.T if tb else b_np
+    sa = np.ascontiguousarray(A[rows, :])
+    sb = np.ascontiguousarray(B[:, cols])
+    ref = oracle.matmult2d(sa, sb, dt=code_of(dtype))
+    got = from_torch(got_t[rows][:, cols].contiguous())
+    assert_close(got, ref, to_f64(sa, bf), to_f64(sb, bf), k, dtype, "sampled block")
+
+
+@pytest.mark.parametrize("dtype,scale", [("bf16", 0.02), (np.float16, 0.02), (np.float32, 1.0), (np.float64, 1.0)],
+                         ids=["bf16", "fp16", "fp32", "fp64"])
+def test_config3_4096_cube(dtype, scale):
+    n = 4096
+    rng = np.random.default_rng(1004)
+    a = randn(rng, (n, n), dtype, scale)
+    b = randn(rng, (n, n), dtype, scale)
+    bf = dtype == "bf16"
+    ta_, tb_ = to_torch(a, DEV, bf), to_torch(b, DEV, bf)
+    out = F.matmult(ta_, tb_)
+    torch.cuda.synchronize()
+    rows = np.r_[0:32, 2040:2072, 4064:4096]
+    cols = np.r_[0:16, 1000:1016, 4080:4096]
+    _sampled_oracle_check(a, b, out, False, False, dtype, rows, cols, n)
+    # whole-matrix cross-check against an independent library GEMM in higher precision
+    if dtype in (np.float32, np.float64):
+        ref = torch.matmul(ta_.double(), tb_.double())
+        tol = 1e-5 * n * ta_.abs().max().item() * tb_.abs().max().item()
+        assert (out.double() - ref).abs().max().item() <= tol
+    else:
+        ref = torch.matmul(ta_.float(), tb_.float())
+        assert ((out.float() - ref).abs().max() / ref.abs().max()).item() <= HALF_REL
+    # linearity, a size-independent property: (2A).B == 2(A.B) exactly in binary floating point
+    out2 = F.matmult(ta_ * 2, tb_)
+    if dtype is np.float16:      # half subnormals (|c| < 6.1e-5) round on a fixed 2^-24 grid
+        assert (out2.float() - 2 * out.float()).abs().max().item() <= 2.0 ** -23
+    else:
+        assert torch.equal(out2, out * 2)
+    # accumulate contract at full size: C0 + A.B
+    acc = out.clone()
+    F.matmult(ta_, tb_, acc)
+    if dtype in (np.float32, np.float64):
+        assert torch.allclose(acc, 2 * out, rtol=1e-5, atol=1e-4)
+    else:
+        assert ((acc.float() - 2 * out.float()).abs().max() / out.float().abs().max()).item() <= HALF_REL
+
+
+def test_skinny_fp32_config5b():
+    rng = np.random.default_rng(1005)
+    a = rng.standard_normal((16, 8192)).astype(np.float32)
+    b = rng.standard_normal((8192, 8192)).astype(np.float32)
+    ta_, tb_ = torch.from_numpy(a).to(DEV), torch.from_numpy(b).to(DEV)
+    out = F.matmult(ta_, tb_)
+    ref = oracle.matmult2d(a, b, kind="tiled")
+    tol = float_tol(8192, a, b)
+    assert np.abs(out.cpu().numpy() - ref).max() <= tol
+    # deterministic: two runs are bit-identical
+    assert torch.equal(F.matmult(ta_, tb_), out)
+    # other flag pairs of the skinny path, ragged sizes, m in (1, 16, 17, 32)
+    for m, k, n, ta, tb in [(1, 300, 1000, False, False), (16, 257, 513, False, True), (17, 1024, 96, True, False),
+                            (32, 640, 2048, True, True), (3, 64, 5, False, False)]:
+        A, B, sa, sb, c0 = make_inputs(rng, m, k, n, np.float32, ta, tb)
+        ref = oracle.matmult2d(sa, sb, c0.copy(), ta, tb)
+        got = dev_matmult(sa, sb, c0, m, k, n, ta, tb, np.float32)
+        assert np.abs(got - ref).max() <= float_tol(k, A, B), (m, k, n, ta, tb)
