@@ -1,0 +1,347 @@
+// 16-bit (Float16 / BFloat16) MFMA GEMM for gfx950, fast path for tile-aligned problems:
+//   C[M,N] (+)= op(A) . op(B),  M % 256 == 0, N % 256 == 0, K % 32 == 0, 16-byte aligned rows.
+// (Everything else goes through the general kernel in gemm_mfma_impl.h.)
+//
+// Shape of the kernel
+//   * 256 x 256 tile of C per workgroup, 4 wavefronts (2 x 2), each owning 128 x 128 =
+//     4 x 4 blocks of v_mfma_f32_32x32x16_{f16,bf16}; 256 accumulator registers per lane.
+//   * K advances in steps of 32 through a 4-deep ring of LDS stages (4 x 32 KiB).  Global
+//     memory is copied straight into LDS (global_load_lds_dwordx4): no staging registers,
+//     three K-steps of loads in flight while one is being multiplied.
+//   * LDS layouts are conflict free for the reads the MFMA operands need:
+//       operand stored K-contiguous  -> [row][32 k] (64 B rows), 16-byte slot kv stored at
+//                                        kv ^ ((row >> 1) & 3); one ds_read_b128 per block;
+//       operand stored MN-contiguous -> [k][256 mn] (512 B rows), 16-byte chunk c stored at
+//                                        c ^ (2 * (k & 3)); ds_read_b64_tr_b16 turns four k-rows
+//                                        into "4 consecutive k per lane", i.e. the transpose
+//                                        is done by the LDS read, never in memory.
+//     Because the DMA writes 64 consecutive 16-byte slots per instruction, the swizzle is
+//     applied by choosing which global chunk each lane fetches.
+//   * The MFMA is issued with the operands swapped (B fragment first), so a lane holds four
+//     consecutive columns of one row of C; the epilogue stages 32-row slabs through LDS in
+//     fp32 and touches C with 16-byte accesses only (C0 is added in fp32 before the single
+//     rounding to the 16-bit type).
+#pragma once
+#include "gemm_mfma_impl.h"
+
+#include <type_traits>
+
+namespace ntg {
+
+typedef short shortx4 __attribute__((ext_vector_type(4)));
+typedef float floatx4v __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+
+#define NTG_WAIT_VMCNT(N) __builtin_amdgcn_s_waitcnt(((N) & 0xF) | (7 << 4) | (15 << 8) | (((N) >> 4) << 14))
+
+template <int DT>
+struct Cvt16;
+template <> struct Cvt16<DT_F16> {
+    static __device__ __forceinline__ float up(uint16_t v) { return (float)__builtin_bit_cast(_Float16, v); }
+    static __device__ __forceinline__ uint16_t down(float v) { return __builtin_bit_cast(uint16_t, (_Float16)v); }
+};
+template <> struct Cvt16<DT_BF16> {
+    static __device__ __forceinline__ float up(uint16_t v) { return __builtin_bit_cast(float, (uint32_t)v << 16); }
+    static __device__ __forceinline__ uint16_t down(float v) { return __builtin_bit_cast(uint16_t, (__bf16)v); }
+};
+
+struct G16 {
+    static constexpr int BM = 256, BN = 256, BK = 32, NST = 4;
+    static constexpr int TILE_BYTES = 256 * BK * 2;      // one operand tile, 16 KiB
+    static constexpr int STAGE_BYTES = 2 * TILE_BYTES;   // 32 KiB
+    static constexpr int LOADS_PER_TILE = 8;             // DMA instructions per wavefront per K-step
+};
+
+// Per-lane BYTE offsets (relative to the tile's first element at K-step 0) of this wavefront's
+// 4 DMA instructions into one operand tile.  Instruction j = 4*wave + jj fills LDS bytes
+// [1024 j, 1024 j + 1024) of the tile:
+//   K-contiguous operand: rows 16 j + lane/4, 16-byte slot lane%4 holds kv = slot ^ ((row>>1)&3)
+//   MN-contiguous operand: k-rows 2 j + lane/32, slot lane%32 holds chunk = slot ^ (2*(krow&3))
+template <bool KC>
+__device__ __forceinline__ void dma_offsets(uint32_t (&off)[4], int64_t ld, int wave, int lane) {
+#pragma unroll
+    for (int jj = 0; jj < 4; ++jj) {
+        const int j = wave * 4 + jj;
+        if constexpr (KC) {
+            const int row = 16 * j + (lane >> 2);
+            const int kv = (lane & 3) ^ ((row >> 1) & 3);
+            off[jj] = (uint32_t)(((int64_t)row * ld + kv * 8) * 2);
+        } else {
+            const int krow = 2 * j + (lane >> 5);
+            const int chunk = (lane & 31) ^ (2 * (krow & 3));
+            off[jj] = (uint32_t)(((int64_t)krow * ld + chunk * 8) * 2);
+        }
+    }
+}
+
+// One DMA instruction: 64 lanes x 16 bytes from  base + off  (uniform base, per-lane offset)
+// to LDS bytes [lds_addr, lds_addr + 1024).  Written as inline assembly so that the only
+// waits on these loads are the explicit s_waitcnt vmcnt(N) of the pipeline: the compiler's
+// own tracking of LDS-DMA writes made every read of one of the four stages wait for all
+// outstanding loads.  The memory clobber keeps LDS reads from being moved across it.
+__device__ __forceinline__ void dma_1k(const void* base, uint32_t off, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :: "s"(lds_addr), "v"(off), "s"(base) : "memory");
+}
+
+__device__ __forceinline__ void dma_tile(const void* base, const uint32_t (&off)[4], uint32_t lds_tile, int wave_u) {
+    // the base is the same for every lane; say so explicitly so that it is kept in scalar registers
+    const uint64_t bu = reinterpret_cast<uint64_t>(base);
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)bu);
+    const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(bu >> 32));
+    const void* sbase = reinterpret_cast<const void*>(((uint64_t)hi << 32) | lo);
+#pragma unroll
+    for (int jj = 0; jj < 4; ++jj) dma_1k(sbase, off[jj], lds_tile + (uint32_t)(wave_u * 4 + jj) * 1024u);
+}
+
+__device__ __forceinline__ uint32_t lds_addr_of(const char* p) {
+    return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const char*)p;
+}
+
+template <int DT, bool TA, bool TB>
+__global__ void __launch_bounds__(256) gemm16_kernel(const GemmParams p) {
+    using E = Elem<DT>;
+    using T = typename E::T;
+    constexpr bool A_KC = !TA, B_KC = TB;
+    constexpr int BK = G16::BK;
+
+    __shared__ __attribute__((aligned(1024))) char st0[G16::STAGE_BYTES];
+    __shared__ __attribute__((aligned(1024))) char st1[G16::STAGE_BYTES];
+    __shared__ __attribute__((aligned(1024))) char st2[G16::STAGE_BYTES];
+    __shared__ __attribute__((aligned(1024))) char st3[G16::STAGE_BYTES];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+
+    const int lid = xcd_contiguous_id(blockIdx.x, gridDim.x);
+    const int tiles = p.tiles_m * p.tiles_n;
+    const int b = lid / tiles;
+    int tm, tn;
+    tile_coords(lid - b * tiles, p.tiles_m, p.tiles_n, 4, tm, tn);
+    const int m0 = tm * G16::BM, n0 = tn * G16::BN;
+
+    const T* A = static_cast<const T*>(p.A) + (int64_t)b * p.sA;
+    const T* B = static_cast<const T*>(p.B) + (int64_t)b * p.sB;
+    T* C = static_cast<T*>(p.C) + (int64_t)b * p.sC;
+
+    // ---- DMA sources: uniform tile base (advances by adv bytes per K-step) + per-lane offsets ----
+    const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+    uint32_t offA[4], offB[4];
+    dma_offsets<A_KC>(offA, p.lda, wave, lane);
+    dma_offsets<B_KC>(offB, p.ldb, wave, lane);
+    const char* baseA = reinterpret_cast<const char*>(A) + (A_KC ? (int64_t)m0 * p.lda : (int64_t)m0) * 2;
+    const char* baseB = reinterpret_cast<const char*>(B) + (B_KC ? (int64_t)n0 * p.ldb : (int64_t)n0) * 2;
+    const int64_t advA = (A_KC ? (int64_t)BK : (int64_t)BK * p.lda) * 2;
+    const int64_t advB = (B_KC ? (int64_t)BK : (int64_t)BK * p.ldb) * 2;
+    auto issue_tile = [&](int kt, const char* stage) {
+        const uint32_t l = lds_addr_of(stage);
+#ifdef NTG_DBG_SAME_K
+        kt &= 3;
+#endif
+        dma_tile(baseA + kt * advA, offA, l, wave_u);
+        dma_tile(baseB + kt * advB, offB, l + G16::TILE_BYTES, wave_u);
+    };
+
+    // ---- per-lane LDS read offsets (bytes inside an operand tile), for k16-step ks ----
+    // K-major: block b of the wavefront, row = wbase + 32 b + lane%32, slot (2 ks + lane/32) ^ ((row>>1)&3)
+    // MN-major: two transposing reads per block; see the header comment
+    auto frag_off_km = [&](int wbase, int blk, int ks) -> int {
+        const int row = wbase + blk * 32 + (lane & 31);
+        const int slot = (2 * ks + (lane >> 5)) ^ ((lane >> 1) & 3);
+        return row * 64 + slot * 16;
+    };
+    auto frag_off_mm = [&](int wbase, int blk, int ks, int half) -> int {
+        const int bl = lane >> 4, s = lane & 15, e = s >> 2, q = s & 3;
+        const int krow = 16 * ks + 8 * (bl >> 1) + 4 * half + e;
+        const int mnl = wbase + blk * 32 + 16 * (bl & 1) + 4 * q;
+        const int chunk = (mnl >> 3) ^ (2 * e);
+        return krow * 512 + chunk * 16 + (mnl & 7) * 2;
+    };
+
+    // One LDS read instruction of an operand's fragment set for k16-step ks.  A K-major
+    // operand takes 4 reads (one ds_read_b128 per block), an MN-major one 8 (two transposing
+    // 8-byte reads per block); read r lands in frag[r / per_block] (half r % per_block).
+    auto read_op = [&](u32x4 (&frag)[4], const char* tile, bool kc, int wbase, int ks, int r) {
+        if (kc) {
+            frag[r] = *reinterpret_cast<const u32x4*>(tile + frag_off_km(wbase, r, ks));
+        } else {
+            const int blk = r >> 1, half = r & 1;
+            const shortx4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                (__attribute__((address_space(3))) shortx4*)(tile + frag_off_mm(wbase, blk, ks, half)));
+            typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+            const u32x2 w = __builtin_bit_cast(u32x2, v);
+            frag[blk][2 * half] = w[0];
+            frag[blk][2 * half + 1] = w[1];
+        }
+    };
+    constexpr int NRA = A_KC ? 4 : 8, NRB = B_KC ? 4 : 8, NR = NRA + NRB;
+
+    floatx16 acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+    const int KT = p.K / BK;
+
+    // prologue: all four stages in flight
+    issue_tile(0, st0);
+    if (1 < KT) issue_tile(1, st1);
+    if (2 < KT) issue_tile(2, st2);
+    if (3 < KT) issue_tile(3, st3);
+
+    u32x4 af[2][4], bf[2][4];   // fragment double buffer: [k16-step parity][block]
+
+    // all reads of one fragment set, back to back (prologue only)
+    auto load_frags = [&](const char* stage, int ks, int buf) {
+#pragma unroll
+        for (int r = 0; r < NRA; ++r) read_op(af[buf], stage, A_KC, wm * 128, ks, r);
+#pragma unroll
+        for (int r = 0; r < NRB; ++r) read_op(bf[buf], stage + G16::TILE_BYTES, B_KC, wn * 128, ks, r);
+    };
+    // 16 MFMAs on fragment set `cur_buf`, with the NR reads of the next set (stage/ks ->
+    // `nxt_buf`) slotted one per MFMA, so LDS latency is always covered by matrix work and
+    // never more than NR (<= 16) reads are outstanding.
+    auto mma_step_prefetch = [&](int cur_buf, const char* stage, int ks, int nxt_buf) {
+#pragma unroll
+        for (int q = 0; q < 16; ++q) {
+            const int i = q >> 2, j = q & 3;
+            E::mma(acc[i][j], bf[cur_buf][j], af[cur_buf][i]);   // D rows <-> n, cols <-> m
+            if (q < NRA) read_op(af[nxt_buf], stage, A_KC, wm * 128, ks, q);
+            else if (q < NR) read_op(bf[nxt_buf], stage + G16::TILE_BYTES, B_KC, wn * 128, ks, q - NRA);
+        }
+#pragma unroll
+        for (int q = 0; q < 16; ++q) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);           // one MFMA
+            if (q < NR) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // one LDS read
+        }
+    };
+
+    // tile 0 must have landed before its first fragments are read
+    if (KT > 3) NTG_WAIT_VMCNT(24); else if (KT > 2) NTG_WAIT_VMCNT(16); else if (KT > 1) NTG_WAIT_VMCNT(8); else NTG_WAIT_VMCNT(0);
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    load_frags(st0, 0, 0);
+
+    // One K-step.  `cur` holds tile kt (its k16-step 0 fragments are already in registers),
+    // `nxt` holds tile kt+1.  The single barrier sits between the two k16-steps: by then every
+    // wavefront has issued and received its last reads of `cur`, so the stage can be handed
+    // back to the DMA at once (tile kt+4), and tile kt+1 -- first touched in the second half --
+    // has had three full K-steps to arrive.
+    auto iteration = [&](int kt, char* cur, const char* nxt) {
+        mma_step_prefetch(0, cur, 1, 1);
+        if (kt + 3 < KT) NTG_WAIT_VMCNT(16); else if (kt + 2 < KT) NTG_WAIT_VMCNT(8); else NTG_WAIT_VMCNT(0);
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // my reads of `cur` are complete
+#ifndef NTG_DBG_NO_BARRIER
+        __builtin_amdgcn_s_barrier();
+#endif
+        asm volatile("" ::: "memory");
+#ifndef NTG_DBG_NO_DMA
+        if (kt + 4 < KT) issue_tile(kt + 4, cur);
+#endif
+        // the last K-step prefetches from a stage nobody writes any more; the data is unused
+        mma_step_prefetch(1, nxt, 0, 0);
+    };
+
+    for (int kt = 0; kt < KT; kt += 4) {
+        iteration(kt, st0, st1);
+        if (kt + 1 < KT) iteration(kt + 1, st1, st2);
+        if (kt + 2 < KT) iteration(kt + 2, st2, st3);
+        if (kt + 3 < KT) iteration(kt + 3, st3, st0);
+    }
+    __builtin_amdgcn_s_barrier();   // all fragment reads done: LDS is free for the epilogue
+    asm volatile("" ::: "memory");
+
+#ifdef NTG_DBG_NO_EPI
+    if (p.K > 0) { if (acc[0][0][0] == 123.f) C[0] = (T)1.f; return; }
+#endif
+    // ---- epilogue: per wavefront, four 32-row slabs through a private fp32 LDS region ----
+    // 32 rows x 512 B per wavefront; 16-byte slot s of row r lives at s ^ (r & 7)
+    char* slab = ((wave & 2) ? st1 : st0) + (wave & 1) * (32 * 512);
+    uint16_t* Cu = reinterpret_cast<uint16_t*>(C);
+    const int col = 8 * (lane & 15);               // this lane's 8 consecutive columns in the slab
+    const int n = n0 + wn * 128 + col;
+    auto epilogue = [&](auto cmode_tag) {
+        constexpr int CM = decltype(cmode_tag)::value;
+        const uint16_t* bias = static_cast<const uint16_t*>(p.bias);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            // C0 of the whole slab is requested before the LDS round trip
+            u32x4 c0[8];
+            if constexpr (CM == C_ACCUMULATE) {
+#pragma unroll
+                for (int t = 0; t < 8; ++t) {
+                    const int m = m0 + wm * 128 + 32 * i + 4 * t + (lane >> 4);
+                    c0[t] = *reinterpret_cast<const u32x4*>(Cu + (int64_t)m * p.ldc + n);
+                }
+            }
+            // lane holds rows m = 32 i + lane%32, cols 32 j + 8 rq + 4 (lane/32) + (0..3)
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int rq = 0; rq < 4; ++rq) {
+                    floatx4v v = {acc[i][j][4 * rq], acc[i][j][4 * rq + 1], acc[i][j][4 * rq + 2], acc[i][j][4 * rq + 3]};
+                    const int slot = 8 * j + 2 * rq + (lane >> 5);
+                    *reinterpret_cast<floatx4v*>(slab + (lane & 31) * 512 + ((slot ^ (lane & 7)) * 16)) = v;
+                }
+            // 32 rows x 128 cols: 8 steps of 4 rows; a lane owns 8 consecutive columns
+#pragma unroll
+            for (int t = 0; t < 8; ++t) {
+                const int row = 4 * t + (lane >> 4);
+                const int sl = 2 * (lane & 15);
+                const floatx4v lo = *reinterpret_cast<const floatx4v*>(slab + row * 512 + ((sl ^ (row & 7)) * 16));
+                const floatx4v hi = *reinterpret_cast<const floatx4v*>(slab + row * 512 + (((sl + 1) ^ (row & 7)) * 16));
+                float v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                const int m = m0 + wm * 128 + 32 * i + row;
+                if constexpr (CM == C_ACCUMULATE) {
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) v[e] += Cvt16<DT>::up((uint16_t)(c0[t][e >> 1] >> (16 * (e & 1))));
+                } else if constexpr (CM == C_BIAS) {
+#pragma unroll
+                    for (int e = 0; e < 8; ++e)
+                        v[e] += Cvt16<DT>::up(bias[(int64_t)b * p.bias_bs + (int64_t)m * p.bias_rs + (int64_t)(n + e) * p.bias_cs]);
+                }
+                u32x4 o;
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    o[e] = (uint32_t)Cvt16<DT>::down(v[2 * e]) | ((uint32_t)Cvt16<DT>::down(v[2 * e + 1]) << 16);
+                *reinterpret_cast<u32x4*>(Cu + (int64_t)m * p.ldc + n) = o;
+            }
+        }
+    };
+    if (p.cmode == C_ACCUMULATE) epilogue(std::integral_constant<int, C_ACCUMULATE>{});
+    else if (p.cmode == C_BIAS) epilogue(std::integral_constant<int, C_BIAS>{});
+    else epilogue(std::integral_constant<int, C_OVERWRITE>{});
+}
+
+// true when the fast kernel's preconditions hold
+static inline bool gemm16_eligible(const GemmParams& p) {
+    return p.M % 256 == 0 && p.N % 256 == 0 && p.K % 32 == 0 && p.K >= 32 &&
+           !p.Aptr && !p.Bptr && !p.Cptr && p.vecA_ok && p.vecB_ok &&
+           p.ldc % 8 == 0 && p.sC % 8 == 0 && p.lda < (1 << 22) && p.ldb < (1 << 22) &&
+           ((reinterpret_cast<uintptr_t>(p.A) & 15) == 0) && ((reinterpret_cast<uintptr_t>(p.B) & 15) == 0) &&
+           ((reinterpret_cast<uintptr_t>(p.C) & 15) == 0);
+}
+
+template <int DT, bool TA, bool TB>
+static hipError_t launch_gemm16_cfg(const GemmParams& pin, hipStream_t s) {
+    GemmParams p = pin;
+    p.tiles_m = p.M / 256;
+    p.tiles_n = p.N / 256;
+    const int64_t blocks = (int64_t)p.tiles_m * p.tiles_n * p.batch;
+    if (blocks > 0x7fffffffLL) return hipErrorInvalidValue;
+    hipLaunchKernelGGL((gemm16_kernel<DT, TA, TB>), dim3((unsigned)blocks), dim3(256), 0, s, p);
+    return hipGetLastError();
+}
+
+template <int DT>
+static hipError_t launch_gemm16(bool ta, bool tb, const GemmParams& p, hipStream_t s) {
+    if (ta) return tb ? launch_gemm16_cfg<DT, true, true>(p, s) : launch_gemm16_cfg<DT, true, false>(p, s);
+    return tb ? launch_gemm16_cfg<DT, false, true>(p, s) : launch_gemm16_cfg<DT, false, false>(p, s);
+}
+
+}  // namespace ntg
