@@ -1,0 +1,218 @@
+#!/usr/bin/env python3
+"""Benchmark of the matmult hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-extras] [--no-cpu]
+
+One "step" is one pass of nt::matmult over the headline workload of BASELINE.json
+(config 3): a 4096 x 4096 x 4096 BFloat16 product, inputs randn*0.02 already resident in
+HBM, fp32 accumulation, C += A.B (the accumulate contract of nt_matmult).  The timed
+region brackets exactly K launches between device synchronisations; the per-launch
+duration used for the roofline comes from HIP events recorded on the launch stream
+inside that region.  Prints ONE JSON line.
+
+Besides the headline value the line carries
+  roofline      achieved vs. MI355X dense-MFMA peak for the dominant kernel,
+  cpu_baseline  the CPU oracle's tiled restatement of the reference's TBB/SIMD GEMM, timed
+                on this host's cores on a bounded sample (reported, not a target),
+  extras        the other dtypes at 4096^3 and the remaining BASELINE configurations.
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_TFLOPS = {"bf16": 2500.0, "fp16": 2500.0, "fp32": 157.3, "fp64": 78.6}   # MI355X dense MFMA
+PEAK_HBM_GBS = 8000.0
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--no-extras", action="store_true", help="only the headline workload")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run a plain 256 MiB device copy (known HBM traffic) so that counter runs "
+                         "(rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE) can be scaled")
+    return ap.parse_args()
+
+
+def read_traffic_note():
+    """HBM bytes per launch of the headline kernel, measured offline with rocprofv3 --pmc
+    (FETCH_SIZE / WRITE_SIZE, scaled by a copy kernel); None until that profile exists."""
+    path = os.path.join(ROOT, "profiles", "gemm16_bf16_4096_hbm_traffic.txt")
+    try:
+        for line in open(path):
+            if line.startswith("hbm_traffic_bytes_per_launch:"):
+                return float(line.split(":", 1)[1].strip())
+    except OSError:
+        pass
+    return None
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU only (no collectives, no sharding); "
+              f"--gpus {args.gpus} is not supported. Re-run with --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    from neurotensor_amd import _lib
+    from neurotensor_amd import functional as F
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    lib = _lib.load()
+    dev = torch.device("cuda:0")
+    torch.manual_seed(1003)
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    def make_gemm(dtype, m, k, n, ta=False, tb=False, batch=1, scale=1.0, mode=_lib.C_ACCUMULATE, ints=False):
+        ashape = (batch, k, m) if ta else (batch, m, k)
+        bshape = (batch, n, k) if tb else (batch, k, n)
+        if ints:
+            a = torch.randint(-8, 9, ashape, device=dev, dtype=dtype)
+            b = torch.randint(-8, 9, bshape, device=dev, dtype=dtype)
+        else:
+            a = (torch.randn(ashape, device=dev) * scale).to(dtype)
+            b = (torch.randn(bshape, device=dev) * scale).to(dtype)
+        c = torch.zeros((batch, m, n), device=dev, dtype=dtype)
+        d = _lib.GemmDesc()
+        d.dtype = F.ntg_dtype(a)
+        d.transpose_a, d.transpose_b, d.c_mode = int(ta), int(tb), mode
+        d.m, d.k, d.n, d.batches = m, k, n, batch
+        d.stride_a, d.stride_b, d.stride_c = m * k, k * n, m * n
+
+        def launch():
+            _lib.check(lib.ntg_gemm_dev(ctypes.byref(d), a.data_ptr(), b.data_ptr(), c.data_ptr(), stream))
+
+        launch.keep = (a, b, c, d)
+        return launch
+
+    def time_steps(fn, steps, warmup):
+        """(wall ms per step over the whole timed region, mean ms per launch from HIP events)."""
+        for _ in range(warmup):
+            fn()
+        torch.cuda.synchronize()
+        evs = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
+        t0 = time.perf_counter()
+        evs[0].record()
+        for i in range(steps):
+            fn()
+            evs[i + 1].record()
+        torch.cuda.synchronize()
+        wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+        ev_ms = sum(evs[i].elapsed_time(evs[i + 1]) for i in range(steps)) / steps
+        return wall_ms, ev_ms
+
+    if args.copy_calibration:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).fill_(3)
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)          # reads 256 MiB, writes 256 MiB
+        torch.cuda.synchronize()
+        del src, dst
+
+    # ---------------- headline: config 3, BFloat16 4096^3, C += A.B ----------------
+    N = 4096
+    flops = 2.0 * N * N * N
+    head = make_gemm(torch.bfloat16, N, N, N, scale=0.02)
+    wall_ms, ev_ms = time_steps(head, args.steps, args.warmup)
+    value = flops / (wall_ms * 1e-3) / 1e12
+    achieved = flops / (ev_ms * 1e-3) / 1e12
+
+    out = {
+        "metric": "matmult TFLOP/s at 4096^3 (BFloat16, fp32 accumulate)",
+        "value": round(value, 2),
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(wall_ms, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": "nt::matmult A[4096,4096].B[4096,4096] BFloat16, inputs randn*0.02 resident in HBM, "
+                               "C += A.B (BASELINE config 3)", "m": N, "k": N, "n": N, "c_mode": "accumulate"},
+        "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_TFLOPS["bf16"], "unit": "TFLOP/s",
+                     "frac": round(achieved / PEAK_TFLOPS["bf16"], 4), "traffic": read_traffic_note(),
+                     "kernel": "ntg::gemm16_kernel<BFloat16, NN>", "launch_ms": round(ev_ms, 5)},
+    }
+
+    # ---------------- extras: the other dtypes and configurations ----------------
+    if not args.no_extras:
+        extras = {}
+        steps, warm = max(5, args.steps // 5), max(2, args.warmup // 3)
+
+        def run(name, fn, work, peak=None, unit="TFLOP/s", scale=1e12, st=steps):
+            _, ms = time_steps(fn, st, warm)
+            rate = work / (ms * 1e-3) / scale
+            e = {"ms": round(ms, 5), "rate": round(rate, 2), "unit": unit}
+            if peak:
+                e["frac_of_peak"] = round(rate / peak, 4)
+            extras[name] = e
+
+        run("c3_fp16_4096", make_gemm(torch.float16, N, N, N, scale=0.02), flops, PEAK_TFLOPS["fp16"])
+        run("c3_bf16_4096_overwrite", make_gemm(torch.bfloat16, N, N, N, scale=0.02, mode=_lib.C_OVERWRITE), flops, PEAK_TFLOPS["bf16"])
+        run("c3_fp32_4096", make_gemm(torch.float32, N, N, N), flops, PEAK_TFLOPS["fp32"])
+        run("c3_fp64_4096", make_gemm(torch.float64, N, N, N), flops, PEAK_TFLOPS["fp64"])
+        run("c1_fp32_512", make_gemm(torch.float32, 512, 512, 512), 2.0 * 512 ** 3, PEAK_TFLOPS["fp32"], st=steps * 4)
+        f2 = 2.0 * 32 * 1024 * 768 * 1024
+        run("c2a_fp32_b32_1024x768x1024", make_gemm(torch.float32, 1024, 768, 1024, batch=32), f2, PEAK_TFLOPS["fp32"])
+        run("c2b_fp32_b32_transpose_b", make_gemm(torch.float32, 1024, 768, 1024, tb=True, batch=32), f2, PEAK_TFLOPS["fp32"])
+        run("c2c_int32_b8_1024", make_gemm(torch.int32, 1024, 1024, 1024, batch=8, ints=True), 2.0 * 8 * 1024 ** 3, None, "Top/s")
+        f4 = 2.0 * 8192 * 4096 * 11008
+        for dt, nm in ((torch.float32, "fp32"), (torch.bfloat16, "bf16")):
+            pk = PEAK_TFLOPS[nm]
+            run(f"c4_linear_fwd_{nm}", make_gemm(dt, 8192, 4096, 11008, tb=True, mode=_lib.C_OVERWRITE, scale=0.1), f4, pk)
+            run(f"c4_linear_dx_{nm}", make_gemm(dt, 8192, 11008, 4096, mode=_lib.C_OVERWRITE, scale=0.1), f4, pk)
+            run(f"c4_linear_dw_{nm}", make_gemm(dt, 11008, 8192, 4096, ta=True, mode=_lib.C_OVERWRITE, scale=0.1), f4, pk)
+        x = torch.randn(64, 256, 56, 56, device=dev)
+        w = torch.randn(256, 256, 3, 3, device=dev) / 48.0
+        run("c5a_conv2d_fp32", lambda: F.conv2d(x, w, padding=1), 2.0 * 200704 * 2304 * 256, PEAK_TFLOPS["fp32"])
+        del x, w
+        skinny_bytes = 4.0 * (16 * 8192 + 8192 * 8192 + 2 * 16 * 8192)
+        run("c5b_skinny_fp32_16x8192x8192", make_gemm(torch.float32, 16, 8192, 8192), skinny_bytes, PEAK_HBM_GBS, "GB/s", 1e9,
+            st=steps * 4)
+        out["extras"] = extras
+
+    # ---------------- CPU baseline: the oracle's restatement of the reference loop nest ----------------
+    if not args.no_cpu:
+        import numpy as np
+
+        import oracle
+        threads = oracle.lib().oracle_tiled_threads(0)
+        rng = np.random.default_rng(1003)
+        a = rng.standard_normal((N, N)).astype(np.float32)
+        b = rng.standard_normal((N, N)).astype(np.float32)
+        c = np.zeros((N, N), np.float32)
+        oracle.matmult2d(a[:256], b, np.zeros((256, N), np.float32), kind="tiled")     # warm the pool
+        reps, t_cpu = 0, 0.0
+        while reps < 1 or (t_cpu < 10.0 and reps < 8):
+            t0 = time.perf_counter()
+            oracle.matmult2d(a, b, c, kind="tiled")
+            t_cpu += time.perf_counter() - t0
+            reps += 1
+        out["cpu_baseline"] = {
+            "value": round(flops * reps / t_cpu / 1e12, 4), "unit": "TFLOP/s", "cores": threads, "kind": "port",
+            "sample": f"Float32 4096x4096x4096, {reps} pass(es) of the tiled/packed k-outer restatement "
+                      f"(tile 16, pack block 7056, thread cap 21 -> {threads} threads); the reference has no BFloat16",
+        }
+
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

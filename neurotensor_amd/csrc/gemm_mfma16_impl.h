@@ -7,7 +7,10 @@
 //     4 x 4 blocks of v_mfma_f32_32x32x16_{f16,bf16}; 256 accumulator registers per lane.
 //   * K advances in steps of 32 through a 4-deep ring of LDS stages (4 x 32 KiB).  Global
 //     memory is copied straight into LDS (global_load_lds_dwordx4): no staging registers,
-//     three K-steps of loads in flight while one is being multiplied.
+//     three to four K-steps of loads in flight while one is being multiplied.  One barrier
+//     per K-step, placed between its two k16 halves; the DMA instructions and the LDS
+//     fragment reads are slotted between the MFMAs one at a time, so neither the CU's single
+//     address unit nor LDS latency ever holds up the matrix pipe.
 //   * LDS layouts are conflict free for the reads the MFMA operands need:
 //       operand stored K-contiguous  -> [row][32 k] (64 B rows), 16-byte slot kv stored at
 //                                        kv ^ ((row >> 1) & 3); one ds_read_b128 per block;
@@ -84,12 +87,7 @@ __device__ __forceinline__ void dma_1k(const void* base, uint32_t off, uint32_t 
                  :: "s"(lds_addr), "v"(off), "s"(base) : "memory");
 }
 
-__device__ __forceinline__ void dma_tile(const void* base, const uint32_t (&off)[4], uint32_t lds_tile, int wave_u) {
-    // the base is the same for every lane; say so explicitly so that it is kept in scalar registers
-    const uint64_t bu = reinterpret_cast<uint64_t>(base);
-    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)bu);
-    const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(bu >> 32));
-    const void* sbase = reinterpret_cast<const void*>(((uint64_t)hi << 32) | lo);
+__device__ __forceinline__ void dma_tile(const void* sbase, const uint32_t (&off)[4], uint32_t lds_tile, int wave_u) {
 #pragma unroll
     for (int jj = 0; jj < 4; ++jj) dma_1k(sbase, off[jj], lds_tile + (uint32_t)(wave_u * 4 + jj) * 1024u);
 }
@@ -135,13 +133,12 @@ __global__ void __launch_bounds__(256) gemm16_kernel(const GemmParams p) {
     const char* baseB = reinterpret_cast<const char*>(B) + (B_KC ? (int64_t)n0 * p.ldb : (int64_t)n0) * 2;
     const int64_t advA = (A_KC ? (int64_t)BK : (int64_t)BK * p.lda) * 2;
     const int64_t advB = (B_KC ? (int64_t)BK : (int64_t)BK * p.ldb) * 2;
-    auto issue_tile = [&](int kt, const char* stage) {
-        const uint32_t l = lds_addr_of(stage);
-#ifdef NTG_DBG_SAME_K
-        kt &= 3;
-#endif
-        dma_tile(baseA + kt * advA, offA, l, wave_u);
-        dma_tile(baseB + kt * advB, offB, l + G16::TILE_BYTES, wave_u);
+    // uniform (scalar) source pointer of one operand tile
+    auto tile_src = [&](const char* base) -> const void* {
+        const uint64_t bu = reinterpret_cast<uint64_t>(base);
+        const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)bu);
+        const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(bu >> 32));
+        return reinterpret_cast<const void*>(((uint64_t)hi << 32) | lo);
     };
 
     // ---- per-lane LDS read offsets (bytes inside an operand tile), for k16-step ks ----
@@ -188,11 +185,21 @@ __global__ void __launch_bounds__(256) gemm16_kernel(const GemmParams p) {
 
     const int KT = p.K / BK;
 
-    // prologue: all four stages in flight
-    issue_tile(0, st0);
-    if (1 < KT) issue_tile(1, st1);
-    if (2 < KT) issue_tile(2, st2);
-    if (3 < KT) issue_tile(3, st3);
+    // K-steps past the end are clamped to the last one: the tail iterations then issue the
+    // same DMA traffic as the steady state (into stages nobody reads any more), which keeps
+    // the loop body free of branches and the vmcnt bookkeeping uniform.
+    const int last = KT - 1;
+    auto srcA = [&](int kt) { return tile_src(baseA + (int64_t)(kt < last ? kt : last) * advA); };
+    auto srcB = [&](int kt) { return tile_src(baseB + (int64_t)(kt < last ? kt : last) * advB); };
+
+    // prologue: tiles 0..2 and the A half of tile 3 in flight (28 instructions)
+    dma_tile(srcA(0), offA, lds_addr_of(st0), wave_u);
+    dma_tile(srcB(0), offB, lds_addr_of(st0) + G16::TILE_BYTES, wave_u);
+    dma_tile(srcA(1), offA, lds_addr_of(st1), wave_u);
+    dma_tile(srcB(1), offB, lds_addr_of(st1) + G16::TILE_BYTES, wave_u);
+    dma_tile(srcA(2), offA, lds_addr_of(st2), wave_u);
+    dma_tile(srcB(2), offB, lds_addr_of(st2) + G16::TILE_BYTES, wave_u);
+    dma_tile(srcA(3), offA, lds_addr_of(st3), wave_u);
 
     u32x4 af[2][4], bf[2][4];   // fragment double buffer: [k16-step parity][block]
 
@@ -205,60 +212,60 @@ __global__ void __launch_bounds__(256) gemm16_kernel(const GemmParams p) {
     };
     // 16 MFMAs on fragment set `cur_buf`, with the NR reads of the next set (stage/ks ->
     // `nxt_buf`) slotted one per MFMA, so LDS latency is always covered by matrix work and
-    // never more than NR (<= 16) reads are outstanding.
-    auto mma_step_prefetch = [&](int cur_buf, const char* stage, int ks, int nxt_buf) {
+    // never more than NR (<= 16) reads are outstanding.  Four DMA instructions (one operand
+    // tile's share of this wavefront) are spread over the step as well -- issued in a burst
+    // right after the barrier, the four wavefronts would queue up behind the CU's one
+    // address unit and stall their MFMA streams.
+    auto mma_step_prefetch = [&](int cur_buf, const char* stage, int ks, int nxt_buf,
+                                 const void* src, const uint32_t (&off)[4], uint32_t lds_tile) {
 #pragma unroll
         for (int q = 0; q < 16; ++q) {
             const int i = q >> 2, j = q & 3;
             E::mma(acc[i][j], bf[cur_buf][j], af[cur_buf][i]);   // D rows <-> n, cols <-> m
             if (q < NRA) read_op(af[nxt_buf], stage, A_KC, wm * 128, ks, q);
             else if (q < NR) read_op(bf[nxt_buf], stage + G16::TILE_BYTES, B_KC, wn * 128, ks, q - NRA);
+            if ((q & 3) == 3) dma_1k(src, off[q >> 2], lds_tile + (uint32_t)(wave_u * 4 + (q >> 2)) * 1024u);
         }
 #pragma unroll
         for (int q = 0; q < 16; ++q) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);           // one MFMA
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);               // one MFMA
             if (q < NR) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // one LDS read
         }
     };
 
     // tile 0 must have landed before its first fragments are read
-    if (KT > 3) NTG_WAIT_VMCNT(24); else if (KT > 2) NTG_WAIT_VMCNT(16); else if (KT > 1) NTG_WAIT_VMCNT(8); else NTG_WAIT_VMCNT(0);
+    NTG_WAIT_VMCNT(20);
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
     load_frags(st0, 0, 0);
 
     // One K-step.  `cur` holds tile kt (its k16-step 0 fragments are already in registers),
-    // `nxt` holds tile kt+1.  The single barrier sits between the two k16-steps: by then every
-    // wavefront has issued and received its last reads of `cur`, so the stage can be handed
-    // back to the DMA at once (tile kt+4), and tile kt+1 -- first touched in the second half --
-    // has had three full K-steps to arrive.
-    auto iteration = [&](int kt, char* cur, const char* nxt) {
-        mma_step_prefetch(0, cur, 1, 1);
-        if (kt + 3 < KT) NTG_WAIT_VMCNT(16); else if (kt + 2 < KT) NTG_WAIT_VMCNT(8); else NTG_WAIT_VMCNT(0);
+    // `nxt` holds tile kt+1, `prv` held tile kt-1.  The single barrier sits between the two
+    // k16-steps: by then every wavefront has issued and received its last reads of `cur`, so
+    // the stage goes back to the DMA at once: the A half of tile kt+4 is fetched during the
+    // second k16-step, its B half during the first k16-step of the next K-step.  Tile kt+1,
+    // first touched in the second half, has had three K-steps to arrive.
+    auto iteration = [&](int kt, char* cur, const char* nxt, char* prv) {
+        mma_step_prefetch(0, cur, 1, 1, srcB(kt + 3), offB, lds_addr_of(prv) + G16::TILE_BYTES);
+        // outstanding now: tiles kt+1, kt+2, kt+3 (8 instructions each): wait for the oldest
+        NTG_WAIT_VMCNT(16);
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // my reads of `cur` are complete
-#ifndef NTG_DBG_NO_BARRIER
         __builtin_amdgcn_s_barrier();
-#endif
         asm volatile("" ::: "memory");
-#ifndef NTG_DBG_NO_DMA
-        if (kt + 4 < KT) issue_tile(kt + 4, cur);
-#endif
-        // the last K-step prefetches from a stage nobody writes any more; the data is unused
-        mma_step_prefetch(1, nxt, 0, 0);
+        // (the last K-step prefetches fragments from a stage holding a clamped tile; unused)
+        mma_step_prefetch(1, nxt, 0, 0, srcA(kt + 4), offA, lds_addr_of(cur));
     };
 
     for (int kt = 0; kt < KT; kt += 4) {
-        iteration(kt, st0, st1);
-        if (kt + 1 < KT) iteration(kt + 1, st1, st2);
-        if (kt + 2 < KT) iteration(kt + 2, st2, st3);
-        if (kt + 3 < KT) iteration(kt + 3, st3, st0);
+        iteration(kt, st0, st1, st3);
+        if (kt + 1 < KT) iteration(kt + 1, st1, st2, st0);
+        if (kt + 2 < KT) iteration(kt + 2, st2, st3, st1);
+        if (kt + 3 < KT) iteration(kt + 3, st3, st0, st2);
     }
+    NTG_WAIT_VMCNT(0);              // clamped tail DMAs have landed
     __builtin_amdgcn_s_barrier();   // all fragment reads done: LDS is free for the epilogue
     asm volatile("" ::: "memory");
 
-#ifdef NTG_DBG_NO_EPI
-    if (p.K > 0) { if (acc[0][0][0] == 123.f) C[0] = (T)1.f; return; }
-#endif
     // ---- epilogue: per wavefront, four 32-row slabs through a private fp32 LDS region ----
     // 32 rows x 512 B per wavefront; 16-byte slot s of row r lives at s ^ (r & 7)
     char* slab = ((wave & 2) ? st1 : st0) + (wave & 1) * (32 * 512);
