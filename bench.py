@@ -100,19 +100,23 @@ def main():
         return launch
 
     def time_steps(fn, steps, warmup):
-        """(wall ms per step over the whole timed region, mean ms per launch from HIP events)."""
+        """(wall ms per step over the whole timed region, mean ms per launch from a pair of HIP
+        events recorded on the launch stream around the same K launches).  One event pair, not
+        one per launch: an event between two kernels drains the queue and would add a gap of
+        several microseconds to every launch."""
         for _ in range(warmup):
             fn()
         torch.cuda.synchronize()
-        evs = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
         t0 = time.perf_counter()
-        evs[0].record()
-        for i in range(steps):
+        e0.record()
+        for _ in range(steps):
             fn()
-            evs[i + 1].record()
+        e1.record()
         torch.cuda.synchronize()
         wall_ms = (time.perf_counter() - t0) * 1e3 / steps
-        ev_ms = sum(evs[i].elapsed_time(evs[i + 1]) for i in range(steps)) / steps
+        ev_ms = e0.elapsed_time(e1) / steps
         return wall_ms, ev_ms
 
     if args.copy_calibration:

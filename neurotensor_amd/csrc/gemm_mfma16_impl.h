@@ -220,7 +220,8 @@ __global__ void __launch_bounds__(256) gemm16_kernel(const GemmParams p) {
                                  const void* src, const uint32_t (&off)[4], uint32_t lds_tile) {
 #pragma unroll
         for (int q = 0; q < 16; ++q) {
-            const int i = q >> 2, j = q & 3;
+            // serpentine order: consecutive MFMAs always share one operand fragment
+            const int i = q >> 2, j = (i & 1) ? 3 - (q & 3) : (q & 3);
             E::mma(acc[i][j], bf[cur_buf][j], af[cur_buf][i]);   // D rows <-> n, cols <-> m
             if (q < NRA) read_op(af[nxt_buf], stage, A_KC, wm * 128, ks, q);
             else if (q < NR) read_op(bf[nxt_buf], stage + G16::TILE_BYTES, B_KC, wn * 128, ks, q - NRA);
