@@ -1,0 +1,541 @@
+// Implementation of the nt_compat facade on the host-pointer C ABI of libntgemm.so.
+// Every validation happens here, before any device work, with the reference's messages.
+#include "nt_compat.h"
+
+#include "../../include/ntgemm.h"
+
+#include <algorithm>
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+#include <fstream>
+#include <random>
+#include <sstream>
+
+namespace nt {
+
+int64_t dtype_size(DType dt) { return ntg_dtype_size(static_cast<int>(dt)); }
+
+const char* dtype_name(DType dt) {
+    switch (dt) {
+    case DType::Float16: return "Float16"; case DType::Float32: return "Float32"; case DType::Float64: return "Float64";
+    case DType::BFloat16: return "BFloat16"; case DType::int8: return "int8"; case DType::int16: return "int16";
+    case DType::int32: return "int32"; case DType::int64: return "int64"; case DType::uint8: return "uint8";
+    case DType::uint16: return "uint16"; case DType::uint32: return "uint32"; case DType::uint64: return "uint64";
+    case DType::Bool: return "Bool"; case DType::TensorObj: return "TensorObj";
+    default: return "unsupported";
+    }
+}
+
+namespace utils {
+void throw_exception(bool ok, const std::string& message) {
+    if (!ok) throw nt_error(message);
+}
+}  // namespace utils
+
+std::string shape_str(const SizeRef& s) {
+    std::ostringstream o;
+    o << "{";
+    for (size_t i = 0; i < s.size(); ++i) o << (i ? "," : "") << s[i];
+    o << "}";
+    return o.str();
+}
+
+static int64_t prod(const SizeRef& s, size_t from = 0, size_t to = (size_t)-1) {
+    int64_t p = 1;
+    for (size_t i = from; i < std::min(to, s.size()); ++i) p *= s[i];
+    return p;
+}
+
+static SizeRef dense_strides(const SizeRef& shape) {
+    SizeRef st(shape.size());
+    int64_t acc = 1;
+    for (int64_t i = (int64_t)shape.size() - 1; i >= 0; --i) { st[i] = acc; acc *= shape[i]; }
+    return st;
+}
+
+// ------------------------------------------------------------------------------------------ Tensor
+
+Tensor::Tensor(SizeRef shape, DType dt) : shape_(std::move(shape)), dtype_(dt) {
+    const int64_t es = dtype_size(dt);
+    utils::throw_exception(es > 0, std::string("dtype ") + dtype_name(dt) + " has no storage in nt_compat");
+    for (int64_t d : shape_) utils::throw_exception(d >= 0, "negative dimension in shape " + shape_str(shape_));
+    strides_ = dense_strides(shape_);
+    const size_t bytes = (size_t)std::max<int64_t>(1, prod(shape_) * es);
+    storage_ = std::shared_ptr<char>(static_cast<char*>(::operator new(bytes)), [](char* p) { ::operator delete(p); });
+}
+
+int64_t Tensor::numel() const { return is_null() ? 0 : prod(shape_); }
+
+bool Tensor::is_contiguous() const {
+    int64_t acc = 1;
+    for (int64_t i = dims() - 1; i >= 0; --i) {
+        if (shape_[i] != 1 && strides_[i] != acc) return false;
+        acc *= shape_[i];
+    }
+    return true;
+}
+
+Tensor Tensor::clone() const {
+    utils::throw_exception(!is_null(), "cannot clone a null tensor");
+    Tensor out(shape_, dtype_);
+    const int64_t es = dtype_size(dtype_), n = numel();
+    if (is_contiguous()) {
+        std::memcpy(out.data_ptr(), data_ptr(), (size_t)(n * es));
+        return out;
+    }
+    const char* src = static_cast<const char*>(data_ptr());
+    char* dst = static_cast<char*>(out.data_ptr());
+    SizeRef idx(shape_.size(), 0);
+    for (int64_t lin = 0; lin < n; ++lin) {
+        int64_t off = 0;
+        for (size_t d = 0; d < idx.size(); ++d) off += idx[d] * strides_[d];
+        std::memcpy(dst + lin * es, src + off * es, (size_t)es);
+        for (int64_t d = (int64_t)idx.size() - 1; d >= 0; --d) {
+            if (++idx[d] < shape_[d]) break;
+            idx[d] = 0;
+        }
+    }
+    return out;
+}
+
+Tensor Tensor::view(SizeRef shape) const {
+    utils::throw_exception(is_contiguous(), "view needs a contiguous tensor");
+    int64_t known = 1, unknown = -1;
+    for (size_t i = 0; i < shape.size(); ++i) {
+        if (shape[i] == -1) { utils::throw_exception(unknown < 0, "only one -1 allowed in view"); unknown = (int64_t)i; }
+        else known *= shape[i];
+    }
+    if (unknown >= 0) { utils::throw_exception(known != 0 && numel() % known == 0, "view shape does not divide numel"); shape[(size_t)unknown] = numel() / known; }
+    utils::throw_exception(prod(shape) == numel(), "view of " + shape_str(shape_) + " as " + shape_str(shape) + " changes numel");
+    Tensor out = *this;
+    out.shape_ = shape;
+    out.strides_ = dense_strides(shape);
+    return out;
+}
+
+Tensor Tensor::transpose(int64_t a, int64_t b) const {
+    const int64_t nd = dims();
+    if (a < 0) a += nd;
+    if (b < 0) b += nd;
+    utils::throw_exception(a >= 0 && a < nd && b >= 0 && b < nd, "transpose dims out of range");
+    Tensor out = *this;
+    std::swap(out.shape_[(size_t)a], out.shape_[(size_t)b]);
+    std::swap(out.strides_[(size_t)a], out.strides_[(size_t)b]);
+    return out;
+}
+
+Tensor Tensor::unsqueeze_front(int64_t n) const {
+    Tensor out = *this;
+    for (int64_t i = 0; i < n; ++i) { out.shape_.insert(out.shape_.begin(), 1); out.strides_.insert(out.strides_.begin(), 0); }
+    return out;
+}
+
+Tensor Tensor::item(int64_t i) const {
+    utils::throw_exception(is_contiguous() && dims() >= 2, "item needs a contiguous tensor of matrices");
+    const int64_t mat = shape_[(size_t)dims() - 1] * shape_[(size_t)dims() - 2];
+    Tensor out = *this;
+    out.shape_ = {shape_[(size_t)dims() - 2], shape_[(size_t)dims() - 1]};
+    out.strides_ = dense_strides(out.shape_);
+    out.offset_ = offset_ + i * mat * dtype_size(dtype_);
+    return out;
+}
+
+template <class T>
+static void sum_as_t(const Tensor& src, Tensor& dst, const SizeRef& tgt_padded) {
+    // src contiguous with shape S; dst contiguous with shape tgt_padded (same rank, dims equal or 1)
+    const SizeRef& S = src.shape();
+    const int64_t n = src.numel();
+    T* d = dst.data<T>();
+    for (int64_t i = 0; i < dst.numel(); ++i) d[i] = T(0);
+    const T* s = src.data<T>();
+    const SizeRef dst_st = dense_strides(tgt_padded);
+    SizeRef idx(S.size(), 0);
+    for (int64_t lin = 0; lin < n; ++lin) {
+        int64_t off = 0;
+        for (size_t k = 0; k < S.size(); ++k) off += (tgt_padded[k] == 1 ? 0 : idx[k]) * dst_st[k];
+        d[off] += s[lin];
+        for (int64_t k = (int64_t)S.size() - 1; k >= 0; --k) {
+            if (++idx[(size_t)k] < S[(size_t)k]) break;
+            idx[(size_t)k] = 0;
+        }
+    }
+}
+
+// grad += in_grad with broadcasting reduced back by sum_as (nt/functional/tensor_files/operators.cpp:175-187)
+Tensor Tensor::sum_leading(const SizeRef& target) const {
+    Tensor src = contiguous();
+    utils::throw_exception((int64_t)target.size() <= dims(), "sum_as target has more dims than the source");
+    SizeRef padded(shape_.size(), 1);
+    for (size_t i = 0; i < target.size(); ++i) padded[shape_.size() - target.size() + i] = target[i];
+    for (size_t i = 0; i < padded.size(); ++i)
+        utils::throw_exception(padded[i] == 1 || padded[i] == shape_[i], "cannot reduce " + shape_str(shape_) + " to " + shape_str(target));
+    Tensor out(target, dtype_);
+    if (dtype_ == DType::Float32) sum_as_t<float>(src, out, padded);
+    else if (dtype_ == DType::Float64) sum_as_t<double>(src, out, padded);
+    else if (dtype_ == DType::int32) sum_as_t<int32_t>(src, out, padded);
+    else if (dtype_ == DType::int64) sum_as_t<int64_t>(src, out, padded);
+    else utils::throw_exception(false, std::string("sum_as is not available for ") + dtype_name(dtype_));
+    return out;
+}
+
+// ------------------------------------------------------------------------------------------ helpers
+
+namespace functional {
+
+Tensor zeros(SizeRef shape, DType dt) {
+    Tensor t(std::move(shape), dt);
+    std::memset(t.data_ptr(), 0, (size_t)(t.numel() * dtype_size(dt)));
+    return t;
+}
+
+static uint16_t f32_to_bf16(float f) {
+    uint32_t x;
+    std::memcpy(&x, &f, 4);
+    if ((x & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((x >> 16) | 0x40u);
+    x += 0x7fffu + ((x >> 16) & 1u);
+    return (uint16_t)(x >> 16);
+}
+
+Tensor randn(SizeRef shape, DType dt, uint64_t seed) {
+    Tensor t(std::move(shape), dt);
+    std::mt19937_64 gen(seed ? seed : 0x9e3779b97f4a7c15ull);
+    std::normal_distribution<double> nd(0.0, 1.0);
+    const int64_t n = t.numel();
+    switch (dt) {
+    case DType::Float32: for (int64_t i = 0; i < n; ++i) t.data<float>()[i] = (float)nd(gen); break;
+    case DType::Float64: for (int64_t i = 0; i < n; ++i) t.data<double>()[i] = nd(gen); break;
+    case DType::BFloat16: for (int64_t i = 0; i < n; ++i) t.data<uint16_t>()[i] = f32_to_bf16((float)nd(gen)); break;
+    case DType::int32: for (int64_t i = 0; i < n; ++i) t.data<int32_t>()[i] = (int32_t)std::lround(nd(gen) * 4.0); break;
+    case DType::int64: for (int64_t i = 0; i < n; ++i) t.data<int64_t>()[i] = (int64_t)std::lround(nd(gen) * 4.0); break;
+    default: utils::throw_exception(false, std::string("randn is not available for ") + dtype_name(dt));
+    }
+    return t;
+}
+
+Tensor from_numpy(const std::string& path) {
+    std::ifstream f(path, std::ios::binary);
+    utils::throw_exception((bool)f, "cannot open " + path);
+    char magic[8];
+    f.read(magic, 8);
+    utils::throw_exception(f && std::memcmp(magic, "\x93NUMPY", 6) == 0, path + " is not a .npy file");
+    uint32_t hlen = 0;
+    if (magic[6] == 1) { uint16_t h16; f.read(reinterpret_cast<char*>(&h16), 2); hlen = h16; }
+    else f.read(reinterpret_cast<char*>(&hlen), 4);
+    std::string hdr(hlen, ' ');
+    f.read(&hdr[0], hlen);
+    auto field = [&](const std::string& key) {
+        size_t p = hdr.find("'" + key + "'");
+        utils::throw_exception(p != std::string::npos, "npy header lacks " + key);
+        return hdr.substr(hdr.find(':', p) + 1);
+    };
+    std::string descr = field("descr");
+    descr = descr.substr(descr.find('\'') + 1);
+    descr = descr.substr(0, descr.find('\''));
+    utils::throw_exception(field("fortran_order").find("False") < 8, "fortran-order .npy is not supported");
+    std::string shp = field("shape");
+    shp = shp.substr(shp.find('(') + 1);
+    shp = shp.substr(0, shp.find(')'));
+    SizeRef shape;
+    std::stringstream ss(shp);
+    std::string tok;
+    while (std::getline(ss, tok, ',')) {
+        bool digit = false;
+        for (char c : tok) digit |= (c >= '0' && c <= '9');
+        if (digit) shape.push_back(std::stoll(tok));
+    }
+    DType dt;
+    const std::string code = descr.substr(1);
+    utils::throw_exception(descr[0] == '<' || descr[0] == '|' || descr[0] == '=', "big-endian .npy is not supported");
+    if (code == "f4") dt = DType::Float32; else if (code == "f8") dt = DType::Float64; else if (code == "f2") dt = DType::Float16;
+    else if (code == "i1") dt = DType::int8; else if (code == "i2") dt = DType::int16; else if (code == "i4") dt = DType::int32;
+    else if (code == "i8") dt = DType::int64; else if (code == "u1") dt = DType::uint8;
+    else { utils::throw_exception(false, "npy dtype " + descr + " is not supported"); dt = DType::Float32; }
+    Tensor t(shape, dt);
+    f.read(static_cast<char*>(t.data_ptr()), (std::streamsize)(t.numel() * dtype_size(dt)));
+    utils::throw_exception((bool)f, path + " is truncated");
+    return t;
+}
+
+bool allclose(const Tensor& a_, const Tensor& b_, double rtol, double atol) {
+    if (a_.is_null() || b_.is_null() || a_.shape() != b_.shape() || a_.dtype() != b_.dtype()) return false;
+    Tensor a = a_.contiguous(), b = b_.contiguous();
+    const int64_t n = a.numel();
+    auto chk = [&](auto* pa, auto* pb) {
+        for (int64_t i = 0; i < n; ++i) {
+            const double x = (double)pa[i], y = (double)pb[i];
+            if (!(std::fabs(x - y) <= atol + rtol * std::fabs(y))) return false;
+        }
+        return true;
+    };
+    switch (a.dtype()) {
+    case DType::Float32: return chk(a.data<float>(), b.data<float>());
+    case DType::Float64: return chk(a.data<double>(), b.data<double>());
+    case DType::int32: return chk(a.data<int32_t>(), b.data<int32_t>());
+    case DType::int64: return chk(a.data<int64_t>(), b.data<int64_t>());
+    default: return std::memcmp(a.data_ptr(), b.data_ptr(), (size_t)(n * dtype_size(a.dtype()))) == 0;
+    }
+}
+
+static void check_status(int rc) {
+    if (rc != NTG_OK) throw utils::nt_error(std::string("gfx950 matmult backend: ") + ntg_last_error());
+}
+
+// A contiguous tensor is used as is; a view whose last two dims are a transposed contiguous
+// matrix flips the flag instead of copying (was_transposed_back, matmult_cpu.cpp:204-250,
+// 268-274, 491-494); anything else is cloned (matmult_cpu.cpp:277-279, 471-473).
+static Tensor matrix_storage(const Tensor& t, bool& trans) {
+    if (t.is_contiguous()) return t;
+    Tensor tt = t.transpose(-1, -2);
+    if (tt.is_contiguous()) { trans = !trans; return tt; }
+    return t.clone();
+}
+
+struct MatmultPlan {
+    Tensor a, b;            // storage tensors (contiguous)
+    bool ta, tb;
+    int64_t m, k, n, nbig, na, nb;
+    SizeRef out_shape;
+};
+
+static MatmultPlan plan_matmult(const Tensor& a_in, const Tensor& b_in, bool trans_a, bool trans_b, bool out_variant) {
+    utils::throw_exception(!a_in.is_null() && !b_in.is_null(), "Cannot perform operation matmult on a null tensor");   // _NT_FUNCTIONAL_ALWAYS_CHECK_
+    utils::throw_exception(a_in.dims() > 1 && b_in.dims() > 1,
+                           "\nRuntimeError: Expected tensors to have dims greater than 1, but instead had dims of " +
+                               std::to_string(a_in.dims()) + " and " + std::to_string(b_in.dims()));
+    utils::throw_exception(a_in.dtype() == b_in.dtype(), std::string("Expected both tensors to have the dtype ") + dtype_name(a_in.dtype()) +
+                                                             " but got " + dtype_name(a_in.dtype()) + " and " + dtype_name(b_in.dtype()));   // :868
+    utils::throw_exception(dtype_size(a_in.dtype()) > 0, std::string("dtype ") + dtype_name(a_in.dtype()) + " has no matmult on this backend");
+    MatmultPlan p;
+    p.ta = trans_a; p.tb = trans_b;
+    p.a = matrix_storage(a_in, p.ta);
+    p.b = matrix_storage(b_in, p.tb);
+    const SizeRef& as = p.a.shape();
+    const SizeRef& bs = p.b.shape();
+    const int64_t ar = as[as.size() - 2], ac = as[as.size() - 1], br = bs[bs.size() - 2], bc = bs[bs.size() - 1];
+    p.m = p.ta ? ac : ar;
+    p.k = p.ta ? ar : ac;
+    const int64_t kb = p.tb ? bc : br;
+    p.n = p.tb ? br : bc;
+    utils::throw_exception(p.k == kb, "Expected dimensions -2 and -1 of shapes (" + shape_str(a_in.shape()) + "," + shape_str(b_in.shape()) +
+                                          ") to be equal for matrix multiplication");   // determine_transposes, :73-90
+    const size_t abd = as.size() - 2, bbd = bs.size() - 2;
+    const SizeRef& big = abd >= bbd ? as : bs;
+    const SizeRef& small = abd >= bbd ? bs : as;
+    const size_t bigd = std::max(abd, bbd), smalld = std::min(abd, bbd);
+    for (size_t i = 0; i < smalld; ++i)
+        utils::throw_exception(big[bigd - smalld + i] == small[i], "Cannot multiply tensors of shapes " + shape_str(a_in.shape()) + " and " +
+                                                                       shape_str(b_in.shape()) + ", outter dimensions do not match");   // :870-872
+    if (out_variant && bbd > abd)
+        utils::throw_exception(!p.ta && !p.tb, "Transposing a and b are not currently supported for tensors of tensors, run "
+                                               "transpose_Tensors(-1, -2).clone(), and then run matrix multiplication over the tensors");   // :952
+    p.nbig = prod(big, 0, bigd);
+    p.na = prod(as, 0, abd);
+    p.nb = prod(bs, 0, bbd);
+    p.out_shape.assign(big.begin(), big.begin() + (long)bigd);
+    p.out_shape.push_back(p.m);
+    p.out_shape.push_back(p.n);
+    return p;
+}
+
+static void run_plan(const MatmultPlan& p, Tensor& c) {
+    if (p.nbig == 0 || p.m == 0 || p.n == 0 || p.k == 0) return;
+    const int64_t es = dtype_size(p.a.dtype());
+    const int dt = static_cast<int>(p.a.dtype());
+    const char* A = static_cast<const char*>(p.a.data_ptr());
+    const char* B = static_cast<const char*>(p.b.data_ptr());
+    char* C = static_cast<char*>(c.data_ptr());
+    if (p.nbig == 1) {
+        check_status(ntg_matmult(dt, A, B, C, p.m, p.k, p.k, p.n, p.ta, p.tb));
+        return;
+    }
+    // item i of the higher-rank operand pairs with item i mod count of the lower-rank one: the
+    // reference repeats the HANDLES (smaller.repeat_, :883), so the pointer tables simply repeat
+    std::vector<const void*> pa((size_t)p.nbig), pb((size_t)p.nbig);
+    std::vector<void*> pc((size_t)p.nbig);
+    for (int64_t i = 0; i < p.nbig; ++i) {
+        pa[(size_t)i] = A + (i % p.na) * p.m * p.k * es;
+        pb[(size_t)i] = B + (i % p.nb) * p.k * p.n * es;
+        pc[(size_t)i] = C + i * p.m * p.n * es;
+    }
+    check_status(ntg_matmult_batch(dt, pa.data(), pb.data(), pc.data(), p.nbig, p.m, p.k, p.k, p.n, p.ta, p.tb));
+}
+
+Tensor matmult(const Tensor& a, const Tensor& b, bool trans_a, bool trans_b) {
+    MatmultPlan p = plan_matmult(a, b, trans_a, trans_b, false);
+    Tensor c = zeros(p.out_shape, a.dtype());      // matmult_cpu.cpp:110, :707
+    run_plan(p, c);
+    return c;
+}
+
+Tensor& matmult(const Tensor& a, const Tensor& b, Tensor& c, bool trans_a, bool trans_b) {
+    utils::throw_exception(!c.is_null(), "Cannot perform operation matmult on a null tensor");
+    utils::throw_exception(c.is_mutable(), "Output from Matmult must be mutable");   // tensor_files/matmult.cpp:21
+    MatmultPlan p = plan_matmult(a, b, trans_a, trans_b, true);
+    const SizeRef& cs = c.shape();
+    const bool same = cs == p.out_shape;
+    const bool same_numel = c.dims() >= 2 && c.numel() == p.nbig * p.m * p.n && cs[cs.size() - 2] == p.m && cs[cs.size() - 1] == p.n;
+    utils::throw_exception(same || (p.nbig > 1 && same_numel), "Got invalid shape for output tensor " + shape_str(cs) + " expected " +
+                                                                   shape_str(p.out_shape));                                         // :137-139, :807-812
+    utils::throw_exception(c.is_contiguous(), "Expected output tensor for matrix multiplication to be contiguous");             // :140
+    utils::throw_exception(c.dtype() == a.dtype(), std::string("Expected dtype ") + dtype_name(a.dtype()) +
+                                                       " for output matrix multiplication, C dtype inputted was " + dtype_name(c.dtype()));   // :141-143
+    run_plan(p, c);                                // accumulates: C += op(a).op(b)
+    return c;
+}
+
+Tensor matmult_cT(const Tensor& a, const Tensor& b) { return functional::matmult(a, b, false, true); }   // tensor_files/matmult.cpp:38
+
+Tensor linear(const Tensor& x_in, const Tensor& w_in, const Tensor& b_in, bool trans_a, bool trans_b) {
+    utils::throw_exception(!x_in.is_null() && !w_in.is_null() && !b_in.is_null(), "Cannot perform operation linear on a null tensor");
+    utils::throw_exception(x_in.dtype() == w_in.dtype() && x_in.dtype() == b_in.dtype(), "linear expects input, weight and bias of one dtype");
+    const int64_t nd = std::max({x_in.dims(), w_in.dims(), b_in.dims()});
+    utils::throw_exception(nd >= 2, "Cannot perform matrix multiplication with dimensions less than 2 got " + std::to_string(nd) +
+                                        " for tensor dimensions");
+    // unsqueeze_as (matmult_cpu.cpp:1712-1713)
+    Tensor x = x_in.unsqueeze_front(nd - x_in.dims()), w = w_in.unsqueeze_front(nd - w_in.dims());
+    Tensor b = b_in.contiguous().unsqueeze_front(nd - b_in.dims());
+    auto strip = [](const Tensor& t) {   // leading batch dims of 1 are dropped (:1693-1696)
+        SizeRef s = t.shape();
+        size_t drop = 0;
+        while (s.size() - drop > 2 && s[drop] == 1) ++drop;
+        SizeRef ns(s.begin() + (long)drop, s.end());
+        if (t.is_contiguous()) return t.view(ns);
+        return t.clone().view(ns);
+    };
+    x = strip(x);
+    w = strip(w);
+    MatmultPlan p = plan_matmult(x, w, trans_a, trans_b, false);
+    const SizeRef& bs = b.shape();
+    const int64_t brow = bs[bs.size() - 2], bcol = bs[bs.size() - 1];
+    utils::throw_exception(brow == p.m || brow == 1, "Got invalid shape for bias (" + shape_str(b_in.shape()) +
+                                                         ") to linear function expected rows to be 1 or " + std::to_string(p.m));    // :1629-1631
+    utils::throw_exception(bcol == p.n || bcol == 1, "Got invalid shape for bias (" + shape_str(b_in.shape()) +
+                                                         ") to linear function expected cols to be 1 or " + std::to_string(p.n));    // :1632-1634
+    SizeRef bb(bs.begin(), bs.end() - 2);
+    while (!bb.empty() && bb[0] == 1) bb.erase(bb.begin());
+    const size_t obd = p.out_shape.size() - 2;
+    utils::throw_exception(bb.size() <= obd, "Error, invalid batch shapes for linear: (" + shape_str(x_in.shape()) + ", " +
+                                                 shape_str(w_in.shape()) + ", " + shape_str(b_in.shape()) + ")");
+    for (size_t i = 0; i < bb.size(); ++i)
+        utils::throw_exception(bb[i] == p.out_shape[obd - bb.size() + i], "Error, invalid batch shapes for linear: (" + shape_str(x_in.shape()) +
+                                                                              ", " + shape_str(w_in.shape()) + ", " + shape_str(b_in.shape()) + ")");
+    const int64_t nbias = prod(bb);
+    Tensor c(p.out_shape, x.dtype());
+    if (p.nbig == 0 || p.m == 0 || p.n == 0) return c;
+    const int64_t es = dtype_size(x.dtype());
+    const int dt = static_cast<int>(x.dtype());
+    // bias broadcast to the output is the initial accumulator (:1637-1647); fused on the device
+    for (int64_t i = 0; i < p.nbig; ++i) {
+        check_status(ntg_linear(dt, static_cast<const char*>(p.a.data_ptr()) + (i % p.na) * p.m * p.k * es,
+                                static_cast<const char*>(p.b.data_ptr()) + (i % p.nb) * p.k * p.n * es,
+                                static_cast<const char*>(b.data_ptr()) + (i % nbias) * brow * bcol * es,
+                                static_cast<char*>(c.data_ptr()) + i * p.m * p.n * es, p.m, p.k, p.n, p.ta, p.tb, brow, bcol));
+    }
+    return c;
+}
+
+MatmultGrads matmult_backward(const Tensor& a, const Tensor& b, const Tensor& grad, bool trans_a, bool trans_b) {
+    // nn/functional/matmult.cpp:37-62
+    MatmultGrads g;
+    g.da = trans_a ? functional::matmult(b, grad, trans_b, true) : functional::matmult(grad, b, false, !trans_b);
+    g.db = trans_b ? functional::matmult(grad, a, true, trans_a) : functional::matmult(a, grad, !trans_a, false);
+    if (g.da.shape() != a.shape()) g.da = g.da.sum_leading(a.shape());     // accumulate_gradient's broadcast reduction
+    if (g.db.shape() != b.shape()) g.db = g.db.sum_leading(b.shape());
+    return g;
+}
+
+LinearGrads linear_backward(const Tensor& x, const Tensor& w, const Tensor& bias, const Tensor& grad, bool trans_a, bool trans_b) {
+    // nn/functional/matmult.cpp:253-275; AutoGrad.cpp:7-25 for the reductions
+    MatmultGrads mg = matmult_backward(x, w, grad, trans_a, trans_b);
+    LinearGrads g;
+    g.dx = mg.da;
+    g.dw = mg.db;
+    g.db = grad.shape() == bias.shape() ? grad.clone() : grad.sum_leading(bias.shape());
+    return g;
+}
+
+static void check_pair_ge(const utils::my_tuple& v, int64_t lo, const std::string& what) {
+    utils::throw_exception(v.first >= lo && v.second >= lo, what);
+}
+
+Tensor unfold2d(const Tensor& x_in, utils::my_tuple k, utils::my_tuple d, utils::my_tuple p, utils::my_tuple s, bool transpose_out) {
+    utils::throw_exception(!x_in.is_null(), "Cannot perform operation unfold2d on a null tensor");
+    utils::throw_exception(x_in.dims() >= 3, "Expected input tensot to unfold to have dims greater than or equal to 3 but got " +
+                                                 std::to_string(x_in.dims()) + "D");
+    Tensor x = x_in.contiguous();
+    const SizeRef& xs = x.shape();
+    const int64_t H = xs[xs.size() - 2], W = xs[xs.size() - 1], C = xs[xs.size() - 3];
+    const int64_t B = x.numel() / std::max<int64_t>(1, C * H * W);
+    const int64_t Lr = (H + 2 * p.first - d.first * (k.first - 1) - 1) / s.first + 1;
+    const int64_t Lc = (W + 2 * p.second - d.second * (k.second - 1) - 1) / s.second + 1;
+    utils::throw_exception(Lr > 0 && Lc > 0 && H + 2 * p.first - d.first * (k.first - 1) - 1 >= 0 && W + 2 * p.second - d.second * (k.second - 1) - 1 >= 0,
+                           "Given input with spatial size (" + std::to_string(H) + ", " + std::to_string(W) +
+                               "), calculated shape of the array of sliding blocks as (" + std::to_string(Lr) + ", " + std::to_string(Lc) +
+                               "), but its components must be at least one.");
+    Tensor col({B, C * k.first * k.second, Lr * Lc}, x.dtype());
+    check_status(ntg_unfold2d(static_cast<int>(x.dtype()), x.data_ptr(), col.data_ptr(), B, C, H, W, k.first, k.second, s.first, s.second,
+                              p.first, p.second, d.first, d.second));
+    if (transpose_out) return col;
+    return col.transpose(-1, -2);
+}
+
+Tensor conv2d(const Tensor& image, const Tensor& kernel, utils::my_tuple s, utils::my_tuple p, utils::my_tuple d, int64_t groups) {
+    utils::throw_exception(!image.is_null() && !kernel.is_null(), "Cannot perform operation conv2d on a null tensor");
+    // conv.cpp:72-79
+    utils::throw_exception(image.dims() >= 3, "Expected to get a 3D or greater tensor as the input for a 2d convolution, but got " +
+                                                  std::to_string(image.dims()) + "D");
+    utils::throw_exception(kernel.dims() == 3 || kernel.dims() == 4, "Expected to get a 4D or 3D tensor as the kernel for a 2d convolution, but got " +
+                                                                         std::to_string(kernel.dims()) + "D");
+    utils::throw_exception(image.dtype() == kernel.dtype(), std::string("Expected both kernel and image to have the same dtype for conv2d but got ") +
+                                                                dtype_name(kernel.dtype()) + " and " + dtype_name(image.dtype()));
+    utils::throw_exception(image.dtype() != DType::Bool && image.dtype() != DType::TensorObj, "Expected to get a number type for image and kernel");
+    check_pair_ge(s, 1, "Conv2d stride cannot be less than 1");
+    check_pair_ge(d, 1, "Conv2d dilation cannot be less than 1");
+    check_pair_ge(p, 0, "Conv2d padding cannot be less than 1");
+    Tensor x = image.contiguous(), w = kernel.contiguous();
+    const SizeRef& xs = x.shape();
+    const int64_t H = xs[xs.size() - 2], W = xs[xs.size() - 1], C = xs[xs.size() - 3];
+    const int64_t B = x.numel() / std::max<int64_t>(1, C * H * W);
+    const SizeRef& ws = w.shape();
+    const int64_t kh = ws[ws.size() - 2], kw = ws[ws.size() - 1], Cg = ws[ws.size() - 3], O = kernel.dims() == 4 ? ws[0] : 1;
+    utils::throw_exception(groups >= 1, "Conv2d groups cannot be less than 1");
+    utils::throw_exception(C % groups == 0, "Expected image channels to be divisible by groups in Conv2d but got " + std::to_string(C) + " % " +
+                                                std::to_string(groups) + " != 0");   // :97
+    utils::throw_exception(Cg * groups == C, "Expected kernel rows times groups to be equal to rows of image Conv2d but got " + std::to_string(Cg) +
+                                                 " * " + std::to_string(groups) + " != " + std::to_string(C));   // :98
+    const int64_t Ro = (H + 2 * p.first - d.first * (kh - 1) - 1) / s.first + 1;
+    const int64_t Co = (W + 2 * p.second - d.second * (kw - 1) - 1) / s.second + 1;
+    utils::throw_exception(Ro > 0 && Co > 0, "conv2d output would be empty");
+    Tensor out({B, O, Ro, Co}, x.dtype());
+    check_status(ntg_conv2d(static_cast<int>(x.dtype()), x.data_ptr(), w.data_ptr(), out.data_ptr(), B, C, H, W, O, kh, kw, s.first, s.second,
+                            p.first, p.second, d.first, d.second, groups));
+    return out;
+}
+
+}  // namespace functional
+
+namespace layers {
+
+Linear::Linear(int64_t in_channels, int64_t out_channels, bool use_bias_, DType dt, uint64_t seed)
+    : use_bias(use_bias_), Weight(functional::randn({in_channels, out_channels}, dt, seed)),
+      Bias(use_bias_ ? functional::randn({out_channels}, dt, seed + 1) : Tensor::Null()) {
+    Weight.set_mutability(false);                  // Linear.cpp:17-19
+    if (use_bias) Bias.set_mutability(false);
+}
+
+Tensor Linear::forward(const Tensor& x) const {
+    if (!use_bias) return functional::matmult(x, Weight);      // TensorGrad linear with a null bias, nn/functional/matmult.cpp:238-241
+    return functional::linear(x, Weight, Bias);
+}
+
+functional::LinearGrads Linear::backward(const Tensor& x, const Tensor& grad) const {
+    if (!use_bias) {
+        functional::MatmultGrads mg = functional::matmult_backward(x, Weight, grad, false, false);
+        return {mg.da, mg.db, Tensor::Null()};
+    }
+    return functional::linear_backward(x, Weight, Bias, grad, false, false);
+}
+
+}  // namespace layers
+}  // namespace nt

@@ -1,0 +1,129 @@
+// nt_compat -- the reference's C++ interface for the dense matmult path, on the gfx950 backend.
+//
+// Mirrors, with the same names, argument meaning and error behaviour:
+//   nt::functional::matmult / matmult_cT / linear   nt/functional/tensor_files/matmult.h:10-13
+//   nt::functional::unfold2d                        nt/functional/tensor_files/colim_transform.cpp:565-588
+//   nt::functional::conv2d                          nt/functional/tensor_files/conv.h:12
+//   nt::matmult / nt::linear / nt::conv2d           nt/nt.h:835-850, 369-517 (positional form of the named-argument facade)
+//   nt::layers::Linear                              nt/nn/layers/Linear.h:10-20
+//   gradient GEMM selection of TensorGrad linear/matmult   nt/nn/functional/matmult.cpp:37-62, 253-275
+//   nt::utils::throw_exception                      nt/utils/utils.h:178-202
+// nt::Tensor is reduced to what the path needs: dtype + shape + strides over ref-counted host
+// storage (contiguous tensors and transposed views).  All arithmetic is done by libntgemm.so
+// through the host-pointer C ABI (include/ntgemm.h); there is no CPU fallback.
+#pragma once
+#include <cstdint>
+#include <initializer_list>
+#include <memory>
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+namespace nt {
+
+// values equal the reference enum (nt/dtype/DType_enum.h:14-20); BFloat16 / uint64 are this backend's extensions
+enum class DType : int {
+    Float16 = 0, Float32 = 1, Float64 = 2, Float128 = 3, Complex32 = 4, Complex64 = 5, Complex128 = 6,
+    int8 = 7, int16 = 8, int32 = 9, int64 = 10, int128 = 11, uint8 = 12, uint16 = 13, uint32 = 14, uint128 = 15,
+    Bool = 16, TensorObj = 17, BFloat16 = 100, uint64 = 101,
+    Half = Float16, Float = Float32, Double = Float64, Char = int8, Short = int16, Integer = int32, Long = int64, Byte = uint8
+};
+int64_t dtype_size(DType dt);
+const char* dtype_name(DType dt);
+
+namespace utils {
+// thrown by every failed check; derives from std::exception like the reference's errors (test_macros.h:89)
+struct nt_error : std::runtime_error { using std::runtime_error::runtime_error; };
+void throw_exception(bool ok, const std::string& message);
+using my_tuple = std::pair<int64_t, int64_t>;
+}  // namespace utils
+
+using SizeRef = std::vector<int64_t>;
+std::string shape_str(const SizeRef& s);
+
+class Tensor {
+public:
+    Tensor() = default;                                           // null tensor
+    Tensor(SizeRef shape, DType dt);                              // uninitialised contiguous tensor
+    static Tensor Null() { return Tensor(); }
+
+    bool is_null() const { return !storage_; }
+    const SizeRef& shape() const { return shape_; }
+    const SizeRef& strides() const { return strides_; }
+    int64_t dims() const { return (int64_t)shape_.size(); }
+    int64_t numel() const;
+    DType dtype() const { return dtype_; }
+    void* data_ptr() { return storage_.get() + offset_; }
+    const void* data_ptr() const { return storage_.get() + offset_; }
+    bool is_contiguous() const;
+    bool is_mutable() const { return mutable_; }
+    Tensor& set_mutability(bool m) { mutable_ = m; return *this; }
+
+    Tensor clone() const;                                         // contiguous copy
+    Tensor contiguous() const { return is_contiguous() ? *this : clone(); }
+    Tensor view(SizeRef shape) const;                             // contiguous tensors only; one -1 allowed
+    Tensor transpose(int64_t a, int64_t b) const;                 // strided view, no copy
+    Tensor unsqueeze_front(int64_t n) const;                      // prepend n dims of 1
+    Tensor item(int64_t batch_index) const;                       // i-th matrix of a contiguous [.., r, c] tensor
+    Tensor sum_leading(const SizeRef& target_shape) const;        // reduce broadcast dims back (sum_as)
+    template <class T> T* data() { return reinterpret_cast<T*>(data_ptr()); }
+    template <class T> const T* data() const { return reinterpret_cast<const T*>(data_ptr()); }
+
+private:
+    std::shared_ptr<char> storage_;
+    int64_t offset_ = 0;        // bytes
+    SizeRef shape_, strides_;   // strides in elements
+    DType dtype_ = DType::Float32;
+    bool mutable_ = true;
+};
+
+namespace functional {
+Tensor zeros(SizeRef shape, DType dt = DType::Float32);
+Tensor randn(SizeRef shape, DType dt = DType::Float32, uint64_t seed = 0);   // seeded N(0,1) (the reference's randn is unseeded)
+Tensor from_numpy(const std::string& path);                                   // .npy, C order, f2/f4/f8/i1/i2/i4/i8/u1
+bool allclose(const Tensor& a, const Tensor& b, double rtol = 1e-5, double atol = 1e-8);   // compare.h:34
+
+Tensor matmult(const Tensor& a, const Tensor& b, bool trans_a = false, bool trans_b = false);
+Tensor& matmult(const Tensor& a, const Tensor& b, Tensor& c, bool trans_a = false, bool trans_b = false);
+Tensor matmult_cT(const Tensor& a, const Tensor& b);
+Tensor linear(const Tensor& input, const Tensor& weight, const Tensor& bias, bool trans_input = false, bool trans_weight = false);
+Tensor unfold2d(const Tensor& x, utils::my_tuple kernel_size, utils::my_tuple dilation = {1, 1}, utils::my_tuple padding = {0, 0},
+                utils::my_tuple stride = {1, 1}, bool transpose_out = true);
+Tensor conv2d(const Tensor& image, const Tensor& kernel, utils::my_tuple stride = {1, 1}, utils::my_tuple padding = {0, 0},
+              utils::my_tuple dilation = {1, 1}, int64_t groups = 1);
+
+// what the backward lambdas of TensorGrad matmult / linear compute (flags only, no transposed copies)
+struct MatmultGrads { Tensor da, db; };
+MatmultGrads matmult_backward(const Tensor& a, const Tensor& b, const Tensor& grad, bool trans_a, bool trans_b);
+struct LinearGrads { Tensor dx, dw, db; };
+LinearGrads linear_backward(const Tensor& x, const Tensor& w, const Tensor& bias, const Tensor& grad, bool trans_a, bool trans_b);
+}  // namespace functional
+
+// positional forms of the named-argument facade (nt.h:835-850)
+inline Tensor matmult(const Tensor& input, const Tensor& other, bool transpose_a = false, bool transpose_b = false) {
+    return functional::matmult(input, other, transpose_a, transpose_b);
+}
+inline Tensor& matmult(const Tensor& input, const Tensor& other, Tensor& out, bool transpose_a = false, bool transpose_b = false) {
+    return functional::matmult(input, other, out, transpose_a, transpose_b);
+}
+inline Tensor linear(const Tensor& input, const Tensor& weight, const Tensor& bias, bool transpose_a = false, bool transpose_b = false) {
+    return functional::linear(input, weight, bias, transpose_a, transpose_b);
+}
+inline Tensor conv2d(const Tensor& image, const Tensor& kernel, utils::my_tuple stride = {1, 1}, utils::my_tuple padding = {0, 0},
+                     utils::my_tuple dilation = {1, 1}, int64_t groups = 1) {
+    return functional::conv2d(image, kernel, stride, padding, dilation, groups);
+}
+
+namespace layers {
+// Weight [in, out], Bias [out]; forward = linear(x, Weight, Bias) (Linear.cpp:10-24)
+class Linear {
+public:
+    Linear(int64_t in_channels, int64_t out_channels, bool use_bias = true, DType dt = DType::Float32, uint64_t seed = 1);
+    Tensor forward(const Tensor& x) const;
+    functional::LinearGrads backward(const Tensor& x, const Tensor& grad) const;
+    bool use_bias;
+    Tensor Weight, Bias;
+};
+}  // namespace layers
+
+}  // namespace nt

@@ -1,0 +1,253 @@
+// Replays the reference's own tests for the matmult path against the nt_compat facade:
+//   tests/src/matmult_test.cpp:10-107 (matmult shapes), :108-189 (batched == per item, bitwise),
+//   :194-307 (linear shapes), tests/src/linear_autograd_test.cpp:126-148 (golden grads),
+//   tests/src/conv_autograd_test.cpp:250-371 (golden conv2d outputs), col_im_autograd_test.cpp:77-95.
+// Same structure as the reference's runner (tests/src/test_macros.h:69-93): each case is a lambda,
+// a thrown exception fails the case.  `--host-only` runs the cases that never reach the device
+// (argument validation must fail BEFORE any device work).  Usage: nt_compat_tests <golden dir> [--host-only]
+#include "../../neurotensor_amd/nt_compat/nt_compat.h"
+
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+#include <functional>
+#include <string>
+
+static int g_failed = 0, g_run = 0;
+
+static void run_test(const char* name, const std::function<void()>& fn) {
+    ++g_run;
+    try {
+        fn();
+        std::printf("[ok]   %s\n", name);
+    } catch (const std::exception& e) {
+        ++g_failed;
+        std::printf("[FAIL] %s: %s\n", name, e.what());
+    }
+}
+
+static void expect_throw(const char* name, const std::function<void()>& fn) {
+    run_test(name, [&] {
+        bool threw = false;
+        try { fn(); } catch (const nt::utils::nt_error&) { threw = true; }
+        nt::utils::throw_exception(threw, "expected an exception");
+    });
+}
+
+using nt::DType;
+using nt::SizeRef;
+using nt::Tensor;
+namespace F = nt::functional;
+
+// double-precision reference of op(a).op(b) for contiguous 2-D float tensors
+static double max_err_vs_double(const Tensor& a, const Tensor& b, const Tensor& c, bool ta, bool tb, const float* c0 = nullptr) {
+    const int64_t ar = a.shape()[0], ac = a.shape()[1], bc = b.shape()[1], br = b.shape()[0];
+    const int64_t m = ta ? ac : ar, k = ta ? ar : ac, n = tb ? br : bc;
+    double worst = 0;
+    for (int64_t i = 0; i < m; ++i)
+        for (int64_t j = 0; j < n; ++j) {
+            double s = c0 ? c0[i * n + j] : 0.0;
+            for (int64_t t = 0; t < k; ++t) {
+                const double av = ta ? a.data<float>()[t * ac + i] : a.data<float>()[i * ac + t];
+                const double bv = tb ? b.data<float>()[j * bc + t] : b.data<float>()[t * bc + j];
+                s += av * bv;
+            }
+            worst = std::fmax(worst, std::fabs(s - c.data<float>()[i * n + j]));
+        }
+    return worst;
+}
+
+static void shape_case(const char* name, SizeRef as, SizeRef bs, bool ta, bool tb, SizeRef expect) {
+    run_test(name, [&] {
+        Tensor a = F::randn(as, DType::Float32, 11), b = F::randn(bs, DType::Float32, 12);
+        Tensor o = nt::matmult(a, b, ta, tb);
+        nt::utils::throw_exception(o.shape() == expect, "Error: Got unexpected shape for (" + nt::shape_str(as) + ") (" + nt::shape_str(bs) +
+                                                            ") = (" + nt::shape_str(o.shape()) + ")");
+        // values: first and last item against a double-precision loop
+        const int64_t items = o.numel() / (expect[expect.size() - 1] * expect[expect.size() - 2]);
+        Tensor ac = a.contiguous(), bc = b.contiguous();
+        const int64_t na = ac.numel() / (as[as.size() - 1] * as[as.size() - 2]), nb = bc.numel() / (bs[bs.size() - 1] * bs[bs.size() - 2]);
+        for (int64_t i : {int64_t(0), items - 1}) {
+            const double err = max_err_vs_double(ac.item(i % na), bc.item(i % nb), o.item(i), ta, tb);
+            nt::utils::throw_exception(err <= 1e-3, "values differ from the double-precision loop by " + std::to_string(err));
+        }
+    });
+}
+
+static void linear_shape_case(const char* name, SizeRef as, SizeRef bs, SizeRef bis, bool ta, bool tb, SizeRef expect) {
+    run_test(name, [&] {
+        Tensor a = F::randn(as, DType::Float32, 21), b = F::randn(bs, DType::Float32, 22), bi = F::randn(bis, DType::Float32, 23);
+        Tensor o = nt::linear(a, b, bi, ta, tb);
+        nt::utils::throw_exception(o.shape() == expect, "Error: Got unexpected shape (" + nt::shape_str(o.shape()) + ")");
+        // linear == matmult + broadcast bias (bias is the initial accumulator)
+        Tensor mm = nt::matmult(a, b, ta, tb);
+        const int64_t n = expect[expect.size() - 1], m = expect[expect.size() - 2];
+        const int64_t brow = bis.size() >= 2 ? bis[bis.size() - 2] : 1, bcol = bis[bis.size() - 1];
+        for (int64_t i = 0; i < o.numel(); ++i) {
+            const int64_t r = (i / n) % m, c = i % n;
+            const float want = mm.data<float>()[i] + bi.data<float>()[(brow == 1 ? 0 : r) * bcol + (bcol == 1 ? 0 : c)];
+            nt::utils::throw_exception(std::fabs(want - o.data<float>()[i]) <= 1e-3, "linear != matmult + bias at " + std::to_string(i));
+        }
+    });
+}
+
+static void host_only_cases() {
+    expect_throw("matmult inner sizes differ", [] { nt::matmult(F::zeros({4, 5}), F::zeros({4, 5})); });
+    expect_throw("matmult inner sizes differ with flags", [] { nt::matmult(F::zeros({4, 5}), F::zeros({4, 6}), true, true); });
+    expect_throw("matmult 1-D operand", [] { nt::matmult(F::zeros({5}), F::zeros({5, 5})); });
+    expect_throw("matmult dtype mismatch", [] { nt::matmult(F::zeros({4, 4}), F::zeros({4, 4}, DType::Float64)); });
+    expect_throw("matmult batch dims do not line up", [] { nt::matmult(F::zeros({2, 3, 4, 4}), F::zeros({2, 4, 4})); });
+    expect_throw("matmult null operand", [] { nt::matmult(Tensor::Null(), F::zeros({4, 4})); });
+    expect_throw("matmult unsupported dtype", [] { Tensor t; nt::matmult(Tensor({2, 2}, DType::Complex64), Tensor({2, 2}, DType::Complex64)); });
+    expect_throw("matmult out wrong shape", [] { Tensor c = F::zeros({4, 5}); nt::matmult(F::zeros({4, 4}), F::zeros({4, 4}), c); });
+    expect_throw("matmult out wrong dtype", [] { Tensor c = F::zeros({4, 4}, DType::Float64); nt::matmult(F::zeros({4, 4}), F::zeros({4, 4}), c); });
+    expect_throw("matmult out immutable", [] { Tensor c = F::zeros({4, 4}); c.set_mutability(false); nt::matmult(F::zeros({4, 4}), F::zeros({4, 4}), c); });
+    expect_throw("matmult out not contiguous", [] { Tensor c = F::zeros({4, 4}).transpose(0, 1); nt::matmult(F::zeros({4, 4}), F::zeros({4, 4}), c); });
+    expect_throw("matmult out with flags on lower-rank a", [] { Tensor c = F::zeros({3, 4, 4}); nt::matmult(F::zeros({4, 4}), F::zeros({3, 4, 4}), c, true, false); });
+    expect_throw("linear bias rows", [] { nt::linear(F::zeros({4, 5}), F::zeros({5, 6}), F::zeros({2, 6})); });
+    expect_throw("linear bias cols", [] { nt::linear(F::zeros({4, 5}), F::zeros({5, 6}), F::zeros({5})); });
+    expect_throw("conv2d kernel dims", [] { nt::conv2d(F::zeros({1, 3, 8, 8}), F::zeros({3, 3})); });
+    expect_throw("conv2d groups", [] { nt::conv2d(F::zeros({1, 3, 8, 8}), F::zeros({4, 3, 3, 3}), {1, 1}, {0, 0}, {1, 1}, 2); });
+    expect_throw("conv2d stride", [] { nt::conv2d(F::zeros({1, 3, 8, 8}), F::zeros({4, 3, 3, 3}), {0, 1}); });
+    expect_throw("unfold2d empty", [] { F::unfold2d(F::zeros({1, 1, 2, 2}), {5, 5}); });
+    run_test("tensor views", [] {
+        Tensor a = F::randn({3, 4, 5}, DType::Float32, 5);
+        Tensor t = a.transpose(-1, -2);
+        nt::utils::throw_exception(!t.is_contiguous() && t.shape() == SizeRef({3, 5, 4}), "transpose view");
+        Tensor c = t.clone();
+        nt::utils::throw_exception(c.is_contiguous() && c.data<float>()[1] == a.data<float>()[5], "clone of a strided view");
+        nt::utils::throw_exception(F::allclose(c.transpose(-1, -2), a), "double transpose");
+        Tensor s = a.sum_leading({5});
+        float want = 0;
+        for (int i = 0; i < 12; ++i) want += a.data<float>()[i * 5 + 2];
+        nt::utils::throw_exception(std::fabs(s.data<float>()[2] - want) < 1e-5, "sum_as");
+    });
+}
+
+static void device_cases(const std::string& g) {
+    shape_case("matmult 2d", {30, 30}, {30, 30}, false, false, {30, 30});
+    shape_case("matmult 2d Ta", {30, 14}, {30, 30}, true, false, {14, 30});
+    shape_case("matmult 2d Tb", {30, 30}, {14, 30}, false, true, {30, 14});
+    shape_case("matmult 2d T(a, b)", {30, 14}, {14, 30}, true, true, {14, 14});
+    shape_case("matmult 3d", {10, 30, 30}, {10, 30, 30}, false, false, {10, 30, 30});
+    shape_case("matmult 3d Ta", {10, 30, 14}, {10, 30, 30}, true, false, {10, 14, 30});
+    shape_case("matmult 3d Tb", {10, 30, 30}, {10, 14, 30}, false, true, {10, 30, 14});
+    shape_case("matmult 3d T(a, b)", {10, 30, 14}, {10, 14, 30}, true, true, {10, 14, 14});
+    shape_case("matmult 3d bigger A", {5, 10, 30, 30}, {10, 30, 30}, false, false, {5, 10, 30, 30});
+    shape_case("matmult 3d Ta bigger A", {5, 10, 30, 14}, {10, 30, 30}, true, false, {5, 10, 14, 30});
+    shape_case("matmult 3d Tb bigger A", {5, 10, 30, 30}, {10, 14, 30}, false, true, {5, 10, 30, 14});
+    shape_case("matmult 3d T(a, b) bigger A", {5, 10, 30, 14}, {10, 14, 30}, true, true, {5, 10, 14, 14});
+    shape_case("matmult 3d bigger B", {10, 30, 30}, {5, 10, 30, 30}, false, false, {5, 10, 30, 30});
+    shape_case("matmult 3d Ta bigger B", {10, 30, 14}, {5, 10, 30, 30}, true, false, {5, 10, 14, 30});
+    shape_case("matmult 3d Tb bigger B", {10, 30, 30}, {5, 10, 14, 30}, false, true, {5, 10, 30, 14});
+    shape_case("matmult 3d T(a, b) bigger B", {10, 30, 14}, {5, 10, 14, 30}, true, true, {5, 10, 14, 14});
+
+    run_test("matmult batched == per item (bitwise)", [] {
+        Tensor a = F::randn({5, 2, 3, 4}, DType::Float32, 31), b = F::randn({5, 2, 4, 3}, DType::Float32, 32);
+        Tensor o = nt::matmult(a, b);
+        for (int64_t i = 0; i < 10; ++i) {
+            Tensor oi = nt::matmult(a.item(i).clone(), b.item(i).clone());
+            nt::utils::throw_exception(std::memcmp(oi.data_ptr(), o.item(i).data_ptr(), 9 * sizeof(float)) == 0, "item differs");
+        }
+    });
+    run_test("matmult transposed view == flag (no copy)", [] {
+        Tensor a = F::randn({6, 40, 30}, DType::Float32, 33), b = F::randn({6, 20, 30}, DType::Float32, 34);
+        Tensor o1 = nt::matmult(a, b, false, true);
+        Tensor o2 = nt::matmult(a, b.transpose(-1, -2));
+        nt::utils::throw_exception(std::memcmp(o1.data_ptr(), o2.data_ptr(), (size_t)o1.numel() * 4) == 0, "view and flag disagree");
+    });
+    run_test("matmult out= accumulates", [] {
+        Tensor a = F::randn({33, 17}, DType::Float32, 35), b = F::randn({17, 29}, DType::Float32, 36);
+        Tensor c0 = F::randn({33, 29}, DType::Float32, 37), c = c0.clone();
+        nt::matmult(a, b, c);
+        nt::utils::throw_exception(max_err_vs_double(a, b, c, false, false, c0.data<float>()) <= 1e-3, "C += A.B");
+    });
+    run_test("matmult int32 / float64 / int64 values", [] {
+        Tensor a = F::randn({19, 23}, DType::int32, 41), b = F::randn({23, 7}, DType::int32, 42);
+        Tensor o = nt::matmult(a, b);
+        for (int64_t i = 0; i < 19; ++i)
+            for (int64_t j = 0; j < 7; ++j) {
+                int64_t s = 0;
+                for (int64_t t = 0; t < 23; ++t) s += (int64_t)a.data<int32_t>()[i * 23 + t] * b.data<int32_t>()[t * 7 + j];
+                nt::utils::throw_exception(o.data<int32_t>()[i * 7 + j] == (int32_t)s, "int32 result not exact");
+            }
+        Tensor x = F::randn({12, 40}, DType::Float64, 43), y = F::randn({40, 9}, DType::Float64, 44);
+        Tensor z = nt::matmult(x, y);
+        double worst = 0;
+        for (int64_t i = 0; i < 12; ++i)
+            for (int64_t j = 0; j < 9; ++j) {
+                double s = 0;
+                for (int64_t t = 0; t < 40; ++t) s += x.data<double>()[i * 40 + t] * y.data<double>()[t * 9 + j];
+                worst = std::fmax(worst, std::fabs(s - z.data<double>()[i * 9 + j]));
+            }
+        nt::utils::throw_exception(worst <= 1e-12, "float64 result off by " + std::to_string(worst));
+    });
+
+    linear_shape_case("linear 2d", {30, 30}, {30, 30}, {30}, false, false, {30, 30});
+    linear_shape_case("linear 2d Ta", {30, 14}, {30, 30}, {30}, true, false, {14, 30});
+    linear_shape_case("linear 2d Tb", {30, 30}, {14, 30}, {30, 14}, false, true, {30, 14});
+    linear_shape_case("linear 2d T(a, b)", {30, 14}, {14, 30}, {14, 14}, true, true, {14, 14});
+    linear_shape_case("linear 3d", {10, 30, 30}, {10, 30, 30}, {30, 30}, false, false, {10, 30, 30});
+    linear_shape_case("linear 3d Ta", {10, 30, 14}, {10, 30, 30}, {14, 30}, true, false, {10, 14, 30});
+    linear_shape_case("linear 3d Tb", {10, 30, 30}, {10, 14, 30}, {30, 14}, false, true, {10, 30, 14});
+    linear_shape_case("linear 3d T(a, b)", {10, 30, 14}, {10, 14, 30}, {14, 14}, true, true, {10, 14, 14});
+    linear_shape_case("linear 3d bigger A", {5, 10, 30, 30}, {10, 30, 30}, {30, 30}, false, false, {5, 10, 30, 30});
+    linear_shape_case("linear 3d Ta bigger A", {5, 10, 30, 14}, {10, 30, 30}, {14, 30}, true, false, {5, 10, 14, 30});
+    linear_shape_case("linear 3d Tb bigger A", {5, 10, 30, 30}, {10, 14, 30}, {30, 14}, false, true, {5, 10, 30, 14});
+    linear_shape_case("linear 3d T(a, b) bigger A", {5, 10, 30, 14}, {10, 14, 30}, {14, 14}, true, true, {5, 10, 14, 14});
+    linear_shape_case("linear 3d bigger B", {10, 30, 30}, {5, 10, 30, 30}, {30, 30}, false, false, {5, 10, 30, 30});
+    linear_shape_case("linear 3d Ta bigger B", {10, 30, 14}, {5, 10, 30, 30}, {14, 30}, true, false, {5, 10, 14, 30});
+    linear_shape_case("linear 3d Tb bigger B", {10, 30, 30}, {5, 10, 14, 30}, {30, 14}, false, true, {5, 10, 30, 14});
+    linear_shape_case("linear 3d T(a, b) bigger B", {10, 30, 14}, {5, 10, 14, 30}, {14, 14}, true, true, {5, 10, 14, 14});
+
+    run_test("Linear Autograd test (golden)", [&] {
+        Tensor x = F::from_numpy(g + "/linear_input.npy"), grad = F::from_numpy(g + "/linear_grad.npy");
+        Tensor w = F::from_numpy(g + "/linear_weight.npy"), b = F::from_numpy(g + "/linear_bias.npy");
+        Tensor o = nt::linear(x, w, b, false, true);
+        nt::utils::throw_exception(o.shape() == SizeRef({3, 4, 3}), "forward shape");
+        F::LinearGrads gr = F::linear_backward(x, w, b, grad, false, true);
+        nt::utils::throw_exception(F::allclose(gr.dx, F::from_numpy(g + "/linear_xgrad.npy"), 1e-5, 1e-6) &&
+                                       F::allclose(gr.dw, F::from_numpy(g + "/linear_wgrad.npy"), 1e-5, 1e-6) &&
+                                       F::allclose(gr.db, F::from_numpy(g + "/linear_bgrad.npy"), 1e-5, 1e-6),
+                                   "Error, grads do not match");
+    });
+    run_test("layers::Linear forward/backward", [] {
+        nt::layers::Linear lin(20, 12);
+        Tensor x = F::randn({7, 20}, DType::Float32, 51), gy = F::randn({7, 12}, DType::Float32, 52);
+        Tensor y = lin.forward(x);
+        nt::utils::throw_exception(y.shape() == SizeRef({7, 12}), "forward shape");
+        Tensor mm = nt::matmult(x, lin.Weight);
+        for (int64_t i = 0; i < y.numel(); ++i)
+            nt::utils::throw_exception(std::fabs(y.data<float>()[i] - mm.data<float>()[i] - lin.Bias.data<float>()[i % 12]) <= 1e-4, "forward value");
+        F::LinearGrads gr = lin.backward(x, gy);
+        nt::utils::throw_exception(gr.dx.shape() == x.shape() && gr.dw.shape() == lin.Weight.shape() && gr.db.shape() == lin.Bias.shape(), "grad shapes");
+        nt::utils::throw_exception(max_err_vs_double(gy, lin.Weight, gr.dx, false, true) <= 1e-3, "dX = dY.W^T");
+        nt::utils::throw_exception(max_err_vs_double(x, gy, gr.dw, true, false) <= 1e-3, "dW = X^T.dY");
+    });
+    for (const char* sfx : {"", "_batched", "_grouped", "_grouped_batched"}) {
+        const std::string name = std::string("conv2d golden") + sfx;
+        run_test(name.c_str(), [&] {
+            const bool grouped = std::strstr(sfx, "grouped") != nullptr;
+            Tensor x = F::from_numpy(g + "/conv2d_input" + sfx + ".npy"), w = F::from_numpy(g + "/conv2d_weight" + sfx + ".npy");
+            Tensor want = F::from_numpy(g + "/conv2d_output" + sfx + ".npy");
+            const int64_t pad = grouped ? 0 : 1;
+            Tensor o = nt::conv2d(x, w, {1, 1}, {pad, pad}, {1, 1}, grouped ? 2 : 1);
+            nt::utils::throw_exception(o.shape() == want.shape(), "output shape " + nt::shape_str(o.shape()));
+            nt::utils::throw_exception(F::allclose(o, want, 1e-4, 1e-4), "conv2d output differs from the fixture");
+        });
+    }
+    run_test("unfold2d golden", [&] {
+        Tensor x = F::from_numpy(g + "/unfold_input.npy"), want = F::from_numpy(g + "/unfold_output.npy");
+        Tensor col = F::unfold2d(x, {3, 2}, {1, 2}, {1, 1}, {2, 2}, true);
+        nt::utils::throw_exception(col.shape() == SizeRef({1, 18, 16}) && std::memcmp(col.data_ptr(), want.data_ptr(), 18 * 16 * 4) == 0, "unfold output");
+    });
+}
+
+int main(int argc, char** argv) {
+    if (argc < 2) { std::fprintf(stderr, "usage: %s <golden dir> [--host-only]\n", argv[0]); return 2; }
+    const bool host_only = argc > 2 && std::strcmp(argv[2], "--host-only") == 0;
+    host_only_cases();
+    if (!host_only) device_cases(argv[1]);
+    std::printf("%d cases, %d failed\n", g_run, g_failed);
+    return g_failed ? 1 : 0;
+}
