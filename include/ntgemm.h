@@ -117,6 +117,28 @@ int ntg_conv2d(int dtype, const void* image, const void* kernel, void* out,
                int64_t s_r, int64_t s_c, int64_t p_r, int64_t p_c, int64_t d_r, int64_t d_c,
                int64_t groups);
 
+/* Replaces nt::functional::cpu::unfold2d_backward_ with transpose_out = true (col2im,
+ * nt/functional/cpu/unfold2d_backward.cpp:9-56, :158): image[batch, channels, height, width]
+ * receives the scatter-add of col[batch, channels*k_r*k_c, Ho*Wo]; accumulate != 0 adds to
+ * the incoming image like the reference does, 0 overwrites it. */
+int ntg_unfold2d_backward(int dtype, const void* col, void* image,
+                          int64_t batch, int64_t channels, int64_t height, int64_t width,
+                          int64_t k_r, int64_t k_c, int64_t s_r, int64_t s_c,
+                          int64_t p_r, int64_t p_c, int64_t d_r, int64_t d_c, int accumulate);
+
+/* Replaces the dim == 2 bodies of nt::functional::conv_dimage (conv.cpp:318-346) and
+ * conv_dkernel (conv.cpp:444-471):
+ *   d_image  (+)= col2im( W2d^T . dY_b )                 [batch, channels, height, width]
+ *   d_kernel (+)= sum_b dY_b . col_b^T                   [out_channels, channels/groups, k_r, k_c]
+ * grad_out is dY [batch, out_channels, Ho, Wo].  Either output may be NULL to skip it.
+ * accumulate != 0 adds into the outputs (the reference's += on the gradient tensors). */
+int ntg_conv2d_backward(int dtype, const void* image, const void* kernel, const void* grad_out,
+                        void* d_image, void* d_kernel,
+                        int64_t batch, int64_t channels, int64_t height, int64_t width,
+                        int64_t out_channels, int64_t k_r, int64_t k_c,
+                        int64_t s_r, int64_t s_c, int64_t p_r, int64_t p_c, int64_t d_r, int64_t d_c,
+                        int64_t groups, int accumulate);
+
 /* ------------------------------------------------------------------------------------ */
 /* Device-pointer entry points (buffers already in HBM; asynchronous on `stream`).        */
 /* `stream` is a hipStream_t passed as void*; NULL is the default stream.                 */
@@ -163,6 +185,19 @@ int ntg_conv2d_dev(int dtype, const void* image, const void* kernel, void* out,
                    int64_t out_channels, int64_t k_r, int64_t k_c,
                    int64_t s_r, int64_t s_c, int64_t p_r, int64_t p_c, int64_t d_r, int64_t d_c,
                    int64_t groups, void* stream);
+
+int ntg_unfold2d_backward_dev(int dtype, const void* col, void* image,
+                              int64_t batch, int64_t channels, int64_t height, int64_t width,
+                              int64_t k_r, int64_t k_c, int64_t s_r, int64_t s_c,
+                              int64_t p_r, int64_t p_c, int64_t d_r, int64_t d_c, int accumulate, void* stream);
+
+/* workspace: ntg_conv2d_workspace_bytes (one im2col-sized buffer, used for col and then d_col) */
+int ntg_conv2d_backward_dev(int dtype, const void* image, const void* kernel, const void* grad_out,
+                            void* d_image, void* d_kernel, void* workspace, int64_t workspace_bytes,
+                            int64_t batch, int64_t channels, int64_t height, int64_t width,
+                            int64_t out_channels, int64_t k_r, int64_t k_c,
+                            int64_t s_r, int64_t s_c, int64_t p_r, int64_t p_c, int64_t d_r, int64_t d_c,
+                            int64_t groups, int accumulate, void* stream);
 
 #ifdef __cplusplus
 }

@@ -58,6 +58,11 @@ hipError_t launch_unfold2d(int64_t elem_size, const void* im, void* col,
                            int64_t k_r, int64_t k_c, int64_t s_r, int64_t s_c,
                            int64_t p_r, int64_t p_c, int64_t d_r, int64_t d_c, hipStream_t s);
 
+hipError_t launch_col2im(int dtype, const void* col, void* im,
+                         int64_t batch, int64_t channels, int64_t height, int64_t width,
+                         int64_t k_r, int64_t k_c, int64_t s_r, int64_t s_c,
+                         int64_t p_r, int64_t p_c, int64_t d_r, int64_t d_c, int accumulate, hipStream_t s);
+
 #ifdef __HIPCC__
 // Workgroup ids are dealt round-robin to the 8 XCDs; make the ids that land on one
 // XCD (its own L2) a contiguous range of logical tile ids.

@@ -405,4 +405,149 @@ int ntg_conv2d(int dtype, const void* image, const void* kernel, void* out,
     return NTG_OK;
 }
 
+int ntg_unfold2d_backward_dev(int dtype, const void* col, void* image,
+                              int64_t batch, int64_t channels, int64_t height, int64_t width,
+                              int64_t k_r, int64_t k_c, int64_t s_r, int64_t s_c,
+                              int64_t p_r, int64_t p_c, int64_t d_r, int64_t d_c, int accumulate, void* stream) {
+    const int64_t es = ntg::elem_size(dtype);
+    if (es == 0) return fail(NTG_ERR_UNSUPPORTED_DTYPE, "dtype %d is not supported", dtype);
+    if (batch < 0 || channels < 0 || height < 0 || width < 0) return fail(NTG_ERR_INVALID_ARGUMENT, "negative size");
+    int64_t Ho, Wo;
+    int rc = unfold_out(height, width, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c, Ho, Wo);
+    if (rc) return rc;
+    if (batch == 0 || channels == 0) return NTG_OK;
+    if (!col || !image) return fail(NTG_ERR_INVALID_ARGUMENT, "null pointer");
+    hipError_t e = ntg::launch_col2im(dtype, col, image, batch, channels, height, width, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c,
+                                      accumulate, static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return hip_fail(e, "col2im launch");
+    return NTG_OK;
+}
+
+int ntg_unfold2d_backward(int dtype, const void* col, void* image,
+                          int64_t batch, int64_t channels, int64_t height, int64_t width,
+                          int64_t k_r, int64_t k_c, int64_t s_r, int64_t s_c,
+                          int64_t p_r, int64_t p_c, int64_t d_r, int64_t d_c, int accumulate) {
+    const int64_t es = ntg::elem_size(dtype);
+    if (es == 0) return fail(NTG_ERR_UNSUPPORTED_DTYPE, "dtype %d is not supported", dtype);
+    if (batch < 0 || channels < 0 || height < 0 || width < 0) return fail(NTG_ERR_INVALID_ARGUMENT, "negative size");
+    int64_t Ho, Wo;
+    int rc = unfold_out(height, width, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c, Ho, Wo);
+    if (rc) return rc;
+    if (batch == 0 || channels == 0) return NTG_OK;
+    if (!col || !image) return fail(NTG_ERR_INVALID_ARGUMENT, "null pointer");
+    const size_t im_bytes = (size_t)(batch * channels * height * width * es);
+    const size_t col_bytes = (size_t)(batch * channels * k_r * k_c * Ho * Wo * es);
+    DeviceMem mem;
+    const size_t oc = align_up(im_bytes, 256);
+    HIP_TRY(mem.alloc(oc + col_bytes));
+    if (accumulate) HIP_TRY(hipMemcpy(mem.at(0), image, im_bytes, hipMemcpyHostToDevice));
+    HIP_TRY(hipMemcpy(mem.at(oc), col, col_bytes, hipMemcpyHostToDevice));
+    rc = ntg_unfold2d_backward_dev(dtype, mem.at(oc), mem.at(0), batch, channels, height, width, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c,
+                                   accumulate, nullptr);
+    if (rc) return rc;
+    HIP_TRY(hipStreamSynchronize(nullptr));
+    HIP_TRY(hipMemcpy(image, mem.at(0), im_bytes, hipMemcpyDeviceToHost));
+    return NTG_OK;
+}
+
+int ntg_conv2d_backward_dev(int dtype, const void* image, const void* kernel, const void* grad_out,
+                            void* d_image, void* d_kernel, void* workspace, int64_t workspace_bytes,
+                            int64_t batch, int64_t channels, int64_t height, int64_t width,
+                            int64_t out_channels, int64_t k_r, int64_t k_c,
+                            int64_t s_r, int64_t s_c, int64_t p_r, int64_t p_c, int64_t d_r, int64_t d_c,
+                            int64_t groups, int accumulate, void* stream) {
+    const int64_t es = ntg::elem_size(dtype);
+    if (es == 0) return fail(NTG_ERR_UNSUPPORTED_DTYPE, "dtype %d is not supported", dtype);
+    if (batch < 0 || channels < 0 || out_channels < 0 || height < 0 || width < 0) return fail(NTG_ERR_INVALID_ARGUMENT, "negative size");
+    if (groups < 1 || channels % groups != 0 || out_channels % groups != 0)
+        return fail(NTG_ERR_INVALID_ARGUMENT, "channels (%lld) and out channels (%lld) must be divisible by groups (%lld)",
+                    (long long)channels, (long long)out_channels, (long long)groups);
+    int64_t Ho, Wo;
+    int rc = unfold_out(height, width, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c, Ho, Wo);
+    if (rc) return rc;
+    if (batch == 0 || out_channels == 0 || channels == 0) return NTG_OK;
+    if (!kernel || !grad_out || (d_kernel && !image)) return fail(NTG_ERR_INVALID_ARGUMENT, "null pointer");
+    const int64_t L = Ho * Wo, ckk = channels * k_r * k_c;
+    const int64_t add = (channels / groups) * k_r * k_c, og = out_channels / groups;
+    const int64_t need = batch * ckk * L * es;
+    if (!workspace || workspace_bytes < need)
+        return fail(NTG_ERR_INVALID_ARGUMENT, "workspace of %lld bytes needed, %lld given", (long long)need, (long long)workspace_bytes);
+    const char* kern = static_cast<const char*>(kernel);
+    const char* gy = static_cast<const char*>(grad_out);
+    char* ws = static_cast<char*>(workspace);
+    ntg_gemm_desc d;
+    if (d_kernel) {
+        // col = im2col(image); per group g:  dW_g [og, add] (+)= sum_b dY_{b,g} [og, L] . col_{b,g}^T  (col_{b,g} stored [add, L])
+        rc = ntg_unfold2d_dev(dtype, image, ws, batch, channels, height, width, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c, stream);
+        if (rc) return rc;
+        for (int64_t g = 0; g < groups; ++g)
+            for (int64_t b = 0; b < batch; ++b) {
+                std::memset(&d, 0, sizeof d);
+                d.dtype = dtype; d.transpose_b = 1;
+                d.c_mode = (b == 0 && !accumulate) ? NTG_C_OVERWRITE : NTG_C_ACCUMULATE;
+                d.m = og; d.k = L; d.n = add;
+                d.lda = L; d.ldb = L; d.ldc = add; d.batches = 1;
+                rc = ntg_gemm_dev(&d, gy + ((b * out_channels + g * og) * L) * es, ws + ((b * ckk + g * add) * L) * es,
+                                  static_cast<char*>(d_kernel) + g * og * add * es, stream);
+                if (rc) return rc;
+            }
+    }
+    if (d_image) {
+        // d_col_{b,g} [add, L] = W_g^T . dY_{b,g}   (W_g stored [og, add] -> transpose_a), then col2im
+        for (int64_t g = 0; g < groups; ++g) {
+            std::memset(&d, 0, sizeof d);
+            d.dtype = dtype; d.transpose_a = 1; d.c_mode = NTG_C_OVERWRITE;
+            d.m = add; d.k = og; d.n = L;
+            d.lda = add; d.ldb = L; d.ldc = L; d.batches = batch;
+            d.stride_a = 0; d.stride_b = out_channels * L; d.stride_c = ckk * L;
+            rc = ntg_gemm_dev(&d, kern + g * og * add * es, gy + g * og * L * es, ws + g * add * L * es, stream);
+            if (rc) return rc;
+        }
+        rc = ntg_unfold2d_backward_dev(dtype, ws, d_image, batch, channels, height, width, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c,
+                                       accumulate, stream);
+        if (rc) return rc;
+    }
+    return NTG_OK;
+}
+
+int ntg_conv2d_backward(int dtype, const void* image, const void* kernel, const void* grad_out,
+                        void* d_image, void* d_kernel,
+                        int64_t batch, int64_t channels, int64_t height, int64_t width,
+                        int64_t out_channels, int64_t k_r, int64_t k_c,
+                        int64_t s_r, int64_t s_c, int64_t p_r, int64_t p_c, int64_t d_r, int64_t d_c,
+                        int64_t groups, int accumulate) {
+    const int64_t es = ntg::elem_size(dtype);
+    if (es == 0) return fail(NTG_ERR_UNSUPPORTED_DTYPE, "dtype %d is not supported", dtype);
+    if (batch < 0 || channels < 0 || out_channels < 0 || height < 0 || width < 0) return fail(NTG_ERR_INVALID_ARGUMENT, "negative size");
+    if (groups < 1 || channels % groups != 0 || out_channels % groups != 0)
+        return fail(NTG_ERR_INVALID_ARGUMENT, "channels (%lld) and out channels (%lld) must be divisible by groups (%lld)",
+                    (long long)channels, (long long)out_channels, (long long)groups);
+    int64_t Ho, Wo;
+    int rc = unfold_out(height, width, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c, Ho, Wo);
+    if (rc) return rc;
+    if (batch == 0 || out_channels == 0 || channels == 0) return NTG_OK;
+    if (!image || !kernel || !grad_out) return fail(NTG_ERR_INVALID_ARGUMENT, "null pointer");
+    const size_t im_bytes = (size_t)(batch * channels * height * width * es);
+    const size_t k_bytes = (size_t)(out_channels * (channels / groups) * k_r * k_c * es);
+    const size_t g_bytes = (size_t)(batch * out_channels * Ho * Wo * es);
+    const int64_t wsb = ntg_conv2d_workspace_bytes(dtype, batch, channels, height, width, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c);
+    DeviceMem mem;
+    const size_t o_k = align_up(im_bytes, 256), o_g = o_k + align_up(k_bytes, 256), o_di = o_g + align_up(g_bytes, 256);
+    const size_t o_dk = o_di + align_up(im_bytes, 256), o_ws = o_dk + align_up(k_bytes, 256);
+    HIP_TRY(mem.alloc(o_ws + (size_t)wsb));
+    HIP_TRY(hipMemcpy(mem.at(0), image, im_bytes, hipMemcpyHostToDevice));
+    HIP_TRY(hipMemcpy(mem.at(o_k), kernel, k_bytes, hipMemcpyHostToDevice));
+    HIP_TRY(hipMemcpy(mem.at(o_g), grad_out, g_bytes, hipMemcpyHostToDevice));
+    if (accumulate && d_image) HIP_TRY(hipMemcpy(mem.at(o_di), d_image, im_bytes, hipMemcpyHostToDevice));
+    if (accumulate && d_kernel) HIP_TRY(hipMemcpy(mem.at(o_dk), d_kernel, k_bytes, hipMemcpyHostToDevice));
+    rc = ntg_conv2d_backward_dev(dtype, mem.at(0), mem.at(o_k), mem.at(o_g), d_image ? mem.at(o_di) : nullptr,
+                                 d_kernel ? mem.at(o_dk) : nullptr, mem.at(o_ws), wsb, batch, channels, height, width, out_channels,
+                                 k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c, groups, accumulate, nullptr);
+    if (rc) return rc;
+    HIP_TRY(hipStreamSynchronize(nullptr));
+    if (d_image) HIP_TRY(hipMemcpy(d_image, mem.at(o_di), im_bytes, hipMemcpyDeviceToHost));
+    if (d_kernel) HIP_TRY(hipMemcpy(d_kernel, mem.at(o_dk), k_bytes, hipMemcpyDeviceToHost));
+    return NTG_OK;
+}
+
 }  // extern "C"

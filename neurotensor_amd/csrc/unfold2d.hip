@@ -36,6 +36,80 @@ __global__ void __launch_bounds__(256) unfold2d_kernel(const T* __restrict__ im,
     }
 }
 
+// col2im, the adjoint of the above (im2col_backward_cpu, nt/functional/cpu/unfold2d_backward.cpp:9-56):
+//   im[b, c, y, x] (+)= sum over taps (i, j) of col[b, c*kh*kw + i*kw + j, h*Wo + w]
+//   with  y = h*s_r - p_r + i*d_r,  x = w*s_c - p_c + j*d_c.
+// Written as a gather -- one lane per image element, taps visited in ascending (i, j), which
+// is the order in which the reference's scatter loop reaches that element -- so there are no
+// atomics and the floating-point sum is reproducible.
+template <class T, class Acc>
+__global__ void __launch_bounds__(256) col2im_kernel(const T* __restrict__ col, T* __restrict__ im, const UnfoldParams u, const int accumulate) {
+    const int64_t total = u.batch * u.channels * u.height * u.width;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += stride) {
+        const int64_t x = idx % u.width;
+        int64_t t = idx / u.width;
+        const int64_t y = t % u.height;
+        t /= u.height;
+        const int64_t c = t % u.channels;
+        const int64_t b = t / u.channels;
+        Acc acc = accumulate ? (Acc)im[idx] : (Acc)0;
+        for (int64_t i = 0; i < u.k_r; ++i) {
+            const int64_t hn = y + u.p_r - i * u.d_r;
+            if (hn < 0 || hn % u.s_r != 0) continue;
+            const int64_t h = hn / u.s_r;
+            if (h >= u.Ho) continue;
+            for (int64_t j = 0; j < u.k_c; ++j) {
+                const int64_t wn = x + u.p_c - j * u.d_c;
+                if (wn < 0 || wn % u.s_c != 0) continue;
+                const int64_t w = wn / u.s_c;
+                if (w >= u.Wo) continue;
+                const int64_t cc = (c * u.k_r + i) * u.k_c + j;
+                acc += (Acc)col[((b * u.ccol + cc) * u.Ho + h) * u.Wo + w];
+            }
+        }
+        im[idx] = (T)acc;
+    }
+}
+
+static hipError_t fill_params(UnfoldParams& u, int64_t batch, int64_t channels, int64_t height, int64_t width,
+                              int64_t k_r, int64_t k_c, int64_t s_r, int64_t s_c, int64_t p_r, int64_t p_c, int64_t d_r, int64_t d_c) {
+    u.batch = batch; u.channels = channels; u.height = height; u.width = width;
+    u.k_r = k_r; u.k_c = k_c; u.s_r = s_r; u.s_c = s_c; u.p_r = p_r; u.p_c = p_c; u.d_r = d_r; u.d_c = d_c;
+    u.Ho = (height + 2 * p_r - d_r * (k_r - 1) - 1) / s_r + 1;
+    u.Wo = (width + 2 * p_c - d_c * (k_c - 1) - 1) / s_c + 1;
+    if (u.Ho <= 0 || u.Wo <= 0) return hipErrorInvalidValue;
+    u.ccol = channels * k_r * k_c;
+    u.total = batch * u.ccol * u.Ho * u.Wo;
+    return hipSuccess;
+}
+
+hipError_t launch_col2im(int dtype, const void* col, void* im,
+                         int64_t batch, int64_t channels, int64_t height, int64_t width,
+                         int64_t k_r, int64_t k_c, int64_t s_r, int64_t s_c,
+                         int64_t p_r, int64_t p_c, int64_t d_r, int64_t d_c, int accumulate, hipStream_t s) {
+    UnfoldParams u;
+    hipError_t e = fill_params(u, batch, channels, height, width, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c);
+    if (e != hipSuccess) return e;
+    const int64_t total = batch * channels * height * width;
+    if (total == 0) return hipSuccess;
+    int64_t blocks = (total + 255) / 256;
+    if (blocks > 256 * 64) blocks = 256 * 64;
+    const dim3 g((unsigned)blocks), b(256);
+    switch (dtype) {
+    case DT_F32: hipLaunchKernelGGL((col2im_kernel<float, float>), g, b, 0, s, (const float*)col, (float*)im, u, accumulate); break;
+    case DT_F64: hipLaunchKernelGGL((col2im_kernel<double, double>), g, b, 0, s, (const double*)col, (double*)im, u, accumulate); break;
+    case DT_F16: hipLaunchKernelGGL((col2im_kernel<_Float16, float>), g, b, 0, s, (const _Float16*)col, (_Float16*)im, u, accumulate); break;
+    case DT_BF16: hipLaunchKernelGGL((col2im_kernel<__bf16, float>), g, b, 0, s, (const __bf16*)col, (__bf16*)im, u, accumulate); break;
+    case DT_I8: case DT_U8: hipLaunchKernelGGL((col2im_kernel<uint8_t, uint8_t>), g, b, 0, s, (const uint8_t*)col, (uint8_t*)im, u, accumulate); break;
+    case DT_I16: case DT_U16: hipLaunchKernelGGL((col2im_kernel<uint16_t, uint16_t>), g, b, 0, s, (const uint16_t*)col, (uint16_t*)im, u, accumulate); break;
+    case DT_I32: case DT_U32: hipLaunchKernelGGL((col2im_kernel<uint32_t, uint32_t>), g, b, 0, s, (const uint32_t*)col, (uint32_t*)im, u, accumulate); break;
+    case DT_I64: case DT_U64: hipLaunchKernelGGL((col2im_kernel<uint64_t, uint64_t>), g, b, 0, s, (const uint64_t*)col, (uint64_t*)im, u, accumulate); break;
+    default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+
 hipError_t launch_unfold2d(int64_t es, const void* im, void* col,
                            int64_t batch, int64_t channels, int64_t height, int64_t width,
                            int64_t k_r, int64_t k_c, int64_t s_r, int64_t s_c,

@@ -277,3 +277,55 @@ def conv2d(image, kernel, stride=1, padding=0, dilation=1, groups=1):
     check(L.ntg_conv2d_dev(dt, x.data_ptr(), w.data_ptr(), out.data_ptr(), ws.data_ptr(), ws_bytes,
                            B, C, H, W, O, kh, kw, s[0], s[1], p[0], p[1], d[0], d[1], groups, _stream()))
     return out
+
+
+def unfold2d_backward(col, output_size, kernel_size, dilation=1, padding=0, stride=1):
+    """functional::unfold2d_backward with transpose_out=true (colim_transform.cpp:592-653):
+    col [B, C*kh*kw, L] -> image gradient [B, C, H, W]."""
+    _require_device(col)
+    k, d, p, s = _pair(kernel_size), _pair(dilation), _pair(padding), _pair(stride)
+    H, W = _pair(output_size)
+    if col.dim() not in (2, 3):
+        raise ValueError(f"Expected to get a shape with a dimensionality of 3D or 2D, but got {col.dim()} dimensions")
+    c3 = col.reshape((1,) + tuple(col.shape)) if col.dim() == 2 else col
+    c3 = c3.contiguous()
+    B = c3.shape[0]
+    if c3.shape[1] % (k[0] * k[1]) != 0:
+        raise ValueError("col rows are not a multiple of the kernel size")
+    C = c3.shape[1] // (k[0] * k[1])
+    Ho = (H + 2 * p[0] - d[0] * (k[0] - 1) - 1) // s[0] + 1
+    Wo = (W + 2 * p[1] - d[1] * (k[1] - 1) - 1) // s[1] + 1
+    if Ho * Wo != c3.shape[2]:
+        raise ValueError(f"col has {c3.shape[2]} sliding blocks, the geometry gives {Ho * Wo}")
+    im = torch.empty((B, C, H, W), dtype=col.dtype, device=col.device)
+    check(load().ntg_unfold2d_backward_dev(ntg_dtype(col), c3.data_ptr(), im.data_ptr(), B, C, H, W,
+                                           k[0], k[1], s[0], s[1], p[0], p[1], d[0], d[1], 0, _stream()))
+    return im
+
+
+def conv2d_backward(image, kernel, grad, stride=1, padding=0, dilation=1, groups=1):
+    """conv_dimage + conv_dkernel for dim == 2 (conv.cpp:318-346, 444-471): returns (d_image, d_kernel)."""
+    _require_device(image, kernel, grad)
+    s, p, d = _pair(stride), _pair(padding), _pair(dilation)
+    x = image.reshape((1,) + tuple(image.shape)) if image.dim() == 3 else image.reshape((-1,) + tuple(image.shape[-3:]))
+    w = kernel.reshape((1,) + tuple(kernel.shape)) if kernel.dim() == 3 else kernel
+    x, w, g = x.contiguous(), w.contiguous(), grad.contiguous()
+    B, C, H, W = x.shape
+    O, Cg, kh, kw = w.shape
+    if C % groups != 0 or Cg * groups != C or O % groups != 0:
+        raise ValueError(f"channels {C}, kernel channels {Cg} and filters {O} do not fit groups={groups}")
+    L = load()
+    dt = ntg_dtype(x)
+    ws_bytes = L.ntg_conv2d_workspace_bytes(dt, B, C, H, W, kh, kw, s[0], s[1], p[0], p[1], d[0], d[1])
+    if ws_bytes < 0:
+        raise ValueError("the array of sliding blocks would be empty")
+    Ho = (H + 2 * p[0] - d[0] * (kh - 1) - 1) // s[0] + 1
+    Wo = (W + 2 * p[1] - d[1] * (kw - 1) - 1) // s[1] + 1
+    if g.numel() != B * O * Ho * Wo:
+        raise ValueError(f"grad has {g.numel()} elements, expected {(B, O, Ho, Wo)}")
+    dx = torch.empty_like(x)
+    dw = torch.empty_like(w)
+    ws = torch.empty((max(ws_bytes, 1),), dtype=torch.uint8, device=x.device)
+    check(L.ntg_conv2d_backward_dev(dt, x.data_ptr(), w.data_ptr(), g.data_ptr(), dx.data_ptr(), dw.data_ptr(), ws.data_ptr(), ws_bytes,
+                                    B, C, H, W, O, kh, kw, s[0], s[1], p[0], p[1], d[0], d[1], groups, 0, _stream()))
+    return dx.reshape(image.shape), dw.reshape(kernel.shape)

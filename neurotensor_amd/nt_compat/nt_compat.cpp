@@ -513,6 +513,46 @@ Tensor conv2d(const Tensor& image, const Tensor& kernel, utils::my_tuple s, util
     return out;
 }
 
+Tensor unfold2d_backward(const Tensor& col_in, utils::my_tuple out, utils::my_tuple k, utils::my_tuple d, utils::my_tuple p, utils::my_tuple s) {
+    utils::throw_exception(!col_in.is_null(), "Cannot perform operation unfold2d_backward on a null tensor");
+    utils::throw_exception(col_in.dims() == 2 || col_in.dims() == 3, "Expected to get a shape with a dimensionality of 3D or 2D, but got " +
+                                                                         std::to_string(col_in.dims()) + " dimensions");   // colim_transform.cpp:594
+    Tensor col = col_in.contiguous();
+    const SizeRef& cs = col.shape();
+    const int64_t B = col.dims() == 3 ? cs[0] : 1, rows = cs[cs.size() - 2], L = cs[cs.size() - 1];
+    utils::throw_exception(rows % (k.first * k.second) == 0, "col rows are not a multiple of the kernel size");
+    const int64_t C = rows / (k.first * k.second);
+    const int64_t Lr = (out.first + 2 * p.first - d.first * (k.first - 1) - 1) / s.first + 1;
+    const int64_t Lc = (out.second + 2 * p.second - d.second * (k.second - 1) - 1) / s.second + 1;
+    utils::throw_exception(Lr > 0 && Lc > 0 && Lr * Lc == L, "Given output_size and kernel geometry do not match the number of sliding blocks");
+    Tensor im({B, C, out.first, out.second}, col.dtype());
+    check_status(ntg_unfold2d_backward(static_cast<int>(col.dtype()), col.data_ptr(), im.data_ptr(), B, C, out.first, out.second, k.first,
+                                       k.second, s.first, s.second, p.first, p.second, d.first, d.second, 0));
+    return im;
+}
+
+ConvGrads conv2d_backward(const Tensor& image, const Tensor& kernel, const Tensor& grad, utils::my_tuple s, utils::my_tuple p,
+                          utils::my_tuple d, int64_t groups) {
+    utils::throw_exception(!image.is_null() && !kernel.is_null() && !grad.is_null(), "Cannot perform operation conv2d backward on a null tensor");
+    utils::throw_exception(image.dims() >= 3 && (kernel.dims() == 3 || kernel.dims() == 4), "conv2d backward expects an image of >= 3 dims and a 3D/4D kernel");
+    utils::throw_exception(image.dtype() == kernel.dtype() && image.dtype() == grad.dtype(), "conv2d backward expects one dtype");
+    Tensor x = image.contiguous(), w = kernel.contiguous(), g = grad.contiguous();
+    const SizeRef& xs = x.shape();
+    const int64_t H = xs[xs.size() - 2], W = xs[xs.size() - 1], C = xs[xs.size() - 3];
+    const int64_t B = x.numel() / std::max<int64_t>(1, C * H * W);
+    const SizeRef& ws = w.shape();
+    const int64_t kh = ws[ws.size() - 2], kw = ws[ws.size() - 1], Cg = ws[ws.size() - 3], O = kernel.dims() == 4 ? ws[0] : 1;
+    utils::throw_exception(groups >= 1 && C % groups == 0 && Cg * groups == C && O % groups == 0, "channels, kernel channels and filters do not fit groups");
+    const int64_t Ro = (H + 2 * p.first - d.first * (kh - 1) - 1) / s.first + 1;
+    const int64_t Co = (W + 2 * p.second - d.second * (kw - 1) - 1) / s.second + 1;
+    utils::throw_exception(Ro > 0 && Co > 0 && g.numel() == B * O * Ro * Co, "grad does not have the shape of the convolution output");
+    ConvGrads out{Tensor(image.shape(), x.dtype()), Tensor(kernel.shape(), x.dtype())};
+    check_status(ntg_conv2d_backward(static_cast<int>(x.dtype()), x.data_ptr(), w.data_ptr(), g.data_ptr(), out.d_image.data_ptr(),
+                                     out.d_kernel.data_ptr(), B, C, H, W, O, kh, kw, s.first, s.second, p.first, p.second, d.first, d.second,
+                                     groups, 0));
+    return out;
+}
+
 }  // namespace functional
 
 namespace layers {

@@ -92,6 +92,13 @@ Tensor unfold2d(const Tensor& x, utils::my_tuple kernel_size, utils::my_tuple di
 Tensor conv2d(const Tensor& image, const Tensor& kernel, utils::my_tuple stride = {1, 1}, utils::my_tuple padding = {0, 0},
               utils::my_tuple dilation = {1, 1}, int64_t groups = 1);
 
+// conv_dimage + conv_dkernel for dim == 2 (conv.h:17-18; conv.cpp:318-346, 444-471) and col2im
+Tensor unfold2d_backward(const Tensor& col, utils::my_tuple output_size, utils::my_tuple kernel_size, utils::my_tuple dilation = {1, 1},
+                         utils::my_tuple padding = {0, 0}, utils::my_tuple stride = {1, 1});
+struct ConvGrads { Tensor d_image, d_kernel; };
+ConvGrads conv2d_backward(const Tensor& image, const Tensor& kernel, const Tensor& grad, utils::my_tuple stride = {1, 1},
+                          utils::my_tuple padding = {0, 0}, utils::my_tuple dilation = {1, 1}, int64_t groups = 1);
+
 // what the backward lambdas of TensorGrad matmult / linear compute (flags only, no transposed copies)
 struct MatmultGrads { Tensor da, db; };
 MatmultGrads matmult_backward(const Tensor& a, const Tensor& b, const Tensor& grad, bool trans_a, bool trans_b);

@@ -234,12 +234,18 @@ static void device_cases(const std::string& g) {
             Tensor o = nt::conv2d(x, w, {1, 1}, {pad, pad}, {1, 1}, grouped ? 2 : 1);
             nt::utils::throw_exception(o.shape() == want.shape(), "output shape " + nt::shape_str(o.shape()));
             nt::utils::throw_exception(F::allclose(o, want, 1e-4, 1e-4), "conv2d output differs from the fixture");
+            // xgrad / wgrad of the same test case (conv_dimage, conv_dkernel)
+            F::ConvGrads gr = F::conv2d_backward(x, w, F::from_numpy(g + "/conv2d_grad" + sfx + ".npy"), {1, 1}, {pad, pad}, {1, 1}, grouped ? 2 : 1);
+            nt::utils::throw_exception(F::allclose(gr.d_image, F::from_numpy(g + "/conv2d_xgrad" + sfx + ".npy"), 1e-4, 1e-4), "xgrad differs from the fixture");
+            nt::utils::throw_exception(F::allclose(gr.d_kernel, F::from_numpy(g + "/conv2d_wgrad" + sfx + ".npy"), 1e-4, 1e-3), "wgrad differs from the fixture");
         });
     }
     run_test("unfold2d golden", [&] {
         Tensor x = F::from_numpy(g + "/unfold_input.npy"), want = F::from_numpy(g + "/unfold_output.npy");
         Tensor col = F::unfold2d(x, {3, 2}, {1, 2}, {1, 1}, {2, 2}, true);
         nt::utils::throw_exception(col.shape() == SizeRef({1, 18, 16}) && std::memcmp(col.data_ptr(), want.data_ptr(), 18 * 16 * 4) == 0, "unfold output");
+        Tensor gi = F::unfold2d_backward(F::from_numpy(g + "/unfold_grad.npy"), {8, 8}, {3, 2}, {1, 2}, {1, 1}, {2, 2});
+        nt::utils::throw_exception(F::allclose(gi, F::from_numpy(g + "/unfold_input_grad.npy"), 1e-5, 1e-6), "unfold input grad");
     });
 }
 

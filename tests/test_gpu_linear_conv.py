@@ -162,6 +162,74 @@ def test_conv2d_golden(golden_dir, sfx, pad, groups):
     assert np.array_equal(y, out)
 
 
+@pytest.mark.parametrize("sfx,pad,groups", CONV_CASES)
+def test_conv2d_backward_golden(golden_dir, sfx, pad, groups):
+    """conv_dimage / conv_dkernel (conv.cpp:318-346, 444-471) against the xgrad / wgrad fixtures of
+    tests/src/conv_autograd_test.cpp:250-371, device and host entry points."""
+    x = load(golden_dir, "conv2d_input" + sfx)
+    w = load(golden_dir, "conv2d_weight" + sfx)
+    g = load(golden_dir, "conv2d_grad" + sfx)
+    xg = load(golden_dir, "conv2d_xgrad" + sfx)
+    wg = load(golden_dir, "conv2d_wgrad" + sfx)
+    dx, dw = F.conv2d_backward(dev(x), dev(w), dev(g), stride=1, padding=pad, dilation=1, groups=groups)
+    dx, dw = dx.cpu().numpy(), dw.cpu().numpy()
+    assert dx.shape == xg.shape and dw.shape == wg.shape
+    assert np.abs(dx - xg).max() <= 1e-4 * max(1.0, np.abs(xg).max())
+    assert np.abs(dw - wg).max() <= 1e-4 * max(1.0, np.abs(wg).max())
+    odx, odw = oracle.conv2d_backward(x, w, g, 1, pad, 1, groups)
+    assert np.abs(dx - odx).max() <= 1e-5 and np.abs(dw - odw).max() <= 1e-4
+    lib = _lib.load()
+    B, C, H, W = x.shape
+    O, _, kh, kw = w.shape
+    hx = np.full(x.shape, np.nan, np.float32)
+    hw = np.full(w.shape, np.nan, np.float32)
+    p = lambda a: np.ascontiguousarray(a).ctypes.data_as(ctypes.c_void_p)
+    _lib.check(lib.ntg_conv2d_backward(_lib.FLOAT32, p(x), p(w), p(g), hx.ctypes.data_as(ctypes.c_void_p),
+                                       hw.ctypes.data_as(ctypes.c_void_p), B, C, H, W, O, kh, kw, 1, 1, pad, pad, 1, 1, groups, 0))
+    assert np.array_equal(hx, dx) and np.array_equal(hw, dw)
+    # accumulate != 0 adds to the incoming gradients, like the reference's += (conv.cpp:466-469)
+    hx2, hw2 = hx.copy(), hw.copy()
+    _lib.check(lib.ntg_conv2d_backward(_lib.FLOAT32, p(x), p(w), p(g), hx2.ctypes.data_as(ctypes.c_void_p),
+                                       hw2.ctypes.data_as(ctypes.c_void_p), B, C, H, W, O, kh, kw, 1, 1, pad, pad, 1, 1, groups, 1))
+    assert np.allclose(hx2, 2 * hx, rtol=1e-5, atol=1e-5) and np.allclose(hw2, 2 * hw, rtol=1e-5, atol=1e-4)
+
+
+def test_unfold_backward_golden_and_random(golden_dir):
+    g = load(golden_dir, "unfold_grad")
+    want = load(golden_dir, "unfold_input_grad")
+    got = F.unfold2d_backward(dev(g), (8, 8), (3, 2), dilation=(1, 2), padding=1, stride=(2, 2)).cpu().numpy()
+    assert np.allclose(got, want, rtol=1e-6, atol=1e-6)
+    rng = np.random.default_rng(950)
+    for dtype in (np.float32, np.float64):
+        for (H, W), k, d, p, s in [((13, 17), (3, 3), 1, 1, 1), ((9, 12), (2, 4), (2, 1), (0, 3), (1, 2)), ((10, 10), (5, 5), 1, 2, 2)]:
+            x = rng.standard_normal((2, 3, H, W)).astype(dtype)
+            col = oracle.unfold2d(x, k, dilation=d, padding=p, stride=s)
+            gcol = rng.standard_normal(col.shape).astype(dtype)
+            ref = oracle.unfold2d_backward(gcol, (H, W), k, dilation=d, padding=p, stride=s)
+            got = F.unfold2d_backward(dev(gcol), (H, W), k, dilation=d, padding=p, stride=s).cpu().numpy()
+            # same tap order as the scatter loop: bit-identical sums
+            assert np.array_equal(got, ref)
+
+
+def test_conv2d_backward_random_vs_oracle():
+    rng = np.random.default_rng(960)
+    x = rng.standard_normal((3, 6, 14, 11)).astype(np.float32)
+    w = rng.standard_normal((8, 3, 3, 2)).astype(np.float32)
+    kw = dict(stride=(2, 1), padding=(1, 2), dilation=(1, 2), groups=2)
+    out = oracle.conv2d(x, w, kw["stride"], kw["padding"], kw["dilation"], kw["groups"])
+    g = rng.standard_normal(out.shape).astype(np.float32)
+    dx, dw = F.conv2d_backward(dev(x), dev(w), dev(g), **kw)
+    odx, odw = oracle.conv2d_backward(x, w, g, kw["stride"], kw["padding"], kw["dilation"], kw["groups"])
+    assert np.abs(dx.cpu().numpy() - odx).max() <= 1e-4
+    assert np.abs(dw.cpu().numpy() - odw).max() <= 1e-3
+    # gradient check against torch autograd in float64 (independent of both implementations)
+    tx = torch.from_numpy(x).double().requires_grad_(True)
+    tw = torch.from_numpy(w).double().requires_grad_(True)
+    torch.nn.functional.conv2d(tx, tw, None, kw["stride"], kw["padding"], kw["dilation"], kw["groups"]).backward(torch.from_numpy(g).double())
+    assert np.abs(dx.cpu().numpy() - tx.grad.numpy()).max() <= 1e-4
+    assert np.abs(dw.cpu().numpy() - tw.grad.numpy()).max() <= 1e-3
+
+
 @pytest.mark.parametrize("dtype", [np.float32, np.float64, np.float16, np.int32])
 def test_conv2d_random_vs_oracle(dtype):
     rng = np.random.default_rng(900)
