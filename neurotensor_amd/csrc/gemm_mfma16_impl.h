@@ -1,6 +1,8 @@
-// 16-bit (Float16 / BFloat16) MFMA GEMM for gfx950, fast path for tile-aligned problems:
-//   C[M,N] (+)= op(A) . op(B),  M % 256 == 0, N % 256 == 0, K % 32 == 0, 16-byte aligned rows.
-// (Everything else goes through the general kernel in gemm_mfma_impl.h.)
+// 16-bit (Float16 / BFloat16) MFMA GEMM for gfx950, fast path:
+//   C[M,N] (+)= op(A) . op(B),  16-byte aligned rows (leading dimensions and contiguous extents
+//   multiples of 8 elements); M, N, K need not be multiples of the 256 x 256 x 32 tile (the
+//   RAGGED instantiation clamps DMA source addresses, zeroes the k tail in registers and
+//   guards the stores).  Everything else goes through the general kernel in gemm_mfma_impl.h.
 //
 // Shape of the kernel
 //   * 256 x 256 tile of C per workgroup, 4 wavefronts (2 x 2), each owning 128 x 128 =
@@ -60,18 +62,31 @@ struct G16 {
 // [1024 j, 1024 j + 1024) of the tile:
 //   K-contiguous operand: rows 16 j + lane/4, 16-byte slot lane%4 holds kv = slot ^ ((row>>1)&3)
 //   MN-contiguous operand: k-rows 2 j + lane/32, slot lane%32 holds chunk = slot ^ (2*(krow&3))
-template <bool KC>
-__device__ __forceinline__ void dma_offsets(uint32_t (&off)[4], int64_t ld, int wave, int lane) {
+// With RAGGED, mn_valid (1..256 rows/columns of the tile that exist) and k_valid (8..32 k of
+// the K-step that exist, a multiple of 8) clamp the SOURCE address into the matrix: lanes
+// whose data does not exist fetch a neighbouring chunk instead.  Rows/columns past the edge
+// only ever reach accumulators that the epilogue does not store; k past the end is zeroed
+// in the fragment registers before it is multiplied.
+template <bool KC, bool RAGGED>
+__device__ __forceinline__ void dma_offsets(uint32_t (&off)[4], int64_t ld, int wave, int lane, int mn_valid, int k_valid) {
 #pragma unroll
     for (int jj = 0; jj < 4; ++jj) {
         const int j = wave * 4 + jj;
         if constexpr (KC) {
-            const int row = 16 * j + (lane >> 2);
-            const int kv = (lane & 3) ^ ((row >> 1) & 3);
+            int row = 16 * j + (lane >> 2);
+            int kv = (lane & 3) ^ ((row >> 1) & 3);
+            if constexpr (RAGGED) {
+                row = row < mn_valid ? row : mn_valid - 1;
+                kv = kv < (k_valid >> 3) ? kv : (k_valid >> 3) - 1;
+            }
             off[jj] = (uint32_t)(((int64_t)row * ld + kv * 8) * 2);
         } else {
-            const int krow = 2 * j + (lane >> 5);
-            const int chunk = (lane & 31) ^ (2 * (krow & 3));
+            int krow = 2 * j + (lane >> 5);
+            int chunk = (lane & 31) ^ (2 * (krow & 3));
+            if constexpr (RAGGED) {
+                krow = krow < k_valid ? krow : k_valid - 1;
+                chunk = chunk < (mn_valid >> 3) ? chunk : (mn_valid >> 3) - 1;
+            }
             off[jj] = (uint32_t)(((int64_t)krow * ld + chunk * 8) * 2);
         }
     }
@@ -96,7 +111,7 @@ __device__ __forceinline__ uint32_t lds_addr_of(const char* p) {
     return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const char*)p;
 }
 
-template <int DT, bool TA, bool TB>
+template <int DT, bool TA, bool TB, bool RAGGED>
 __global__ void __launch_bounds__(256) gemm16_kernel(const GemmParams p) {
     using E = Elem<DT>;
     using T = typename E::T;
@@ -126,9 +141,17 @@ __global__ void __launch_bounds__(256) gemm16_kernel(const GemmParams p) {
 
     // ---- DMA sources: uniform tile base (advances by adv bytes per K-step) + per-lane offsets ----
     const int wave_u = __builtin_amdgcn_readfirstlane(wave);
-    uint32_t offA[4], offB[4];
-    dma_offsets<A_KC>(offA, p.lda, wave, lane);
-    dma_offsets<B_KC>(offB, p.ldb, wave, lane);
+    const int KT = (p.K + BK - 1) / BK;
+    const int last = KT - 1;
+    const int kr = p.K - last * BK;                                  // k that exist in the last K-step (8..32)
+    const int mvalid = p.M - m0 < G16::BM ? p.M - m0 : G16::BM;
+    const int nvalid = p.N - n0 < G16::BN ? p.N - n0 : G16::BN;
+    uint32_t offA[4], offB[4];      // K-steps before the last
+    uint32_t offAt[4], offBt[4];    // the last K-step (RAGGED: k clamped to what exists)
+    dma_offsets<A_KC, RAGGED>(offA, p.lda, wave, lane, mvalid, BK);
+    dma_offsets<B_KC, RAGGED>(offB, p.ldb, wave, lane, nvalid, BK);
+    dma_offsets<A_KC, RAGGED>(offAt, p.lda, wave, lane, mvalid, kr);
+    dma_offsets<B_KC, RAGGED>(offBt, p.ldb, wave, lane, nvalid, kr);
     const char* baseA = reinterpret_cast<const char*>(A) + (A_KC ? (int64_t)m0 * p.lda : (int64_t)m0) * 2;
     const char* baseB = reinterpret_cast<const char*>(B) + (B_KC ? (int64_t)n0 * p.ldb : (int64_t)n0) * 2;
     const int64_t advA = (A_KC ? (int64_t)BK : (int64_t)BK * p.lda) * 2;
@@ -183,23 +206,20 @@ __global__ void __launch_bounds__(256) gemm16_kernel(const GemmParams p) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-    const int KT = p.K / BK;
-
     // K-steps past the end are clamped to the last one: the tail iterations then issue the
     // same DMA traffic as the steady state (into stages nobody reads any more), which keeps
     // the loop body free of branches and the vmcnt bookkeeping uniform.
-    const int last = KT - 1;
     auto srcA = [&](int kt) { return tile_src(baseA + (int64_t)(kt < last ? kt : last) * advA); };
     auto srcB = [&](int kt) { return tile_src(baseB + (int64_t)(kt < last ? kt : last) * advB); };
 
     // prologue: tiles 0..2 and the A half of tile 3 in flight (28 instructions)
-    dma_tile(srcA(0), offA, lds_addr_of(st0), wave_u);
-    dma_tile(srcB(0), offB, lds_addr_of(st0) + G16::TILE_BYTES, wave_u);
-    dma_tile(srcA(1), offA, lds_addr_of(st1), wave_u);
-    dma_tile(srcB(1), offB, lds_addr_of(st1) + G16::TILE_BYTES, wave_u);
-    dma_tile(srcA(2), offA, lds_addr_of(st2), wave_u);
-    dma_tile(srcB(2), offB, lds_addr_of(st2) + G16::TILE_BYTES, wave_u);
-    dma_tile(srcA(3), offA, lds_addr_of(st3), wave_u);
+    dma_tile(srcA(0), 0 >= last ? offAt : offA, lds_addr_of(st0), wave_u);
+    dma_tile(srcB(0), 0 >= last ? offBt : offB, lds_addr_of(st0) + G16::TILE_BYTES, wave_u);
+    dma_tile(srcA(1), 1 >= last ? offAt : offA, lds_addr_of(st1), wave_u);
+    dma_tile(srcB(1), 1 >= last ? offBt : offB, lds_addr_of(st1) + G16::TILE_BYTES, wave_u);
+    dma_tile(srcA(2), 2 >= last ? offAt : offA, lds_addr_of(st2), wave_u);
+    dma_tile(srcB(2), 2 >= last ? offBt : offB, lds_addr_of(st2) + G16::TILE_BYTES, wave_u);
+    dma_tile(srcA(3), 3 >= last ? offAt : offA, lds_addr_of(st3), wave_u);
 
     u32x4 af[2][4], bf[2][4];   // fragment double buffer: [k16-step parity][block]
 
@@ -217,7 +237,11 @@ __global__ void __launch_bounds__(256) gemm16_kernel(const GemmParams p) {
     // right after the barrier, the four wavefronts would queue up behind the CU's one
     // address unit and stall their MFMA streams.
     auto mma_step_prefetch = [&](int cur_buf, const char* stage, int ks, int nxt_buf,
-                                 const void* src, const uint32_t (&off)[4], uint32_t lds_tile) {
+                                 const void* src, const uint32_t (&off_main)[4], const uint32_t (&off_tail)[4], bool tail_tile,
+                                 uint32_t lds_tile) {
+        uint32_t off[4];
+#pragma unroll
+        for (int x = 0; x < 4; ++x) off[x] = (RAGGED && tail_tile) ? off_tail[x] : off_main[x];
 #pragma unroll
         for (int q = 0; q < 16; ++q) {
             // serpentine order: consecutive MFMAs always share one operand fragment
@@ -246,15 +270,31 @@ __global__ void __launch_bounds__(256) gemm16_kernel(const GemmParams p) {
     // the stage goes back to the DMA at once: the A half of tile kt+4 is fetched during the
     // second k16-step, its B half during the first k16-step of the next K-step.  Tile kt+1,
     // first touched in the second half, has had three K-steps to arrive.
+    // RAGGED: zero the k >= K part of a fragment set of the last K-step.  Every lane's fragment
+    // covers 8 consecutive k starting at 16 ks + 8 (lane / 32) in both LDS layouts, and K is a
+    // multiple of 8, so a lane's fragment is either entirely real or entirely past the end.
+    auto mask_tail = [&](int buf, int ks) {
+        const bool ok = 16 * ks + 8 * (lane >> 5) < kr;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                af[buf][i][e] = ok ? af[buf][i][e] : 0u;
+                bf[buf][i][e] = ok ? bf[buf][i][e] : 0u;
+            }
+    };
+
     auto iteration = [&](int kt, char* cur, const char* nxt, char* prv) {
-        mma_step_prefetch(0, cur, 1, 1, srcB(kt + 3), offB, lds_addr_of(prv) + G16::TILE_BYTES);
+        if (RAGGED && kt == last && kr < BK) mask_tail(0, 0);
+        mma_step_prefetch(0, cur, 1, 1, srcB(kt + 3), offB, offBt, kt + 3 >= last, lds_addr_of(prv) + G16::TILE_BYTES);
         // outstanding now: tiles kt+1, kt+2, kt+3 (8 instructions each): wait for the oldest
         NTG_WAIT_VMCNT(16);
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // my reads of `cur` are complete
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
+        if (RAGGED && kt == last && kr < BK) mask_tail(1, 1);
         // (the last K-step prefetches fragments from a stage holding a clamped tile; unused)
-        mma_step_prefetch(1, nxt, 0, 0, srcA(kt + 4), offA, lds_addr_of(cur));
+        mma_step_prefetch(1, nxt, 0, 0, srcA(kt + 4), offA, offAt, kt + 4 >= last, lds_addr_of(cur));
     };
 
     for (int kt = 0; kt < KT; kt += 4) {
@@ -284,7 +324,8 @@ __global__ void __launch_bounds__(256) gemm16_kernel(const GemmParams p) {
 #pragma unroll
                 for (int t = 0; t < 8; ++t) {
                     const int m = m0 + wm * 128 + 32 * i + 4 * t + (lane >> 4);
-                    c0[t] = *reinterpret_cast<const u32x4*>(Cu + (int64_t)m * p.ldc + n);
+                    if (!RAGGED || (m < p.M && n < p.N)) c0[t] = *reinterpret_cast<const u32x4*>(Cu + (int64_t)m * p.ldc + n);
+                    else c0[t] = u32x4{0u, 0u, 0u, 0u};
                 }
             }
             // lane holds rows m = 32 i + lane%32, cols 32 j + 8 rq + 4 (lane/32) + (0..3)
@@ -305,6 +346,7 @@ __global__ void __launch_bounds__(256) gemm16_kernel(const GemmParams p) {
                 const floatx4v hi = *reinterpret_cast<const floatx4v*>(slab + row * 512 + (((sl + 1) ^ (row & 7)) * 16));
                 float v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
                 const int m = m0 + wm * 128 + 32 * i + row;
+                if (RAGGED && (m >= p.M || n >= p.N)) continue;     // N % 8 == 0: a lane's 8 columns exist or not together
                 if constexpr (CM == C_ACCUMULATE) {
 #pragma unroll
                     for (int e = 0; e < 8; ++e) v[e] += Cvt16<DT>::up((uint16_t)(c0[t][e >> 1] >> (16 * (e & 1))));
@@ -326,9 +368,11 @@ __global__ void __launch_bounds__(256) gemm16_kernel(const GemmParams p) {
     else epilogue(std::integral_constant<int, C_OVERWRITE>{});
 }
 
-// true when the fast kernel's preconditions hold
-static inline bool gemm16_eligible(const GemmParams& p) {
-    return p.M % 256 == 0 && p.N % 256 == 0 && p.K % 32 == 0 && p.K >= 32 &&
+// true when the fast kernel can serve the problem: 16-byte aligned rows everywhere (leading
+// dimensions, batch strides, base pointers) and every contiguous extent a multiple of 8
+// elements.  M, N and K themselves may be ragged with respect to the 256 x 256 x 32 tile.
+static inline bool gemm16_eligible(const GemmParams& p, bool ta) {
+    return p.K >= 8 && p.K % 8 == 0 && p.N % 8 == 0 && (!ta || p.M % 8 == 0) &&
            !p.Aptr && !p.Bptr && !p.Cptr && p.vecA_ok && p.vecB_ok &&
            p.ldc % 8 == 0 && p.sC % 8 == 0 && p.lda < (1 << 22) && p.ldb < (1 << 22) &&
            ((reinterpret_cast<uintptr_t>(p.A) & 15) == 0) && ((reinterpret_cast<uintptr_t>(p.B) & 15) == 0) &&
@@ -338,11 +382,14 @@ static inline bool gemm16_eligible(const GemmParams& p) {
 template <int DT, bool TA, bool TB>
 static hipError_t launch_gemm16_cfg(const GemmParams& pin, hipStream_t s) {
     GemmParams p = pin;
-    p.tiles_m = p.M / 256;
-    p.tiles_n = p.N / 256;
+    p.tiles_m = (p.M + 255) / 256;
+    p.tiles_n = (p.N + 255) / 256;
     const int64_t blocks = (int64_t)p.tiles_m * p.tiles_n * p.batch;
     if (blocks > 0x7fffffffLL) return hipErrorInvalidValue;
-    hipLaunchKernelGGL((gemm16_kernel<DT, TA, TB>), dim3((unsigned)blocks), dim3(256), 0, s, p);
+    if (p.M % 256 == 0 && p.N % 256 == 0 && p.K % 32 == 0)
+        hipLaunchKernelGGL((gemm16_kernel<DT, TA, TB, false>), dim3((unsigned)blocks), dim3(256), 0, s, p);
+    else
+        hipLaunchKernelGGL((gemm16_kernel<DT, TA, TB, true>), dim3((unsigned)blocks), dim3(256), 0, s, p);
     return hipGetLastError();
 }
 

@@ -307,6 +307,43 @@ def test_config3_4096_cube(dtype, scale):
         assert ((acc.float() - 2 * out.float()).abs().max() / out.float().abs().max()).item() <= HALF_REL
 
 
+@pytest.mark.parametrize("dtype", ["bf16", np.float16], ids=["bf16", "fp16"])
+@pytest.mark.parametrize("shape", [(2056, 1000, 2312), (1800, 1016, 3080), (2304, 992, 1928), (3000, 40, 2056), (2056, 8, 2056)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_ragged_16bit_dma_kernel(dtype, shape):
+    """M, N, K that are not multiples of the 256 x 256 x 32 tile (but keep 16-byte rows) stay on the
+    DMA-fed kernel: edge rows/columns, the k tail (8, 24, none, 8-only) and all three C modes."""
+    m, k, n = shape
+    bf = dtype == "bf16"
+    rng = np.random.default_rng(1100 + k)
+    for ta, tb in TRANS:
+        a = randn(rng, (m, k), dtype, 0.25)
+        b = randn(rng, (k, n), dtype, 0.25)
+        sa = np.ascontiguousarray(a.T) if ta else a
+        sb = np.ascontiguousarray(b.T) if tb else b
+        ta_, tb_ = to_torch(sa, DEV, bf), to_torch(sb, DEV, bf)
+        ref = torch.matmul(to_torch(a, DEV, bf).float(), to_torch(b, DEV, bf).float())
+        scale = ref.abs().max().item()
+        # C sits inside a larger buffer of sentinels: nothing outside [m, n] may be written
+        guard = torch.full((m + 2, n), 7.0, device=DEV).to(ta_.dtype)
+        c = guard[1:m + 1]
+        c.zero_()
+        out = F.matmult(ta_, tb_, c, ta, tb, accumulate=False)
+        assert ((out.float() - ref).abs().max() / scale).item() <= HALF_REL, (shape, ta, tb)
+        assert torch.all(guard[0] == 7.0) and torch.all(guard[m + 1] == 7.0)
+        F.matmult(ta_, tb_, c, ta, tb)                                   # accumulate: 2 * A.B
+        assert ((c.float() - 2 * ref).abs().max() / scale).item() <= 2 * HALF_REL
+        # oracle on the last rows / columns and on an interior block
+        rows = np.r_[0:8, m - 8:m]
+        cols = np.r_[0:8, n - 8:n]
+        _sampled_oracle_check(sa, sb, out := F.matmult(ta_, tb_, None, ta, tb), ta, tb, dtype, rows, cols, k)
+    # bias mode on a ragged shape
+    bias = randn(rng, (n,), dtype)
+    y = F.linear(to_torch(a, DEV, bf), to_torch(b, DEV, bf), to_torch(bias, DEV, bf))
+    refy = ref + to_torch(bias, DEV, bf).float()
+    assert ((y.float() - refy).abs().max() / refy.abs().max()).item() <= HALF_REL
+
+
 def test_skinny_fp32_config5b():
     rng = np.random.default_rng(1005)
     a = rng.standard_normal((16, 8192)).astype(np.float32)
