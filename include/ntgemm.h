@@ -174,7 +174,14 @@ int ntg_unfold2d_dev(int dtype, const void* image, void* col,
                      int64_t k_r, int64_t k_c, int64_t s_r, int64_t s_c,
                      int64_t p_r, int64_t p_c, int64_t d_r, int64_t d_c, void* stream);
 
-/* bytes of device workspace ntg_conv2d_dev needs (the im2col buffer). */
+/* Bytes of device workspace ntg_conv2d_dev needs.  0 for the floating dtypes: their GEMM gathers
+ * the im2col operand (nt/functional/cpu/unfold2d.cpp:12-112) from the image tile by tile and the
+ * unfolded matrix of conv.cpp:87-94 is never stored; the integer dtypes unfold into the workspace. */
+int64_t ntg_conv2d_forward_workspace_bytes(int dtype, int64_t batch, int64_t channels, int64_t height, int64_t width,
+                                           int64_t k_r, int64_t k_c, int64_t s_r, int64_t s_c,
+                                           int64_t p_r, int64_t p_c, int64_t d_r, int64_t d_c);
+
+/* bytes of the full im2col buffer (what ntg_unfold2d_dev writes and ntg_conv2d_backward_dev needs). */
 int64_t ntg_conv2d_workspace_bytes(int dtype, int64_t batch, int64_t channels, int64_t height, int64_t width,
                                    int64_t k_r, int64_t k_c, int64_t s_r, int64_t s_c,
                                    int64_t p_r, int64_t p_c, int64_t d_r, int64_t d_c);

@@ -7,4 +7,11 @@ hipError_t launch_gemm_mfma_f32(bool ta, bool tb, const GemmParams& p, hipStream
     if (big_tiles >= 192) return launch_trans<DT_F32, 2, 2, 32>(ta, tb, p, s);
     return launch_trans<DT_F32, 1, 1, 32>(ta, tb, p, s);
 }
+// conv2d / conv_dkernel with op(B) gathered from the image (tb: col^T)
+hipError_t launch_conv_mfma_f32(bool tb, const GemmParams& p, hipStream_t s) {
+    const int64_t big_tiles = (int64_t)((p.M + 127) / 128) * ((p.N + 127) / 128) * p.batch;
+    if (big_tiles >= 192)
+        return tb ? launch_conv_cfg<DT_F32, true, 2, 2, 32>(p, s) : launch_conv_cfg<DT_F32, false, 2, 2, 32>(p, s);
+    return tb ? launch_conv_cfg<DT_F32, true, 1, 1, 32>(p, s) : launch_conv_cfg<DT_F32, false, 1, 1, 32>(p, s);
+}
 }  // namespace ntg

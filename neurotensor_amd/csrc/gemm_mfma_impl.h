@@ -83,6 +83,35 @@ __device__ __forceinline__ u32x4 ldvec(const T* src, bool outer_ok, int c0, int 
     }
 }
 
+// Implicit im2col: one 16-byte vector of VE consecutive l (output pixels) of row kk (channel, tap)
+// of the matrix described by ConvGeom, gathered from the image.  Loads are unconditional (a
+// clamped address, then a select) so that all of a tile's loads are in flight together.
+template <class T, int VE>
+__device__ __forceinline__ u32x4 conv_gather(const T* __restrict__ im, const ConvGeom& g, int kk, bool kk_ok, int l0, int l_end) {
+    const uint32_t c = fast_div((uint32_t)kk, g.div_krc);
+    const uint32_t rem = (uint32_t)kk - c * (uint32_t)g.k_rc;
+    const uint32_t r = fast_div(rem, g.div_kc);
+    const uint32_t q = rem - r * (uint32_t)g.k_c;
+    const int base = (int)c * g.HW;
+    const int dh = kk_ok ? (int)r * g.d_r - g.p_r : -(1 << 29);   // far outside the image => every tap reads as padding
+    const int dw = (int)q * g.d_c - g.p_c;
+    T tmp[VE];
+#pragma unroll
+    for (int e = 0; e < VE; ++e) {
+        const int l = l0 + e;
+        const uint32_t oh = fast_div((uint32_t)l, g.div_wo);
+        const uint32_t ow = (uint32_t)l - oh * (uint32_t)g.Wo;
+        const int ih = (l < l_end ? (int)oh * g.s_r : -(1 << 29)) + dh;
+        const int iw = (int)ow * g.s_c + dw;
+        const bool ok = (unsigned)ih < (unsigned)g.H && (unsigned)iw < (unsigned)g.W;
+        const T v = im[ok ? base + ih * g.W + iw : 0];
+        tmp[e] = ok ? v : (T)0.0f;
+    }
+    u32x4 out;
+    __builtin_memcpy(&out, tmp, 16);
+    return out;
+}
+
 // One operand's BMN x BK tile: global -> registers -> LDS.
 //   KC: stored K-contiguous in global memory (A without transpose_a, B with transpose_b)
 //   KM: K-major LDS layout
@@ -132,6 +161,40 @@ struct TileLoader {
                     for (int i = 0; i < 8; ++i) {
                         const int k = k0 + kg * 8 + i;
                         v[q * 8 + i] = ldvec<T, VE, ALIGNED>(base + (int64_t)k * ld + mn, k < K, mn, MN, vec_ok);
+                    }
+                }
+            }
+        }
+    }
+
+    // Same tile, but the operand is the never-stored im2col matrix of `im`: the "rows" the
+    // vectors run along are output pixels l, the other index is kk = (channel, tap).
+    //   !KC: tile = col[k0.., mn0..]   (k = kk, mn = l)      KC: tile = col^T  (mn = kk, k = l)
+    __device__ __forceinline__ void load_conv(const T* im, const ConvGeom& g, int mn0, int k0, int MN, int K, int tid) {
+        if constexpr (!TRANSPOSE && KC) {
+#pragma unroll
+            for (int p = 0; p < NV; ++p) {
+                const int vi = tid + p * 256;
+                const int row = vi / KV, kv = vi % KV;
+                v[p] = conv_gather<T, VE>(im, g, mn0 + row, mn0 + row < MN, k0 + kv * VE, K);
+            }
+        } else if constexpr (!TRANSPOSE) {
+#pragma unroll
+            for (int p = 0; p < NV; ++p) {
+                const int vi = tid + p * 256;
+                const int kr = vi / MV, mv = vi % MV;
+                v[p] = conv_gather<T, VE>(im, g, k0 + kr, k0 + kr < K, mn0 + mv * VE, MN);
+            }
+        } else {
+#pragma unroll
+            for (int q = 0; q < NQ; ++q) {
+                const int sb = tid + q * 256;
+                if (NSB % 256 == 0 || sb < NSB) {
+                    const int kg = sb % KG, mv = sb / KG;
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) {
+                        const int k = k0 + kg * 8 + i;
+                        v[q * 8 + i] = conv_gather<T, VE>(im, g, k, k < K, mn0 + mv * 8, MN);
                     }
                 }
             }
@@ -193,7 +256,8 @@ struct GemmShape {
     static constexpr int GROUP_M = (1024 / BM) > 0 ? (1024 / BM) : 1;
 };
 
-template <int DT, bool TA, bool TB, int WBM, int WBN, int BK, bool ALIGNED>
+// CONV: op(B) is the implicit im2col matrix of the image at p.B (p.conv), see load_conv.
+template <int DT, bool TA, bool TB, int WBM, int WBN, int BK, bool ALIGNED, bool CONV = false>
 __global__ void __launch_bounds__(256) gemm_mfma_kernel(const GemmParams p) {
     using SH = GemmShape<DT, TA, TB, WBM, WBN, BK>;
     using E = Elem<DT>;
@@ -241,8 +305,13 @@ __global__ void __launch_bounds__(256) gemm_mfma_kernel(const GemmParams p) {
     LB lb;
     const int KT = (p.K + BK - 1) / BK;
 
+    auto load_b = [&](int k0) {
+        if constexpr (CONV) lb.load_conv(B, p.conv, n0, k0, p.N, p.K, tid);
+        else lb.load(B, p.ldb, n0, k0, p.N, p.K, vecB, tid);
+    };
+
     la.load(A, p.lda, m0, 0, p.M, p.K, vecA, tid);
-    lb.load(B, p.ldb, n0, 0, p.N, p.K, vecB, tid);
+    load_b(0);
     la.store(smem, tid);
     lb.store(smem + SH::LDS_A, tid);
     __syncthreads();
@@ -253,7 +322,7 @@ __global__ void __launch_bounds__(256) gemm_mfma_kernel(const GemmParams p) {
         const bool more = (kt + 1 < KT);
         if (more) {
             la.load(A, p.lda, m0, (kt + 1) * BK, p.M, p.K, vecA, tid);
-            lb.load(B, p.ldb, n0, (kt + 1) * BK, p.N, p.K, vecB, tid);
+            load_b((kt + 1) * BK);
         }
 
         if constexpr (IS16) {
@@ -380,6 +449,23 @@ static hipError_t launch_cfg(const GemmParams& pin, hipStream_t s) {
         if (attr != hipSuccess) return attr;
         hipLaunchKernelGGL(k, dim3((unsigned)blocks), dim3(256), SH::LDS_TOTAL, s, p);
     }
+    return hipGetLastError();
+}
+
+// op(B) = implicit im2col matrix (TB: transposed); always the guarded kernel
+template <int DT, bool TB, int WBM, int WBN, int BK>
+static hipError_t launch_conv_cfg(const GemmParams& pin, hipStream_t s) {
+    using SH = GemmShape<DT, false, TB, WBM, WBN, BK>;
+    GemmParams p = pin;
+    p.tiles_m = (p.M + SH::BM - 1) / SH::BM;
+    p.tiles_n = (p.N + SH::BN - 1) / SH::BN;
+    const int64_t blocks = (int64_t)p.tiles_m * p.tiles_n * p.batch;
+    if (blocks <= 0) return hipSuccess;
+    if (blocks > 0x7fffffffLL) return hipErrorInvalidValue;
+    auto k = gemm_mfma_kernel<DT, false, TB, WBM, WBN, BK, false, true>;
+    static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(k), hipFuncAttributeMaxDynamicSharedMemorySize, SH::LDS_TOTAL);
+    if (attr != hipSuccess) return attr;
+    hipLaunchKernelGGL(k, dim3((unsigned)blocks), dim3(256), SH::LDS_TOTAL, s, p);
     return hipGetLastError();
 }
 

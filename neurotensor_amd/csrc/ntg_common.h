@@ -20,6 +20,31 @@ enum CMode : int {
     C_BIAS = 2         // C  = bias (+) op(A).op(B) (cpu::linear, matmult_cpu.cpp:1637-1647)
 };
 
+// Unsigned division by a divisor fixed at launch (round-up multiplier form): exact for every
+// 32-bit n.  q = (t + ((n - t) >> s1)) >> s2  with  t = mulhi(m, n).
+struct FastDiv { uint32_t m, s1, s2; };
+static inline FastDiv make_fastdiv(uint32_t d) {
+    uint32_t l = 0;
+    while ((1ull << l) < d) ++l;
+    FastDiv f;
+    f.m = (uint32_t)(((1ull << 32) * ((1ull << l) - d)) / d + 1);
+    f.s1 = l < 1 ? l : 1;
+    f.s2 = l > 0 ? l - 1 : 0;
+    return f;
+}
+
+// Geometry of an operand that is the im2col matrix of an image and is never stored:
+//   col(kk, l) = im[c, oh*s_r - p_r + r*d_r, ow*s_c - p_c + q*d_c]   (0 in the padding)
+//   kk = (c*k_r + r)*k_c + q,   l = oh*Wo + ow
+// (the matrix nt::functional::unfold2d(..., transpose_out = true) would produce,
+// nt/functional/cpu/unfold2d.cpp:12-112).
+struct ConvGeom {
+    int H, W, HW;
+    int s_r, s_c, p_r, p_c, d_r, d_c;
+    int k_c, k_rc, Wo;
+    FastDiv div_krc, div_kc, div_wo;
+};
+
 struct GemmParams {
     const void* A;
     const void* B;
@@ -37,6 +62,7 @@ struct GemmParams {
     int cmode;
     int tiles_m, tiles_n;
     int vecA_ok, vecB_ok;    // 16-byte vector loads are legal for every row of A / B
+    ConvGeom conv;           // used by the implicit-im2col kernels only: B = image, op(B) = col or col^T
 };
 
 static inline int64_t elem_size(int dt) {
@@ -53,6 +79,8 @@ static inline int64_t elem_size(int dt) {
 hipError_t launch_gemm_mfma(int dtype, bool ta, bool tb, const GemmParams& p, hipStream_t s);
 hipError_t launch_gemm_valu(int dtype, bool ta, bool tb, const GemmParams& p, hipStream_t s);
 hipError_t launch_gemm_skinny(int dtype, bool ta, bool tb, const GemmParams& p, hipStream_t s, bool* handled);
+// op(B) is the im2col matrix of the image at p.B (tb: its transpose); floating dtypes only
+hipError_t launch_conv_mfma(int dtype, bool tb, const GemmParams& p, hipStream_t s);
 hipError_t launch_unfold2d(int64_t elem_size, const void* im, void* col,
                            int64_t batch, int64_t channels, int64_t height, int64_t width,
                            int64_t k_r, int64_t k_c, int64_t s_r, int64_t s_c,
@@ -64,6 +92,11 @@ hipError_t launch_col2im(int dtype, const void* col, void* im,
                          int64_t p_r, int64_t p_c, int64_t d_r, int64_t d_c, int accumulate, hipStream_t s);
 
 #ifdef __HIPCC__
+__device__ __forceinline__ uint32_t fast_div(uint32_t n, const FastDiv& f) {
+    const uint32_t t = __umulhi(f.m, n);
+    return (t + ((n - t) >> f.s1)) >> f.s2;
+}
+
 // Workgroup ids are dealt round-robin to the 8 XCDs; make the ids that land on one
 // XCD (its own L2) a contiguous range of logical tile ids.
 __device__ __forceinline__ int xcd_contiguous_id(int bid, int nb) {

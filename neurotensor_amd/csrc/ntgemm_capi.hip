@@ -18,6 +18,20 @@ hipError_t launch_gemm_mfma_f64(bool ta, bool tb, const GemmParams& p, hipStream
 hipError_t launch_gemm_mfma_f16(bool ta, bool tb, const GemmParams& p, hipStream_t s);
 hipError_t launch_gemm_mfma_bf16(bool ta, bool tb, const GemmParams& p, hipStream_t s);
 hipError_t launch_gemm_skinny(int dtype, bool ta, bool tb, const GemmParams& p, hipStream_t s, bool* handled);
+hipError_t launch_conv_mfma_f32(bool tb, const GemmParams& p, hipStream_t s);
+hipError_t launch_conv_mfma_f64(bool tb, const GemmParams& p, hipStream_t s);
+hipError_t launch_conv_mfma_f16(bool tb, const GemmParams& p, hipStream_t s);
+hipError_t launch_conv_mfma_bf16(bool tb, const GemmParams& p, hipStream_t s);
+
+hipError_t launch_conv_mfma(int dtype, bool tb, const GemmParams& p, hipStream_t s) {
+    switch (dtype) {
+    case DT_F32: return launch_conv_mfma_f32(tb, p, s);
+    case DT_F64: return launch_conv_mfma_f64(tb, p, s);
+    case DT_F16: return launch_conv_mfma_f16(tb, p, s);
+    case DT_BF16: return launch_conv_mfma_bf16(tb, p, s);
+    default: return hipErrorInvalidValue;
+    }
+}
 }  // namespace ntg
 
 namespace {
@@ -319,6 +333,38 @@ int ntg_unfold2d(int dtype, const void* image, void* col,
     return NTG_OK;
 }
 
+// The floating dtypes gather the im2col operand inside the GEMM (no col buffer) when every
+// index the kernel forms fits 32 bits with room for its out-of-range sentinels.
+static bool conv_implicit(int dtype, int64_t channels, int64_t height, int64_t width, int64_t k_r, int64_t k_c,
+                          int64_t s_r, int64_t s_c, int64_t p_r, int64_t p_c, int64_t d_r, int64_t d_c, int64_t Ho, int64_t Wo) {
+    if (is_int_dtype(dtype)) return false;
+    const int64_t lim = 1 << 24;
+    if (height >= lim || width >= lim || s_r >= lim || s_c >= lim || p_r >= lim || p_c >= lim) return false;
+    if (k_r * d_r >= lim || k_c * d_c >= lim || Ho * s_r >= lim || Wo * s_c >= lim) return false;
+    if (channels * height * width >= 0x7fffffffLL || channels * k_r * k_c >= 0x7fffffffLL || Ho * Wo >= 0x7fffffffLL) return false;
+    return channels * height * width > 0;
+}
+
+static void fill_conv_geom(ntg::ConvGeom& g, int64_t height, int64_t width, int64_t k_r, int64_t k_c, int64_t s_r, int64_t s_c,
+                           int64_t p_r, int64_t p_c, int64_t d_r, int64_t d_c, int64_t Wo) {
+    g.H = (int)height; g.W = (int)width; g.HW = (int)(height * width);
+    g.s_r = (int)s_r; g.s_c = (int)s_c; g.p_r = (int)p_r; g.p_c = (int)p_c; g.d_r = (int)d_r; g.d_c = (int)d_c;
+    g.k_c = (int)k_c; g.k_rc = (int)(k_r * k_c); g.Wo = (int)Wo;
+    g.div_krc = ntg::make_fastdiv((uint32_t)(k_r * k_c));
+    g.div_kc = ntg::make_fastdiv((uint32_t)k_c);
+    g.div_wo = ntg::make_fastdiv((uint32_t)Wo);
+}
+
+int64_t ntg_conv2d_forward_workspace_bytes(int dtype, int64_t batch, int64_t channels, int64_t height, int64_t width,
+                                           int64_t k_r, int64_t k_c, int64_t s_r, int64_t s_c,
+                                           int64_t p_r, int64_t p_c, int64_t d_r, int64_t d_c) {
+    const int64_t es = ntg::elem_size(dtype);
+    int64_t Ho, Wo;
+    if (es == 0 || unfold_out(height, width, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c, Ho, Wo)) return -1;
+    if (conv_implicit(dtype, channels, height, width, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c, Ho, Wo)) return 0;
+    return batch * channels * k_r * k_c * Ho * Wo * es;
+}
+
 int64_t ntg_conv2d_workspace_bytes(int dtype, int64_t batch, int64_t channels, int64_t height, int64_t width,
                                    int64_t k_r, int64_t k_c, int64_t s_r, int64_t s_c,
                                    int64_t p_r, int64_t p_c, int64_t d_r, int64_t d_c) {
@@ -346,16 +392,35 @@ int ntg_conv2d_dev(int dtype, const void* image, const void* kernel, void* out,
     if (rc) return rc;
     if (batch == 0 || out_channels == 0) return NTG_OK;
     if (!image || !kernel || !out) return fail(NTG_ERR_INVALID_ARGUMENT, "null pointer");
-    const int64_t need = batch * channels * k_r * k_c * Ho * Wo * es;
-    if (need > 0 && (!workspace || workspace_bytes < need))
-        return fail(NTG_ERR_INVALID_ARGUMENT, "workspace of %lld bytes needed, %lld given", (long long)need, (long long)workspace_bytes);
-    rc = ntg_unfold2d_dev(dtype, image, workspace, batch, channels, height, width, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c, stream);
-    if (rc) return rc;
     // Per image b and group g:  out_b[g*og:(g+1)*og, L] = W_g[og, add] . col_b[g*add:(g+1)*add, L].
     // The reference forms (col_b^T . W_g^T) and swaps rows/columns afterwards (conv.cpp:94);
     // each output element is the same ascending-k sum of the same products.
     const int64_t L = Ho * Wo, ckk = channels * k_r * k_c;
     const int64_t add = (channels / groups) * k_r * k_c, og = out_channels / groups;
+    if (conv_implicit(dtype, channels, height, width, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c, Ho, Wo)) {
+        // col_b is never stored: the GEMM's B loader gathers it from the image
+        for (int64_t g = 0; g < groups; ++g) {
+            ntg::GemmParams p;
+            std::memset(&p, 0, sizeof p);
+            p.M = (int)og; p.K = (int)add; p.N = (int)L; p.batch = (int)batch;
+            p.A = static_cast<const char*>(kernel) + g * og * add * es;
+            p.B = static_cast<const char*>(image) + g * (channels / groups) * height * width * es;
+            p.C = static_cast<char*>(out) + g * og * L * es;
+            p.lda = add; p.ldb = L; p.ldc = L;
+            p.sA = 0; p.sB = channels * height * width; p.sC = out_channels * L;
+            p.cmode = ntg::C_OVERWRITE;
+            p.vecA_ok = (add * es) % 16 == 0;
+            fill_conv_geom(p.conv, height, width, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c, Wo);
+            hipError_t e = ntg::launch_conv_mfma(dtype, false, p, static_cast<hipStream_t>(stream));
+            if (e != hipSuccess) return hip_fail(e, "implicit conv2d launch");
+        }
+        return NTG_OK;
+    }
+    const int64_t need = batch * channels * k_r * k_c * Ho * Wo * es;
+    if (need > 0 && (!workspace || workspace_bytes < need))
+        return fail(NTG_ERR_INVALID_ARGUMENT, "workspace of %lld bytes needed, %lld given", (long long)need, (long long)workspace_bytes);
+    rc = ntg_unfold2d_dev(dtype, image, workspace, batch, channels, height, width, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c, stream);
+    if (rc) return rc;
     for (int64_t g = 0; g < groups; ++g) {
         ntg_gemm_desc d;
         std::memset(&d, 0, sizeof d);
@@ -391,7 +456,7 @@ int ntg_conv2d(int dtype, const void* image, const void* kernel, void* out,
     const size_t im_bytes = (size_t)(batch * channels * height * width * es);
     const size_t k_bytes = (size_t)(out_channels * (channels / groups) * k_r * k_c * es);
     const size_t o_bytes = (size_t)(batch * out_channels * Ho * Wo * es);
-    const int64_t ws = ntg_conv2d_workspace_bytes(dtype, batch, channels, height, width, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c);
+    const int64_t ws = ntg_conv2d_forward_workspace_bytes(dtype, batch, channels, height, width, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c);
     DeviceMem mem;
     const size_t ok_ = align_up(im_bytes, 256), oo = ok_ + align_up(k_bytes, 256), ow = oo + align_up(o_bytes, 256);
     HIP_TRY(mem.alloc(ow + (size_t)ws));

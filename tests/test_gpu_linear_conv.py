@@ -247,6 +247,57 @@ def test_conv2d_random_vs_oracle(dtype):
         F.conv2d(dev(x), dev(w), groups=4)
 
 
+IMPLICIT_GEOMS = [
+    # (B, C, H, W, O, kh, kw, stride, padding, dilation, groups)
+    (2, 8, 20, 23, 16, 3, 3, 1, 1, 1, 1),
+    (3, 6, 17, 9, 9, 2, 4, (2, 1), (0, 3), (2, 1), 3),
+    (2, 5, 12, 12, 7, 5, 5, 2, 2, 1, 1),
+    (1, 3, 7, 31, 4, 1, 1, 1, 0, 1, 1),
+    (2, 4, 9, 9, 6, 3, 3, 3, (4, 0), (1, 2), 2),          # padding wider than the kernel reach
+    (16, 64, 28, 28, 128, 3, 3, 1, 1, 1, 1),               # enough tiles for the large-tile kernels
+    (24, 32, 33, 35, 96, 3, 3, 2, 1, 1, 2),
+]
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64, np.float16, "bf16"], ids=["fp32", "fp64", "fp16", "bf16"])
+@pytest.mark.parametrize("geom", IMPLICIT_GEOMS, ids=lambda g: "-".join(str(v).replace(" ", "") for v in g))
+def test_conv2d_implicit_gather(dtype, geom):
+    """The floating dtypes never store the unfolded matrix: the GEMM gathers it.  It must equal
+    W_g . unfold2d(x) formed explicitly (bit for bit where both use the same kernel), the oracle on
+    the small cases and torch's conv2d in double on all."""
+    B, C, H, W, O, kh, kw, s, p, d, groups = geom
+    bf = dtype == "bf16"
+    rng = np.random.default_rng(1300 + C + H)
+    x = randn(rng, (B, C, H, W), dtype)
+    w = randn(rng, (O, C // groups, kh, kw), dtype, 1.0 / np.sqrt(C // groups * kh * kw))
+    tx, tw = to_torch(x, DEV, bf), to_torch(w, DEV, bf)
+    lib = _lib.load()
+    assert lib.ntg_conv2d_forward_workspace_bytes(F.ntg_dtype(tx), B, C, H, W, kh, kw, 1, 1, 0, 0, 1, 1) == 0
+    out = F.conv2d(tx, tw, stride=s, padding=p, dilation=d, groups=groups)
+    ref = torch.nn.functional.conv2d(tx.double(), tw.double(), None, s, p, d, groups)
+    assert out.shape == ref.shape
+    K = C // groups * kh * kw
+    scale = ref.abs().max().item()
+    if dtype in (np.float32, np.float64):
+        tol = 1e-5 * K * float(tx.abs().max() * tw.abs().max())
+        assert (out.double() - ref).abs().max().item() <= tol
+        # explicit form with the same GEMM: unfold2d, then W_g . col_b per group
+        col = F.unfold2d(tx, (kh, kw), dilation=d, padding=p, stride=s)                    # [B, C*kh*kw, L]
+        og = O // groups
+        for g in range(groups):
+            wg = tw[g * og:(g + 1) * og].reshape(og, K).contiguous()
+            cg = col[:, g * K:(g + 1) * K].contiguous()
+            exp = F.matmult(wg.expand(B, og, K).contiguous(), cg)
+            got = out[:, g * og:(g + 1) * og].reshape(B, og, -1)
+            assert (got.double() - exp.double()).abs().max().item() <= tol * 1e-1
+    else:
+        assert ((out.double() - ref).abs().max().item()) <= HALF_REL * scale
+    if B * C * H * W <= 20000 and not bf:
+        oref = oracle.conv2d(x, w, s, p, d, groups)
+        err = np.abs(out.cpu().numpy().astype(np.float64) - oref.astype(np.float64)).max()
+        assert err <= (HALF_REL * scale if dtype == np.float16 else 1e-5 * K * np.abs(x).max() * np.abs(w).max())
+
+
 def test_config5a_conv2d_resnet_block():
     """image [64,256,56,56], weight [256,256,3,3], stride 1, pad 1 (GEMM M=200704, K=2304, N=256)."""
     rng = np.random.default_rng(1007)
