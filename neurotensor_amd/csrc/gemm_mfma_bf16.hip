@@ -7,11 +7,9 @@ hipError_t launch_gemm_mfma_bf16(bool ta, bool tb, const GemmParams& p, hipStrea
     if (big_tiles >= 256) return launch_trans<DT_BF16, 4, 4, 64>(ta, tb, p, s);   // 256 x 256 x 64
     return launch_trans<DT_BF16, 2, 2, 64>(ta, tb, p, s);                          // 128 x 128 x 64
 }
-// conv2d / conv_dkernel with op(B) gathered from the image (tb: col^T)
+// conv2d / conv_dkernel with op(B) gathered from the image (tb: col^T).  128 x 128 x 64 tiles, two
+// workgroups per CU: the gather's registers do not fit beside a 256 x 256 accumulator.
 hipError_t launch_conv_mfma_bf16(bool tb, const GemmParams& p, hipStream_t s) {
-    const int64_t big_tiles = (int64_t)((p.M + 255) / 256) * ((p.N + 255) / 256) * p.batch;
-    if (big_tiles >= 192)
-        return tb ? launch_conv_cfg<DT_BF16, true, 4, 4, 64>(p, s) : launch_conv_cfg<DT_BF16, false, 4, 4, 64>(p, s);
     return tb ? launch_conv_cfg<DT_BF16, true, 2, 2, 64>(p, s) : launch_conv_cfg<DT_BF16, false, 2, 2, 64>(p, s);
 }
 }  // namespace ntg

@@ -63,15 +63,21 @@ template <int R> __device__ __forceinline__ int acc_row(int r, int lane);
 template <> __device__ __forceinline__ int acc_row<32>(int r, int lane) { return 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3); }
 template <> __device__ __forceinline__ int acc_row<16>(int r, int lane) { return 4 * r + (lane >> 4); }
 
+// Pointers into the operands carry the global address space, so that their loads and stores
+// are global_* instructions (vmcnt only) and never share the LDS counter with the ds_reads.
+#define NTG_GLOBAL __attribute__((address_space(1)))
+template <class T> using gptr = const NTG_GLOBAL T*;
+template <class T> using gptr_mut = NTG_GLOBAL T*;
+
 template <class T, int VE, bool ALIGNED>
-__device__ __forceinline__ u32x4 ldvec(const T* src, bool outer_ok, int c0, int cmax, bool vec_ok) {
+__device__ __forceinline__ u32x4 ldvec(gptr<T> src, bool outer_ok, int c0, int cmax, bool vec_ok) {
     if constexpr (ALIGNED) {
-        return *reinterpret_cast<const u32x4*>(src);
+        return *reinterpret_cast<gptr<u32x4>>(src);
     } else {
         u32x4 r = {0u, 0u, 0u, 0u};
         if (outer_ok) {
             if (vec_ok && c0 + VE <= cmax) {
-                r = *reinterpret_cast<const u32x4*>(src);
+                r = *reinterpret_cast<gptr<u32x4>>(src);
             } else {
                 T tmp[VE];
 #pragma unroll
@@ -83,33 +89,65 @@ __device__ __forceinline__ u32x4 ldvec(const T* src, bool outer_ok, int c0, int 
     }
 }
 
-// Implicit im2col: one 16-byte vector of VE consecutive l (output pixels) of row kk (channel, tap)
-// of the matrix described by ConvGeom, gathered from the image.  Loads are unconditional (a
-// clamped address, then a select) so that all of a tile's loads are in flight together.
-template <class T, int VE>
-__device__ __forceinline__ u32x4 conv_gather(const T* __restrict__ im, const ConvGeom& g, int kk, bool kk_ok, int l0, int l_end) {
+// Implicit im2col.  Element (kk, l) of the never-stored matrix described by ConvGeom is
+//   im[c, oh*s_r - p_r + r*d_r, ow*s_c - p_c + q*d_c]     kk = (c, r, q),  l = (oh, ow)
+// Its coordinates and byte offset split into a part that depends on kk only (ConvRow) and a part
+// that depends on l only (ConvCol); whichever of the two is fixed for a thread over the whole
+// k loop is computed once.  Indices outside the matrix get coordinates far outside the image,
+// so they read as padding.
+struct ConvRow { uint32_t roff; int dh, dw; };
+struct ConvCol { uint32_t off0; int ih0, iw0; };
+
+template <class T>
+__device__ __forceinline__ ConvRow conv_row(const ConvGeom& g, int kk, bool valid) {
     const uint32_t c = fast_div((uint32_t)kk, g.div_krc);
-    const uint32_t rem = (uint32_t)kk - c * (uint32_t)g.k_rc;
+    const uint32_t rem = (uint32_t)kk - __umul24(c, (uint32_t)g.k_rc);
     const uint32_t r = fast_div(rem, g.div_kc);
-    const uint32_t q = rem - r * (uint32_t)g.k_c;
-    const int base = (int)c * g.HW;
-    const int dh = kk_ok ? (int)r * g.d_r - g.p_r : -(1 << 29);   // far outside the image => every tap reads as padding
-    const int dw = (int)q * g.d_c - g.p_c;
-    T tmp[VE];
+    const uint32_t q = rem - __umul24(r, (uint32_t)g.k_c);
+    ConvRow o;
+    o.dh = valid ? (int)__umul24(r, (uint32_t)g.d_r) - g.p_r : -(1 << 29);
+    o.dw = (int)__umul24(q, (uint32_t)g.d_c) - g.p_c;
+    o.roff = (c * (uint32_t)g.HW + (uint32_t)o.dh * (uint32_t)g.W + (uint32_t)o.dw) * (uint32_t)sizeof(T);
+    return o;
+}
+
+template <class T>
+__device__ __forceinline__ ConvCol conv_col(const ConvGeom& g, int l, bool valid) {
+    const uint32_t oh = fast_div((uint32_t)l, g.div_wo);
+    const uint32_t ow = (uint32_t)l - oh * (uint32_t)g.Wo;
+    ConvCol o;
+    o.ih0 = valid ? (int)__umul24(oh, (uint32_t)g.s_r) : -(1 << 29);
+    o.iw0 = (int)__umul24(ow, (uint32_t)g.s_c);
+    o.off0 = ((uint32_t)o.ih0 * (uint32_t)g.W + (uint32_t)o.iw0) * (uint32_t)sizeof(T);
+    return o;
+}
+
+// One element of the gather.  The load is unconditional (padding reads element 0 instead) and
+// nothing here consumes the loaded value, so all of a tile's loads stay in flight; `ok` goes into
+// a bit mask and conv_mask() zeroes the padding when the tile is written to LDS.
+template <class T>
+__device__ __forceinline__ T conv_load(gptr<T> im, const ConvGeom& g, const ConvRow& row, const ConvCol& col, bool& ok) {
+    const int ih = col.ih0 + row.dh;
+    const int iw = col.iw0 + row.dw;
+    ok = ((unsigned)ih < (unsigned)g.H) & ((unsigned)iw < (unsigned)g.W);   // no short circuit: keeps the gather branch-free
+    const uint32_t boff = ok ? col.off0 + row.roff : 0u;
+    return *reinterpret_cast<gptr<T>>(reinterpret_cast<gptr<char>>(im) + boff);
+}
+
+template <class T, int VE>
+__device__ __forceinline__ u32x4 conv_mask(u32x4 v, uint32_t okm) {
+    auto bit = [&](int e) { return (uint32_t)(((int32_t)(okm << (31 - e))) >> 31); };   // all ones / all zeros
+    if constexpr (sizeof(T) == 4) {
 #pragma unroll
-    for (int e = 0; e < VE; ++e) {
-        const int l = l0 + e;
-        const uint32_t oh = fast_div((uint32_t)l, g.div_wo);
-        const uint32_t ow = (uint32_t)l - oh * (uint32_t)g.Wo;
-        const int ih = (l < l_end ? (int)oh * g.s_r : -(1 << 29)) + dh;
-        const int iw = (int)ow * g.s_c + dw;
-        const bool ok = (unsigned)ih < (unsigned)g.H && (unsigned)iw < (unsigned)g.W;
-        const T v = im[ok ? base + ih * g.W + iw : 0];
-        tmp[e] = ok ? v : (T)0.0f;
+        for (int e = 0; e < 4; ++e) v[e] &= bit(e);
+    } else if constexpr (sizeof(T) == 8) {
+#pragma unroll
+        for (int e = 0; e < 2; ++e) { v[2 * e] &= bit(e); v[2 * e + 1] &= bit(e); }
+    } else {
+#pragma unroll
+        for (int d = 0; d < 4; ++d) v[d] &= __builtin_amdgcn_perm(bit(2 * d + 1), bit(2 * d), 0x07060100u);
     }
-    u32x4 out;
-    __builtin_memcpy(&out, tmp, 16);
-    return out;
+    return v;
 }
 
 // One operand's BMN x BK tile: global -> registers -> LDS.
@@ -133,7 +171,7 @@ struct TileLoader {
 
     u32x4 v[NV];
 
-    __device__ __forceinline__ void load(const T* base, int64_t ld, int mn0, int k0, int MN, int K, bool vec_ok, int tid) {
+    __device__ __forceinline__ void load(gptr<T> base, int64_t ld, int mn0, int k0, int MN, int K, bool vec_ok, int tid) {
         if constexpr (!TRANSPOSE && KC) {
 #pragma unroll
             for (int p = 0; p < NV; ++p) {
@@ -167,38 +205,103 @@ struct TileLoader {
         }
     }
 
-    // Same tile, but the operand is the never-stored im2col matrix of `im`: the "rows" the
-    // vectors run along are output pixels l, the other index is kk = (channel, tap).
+    // Same tile, but the operand is the never-stored im2col matrix of `im`: the vectors run
+    // along output pixels l, the other index is kk = (channel, tap).
     //   !KC: tile = col[k0.., mn0..]   (k = kk, mn = l)      KC: tile = col^T  (mn = kk, k = l)
-    __device__ __forceinline__ void load_conv(const T* im, const ConvGeom& g, int mn0, int k0, int MN, int K, int tid) {
+    // conv_setup() computes what stays fixed for the thread, load_conv() gathers one tile and
+    // conv_finish() zeroes the padding before store().
+    static constexpr int NFIX = !KC ? (TRANSPOSE ? NQ * 8 : VE) : NV;
+    static constexpr int NE = NV * VE;              // elements a thread gathers per tile
+    ConvCol ccol[!KC ? NFIX : VE];                  // !KC: fixed columns;  KC: this tile's columns
+    ConvRow crow[KC ? NFIX : 1];                    //  KC: fixed rows;    !KC: the row being gathered
+    uint32_t okm[NV];
+    uint32_t raw16[sizeof(T) == 2 ? NV * VE : 1];
+
+    __device__ __forceinline__ void conv_setup(const ConvGeom& g, int mn0, int MN, int tid) {
         if constexpr (!TRANSPOSE && KC) {
+            static_assert(256 % KV == 0, "a thread keeps the same k offsets for every vector it loads");
 #pragma unroll
             for (int p = 0; p < NV; ++p) {
-                const int vi = tid + p * 256;
-                const int row = vi / KV, kv = vi % KV;
-                v[p] = conv_gather<T, VE>(im, g, mn0 + row, mn0 + row < MN, k0 + kv * VE, K);
+                const int row = (tid + p * 256) / KV;
+                crow[p] = conv_row<T>(g, mn0 + row, mn0 + row < MN);
             }
         } else if constexpr (!TRANSPOSE) {
+            static_assert(256 % MV == 0, "a thread keeps the same columns for every vector it loads");
+            const int mv = tid % MV;
 #pragma unroll
-            for (int p = 0; p < NV; ++p) {
-                const int vi = tid + p * 256;
-                const int kr = vi / MV, mv = vi % MV;
-                v[p] = conv_gather<T, VE>(im, g, k0 + kr, k0 + kr < K, mn0 + mv * VE, MN);
-            }
+            for (int e = 0; e < VE; ++e) ccol[e] = conv_col<T>(g, mn0 + mv * VE + e, mn0 + mv * VE + e < MN);
         } else {
 #pragma unroll
             for (int q = 0; q < NQ; ++q) {
-                const int sb = tid + q * 256;
-                if (NSB % 256 == 0 || sb < NSB) {
-                    const int kg = sb % KG, mv = sb / KG;
+                const int mv = (tid + q * 256) / KG;      // threads past NSB sub-blocks compute unused columns
 #pragma unroll
-                    for (int i = 0; i < 8; ++i) {
-                        const int k = k0 + kg * 8 + i;
-                        v[q * 8 + i] = conv_gather<T, VE>(im, g, k, k < K, mn0 + mv * 8, MN);
-                    }
-                }
+                for (int e = 0; e < 8; ++e) ccol[q * 8 + e] = conv_col<T>(g, mn0 + mv * 8 + e, mn0 + mv * 8 + e < MN);
             }
         }
+    }
+
+    // element idx (0 .. NE-1, a compile-time constant after unrolling) of the tile at k0
+    __device__ __forceinline__ void conv_elem(int idx, gptr<T> im, const ConvGeom& g, int k0, int K, int tid) {
+        const int pv = idx / VE, e = idx % VE;
+        if constexpr (TRANSPOSE && NSB % 256 != 0) {
+            if (tid + (pv / 8) * 256 >= NSB) return;      // whole wavefronts: this thread owns no sub-block here
+        }
+        bool ok;
+        T x;
+        if constexpr (!TRANSPOSE && KC) {
+            if (idx == 0) {
+                const int kv = tid % KV;
+#pragma unroll
+                for (int c = 0; c < VE; ++c) ccol[c] = conv_col<T>(g, k0 + kv * VE + c, k0 + kv * VE + c < K);
+            }
+            x = conv_load<T>(im, g, crow[pv], ccol[e], ok);
+        } else if constexpr (!TRANSPOSE) {
+            if (e == 0) {
+                const int kr = (tid + pv * 256) / MV;
+                crow[0] = conv_row<T>(g, k0 + kr, k0 + kr < K);
+            }
+            x = conv_load<T>(im, g, crow[0], ccol[e], ok);
+        } else {
+            const int q = pv / 8, i = pv % 8;
+            if (e == 0) {
+                const int k = k0 + ((tid + q * 256) % KG) * 8 + i;
+                crow[0] = conv_row<T>(g, k, k < K);
+            }
+            x = conv_load<T>(im, g, crow[0], ccol[q * 8 + e], ok);
+        }
+        if (e == 0) okm[pv] = 0;
+        okm[pv] |= ok ? (1u << e) : 0u;
+        if constexpr (sizeof(T) == 4) {
+            v[pv][e] = __builtin_bit_cast(uint32_t, x);
+        } else if constexpr (sizeof(T) == 8) {
+            const uint64_t bits = __builtin_bit_cast(uint64_t, x);
+            v[pv][2 * e] = (uint32_t)bits;
+            v[pv][2 * e + 1] = (uint32_t)(bits >> 32);
+        } else {
+            raw16[idx] = __builtin_bit_cast(uint16_t, x);   // packed in conv_finish(): packing here would wait for the load
+        }
+    }
+
+    // slice s of ns of a tile's gather: the kernel spreads the slices between its MFMAs
+    __device__ __forceinline__ void conv_slice(int s, int ns, gptr<T> im, const ConvGeom& g, int k0, int K, int tid) {
+#pragma unroll
+        for (int idx = 0; idx < NE; ++idx)
+            if (idx >= s * NE / ns && idx < (s + 1) * NE / ns) conv_elem(idx, im, g, k0, K, tid);
+    }
+
+    __device__ __forceinline__ void load_conv(gptr<T> im, const ConvGeom& g, int k0, int K, int tid) {
+        conv_slice(0, 1, im, g, k0, K, tid);
+    }
+
+    __device__ __forceinline__ void conv_finish() {
+        if constexpr (sizeof(T) == 2) {
+#pragma unroll
+            for (int p = 0; p < NV; ++p)
+#pragma unroll
+                for (int d = 0; d < 4; ++d) v[p][d] = raw16[p * 8 + 2 * d] | (raw16[p * 8 + 2 * d + 1] << 16);
+        }
+#pragma unroll
+        for (int p = 0; p < NV; ++p) v[p] = conv_mask<T, VE>(v[p], okm[p]);
     }
 
     __device__ __forceinline__ void store(char* lds, int tid) const {
@@ -287,9 +390,9 @@ __global__ void __launch_bounds__(256) gemm_mfma_kernel(const GemmParams p) {
     tile_coords(lid - b * tiles, p.tiles_m, p.tiles_n, SH::GROUP_M, tm, tn);
     const int m0 = tm * BM, n0 = tn * BN;
 
-    const T* A = p.Aptr ? static_cast<const T*>(p.Aptr[b]) : static_cast<const T*>(p.A) + (int64_t)b * p.sA;
-    const T* B = p.Bptr ? static_cast<const T*>(p.Bptr[b]) : static_cast<const T*>(p.B) + (int64_t)b * p.sB;
-    T* C = p.Cptr ? static_cast<T*>(p.Cptr[b]) : static_cast<T*>(p.C) + (int64_t)b * p.sC;
+    const gptr<T> A = (gptr<T>)(p.Aptr ? static_cast<const T*>(((gptr<const void*>)p.Aptr)[b]) : static_cast<const T*>(p.A) + (int64_t)b * p.sA);
+    const gptr<T> B = (gptr<T>)(p.Bptr ? static_cast<const T*>(((gptr<const void*>)p.Bptr)[b]) : static_cast<const T*>(p.B) + (int64_t)b * p.sB);
+    const gptr_mut<T> C = (gptr_mut<T>)(p.Cptr ? static_cast<T*>(((gptr<void*>)p.Cptr)[b]) : static_cast<T*>(p.C) + (int64_t)b * p.sC);
     const bool vecA = p.vecA_ok && ((reinterpret_cast<uintptr_t>(A) & 15) == 0);
     const bool vecB = p.vecB_ok && ((reinterpret_cast<uintptr_t>(B) & 15) == 0);
 
@@ -306,12 +409,14 @@ __global__ void __launch_bounds__(256) gemm_mfma_kernel(const GemmParams p) {
     const int KT = (p.K + BK - 1) / BK;
 
     auto load_b = [&](int k0) {
-        if constexpr (CONV) lb.load_conv(B, p.conv, n0, k0, p.N, p.K, tid);
+        if constexpr (CONV) lb.load_conv(B, p.conv, k0, p.K, tid);
         else lb.load(B, p.ldb, n0, k0, p.N, p.K, vecB, tid);
     };
+    if constexpr (CONV) lb.conv_setup(p.conv, n0, p.N, tid);
 
     la.load(A, p.lda, m0, 0, p.M, p.K, vecA, tid);
     load_b(0);
+    if constexpr (CONV) lb.conv_finish();
     la.store(smem, tid);
     lb.store(smem + SH::LDS_A, tid);
     __syncthreads();
@@ -319,11 +424,24 @@ __global__ void __launch_bounds__(256) gemm_mfma_kernel(const GemmParams p) {
     for (int kt = 0; kt < KT; ++kt) {
         const char* sA = smem + (kt & 1) * SH::STAGE;
         const char* sB = sA + SH::LDS_A;
-        const bool more = (kt + 1 < KT);
+        // The gathering kernels load unconditionally (the last pass re-reads the last tile into the
+        // idle stage), so that the loop body is one scheduling region and the address arithmetic
+        // of the gather can sit in the shadow of the MFMAs.
+        const bool more = CONV || (kt + 1 < KT);
+        const int k_next = (CONV && kt + 1 >= KT ? kt : kt + 1) * BK;
         if (more) {
-            la.load(A, p.lda, m0, (kt + 1) * BK, p.M, p.K, vecA, tid);
-            load_b((kt + 1) * BK);
+            la.load(A, p.lda, m0, k_next, p.M, p.K, vecA, tid);
+            if constexpr (!CONV) load_b(k_next);
         }
+        // CONV: slice `step` of NSTEP of the next tile's gather follows each group of MFMAs; only LDS
+        // reads and scalar work may move across the fence, so the slice stays with its group.
+        constexpr int NSTEP = IS16 ? BK / 16 : BK / G;
+        auto gather_slice = [&](int step) {
+            if constexpr (CONV) {
+                lb.conv_slice(step, NSTEP, B, p.conv, k_next, p.K, tid);
+                __builtin_amdgcn_sched_barrier(0x104);
+            }
+        };
 
         if constexpr (IS16) {
             constexpr int KQ = BK / 16;
@@ -340,6 +458,7 @@ __global__ void __launch_bounds__(256) gemm_mfma_kernel(const GemmParams p) {
                 for (int i = 0; i < WBM; ++i)
 #pragma unroll
                     for (int j = 0; j < WBN; ++j) E::mma(acc[i][j], af[i], bf[j]);
+                gather_slice(kq);
             }
         } else {
             constexpr int KQ = BK / (G * VE);
@@ -382,16 +501,22 @@ __global__ void __launch_bounds__(256) gemm_mfma_kernel(const GemmParams p) {
                     }
                 }
 #pragma unroll
-                for (int e = 0; e < VE; ++e)
+                for (int e = 0; e < VE; ++e) {
 #pragma unroll
                     for (int i = 0; i < WBM; ++i)
 #pragma unroll
                         for (int j = 0; j < WBN; ++j) E::mma(acc[i][j], af[i][e], bf[j][e]);
+                    gather_slice(kq * VE + e);
+                }
             }
         }
-
         if (more) {
             char* dA = smem + ((kt + 1) & 1) * SH::STAGE;
+            if constexpr (CONV) {
+                // the gathered values are first touched here, after the MFMAs of this tile
+                __builtin_amdgcn_sched_barrier(0);
+                lb.conv_finish();
+            }
             la.store(dA, tid);
             lb.store(dA + SH::LDS_A, tid);
         }
@@ -401,7 +526,7 @@ __global__ void __launch_bounds__(256) gemm_mfma_kernel(const GemmParams p) {
     // epilogue: every lane owns ACCN elements per block; C0 comes from C (accumulate),
     // from the broadcast bias (linear) or is zero (overwrite)
     const int cmode = p.cmode;
-    const T* bias = static_cast<const T*>(p.bias);
+    const gptr<T> bias = (gptr<T>)static_cast<const T*>(p.bias);
 #pragma unroll
     for (int i = 0; i < WBM; ++i) {
 #pragma unroll
@@ -411,8 +536,8 @@ __global__ void __launch_bounds__(256) gemm_mfma_kernel(const GemmParams p) {
             for (int r = 0; r < E::ACCN; ++r) {
                 const int lrow = acc_row<R>(r, lane);
                 const int m = m0 + (A_KM ? (wm * WBM + i) * R + lrow : (wm * R + lrow) * WBM + i);
-                if (ALIGNED || (m < p.M && n < p.N)) {
-                    T* cp = C + (int64_t)m * p.ldc + n;
+                if ((ALIGNED && !CONV) || (m < p.M && n < p.N)) {
+                    const gptr_mut<T> cp = C + (int64_t)m * p.ldc + n;
                     AccS val = acc[i][j][r];
                     if (cmode == C_ACCUMULATE) val += (AccS)(*cp);
                     else if (cmode == C_BIAS) val += (AccS)bias[(int64_t)b * p.bias_bs + (int64_t)m * p.bias_rs + (int64_t)n * p.bias_cs];
@@ -452,7 +577,8 @@ static hipError_t launch_cfg(const GemmParams& pin, hipStream_t s) {
     return hipGetLastError();
 }
 
-// op(B) = implicit im2col matrix (TB: transposed); always the guarded kernel
+// op(B) = implicit im2col matrix (TB: transposed).  ALIGNED here speaks of A only (whole tiles,
+// 16-byte rows); the gathered operand and the stores are always guarded.
 template <int DT, bool TB, int WBM, int WBN, int BK>
 static hipError_t launch_conv_cfg(const GemmParams& pin, hipStream_t s) {
     using SH = GemmShape<DT, false, TB, WBM, WBN, BK>;
@@ -462,10 +588,20 @@ static hipError_t launch_conv_cfg(const GemmParams& pin, hipStream_t s) {
     const int64_t blocks = (int64_t)p.tiles_m * p.tiles_n * p.batch;
     if (blocks <= 0) return hipSuccess;
     if (blocks > 0x7fffffffLL) return hipErrorInvalidValue;
-    auto k = gemm_mfma_kernel<DT, false, TB, WBM, WBN, BK, false, true>;
-    static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(k), hipFuncAttributeMaxDynamicSharedMemorySize, SH::LDS_TOTAL);
-    if (attr != hipSuccess) return attr;
-    hipLaunchKernelGGL(k, dim3((unsigned)blocks), dim3(256), SH::LDS_TOTAL, s, p);
+    constexpr int VE = Elem<DT>::VE;
+    const bool a_aligned = (p.M % SH::BM == 0) && (p.K % BK == 0) && p.vecA_ok && !p.Aptr &&
+                           ((reinterpret_cast<uintptr_t>(p.A) & 15) == 0) && (p.sA % VE == 0);
+    if (a_aligned) {
+        auto k = gemm_mfma_kernel<DT, false, TB, WBM, WBN, BK, true, true>;
+        static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(k), hipFuncAttributeMaxDynamicSharedMemorySize, SH::LDS_TOTAL);
+        if (attr != hipSuccess) return attr;
+        hipLaunchKernelGGL(k, dim3((unsigned)blocks), dim3(256), SH::LDS_TOTAL, s, p);
+    } else {
+        auto k = gemm_mfma_kernel<DT, false, TB, WBM, WBN, BK, false, true>;
+        static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(k), hipFuncAttributeMaxDynamicSharedMemorySize, SH::LDS_TOTAL);
+        if (attr != hipSuccess) return attr;
+        hipLaunchKernelGGL(k, dim3((unsigned)blocks), dim3(256), SH::LDS_TOTAL, s, p);
+    }
     return hipGetLastError();
 }
 

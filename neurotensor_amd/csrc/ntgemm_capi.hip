@@ -341,7 +341,9 @@ static bool conv_implicit(int dtype, int64_t channels, int64_t height, int64_t w
     const int64_t lim = 1 << 24;
     if (height >= lim || width >= lim || s_r >= lim || s_c >= lim || p_r >= lim || p_c >= lim) return false;
     if (k_r * d_r >= lim || k_c * d_c >= lim || Ho * s_r >= lim || Wo * s_c >= lim) return false;
-    if (channels * height * width >= 0x7fffffffLL || channels * k_r * k_c >= 0x7fffffffLL || Ho * Wo >= 0x7fffffffLL) return false;
+    if (channels >= lim || k_r * k_c >= lim) return false;
+    // byte offsets inside one image are formed in 32 bits
+    if (channels * height * width * ntg::elem_size(dtype) >= 0x7fffffffLL || channels * k_r * k_c >= 0x7fffffffLL || Ho * Wo >= 0x7fffffffLL) return false;
     return channels * height * width > 0;
 }
 
