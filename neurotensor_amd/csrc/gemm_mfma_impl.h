@@ -91,22 +91,25 @@ __device__ __forceinline__ u32x4 ldvec(gptr<T> src, bool outer_ok, int c0, int c
 
 // Implicit im2col.  Element (kk, l) of the never-stored matrix described by ConvGeom is
 //   im[c, oh*s_r - p_r + r*d_r, ow*s_c - p_c + q*d_c]     kk = (c, r, q),  l = (oh, ow)
-// Its coordinates and byte offset split into a part that depends on kk only (ConvRow) and a part
-// that depends on l only (ConvCol); whichever of the two is fixed for a thread over the whole
-// k loop is computed once.  Indices outside the matrix get coordinates far outside the image,
-// so they read as padding.
-struct ConvRow { uint32_t roff; int dh, dw; };
+// Its byte offset is the sum of a term in kk (ConvRow::roff) and a term in l (ConvCol::off0);
+// whichever of the two is fixed for a thread over the whole k loop is computed once.
+// Every load is unconditional: the offset is clamped into the image (a padding tap reads some
+// neighbouring element), nothing consumes the value, so all of a tile's loads stay in flight; one
+// bit per element says whether it is real, and conv_mask() zeroes the rest when the tile is
+// written to LDS.  The bit of element e sits at bit 8*(e%4) of mask word e/4.
+struct ConvRow { uint32_t roff, r, q; int dh, dw; bool valid; };
 struct ConvCol { uint32_t off0; int ih0, iw0; };
 
 template <class T>
 __device__ __forceinline__ ConvRow conv_row(const ConvGeom& g, int kk, bool valid) {
     const uint32_t c = fast_div((uint32_t)kk, g.div_krc);
     const uint32_t rem = (uint32_t)kk - __umul24(c, (uint32_t)g.k_rc);
-    const uint32_t r = fast_div(rem, g.div_kc);
-    const uint32_t q = rem - __umul24(r, (uint32_t)g.k_c);
     ConvRow o;
-    o.dh = valid ? (int)__umul24(r, (uint32_t)g.d_r) - g.p_r : -(1 << 29);
-    o.dw = (int)__umul24(q, (uint32_t)g.d_c) - g.p_c;
+    o.r = fast_div(rem, g.div_kc);
+    o.q = rem - __umul24(o.r, (uint32_t)g.k_c);
+    o.valid = valid;
+    o.dh = valid ? (int)__umul24(o.r, (uint32_t)g.d_r) - g.p_r : -(1 << 29);   // far outside: every tap is padding
+    o.dw = (int)__umul24(o.q, (uint32_t)g.d_c) - g.p_c;
     o.roff = (c * (uint32_t)g.HW + (uint32_t)o.dh * (uint32_t)g.W + (uint32_t)o.dw) * (uint32_t)sizeof(T);
     return o;
 }
@@ -122,21 +125,30 @@ __device__ __forceinline__ ConvCol conv_col(const ConvGeom& g, int l, bool valid
     return o;
 }
 
-// One element of the gather.  The load is unconditional (padding reads element 0 instead) and
-// nothing here consumes the loaded value, so all of a tile's loads stay in flight; `ok` goes into
-// a bit mask and conv_mask() zeroes the padding when the tile is written to LDS.
+// For a fixed column: bit r of `hm` / bit q of `wm` say whether tap row r / tap column q falls
+// inside the image (kernels up to 8 x 8; larger ones use the stored im2col matrix).
+__device__ __forceinline__ void conv_tap_masks(const ConvGeom& g, const ConvCol& col, uint32_t& hm, uint32_t& wm) {
+    hm = 0;
+    wm = 0;
+#pragma unroll
+    for (int t = 0; t < 8; ++t) {
+        hm |= ((t < g.k_r) & ((unsigned)(col.ih0 + t * g.d_r - g.p_r) < (unsigned)g.H)) ? (1u << t) : 0u;
+        wm |= ((t < g.k_c) & ((unsigned)(col.iw0 + t * g.d_c - g.p_c) < (unsigned)g.W)) ? (1u << t) : 0u;
+    }
+}
+
 template <class T>
-__device__ __forceinline__ T conv_load(gptr<T> im, const ConvGeom& g, const ConvRow& row, const ConvCol& col, bool& ok) {
-    const int ih = col.ih0 + row.dh;
-    const int iw = col.iw0 + row.dw;
-    ok = ((unsigned)ih < (unsigned)g.H) & ((unsigned)iw < (unsigned)g.W);   // no short circuit: keeps the gather branch-free
-    const uint32_t boff = ok ? col.off0 + row.roff : 0u;
-    return *reinterpret_cast<gptr<T>>(reinterpret_cast<gptr<char>>(im) + boff);
+__device__ __forceinline__ T conv_load(gptr<T> im, const ConvGeom& g, uint32_t off) {
+    const int lim = g.last * (int)sizeof(T);
+    int boff = (int)off;
+    boff = boff < 0 ? 0 : boff;
+    boff = boff > lim ? lim : boff;
+    return *reinterpret_cast<gptr<T>>(reinterpret_cast<gptr<char>>(im) + (uint32_t)boff);
 }
 
 template <class T, int VE>
-__device__ __forceinline__ u32x4 conv_mask(u32x4 v, uint32_t okm) {
-    auto bit = [&](int e) { return (uint32_t)(((int32_t)(okm << (31 - e))) >> 31); };   // all ones / all zeros
+__device__ __forceinline__ u32x4 conv_mask(u32x4 v, const uint32_t* okm) {
+    auto bit = [&](int e) { return (uint32_t)(((int32_t)(okm[e >> 2] << (31 - 8 * (e & 3)))) >> 31); };   // all ones / all zeros
     if constexpr (sizeof(T) == 4) {
 #pragma unroll
         for (int e = 0; e < 4; ++e) v[e] &= bit(e);
@@ -212,9 +224,13 @@ struct TileLoader {
     // conv_finish() zeroes the padding before store().
     static constexpr int NFIX = !KC ? (TRANSPOSE ? NQ * 8 : VE) : NV;
     static constexpr int NE = NV * VE;              // elements a thread gathers per tile
-    ConvCol ccol[!KC ? NFIX : VE];                  // !KC: fixed columns;  KC: this tile's columns
+    static constexpr int NW = (VE + 3) / 4;         // mask words per vector
+    uint32_t coff[!KC ? NFIX : 1];                  // !KC: byte offsets of the thread's fixed columns ...
+    uint32_t hpk[!KC ? (NFIX + 3) / 4 : 1];         //      ... and their tap masks, 8 bits per column
+    uint32_t wpk[!KC ? (NFIX + 3) / 4 : 1];
+    ConvCol ccol[KC ? VE : 1];                      //  KC: this tile's columns
     ConvRow crow[KC ? NFIX : 1];                    //  KC: fixed rows;    !KC: the row being gathered
-    uint32_t okm[NV];
+    uint32_t okm[NV][NW];
     uint32_t raw16[sizeof(T) == 2 ? NV * VE : 1];
 
     __device__ __forceinline__ void conv_setup(const ConvGeom& g, int mn0, int MN, int tid) {
@@ -225,17 +241,20 @@ struct TileLoader {
                 const int row = (tid + p * 256) / KV;
                 crow[p] = conv_row<T>(g, mn0 + row, mn0 + row < MN);
             }
-        } else if constexpr (!TRANSPOSE) {
-            static_assert(256 % MV == 0, "a thread keeps the same columns for every vector it loads");
-            const int mv = tid % MV;
-#pragma unroll
-            for (int e = 0; e < VE; ++e) ccol[e] = conv_col<T>(g, mn0 + mv * VE + e, mn0 + mv * VE + e < MN);
         } else {
+            static_assert(TRANSPOSE || 256 % MV == 0, "a thread keeps the same columns for every vector it loads");
 #pragma unroll
-            for (int q = 0; q < NQ; ++q) {
-                const int mv = (tid + q * 256) / KG;      // threads past NSB sub-blocks compute unused columns
+            for (int i = 0; i < (NFIX + 3) / 4; ++i) hpk[i] = wpk[i] = 0;
 #pragma unroll
-                for (int e = 0; e < 8; ++e) ccol[q * 8 + e] = conv_col<T>(g, mn0 + mv * 8 + e, mn0 + mv * 8 + e < MN);
+            for (int i = 0; i < NFIX; ++i) {
+                // threads past NSB sub-blocks compute columns they never use
+                const int l = TRANSPOSE ? mn0 + ((tid + (i / 8) * 256) / KG) * 8 + (i % 8) : mn0 + (tid % MV) * VE + i;
+                const ConvCol c = conv_col<T>(g, l, l < MN);
+                uint32_t hm, wm;
+                conv_tap_masks(g, c, hm, wm);
+                coff[i] = c.off0;
+                hpk[i / 4] |= hm << (8 * (i % 4));
+                wpk[i / 4] |= wm << (8 * (i % 4));
             }
         }
     }
@@ -246,7 +265,6 @@ struct TileLoader {
         if constexpr (TRANSPOSE && NSB % 256 != 0) {
             if (tid + (pv / 8) * 256 >= NSB) return;      // whole wavefronts: this thread owns no sub-block here
         }
-        bool ok;
         T x;
         if constexpr (!TRANSPOSE && KC) {
             if (idx == 0) {
@@ -254,23 +272,24 @@ struct TileLoader {
 #pragma unroll
                 for (int c = 0; c < VE; ++c) ccol[c] = conv_col<T>(g, k0 + kv * VE + c, k0 + kv * VE + c < K);
             }
-            x = conv_load<T>(im, g, crow[pv], ccol[e], ok);
-        } else if constexpr (!TRANSPOSE) {
-            if (e == 0) {
-                const int kr = (tid + pv * 256) / MV;
-                crow[0] = conv_row<T>(g, k0 + kr, k0 + kr < K);
-            }
-            x = conv_load<T>(im, g, crow[0], ccol[e], ok);
+            const int ih = ccol[e].ih0 + crow[pv].dh;
+            const int iw = ccol[e].iw0 + crow[pv].dw;
+            const bool ok = ((unsigned)ih < (unsigned)g.H) & ((unsigned)iw < (unsigned)g.W);   // no short circuit: branch-free
+            if (e % 4 == 0) okm[pv][e / 4] = 0;
+            okm[pv][e / 4] |= ok ? (1u << (8 * (e % 4))) : 0u;
+            x = conv_load<T>(im, g, ccol[e].off0 + crow[pv].roff);
         } else {
-            const int q = pv / 8, i = pv % 8;
+            const int cb = TRANSPOSE ? (pv / 8) * 8 : 0;      // first fixed column of this vector
             if (e == 0) {
-                const int k = k0 + ((tid + q * 256) % KG) * 8 + i;
-                crow[0] = conv_row<T>(g, k, k < K);
+                const int kk = TRANSPOSE ? k0 + ((tid + (pv / 8) * 256) % KG) * 8 + (pv % 8) : k0 + (tid + pv * 256) / MV;
+                crow[0] = conv_row<T>(g, kk, kk < K);
             }
-            x = conv_load<T>(im, g, crow[0], ccol[q * 8 + e], ok);
+            if (e % 4 == 0) {
+                const uint32_t m = (hpk[(cb + e) / 4] >> crow[0].r) & (wpk[(cb + e) / 4] >> crow[0].q) & 0x01010101u;
+                okm[pv][e / 4] = crow[0].valid ? m : 0u;
+            }
+            x = conv_load<T>(im, g, coff[cb + e] + crow[0].roff);
         }
-        if (e == 0) okm[pv] = 0;
-        okm[pv] |= ok ? (1u << e) : 0u;
         if constexpr (sizeof(T) == 4) {
             v[pv][e] = __builtin_bit_cast(uint32_t, x);
         } else if constexpr (sizeof(T) == 8) {

@@ -41,7 +41,8 @@ static inline FastDiv make_fastdiv(uint32_t d) {
 struct ConvGeom {
     int H, W, HW;
     int s_r, s_c, p_r, p_c, d_r, d_c;
-    int k_c, k_rc, Wo;
+    int k_r, k_c, k_rc, Wo;
+    int last;                // index of the last element of the image slice at p.B (loads are clamped to it)
     FastDiv div_krc, div_kc, div_wo;
 };
 

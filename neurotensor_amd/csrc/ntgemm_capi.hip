@@ -338,6 +338,7 @@ int ntg_unfold2d(int dtype, const void* image, void* col,
 static bool conv_implicit(int dtype, int64_t channels, int64_t height, int64_t width, int64_t k_r, int64_t k_c,
                           int64_t s_r, int64_t s_c, int64_t p_r, int64_t p_c, int64_t d_r, int64_t d_c, int64_t Ho, int64_t Wo) {
     if (is_int_dtype(dtype)) return false;
+    if (k_r > 8 || k_c > 8) return false;   // the kernels keep one byte of tap mask per output pixel
     const int64_t lim = 1 << 24;
     if (height >= lim || width >= lim || s_r >= lim || s_c >= lim || p_r >= lim || p_c >= lim) return false;
     if (k_r * d_r >= lim || k_c * d_c >= lim || Ho * s_r >= lim || Wo * s_c >= lim) return false;
@@ -347,11 +348,12 @@ static bool conv_implicit(int dtype, int64_t channels, int64_t height, int64_t w
     return channels * height * width > 0;
 }
 
-static void fill_conv_geom(ntg::ConvGeom& g, int64_t height, int64_t width, int64_t k_r, int64_t k_c, int64_t s_r, int64_t s_c,
+static void fill_conv_geom(ntg::ConvGeom& g, int64_t slice_channels, int64_t height, int64_t width, int64_t k_r, int64_t k_c, int64_t s_r, int64_t s_c,
                            int64_t p_r, int64_t p_c, int64_t d_r, int64_t d_c, int64_t Wo) {
     g.H = (int)height; g.W = (int)width; g.HW = (int)(height * width);
     g.s_r = (int)s_r; g.s_c = (int)s_c; g.p_r = (int)p_r; g.p_c = (int)p_c; g.d_r = (int)d_r; g.d_c = (int)d_c;
-    g.k_c = (int)k_c; g.k_rc = (int)(k_r * k_c); g.Wo = (int)Wo;
+    g.k_r = (int)k_r; g.k_c = (int)k_c; g.k_rc = (int)(k_r * k_c); g.Wo = (int)Wo;
+    g.last = (int)(slice_channels * height * width - 1);
     g.div_krc = ntg::make_fastdiv((uint32_t)(k_r * k_c));
     g.div_kc = ntg::make_fastdiv((uint32_t)k_c);
     g.div_wo = ntg::make_fastdiv((uint32_t)Wo);
@@ -412,7 +414,7 @@ int ntg_conv2d_dev(int dtype, const void* image, const void* kernel, void* out,
             p.sA = 0; p.sB = channels * height * width; p.sC = out_channels * L;
             p.cmode = ntg::C_OVERWRITE;
             p.vecA_ok = (add * es) % 16 == 0;
-            fill_conv_geom(p.conv, height, width, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c, Wo);
+            fill_conv_geom(p.conv, channels / groups, height, width, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c, Wo);
             hipError_t e = ntg::launch_conv_mfma(dtype, false, p, static_cast<hipStream_t>(stream));
             if (e != hipSuccess) return hip_fail(e, "implicit conv2d launch");
         }
