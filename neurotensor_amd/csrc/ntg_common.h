@@ -92,6 +92,11 @@ hipError_t launch_col2im(int dtype, const void* col, void* im,
                          int64_t k_r, int64_t k_c, int64_t s_r, int64_t s_c,
                          int64_t p_r, int64_t p_c, int64_t d_r, int64_t d_c, int accumulate, hipStream_t s);
 
+// conv2d backward helpers (unfold2d.hip): ordered sum of per-image weight gradients; weights of
+// the gradient-to-image convolution
+hipError_t launch_reduce_batch(int dtype, const void* part, void* out, int64_t batch, int64_t n, int accumulate, hipStream_t s);
+hipError_t launch_flip_weights(int64_t elem_size, const void* w, void* wt, int64_t groups, int64_t og, int64_t cg, int64_t taps, hipStream_t s);
+
 #ifdef __HIPCC__
 __device__ __forceinline__ uint32_t fast_div(uint32_t n, const FastDiv& f) {
     const uint32_t t = __umulhi(f.m, n);

@@ -544,7 +544,63 @@ int ntg_conv2d_backward_dev(int dtype, const void* image, const void* kernel, co
     const char* kern = static_cast<const char*>(kernel);
     const char* gy = static_cast<const char*>(grad_out);
     char* ws = static_cast<char*>(workspace);
+    hipStream_t hs = static_cast<hipStream_t>(stream);
+    const int64_t cg = channels / groups, HW = height * width;
     ntg_gemm_desc d;
+    // Floating dtypes: neither gradient needs the stored im2col matrix.
+    //   dW: one batched GEMM  P_b,g [og, add] = dY_{b,g} [og, L] . col_{b,g}^T  with col gathered from the image by the
+    //       B loader, then the per-image results are summed in batch order (the same additions, in the same order, as
+    //       accumulating one GEMM per image into dW).
+    //   dX (stride 1): the convolution of dY with the channel-swapped, tap-reversed kernel and padding d*(k-1) - p,
+    //       again as an implicit GEMM; one sum over (oc, i, j) per element instead of the reference's GEMM over oc
+    //       followed by col2im over (i, j) -- same terms, different rounding order, inside the stated tolerance.
+    const bool gather_dw = d_kernel && conv_implicit(dtype, channels, height, width, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c, Ho, Wo) &&
+                           batch * out_channels * add * es <= workspace_bytes;
+    const int64_t q_r = d_r * (k_r - 1) - p_r, q_c = d_c * (k_c - 1) - p_c;   // padding of the gradient-to-image convolution
+    const bool gather_dx = d_image && s_r == 1 && s_c == 1 && q_r > -(1 << 24) && q_c > -(1 << 24) &&
+                           conv_implicit(dtype, out_channels, Ho, Wo, k_r, k_c, 1, 1, q_r < 0 ? 0 : q_r, q_c < 0 ? 0 : q_c, d_r, d_c, height, width) &&
+                           out_channels * cg * k_r * k_c * es <= workspace_bytes;
+    if (gather_dw) {
+        for (int64_t g = 0; g < groups; ++g) {
+            ntg::GemmParams p;
+            std::memset(&p, 0, sizeof p);
+            p.M = (int)og; p.K = (int)L; p.N = (int)add; p.batch = (int)batch;
+            p.A = gy + g * og * L * es;
+            p.B = static_cast<const char*>(image) + g * cg * HW * es;
+            p.C = ws + g * og * add * es;
+            p.lda = L; p.ldb = L; p.ldc = add;
+            p.sA = out_channels * L; p.sB = channels * HW; p.sC = out_channels * add;
+            p.cmode = ntg::C_OVERWRITE;
+            p.vecA_ok = (L * es) % 16 == 0 && (p.sA * es) % 16 == 0;
+            fill_conv_geom(p.conv, cg, height, width, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c, Wo);
+            hipError_t e = ntg::launch_conv_mfma(dtype, true, p, hs);
+            if (e != hipSuccess) return hip_fail(e, "implicit conv_dkernel launch");
+        }
+        hipError_t e = ntg::launch_reduce_batch(dtype, ws, d_kernel, batch, out_channels * add, accumulate, hs);
+        if (e != hipSuccess) return hip_fail(e, "weight gradient reduction launch");
+    }
+    if (gather_dx) {
+        const int64_t taps = k_r * k_c;
+        hipError_t e = ntg::launch_flip_weights(es, kernel, ws, groups, og, cg, taps, hs);
+        if (e != hipSuccess) return hip_fail(e, "weight flip launch");
+        for (int64_t g = 0; g < groups; ++g) {
+            ntg::GemmParams p;
+            std::memset(&p, 0, sizeof p);
+            p.M = (int)cg; p.K = (int)(og * taps); p.N = (int)HW; p.batch = (int)batch;
+            p.A = ws + g * cg * og * taps * es;
+            p.B = gy + g * og * L * es;
+            p.C = static_cast<char*>(d_image) + g * cg * HW * es;
+            p.lda = og * taps; p.ldb = HW; p.ldc = HW;
+            p.sA = 0; p.sB = out_channels * L; p.sC = channels * HW;
+            p.cmode = accumulate ? ntg::C_ACCUMULATE : ntg::C_OVERWRITE;
+            p.vecA_ok = (og * taps * es) % 16 == 0;
+            fill_conv_geom(p.conv, og, Ho, Wo, k_r, k_c, 1, 1, q_r, q_c, d_r, d_c, width);
+            e = ntg::launch_conv_mfma(dtype, false, p, hs);
+            if (e != hipSuccess) return hip_fail(e, "implicit conv_dimage launch");
+        }
+    }
+    if (gather_dw) d_kernel = nullptr;    // done
+    if (gather_dx) d_image = nullptr;
     if (d_kernel) {
         // col = im2col(image); per group g:  dW_g [og, add] (+)= sum_b dY_{b,g} [og, L] . col_{b,g}^T  (col_{b,g} stored [add, L])
         rc = ntg_unfold2d_dev(dtype, image, ws, batch, channels, height, width, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c, stream);

@@ -72,6 +72,70 @@ __global__ void __launch_bounds__(256) col2im_kernel(const T* __restrict__ col, 
     }
 }
 
+// out[i] (+)= sum over b of part[b*n + i], b ascending: the order in which per-image weight
+// gradients are added up by the reference's batch loop (conv.cpp:466-469).
+template <class T, class Acc>
+__global__ void __launch_bounds__(256) reduce_batch_kernel(const T* __restrict__ part, T* __restrict__ out, const int64_t batch,
+                                                           const int64_t n, const int accumulate) {
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+        Acc acc = accumulate ? (Acc)out[i] : (Acc)0;
+        for (int64_t b = 0; b < batch; ++b) acc += (Acc)part[b * n + i];
+        out[i] = (T)acc;
+    }
+}
+
+// wt[g][c][oc][t] = w[g*og + oc][c][taps-1-t]: the kernel with input/output channels swapped
+// inside each group and both tap axes reversed, i.e. the weights of the convolution that maps
+// the output gradient back to the image.
+template <class T>
+__global__ void __launch_bounds__(256) flip_weights_kernel(const T* __restrict__ w, T* __restrict__ wt, const int64_t groups,
+                                                           const int64_t og, const int64_t cg, const int64_t taps) {
+    const int64_t total = groups * og * cg * taps;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += stride) {
+        const int64_t t = idx % taps;
+        int64_t r = idx / taps;
+        const int64_t oc = r % og;
+        r /= og;
+        const int64_t c = r % cg;
+        const int64_t g = r / cg;
+        wt[idx] = w[((g * og + oc) * cg + c) * taps + (taps - 1 - t)];
+    }
+}
+
+static unsigned grid_for(int64_t total) {
+    int64_t blocks = (total + 255) / 256;
+    if (blocks > 256 * 64) blocks = 256 * 64;
+    return (unsigned)(blocks < 1 ? 1 : blocks);
+}
+
+hipError_t launch_reduce_batch(int dtype, const void* part, void* out, int64_t batch, int64_t n, int accumulate, hipStream_t s) {
+    if (n == 0) return hipSuccess;
+    const dim3 g(grid_for(n)), b(256);
+    switch (dtype) {
+    case DT_F32: hipLaunchKernelGGL((reduce_batch_kernel<float, float>), g, b, 0, s, (const float*)part, (float*)out, batch, n, accumulate); break;
+    case DT_F64: hipLaunchKernelGGL((reduce_batch_kernel<double, double>), g, b, 0, s, (const double*)part, (double*)out, batch, n, accumulate); break;
+    case DT_F16: hipLaunchKernelGGL((reduce_batch_kernel<_Float16, float>), g, b, 0, s, (const _Float16*)part, (_Float16*)out, batch, n, accumulate); break;
+    case DT_BF16: hipLaunchKernelGGL((reduce_batch_kernel<__bf16, float>), g, b, 0, s, (const __bf16*)part, (__bf16*)out, batch, n, accumulate); break;
+    default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+
+hipError_t launch_flip_weights(int64_t es, const void* w, void* wt, int64_t groups, int64_t og, int64_t cg, int64_t taps, hipStream_t s) {
+    const int64_t total = groups * og * cg * taps;
+    if (total == 0) return hipSuccess;
+    const dim3 g(grid_for(total)), b(256);
+    switch (es) {
+    case 2: hipLaunchKernelGGL(flip_weights_kernel<uint16_t>, g, b, 0, s, (const uint16_t*)w, (uint16_t*)wt, groups, og, cg, taps); break;
+    case 4: hipLaunchKernelGGL(flip_weights_kernel<uint32_t>, g, b, 0, s, (const uint32_t*)w, (uint32_t*)wt, groups, og, cg, taps); break;
+    case 8: hipLaunchKernelGGL(flip_weights_kernel<uint64_t>, g, b, 0, s, (const uint64_t*)w, (uint64_t*)wt, groups, og, cg, taps); break;
+    default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+
 static hipError_t fill_params(UnfoldParams& u, int64_t batch, int64_t channels, int64_t height, int64_t width,
                               int64_t k_r, int64_t k_c, int64_t s_r, int64_t s_c, int64_t p_r, int64_t p_c, int64_t d_r, int64_t d_c) {
     u.batch = batch; u.channels = channels; u.height = height; u.width = width;

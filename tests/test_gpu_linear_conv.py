@@ -230,6 +230,64 @@ def test_conv2d_backward_random_vs_oracle():
     assert np.abs(dw.cpu().numpy() - tw.grad.numpy()).max() <= 1e-3
 
 
+BACKWARD_GEOMS = [
+    # (B, C, H, W, O, kh, kw, stride, padding, dilation, groups)
+    (2, 8, 20, 23, 16, 3, 3, 1, 1, 1, 1),                  # stride 1: both gradients as implicit GEMMs
+    (3, 6, 17, 9, 9, 2, 4, 1, (0, 3), (2, 1), 3),          # groups, asymmetric taps / padding / dilation
+    (2, 4, 11, 12, 6, 3, 3, 1, (3, 4), 1, 2),              # padding beyond the kernel reach (negative padding of the dX conv)
+    (1, 3, 7, 31, 4, 1, 1, 1, 0, 1, 1),
+    (2, 5, 12, 12, 7, 5, 5, 2, 2, 1, 1),                   # stride 2: dX through the stored col matrix + col2im
+    (4, 32, 30, 28, 64, 3, 3, 1, 1, 1, 1),
+    (8, 64, 28, 28, 128, 3, 3, 1, 1, 1, 1),                # enough tiles for the large-tile kernels
+]
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64, np.float16, "bf16"], ids=["fp32", "fp64", "fp16", "bf16"])
+@pytest.mark.parametrize("geom", BACKWARD_GEOMS, ids=lambda g: "-".join(str(v).replace(" ", "") for v in g))
+def test_conv2d_backward_geometries(dtype, geom):
+    """conv_dimage / conv_dkernel against torch autograd in double (and the oracle on the small cases),
+    with and without accumulation into existing gradients."""
+    B, C, H, W, O, kh, kw, s, p, d, groups = geom
+    bf = dtype == "bf16"
+    rng = np.random.default_rng(1400 + C + H)
+    x = randn(rng, (B, C, H, W), dtype)
+    w = randn(rng, (O, C // groups, kh, kw), dtype, 1.0 / np.sqrt(C // groups * kh * kw))
+    tx, tw = to_torch(x, DEV, bf), to_torch(w, DEV, bf)
+    rx = tx.double().requires_grad_(True)
+    rw = tw.double().requires_grad_(True)
+    ry = torch.nn.functional.conv2d(rx, rw, None, s, p, d, groups)
+    g = randn(rng, tuple(ry.shape), dtype)
+    tg = to_torch(g, DEV, bf)
+    ry.backward(tg.double())
+    dx, dw = F.conv2d_backward(tx, tw, tg, stride=s, padding=p, dilation=d, groups=groups)
+    assert dx.shape == tx.shape and dw.shape == tw.shape
+    sx, sw = rx.grad.abs().max().item(), rw.grad.abs().max().item()
+    if dtype in (np.float32, np.float64):
+        kx = O // groups * kh * kw
+        kw_ = B * ry.shape[2] * ry.shape[3]
+        tolx = 1e-5 * kx * float(tg.abs().max().item() * tw.abs().max().item())
+        tolw = 1e-5 * kw_ * float(tg.abs().max().item() * tx.abs().max().item())
+    else:
+        tolx, tolw = HALF_REL * sx, HALF_REL * sw
+    assert (dx.double() - rx.grad).abs().max().item() <= tolx
+    assert (dw.double() - rw.grad).abs().max().item() <= tolw
+    if B * C * H * W <= 20000 and dtype in (np.float32, np.float64):      # the oracle's col2im is fp32 / fp64 only
+        odx, odw = oracle.conv2d_backward(x, w, g, s, p, d, groups)
+        assert np.abs(dx.cpu().numpy().astype(np.float64) - odx.astype(np.float64)).max() <= tolx
+        assert np.abs(dw.cpu().numpy().astype(np.float64) - odw.astype(np.float64)).max() <= tolw
+    # accumulate: the gradients are added to what the buffers hold
+    dx2, dw2 = dx.clone(), dw.clone()
+    lib = _lib.load()
+    ws_bytes = lib.ntg_conv2d_workspace_bytes(F.ntg_dtype(tx), B, C, H, W, kh, kw, *F._pair(s), *F._pair(p), *F._pair(d))
+    ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=DEV)
+    st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    _lib.check(lib.ntg_conv2d_backward_dev(F.ntg_dtype(tx), tx.data_ptr(), tw.data_ptr(), tg.data_ptr(), dx2.data_ptr(), dw2.data_ptr(),
+                                           ws.data_ptr(), ws_bytes, B, C, H, W, O, kh, kw, *F._pair(s), *F._pair(p), *F._pair(d),
+                                           groups, 1, st))
+    assert (dx2.double() - 2 * rx.grad).abs().max().item() <= 2 * tolx + (0 if dtype in (np.float32, np.float64) else HALF_REL * sx)
+    assert (dw2.double() - 2 * rw.grad).abs().max().item() <= 2 * tolw + (0 if dtype in (np.float32, np.float64) else HALF_REL * sw)
+
+
 @pytest.mark.parametrize("dtype", [np.float32, np.float64, np.float16, np.int32])
 def test_conv2d_random_vs_oracle(dtype):
     rng = np.random.default_rng(900)
