@@ -7,6 +7,7 @@
 
 #include <cstdarg>
 #include <cstdio>
+#include <algorithm>
 #include <cstring>
 #include <map>
 #include <string>
@@ -519,6 +520,37 @@ int ntg_unfold2d_backward(int dtype, const void* col, void* image,
     return NTG_OK;
 }
 
+// Which conv2d-backward gradients run as implicit GEMMs, and the workspace the call needs.
+struct ConvBackwardPlan { bool gather_dw, gather_dx; int64_t q_r, q_c, need; };
+static ConvBackwardPlan plan_conv_backward(int dtype, bool want_dx, bool want_dw, int64_t batch, int64_t channels, int64_t height, int64_t width,
+                                           int64_t out_channels, int64_t k_r, int64_t k_c, int64_t s_r, int64_t s_c, int64_t p_r, int64_t p_c,
+                                           int64_t d_r, int64_t d_c, int64_t groups, int64_t Ho, int64_t Wo) {
+    const int64_t es = ntg::elem_size(dtype);
+    const int64_t cg = channels / groups, taps = k_r * k_c;
+    ConvBackwardPlan pl;
+    pl.q_r = d_r * (k_r - 1) - p_r;   // padding of the gradient-to-image convolution
+    pl.q_c = d_c * (k_c - 1) - p_c;
+    pl.gather_dw = want_dw && conv_implicit(dtype, channels, height, width, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c, Ho, Wo);
+    pl.gather_dx = want_dx && s_r == 1 && s_c == 1 && pl.q_r > -(1 << 24) && pl.q_c > -(1 << 24) &&
+                   conv_implicit(dtype, out_channels, Ho, Wo, k_r, k_c, 1, 1, pl.q_r < 0 ? 0 : pl.q_r, pl.q_c < 0 ? 0 : pl.q_c, d_r, d_c, height, width);
+    const int64_t col = batch * channels * taps * Ho * Wo * es;
+    int64_t need = 0;
+    if (want_dw) need = std::max(need, pl.gather_dw ? batch * out_channels * cg * taps * es : col);
+    if (want_dx) need = std::max(need, pl.gather_dx ? out_channels * cg * taps * es : col);
+    pl.need = need;
+    return pl;
+}
+
+int64_t ntg_conv2d_backward_workspace_bytes(int dtype, int64_t batch, int64_t channels, int64_t height, int64_t width,
+                                            int64_t out_channels, int64_t k_r, int64_t k_c, int64_t s_r, int64_t s_c,
+                                            int64_t p_r, int64_t p_c, int64_t d_r, int64_t d_c, int64_t groups) {
+    int64_t Ho, Wo;
+    if (ntg::elem_size(dtype) == 0 || groups < 1 || channels % groups != 0 || out_channels % groups != 0 ||
+        unfold_out(height, width, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c, Ho, Wo)) return -1;
+    return plan_conv_backward(dtype, true, true, batch, channels, height, width, out_channels, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c,
+                              groups, Ho, Wo).need;
+}
+
 int ntg_conv2d_backward_dev(int dtype, const void* image, const void* kernel, const void* grad_out,
                             void* d_image, void* d_kernel, void* workspace, int64_t workspace_bytes,
                             int64_t batch, int64_t channels, int64_t height, int64_t width,
@@ -538,9 +570,10 @@ int ntg_conv2d_backward_dev(int dtype, const void* image, const void* kernel, co
     if (!kernel || !grad_out || (d_kernel && !image)) return fail(NTG_ERR_INVALID_ARGUMENT, "null pointer");
     const int64_t L = Ho * Wo, ckk = channels * k_r * k_c;
     const int64_t add = (channels / groups) * k_r * k_c, og = out_channels / groups;
-    const int64_t need = batch * ckk * L * es;
-    if (!workspace || workspace_bytes < need)
-        return fail(NTG_ERR_INVALID_ARGUMENT, "workspace of %lld bytes needed, %lld given", (long long)need, (long long)workspace_bytes);
+    const ConvBackwardPlan plan = plan_conv_backward(dtype, d_image != nullptr, d_kernel != nullptr, batch, channels, height, width,
+                                                     out_channels, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c, groups, Ho, Wo);
+    if (plan.need > 0 && (!workspace || workspace_bytes < plan.need))
+        return fail(NTG_ERR_INVALID_ARGUMENT, "workspace of %lld bytes needed, %lld given", (long long)plan.need, (long long)workspace_bytes);
     const char* kern = static_cast<const char*>(kernel);
     const char* gy = static_cast<const char*>(grad_out);
     char* ws = static_cast<char*>(workspace);
@@ -554,12 +587,8 @@ int ntg_conv2d_backward_dev(int dtype, const void* image, const void* kernel, co
     //   dX (stride 1): the convolution of dY with the channel-swapped, tap-reversed kernel and padding d*(k-1) - p,
     //       again as an implicit GEMM; one sum over (oc, i, j) per element instead of the reference's GEMM over oc
     //       followed by col2im over (i, j) -- same terms, different rounding order, inside the stated tolerance.
-    const bool gather_dw = d_kernel && conv_implicit(dtype, channels, height, width, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c, Ho, Wo) &&
-                           batch * out_channels * add * es <= workspace_bytes;
-    const int64_t q_r = d_r * (k_r - 1) - p_r, q_c = d_c * (k_c - 1) - p_c;   // padding of the gradient-to-image convolution
-    const bool gather_dx = d_image && s_r == 1 && s_c == 1 && q_r > -(1 << 24) && q_c > -(1 << 24) &&
-                           conv_implicit(dtype, out_channels, Ho, Wo, k_r, k_c, 1, 1, q_r < 0 ? 0 : q_r, q_c < 0 ? 0 : q_c, d_r, d_c, height, width) &&
-                           out_channels * cg * k_r * k_c * es <= workspace_bytes;
+    const bool gather_dw = plan.gather_dw, gather_dx = plan.gather_dx;
+    const int64_t q_r = plan.q_r, q_c = plan.q_c;
     if (gather_dw) {
         for (int64_t g = 0; g < groups; ++g) {
             ntg::GemmParams p;
@@ -655,7 +684,8 @@ int ntg_conv2d_backward(int dtype, const void* image, const void* kernel, const 
     const size_t im_bytes = (size_t)(batch * channels * height * width * es);
     const size_t k_bytes = (size_t)(out_channels * (channels / groups) * k_r * k_c * es);
     const size_t g_bytes = (size_t)(batch * out_channels * Ho * Wo * es);
-    const int64_t wsb = ntg_conv2d_workspace_bytes(dtype, batch, channels, height, width, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c);
+    const int64_t wsb = ntg_conv2d_backward_workspace_bytes(dtype, batch, channels, height, width, out_channels, k_r, k_c, s_r, s_c,
+                                                            p_r, p_c, d_r, d_c, groups);
     DeviceMem mem;
     const size_t o_k = align_up(im_bytes, 256), o_g = o_k + align_up(k_bytes, 256), o_di = o_g + align_up(g_bytes, 256);
     const size_t o_dk = o_di + align_up(im_bytes, 256), o_ws = o_dk + align_up(k_bytes, 256);

@@ -278,7 +278,8 @@ def test_conv2d_backward_geometries(dtype, geom):
     # accumulate: the gradients are added to what the buffers hold
     dx2, dw2 = dx.clone(), dw.clone()
     lib = _lib.load()
-    ws_bytes = lib.ntg_conv2d_workspace_bytes(F.ntg_dtype(tx), B, C, H, W, kh, kw, *F._pair(s), *F._pair(p), *F._pair(d))
+    ws_bytes = lib.ntg_conv2d_backward_workspace_bytes(F.ntg_dtype(tx), B, C, H, W, O, kh, kw, *F._pair(s), *F._pair(p), *F._pair(d), groups)
+    assert ws_bytes > 0
     ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=DEV)
     st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
     _lib.check(lib.ntg_conv2d_backward_dev(F.ntg_dtype(tx), tx.data_ptr(), tw.data_ptr(), tg.data_ptr(), dx2.data_ptr(), dw2.data_ptr(),
