@@ -214,6 +214,25 @@ int ntg_conv2d_backward_dev(int dtype, const void* image, const void* kernel, co
                             int64_t s_r, int64_t s_c, int64_t p_r, int64_t p_c, int64_t d_r, int64_t d_c,
                             int64_t groups, int accumulate, void* stream);
 
+/* functional::conv_transpose2d (nt/functional/tensor_files/conv.cpp:614-676; conv_transpose1d :538-612 is the same call
+ * with in_h == 1 and k_r == 1).  input [batch, in_channels, in_h, in_w], kernel [in_channels, out_channels/groups, k_r, k_c],
+ * out [batch, out_channels, (in_h-1)*s_r - 2*p_r + d_r*(k_r-1) + 1 + op_r, likewise for columns].  The reference dilates the
+ * input by the stride, pads it by output_padding, unfolds it and multiplies by the channel-swapped, tap-reversed kernel;
+ * this backend computes the same sums as the image gradient of the matching convolution.  output_padding must be smaller
+ * than stride. */
+int64_t ntg_conv_transpose2d_workspace_bytes(int dtype, int64_t batch, int64_t in_channels, int64_t in_h, int64_t in_w,
+                                             int64_t out_channels, int64_t k_r, int64_t k_c, int64_t s_r, int64_t s_c,
+                                             int64_t p_r, int64_t p_c, int64_t d_r, int64_t d_c, int64_t op_r, int64_t op_c, int64_t groups);
+int ntg_conv_transpose2d_dev(int dtype, const void* input, const void* kernel, void* out, void* workspace, int64_t workspace_bytes,
+                             int64_t batch, int64_t in_channels, int64_t in_h, int64_t in_w, int64_t out_channels,
+                             int64_t k_r, int64_t k_c, int64_t s_r, int64_t s_c, int64_t p_r, int64_t p_c, int64_t d_r, int64_t d_c,
+                             int64_t op_r, int64_t op_c, int64_t groups, void* stream);
+/* host pointers, synchronous */
+int ntg_conv_transpose2d(int dtype, const void* input, const void* kernel, void* out,
+                         int64_t batch, int64_t in_channels, int64_t in_h, int64_t in_w, int64_t out_channels,
+                         int64_t k_r, int64_t k_c, int64_t s_r, int64_t s_c, int64_t p_r, int64_t p_c, int64_t d_r, int64_t d_c,
+                         int64_t op_r, int64_t op_c, int64_t groups);
+
 #ifdef __cplusplus
 }
 #endif

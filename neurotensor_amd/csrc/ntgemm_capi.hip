@@ -664,6 +664,102 @@ int ntg_conv2d_backward_dev(int dtype, const void* image, const void* kernel, co
     return NTG_OK;
 }
 
+// conv_transpose2d = the image gradient of the convolution whose output is `input`: per group
+// out_g [cog, Rout*Cout] = flipped, channel-swapped kernel . unfold(zero-dilated input), which is what
+// the reference forms explicitly (conv.cpp:614-676: dilate by stride, pad by output_padding, unfold2d
+// with padding d*(k-1) - p and stride 1, matmult with w.transpose(0,1).flip).  Here it is the
+// conv_dimage path of ntg_conv2d_backward_dev with the roles renamed; kernel is [in_channels,
+// out_channels/groups, k_r, k_c] as in the reference.
+static int conv_transpose_out(int64_t in_h, int64_t in_w, int64_t k_r, int64_t k_c, int64_t s_r, int64_t s_c, int64_t p_r, int64_t p_c,
+                              int64_t d_r, int64_t d_c, int64_t op_r, int64_t op_c, int64_t& out_h, int64_t& out_w) {
+    if (k_r < 1 || k_c < 1) return fail(NTG_ERR_INVALID_ARGUMENT, "kernel size must be >= 1");
+    if (s_r < 1 || s_c < 1) return fail(NTG_ERR_INVALID_ARGUMENT, "Conv2d Transpose stride cannot be less than 1 but got (%lld, %lld)", (long long)s_r, (long long)s_c);
+    if (d_r < 1 || d_c < 1) return fail(NTG_ERR_INVALID_ARGUMENT, "Conv2d Transpose dilation cannot be less than 1 but got (%lld, %lld)", (long long)d_r, (long long)d_c);
+    if (p_r < 0 || p_c < 0) return fail(NTG_ERR_INVALID_ARGUMENT, "Conv2d Transpose padding cannot be less than 0 but got (%lld, %lld)", (long long)p_r, (long long)p_c);
+    if (op_r < 0 || op_c < 0) return fail(NTG_ERR_INVALID_ARGUMENT, "Conv2d Transpose output_padding cannot be less than 0 but got (%lld, %lld)", (long long)op_r, (long long)op_c);
+    // the reference accepts any output_padding; rows past the reach of the kernel would be zero.  This backend needs the
+    // forward convolution of the result to reproduce the input size, which holds for output_padding < stride.
+    if (op_r >= s_r || op_c >= s_c) return fail(NTG_ERR_INVALID_ARGUMENT, "output_padding (%lld, %lld) must be smaller than stride (%lld, %lld)",
+                                                (long long)op_r, (long long)op_c, (long long)s_r, (long long)s_c);
+    if (in_h < 1 || in_w < 1) return fail(NTG_ERR_INVALID_ARGUMENT, "empty input");
+    out_h = (in_h - 1) * s_r - 2 * p_r + d_r * (k_r - 1) + 1 + op_r;
+    out_w = (in_w - 1) * s_c - 2 * p_c + d_c * (k_c - 1) + 1 + op_c;
+    if (out_h < 1 || out_w < 1) return fail(NTG_ERR_INVALID_ARGUMENT, "the output of the transposed convolution would be empty");
+    // a padding wider than the kernel reach would make the matching convolution read fewer input rows than exist
+    if ((out_h + 2 * p_r - d_r * (k_r - 1) - 1) / s_r + 1 != in_h || (out_w + 2 * p_c - d_c * (k_c - 1) - 1) / s_c + 1 != in_w)
+        return fail(NTG_ERR_INVALID_ARGUMENT, "geometry is not the transpose of a convolution");
+    return NTG_OK;
+}
+
+int64_t ntg_conv_transpose2d_workspace_bytes(int dtype, int64_t batch, int64_t in_channels, int64_t in_h, int64_t in_w,
+                                             int64_t out_channels, int64_t k_r, int64_t k_c, int64_t s_r, int64_t s_c,
+                                             int64_t p_r, int64_t p_c, int64_t d_r, int64_t d_c, int64_t op_r, int64_t op_c, int64_t groups) {
+    int64_t oh, ow, Ho, Wo;
+    if (ntg::elem_size(dtype) == 0 || groups < 1 || in_channels % groups != 0 || out_channels % groups != 0 ||
+        conv_transpose_out(in_h, in_w, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c, op_r, op_c, oh, ow) ||
+        unfold_out(oh, ow, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c, Ho, Wo)) return -1;
+    return plan_conv_backward(dtype, true, false, batch, out_channels, oh, ow, in_channels, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c,
+                              groups, Ho, Wo).need;
+}
+
+int ntg_conv_transpose2d_dev(int dtype, const void* input, const void* kernel, void* out, void* workspace, int64_t workspace_bytes,
+                             int64_t batch, int64_t in_channels, int64_t in_h, int64_t in_w, int64_t out_channels,
+                             int64_t k_r, int64_t k_c, int64_t s_r, int64_t s_c, int64_t p_r, int64_t p_c, int64_t d_r, int64_t d_c,
+                             int64_t op_r, int64_t op_c, int64_t groups, void* stream) {
+    if (ntg::elem_size(dtype) == 0) return fail(NTG_ERR_UNSUPPORTED_DTYPE, "dtype %d is not supported", dtype);
+    if (batch < 0 || in_channels < 0 || out_channels < 0) return fail(NTG_ERR_INVALID_ARGUMENT, "negative size");
+    if (groups < 1) return fail(NTG_ERR_INVALID_ARGUMENT, "groups must be >= 1");
+    if (in_channels % groups != 0)
+        return fail(NTG_ERR_INVALID_ARGUMENT, "Expected image channels to be divisible by groups in Conv2d Transpose but got %lld %% %lld != 0",
+                    (long long)in_channels, (long long)groups);
+    if (out_channels % groups != 0) return fail(NTG_ERR_INVALID_ARGUMENT, "out channels (%lld) not divisible by groups (%lld)", (long long)out_channels, (long long)groups);
+    int64_t oh, ow;
+    int rc = conv_transpose_out(in_h, in_w, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c, op_r, op_c, oh, ow);
+    if (rc) return rc;
+    if (batch == 0 || out_channels == 0) return NTG_OK;
+    if (in_channels == 0) {
+        hipError_t e = ntg::launch_col2im(dtype, nullptr, out, batch, out_channels, oh, ow, 0, 0, 1, 1, 0, 0, 1, 1, 0, static_cast<hipStream_t>(stream));
+        if (e != hipSuccess) return hip_fail(e, "zero fill");
+        return NTG_OK;
+    }
+    return ntg_conv2d_backward_dev(dtype, nullptr, kernel, input, out, nullptr, workspace, workspace_bytes, batch, out_channels, oh, ow,
+                                   in_channels, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c, groups, 0, stream);
+}
+
+int ntg_conv_transpose2d(int dtype, const void* input, const void* kernel, void* out,
+                         int64_t batch, int64_t in_channels, int64_t in_h, int64_t in_w, int64_t out_channels,
+                         int64_t k_r, int64_t k_c, int64_t s_r, int64_t s_c, int64_t p_r, int64_t p_c, int64_t d_r, int64_t d_c,
+                         int64_t op_r, int64_t op_c, int64_t groups) {
+    const int64_t es = ntg::elem_size(dtype);
+    if (es == 0) return fail(NTG_ERR_UNSUPPORTED_DTYPE, "dtype %d is not supported", dtype);
+    if (batch < 0 || in_channels < 0 || out_channels < 0) return fail(NTG_ERR_INVALID_ARGUMENT, "negative size");
+    if (groups < 1 || in_channels % groups != 0 || out_channels % groups != 0)
+        return fail(NTG_ERR_INVALID_ARGUMENT, "channels (%lld) and out channels (%lld) must be divisible by groups (%lld)",
+                    (long long)in_channels, (long long)out_channels, (long long)groups);
+    int64_t oh, ow;
+    int rc = conv_transpose_out(in_h, in_w, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c, op_r, op_c, oh, ow);
+    if (rc) return rc;
+    if (batch == 0 || out_channels == 0) return NTG_OK;
+    if (!input || !kernel || !out) return fail(NTG_ERR_INVALID_ARGUMENT, "null pointer");
+    const size_t in_bytes = (size_t)(batch * in_channels * in_h * in_w * es);
+    const size_t k_bytes = (size_t)(in_channels * (out_channels / groups) * k_r * k_c * es);
+    const size_t o_bytes = (size_t)(batch * out_channels * oh * ow * es);
+    const int64_t wsb = ntg_conv_transpose2d_workspace_bytes(dtype, batch, in_channels, in_h, in_w, out_channels, k_r, k_c, s_r, s_c,
+                                                             p_r, p_c, d_r, d_c, op_r, op_c, groups);
+    if (wsb < 0) return fail(NTG_ERR_INVALID_ARGUMENT, "invalid geometry");
+    DeviceMem mem;
+    const size_t o_k = align_up(in_bytes, 256), o_o = o_k + align_up(k_bytes, 256), o_ws = o_o + align_up(o_bytes, 256);
+    HIP_TRY(mem.alloc(o_ws + (size_t)wsb));
+    if (in_bytes) HIP_TRY(hipMemcpy(mem.at(0), input, in_bytes, hipMemcpyHostToDevice));
+    if (k_bytes) HIP_TRY(hipMemcpy(mem.at(o_k), kernel, k_bytes, hipMemcpyHostToDevice));
+    rc = ntg_conv_transpose2d_dev(dtype, mem.at(0), mem.at(o_k), mem.at(o_o), mem.at(o_ws), wsb, batch, in_channels, in_h, in_w, out_channels,
+                                  k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c, op_r, op_c, groups, nullptr);
+    if (rc) return rc;
+    HIP_TRY(hipStreamSynchronize(nullptr));
+    HIP_TRY(hipMemcpy(out, mem.at(o_o), o_bytes, hipMemcpyDeviceToHost));
+    return NTG_OK;
+}
+
 int ntg_conv2d_backward(int dtype, const void* image, const void* kernel, const void* grad_out,
                         void* d_image, void* d_kernel,
                         int64_t batch, int64_t channels, int64_t height, int64_t width,

@@ -329,3 +329,105 @@ def conv2d_backward(image, kernel, grad, stride=1, padding=0, dilation=1, groups
     check(L.ntg_conv2d_backward_dev(dt, x.data_ptr(), w.data_ptr(), g.data_ptr(), dx.data_ptr(), dw.data_ptr(), ws.data_ptr(), ws_bytes,
                                     B, C, H, W, O, kh, kw, s[0], s[1], p[0], p[1], d[0], d[1], groups, 0, _stream()))
     return dx.reshape(image.shape), dw.reshape(kernel.shape)
+
+
+def conv1d(image, kernel, stride=1, padding=0, dilation=1, groups=1):
+    """functional::conv1d (tensor_files/conv.cpp:13-67): unfold1d then matmult; image [.., C, W], kernel [O, C/groups, k]
+    -> [B, O, Wo].  A convolution over one axis is the two-axis one with a single image row and a single tap row."""
+    _require_device(image, kernel)
+    if image.dim() < 2:
+        raise ValueError(f"Expected to get a 2D or greater tensor as the input for a 1d convolution, but got {image.dim()}D")
+    if kernel.dim() not in (2, 3):
+        raise ValueError(f"Expected to get a 3D or 2D tensor as the kernel for a 1d convolution, but got {kernel.dim()}D")
+    if stride < 1:
+        raise ValueError(f"Conv1d stride cannot be less than 1 but got {stride}")
+    if dilation < 1:
+        raise ValueError(f"Conv1d dilation cannot be less than 1 but got {dilation}")
+    if padding < 0:
+        raise ValueError(f"Conv1d padding cannot be less than 1 but got {padding}")
+    x = image.reshape((1,) + tuple(image.shape)) if image.dim() == 2 else image.reshape((-1,) + tuple(image.shape[-2:]))
+    w = kernel.reshape((1,) + tuple(kernel.shape)) if kernel.dim() == 2 else kernel
+    out = conv2d(x.unsqueeze(2), w.unsqueeze(2), (1, stride), (0, padding), (1, dilation), groups)
+    return out.squeeze(2)
+
+
+def conv1d_backward(image, kernel, grad, stride=1, padding=0, dilation=1, groups=1):
+    """Gradients of conv1d with respect to image and kernel (conv_dimage / conv_dkernel with dim == 1)."""
+    x = image.reshape((1,) + tuple(image.shape)) if image.dim() == 2 else image.reshape((-1,) + tuple(image.shape[-2:]))
+    w = kernel.reshape((1,) + tuple(kernel.shape)) if kernel.dim() == 2 else kernel
+    dx, dw = conv2d_backward(x.unsqueeze(2), w.unsqueeze(2), grad.reshape(x.shape[0], w.shape[0], 1, -1),
+                             (1, stride), (0, padding), (1, dilation), groups)
+    return dx.squeeze(2).reshape(image.shape), dw.squeeze(2).reshape(kernel.shape)
+
+
+def conv_transpose2d(image, kernel, stride=1, padding=0, output_padding=0, dilation=1, groups=1):
+    """functional::conv_transpose2d (tensor_files/conv.cpp:614-676): image [.., Cin, H, W], kernel [Cin, Cout/groups, kh, kw]
+    -> [B, Cout, (H-1)*s - 2p + d(kh-1) + 1 + output_padding, ...]."""
+    _require_device(image, kernel)
+    if image.dim() < 3:
+        raise ValueError(f"Expected to get a 3D or greater tensor as the input for a conv2d transpose, but got {image.dim()}D")
+    if kernel.dim() not in (3, 4):
+        raise ValueError(f"Expected to get a 4D or 3D tensor as the kernel for a conv2d transpose, but got {kernel.dim()}D")
+    if image.dtype != kernel.dtype:
+        raise ValueError(f"Expected both kernel and image to have the same dtype for conv2d transpose but got {kernel.dtype} and {image.dtype}")
+    s, p, op, d = _pair(stride), _pair(padding), _pair(output_padding), _pair(dilation)
+    if min(s) < 1:
+        raise ValueError(f"Conv2d Transpose stride cannot be less than 1 but got {s}")
+    if min(d) < 1:
+        raise ValueError(f"Conv2d Transpose dilation cannot be less than 1 but got {d}")
+    if min(op) < 0:
+        raise ValueError(f"Conv2d Transpose output_padding cannot be less than 1 but got {op}")
+    if min(p) < 0:
+        raise ValueError(f"Conv2d Transpose padding cannot be less than 1 but got {p}")
+    if groups < 1:
+        raise ValueError(f"Expected groups for a convolution to be greater than 0 but got {groups}")
+    x = image.reshape((1,) + tuple(image.shape)) if image.dim() == 3 else image.reshape((-1,) + tuple(image.shape[-3:]))
+    w = kernel.reshape((1,) + tuple(kernel.shape)) if kernel.dim() == 3 else kernel
+    x, w = x.contiguous(), w.contiguous()
+    B, Cin, H, W = x.shape
+    if w.shape[0] != Cin:
+        raise ValueError(f"Expected image channels to be the same as the kernel batches for conv_transpose2d but got {tuple(x.shape)} and {tuple(w.shape)}")
+    if Cin % groups != 0:
+        raise ValueError(f"Expected image channels to be divisible by groups in Conv2d Transpose but got {Cin} % {groups} != 0")
+    _, Cog, kh, kw = w.shape
+    Cout = Cog * groups
+    L = load()
+    dt = ntg_dtype(x)
+    args = (B, Cin, H, W, Cout, kh, kw, s[0], s[1], p[0], p[1], d[0], d[1], op[0], op[1], groups)
+    ws_bytes = L.ntg_conv_transpose2d_workspace_bytes(dt, *args)
+    if ws_bytes < 0:
+        raise ValueError("conv_transpose2d: " + L.ntg_last_error().decode() if L.ntg_last_error() else "invalid geometry")
+    R = (H - 1) * s[0] - 2 * p[0] + d[0] * (kh - 1) + 1 + op[0]
+    Cc = (W - 1) * s[1] - 2 * p[1] + d[1] * (kw - 1) + 1 + op[1]
+    out = torch.empty((B, Cout, R, Cc), dtype=x.dtype, device=x.device)
+    ws = torch.empty((max(ws_bytes, 1),), dtype=torch.uint8, device=x.device)
+    check(L.ntg_conv_transpose2d_dev(dt, x.data_ptr(), w.data_ptr(), out.data_ptr(), ws.data_ptr(), ws_bytes, *args, _stream()))
+    return out
+
+
+def conv_transpose2d_backward(image, kernel, grad, stride=1, padding=0, output_padding=0, dilation=1, groups=1):
+    """Gradients of conv_transpose2d: d_image = conv2d(grad, kernel) and d_kernel = conv_dkernel with the roles of image
+    and output gradient exchanged (the transposed convolution is the adjoint of that convolution)."""
+    s, p, d = _pair(stride), _pair(padding), _pair(dilation)
+    x = image.reshape((1,) + tuple(image.shape)) if image.dim() == 3 else image.reshape((-1,) + tuple(image.shape[-3:]))
+    w = kernel.reshape((1,) + tuple(kernel.shape)) if kernel.dim() == 3 else kernel
+    g = grad.reshape((x.shape[0], w.shape[1] * groups) + tuple(grad.shape[-2:])).contiguous()
+    dx = conv2d(g, w, s, p, d, groups)
+    _, dw = conv2d_backward(g, w, x.contiguous(), s, p, d, groups)
+    return dx.reshape(image.shape), dw.reshape(kernel.shape)
+
+
+def conv_transpose1d(image, kernel, stride=1, padding=0, output_padding=0, dilation=1, groups=1):
+    """functional::conv_transpose1d (tensor_files/conv.cpp:538-612): image [.., Cin, W], kernel [Cin, Cout/groups, k]."""
+    x = image.reshape((1,) + tuple(image.shape)) if image.dim() == 2 else image.reshape((-1,) + tuple(image.shape[-2:]))
+    w = kernel.reshape((1,) + tuple(kernel.shape)) if kernel.dim() == 2 else kernel
+    out = conv_transpose2d(x.unsqueeze(2), w.unsqueeze(2), (1, stride), (0, padding), (0, output_padding), (1, dilation), groups)
+    return out.squeeze(2)
+
+
+def conv_transpose1d_backward(image, kernel, grad, stride=1, padding=0, output_padding=0, dilation=1, groups=1):
+    x = image.reshape((1,) + tuple(image.shape)) if image.dim() == 2 else image.reshape((-1,) + tuple(image.shape[-2:]))
+    w = kernel.reshape((1,) + tuple(kernel.shape)) if kernel.dim() == 2 else kernel
+    dx, dw = conv_transpose2d_backward(x.unsqueeze(2), w.unsqueeze(2), grad.unsqueeze(-2), (1, stride), (0, padding),
+                                       (0, output_padding), (1, dilation), groups)
+    return dx.squeeze(2).reshape(image.shape), dw.squeeze(2).reshape(kernel.shape)

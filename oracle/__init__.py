@@ -326,3 +326,78 @@ def conv2d_backward(image, kernel, grad, stride=1, padding=0, dilation=1, groups
         dk[g * og:(g + 1) * og] = per_item.sum(axis=0)
     dimg = unfold2d_backward(dcol, (H, W), (kh, kw), d, p, s, channels=C)
     return dimg, dk.reshape(kernel.shape)
+
+
+def conv1d(image, kernel, stride=1, padding=0, dilation=1, groups=1, kind="closed"):
+    """functional::conv1d (conv.cpp:13-67): unfold1d (window index c*k + j, the one-row case of the
+    2-d unfold) then the same matmult / group split as conv2d."""
+    x = image.reshape((1,) + image.shape) if image.ndim == 2 else image.reshape((-1,) + image.shape[-2:])
+    w = kernel.reshape((1,) + kernel.shape) if kernel.ndim == 2 else kernel
+    out = conv2d(x[:, :, None, :], w[:, :, None, :], (1, stride), (0, padding), (1, dilation), groups, kind)
+    return out[:, :, 0, :]
+
+
+def conv1d_backward(image, kernel, grad, stride=1, padding=0, dilation=1, groups=1, kind="closed"):
+    x = image.reshape((1,) + image.shape) if image.ndim == 2 else image.reshape((-1,) + image.shape[-2:])
+    w = kernel.reshape((1,) + kernel.shape) if kernel.ndim == 2 else kernel
+    g = np.ascontiguousarray(grad).reshape(x.shape[0], w.shape[0], 1, -1)
+    dx, dw = conv2d_backward(np.ascontiguousarray(x[:, :, None, :]), np.ascontiguousarray(w[:, :, None, :]), g,
+                             (1, stride), (0, padding), (1, dilation), groups, kind)
+    return dx[:, :, 0, :].reshape(image.shape), dw[:, :, 0, :].reshape(kernel.shape)
+
+
+def conv_transpose2d(image, kernel, stride=1, padding=0, output_padding=0, dilation=1, groups=1, kind="closed"):
+    """functional::conv_transpose2d (conv.cpp:614-676): zero-dilate the input by the stride (:632-634), pad bottom/right
+    by output_padding (:635-637), unfold2d with padding d*(k-1) - p and stride 1 (:639-641), then per group
+    matmult(w.transpose(0,1).flip(-1,-2) viewed [Cout/g, Cin/g*kh*kw], col) (:645-675)."""
+    x = image.reshape((1,) + image.shape) if image.ndim == 3 else image.reshape((-1,) + image.shape[-3:])
+    w = kernel.reshape((1,) + kernel.shape) if kernel.ndim == 3 else kernel
+    s, p, op, d = _pair(stride), _pair(padding), _pair(output_padding), _pair(dilation)
+    B, Cin, H, W = x.shape
+    _, Cog, kh, kw = w.shape
+    assert w.shape[0] == Cin and Cin % groups == 0
+    xd = np.zeros((B, Cin, (H - 1) * s[0] + 1 + op[0], (W - 1) * s[1] + 1 + op[1]), dtype=x.dtype)
+    xd[:, :, 0:(H - 1) * s[0] + 1:s[0], 0:(W - 1) * s[1] + 1:s[1]] = x
+    ph, pw = (kh - 1) * d[0] - p[0], (kw - 1) * d[1] - p[1]
+    assert ph >= 0 and pw >= 0, "padding wider than the kernel reach is not representable by unfold2d"
+    col = unfold2d(xd, (kh, kw), d, (ph, pw), 1, True)                               # [B, Cin*kh*kw, R*C]
+    R = (H - 1) * s[0] - 2 * p[0] + d[0] * (kh - 1) + 1 + op[0]
+    Cc = (W - 1) * s[1] - 2 * p[1] + d[1] * (kw - 1) + 1 + op[1]
+    wt = np.ascontiguousarray(w.transpose(1, 0, 2, 3)[:, :, ::-1, ::-1])              # [Cout/g, Cin, kh, kw]
+    cig = Cin // groups
+    add = cig * kh * kw
+    out = np.zeros((B, Cog * groups, R * Cc), dtype=x.dtype)
+    for g in range(groups):
+        kg = np.ascontiguousarray(wt[:, g * cig:(g + 1) * cig].reshape(Cog, -1))
+        colg = np.ascontiguousarray(col[:, g * add:(g + 1) * add, :])
+        out[:, g * Cog:(g + 1) * Cog, :] = matmult(kg, colg, None, False, False, kind=kind)
+    return out.reshape(B, Cog * groups, R, Cc)
+
+
+def conv_transpose2d_backward(image, kernel, grad, stride=1, padding=0, output_padding=0, dilation=1, groups=1, kind="closed"):
+    """The transposed convolution is the adjoint of conv2d with the same kernel, so its image gradient is conv2d(grad, kernel)
+    and its kernel gradient is conv_dkernel with image and output gradient exchanged.  (The reference reaches the same sums
+    through the saved unfolded input and flipped kernel; pinned by the conv_transpose*_{xgrad,wgrad} fixtures.)"""
+    x = image.reshape((1,) + image.shape) if image.ndim == 3 else image.reshape((-1,) + image.shape[-3:])
+    w = kernel.reshape((1,) + kernel.shape) if kernel.ndim == 3 else kernel
+    g = np.ascontiguousarray(grad).reshape((x.shape[0], w.shape[1] * groups) + grad.shape[-2:])
+    dx = conv2d(g, w, stride, padding, dilation, groups, kind)
+    _, dw = conv2d_backward(g, w, np.ascontiguousarray(x), stride, padding, dilation, groups, kind)
+    return dx.reshape(image.shape), dw.reshape(kernel.shape)
+
+
+def conv_transpose1d(image, kernel, stride=1, padding=0, output_padding=0, dilation=1, groups=1, kind="closed"):
+    """functional::conv_transpose1d (conv.cpp:538-612), the one-row case of conv_transpose2d."""
+    x = image.reshape((1,) + image.shape) if image.ndim == 2 else image.reshape((-1,) + image.shape[-2:])
+    w = kernel.reshape((1,) + kernel.shape) if kernel.ndim == 2 else kernel
+    out = conv_transpose2d(x[:, :, None, :], w[:, :, None, :], (1, stride), (0, padding), (0, output_padding), (1, dilation), groups, kind)
+    return out[:, :, 0, :]
+
+
+def conv_transpose1d_backward(image, kernel, grad, stride=1, padding=0, output_padding=0, dilation=1, groups=1, kind="closed"):
+    x = image.reshape((1,) + image.shape) if image.ndim == 2 else image.reshape((-1,) + image.shape[-2:])
+    w = kernel.reshape((1,) + kernel.shape) if kernel.ndim == 2 else kernel
+    dx, dw = conv_transpose2d_backward(np.ascontiguousarray(x[:, :, None, :]), np.ascontiguousarray(w[:, :, None, :]),
+                                       np.ascontiguousarray(grad)[..., None, :], (1, stride), (0, padding), (0, output_padding),
+                                       (1, dilation), groups, kind)
+    return dx[:, :, 0, :].reshape(image.shape), dw[:, :, 0, :].reshape(kernel.shape)

@@ -357,6 +357,93 @@ def test_conv2d_implicit_gather(dtype, geom):
         assert err <= (HALF_REL * scale if dtype == np.float16 else 1e-5 * K * np.abs(x).max() * np.abs(w).max())
 
 
+def _gpu_family(golden_dir, name, sfx, fwd, bwd, ofwd, obwd, kw):
+    x, w, exp, g, xg, wg = (load(golden_dir, f"{name}_{part}{sfx}") for part in ("input", "weight", "output", "grad", "xgrad", "wgrad"))
+    out = fwd(dev(x), dev(w), **kw).cpu().numpy()
+    assert out.shape == exp.shape
+    assert np.abs(out - exp).max() <= 1e-4 * max(1.0, np.abs(exp).max())
+    assert np.abs(out - ofwd(x, w, **kw)).max() <= 1e-5 * max(1.0, np.abs(exp).max())
+    dx, dw = bwd(dev(x), dev(w), dev(g), **kw)
+    dx, dw = dx.cpu().numpy(), dw.cpu().numpy()
+    assert dx.shape == xg.shape and dw.shape == wg.shape
+    assert np.abs(dx - xg).max() <= 1e-4 * max(1.0, np.abs(xg).max())
+    assert np.abs(dw - wg).max() <= 1e-4 * max(1.0, np.abs(wg).max())
+    odx, odw = obwd(x, w, g, **kw)
+    assert np.abs(dx - odx).max() <= 1e-5 * max(1.0, np.abs(xg).max())
+    assert np.abs(dw - odw).max() <= 1e-5 * max(1.0, np.abs(wg).max())
+
+
+@pytest.mark.parametrize("sfx,kw", [("", dict(stride=1, padding=1)), ("_grouped", dict(stride=1, groups=2)),
+                                    ("_batched", dict(stride=1, padding=1)), ("_grouped_batched", dict(stride=1, groups=2))])
+def test_conv1d_golden(golden_dir, sfx, kw):
+    """tests/src/conv_autograd_test.cpp:125-247 (conv1d outputs and gradients) on the GPU path."""
+    _gpu_family(golden_dir, "conv1d", sfx, F.conv1d, F.conv1d_backward, oracle.conv1d, oracle.conv1d_backward, kw)
+
+
+@pytest.mark.parametrize("sfx,kw", [("", dict(stride=2, output_padding=1)), ("_grouped", dict(stride=1, groups=2, padding=1)),
+                                    ("_grouped_bigger", dict(stride=1, groups=5, padding=1)),
+                                    ("_batched", dict(stride=2, output_padding=1, padding=1)),
+                                    ("_grouped_batched", dict(stride=1, groups=2, padding=1))])
+def test_conv_transpose1d_golden(golden_dir, sfx, kw):
+    """tests/src/conv_autograd_test.cpp:555-716 on the GPU path."""
+    _gpu_family(golden_dir, "conv_transpose1d", sfx, F.conv_transpose1d, F.conv_transpose1d_backward,
+                oracle.conv_transpose1d, oracle.conv_transpose1d_backward, kw)
+
+
+@pytest.mark.parametrize("sfx,kw", [("", dict(stride=2, output_padding=1)), ("_grouped", dict(stride=1, groups=5, padding=1)),
+                                    ("_batched", dict(stride=2, output_padding=1, padding=1)),
+                                    ("_grouped_batched", dict(stride=1, groups=2, padding=1))])
+def test_conv_transpose2d_golden(golden_dir, sfx, kw):
+    """tests/src/conv_autograd_test.cpp:720-846 on the GPU path, device and host entry points."""
+    _gpu_family(golden_dir, "conv_transpose2d", sfx, F.conv_transpose2d, F.conv_transpose2d_backward,
+                oracle.conv_transpose2d, oracle.conv_transpose2d_backward, kw)
+    x = load(golden_dir, "conv_transpose2d_input" + sfx)
+    w = load(golden_dir, "conv_transpose2d_weight" + sfx)
+    exp = load(golden_dir, "conv_transpose2d_output" + sfx)
+    lib = _lib.load()
+    B, Cin, H, W = x.shape
+    _, Cog, kh, kw_ = w.shape
+    groups = kw.get("groups", 1)
+    s, p, op = kw.get("stride", 1), kw.get("padding", 0), kw.get("output_padding", 0)
+    y = np.full(exp.shape, np.nan, np.float32)
+    ptr = lambda a: np.ascontiguousarray(a).ctypes.data_as(ctypes.c_void_p)
+    _lib.check(lib.ntg_conv_transpose2d(_lib.FLOAT32, ptr(x), ptr(w), y.ctypes.data_as(ctypes.c_void_p), B, Cin, H, W, Cog * groups,
+                                        kh, kw_, s, s, p, p, 1, 1, op, op, groups))
+    assert np.array_equal(y, F.conv_transpose2d(dev(x), dev(w), **kw).cpu().numpy())
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64, np.float16, "bf16", np.int32], ids=["fp32", "fp64", "fp16", "bf16", "int32"])
+def test_conv_transpose2d_random_vs_torch(dtype):
+    """Strides, dilations, groups and output_padding against torch's conv_transpose2d in double; integers bit-exact."""
+    bf = dtype == "bf16"
+    rng = np.random.default_rng(1500)
+    for (B, Cin, H, W, Cout, kh, kw_, s, p, op, d, groups) in [
+            (2, 6, 9, 11, 8, 3, 3, 1, 1, 0, 1, 2), (3, 4, 7, 6, 6, 2, 4, (2, 3), (1, 0), (1, 2), (2, 1), 1),
+            (2, 8, 13, 12, 4, 5, 3, 2, 2, 1, 1, 4), (4, 32, 20, 20, 48, 3, 3, 1, 1, 0, 1, 1)]:
+        if dtype == np.int32:
+            x = rng.integers(-4, 5, (B, Cin, H, W)).astype(np.int32)
+            w = rng.integers(-4, 5, (Cin, Cout // groups, kh, kw_)).astype(np.int32)
+        else:
+            x = randn(rng, (B, Cin, H, W), dtype)
+            w = randn(rng, (Cin, Cout // groups, kh, kw_), dtype, 1.0 / np.sqrt(Cin // groups * kh * kw_))
+        tx, tw = to_torch(x, DEV, bf), to_torch(w, DEV, bf)
+        out = F.conv_transpose2d(tx, tw, stride=s, padding=p, output_padding=op, dilation=d, groups=groups)
+        ref = torch.nn.functional.conv_transpose2d(tx.double().cpu(), tw.double().cpu(), None, s, p, op, groups, d)
+        assert tuple(out.shape) == tuple(ref.shape)
+        got = out.double().cpu()
+        if dtype == np.int32:
+            assert torch.equal(got, ref)
+        elif dtype in (np.float32, np.float64):
+            K = Cin // groups * kh * kw_
+            assert (got - ref).abs().max().item() <= 1e-5 * K * float(tx.abs().max().item() * tw.abs().max().item())
+        else:
+            assert (got - ref).abs().max().item() <= HALF_REL * ref.abs().max().item()
+    with pytest.raises(ValueError):
+        F.conv_transpose2d(tx, tw[:-1])
+    with pytest.raises((ValueError, _lib.NtgError)):
+        F.conv_transpose2d(tx, tw, stride=1, output_padding=1)
+
+
 def test_config5a_conv2d_resnet_block():
     """image [64,256,56,56], weight [256,256,3,3], stride 1, pad 1 (GEMM M=200704, K=2304, N=256)."""
     rng = np.random.default_rng(1007)
