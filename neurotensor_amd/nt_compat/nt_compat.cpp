@@ -553,6 +553,99 @@ ConvGrads conv2d_backward(const Tensor& image, const Tensor& kernel, const Tenso
     return out;
 }
 
+// [.., C, W] -> [B, C, 1, W] (contiguous view)
+static Tensor as_one_row(const Tensor& t, int64_t lead_if_low, const char* what) {
+    utils::throw_exception(!t.is_null(), std::string("Cannot perform operation ") + what + " on a null tensor");
+    Tensor c = t.contiguous();
+    const SizeRef& s = c.shape();
+    utils::throw_exception(s.size() >= 2, std::string("Expected to get a 2D or greater tensor for ") + what + ", but got " + std::to_string(s.size()) + "D");
+    const int64_t W = s[s.size() - 1], C = s[s.size() - 2];
+    const int64_t B = s.size() == 2 ? lead_if_low : c.numel() / std::max<int64_t>(1, C * W);
+    (void)lead_if_low;
+    return c.view({s.size() == 2 ? 1 : B, C, 1, W});
+}
+
+Tensor conv1d(const Tensor& image, const Tensor& kernel, int64_t stride, int64_t padding, int64_t dilation, int64_t groups) {
+    utils::throw_exception(!image.is_null() && !kernel.is_null(), "Cannot perform operation conv1d on a null tensor");
+    // conv.cpp:16-23
+    utils::throw_exception(image.dims() >= 2, "Expected to get a 2D or greater tensor as the input for a 1d convolution, but got " + std::to_string(image.dims()) + "D");
+    utils::throw_exception(kernel.dims() == 3 || kernel.dims() == 2, "Expected to get a 3D or 2D tensor as the kernel for a 1d convolution, but got " + std::to_string(kernel.dims()) + "D");
+    utils::throw_exception(stride >= 1, "Conv1d stride cannot be less than 1 but got " + std::to_string(stride));
+    utils::throw_exception(dilation >= 1, "Conv1d dilation cannot be less than 1 but got " + std::to_string(dilation));
+    utils::throw_exception(padding >= 0, "Conv1d padding cannot be less than 1 but got " + std::to_string(padding));
+    Tensor x = as_one_row(image, 1, "conv1d"), w = as_one_row(kernel, 1, "conv1d");
+    Tensor o = functional::conv2d(x, w, {1, stride}, {0, padding}, {1, dilation}, groups);
+    return o.view({o.shape()[0], o.shape()[1], o.shape()[3]});
+}
+
+ConvGrads conv1d_backward(const Tensor& image, const Tensor& kernel, const Tensor& grad, int64_t stride, int64_t padding, int64_t dilation,
+                          int64_t groups) {
+    Tensor x = as_one_row(image, 1, "conv1d backward"), w = as_one_row(kernel, 1, "conv1d backward");
+    ConvGrads g = functional::conv2d_backward(x, w, grad.contiguous(), {1, stride}, {0, padding}, {1, dilation}, groups);
+    return {g.d_image.view(image.shape()), g.d_kernel.view(kernel.shape())};
+}
+
+Tensor conv_transpose2d(const Tensor& image, const Tensor& kernel, utils::my_tuple s, utils::my_tuple p, utils::my_tuple op, utils::my_tuple d,
+                        int64_t groups) {
+    utils::throw_exception(!image.is_null() && !kernel.is_null(), "Cannot perform operation conv_transpose2d on a null tensor");
+    // conv.cpp:617-631
+    utils::throw_exception(image.dims() >= 3, "Expected to get a 3D or greater tensor as the input for a conv2d transpose, but got " + std::to_string(image.dims()) + "D");
+    utils::throw_exception(kernel.dims() == 4 || kernel.dims() == 3, "Expected to get a 4D or 3D tensor as the kernel for a conv2d transpose, but got " + std::to_string(kernel.dims()) + "D");
+    utils::throw_exception(image.dtype() == kernel.dtype(), std::string("Expected both kernel and image to have the same dtype for conv2d transpose but got ") +
+                                                                dtype_name(kernel.dtype()) + " and " + dtype_name(image.dtype()));
+    check_pair_ge(s, 1, "Conv2d Transpose stride cannot be less than 1");
+    check_pair_ge(d, 1, "Conv2d Transpose dilation cannot be less than 1");
+    check_pair_ge(op, 0, "Conv2d Transpose output_padding cannot be less than 1");
+    check_pair_ge(p, 0, "Conv2d Transpose padding cannot be less than 1");
+    utils::throw_exception(groups > 0, "Expected groups for a convolution to be greater than 0 but got " + std::to_string(groups));
+    Tensor x = image.contiguous(), w = kernel.contiguous();
+    const SizeRef& xs = x.shape();
+    const int64_t H = xs[xs.size() - 2], W = xs[xs.size() - 1], Cin = xs[xs.size() - 3];
+    const int64_t B = x.numel() / std::max<int64_t>(1, Cin * H * W);
+    const SizeRef& ws = w.shape();
+    const int64_t kh = ws[ws.size() - 2], kw = ws[ws.size() - 1], Cog = ws[ws.size() - 3], Wb = kernel.dims() == 4 ? ws[0] : 1;
+    utils::throw_exception(Cin == Wb, "Expected image channels to be the same as the kernel batches for conv_transpose2d but got " +
+                                          shape_str(x.shape()) + " and " + shape_str(w.shape()));
+    utils::throw_exception(Cin % groups == 0, "Expected image channels to be divisible by groups in Conv2d Transpose but got " + std::to_string(Cin) +
+                                                  " % " + std::to_string(groups) + " != 0");
+    const int64_t R = (H - 1) * s.first - 2 * p.first + d.first * (kh - 1) + 1 + op.first;
+    const int64_t Cc = (W - 1) * s.second - 2 * p.second + d.second * (kw - 1) + 1 + op.second;
+    utils::throw_exception(R > 0 && Cc > 0, "conv_transpose2d output would be empty");
+    Tensor out({B, Cog * groups, R, Cc}, x.dtype());
+    check_status(ntg_conv_transpose2d(static_cast<int>(x.dtype()), x.data_ptr(), w.data_ptr(), out.data_ptr(), B, Cin, H, W, Cog * groups, kh, kw,
+                                      s.first, s.second, p.first, p.second, d.first, d.second, op.first, op.second, groups));
+    return out;
+}
+
+ConvGrads conv_transpose2d_backward(const Tensor& image, const Tensor& kernel, const Tensor& grad, utils::my_tuple s, utils::my_tuple p,
+                                    utils::my_tuple op, utils::my_tuple d, int64_t groups) {
+    (void)op;   // the output size is the gradient's
+    utils::throw_exception(!image.is_null() && !kernel.is_null() && !grad.is_null(), "Cannot perform operation conv_transpose2d backward on a null tensor");
+    Tensor x = image.contiguous(), g = grad.contiguous();
+    Tensor dx = functional::conv2d(g, kernel, s, p, d, groups);
+    utils::throw_exception(dx.numel() == x.numel(), "grad does not have the shape of the transposed convolution's output");
+    ConvGrads kg = functional::conv2d_backward(g, kernel, x, s, p, d, groups);
+    return {dx.view(image.shape()), kg.d_kernel};
+}
+
+Tensor conv_transpose1d(const Tensor& image, const Tensor& kernel, int64_t stride, int64_t padding, int64_t output_padding, int64_t dilation,
+                        int64_t groups) {
+    utils::throw_exception(!image.is_null() && !kernel.is_null(), "Cannot perform operation conv_transpose1d on a null tensor");
+    utils::throw_exception(image.dims() >= 2, "Expected to get a 2D or greater tensor as the input for a conv1d transpose, but got " + std::to_string(image.dims()) + "D");
+    utils::throw_exception(kernel.dims() == 3 || kernel.dims() == 2, "Expected to get a 3D or 2D tensor as the kernel for a conv1d transpose, but got " + std::to_string(kernel.dims()) + "D");
+    Tensor x = as_one_row(image, 1, "conv_transpose1d"), w = as_one_row(kernel, 1, "conv_transpose1d");
+    Tensor o = functional::conv_transpose2d(x, w, {1, stride}, {0, padding}, {0, output_padding}, {1, dilation}, groups);
+    return o.view({o.shape()[0], o.shape()[1], o.shape()[3]});
+}
+
+ConvGrads conv_transpose1d_backward(const Tensor& image, const Tensor& kernel, const Tensor& grad, int64_t stride, int64_t padding,
+                                    int64_t output_padding, int64_t dilation, int64_t groups) {
+    Tensor x = as_one_row(image, 1, "conv_transpose1d backward"), w = as_one_row(kernel, 1, "conv_transpose1d backward");
+    Tensor g = as_one_row(grad, 1, "conv_transpose1d backward");
+    ConvGrads r = functional::conv_transpose2d_backward(x, w, g, {1, stride}, {0, padding}, {0, output_padding}, {1, dilation}, groups);
+    return {r.d_image.view(image.shape()), r.d_kernel.view(kernel.shape())};
+}
+
 }  // namespace functional
 
 namespace layers {

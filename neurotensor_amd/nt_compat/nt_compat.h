@@ -4,6 +4,7 @@
 //   nt::functional::matmult / matmult_cT / linear   nt/functional/tensor_files/matmult.h:10-13
 //   nt::functional::unfold2d                        nt/functional/tensor_files/colim_transform.cpp:565-588
 //   nt::functional::conv2d                          nt/functional/tensor_files/conv.h:12
+//   nt::functional::conv1d / conv_transpose1d / conv_transpose2d   nt/functional/tensor_files/conv.cpp:13-67, 538-676
 //   nt::matmult / nt::linear / nt::conv2d           nt/nt.h:835-850, 369-517 (positional form of the named-argument facade)
 //   nt::layers::Linear                              nt/nn/layers/Linear.h:10-20
 //   gradient GEMM selection of TensorGrad linear/matmult   nt/nn/functional/matmult.cpp:37-62, 253-275
@@ -99,6 +100,22 @@ struct ConvGrads { Tensor d_image, d_kernel; };
 ConvGrads conv2d_backward(const Tensor& image, const Tensor& kernel, const Tensor& grad, utils::my_tuple stride = {1, 1},
                           utils::my_tuple padding = {0, 0}, utils::my_tuple dilation = {1, 1}, int64_t groups = 1);
 
+// conv1d (conv.cpp:13-67), conv_transpose1d (:538-612), conv_transpose2d (:614-676) and their gradients.  The one-axis
+// forms are the two-axis ones with a single row; a transposed convolution is the image gradient of the convolution with
+// the same kernel, and its own gradients are that convolution and its kernel gradient with the operands exchanged.
+Tensor conv1d(const Tensor& image, const Tensor& kernel, int64_t stride = 1, int64_t padding = 0, int64_t dilation = 1, int64_t groups = 1);
+ConvGrads conv1d_backward(const Tensor& image, const Tensor& kernel, const Tensor& grad, int64_t stride = 1, int64_t padding = 0,
+                          int64_t dilation = 1, int64_t groups = 1);
+Tensor conv_transpose2d(const Tensor& image, const Tensor& kernel, utils::my_tuple stride = {1, 1}, utils::my_tuple padding = {0, 0},
+                        utils::my_tuple output_padding = {0, 0}, utils::my_tuple dilation = {1, 1}, int64_t groups = 1);
+ConvGrads conv_transpose2d_backward(const Tensor& image, const Tensor& kernel, const Tensor& grad, utils::my_tuple stride = {1, 1},
+                                    utils::my_tuple padding = {0, 0}, utils::my_tuple output_padding = {0, 0},
+                                    utils::my_tuple dilation = {1, 1}, int64_t groups = 1);
+Tensor conv_transpose1d(const Tensor& image, const Tensor& kernel, int64_t stride = 1, int64_t padding = 0, int64_t output_padding = 0,
+                        int64_t dilation = 1, int64_t groups = 1);
+ConvGrads conv_transpose1d_backward(const Tensor& image, const Tensor& kernel, const Tensor& grad, int64_t stride = 1, int64_t padding = 0,
+                                    int64_t output_padding = 0, int64_t dilation = 1, int64_t groups = 1);
+
 // what the backward lambdas of TensorGrad matmult / linear compute (flags only, no transposed copies)
 struct MatmultGrads { Tensor da, db; };
 MatmultGrads matmult_backward(const Tensor& a, const Tensor& b, const Tensor& grad, bool trans_a, bool trans_b);
@@ -119,6 +136,18 @@ inline Tensor linear(const Tensor& input, const Tensor& weight, const Tensor& bi
 inline Tensor conv2d(const Tensor& image, const Tensor& kernel, utils::my_tuple stride = {1, 1}, utils::my_tuple padding = {0, 0},
                      utils::my_tuple dilation = {1, 1}, int64_t groups = 1) {
     return functional::conv2d(image, kernel, stride, padding, dilation, groups);
+}
+
+inline Tensor conv1d(const Tensor& image, const Tensor& kernel, int64_t stride = 1, int64_t padding = 0, int64_t dilation = 1, int64_t groups = 1) {
+    return functional::conv1d(image, kernel, stride, padding, dilation, groups);
+}
+inline Tensor conv_transpose1d(const Tensor& image, const Tensor& kernel, int64_t stride = 1, int64_t padding = 0, int64_t output_padding = 0,
+                               int64_t dilation = 1, int64_t groups = 1) {
+    return functional::conv_transpose1d(image, kernel, stride, padding, output_padding, dilation, groups);
+}
+inline Tensor conv_transpose2d(const Tensor& image, const Tensor& kernel, utils::my_tuple stride = {1, 1}, utils::my_tuple padding = {0, 0},
+                               utils::my_tuple output_padding = {0, 0}, utils::my_tuple dilation = {1, 1}, int64_t groups = 1) {
+    return functional::conv_transpose2d(image, kernel, stride, padding, output_padding, dilation, groups);
 }
 
 namespace layers {

@@ -109,6 +109,10 @@ static void host_only_cases() {
     expect_throw("conv2d kernel dims", [] { nt::conv2d(F::zeros({1, 3, 8, 8}), F::zeros({3, 3})); });
     expect_throw("conv2d groups", [] { nt::conv2d(F::zeros({1, 3, 8, 8}), F::zeros({4, 3, 3, 3}), {1, 1}, {0, 0}, {1, 1}, 2); });
     expect_throw("conv2d stride", [] { nt::conv2d(F::zeros({1, 3, 8, 8}), F::zeros({4, 3, 3, 3}), {0, 1}); });
+    expect_throw("conv1d image dims", [] { nt::conv1d(F::zeros({8}), F::zeros({4, 3, 3})); });
+    expect_throw("conv1d stride", [] { nt::conv1d(F::zeros({1, 3, 8}), F::zeros({4, 3, 3}), 0); });
+    expect_throw("conv_transpose2d channels", [] { nt::conv_transpose2d(F::zeros({1, 3, 8, 8}), F::zeros({4, 3, 3, 3})); });
+    expect_throw("conv_transpose2d output_padding", [] { nt::conv_transpose2d(F::zeros({1, 3, 8, 8}), F::zeros({3, 4, 3, 3}), {1, 1}, {0, 0}, {-1, 0}); });
     expect_throw("unfold2d empty", [] { F::unfold2d(F::zeros({1, 1, 2, 2}), {5, 5}); });
     run_test("tensor views", [] {
         Tensor a = F::randn({3, 4, 5}, DType::Float32, 5);
@@ -238,6 +242,46 @@ static void device_cases(const std::string& g) {
             F::ConvGrads gr = F::conv2d_backward(x, w, F::from_numpy(g + "/conv2d_grad" + sfx + ".npy"), {1, 1}, {pad, pad}, {1, 1}, grouped ? 2 : 1);
             nt::utils::throw_exception(F::allclose(gr.d_image, F::from_numpy(g + "/conv2d_xgrad" + sfx + ".npy"), 1e-4, 1e-4), "xgrad differs from the fixture");
             nt::utils::throw_exception(F::allclose(gr.d_kernel, F::from_numpy(g + "/conv2d_wgrad" + sfx + ".npy"), 1e-4, 1e-3), "wgrad differs from the fixture");
+        });
+    }
+    // tests/src/conv_autograd_test.cpp:125-247 (conv1d), :555-716 (conv_transpose1d), :720-846 (conv_transpose2d)
+    auto close = [](const Tensor& a, const Tensor& b, const char* what) {
+        nt::utils::throw_exception(a.shape() == b.shape(), std::string(what) + " shape " + nt::shape_str(a.shape()));
+        nt::utils::throw_exception(F::allclose(a, b, 1e-4, 1e-3), std::string(what) + " differs from the fixture");
+    };
+    auto fixture = [&](const std::string& fam, const char* part, const char* sfx) { return F::from_numpy(g + "/" + fam + "_" + part + sfx + ".npy"); };
+    for (const char* sfx : {"", "_batched", "_grouped", "_grouped_batched"}) {
+        run_test((std::string("conv1d golden") + sfx).c_str(), [&] {
+            const bool grouped = std::strstr(sfx, "grouped") != nullptr;
+            Tensor x = fixture("conv1d", "input", sfx), w = fixture("conv1d", "weight", sfx);
+            Tensor o = nt::conv1d(x, w, 1, grouped ? 0 : 1, 1, grouped ? 2 : 1);
+            close(o, fixture("conv1d", "output", sfx), "conv1d output");
+            F::ConvGrads gr = F::conv1d_backward(x, w, fixture("conv1d", "grad", sfx), 1, grouped ? 0 : 1, 1, grouped ? 2 : 1);
+            close(gr.d_image, fixture("conv1d", "xgrad", sfx), "conv1d xgrad");
+            close(gr.d_kernel, fixture("conv1d", "wgrad", sfx), "conv1d wgrad");
+        });
+    }
+    struct TCase { const char* sfx; int64_t stride, padding, output_padding, groups; };
+    for (const TCase& c : {TCase{"", 2, 0, 1, 1}, TCase{"_grouped", 1, 1, 0, 2}, TCase{"_grouped_bigger", 1, 1, 0, 5}, TCase{"_batched", 2, 1, 1, 1},
+                           TCase{"_grouped_batched", 1, 1, 0, 2}}) {
+        run_test((std::string("conv_transpose1d golden") + c.sfx).c_str(), [&] {
+            Tensor x = fixture("conv_transpose1d", "input", c.sfx), w = fixture("conv_transpose1d", "weight", c.sfx);
+            Tensor o = nt::conv_transpose1d(x, w, c.stride, c.padding, c.output_padding, 1, c.groups);
+            close(o, fixture("conv_transpose1d", "output", c.sfx), "conv_transpose1d output");
+            F::ConvGrads gr = F::conv_transpose1d_backward(x, w, fixture("conv_transpose1d", "grad", c.sfx), c.stride, c.padding, c.output_padding, 1, c.groups);
+            close(gr.d_image, fixture("conv_transpose1d", "xgrad", c.sfx), "conv_transpose1d xgrad");
+            close(gr.d_kernel, fixture("conv_transpose1d", "wgrad", c.sfx), "conv_transpose1d wgrad");
+        });
+    }
+    for (const TCase& c : {TCase{"", 2, 0, 1, 1}, TCase{"_grouped", 1, 1, 0, 5}, TCase{"_batched", 2, 1, 1, 1}, TCase{"_grouped_batched", 1, 1, 0, 2}}) {
+        run_test((std::string("conv_transpose2d golden") + c.sfx).c_str(), [&] {
+            Tensor x = fixture("conv_transpose2d", "input", c.sfx), w = fixture("conv_transpose2d", "weight", c.sfx);
+            Tensor o = nt::conv_transpose2d(x, w, {c.stride, c.stride}, {c.padding, c.padding}, {c.output_padding, c.output_padding}, {1, 1}, c.groups);
+            close(o, fixture("conv_transpose2d", "output", c.sfx), "conv_transpose2d output");
+            F::ConvGrads gr = F::conv_transpose2d_backward(x, w, fixture("conv_transpose2d", "grad", c.sfx), {c.stride, c.stride}, {c.padding, c.padding},
+                                                           {c.output_padding, c.output_padding}, {1, 1}, c.groups);
+            close(gr.d_image, fixture("conv_transpose2d", "xgrad", c.sfx), "conv_transpose2d xgrad");
+            close(gr.d_kernel, fixture("conv_transpose2d", "wgrad", c.sfx), "conv_transpose2d wgrad");
         });
     }
     run_test("unfold2d golden", [&] {
