@@ -233,6 +233,47 @@ int ntg_conv_transpose2d(int dtype, const void* input, const void* kernel, void*
                          int64_t k_r, int64_t k_c, int64_t s_r, int64_t s_c, int64_t p_r, int64_t p_c, int64_t d_r, int64_t d_c,
                          int64_t op_r, int64_t op_c, int64_t groups);
 
+/* ---- convolutions over 1..4 spatial axes -----------------------------------------------------------------------
+ * functional::conv3d (nt/functional/tensor_files/conv.cpp:122-175), convnd (:177-316), conv_dimage / conv_dkernel for
+ * dim == 3 and the dynamic case (:347, :472), conv_transpose3d (:678-745), conv_transposend (:747-905); unfold3d / unfoldnd
+ * and their adjoints (nt/functional/cpu/unfold3d.cpp:9-80, unfoldnd.cpp, unfold3d_backward.cpp, unfoldnd_backward.cpp).
+ * size / kernel_size / stride / padding / dilation / output_padding point to `ndim` values, slowest axis first
+ * (depth, rows, columns).  image [batch, channels, size...], kernel [out_channels, channels/groups, kernel_size...]
+ * (transposed: [in_channels, out_channels/groups, kernel_size...]).  ndim 1 and 2 run on the conv2d entry points above;
+ * ndim 3 and 4 unfold into the workspace like the reference.  `backward` selects the workspace of the gradient call. */
+int ntg_unfoldnd_dev(int dtype, const void* image, void* col, int64_t batch, int64_t channels, int ndim, const int64_t* size,
+                     const int64_t* kernel_size, const int64_t* stride, const int64_t* padding, const int64_t* dilation, void* stream);
+int ntg_unfoldnd_backward_dev(int dtype, const void* col, void* image, int64_t batch, int64_t channels, int ndim, const int64_t* size,
+                              const int64_t* kernel_size, const int64_t* stride, const int64_t* padding, const int64_t* dilation,
+                              int accumulate, void* stream);
+int64_t ntg_convnd_workspace_bytes(int dtype, int64_t batch, int64_t channels, int64_t out_channels, int ndim, const int64_t* size,
+                                   const int64_t* kernel_size, const int64_t* stride, const int64_t* padding, const int64_t* dilation,
+                                   int64_t groups, int backward);
+int ntg_convnd_dev(int dtype, const void* image, const void* kernel, void* out, void* workspace, int64_t workspace_bytes,
+                   int64_t batch, int64_t channels, int64_t out_channels, int ndim, const int64_t* size, const int64_t* kernel_size,
+                   const int64_t* stride, const int64_t* padding, const int64_t* dilation, int64_t groups, void* stream);
+int ntg_convnd_backward_dev(int dtype, const void* image, const void* kernel, const void* grad_out, void* d_image, void* d_kernel,
+                            void* workspace, int64_t workspace_bytes, int64_t batch, int64_t channels, int64_t out_channels, int ndim,
+                            const int64_t* size, const int64_t* kernel_size, const int64_t* stride, const int64_t* padding,
+                            const int64_t* dilation, int64_t groups, int accumulate, void* stream);
+int64_t ntg_conv_transposend_workspace_bytes(int dtype, int64_t batch, int64_t in_channels, int64_t out_channels, int ndim,
+                                             const int64_t* in_size, const int64_t* kernel_size, const int64_t* stride,
+                                             const int64_t* padding, const int64_t* dilation, const int64_t* output_padding, int64_t groups);
+int ntg_conv_transposend_dev(int dtype, const void* input, const void* kernel, void* out, void* workspace, int64_t workspace_bytes,
+                             int64_t batch, int64_t in_channels, int64_t out_channels, int ndim, const int64_t* in_size,
+                             const int64_t* kernel_size, const int64_t* stride, const int64_t* padding, const int64_t* dilation,
+                             const int64_t* output_padding, int64_t groups, void* stream);
+/* host pointers, synchronous */
+int ntg_convnd(int dtype, const void* image, const void* kernel, void* out, int64_t batch, int64_t channels, int64_t out_channels, int ndim,
+               const int64_t* size, const int64_t* kernel_size, const int64_t* stride, const int64_t* padding, const int64_t* dilation,
+               int64_t groups);
+int ntg_convnd_backward(int dtype, const void* image, const void* kernel, const void* grad_out, void* d_image, void* d_kernel,
+                        int64_t batch, int64_t channels, int64_t out_channels, int ndim, const int64_t* size, const int64_t* kernel_size,
+                        const int64_t* stride, const int64_t* padding, const int64_t* dilation, int64_t groups, int accumulate);
+int ntg_conv_transposend(int dtype, const void* input, const void* kernel, void* out, int64_t batch, int64_t in_channels,
+                         int64_t out_channels, int ndim, const int64_t* in_size, const int64_t* kernel_size, const int64_t* stride,
+                         const int64_t* padding, const int64_t* dilation, const int64_t* output_padding, int64_t groups);
+
 #ifdef __cplusplus
 }
 #endif

@@ -42,6 +42,7 @@ class NtgError(RuntimeError):
 
 # every symbol include/ntgemm.h declares, with its ctypes signature
 _i64, _vp, _ci = ctypes.c_int64, ctypes.c_void_p, ctypes.c_int
+_pi64 = ctypes.POINTER(ctypes.c_int64)
 _pp = ctypes.POINTER(ctypes.c_void_p)
 SIGNATURES = {
     "ntg_last_error": (ctypes.c_char_p, []),
@@ -63,6 +64,16 @@ SIGNATURES = {
     "ntg_conv_transpose2d_workspace_bytes": (_i64, [_ci] + [_i64] * 16),
     "ntg_conv_transpose2d_dev": (_ci, [_ci, _vp, _vp, _vp, _vp, _i64] + [_i64] * 16 + [_vp]),
     "ntg_conv_transpose2d": (_ci, [_ci, _vp, _vp, _vp] + [_i64] * 16),
+    "ntg_unfoldnd_dev": (_ci, [_ci, _vp, _vp, _i64, _i64, _ci] + [_pi64] * 5 + [_vp]),
+    "ntg_unfoldnd_backward_dev": (_ci, [_ci, _vp, _vp, _i64, _i64, _ci] + [_pi64] * 5 + [_ci, _vp]),
+    "ntg_convnd_workspace_bytes": (_i64, [_ci, _i64, _i64, _i64, _ci] + [_pi64] * 5 + [_i64, _ci]),
+    "ntg_convnd_dev": (_ci, [_ci, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _ci] + [_pi64] * 5 + [_i64, _vp]),
+    "ntg_convnd_backward_dev": (_ci, [_ci, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _ci] + [_pi64] * 5 + [_i64, _ci, _vp]),
+    "ntg_conv_transposend_workspace_bytes": (_i64, [_ci, _i64, _i64, _i64, _ci] + [_pi64] * 6 + [_i64]),
+    "ntg_conv_transposend_dev": (_ci, [_ci, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _ci] + [_pi64] * 6 + [_i64, _vp]),
+    "ntg_convnd": (_ci, [_ci, _vp, _vp, _vp, _i64, _i64, _i64, _ci] + [_pi64] * 5 + [_i64]),
+    "ntg_convnd_backward": (_ci, [_ci, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _ci] + [_pi64] * 5 + [_i64, _ci]),
+    "ntg_conv_transposend": (_ci, [_ci, _vp, _vp, _vp, _i64, _i64, _i64, _ci] + [_pi64] * 6 + [_i64]),
     "ntg_conv2d_dev": (_ci, [_ci, _vp, _vp, _vp, _vp, _i64] + [_i64] * 14 + [_vp]),
     "ntg_unfold2d_backward": (_ci, [_ci, _vp, _vp] + [_i64] * 12 + [_ci]),
     "ntg_unfold2d_backward_dev": (_ci, [_ci, _vp, _vp] + [_i64] * 12 + [_ci, _vp]),

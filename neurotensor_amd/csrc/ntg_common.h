@@ -92,6 +92,17 @@ hipError_t launch_col2im(int dtype, const void* col, void* im,
                          int64_t k_r, int64_t k_c, int64_t s_r, int64_t s_c,
                          int64_t p_r, int64_t p_c, int64_t d_r, int64_t d_c, int accumulate, hipStream_t s);
 
+// unfold / col2im over 1..NTG_MAX_SPATIAL axes (slowest first); filled by the C API
+#define NTG_MAX_SPATIAL 4
+struct UnfoldNdParams {
+    int nd;
+    int64_t batch, channels;
+    int64_t size[NTG_MAX_SPATIAL], k[NTG_MAX_SPATIAL], s[NTG_MAX_SPATIAL], p[NTG_MAX_SPATIAL], d[NTG_MAX_SPATIAL], out[NTG_MAX_SPATIAL];
+    int64_t taps, L, vol, ccol, total;   // prod k, prod out, prod size, channels*taps, batch*ccol*L
+};
+hipError_t launch_unfoldnd(int64_t elem_size, const void* im, void* col, const UnfoldNdParams& u, hipStream_t s);
+hipError_t launch_col2imnd(int dtype, const void* col, void* im, const UnfoldNdParams& u, int accumulate, hipStream_t s);
+
 // conv2d backward helpers (unfold2d.hip): ordered sum of per-image weight gradients; weights of
 // the gradient-to-image convolution
 hipError_t launch_reduce_batch(int dtype, const void* part, void* out, int64_t batch, int64_t n, int accumulate, hipStream_t s);

@@ -801,4 +801,330 @@ int ntg_conv2d_backward(int dtype, const void* image, const void* kernel, const 
     return NTG_OK;
 }
 
+// ---------------------------------------------------------------------------------------------------
+// Convolutions over 1..4 spatial axes (conv3d conv.cpp:122-175, convnd :177-316, their gradients :347, :472 and
+// conv_transpose3d / conv_transposend :678-905): unfold -> matmult like the reference.  One and two axes go to
+// the 2-d entry points above (implicit GEMM); three and four axes store the unfolded matrix.
+// Geometry arrays hold `ndim` entries, slowest axis first (depth, rows, columns).
+static int fill_nd(ntg::UnfoldNdParams& u, int64_t batch, int64_t channels, int ndim, const int64_t* size, const int64_t* k,
+                   const int64_t* s, const int64_t* p, const int64_t* d) {
+    if (ndim < 1 || ndim > NTG_MAX_SPATIAL) return fail(NTG_ERR_INVALID_ARGUMENT, "ndim must be 1..%d but got %d", NTG_MAX_SPATIAL, ndim);
+    if (!size || !k || !s || !p || !d) return fail(NTG_ERR_INVALID_ARGUMENT, "null geometry array");
+    if (batch < 0 || channels < 0) return fail(NTG_ERR_INVALID_ARGUMENT, "negative size");
+    std::memset(&u, 0, sizeof u);
+    u.nd = ndim; u.batch = batch; u.channels = channels;
+    u.taps = 1; u.L = 1; u.vol = 1;
+    for (int a = 0; a < ndim; ++a) {
+        if (size[a] < 0) return fail(NTG_ERR_INVALID_ARGUMENT, "negative size");
+        if (k[a] < 1 || s[a] < 1 || d[a] < 1 || p[a] < 0) return fail(NTG_ERR_INVALID_ARGUMENT, "kernel/stride/dilation must be >= 1 and padding >= 0");
+        const int64_t span = size[a] + 2 * p[a] - d[a] * (k[a] - 1) - 1;
+        const int64_t o = span / s[a] + 1;
+        if (span < 0 || o <= 0) return fail(NTG_ERR_INVALID_ARGUMENT, "the array of sliding blocks would be empty (axis %d)", a);
+        u.size[a] = size[a]; u.k[a] = k[a]; u.s[a] = s[a]; u.p[a] = p[a]; u.d[a] = d[a]; u.out[a] = o;
+        u.taps *= k[a]; u.L *= o; u.vol *= size[a];
+    }
+    u.ccol = channels * u.taps;
+    u.total = batch * u.ccol * u.L;
+    return NTG_OK;
+}
+
+// trailing two axes of a 1- or 2-axis geometry as (rows, columns) for the 2-d entry points
+struct Geo2 { int64_t h, w, kr, kc, sr, sc, pr, pc, dr, dc; };
+static Geo2 as_2d(int ndim, const int64_t* size, const int64_t* k, const int64_t* s, const int64_t* p, const int64_t* d) {
+    if (ndim == 1) return {1, size[0], 1, k[0], 1, s[0], 0, p[0], 1, d[0]};
+    return {size[0], size[1], k[0], k[1], s[0], s[1], p[0], p[1], d[0], d[1]};
+}
+
+int ntg_unfoldnd_dev(int dtype, const void* image, void* col, int64_t batch, int64_t channels, int ndim, const int64_t* size,
+                     const int64_t* kernel_size, const int64_t* stride, const int64_t* padding, const int64_t* dilation, void* stream) {
+    const int64_t es = ntg::elem_size(dtype);
+    if (es == 0) return fail(NTG_ERR_UNSUPPORTED_DTYPE, "dtype %d is not supported", dtype);
+    ntg::UnfoldNdParams u;
+    int rc = fill_nd(u, batch, channels, ndim, size, kernel_size, stride, padding, dilation);
+    if (rc) return rc;
+    if (u.total == 0) return NTG_OK;
+    if (!image || !col) return fail(NTG_ERR_INVALID_ARGUMENT, "null pointer");
+    hipError_t e = ntg::launch_unfoldnd(es, image, col, u, static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return hip_fail(e, "unfoldnd launch");
+    return NTG_OK;
+}
+
+int ntg_unfoldnd_backward_dev(int dtype, const void* col, void* image, int64_t batch, int64_t channels, int ndim, const int64_t* size,
+                              const int64_t* kernel_size, const int64_t* stride, const int64_t* padding, const int64_t* dilation,
+                              int accumulate, void* stream) {
+    if (ntg::elem_size(dtype) == 0) return fail(NTG_ERR_UNSUPPORTED_DTYPE, "dtype %d is not supported", dtype);
+    ntg::UnfoldNdParams u;
+    int rc = fill_nd(u, batch, channels, ndim, size, kernel_size, stride, padding, dilation);
+    if (rc) return rc;
+    if (batch * channels * u.vol == 0) return NTG_OK;
+    if (!image || !col) return fail(NTG_ERR_INVALID_ARGUMENT, "null pointer");
+    hipError_t e = ntg::launch_col2imnd(dtype, col, image, u, accumulate, static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return hip_fail(e, "col2imnd launch");
+    return NTG_OK;
+}
+
+static int check_groups(int64_t channels, int64_t out_channels, int64_t groups) {
+    if (channels < 0 || out_channels < 0) return fail(NTG_ERR_INVALID_ARGUMENT, "negative size");
+    if (groups < 1) return fail(NTG_ERR_INVALID_ARGUMENT, "groups must be >= 1");
+    if (channels % groups != 0) return fail(NTG_ERR_INVALID_ARGUMENT, "image channels (%lld) not divisible by groups (%lld)", (long long)channels, (long long)groups);
+    if (out_channels % groups != 0) return fail(NTG_ERR_INVALID_ARGUMENT, "out channels (%lld) not divisible by groups (%lld)", (long long)out_channels, (long long)groups);
+    return NTG_OK;
+}
+
+int64_t ntg_convnd_workspace_bytes(int dtype, int64_t batch, int64_t channels, int64_t out_channels, int ndim, const int64_t* size,
+                                   const int64_t* kernel_size, const int64_t* stride, const int64_t* padding, const int64_t* dilation,
+                                   int64_t groups, int backward) {
+    const int64_t es = ntg::elem_size(dtype);
+    ntg::UnfoldNdParams u;
+    if (es == 0 || check_groups(channels, out_channels, groups) || fill_nd(u, batch, channels, ndim, size, kernel_size, stride, padding, dilation)) return -1;
+    if (ndim <= 2) {
+        const Geo2 g = as_2d(ndim, size, kernel_size, stride, padding, dilation);
+        return backward ? ntg_conv2d_backward_workspace_bytes(dtype, batch, channels, g.h, g.w, out_channels, g.kr, g.kc, g.sr, g.sc, g.pr, g.pc, g.dr, g.dc, groups)
+                        : ntg_conv2d_forward_workspace_bytes(dtype, batch, channels, g.h, g.w, g.kr, g.kc, g.sr, g.sc, g.pr, g.pc, g.dr, g.dc);
+    }
+    return u.total * es;
+}
+
+int ntg_convnd_dev(int dtype, const void* image, const void* kernel, void* out, void* workspace, int64_t workspace_bytes,
+                   int64_t batch, int64_t channels, int64_t out_channels, int ndim, const int64_t* size, const int64_t* kernel_size,
+                   const int64_t* stride, const int64_t* padding, const int64_t* dilation, int64_t groups, void* stream) {
+    const int64_t es = ntg::elem_size(dtype);
+    if (es == 0) return fail(NTG_ERR_UNSUPPORTED_DTYPE, "dtype %d is not supported", dtype);
+    int rc = check_groups(channels, out_channels, groups);
+    if (rc) return rc;
+    ntg::UnfoldNdParams u;
+    rc = fill_nd(u, batch, channels, ndim, size, kernel_size, stride, padding, dilation);
+    if (rc) return rc;
+    if (ndim <= 2) {
+        const Geo2 g = as_2d(ndim, size, kernel_size, stride, padding, dilation);
+        return ntg_conv2d_dev(dtype, image, kernel, out, workspace, workspace_bytes, batch, channels, g.h, g.w, out_channels, g.kr, g.kc,
+                              g.sr, g.sc, g.pr, g.pc, g.dr, g.dc, groups, stream);
+    }
+    if (batch == 0 || out_channels == 0) return NTG_OK;
+    if (!image || !kernel || !out) return fail(NTG_ERR_INVALID_ARGUMENT, "null pointer");
+    const int64_t need = u.total * es;
+    if (need > 0 && (!workspace || workspace_bytes < need))
+        return fail(NTG_ERR_INVALID_ARGUMENT, "workspace of %lld bytes needed, %lld given", (long long)need, (long long)workspace_bytes);
+    hipError_t e = ntg::launch_unfoldnd(es, image, workspace, u, static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return hip_fail(e, "unfoldnd launch");
+    // out_b[g*og:(g+1)*og, L] = W_g[og, add] . col_b[g*add:(g+1)*add, L]   (the reference's (col^T . W^T)^T, conv.cpp:143, :171)
+    const int64_t add = (channels / groups) * u.taps, og = out_channels / groups;
+    for (int64_t g = 0; g < groups; ++g) {
+        ntg_gemm_desc d;
+        std::memset(&d, 0, sizeof d);
+        d.dtype = dtype; d.c_mode = NTG_C_OVERWRITE;
+        d.m = og; d.k = add; d.n = u.L;
+        d.lda = add; d.ldb = u.L; d.ldc = u.L;
+        d.batches = batch;
+        d.stride_a = 0; d.stride_b = u.ccol * u.L; d.stride_c = out_channels * u.L;
+        rc = ntg_gemm_dev(&d, static_cast<const char*>(kernel) + g * og * add * es, static_cast<const char*>(workspace) + g * add * u.L * es,
+                          static_cast<char*>(out) + g * og * u.L * es, stream);
+        if (rc) return rc;
+    }
+    return NTG_OK;
+}
+
+int ntg_convnd_backward_dev(int dtype, const void* image, const void* kernel, const void* grad_out, void* d_image, void* d_kernel,
+                            void* workspace, int64_t workspace_bytes, int64_t batch, int64_t channels, int64_t out_channels, int ndim,
+                            const int64_t* size, const int64_t* kernel_size, const int64_t* stride, const int64_t* padding,
+                            const int64_t* dilation, int64_t groups, int accumulate, void* stream) {
+    const int64_t es = ntg::elem_size(dtype);
+    if (es == 0) return fail(NTG_ERR_UNSUPPORTED_DTYPE, "dtype %d is not supported", dtype);
+    int rc = check_groups(channels, out_channels, groups);
+    if (rc) return rc;
+    ntg::UnfoldNdParams u;
+    rc = fill_nd(u, batch, channels, ndim, size, kernel_size, stride, padding, dilation);
+    if (rc) return rc;
+    if (ndim <= 2) {
+        const Geo2 g = as_2d(ndim, size, kernel_size, stride, padding, dilation);
+        return ntg_conv2d_backward_dev(dtype, image, kernel, grad_out, d_image, d_kernel, workspace, workspace_bytes, batch, channels, g.h, g.w,
+                                       out_channels, g.kr, g.kc, g.sr, g.sc, g.pr, g.pc, g.dr, g.dc, groups, accumulate, stream);
+    }
+    if (batch == 0 || out_channels == 0 || channels == 0) return NTG_OK;
+    if (!kernel || !grad_out || (d_kernel && !image)) return fail(NTG_ERR_INVALID_ARGUMENT, "null pointer");
+    const int64_t need = u.total * es;
+    if (!workspace || workspace_bytes < need)
+        return fail(NTG_ERR_INVALID_ARGUMENT, "workspace of %lld bytes needed, %lld given", (long long)need, (long long)workspace_bytes);
+    const int64_t L = u.L, add = (channels / groups) * u.taps, og = out_channels / groups;
+    const char* kern = static_cast<const char*>(kernel);
+    const char* gy = static_cast<const char*>(grad_out);
+    char* ws = static_cast<char*>(workspace);
+    ntg_gemm_desc d;
+    if (d_kernel) {
+        hipError_t e = ntg::launch_unfoldnd(es, image, ws, u, static_cast<hipStream_t>(stream));
+        if (e != hipSuccess) return hip_fail(e, "unfoldnd launch");
+        for (int64_t g = 0; g < groups; ++g)
+            for (int64_t b = 0; b < batch; ++b) {
+                std::memset(&d, 0, sizeof d);
+                d.dtype = dtype; d.transpose_b = 1;
+                d.c_mode = (b == 0 && !accumulate) ? NTG_C_OVERWRITE : NTG_C_ACCUMULATE;
+                d.m = og; d.k = L; d.n = add;
+                d.lda = L; d.ldb = L; d.ldc = add; d.batches = 1;
+                rc = ntg_gemm_dev(&d, gy + ((b * out_channels + g * og) * L) * es, ws + ((b * u.ccol + g * add) * L) * es,
+                                  static_cast<char*>(d_kernel) + g * og * add * es, stream);
+                if (rc) return rc;
+            }
+    }
+    if (d_image) {
+        for (int64_t g = 0; g < groups; ++g) {
+            std::memset(&d, 0, sizeof d);
+            d.dtype = dtype; d.transpose_a = 1; d.c_mode = NTG_C_OVERWRITE;
+            d.m = add; d.k = og; d.n = L;
+            d.lda = add; d.ldb = L; d.ldc = L; d.batches = batch;
+            d.stride_a = 0; d.stride_b = out_channels * L; d.stride_c = u.ccol * L;
+            rc = ntg_gemm_dev(&d, kern + g * og * add * es, gy + g * og * L * es, ws + g * add * L * es, stream);
+            if (rc) return rc;
+        }
+        hipError_t e = ntg::launch_col2imnd(dtype, ws, d_image, u, accumulate, static_cast<hipStream_t>(stream));
+        if (e != hipSuccess) return hip_fail(e, "col2imnd launch");
+    }
+    return NTG_OK;
+}
+
+// output size of the transposed convolution per axis; the geometry of the convolution it is the adjoint of
+static int transpose_nd_out(int ndim, const int64_t* in_size, const int64_t* k, const int64_t* s, const int64_t* p, const int64_t* d,
+                            const int64_t* op, int64_t* out_size) {
+    if (ndim < 1 || ndim > NTG_MAX_SPATIAL) return fail(NTG_ERR_INVALID_ARGUMENT, "ndim must be 1..%d but got %d", NTG_MAX_SPATIAL, ndim);
+    if (!in_size || !k || !s || !p || !d || !op) return fail(NTG_ERR_INVALID_ARGUMENT, "null geometry array");
+    for (int a = 0; a < ndim; ++a) {
+        if (k[a] < 1 || s[a] < 1 || d[a] < 1 || p[a] < 0 || op[a] < 0)
+            return fail(NTG_ERR_INVALID_ARGUMENT, "kernel/stride/dilation must be >= 1 and padding/output_padding >= 0");
+        if (op[a] >= s[a]) return fail(NTG_ERR_INVALID_ARGUMENT, "output_padding (%lld) must be smaller than stride (%lld)", (long long)op[a], (long long)s[a]);
+        if (in_size[a] < 1) return fail(NTG_ERR_INVALID_ARGUMENT, "empty input");
+        out_size[a] = (in_size[a] - 1) * s[a] - 2 * p[a] + d[a] * (k[a] - 1) + 1 + op[a];
+        if (out_size[a] < 1) return fail(NTG_ERR_INVALID_ARGUMENT, "the output of the transposed convolution would be empty");
+    }
+    return NTG_OK;
+}
+
+int64_t ntg_conv_transposend_workspace_bytes(int dtype, int64_t batch, int64_t in_channels, int64_t out_channels, int ndim,
+                                             const int64_t* in_size, const int64_t* kernel_size, const int64_t* stride,
+                                             const int64_t* padding, const int64_t* dilation, const int64_t* output_padding, int64_t groups) {
+    int64_t os[NTG_MAX_SPATIAL];
+    if (ntg::elem_size(dtype) == 0 || check_groups(in_channels, out_channels, groups) ||
+        transpose_nd_out(ndim, in_size, kernel_size, stride, padding, dilation, output_padding, os)) return -1;
+    if (ndim <= 2) {
+        const Geo2 g = as_2d(ndim, in_size, kernel_size, stride, padding, dilation);
+        return ntg_conv_transpose2d_workspace_bytes(dtype, batch, in_channels, g.h, g.w, out_channels, g.kr, g.kc, g.sr, g.sc, g.pr, g.pc, g.dr, g.dc,
+                                                    ndim == 1 ? 0 : output_padding[0], output_padding[ndim - 1], groups);
+    }
+    return ntg_convnd_workspace_bytes(dtype, batch, out_channels, in_channels, ndim, os, kernel_size, stride, padding, dilation, groups, 1);
+}
+
+int ntg_conv_transposend_dev(int dtype, const void* input, const void* kernel, void* out, void* workspace, int64_t workspace_bytes,
+                             int64_t batch, int64_t in_channels, int64_t out_channels, int ndim, const int64_t* in_size,
+                             const int64_t* kernel_size, const int64_t* stride, const int64_t* padding, const int64_t* dilation,
+                             const int64_t* output_padding, int64_t groups, void* stream) {
+    if (ntg::elem_size(dtype) == 0) return fail(NTG_ERR_UNSUPPORTED_DTYPE, "dtype %d is not supported", dtype);
+    int rc = check_groups(in_channels, out_channels, groups);
+    if (rc) return rc;
+    int64_t os[NTG_MAX_SPATIAL];
+    rc = transpose_nd_out(ndim, in_size, kernel_size, stride, padding, dilation, output_padding, os);
+    if (rc) return rc;
+    if (ndim <= 2) {
+        const Geo2 g = as_2d(ndim, in_size, kernel_size, stride, padding, dilation);
+        return ntg_conv_transpose2d_dev(dtype, input, kernel, out, workspace, workspace_bytes, batch, in_channels, g.h, g.w, out_channels, g.kr, g.kc,
+                                        g.sr, g.sc, g.pr, g.pc, g.dr, g.dc, ndim == 1 ? 0 : output_padding[0], output_padding[ndim - 1], groups, stream);
+    }
+    if (batch == 0 || out_channels == 0) return NTG_OK;
+    if (in_channels == 0) return fail(NTG_ERR_INVALID_ARGUMENT, "empty input");
+    // the image gradient of the convolution [out_channels -> in_channels] over an image of the output's size
+    return ntg_convnd_backward_dev(dtype, nullptr, kernel, input, out, nullptr, workspace, workspace_bytes, batch, out_channels, in_channels, ndim,
+                                   os, kernel_size, stride, padding, dilation, groups, 0, stream);
+}
+
+// host-pointer forms (synchronous)
+int ntg_convnd(int dtype, const void* image, const void* kernel, void* out, int64_t batch, int64_t channels, int64_t out_channels, int ndim,
+               const int64_t* size, const int64_t* kernel_size, const int64_t* stride, const int64_t* padding, const int64_t* dilation, int64_t groups) {
+    const int64_t es = ntg::elem_size(dtype);
+    if (es == 0) return fail(NTG_ERR_UNSUPPORTED_DTYPE, "dtype %d is not supported", dtype);
+    int rc = check_groups(channels, out_channels, groups);
+    if (rc) return rc;
+    ntg::UnfoldNdParams u;
+    rc = fill_nd(u, batch, channels, ndim, size, kernel_size, stride, padding, dilation);
+    if (rc) return rc;
+    if (batch == 0 || out_channels == 0) return NTG_OK;
+    if (!image || !kernel || !out) return fail(NTG_ERR_INVALID_ARGUMENT, "null pointer");
+    const size_t im_bytes = (size_t)(batch * channels * u.vol * es), k_bytes = (size_t)(out_channels * (channels / groups) * u.taps * es);
+    const size_t o_bytes = (size_t)(batch * out_channels * u.L * es);
+    const int64_t wsb = ntg_convnd_workspace_bytes(dtype, batch, channels, out_channels, ndim, size, kernel_size, stride, padding, dilation, groups, 0);
+    DeviceMem mem;
+    const size_t o_k = align_up(im_bytes, 256), o_o = o_k + align_up(k_bytes, 256), o_ws = o_o + align_up(o_bytes, 256);
+    HIP_TRY(mem.alloc(o_ws + (size_t)wsb));
+    if (im_bytes) HIP_TRY(hipMemcpy(mem.at(0), image, im_bytes, hipMemcpyHostToDevice));
+    if (k_bytes) HIP_TRY(hipMemcpy(mem.at(o_k), kernel, k_bytes, hipMemcpyHostToDevice));
+    rc = ntg_convnd_dev(dtype, mem.at(0), mem.at(o_k), mem.at(o_o), mem.at(o_ws), wsb, batch, channels, out_channels, ndim, size, kernel_size,
+                        stride, padding, dilation, groups, nullptr);
+    if (rc) return rc;
+    HIP_TRY(hipStreamSynchronize(nullptr));
+    HIP_TRY(hipMemcpy(out, mem.at(o_o), o_bytes, hipMemcpyDeviceToHost));
+    return NTG_OK;
+}
+
+int ntg_convnd_backward(int dtype, const void* image, const void* kernel, const void* grad_out, void* d_image, void* d_kernel,
+                        int64_t batch, int64_t channels, int64_t out_channels, int ndim, const int64_t* size, const int64_t* kernel_size,
+                        const int64_t* stride, const int64_t* padding, const int64_t* dilation, int64_t groups, int accumulate) {
+    const int64_t es = ntg::elem_size(dtype);
+    if (es == 0) return fail(NTG_ERR_UNSUPPORTED_DTYPE, "dtype %d is not supported", dtype);
+    int rc = check_groups(channels, out_channels, groups);
+    if (rc) return rc;
+    ntg::UnfoldNdParams u;
+    rc = fill_nd(u, batch, channels, ndim, size, kernel_size, stride, padding, dilation);
+    if (rc) return rc;
+    if (batch == 0 || out_channels == 0 || channels == 0) return NTG_OK;
+    if (!image || !kernel || !grad_out) return fail(NTG_ERR_INVALID_ARGUMENT, "null pointer");
+    const size_t im_bytes = (size_t)(batch * channels * u.vol * es), k_bytes = (size_t)(out_channels * (channels / groups) * u.taps * es);
+    const size_t g_bytes = (size_t)(batch * out_channels * u.L * es);
+    const int64_t wsb = ntg_convnd_workspace_bytes(dtype, batch, channels, out_channels, ndim, size, kernel_size, stride, padding, dilation, groups, 1);
+    DeviceMem mem;
+    const size_t o_k = align_up(im_bytes, 256), o_g = o_k + align_up(k_bytes, 256), o_di = o_g + align_up(g_bytes, 256);
+    const size_t o_dk = o_di + align_up(im_bytes, 256), o_ws = o_dk + align_up(k_bytes, 256);
+    HIP_TRY(mem.alloc(o_ws + (size_t)wsb));
+    HIP_TRY(hipMemcpy(mem.at(0), image, im_bytes, hipMemcpyHostToDevice));
+    HIP_TRY(hipMemcpy(mem.at(o_k), kernel, k_bytes, hipMemcpyHostToDevice));
+    HIP_TRY(hipMemcpy(mem.at(o_g), grad_out, g_bytes, hipMemcpyHostToDevice));
+    if (accumulate && d_image) HIP_TRY(hipMemcpy(mem.at(o_di), d_image, im_bytes, hipMemcpyHostToDevice));
+    if (accumulate && d_kernel) HIP_TRY(hipMemcpy(mem.at(o_dk), d_kernel, k_bytes, hipMemcpyHostToDevice));
+    rc = ntg_convnd_backward_dev(dtype, mem.at(0), mem.at(o_k), mem.at(o_g), d_image ? mem.at(o_di) : nullptr, d_kernel ? mem.at(o_dk) : nullptr,
+                                 mem.at(o_ws), wsb, batch, channels, out_channels, ndim, size, kernel_size, stride, padding, dilation, groups,
+                                 accumulate, nullptr);
+    if (rc) return rc;
+    HIP_TRY(hipStreamSynchronize(nullptr));
+    if (d_image) HIP_TRY(hipMemcpy(d_image, mem.at(o_di), im_bytes, hipMemcpyDeviceToHost));
+    if (d_kernel) HIP_TRY(hipMemcpy(d_kernel, mem.at(o_dk), k_bytes, hipMemcpyDeviceToHost));
+    return NTG_OK;
+}
+
+int ntg_conv_transposend(int dtype, const void* input, const void* kernel, void* out, int64_t batch, int64_t in_channels, int64_t out_channels,
+                         int ndim, const int64_t* in_size, const int64_t* kernel_size, const int64_t* stride, const int64_t* padding,
+                         const int64_t* dilation, const int64_t* output_padding, int64_t groups) {
+    const int64_t es = ntg::elem_size(dtype);
+    if (es == 0) return fail(NTG_ERR_UNSUPPORTED_DTYPE, "dtype %d is not supported", dtype);
+    int rc = check_groups(in_channels, out_channels, groups);
+    if (rc) return rc;
+    int64_t os[NTG_MAX_SPATIAL];
+    rc = transpose_nd_out(ndim, in_size, kernel_size, stride, padding, dilation, output_padding, os);
+    if (rc) return rc;
+    if (batch == 0 || out_channels == 0) return NTG_OK;
+    if (!input || !kernel || !out) return fail(NTG_ERR_INVALID_ARGUMENT, "null pointer");
+    int64_t in_vol = 1, out_vol = 1, taps = 1;
+    for (int a = 0; a < ndim; ++a) { in_vol *= in_size[a]; out_vol *= os[a]; taps *= kernel_size[a]; }
+    const size_t in_bytes = (size_t)(batch * in_channels * in_vol * es), k_bytes = (size_t)(in_channels * (out_channels / groups) * taps * es);
+    const size_t o_bytes = (size_t)(batch * out_channels * out_vol * es);
+    const int64_t wsb = ntg_conv_transposend_workspace_bytes(dtype, batch, in_channels, out_channels, ndim, in_size, kernel_size, stride, padding,
+                                                             dilation, output_padding, groups);
+    if (wsb < 0) return fail(NTG_ERR_INVALID_ARGUMENT, "invalid geometry");
+    DeviceMem mem;
+    const size_t o_k = align_up(in_bytes, 256), o_o = o_k + align_up(k_bytes, 256), o_ws = o_o + align_up(o_bytes, 256);
+    HIP_TRY(mem.alloc(o_ws + (size_t)wsb));
+    if (in_bytes) HIP_TRY(hipMemcpy(mem.at(0), input, in_bytes, hipMemcpyHostToDevice));
+    if (k_bytes) HIP_TRY(hipMemcpy(mem.at(o_k), kernel, k_bytes, hipMemcpyHostToDevice));
+    rc = ntg_conv_transposend_dev(dtype, mem.at(0), mem.at(o_k), mem.at(o_o), mem.at(o_ws), wsb, batch, in_channels, out_channels, ndim, in_size,
+                                  kernel_size, stride, padding, dilation, output_padding, groups, nullptr);
+    if (rc) return rc;
+    HIP_TRY(hipStreamSynchronize(nullptr));
+    HIP_TRY(hipMemcpy(out, mem.at(o_o), o_bytes, hipMemcpyDeviceToHost));
+    return NTG_OK;
+}
+
 }  // extern "C"

@@ -136,6 +136,100 @@ hipError_t launch_flip_weights(int64_t es, const void* w, void* wt, int64_t grou
     return hipGetLastError();
 }
 
+// ---- the same two transforms over up to NTG_MAX_SPATIAL axes (unfold3d / unfoldnd and their adjoints:
+// nt/functional/cpu/unfold3d.cpp:9-80, unfoldnd.cpp, unfold3d_backward.cpp, unfoldnd_backward.cpp).
+// Row index of col: ((c*k0 + t0)*k1 + t1)*... ; column index: (o0*out1 + o1)*... ; last axis fastest.
+template <class T>
+__global__ void __launch_bounds__(256) unfoldnd_kernel(const T* __restrict__ im, T* __restrict__ col, const UnfoldNdParams u) {
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < u.total; idx += stride) {
+        int64_t l = idx % u.L;
+        int64_t t = idx / u.L;
+        const int64_t c = t % u.ccol;
+        const int64_t b = t / u.ccol;
+        int64_t tap = c % u.taps;
+        const int64_t c_im = c / u.taps;
+        int64_t off = 0, mult = 1;
+        bool ok = true;
+        for (int a = u.nd - 1; a >= 0; --a) {
+            const int64_t o = l % u.out[a];
+            l /= u.out[a];
+            const int64_t kk = tap % u.k[a];
+            tap /= u.k[a];
+            const int64_t pos = o * u.s[a] - u.p[a] + kk * u.d[a];
+            ok = ok && pos >= 0 && pos < u.size[a];
+            off += pos * mult;
+            mult *= u.size[a];
+        }
+        T v = 0;
+        if (ok) v = im[(b * u.channels + c_im) * u.vol + off];
+        col[idx] = v;
+    }
+}
+
+// gather form of the adjoint: taps visited in ascending order, as the reference's scatter loop reaches an element
+template <class T, class Acc>
+__global__ void __launch_bounds__(256) col2imnd_kernel(const T* __restrict__ col, T* __restrict__ im, const UnfoldNdParams u, const int accumulate) {
+    const int64_t total = u.batch * u.channels * u.vol;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += stride) {
+        int64_t pos[NTG_MAX_SPATIAL];
+        int64_t r = idx;
+        for (int a = u.nd - 1; a >= 0; --a) {
+            pos[a] = r % u.size[a];
+            r /= u.size[a];
+        }
+        const int64_t c = r % u.channels;
+        const int64_t b = r / u.channels;
+        Acc acc = accumulate ? (Acc)im[idx] : (Acc)0;
+        for (int64_t tap = 0; tap < u.taps; ++tap) {
+            int64_t tt = tap, l = 0, mult = 1;
+            bool ok = true;
+            for (int a = u.nd - 1; a >= 0 && ok; --a) {
+                const int64_t kk = tt % u.k[a];
+                tt /= u.k[a];
+                const int64_t on = pos[a] + u.p[a] - kk * u.d[a];
+                if (on < 0 || on % u.s[a] != 0 || on / u.s[a] >= u.out[a]) { ok = false; break; }
+                l += (on / u.s[a]) * mult;
+                mult *= u.out[a];
+            }
+            if (ok) acc += (Acc)col[((b * u.ccol + c * u.taps + tap) * u.L) + l];
+        }
+        im[idx] = (T)acc;
+    }
+}
+
+hipError_t launch_unfoldnd(int64_t es, const void* im, void* col, const UnfoldNdParams& u, hipStream_t s) {
+    if (u.total == 0) return hipSuccess;
+    const dim3 g(grid_for(u.total)), b(256);
+    switch (es) {
+    case 1: hipLaunchKernelGGL(unfoldnd_kernel<uint8_t>, g, b, 0, s, (const uint8_t*)im, (uint8_t*)col, u); break;
+    case 2: hipLaunchKernelGGL(unfoldnd_kernel<uint16_t>, g, b, 0, s, (const uint16_t*)im, (uint16_t*)col, u); break;
+    case 4: hipLaunchKernelGGL(unfoldnd_kernel<uint32_t>, g, b, 0, s, (const uint32_t*)im, (uint32_t*)col, u); break;
+    case 8: hipLaunchKernelGGL(unfoldnd_kernel<uint64_t>, g, b, 0, s, (const uint64_t*)im, (uint64_t*)col, u); break;
+    default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+
+hipError_t launch_col2imnd(int dtype, const void* col, void* im, const UnfoldNdParams& u, int accumulate, hipStream_t s) {
+    const int64_t total = u.batch * u.channels * u.vol;
+    if (total == 0) return hipSuccess;
+    const dim3 g(grid_for(total)), b(256);
+    switch (dtype) {
+    case DT_F32: hipLaunchKernelGGL((col2imnd_kernel<float, float>), g, b, 0, s, (const float*)col, (float*)im, u, accumulate); break;
+    case DT_F64: hipLaunchKernelGGL((col2imnd_kernel<double, double>), g, b, 0, s, (const double*)col, (double*)im, u, accumulate); break;
+    case DT_F16: hipLaunchKernelGGL((col2imnd_kernel<_Float16, float>), g, b, 0, s, (const _Float16*)col, (_Float16*)im, u, accumulate); break;
+    case DT_BF16: hipLaunchKernelGGL((col2imnd_kernel<__bf16, float>), g, b, 0, s, (const __bf16*)col, (__bf16*)im, u, accumulate); break;
+    case DT_I8: case DT_U8: hipLaunchKernelGGL((col2imnd_kernel<uint8_t, uint8_t>), g, b, 0, s, (const uint8_t*)col, (uint8_t*)im, u, accumulate); break;
+    case DT_I16: case DT_U16: hipLaunchKernelGGL((col2imnd_kernel<uint16_t, uint16_t>), g, b, 0, s, (const uint16_t*)col, (uint16_t*)im, u, accumulate); break;
+    case DT_I32: case DT_U32: hipLaunchKernelGGL((col2imnd_kernel<uint32_t, uint32_t>), g, b, 0, s, (const uint32_t*)col, (uint32_t*)im, u, accumulate); break;
+    case DT_I64: case DT_U64: hipLaunchKernelGGL((col2imnd_kernel<uint64_t, uint64_t>), g, b, 0, s, (const uint64_t*)col, (uint64_t*)im, u, accumulate); break;
+    default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+
 static hipError_t fill_params(UnfoldParams& u, int64_t batch, int64_t channels, int64_t height, int64_t width,
                               int64_t k_r, int64_t k_c, int64_t s_r, int64_t s_c, int64_t p_r, int64_t p_c, int64_t d_r, int64_t d_c) {
     u.batch = batch; u.channels = channels; u.height = height; u.width = width;

@@ -431,3 +431,138 @@ def conv_transpose1d_backward(image, kernel, grad, stride=1, padding=0, output_p
     dx, dw = conv_transpose2d_backward(x.unsqueeze(2), w.unsqueeze(2), grad.unsqueeze(-2), (1, stride), (0, padding),
                                        (0, output_padding), (1, dilation), groups)
     return dx.squeeze(2).reshape(image.shape), dw.squeeze(2).reshape(kernel.shape)
+
+
+# ---- convolutions over N spatial axes: conv3d / convnd / conv_transpose3d (tensor_files/conv.cpp:122-316, 678-905) ----
+def _ntuple(v, n):
+    return tuple(int(x) for x in v) if isinstance(v, (tuple, list)) else (int(v),) * n
+
+
+def _i64arr(vals):
+    return (ctypes.c_int64 * len(vals))(*vals)
+
+
+def convnd(image, kernel, stride=1, padding=0, dilation=1, groups=1):
+    """functional::conv3d / convnd: image [B, C, *size], kernel [O, C/groups, *k] with 1..4 spatial axes -> [B, O, *out]."""
+    _require_device(image, kernel)
+    nd = kernel.dim() - 2
+    if nd < 1 or nd > 4:
+        raise ValueError(f"Expected a kernel with 1 to 4 spatial dimensions but got {nd}")
+    if image.dim() != nd + 2:
+        raise ValueError(f"Expected to get a {nd + 2}D tensor as the input for a {nd}d convolution, but got {image.dim()}D")
+    if image.dtype != kernel.dtype:
+        raise ValueError(f"Expected both kernel and image to have the same dtype for conv{nd}d but got {kernel.dtype} and {image.dtype}")
+    s, p, d = _ntuple(stride, nd), _ntuple(padding, nd), _ntuple(dilation, nd)
+    if min(s) < 1:
+        raise ValueError(f"Conv{nd}d stride cannot be less than 1 but got {s}")
+    if min(d) < 1:
+        raise ValueError(f"Conv{nd}d dilation cannot be less than 1 but got {d}")
+    if min(p) < 0:
+        raise ValueError(f"Conv{nd}d padding cannot be less than 1 but got {p}")
+    x, w = image.contiguous(), kernel.contiguous()
+    B, C = x.shape[:2]
+    O, Cg = w.shape[:2]
+    size, k = tuple(x.shape[2:]), tuple(w.shape[2:])
+    if groups < 1 or C % groups != 0 or Cg * groups != C or O % groups != 0:
+        raise ValueError(f"Expected kernel rows times groups to be equal to rows of image Conv{nd}d but got {Cg} * {groups} != {C}")
+    out = tuple((size[a] + 2 * p[a] - d[a] * (k[a] - 1) - 1) // s[a] + 1 for a in range(nd))
+    if min(out) <= 0:
+        raise ValueError("the array of sliding blocks would be empty")
+    L = load()
+    dt = ntg_dtype(x)
+    geo = (_i64arr(size), _i64arr(k), _i64arr(s), _i64arr(p), _i64arr(d))
+    ws_bytes = L.ntg_convnd_workspace_bytes(dt, B, C, O, nd, *geo, groups, 0)
+    if ws_bytes < 0:
+        raise ValueError("invalid convolution geometry")
+    y = torch.empty((B, O) + out, dtype=x.dtype, device=x.device)
+    ws = torch.empty((max(ws_bytes, 1),), dtype=torch.uint8, device=x.device)
+    check(L.ntg_convnd_dev(dt, x.data_ptr(), w.data_ptr(), y.data_ptr(), ws.data_ptr(), ws_bytes, B, C, O, nd, *geo, groups, _stream()))
+    return y
+
+
+def convnd_backward(image, kernel, grad, stride=1, padding=0, dilation=1, groups=1):
+    """conv_dimage + conv_dkernel for 1..4 spatial axes (conv.cpp:318-535): returns (d_image, d_kernel)."""
+    _require_device(image, kernel, grad)
+    nd = kernel.dim() - 2
+    s, p, d = _ntuple(stride, nd), _ntuple(padding, nd), _ntuple(dilation, nd)
+    x, w, g = image.contiguous(), kernel.contiguous(), grad.contiguous()
+    B, C = x.shape[:2]
+    O = w.shape[0]
+    size, k = tuple(x.shape[2:]), tuple(w.shape[2:])
+    L = load()
+    dt = ntg_dtype(x)
+    geo = (_i64arr(size), _i64arr(k), _i64arr(s), _i64arr(p), _i64arr(d))
+    ws_bytes = L.ntg_convnd_workspace_bytes(dt, B, C, O, nd, *geo, groups, 1)
+    if ws_bytes < 0:
+        raise ValueError("invalid convolution geometry")
+    dx, dw = torch.empty_like(x), torch.empty_like(w)
+    ws = torch.empty((max(ws_bytes, 1),), dtype=torch.uint8, device=x.device)
+    check(L.ntg_convnd_backward_dev(dt, x.data_ptr(), w.data_ptr(), g.data_ptr(), dx.data_ptr(), dw.data_ptr(), ws.data_ptr(), ws_bytes,
+                                    B, C, O, nd, *geo, groups, 0, _stream()))
+    return dx, dw
+
+
+def conv3d(image, kernel, stride=1, padding=0, dilation=1, groups=1):
+    """functional::conv3d (conv.cpp:122-175): image [.., C, D, H, W], kernel [O, C/groups, kd, kh, kw]."""
+    if image.dim() < 4:
+        raise ValueError(f"Expected to get a 4D or greater tensor as the input for a 3d convolution, but got {image.dim()}D")
+    if kernel.dim() not in (4, 5):
+        raise ValueError(f"Expected to get a 5D or 4D tensor as the kernel for a 3d convolution, but got {kernel.dim()}D")
+    x = image.reshape((1,) + tuple(image.shape)) if image.dim() == 4 else image.reshape((-1,) + tuple(image.shape[-4:]))
+    w = kernel.reshape((1,) + tuple(kernel.shape)) if kernel.dim() == 4 else kernel
+    return convnd(x, w, stride, padding, dilation, groups)
+
+
+def conv3d_backward(image, kernel, grad, stride=1, padding=0, dilation=1, groups=1):
+    x = image.reshape((1,) + tuple(image.shape)) if image.dim() == 4 else image.reshape((-1,) + tuple(image.shape[-4:]))
+    w = kernel.reshape((1,) + tuple(kernel.shape)) if kernel.dim() == 4 else kernel
+    dx, dw = convnd_backward(x, w, grad, stride, padding, dilation, groups)
+    return dx.reshape(image.shape), dw.reshape(kernel.shape)
+
+
+def conv_transposend(image, kernel, stride=1, padding=0, output_padding=0, dilation=1, groups=1):
+    """functional::conv_transpose3d / conv_transposend (conv.cpp:678-905): image [B, Cin, *size], kernel [Cin, Cout/groups, *k]."""
+    _require_device(image, kernel)
+    nd = kernel.dim() - 2
+    if image.dim() != nd + 2:
+        raise ValueError(f"Expected to get a {nd + 2}D tensor as the input for a conv{nd}d transpose, but got {image.dim()}D")
+    s, p, op, d = _ntuple(stride, nd), _ntuple(padding, nd), _ntuple(output_padding, nd), _ntuple(dilation, nd)
+    x, w = image.contiguous(), kernel.contiguous()
+    B, Cin = x.shape[:2]
+    if w.shape[0] != Cin:
+        raise ValueError(f"Expected image channels to be the same as the kernel batches for conv_transpose{nd}d but got {tuple(x.shape)} and {tuple(w.shape)}")
+    if groups < 1 or Cin % groups != 0:
+        raise ValueError(f"Expected image channels to be divisible by groups in Conv{nd}d Transpose but got {Cin} % {groups} != 0")
+    Cout = w.shape[1] * groups
+    size, k = tuple(x.shape[2:]), tuple(w.shape[2:])
+    out = tuple((size[a] - 1) * s[a] - 2 * p[a] + d[a] * (k[a] - 1) + 1 + op[a] for a in range(nd))
+    L = load()
+    dt = ntg_dtype(x)
+    geo = (_i64arr(size), _i64arr(k), _i64arr(s), _i64arr(p), _i64arr(d), _i64arr(op))
+    ws_bytes = L.ntg_conv_transposend_workspace_bytes(dt, B, Cin, Cout, nd, *geo, groups)
+    if ws_bytes < 0:
+        raise ValueError("invalid transposed-convolution geometry: " + L.ntg_last_error().decode())
+    y = torch.empty((B, Cout) + out, dtype=x.dtype, device=x.device)
+    ws = torch.empty((max(ws_bytes, 1),), dtype=torch.uint8, device=x.device)
+    check(L.ntg_conv_transposend_dev(dt, x.data_ptr(), w.data_ptr(), y.data_ptr(), ws.data_ptr(), ws_bytes, B, Cin, Cout, nd, *geo, groups,
+                                     _stream()))
+    return y
+
+
+def conv_transposend_backward(image, kernel, grad, stride=1, padding=0, output_padding=0, dilation=1, groups=1):
+    """Gradients of the transposed convolution through its adjoint: d_image = convnd(grad, kernel), d_kernel = conv_dkernel
+    with image and output gradient exchanged."""
+    g = grad.contiguous()
+    dx = convnd(g, kernel, stride, padding, dilation, groups)
+    _, dw = convnd_backward(g, kernel, image.contiguous(), stride, padding, dilation, groups)
+    return dx.reshape(image.shape), dw
+
+
+def conv_transpose3d(image, kernel, stride=1, padding=0, output_padding=0, dilation=1, groups=1):
+    if image.dim() < 4:
+        raise ValueError(f"Expected to get a 4D or greater tensor as the input for a conv3d transpose, but got {image.dim()}D")
+    if kernel.dim() not in (4, 5):
+        raise ValueError(f"Expected to get a 5D or 4D tensor as the kernel for a conv3d transpose, but got {kernel.dim()}D")
+    x = image.reshape((1,) + tuple(image.shape)) if image.dim() == 4 else image.reshape((-1,) + tuple(image.shape[-4:]))
+    w = kernel.reshape((1,) + tuple(kernel.shape)) if kernel.dim() == 4 else kernel
+    return conv_transposend(x, w, stride, padding, output_padding, dilation, groups)

@@ -401,3 +401,123 @@ def conv_transpose1d_backward(image, kernel, grad, stride=1, padding=0, output_p
                                        np.ascontiguousarray(grad)[..., None, :], (1, stride), (0, padding), (0, output_padding),
                                        (1, dilation), groups, kind)
     return dx[:, :, 0, :].reshape(image.shape), dw[:, :, 0, :].reshape(kernel.shape)
+
+
+# ---- convolutions over N spatial axes (conv3d conv.cpp:122-175, convnd :177-316, conv_transpose3d :678-745) ----
+def _ntuple(v, n):
+    return tuple(int(x) for x in v) if isinstance(v, (tuple, list)) else (int(v),) * n
+
+
+def unfoldnd(x, kernel_size, dilation=1, padding=0, stride=1):
+    """functional::unfold3d / unfoldnd with transpose_out=true: x [B, C, *size] -> col [B, C*prod(k), prod(out)];
+    row index ((c*k0 + t0)*k1 + t1)..., column index (o0*out1 + o1)... (nt/functional/cpu/unfold3d.cpp:9-80).
+    Pure data movement, written with numpy slicing (one strided copy per tap)."""
+    x = np.ascontiguousarray(x)
+    nd = x.ndim - 2
+    k, d, p, s = _ntuple(kernel_size, nd), _ntuple(dilation, nd), _ntuple(padding, nd), _ntuple(stride, nd)
+    B, C = x.shape[:2]
+    size = x.shape[2:]
+    out = tuple((size[a] + 2 * p[a] - d[a] * (k[a] - 1) - 1) // s[a] + 1 for a in range(nd))
+    if min(out) <= 0:
+        raise ValueError("the array of sliding blocks would be empty")
+    xp = np.zeros((B, C) + tuple(size[a] + 2 * p[a] for a in range(nd)), dtype=x.dtype)
+    xp[(slice(None), slice(None)) + tuple(slice(p[a], p[a] + size[a]) for a in range(nd))] = x
+    col = np.zeros((B, C) + k + out, dtype=x.dtype)
+    for tap in np.ndindex(*k):
+        src = tuple(slice(tap[a] * d[a], tap[a] * d[a] + (out[a] - 1) * s[a] + 1, s[a]) for a in range(nd))
+        col[(slice(None), slice(None)) + tap] = xp[(slice(None), slice(None)) + src]
+    return col.reshape(B, C * int(np.prod(k)), int(np.prod(out))), out
+
+
+def unfoldnd_backward(col, size, kernel_size, dilation=1, padding=0, stride=1):
+    """The adjoint of unfoldnd (unfold3d_backward.cpp / unfoldnd_backward.cpp): taps are added in ascending order."""
+    nd = len(size)
+    k, d, p, s = _ntuple(kernel_size, nd), _ntuple(dilation, nd), _ntuple(padding, nd), _ntuple(stride, nd)
+    out = tuple((size[a] + 2 * p[a] - d[a] * (k[a] - 1) - 1) // s[a] + 1 for a in range(nd))
+    B = col.shape[0]
+    C = col.shape[1] // int(np.prod(k))
+    c6 = col.reshape((B, C) + k + out)
+    xp = np.zeros((B, C) + tuple(size[a] + 2 * p[a] for a in range(nd)), dtype=col.dtype)
+    for tap in np.ndindex(*k):
+        dst = tuple(slice(tap[a] * d[a], tap[a] * d[a] + (out[a] - 1) * s[a] + 1, s[a]) for a in range(nd))
+        xp[(slice(None), slice(None)) + dst] += c6[(slice(None), slice(None)) + tap]
+    return np.ascontiguousarray(xp[(slice(None), slice(None)) + tuple(slice(p[a], p[a] + size[a]) for a in range(nd))])
+
+
+def convnd(image, kernel, stride=1, padding=0, dilation=1, groups=1, kind="closed"):
+    """conv3d / convnd: unfold, then per group matmult(col_g, W_g, true, true) transposed back (conv.cpp:134-174)."""
+    x = np.ascontiguousarray(image)
+    w = np.ascontiguousarray(kernel)
+    nd = w.ndim - 2
+    B, C = x.shape[:2]
+    O = w.shape[0]
+    col, out = unfoldnd(x, w.shape[2:], dilation, padding, stride)
+    add = (C // groups) * int(np.prod(w.shape[2:]))
+    og = O // groups
+    res = np.zeros((B, O, col.shape[2]), dtype=x.dtype)
+    for g in range(groups):
+        colg = np.ascontiguousarray(col[:, g * add:(g + 1) * add, :])
+        wg = np.ascontiguousarray(w[g * og:(g + 1) * og].reshape(og, -1))
+        res[:, g * og:(g + 1) * og, :] = matmult(colg, wg, None, True, True, kind=kind).transpose(0, 2, 1)
+    return res.reshape((B, O) + out)
+
+
+def convnd_backward(image, kernel, grad, stride=1, padding=0, dilation=1, groups=1, kind="closed"):
+    """conv_dimage / conv_dkernel for any number of axes (conv.cpp:318-535): d_col = W_g^T . dY then the unfold adjoint;
+    d_kernel = sum over the batch of dY_b . col_b^T."""
+    x = np.ascontiguousarray(image)
+    w = np.ascontiguousarray(kernel)
+    B, C = x.shape[:2]
+    O = w.shape[0]
+    col, out = unfoldnd(x, w.shape[2:], dilation, padding, stride)
+    g3 = np.ascontiguousarray(grad).reshape(B, O, -1)
+    add = (C // groups) * int(np.prod(w.shape[2:]))
+    og = O // groups
+    dcol = np.zeros_like(col)
+    dk = np.zeros((O, add), dtype=x.dtype)
+    for g in range(groups):
+        wg = np.ascontiguousarray(w[g * og:(g + 1) * og].reshape(og, -1))
+        gg = np.ascontiguousarray(g3[:, g * og:(g + 1) * og, :])
+        dcol[:, g * add:(g + 1) * add, :] = matmult(wg, gg, None, True, False, kind=kind)
+        colg = np.ascontiguousarray(col[:, g * add:(g + 1) * add, :])
+        dk[g * og:(g + 1) * og] = matmult(gg, colg, None, False, True, kind=kind).sum(axis=0)
+    dimg = unfoldnd_backward(dcol, x.shape[2:], w.shape[2:], dilation, padding, stride)
+    return dimg, dk.reshape(w.shape)
+
+
+def conv_transposend(image, kernel, stride=1, padding=0, output_padding=0, dilation=1, groups=1, kind="closed"):
+    """conv_transpose3d / conv_transposend (conv.cpp:678-905): zero-dilate by the stride, pad the far side by output_padding,
+    unfold with padding d*(k-1) - p and stride 1, matmult with the channel-swapped, tap-reversed kernel per group."""
+    x = np.ascontiguousarray(image)
+    w = np.ascontiguousarray(kernel)
+    nd = w.ndim - 2
+    s, p, op, d = _ntuple(stride, nd), _ntuple(padding, nd), _ntuple(output_padding, nd), _ntuple(dilation, nd)
+    B, Cin = x.shape[:2]
+    size = x.shape[2:]
+    k = w.shape[2:]
+    Cog = w.shape[1]
+    xd = np.zeros((B, Cin) + tuple((size[a] - 1) * s[a] + 1 + op[a] for a in range(nd)), dtype=x.dtype)
+    xd[(slice(None), slice(None)) + tuple(slice(0, (size[a] - 1) * s[a] + 1, s[a]) for a in range(nd))] = x
+    pad = tuple((k[a] - 1) * d[a] - p[a] for a in range(nd))
+    assert min(pad) >= 0
+    col, out = unfoldnd(xd, k, d, pad, 1)
+    flip = (slice(None), slice(None)) + (slice(None, None, -1),) * nd
+    wt = np.ascontiguousarray(np.swapaxes(w, 0, 1)[flip])                      # [Cout/g, Cin, *k]
+    cig = Cin // groups
+    add = cig * int(np.prod(k))
+    res = np.zeros((B, Cog * groups, col.shape[2]), dtype=x.dtype)
+    for g in range(groups):
+        kg = np.ascontiguousarray(wt[:, g * cig:(g + 1) * cig].reshape(Cog, -1))
+        colg = np.ascontiguousarray(col[:, g * add:(g + 1) * add, :])
+        res[:, g * Cog:(g + 1) * Cog, :] = matmult(kg, colg, None, False, False, kind=kind)
+    return res.reshape((B, Cog * groups) + out)
+
+
+def conv_transposend_backward(image, kernel, grad, stride=1, padding=0, output_padding=0, dilation=1, groups=1, kind="closed"):
+    """Adjoint relations as for conv_transpose2d_backward."""
+    x = np.ascontiguousarray(image)
+    w = np.ascontiguousarray(kernel)
+    g = np.ascontiguousarray(grad)
+    dx = convnd(g, w, stride, padding, dilation, groups, kind)
+    _, dw = convnd_backward(g, w, x, stride, padding, dilation, groups, kind)
+    return dx.reshape(x.shape), dw

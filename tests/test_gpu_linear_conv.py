@@ -444,6 +444,81 @@ def test_conv_transpose2d_random_vs_torch(dtype):
         F.conv_transpose2d(tx, tw, stride=1, output_padding=1)
 
 
+@pytest.mark.parametrize("sfx,kw", [("", dict(stride=1, padding=1)), ("_grouped", dict(stride=1, groups=2)),
+                                    ("_batched", dict(stride=1, padding=1)), ("_grouped_batched", dict(stride=1, groups=2))])
+def test_conv3d_golden(golden_dir, sfx, kw):
+    """tests/src/conv_autograd_test.cpp:375-497 on the GPU path."""
+    _gpu_family(golden_dir, "conv3d", sfx, F.conv3d, F.conv3d_backward, oracle.convnd, oracle.convnd_backward, kw)
+
+
+@pytest.mark.parametrize("sfx,kw", [("", dict(stride=2, output_padding=1)), ("_grouped_batched", dict(stride=1, groups=2, padding=1))])
+def test_conv_transpose3d_golden(golden_dir, sfx, kw):
+    """tests/src/conv_autograd_test.cpp:847-971 on the GPU path."""
+    _gpu_family(golden_dir, "conv_transpose3d", sfx, F.conv_transpose3d, F.conv_transposend_backward,
+                oracle.conv_transposend, oracle.conv_transposend_backward, kw)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64, np.float16, "bf16", np.int32], ids=["fp32", "fp64", "fp16", "bf16", "int32"])
+def test_conv3d_and_transpose_random_vs_torch(dtype):
+    """conv3d / conv_transpose3d forward and gradients with strides, dilations, padding and groups against torch in double;
+    the unfold itself bit-exact against the oracle; 4 spatial axes against the oracle."""
+    bf = dtype == "bf16"
+    ints = dtype == np.int32
+    rng = np.random.default_rng(1600)
+    for (B, C, size, O, k, s, p, d, groups) in [(2, 4, (6, 7, 8), 6, (2, 3, 2), (1, 2, 1), (1, 0, 2), (2, 1, 1), 2),
+                                                (3, 3, (9, 8, 7), 5, (3, 3, 3), 1, 1, 1, 1), (2, 8, (5, 10, 6), 4, (1, 2, 3), 2, (0, 1, 1), 1, 4)]:
+        if ints:
+            x = rng.integers(-4, 5, (B, C) + size).astype(np.int32)
+            w = rng.integers(-4, 5, (O, C // groups) + k).astype(np.int32)
+        else:
+            x = randn(rng, (B, C) + size, dtype)
+            w = randn(rng, (O, C // groups) + k, dtype, 1.0 / np.sqrt(C // groups * np.prod(k)))
+        tx, tw = to_torch(x, DEV, bf), to_torch(w, DEV, bf)
+        y = F.conv3d(tx, tw, stride=s, padding=p, dilation=d, groups=groups)
+        rx = tx.double().cpu().requires_grad_(not ints)
+        rw = tw.double().cpu().requires_grad_(not ints)
+        ry = torch.nn.functional.conv3d(rx, rw, None, s, p, d, groups)
+        assert tuple(y.shape) == tuple(ry.shape)
+        K = C // groups * int(np.prod(k))
+        if ints:
+            assert torch.equal(y.double().cpu(), ry)
+            continue
+        tol = (1e-5 * K * float(tx.abs().max().item() * tw.abs().max().item())) if dtype in (np.float32, np.float64) else HALF_REL * ry.abs().max().item()
+        assert (y.double().cpu() - ry.detach()).abs().max().item() <= tol
+        g = randn(rng, tuple(ry.shape), dtype)
+        tg = to_torch(g, DEV, bf)
+        ry.backward(tg.double().cpu())
+        dx, dw = F.conv3d_backward(tx, tw, tg, stride=s, padding=p, dilation=d, groups=groups)
+        rel = 1e-4 if dtype in (np.float32, np.float64) else HALF_REL
+        assert (dx.double().cpu() - rx.grad).abs().max().item() <= rel * max(1.0, rx.grad.abs().max().item())
+        assert (dw.double().cpu() - rw.grad).abs().max().item() <= rel * max(1.0, rw.grad.abs().max().item())
+        # transposed: the same kernel tensor read as [Cin = O, Cout/groups = C/groups, *k]
+        xt = to_torch(randn(rng, tuple(ry.shape), dtype), DEV, bf)
+        yt = F.conv_transpose3d(xt, tw, stride=s, padding=p, dilation=d, groups=groups)
+        rt = torch.nn.functional.conv_transpose3d(xt.double().cpu(), tw.double().cpu(), None, s, p, 0, groups, d)
+        assert tuple(yt.shape) == tuple(rt.shape)
+        assert (yt.double().cpu() - rt).abs().max().item() <= rel * max(1.0, rt.abs().max().item()) * (10 if dtype in (np.float32, np.float64) else 1)
+    # 4 spatial axes, and the unfold alone
+    x4 = randn(rng, (2, 3, 4, 5, 4, 6), np.float32)
+    w4 = randn(rng, (4, 3, 2, 2, 1, 3), np.float32, 0.3)
+    y4 = F.convnd(dev(x4), dev(w4), stride=(1, 2, 1, 1), padding=(1, 0, 0, 1), dilation=1)
+    assert np.abs(y4.cpu().numpy() - oracle.convnd(x4, w4, (1, 2, 1, 1), (1, 0, 0, 1), 1)).max() <= 1e-4
+    lib = _lib.load()
+    x3 = randn(rng, (2, 3, 6, 5, 7), np.float32)
+    ref_col, out = oracle.unfoldnd(x3, (2, 3, 2), (2, 1, 1), (1, 0, 2), (1, 2, 1))
+    col = torch.empty(ref_col.shape, dtype=torch.float32, device=DEV)
+    arr = lambda v: (ctypes.c_int64 * 3)(*v)
+    st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    _lib.check(lib.ntg_unfoldnd_dev(_lib.FLOAT32, dev(x3).data_ptr(), col.data_ptr(), 2, 3, 3, arr((6, 5, 7)), arr((2, 3, 2)), arr((1, 2, 1)),
+                                    arr((1, 0, 2)), arr((2, 1, 1)), st))
+    assert np.array_equal(col.cpu().numpy(), ref_col)
+    gcol = randn(rng, ref_col.shape, np.float32)
+    back = torch.empty((2, 3, 6, 5, 7), dtype=torch.float32, device=DEV)
+    _lib.check(lib.ntg_unfoldnd_backward_dev(_lib.FLOAT32, dev(gcol).data_ptr(), back.data_ptr(), 2, 3, 3, arr((6, 5, 7)), arr((2, 3, 2)),
+                                             arr((1, 2, 1)), arr((1, 0, 2)), arr((2, 1, 1)), 0, st))
+    assert np.array_equal(back.cpu().numpy(), oracle.unfoldnd_backward(gcol, (6, 5, 7), (2, 3, 2), (2, 1, 1), (1, 0, 2), (1, 2, 1)))
+
+
 def test_config5a_conv2d_resnet_block():
     """image [64,256,56,56], weight [256,256,3,3], stride 1, pad 1 (GEMM M=200704, K=2304, N=256)."""
     rng = np.random.default_rng(1007)
