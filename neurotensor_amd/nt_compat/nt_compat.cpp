@@ -646,6 +646,90 @@ ConvGrads conv_transpose1d_backward(const Tensor& image, const Tensor& kernel, c
     return {r.d_image.view(image.shape()), r.d_kernel.view(kernel.shape())};
 }
 
+// image [.., C, D, H, W] / kernel [O, C/g, kd, kh, kw] -> batch, channels, sizes (contiguous inputs)
+struct Vol3 { int64_t B, C, size[3]; };
+static Vol3 vol3(const Tensor& t, bool is_kernel, const char* what) {
+    const SizeRef& s = t.shape();
+    utils::throw_exception(s.size() >= 4, std::string("Expected to get a 4D or greater tensor for ") + what + ", but got " + std::to_string(s.size()) + "D");
+    utils::throw_exception(!is_kernel || s.size() <= 5, std::string("Expected to get a 5D or 4D tensor as the kernel for ") + what);
+    Vol3 v;
+    for (int a = 0; a < 3; ++a) v.size[a] = s[s.size() - 3 + a];
+    v.C = s[s.size() - 4];
+    v.B = t.numel() / std::max<int64_t>(1, v.C * v.size[0] * v.size[1] * v.size[2]);
+    return v;
+}
+
+Tensor conv3d(const Tensor& image, const Tensor& kernel, utils::my_n_tuple<3> s, utils::my_n_tuple<3> p, utils::my_n_tuple<3> d, int64_t groups) {
+    utils::throw_exception(!image.is_null() && !kernel.is_null(), "Cannot perform operation conv3d on a null tensor");
+    utils::throw_exception(image.dtype() == kernel.dtype(), "Expected both kernel and image to have the same dtype for conv3d");
+    for (int a = 0; a < 3; ++a) {   // conv.cpp:129-131
+        utils::throw_exception(s[a] >= 1, "Conv3d stride cannot be less than 1");
+        utils::throw_exception(d[a] >= 1, "Conv3d dilation cannot be less than 1");
+        utils::throw_exception(p[a] >= 0, "Conv3d padding cannot be less than 1");
+    }
+    Tensor x = image.contiguous(), w = kernel.contiguous();
+    const Vol3 xv = vol3(x, false, "a 3d convolution"), wv = vol3(w, true, "a 3d convolution");
+    const int64_t O = wv.B;
+    utils::throw_exception(groups >= 1 && xv.C % groups == 0 && wv.C * groups == xv.C && O % groups == 0,
+                           "Expected kernel rows times groups to be equal to rows of image Conv3d");
+    int64_t out[3];
+    for (int a = 0; a < 3; ++a) {
+        out[a] = (xv.size[a] + 2 * p[a] - d[a] * (wv.size[a] - 1) - 1) / s[a] + 1;
+        utils::throw_exception(out[a] > 0, "conv3d output would be empty");
+    }
+    Tensor y({xv.B, O, out[0], out[1], out[2]}, x.dtype());
+    check_status(ntg_convnd(static_cast<int>(x.dtype()), x.data_ptr(), w.data_ptr(), y.data_ptr(), xv.B, xv.C, O, 3, xv.size, wv.size, s.data(),
+                            p.data(), d.data(), groups));
+    return y;
+}
+
+ConvGrads conv3d_backward(const Tensor& image, const Tensor& kernel, const Tensor& grad, utils::my_n_tuple<3> s, utils::my_n_tuple<3> p,
+                          utils::my_n_tuple<3> d, int64_t groups) {
+    utils::throw_exception(!image.is_null() && !kernel.is_null() && !grad.is_null(), "Cannot perform operation conv3d backward on a null tensor");
+    Tensor x = image.contiguous(), w = kernel.contiguous(), g = grad.contiguous();
+    const Vol3 xv = vol3(x, false, "conv3d backward"), wv = vol3(w, true, "conv3d backward");
+    int64_t L = 1;
+    for (int a = 0; a < 3; ++a) L *= (xv.size[a] + 2 * p[a] - d[a] * (wv.size[a] - 1) - 1) / s[a] + 1;
+    utils::throw_exception(g.numel() == xv.B * wv.B * L, "grad does not have the shape of the convolution output");
+    ConvGrads out{Tensor(image.shape(), x.dtype()), Tensor(kernel.shape(), x.dtype())};
+    check_status(ntg_convnd_backward(static_cast<int>(x.dtype()), x.data_ptr(), w.data_ptr(), g.data_ptr(), out.d_image.data_ptr(),
+                                     out.d_kernel.data_ptr(), xv.B, xv.C, wv.B, 3, xv.size, wv.size, s.data(), p.data(), d.data(), groups, 0));
+    return out;
+}
+
+Tensor conv_transpose3d(const Tensor& image, const Tensor& kernel, utils::my_n_tuple<3> s, utils::my_n_tuple<3> p, utils::my_n_tuple<3> op,
+                        utils::my_n_tuple<3> d, int64_t groups) {
+    utils::throw_exception(!image.is_null() && !kernel.is_null(), "Cannot perform operation conv_transpose3d on a null tensor");
+    utils::throw_exception(image.dtype() == kernel.dtype(), "Expected both kernel and image to have the same dtype for conv3d transpose");
+    for (int a = 0; a < 3; ++a) {   // conv.cpp:687-691
+        utils::throw_exception(s[a] >= 1, "Conv3d Transpose stride cannot be less than 1");
+        utils::throw_exception(d[a] >= 1, "Conv3d Transpose dilation cannot be less than 1");
+        utils::throw_exception(op[a] >= 0, "Conv3d Transpose output_padding cannot be less than 1");
+        utils::throw_exception(p[a] >= 0, "Conv3d Transpose padding cannot be less than 1");
+    }
+    utils::throw_exception(groups > 0, "Expected groups for a convolution to be greater than 0 but got " + std::to_string(groups));
+    Tensor x = image.contiguous(), w = kernel.contiguous();
+    const Vol3 xv = vol3(x, false, "a conv3d transpose"), wv = vol3(w, true, "a conv3d transpose");
+    utils::throw_exception(xv.C == wv.B, "Expected image channels to be the same as the kernel batches for conv_transpose3d but got " +
+                                             shape_str(x.shape()) + " and " + shape_str(w.shape()));
+    utils::throw_exception(xv.C % groups == 0, "Expected image channels to be divisible by groups in Conv3d Transpose");
+    int64_t out[3];
+    for (int a = 0; a < 3; ++a) out[a] = (xv.size[a] - 1) * s[a] - 2 * p[a] + d[a] * (wv.size[a] - 1) + 1 + op[a];
+    Tensor y({xv.B, wv.C * groups, out[0], out[1], out[2]}, x.dtype());
+    check_status(ntg_conv_transposend(static_cast<int>(x.dtype()), x.data_ptr(), w.data_ptr(), y.data_ptr(), xv.B, xv.C, wv.C * groups, 3, xv.size,
+                                      wv.size, s.data(), p.data(), d.data(), op.data(), groups));
+    return y;
+}
+
+ConvGrads conv_transpose3d_backward(const Tensor& image, const Tensor& kernel, const Tensor& grad, utils::my_n_tuple<3> s, utils::my_n_tuple<3> p,
+                                    utils::my_n_tuple<3> op, utils::my_n_tuple<3> d, int64_t groups) {
+    (void)op;
+    Tensor dx = functional::conv3d(grad.contiguous(), kernel, s, p, d, groups);
+    utils::throw_exception(dx.numel() == image.numel(), "grad does not have the shape of the transposed convolution's output");
+    ConvGrads kg = functional::conv3d_backward(grad.contiguous(), kernel, image.contiguous(), s, p, d, groups);
+    return {dx.view(image.shape()), kg.d_kernel};
+}
+
 }  // namespace functional
 
 namespace layers {

@@ -13,6 +13,7 @@
 // storage (contiguous tensors and transposed views).  All arithmetic is done by libntgemm.so
 // through the host-pointer C ABI (include/ntgemm.h); there is no CPU fallback.
 #pragma once
+#include <array>
 #include <cstdint>
 #include <initializer_list>
 #include <memory>
@@ -37,6 +38,7 @@ namespace utils {
 struct nt_error : std::runtime_error { using std::runtime_error::runtime_error; };
 void throw_exception(bool ok, const std::string& message);
 using my_tuple = std::pair<int64_t, int64_t>;
+template <size_t N> using my_n_tuple = std::array<int64_t, N>;
 }  // namespace utils
 
 using SizeRef = std::vector<int64_t>;
@@ -116,6 +118,17 @@ Tensor conv_transpose1d(const Tensor& image, const Tensor& kernel, int64_t strid
 ConvGrads conv_transpose1d_backward(const Tensor& image, const Tensor& kernel, const Tensor& grad, int64_t stride = 1, int64_t padding = 0,
                                     int64_t output_padding = 0, int64_t dilation = 1, int64_t groups = 1);
 
+// conv3d (conv.cpp:122-175), conv_transpose3d (:678-745) and their gradients
+Tensor conv3d(const Tensor& image, const Tensor& kernel, utils::my_n_tuple<3> stride = {1, 1, 1}, utils::my_n_tuple<3> padding = {0, 0, 0},
+              utils::my_n_tuple<3> dilation = {1, 1, 1}, int64_t groups = 1);
+ConvGrads conv3d_backward(const Tensor& image, const Tensor& kernel, const Tensor& grad, utils::my_n_tuple<3> stride = {1, 1, 1},
+                          utils::my_n_tuple<3> padding = {0, 0, 0}, utils::my_n_tuple<3> dilation = {1, 1, 1}, int64_t groups = 1);
+Tensor conv_transpose3d(const Tensor& image, const Tensor& kernel, utils::my_n_tuple<3> stride = {1, 1, 1}, utils::my_n_tuple<3> padding = {0, 0, 0},
+                        utils::my_n_tuple<3> output_padding = {0, 0, 0}, utils::my_n_tuple<3> dilation = {1, 1, 1}, int64_t groups = 1);
+ConvGrads conv_transpose3d_backward(const Tensor& image, const Tensor& kernel, const Tensor& grad, utils::my_n_tuple<3> stride = {1, 1, 1},
+                                    utils::my_n_tuple<3> padding = {0, 0, 0}, utils::my_n_tuple<3> output_padding = {0, 0, 0},
+                                    utils::my_n_tuple<3> dilation = {1, 1, 1}, int64_t groups = 1);
+
 // what the backward lambdas of TensorGrad matmult / linear compute (flags only, no transposed copies)
 struct MatmultGrads { Tensor da, db; };
 MatmultGrads matmult_backward(const Tensor& a, const Tensor& b, const Tensor& grad, bool trans_a, bool trans_b);
@@ -148,6 +161,16 @@ inline Tensor conv_transpose1d(const Tensor& image, const Tensor& kernel, int64_
 inline Tensor conv_transpose2d(const Tensor& image, const Tensor& kernel, utils::my_tuple stride = {1, 1}, utils::my_tuple padding = {0, 0},
                                utils::my_tuple output_padding = {0, 0}, utils::my_tuple dilation = {1, 1}, int64_t groups = 1) {
     return functional::conv_transpose2d(image, kernel, stride, padding, output_padding, dilation, groups);
+}
+
+inline Tensor conv3d(const Tensor& image, const Tensor& kernel, utils::my_n_tuple<3> stride = {1, 1, 1}, utils::my_n_tuple<3> padding = {0, 0, 0},
+                     utils::my_n_tuple<3> dilation = {1, 1, 1}, int64_t groups = 1) {
+    return functional::conv3d(image, kernel, stride, padding, dilation, groups);
+}
+inline Tensor conv_transpose3d(const Tensor& image, const Tensor& kernel, utils::my_n_tuple<3> stride = {1, 1, 1},
+                               utils::my_n_tuple<3> padding = {0, 0, 0}, utils::my_n_tuple<3> output_padding = {0, 0, 0},
+                               utils::my_n_tuple<3> dilation = {1, 1, 1}, int64_t groups = 1) {
+    return functional::conv_transpose3d(image, kernel, stride, padding, output_padding, dilation, groups);
 }
 
 namespace layers {

@@ -109,6 +109,8 @@ static void host_only_cases() {
     expect_throw("conv2d kernel dims", [] { nt::conv2d(F::zeros({1, 3, 8, 8}), F::zeros({3, 3})); });
     expect_throw("conv2d groups", [] { nt::conv2d(F::zeros({1, 3, 8, 8}), F::zeros({4, 3, 3, 3}), {1, 1}, {0, 0}, {1, 1}, 2); });
     expect_throw("conv2d stride", [] { nt::conv2d(F::zeros({1, 3, 8, 8}), F::zeros({4, 3, 3, 3}), {0, 1}); });
+    expect_throw("conv3d stride", [] { nt::conv3d(F::zeros({1, 3, 4, 8, 8}), F::zeros({4, 3, 3, 3, 3}), {1, 0, 1}); });
+    expect_throw("conv3d groups", [] { nt::conv3d(F::zeros({1, 3, 4, 8, 8}), F::zeros({4, 3, 3, 3, 3}), {1, 1, 1}, {0, 0, 0}, {1, 1, 1}, 2); });
     expect_throw("conv1d image dims", [] { nt::conv1d(F::zeros({8}), F::zeros({4, 3, 3})); });
     expect_throw("conv1d stride", [] { nt::conv1d(F::zeros({1, 3, 8}), F::zeros({4, 3, 3}), 0); });
     expect_throw("conv_transpose2d channels", [] { nt::conv_transpose2d(F::zeros({1, 3, 8, 8}), F::zeros({4, 3, 3, 3})); });
@@ -282,6 +284,31 @@ static void device_cases(const std::string& g) {
                                                            {c.output_padding, c.output_padding}, {1, 1}, c.groups);
             close(gr.d_image, fixture("conv_transpose2d", "xgrad", c.sfx), "conv_transpose2d xgrad");
             close(gr.d_kernel, fixture("conv_transpose2d", "wgrad", c.sfx), "conv_transpose2d wgrad");
+        });
+    }
+    // tests/src/conv_autograd_test.cpp:375-497 (conv3d), :847-971 (conv_transpose3d)
+    for (const char* sfx : {"", "_batched", "_grouped", "_grouped_batched"}) {
+        run_test((std::string("conv3d golden") + sfx).c_str(), [&] {
+            const bool grouped = std::strstr(sfx, "grouped") != nullptr;
+            const int64_t pad = grouped ? 0 : 1, groups = grouped ? 2 : 1;
+            Tensor x = fixture("conv3d", "input", sfx), w = fixture("conv3d", "weight", sfx);
+            Tensor o = nt::conv3d(x, w, {1, 1, 1}, {pad, pad, pad}, {1, 1, 1}, groups);
+            close(o, fixture("conv3d", "output", sfx), "conv3d output");
+            F::ConvGrads gr = F::conv3d_backward(x, w, fixture("conv3d", "grad", sfx), {1, 1, 1}, {pad, pad, pad}, {1, 1, 1}, groups);
+            close(gr.d_image, fixture("conv3d", "xgrad", sfx), "conv3d xgrad");
+            close(gr.d_kernel, fixture("conv3d", "wgrad", sfx), "conv3d wgrad");
+        });
+    }
+    for (const TCase& c : {TCase{"", 2, 0, 1, 1}, TCase{"_grouped_batched", 1, 1, 0, 2}}) {
+        run_test((std::string("conv_transpose3d golden") + c.sfx).c_str(), [&] {
+            Tensor x = fixture("conv_transpose3d", "input", c.sfx), w = fixture("conv_transpose3d", "weight", c.sfx);
+            const nt::utils::my_n_tuple<3> s{c.stride, c.stride, c.stride}, p{c.padding, c.padding, c.padding},
+                op{c.output_padding, c.output_padding, c.output_padding}, d{1, 1, 1};
+            Tensor o = nt::conv_transpose3d(x, w, s, p, op, d, c.groups);
+            close(o, fixture("conv_transpose3d", "output", c.sfx), "conv_transpose3d output");
+            F::ConvGrads gr = F::conv_transpose3d_backward(x, w, fixture("conv_transpose3d", "grad", c.sfx), s, p, op, d, c.groups);
+            close(gr.d_image, fixture("conv_transpose3d", "xgrad", c.sfx), "conv_transpose3d xgrad");
+            close(gr.d_kernel, fixture("conv_transpose3d", "wgrad", c.sfx), "conv_transpose3d wgrad");
         });
     }
     run_test("unfold2d golden", [&] {
