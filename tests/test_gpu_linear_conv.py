@@ -519,6 +519,39 @@ def test_conv3d_and_transpose_random_vs_torch(dtype):
     assert np.array_equal(back.cpu().numpy(), oracle.unfoldnd_backward(gcol, (6, 5, 7), (2, 3, 2), (2, 1, 1), (1, 0, 2), (1, 2, 1)))
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float16], ids=["fp32", "fp16"])
+def test_conv2d_wide_kernels_and_empty_inputs(dtype):
+    """Kernels wider than 8 taps on an axis leave the implicit-GEMM path (one byte of tap mask per pixel) for the stored
+    im2col matrix; zero-sized batches and channels return without touching memory; bad geometry is an error."""
+    rng = np.random.default_rng(1700)
+    lib = _lib.load()
+    for (B, C, H, W, O, kh, kw_, s, p, d, groups) in [(2, 4, 20, 15, 6, 9, 3, 1, (4, 1), 1, 2), (3, 2, 8, 30, 4, 2, 11, (1, 2), (0, 5), 1, 1)]:
+        x = randn(rng, (B, C, H, W), dtype)
+        w = randn(rng, (O, C // groups, kh, kw_), dtype, 1.0 / np.sqrt(C // groups * kh * kw_))
+        tx, tw = dev(x), dev(w)
+        assert lib.ntg_conv2d_forward_workspace_bytes(F.ntg_dtype(tx), B, C, H, W, kh, kw_, *F._pair(s), *F._pair(p), *F._pair(d)) > 0
+        rx, rw = tx.double().cpu().requires_grad_(True), tw.double().cpu().requires_grad_(True)
+        ry = torch.nn.functional.conv2d(rx, rw, None, s, p, d, groups)
+        y = F.conv2d(tx, tw, stride=s, padding=p, dilation=d, groups=groups)
+        tol = 1e-4 if dtype == np.float32 else HALF_REL * ry.abs().max().item()
+        assert (y.double().cpu() - ry.detach()).abs().max().item() <= tol
+        g = dev(randn(rng, tuple(ry.shape), dtype))
+        ry.backward(g.double().cpu())
+        dx, dw = F.conv2d_backward(tx, tw, g, stride=s, padding=p, dilation=d, groups=groups)
+        assert (dx.double().cpu() - rx.grad).abs().max().item() <= (1e-4 if dtype == np.float32 else HALF_REL * rx.grad.abs().max().item())
+        assert (dw.double().cpu() - rw.grad).abs().max().item() <= (1e-3 if dtype == np.float32 else HALF_REL * rw.grad.abs().max().item())
+    # empty batch / no filters: nothing to do, no error
+    st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    dt = F.ntg_dtype(tx)
+    _lib.check(lib.ntg_conv2d_dev(dt, None, None, None, None, 0, 0, 3, 8, 8, 4, 3, 3, 1, 1, 1, 1, 1, 1, 1, st))
+    _lib.check(lib.ntg_conv2d_dev(dt, tx.data_ptr(), tw.data_ptr(), None, None, 0, 2, 3, 8, 8, 0, 3, 3, 1, 1, 1, 1, 1, 1, 1, st))
+    _lib.check(lib.ntg_conv2d_backward_dev(dt, None, None, None, None, None, None, 0, 0, 3, 8, 8, 4, 3, 3, 1, 1, 1, 1, 1, 1, 1, 0, st))
+    # kernel larger than the padded image, channels not divisible by groups
+    assert lib.ntg_conv2d_dev(dt, tx.data_ptr(), tw.data_ptr(), tx.data_ptr(), None, 0, 1, 3, 4, 4, 4, 7, 7, 1, 1, 1, 1, 1, 1, 1, st) == 1
+    assert lib.ntg_conv2d_dev(dt, tx.data_ptr(), tw.data_ptr(), tx.data_ptr(), None, 0, 1, 3, 8, 8, 4, 3, 3, 1, 1, 1, 1, 1, 1, 2, st) == 1
+    assert b"groups" in lib.ntg_last_error()
+
+
 def test_config5a_conv2d_resnet_block():
     """image [64,256,56,56], weight [256,256,3,3], stride 1, pad 1 (GEMM M=200704, K=2304, N=256)."""
     rng = np.random.default_rng(1007)
