@@ -20,7 +20,7 @@
  *
  * Pinning (see tests/test_oracle_*.py):
  *   fp32 linear grads / conv2d output+grads / unfold  <- the reference's own
- *       committed PyTorch fixtures (tests/golden/*.npy).
+ *       committed PyTorch fixtures (the .npy files under tests/golden).
  *   fp32/fp64 GEMM  <- numpy float64 GEMM, identity/permutation operands,
  *       explicit-transpose equivalence (bitwise), batch == per item (bitwise),
  *       tiled == closed form (bitwise), naive triple loop on tiny inputs.

@@ -66,6 +66,29 @@ def test_argument_errors_do_not_need_a_device():
     rc = lib.ntg_unfold2d(_lib.FLOAT32, p, p, 1, 1, 2, 2, 5, 5, 1, 1, 0, 0, 1, 1)
     assert rc == 1
     assert lib.ntg_conv2d_workspace_bytes(_lib.FLOAT32, 1, 3, 8, 8, 3, 3, 1, 1, 1, 1, 1, 1) == 27 * 64 * 4
+    # implicit-GEMM convolutions need no workspace; integers and kernels wider than 8 taps unfold
+    assert lib.ntg_conv2d_forward_workspace_bytes(_lib.FLOAT32, 1, 3, 8, 8, 3, 3, 1, 1, 1, 1, 1, 1) == 0
+    assert lib.ntg_conv2d_forward_workspace_bytes(_lib.INT32, 1, 3, 8, 8, 3, 3, 1, 1, 1, 1, 1, 1) == 27 * 64 * 4
+    assert lib.ntg_conv2d_forward_workspace_bytes(_lib.FLOAT32, 1, 3, 16, 16, 9, 3, 1, 1, 4, 1, 1, 1) == 27 * 3 * 256 * 4
+    # per-image weight gradients [B, O, C/g * taps] instead of the im2col matrix
+    assert lib.ntg_conv2d_backward_workspace_bytes(_lib.FLOAT32, 2, 4, 8, 8, 6, 3, 3, 1, 1, 1, 1, 1, 1, 2) == 2 * 6 * 2 * 9 * 4
+    assert lib.ntg_conv2d_backward_workspace_bytes(_lib.FLOAT32, 2, 4, 8, 8, 6, 3, 3, 1, 1, 1, 1, 1, 1, 3) == -1
+    # transposed convolution: output_padding must stay below the stride; sizes follow (in-1)*s - 2p + d(k-1) + 1 + op
+    assert lib.ntg_conv_transpose2d_workspace_bytes(_lib.FLOAT32, 1, 3, 9, 7, 8, 3, 3, 2, 2, 0, 0, 1, 1, 2, 1, 1) == -1
+    assert lib.ntg_conv_transpose2d_workspace_bytes(_lib.FLOAT32, 1, 3, 9, 7, 8, 3, 3, 2, 2, 0, 0, 1, 1, 1, 1, 1) > 0
+    assert lib.ntg_conv_transpose2d(_lib.FLOAT32, p, p, p, 1, 3, 9, 7, 8, 3, 3, 2, 2, 0, 0, 1, 1, 2, 1, 1) == 1
+    assert b"output_padding" in lib.ntg_last_error()
+    assert lib.ntg_conv_transpose2d(_lib.FLOAT32, p, p, p, 1, 3, 9, 7, 8, 3, 3, 2, 2, 0, 0, 1, 1, 1, 1, 2) == 1    # 3 % 2 groups
+    # N-d geometry arrays
+    arr = lambda *v: (ctypes.c_int64 * len(v))(*v)
+    assert lib.ntg_convnd_workspace_bytes(_lib.FLOAT32, 2, 3, 4, 3, arr(5, 6, 7), arr(2, 3, 2), arr(1, 2, 1), arr(1, 0, 2), arr(2, 1, 1), 1, 0) \
+        == 2 * 3 * 12 * (5 * 2 * 10) * 4
+    assert lib.ntg_convnd_workspace_bytes(_lib.FLOAT32, 2, 3, 4, 5, arr(5, 6, 7), arr(2, 3, 2), arr(1, 2, 1), arr(1, 0, 2), arr(2, 1, 1), 1, 0) == -1
+    assert lib.ntg_convnd(_lib.FLOAT32, p, p, p, 1, 3, 4, 3, arr(5, 6, 7), arr(2, 3, 9), arr(1, 1, 1), arr(0, 0, 0), arr(1, 1, 1), 1) == 1
+    assert b"sliding blocks" in lib.ntg_last_error()
+    assert lib.ntg_convnd(_lib.FLOAT32, p, p, p, 0, 3, 4, 3, arr(5, 6, 7), arr(2, 3, 2), arr(1, 1, 1), arr(0, 0, 0), arr(1, 1, 1), 1) == 0
+    assert lib.ntg_conv_transposend(_lib.FLOAT32, p, p, p, 1, 3, 4, 3, arr(5, 6, 7), arr(2, 3, 2), arr(1, 1, 1), arr(0, 0, 0), arr(1, 1, 1),
+                                    arr(0, 1, 0), 1) == 1
     d = _lib.GemmDesc()
     d.dtype, d.m, d.k, d.n, d.batches, d.c_mode = _lib.FLOAT32, 4, 4, 4, 1, 7
     assert lib.ntg_gemm_dev(ctypes.byref(d), p, p, p, None) == 1
