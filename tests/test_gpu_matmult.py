@@ -344,6 +344,45 @@ def test_ragged_16bit_dma_kernel(dtype, shape):
     assert ((y.float() - refy).abs().max() / refy.abs().max()).item() <= HALF_REL
 
 
+@pytest.mark.parametrize("dtype", ["bf16", np.float32, np.int32], ids=["bf16", "fp32", "int32"])
+def test_operands_beyond_2_31_elements(dtype):
+    """A holds more than 2^31 elements (4.4 - 9.6 GB): every row offset in the loaders and the stores is 64-bit.
+    The rows past the 2^31-element mark are checked against torch on that slice."""
+    bf = dtype == "bf16"
+    if bf:
+        m, k, n, td = 66000, 33000, 256, torch.bfloat16
+    elif dtype == np.float32:
+        m, k, n, td = 40000, 60000, 128, torch.float32
+    else:
+        m, k, n, td = 50000, 45000, 8, torch.int32
+    assert m * k > 2 ** 31
+    torch.manual_seed(5)
+    if dtype == np.int32:
+        a = torch.randint(-8, 9, (m, k), device=DEV, dtype=td)
+        b = torch.randint(-8, 9, (k, n), device=DEV, dtype=td)
+    else:
+        a = torch.empty((m, k), device=DEV, dtype=td).normal_(0, 0.05 if bf else 1.0)
+        b = torch.empty((k, n), device=DEV, dtype=td).normal_(0, 0.05 if bf else 1.0)
+    c = F.matmult(a, b)
+    for lo in (0, m - 300):
+        rows = slice(lo, lo + 300)
+        if dtype == np.int32:
+            ref = (a[rows].double() @ b.double())                       # |sum| < 2^53: exact
+            assert torch.equal(c[rows].double(), ref)
+        else:
+            ref = a[rows].double() @ b.double()
+            err = (c[rows].double() - ref).abs().max().item()
+            tol = HALF_REL * ref.abs().max().item() if bf else 1e-5 * k * float(a[rows].abs().max().item() * b.abs().max().item())
+            assert err <= tol, (lo, err, tol)
+    # transpose_a: A stored [k, m] with the same footprint
+    if not bf:
+        return
+    at = torch.empty((k, m), device=DEV, dtype=td).normal_(0, 0.05)
+    ct = F.matmult(at, b, None, True, False)
+    ref = at[:, m - 256:].double().t() @ b.double()
+    assert (ct[m - 256:].double() - ref).abs().max().item() <= HALF_REL * ref.abs().max().item()
+
+
 def test_skinny_fp32_config5b():
     rng = np.random.default_rng(1005)
     a = rng.standard_normal((16, 8192)).astype(np.float32)
