@@ -383,6 +383,45 @@ def test_operands_beyond_2_31_elements(dtype):
     assert (ct[m - 256:].double() - ref).abs().max().item() <= HALF_REL * ref.abs().max().item()
 
 
+@pytest.mark.parametrize("dtype", ["bf16", np.float16], ids=["bf16", "fp16"])
+@pytest.mark.parametrize("m", [1, 7, 16, 17, 32])
+def test_skinny_16bit(dtype, m):
+    """m <= 32 in Float16 / BFloat16 streams B once through the HBM-bound kernel: every transpose pair, strip widths of
+    2, 4 and 8 columns per lane, the guarded (ragged / unaligned) instantiation, all three C modes, batches."""
+    bf = dtype == "bf16"
+    rng = np.random.default_rng(1800 + m)
+    for (k, n, batch) in [(4096, 8192, 1), (1024, 2048, 1), (512, 256, 3), (1000, 520, 2), (136, 24, 1), (2048, 1030, 1)]:
+        for ta, tb in TRANS:
+            a = randn(rng, (batch, m, k), dtype, 0.25)
+            b = randn(rng, (batch, k, n), dtype, 0.25)
+            sa = np.ascontiguousarray(a.transpose(0, 2, 1)) if ta else a
+            sb = np.ascontiguousarray(b.transpose(0, 2, 1)) if tb else b
+            ta_, tb_ = to_torch(sa, DEV, bf), to_torch(sb, DEV, bf)
+            ref = torch.matmul(to_torch(a, DEV, bf).double(), to_torch(b, DEV, bf).double())
+            scale = ref.abs().max().item()
+            out = F.matmult(ta_, tb_, None, ta, tb)
+            assert tuple(out.shape) == (batch, m, n)
+            assert ((out.double() - ref).abs().max() / scale).item() <= HALF_REL, (m, k, n, batch, ta, tb)
+            c0 = to_torch(randn(rng, (batch, m, n), dtype), DEV, bf)
+            c = c0.clone()
+            F.matmult(ta_, tb_, c, ta, tb)                                        # C += A.B
+            assert ((c.double() - (ref + c0.double())).abs().max() / scale).item() <= HALF_REL
+    # deterministic: two launches give identical bits; the oracle agrees on a small case
+    a = randn(rng, (m, 512), dtype)
+    b = randn(rng, (512, 64), dtype)
+    ta_, tb_ = to_torch(a, DEV, bf), to_torch(b, DEV, bf)
+    o1, o2 = F.matmult(ta_, tb_), F.matmult(ta_, tb_)
+    assert torch.equal(o1, o2)
+    want = to_f64(oracle.matmult2d(a, b, dt=code_of(dtype)), bf)
+    got = o1.double().cpu().numpy()
+    assert np.abs(got - want).max() <= HALF_REL * np.abs(want).max()
+    # bias mode (linear with a small batch)
+    bias = randn(rng, (64,), dtype)
+    y = F.linear(ta_, tb_, to_torch(bias, DEV, bf))
+    refy = ta_.double() @ tb_.double() + to_torch(bias, DEV, bf).double()
+    assert ((y.double() - refy).abs().max() / refy.abs().max()).item() <= HALF_REL
+
+
 def test_skinny_fp32_config5b():
     rng = np.random.default_rng(1005)
     a = rng.standard_normal((16, 8192)).astype(np.float32)
