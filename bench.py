@@ -92,11 +92,15 @@ def main():
         d.transpose_a, d.transpose_b, d.c_mode = int(ta), int(tb), mode
         d.m, d.k, d.n, d.batches = m, k, n, batch
         d.stride_a, d.stride_b, d.stride_c = m * k, k * n, m * n
+        ws_bytes = lib.ntg_gemm_workspace_bytes(ctypes.byref(d))     # > 0 only for few-tile, deep-k shapes (split along k)
+        ws = torch.empty((ws_bytes,), dtype=torch.uint8, device=dev) if ws_bytes > 0 else None
+        if ws is not None:
+            d.workspace, d.workspace_bytes = ws.data_ptr(), ws_bytes
 
         def launch():
             _lib.check(lib.ntg_gemm_dev(ctypes.byref(d), a.data_ptr(), b.data_ptr(), c.data_ptr(), stream))
 
-        launch.keep = (a, b, c, d)
+        launch.keep = (a, b, c, d, ws)
         return launch
 
     def time_steps(fn, steps, warmup):
@@ -183,6 +187,12 @@ def main():
             run(f"c4_linear_fwd_{nm}", make_gemm(dt, 8192, 4096, 11008, tb=True, mode=_lib.C_OVERWRITE, scale=0.1), f4, pk)
             run(f"c4_linear_dx_{nm}", make_gemm(dt, 8192, 11008, 4096, mode=_lib.C_OVERWRITE, scale=0.1), f4, pk)
             run(f"c4_linear_dw_{nm}", make_gemm(dt, 11008, 8192, 4096, ta=True, mode=_lib.C_OVERWRITE, scale=0.1), f4, pk)
+        # the same Linear layer on 16 and 256 rows (inference-sized batches): HBM-bound streaming kernel, split along k
+        wbytes = 2.0 * 4096 * 11008
+        run("linear_bf16_16_rows_4096x11008", make_gemm(torch.bfloat16, 16, 4096, 11008, mode=_lib.C_OVERWRITE, scale=0.1),
+            wbytes + 2.0 * 16 * (4096 + 11008), PEAK_HBM_GBS, "GB/s", 1e9, st=steps * 4)
+        run("linear_bf16_256_rows_4096x11008", make_gemm(torch.bfloat16, 256, 4096, 11008, mode=_lib.C_OVERWRITE, scale=0.1),
+            2.0 * 256 * 4096 * 11008, PEAK_TFLOPS["bf16"], st=steps * 2)
         x = torch.randn(64, 256, 56, 56, device=dev)
         w = torch.randn(256, 256, 3, 3, device=dev) / 48.0
         run("c5a_conv2d_fp32", lambda: F.conv2d(x, w, padding=1), 2.0 * 200704 * 2304 * 256, PEAK_TFLOPS["fp32"])

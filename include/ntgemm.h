@@ -155,7 +155,14 @@ typedef struct ntg_gemm_desc {
     int64_t stride_a, stride_b, stride_c;   /* elements between items; 0 on A/B = broadcast */
     const void* bias;           /* device pointer, NTG_C_BIAS only */
     int64_t bias_batch_stride, bias_row_stride, bias_col_stride;   /* elements; 0 = broadcast */
+    void* workspace;            /* optional device scratch, 16-byte aligned, ntg_gemm_workspace_bytes(desc) bytes: lets a   */
+    int64_t workspace_bytes;    /* single product with few output tiles and a deep k be split along k (deterministic)      */
 } ntg_gemm_desc;
+
+/* Bytes of workspace with which ntg_gemm_dev can split the product along k (0: it would not split).  Without a
+ * workspace the same result is computed by one pass over k; only the speed of shapes such as [256, 8192] x [8192, 8192]
+ * differs.  The reference has no counterpart: its k loop is always serial (nt_matmult.hpp:196). */
+int64_t ntg_gemm_workspace_bytes(const ntg_gemm_desc* desc);
 
 /* nt_matmult<T> on device buffers: C += op(A).op(B), dense leading dimensions. */
 int ntg_matmult_dev(int dtype, const void* dA, const void* dB, void* dC,

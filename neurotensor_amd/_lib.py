@@ -29,6 +29,7 @@ class GemmDesc(ctypes.Structure):
         ("stride_a", ctypes.c_int64), ("stride_b", ctypes.c_int64), ("stride_c", ctypes.c_int64),
         ("bias", ctypes.c_void_p),
         ("bias_batch_stride", ctypes.c_int64), ("bias_row_stride", ctypes.c_int64), ("bias_col_stride", ctypes.c_int64),
+        ("workspace", ctypes.c_void_p), ("workspace_bytes", ctypes.c_int64),
     ]
 
 
@@ -56,6 +57,7 @@ SIGNATURES = {
     "ntg_conv2d": (_ci, [_ci, _vp, _vp, _vp] + [_i64] * 14),
     "ntg_matmult_dev": (_ci, [_ci, _vp, _vp, _vp, _i64, _i64, _i64, _ci, _ci, _vp]),
     "ntg_gemm_dev": (_ci, [ctypes.POINTER(GemmDesc), _vp, _vp, _vp, _vp]),
+    "ntg_gemm_workspace_bytes": (_i64, [ctypes.POINTER(GemmDesc)]),
     "ntg_gemm_ptrs_dev": (_ci, [ctypes.POINTER(GemmDesc), _vp, _vp, _vp, _vp]),
     "ntg_unfold2d_dev": (_ci, [_ci, _vp, _vp] + [_i64] * 12 + [_vp]),
     "ntg_conv2d_workspace_bytes": (_i64, [_ci] + [_i64] * 12),

@@ -347,6 +347,13 @@ __global__ void __launch_bounds__(256) gemm16_kernel(const GemmParams p) {
                 float v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
                 const int m = m0 + wm * 128 + 32 * i + row;
                 if (RAGGED && (m >= p.M || n >= p.N)) continue;     // N % 8 == 0: a lane's 8 columns exist or not together
+                if constexpr (CM == C_PARTIAL) {
+                    // split-K: the fp32 sums of this k range go to a float matrix; rounding happens after the reduction
+                    float* wp = static_cast<float*>(p.C) + (int64_t)b * p.sC + (int64_t)m * p.ldc + n;
+                    *reinterpret_cast<floatx4v*>(wp) = lo;
+                    *reinterpret_cast<floatx4v*>(wp + 4) = hi;
+                    continue;
+                }
                 if constexpr (CM == C_ACCUMULATE) {
 #pragma unroll
                     for (int e = 0; e < 8; ++e) v[e] += Cvt16<DT>::up((uint16_t)(c0[t][e >> 1] >> (16 * (e & 1))));
@@ -364,6 +371,7 @@ __global__ void __launch_bounds__(256) gemm16_kernel(const GemmParams p) {
         }
     };
     if (p.cmode == C_ACCUMULATE) epilogue(std::integral_constant<int, C_ACCUMULATE>{});
+    else if (p.cmode == C_PARTIAL) epilogue(std::integral_constant<int, C_PARTIAL>{});
     else if (p.cmode == C_BIAS) epilogue(std::integral_constant<int, C_BIAS>{});
     else epilogue(std::integral_constant<int, C_OVERWRITE>{});
 }

@@ -3,7 +3,7 @@
 namespace ntg {
 hipError_t launch_gemm_mfma_f64(bool ta, bool tb, const GemmParams& p, hipStream_t s) {
     const int64_t big_tiles = (int64_t)((p.M + 127) / 128) * ((p.N + 127) / 128) * p.batch;
-    if (big_tiles >= 192) return launch_trans<DT_F64, 4, 4, 16>(ta, tb, p, s);   // 128 x 128 x 16 tile
+    if (big_tiles >= 192 && p.M > 64 && p.N > 64) return launch_trans<DT_F64, 4, 4, 16>(ta, tb, p, s);   // a 128-wide tile would be half empty   // 128 x 128 x 16 tile
     return launch_trans<DT_F64, 2, 2, 16>(ta, tb, p, s);                          // 64 x 64 x 16 tile
 }
 // conv2d / conv_dkernel with op(B) gathered from the image (tb: col^T)

@@ -17,7 +17,8 @@ enum DType : int {
 enum CMode : int {
     C_OVERWRITE = 0,   // C  = op(A).op(B)          (caller knows C would be zeros)
     C_ACCUMULATE = 1,  // C += op(A).op(B)          (contract of nt_matmult, nt_matmult.hpp:370-378)
-    C_BIAS = 2         // C  = bias (+) op(A).op(B) (cpu::linear, matmult_cpu.cpp:1637-1647)
+    C_BIAS = 2,        // C  = bias (+) op(A).op(B) (cpu::linear, matmult_cpu.cpp:1637-1647)
+    C_PARTIAL = 3      // internal (split-K): write the fp32 accumulators to a float matrix at C; 16-bit DMA kernel only
 };
 
 // Unsigned division by a divisor fixed at launch (round-up multiplier form): exact for every
@@ -102,6 +103,9 @@ struct UnfoldNdParams {
 };
 hipError_t launch_unfoldnd(int64_t elem_size, const void* im, void* col, const UnfoldNdParams& u, hipStream_t s);
 hipError_t launch_col2imnd(int dtype, const void* col, void* im, const UnfoldNdParams& u, int accumulate, hipStream_t s);
+
+// split-K: out (+)= sum over s of part[s] (s ascending), fp32 accumulation for the 16-bit dtypes whose partials are float
+hipError_t launch_splitk_reduce(int dtype, const void* part, int splits, const GemmParams& p, hipStream_t s);
 
 // conv2d backward helpers (unfold2d.hip): ordered sum of per-image weight gradients; weights of
 // the gradient-to-image convolution

@@ -79,10 +79,8 @@ bool is_int_dtype(int dt) {
 }
 
 // Fills the derived fields and launches the kernel family for the dtype.
-int run_gemm(ntg::GemmParams p, int dtype, bool ta, bool tb, hipStream_t s) {
+int launch_gemm(ntg::GemmParams p, int dtype, bool ta, bool tb, hipStream_t s) {
     const int64_t es = ntg::elem_size(dtype);
-    if (es == 0) return fail(NTG_ERR_UNSUPPORTED_DTYPE, "dtype %d is not supported by the gfx950 matmult backend", dtype);
-    if (p.M == 0 || p.N == 0 || p.batch == 0) return NTG_OK;
     const int64_t ve = 16 / es;
     p.vecA_ok = (p.lda % ve == 0) && (p.Aptr || p.sA % ve == 0);
     p.vecB_ok = (p.ldb % ve == 0) && (p.Bptr || p.sB % ve == 0);
@@ -104,6 +102,64 @@ int run_gemm(ntg::GemmParams p, int dtype, bool ta, bool tb, hipStream_t s) {
     }
     if (e != hipSuccess) return hip_fail(e, "gemm launch");
     return NTG_OK;
+}
+
+// Split-K.  A single product whose output tiles cannot occupy the 256 CUs but whose K is deep (a Linear layer on a few
+// hundred rows) is cut into `splits` equal k ranges, computed as one batched launch of the ordinary kernels into a
+// workspace [splits][M][N] (fp32 sums for the 16-bit dtypes, so nothing is rounded early), and added up in ascending
+// range order by a second kernel.  Deterministic; applied only when the caller supplies the workspace.
+struct SplitPlan { int splits; int64_t kc; int64_t bytes; };
+
+SplitPlan plan_splitk(const ntg::GemmParams& p, int dtype, bool ta) {
+    SplitPlan none{1, p.K, 0};
+    const int64_t es = ntg::elem_size(dtype);
+    if (is_int_dtype(dtype) || es == 0 || p.batch != 1 || p.Aptr || p.Bptr || p.Cptr) return none;
+    if (p.M <= 32 && dtype != ntg::DT_F64) return none;                       // the streaming kernels take these
+    const bool half = dtype == ntg::DT_F16 || dtype == ntg::DT_BF16;
+    if (half) {
+        // only the DMA-fed kernel writes fp32 partial sums: 16-byte rows everywhere
+        if (p.K % 8 || p.N % 8 || (ta && p.M % 8) || p.lda % 8 || p.ldb % 8 || p.lda >= (1 << 22) || p.ldb >= (1 << 22)) return none;
+        if ((reinterpret_cast<uintptr_t>(p.A) & 15) || (reinterpret_cast<uintptr_t>(p.B) & 15)) return none;
+    }
+    // workgroups the kernels want in flight: one 256 x 256 tile per CU for the 16-bit kernel (its LDS ring fills the CU),
+    // two 128 x 128 (or more 64 x 64) tiles per CU for fp32 / fp64
+    const int64_t tile = half ? 256 : ((p.M <= 64 || p.N <= 64) ? 64 : 128), kstep = dtype == ntg::DT_F64 ? 16 : 32;
+    const int64_t target = half ? 256 : 512;
+    const int64_t tiles = ((p.M + tile - 1) / tile) * ((p.N + tile - 1) / tile);
+    if (2 * tiles > target) return none;
+    int64_t smax = target / tiles;
+    if (smax > 16) smax = 16;
+    for (int64_t sp = smax; sp >= 2; --sp) {
+        if (p.K % (sp * kstep) != 0 || p.K / sp < 512) continue;   // short k ranges do not pay for the second pass
+        if (half && tiles * sp < 48) return none;                             // too small for the DMA-fed kernel anyway
+        return SplitPlan{(int)sp, p.K / sp, sp * (int64_t)p.M * p.N * (half ? 4 : es)};
+    }
+    return none;
+}
+
+int run_gemm(ntg::GemmParams p, int dtype, bool ta, bool tb, hipStream_t s, void* workspace = nullptr, int64_t workspace_bytes = 0) {
+    const int64_t es = ntg::elem_size(dtype);
+    if (es == 0) return fail(NTG_ERR_UNSUPPORTED_DTYPE, "dtype %d is not supported by the gfx950 matmult backend", dtype);
+    if (p.M == 0 || p.N == 0 || p.batch == 0) return NTG_OK;
+    const SplitPlan plan = plan_splitk(p, dtype, ta);
+    if (plan.splits > 1 && workspace && workspace_bytes >= plan.bytes && (reinterpret_cast<uintptr_t>(workspace) & 15) == 0) {
+        ntg::GemmParams q = p;
+        q.K = (int)plan.kc;
+        q.batch = plan.splits;
+        q.sA = ta ? plan.kc * p.lda : plan.kc;
+        q.sB = tb ? plan.kc : plan.kc * p.ldb;
+        q.C = workspace;
+        q.ldc = p.N;
+        q.sC = (int64_t)p.M * p.N;
+        q.cmode = (dtype == ntg::DT_F16 || dtype == ntg::DT_BF16) ? ntg::C_PARTIAL : ntg::C_OVERWRITE;
+        q.bias = nullptr;
+        int rc = launch_gemm(q, dtype, ta, tb, s);
+        if (rc) return rc;
+        hipError_t e = ntg::launch_splitk_reduce(dtype, workspace, plan.splits, p, s);
+        if (e != hipSuccess) return hip_fail(e, "split-K reduction launch");
+        return NTG_OK;
+    }
+    return launch_gemm(p, dtype, ta, tb, s);
 }
 
 int check_sizes(int64_t m, int64_t k, int64_t n, int64_t batches) {
@@ -156,7 +212,14 @@ int ntg_gemm_dev(const ntg_gemm_desc* d, const void* dA, const void* dB, void* d
     if (!dA || !dB || !dC) return fail(NTG_ERR_INVALID_ARGUMENT, "null matrix pointer");
     if (p.batch > 1 && p.sC == 0) return fail(NTG_ERR_INVALID_ARGUMENT, "stride_c must be non-zero for a batch (outputs may not alias)");
     p.A = dA; p.B = dB; p.C = dC;
-    return run_gemm(p, d->dtype, d->transpose_a != 0, d->transpose_b != 0, static_cast<hipStream_t>(stream));
+    return run_gemm(p, d->dtype, d->transpose_a != 0, d->transpose_b != 0, static_cast<hipStream_t>(stream), d->workspace, d->workspace_bytes);
+}
+
+int64_t ntg_gemm_workspace_bytes(const ntg_gemm_desc* d) {
+    ntg::GemmParams p;
+    if (desc_to_params(d, p)) return -1;
+    if (p.M == 0 || p.N == 0 || p.batch == 0) return 0;
+    return plan_splitk(p, d->dtype, d->transpose_a != 0).bytes;      // pointers taken as 16-byte aligned
 }
 
 int ntg_gemm_ptrs_dev(const ntg_gemm_desc* d, const void* const* dA, const void* const* dB, void* const* dC, void* stream) {
@@ -212,7 +275,14 @@ int ntg_matmult_batch(int dtype, const void* const* A, const void* const* B, voi
     const size_t c_off = off;
     off += align_up(c_bytes, 256) * (size_t)batches;
     const size_t tab_off = off;
-    off += 3 * sizeof(void*) * (size_t)batches;
+    off += align_up(3 * sizeof(void*) * (size_t)batches, 256);
+    ntg_gemm_desc d;
+    std::memset(&d, 0, sizeof d);
+    d.dtype = dtype; d.transpose_a = transpose_a; d.transpose_b = transpose_b; d.c_mode = NTG_C_ACCUMULATE;
+    d.m = m; d.k = k; d.n = n; d.batches = batches;
+    const size_t ws_off = off;
+    const int64_t ws_bytes = batches == 1 ? ntg_gemm_workspace_bytes(&d) : 0;
+    if (ws_bytes > 0) off += (size_t)ws_bytes;
 
     DeviceMem mem;
     HIP_TRY(mem.alloc(off));
@@ -230,11 +300,8 @@ int ntg_matmult_batch(int dtype, const void* const* A, const void* const* B, voi
     }
     HIP_TRY(hipMemcpy(mem.at(tab_off), tab.data(), tab.size() * sizeof(void*), hipMemcpyHostToDevice));
 
-    ntg_gemm_desc d;
-    std::memset(&d, 0, sizeof d);
-    d.dtype = dtype; d.transpose_a = transpose_a; d.transpose_b = transpose_b; d.c_mode = NTG_C_ACCUMULATE;
-    d.m = m; d.k = k; d.n = n; d.batches = batches;
     void** dtab = reinterpret_cast<void**>(mem.at(tab_off));
+    if (ws_bytes > 0) { d.workspace = mem.at(ws_off); d.workspace_bytes = ws_bytes; }
     if (batches == 1) {
         rc = ntg_gemm_dev(&d, tab[0], tab[1], tab[2], nullptr);
     } else {

@@ -85,6 +85,45 @@ __global__ void __launch_bounds__(256) reduce_batch_kernel(const T* __restrict__
     }
 }
 
+static unsigned grid_for(int64_t total) {
+    int64_t blocks = (total + 255) / 256;
+    if (blocks > 256 * 64) blocks = 256 * 64;
+    return (unsigned)(blocks < 1 ? 1 : blocks);
+}
+
+// Split-K epilogue: C (+)= sum over the k ranges of part[s][m][n], s ascending, starting from C0 (the incoming C, the
+// broadcast bias, or zero).  One rounding to T at the end.
+template <class T, class P, class Acc>
+__global__ void __launch_bounds__(256) splitk_reduce_kernel(const P* __restrict__ part, const int splits, const GemmParams p) {
+    const int64_t total = (int64_t)p.M * p.N;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    T* C = static_cast<T*>(p.C);
+    const T* bias = static_cast<const T*>(p.bias);
+    for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += stride) {
+        const int64_t m = idx / p.N, n = idx - m * p.N;
+        T* cp = C + m * p.ldc + n;
+        Acc acc = (Acc)0;
+        if (p.cmode == C_ACCUMULATE) acc = (Acc)*cp;
+        else if (p.cmode == C_BIAS) acc = (Acc)bias[m * p.bias_rs + n * p.bias_cs];
+        for (int s = 0; s < splits; ++s) acc += (Acc)part[(int64_t)s * total + idx];
+        *cp = (T)acc;
+    }
+}
+
+hipError_t launch_splitk_reduce(int dtype, const void* part, int splits, const GemmParams& p, hipStream_t s) {
+    const int64_t total = (int64_t)p.M * p.N;
+    if (total == 0) return hipSuccess;
+    const dim3 g(grid_for(total)), b(256);
+    switch (dtype) {
+    case DT_F32: hipLaunchKernelGGL((splitk_reduce_kernel<float, float, float>), g, b, 0, s, (const float*)part, splits, p); break;
+    case DT_F64: hipLaunchKernelGGL((splitk_reduce_kernel<double, double, double>), g, b, 0, s, (const double*)part, splits, p); break;
+    case DT_F16: hipLaunchKernelGGL((splitk_reduce_kernel<_Float16, float, float>), g, b, 0, s, (const float*)part, splits, p); break;
+    case DT_BF16: hipLaunchKernelGGL((splitk_reduce_kernel<__bf16, float, float>), g, b, 0, s, (const float*)part, splits, p); break;
+    default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+
 // wt[g][c][oc][t] = w[g*og + oc][c][taps-1-t]: the kernel with input/output channels swapped
 // inside each group and both tap axes reversed, i.e. the weights of the convolution that maps
 // the output gradient back to the image.
@@ -104,11 +143,6 @@ __global__ void __launch_bounds__(256) flip_weights_kernel(const T* __restrict__
     }
 }
 
-static unsigned grid_for(int64_t total) {
-    int64_t blocks = (total + 255) / 256;
-    if (blocks > 256 * 64) blocks = 256 * 64;
-    return (unsigned)(blocks < 1 ? 1 : blocks);
-}
 
 hipError_t launch_reduce_batch(int dtype, const void* part, void* out, int64_t batch, int64_t n, int accumulate, hipStream_t s) {
     if (n == 0) return hipSuccess;

@@ -73,8 +73,14 @@ def _launch(a, b, c, m, k, n, ta, tb, batches, sa, sb, sc, c_mode, bias=None, bi
     if bias is not None:
         d.bias = bias.data_ptr() + bias_off * es
         d.bias_batch_stride, d.bias_row_stride, d.bias_col_stride = bias_strides
-    check(load().ntg_gemm_dev(ctypes.byref(d), a.data_ptr() + a_off * es, b.data_ptr() + b_off * es,
-                              c.data_ptr() + c_off * es, _stream()))
+    L = load()
+    ws_bytes = L.ntg_gemm_workspace_bytes(ctypes.byref(d))      # > 0: few output tiles, deep k -> split along k
+    ws = None
+    if ws_bytes > 0:
+        ws = torch.empty((ws_bytes,), dtype=torch.uint8, device=a.device)
+        d.workspace, d.workspace_bytes = ws.data_ptr(), ws_bytes
+    check(L.ntg_gemm_dev(ctypes.byref(d), a.data_ptr() + a_off * es, b.data_ptr() + b_off * es,
+                         c.data_ptr() + c_off * es, _stream()))
 
 
 def matmult(a, b, out=None, transpose_a=False, transpose_b=False, accumulate=None):

@@ -41,7 +41,7 @@ def test_dtype_sizes_follow_nt_dtype_values():
 
 
 def test_desc_struct_layout():
-    assert ctypes.sizeof(_lib.GemmDesc) == 16 + 8 * 3 + 8 * 3 + 8 + 8 * 3 + 8 + 8 * 3
+    assert ctypes.sizeof(_lib.GemmDesc) == 16 + 8 * 3 + 8 * 3 + 8 + 8 * 3 + 8 + 8 * 3 + 8 + 8
 
 
 def test_argument_errors_do_not_need_a_device():

@@ -422,6 +422,57 @@ def test_skinny_16bit(dtype, m):
     assert ((y.double() - refy).abs().max() / refy.abs().max()).item() <= HALF_REL
 
 
+@pytest.mark.parametrize("dtype", ["bf16", np.float16, np.float32, np.float64], ids=["bf16", "fp16", "fp32", "fp64"])
+def test_split_k_medium_rows(dtype):
+    """Few output tiles and a deep k: ntg_gemm_workspace_bytes offers a workspace and the product is split along k
+    (fp32 partial sums for the 16-bit dtypes, ordered reduction).  Every transpose pair and C mode; the result must also
+    equal the unsplit run to rounding, and two runs must be bit-identical."""
+    bf = dtype == "bf16"
+    half = bf or dtype == np.float16
+    rng = np.random.default_rng(1900)
+    lib = _lib.load()
+    for (m, k, n) in [(256, 4096, 2048), (520, 2048, 1032), (64, 8192, 1024), (1024, 3072, 1024)]:
+        for ta, tb in TRANS:
+            a = randn(rng, (m, k), dtype, 0.25)
+            b = randn(rng, (k, n), dtype, 0.25)
+            sa = np.ascontiguousarray(a.T) if ta else a
+            sb = np.ascontiguousarray(b.T) if tb else b
+            ta_, tb_ = to_torch(sa, DEV, bf), to_torch(sb, DEV, bf)
+            d = _lib.GemmDesc()
+            d.dtype, d.transpose_a, d.transpose_b, d.c_mode = F.ntg_dtype(ta_), int(ta), int(tb), _lib.C_OVERWRITE
+            d.m, d.k, d.n, d.batches = m, k, n, 1
+            ws_bytes = lib.ntg_gemm_workspace_bytes(ctypes.byref(d))
+            assert ws_bytes > 0, (m, k, n)
+            assert ws_bytes % (m * n * (4 if half else a.itemsize)) == 0
+            ref = to_torch(a, DEV, bf).double() @ to_torch(b, DEV, bf).double()
+            scale = ref.abs().max().item()
+            tol = HALF_REL * scale if half else 1e-5 * k * float(np.abs(to_f64(a, bf)).max() * np.abs(to_f64(b, bf)).max())
+            out = F.matmult(ta_, tb_, None, ta, tb)                                # functional passes the workspace
+            assert (out.double() - ref).abs().max().item() <= tol
+            assert torch.equal(out, F.matmult(ta_, tb_, None, ta, tb))
+            # the same product without a workspace (one pass over k)
+            st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+            plain = torch.empty_like(out)
+            _lib.check(lib.ntg_gemm_dev(ctypes.byref(d), ta_.data_ptr(), tb_.data_ptr(), plain.data_ptr(), st))
+            assert (plain.double() - ref).abs().max().item() <= tol
+            assert (plain.double() - out.double()).abs().max().item() <= (2 * HALF_REL * scale / 8 if half else tol)
+            # C += and bias
+            c0 = to_torch(randn(rng, (m, n), dtype), DEV, bf)
+            c = c0.clone()
+            F.matmult(ta_, tb_, c, ta, tb)
+            assert (c.double() - (ref + c0.double())).abs().max().item() <= tol + (HALF_REL * scale if half else 0)
+        bias = to_torch(randn(rng, (n,), dtype), DEV, bf)
+        y = F.linear(to_torch(a, DEV, bf), to_torch(b, DEV, bf), bias)
+        refy = to_torch(a, DEV, bf).double() @ to_torch(b, DEV, bf).double() + bias.double()
+        assert (y.double() - refy).abs().max().item() <= tol + (HALF_REL * scale if half else 0)
+    # no split where it does not apply: many tiles, shallow k, batches
+    for (m, k, n, bt) in [(4096, 4096, 4096, 1), (256, 128, 256, 1), (256, 4096, 2048, 2)]:
+        d = _lib.GemmDesc()
+        d.dtype, d.m, d.k, d.n, d.batches = F.ntg_dtype(ta_), m, k, n, bt
+        d.stride_a, d.stride_b, d.stride_c = m * k, k * n, m * n
+        assert lib.ntg_gemm_workspace_bytes(ctypes.byref(d)) == 0
+
+
 def test_skinny_fp32_config5b():
     rng = np.random.default_rng(1005)
     a = rng.standard_normal((16, 8192)).astype(np.float32)
