@@ -554,15 +554,14 @@ ConvGrads conv2d_backward(const Tensor& image, const Tensor& kernel, const Tenso
 }
 
 // [.., C, W] -> [B, C, 1, W] (contiguous view)
-static Tensor as_one_row(const Tensor& t, int64_t lead_if_low, const char* what) {
+static Tensor as_one_row(const Tensor& t, const char* what) {
     utils::throw_exception(!t.is_null(), std::string("Cannot perform operation ") + what + " on a null tensor");
     Tensor c = t.contiguous();
     const SizeRef& s = c.shape();
     utils::throw_exception(s.size() >= 2, std::string("Expected to get a 2D or greater tensor for ") + what + ", but got " + std::to_string(s.size()) + "D");
     const int64_t W = s[s.size() - 1], C = s[s.size() - 2];
-    const int64_t B = s.size() == 2 ? lead_if_low : c.numel() / std::max<int64_t>(1, C * W);
-    (void)lead_if_low;
-    return c.view({s.size() == 2 ? 1 : B, C, 1, W});
+    const int64_t B = s.size() == 2 ? 1 : c.numel() / std::max<int64_t>(1, C * W);
+    return c.view({B, C, 1, W});
 }
 
 Tensor conv1d(const Tensor& image, const Tensor& kernel, int64_t stride, int64_t padding, int64_t dilation, int64_t groups) {
@@ -573,14 +572,14 @@ Tensor conv1d(const Tensor& image, const Tensor& kernel, int64_t stride, int64_t
     utils::throw_exception(stride >= 1, "Conv1d stride cannot be less than 1 but got " + std::to_string(stride));
     utils::throw_exception(dilation >= 1, "Conv1d dilation cannot be less than 1 but got " + std::to_string(dilation));
     utils::throw_exception(padding >= 0, "Conv1d padding cannot be less than 1 but got " + std::to_string(padding));
-    Tensor x = as_one_row(image, 1, "conv1d"), w = as_one_row(kernel, 1, "conv1d");
+    Tensor x = as_one_row(image, "conv1d"), w = as_one_row(kernel, "conv1d");
     Tensor o = functional::conv2d(x, w, {1, stride}, {0, padding}, {1, dilation}, groups);
     return o.view({o.shape()[0], o.shape()[1], o.shape()[3]});
 }
 
 ConvGrads conv1d_backward(const Tensor& image, const Tensor& kernel, const Tensor& grad, int64_t stride, int64_t padding, int64_t dilation,
                           int64_t groups) {
-    Tensor x = as_one_row(image, 1, "conv1d backward"), w = as_one_row(kernel, 1, "conv1d backward");
+    Tensor x = as_one_row(image, "conv1d backward"), w = as_one_row(kernel, "conv1d backward");
     ConvGrads g = functional::conv2d_backward(x, w, grad.contiguous(), {1, stride}, {0, padding}, {1, dilation}, groups);
     return {g.d_image.view(image.shape()), g.d_kernel.view(kernel.shape())};
 }
@@ -633,15 +632,15 @@ Tensor conv_transpose1d(const Tensor& image, const Tensor& kernel, int64_t strid
     utils::throw_exception(!image.is_null() && !kernel.is_null(), "Cannot perform operation conv_transpose1d on a null tensor");
     utils::throw_exception(image.dims() >= 2, "Expected to get a 2D or greater tensor as the input for a conv1d transpose, but got " + std::to_string(image.dims()) + "D");
     utils::throw_exception(kernel.dims() == 3 || kernel.dims() == 2, "Expected to get a 3D or 2D tensor as the kernel for a conv1d transpose, but got " + std::to_string(kernel.dims()) + "D");
-    Tensor x = as_one_row(image, 1, "conv_transpose1d"), w = as_one_row(kernel, 1, "conv_transpose1d");
+    Tensor x = as_one_row(image, "conv_transpose1d"), w = as_one_row(kernel, "conv_transpose1d");
     Tensor o = functional::conv_transpose2d(x, w, {1, stride}, {0, padding}, {0, output_padding}, {1, dilation}, groups);
     return o.view({o.shape()[0], o.shape()[1], o.shape()[3]});
 }
 
 ConvGrads conv_transpose1d_backward(const Tensor& image, const Tensor& kernel, const Tensor& grad, int64_t stride, int64_t padding,
                                     int64_t output_padding, int64_t dilation, int64_t groups) {
-    Tensor x = as_one_row(image, 1, "conv_transpose1d backward"), w = as_one_row(kernel, 1, "conv_transpose1d backward");
-    Tensor g = as_one_row(grad, 1, "conv_transpose1d backward");
+    Tensor x = as_one_row(image, "conv_transpose1d backward"), w = as_one_row(kernel, "conv_transpose1d backward");
+    Tensor g = as_one_row(grad, "conv_transpose1d backward");
     ConvGrads r = functional::conv_transpose2d_backward(x, w, g, {1, stride}, {0, padding}, {0, output_padding}, {1, dilation}, groups);
     return {r.d_image.view(image.shape()), r.d_kernel.view(kernel.shape())};
 }
