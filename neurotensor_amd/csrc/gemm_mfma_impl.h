@@ -97,41 +97,64 @@ __device__ __forceinline__ u32x4 ldvec(gptr<T> src, bool outer_ok, int c0, int c
 // neighbouring element), nothing consumes the value, so all of a tile's loads stay in flight; one
 // bit per element says whether it is real, and conv_mask() zeroes the rest when the tile is
 // written to LDS.  The bit of element e sits at bit 8*(e%4) of mask word e/4.
-struct ConvRow { uint32_t roff, r, q; int dh, dw; bool valid; };
-struct ConvCol { uint32_t off0; int ih0, iw0; };
+// ND = 2 or 3 spatial axes (compile time: the two-axis kernels carry no depth arithmetic)
+struct ConvRow { uint32_t roff, t, r, q; int dd, dh, dw; bool valid; };
+struct ConvCol { uint32_t off0; int id0, ih0, iw0; };
 
-template <class T>
+template <class T, int ND>
 __device__ __forceinline__ ConvRow conv_row(const ConvGeom& g, int kk, bool valid) {
-    const uint32_t c = fast_div((uint32_t)kk, g.div_krc);
-    const uint32_t rem = (uint32_t)kk - __umul24(c, (uint32_t)g.k_rc);
     ConvRow o;
+    uint32_t c, rem;
+    if constexpr (ND == 3) {
+        c = fast_div((uint32_t)kk, g.div_kdrc);
+        const uint32_t rem3 = (uint32_t)kk - __umul24(c, (uint32_t)g.k_drc);
+        o.t = fast_div(rem3, g.div_krc);
+        rem = rem3 - __umul24(o.t, (uint32_t)g.k_rc);
+        o.dd = (int)__umul24(o.t, (uint32_t)g.d_d) - g.p_d;
+    } else {
+        c = fast_div((uint32_t)kk, g.div_krc);
+        rem = (uint32_t)kk - __umul24(c, (uint32_t)g.k_rc);
+        o.t = 0;
+        o.dd = 0;
+    }
     o.r = fast_div(rem, g.div_kc);
     o.q = rem - __umul24(o.r, (uint32_t)g.k_c);
     o.valid = valid;
     o.dh = valid ? (int)__umul24(o.r, (uint32_t)g.d_r) - g.p_r : -(1 << 29);   // far outside: every tap is padding
     o.dw = (int)__umul24(o.q, (uint32_t)g.d_c) - g.p_c;
-    o.roff = (c * (uint32_t)g.HW + (uint32_t)o.dh * (uint32_t)g.W + (uint32_t)o.dw) * (uint32_t)sizeof(T);
+    o.roff = (c * (uint32_t)g.chan + ((uint32_t)o.dd * (uint32_t)g.H + (uint32_t)o.dh) * (uint32_t)g.W + (uint32_t)o.dw) * (uint32_t)sizeof(T);
     return o;
 }
 
-template <class T>
+template <class T, int ND>
 __device__ __forceinline__ ConvCol conv_col(const ConvGeom& g, int l, bool valid) {
-    const uint32_t oh = fast_div((uint32_t)l, g.div_wo);
-    const uint32_t ow = (uint32_t)l - oh * (uint32_t)g.Wo;
     ConvCol o;
+    uint32_t rem = (uint32_t)l;
+    o.id0 = 0;
+    if constexpr (ND == 3) {
+        const uint32_t od = fast_div((uint32_t)l, g.div_howo);
+        rem = (uint32_t)l - od * (uint32_t)g.HoWo;
+        o.id0 = (int)__umul24(od, (uint32_t)g.s_d);
+    }
+    const uint32_t oh = fast_div(rem, g.div_wo);
+    const uint32_t ow = rem - oh * (uint32_t)g.Wo;
     o.ih0 = valid ? (int)__umul24(oh, (uint32_t)g.s_r) : -(1 << 29);
     o.iw0 = (int)__umul24(ow, (uint32_t)g.s_c);
-    o.off0 = ((uint32_t)o.ih0 * (uint32_t)g.W + (uint32_t)o.iw0) * (uint32_t)sizeof(T);
+    o.off0 = (((uint32_t)o.id0 * (uint32_t)g.H + (uint32_t)o.ih0) * (uint32_t)g.W + (uint32_t)o.iw0) * (uint32_t)sizeof(T);
     return o;
 }
 
-// For a fixed column: bit r of `hm` / bit q of `wm` say whether tap row r / tap column q falls
-// inside the image (kernels up to 8 x 8; larger ones use the stored im2col matrix).
-__device__ __forceinline__ void conv_tap_masks(const ConvGeom& g, const ConvCol& col, uint32_t& hm, uint32_t& wm) {
+// For a fixed column: bit t of `dm` / bit r of `hm` / bit q of `wm` say whether that tap plane / row / column falls
+// inside the image (kernels up to 8 taps per axis; larger ones use the stored im2col matrix).
+template <int ND>
+__device__ __forceinline__ void conv_tap_masks(const ConvGeom& g, const ConvCol& col, uint32_t& dm, uint32_t& hm, uint32_t& wm) {
+    dm = 0xffu;
     hm = 0;
     wm = 0;
+    if constexpr (ND == 3) dm = 0;
 #pragma unroll
     for (int t = 0; t < 8; ++t) {
+        if constexpr (ND == 3) dm |= ((t < g.k_d) & ((unsigned)(col.id0 + t * g.d_d - g.p_d) < (unsigned)g.D)) ? (1u << t) : 0u;
         hm |= ((t < g.k_r) & ((unsigned)(col.ih0 + t * g.d_r - g.p_r) < (unsigned)g.H)) ? (1u << t) : 0u;
         wm |= ((t < g.k_c) & ((unsigned)(col.iw0 + t * g.d_c - g.p_c) < (unsigned)g.W)) ? (1u << t) : 0u;
     }
@@ -228,38 +251,42 @@ struct TileLoader {
     uint32_t coff[!KC ? NFIX : 1];                  // !KC: byte offsets of the thread's fixed columns ...
     uint32_t hpk[!KC ? (NFIX + 3) / 4 : 1];         //      ... and their tap masks, 8 bits per column
     uint32_t wpk[!KC ? (NFIX + 3) / 4 : 1];
+    uint32_t dpk[!KC ? (NFIX + 3) / 4 : 1];         //      (depth taps; three spatial axes only)
     ConvCol ccol[KC ? VE : 1];                      //  KC: this tile's columns
     ConvRow crow[KC ? NFIX : 1];                    //  KC: fixed rows;    !KC: the row being gathered
     uint32_t okm[NV][NW];
     uint32_t raw16[sizeof(T) == 2 ? NV * VE : 1];
 
+    template <int ND>
     __device__ __forceinline__ void conv_setup(const ConvGeom& g, int mn0, int MN, int tid) {
         if constexpr (!TRANSPOSE && KC) {
             static_assert(256 % KV == 0, "a thread keeps the same k offsets for every vector it loads");
 #pragma unroll
             for (int p = 0; p < NV; ++p) {
                 const int row = (tid + p * 256) / KV;
-                crow[p] = conv_row<T>(g, mn0 + row, mn0 + row < MN);
+                crow[p] = conv_row<T, ND>(g, mn0 + row, mn0 + row < MN);
             }
         } else {
             static_assert(TRANSPOSE || 256 % MV == 0, "a thread keeps the same columns for every vector it loads");
 #pragma unroll
-            for (int i = 0; i < (NFIX + 3) / 4; ++i) hpk[i] = wpk[i] = 0;
+            for (int i = 0; i < (NFIX + 3) / 4; ++i) hpk[i] = wpk[i] = dpk[i] = 0;
 #pragma unroll
             for (int i = 0; i < NFIX; ++i) {
                 // threads past NSB sub-blocks compute columns they never use
                 const int l = TRANSPOSE ? mn0 + ((tid + (i / 8) * 256) / KG) * 8 + (i % 8) : mn0 + (tid % MV) * VE + i;
-                const ConvCol c = conv_col<T>(g, l, l < MN);
-                uint32_t hm, wm;
-                conv_tap_masks(g, c, hm, wm);
+                const ConvCol c = conv_col<T, ND>(g, l, l < MN);
+                uint32_t dm, hm, wm;
+                conv_tap_masks<ND>(g, c, dm, hm, wm);
                 coff[i] = c.off0;
                 hpk[i / 4] |= hm << (8 * (i % 4));
                 wpk[i / 4] |= wm << (8 * (i % 4));
+                dpk[i / 4] |= dm << (8 * (i % 4));
             }
         }
     }
 
     // element idx (0 .. NE-1, a compile-time constant after unrolling) of the tile at k0
+    template <int ND>
     __device__ __forceinline__ void conv_elem(int idx, gptr<T> im, const ConvGeom& g, int k0, int K, int tid) {
         const int pv = idx / VE, e = idx % VE;
         if constexpr (TRANSPOSE && NSB % 256 != 0) {
@@ -270,11 +297,12 @@ struct TileLoader {
             if (idx == 0) {
                 const int kv = tid % KV;
 #pragma unroll
-                for (int c = 0; c < VE; ++c) ccol[c] = conv_col<T>(g, k0 + kv * VE + c, k0 + kv * VE + c < K);
+                for (int c = 0; c < VE; ++c) ccol[c] = conv_col<T, ND>(g, k0 + kv * VE + c, k0 + kv * VE + c < K);
             }
             const int ih = ccol[e].ih0 + crow[pv].dh;
             const int iw = ccol[e].iw0 + crow[pv].dw;
-            const bool ok = ((unsigned)ih < (unsigned)g.H) & ((unsigned)iw < (unsigned)g.W);   // no short circuit: branch-free
+            bool ok = ((unsigned)ih < (unsigned)g.H) & ((unsigned)iw < (unsigned)g.W);   // no short circuit: branch-free
+            if constexpr (ND == 3) ok = ok & ((unsigned)(ccol[e].id0 + crow[pv].dd) < (unsigned)g.D);
             if (e % 4 == 0) okm[pv][e / 4] = 0;
             okm[pv][e / 4] |= ok ? (1u << (8 * (e % 4))) : 0u;
             x = conv_load<T>(im, g, ccol[e].off0 + crow[pv].roff);
@@ -282,10 +310,11 @@ struct TileLoader {
             const int cb = TRANSPOSE ? (pv / 8) * 8 : 0;      // first fixed column of this vector
             if (e == 0) {
                 const int kk = TRANSPOSE ? k0 + ((tid + (pv / 8) * 256) % KG) * 8 + (pv % 8) : k0 + (tid + pv * 256) / MV;
-                crow[0] = conv_row<T>(g, kk, kk < K);
+                crow[0] = conv_row<T, ND>(g, kk, kk < K);
             }
             if (e % 4 == 0) {
-                const uint32_t m = (hpk[(cb + e) / 4] >> crow[0].r) & (wpk[(cb + e) / 4] >> crow[0].q) & 0x01010101u;
+                uint32_t m = (hpk[(cb + e) / 4] >> crow[0].r) & (wpk[(cb + e) / 4] >> crow[0].q) & 0x01010101u;
+                if constexpr (ND == 3) m &= dpk[(cb + e) / 4] >> crow[0].t;
                 okm[pv][e / 4] = crow[0].valid ? m : 0u;
             }
             x = conv_load<T>(im, g, coff[cb + e] + crow[0].roff);
@@ -302,14 +331,16 @@ struct TileLoader {
     }
 
     // slice s of ns of a tile's gather: the kernel spreads the slices between its MFMAs
+    template <int ND>
     __device__ __forceinline__ void conv_slice(int s, int ns, gptr<T> im, const ConvGeom& g, int k0, int K, int tid) {
 #pragma unroll
         for (int idx = 0; idx < NE; ++idx)
-            if (idx >= s * NE / ns && idx < (s + 1) * NE / ns) conv_elem(idx, im, g, k0, K, tid);
+            if (idx >= s * NE / ns && idx < (s + 1) * NE / ns) conv_elem<ND>(idx, im, g, k0, K, tid);
     }
 
+    template <int ND>
     __device__ __forceinline__ void load_conv(gptr<T> im, const ConvGeom& g, int k0, int K, int tid) {
-        conv_slice(0, 1, im, g, k0, K, tid);
+        conv_slice<ND>(0, 1, im, g, k0, K, tid);
     }
 
     __device__ __forceinline__ void conv_finish() {
@@ -378,8 +409,8 @@ struct GemmShape {
     static constexpr int GROUP_M = (1024 / BM) > 0 ? (1024 / BM) : 1;
 };
 
-// CONV: op(B) is the implicit im2col matrix of the image at p.B (p.conv), see load_conv.
-template <int DT, bool TA, bool TB, int WBM, int WBN, int BK, bool ALIGNED, bool CONV = false>
+// CONV = 2 / 3: op(B) is the implicit im2col matrix (two / three spatial axes) of the image at p.B (p.conv), see load_conv.
+template <int DT, bool TA, bool TB, int WBM, int WBN, int BK, bool ALIGNED, int CONV = 0>
 __global__ void __launch_bounds__(256) gemm_mfma_kernel(const GemmParams p) {
     using SH = GemmShape<DT, TA, TB, WBM, WBN, BK>;
     using E = Elem<DT>;
@@ -428,14 +459,14 @@ __global__ void __launch_bounds__(256) gemm_mfma_kernel(const GemmParams p) {
     const int KT = (p.K + BK - 1) / BK;
 
     auto load_b = [&](int k0) {
-        if constexpr (CONV) lb.load_conv(B, p.conv, k0, p.K, tid);
+        if constexpr (CONV != 0) lb.template load_conv<CONV>(B, p.conv, k0, p.K, tid);
         else lb.load(B, p.ldb, n0, k0, p.N, p.K, vecB, tid);
     };
-    if constexpr (CONV) lb.conv_setup(p.conv, n0, p.N, tid);
+    if constexpr (CONV != 0) lb.template conv_setup<CONV>(p.conv, n0, p.N, tid);
 
     la.load(A, p.lda, m0, 0, p.M, p.K, vecA, tid);
     load_b(0);
-    if constexpr (CONV) lb.conv_finish();
+    if constexpr (CONV != 0) lb.conv_finish();
     la.store(smem, tid);
     lb.store(smem + SH::LDS_A, tid);
     __syncthreads();
@@ -446,18 +477,18 @@ __global__ void __launch_bounds__(256) gemm_mfma_kernel(const GemmParams p) {
         // The gathering kernels load unconditionally (the last pass re-reads the last tile into the
         // idle stage), so that the loop body is one scheduling region and the address arithmetic
         // of the gather can sit in the shadow of the MFMAs.
-        const bool more = CONV || (kt + 1 < KT);
-        const int k_next = (CONV && kt + 1 >= KT ? kt : kt + 1) * BK;
+        const bool more = CONV != 0 || (kt + 1 < KT);
+        const int k_next = (CONV != 0 && kt + 1 >= KT ? kt : kt + 1) * BK;
         if (more) {
             la.load(A, p.lda, m0, k_next, p.M, p.K, vecA, tid);
-            if constexpr (!CONV) load_b(k_next);
+            if constexpr (CONV == 0) load_b(k_next);
         }
         // CONV: slice `step` of NSTEP of the next tile's gather follows each group of MFMAs; only LDS
         // reads and scalar work may move across the fence, so the slice stays with its group.
         constexpr int NSTEP = IS16 ? BK / 16 : BK / G;
         auto gather_slice = [&](int step) {
-            if constexpr (CONV) {
-                lb.conv_slice(step, NSTEP, B, p.conv, k_next, p.K, tid);
+            if constexpr (CONV != 0) {
+                lb.template conv_slice<CONV>(step, NSTEP, B, p.conv, k_next, p.K, tid);
                 __builtin_amdgcn_sched_barrier(0x104);
             }
         };
@@ -531,7 +562,7 @@ __global__ void __launch_bounds__(256) gemm_mfma_kernel(const GemmParams p) {
         }
         if (more) {
             char* dA = smem + ((kt + 1) & 1) * SH::STAGE;
-            if constexpr (CONV) {
+            if constexpr (CONV != 0) {
                 // the gathered values are first touched here, after the MFMAs of this tile
                 __builtin_amdgcn_sched_barrier(0);
                 lb.conv_finish();
@@ -555,7 +586,7 @@ __global__ void __launch_bounds__(256) gemm_mfma_kernel(const GemmParams p) {
             for (int r = 0; r < E::ACCN; ++r) {
                 const int lrow = acc_row<R>(r, lane);
                 const int m = m0 + (A_KM ? (wm * WBM + i) * R + lrow : (wm * R + lrow) * WBM + i);
-                if ((ALIGNED && !CONV) || (m < p.M && n < p.N)) {
+                if ((ALIGNED && CONV == 0) || (m < p.M && n < p.N)) {
                     const gptr_mut<T> cp = C + (int64_t)m * p.ldc + n;
                     AccS val = acc[i][j][r];
                     if (cmode == C_ACCUMULATE) val += (AccS)(*cp);
@@ -598,7 +629,7 @@ static hipError_t launch_cfg(const GemmParams& pin, hipStream_t s) {
 
 // op(B) = implicit im2col matrix (TB: transposed).  ALIGNED here speaks of A only (whole tiles,
 // 16-byte rows); the gathered operand and the stores are always guarded.
-template <int DT, bool TB, int WBM, int WBN, int BK>
+template <int DT, bool TB, int ND, int WBM, int WBN, int BK>
 static hipError_t launch_conv_cfg(const GemmParams& pin, hipStream_t s) {
     using SH = GemmShape<DT, false, TB, WBM, WBN, BK>;
     GemmParams p = pin;
@@ -611,12 +642,12 @@ static hipError_t launch_conv_cfg(const GemmParams& pin, hipStream_t s) {
     const bool a_aligned = (p.M % SH::BM == 0) && (p.K % BK == 0) && p.vecA_ok && !p.Aptr &&
                            ((reinterpret_cast<uintptr_t>(p.A) & 15) == 0) && (p.sA % VE == 0);
     if (a_aligned) {
-        auto k = gemm_mfma_kernel<DT, false, TB, WBM, WBN, BK, true, true>;
+        auto k = gemm_mfma_kernel<DT, false, TB, WBM, WBN, BK, true, ND>;
         static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(k), hipFuncAttributeMaxDynamicSharedMemorySize, SH::LDS_TOTAL);
         if (attr != hipSuccess) return attr;
         hipLaunchKernelGGL(k, dim3((unsigned)blocks), dim3(256), SH::LDS_TOTAL, s, p);
     } else {
-        auto k = gemm_mfma_kernel<DT, false, TB, WBM, WBN, BK, false, true>;
+        auto k = gemm_mfma_kernel<DT, false, TB, WBM, WBN, BK, false, ND>;
         static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(k), hipFuncAttributeMaxDynamicSharedMemorySize, SH::LDS_TOTAL);
         if (attr != hipSuccess) return attr;
         hipLaunchKernelGGL(k, dim3((unsigned)blocks), dim3(256), SH::LDS_TOTAL, s, p);

@@ -35,16 +35,16 @@ static inline FastDiv make_fastdiv(uint32_t d) {
 }
 
 // Geometry of an operand that is the im2col matrix of an image and is never stored:
-//   col(kk, l) = im[c, oh*s_r - p_r + r*d_r, ow*s_c - p_c + q*d_c]   (0 in the padding)
-//   kk = (c*k_r + r)*k_c + q,   l = oh*Wo + ow
-// (the matrix nt::functional::unfold2d(..., transpose_out = true) would produce,
-// nt/functional/cpu/unfold2d.cpp:12-112).
+//   col(kk, l) = im[c, od*s_d - p_d + t*d_d, oh*s_r - p_r + r*d_r, ow*s_c - p_c + q*d_c]   (0 in the padding)
+//   kk = ((c*k_d + t)*k_r + r)*k_c + q,   l = (od*Ho + oh)*Wo + ow
+// (the matrix nt::functional::unfold2d / unfold3d(..., transpose_out = true) would produce,
+// nt/functional/cpu/unfold2d.cpp:12-112, unfold3d.cpp:9-80).  Two spatial axes: D = k_d = s_d = d_d = 1, p_d = 0.
 struct ConvGeom {
-    int H, W, HW;
-    int s_r, s_c, p_r, p_c, d_r, d_c;
-    int k_r, k_c, k_rc, Wo;
+    int D, H, W, chan;       // chan = D*H*W, the channel stride
+    int s_d, s_r, s_c, p_d, p_r, p_c, d_d, d_r, d_c;
+    int k_d, k_r, k_c, k_rc, k_drc, Wo, HoWo;
     int last;                // index of the last element of the image slice at p.B (loads are clamped to it)
-    FastDiv div_krc, div_kc, div_wo;
+    FastDiv div_kdrc, div_krc, div_kc, div_wo, div_howo;
 };
 
 struct GemmParams {

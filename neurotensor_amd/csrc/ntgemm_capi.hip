@@ -19,17 +19,17 @@ hipError_t launch_gemm_mfma_f64(bool ta, bool tb, const GemmParams& p, hipStream
 hipError_t launch_gemm_mfma_f16(bool ta, bool tb, const GemmParams& p, hipStream_t s);
 hipError_t launch_gemm_mfma_bf16(bool ta, bool tb, const GemmParams& p, hipStream_t s);
 hipError_t launch_gemm_skinny(int dtype, bool ta, bool tb, const GemmParams& p, hipStream_t s, bool* handled);
-hipError_t launch_conv_mfma_f32(bool tb, const GemmParams& p, hipStream_t s);
-hipError_t launch_conv_mfma_f64(bool tb, const GemmParams& p, hipStream_t s);
-hipError_t launch_conv_mfma_f16(bool tb, const GemmParams& p, hipStream_t s);
-hipError_t launch_conv_mfma_bf16(bool tb, const GemmParams& p, hipStream_t s);
+hipError_t launch_conv_mfma_f32(bool tb, int nd, const GemmParams& p, hipStream_t s);
+hipError_t launch_conv_mfma_f64(bool tb, int nd, const GemmParams& p, hipStream_t s);
+hipError_t launch_conv_mfma_f16(bool tb, int nd, const GemmParams& p, hipStream_t s);
+hipError_t launch_conv_mfma_bf16(bool tb, int nd, const GemmParams& p, hipStream_t s);
 
-hipError_t launch_conv_mfma(int dtype, bool tb, const GemmParams& p, hipStream_t s) {
+hipError_t launch_conv_mfma(int dtype, bool tb, int nd, const GemmParams& p, hipStream_t s) {
     switch (dtype) {
-    case DT_F32: return launch_conv_mfma_f32(tb, p, s);
-    case DT_F64: return launch_conv_mfma_f64(tb, p, s);
-    case DT_F16: return launch_conv_mfma_f16(tb, p, s);
-    case DT_BF16: return launch_conv_mfma_bf16(tb, p, s);
+    case DT_F32: return launch_conv_mfma_f32(tb, nd, p, s);
+    case DT_F64: return launch_conv_mfma_f64(tb, nd, p, s);
+    case DT_F16: return launch_conv_mfma_f16(tb, nd, p, s);
+    case DT_BF16: return launch_conv_mfma_bf16(tb, nd, p, s);
     default: return hipErrorInvalidValue;
     }
 }
@@ -401,30 +401,163 @@ int ntg_unfold2d(int dtype, const void* image, void* col,
     return NTG_OK;
 }
 
-// The floating dtypes gather the im2col operand inside the GEMM (no col buffer) when every
-// index the kernel forms fits 32 bits with room for its out-of-range sentinels.
-static bool conv_implicit(int dtype, int64_t channels, int64_t height, int64_t width, int64_t k_r, int64_t k_c,
-                          int64_t s_r, int64_t s_c, int64_t p_r, int64_t p_c, int64_t d_r, int64_t d_c, int64_t Ho, int64_t Wo) {
-    if (is_int_dtype(dtype)) return false;
-    if (k_r > 8 || k_c > 8) return false;   // the kernels keep one byte of tap mask per output pixel
-    const int64_t lim = 1 << 24;
-    if (height >= lim || width >= lim || s_r >= lim || s_c >= lim || p_r >= lim || p_c >= lim) return false;
-    if (k_r * d_r >= lim || k_c * d_c >= lim || Ho * s_r >= lim || Wo * s_c >= lim) return false;
-    if (channels >= lim || k_r * k_c >= lim) return false;
-    // byte offsets inside one image are formed in 32 bits
-    if (channels * height * width * ntg::elem_size(dtype) >= 0x7fffffffLL || channels * k_r * k_c >= 0x7fffffffLL || Ho * Wo >= 0x7fffffffLL) return false;
-    return channels * height * width > 0;
+// Geometry of a convolution over two or three spatial axes; axis 0 is the depth (size 1, one tap for two axes).
+struct Geo3 {
+    int nd;
+    int64_t sz[3], k[3], s[3], p[3], d[3], o[3];
+    int64_t vol() const { return sz[0] * sz[1] * sz[2]; }
+    int64_t taps() const { return k[0] * k[1] * k[2]; }
+    int64_t L() const { return o[0] * o[1] * o[2]; }
+};
+
+static Geo3 geo2(int64_t height, int64_t width, int64_t k_r, int64_t k_c, int64_t s_r, int64_t s_c, int64_t p_r, int64_t p_c,
+                 int64_t d_r, int64_t d_c, int64_t Ho, int64_t Wo) {
+    return Geo3{2, {1, height, width}, {1, k_r, k_c}, {1, s_r, s_c}, {0, p_r, p_c}, {1, d_r, d_c}, {1, Ho, Wo}};
 }
 
-static void fill_conv_geom(ntg::ConvGeom& g, int64_t slice_channels, int64_t height, int64_t width, int64_t k_r, int64_t k_c, int64_t s_r, int64_t s_c,
-                           int64_t p_r, int64_t p_c, int64_t d_r, int64_t d_c, int64_t Wo) {
-    g.H = (int)height; g.W = (int)width; g.HW = (int)(height * width);
-    g.s_r = (int)s_r; g.s_c = (int)s_c; g.p_r = (int)p_r; g.p_c = (int)p_c; g.d_r = (int)d_r; g.d_c = (int)d_c;
-    g.k_r = (int)k_r; g.k_c = (int)k_c; g.k_rc = (int)(k_r * k_c); g.Wo = (int)Wo;
-    g.last = (int)(slice_channels * height * width - 1);
-    g.div_krc = ntg::make_fastdiv((uint32_t)(k_r * k_c));
-    g.div_kc = ntg::make_fastdiv((uint32_t)k_c);
-    g.div_wo = ntg::make_fastdiv((uint32_t)Wo);
+// The geometry of the convolution that maps the output gradient back to the image (all strides 1): its "image" is the
+// gradient, its outputs are the image elements, its padding is d*(k-1) - p (negative = the image is cropped).
+static Geo3 geo_dimage(const Geo3& g) {
+    Geo3 t = g;
+    for (int a = 0; a < 3; ++a) {
+        t.sz[a] = g.o[a]; t.o[a] = g.sz[a]; t.s[a] = 1;
+        t.p[a] = g.d[a] * (g.k[a] - 1) - g.p[a];
+    }
+    return t;
+}
+
+// The floating dtypes gather the im2col operand inside the GEMM (no col buffer) when every index the kernel forms fits
+// 32 bits with room for its out-of-range sentinels and the kernel has at most 8 taps per axis (one byte of tap mask).
+static bool conv_implicit_g(int dtype, int64_t channels, const Geo3& g) {
+    if (is_int_dtype(dtype)) return false;
+    const int64_t lim = 1 << 24;
+    for (int a = 0; a < 3; ++a) {
+        if (g.k[a] > 8) return false;
+        if (g.sz[a] >= lim || g.s[a] >= lim || g.p[a] >= lim || g.p[a] <= -lim) return false;
+        if (g.k[a] * g.d[a] >= lim || g.o[a] * g.s[a] >= lim) return false;
+    }
+    if (channels >= lim || g.taps() >= lim) return false;
+    // byte offsets inside one image are formed in 32 bits
+    if (channels * g.vol() * ntg::elem_size(dtype) >= 0x7fffffffLL || channels * g.taps() >= 0x7fffffffLL || g.L() >= 0x7fffffffLL) return false;
+    return channels * g.vol() > 0;
+}
+
+static bool conv_implicit(int dtype, int64_t channels, int64_t height, int64_t width, int64_t k_r, int64_t k_c,
+                          int64_t s_r, int64_t s_c, int64_t p_r, int64_t p_c, int64_t d_r, int64_t d_c, int64_t Ho, int64_t Wo) {
+    return conv_implicit_g(dtype, channels, geo2(height, width, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c, Ho, Wo));
+}
+
+static void fill_conv_geom(ntg::ConvGeom& c, int64_t slice_channels, const Geo3& g) {
+    c.D = (int)g.sz[0]; c.H = (int)g.sz[1]; c.W = (int)g.sz[2]; c.chan = (int)g.vol();
+    c.s_d = (int)g.s[0]; c.s_r = (int)g.s[1]; c.s_c = (int)g.s[2];
+    c.p_d = (int)g.p[0]; c.p_r = (int)g.p[1]; c.p_c = (int)g.p[2];
+    c.d_d = (int)g.d[0]; c.d_r = (int)g.d[1]; c.d_c = (int)g.d[2];
+    c.k_d = (int)g.k[0]; c.k_r = (int)g.k[1]; c.k_c = (int)g.k[2];
+    c.k_rc = (int)(g.k[1] * g.k[2]); c.k_drc = (int)g.taps();
+    c.Wo = (int)g.o[2]; c.HoWo = (int)(g.o[1] * g.o[2]);
+    c.last = (int)(slice_channels * g.vol() - 1);
+    c.div_kdrc = ntg::make_fastdiv((uint32_t)c.k_drc);
+    c.div_krc = ntg::make_fastdiv((uint32_t)c.k_rc);
+    c.div_kc = ntg::make_fastdiv((uint32_t)c.k_c);
+    c.div_wo = ntg::make_fastdiv((uint32_t)c.Wo);
+    c.div_howo = ntg::make_fastdiv((uint32_t)c.HoWo);
+}
+
+// out_b[g*og:(g+1)*og, L] = W_g[og, add] . col_b[g*add:(g+1)*add, L] with col_b gathered from the image by the B loader.
+// The reference forms (col_b^T . W_g^T) and swaps rows/columns afterwards (conv.cpp:94, :143); each output element is the
+// same ascending-k sum of the same products.
+static int conv_forward_gather(int dtype, const void* image, const void* kernel, void* out, int64_t batch, int64_t channels,
+                               int64_t out_channels, const Geo3& g, int64_t groups, hipStream_t hs) {
+    const int64_t es = ntg::elem_size(dtype), cg = channels / groups, og = out_channels / groups;
+    const int64_t L = g.L(), add = cg * g.taps(), vol = g.vol();
+    for (int64_t gi = 0; gi < groups; ++gi) {
+        ntg::GemmParams p;
+        std::memset(&p, 0, sizeof p);
+        p.M = (int)og; p.K = (int)add; p.N = (int)L; p.batch = (int)batch;
+        p.A = static_cast<const char*>(kernel) + gi * og * add * es;
+        p.B = static_cast<const char*>(image) + gi * cg * vol * es;
+        p.C = static_cast<char*>(out) + gi * og * L * es;
+        p.lda = add; p.ldb = L; p.ldc = L;
+        p.sA = 0; p.sB = channels * vol; p.sC = out_channels * L;
+        p.cmode = ntg::C_OVERWRITE;
+        p.vecA_ok = (add * es) % 16 == 0;
+        fill_conv_geom(p.conv, cg, g);
+        hipError_t e = ntg::launch_conv_mfma(dtype, false, g.nd, p, hs);
+        if (e != hipSuccess) return hip_fail(e, "implicit convolution launch");
+    }
+    return NTG_OK;
+}
+
+// dW: one batched GEMM  P_{b,g} [og, add] = dY_{b,g} [og, L] . col_{b,g}^T  with col gathered from the image, into
+// ws [B][O][add]; then the per-image results are summed in batch order (the same additions, in the same order, as
+// accumulating one GEMM per image into dW, conv.cpp:466-469).
+static int conv_dkernel_gather(int dtype, const void* image, const void* grad_out, void* d_kernel, void* ws, int64_t batch,
+                               int64_t channels, int64_t out_channels, const Geo3& g, int64_t groups, int accumulate, hipStream_t hs) {
+    const int64_t es = ntg::elem_size(dtype), cg = channels / groups, og = out_channels / groups;
+    const int64_t L = g.L(), add = cg * g.taps(), vol = g.vol();
+    for (int64_t gi = 0; gi < groups; ++gi) {
+        ntg::GemmParams p;
+        std::memset(&p, 0, sizeof p);
+        p.M = (int)og; p.K = (int)L; p.N = (int)add; p.batch = (int)batch;
+        p.A = static_cast<const char*>(grad_out) + gi * og * L * es;
+        p.B = static_cast<const char*>(image) + gi * cg * vol * es;
+        p.C = static_cast<char*>(ws) + gi * og * add * es;
+        p.lda = L; p.ldb = L; p.ldc = add;
+        p.sA = out_channels * L; p.sB = channels * vol; p.sC = out_channels * add;
+        p.cmode = ntg::C_OVERWRITE;
+        p.vecA_ok = (L * es) % 16 == 0 && (p.sA * es) % 16 == 0;
+        fill_conv_geom(p.conv, cg, g);
+        hipError_t e = ntg::launch_conv_mfma(dtype, true, g.nd, p, hs);
+        if (e != hipSuccess) return hip_fail(e, "implicit conv_dkernel launch");
+    }
+    hipError_t e = ntg::launch_reduce_batch(dtype, ws, d_kernel, batch, out_channels * add, accumulate, hs);
+    if (e != hipSuccess) return hip_fail(e, "weight gradient reduction launch");
+    return NTG_OK;
+}
+
+// dX (all strides 1): the convolution of dY with the channel-swapped, tap-reversed kernel (written to ws) and padding
+// d*(k-1) - p, again as an implicit GEMM; one sum over (oc, taps) per element instead of the reference's GEMM over oc
+// followed by col2im over the taps -- same terms, different rounding order, inside the stated tolerance.
+static int conv_dimage_gather(int dtype, const void* kernel, const void* grad_out, void* d_image, void* ws, int64_t batch,
+                              int64_t channels, int64_t out_channels, const Geo3& g, int64_t groups, int accumulate, hipStream_t hs) {
+    const int64_t es = ntg::elem_size(dtype), cg = channels / groups, og = out_channels / groups;
+    const int64_t L = g.L(), taps = g.taps(), vol = g.vol();
+    hipError_t e = ntg::launch_flip_weights(es, kernel, ws, groups, og, cg, taps, hs);
+    if (e != hipSuccess) return hip_fail(e, "weight flip launch");
+    const Geo3 t = geo_dimage(g);
+    for (int64_t gi = 0; gi < groups; ++gi) {
+        ntg::GemmParams p;
+        std::memset(&p, 0, sizeof p);
+        p.M = (int)cg; p.K = (int)(og * taps); p.N = (int)vol; p.batch = (int)batch;
+        p.A = static_cast<const char*>(ws) + gi * cg * og * taps * es;
+        p.B = static_cast<const char*>(grad_out) + gi * og * L * es;
+        p.C = static_cast<char*>(d_image) + gi * cg * vol * es;
+        p.lda = og * taps; p.ldb = vol; p.ldc = vol;
+        p.sA = 0; p.sB = out_channels * L; p.sC = channels * vol;
+        p.cmode = accumulate ? ntg::C_ACCUMULATE : ntg::C_OVERWRITE;
+        p.vecA_ok = (og * taps * es) % 16 == 0;
+        fill_conv_geom(p.conv, og, t);
+        e = ntg::launch_conv_mfma(dtype, false, g.nd, p, hs);
+        if (e != hipSuccess) return hip_fail(e, "implicit conv_dimage launch");
+    }
+    return NTG_OK;
+}
+
+// Which backward gradients run as implicit GEMMs, and the workspace the call needs.
+struct ConvBackwardPlan { bool gather_dw, gather_dx; int64_t need; };
+static ConvBackwardPlan plan_conv_backward_g(int dtype, bool want_dx, bool want_dw, int64_t batch, int64_t channels, int64_t out_channels,
+                                             const Geo3& g, int64_t groups) {
+    const int64_t es = ntg::elem_size(dtype);
+    const int64_t cg = channels / groups, taps = g.taps();
+    ConvBackwardPlan pl;
+    pl.gather_dw = want_dw && conv_implicit_g(dtype, channels, g);
+    pl.gather_dx = want_dx && g.s[0] == 1 && g.s[1] == 1 && g.s[2] == 1 && conv_implicit_g(dtype, out_channels, geo_dimage(g));
+    const int64_t col = batch * channels * taps * g.L() * es;
+    int64_t need = 0;
+    if (want_dw) need = std::max(need, pl.gather_dw ? batch * out_channels * cg * taps * es : col);
+    if (want_dx) need = std::max(need, pl.gather_dx ? out_channels * cg * taps * es : col);
+    pl.need = need;
+    return pl;
 }
 
 int64_t ntg_conv2d_forward_workspace_bytes(int dtype, int64_t batch, int64_t channels, int64_t height, int64_t width,
@@ -464,29 +597,12 @@ int ntg_conv2d_dev(int dtype, const void* image, const void* kernel, void* out,
     if (rc) return rc;
     if (batch == 0 || out_channels == 0) return NTG_OK;
     if (!image || !kernel || !out) return fail(NTG_ERR_INVALID_ARGUMENT, "null pointer");
-    // Per image b and group g:  out_b[g*og:(g+1)*og, L] = W_g[og, add] . col_b[g*add:(g+1)*add, L].
-    // The reference forms (col_b^T . W_g^T) and swaps rows/columns afterwards (conv.cpp:94);
-    // each output element is the same ascending-k sum of the same products.
     const int64_t L = Ho * Wo, ckk = channels * k_r * k_c;
     const int64_t add = (channels / groups) * k_r * k_c, og = out_channels / groups;
-    if (conv_implicit(dtype, channels, height, width, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c, Ho, Wo)) {
-        // col_b is never stored: the GEMM's B loader gathers it from the image
-        for (int64_t g = 0; g < groups; ++g) {
-            ntg::GemmParams p;
-            std::memset(&p, 0, sizeof p);
-            p.M = (int)og; p.K = (int)add; p.N = (int)L; p.batch = (int)batch;
-            p.A = static_cast<const char*>(kernel) + g * og * add * es;
-            p.B = static_cast<const char*>(image) + g * (channels / groups) * height * width * es;
-            p.C = static_cast<char*>(out) + g * og * L * es;
-            p.lda = add; p.ldb = L; p.ldc = L;
-            p.sA = 0; p.sB = channels * height * width; p.sC = out_channels * L;
-            p.cmode = ntg::C_OVERWRITE;
-            p.vecA_ok = (add * es) % 16 == 0;
-            fill_conv_geom(p.conv, channels / groups, height, width, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c, Wo);
-            hipError_t e = ntg::launch_conv_mfma(dtype, false, p, static_cast<hipStream_t>(stream));
-            if (e != hipSuccess) return hip_fail(e, "implicit conv2d launch");
-        }
-        return NTG_OK;
+    {
+        const Geo3 g = geo2(height, width, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c, Ho, Wo);
+        if (conv_implicit_g(dtype, channels, g))      // col_b is never stored: the GEMM's B loader gathers it from the image
+            return conv_forward_gather(dtype, image, kernel, out, batch, channels, out_channels, g, groups, static_cast<hipStream_t>(stream));
     }
     const int64_t need = batch * channels * k_r * k_c * Ho * Wo * es;
     if (need > 0 && (!workspace || workspace_bytes < need))
@@ -587,25 +703,11 @@ int ntg_unfold2d_backward(int dtype, const void* col, void* image,
     return NTG_OK;
 }
 
-// Which conv2d-backward gradients run as implicit GEMMs, and the workspace the call needs.
-struct ConvBackwardPlan { bool gather_dw, gather_dx; int64_t q_r, q_c, need; };
 static ConvBackwardPlan plan_conv_backward(int dtype, bool want_dx, bool want_dw, int64_t batch, int64_t channels, int64_t height, int64_t width,
                                            int64_t out_channels, int64_t k_r, int64_t k_c, int64_t s_r, int64_t s_c, int64_t p_r, int64_t p_c,
                                            int64_t d_r, int64_t d_c, int64_t groups, int64_t Ho, int64_t Wo) {
-    const int64_t es = ntg::elem_size(dtype);
-    const int64_t cg = channels / groups, taps = k_r * k_c;
-    ConvBackwardPlan pl;
-    pl.q_r = d_r * (k_r - 1) - p_r;   // padding of the gradient-to-image convolution
-    pl.q_c = d_c * (k_c - 1) - p_c;
-    pl.gather_dw = want_dw && conv_implicit(dtype, channels, height, width, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c, Ho, Wo);
-    pl.gather_dx = want_dx && s_r == 1 && s_c == 1 && pl.q_r > -(1 << 24) && pl.q_c > -(1 << 24) &&
-                   conv_implicit(dtype, out_channels, Ho, Wo, k_r, k_c, 1, 1, pl.q_r < 0 ? 0 : pl.q_r, pl.q_c < 0 ? 0 : pl.q_c, d_r, d_c, height, width);
-    const int64_t col = batch * channels * taps * Ho * Wo * es;
-    int64_t need = 0;
-    if (want_dw) need = std::max(need, pl.gather_dw ? batch * out_channels * cg * taps * es : col);
-    if (want_dx) need = std::max(need, pl.gather_dx ? out_channels * cg * taps * es : col);
-    pl.need = need;
-    return pl;
+    return plan_conv_backward_g(dtype, want_dx, want_dw, batch, channels, out_channels,
+                                geo2(height, width, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c, Ho, Wo), groups);
 }
 
 int64_t ntg_conv2d_backward_workspace_bytes(int dtype, int64_t batch, int64_t channels, int64_t height, int64_t width,
@@ -645,55 +747,17 @@ int ntg_conv2d_backward_dev(int dtype, const void* image, const void* kernel, co
     const char* gy = static_cast<const char*>(grad_out);
     char* ws = static_cast<char*>(workspace);
     hipStream_t hs = static_cast<hipStream_t>(stream);
-    const int64_t cg = channels / groups, HW = height * width;
     ntg_gemm_desc d;
-    // Floating dtypes: neither gradient needs the stored im2col matrix.
-    //   dW: one batched GEMM  P_b,g [og, add] = dY_{b,g} [og, L] . col_{b,g}^T  with col gathered from the image by the
-    //       B loader, then the per-image results are summed in batch order (the same additions, in the same order, as
-    //       accumulating one GEMM per image into dW).
-    //   dX (stride 1): the convolution of dY with the channel-swapped, tap-reversed kernel and padding d*(k-1) - p,
-    //       again as an implicit GEMM; one sum over (oc, i, j) per element instead of the reference's GEMM over oc
-    //       followed by col2im over (i, j) -- same terms, different rounding order, inside the stated tolerance.
+    // Floating dtypes: neither gradient needs the stored im2col matrix (conv_dkernel_gather, conv_dimage_gather).
     const bool gather_dw = plan.gather_dw, gather_dx = plan.gather_dx;
-    const int64_t q_r = plan.q_r, q_c = plan.q_c;
+    const Geo3 geo = geo2(height, width, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c, Ho, Wo);
     if (gather_dw) {
-        for (int64_t g = 0; g < groups; ++g) {
-            ntg::GemmParams p;
-            std::memset(&p, 0, sizeof p);
-            p.M = (int)og; p.K = (int)L; p.N = (int)add; p.batch = (int)batch;
-            p.A = gy + g * og * L * es;
-            p.B = static_cast<const char*>(image) + g * cg * HW * es;
-            p.C = ws + g * og * add * es;
-            p.lda = L; p.ldb = L; p.ldc = add;
-            p.sA = out_channels * L; p.sB = channels * HW; p.sC = out_channels * add;
-            p.cmode = ntg::C_OVERWRITE;
-            p.vecA_ok = (L * es) % 16 == 0 && (p.sA * es) % 16 == 0;
-            fill_conv_geom(p.conv, cg, height, width, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c, Wo);
-            hipError_t e = ntg::launch_conv_mfma(dtype, true, p, hs);
-            if (e != hipSuccess) return hip_fail(e, "implicit conv_dkernel launch");
-        }
-        hipError_t e = ntg::launch_reduce_batch(dtype, ws, d_kernel, batch, out_channels * add, accumulate, hs);
-        if (e != hipSuccess) return hip_fail(e, "weight gradient reduction launch");
+        rc = conv_dkernel_gather(dtype, image, grad_out, d_kernel, ws, batch, channels, out_channels, geo, groups, accumulate, hs);
+        if (rc) return rc;
     }
     if (gather_dx) {
-        const int64_t taps = k_r * k_c;
-        hipError_t e = ntg::launch_flip_weights(es, kernel, ws, groups, og, cg, taps, hs);
-        if (e != hipSuccess) return hip_fail(e, "weight flip launch");
-        for (int64_t g = 0; g < groups; ++g) {
-            ntg::GemmParams p;
-            std::memset(&p, 0, sizeof p);
-            p.M = (int)cg; p.K = (int)(og * taps); p.N = (int)HW; p.batch = (int)batch;
-            p.A = ws + g * cg * og * taps * es;
-            p.B = gy + g * og * L * es;
-            p.C = static_cast<char*>(d_image) + g * cg * HW * es;
-            p.lda = og * taps; p.ldb = HW; p.ldc = HW;
-            p.sA = 0; p.sB = out_channels * L; p.sC = channels * HW;
-            p.cmode = accumulate ? ntg::C_ACCUMULATE : ntg::C_OVERWRITE;
-            p.vecA_ok = (og * taps * es) % 16 == 0;
-            fill_conv_geom(p.conv, og, Ho, Wo, k_r, k_c, 1, 1, q_r, q_c, d_r, d_c, width);
-            e = ntg::launch_conv_mfma(dtype, false, p, hs);
-            if (e != hipSuccess) return hip_fail(e, "implicit conv_dimage launch");
-        }
+        rc = conv_dimage_gather(dtype, kernel, grad_out, d_image, ws, batch, channels, out_channels, geo, groups, accumulate, hs);
+        if (rc) return rc;
     }
     if (gather_dw) d_kernel = nullptr;    // done
     if (gather_dx) d_image = nullptr;
@@ -902,6 +966,12 @@ static Geo2 as_2d(int ndim, const int64_t* size, const int64_t* k, const int64_t
     return {size[0], size[1], k[0], k[1], s[0], s[1], p[0], p[1], d[0], d[1]};
 }
 
+static Geo3 geo_from(const ntg::UnfoldNdParams& u) {
+    Geo3 g{3, {1, 1, 1}, {1, 1, 1}, {1, 1, 1}, {0, 0, 0}, {1, 1, 1}, {1, 1, 1}};
+    for (int a = 0; a < 3; ++a) { g.sz[a] = u.size[a]; g.k[a] = u.k[a]; g.s[a] = u.s[a]; g.p[a] = u.p[a]; g.d[a] = u.d[a]; g.o[a] = u.out[a]; }
+    return g;
+}
+
 int ntg_unfoldnd_dev(int dtype, const void* image, void* col, int64_t batch, int64_t channels, int ndim, const int64_t* size,
                      const int64_t* kernel_size, const int64_t* stride, const int64_t* padding, const int64_t* dilation, void* stream) {
     const int64_t es = ntg::elem_size(dtype);
@@ -949,6 +1019,11 @@ int64_t ntg_convnd_workspace_bytes(int dtype, int64_t batch, int64_t channels, i
         return backward ? ntg_conv2d_backward_workspace_bytes(dtype, batch, channels, g.h, g.w, out_channels, g.kr, g.kc, g.sr, g.sc, g.pr, g.pc, g.dr, g.dc, groups)
                         : ntg_conv2d_forward_workspace_bytes(dtype, batch, channels, g.h, g.w, g.kr, g.kc, g.sr, g.sc, g.pr, g.pc, g.dr, g.dc);
     }
+    if (ndim == 3) {
+        const Geo3 g = geo_from(u);
+        if (backward) return plan_conv_backward_g(dtype, true, true, batch, channels, out_channels, g, groups).need;
+        if (conv_implicit_g(dtype, channels, g)) return 0;
+    }
     return u.total * es;
 }
 
@@ -969,6 +1044,11 @@ int ntg_convnd_dev(int dtype, const void* image, const void* kernel, void* out, 
     }
     if (batch == 0 || out_channels == 0) return NTG_OK;
     if (!image || !kernel || !out) return fail(NTG_ERR_INVALID_ARGUMENT, "null pointer");
+    if (ndim == 3) {
+        const Geo3 g = geo_from(u);
+        if (conv_implicit_g(dtype, channels, g))      // three axes, floating dtype: gathered inside the GEMM, no col buffer
+            return conv_forward_gather(dtype, image, kernel, out, batch, channels, out_channels, g, groups, static_cast<hipStream_t>(stream));
+    }
     const int64_t need = u.total * es;
     if (need > 0 && (!workspace || workspace_bytes < need))
         return fail(NTG_ERR_INVALID_ARGUMENT, "workspace of %lld bytes needed, %lld given", (long long)need, (long long)workspace_bytes);
@@ -1009,7 +1089,27 @@ int ntg_convnd_backward_dev(int dtype, const void* image, const void* kernel, co
     }
     if (batch == 0 || out_channels == 0 || channels == 0) return NTG_OK;
     if (!kernel || !grad_out || (d_kernel && !image)) return fail(NTG_ERR_INVALID_ARGUMENT, "null pointer");
-    const int64_t need = u.total * es;
+    int64_t need = u.total * es;
+    if (ndim == 3) {
+        const Geo3 g = geo_from(u);
+        const ConvBackwardPlan plan = plan_conv_backward_g(dtype, d_image != nullptr, d_kernel != nullptr, batch, channels, out_channels, g, groups);
+        need = plan.need;
+        if (need > 0 && (!workspace || workspace_bytes < need))
+            return fail(NTG_ERR_INVALID_ARGUMENT, "workspace of %lld bytes needed, %lld given", (long long)need, (long long)workspace_bytes);
+        if (plan.gather_dw) {
+            rc = conv_dkernel_gather(dtype, image, grad_out, d_kernel, workspace, batch, channels, out_channels, g, groups, accumulate,
+                                     static_cast<hipStream_t>(stream));
+            if (rc) return rc;
+            d_kernel = nullptr;
+        }
+        if (plan.gather_dx) {
+            rc = conv_dimage_gather(dtype, kernel, grad_out, d_image, workspace, batch, channels, out_channels, g, groups, accumulate,
+                                    static_cast<hipStream_t>(stream));
+            if (rc) return rc;
+            d_image = nullptr;
+        }
+        if (!d_kernel && !d_image) return NTG_OK;
+    }
     if (!workspace || workspace_bytes < need)
         return fail(NTG_ERR_INVALID_ARGUMENT, "workspace of %lld bytes needed, %lld given", (long long)need, (long long)workspace_bytes);
     const int64_t L = u.L, add = (channels / groups) * u.taps, og = out_channels / groups;
