@@ -247,7 +247,9 @@ int ntg_conv_transpose2d(int dtype, const void* input, const void* kernel, void*
  * size / kernel_size / stride / padding / dilation / output_padding point to `ndim` values, slowest axis first
  * (depth, rows, columns).  image [batch, channels, size...], kernel [out_channels, channels/groups, kernel_size...]
  * (transposed: [in_channels, out_channels/groups, kernel_size...]).  ndim 1 and 2 run on the conv2d entry points above;
- * ndim 3 and 4 unfold into the workspace like the reference.  `backward` selects the workspace of the gradient call. */
+ * ndim 3 gathers the unfolded operand inside the GEMM for the floating dtypes (workspace as for conv2d); ndim 4, the
+ * integer dtypes and kernels wider than 8 taps unfold into the workspace like the reference.  `backward` selects the
+ * workspace of the gradient call. */
 int ntg_unfoldnd_dev(int dtype, const void* image, void* col, int64_t batch, int64_t channels, int ndim, const int64_t* size,
                      const int64_t* kernel_size, const int64_t* stride, const int64_t* padding, const int64_t* dilation, void* stream);
 int ntg_unfoldnd_backward_dev(int dtype, const void* col, void* image, int64_t batch, int64_t channels, int ndim, const int64_t* size,
