@@ -81,7 +81,9 @@ def test_argument_errors_do_not_need_a_device():
     assert lib.ntg_conv_transpose2d(_lib.FLOAT32, p, p, p, 1, 3, 9, 7, 8, 3, 3, 2, 2, 0, 0, 1, 1, 1, 1, 2) == 1    # 3 % 2 groups
     # N-d geometry arrays
     arr = lambda *v: (ctypes.c_int64 * len(v))(*v)
-    assert lib.ntg_convnd_workspace_bytes(_lib.FLOAT32, 2, 3, 4, 3, arr(5, 6, 7), arr(2, 3, 2), arr(1, 2, 1), arr(1, 0, 2), arr(2, 1, 1), 1, 0) \
+    # three spatial axes: floats gather the operand inside the product, integers unfold [B, C*taps, L] first
+    assert lib.ntg_convnd_workspace_bytes(_lib.FLOAT32, 2, 3, 4, 3, arr(5, 6, 7), arr(2, 3, 2), arr(1, 2, 1), arr(1, 0, 2), arr(2, 1, 1), 1, 0) == 0
+    assert lib.ntg_convnd_workspace_bytes(_lib.INT32, 2, 3, 4, 3, arr(5, 6, 7), arr(2, 3, 2), arr(1, 2, 1), arr(1, 0, 2), arr(2, 1, 1), 1, 0) \
         == 2 * 3 * 12 * (5 * 2 * 10) * 4
     assert lib.ntg_convnd_workspace_bytes(_lib.FLOAT32, 2, 3, 4, 5, arr(5, 6, 7), arr(2, 3, 2), arr(1, 2, 1), arr(1, 0, 2), arr(2, 1, 1), 1, 0) == -1
     assert lib.ntg_convnd(_lib.FLOAT32, p, p, p, 1, 3, 4, 3, arr(5, 6, 7), arr(2, 3, 9), arr(1, 1, 1), arr(0, 0, 0), arr(1, 1, 1), 1) == 1
