@@ -120,19 +120,38 @@ SplitPlan plan_splitk(const ntg::GemmParams& p, int dtype, bool ta) {
         // only the DMA-fed kernel writes fp32 partial sums: 16-byte rows everywhere
         if (p.K % 8 || p.N % 8 || (ta && p.M % 8) || p.lda % 8 || p.ldb % 8 || p.lda >= (1 << 22) || p.ldb >= (1 << 22)) return none;
         if ((reinterpret_cast<uintptr_t>(p.A) & 15) || (reinterpret_cast<uintptr_t>(p.B) & 15)) return none;
+        // The DMA-fed kernel at its 128 x 128 tile (larger problems fill the chip by themselves).  Measured on MI355X:
+        // a workgroup alone on its CU takes about 0.215 us per 32-wide K-step, n >= 2 sharing a CU about 0.26 n us;
+        // launching the reduction and writing/reading the fp32 partial sums costs about 6 us + 8 S M N bytes at 4 TB/s.
+        // Pick the S with the smallest estimate (S = 1: no split).
+        if (ntg::gemm16_tile_edge(p.M, p.N, 1) != 128) return none;
+        const int64_t tiles = ((p.M + 127) / 128) * ((p.N + 127) / 128);
+        auto estimate_us = [&](int64_t sp) {
+            const int64_t per_cu = (tiles * sp + 255) / 256;
+            const double step = per_cu == 1 ? 0.215 : 0.26 * (double)per_cu;
+            const double second_pass = sp == 1 ? 0.0 : 6.0 + 8.0 * (double)sp * (double)p.M * (double)p.N / 4.0e6;
+            return (double)(p.K / sp / 32) * step + second_pass;
+        };
+        int64_t best = 1;
+        double best_us = estimate_us(1);
+        for (int64_t sp = 2; sp <= 16; ++sp) {
+            if (p.K % (sp * 32) != 0 || p.K / sp < 256) continue;
+            const double us = estimate_us(sp);
+            if (us < 0.9 * best_us) { best = sp; best_us = us; }      // a split must win clearly
+        }
+        if (best == 1) return none;
+        return SplitPlan{(int)best, p.K / best, best * (int64_t)p.M * p.N * 4};
     }
-    // workgroups the kernels want in flight: one 256 x 256 tile per CU for the 16-bit kernel (its LDS ring fills the CU),
-    // two 128 x 128 (or more 64 x 64) tiles per CU for fp32 / fp64
-    const int64_t tile = half ? 256 : ((p.M <= 64 || p.N <= 64) ? 64 : 128), kstep = dtype == ntg::DT_F64 ? 16 : 32;
-    const int64_t target = half ? 256 : 512;
+    // fp32 / fp64: two 128 x 128 (or more 64 x 64) tiles per CU wanted in flight
+    const int64_t tile = (p.M <= 64 || p.N <= 64) ? 64 : 128, kstep = dtype == ntg::DT_F64 ? 16 : 32;
+    const int64_t target = 512;
     const int64_t tiles = ((p.M + tile - 1) / tile) * ((p.N + tile - 1) / tile);
     if (2 * tiles > target) return none;
     int64_t smax = target / tiles;
     if (smax > 16) smax = 16;
     for (int64_t sp = smax; sp >= 2; --sp) {
         if (p.K % (sp * kstep) != 0 || p.K / sp < 512) continue;   // short k ranges do not pay for the second pass
-        if (half && tiles * sp < 48) return none;                             // too small for the DMA-fed kernel anyway
-        return SplitPlan{(int)sp, p.K / sp, sp * (int64_t)p.M * p.N * (half ? 4 : es)};
+        return SplitPlan{(int)sp, p.K / sp, sp * (int64_t)p.M * p.N * es};
     }
     return none;
 }

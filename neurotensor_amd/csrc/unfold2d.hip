@@ -110,19 +110,73 @@ __global__ void __launch_bounds__(256) splitk_reduce_kernel(const P* __restrict_
     }
 }
 
+// The same sum, four consecutive columns per thread with 16-byte accesses to the partial sums (rows of C and of the
+// partial matrices must start on a multiple of four elements); the partial loads of four k ranges are in flight together.
+template <class T, class P, class Acc>
+__global__ void __launch_bounds__(256) splitk_reduce_vec_kernel(const P* __restrict__ part, const int splits, const GemmParams p) {
+    typedef T TV __attribute__((ext_vector_type(4)));
+    typedef P PV __attribute__((ext_vector_type(4)));
+    const int64_t nq = p.N / 4, total = (int64_t)p.M * p.N, quads = (int64_t)p.M * nq;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    T* C = static_cast<T*>(p.C);
+    const T* bias = static_cast<const T*>(p.bias);
+    for (int64_t q = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; q < quads; q += stride) {
+        const int64_t m = q / nq, n = (q - m * nq) * 4;
+        TV* cp = reinterpret_cast<TV*>(C + m * p.ldc + n);
+        Acc acc[4] = {(Acc)0, (Acc)0, (Acc)0, (Acc)0};
+        if (p.cmode == C_ACCUMULATE) {
+            const TV c0 = *cp;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) acc[e] = (Acc)c0[e];
+        } else if (p.cmode == C_BIAS) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) acc[e] = (Acc)bias[m * p.bias_rs + (n + e) * p.bias_cs];
+        }
+        const P* pp = part + q * 4;
+        int s = 0;
+        for (; s + 4 <= splits; s += 4) {
+            PV v[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) v[u] = *reinterpret_cast<const PV*>(pp + (int64_t)(s + u) * total);
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) acc[e] += (Acc)v[u][e];
+        }
+        for (; s < splits; ++s) {
+            const PV v = *reinterpret_cast<const PV*>(pp + (int64_t)s * total);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) acc[e] += (Acc)v[e];
+        }
+        TV o;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) o[e] = (T)acc[e];
+        *cp = o;
+    }
+}
+
+template <class T, class P, class Acc>
+static void launch_splitk_reduce_t(const void* part, int splits, const GemmParams& p, hipStream_t s) {
+    const int64_t total = (int64_t)p.M * p.N;
+    const bool vec = p.N % 4 == 0 && p.ldc % 4 == 0 && (reinterpret_cast<uintptr_t>(p.C) % (4 * sizeof(T))) == 0 &&
+                     (reinterpret_cast<uintptr_t>(part) % (4 * sizeof(P))) == 0;
+    if (vec) hipLaunchKernelGGL((splitk_reduce_vec_kernel<T, P, Acc>), dim3(grid_for(total / 4)), dim3(256), 0, s, (const P*)part, splits, p);
+    else hipLaunchKernelGGL((splitk_reduce_kernel<T, P, Acc>), dim3(grid_for(total)), dim3(256), 0, s, (const P*)part, splits, p);
+}
+
 hipError_t launch_splitk_reduce(int dtype, const void* part, int splits, const GemmParams& p, hipStream_t s) {
     const int64_t total = (int64_t)p.M * p.N;
     if (total == 0) return hipSuccess;
-    const dim3 g(grid_for(total)), b(256);
     switch (dtype) {
-    case DT_F32: hipLaunchKernelGGL((splitk_reduce_kernel<float, float, float>), g, b, 0, s, (const float*)part, splits, p); break;
-    case DT_F64: hipLaunchKernelGGL((splitk_reduce_kernel<double, double, double>), g, b, 0, s, (const double*)part, splits, p); break;
-    case DT_F16: hipLaunchKernelGGL((splitk_reduce_kernel<_Float16, float, float>), g, b, 0, s, (const float*)part, splits, p); break;
-    case DT_BF16: hipLaunchKernelGGL((splitk_reduce_kernel<__bf16, float, float>), g, b, 0, s, (const float*)part, splits, p); break;
+    case DT_F32: launch_splitk_reduce_t<float, float, float>(part, splits, p, s); break;
+    case DT_F64: launch_splitk_reduce_t<double, double, double>(part, splits, p, s); break;
+    case DT_F16: launch_splitk_reduce_t<_Float16, float, float>(part, splits, p, s); break;
+    case DT_BF16: launch_splitk_reduce_t<__bf16, float, float>(part, splits, p, s); break;
     default: return hipErrorInvalidValue;
     }
     return hipGetLastError();
 }
+
 
 // wt[g][c][oc][t] = w[g*og + oc][c][taps-1-t]: the kernel with input/output channels swapped
 // inside each group and both tap axes reversed, i.e. the weights of the convolution that maps

@@ -308,11 +308,14 @@ def test_config3_4096_cube(dtype, scale):
 
 
 @pytest.mark.parametrize("dtype", ["bf16", np.float16], ids=["bf16", "fp16"])
-@pytest.mark.parametrize("shape", [(2056, 1000, 2312), (1800, 1016, 3080), (2304, 992, 1928), (3000, 40, 2056), (2056, 8, 2056)],
+@pytest.mark.parametrize("shape", [(2056, 1000, 2312), (1800, 1016, 3080), (2304, 992, 1928), (3000, 40, 2056), (2056, 8, 2056),
+                                   (3080, 1016, 3336), (4104, 40, 2056), (1024, 512, 1536), (128, 96, 128), (136, 72, 8)],
                          ids=lambda s: "x".join(map(str, s)))
 def test_ragged_16bit_dma_kernel(dtype, shape):
-    """M, N, K that are not multiples of the 256 x 256 x 32 tile (but keep 16-byte rows) stay on the
-    DMA-fed kernel: edge rows/columns, the k tail (8, 24, none, 8-only) and all three C modes."""
+    """M, N, K that are not multiples of the tile (but keep 16-byte rows) stay on the DMA-fed kernel: edge
+    rows/columns, the k tail (8, 24, none, 8-only) and all three C modes.  Up to 128 tiles of 256 x 256 the kernel
+    runs with 128 x 128 tiles (the first five shapes, ragged; the last three, two of them aligned), above that
+    with 256 x 256 tiles (3080 x 3336 and 4104 x 2056: 182 and 153 large tiles)."""
     m, k, n = shape
     bf = dtype == "bf16"
     rng = np.random.default_rng(1100 + k)
@@ -431,7 +434,7 @@ def test_split_k_medium_rows(dtype):
     half = bf or dtype == np.float16
     rng = np.random.default_rng(1900)
     lib = _lib.load()
-    for (m, k, n) in [(256, 4096, 2048), (520, 2048, 1032), (64, 8192, 1024), (1024, 3072, 1024)]:
+    for (m, k, n) in [(256, 4096, 2048), (520, 4096, 1032), (64, 8192, 1024), (1024, 6144, 1024)]:
         for ta, tb in TRANS:
             a = randn(rng, (m, k), dtype, 0.25)
             b = randn(rng, (k, n), dtype, 0.25)
