@@ -156,7 +156,7 @@ def main():
                                "C += A.B (BASELINE config 3)", "m": N, "k": N, "n": N, "c_mode": "accumulate"},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_TFLOPS["bf16"], "unit": "TFLOP/s",
                      "frac": round(achieved / PEAK_TFLOPS["bf16"], 4), "traffic": read_traffic_note(),
-                     "kernel": "ntg::gemm16_kernel<BFloat16, NN>", "launch_ms": round(ev_ms, 5)},
+                     "kernel": "ntg::gemm_ring_kernel<BFloat16, NN>", "launch_ms": round(ev_ms, 5)},
     }
 
     # ---------------- extras: the other dtypes and configurations ----------------

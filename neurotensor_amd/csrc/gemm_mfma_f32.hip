@@ -1,8 +1,23 @@
-// Float32 instantiations of the MFMA GEMM (v_mfma_f32_32x32x2_f32).
-#include "gemm_mfma_impl.h"
+// Float32 instantiations of the MFMA GEMMs (v_mfma_f32_32x32x2_f32): the DMA-fed LDS ring for 16-byte aligned rows,
+// the register-staged kernel for everything else and for the gathering convolutions.
+#include "gemm_ring_impl.h"
 namespace ntg {
+// Tile edge of the DMA-fed kernel for Float32 (64 or 128).  The 32x32x2 MFMA is slow enough that LDS traffic never
+// binds, so the tile only decides how evenly the work spreads: a CU's time is the number of tiles it is handed
+// times the tile's MFMA time; 64 x 64 tiles balance four times finer and lose about 7 % to their single
+// accumulator block per wavefront.
+static int ring_f32_tile_edge(const GemmParams& p) {
+    const int64_t t128 = (int64_t)((p.M + 127) / 128) * ((p.N + 127) / 128) * p.batch;
+    const int64_t t64 = (int64_t)((p.M + 63) / 64) * ((p.N + 63) / 64) * p.batch;
+    const double cost128 = (double)((t128 + 255) / 256), cost64 = 1.07 * 0.25 * (double)((t64 + 255) / 256);
+    return cost64 < cost128 ? 64 : 128;
+}
+
 hipError_t launch_gemm_mfma_f32(bool ta, bool tb, const GemmParams& p, hipStream_t s) {
-    // 128 x 128 x 32 tiles unless that leaves most of the 256 CUs idle; then 64 x 64 x 32
+    if (ring_eligible(p, ta, 4))
+        return ring_f32_tile_edge(p) == 64 ? launch_ring_wb<DT_F32, 1>(ta, tb, p, s) : launch_ring_wb<DT_F32, 2>(ta, tb, p, s);
+    // rows that are not 16-byte aligned (or pointer tables): register-staged kernel, 128 x 128 x 32 tiles unless that
+    // leaves most of the 256 CUs idle; then 64 x 64 x 32
     const int64_t big_tiles = (int64_t)((p.M + 127) / 128) * ((p.N + 127) / 128) * p.batch;
     if (big_tiles >= 192 && p.M > 64 && p.N > 64) return launch_trans<DT_F32, 2, 2, 32>(ta, tb, p, s);   // a 128-wide tile would be half empty
     return launch_trans<DT_F32, 1, 1, 32>(ta, tb, p, s);

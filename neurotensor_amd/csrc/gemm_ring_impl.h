@@ -1,35 +1,41 @@
-// 16-bit (Float16 / BFloat16) MFMA GEMM for gfx950, fast path:
+// DMA-fed MFMA GEMM for gfx950 (Float16, BFloat16, Float32), the fast path:
 //   C[M,N] (+)= op(A) . op(B),  16-byte aligned rows (leading dimensions and contiguous extents
-//   multiples of 8 elements); M, N, K need not be multiples of the tile (the
-//   RAGGED instantiation clamps DMA source addresses, zeroes the k tail in registers and
+//   multiples of one 16-byte chunk: 8 or 4 elements); M, N, K need not be multiples of the tile
+//   (the RAGGED instantiation clamps DMA source addresses, zeroes the k tail in registers and
 //   guards the stores).  Everything else goes through the general kernel in gemm_mfma_impl.h.
 //
 // Shape of the kernel
-//   * 256 x 256 tile of C per workgroup, 4 wavefronts (2 x 2), each owning 128 x 128 =
-//     4 x 4 blocks of v_mfma_f32_32x32x16_{f16,bf16}; 256 accumulator registers per lane.
-//     A second instantiation (WB = 2) has 128 x 128 tiles, 64 x 64 per wavefront, half the
-//     LDS and two workgroups per CU: problems of up to 128 large tiles run on it, so that
-//     mid-sized products still put a workgroup on every CU.  The numbers below are the large
-//     tile's; the small one halves the per-operand tile, DMA and read counts.
-//   * K advances in steps of 32 through a 4-deep ring of LDS stages (4 x 32 KiB).  Global
+//   * One workgroup = 4 wavefronts (2 x 2), each owning WB x WB blocks of 32 x 32:
+//       WB = 4: 256 x 256 tile, 256 accumulator registers per lane, one workgroup per CU (16-bit, large products);
+//       WB = 2: 128 x 128 tile, half the LDS, two workgroups per CU (16-bit up to 128 large tiles, so that
+//               mid-sized products still put a workgroup on every CU; Float32);
+//       WB = 1: 64 x 64 tile (Float32 when that spreads the work more evenly over the 256 CUs).
+//     The numbers below are the large tile's; the smaller ones scale the per-operand tile, DMA and read counts.
+//   * 16-bit: v_mfma_f32_32x32x16_{f16,bf16} on 16-byte fragments (8 k per lane).  Float32: the same 16-byte
+//     fragment holds 4 k, element e feeding the e-th of four v_mfma_f32_32x32x2_f32 -- all byte geometry (tiles,
+//     stages, DMA instructions, K-major reads) is shared; a K-step is 64 bytes of k per row (32 or 16 elements).
+//   * K advances through a 4-deep ring of LDS stages (4 x 32 KiB).  Global
 //     memory is copied straight into LDS (global_load_lds_dwordx4): no staging registers,
 //     three to four K-steps of loads in flight while one is being multiplied.  One barrier
-//     per K-step, placed between its two k16 halves; the DMA instructions and the LDS
+//     per K-step, placed between its two halves; the DMA instructions and the LDS
 //     fragment reads are slotted between the MFMAs one at a time, so neither the CU's single
 //     address unit nor LDS latency ever holds up the matrix pipe.
 //   * LDS layouts are conflict free for the reads the MFMA operands need:
-//       operand stored K-contiguous  -> [row][32 k] (64 B rows), 16-byte slot kv stored at
+//       operand stored K-contiguous  -> [row][64 B of k], 16-byte slot kv stored at
 //                                        kv ^ ((row >> 1) & 3); one ds_read_b128 per block;
-//       operand stored MN-contiguous -> [k][256 mn] (512 B rows), 16-byte chunk c stored at
+//       operand stored MN-contiguous -> [k][tile edge], 16-bit: 16-byte chunk c stored at
 //                                        c ^ (2 * (k & 3)); ds_read_b64_tr_b16 turns four k-rows
 //                                        into "4 consecutive k per lane", i.e. the transpose
-//                                        is done by the LDS read, never in memory.
+//                                        is done by the LDS read, never in memory;
+//                                        Float32: chunk c at c ^ (8 * ((k >> 2) & 1)), one
+//                                        ds_read_b32 per block and k (32 consecutive floats per
+//                                        half-wavefront, the halves in different bank halves).
 //     Because the DMA writes 64 consecutive 16-byte slots per instruction, the swizzle is
 //     applied by choosing which global chunk each lane fetches.
 //   * The MFMA is issued with the operands swapped (B fragment first), so a lane holds four
 //     consecutive columns of one row of C; the epilogue stages 32-row slabs through LDS in
 //     fp32 and touches C with 16-byte accesses only (C0 is added in fp32 before the single
-//     rounding to the 16-bit type).
+//     rounding to a 16-bit type).
 #pragma once
 #include "gemm_mfma_impl.h"
 
@@ -55,30 +61,36 @@ template <> struct Cvt16<DT_BF16> {
 };
 
 // WB = 32 x 32 blocks per wavefront along each of m and n: 4 -> 256 x 256 tile, 2 -> 128 x 128 tile
-template <int WB>
-struct G16 {
-    static constexpr int BM = 64 * WB, BN = 64 * WB, BK = 32, NST = 4;
+// ES = bytes per element (2: Float16 / BFloat16, 4: Float32).  A K-step is 64 bytes of k for every row (32 or 16
+// elements), so the byte geometry of tiles, stages and DMA instructions is the same for both element sizes.
+template <int WB, int ES>
+struct RingGeom {
+    static constexpr int BM = 64 * WB, BN = 64 * WB, BK = 64 / ES, NST = 4;
+    static constexpr int VEL = 16 / ES;                  // elements per 16-byte chunk
     static constexpr int WT = 32 * WB;                   // edge of a wavefront's share of the tile
-    static constexpr int TILE_BYTES = BM * BK * 2;       // one operand tile, 16 / 8 KiB
+    static constexpr int TILE_BYTES = BM * 64;           // one operand tile, 16 / 8 KiB
     static constexpr int STAGE_BYTES = 2 * TILE_BYTES;   // 32 / 16 KiB
-    static constexpr int MN_ROW_BYTES = BM * 2;          // one k-row of an MN-contiguous operand tile
-    static constexpr int CHUNKS = BM / 8;                // 16-byte chunks in such a row
+    static constexpr int MN_ROW_BYTES = BM * ES;         // one k-row of an MN-contiguous operand tile
+    static constexpr int CHUNKS = MN_ROW_BYTES / 16;     // 16-byte chunks in such a row (16 .. 64)
+    static constexpr int ROWS_PER_DMA = 64 / CHUNKS;     // k-rows of such a tile that one DMA instruction fills (1 .. 4)
 };
 
 // Per-lane BYTE offsets (relative to the tile's first element at K-step 0) of this wavefront's
 // WB DMA instructions into one operand tile.  Instruction j = WB*wave + jj fills LDS bytes
 // [1024 j, 1024 j + 1024) of the tile:
 //   K-contiguous operand: rows 16 j + lane/4, 16-byte slot lane%4 holds kv = slot ^ ((row>>1)&3)
-//   MN-contiguous operand (CH = 8 WB chunks per k-row): k-rows (64/CH) j + lane/CH, slot lane%CH
-//                          holds chunk = slot ^ (2*(krow&3))
-// With RAGGED, mn_valid (1..BM rows/columns of the tile that exist) and k_valid (8..32 k of
-// the K-step that exist, a multiple of 8) clamp the SOURCE address into the matrix: lanes
+//   MN-contiguous operand (CH chunks per k-row): k-rows (64/CH) j + lane/CH, slot lane%CH holds
+//                          chunk = slot ^ (2*(krow&3)) for 16-bit elements (what the transposing
+//                          reads need), slot ^ (8*((krow>>2)&1)) for Float32 (the two k-rows that one
+//                          ds_read_b32 touches land in different halves of the 64 banks)
+// With RAGGED, mn_valid (1..BM rows/columns of the tile that exist) and k_valid (k of the
+// K-step that exist, a multiple of one chunk) clamp the SOURCE address into the matrix: lanes
 // whose data does not exist fetch a neighbouring chunk instead.  Rows/columns past the edge
 // only ever reach accumulators that the epilogue does not store; k past the end is zeroed
 // in the fragment registers before it is multiplied.
-template <bool KC, bool RAGGED, int WB>
+template <bool KC, bool RAGGED, int WB, int ES>
 __device__ __forceinline__ void dma_offsets(uint32_t (&off)[WB], int64_t ld, int wave, int lane, int mn_valid, int k_valid) {
-    constexpr int CH = G16<WB>::CHUNKS;
+    constexpr int CH = RingGeom<WB, ES>::CHUNKS, VEL = RingGeom<WB, ES>::VEL;
 #pragma unroll
     for (int jj = 0; jj < WB; ++jj) {
         const int j = wave * WB + jj;
@@ -87,17 +99,17 @@ __device__ __forceinline__ void dma_offsets(uint32_t (&off)[WB], int64_t ld, int
             int kv = (lane & 3) ^ ((row >> 1) & 3);
             if constexpr (RAGGED) {
                 row = row < mn_valid ? row : mn_valid - 1;
-                kv = kv < (k_valid >> 3) ? kv : (k_valid >> 3) - 1;
+                kv = kv < k_valid / VEL ? kv : k_valid / VEL - 1;
             }
-            off[jj] = (uint32_t)(((int64_t)row * ld + kv * 8) * 2);
+            off[jj] = (uint32_t)(((int64_t)row * ld + kv * VEL) * ES);
         } else {
             int krow = (64 / CH) * j + lane / CH;
-            int chunk = (lane % CH) ^ (2 * (krow & 3));
+            int chunk = (lane % CH) ^ (ES == 2 ? 2 * (krow & 3) : 8 * ((krow >> 2) & 1));
             if constexpr (RAGGED) {
                 krow = krow < k_valid ? krow : k_valid - 1;
-                chunk = chunk < (mn_valid >> 3) ? chunk : (mn_valid >> 3) - 1;
+                chunk = chunk < mn_valid / VEL ? chunk : mn_valid / VEL - 1;
             }
-            off[jj] = (uint32_t)(((int64_t)krow * ld + chunk * 8) * 2);
+            off[jj] = (uint32_t)(((int64_t)krow * ld + chunk * VEL) * ES);
         }
     }
 }
@@ -123,10 +135,11 @@ __device__ __forceinline__ uint32_t lds_addr_of(const char* p) {
 }
 
 template <int DT, bool TA, bool TB, bool RAGGED, int WB>
-__global__ void __launch_bounds__(256) gemm16_kernel(const GemmParams p) {
+__global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
     using E = Elem<DT>;
     using T = typename E::T;
-    using G = G16<WB>;
+    constexpr int ES = sizeof(T);
+    using G = RingGeom<WB, ES>;
     constexpr bool A_KC = !TA, B_KC = TB;
     constexpr int BK = G::BK;
     constexpr int WT = G::WT;
@@ -156,19 +169,19 @@ __global__ void __launch_bounds__(256) gemm16_kernel(const GemmParams p) {
     const int wave_u = __builtin_amdgcn_readfirstlane(wave);
     const int KT = (p.K + BK - 1) / BK;
     const int last = KT - 1;
-    const int kr = p.K - last * BK;                                  // k that exist in the last K-step (8..32)
+    const int kr = p.K - last * BK;                                  // k that exist in the last K-step (a multiple of one chunk)
     const int mvalid = p.M - m0 < G::BM ? p.M - m0 : G::BM;
     const int nvalid = p.N - n0 < G::BN ? p.N - n0 : G::BN;
     uint32_t offA[WB], offB[WB];      // K-steps before the last
     uint32_t offAt[WB], offBt[WB];    // the last K-step (RAGGED: k clamped to what exists)
-    dma_offsets<A_KC, RAGGED, WB>(offA, p.lda, wave, lane, mvalid, BK);
-    dma_offsets<B_KC, RAGGED, WB>(offB, p.ldb, wave, lane, nvalid, BK);
-    dma_offsets<A_KC, RAGGED, WB>(offAt, p.lda, wave, lane, mvalid, kr);
-    dma_offsets<B_KC, RAGGED, WB>(offBt, p.ldb, wave, lane, nvalid, kr);
-    const char* baseA = reinterpret_cast<const char*>(A) + (A_KC ? (int64_t)m0 * p.lda : (int64_t)m0) * 2;
-    const char* baseB = reinterpret_cast<const char*>(B) + (B_KC ? (int64_t)n0 * p.ldb : (int64_t)n0) * 2;
-    const int64_t advA = (A_KC ? (int64_t)BK : (int64_t)BK * p.lda) * 2;
-    const int64_t advB = (B_KC ? (int64_t)BK : (int64_t)BK * p.ldb) * 2;
+    dma_offsets<A_KC, RAGGED, WB, ES>(offA, p.lda, wave, lane, mvalid, BK);
+    dma_offsets<B_KC, RAGGED, WB, ES>(offB, p.ldb, wave, lane, nvalid, BK);
+    dma_offsets<A_KC, RAGGED, WB, ES>(offAt, p.lda, wave, lane, mvalid, kr);
+    dma_offsets<B_KC, RAGGED, WB, ES>(offBt, p.ldb, wave, lane, nvalid, kr);
+    const char* baseA = reinterpret_cast<const char*>(A) + (A_KC ? (int64_t)m0 * p.lda : (int64_t)m0) * ES;
+    const char* baseB = reinterpret_cast<const char*>(B) + (B_KC ? (int64_t)n0 * p.ldb : (int64_t)n0) * ES;
+    const int64_t advA = (A_KC ? (int64_t)BK : (int64_t)BK * p.lda) * ES;
+    const int64_t advB = (B_KC ? (int64_t)BK : (int64_t)BK * p.ldb) * ES;
     // uniform (scalar) source pointer of one operand tile
     auto tile_src = [&](const char* base) -> const void* {
         const uint64_t bu = reinterpret_cast<uint64_t>(base);
@@ -177,9 +190,14 @@ __global__ void __launch_bounds__(256) gemm16_kernel(const GemmParams p) {
         return reinterpret_cast<const void*>(((uint64_t)hi << 32) | lo);
     };
 
-    // ---- per-lane LDS read offsets (bytes inside an operand tile), for k16-step ks ----
+    // ---- per-lane LDS read offsets (bytes inside an operand tile), for half-step ks (0, 1) of a K-step ----
+    // A lane's fragment of one block is 16 bytes of k: lanes 0..31 hold the first 16 bytes of the half-step of
+    // their row, lanes 32..63 the second (8 + 8 consecutive k of 16-bit elements for one 32x32x16 MFMA; 4 + 4 of
+    // Float32, element e of both halves feeding the e-th of four 32x32x2 MFMAs -- the order of k inside a half-step
+    // is the same permutation for A and B).
     // K-major: block b of the wavefront, row = wbase + 32 b + lane%32, slot (2 ks + lane/32) ^ ((row>>1)&3)
-    // MN-major: two transposing reads per block; see the header comment
+    // MN-major, 16-bit: two transposing reads per block; see the header comment
+    // MN-major, Float32: four ds_read_b32 per block, element e from k-row 8 ks + 4 (lane/32) + e
     auto frag_off_km = [&](int wbase, int blk, int ks) -> int {
         const int row = wbase + blk * 32 + (lane & 31);
         const int slot = (2 * ks + (lane >> 5)) ^ ((lane >> 1) & 3);
@@ -192,13 +210,20 @@ __global__ void __launch_bounds__(256) gemm16_kernel(const GemmParams p) {
         const int chunk = (mnl >> 3) ^ (2 * e);
         return krow * G::MN_ROW_BYTES + chunk * 16 + (mnl & 7) * 2;
     };
+    auto frag_off_mm32 = [&](int wbase, int blk, int ks, int e) -> int {
+        const int krow = 8 * ks + 4 * (lane >> 5) + e;
+        const int mnl = wbase + blk * 32 + (lane & 31);
+        return krow * G::MN_ROW_BYTES + ((mnl * 4) ^ (128 * (lane >> 5)));      // (krow >> 2) & 1 == lane / 32
+    };
 
     // One LDS read instruction of an operand's fragment set for k16-step ks.  A K-major
     // operand takes WB reads (one ds_read_b128 per block), an MN-major one 2 WB (two transposing
-    // 8-byte reads per block); read r lands in frag[r / per_block] (half r % per_block).
+    // 8-byte reads per block; Float32: 4 WB four-byte reads); read r lands in frag[r / per_block].
     auto read_op = [&](u32x4 (&frag)[WB], const char* tile, bool kc, int wbase, int ks, int r) {
         if (kc) {
             frag[r] = *reinterpret_cast<const u32x4*>(tile + frag_off_km(wbase, r, ks));
+        } else if constexpr (ES == 4) {
+            frag[r >> 2][r & 3] = *reinterpret_cast<const uint32_t*>(tile + frag_off_mm32(wbase, r >> 2, ks, r & 3));
         } else {
             const int blk = r >> 1, half = r & 1;
             const shortx4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
@@ -209,8 +234,10 @@ __global__ void __launch_bounds__(256) gemm16_kernel(const GemmParams p) {
             frag[blk][2 * half + 1] = w[1];
         }
     };
-    constexpr int NRA = A_KC ? WB : 2 * WB, NRB = B_KC ? WB : 2 * WB, NR = NRA + NRB;
-    constexpr int NMMA = WB * WB;                        // MFMAs per k16-step
+    constexpr int MNR = ES == 2 ? 2 * WB : 4 * WB;       // reads of an MN-major operand per half-step
+    constexpr int NRA = A_KC ? WB : MNR, NRB = B_KC ? WB : MNR, NR = NRA + NRB;
+    constexpr int MPP = ES == 2 ? 1 : 4;                 // MFMAs per pair of fragments
+    constexpr int NMMA = WB * WB * MPP;                  // MFMAs per half-step
     constexpr int RPM = (NR + NMMA - 1) / NMMA;          // LDS reads slotted behind each MFMA
 
     floatx16 acc[WB][WB];
@@ -253,21 +280,29 @@ __global__ void __launch_bounds__(256) gemm16_kernel(const GemmParams p) {
     // behind the CU's one address unit and stall their MFMA streams.
     auto mma_step_prefetch = [&](int cur_buf, const char* stage, int ks, int nxt_buf,
                                  const void* src, const uint32_t (&off_main)[WB], const uint32_t (&off_tail)[WB], bool tail_tile,
-                                 uint32_t lds_tile) {
+                                 uint32_t lds_tile) __attribute__((always_inline)) {
         uint32_t off[WB];
 #pragma unroll
         for (int x = 0; x < WB; ++x) off[x] = (RAGGED && tail_tile) ? off_tail[x] : off_main[x];
 #pragma unroll
         for (int q = 0; q < NMMA; ++q) {
             // serpentine order: consecutive MFMAs always share one operand fragment
-            const int i = q / WB, j = (i & 1) ? WB - 1 - (q % WB) : (q % WB);
-            E::mma(acc[i][j], bf[cur_buf][j], af[cur_buf][i]);   // D rows <-> n, cols <-> m
+            const int e = q / (WB * WB), pr = q % (WB * WB);
+            const int i = pr / WB, j = (i & 1) ? WB - 1 - (pr % WB) : (pr % WB);
+            if constexpr (ES == 2) {
+                E::mma(acc[i][j], bf[cur_buf][j], af[cur_buf][i]);   // D rows <-> n, cols <-> m
+            } else {
+                // (copies first: __builtin_bit_cast applied to a vector-element lvalue reads element 0)
+                const uint32_t bu = bf[cur_buf][j][e], au = af[cur_buf][i][e];
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(__builtin_bit_cast(float, bu), __builtin_bit_cast(float, au), acc[i][j], 0, 0, 0);
+            }
 #pragma unroll
             for (int r = q * RPM; r < (q + 1) * RPM; ++r) {
                 if (r < NRA) read_op(af[nxt_buf], stage, A_KC, wm * WT, ks, r);
                 else if (r < NR) read_op(bf[nxt_buf], stage + G::TILE_BYTES, B_KC, wn * WT, ks, r - NRA);
             }
-            if (q % WB == WB - 1) dma_1k(src, off[q / WB], lds_tile + (uint32_t)(wave_u * WB + q / WB) * 1024u);
+            constexpr int DGAP = NMMA / WB;                      // MFMAs between two DMA instructions
+            if (q % DGAP == DGAP - 1) dma_1k(src, off[q / DGAP], lds_tile + (uint32_t)(wave_u * WB + q / DGAP) * 1024u);
         }
 #pragma unroll
         for (int q = 0; q < NMMA; ++q) {
@@ -291,10 +326,11 @@ __global__ void __launch_bounds__(256) gemm16_kernel(const GemmParams p) {
     // second k16-step, its B half during the first k16-step of the next K-step.  Tile kt+1,
     // first touched in the second half, has had three K-steps to arrive.
     // RAGGED: zero the k >= K part of a fragment set of the last K-step.  Every lane's fragment
-    // covers 8 consecutive k starting at 16 ks + 8 (lane / 32) in both LDS layouts, and K is a
-    // multiple of 8, so a lane's fragment is either entirely real or entirely past the end.
+    // covers one chunk of consecutive k (8 or 4) starting at (BK/2) ks + (BK/4) (lane / 32) in both
+    // LDS layouts, and K is a multiple of the chunk, so a lane's fragment is either entirely real or
+    // entirely past the end.
     auto mask_tail = [&](int buf, int ks) {
-        const bool ok = 16 * ks + 8 * (lane >> 5) < kr;
+        const bool ok = (BK / 2) * ks + (BK / 4) * (lane >> 5) < kr;
 #pragma unroll
         for (int i = 0; i < WB; ++i)
 #pragma unroll
@@ -304,7 +340,8 @@ __global__ void __launch_bounds__(256) gemm16_kernel(const GemmParams p) {
             }
     };
 
-    auto iteration = [&](int kt, char* cur, const char* nxt, char* prv) {
+    // (inlined by force: as a call, the stage pointers would arrive in vector registers and could not feed M0)
+    auto iteration = [&](int kt, char* cur, const char* nxt, char* prv) __attribute__((always_inline)) {
         if (RAGGED && kt == last && kr < BK) mask_tail(0, 0);
         mma_step_prefetch(0, cur, 1, 1, srcB(kt + 3), offB, offBt, kt + 3 >= last, lds_addr_of(prv) + G::TILE_BYTES);
         // outstanding now: tiles kt+1, kt+2, kt+3 (2 WB instructions each): wait for the oldest
@@ -333,22 +370,27 @@ __global__ void __launch_bounds__(256) gemm16_kernel(const GemmParams p) {
     // read-back moves RPS rows.
     constexpr int SROW = WT * 4, LPR = WT / 8, RPS = 64 / LPR, NSTEP = 32 / RPS;
     char* slab = ((wave & 2) ? st1 : st0) + (wave & 1) * (32 * SROW);
-    uint16_t* Cu = reinterpret_cast<uint16_t*>(C);
+    char* Cb = reinterpret_cast<char*>(C);
     const int col = 8 * (lane % LPR);              // this lane's 8 consecutive columns in the slab
     const int n = n0 + wn * WT + col;
+    constexpr int NV = ES / 2;                     // 16-byte vectors of C per lane and row: 8 columns of 2 or 4 bytes
     auto epilogue = [&](auto cmode_tag) {
         constexpr int CM = decltype(cmode_tag)::value;
-        const uint16_t* bias = static_cast<const uint16_t*>(p.bias);
+        const T* bias = static_cast<const T*>(p.bias);
 #pragma unroll
         for (int i = 0; i < WB; ++i) {
             // C0 of the whole slab is requested before the LDS round trip
-            u32x4 c0[NSTEP];
+            u32x4 c0[NSTEP][NV];
             if constexpr (CM == C_ACCUMULATE) {
 #pragma unroll
                 for (int t = 0; t < NSTEP; ++t) {
                     const int m = m0 + wm * WT + 32 * i + RPS * t + lane / LPR;
-                    if (!RAGGED || (m < p.M && n < p.N)) c0[t] = *reinterpret_cast<const u32x4*>(Cu + (int64_t)m * p.ldc + n);
-                    else c0[t] = u32x4{0u, 0u, 0u, 0u};
+#pragma unroll
+                    for (int v = 0; v < NV; ++v) {
+                        if (!RAGGED || (m < p.M && n + 4 * v < p.N))
+                            c0[t][v] = *reinterpret_cast<const u32x4*>(Cb + ((int64_t)m * p.ldc + n) * ES + 16 * v);
+                        else c0[t][v] = u32x4{0u, 0u, 0u, 0u};
+                    }
                 }
             }
             // lane holds rows m = 32 i + lane%32, cols 32 j + 8 rq + 4 (lane/32) + (0..3)
@@ -369,27 +411,39 @@ __global__ void __launch_bounds__(256) gemm16_kernel(const GemmParams p) {
                 const floatx4v hi = *reinterpret_cast<const floatx4v*>(slab + row * SROW + (((sl + 1) ^ (row & 7)) * 16));
                 float v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
                 const int m = m0 + wm * WT + 32 * i + row;
-                if (RAGGED && (m >= p.M || n >= p.N)) continue;     // N % 8 == 0: a lane's 8 columns exist or not together
+                // 16-bit: N % 8 == 0, a lane's 8 columns exist or not together; Float32: N % 4 == 0, the halves separately
+                if (RAGGED && (m >= p.M || n >= p.N)) continue;
+                const bool hi_ok = !RAGGED || ES == 2 || n + 4 < p.N;
                 if constexpr (CM == C_PARTIAL) {
                     // split-K: the fp32 sums of this k range go to a float matrix; rounding happens after the reduction
                     float* wp = static_cast<float*>(p.C) + (int64_t)b * p.sC + (int64_t)m * p.ldc + n;
                     *reinterpret_cast<floatx4v*>(wp) = lo;
-                    *reinterpret_cast<floatx4v*>(wp + 4) = hi;
+                    if (hi_ok) *reinterpret_cast<floatx4v*>(wp + 4) = hi;
                     continue;
                 }
                 if constexpr (CM == C_ACCUMULATE) {
 #pragma unroll
-                    for (int e = 0; e < 8; ++e) v[e] += Cvt16<DT>::up((uint16_t)(c0[t][e >> 1] >> (16 * (e & 1))));
+                    for (int e = 0; e < 8; ++e) {
+                        if constexpr (ES == 2) v[e] += Cvt16<DT>::up((uint16_t)(c0[t][0][e >> 1] >> (16 * (e & 1))));
+                        else { const uint32_t cu = c0[t][e >> 2][e & 3]; v[e] += __builtin_bit_cast(float, cu); }
+                    }
                 } else if constexpr (CM == C_BIAS) {
 #pragma unroll
                     for (int e = 0; e < 8; ++e)
-                        v[e] += Cvt16<DT>::up(bias[(int64_t)b * p.bias_bs + (int64_t)m * p.bias_rs + (int64_t)(n + e) * p.bias_cs]);
+                        if (ES == 2 || e < 4 || hi_ok)
+                            v[e] += (float)bias[(int64_t)b * p.bias_bs + (int64_t)m * p.bias_rs + (int64_t)(n + e) * p.bias_cs];
                 }
-                u32x4 o;
+                char* cp = Cb + ((int64_t)m * p.ldc + n) * ES;
+                if constexpr (ES == 2) {
+                    u32x4 o;
 #pragma unroll
-                for (int e = 0; e < 4; ++e)
-                    o[e] = (uint32_t)Cvt16<DT>::down(v[2 * e]) | ((uint32_t)Cvt16<DT>::down(v[2 * e + 1]) << 16);
-                *reinterpret_cast<u32x4*>(Cu + (int64_t)m * p.ldc + n) = o;
+                    for (int e = 0; e < 4; ++e)
+                        o[e] = (uint32_t)Cvt16<DT>::down(v[2 * e]) | ((uint32_t)Cvt16<DT>::down(v[2 * e + 1]) << 16);
+                    *reinterpret_cast<u32x4*>(cp) = o;
+                } else {
+                    *reinterpret_cast<floatx4v*>(cp) = floatx4v{v[0], v[1], v[2], v[3]};
+                    if (hi_ok) *reinterpret_cast<floatx4v*>(cp + 16) = floatx4v{v[4], v[5], v[6], v[7]};
+                }
             }
         }
     };
@@ -400,41 +454,44 @@ __global__ void __launch_bounds__(256) gemm16_kernel(const GemmParams p) {
 }
 
 // true when the fast kernel can serve the problem: 16-byte aligned rows everywhere (leading
-// dimensions, batch strides, base pointers) and every contiguous extent a multiple of 8
-// elements.  M, N and K themselves may be ragged with respect to the tile.
-static inline bool gemm16_eligible(const GemmParams& p, bool ta) {
-    return p.K >= 8 && p.K % 8 == 0 && p.N % 8 == 0 && (!ta || p.M % 8 == 0) &&
+// dimensions, batch strides, base pointers) and every contiguous extent a multiple of one 16-byte
+// chunk (es = element size: 8 or 4 elements).  M, N and K themselves may be ragged with respect
+// to the tile.  Per-lane DMA offsets are 32-bit: 256 rows of lda elements must stay below 4 GiB.
+static inline bool ring_eligible(const GemmParams& p, bool ta, int es = 2) {
+    const int vel = 16 / es;
+    const int64_t ldmax = es == 2 ? (1 << 22) : (1 << 21);
+    return p.K >= vel && p.K % vel == 0 && p.N % vel == 0 && (!ta || p.M % vel == 0) &&
            !p.Aptr && !p.Bptr && !p.Cptr && p.vecA_ok && p.vecB_ok &&
-           p.ldc % 8 == 0 && p.sC % 8 == 0 && p.lda < (1 << 22) && p.ldb < (1 << 22) &&
+           p.ldc % vel == 0 && p.sC % vel == 0 && p.lda < ldmax && p.ldb < ldmax &&
            ((reinterpret_cast<uintptr_t>(p.A) & 15) == 0) && ((reinterpret_cast<uintptr_t>(p.B) & 15) == 0) &&
            ((reinterpret_cast<uintptr_t>(p.C) & 15) == 0);
 }
 
 template <int DT, bool TA, bool TB, int WB>
-static hipError_t launch_gemm16_cfg(const GemmParams& pin, hipStream_t s) {
-    constexpr int TE = G16<WB>::BM;
+static hipError_t launch_ring_cfg(const GemmParams& pin, hipStream_t s) {
+    constexpr int TE = RingGeom<WB, (int)sizeof(typename Elem<DT>::T)>::BM, BK = RingGeom<WB, (int)sizeof(typename Elem<DT>::T)>::BK;
     GemmParams p = pin;
     p.tiles_m = (p.M + TE - 1) / TE;
     p.tiles_n = (p.N + TE - 1) / TE;
     const int64_t blocks = (int64_t)p.tiles_m * p.tiles_n * p.batch;
     if (blocks > 0x7fffffffLL) return hipErrorInvalidValue;
-    if (p.M % TE == 0 && p.N % TE == 0 && p.K % 32 == 0)
-        hipLaunchKernelGGL((gemm16_kernel<DT, TA, TB, false, WB>), dim3((unsigned)blocks), dim3(256), 0, s, p);
+    if (p.M % TE == 0 && p.N % TE == 0 && p.K % BK == 0)
+        hipLaunchKernelGGL((gemm_ring_kernel<DT, TA, TB, false, WB>), dim3((unsigned)blocks), dim3(256), 0, s, p);
     else
-        hipLaunchKernelGGL((gemm16_kernel<DT, TA, TB, true, WB>), dim3((unsigned)blocks), dim3(256), 0, s, p);
+        hipLaunchKernelGGL((gemm_ring_kernel<DT, TA, TB, true, WB>), dim3((unsigned)blocks), dim3(256), 0, s, p);
     return hipGetLastError();
 }
 
 template <int DT, int WB>
-static hipError_t launch_gemm16_wb(bool ta, bool tb, const GemmParams& p, hipStream_t s) {
-    if (ta) return tb ? launch_gemm16_cfg<DT, true, true, WB>(p, s) : launch_gemm16_cfg<DT, true, false, WB>(p, s);
-    return tb ? launch_gemm16_cfg<DT, false, true, WB>(p, s) : launch_gemm16_cfg<DT, false, false, WB>(p, s);
+static hipError_t launch_ring_wb(bool ta, bool tb, const GemmParams& p, hipStream_t s) {
+    if (ta) return tb ? launch_ring_cfg<DT, true, true, WB>(p, s) : launch_ring_cfg<DT, true, false, WB>(p, s);
+    return tb ? launch_ring_cfg<DT, false, true, WB>(p, s) : launch_ring_cfg<DT, false, false, WB>(p, s);
 }
 
 template <int DT>
-static hipError_t launch_gemm16(bool ta, bool tb, const GemmParams& p, hipStream_t s) {
-    if (gemm16_tile_edge(p.M, p.N, p.batch) == 256) return launch_gemm16_wb<DT, 4>(ta, tb, p, s);
-    return launch_gemm16_wb<DT, 2>(ta, tb, p, s);
+static hipError_t launch_ring16(bool ta, bool tb, const GemmParams& p, hipStream_t s) {
+    if (ring16_tile_edge(p.M, p.N, p.batch) == 256) return launch_ring_wb<DT, 4>(ta, tb, p, s);
+    return launch_ring_wb<DT, 2>(ta, tb, p, s);
 }
 
 }  // namespace ntg

@@ -70,7 +70,7 @@ struct GemmParams {
 // Tile edge the DMA-fed 16-bit kernel uses for M x N x batch: 256 x 256 tiles need about half the LDS traffic per
 // flop, but the 256 CUs idle below one tile each; four times as many 128 x 128 workgroups (two fit on a CU) are
 // quicker up to 128 large tiles.
-static inline int gemm16_tile_edge(int64_t M, int64_t N, int64_t batch) {
+static inline int ring16_tile_edge(int64_t M, int64_t N, int64_t batch) {
     const int64_t t256 = ((M + 255) / 256) * ((N + 255) / 256) * batch;
     return t256 > 128 ? 256 : 128;
 }

@@ -124,7 +124,7 @@ SplitPlan plan_splitk(const ntg::GemmParams& p, int dtype, bool ta) {
         // a workgroup alone on its CU takes about 0.215 us per 32-wide K-step, n >= 2 sharing a CU about 0.26 n us;
         // launching the reduction and writing/reading the fp32 partial sums costs about 6 us + 8 S M N bytes at 4 TB/s.
         // Pick the S with the smallest estimate (S = 1: no split).
-        if (ntg::gemm16_tile_edge(p.M, p.N, 1) != 128) return none;
+        if (ntg::ring16_tile_edge(p.M, p.N, 1) != 128) return none;
         const int64_t tiles = ((p.M + 127) / 128) * ((p.N + 127) / 128);
         auto estimate_us = [&](int64_t sp) {
             const int64_t per_cu = (tiles * sp + 255) / 256;
@@ -142,11 +142,13 @@ SplitPlan plan_splitk(const ntg::GemmParams& p, int dtype, bool ta) {
         if (best == 1) return none;
         return SplitPlan{(int)best, p.K / best, best * (int64_t)p.M * p.N * 4};
     }
-    // fp32 / fp64: two 128 x 128 (or more 64 x 64) tiles per CU wanted in flight
-    const int64_t tile = (p.M <= 64 || p.N <= 64) ? 64 : 128, kstep = dtype == ntg::DT_F64 ? 16 : 32;
+    // fp64: two 128 x 128 (or more 64 x 64) tiles per CU wanted in flight; fp32 (whose kernel goes down to 64 x 64
+    // tiles by itself) only when those leave CUs without any tile
+    const bool f32 = dtype == ntg::DT_F32;
+    const int64_t tile = (f32 || p.M <= 64 || p.N <= 64) ? 64 : 128, kstep = f32 ? 32 : 16;
     const int64_t target = 512;
     const int64_t tiles = ((p.M + tile - 1) / tile) * ((p.N + tile - 1) / tile);
-    if (2 * tiles > target) return none;
+    if ((f32 ? 1 : 2) * tiles > (f32 ? 255 : target)) return none;
     int64_t smax = target / tiles;
     if (smax > 16) smax = 16;
     for (int64_t sp = smax; sp >= 2; --sp) {

@@ -434,7 +434,7 @@ def test_split_k_medium_rows(dtype):
     half = bf or dtype == np.float16
     rng = np.random.default_rng(1900)
     lib = _lib.load()
-    for (m, k, n) in [(256, 4096, 2048), (520, 4096, 1032), (64, 8192, 1024), (1024, 6144, 1024)]:
+    for (m, k, n) in [(256, 4096, 2048), (520, 4096, 1032), (64, 8192, 1024), (768, 6144, 1024)]:
         for ta, tb in TRANS:
             a = randn(rng, (m, k), dtype, 0.25)
             b = randn(rng, (k, n), dtype, 0.25)
