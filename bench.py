@@ -49,7 +49,7 @@ def parse_args():
 def read_traffic_note():
     """HBM bytes per launch of the headline kernel, measured offline with rocprofv3 --pmc
     (FETCH_SIZE / WRITE_SIZE, scaled by a copy kernel); None until that profile exists."""
-    path = os.path.join(ROOT, "profiles", "gemm16_bf16_4096_hbm_traffic.txt")
+    path = os.path.join(ROOT, "profiles", "gemm_ring_bf16_4096_hbm_traffic.txt")
     try:
         for line in open(path):
             if line.startswith("hbm_traffic_bytes_per_launch:"):
