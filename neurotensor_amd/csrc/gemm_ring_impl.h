@@ -124,6 +124,15 @@ __device__ __forceinline__ void dma_1k(const void* base, uint32_t off, uint32_t 
                  :: "s"(lds_addr), "v"(off), "s"(base) : "memory");
 }
 
+// One gathering DMA instruction: 64 lanes x 4 bytes, every lane from its own address, to LDS bytes
+// [lds_addr, lds_addr + 256).
+__device__ __forceinline__ void dma_dword(const void* addr, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off"
+                 :: "s"(lds_addr), "v"(addr) : "memory");
+}
+// what the padding taps of a gathered convolution operand read
+static __device__ const uint32_t ring_zero_word[4] = {0u, 0u, 0u, 0u};
+
 template <int WB>
 __device__ __forceinline__ void dma_tile(const void* sbase, const uint32_t (&off)[WB], uint32_t lds_tile, int wave_u) {
 #pragma unroll
@@ -134,15 +143,27 @@ __device__ __forceinline__ uint32_t lds_addr_of(const char* p) {
     return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const char*)p;
 }
 
-template <int DT, bool TA, bool TB, bool RAGGED, int WB>
+// CONV = 0: plain product.  CONV = 1 / 2 (Float32, two spatial axes): op(B) is the never-stored im2col matrix col[kk][l]
+// of the image at p.B (1: convolution, C[o][l]; 2: its transpose col^T[l][kk], the weight gradient C[o][kk]), described by
+// p.conv.  Its LDS tile is [k-row][BN floats]; one DMA instruction gathers 64 consecutive columns of one k-row, the
+// address being a wave-uniform term of the k-row plus a per-lane term of the column that is fixed for the whole K loop
+// (convolution: the tap (c, r, q) is uniform, the pixel per lane; weight gradient: the other way round).  Padding taps
+// and columns / k-rows past the edge read a zero word instead, so the tile in LDS is exact and the multiply loop is the
+// plain one.  Wavefront w gathers k-rows 4 w .. 4 w + 3 of every K-step.
+template <int DT, bool TA, bool TB, bool RAGGED, int WB, int CONV = 0>
 __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
     using E = Elem<DT>;
     using T = typename E::T;
     constexpr int ES = sizeof(T);
     using G = RingGeom<WB, ES>;
-    constexpr bool A_KC = !TA, B_KC = TB;
+    constexpr bool A_KC = !TA, B_KC = CONV ? false : TB;
     constexpr int BK = G::BK;
     constexpr int WT = G::WT;
+    static_assert(CONV == 0 || (ES == 4 && !TA && RAGGED), "gathered operands: Float32, A stored [m][k], guarded edges");
+    constexpr int NA = WB, NB = CONV ? 4 * WB : WB;      // DMA instructions per wavefront and K-step for the A / B tile
+    // B instructions issued in the first / second half-step (the second also carries the A tile's).  Splitting a gathered
+    // tile between the two was measured slower than issuing all of it in the first.
+    constexpr int NB1 = NB, NB2 = NB - NB1;
 
     __shared__ __attribute__((aligned(1024))) char st0[G::STAGE_BYTES];
     __shared__ __attribute__((aligned(1024))) char st1[G::STAGE_BYTES];
@@ -182,6 +203,107 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
     const char* baseB = reinterpret_cast<const char*>(B) + (B_KC ? (int64_t)n0 * p.ldb : (int64_t)n0) * ES;
     const int64_t advA = (A_KC ? (int64_t)BK : (int64_t)BK * p.lda) * ES;
     const int64_t advB = (B_KC ? (int64_t)BK : (int64_t)BK * p.ldb) * ES;
+    // ---- gathered operand: per-lane constants of this lane's WB columns (64 h + lane) of the tile ----
+    //   convolution:      lanepart = byte offset of the output pixel's window origin without padding, cmask = one bit per
+    //                     tap row (bits 0..7) and tap column (bits 8..15) that falls inside the image; 0 past the edge
+    //   weight gradient:  lanepart = byte offset of the tap inside the image slice, cmask = r*d_r | q*d_c << 16,
+    //                     0x80008000 (never inside) past the edge
+    uint32_t lanepart[WB], cmask[WB];
+    if constexpr (CONV != 0) {
+        const ConvGeom& g = p.conv;
+#pragma unroll
+        for (int h = 0; h < WB; ++h) {
+            const int n = n0 + 64 * h + lane;
+            if constexpr (CONV == 1) {
+                const uint32_t l = n < p.N ? (uint32_t)n : 0u;
+                const uint32_t oh = fast_div(l, g.div_wo), ow = l - oh * (uint32_t)g.Wo;
+                const int ih0 = (int)oh * g.s_r - g.p_r, iw0 = (int)ow * g.s_c - g.p_c;
+                uint32_t m = 0;
+#pragma unroll
+                for (int t = 0; t < 8; ++t) {
+                    if (t < g.k_r && (unsigned)(ih0 + t * g.d_r) < (unsigned)g.H) m |= 1u << t;
+                    if (t < g.k_c && (unsigned)(iw0 + t * g.d_c) < (unsigned)g.W) m |= 256u << t;
+                }
+                cmask[h] = n < p.N ? m : 0u;
+                lanepart[h] = (oh * (uint32_t)g.s_r * (uint32_t)g.W + ow * (uint32_t)g.s_c) * 4u;
+            } else {
+                const uint32_t kk = n < p.N ? (uint32_t)n : 0u;
+                const uint32_t c = fast_div(kk, g.div_krc), rem = kk - c * (uint32_t)g.k_rc;
+                const uint32_t r = fast_div(rem, g.div_kc), q = rem - r * (uint32_t)g.k_c;
+                cmask[h] = n < p.N ? (r * (uint32_t)g.d_r) | ((q * (uint32_t)g.d_c) << 16) : 0x80008000u;
+                lanepart[h] = (c * (uint32_t)g.chan + r * (uint32_t)g.d_r * (uint32_t)g.W + q * (uint32_t)g.d_c) * 4u;
+            }
+        }
+    }
+    // Wave-uniform state of the four k-rows (4 wave + i) this wavefront gathers, kept in scalar registers and advanced
+    // by one K-step (16 k) after each use, so the loop body holds no division: a k-row index is the mixed-radix number
+    // (hi, mid, lo) = (c, r, q) with radices (k_r, k_c) for the convolution, (-, oh, ow) with radix Wo for the weight
+    // gradient; adding 16 = (d_hi, d_mid, d_lo) needs one carry per digit.  st_up is the byte offset that the digits
+    // contribute (padding included, so it may be negative).
+    int st_lo[4], st_mid[4], st_up[4], st_k[4];
+    int cv_r0 = 1, cv_r1 = 1, cv_dlo = 0, cv_dmid = 0, cv_dup = 0, cv_carry_lo = 0, cv_carry_mid = 0;
+    if constexpr (CONV != 0) {
+        const ConvGeom& g = p.conv;
+        const int s_lo = (CONV == 1 ? g.d_c : g.s_c) * 4, s_mid = (CONV == 1 ? g.d_r : g.s_r) * g.W * 4, s_hi = g.chan * 4;
+        cv_r0 = CONV == 1 ? g.k_c : g.Wo;
+        cv_r1 = CONV == 1 ? g.k_r : 0x7fffffff;
+        const FastDiv& dv0 = CONV == 1 ? g.div_kc : g.div_wo;
+        const uint32_t t16 = fast_div((uint32_t)BK, dv0);
+        cv_dlo = BK - (int)t16 * cv_r0;
+        const uint32_t h16 = CONV == 1 ? t16 / (uint32_t)cv_r1 : 0u;
+        cv_dmid = (int)t16 - (int)h16 * (CONV == 1 ? cv_r1 : 0);
+        cv_dup = (int)h16 * s_hi + cv_dmid * s_mid + cv_dlo * s_lo;
+        cv_carry_lo = s_mid - cv_r0 * s_lo;
+        cv_carry_mid = CONV == 1 ? s_hi - cv_r1 * s_mid : 0;
+        const int base0 = -(g.p_r * g.W + g.p_c) * 4;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const uint32_t idx = (uint32_t)(4 * wave_u + i);
+            const uint32_t t = fast_div(idx, dv0);
+            st_lo[i] = (int)(idx - t * (uint32_t)cv_r0);
+            const uint32_t hi = CONV == 1 ? t / (uint32_t)cv_r1 : 0u;
+            st_mid[i] = (int)t - (int)hi * (CONV == 1 ? cv_r1 : 0);
+            st_up[i] = base0 + (int)hi * s_hi + st_mid[i] * s_mid + st_lo[i] * s_lo;
+            st_k[i] = (int)idx;
+        }
+    }
+    // Instruction x (0 .. 4 WB - 1) of this wavefront's share of the NEXT gathered tile (tiles are gathered in K order):
+    // k-row 4 wave + x / WB, columns 64 (x % WB) .. + 63; the k-row's state moves on after its last instruction.
+    auto conv_dma = [&](int x, uint32_t lds_tile) __attribute__((always_inline)) {
+        if constexpr (CONV != 0) {
+            const ConvGeom& g = p.conv;
+            const int i = x / WB, h = x % WB;
+            const int krow = 4 * wave_u + i;
+            const char* img = reinterpret_cast<const char*>(B);
+            const bool krow_ok = st_k[i] < p.K;                    // uniform
+            bool ok;
+            if constexpr (CONV == 1) {
+                const uint32_t sr = krow_ok ? (uint32_t)st_mid[i] : 31u, sq = 8u + (uint32_t)st_lo[i];
+                ok = ((cmask[h] >> sr) & (cmask[h] >> sq) & 1u) != 0u;
+            } else {
+                const int ih0 = krow_ok ? st_mid[i] * g.s_r - g.p_r : -(1 << 20), iw0 = st_lo[i] * g.s_c - g.p_c;
+                ok = ((uint32_t)(ih0 + (int)(cmask[h] & 0xffffu)) < (uint32_t)g.H) & ((uint32_t)(iw0 + (int)(cmask[h] >> 16)) < (uint32_t)g.W);
+            }
+            const char* src = ok ? img + (int64_t)st_up[i] + lanepart[h] : reinterpret_cast<const char*>(ring_zero_word);
+            dma_dword(src, lds_tile + (uint32_t)(krow * G::MN_ROW_BYTES + h * 256));
+            if (h == WB - 1) {
+                int lo = st_lo[i] + cv_dlo, mid = st_mid[i] + cv_dmid, up = st_up[i] + cv_dup;
+                const bool c0 = lo >= cv_r0;
+                lo = c0 ? lo - cv_r0 : lo;
+                mid = c0 ? mid + 1 : mid;
+                up = c0 ? up + cv_carry_lo : up;
+                const bool c1 = mid >= cv_r1;
+                mid = c1 ? mid - cv_r1 : mid;
+                up = c1 ? up + cv_carry_mid : up;
+                st_lo[i] = lo; st_mid[i] = mid; st_up[i] = up; st_k[i] += BK;
+            }
+        }
+    };
+    auto conv_tile = [&](uint32_t lds_tile) __attribute__((always_inline)) {
+#pragma unroll
+        for (int x = 0; x < 4 * WB; ++x) conv_dma(x, lds_tile);
+    };
+
     // uniform (scalar) source pointer of one operand tile
     auto tile_src = [&](const char* base) -> const void* {
         const uint64_t bu = reinterpret_cast<uint64_t>(base);
@@ -213,6 +335,7 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
     auto frag_off_mm32 = [&](int wbase, int blk, int ks, int e) -> int {
         const int krow = 8 * ks + 4 * (lane >> 5) + e;
         const int mnl = wbase + blk * 32 + (lane & 31);
+        if constexpr (CONV != 0) return krow * G::MN_ROW_BYTES + mnl * 4;          // gathered tiles are stored unswizzled
         return krow * G::MN_ROW_BYTES + ((mnl * 4) ^ (128 * (lane >> 5)));      // (krow >> 2) & 1 == lane / 32
     };
 
@@ -254,13 +377,17 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
     auto srcA = [&](int kt) { return tile_src(baseA + (int64_t)(kt < last ? kt : last) * advA); };
     auto srcB = [&](int kt) { return tile_src(baseB + (int64_t)(kt < last ? kt : last) * advB); };
 
-    // prologue: tiles 0..2 and the A half of tile 3 in flight (7 WB instructions)
+    // prologue: tiles 0..2 and the A half of tile 3 in flight (3 (NA + NB) + NA instructions)
+    auto b_tile = [&](int kt, uint32_t lds_tile) __attribute__((always_inline)) {
+        if constexpr (CONV != 0) conv_tile(lds_tile);      // (tiles past the last one are all zeros; nobody reads them)
+        else dma_tile<WB>(srcB(kt), kt >= last ? offBt : offB, lds_tile, wave_u);
+    };
     dma_tile<WB>(srcA(0), 0 >= last ? offAt : offA, lds_addr_of(st0), wave_u);
-    dma_tile<WB>(srcB(0), 0 >= last ? offBt : offB, lds_addr_of(st0) + G::TILE_BYTES, wave_u);
+    b_tile(0, lds_addr_of(st0) + G::TILE_BYTES);
     dma_tile<WB>(srcA(1), 1 >= last ? offAt : offA, lds_addr_of(st1), wave_u);
-    dma_tile<WB>(srcB(1), 1 >= last ? offBt : offB, lds_addr_of(st1) + G::TILE_BYTES, wave_u);
+    b_tile(1, lds_addr_of(st1) + G::TILE_BYTES);
     dma_tile<WB>(srcA(2), 2 >= last ? offAt : offA, lds_addr_of(st2), wave_u);
-    dma_tile<WB>(srcB(2), 2 >= last ? offBt : offB, lds_addr_of(st2) + G::TILE_BYTES, wave_u);
+    b_tile(2, lds_addr_of(st2) + G::TILE_BYTES);
     dma_tile<WB>(srcA(3), 3 >= last ? offAt : offA, lds_addr_of(st3), wave_u);
 
     u32x4 af[2][WB], bf[2][WB];   // fragment double buffer: [k16-step parity][block]
@@ -278,12 +405,9 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
     // instructions (one operand tile's share of this wavefront) are spread over the step as
     // well -- issued in a burst right after the barrier, the four wavefronts would queue up
     // behind the CU's one address unit and stall their MFMA streams.
-    auto mma_step_prefetch = [&](int cur_buf, const char* stage, int ks, int nxt_buf,
-                                 const void* src, const uint32_t (&off_main)[WB], const uint32_t (&off_tail)[WB], bool tail_tile,
-                                 uint32_t lds_tile) __attribute__((always_inline)) {
-        uint32_t off[WB];
-#pragma unroll
-        for (int x = 0; x < WB; ++x) off[x] = (RAGGED && tail_tile) ? off_tail[x] : off_main[x];
+    // `issue(x)` emits DMA instruction x of the NDMA that this step carries.
+    auto mma_step_prefetch = [&](int cur_buf, const char* stage, int ks, int nxt_buf, auto ndma_tag, auto ngather_tag, auto&& issue) __attribute__((always_inline)) {
+        constexpr int NDMA = decltype(ndma_tag)::value, NGATHER = decltype(ngather_tag)::value;
 #pragma unroll
         for (int q = 0; q < NMMA; ++q) {
             // serpentine order: consecutive MFMAs always share one operand fragment
@@ -301,8 +425,12 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
                 if (r < NRA) read_op(af[nxt_buf], stage, A_KC, wm * WT, ks, r);
                 else if (r < NR) read_op(bf[nxt_buf], stage + G::TILE_BYTES, B_KC, wn * WT, ks, r - NRA);
             }
-            constexpr int DGAP = NMMA / WB;                      // MFMAs between two DMA instructions
-            if (q % DGAP == DGAP - 1) dma_1k(src, off[q / DGAP], lds_tile + (uint32_t)(wave_u * WB + q / DGAP) * 1024u);
+            constexpr int DGAP = NMMA >= NDMA ? NMMA / NDMA : 1, DPER = NMMA >= NDMA ? 1 : NDMA / NMMA;   // MFMAs between two DMA instructions / DMA instructions per MFMA
+            if (q % DGAP == DGAP - 1) {
+#pragma unroll
+                for (int x = 0; x < DPER; ++x)
+                    if ((q / DGAP) * DPER + x < NDMA) issue((q / DGAP) * DPER + x);
+            }
         }
 #pragma unroll
         for (int q = 0; q < NMMA; ++q) {
@@ -310,11 +438,16 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
             const int nrd = NR - q * RPM < RPM ? NR - q * RPM : RPM;
             if (nrd == 2) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0); // its LDS reads
             else if (nrd == 1) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            if constexpr (NGATHER > 0) {
+                // the gather's address arithmetic, dealt out evenly: what does not fit under one MFMA delays the next
+                __builtin_amdgcn_sched_group_barrier(0x002, (8 * NGATHER + NMMA - 1) / NMMA + 1, 0);   // VALU
+                __builtin_amdgcn_sched_group_barrier(0x004, (10 * NGATHER + NMMA - 1) / NMMA, 0);      // SALU
+            }
         }
     };
 
     // tile 0 must have landed before its first fragments are read
-    NTG_WAIT_VMCNT(5 * WB);
+    NTG_WAIT_VMCNT(2 * (NA + NB) + NA);
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
     load_frags(st0, 0, 0);
@@ -343,15 +476,34 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
     // (inlined by force: as a call, the stage pointers would arrive in vector registers and could not feed M0)
     auto iteration = [&](int kt, char* cur, const char* nxt, char* prv) __attribute__((always_inline)) {
         if (RAGGED && kt == last && kr < BK) mask_tail(0, 0);
-        mma_step_prefetch(0, cur, 1, 1, srcB(kt + 3), offB, offBt, kt + 3 >= last, lds_addr_of(prv) + G::TILE_BYTES);
-        // outstanding now: tiles kt+1, kt+2, kt+3 (2 WB instructions each): wait for the oldest
-        NTG_WAIT_VMCNT(4 * WB);
+        {
+            const void* src = nullptr;
+            if constexpr (CONV == 0) src = srcB(kt + 3);
+            const bool tail = kt + 3 >= last;
+            const uint32_t lds_tile = lds_addr_of(prv) + G::TILE_BYTES;
+            mma_step_prefetch(0, cur, 1, 1, std::integral_constant<int, NB1>{}, std::integral_constant<int, (CONV ? NB1 : 0)>{},
+                              [&](int x) __attribute__((always_inline)) {
+                if constexpr (CONV != 0) conv_dma(x, lds_tile);
+                else dma_1k(src, (RAGGED && tail) ? offBt[x] : offB[x], lds_tile + (uint32_t)(wave_u * WB + x) * 1024u);
+            });
+        }
+        // issued since the last instruction of tile kt+1: A(kt+2), B(kt+2), A(kt+3) and the first NB1 of B(kt+3)
+        NTG_WAIT_VMCNT(2 * (NA + NB) - NB2);
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // my reads of `cur` are complete
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
         if (RAGGED && kt == last && kr < BK) mask_tail(1, 1);
         // (the last K-step prefetches fragments from a stage holding a clamped tile; unused)
-        mma_step_prefetch(1, nxt, 0, 0, srcA(kt + 4), offA, offAt, kt + 4 >= last, lds_addr_of(cur));
+        {
+            const void* src = srcA(kt + 4);
+            const bool tail = kt + 4 >= last;
+            const uint32_t lds_tile = lds_addr_of(cur), lds_gather = lds_addr_of(prv) + G::TILE_BYTES;
+            mma_step_prefetch(1, nxt, 0, 0, std::integral_constant<int, NB2 + NA>{}, std::integral_constant<int, NB2>{},
+                              [&](int x) __attribute__((always_inline)) {
+                if (x < NB2) conv_dma(NB1 + x, lds_gather);       // rest of B(kt+3)
+                else dma_1k(src, (RAGGED && tail) ? offAt[x - NB2] : offA[x - NB2], lds_tile + (uint32_t)(wave_u * WB + x - NB2) * 1024u);
+            });
+        }
     };
 
     for (int kt = 0; kt < KT; kt += 4) {
@@ -479,6 +631,21 @@ static hipError_t launch_ring_cfg(const GemmParams& pin, hipStream_t s) {
         hipLaunchKernelGGL((gemm_ring_kernel<DT, TA, TB, false, WB>), dim3((unsigned)blocks), dim3(256), 0, s, p);
     else
         hipLaunchKernelGGL((gemm_ring_kernel<DT, TA, TB, true, WB>), dim3((unsigned)blocks), dim3(256), 0, s, p);
+    return hipGetLastError();
+}
+
+// convolution (tb = false) or weight gradient (tb = true) with op(B) gathered from the image; Float32, two spatial axes
+template <int WB>
+static hipError_t launch_ring_conv_cfg(bool tb, const GemmParams& pin, hipStream_t s) {
+    constexpr int TE = RingGeom<WB, 4>::BM;
+    GemmParams p = pin;
+    p.tiles_m = (p.M + TE - 1) / TE;
+    p.tiles_n = (p.N + TE - 1) / TE;
+    const int64_t blocks = (int64_t)p.tiles_m * p.tiles_n * p.batch;
+    if (blocks <= 0) return hipSuccess;
+    if (blocks > 0x7fffffffLL) return hipErrorInvalidValue;
+    if (tb) hipLaunchKernelGGL((gemm_ring_kernel<DT_F32, false, false, true, WB, 2>), dim3((unsigned)blocks), dim3(256), 0, s, p);
+    else hipLaunchKernelGGL((gemm_ring_kernel<DT_F32, false, false, true, WB, 1>), dim3((unsigned)blocks), dim3(256), 0, s, p);
     return hipGetLastError();
 }
 
