@@ -347,6 +347,39 @@ def test_ragged_16bit_dma_kernel(dtype, shape):
     assert ((y.float() - refy).abs().max() / refy.abs().max()).item() <= HALF_REL
 
 
+@pytest.mark.parametrize("shape", [(1860, 260, 1860), (2052, 1000, 2308), (1028, 132, 516), (68, 20, 4), (132, 16, 260)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_ragged_fp32_ring_kernel(shape):
+    """Float32 with 16-byte rows (sizes multiples of 4) stays on the DMA-fed kernel: 1860 x 1860 runs on 128 x 128 tiles,
+    the others on 64 x 64; edge rows / columns, a last 16-byte chunk of C of which only the first half exists
+    (n % 8 == 4), k tails of 4, 8, 4 and none, all three C modes, nothing written outside [m, n]."""
+    m, k, n = shape
+    rng = np.random.default_rng(1300 + k)
+    for ta, tb in TRANS:
+        a = randn(rng, (m, k), np.float32)
+        b = randn(rng, (k, n), np.float32)
+        sa = np.ascontiguousarray(a.T) if ta else a
+        sb = np.ascontiguousarray(b.T) if tb else b
+        ta_, tb_ = to_torch(sa, DEV, False), to_torch(sb, DEV, False)
+        ref = torch.matmul(to_torch(a, DEV, False).double(), to_torch(b, DEV, False).double())
+        tol = 1e-5 * k * float(np.abs(a).max() * np.abs(b).max())
+        guard = torch.full((m + 2, n), 7.0, device=DEV)
+        c = guard[1:m + 1]
+        c.zero_()
+        out = F.matmult(ta_, tb_, c, ta, tb, accumulate=False)
+        assert (out.double() - ref).abs().max().item() <= tol, (shape, ta, tb)
+        assert torch.all(guard[0] == 7.0) and torch.all(guard[m + 1] == 7.0)
+        F.matmult(ta_, tb_, c, ta, tb)                                   # accumulate: 2 * A.B
+        assert (c.double() - 2 * ref).abs().max().item() <= 2 * tol
+        assert torch.all(guard[0] == 7.0) and torch.all(guard[m + 1] == 7.0)
+        rows = np.r_[0:4, m - 4:m]
+        cols = np.r_[0:4, n - 4:n]
+        _sampled_oracle_check(sa, sb, F.matmult(ta_, tb_, None, ta, tb), ta, tb, np.float32, rows, cols, k)
+    bias = randn(rng, (n,), np.float32)
+    y = F.linear(to_torch(a, DEV, False), to_torch(b, DEV, False), to_torch(bias, DEV, False))
+    assert (y.double() - (ref + to_torch(bias, DEV, False).double())).abs().max().item() <= tol
+
+
 @pytest.mark.parametrize("dtype", ["bf16", np.float32, np.int32], ids=["bf16", "fp32", "int32"])
 def test_operands_beyond_2_31_elements(dtype):
     """A holds more than 2^31 elements (4.4 - 9.6 GB): every row offset in the loaders and the stores is 64-bit.
