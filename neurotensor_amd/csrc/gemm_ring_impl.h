@@ -104,7 +104,7 @@ __device__ __forceinline__ void dma_offsets(uint32_t (&off)[WB], int64_t ld, int
             off[jj] = (uint32_t)(((int64_t)row * ld + kv * VEL) * ES);
         } else {
             int krow = (64 / CH) * j + lane / CH;
-            int chunk = (lane % CH) ^ (ES == 2 ? 2 * (krow & 3) : 8 * ((krow >> 2) & 1));
+            int chunk = (lane % CH) ^ (ES == 2 ? 2 * (krow & 3) : ES == 4 ? 8 * ((krow >> 2) & 1) : 0);   // Float64: stored as is
             if constexpr (RAGGED) {
                 krow = krow < k_valid ? krow : k_valid - 1;
                 chunk = chunk < mn_valid / VEL ? chunk : mn_valid / VEL - 1;

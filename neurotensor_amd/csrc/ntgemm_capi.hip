@@ -142,13 +142,11 @@ SplitPlan plan_splitk(const ntg::GemmParams& p, int dtype, bool ta) {
         if (best == 1) return none;
         return SplitPlan{(int)best, p.K / best, best * (int64_t)p.M * p.N * 4};
     }
-    // fp64: two 128 x 128 (or more 64 x 64) tiles per CU wanted in flight; fp32 (whose kernel goes down to 64 x 64
-    // tiles by itself) only when those leave CUs without any tile
-    const bool f32 = dtype == ntg::DT_F32;
-    const int64_t tile = (f32 || p.M <= 64 || p.N <= 64) ? 64 : 128, kstep = f32 ? 32 : 16;
+    // fp32 / fp64: their kernels go down to 64 x 64 tiles by themselves; split only when those leave CUs without any tile
+    const int64_t tile = 64, kstep = 32;
     const int64_t target = 512;
     const int64_t tiles = ((p.M + tile - 1) / tile) * ((p.N + tile - 1) / tile);
-    if ((f32 ? 1 : 2) * tiles > (f32 ? 255 : target)) return none;
+    if (tiles > 255) return none;
     int64_t smax = target / tiles;
     if (smax > 16) smax = 16;
     for (int64_t sp = smax; sp >= 2; --sp) {

@@ -347,23 +347,25 @@ def test_ragged_16bit_dma_kernel(dtype, shape):
     assert ((y.float() - refy).abs().max() / refy.abs().max()).item() <= HALF_REL
 
 
-@pytest.mark.parametrize("shape", [(1860, 260, 1860), (2052, 1000, 2308), (1028, 132, 516), (68, 20, 4), (132, 16, 260)],
+@pytest.mark.parametrize("dtype", [np.float32, np.float64], ids=["fp32", "fp64"])
+@pytest.mark.parametrize("shape", [(1860, 260, 1860), (2052, 1000, 2308), (1028, 132, 516), (68, 20, 4), (132, 16, 260), (130, 22, 66)],
                          ids=lambda s: "x".join(map(str, s)))
-def test_ragged_fp32_ring_kernel(shape):
-    """Float32 with 16-byte rows (sizes multiples of 4) stays on the DMA-fed kernel: 1860 x 1860 runs on 128 x 128 tiles,
-    the others on 64 x 64; edge rows / columns, a last 16-byte chunk of C of which only the first half exists
-    (n % 8 == 4), k tails of 4, 8, 4 and none, all three C modes, nothing written outside [m, n]."""
+def test_ragged_fp32_fp64_ring_kernels(dtype, shape):
+    """Float32 / Float64 with 16-byte rows (sizes multiples of 4 / 2) stay on the DMA-fed kernels: 1860 x 1860 runs on
+    128 x 128 tiles, the others on 64 x 64; edge rows / columns, a last 16-byte chunk of C of which only the first half
+    exists (fp32, n % 8 == 4), k tails (fp32: 4, 8, 4, none; fp64: 4, none, 4, 4, none, 6), all three C modes, nothing
+    written outside [m, n].  130 x 22 x 66 has 8-byte but not 16-byte rows in fp32: the register-staged kernel."""
     m, k, n = shape
     rng = np.random.default_rng(1300 + k)
     for ta, tb in TRANS:
-        a = randn(rng, (m, k), np.float32)
-        b = randn(rng, (k, n), np.float32)
+        a = randn(rng, (m, k), dtype)
+        b = randn(rng, (k, n), dtype)
         sa = np.ascontiguousarray(a.T) if ta else a
         sb = np.ascontiguousarray(b.T) if tb else b
         ta_, tb_ = to_torch(sa, DEV, False), to_torch(sb, DEV, False)
         ref = torch.matmul(to_torch(a, DEV, False).double(), to_torch(b, DEV, False).double())
         tol = 1e-5 * k * float(np.abs(a).max() * np.abs(b).max())
-        guard = torch.full((m + 2, n), 7.0, device=DEV)
+        guard = torch.full((m + 2, n), 7.0, device=DEV, dtype=ta_.dtype)
         c = guard[1:m + 1]
         c.zero_()
         out = F.matmult(ta_, tb_, c, ta, tb, accumulate=False)
@@ -374,8 +376,8 @@ def test_ragged_fp32_ring_kernel(shape):
         assert torch.all(guard[0] == 7.0) and torch.all(guard[m + 1] == 7.0)
         rows = np.r_[0:4, m - 4:m]
         cols = np.r_[0:4, n - 4:n]
-        _sampled_oracle_check(sa, sb, F.matmult(ta_, tb_, None, ta, tb), ta, tb, np.float32, rows, cols, k)
-    bias = randn(rng, (n,), np.float32)
+        _sampled_oracle_check(sa, sb, F.matmult(ta_, tb_, None, ta, tb), ta, tb, dtype, rows, cols, k)
+    bias = randn(rng, (n,), dtype)
     y = F.linear(to_torch(a, DEV, False), to_torch(b, DEV, False), to_torch(bias, DEV, False))
     assert (y.double() - (ref + to_torch(bias, DEV, False).double())).abs().max().item() <= tol
 
