@@ -36,6 +36,45 @@ __global__ void __launch_bounds__(256) unfold2d_kernel(const T* __restrict__ im,
     }
 }
 
+// The same matrix, 16 bytes of consecutive outputs per lane (V = 16 / sizeof(T) elements of one row of col) and 32-bit
+// index arithmetic with multiply-shift divisions: for L = Ho*Wo a multiple of V every vector lies inside one row
+// (b, kk) of col and is 16-byte aligned.  One workgroup covers 256 vectors of one row, so b and the tap (c, i, j) are
+// uniform; a lane splits its first l into (h, w) once and walks on element by element (the vector may cross the end
+// of an output row).
+struct UnfoldVecParams {
+    int channels, height, width, k_c, s_r, s_c, p_r, p_c, d_r, d_c, Wo, ccol, vec_per_row, blocks_per_row;
+    FastDiv div_bpr, div_ccol, div_krc, div_kc, div_wo;
+    int k_rc;
+    int64_t L;
+};
+
+template <class T>
+__global__ void __launch_bounds__(256) unfold2d_vec_kernel(const T* __restrict__ im, T* __restrict__ col, const UnfoldVecParams u) {
+    constexpr int V = 16 / (int)sizeof(T);
+    const uint32_t row = fast_div(blockIdx.x, u.div_bpr);
+    const uint32_t lv = (blockIdx.x - row * (uint32_t)u.blocks_per_row) * 256u + threadIdx.x;
+    if (lv >= (uint32_t)u.vec_per_row) return;
+    const uint32_t b = fast_div(row, u.div_ccol), kk = row - b * (uint32_t)u.ccol;
+    const uint32_t c = fast_div(kk, u.div_krc), rem = kk - c * (uint32_t)u.k_rc;
+    const uint32_t i = fast_div(rem, u.div_kc), j = rem - i * (uint32_t)u.k_c;
+    const T* plane = im + ((int64_t)b * u.channels + c) * ((int64_t)u.height * u.width);
+    const uint32_t l0 = lv * V;
+    uint32_t h = fast_div(l0, u.div_wo), w = l0 - h * (uint32_t)u.Wo;
+    const int dh = (int)i * u.d_r - u.p_r, dw = (int)j * u.d_c - u.p_c;
+    T v[V];
+#pragma unroll
+    for (int e = 0; e < V; ++e) {
+        const int hp = (int)h * u.s_r + dh, wp = (int)w * u.s_c + dw;
+        const bool ok = (unsigned)hp < (unsigned)u.height && (unsigned)wp < (unsigned)u.width;
+        v[e] = ok ? plane[(int64_t)hp * u.width + wp] : (T)0;
+        if (++w == (uint32_t)u.Wo) { w = 0; ++h; }
+    }
+    typedef uint32_t u32x4v __attribute__((ext_vector_type(4)));
+    u32x4v o;
+    __builtin_memcpy(&o, v, 16);
+    *reinterpret_cast<u32x4v*>(col + (int64_t)row * u.L + l0) = o;
+}
+
 // col2im, the adjoint of the above (im2col_backward_cpu, nt/functional/cpu/unfold2d_backward.cpp:9-56):
 //   im[b, c, y, x] (+)= sum over taps (i, j) of col[b, c*kh*kw + i*kw + j, h*Wo + w]
 //   with  y = h*s_r - p_r + i*d_r,  x = w*s_c - p_c + j*d_c.
@@ -369,6 +408,35 @@ hipError_t launch_unfold2d(int64_t es, const void* im, void* col,
     u.ccol = channels * k_r * k_c;
     u.total = batch * u.ccol * u.Ho * u.Wo;
     if (u.total == 0) return hipSuccess;
+    {
+        // 16-byte stores when every row of col is a whole number of vectors and all sizes fit 32-bit arithmetic
+        const int64_t L = u.Ho * u.Wo, V = 16 / es, rows = batch * u.ccol;
+        const int64_t lim = 1 << 24;
+        if (L % V == 0 && (reinterpret_cast<uintptr_t>(col) & 15) == 0 && L < 0x7fffffffLL && rows < 0x7fffffffLL &&
+            height < lim && width < lim && k_r * d_r < lim && k_c * d_c < lim && u.Ho * s_r < lim && u.Wo * s_c < lim && p_r < lim && p_c < lim &&
+            p_r > -lim && p_c > -lim && u.ccol < 0x7fffffffLL) {
+            UnfoldVecParams q;
+            q.channels = (int)channels; q.height = (int)height; q.width = (int)width; q.k_c = (int)k_c;
+            q.s_r = (int)s_r; q.s_c = (int)s_c; q.p_r = (int)p_r; q.p_c = (int)p_c; q.d_r = (int)d_r; q.d_c = (int)d_c;
+            q.Wo = (int)u.Wo; q.ccol = (int)u.ccol; q.k_rc = (int)(k_r * k_c); q.L = L;
+            q.vec_per_row = (int)(L / V);
+            q.blocks_per_row = (q.vec_per_row + 255) / 256;
+            const int64_t nblocks = rows * q.blocks_per_row;
+            if (nblocks <= 0x7fffffffLL) {
+                q.div_bpr = make_fastdiv((uint32_t)q.blocks_per_row); q.div_ccol = make_fastdiv((uint32_t)q.ccol);
+                q.div_krc = make_fastdiv((uint32_t)q.k_rc); q.div_kc = make_fastdiv((uint32_t)q.k_c); q.div_wo = make_fastdiv((uint32_t)q.Wo);
+                const dim3 g((unsigned)nblocks), t(256);
+                switch (es) {
+                case 1: hipLaunchKernelGGL(unfold2d_vec_kernel<uint8_t>, g, t, 0, s, (const uint8_t*)im, (uint8_t*)col, q); break;
+                case 2: hipLaunchKernelGGL(unfold2d_vec_kernel<uint16_t>, g, t, 0, s, (const uint16_t*)im, (uint16_t*)col, q); break;
+                case 4: hipLaunchKernelGGL(unfold2d_vec_kernel<uint32_t>, g, t, 0, s, (const uint32_t*)im, (uint32_t*)col, q); break;
+                case 8: hipLaunchKernelGGL(unfold2d_vec_kernel<uint64_t>, g, t, 0, s, (const uint64_t*)im, (uint64_t*)col, q); break;
+                default: return hipErrorInvalidValue;
+                }
+                return hipGetLastError();
+            }
+        }
+    }
     int64_t blocks = (u.total + 255) / 256;
     if (blocks > 256 * 64) blocks = 256 * 64;   // grid-stride beyond 64 workgroups per CU
     switch (es) {
