@@ -1,7 +1,6 @@
 // Float32 instantiations of the MFMA GEMMs (v_mfma_f32_32x32x2_f32): the DMA-fed LDS ring for 16-byte aligned rows,
 // the register-staged kernel for everything else and for the gathering convolutions.
 #include "gemm_ring_impl.h"
-#include <stdlib.h>
 namespace ntg {
 // Tile edge of the DMA-fed kernel for Float32 (64 or 128).  The 32x32x2 MFMA is slow enough that LDS traffic never
 // binds, so the tile only decides how evenly the work spreads: a CU's time is the number of tiles it is handed
@@ -36,13 +35,10 @@ static bool ring_conv_eligible(const GemmParams& p) {
     return p.K % 4 == 0 && p.N % 4 == 0 && p.ldc % 4 == 0 && p.sC % 4 == 0 && p.vecA_ok && p.lda % 4 == 0 && p.sA % 4 == 0 &&
            p.lda < (1 << 21) && !p.Aptr && !p.Bptr && !p.Cptr &&
            ((reinterpret_cast<uintptr_t>(p.A) & 15) == 0) && ((reinterpret_cast<uintptr_t>(p.C) & 15) == 0) &&
-           ((reinterpret_cast<uintptr_t>(p.B) & 3) == 0) && (p.sB % 1 == 0);
+           ((reinterpret_cast<uintptr_t>(p.B) & 3) == 0);
 }
 hipError_t launch_conv_mfma_f32(bool tb, int nd, const GemmParams& p, hipStream_t s) {
-    if (nd == 2 && ring_conv_eligible(p)) {
-        static const int off = getenv("NTG_NO_RING_CONV") ? 1 : 0;
-        if (!off) return p.M > 64 ? launch_ring_conv_cfg<2>(tb, p, s) : launch_ring_conv_cfg<1>(tb, p, s);
-    }
+    if (nd == 2 && ring_conv_eligible(p)) return p.M > 64 ? launch_ring_conv_cfg<2>(tb, p, s) : launch_ring_conv_cfg<1>(tb, p, s);
     return nd == 3 ? launch_conv_nd_f32<3>(tb, p, s) : launch_conv_nd_f32<2>(tb, p, s);
 }
 }  // namespace ntg
