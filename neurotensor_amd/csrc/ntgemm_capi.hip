@@ -142,17 +142,25 @@ SplitPlan plan_splitk(const ntg::GemmParams& p, int dtype, bool ta) {
         if (best == 1) return none;
         return SplitPlan{(int)best, p.K / best, best * (int64_t)p.M * p.N * 4};
     }
-    // fp32 / fp64: their kernels go down to 64 x 64 tiles by themselves; split only when those leave CUs without any tile
-    const int64_t tile = 64, kstep = 32;
-    const int64_t target = 512;
-    const int64_t tiles = ((p.M + tile - 1) / tile) * ((p.N + tile - 1) / tile);
+    // fp32 / fp64: their kernels go down to 64 x 64 tiles by themselves; a split pays only when those leave CUs without a
+    // tile.  Same kind of estimate: a CU spends about 14.4 ns (fp32) / 28.8 ns (fp64) per k on each 64 x 64 tile it is
+    // handed; the second pass costs about 5 us + the partial sums written and read at 4 TB/s.
+    const int64_t tiles = ((p.M + 63) / 64) * ((p.N + 63) / 64);
     if (tiles > 255) return none;
-    int64_t smax = target / tiles;
-    if (smax > 16) smax = 16;
-    for (int64_t sp = smax; sp >= 2; --sp) {
-        if (p.K % (sp * kstep) != 0 || p.K / sp < 512) continue;   // short k ranges do not pay for the second pass
-        return SplitPlan{(int)sp, p.K / sp, sp * (int64_t)p.M * p.N * es};
+    const double per_k = dtype == ntg::DT_F32 ? 0.0144 : 0.0288;
+    auto estimate_us = [&](int64_t sp) {
+        const double rounds = (double)((tiles * sp + 255) / 256);
+        const double second_pass = sp == 1 ? 0.0 : 5.0 + 2.0 * (double)sp * (double)p.M * (double)p.N * (double)es / 4.0e6;
+        return rounds * (double)(p.K / sp) * per_k + second_pass;
+    };
+    int64_t best = 1;
+    double best_us = estimate_us(1);
+    for (int64_t sp = 2; sp <= 16; ++sp) {
+        if (p.K % (sp * 32) != 0 || p.K / sp < 64) continue;
+        const double us = estimate_us(sp);
+        if (us < 0.9 * best_us) { best = sp; best_us = us; }
     }
+    if (best > 1) return SplitPlan{(int)best, p.K / best, best * (int64_t)p.M * p.N * es};
     return none;
 }
 
