@@ -120,6 +120,13 @@ hipError_t launch_splitk_reduce(int dtype, const void* part, int splits, const G
 hipError_t launch_reduce_batch(int dtype, const void* part, void* out, int64_t batch, int64_t n, int accumulate, hipStream_t s);
 hipError_t launch_flip_weights(int64_t elem_size, const void* w, void* wt, int64_t groups, int64_t og, int64_t cg, int64_t taps, hipStream_t s);
 
+// grid of a grid-stride element-wise kernel (256 lanes per workgroup, at most 64 workgroups per CU)
+static inline unsigned grid_for(int64_t total) {
+    int64_t blocks = (total + 255) / 256;
+    if (blocks > 256 * 64) blocks = 256 * 64;
+    return (unsigned)(blocks < 1 ? 1 : blocks);
+}
+
 #ifdef __HIPCC__
 __device__ __forceinline__ uint32_t fast_div(uint32_t n, const FastDiv& f) {
     const uint32_t t = __umulhi(f.m, n);

@@ -111,158 +111,6 @@ __global__ void __launch_bounds__(256) col2im_kernel(const T* __restrict__ col, 
     }
 }
 
-// out[i] (+)= sum over b of part[b*n + i], b ascending: the order in which per-image weight
-// gradients are added up by the reference's batch loop (conv.cpp:466-469).
-template <class T, class Acc>
-__global__ void __launch_bounds__(256) reduce_batch_kernel(const T* __restrict__ part, T* __restrict__ out, const int64_t batch,
-                                                           const int64_t n, const int accumulate) {
-    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
-        Acc acc = accumulate ? (Acc)out[i] : (Acc)0;
-        for (int64_t b = 0; b < batch; ++b) acc += (Acc)part[b * n + i];
-        out[i] = (T)acc;
-    }
-}
-
-static unsigned grid_for(int64_t total) {
-    int64_t blocks = (total + 255) / 256;
-    if (blocks > 256 * 64) blocks = 256 * 64;
-    return (unsigned)(blocks < 1 ? 1 : blocks);
-}
-
-// Split-K epilogue: C (+)= sum over the k ranges of part[s][m][n], s ascending, starting from C0 (the incoming C, the
-// broadcast bias, or zero).  One rounding to T at the end.
-template <class T, class P, class Acc>
-__global__ void __launch_bounds__(256) splitk_reduce_kernel(const P* __restrict__ part, const int splits, const GemmParams p) {
-    const int64_t total = (int64_t)p.M * p.N;
-    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-    T* C = static_cast<T*>(p.C);
-    const T* bias = static_cast<const T*>(p.bias);
-    for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += stride) {
-        const int64_t m = idx / p.N, n = idx - m * p.N;
-        T* cp = C + m * p.ldc + n;
-        Acc acc = (Acc)0;
-        if (p.cmode == C_ACCUMULATE) acc = (Acc)*cp;
-        else if (p.cmode == C_BIAS) acc = (Acc)bias[m * p.bias_rs + n * p.bias_cs];
-        for (int s = 0; s < splits; ++s) acc += (Acc)part[(int64_t)s * total + idx];
-        *cp = (T)acc;
-    }
-}
-
-// The same sum, four consecutive columns per thread with 16-byte accesses to the partial sums (rows of C and of the
-// partial matrices must start on a multiple of four elements); the partial loads of four k ranges are in flight together.
-template <class T, class P, class Acc>
-__global__ void __launch_bounds__(256) splitk_reduce_vec_kernel(const P* __restrict__ part, const int splits, const GemmParams p) {
-    typedef T TV __attribute__((ext_vector_type(4)));
-    typedef P PV __attribute__((ext_vector_type(4)));
-    const int64_t nq = p.N / 4, total = (int64_t)p.M * p.N, quads = (int64_t)p.M * nq;
-    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-    T* C = static_cast<T*>(p.C);
-    const T* bias = static_cast<const T*>(p.bias);
-    for (int64_t q = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; q < quads; q += stride) {
-        const int64_t m = q / nq, n = (q - m * nq) * 4;
-        TV* cp = reinterpret_cast<TV*>(C + m * p.ldc + n);
-        Acc acc[4] = {(Acc)0, (Acc)0, (Acc)0, (Acc)0};
-        if (p.cmode == C_ACCUMULATE) {
-            const TV c0 = *cp;
-#pragma unroll
-            for (int e = 0; e < 4; ++e) acc[e] = (Acc)c0[e];
-        } else if (p.cmode == C_BIAS) {
-#pragma unroll
-            for (int e = 0; e < 4; ++e) acc[e] = (Acc)bias[m * p.bias_rs + (n + e) * p.bias_cs];
-        }
-        const P* pp = part + q * 4;
-        int s = 0;
-        for (; s + 4 <= splits; s += 4) {
-            PV v[4];
-#pragma unroll
-            for (int u = 0; u < 4; ++u) v[u] = *reinterpret_cast<const PV*>(pp + (int64_t)(s + u) * total);
-#pragma unroll
-            for (int u = 0; u < 4; ++u)
-#pragma unroll
-                for (int e = 0; e < 4; ++e) acc[e] += (Acc)v[u][e];
-        }
-        for (; s < splits; ++s) {
-            const PV v = *reinterpret_cast<const PV*>(pp + (int64_t)s * total);
-#pragma unroll
-            for (int e = 0; e < 4; ++e) acc[e] += (Acc)v[e];
-        }
-        TV o;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) o[e] = (T)acc[e];
-        *cp = o;
-    }
-}
-
-template <class T, class P, class Acc>
-static void launch_splitk_reduce_t(const void* part, int splits, const GemmParams& p, hipStream_t s) {
-    const int64_t total = (int64_t)p.M * p.N;
-    const bool vec = p.N % 4 == 0 && p.ldc % 4 == 0 && (reinterpret_cast<uintptr_t>(p.C) % (4 * sizeof(T))) == 0 &&
-                     (reinterpret_cast<uintptr_t>(part) % (4 * sizeof(P))) == 0;
-    if (vec) hipLaunchKernelGGL((splitk_reduce_vec_kernel<T, P, Acc>), dim3(grid_for(total / 4)), dim3(256), 0, s, (const P*)part, splits, p);
-    else hipLaunchKernelGGL((splitk_reduce_kernel<T, P, Acc>), dim3(grid_for(total)), dim3(256), 0, s, (const P*)part, splits, p);
-}
-
-hipError_t launch_splitk_reduce(int dtype, const void* part, int splits, const GemmParams& p, hipStream_t s) {
-    const int64_t total = (int64_t)p.M * p.N;
-    if (total == 0) return hipSuccess;
-    switch (dtype) {
-    case DT_F32: launch_splitk_reduce_t<float, float, float>(part, splits, p, s); break;
-    case DT_F64: launch_splitk_reduce_t<double, double, double>(part, splits, p, s); break;
-    case DT_F16: launch_splitk_reduce_t<_Float16, float, float>(part, splits, p, s); break;
-    case DT_BF16: launch_splitk_reduce_t<__bf16, float, float>(part, splits, p, s); break;
-    default: return hipErrorInvalidValue;
-    }
-    return hipGetLastError();
-}
-
-
-// wt[g][c][oc][t] = w[g*og + oc][c][taps-1-t]: the kernel with input/output channels swapped
-// inside each group and both tap axes reversed, i.e. the weights of the convolution that maps
-// the output gradient back to the image.
-template <class T>
-__global__ void __launch_bounds__(256) flip_weights_kernel(const T* __restrict__ w, T* __restrict__ wt, const int64_t groups,
-                                                           const int64_t og, const int64_t cg, const int64_t taps) {
-    const int64_t total = groups * og * cg * taps;
-    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-    for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += stride) {
-        const int64_t t = idx % taps;
-        int64_t r = idx / taps;
-        const int64_t oc = r % og;
-        r /= og;
-        const int64_t c = r % cg;
-        const int64_t g = r / cg;
-        wt[idx] = w[((g * og + oc) * cg + c) * taps + (taps - 1 - t)];
-    }
-}
-
-
-hipError_t launch_reduce_batch(int dtype, const void* part, void* out, int64_t batch, int64_t n, int accumulate, hipStream_t s) {
-    if (n == 0) return hipSuccess;
-    const dim3 g(grid_for(n)), b(256);
-    switch (dtype) {
-    case DT_F32: hipLaunchKernelGGL((reduce_batch_kernel<float, float>), g, b, 0, s, (const float*)part, (float*)out, batch, n, accumulate); break;
-    case DT_F64: hipLaunchKernelGGL((reduce_batch_kernel<double, double>), g, b, 0, s, (const double*)part, (double*)out, batch, n, accumulate); break;
-    case DT_F16: hipLaunchKernelGGL((reduce_batch_kernel<_Float16, float>), g, b, 0, s, (const _Float16*)part, (_Float16*)out, batch, n, accumulate); break;
-    case DT_BF16: hipLaunchKernelGGL((reduce_batch_kernel<__bf16, float>), g, b, 0, s, (const __bf16*)part, (__bf16*)out, batch, n, accumulate); break;
-    default: return hipErrorInvalidValue;
-    }
-    return hipGetLastError();
-}
-
-hipError_t launch_flip_weights(int64_t es, const void* w, void* wt, int64_t groups, int64_t og, int64_t cg, int64_t taps, hipStream_t s) {
-    const int64_t total = groups * og * cg * taps;
-    if (total == 0) return hipSuccess;
-    const dim3 g(grid_for(total)), b(256);
-    switch (es) {
-    case 2: hipLaunchKernelGGL(flip_weights_kernel<uint16_t>, g, b, 0, s, (const uint16_t*)w, (uint16_t*)wt, groups, og, cg, taps); break;
-    case 4: hipLaunchKernelGGL(flip_weights_kernel<uint32_t>, g, b, 0, s, (const uint32_t*)w, (uint32_t*)wt, groups, og, cg, taps); break;
-    case 8: hipLaunchKernelGGL(flip_weights_kernel<uint64_t>, g, b, 0, s, (const uint64_t*)w, (uint64_t*)wt, groups, og, cg, taps); break;
-    default: return hipErrorInvalidValue;
-    }
-    return hipGetLastError();
-}
-
 // ---- the same two transforms over up to NTG_MAX_SPATIAL axes (unfold3d / unfoldnd and their adjoints:
 // nt/functional/cpu/unfold3d.cpp:9-80, unfoldnd.cpp, unfold3d_backward.cpp, unfoldnd_backward.cpp).
 // Row index of col: ((c*k0 + t0)*k1 + t1)*... ; column index: (o0*out1 + o1)*... ; last axis fastest.
