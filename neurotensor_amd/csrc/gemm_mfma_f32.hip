@@ -38,7 +38,8 @@ static bool ring_conv_eligible(const GemmParams& p) {
            ((reinterpret_cast<uintptr_t>(p.B) & 3) == 0);
 }
 hipError_t launch_conv_mfma_f32(bool tb, int nd, const GemmParams& p, hipStream_t s) {
-    if (nd == 2 && ring_conv_eligible(p)) return p.M > 64 ? launch_ring_conv_cfg<2>(tb, p, s) : launch_ring_conv_cfg<1>(tb, p, s);
+    // tile edge by the same evenness rule as the plain product (padding of M = O/g and N = Ho*Wo to the tile counts as work)
+    if (nd == 2 && ring_conv_eligible(p)) return ring_f32_tile_edge(p) == 128 ? launch_ring_conv_cfg<2>(tb, p, s) : launch_ring_conv_cfg<1>(tb, p, s);
     return nd == 3 ? launch_conv_nd_f32<3>(tb, p, s) : launch_conv_nd_f32<2>(tb, p, s);
 }
 }  // namespace ntg
