@@ -96,6 +96,43 @@ def test_argument_errors_do_not_need_a_device():
     assert lib.ntg_gemm_dev(ctypes.byref(d), p, p, p, None) == 1
 
 
+def test_split_k_planner_needs_no_device():
+    """ntg_gemm_workspace_bytes is host arithmetic: which products are offered a split along k, and into how many ranges
+    (bytes = ranges x m x n x 4 for the 16-bit dtypes, whose partial sums are fp32; x element size otherwise)."""
+    lib = _lib.load()
+
+    def ws(dtype, m, k, n, batches=1, ta=0, tb=0, lda=0):
+        d = _lib.GemmDesc()
+        d.dtype, d.transpose_a, d.transpose_b, d.c_mode = dtype, ta, tb, _lib.C_OVERWRITE
+        d.m, d.k, d.n, d.batches, d.lda = m, k, n, batches, lda
+        return lib.ntg_gemm_workspace_bytes(ctypes.byref(d))
+
+    def ranges(dtype, m, k, n, es):
+        b = ws(dtype, m, k, n)
+        assert b % (m * n * es) == 0
+        return b // (m * n * es)
+
+    # full-chip products are never split; integers, batches and the streaming (m <= 32) shapes neither
+    for dt in (_lib.BFLOAT16, _lib.FLOAT16, _lib.FLOAT32, _lib.FLOAT64):
+        assert ws(dt, 4096, 4096, 4096) == 0
+        assert ws(dt, 256, 8192, 2048, batches=2) == 0
+    assert ws(_lib.INT32, 64, 8192, 64) == 0
+    assert ws(_lib.FLOAT32, 16, 8192, 8192) == 0 and ws(_lib.BFLOAT16, 32, 8192, 8192) == 0
+    # 16-bit, 128 x 128 tiles: 64 tiles and k = 8192 -> four ranges; one tile and k = 16384 -> sixteen
+    assert ranges(_lib.BFLOAT16, 128, 8192, 8192, 4) == 4
+    assert ranges(_lib.FLOAT16, 128, 16384, 128, 4) == 16
+    # a short k does not pay for the second pass; a product that already has a tile for most CUs does not either
+    assert ws(_lib.BFLOAT16, 1024, 1024, 1024) == 0
+    assert ws(_lib.BFLOAT16, 1536, 4096, 1536) == 0
+    # rows that are not 16-byte multiples cannot use the kernel that writes fp32 partial sums
+    assert ws(_lib.BFLOAT16, 128, 8192, 8190) == 0 and ws(_lib.BFLOAT16, 128, 8192, 8192, lda=8196) == 0
+    # fp32 / fp64, 64 x 64 tiles: 16 tiles and k = 1024 -> eight ranges of 128; 256 or more tiles -> none
+    assert ranges(_lib.FLOAT32, 256, 1024, 256, 4) == 8
+    assert ranges(_lib.FLOAT64, 256, 1024, 256, 8) == 8
+    assert ws(_lib.FLOAT32, 1024, 4096, 1024) == 0 and ws(_lib.FLOAT64, 1024, 4096, 1024) == 0
+    assert ws(_lib.FLOAT32, 768, 768, 768) == 0
+
+
 def test_missing_library_fails_loudly(monkeypatch, tmp_path):
     monkeypatch.setattr(_lib, "_lib", None)
     monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "libntgemm.so"))
