@@ -339,7 +339,7 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
         return krow * G::MN_ROW_BYTES + ((mnl * 4) ^ (128 * (lane >> 5)));      // (krow >> 2) & 1 == lane / 32
     };
 
-    // One LDS read instruction of an operand's fragment set for k16-step ks.  A K-major
+    // One LDS read instruction of an operand's fragment set for half-step ks.  A K-major
     // operand takes WB reads (one ds_read_b128 per block), an MN-major one 2 WB (two transposing
     // 8-byte reads per block; Float32: 4 WB four-byte reads); read r lands in frag[r / per_block].
     auto read_op = [&](u32x4 (&frag)[WB], const char* tile, bool kc, int wbase, int ks, int r) {
@@ -390,7 +390,7 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
     b_tile(2, lds_addr_of(st2) + G::TILE_BYTES);
     dma_tile<WB>(srcA(3), 3 >= last ? offAt : offA, lds_addr_of(st3), wave_u);
 
-    u32x4 af[2][WB], bf[2][WB];   // fragment double buffer: [k16-step parity][block]
+    u32x4 af[2][WB], bf[2][WB];   // fragment double buffer: [half-step parity][block]
 
     // all reads of one fragment set, back to back (prologue only)
     auto load_frags = [&](const char* stage, int ks, int buf) {
@@ -399,9 +399,9 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
 #pragma unroll
         for (int r = 0; r < NRB; ++r) read_op(bf[buf], stage + G::TILE_BYTES, B_KC, wn * WT, ks, r);
     };
-    // WB^2 MFMAs on fragment set `cur_buf`, with the NR reads of the next set (stage/ks ->
-    // `nxt_buf`) slotted RPM (one; up to two for the 128 x 128 tile) per MFMA, so LDS latency is
-    // always covered by matrix work and never more than NR (<= 16) reads are outstanding.  WB DMA
+    // The NMMA MFMAs of one half-step on fragment set `cur_buf`, with the NR reads of the next set (stage/ks ->
+    // `nxt_buf`) slotted RPM (one; two for the small 16-bit tiles) per MFMA, so LDS latency is
+    // always covered by matrix work and only a few reads are outstanding at a time.  The step's DMA
     // instructions (one operand tile's share of this wavefront) are spread over the step as
     // well -- issued in a burst right after the barrier, the four wavefronts would queue up
     // behind the CU's one address unit and stall their MFMA streams.
@@ -452,11 +452,11 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
     asm volatile("" ::: "memory");
     load_frags(st0, 0, 0);
 
-    // One K-step.  `cur` holds tile kt (its k16-step 0 fragments are already in registers),
+    // One K-step.  `cur` holds tile kt (its half-step 0 fragments are already in registers),
     // `nxt` holds tile kt+1, `prv` held tile kt-1.  The single barrier sits between the two
-    // k16-steps: by then every wavefront has issued and received its last reads of `cur`, so
+    // half-steps: by then every wavefront has issued and received its last reads of `cur`, so
     // the stage goes back to the DMA at once: the A half of tile kt+4 is fetched during the
-    // second k16-step, its B half during the first k16-step of the next K-step.  Tile kt+1,
+    // second half-step, its B half during the first half-step of the next K-step.  Tile kt+1,
     // first touched in the second half, has had three K-steps to arrive.
     // RAGGED: zero the k >= K part of a fragment set of the last K-step.  Every lane's fragment
     // covers one chunk of consecutive k (8 or 4) starting at (BK/2) ks + (BK/4) (lane / 32) in both
