@@ -436,7 +436,9 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
         for (int q = 0; q < NMMA; ++q) {
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);               // one MFMA
             const int nrd = NR - q * RPM < RPM ? NR - q * RPM : RPM;
-            if (nrd == 2) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0); // its LDS reads
+            if (nrd == 4) __builtin_amdgcn_sched_group_barrier(0x100, 4, 0); // its LDS reads
+            else if (nrd == 3) __builtin_amdgcn_sched_group_barrier(0x100, 3, 0);
+            else if (nrd == 2) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
             else if (nrd == 1) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
             if constexpr (NGATHER > 0) {
                 // the gather's address arithmetic, dealt out evenly: what does not fit under one MFMA delays the next
@@ -657,7 +659,9 @@ static hipError_t launch_ring_wb(bool ta, bool tb, const GemmParams& p, hipStrea
 
 template <int DT>
 static hipError_t launch_ring16(bool ta, bool tb, const GemmParams& p, hipStream_t s) {
-    if (ring16_tile_edge(p.M, p.N, p.batch) == 256) return launch_ring_wb<DT, 4>(ta, tb, p, s);
+    const int te = ring16_tile_edge(p.M, p.N, p.K, p.batch);
+    if (te == 256) return launch_ring_wb<DT, 4>(ta, tb, p, s);
+    if (te == 64) return launch_ring_wb<DT, 1>(ta, tb, p, s);
     return launch_ring_wb<DT, 2>(ta, tb, p, s);
 }
 

@@ -67,12 +67,23 @@ struct GemmParams {
     ConvGeom conv;           // used by the implicit-im2col kernels only: B = image, op(B) = col or col^T
 };
 
-// Tile edge the DMA-fed 16-bit kernel uses for M x N x batch: 256 x 256 tiles need about half the LDS traffic per
-// flop, but the 256 CUs idle below one tile each; four times as many 128 x 128 workgroups (two fit on a CU) are
-// quicker up to 128 large tiles.
-static inline int ring16_tile_edge(int64_t M, int64_t N, int64_t batch) {
-    const int64_t t256 = ((M + 255) / 256) * ((N + 255) / 256) * batch;
-    return t256 > 128 ? 256 : 128;
+// Tile edge (256, 128 or 64) the DMA-fed 16-bit kernel uses for M x N x K x batch.  Larger tiles need less LDS traffic per
+// flop (a CU sustains about 0.5 / 0.4 / 0.25 of its MFMA peak on 256 / 128 / 64-wide tiles at full load, 0.64 on 256-wide
+// tiles while most CUs are idle and the clock is high), smaller ones spread the work over the 256 CUs more evenly,
+// waste less on the padding of M and N, and hide a tile's prologue and epilogue (about 3 / 1.5 / 0.6 us of exposed
+// latency per tile) behind their neighbours on the CU.  Estimated time = tiles per CU x (tile time + exposed latency).
+static inline int ring16_tile_edge(int64_t M, int64_t N, int64_t K, int64_t batch) {
+    const double cu_flops_per_us = 9.77e6;                      // 2500 TFLOP/s over 256 CUs
+    int best = 256;
+    double best_us = 0.0;
+    for (int t = 256; t >= 64; t /= 2) {
+        const int64_t nt = ((M + t - 1) / t) * ((N + t - 1) / t) * batch;
+        const double f = t == 256 ? (nt >= 192 ? 0.5 : 0.64) : t == 128 ? 0.4 : 0.25;
+        const double latency = t == 256 ? 3.0 : t == 128 ? 1.5 : 0.6;
+        const double us = (double)((nt + 255) / 256) * (2.0 * t * t * (double)K / (cu_flops_per_us * f) + latency);
+        if (t == 256 || us < best_us) { best = t; best_us = us; }
+    }
+    return best;
 }
 
 static inline int64_t elem_size(int dt) {

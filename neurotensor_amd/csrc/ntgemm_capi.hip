@@ -124,7 +124,7 @@ SplitPlan plan_splitk(const ntg::GemmParams& p, int dtype, bool ta) {
         // a workgroup alone on its CU takes about 0.215 us per 32-wide K-step, n >= 2 sharing a CU about 0.26 n us;
         // launching the reduction and writing/reading the fp32 partial sums costs about 6 us + 8 S M N bytes at 4 TB/s.
         // Pick the S with the smallest estimate (S = 1: no split).
-        if (ntg::ring16_tile_edge(p.M, p.N, 1) != 128) return none;
+        if (ntg::ring16_tile_edge(p.M, p.N, p.K, 1) == 256) return none;
         const int64_t tiles = ((p.M + 127) / 128) * ((p.N + 127) / 128);
         auto estimate_us = [&](int64_t sp) {
             const int64_t per_cu = (tiles * sp + 255) / 256;

@@ -309,13 +309,13 @@ def test_config3_4096_cube(dtype, scale):
 
 @pytest.mark.parametrize("dtype", ["bf16", np.float16], ids=["bf16", "fp16"])
 @pytest.mark.parametrize("shape", [(2056, 1000, 2312), (1800, 1016, 3080), (2304, 992, 1928), (3000, 40, 2056), (2056, 8, 2056),
-                                   (3080, 1016, 3336), (4104, 40, 2056), (1024, 512, 1536), (128, 96, 128), (136, 72, 8)],
+                                   (3848, 1000, 4088), (4104, 40, 2056), (1024, 512, 1536), (128, 96, 128), (136, 72, 8)],
                          ids=lambda s: "x".join(map(str, s)))
 def test_ragged_16bit_dma_kernel(dtype, shape):
     """M, N, K that are not multiples of the tile (but keep 16-byte rows) stay on the DMA-fed kernel: edge
-    rows/columns, the k tail (8, 24, none, 8-only) and all three C modes.  Up to 128 tiles of 256 x 256 the kernel
-    runs with 128 x 128 tiles (the first five shapes, ragged; the last three, two of them aligned), above that
-    with 256 x 256 tiles (3080 x 3336 and 4104 x 2056: 182 and 153 large tiles)."""
+    rows/columns, the k tail (8, 24, none, 8-only) and all three C modes.  The tile edge follows the kernel's cost
+    estimate: 3848 x 4088 (16 x 16 large tiles, one per CU) runs on 256 x 256 tiles, 2056 x 2312 and 2304 x 1928 on
+    128 x 128, the others (short k, or few tiles) on 64 x 64; two shapes are tile-aligned."""
     m, k, n = shape
     bf = dtype == "bf16"
     rng = np.random.default_rng(1100 + k)
