@@ -27,7 +27,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
-PEAK_TFLOPS = {"bf16": 2500.0, "fp16": 2500.0, "fp32": 157.3, "fp64": 78.6}   # MI355X dense MFMA
+PEAK_TFLOPS = {"bf16": 2500.0, "fp16": 2500.0, "fp32": 157.3, "fp64": 78.6, "int8": 5000.0}   # MI355X dense MFMA (int8: Top/s)
 PEAK_HBM_GBS = 8000.0
 
 
@@ -83,8 +83,9 @@ def main():
         ashape = (batch, k, m) if ta else (batch, m, k)
         bshape = (batch, n, k) if tb else (batch, k, n)
         if ints:
-            a = torch.randint(-8, 9, ashape, device=dev, dtype=dtype)
-            b = torch.randint(-8, 9, bshape, device=dev, dtype=dtype)
+            lo, hi = (-128, 128) if dtype == torch.int8 else (-8, 9)      # int8: the full value range
+            a = torch.randint(lo, hi, ashape, device=dev, dtype=dtype)
+            b = torch.randint(lo, hi, bshape, device=dev, dtype=dtype)
         else:
             a = (torch.randn(ashape, device=dev) * scale).to(dtype)
             b = (torch.randn(bshape, device=dev) * scale).to(dtype)
@@ -190,6 +191,7 @@ def main():
         run("c2a_fp32_b32_1024x768x1024", make_gemm(torch.float32, 1024, 768, 1024, batch=32), f2, PEAK_TFLOPS["fp32"])
         run("c2b_fp32_b32_transpose_b", make_gemm(torch.float32, 1024, 768, 1024, tb=True, batch=32), f2, PEAK_TFLOPS["fp32"])
         run("c2c_int32_b8_1024", make_gemm(torch.int32, 1024, 1024, 1024, batch=8, ints=True), 2.0 * 8 * 1024 ** 3, None, "Top/s")
+        run("c3_int8_4096", make_gemm(torch.int8, N, N, N, ints=True, mode=_lib.C_OVERWRITE), flops, PEAK_TFLOPS["int8"], "Top/s")
         f4 = 2.0 * 8192 * 4096 * 11008
         for dt, nm in ((torch.float32, "fp32"), (torch.bfloat16, "bf16")):
             pk = PEAK_TFLOPS[nm]

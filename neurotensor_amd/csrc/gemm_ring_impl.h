@@ -49,6 +49,18 @@ typedef __attribute__((address_space(3))) void* lds_ptr_t;
 
 #define NTG_WAIT_VMCNT(N) __builtin_amdgcn_s_waitcnt(((N) & 0xF) | (7 << 4) | (15 << 8) | (((N) >> 4) << 14))
 
+// Int8 / UInt8 (one kernel: products and sums are taken modulo 2^32 in the accumulators and the low 8 bits of
+// the result are the same for both signednesses, which is the reference's wrapping arithmetic in the element type)
+typedef int intx16 __attribute__((ext_vector_type(16)));
+typedef int intx4 __attribute__((ext_vector_type(4)));
+typedef int intx2v __attribute__((ext_vector_type(2)));
+template <> struct Elem<DT_I8> {
+    using T = uint8_t; using AccS = int; using AccV = intx16;
+    static __device__ __forceinline__ void mma(AccV& c, u32x4 a, u32x4 b) {
+        c = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(intx4, a), __builtin_bit_cast(intx4, b), c, 0, 0, 0);
+    }
+};
+
 template <int DT>
 struct Cvt16;
 template <> struct Cvt16<DT_F16> {
@@ -81,13 +93,19 @@ struct RingGeom {
 //   K-contiguous operand: rows 16 j + lane/4, 16-byte slot lane%4 holds kv = slot ^ ((row>>1)&3)
 //   MN-contiguous operand (CH chunks per k-row): k-rows (64/CH) j + lane/CH, slot lane%CH holds
 //                          chunk = slot ^ (2*(krow&3)) for 16-bit elements (what the transposing
-//                          reads need), slot ^ (8*((krow>>2)&1)) for Float32 (the two k-rows that one
+//                          reads need), slot ^ mn8_swizzle(krow) for 8-bit elements,
+//                          slot ^ (8*((krow>>2)&1)) for Float32 (the two k-rows that one
 //                          ds_read_b32 touches land in different halves of the 64 banks)
 // With RAGGED, mn_valid (1..BM rows/columns of the tile that exist) and k_valid (k of the
 // K-step that exist, a multiple of one chunk) clamp the SOURCE address into the matrix: lanes
 // whose data does not exist fetch a neighbouring chunk instead.  Rows/columns past the edge
 // only ever reach accumulators that the epilogue does not store; k past the end is zeroed
 // in the fragment registers before it is multiplied.
+// 8-bit MN-contiguous tiles: chunk c of k-row krow is stored at c ^ mn8_swizzle(krow), which puts the eight k-rows that
+// one transposing read touches into different 16-byte bank groups (CH = chunks per k-row)
+template <int CH>
+__device__ __forceinline__ int mn8_swizzle(int krow) { return CH >= 8 ? (krow & 7) : ((krow & 7) >> 1); }
+
 template <bool KC, bool RAGGED, int WB, int ES>
 __device__ __forceinline__ void dma_offsets(uint32_t (&off)[WB], int64_t ld, int wave, int lane, int mn_valid, int k_valid) {
     constexpr int CH = RingGeom<WB, ES>::CHUNKS, VEL = RingGeom<WB, ES>::VEL;
@@ -104,7 +122,7 @@ __device__ __forceinline__ void dma_offsets(uint32_t (&off)[WB], int64_t ld, int
             off[jj] = (uint32_t)(((int64_t)row * ld + kv * VEL) * ES);
         } else {
             int krow = (64 / CH) * j + lane / CH;
-            int chunk = (lane % CH) ^ (ES == 2 ? 2 * (krow & 3) : ES == 4 ? 8 * ((krow >> 2) & 1) : 0);   // Float64: stored as is
+            int chunk = (lane % CH) ^ (ES == 2 ? 2 * (krow & 3) : ES == 4 ? 8 * ((krow >> 2) & 1) : ES == 1 ? mn8_swizzle<CH>(krow) : 0);   // Float64: stored as is
             if constexpr (RAGGED) {
                 krow = krow < k_valid ? krow : k_valid - 1;
                 chunk = chunk < mn_valid / VEL ? chunk : mn_valid / VEL - 1;
@@ -332,6 +350,16 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
         const int chunk = (mnl >> 3) ^ (2 * e);
         return krow * G::MN_ROW_BYTES + chunk * 16 + (mnl & 7) * 2;
     };
+    // 8-bit: ds_read_b64_tr_b8 works on groups of 16 lanes; lane i of a group reads the 8 bytes (mn) 8 (i & 1) .. + 7 of
+    // k-row i >> 1 and receives, as lane s, the 8 consecutive k of mn s.  Read t (0, 1) of a block covers
+    // k = 32 ks + 16 (lane / 32) + 8 t .. + 7 for mn = 32 blk + lane % 32.
+    auto frag_off_mm8 = [&](int wbase, int blk, int ks, int t) -> int {
+        const int grp = lane >> 4, i = lane & 15;
+        const int krow = 32 * ks + 16 * (grp >> 1) + 8 * t + (i >> 1);
+        const int mnl = wbase + blk * 32 + 16 * (grp & 1) + 8 * (i & 1);
+        const int chunk = (mnl >> 4) ^ mn8_swizzle<G::CHUNKS>(krow);
+        return krow * G::MN_ROW_BYTES + chunk * 16 + (mnl & 15);
+    };
     auto frag_off_mm32 = [&](int wbase, int blk, int ks, int e) -> int {
         const int krow = 8 * ks + 4 * (lane >> 5) + e;
         const int mnl = wbase + blk * 32 + (lane & 31);
@@ -347,6 +375,12 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
             frag[r] = *reinterpret_cast<const u32x4*>(tile + frag_off_km(wbase, r, ks));
         } else if constexpr (ES == 4) {
             frag[r >> 2][r & 3] = *reinterpret_cast<const uint32_t*>(tile + frag_off_mm32(wbase, r >> 2, ks, r & 3));
+        } else if constexpr (ES == 1) {
+            const int blk = r >> 1, t = r & 1;
+            const intx2v v = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
+                (__attribute__((address_space(3))) intx2v*)(tile + frag_off_mm8(wbase, blk, ks, t)));
+            frag[blk][2 * t] = (uint32_t)v[0];
+            frag[blk][2 * t + 1] = (uint32_t)v[1];
         } else {
             const int blk = r >> 1, half = r & 1;
             const shortx4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
@@ -357,19 +391,21 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
             frag[blk][2 * half + 1] = w[1];
         }
     };
-    constexpr int MNR = ES == 2 ? 2 * WB : 4 * WB;       // reads of an MN-major operand per half-step
+    constexpr int MNR = ES == 4 ? 4 * WB : 2 * WB;       // reads of an MN-major operand per half-step
     constexpr int NRA = A_KC ? WB : MNR, NRB = B_KC ? WB : MNR, NR = NRA + NRB;
-    constexpr int MPP = ES == 2 ? 1 : 4;                 // MFMAs per pair of fragments
+    constexpr int MPP = ES == 4 ? 4 : 1;                 // MFMAs per pair of fragments
     constexpr int NMMA = WB * WB * MPP;                  // MFMAs per half-step
     constexpr int RPM = (NR + NMMA - 1) / NMMA;          // LDS reads slotted behind each MFMA
 
-    floatx16 acc[WB][WB];
+    using AccV = typename E::AccV;
+    using AccS = typename E::AccS;
+    AccV acc[WB][WB];
 #pragma unroll
     for (int i = 0; i < WB; ++i)
 #pragma unroll
         for (int j = 0; j < WB; ++j)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = (AccS)0;
 
     // K-steps past the end are clamped to the last one: the tail iterations then issue the
     // same DMA traffic as the steady state (into stages nobody reads any more), which keeps
@@ -413,7 +449,7 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
             // serpentine order: consecutive MFMAs always share one operand fragment
             const int e = q / (WB * WB), pr = q % (WB * WB);
             const int i = pr / WB, j = (i & 1) ? WB - 1 - (pr % WB) : (pr % WB);
-            if constexpr (ES == 2) {
+            if constexpr (ES != 4) {
                 E::mma(acc[i][j], bf[cur_buf][j], af[cur_buf][i]);   // D rows <-> n, cols <-> m
             } else {
                 // (copies first: __builtin_bit_cast applied to a vector-element lvalue reads element 0)
@@ -527,7 +563,9 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
     char* Cb = reinterpret_cast<char*>(C);
     const int col = 8 * (lane % LPR);              // this lane's 8 consecutive columns in the slab
     const int n = n0 + wn * WT + col;
-    constexpr int NV = ES / 2;                     // 16-byte vectors of C per lane and row: 8 columns of 2 or 4 bytes
+    constexpr int NV = ES == 4 ? 2 : 1;            // 16-byte vectors of C per lane and row: 8 columns of 1 (half a vector), 2 or 4 bytes
+    typedef AccS accx4 __attribute__((ext_vector_type(4)));
+    typedef uint32_t u32x2v __attribute__((ext_vector_type(2)));
     auto epilogue = [&](auto cmode_tag) {
         constexpr int CM = decltype(cmode_tag)::value;
         const T* bias = static_cast<const T*>(p.bias);
@@ -541,9 +579,14 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
                     const int m = m0 + wm * WT + 32 * i + RPS * t + lane / LPR;
 #pragma unroll
                     for (int v = 0; v < NV; ++v) {
-                        if (!RAGGED || (m < p.M && n + 4 * v < p.N))
-                            c0[t][v] = *reinterpret_cast<const u32x4*>(Cb + ((int64_t)m * p.ldc + n) * ES + 16 * v);
-                        else c0[t][v] = u32x4{0u, 0u, 0u, 0u};
+                        if (!RAGGED || (m < p.M && n + 4 * v < p.N)) {
+                            if constexpr (ES == 1) {
+                                const u32x2v c8 = *reinterpret_cast<const u32x2v*>(Cb + (int64_t)m * p.ldc + n);
+                                c0[t][v] = u32x4{c8[0], c8[1], 0u, 0u};
+                            } else {
+                                c0[t][v] = *reinterpret_cast<const u32x4*>(Cb + ((int64_t)m * p.ldc + n) * ES + 16 * v);
+                            }
+                        } else c0[t][v] = u32x4{0u, 0u, 0u, 0u};
                     }
                 }
             }
@@ -552,40 +595,41 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
             for (int j = 0; j < WB; ++j)
 #pragma unroll
                 for (int rq = 0; rq < 4; ++rq) {
-                    floatx4v v = {acc[i][j][4 * rq], acc[i][j][4 * rq + 1], acc[i][j][4 * rq + 2], acc[i][j][4 * rq + 3]};
+                    accx4 v = {acc[i][j][4 * rq], acc[i][j][4 * rq + 1], acc[i][j][4 * rq + 2], acc[i][j][4 * rq + 3]};
                     const int slot = 8 * j + 2 * rq + (lane >> 5);
-                    *reinterpret_cast<floatx4v*>(slab + (lane & 31) * SROW + ((slot ^ (lane & 7)) * 16)) = v;
+                    *reinterpret_cast<accx4*>(slab + (lane & 31) * SROW + ((slot ^ (lane & 7)) * 16)) = v;
                 }
             // 32 rows x WT cols: NSTEP steps of RPS rows; a lane owns 8 consecutive columns
 #pragma unroll
             for (int t = 0; t < NSTEP; ++t) {
                 const int row = RPS * t + lane / LPR;
                 const int sl = 2 * (lane % LPR);
-                const floatx4v lo = *reinterpret_cast<const floatx4v*>(slab + row * SROW + ((sl ^ (row & 7)) * 16));
-                const floatx4v hi = *reinterpret_cast<const floatx4v*>(slab + row * SROW + (((sl + 1) ^ (row & 7)) * 16));
-                float v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                const accx4 lo = *reinterpret_cast<const accx4*>(slab + row * SROW + ((sl ^ (row & 7)) * 16));
+                const accx4 hi = *reinterpret_cast<const accx4*>(slab + row * SROW + (((sl + 1) ^ (row & 7)) * 16));
+                AccS v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
                 const int m = m0 + wm * WT + 32 * i + row;
                 // 16-bit: N % 8 == 0, a lane's 8 columns exist or not together; Float32: N % 4 == 0, the halves separately
                 if (RAGGED && (m >= p.M || n >= p.N)) continue;
-                const bool hi_ok = !RAGGED || ES == 2 || n + 4 < p.N;
-                if constexpr (CM == C_PARTIAL) {
+                const bool hi_ok = !RAGGED || ES != 4 || n + 4 < p.N;
+                if constexpr (CM == C_PARTIAL && ES != 1) {
                     // split-K: the fp32 sums of this k range go to a float matrix; rounding happens after the reduction
                     float* wp = static_cast<float*>(p.C) + (int64_t)b * p.sC + (int64_t)m * p.ldc + n;
-                    *reinterpret_cast<floatx4v*>(wp) = lo;
-                    if (hi_ok) *reinterpret_cast<floatx4v*>(wp + 4) = hi;
+                    *reinterpret_cast<accx4*>(wp) = lo;
+                    if (hi_ok) *reinterpret_cast<accx4*>(wp + 4) = hi;
                     continue;
                 }
                 if constexpr (CM == C_ACCUMULATE) {
 #pragma unroll
                     for (int e = 0; e < 8; ++e) {
                         if constexpr (ES == 2) v[e] += Cvt16<DT>::up((uint16_t)(c0[t][0][e >> 1] >> (16 * (e & 1))));
+                        else if constexpr (ES == 1) v[e] += (int)((c0[t][0][e >> 2] >> (8 * (e & 3))) & 0xffu);
                         else { const uint32_t cu = c0[t][e >> 2][e & 3]; v[e] += __builtin_bit_cast(float, cu); }
                     }
                 } else if constexpr (CM == C_BIAS) {
 #pragma unroll
                     for (int e = 0; e < 8; ++e)
-                        if (ES == 2 || e < 4 || hi_ok)
-                            v[e] += (float)bias[(int64_t)b * p.bias_bs + (int64_t)m * p.bias_rs + (int64_t)(n + e) * p.bias_cs];
+                        if (ES != 4 || e < 4 || hi_ok)
+                            v[e] += (AccS)bias[(int64_t)b * p.bias_bs + (int64_t)m * p.bias_rs + (int64_t)(n + e) * p.bias_cs];
                 }
                 char* cp = Cb + ((int64_t)m * p.ldc + n) * ES;
                 if constexpr (ES == 2) {
@@ -594,9 +638,16 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
                     for (int e = 0; e < 4; ++e)
                         o[e] = (uint32_t)Cvt16<DT>::down(v[2 * e]) | ((uint32_t)Cvt16<DT>::down(v[2 * e + 1]) << 16);
                     *reinterpret_cast<u32x4*>(cp) = o;
+                } else if constexpr (ES == 1) {
+                    u32x2v o;                       // the low 8 bits of each sum: wrapping arithmetic in the element type
+#pragma unroll
+                    for (int h = 0; h < 2; ++h)
+                        o[h] = ((uint32_t)v[4 * h] & 0xffu) | (((uint32_t)v[4 * h + 1] & 0xffu) << 8) |
+                               (((uint32_t)v[4 * h + 2] & 0xffu) << 16) | ((uint32_t)v[4 * h + 3] << 24);
+                    *reinterpret_cast<u32x2v*>(cp) = o;
                 } else {
-                    *reinterpret_cast<floatx4v*>(cp) = floatx4v{v[0], v[1], v[2], v[3]};
-                    if (hi_ok) *reinterpret_cast<floatx4v*>(cp + 16) = floatx4v{v[4], v[5], v[6], v[7]};
+                    *reinterpret_cast<accx4*>(cp) = accx4{v[0], v[1], v[2], v[3]};
+                    if (hi_ok) *reinterpret_cast<accx4*>(cp + 16) = accx4{v[4], v[5], v[6], v[7]};
                 }
             }
         }
@@ -613,7 +664,7 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
 // to the tile.  Per-lane DMA offsets are 32-bit: 256 rows of lda elements must stay below 4 GiB.
 static inline bool ring_eligible(const GemmParams& p, bool ta, int es = 2) {
     const int vel = 16 / es;
-    const int64_t ldmax = es == 2 ? (1 << 22) : (1 << 21);
+    const int64_t ldmax = (int64_t)(1 << 23) / es;
     return p.K >= vel && p.K % vel == 0 && p.N % vel == 0 && (!ta || p.M % vel == 0) &&
            !p.Aptr && !p.Bptr && !p.Cptr && p.vecA_ok && p.vecB_ok &&
            p.ldc % vel == 0 && p.sC % vel == 0 && p.lda < ldmax && p.ldb < ldmax &&

@@ -99,6 +99,7 @@ static inline int64_t elem_size(int dt) {
 // launchers implemented in the .hip files; all return a hipError_t
 hipError_t launch_gemm_mfma(int dtype, bool ta, bool tb, const GemmParams& p, hipStream_t s);
 hipError_t launch_gemm_valu(int dtype, bool ta, bool tb, const GemmParams& p, hipStream_t s);
+hipError_t launch_gemm_mfma_i8(int dtype, bool ta, bool tb, const GemmParams& p, hipStream_t s);   // Int8 / UInt8: MFMA where rows are 16-byte multiples
 hipError_t launch_gemm_skinny(int dtype, bool ta, bool tb, const GemmParams& p, hipStream_t s, bool* handled);
 // op(B) is the im2col matrix of the image at p.B (tb: its transpose); floating dtypes only
 hipError_t launch_conv_mfma(int dtype, bool tb, const GemmParams& p, hipStream_t s);

@@ -85,7 +85,9 @@ int launch_gemm(ntg::GemmParams p, int dtype, bool ta, bool tb, hipStream_t s) {
     p.vecA_ok = (p.lda % ve == 0) && (p.Aptr || p.sA % ve == 0);
     p.vecB_ok = (p.ldb % ve == 0) && (p.Bptr || p.sB % ve == 0);
     hipError_t e;
-    if (is_int_dtype(dtype)) {
+    if (dtype == ntg::DT_I8 || dtype == ntg::DT_U8) {
+        e = ntg::launch_gemm_mfma_i8(dtype, ta, tb, p, s);
+    } else if (is_int_dtype(dtype)) {
         e = ntg::launch_gemm_valu(dtype, ta, tb, p, s);
     } else {
         bool handled = false;

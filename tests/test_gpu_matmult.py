@@ -131,6 +131,54 @@ def test_device_integers_bit_exact(dtype, shape):
         assert got.tobytes() == ref.tobytes()
 
 
+@pytest.mark.parametrize("dtype", [np.int8, np.uint8], ids=["int8", "uint8"])
+@pytest.mark.parametrize("shape", [(128, 64, 128), (256, 192, 256), (272, 80, 144), (1040, 528, 2064), (4096, 1024, 4096), (48, 16, 16)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_int8_matrix_pipe_bit_exact(dtype, shape):
+    """Int8 / UInt8 with 16-byte rows (sizes multiples of 16) run on v_mfma_i32_32x32x32_i8: every result byte must equal the
+    reference's wrapping arithmetic over the full value range, in all four transpose forms (both LDS layouts, the
+    transposing 8-bit reads), on 64-, 128- and 256-wide tiles, ragged edges and k tails, all three C modes, batches; and
+    must equal the vector-ALU kernel (the same product with rows that are not 16-byte multiples takes that path)."""
+    m, k, n = shape
+    rng = np.random.default_rng(3100 + m)
+
+    def exact(x, y):      # |sum| < 2^27: exact in float64, and BLAS-fast (numpy has no fast integer matmul)
+        return (x.astype(np.float64) @ y.astype(np.float64)).astype(np.int64)
+
+    info = np.iinfo(dtype)
+    big = m >= 4096
+    for ta, tb in TRANS:
+        a = rng.integers(info.min, info.max, (m, k), dtype=dtype, endpoint=True)
+        b = rng.integers(info.min, info.max, (k, n), dtype=dtype, endpoint=True)
+        c0 = rng.integers(info.min, info.max, (m, n), dtype=dtype, endpoint=True)
+        sa = np.ascontiguousarray(a.T) if ta else a
+        sb = np.ascontiguousarray(b.T) if tb else b
+        # exact reference, then wrap to 8 bits
+        ref = (exact(a, b) + c0.astype(np.int64)).astype(dtype)
+        got = dev_matmult(sa, sb, c0, m, k, n, ta, tb, dtype)
+        assert got.tobytes() == ref.tobytes(), (shape, ta, tb)
+        if not big:
+            assert oracle.matmult2d(sa, sb, c0.copy(), ta, tb).tobytes() == ref.tobytes()
+        got0 = dev_matmult(sa, sb, c0, m, k, n, ta, tb, dtype, mode=_lib.C_OVERWRITE)
+        assert got0.tobytes() == (exact(a, b)).astype(dtype).tobytes()
+        if big:
+            break
+    # bias mode and a batch with a broadcast operand, through the dispatcher mirror
+    ta_, tb_ = to_torch(a, DEV, False), to_torch(b, DEV, False)
+    bias = rng.integers(info.min, info.max, (n,), dtype=dtype, endpoint=True)
+    y = F.linear(ta_, tb_, to_torch(bias, DEV, False))
+    refy = (exact(a, b) + bias.astype(np.int64)).astype(dtype)
+    assert from_torch(y).tobytes() == refy.tobytes()
+    if not big:
+        a3 = rng.integers(info.min, info.max, (3, m, k), dtype=dtype, endpoint=True)
+        out = F.matmult(to_torch(a3, DEV, False), tb_)
+        ref3 = np.stack([exact(a3[i], b).astype(dtype) for i in range(3)])
+        assert from_torch(out).tobytes() == ref3.tobytes()
+        # the same values through the vector-ALU kernel: drop one column of B (rows are no longer 16-byte multiples)
+        outv = F.matmult(ta_, to_torch(np.ascontiguousarray(b[:, :n - 1]), DEV, False))
+        assert from_torch(outv).tobytes() == exact(a, b[:, :n - 1]).astype(dtype).tobytes()
+
+
 @pytest.mark.parametrize("dtype", [np.float32, np.float16, "bf16", np.float64])
 def test_c_modes(dtype):
     """overwrite ignores the incoming C (even NaN); accumulate adds to it."""
