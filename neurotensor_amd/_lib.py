@@ -62,6 +62,7 @@ SIGNATURES = {
     "ntg_unfold2d_dev": (_ci, [_ci, _vp, _vp] + [_i64] * 12 + [_vp]),
     "ntg_conv2d_workspace_bytes": (_i64, [_ci] + [_i64] * 12),
     "ntg_conv2d_forward_workspace_bytes": (_i64, [_ci] + [_i64] * 12),
+    "ntg_conv2d_fast_workspace_bytes": (_i64, [_ci] + [_i64] * 14),
     "ntg_conv2d_backward_workspace_bytes": (_i64, [_ci] + [_i64] * 14),
     "ntg_conv_transpose2d_workspace_bytes": (_i64, [_ci] + [_i64] * 16),
     "ntg_conv_transpose2d_dev": (_ci, [_ci, _vp, _vp, _vp, _vp, _i64] + [_i64] * 16 + [_vp]),

@@ -42,4 +42,7 @@ hipError_t launch_conv_mfma_f32(bool tb, int nd, const GemmParams& p, hipStream_
     if (nd == 2 && ring_conv_eligible(p)) return ring_f32_tile_edge(p) == 128 ? launch_ring_conv_cfg<2>(tb, p, s) : launch_ring_conv_cfg<1>(tb, p, s);
     return nd == 3 ? launch_conv_nd_f32<3>(tb, p, s) : launch_conv_nd_f32<2>(tb, p, s);
 }
+hipError_t launch_conv_nhwc_f32(const GemmParams& p, hipStream_t s) {
+    return ring_f32_tile_edge(p) == 128 ? launch_ring_nhwc_cfg<DT_F32, 2>(p, s) : launch_ring_nhwc_cfg<DT_F32, 1>(p, s);
+}
 }  // namespace ntg

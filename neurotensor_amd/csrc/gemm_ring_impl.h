@@ -149,7 +149,7 @@ __device__ __forceinline__ void dma_dword(const void* addr, uint32_t lds_addr) {
                  :: "s"(lds_addr), "v"(addr) : "memory");
 }
 // what the padding taps of a gathered convolution operand read
-static __device__ const uint32_t ring_zero_word[4] = {0u, 0u, 0u, 0u};
+static __device__ __attribute__((aligned(16))) const uint32_t ring_zero_word[4] = {0u, 0u, 0u, 0u};
 
 template <int WB>
 __device__ __forceinline__ void dma_tile(const void* sbase, const uint32_t (&off)[WB], uint32_t lds_tile, int wave_u) {
@@ -174,11 +174,14 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
     using T = typename E::T;
     constexpr int ES = sizeof(T);
     using G = RingGeom<WB, ES>;
-    constexpr bool A_KC = !TA, B_KC = CONV ? false : TB;
+    constexpr bool GATHER4 = CONV == 1 || CONV == 2;     // op(B) gathered element by element from an NCHW image
+    constexpr bool GATHER16 = CONV == 3;                 // op(B) = col^T gathered in 16-byte pieces from a channels-last image
+    constexpr bool A_KC = !TA, B_KC = GATHER4 ? false : GATHER16 ? true : TB;
     constexpr int BK = G::BK;
     constexpr int WT = G::WT;
-    static_assert(CONV == 0 || (ES == 4 && !TA && RAGGED), "gathered operands: Float32, A stored [m][k], guarded edges");
-    constexpr int NA = WB, NB = CONV ? 4 * WB : WB;      // DMA instructions per wavefront and K-step for the A / B tile
+    static_assert(!GATHER4 || (ES == 4 && !TA && RAGGED), "gathered operands: Float32, A stored [m][k], guarded edges");
+    static_assert(!GATHER16 || ((ES == 4 || ES == 2) && !TA && RAGGED), "channels-last gather: 16/32-bit floats, A stored [m][k], guarded edges");
+    constexpr int NA = WB, NB = GATHER4 ? 4 * WB : WB;   // DMA instructions per wavefront and K-step for the A / B tile
     // B instructions issued in the first / second half-step (the second also carries the A tile's).  Splitting a gathered
     // tile between the two was measured slower than issuing all of it in the first.
     constexpr int NB1 = NB, NB2 = NB - NB1;
@@ -227,7 +230,7 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
     //   weight gradient:  lanepart = byte offset of the tap inside the image slice, cmask = r*d_r | q*d_c << 16,
     //                     0x80008000 (never inside) past the edge
     uint32_t lanepart[WB], cmask[WB];
-    if constexpr (CONV != 0) {
+    if constexpr (GATHER4) {
         const ConvGeom& g = p.conv;
 #pragma unroll
         for (int h = 0; h < WB; ++h) {
@@ -260,7 +263,7 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
     // contribute (padding included, so it may be negative).
     int st_lo[4], st_mid[4], st_up[4], st_k[4];
     int cv_r0 = 1, cv_r1 = 1, cv_dlo = 0, cv_dmid = 0, cv_dup = 0, cv_carry_lo = 0, cv_carry_mid = 0;
-    if constexpr (CONV != 0) {
+    if constexpr (GATHER4) {
         const ConvGeom& g = p.conv;
         const int s_lo = (CONV == 1 ? g.d_c : g.s_c) * 4, s_mid = (CONV == 1 ? g.d_r : g.s_r) * g.W * 4, s_hi = g.chan * 4;
         cv_r0 = CONV == 1 ? g.k_c : g.Wo;
@@ -288,7 +291,7 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
     // Instruction x (0 .. 4 WB - 1) of this wavefront's share of the NEXT gathered tile (tiles are gathered in K order):
     // k-row 4 wave + x / WB, columns 64 (x % WB) .. + 63; the k-row's state moves on after its last instruction.
     auto conv_dma = [&](int x, uint32_t lds_tile) __attribute__((always_inline)) {
-        if constexpr (CONV != 0) {
+        if constexpr (GATHER4) {
             const ConvGeom& g = p.conv;
             const int i = x / WB, h = x % WB;
             const int krow = 4 * wave_u + i;
@@ -320,6 +323,60 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
     auto conv_tile = [&](uint32_t lds_tile) __attribute__((always_inline)) {
 #pragma unroll
         for (int x = 0; x < 4 * WB; ++x) conv_dma(x, lds_tile);
+    };
+
+    // ---- channels-last gather (CONV = 3): the image at p.B is stored [pixel][channel] (p.conv.chan = channels per pixel),
+    // the weights at A [m][(r, q, c)], so a K-step is 64 bytes of consecutive channels of ONE tap for every output pixel:
+    // the B tile [pixel row][64 B] is filled by the same WB 16-byte DMA instructions per wavefront as a stored K-major
+    // operand, each lane's address being a wave-uniform term of the K-step (tap and first channel, advanced by counters
+    // in scalar registers) plus a per-lane term of its output pixel and 16-byte slot; padding taps read zeros.
+    uint32_t lanepart3[WB], cmask3[WB];
+    int k3_c0 = 0, k3_q = 0, k3_r = 0, k3_up = 0, k3_k = 0, k3_cg = 1;
+    if constexpr (GATHER16) {
+        const ConvGeom& g = p.conv;
+        k3_cg = p.K / g.k_rc;
+        k3_up = -(g.p_r * g.W + g.p_c) * g.chan * ES;
+#pragma unroll
+        for (int x = 0; x < WB; ++x) {
+            const int row = 16 * (wave * WB + x) + (lane >> 2);
+            const int n = n0 + row;
+            const uint32_t l = n < p.N ? (uint32_t)n : 0u;
+            const uint32_t oh = fast_div(l, g.div_wo), ow = l - oh * (uint32_t)g.Wo;
+            const int ih0 = (int)oh * g.s_r - g.p_r, iw0 = (int)ow * g.s_c - g.p_c;
+            uint32_t m = 0;
+#pragma unroll
+            for (int t = 0; t < 8; ++t) {
+                if (t < g.k_r && (unsigned)(ih0 + t * g.d_r) < (unsigned)g.H) m |= 1u << t;
+                if (t < g.k_c && (unsigned)(iw0 + t * g.d_c) < (unsigned)g.W) m |= 256u << t;
+            }
+            cmask3[x] = n < p.N ? m : 0u;
+            const uint32_t kv = (uint32_t)((lane & 3) ^ ((row >> 1) & 3));
+            lanepart3[x] = (oh * (uint32_t)g.s_r * (uint32_t)g.W + ow * (uint32_t)g.s_c) * (uint32_t)g.chan * (uint32_t)ES + kv * 16u;
+        }
+    }
+    // instruction x (0 .. WB - 1) of this wavefront's share of the NEXT gathered tile; the K-step's counters move on after the last
+    auto conv3_dma = [&](int x, uint32_t lds_tile) __attribute__((always_inline)) {
+        if constexpr (GATHER16) {
+            const ConvGeom& g = p.conv;
+            const char* img = reinterpret_cast<const char*>(B);
+            const uint32_t sr = k3_k < p.K ? (uint32_t)k3_r : 31u, sq = 8u + (uint32_t)k3_q;
+            const bool ok = ((cmask3[x] >> sr) & (cmask3[x] >> sq) & 1u) != 0u;
+            const char* src = ok ? img + (int64_t)k3_up + lanepart3[x] : reinterpret_cast<const char*>(ring_zero_word);
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+                         :: "s"(lds_tile + (uint32_t)(wave_u * WB + x) * 1024u), "v"(src) : "memory");
+            if (x == WB - 1) {
+                int c0 = k3_c0 + BK, up = k3_up + BK * ES, q = k3_q, r = k3_r;
+                const bool w0 = c0 >= k3_cg;
+                c0 = w0 ? c0 - k3_cg : c0;
+                up = w0 ? up - k3_cg * ES + g.d_c * g.chan * ES : up;
+                q = w0 ? q + 1 : q;
+                const bool w1 = q >= g.k_c;
+                q = w1 ? 0 : q;
+                up = w1 ? up - g.k_c * g.d_c * g.chan * ES + g.d_r * g.W * g.chan * ES : up;
+                r = w1 ? r + 1 : r;
+                k3_c0 = c0; k3_up = up; k3_q = q; k3_r = r; k3_k += BK;
+            }
+        }
     };
 
     // uniform (scalar) source pointer of one operand tile
@@ -363,7 +420,7 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
     auto frag_off_mm32 = [&](int wbase, int blk, int ks, int e) -> int {
         const int krow = 8 * ks + 4 * (lane >> 5) + e;
         const int mnl = wbase + blk * 32 + (lane & 31);
-        if constexpr (CONV != 0) return krow * G::MN_ROW_BYTES + mnl * 4;          // gathered tiles are stored unswizzled
+        if constexpr (GATHER4) return krow * G::MN_ROW_BYTES + mnl * 4;            // gathered tiles are stored unswizzled
         return krow * G::MN_ROW_BYTES + ((mnl * 4) ^ (128 * (lane >> 5)));      // (krow >> 2) & 1 == lane / 32
     };
 
@@ -415,7 +472,11 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
 
     // prologue: tiles 0..2 and the A half of tile 3 in flight (3 (NA + NB) + NA instructions)
     auto b_tile = [&](int kt, uint32_t lds_tile) __attribute__((always_inline)) {
-        if constexpr (CONV != 0) conv_tile(lds_tile);      // (tiles past the last one are all zeros; nobody reads them)
+        if constexpr (GATHER4) conv_tile(lds_tile);        // (tiles past the last one are all zeros; nobody reads them)
+        else if constexpr (GATHER16) {
+#pragma unroll
+            for (int x = 0; x < WB; ++x) conv3_dma(x, lds_tile);
+        }
         else dma_tile<WB>(srcB(kt), kt >= last ? offBt : offB, lds_tile, wave_u);
     };
     dma_tile<WB>(srcA(0), 0 >= last ? offAt : offA, lds_addr_of(st0), wave_u);
@@ -521,7 +582,8 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
             const uint32_t lds_tile = lds_addr_of(prv) + G::TILE_BYTES;
             mma_step_prefetch(0, cur, 1, 1, std::integral_constant<int, NB1>{}, std::integral_constant<int, (CONV ? NB1 : 0)>{},
                               [&](int x) __attribute__((always_inline)) {
-                if constexpr (CONV != 0) conv_dma(x, lds_tile);
+                if constexpr (GATHER4) conv_dma(x, lds_tile);
+                else if constexpr (GATHER16) conv3_dma(x, lds_tile);
                 else dma_1k(src, (RAGGED && tail) ? offBt[x] : offB[x], lds_tile + (uint32_t)(wave_u * WB + x) * 1024u);
             });
         }
@@ -564,6 +626,8 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
     const int col = 8 * (lane % LPR);              // this lane's 8 consecutive columns in the slab
     const int n = n0 + wn * WT + col;
     constexpr int NV = ES == 4 ? 2 : 1;            // 16-byte vectors of C per lane and row: 8 columns of 1 (half a vector), 2 or 4 bytes
+    // (only the channels-last convolution meets rows of C that are not 16-byte multiples; uniform)
+    const bool c_rows_16 = !GATHER16 || (p.ldc % G::VEL == 0 && p.sC % G::VEL == 0 && (reinterpret_cast<uintptr_t>(p.C) & 15) == 0);
     typedef AccS accx4 __attribute__((ext_vector_type(4)));
     typedef uint32_t u32x2v __attribute__((ext_vector_type(2)));
     auto epilogue = [&](auto cmode_tag) {
@@ -575,7 +639,7 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
             u32x4 c0[NSTEP][NV];
             if constexpr (CM == C_ACCUMULATE) {
 #pragma unroll
-                for (int t = 0; t < NSTEP; ++t) {
+                for (int t = 0; t < NSTEP && c_rows_16; ++t) {
                     const int m = m0 + wm * WT + 32 * i + RPS * t + lane / LPR;
 #pragma unroll
                     for (int v = 0; v < NV; ++v) {
@@ -610,6 +674,21 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
                 const int m = m0 + wm * WT + 32 * i + row;
                 // 16-bit: N % 8 == 0, a lane's 8 columns exist or not together; Float32: N % 4 == 0, the halves separately
                 if (RAGGED && (m >= p.M || n >= p.N)) continue;
+                if constexpr (GATHER16) {
+                    // output planes whose rows are not 16-byte multiples (Ho*Wo = 49, 900, ...): element-wise stores
+                    if (!c_rows_16) {
+                        T* ce = reinterpret_cast<T*>(Cb) + (int64_t)m * p.ldc + n;
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) {
+                            if (n + e >= p.N) break;
+                            AccS val = v[e];
+                            if constexpr (CM == C_ACCUMULATE) val += (AccS)ce[e];
+                            else if constexpr (CM == C_BIAS) val += (AccS)bias[(int64_t)b * p.bias_bs + (int64_t)m * p.bias_rs + (int64_t)(n + e) * p.bias_cs];
+                            ce[e] = (T)val;
+                        }
+                        continue;
+                    }
+                }
                 const bool hi_ok = !RAGGED || ES != 4 || n + 4 < p.N;
                 if constexpr (CM == C_PARTIAL && ES != 1) {
                     // split-K: the fp32 sums of this k range go to a float matrix; rounding happens after the reduction
@@ -699,6 +778,20 @@ static hipError_t launch_ring_conv_cfg(bool tb, const GemmParams& pin, hipStream
     if (blocks > 0x7fffffffLL) return hipErrorInvalidValue;
     if (tb) hipLaunchKernelGGL((gemm_ring_kernel<DT_F32, false, false, true, WB, 2>), dim3((unsigned)blocks), dim3(256), 0, s, p);
     else hipLaunchKernelGGL((gemm_ring_kernel<DT_F32, false, false, true, WB, 1>), dim3((unsigned)blocks), dim3(256), 0, s, p);
+    return hipGetLastError();
+}
+
+// convolution with op(B) gathered in 16-byte pieces from a channels-last image (see CONV = 3)
+template <int DT, int WB>
+static hipError_t launch_ring_nhwc_cfg(const GemmParams& pin, hipStream_t s) {
+    constexpr int TE = RingGeom<WB, (int)sizeof(typename Elem<DT>::T)>::BM;
+    GemmParams p = pin;
+    p.tiles_m = (p.M + TE - 1) / TE;
+    p.tiles_n = (p.N + TE - 1) / TE;
+    const int64_t blocks = (int64_t)p.tiles_m * p.tiles_n * p.batch;
+    if (blocks <= 0) return hipSuccess;
+    if (blocks > 0x7fffffffLL) return hipErrorInvalidValue;
+    hipLaunchKernelGGL((gemm_ring_kernel<DT, false, true, true, WB, 3>), dim3((unsigned)blocks), dim3(256), 0, s, p);
     return hipGetLastError();
 }
 

@@ -24,6 +24,18 @@ hipError_t launch_conv_mfma_f64(bool tb, int nd, const GemmParams& p, hipStream_
 hipError_t launch_conv_mfma_f16(bool tb, int nd, const GemmParams& p, hipStream_t s);
 hipError_t launch_conv_mfma_bf16(bool tb, int nd, const GemmParams& p, hipStream_t s);
 
+hipError_t launch_conv_nhwc_f32(const GemmParams& p, hipStream_t s);
+hipError_t launch_conv_nhwc_f16(const GemmParams& p, hipStream_t s);
+hipError_t launch_conv_nhwc_bf16(const GemmParams& p, hipStream_t s);
+hipError_t launch_conv_nhwc(int dtype, const GemmParams& p, hipStream_t s) {
+    switch (dtype) {
+    case DT_F32: return launch_conv_nhwc_f32(p, s);
+    case DT_F16: return launch_conv_nhwc_f16(p, s);
+    case DT_BF16: return launch_conv_nhwc_bf16(p, s);
+    default: return hipErrorInvalidValue;
+    }
+}
+
 hipError_t launch_conv_mfma(int dtype, bool tb, int nd, const GemmParams& p, hipStream_t s) {
     switch (dtype) {
     case DT_F32: return launch_conv_mfma_f32(tb, nd, p, s);
@@ -517,6 +529,80 @@ static int conv_forward_gather(int dtype, const void* image, const void* kernel,
     return NTG_OK;
 }
 
+// A 1x1 kernel with unit stride and no padding unfolds the image onto itself (col_b == x_b as a [C, H*W] matrix), so the
+// convolution is the batched product W_g . x_b on the image where it lies.  Integer dtypes always take it; the floating
+// ones when rows of the image and of W are 16-byte multiples (what the DMA-fed kernels need), else they gather.
+static bool conv_pointwise(const Geo3& g) {
+    for (int a = 0; a < 3; ++a)
+        if (g.k[a] != 1 || g.s[a] != 1 || g.p[a] != 0) return false;
+    return true;
+}
+static bool conv_pointwise_ok(int dtype, int64_t channels, int64_t groups, const Geo3& g) {
+    if (!conv_pointwise(g)) return false;
+    if (is_int_dtype(dtype)) return true;
+    const int64_t es = ntg::elem_size(dtype);
+    return (g.L() * es) % 16 == 0 && (channels / groups * es) % 16 == 0;
+}
+static int conv_forward_pointwise(int dtype, const void* image, const void* kernel, void* out, int64_t batch, int64_t channels,
+                                  int64_t out_channels, const Geo3& g, int64_t groups, void* stream) {
+    const int64_t es = ntg::elem_size(dtype), cg = channels / groups, og = out_channels / groups, L = g.L();
+    for (int64_t gi = 0; gi < groups; ++gi) {
+        ntg_gemm_desc d;
+        std::memset(&d, 0, sizeof d);
+        d.dtype = dtype; d.c_mode = NTG_C_OVERWRITE;
+        d.m = og; d.k = cg; d.n = L;
+        d.lda = cg; d.ldb = L; d.ldc = L;
+        d.batches = batch;
+        d.stride_a = 0; d.stride_b = channels * L; d.stride_c = out_channels * L;
+        int rc = ntg_gemm_dev(&d, static_cast<const char*>(kernel) + gi * og * cg * es, static_cast<const char*>(image) + gi * cg * L * es,
+                              static_cast<char*>(out) + gi * og * L * es, stream);
+        if (rc) return rc;
+    }
+    return NTG_OK;
+}
+
+// Channels-last form of the same convolution, for the floating dtypes up to 32 bits: the image is first copied to
+// [B][pixel][C] and the weights to [O][(taps, c)] in the workspace; then one K-step of the product is 64 bytes of consecutive
+// channels of one tap, and the kernel's DMA gathers the operand in 16-byte pieces instead of element by element.
+static bool conv_nhwc_ok(int dtype, int64_t channels, int64_t out_channels, int64_t groups, const Geo3& g) {
+    if (dtype != ntg::DT_F32 && dtype != ntg::DT_F16 && dtype != ntg::DT_BF16) return false;
+    if (g.nd != 2 || !conv_implicit_g(dtype, channels, g)) return false;
+    const int64_t es = ntg::elem_size(dtype), cg = channels / groups;
+    return cg % (64 / es) == 0 && out_channels > 0 && channels * g.vol() * es < 0x7fffffffLL;
+}
+static int64_t conv_nhwc_workspace(int dtype, int64_t batch, int64_t channels, int64_t out_channels, int64_t groups, const Geo3& g) {
+    const int64_t es = ntg::elem_size(dtype);
+    return (int64_t)align_up((size_t)(batch * channels * g.vol() * es), 256) + out_channels * (channels / groups) * g.taps() * es;
+}
+static int conv_forward_nhwc(int dtype, const void* image, const void* kernel, void* out, void* ws, int64_t batch, int64_t channels,
+                             int64_t out_channels, const Geo3& g, int64_t groups, hipStream_t hs) {
+    const int64_t es = ntg::elem_size(dtype), cg = channels / groups, og = out_channels / groups;
+    const int64_t L = g.L(), taps = g.taps(), vol = g.vol(), K = taps * cg;
+    char* ws_img = static_cast<char*>(ws);
+    char* ws_w = ws_img + align_up((size_t)(batch * channels * vol * es), 256);
+    hipError_t e = ntg::launch_nchw_to_nhwc(es, image, ws_img, batch, channels, vol, hs);
+    if (e != hipSuccess) return hip_fail(e, "channels-last copy launch");
+    e = ntg::launch_weights_channels_last(es, kernel, ws_w, out_channels, cg, taps, hs);
+    if (e != hipSuccess) return hip_fail(e, "weight permutation launch");
+    for (int64_t gi = 0; gi < groups; ++gi) {
+        ntg::GemmParams p;
+        std::memset(&p, 0, sizeof p);
+        p.M = (int)og; p.K = (int)K; p.N = (int)L; p.batch = (int)batch;
+        p.A = ws_w + gi * og * K * es;
+        p.B = ws_img + gi * cg * es;
+        p.C = static_cast<char*>(out) + gi * og * L * es;
+        p.lda = K; p.ldb = channels; p.ldc = L;
+        p.sA = 0; p.sB = channels * vol; p.sC = out_channels * L;
+        p.cmode = ntg::C_OVERWRITE;
+        p.vecA_ok = 1; p.vecB_ok = 1;
+        fill_conv_geom(p.conv, cg, g);
+        p.conv.chan = (int)channels;               // elements from one pixel to the next
+        e = ntg::launch_conv_nhwc(dtype, p, hs);
+        if (e != hipSuccess) return hip_fail(e, "channels-last convolution launch");
+    }
+    return NTG_OK;
+}
+
 // dW: one batched GEMM  P_{b,g} [og, add] = dY_{b,g} [og, L] . col_{b,g}^T  with col gathered from the image, into
 // ws [B][O][add]; then the per-image results are summed in batch order (the same additions, in the same order, as
 // accumulating one GEMM per image into dW, conv.cpp:466-469).
@@ -589,6 +675,19 @@ static ConvBackwardPlan plan_conv_backward_g(int dtype, bool want_dx, bool want_
     return pl;
 }
 
+int64_t ntg_conv2d_fast_workspace_bytes(int dtype, int64_t batch, int64_t channels, int64_t height, int64_t width,
+                                        int64_t out_channels, int64_t k_r, int64_t k_c, int64_t s_r, int64_t s_c,
+                                        int64_t p_r, int64_t p_c, int64_t d_r, int64_t d_c, int64_t groups) {
+    const int64_t es = ntg::elem_size(dtype);
+    int64_t Ho, Wo;
+    if (es == 0 || unfold_out(height, width, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c, Ho, Wo)) return -1;
+    const Geo3 g = geo2(height, width, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c, Ho, Wo);
+    const bool groups_ok = groups >= 1 && channels % groups == 0 && out_channels % groups == 0;      // (the call itself reports bad groups)
+    if (groups_ok && conv_pointwise_ok(dtype, channels, groups, g)) return 0;
+    if (groups_ok && conv_nhwc_ok(dtype, channels, out_channels, groups, g)) return conv_nhwc_workspace(dtype, batch, channels, out_channels, groups, g);
+    return ntg_conv2d_forward_workspace_bytes(dtype, batch, channels, height, width, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c);
+}
+
 int64_t ntg_conv2d_forward_workspace_bytes(int dtype, int64_t batch, int64_t channels, int64_t height, int64_t width,
                                            int64_t k_r, int64_t k_c, int64_t s_r, int64_t s_c,
                                            int64_t p_r, int64_t p_c, int64_t d_r, int64_t d_c) {
@@ -596,6 +695,7 @@ int64_t ntg_conv2d_forward_workspace_bytes(int dtype, int64_t batch, int64_t cha
     int64_t Ho, Wo;
     if (es == 0 || unfold_out(height, width, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c, Ho, Wo)) return -1;
     if (conv_implicit(dtype, channels, height, width, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c, Ho, Wo)) return 0;
+    if (conv_pointwise(geo2(height, width, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c, Ho, Wo))) return 0;
     return batch * channels * k_r * k_c * Ho * Wo * es;
 }
 
@@ -630,6 +730,13 @@ int ntg_conv2d_dev(int dtype, const void* image, const void* kernel, void* out,
     const int64_t add = (channels / groups) * k_r * k_c, og = out_channels / groups;
     {
         const Geo3 g = geo2(height, width, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c, Ho, Wo);
+        if (conv_pointwise_ok(dtype, channels, groups, g) &&
+            (is_int_dtype(dtype) || ((reinterpret_cast<uintptr_t>(image) | reinterpret_cast<uintptr_t>(kernel) | reinterpret_cast<uintptr_t>(out)) & 15) == 0))
+            return conv_forward_pointwise(dtype, image, kernel, out, batch, channels, out_channels, g, groups, stream);
+        // with the workspace of ntg_conv2d_fast_workspace_bytes: channels-last copy of the image, 16-byte gathers
+        if (conv_nhwc_ok(dtype, channels, out_channels, groups, g) && workspace && (reinterpret_cast<uintptr_t>(workspace) & 15) == 0 &&
+            workspace_bytes >= conv_nhwc_workspace(dtype, batch, channels, out_channels, groups, g))
+            return conv_forward_nhwc(dtype, image, kernel, out, workspace, batch, channels, out_channels, g, groups, static_cast<hipStream_t>(stream));
         if (conv_implicit_g(dtype, channels, g))      // col_b is never stored: the GEMM's B loader gathers it from the image
             return conv_forward_gather(dtype, image, kernel, out, batch, channels, out_channels, g, groups, static_cast<hipStream_t>(stream));
     }
@@ -673,7 +780,7 @@ int ntg_conv2d(int dtype, const void* image, const void* kernel, void* out,
     const size_t im_bytes = (size_t)(batch * channels * height * width * es);
     const size_t k_bytes = (size_t)(out_channels * (channels / groups) * k_r * k_c * es);
     const size_t o_bytes = (size_t)(batch * out_channels * Ho * Wo * es);
-    const int64_t ws = ntg_conv2d_forward_workspace_bytes(dtype, batch, channels, height, width, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c);
+    const int64_t ws = ntg_conv2d_fast_workspace_bytes(dtype, batch, channels, height, width, out_channels, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c, groups);
     DeviceMem mem;
     const size_t ok_ = align_up(im_bytes, 256), oo = ok_ + align_up(k_bytes, 256), ow = oo + align_up(o_bytes, 256);
     HIP_TRY(mem.alloc(ow + (size_t)ws));

@@ -152,4 +152,65 @@ hipError_t launch_flip_weights(int64_t es, const void* w, void* wt, int64_t grou
     return hipGetLastError();
 }
 
+// out[b][p][c] = in[b][c][p]: an image batch from channel planes to channels-last, 64 x 64 tiles through LDS so that
+// both the loads (along p) and the stores (along c) are coalesced.
+template <class T>
+__global__ void __launch_bounds__(256) nchw_to_nhwc_kernel(const T* __restrict__ in, T* __restrict__ out, const int64_t C, const int64_t P) {
+    __shared__ T tile[64][65];
+    const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+    const int64_t p0 = (int64_t)blockIdx.x * 64, c0 = (int64_t)blockIdx.y * 64, b = blockIdx.z;
+    const T* src = in + b * C * P;
+    T* dst = out + b * C * P;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        const int64_t c = c0 + ty + 4 * i, pp = p0 + tx;
+        if (c < C && pp < P) tile[ty + 4 * i][tx] = src[c * P + pp];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        const int64_t pp = p0 + ty + 4 * i, c = c0 + tx;
+        if (c < C && pp < P) dst[pp * C + c] = tile[tx][ty + 4 * i];
+    }
+}
+
+hipError_t launch_nchw_to_nhwc(int64_t es, const void* in, void* out, int64_t batch, int64_t C, int64_t P, hipStream_t s) {
+    if (batch * C * P == 0) return hipSuccess;
+    const int64_t gx = (P + 63) / 64, gy = (C + 63) / 64;
+    if (gx > 0x7fffffffLL || gy > 65535 || batch > 65535) return hipErrorInvalidValue;
+    const dim3 g((unsigned)gx, (unsigned)gy, (unsigned)batch), t(256);
+    switch (es) {
+    case 2: hipLaunchKernelGGL(nchw_to_nhwc_kernel<uint16_t>, g, t, 0, s, (const uint16_t*)in, (uint16_t*)out, C, P); break;
+    case 4: hipLaunchKernelGGL(nchw_to_nhwc_kernel<uint32_t>, g, t, 0, s, (const uint32_t*)in, (uint32_t*)out, C, P); break;
+    default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+
+// wp[o][t][c] = w[o][c][t]: convolution weights with the channel index fastest (the k order of the channels-last gather)
+template <class T>
+__global__ void __launch_bounds__(256) weights_channels_last_kernel(const T* __restrict__ w, T* __restrict__ wp, const int64_t rows,
+                                                                    const int64_t cg, const int64_t taps) {
+    const int64_t total = rows * cg * taps;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += stride) {
+        const int64_t c = idx % cg;
+        const int64_t t = (idx / cg) % taps;
+        const int64_t o = idx / (cg * taps);
+        wp[idx] = w[(o * cg + c) * taps + t];
+    }
+}
+
+hipError_t launch_weights_channels_last(int64_t es, const void* w, void* wp, int64_t rows, int64_t cg, int64_t taps, hipStream_t s) {
+    const int64_t total = rows * cg * taps;
+    if (total == 0) return hipSuccess;
+    const dim3 g(grid_for(total)), t(256);
+    switch (es) {
+    case 2: hipLaunchKernelGGL(weights_channels_last_kernel<uint16_t>, g, t, 0, s, (const uint16_t*)w, (uint16_t*)wp, rows, cg, taps); break;
+    case 4: hipLaunchKernelGGL(weights_channels_last_kernel<uint32_t>, g, t, 0, s, (const uint32_t*)w, (uint32_t*)wp, rows, cg, taps); break;
+    default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+
 }  // namespace ntg

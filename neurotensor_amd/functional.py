@@ -273,7 +273,7 @@ def conv2d(image, kernel, stride=1, padding=0, dilation=1, groups=1):
         raise ValueError(f"Expected kernel rows times groups to be equal to rows of image Conv2d but got {Cg} * {groups} != {C}")
     L = load()
     dt = ntg_dtype(x)
-    ws_bytes = L.ntg_conv2d_forward_workspace_bytes(dt, B, C, H, W, kh, kw, s[0], s[1], p[0], p[1], d[0], d[1])
+    ws_bytes = L.ntg_conv2d_fast_workspace_bytes(dt, B, C, H, W, O, kh, kw, s[0], s[1], p[0], p[1], d[0], d[1], groups)
     if ws_bytes < 0:
         raise ValueError("the array of sliding blocks would be empty")
     Ho = (H + 2 * p[0] - d[0] * (kh - 1) - 1) // s[0] + 1

@@ -70,6 +70,20 @@ def test_argument_errors_do_not_need_a_device():
     assert lib.ntg_conv2d_forward_workspace_bytes(_lib.FLOAT32, 1, 3, 8, 8, 3, 3, 1, 1, 1, 1, 1, 1) == 0
     assert lib.ntg_conv2d_forward_workspace_bytes(_lib.INT32, 1, 3, 8, 8, 3, 3, 1, 1, 1, 1, 1, 1) == 27 * 64 * 4
     assert lib.ntg_conv2d_forward_workspace_bytes(_lib.FLOAT32, 1, 3, 16, 16, 9, 3, 1, 1, 4, 1, 1, 1) == 27 * 3 * 256 * 4
+    # a 1x1 kernel with unit stride and no padding is a product on the image where it lies: no buffer for any dtype
+    assert lib.ntg_conv2d_forward_workspace_bytes(_lib.INT32, 2, 3, 8, 8, 1, 1, 1, 1, 0, 0, 1, 1) == 0
+    assert lib.ntg_conv2d_forward_workspace_bytes(_lib.INT32, 2, 3, 8, 8, 1, 1, 2, 1, 0, 0, 1, 1) == 2 * 3 * 4 * 8 * 4
+    # the faster forward form: channels-last copy of the image (256-byte aligned) + permuted weights, when the channels of
+    # a group fill whole 64-byte runs; else what the plain query says
+    fast = lib.ntg_conv2d_fast_workspace_bytes
+    assert fast(_lib.BFLOAT16, 2, 64, 7, 7, 48, 3, 3, 1, 1, 1, 1, 1, 1, 2) == 12544 + 48 * 32 * 9 * 2    # 2*64*49*2 = 12544
+    assert fast(_lib.FLOAT32, 1, 16, 5, 5, 8, 3, 3, 1, 1, 1, 1, 1, 1, 1) == 1792 + 8 * 16 * 9 * 4        # 1600 -> 1792
+    assert fast(_lib.BFLOAT16, 1, 16, 5, 5, 8, 3, 3, 1, 1, 1, 1, 1, 1, 1) == 0                            # 32 bytes of channels: gathers
+    assert fast(_lib.FLOAT64, 1, 16, 5, 5, 8, 3, 3, 1, 1, 1, 1, 1, 1, 1) == 0
+    assert fast(_lib.INT32, 1, 16, 5, 5, 8, 3, 3, 1, 1, 1, 1, 1, 1, 1) == 16 * 9 * 25 * 4
+    assert fast(_lib.FLOAT32, 4, 64, 8, 8, 32, 1, 1, 1, 1, 0, 0, 1, 1, 1) == 0                            # 1x1: product in place
+    assert fast(_lib.FLOAT32, 4, 64, 7, 7, 32, 1, 1, 1, 1, 0, 0, 1, 1, 1) == 50176 + 32 * 64 * 4   # rows of 196 bytes
+    assert fast(_lib.FLOAT32, 1, 16, 2, 2, 8, 3, 3, 1, 1, 0, 0, 1, 1, 1) == -1                            # kernel larger than the image
     # per-image weight gradients [B, O, C/g * taps] instead of the im2col matrix
     assert lib.ntg_conv2d_backward_workspace_bytes(_lib.FLOAT32, 2, 4, 8, 8, 6, 3, 3, 1, 1, 1, 1, 1, 1, 2) == 2 * 6 * 2 * 9 * 4
     assert lib.ntg_conv2d_backward_workspace_bytes(_lib.FLOAT32, 2, 4, 8, 8, 6, 3, 3, 1, 1, 1, 1, 1, 1, 3) == -1

@@ -315,6 +315,10 @@ IMPLICIT_GEOMS = [
     (2, 4, 9, 9, 6, 3, 3, 3, (4, 0), (1, 2), 2),          # padding wider than the kernel reach
     (16, 64, 28, 28, 128, 3, 3, 1, 1, 1, 1),               # enough tiles for the large-tile kernels
     (24, 32, 33, 35, 96, 3, 3, 2, 1, 1, 2),
+    # channel counts that fill whole 64-byte runs (the channels-last gather) with output planes of odd size
+    (4, 64, 15, 15, 40, 3, 3, 1, 1, 1, 1),                 # Ho*Wo = 225
+    (3, 64, 14, 14, 48, 3, 3, 2, 1, 1, 2),                 # Ho*Wo = 49, two groups of 32 channels
+    (2, 128, 19, 11, 72, 3, 2, 1, (2, 0), (2, 1), 1),               # Ho*Wo = 190
 ]
 
 
@@ -355,6 +359,37 @@ def test_conv2d_implicit_gather(dtype, geom):
         oref = oracle.conv2d(x, w, s, p, d, groups)
         err = np.abs(out.cpu().numpy().astype(np.float64) - oref.astype(np.float64)).max()
         assert err <= (HALF_REL * scale if dtype == np.float16 else 1e-5 * K * np.abs(x).max() * np.abs(w).max())
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64, np.float16, "bf16", np.int32, np.int8], ids=["fp32", "fp64", "fp16", "bf16", "int32", "int8"])
+def test_conv2d_pointwise_is_a_product_on_the_image(dtype):
+    """1x1 kernel, stride 1, no padding: unfold2d is the identity (conv.cpp:94 multiplies by the image itself), so the
+    library runs W_g . x_b in place without a col buffer -- every dtype, grouped, aligned rows or not.  Integers bit-exact
+    against the oracle's conv2d, floats against torch in double."""
+    bf = dtype == "bf16"
+    integer = dtype in (np.int32, np.int8)
+    rng = np.random.default_rng(1900)
+    lib = _lib.load()
+    for (B, C, H, W, O, groups) in [(3, 64, 8, 12, 40, 1), (2, 96, 7, 7, 64, 2), (5, 24, 9, 5, 18, 3)]:
+        if integer:
+            x = rng.integers(-100, 100, (B, C, H, W)).astype(dtype)
+            w = rng.integers(-100, 100, (O, C // groups, 1, 1)).astype(dtype)
+        else:
+            x = randn(rng, (B, C, H, W), dtype)
+            w = randn(rng, (O, C // groups, 1, 1), dtype, 1.0 / np.sqrt(C // groups))
+        tx, tw = to_torch(x, DEV, bf), to_torch(w, DEV, bf)
+        assert lib.ntg_conv2d_forward_workspace_bytes(F.ntg_dtype(tx), B, C, H, W, 1, 1, 1, 1, 0, 0, 1, 1) == 0
+        out = F.conv2d(tx, tw, groups=groups)
+        assert tuple(out.shape) == (B, O, H, W)
+        if integer:
+            assert np.array_equal(out.cpu().numpy(), oracle.conv2d(x, w, 1, 0, 1, groups))
+            continue
+        ref = torch.nn.functional.conv2d(tx.double(), tw.double(), None, 1, 0, 1, groups)
+        err = (out.double() - ref).abs().max().item()
+        if dtype in (np.float32, np.float64):
+            assert err <= 1e-5 * (C // groups) * float(tx.abs().max() * tw.abs().max())
+        else:
+            assert err <= HALF_REL * ref.abs().max().item()
 
 
 def _gpu_family(golden_dir, name, sfx, fwd, bwd, ofwd, obwd, kw):
