@@ -217,7 +217,10 @@ int ntg_unfold2d_backward_dev(int dtype, const void* col, void* image,
 /* Bytes of device workspace ntg_conv2d_backward_dev needs when both gradients are requested.  Floating dtypes with
  * kernels up to 8x8 compute conv_dkernel (conv.cpp:444-471) without the stored im2col matrix (workspace = the per-image
  * weight gradients, batch * out_channels * channels/groups * k_r * k_c elements) and, at stride 1, conv_dimage
- * (conv.cpp:318-346) as well; every other case needs the im2col-sized buffer (ntg_conv2d_workspace_bytes). */
+ * (conv.cpp:318-346) as well; every other case needs the im2col-sized buffer (ntg_conv2d_workspace_bytes).  Where
+ * conv_dimage can run in its channels-last form (Float32 / Float16 / BFloat16, two axes, stride 1, the out channels of a
+ * group filling whole 64-byte runs) the figure also covers a channels-last copy of grad_out plus the flipped weights; the
+ * call still accepts the smaller amount and then gathers from grad_out as it lies. */
 int64_t ntg_conv2d_backward_workspace_bytes(int dtype, int64_t batch, int64_t channels, int64_t height, int64_t width,
                                             int64_t out_channels, int64_t k_r, int64_t k_c, int64_t s_r, int64_t s_c,
                                             int64_t p_r, int64_t p_c, int64_t d_r, int64_t d_c, int64_t groups);

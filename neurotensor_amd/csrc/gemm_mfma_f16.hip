@@ -19,4 +19,10 @@ hipError_t launch_conv_nhwc_f16(const GemmParams& p, hipStream_t s) {
     if (te == 64) return launch_ring_nhwc_cfg<DT_F16, 1>(p, s);
     return launch_ring_nhwc_cfg<DT_F16, 2>(p, s);
 }
+hipError_t launch_conv_nhwc_dw_f16(const GemmParams& p, hipStream_t s) {
+    const int te = ring16_tile_edge(p.M, p.N, p.K, p.batch);
+    if (te == 256) return launch_ring_nhwc_dw_cfg<DT_F16, 4>(p, s);
+    if (te == 64) return launch_ring_nhwc_dw_cfg<DT_F16, 1>(p, s);
+    return launch_ring_nhwc_dw_cfg<DT_F16, 2>(p, s);
+}
 }  // namespace ntg

@@ -45,4 +45,7 @@ hipError_t launch_conv_mfma_f32(bool tb, int nd, const GemmParams& p, hipStream_
 hipError_t launch_conv_nhwc_f32(const GemmParams& p, hipStream_t s) {
     return ring_f32_tile_edge(p) == 128 ? launch_ring_nhwc_cfg<DT_F32, 2>(p, s) : launch_ring_nhwc_cfg<DT_F32, 1>(p, s);
 }
+hipError_t launch_conv_nhwc_dw_f32(const GemmParams& p, hipStream_t s) {
+    return ring_f32_tile_edge(p) == 128 ? launch_ring_nhwc_dw_cfg<DT_F32, 2>(p, s) : launch_ring_nhwc_dw_cfg<DT_F32, 1>(p, s);
+}
 }  // namespace ntg

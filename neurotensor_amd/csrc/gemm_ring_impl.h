@@ -176,11 +176,13 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
     using G = RingGeom<WB, ES>;
     constexpr bool GATHER4 = CONV == 1 || CONV == 2;     // op(B) gathered element by element from an NCHW image
     constexpr bool GATHER16 = CONV == 3;                 // op(B) = col^T gathered in 16-byte pieces from a channels-last image
-    constexpr bool A_KC = !TA, B_KC = GATHER4 ? false : GATHER16 ? true : TB;
+    constexpr bool GATHERW = CONV == 4;                  // op(B) = col^T of a channels-last image, 16-byte pieces along the channels (weight gradient)
+    constexpr bool A_KC = !TA, B_KC = GATHER4 ? false : GATHER16 ? true : GATHERW ? false : TB;
     constexpr int BK = G::BK;
     constexpr int WT = G::WT;
     static_assert(!GATHER4 || (ES == 4 && !TA && RAGGED), "gathered operands: Float32, A stored [m][k], guarded edges");
     static_assert(!GATHER16 || ((ES == 4 || ES == 2) && !TA && RAGGED), "channels-last gather: 16/32-bit floats, A stored [m][k], guarded edges");
+    static_assert(!GATHERW || ((ES == 4 || ES == 2) && !TA && !TB && RAGGED), "channels-last weight gradient: 16/32-bit floats, A stored [m][k], guarded edges");
     constexpr int NA = WB, NB = GATHER4 ? 4 * WB : WB;   // DMA instructions per wavefront and K-step for the A / B tile
     // B instructions issued in the first / second half-step (the second also carries the A tile's).  Splitting a gathered
     // tile between the two was measured slower than issuing all of it in the first.
@@ -379,6 +381,49 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
         }
     };
 
+    // ---- channels-last weight gradient (CONV = 4): C[o][(r, q, c)] = sum over output pixels l of A[o][l] * x[pixel(l, r, q)][c].
+    // The B tile is the MN-major one of a stored [k][n] operand (k = output pixel, n = (tap, channel)), filled by the same
+    // WB 16-byte DMA instructions per wavefront; a lane's 16 bytes are channels c .. of ONE tap for the whole K loop
+    // (tap reach and byte offset kept per lane), and its k-row moves on by BK output pixels per K-step: the pixel is
+    // split into (row, column) with one multiply-shift division per instruction.  Padding and k >= K read zeros.
+    int krow4[WB], noff4[WB];
+    uint32_t tap4[WB];
+    int k4_k = 0;
+    if constexpr (GATHERW) {
+        const ConvGeom& g = p.conv;
+        constexpr int CH = G::CHUNKS;
+        const uint32_t cgc = (uint32_t)p.N / (uint32_t)g.k_rc;               // channels of the slice: N = taps * channels
+#pragma unroll
+        for (int x = 0; x < WB; ++x) {
+            const int j = wave * WB + x;
+            const int krow = (64 / CH) * j + lane / CH;
+            const int chunk = (lane % CH) ^ (ES == 2 ? 2 * (krow & 3) : 8 * ((krow >> 2) & 1));
+            const int n = n0 + chunk * G::VEL;
+            const uint32_t nn = n < p.N ? (uint32_t)n : 0u;
+            const uint32_t t = nn / cgc, c = nn - t * cgc;
+            const uint32_t r = fast_div(t, g.div_kc), q = t - r * (uint32_t)g.k_c;
+            krow4[x] = n < p.N ? krow : 0x40000000;                       // columns past the edge: never inside
+            tap4[x] = (r * (uint32_t)g.d_r) | ((q * (uint32_t)g.d_c) << 16);
+            noff4[x] = (((int)(r * (uint32_t)g.d_r) - g.p_r) * g.W + ((int)(q * (uint32_t)g.d_c) - g.p_c)) * g.chan * ES + (int)c * ES;
+        }
+    }
+    auto conv4_dma = [&](int x, uint32_t lds_tile) __attribute__((always_inline)) {
+        if constexpr (GATHERW) {
+            const ConvGeom& g = p.conv;
+            const char* img = reinterpret_cast<const char*>(B);
+            const uint32_t l = (uint32_t)(k4_k + krow4[x]);
+            const uint32_t oh = fast_div(l, g.div_wo), ow = l - oh * (uint32_t)g.Wo;
+            const int ih0 = (int)oh * g.s_r - g.p_r, iw0 = (int)ow * g.s_c - g.p_c;
+            const bool ok = (l < (uint32_t)p.K) & ((uint32_t)(ih0 + (int)(tap4[x] & 0xffffu)) < (uint32_t)g.H) &
+                            ((uint32_t)(iw0 + (int)(tap4[x] >> 16)) < (uint32_t)g.W);
+            const int off = (int)((oh * (uint32_t)g.s_r * (uint32_t)g.W + ow * (uint32_t)g.s_c) * (uint32_t)g.chan * (uint32_t)ES) + noff4[x];
+            const char* src = ok ? img + (int64_t)off : reinterpret_cast<const char*>(ring_zero_word);
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+                         :: "s"(lds_tile + (uint32_t)(wave_u * WB + x) * 1024u), "v"(src) : "memory");
+            if (x == WB - 1) k4_k += BK;
+        }
+    };
+
     // uniform (scalar) source pointer of one operand tile
     auto tile_src = [&](const char* base) -> const void* {
         const uint64_t bu = reinterpret_cast<uint64_t>(base);
@@ -476,6 +521,9 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
         else if constexpr (GATHER16) {
 #pragma unroll
             for (int x = 0; x < WB; ++x) conv3_dma(x, lds_tile);
+        } else if constexpr (GATHERW) {
+#pragma unroll
+            for (int x = 0; x < WB; ++x) conv4_dma(x, lds_tile);
         }
         else dma_tile<WB>(srcB(kt), kt >= last ? offBt : offB, lds_tile, wave_u);
     };
@@ -539,7 +587,8 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
             else if (nrd == 1) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
             if constexpr (NGATHER > 0) {
                 // the gather's address arithmetic, dealt out evenly: what does not fit under one MFMA delays the next
-                __builtin_amdgcn_sched_group_barrier(0x002, (8 * NGATHER + NMMA - 1) / NMMA + 1, 0);   // VALU
+                constexpr int VPG = GATHERW ? 20 : 8;          // vector instructions per gathering DMA, roughly
+                __builtin_amdgcn_sched_group_barrier(0x002, (VPG * NGATHER + NMMA - 1) / NMMA + 1, 0);   // VALU
                 __builtin_amdgcn_sched_group_barrier(0x004, (10 * NGATHER + NMMA - 1) / NMMA, 0);      // SALU
             }
         }
@@ -584,6 +633,7 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
                               [&](int x) __attribute__((always_inline)) {
                 if constexpr (GATHER4) conv_dma(x, lds_tile);
                 else if constexpr (GATHER16) conv3_dma(x, lds_tile);
+                else if constexpr (GATHERW) conv4_dma(x, lds_tile);
                 else dma_1k(src, (RAGGED && tail) ? offBt[x] : offB[x], lds_tile + (uint32_t)(wave_u * WB + x) * 1024u);
             });
         }
@@ -792,6 +842,20 @@ static hipError_t launch_ring_nhwc_cfg(const GemmParams& pin, hipStream_t s) {
     if (blocks <= 0) return hipSuccess;
     if (blocks > 0x7fffffffLL) return hipErrorInvalidValue;
     hipLaunchKernelGGL((gemm_ring_kernel<DT, false, true, true, WB, 3>), dim3((unsigned)blocks), dim3(256), 0, s, p);
+    return hipGetLastError();
+}
+
+// weight gradient of a convolution with op(B) gathered from a channels-last image (see CONV = 4)
+template <int DT, int WB>
+static hipError_t launch_ring_nhwc_dw_cfg(const GemmParams& pin, hipStream_t s) {
+    constexpr int TE = RingGeom<WB, (int)sizeof(typename Elem<DT>::T)>::BM;
+    GemmParams p = pin;
+    p.tiles_m = (p.M + TE - 1) / TE;
+    p.tiles_n = (p.N + TE - 1) / TE;
+    const int64_t blocks = (int64_t)p.tiles_m * p.tiles_n * p.batch;
+    if (blocks <= 0) return hipSuccess;
+    if (blocks > 0x7fffffffLL) return hipErrorInvalidValue;
+    hipLaunchKernelGGL((gemm_ring_kernel<DT, false, false, true, WB, 4>), dim3((unsigned)blocks), dim3(256), 0, s, p);
     return hipGetLastError();
 }
 

@@ -36,6 +36,18 @@ hipError_t launch_conv_nhwc(int dtype, const GemmParams& p, hipStream_t s) {
     }
 }
 
+hipError_t launch_conv_nhwc_dw_f32(const GemmParams& p, hipStream_t s);
+hipError_t launch_conv_nhwc_dw_f16(const GemmParams& p, hipStream_t s);
+hipError_t launch_conv_nhwc_dw_bf16(const GemmParams& p, hipStream_t s);
+hipError_t launch_conv_nhwc_dw(int dtype, const GemmParams& p, hipStream_t s) {
+    switch (dtype) {
+    case DT_F32: return launch_conv_nhwc_dw_f32(p, s);
+    case DT_F16: return launch_conv_nhwc_dw_f16(p, s);
+    case DT_BF16: return launch_conv_nhwc_dw_bf16(p, s);
+    default: return hipErrorInvalidValue;
+    }
+}
+
 hipError_t launch_conv_mfma(int dtype, bool tb, int nd, const GemmParams& p, hipStream_t s) {
     switch (dtype) {
     case DT_F32: return launch_conv_mfma_f32(tb, nd, p, s);
@@ -658,8 +670,91 @@ static int conv_dimage_gather(int dtype, const void* kernel, const void* grad_ou
     return NTG_OK;
 }
 
+// The same gradient through the channels-last kernel: dY is copied to [B][pixel][O] and the flipped weights to
+// [C][(taps, oc)] in the workspace, when the out channels of a group fill whole 64-byte runs.
+static bool conv_dimage_nhwc_ok(int dtype, int64_t channels, int64_t out_channels, int64_t groups, const Geo3& g) {
+    return conv_nhwc_ok(dtype, out_channels, channels, groups, geo_dimage(g));
+}
+static int64_t conv_dimage_nhwc_workspace(int dtype, int64_t batch, int64_t channels, int64_t out_channels, int64_t groups, const Geo3& g) {
+    return conv_nhwc_workspace(dtype, batch, out_channels, channels, groups, geo_dimage(g));
+}
+static int conv_dimage_nhwc(int dtype, const void* kernel, const void* grad_out, void* d_image, void* ws, int64_t batch,
+                            int64_t channels, int64_t out_channels, const Geo3& g, int64_t groups, int accumulate, hipStream_t hs) {
+    const int64_t es = ntg::elem_size(dtype), cg = channels / groups, og = out_channels / groups;
+    const int64_t L = g.L(), taps = g.taps(), vol = g.vol(), K = taps * og;
+    char* ws_gy = static_cast<char*>(ws);
+    char* ws_w = ws_gy + align_up((size_t)(batch * out_channels * L * es), 256);
+    hipError_t e = ntg::launch_nchw_to_nhwc(es, grad_out, ws_gy, batch, out_channels, L, hs);
+    if (e != hipSuccess) return hip_fail(e, "channels-last copy launch");
+    e = ntg::launch_flip_weights_channels_last(es, kernel, ws_w, groups, og, cg, taps, hs);
+    if (e != hipSuccess) return hip_fail(e, "weight flip launch");
+    const Geo3 t = geo_dimage(g);
+    for (int64_t gi = 0; gi < groups; ++gi) {
+        ntg::GemmParams p;
+        std::memset(&p, 0, sizeof p);
+        p.M = (int)cg; p.K = (int)K; p.N = (int)vol; p.batch = (int)batch;
+        p.A = ws_w + gi * cg * K * es;
+        p.B = ws_gy + gi * og * es;
+        p.C = static_cast<char*>(d_image) + gi * cg * vol * es;
+        p.lda = K; p.ldb = out_channels; p.ldc = vol;
+        p.sA = 0; p.sB = out_channels * L; p.sC = channels * vol;
+        p.cmode = accumulate ? ntg::C_ACCUMULATE : ntg::C_OVERWRITE;
+        p.vecA_ok = 1; p.vecB_ok = 1;
+        fill_conv_geom(p.conv, og, t);
+        p.conv.chan = (int)out_channels;
+        e = ntg::launch_conv_nhwc(dtype, p, hs);
+        if (e != hipSuccess) return hip_fail(e, "channels-last conv_dimage launch");
+    }
+    return NTG_OK;
+}
+
+// dW through the channels-last kernel: the image is copied to [B][pixel][C]; per image and group
+// P_{b,g} [og][(taps, c)] = dY_{b,g} [og, L] . col^T gathered 16 bytes of channels at a time; the per-image results are
+// summed in batch order into the kernel's [O][c][taps] layout.  Needs rows of dY and the channels of a group to be
+// 16-byte multiples.
+static bool conv_dkernel_nhwc_ok(int dtype, int64_t channels, int64_t out_channels, int64_t groups, const Geo3& g) {
+    if (dtype != ntg::DT_F32 && dtype != ntg::DT_F16 && dtype != ntg::DT_BF16) return false;
+    if (g.nd != 2 || !conv_implicit_g(dtype, channels, g)) return false;
+    const int64_t es = ntg::elem_size(dtype), cg = channels / groups;
+    if (g.k[1] * g.d[1] >= 32768 || g.k[2] * g.d[2] >= 32768) return false;      // tap reach packed in 16 bits
+    return (cg * es) % 16 == 0 && (g.L() * es) % 16 == 0 && out_channels > 0 && cg * g.taps() < 0x7fffffffLL;
+}
+static int64_t conv_dkernel_nhwc_workspace(int dtype, int64_t batch, int64_t channels, int64_t out_channels, int64_t groups, const Geo3& g) {
+    const int64_t es = ntg::elem_size(dtype);
+    return (int64_t)align_up((size_t)(batch * channels * g.vol() * es), 256) + batch * out_channels * (channels / groups) * g.taps() * es;
+}
+static int conv_dkernel_nhwc(int dtype, const void* image, const void* grad_out, void* d_kernel, void* ws, int64_t batch,
+                             int64_t channels, int64_t out_channels, const Geo3& g, int64_t groups, int accumulate, hipStream_t hs) {
+    const int64_t es = ntg::elem_size(dtype), cg = channels / groups, og = out_channels / groups;
+    const int64_t L = g.L(), taps = g.taps(), vol = g.vol(), N = taps * cg;
+    char* ws_img = static_cast<char*>(ws);
+    char* ws_part = ws_img + align_up((size_t)(batch * channels * vol * es), 256);
+    hipError_t e = ntg::launch_nchw_to_nhwc(es, image, ws_img, batch, channels, vol, hs);
+    if (e != hipSuccess) return hip_fail(e, "channels-last copy launch");
+    for (int64_t gi = 0; gi < groups; ++gi) {
+        ntg::GemmParams p;
+        std::memset(&p, 0, sizeof p);
+        p.M = (int)og; p.K = (int)L; p.N = (int)N; p.batch = (int)batch;
+        p.A = static_cast<const char*>(grad_out) + gi * og * L * es;
+        p.B = ws_img + gi * cg * es;
+        p.C = ws_part + gi * og * N * es;
+        p.lda = L; p.ldb = channels; p.ldc = N;
+        p.sA = out_channels * L; p.sB = channels * vol; p.sC = out_channels * N;
+        p.cmode = ntg::C_OVERWRITE;
+        p.vecA_ok = 1; p.vecB_ok = 1;
+        fill_conv_geom(p.conv, cg, g);
+        p.conv.chan = (int)channels;               // elements from one pixel to the next
+        e = ntg::launch_conv_nhwc_dw(dtype, p, hs);
+        if (e != hipSuccess) return hip_fail(e, "channels-last conv_dkernel launch");
+    }
+    // (groups are consecutive row blocks of both layouts, so one pass covers them all)
+    e = ntg::launch_reduce_batch_taps_last(dtype, ws_part, d_kernel, batch, out_channels, cg, taps, accumulate, hs);
+    if (e != hipSuccess) return hip_fail(e, "weight gradient reduction launch");
+    return NTG_OK;
+}
+
 // Which backward gradients run as implicit GEMMs, and the workspace the call needs.
-struct ConvBackwardPlan { bool gather_dw, gather_dx; int64_t need; };
+struct ConvBackwardPlan { bool gather_dw, gather_dx, nhwc_dx, nhwc_dw; int64_t need, need_nhwc_dx, need_nhwc_dw; };
 static ConvBackwardPlan plan_conv_backward_g(int dtype, bool want_dx, bool want_dw, int64_t batch, int64_t channels, int64_t out_channels,
                                              const Geo3& g, int64_t groups) {
     const int64_t es = ntg::elem_size(dtype);
@@ -672,6 +767,11 @@ static ConvBackwardPlan plan_conv_backward_g(int dtype, bool want_dx, bool want_
     if (want_dw) need = std::max(need, pl.gather_dw ? batch * out_channels * cg * taps * es : col);
     if (want_dx) need = std::max(need, pl.gather_dx ? out_channels * cg * taps * es : col);
     pl.need = need;
+    // the channels-last form of dX is taken when the caller's workspace also holds the copy of dY
+    pl.nhwc_dx = pl.gather_dx && g.nd == 2 && conv_dimage_nhwc_ok(dtype, channels, out_channels, groups, g);
+    pl.need_nhwc_dx = pl.nhwc_dx ? conv_dimage_nhwc_workspace(dtype, batch, channels, out_channels, groups, g) : 0;
+    pl.nhwc_dw = pl.gather_dw && conv_dkernel_nhwc_ok(dtype, channels, out_channels, groups, g);
+    pl.need_nhwc_dw = pl.nhwc_dw ? conv_dkernel_nhwc_workspace(dtype, batch, channels, out_channels, groups, g) : 0;
     return pl;
 }
 
@@ -852,8 +952,10 @@ int64_t ntg_conv2d_backward_workspace_bytes(int dtype, int64_t batch, int64_t ch
     int64_t Ho, Wo;
     if (ntg::elem_size(dtype) == 0 || groups < 1 || channels % groups != 0 || out_channels % groups != 0 ||
         unfold_out(height, width, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c, Ho, Wo)) return -1;
-    return plan_conv_backward(dtype, true, true, batch, channels, height, width, out_channels, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c,
-                              groups, Ho, Wo).need;
+    // the larger of what the call needs at least and what lets dX take its channels-last form (copy of dY + flipped weights)
+    const ConvBackwardPlan pl = plan_conv_backward(dtype, true, true, batch, channels, height, width, out_channels, k_r, k_c, s_r, s_c, p_r, p_c,
+                                                   d_r, d_c, groups, Ho, Wo);
+    return std::max(pl.need, std::max(pl.need_nhwc_dx, pl.need_nhwc_dw));
 }
 
 int ntg_conv2d_backward_dev(int dtype, const void* image, const void* kernel, const void* grad_out,
@@ -888,11 +990,17 @@ int ntg_conv2d_backward_dev(int dtype, const void* image, const void* kernel, co
     const bool gather_dw = plan.gather_dw, gather_dx = plan.gather_dx;
     const Geo3 geo = geo2(height, width, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c, Ho, Wo);
     if (gather_dw) {
-        rc = conv_dkernel_gather(dtype, image, grad_out, d_kernel, ws, batch, channels, out_channels, geo, groups, accumulate, hs);
+        if (plan.nhwc_dw && workspace_bytes >= plan.need_nhwc_dw && ((reinterpret_cast<uintptr_t>(ws) | reinterpret_cast<uintptr_t>(grad_out)) & 15) == 0)
+            rc = conv_dkernel_nhwc(dtype, image, grad_out, d_kernel, ws, batch, channels, out_channels, geo, groups, accumulate, hs);
+        else
+            rc = conv_dkernel_gather(dtype, image, grad_out, d_kernel, ws, batch, channels, out_channels, geo, groups, accumulate, hs);
         if (rc) return rc;
     }
     if (gather_dx) {
-        rc = conv_dimage_gather(dtype, kernel, grad_out, d_image, ws, batch, channels, out_channels, geo, groups, accumulate, hs);
+        if (plan.nhwc_dx && workspace_bytes >= plan.need_nhwc_dx && (reinterpret_cast<uintptr_t>(ws) & 15) == 0)
+            rc = conv_dimage_nhwc(dtype, kernel, grad_out, d_image, ws, batch, channels, out_channels, geo, groups, accumulate, hs);
+        else
+            rc = conv_dimage_gather(dtype, kernel, grad_out, d_image, ws, batch, channels, out_channels, geo, groups, accumulate, hs);
         if (rc) return rc;
     }
     if (gather_dw) d_kernel = nullptr;    // done

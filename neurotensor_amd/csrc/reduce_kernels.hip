@@ -19,6 +19,22 @@ __global__ void __launch_bounds__(256) reduce_batch_kernel(const T* __restrict__
 }
 
 
+// The same ordered sum for per-image weight gradients held channels-last, part[b][o][t][c], into the kernel's own layout
+// out[o][c][t]: threads follow the partial sums (coalesced reads of the large side), the small result is written scattered.
+template <class T, class Acc>
+__global__ void __launch_bounds__(256) reduce_batch_taps_last_kernel(const T* __restrict__ part, T* __restrict__ out, const int64_t batch,
+                                                                     const int64_t rows, const int64_t cg, const int64_t taps, const int accumulate) {
+    const int64_t n = rows * cg * taps;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+        const int64_t c = i % cg, t = (i / cg) % taps, o = i / (cg * taps);
+        T* dst = out + (o * cg + c) * taps + t;
+        Acc acc = accumulate ? (Acc)*dst : (Acc)0;
+        for (int64_t b = 0; b < batch; ++b) acc += (Acc)part[b * n + i];
+        *dst = (T)acc;
+    }
+}
+
 // Split-K epilogue: C (+)= sum over the k ranges of part[s][m][n], s ascending, starting from C0 (the incoming C, the
 // broadcast bias, or zero).  One rounding to T at the end.
 template <class T, class P, class Acc>
@@ -139,6 +155,20 @@ hipError_t launch_reduce_batch(int dtype, const void* part, void* out, int64_t b
     return hipGetLastError();
 }
 
+hipError_t launch_reduce_batch_taps_last(int dtype, const void* part, void* out, int64_t batch, int64_t rows, int64_t cg, int64_t taps,
+                                         int accumulate, hipStream_t s) {
+    const int64_t n = rows * cg * taps;
+    if (n == 0) return hipSuccess;
+    const dim3 g(grid_for(n)), b(256);
+    switch (dtype) {
+    case DT_F32: hipLaunchKernelGGL((reduce_batch_taps_last_kernel<float, float>), g, b, 0, s, (const float*)part, (float*)out, batch, rows, cg, taps, accumulate); break;
+    case DT_F16: hipLaunchKernelGGL((reduce_batch_taps_last_kernel<_Float16, float>), g, b, 0, s, (const _Float16*)part, (_Float16*)out, batch, rows, cg, taps, accumulate); break;
+    case DT_BF16: hipLaunchKernelGGL((reduce_batch_taps_last_kernel<__bf16, float>), g, b, 0, s, (const __bf16*)part, (__bf16*)out, batch, rows, cg, taps, accumulate); break;
+    default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+
 hipError_t launch_flip_weights(int64_t es, const void* w, void* wt, int64_t groups, int64_t og, int64_t cg, int64_t taps, hipStream_t s) {
     const int64_t total = groups * og * cg * taps;
     if (total == 0) return hipSuccess;
@@ -199,6 +229,36 @@ __global__ void __launch_bounds__(256) weights_channels_last_kernel(const T* __r
         const int64_t o = idx / (cg * taps);
         wp[idx] = w[(o * cg + c) * taps + t];
     }
+}
+
+// wt[g][c][t][oc] = w[g*og + oc][c][taps-1-t]: the weights of the convolution that maps the output gradient back to the
+// image (channel axes swapped inside each group, taps reversed), with the out channels of one tap consecutive.
+template <class T>
+__global__ void __launch_bounds__(256) flip_weights_channels_last_kernel(const T* __restrict__ w, T* __restrict__ wt, const int64_t groups,
+                                                                         const int64_t og, const int64_t cg, const int64_t taps) {
+    const int64_t total = groups * og * cg * taps;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += stride) {
+        const int64_t oc = idx % og;
+        int64_t r = idx / og;
+        const int64_t t = r % taps;
+        r /= taps;
+        const int64_t c = r % cg;
+        const int64_t g = r / cg;
+        wt[idx] = w[((g * og + oc) * cg + c) * taps + (taps - 1 - t)];
+    }
+}
+
+hipError_t launch_flip_weights_channels_last(int64_t es, const void* w, void* wt, int64_t groups, int64_t og, int64_t cg, int64_t taps, hipStream_t s) {
+    const int64_t total = groups * og * cg * taps;
+    if (total == 0) return hipSuccess;
+    const dim3 g(grid_for(total)), t(256);
+    switch (es) {
+    case 2: hipLaunchKernelGGL(flip_weights_channels_last_kernel<uint16_t>, g, t, 0, s, (const uint16_t*)w, (uint16_t*)wt, groups, og, cg, taps); break;
+    case 4: hipLaunchKernelGGL(flip_weights_channels_last_kernel<uint32_t>, g, t, 0, s, (const uint32_t*)w, (uint32_t*)wt, groups, og, cg, taps); break;
+    default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
 }
 
 hipError_t launch_weights_channels_last(int64_t es, const void* w, void* wp, int64_t rows, int64_t cg, int64_t taps, hipStream_t s) {

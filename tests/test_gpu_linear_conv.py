@@ -239,6 +239,9 @@ BACKWARD_GEOMS = [
     (2, 5, 12, 12, 7, 5, 5, 2, 2, 1, 1),                   # stride 2: dX through the stored col matrix + col2im
     (4, 32, 30, 28, 64, 3, 3, 1, 1, 1, 1),
     (8, 64, 28, 28, 128, 3, 3, 1, 1, 1, 1),                # enough tiles for the large-tile kernels
+    (3, 48, 15, 13, 64, 3, 3, 1, 1, 1, 2),                 # channels-last dX with image planes of odd size (195), two groups
+    (2, 16, 9, 11, 96, 3, 2, 1, (2, 0), (2, 1), 1),
+    (2, 16, 12, 16, 24, 3, 3, (2, 1), (1, 2), (1, 2), 2),  # channels-last dW with stride, dilation and groups (L = 96)
 ]
 
 
