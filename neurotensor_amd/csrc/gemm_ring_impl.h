@@ -865,12 +865,36 @@ static hipError_t launch_ring_wb(bool ta, bool tb, const GemmParams& p, hipStrea
     return tb ? launch_ring_cfg<DT, false, true, WB>(p, s) : launch_ring_cfg<DT, false, false, WB>(p, s);
 }
 
+// items [b0, b0 + nb) of a strided batch as a product of their own
+static inline GemmParams ring_batch_range(const GemmParams& p, int64_t es, int b0, int nb) {
+    GemmParams q = p;
+    q.A = static_cast<const char*>(p.A) + (int64_t)b0 * p.sA * es;
+    q.B = static_cast<const char*>(p.B) + (int64_t)b0 * p.sB * es;
+    q.C = static_cast<char*>(p.C) + (int64_t)b0 * p.sC * es;
+    if (p.bias) q.bias = static_cast<const char*>(p.bias) + (int64_t)b0 * p.bias_bs * es;
+    q.batch = nb;
+    return q;
+}
+
+// 16-bit products: tile edge from the cost estimate; a batch that leaves a small rest of tiles after whole rounds
+// over the CUs goes out as two launches (see ring16_plan).  launch(edge, params) starts one of them.
+template <class Launch>
+static hipError_t launch_ring16_planned(const GemmParams& p, hipStream_t s, Launch&& launch) {
+    Ring16Plan pl = ring16_plan(p.M, p.N, p.K, p.batch);
+    if (p.cmode == C_PARTIAL || p.Aptr || p.Bptr || p.Cptr) pl.head = p.batch;
+    if (pl.head >= p.batch) return launch(pl.edge, p);
+    const hipError_t e = launch(pl.edge, ring_batch_range(p, 2, 0, pl.head));
+    if (e != hipSuccess) return e;
+    return launch(pl.tail_edge, ring_batch_range(p, 2, pl.head, p.batch - pl.head));
+}
+
 template <int DT>
 static hipError_t launch_ring16(bool ta, bool tb, const GemmParams& p, hipStream_t s) {
-    const int te = ring16_tile_edge(p.M, p.N, p.K, p.batch);
-    if (te == 256) return launch_ring_wb<DT, 4>(ta, tb, p, s);
-    if (te == 64) return launch_ring_wb<DT, 1>(ta, tb, p, s);
-    return launch_ring_wb<DT, 2>(ta, tb, p, s);
+    return launch_ring16_planned(p, s, [&](int te, const GemmParams& q) {
+        if (te == 256) return launch_ring_wb<DT, 4>(ta, tb, q, s);
+        if (te == 64) return launch_ring_wb<DT, 1>(ta, tb, q, s);
+        return launch_ring_wb<DT, 2>(ta, tb, q, s);
+    });
 }
 
 }  // namespace ntg

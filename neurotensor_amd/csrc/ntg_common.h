@@ -72,18 +72,43 @@ struct GemmParams {
 // tiles while most CUs are idle and the clock is high), smaller ones spread the work over the 256 CUs more evenly,
 // waste less on the padding of M and N, and hide a tile's prologue and epilogue (about 3 / 1.5 / 0.6 us of exposed
 // latency per tile) behind their neighbours on the CU.  Estimated time = tiles per CU x (tile time + exposed latency).
-static inline int ring16_tile_edge(int64_t M, int64_t N, int64_t K, int64_t batch) {
+static inline double ring16_cost_us(int t, int64_t nt, int64_t K) {
     const double cu_flops_per_us = 9.77e6;                      // 2500 TFLOP/s over 256 CUs
+    const double f = t == 256 ? (nt >= 192 ? 0.5 : 0.64) : t == 128 ? 0.4 : 0.25;
+    const double latency = t == 256 ? 3.0 : t == 128 ? 1.5 : 0.6;
+    return (double)((nt + 255) / 256) * (2.0 * t * t * (double)K / (cu_flops_per_us * f) + latency);
+}
+static inline int64_t ring16_tiles(int t, int64_t M, int64_t N, int64_t batch) { return ((M + t - 1) / t) * ((N + t - 1) / t) * batch; }
+static inline int ring16_tile_edge(int64_t M, int64_t N, int64_t K, int64_t batch) {
     int best = 256;
     double best_us = 0.0;
     for (int t = 256; t >= 64; t /= 2) {
-        const int64_t nt = ((M + t - 1) / t) * ((N + t - 1) / t) * batch;
-        const double f = t == 256 ? (nt >= 192 ? 0.5 : 0.64) : t == 128 ? 0.4 : 0.25;
-        const double latency = t == 256 ? 3.0 : t == 128 ? 1.5 : 0.6;
-        const double us = (double)((nt + 255) / 256) * (2.0 * t * t * (double)K / (cu_flops_per_us * f) + latency);
+        const double us = ring16_cost_us(t, ring16_tiles(t, M, N, batch), K);
         if (t == 256 || us < best_us) { best = t; best_us = us; }
     }
     return best;
+}
+
+// A batched product whose tiles fill the 256 CUs a whole number of times plus a small rest would spend a full tile time
+// on that rest.  The plan then gives the first `head` items the chosen tile (as many as fit in whole rounds) and the
+// remaining ones a tile chosen for them alone (usually the next smaller one, spread over all CUs), as two launches; the
+// estimate has to improve by 7 % (the second launch costs a few microseconds).  head == batch: one launch.
+struct Ring16Plan { int edge, head, tail_edge; };
+static inline Ring16Plan ring16_plan(int64_t M, int64_t N, int64_t K, int64_t batch) {
+    Ring16Plan pl;
+    pl.edge = pl.tail_edge = ring16_tile_edge(M, N, K, batch);
+    pl.head = (int)batch;
+    if (batch < 2 || pl.edge == 64) return pl;
+    const int64_t per_item = ring16_tiles(pl.edge, M, N, 1), total = per_item * batch;
+    const int64_t full = total / 256;
+    if (full < 1 || total % 256 == 0) return pl;
+    const int64_t head = full * 256 / per_item;
+    if (head < 1 || head >= batch) return pl;
+    const int tail_edge = ring16_tile_edge(M, N, K, batch - head);
+    const double split_us = ring16_cost_us(pl.edge, per_item * head, K) +
+                            ring16_cost_us(tail_edge, ring16_tiles(tail_edge, M, N, batch - head), K) + 2.0;
+    if (split_us < 0.93 * ring16_cost_us(pl.edge, total, K)) { pl.head = (int)head; pl.tail_edge = tail_edge; }
+    return pl;
 }
 
 static inline int64_t elem_size(int dt) {

@@ -1073,8 +1073,9 @@ int64_t ntg_conv_transpose2d_workspace_bytes(int dtype, int64_t batch, int64_t i
     if (ntg::elem_size(dtype) == 0 || groups < 1 || in_channels % groups != 0 || out_channels % groups != 0 ||
         conv_transpose_out(in_h, in_w, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c, op_r, op_c, oh, ow) ||
         unfold_out(oh, ow, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c, Ho, Wo)) return -1;
-    return plan_conv_backward(dtype, true, false, batch, out_channels, oh, ow, in_channels, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c,
-                              groups, Ho, Wo).need;
+    const ConvBackwardPlan pl = plan_conv_backward(dtype, true, false, batch, out_channels, oh, ow, in_channels, k_r, k_c, s_r, s_c, p_r, p_c,
+                                                   d_r, d_c, groups, Ho, Wo);
+    return std::max(pl.need, pl.need_nhwc_dx);      // (the larger amount lets the stride-1 case run channels-last)
 }
 
 int ntg_conv_transpose2d_dev(int dtype, const void* input, const void* kernel, void* out, void* workspace, int64_t workspace_bytes,

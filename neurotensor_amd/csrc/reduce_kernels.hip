@@ -204,15 +204,56 @@ __global__ void __launch_bounds__(256) nchw_to_nhwc_kernel(const T* __restrict__
     }
 }
 
+// The same copy with 16-byte accesses on both sides (C and P multiples of one 16-byte vector, aligned pointers): a
+// thread loads VEC pixels of one channel, the tile goes through LDS as single elements (row pitch chosen so that the
+// column-wise read-back spreads over the banks), and a thread stores VEC channels of one pixel.
+template <class T>
+__global__ void __launch_bounds__(256) nchw_to_nhwc_vec_kernel(const T* __restrict__ in, T* __restrict__ out, const int64_t C, const int64_t P) {
+    constexpr int VEC = 16 / (int)sizeof(T), VPR = 64 / VEC;            // elements per vector, vectors per tile row
+    constexpr int PITCH = sizeof(T) == 2 ? 66 : 65;                     // elements: 33 / 65 words
+    typedef T TV __attribute__((ext_vector_type(VEC)));
+    __shared__ T tile[64 * PITCH];
+    const int64_t p0 = (int64_t)blockIdx.x * 64, c0 = (int64_t)blockIdx.y * 64, b = blockIdx.z;
+    const T* src = in + b * C * P;
+    T* dst = out + b * C * P;
+#pragma unroll
+    for (int i = 0; i < 64 * VPR / 256; ++i) {
+        const int v = threadIdx.x + 256 * i, c = v / VPR, pv = v % VPR;
+        if (c0 + c < C && p0 + pv * VEC < P) {
+            const TV x = *reinterpret_cast<const TV*>(src + (c0 + c) * P + p0 + pv * VEC);
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) tile[c * PITCH + pv * VEC + e] = x[e];
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 64 * VPR / 256; ++i) {
+        const int v = threadIdx.x + 256 * i, pp = v / VPR, cv = v % VPR;
+        if (c0 + cv * VEC < C && p0 + pp < P) {
+            TV x;
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) x[e] = tile[(cv * VEC + e) * PITCH + pp];
+            *reinterpret_cast<TV*>(dst + (p0 + pp) * C + c0 + cv * VEC) = x;
+        }
+    }
+}
+
 hipError_t launch_nchw_to_nhwc(int64_t es, const void* in, void* out, int64_t batch, int64_t C, int64_t P, hipStream_t s) {
     if (batch * C * P == 0) return hipSuccess;
     const int64_t gx = (P + 63) / 64, gy = (C + 63) / 64;
-    if (gx > 0x7fffffffLL || gy > 65535 || batch > 65535) return hipErrorInvalidValue;
-    const dim3 g((unsigned)gx, (unsigned)gy, (unsigned)batch), t(256);
-    switch (es) {
-    case 2: hipLaunchKernelGGL(nchw_to_nhwc_kernel<uint16_t>, g, t, 0, s, (const uint16_t*)in, (uint16_t*)out, C, P); break;
-    case 4: hipLaunchKernelGGL(nchw_to_nhwc_kernel<uint32_t>, g, t, 0, s, (const uint32_t*)in, (uint32_t*)out, C, P); break;
-    default: return hipErrorInvalidValue;
+    if (gx > 0x7fffffffLL || gy > 65535) return hipErrorInvalidValue;
+    const int64_t vec = 16 / es;
+    const bool vec_ok = C % vec == 0 && P % vec == 0 && ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) & 15) == 0;
+    for (int64_t b0 = 0; b0 < batch; b0 += 65535) {                    // (grid z limit)
+        const int64_t nb = batch - b0 < 65535 ? batch - b0 : 65535;
+        const dim3 g((unsigned)gx, (unsigned)gy, (unsigned)nb), t(256);
+        const char* src = static_cast<const char*>(in) + b0 * C * P * es;
+        char* dst = static_cast<char*>(out) + b0 * C * P * es;
+        if (es == 2 && vec_ok) hipLaunchKernelGGL(nchw_to_nhwc_vec_kernel<uint16_t>, g, t, 0, s, (const uint16_t*)src, (uint16_t*)dst, C, P);
+        else if (es == 4 && vec_ok) hipLaunchKernelGGL(nchw_to_nhwc_vec_kernel<uint32_t>, g, t, 0, s, (const uint32_t*)src, (uint32_t*)dst, C, P);
+        else if (es == 2) hipLaunchKernelGGL(nchw_to_nhwc_kernel<uint16_t>, g, t, 0, s, (const uint16_t*)src, (uint16_t*)dst, C, P);
+        else if (es == 4) hipLaunchKernelGGL(nchw_to_nhwc_kernel<uint32_t>, g, t, 0, s, (const uint32_t*)src, (uint32_t*)dst, C, P);
+        else return hipErrorInvalidValue;
     }
     return hipGetLastError();
 }

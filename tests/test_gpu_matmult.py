@@ -395,6 +395,40 @@ def test_ragged_16bit_dma_kernel(dtype, shape):
     assert ((y.float() - refy).abs().max() / refy.abs().max()).item() <= HALF_REL
 
 
+@pytest.mark.parametrize("dtype", ["bf16", np.float16], ids=["bf16", "fp16"])
+@pytest.mark.parametrize("shape", [(33, 128, 512, 1000), (70, 250, 512, 256), (270, 128, 1032, 264)], ids=lambda s: "x".join(map(str, s)))
+def test_batched_16bit_two_launch_plan(dtype, shape):
+    """Batches whose tiles fill the CUs a whole number of times plus a small rest go out as two launches (the first items
+    on the chosen tile, the rest on a smaller one): 33 -> 32 + 1, 70 -> 64 + 6, 270 -> 256 + 14 items.  Every item must
+    come out the same whichever launch computed it: all three C modes, broadcast A, ragged edges."""
+    batch, m, k, n = shape
+    bf = dtype == "bf16"
+    rng = np.random.default_rng(2100 + batch)
+    a = to_torch(randn(rng, (batch, m, k), dtype, 0.25), DEV, bf)
+    b = to_torch(randn(rng, (batch, k, n), dtype, 0.25), DEV, bf)
+    ref = torch.matmul(a.float(), b.float())
+    scale = ref.abs().max().item()
+    guard = torch.full((batch + 2, m, n), 7.0, device=DEV).to(a.dtype)
+    c = guard[1:batch + 1]
+    c.zero_()
+    out = F.matmult(a, b, c, accumulate=False)
+    assert ((out.float() - ref).abs().max() / scale).item() <= HALF_REL
+    assert torch.all(guard[0] == 7.0) and torch.all(guard[batch + 1] == 7.0)
+    # identical operands in the first and the last item: the two launches must agree bit for bit
+    a2, b2 = a.clone(), b.clone()
+    a2[batch - 1], b2[batch - 1] = a2[0], b2[0]
+    out2 = F.matmult(a2, b2)
+    assert torch.equal(out2[0], out2[batch - 1])
+    F.matmult(a, b, c)                                               # accumulate: 2 * A.B
+    assert ((c.float() - 2 * ref).abs().max() / scale).item() <= 2 * HALF_REL
+    # one A for every item (stride 0), B stored [n, k], bias broadcast over the batch
+    w = to_torch(randn(rng, (n, k), dtype, 0.25), DEV, bf)
+    bias = to_torch(randn(rng, (n,), dtype), DEV, bf)
+    y = F.linear(a, w, bias, False, True)
+    refy = torch.matmul(a.float(), w.float().T) + bias.float()
+    assert ((y.float() - refy).abs().max() / refy.abs().max()).item() <= HALF_REL
+
+
 @pytest.mark.parametrize("dtype", [np.float32, np.float64], ids=["fp32", "fp64"])
 @pytest.mark.parametrize("shape", [(1860, 260, 1860), (2052, 1000, 2308), (1028, 132, 516), (68, 20, 4), (132, 16, 260), (130, 22, 66)],
                          ids=lambda s: "x".join(map(str, s)))
