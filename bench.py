@@ -210,8 +210,14 @@ def main():
         run("mid_fp32_2048", make_gemm(torch.float32, 2048, 2048, 2048, mode=_lib.C_OVERWRITE), f2k, PEAK_TFLOPS["fp32"], st=steps * 2)
         x = torch.randn(64, 256, 56, 56, device=dev)
         w = torch.randn(256, 256, 3, 3, device=dev) / 48.0
-        run("c5a_conv2d_fp32", lambda: F.conv2d(x, w, padding=1), 2.0 * 200704 * 2304 * 256, PEAK_TFLOPS["fp32"])
-        del x, w
+        fc = 2.0 * 200704 * 2304 * 256
+        run("c5a_conv2d_fp32", lambda: F.conv2d(x, w, padding=1), fc, PEAK_TFLOPS["fp32"])
+        g = torch.randn(64, 256, 56, 56, device=dev)
+        run("c5a_conv2d_backward_fp32", lambda: F.conv2d_backward(x, w, g, padding=1), 2.0 * fc, PEAK_TFLOPS["fp32"])
+        xh, wh, gh = x.bfloat16(), w.bfloat16(), g.bfloat16()
+        run("c5a_conv2d_bf16", lambda: F.conv2d(xh, wh, padding=1), fc, PEAK_TFLOPS["bf16"], st=steps * 2)
+        run("c5a_conv2d_backward_bf16", lambda: F.conv2d_backward(xh, wh, gh, padding=1), 2.0 * fc, PEAK_TFLOPS["bf16"], st=steps * 2)
+        del x, w, g, xh, wh, gh
         skinny_bytes = 4.0 * (16 * 8192 + 8192 * 8192 + 2 * 16 * 8192)
         run("c5b_skinny_fp32_16x8192x8192", make_gemm(torch.float32, 16, 8192, 8192), skinny_bytes, PEAK_HBM_GBS, "GB/s", 1e9,
             st=steps * 4)
