@@ -189,7 +189,7 @@ int64_t ntg_conv2d_forward_workspace_bytes(int dtype, int64_t batch, int64_t cha
                                            int64_t p_r, int64_t p_c, int64_t d_r, int64_t d_c);
 
 /* Bytes of device workspace with which ntg_conv2d_dev runs its fastest form.  For Float16 / BFloat16 / Float32 whose
- * channels per group fill whole 64-byte K-steps (a multiple of 32 / 32 / 16) and whose output planes have 16-byte rows,
+ * channels per group fill whole 64-byte K-steps (a multiple of 32 / 32 / 16)
  * that is a channels-last copy of the image plus the weights with the channel index fastest; the convolution
  * (conv.cpp:86-118) then gathers its operand in 16-byte pieces.  Otherwise the figure of
  * ntg_conv2d_forward_workspace_bytes.  ntg_conv2d_dev accepts any smaller workspace and falls back to its other forms. */

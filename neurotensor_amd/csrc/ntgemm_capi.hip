@@ -194,6 +194,25 @@ int run_gemm(ntg::GemmParams p, int dtype, bool ta, bool tb, hipStream_t s, void
     const int64_t es = ntg::elem_size(dtype);
     if (es == 0) return fail(NTG_ERR_UNSUPPORTED_DTYPE, "dtype %d is not supported by the gfx950 matmult backend", dtype);
     if (p.M == 0 || p.N == 0 || p.batch == 0) return NTG_OK;
+    if (p.K == 0) {
+        // empty sum: C keeps what it holds, or becomes the bias / zero.  The product kernels assume at least one k.
+        if (p.cmode == ntg::C_ACCUMULATE) return NTG_OK;
+        if (p.Cptr) return fail(NTG_ERR_INVALID_ARGUMENT, "k = 0 with a C mode other than accumulate needs strided operands");
+        hipError_t e = hipSuccess;
+        if (is_int_dtype(dtype)) {
+            e = ntg::launch_gemm_valu(dtype, ta, tb, p, s);                 // its k loop runs zero times
+        } else {
+            for (int b = 0; b < p.batch && e == hipSuccess; ++b) {
+                ntg::GemmParams q = p;
+                q.batch = 1;
+                q.C = static_cast<char*>(p.C) + (int64_t)b * p.sC * es;
+                if (p.bias) q.bias = static_cast<const char*>(p.bias) + (int64_t)b * p.bias_bs * es;
+                e = ntg::launch_splitk_reduce(dtype, nullptr, 0, q, s);     // C0 plus no partial sums
+            }
+        }
+        if (e != hipSuccess) return hip_fail(e, "empty-k launch");
+        return NTG_OK;
+    }
     const SplitPlan plan = plan_splitk(p, dtype, ta);
     if (plan.splits > 1 && workspace && workspace_bytes >= plan.bytes && (reinterpret_cast<uintptr_t>(workspace) & 15) == 0) {
         ntg::GemmParams q = p;
@@ -576,11 +595,18 @@ static int conv_forward_pointwise(int dtype, const void* image, const void* kern
 // Channels-last form of the same convolution, for the floating dtypes up to 32 bits: the image is first copied to
 // [B][pixel][C] and the weights to [O][(taps, c)] in the workspace; then one K-step of the product is 64 bytes of consecutive
 // channels of one tap, and the kernel's DMA gathers the operand in 16-byte pieces instead of element by element.
+// byte offsets inside a channels-last image are formed in 32 bits from two terms (the pixel of the window origin, and the
+// tap reach with the padding taken off): both must stay below 2^30
+static bool conv_nhwc_offsets_fit(int64_t channels, int64_t es, const Geo3& g) {
+    const int64_t pr = g.p[1] < 0 ? -g.p[1] : g.p[1], pc = g.p[2] < 0 ? -g.p[2] : g.p[2];
+    const int64_t reach = ((pr + g.k[1] * g.d[1]) * g.sz[2] + pc + g.k[2] * g.d[2]) * channels * es;
+    return channels * g.vol() * es < (1LL << 30) && reach < (1LL << 30);
+}
 static bool conv_nhwc_ok(int dtype, int64_t channels, int64_t out_channels, int64_t groups, const Geo3& g) {
     if (dtype != ntg::DT_F32 && dtype != ntg::DT_F16 && dtype != ntg::DT_BF16) return false;
     if (g.nd != 2 || !conv_implicit_g(dtype, channels, g)) return false;
     const int64_t es = ntg::elem_size(dtype), cg = channels / groups;
-    return cg % (64 / es) == 0 && out_channels > 0 && channels * g.vol() * es < 0x7fffffffLL;
+    return cg % (64 / es) == 0 && out_channels > 0 && conv_nhwc_offsets_fit(channels, es, g);
 }
 static int64_t conv_nhwc_workspace(int dtype, int64_t batch, int64_t channels, int64_t out_channels, int64_t groups, const Geo3& g) {
     const int64_t es = ntg::elem_size(dtype);
@@ -717,7 +743,8 @@ static bool conv_dkernel_nhwc_ok(int dtype, int64_t channels, int64_t out_channe
     if (g.nd != 2 || !conv_implicit_g(dtype, channels, g)) return false;
     const int64_t es = ntg::elem_size(dtype), cg = channels / groups;
     if (g.k[1] * g.d[1] >= 32768 || g.k[2] * g.d[2] >= 32768) return false;      // tap reach packed in 16 bits
-    return (cg * es) % 16 == 0 && (g.L() * es) % 16 == 0 && out_channels > 0 && cg * g.taps() < 0x7fffffffLL;
+    return (cg * es) % 16 == 0 && (g.L() * es) % 16 == 0 && out_channels > 0 && cg * g.taps() < 0x7fffffffLL &&
+           conv_nhwc_offsets_fit(channels, es, g);
 }
 static int64_t conv_dkernel_nhwc_workspace(int dtype, int64_t batch, int64_t channels, int64_t out_channels, int64_t groups, const Geo3& g) {
     const int64_t es = ntg::elem_size(dtype);

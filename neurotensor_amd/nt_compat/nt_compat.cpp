@@ -1,8 +1,11 @@
-// Implementation of the nt_compat facade on the host-pointer C ABI of libntgemm.so.
+// Implementation of the nt_compat facade on the C ABI of libntgemm.so: host tensors through the host-pointer
+// entry points, device tensors (DeviceType::HIP) through the `_dev` ones on the default stream.
 // Every validation happens here, before any device work, with the reference's messages.
 #include "nt_compat.h"
 
 #include "../../include/ntgemm.h"
+
+#include <hip/hip_runtime_api.h>
 
 #include <algorithm>
 #include <cmath>
@@ -56,13 +59,64 @@ static SizeRef dense_strides(const SizeRef& shape) {
 
 // ------------------------------------------------------------------------------------------ Tensor
 
-Tensor::Tensor(SizeRef shape, DType dt) : shape_(std::move(shape)), dtype_(dt) {
+static void hip_check(hipError_t e, const char* what) {
+    if (e != hipSuccess) throw utils::nt_error(std::string(what) + ": " + hipGetErrorString(e));
+}
+
+static std::shared_ptr<char> device_alloc(size_t bytes) {
+    void* p = nullptr;
+    hip_check(hipMalloc(&p, bytes), "hipMalloc");
+    return std::shared_ptr<char>(static_cast<char*>(p), [](char* q) { (void)hipFree(q); });
+}
+
+// Scratch for the `_dev` convolutions: one buffer per thread that only grows.  All device work of this facade is
+// issued on the default stream, so a later call reuses it safely after the earlier one in stream order.
+static void* device_workspace(int64_t bytes) {
+    static thread_local std::shared_ptr<char> buf;
+    static thread_local int64_t cap = 0;
+    if (bytes <= 0) return nullptr;
+    if (bytes > cap) {
+        hip_check(hipDeviceSynchronize(), "hipDeviceSynchronize");     // kernels may still use the smaller buffer
+        buf.reset();
+        buf = device_alloc((size_t)bytes);
+        cap = bytes;
+    }
+    return buf.get();
+}
+
+Tensor::Tensor(SizeRef shape, DType dt, DeviceType dev) : shape_(std::move(shape)), dtype_(dt), device_(dev) {
     const int64_t es = dtype_size(dt);
     utils::throw_exception(es > 0, std::string("dtype ") + dtype_name(dt) + " has no storage in nt_compat");
+    utils::throw_exception(dev == DeviceType::CPU || dev == DeviceType::HIP, "nt_compat tensors live on DeviceType::CPU or DeviceType::HIP");
     for (int64_t d : shape_) utils::throw_exception(d >= 0, "negative dimension in shape " + shape_str(shape_));
     strides_ = dense_strides(shape_);
     const size_t bytes = (size_t)std::max<int64_t>(1, prod(shape_) * es);
-    storage_ = std::shared_ptr<char>(static_cast<char*>(::operator new(bytes)), [](char* p) { ::operator delete(p); });
+    if (dev == DeviceType::HIP) storage_ = device_alloc(bytes);
+    else storage_ = std::shared_ptr<char>(static_cast<char*>(::operator new(bytes)), [](char* p) { ::operator delete(p); });
+}
+
+Tensor Tensor::to(DeviceType dev) const {
+    utils::throw_exception(!is_null(), "cannot move a null tensor");
+    utils::throw_exception(dev == DeviceType::CPU || dev == DeviceType::HIP, "nt_compat tensors live on DeviceType::CPU or DeviceType::HIP");
+    if (dev == device_) return *this;
+    const int64_t es = dtype_size(dtype_);
+    if (dev == DeviceType::HIP) {
+        const Tensor src = contiguous();
+        Tensor out(shape_, dtype_, DeviceType::HIP);
+        if (numel()) hip_check(hipMemcpy(out.data_ptr(), src.data_ptr(), (size_t)(numel() * es), hipMemcpyHostToDevice), "hipMemcpy to device");
+        out.mutable_ = mutable_;
+        return out;
+    }
+    // device -> host: the elements the view spans are copied as they lie, the strides are applied on the host
+    int64_t span = numel() ? 1 : 0;
+    for (size_t d = 0; d < shape_.size() && numel(); ++d) span += (shape_[d] - 1) * strides_[d];
+    Tensor raw({std::max<int64_t>(span, 1)}, dtype_);
+    if (span) hip_check(hipMemcpy(raw.data_ptr(), data_ptr(), (size_t)(span * es), hipMemcpyDeviceToHost), "hipMemcpy to host");
+    Tensor out = raw;
+    out.shape_ = shape_;
+    out.strides_ = strides_;
+    out.mutable_ = mutable_;
+    return out.is_contiguous() ? out : out.clone();
 }
 
 int64_t Tensor::numel() const { return is_null() ? 0 : prod(shape_); }
@@ -78,6 +132,12 @@ bool Tensor::is_contiguous() const {
 
 Tensor Tensor::clone() const {
     utils::throw_exception(!is_null(), "cannot clone a null tensor");
+    if (is_device()) {
+        if (!is_contiguous()) return cpu().to(DeviceType::HIP);      // (strided device views are rare on this path: via the host)
+        Tensor out(shape_, dtype_, DeviceType::HIP);
+        if (numel()) hip_check(hipMemcpy(out.data_ptr(), data_ptr(), (size_t)(numel() * dtype_size(dtype_)), hipMemcpyDeviceToDevice), "hipMemcpy on device");
+        return out;
+    }
     Tensor out(shape_, dtype_);
     const int64_t es = dtype_size(dtype_), n = numel();
     if (is_contiguous()) {
@@ -170,6 +230,37 @@ Tensor Tensor::sum_leading(const SizeRef& target) const {
     for (size_t i = 0; i < target.size(); ++i) padded[shape_.size() - target.size() + i] = target[i];
     for (size_t i = 0; i < padded.size(); ++i)
         utils::throw_exception(padded[i] == 1 || padded[i] == shape_[i], "cannot reduce " + shape_str(shape_) + " to " + shape_str(target));
+    if (is_device()) {
+        // Sum over leading dims only (bias and broadcast-batch gradients): ones[1, R] . src[R, T] on the device.
+        size_t j = 0;
+        while (j < padded.size() && padded[j] == 1) ++j;
+        bool tail_equal = true;
+        for (size_t i = j; i < padded.size(); ++i) tail_equal = tail_equal && padded[i] == shape_[i];
+        const int64_t R = prod(shape_, 0, j), T = prod(shape_, j);
+        if (!tail_equal || R == 0 || T == 0) return src.cpu().sum_leading(target).to(DeviceType::HIP);
+        Tensor ones_h({1, R}, dtype_);
+        switch (dtype_) {
+        case DType::Float32: std::fill_n(ones_h.data<float>(), R, 1.0f); break;
+        case DType::Float64: std::fill_n(ones_h.data<double>(), R, 1.0); break;
+        case DType::Float16: std::fill_n(ones_h.data<uint16_t>(), R, (uint16_t)0x3c00); break;
+        case DType::BFloat16: std::fill_n(ones_h.data<uint16_t>(), R, (uint16_t)0x3f80); break;
+        case DType::int8: case DType::uint8: std::fill_n(ones_h.data<uint8_t>(), R, (uint8_t)1); break;
+        case DType::int16: case DType::uint16: std::fill_n(ones_h.data<uint16_t>(), R, (uint16_t)1); break;
+        case DType::int32: case DType::uint32: std::fill_n(ones_h.data<uint32_t>(), R, 1u); break;
+        case DType::int64: case DType::uint64: std::fill_n(ones_h.data<uint64_t>(), R, (uint64_t)1); break;
+        default: utils::throw_exception(false, std::string("sum_as is not available for ") + dtype_name(dtype_));
+        }
+        const Tensor ones = ones_h.to(DeviceType::HIP);
+        Tensor out(target, dtype_, DeviceType::HIP);
+        ntg_gemm_desc d;
+        std::memset(&d, 0, sizeof d);
+        d.dtype = static_cast<int>(dtype_); d.c_mode = NTG_C_OVERWRITE;
+        d.m = 1; d.k = R; d.n = T; d.batches = 1;
+        if (ntg_gemm_dev(&d, ones.data_ptr(), src.data_ptr(), out.data_ptr(), nullptr) != NTG_OK)
+            throw utils::nt_error(std::string("gfx950 matmult backend: ") + ntg_last_error());
+        hip_check(hipStreamSynchronize(nullptr), "hipStreamSynchronize");      // `ones` is freed on return
+        return out;
+    }
     Tensor out(target, dtype_);
     if (dtype_ == DType::Float32) sum_as_t<float>(src, out, padded);
     else if (dtype_ == DType::Float64) sum_as_t<double>(src, out, padded);
@@ -183,9 +274,11 @@ Tensor Tensor::sum_leading(const SizeRef& target) const {
 
 namespace functional {
 
-Tensor zeros(SizeRef shape, DType dt) {
-    Tensor t(std::move(shape), dt);
-    std::memset(t.data_ptr(), 0, (size_t)(t.numel() * dtype_size(dt)));
+Tensor zeros(SizeRef shape, DType dt, DeviceType dev) {
+    Tensor t(std::move(shape), dt, dev);
+    const size_t bytes = (size_t)(t.numel() * dtype_size(dt));
+    if (dev == DeviceType::HIP) { if (bytes) hip_check(hipMemset(t.data_ptr(), 0, bytes), "hipMemset"); }
+    else std::memset(t.data_ptr(), 0, bytes);
     return t;
 }
 
@@ -259,7 +352,7 @@ Tensor from_numpy(const std::string& path) {
 
 bool allclose(const Tensor& a_, const Tensor& b_, double rtol, double atol) {
     if (a_.is_null() || b_.is_null() || a_.shape() != b_.shape() || a_.dtype() != b_.dtype()) return false;
-    Tensor a = a_.contiguous(), b = b_.contiguous();
+    Tensor a = a_.cpu().contiguous(), b = b_.cpu().contiguous();
     const int64_t n = a.numel();
     auto chk = [&](auto* pa, auto* pb) {
         for (int64_t i = 0; i < n; ++i) {
@@ -338,13 +431,57 @@ static MatmultPlan plan_matmult(const Tensor& a_in, const Tensor& b_in, bool tra
     return p;
 }
 
-static void run_plan(const MatmultPlan& p, Tensor& c) {
+// operands of one operation live in the same memory
+static DeviceType common_device(std::initializer_list<const Tensor*> ts, const char* op) {
+    DeviceType dev = DeviceType::CPU;
+    bool first = true;
+    for (const Tensor* t : ts) {
+        if (t->is_null()) continue;
+        if (first) { dev = t->device(); first = false; }
+        utils::throw_exception(t->device() == dev, std::string("Expected all tensors of ") + op + " to be on the same device");
+    }
+    return dev;
+}
+
+// Batched product on device buffers.  Item i of the higher-rank operand pairs with item i mod count of the lower-rank
+// one (and of the bias); the lower-rank batch dims equal the trailing ones of the higher-rank operand, so the items come
+// in nbig / chunk consecutive chunks inside which every operand is either strided or one matrix.
+static void device_gemm(int dt, int64_t es, bool ta, bool tb, int mode, int64_t m, int64_t k, int64_t n, int64_t nbig,
+                        const char* A, int64_t na, const char* B, int64_t nb, char* C,
+                        const char* bias = nullptr, int64_t nbias = 1, int64_t brow = 1, int64_t bcol = 1) {
+    int64_t chunk = nbig;
+    for (int64_t cnt : {na, nb, nbias})
+        if (cnt > 1 && cnt < chunk) chunk = cnt;
+    for (int64_t i0 = 0; i0 < nbig; i0 += chunk) {
+        ntg_gemm_desc d;
+        std::memset(&d, 0, sizeof d);
+        d.dtype = dt; d.transpose_a = ta; d.transpose_b = tb; d.c_mode = mode;
+        d.m = m; d.k = k; d.n = n; d.batches = chunk;
+        d.stride_a = na > 1 ? m * k : 0;
+        d.stride_b = nb > 1 ? k * n : 0;
+        d.stride_c = m * n;
+        if (bias) {
+            d.bias = bias + (nbias > 1 ? (i0 % nbias) * brow * bcol * es : 0);
+            d.bias_batch_stride = nbias > 1 ? brow * bcol : 0;
+            d.bias_row_stride = brow > 1 ? bcol : 0;
+            d.bias_col_stride = bcol > 1 ? 1 : 0;
+        }
+        check_status(ntg_gemm_dev(&d, A + (na > 1 ? (i0 % na) * m * k * es : 0), B + (nb > 1 ? (i0 % nb) * k * n * es : 0),
+                                  C + i0 * m * n * es, nullptr));
+    }
+}
+
+static void run_plan(const MatmultPlan& p, Tensor& c, bool overwrite = false) {
     if (p.nbig == 0 || p.m == 0 || p.n == 0 || p.k == 0) return;
     const int64_t es = dtype_size(p.a.dtype());
     const int dt = static_cast<int>(p.a.dtype());
     const char* A = static_cast<const char*>(p.a.data_ptr());
     const char* B = static_cast<const char*>(p.b.data_ptr());
     char* C = static_cast<char*>(c.data_ptr());
+    if (c.is_device()) {
+        device_gemm(dt, es, p.ta, p.tb, overwrite ? NTG_C_OVERWRITE : NTG_C_ACCUMULATE, p.m, p.k, p.n, p.nbig, A, p.na, B, p.nb, C);
+        return;
+    }
     if (p.nbig == 1) {
         check_status(ntg_matmult(dt, A, B, C, p.m, p.k, p.k, p.n, p.ta, p.tb));
         return;
@@ -363,6 +500,13 @@ static void run_plan(const MatmultPlan& p, Tensor& c) {
 
 Tensor matmult(const Tensor& a, const Tensor& b, bool trans_a, bool trans_b) {
     MatmultPlan p = plan_matmult(a, b, trans_a, trans_b, false);
+    if (common_device({&a, &b}, "matmult") == DeviceType::HIP) {
+        // C = op(a).op(b) written in one pass (zeros + accumulate would read and write C once more)
+        if (p.k == 0) return zeros(p.out_shape, a.dtype(), DeviceType::HIP);
+        Tensor c(p.out_shape, a.dtype(), DeviceType::HIP);
+        run_plan(p, c, true);
+        return c;
+    }
     Tensor c = zeros(p.out_shape, a.dtype());      // matmult_cpu.cpp:110, :707
     run_plan(p, c);
     return c;
@@ -372,6 +516,7 @@ Tensor& matmult(const Tensor& a, const Tensor& b, Tensor& c, bool trans_a, bool 
     utils::throw_exception(!c.is_null(), "Cannot perform operation matmult on a null tensor");
     utils::throw_exception(c.is_mutable(), "Output from Matmult must be mutable");   // tensor_files/matmult.cpp:21
     MatmultPlan p = plan_matmult(a, b, trans_a, trans_b, true);
+    common_device({&a, &b, &c}, "matmult");
     const SizeRef& cs = c.shape();
     const bool same = cs == p.out_shape;
     const bool same_numel = c.dims() >= 2 && c.numel() == p.nbig * p.m * p.n && cs[cs.size() - 2] == p.m && cs[cs.size() - 1] == p.n;
@@ -421,10 +566,17 @@ Tensor linear(const Tensor& x_in, const Tensor& w_in, const Tensor& b_in, bool t
         utils::throw_exception(bb[i] == p.out_shape[obd - bb.size() + i], "Error, invalid batch shapes for linear: (" + shape_str(x_in.shape()) +
                                                                               ", " + shape_str(w_in.shape()) + ", " + shape_str(b_in.shape()) + ")");
     const int64_t nbias = prod(bb);
-    Tensor c(p.out_shape, x.dtype());
+    const DeviceType dev = common_device({&x_in, &w_in, &b_in}, "linear");
+    Tensor c(p.out_shape, x.dtype(), dev);
     if (p.nbig == 0 || p.m == 0 || p.n == 0) return c;
     const int64_t es = dtype_size(x.dtype());
     const int dt = static_cast<int>(x.dtype());
+    if (dev == DeviceType::HIP) {
+        device_gemm(dt, es, p.ta, p.tb, NTG_C_BIAS, p.m, p.k, p.n, p.nbig, static_cast<const char*>(p.a.data_ptr()), p.na,
+                    static_cast<const char*>(p.b.data_ptr()), p.nb, static_cast<char*>(c.data_ptr()),
+                    static_cast<const char*>(b.data_ptr()), nbias, brow, bcol);
+        return c;
+    }
     // bias broadcast to the output is the initial accumulator (:1637-1647); fused on the device
     for (int64_t i = 0; i < p.nbig; ++i) {
         check_status(ntg_linear(dt, static_cast<const char*>(p.a.data_ptr()) + (i % p.na) * p.m * p.k * es,
@@ -473,9 +625,13 @@ Tensor unfold2d(const Tensor& x_in, utils::my_tuple k, utils::my_tuple d, utils:
                            "Given input with spatial size (" + std::to_string(H) + ", " + std::to_string(W) +
                                "), calculated shape of the array of sliding blocks as (" + std::to_string(Lr) + ", " + std::to_string(Lc) +
                                "), but its components must be at least one.");
-    Tensor col({B, C * k.first * k.second, Lr * Lc}, x.dtype());
-    check_status(ntg_unfold2d(static_cast<int>(x.dtype()), x.data_ptr(), col.data_ptr(), B, C, H, W, k.first, k.second, s.first, s.second,
-                              p.first, p.second, d.first, d.second));
+    Tensor col({B, C * k.first * k.second, Lr * Lc}, x.dtype(), x.device());
+    if (x.is_device())
+        check_status(ntg_unfold2d_dev(static_cast<int>(x.dtype()), x.data_ptr(), col.data_ptr(), B, C, H, W, k.first, k.second, s.first, s.second,
+                                      p.first, p.second, d.first, d.second, nullptr));
+    else
+        check_status(ntg_unfold2d(static_cast<int>(x.dtype()), x.data_ptr(), col.data_ptr(), B, C, H, W, k.first, k.second, s.first, s.second,
+                                  p.first, p.second, d.first, d.second));
     if (transpose_out) return col;
     return col.transpose(-1, -2);
 }
@@ -507,8 +663,17 @@ Tensor conv2d(const Tensor& image, const Tensor& kernel, utils::my_tuple s, util
     const int64_t Ro = (H + 2 * p.first - d.first * (kh - 1) - 1) / s.first + 1;
     const int64_t Co = (W + 2 * p.second - d.second * (kw - 1) - 1) / s.second + 1;
     utils::throw_exception(Ro > 0 && Co > 0, "conv2d output would be empty");
-    Tensor out({B, O, Ro, Co}, x.dtype());
-    check_status(ntg_conv2d(static_cast<int>(x.dtype()), x.data_ptr(), w.data_ptr(), out.data_ptr(), B, C, H, W, O, kh, kw, s.first, s.second,
+    const DeviceType dev = common_device({&image, &kernel}, "conv2d");
+    Tensor out({B, O, Ro, Co}, x.dtype(), dev);
+    const int dt = static_cast<int>(x.dtype());
+    if (dev == DeviceType::HIP) {
+        const int64_t wsb = ntg_conv2d_fast_workspace_bytes(dt, B, C, H, W, O, kh, kw, s.first, s.second, p.first, p.second, d.first, d.second, groups);
+        utils::throw_exception(wsb >= 0, "conv2d output would be empty");
+        check_status(ntg_conv2d_dev(dt, x.data_ptr(), w.data_ptr(), out.data_ptr(), device_workspace(wsb), wsb, B, C, H, W, O, kh, kw,
+                                    s.first, s.second, p.first, p.second, d.first, d.second, groups, nullptr));
+        return out;
+    }
+    check_status(ntg_conv2d(dt, x.data_ptr(), w.data_ptr(), out.data_ptr(), B, C, H, W, O, kh, kw, s.first, s.second,
                             p.first, p.second, d.first, d.second, groups));
     return out;
 }
@@ -525,9 +690,13 @@ Tensor unfold2d_backward(const Tensor& col_in, utils::my_tuple out, utils::my_tu
     const int64_t Lr = (out.first + 2 * p.first - d.first * (k.first - 1) - 1) / s.first + 1;
     const int64_t Lc = (out.second + 2 * p.second - d.second * (k.second - 1) - 1) / s.second + 1;
     utils::throw_exception(Lr > 0 && Lc > 0 && Lr * Lc == L, "Given output_size and kernel geometry do not match the number of sliding blocks");
-    Tensor im({B, C, out.first, out.second}, col.dtype());
-    check_status(ntg_unfold2d_backward(static_cast<int>(col.dtype()), col.data_ptr(), im.data_ptr(), B, C, out.first, out.second, k.first,
-                                       k.second, s.first, s.second, p.first, p.second, d.first, d.second, 0));
+    Tensor im({B, C, out.first, out.second}, col.dtype(), col.device());
+    if (col.is_device())
+        check_status(ntg_unfold2d_backward_dev(static_cast<int>(col.dtype()), col.data_ptr(), im.data_ptr(), B, C, out.first, out.second, k.first,
+                                               k.second, s.first, s.second, p.first, p.second, d.first, d.second, 0, nullptr));
+    else
+        check_status(ntg_unfold2d_backward(static_cast<int>(col.dtype()), col.data_ptr(), im.data_ptr(), B, C, out.first, out.second, k.first,
+                                           k.second, s.first, s.second, p.first, p.second, d.first, d.second, 0));
     return im;
 }
 
@@ -546,8 +715,18 @@ ConvGrads conv2d_backward(const Tensor& image, const Tensor& kernel, const Tenso
     const int64_t Ro = (H + 2 * p.first - d.first * (kh - 1) - 1) / s.first + 1;
     const int64_t Co = (W + 2 * p.second - d.second * (kw - 1) - 1) / s.second + 1;
     utils::throw_exception(Ro > 0 && Co > 0 && g.numel() == B * O * Ro * Co, "grad does not have the shape of the convolution output");
-    ConvGrads out{Tensor(image.shape(), x.dtype()), Tensor(kernel.shape(), x.dtype())};
-    check_status(ntg_conv2d_backward(static_cast<int>(x.dtype()), x.data_ptr(), w.data_ptr(), g.data_ptr(), out.d_image.data_ptr(),
+    const DeviceType dev = common_device({&image, &kernel, &grad}, "conv2d backward");
+    ConvGrads out{Tensor(image.shape(), x.dtype(), dev), Tensor(kernel.shape(), x.dtype(), dev)};
+    const int dt = static_cast<int>(x.dtype());
+    if (dev == DeviceType::HIP) {
+        const int64_t wsb = ntg_conv2d_backward_workspace_bytes(dt, B, C, H, W, O, kh, kw, s.first, s.second, p.first, p.second, d.first, d.second, groups);
+        utils::throw_exception(wsb >= 0, "conv2d backward: geometry has no output");
+        check_status(ntg_conv2d_backward_dev(dt, x.data_ptr(), w.data_ptr(), g.data_ptr(), out.d_image.data_ptr(), out.d_kernel.data_ptr(),
+                                             device_workspace(wsb), wsb, B, C, H, W, O, kh, kw, s.first, s.second, p.first, p.second,
+                                             d.first, d.second, groups, 0, nullptr));
+        return out;
+    }
+    check_status(ntg_conv2d_backward(dt, x.data_ptr(), w.data_ptr(), g.data_ptr(), out.d_image.data_ptr(),
                                      out.d_kernel.data_ptr(), B, C, H, W, O, kh, kw, s.first, s.second, p.first, p.second, d.first, d.second,
                                      groups, 0));
     return out;
@@ -610,8 +789,21 @@ Tensor conv_transpose2d(const Tensor& image, const Tensor& kernel, utils::my_tup
     const int64_t R = (H - 1) * s.first - 2 * p.first + d.first * (kh - 1) + 1 + op.first;
     const int64_t Cc = (W - 1) * s.second - 2 * p.second + d.second * (kw - 1) + 1 + op.second;
     utils::throw_exception(R > 0 && Cc > 0, "conv_transpose2d output would be empty");
-    Tensor out({B, Cog * groups, R, Cc}, x.dtype());
-    check_status(ntg_conv_transpose2d(static_cast<int>(x.dtype()), x.data_ptr(), w.data_ptr(), out.data_ptr(), B, Cin, H, W, Cog * groups, kh, kw,
+    const DeviceType dev = common_device({&image, &kernel}, "conv_transpose2d");
+    Tensor out({B, Cog * groups, R, Cc}, x.dtype(), dev);
+    const int dt = static_cast<int>(x.dtype());
+    if (dev == DeviceType::HIP) {
+        const int64_t wsb = ntg_conv_transpose2d_workspace_bytes(dt, B, Cin, H, W, Cog * groups, kh, kw, s.first, s.second, p.first, p.second,
+                                                                 d.first, d.second, op.first, op.second, groups);
+        if (wsb >= 0) {
+            check_status(ntg_conv_transpose2d_dev(dt, x.data_ptr(), w.data_ptr(), out.data_ptr(), device_workspace(wsb), wsb, B, Cin, H, W,
+                                                  Cog * groups, kh, kw, s.first, s.second, p.first, p.second, d.first, d.second, op.first,
+                                                  op.second, groups, nullptr));
+            return out;
+        }
+        // (geometry errors are reported by the host entry point below, with its message)
+    }
+    check_status(ntg_conv_transpose2d(dt, x.data_ptr(), w.data_ptr(), out.data_ptr(), B, Cin, H, W, Cog * groups, kh, kw,
                                       s.first, s.second, p.first, p.second, d.first, d.second, op.first, op.second, groups));
     return out;
 }
@@ -661,6 +853,8 @@ static Vol3 vol3(const Tensor& t, bool is_kernel, const char* what) {
 Tensor conv3d(const Tensor& image, const Tensor& kernel, utils::my_n_tuple<3> s, utils::my_n_tuple<3> p, utils::my_n_tuple<3> d, int64_t groups) {
     utils::throw_exception(!image.is_null() && !kernel.is_null(), "Cannot perform operation conv3d on a null tensor");
     utils::throw_exception(image.dtype() == kernel.dtype(), "Expected both kernel and image to have the same dtype for conv3d");
+    if (common_device({&image, &kernel}, "conv3d") == DeviceType::HIP)      // the three-axis forms take device tensors through host memory
+        return functional::conv3d(image.cpu(), kernel.cpu(), s, p, d, groups).to(DeviceType::HIP);
     for (int a = 0; a < 3; ++a) {   // conv.cpp:129-131
         utils::throw_exception(s[a] >= 1, "Conv3d stride cannot be less than 1");
         utils::throw_exception(d[a] >= 1, "Conv3d dilation cannot be less than 1");
@@ -685,6 +879,10 @@ Tensor conv3d(const Tensor& image, const Tensor& kernel, utils::my_n_tuple<3> s,
 ConvGrads conv3d_backward(const Tensor& image, const Tensor& kernel, const Tensor& grad, utils::my_n_tuple<3> s, utils::my_n_tuple<3> p,
                           utils::my_n_tuple<3> d, int64_t groups) {
     utils::throw_exception(!image.is_null() && !kernel.is_null() && !grad.is_null(), "Cannot perform operation conv3d backward on a null tensor");
+    if (common_device({&image, &kernel, &grad}, "conv3d backward") == DeviceType::HIP) {
+        ConvGrads h = functional::conv3d_backward(image.cpu(), kernel.cpu(), grad.cpu(), s, p, d, groups);
+        return {h.d_image.to(DeviceType::HIP), h.d_kernel.to(DeviceType::HIP)};
+    }
     Tensor x = image.contiguous(), w = kernel.contiguous(), g = grad.contiguous();
     const Vol3 xv = vol3(x, false, "conv3d backward"), wv = vol3(w, true, "conv3d backward");
     int64_t L = 1;
@@ -700,6 +898,8 @@ Tensor conv_transpose3d(const Tensor& image, const Tensor& kernel, utils::my_n_t
                         utils::my_n_tuple<3> d, int64_t groups) {
     utils::throw_exception(!image.is_null() && !kernel.is_null(), "Cannot perform operation conv_transpose3d on a null tensor");
     utils::throw_exception(image.dtype() == kernel.dtype(), "Expected both kernel and image to have the same dtype for conv3d transpose");
+    if (common_device({&image, &kernel}, "conv_transpose3d") == DeviceType::HIP)
+        return functional::conv_transpose3d(image.cpu(), kernel.cpu(), s, p, op, d, groups).to(DeviceType::HIP);
     for (int a = 0; a < 3; ++a) {   // conv.cpp:687-691
         utils::throw_exception(s[a] >= 1, "Conv3d Transpose stride cannot be less than 1");
         utils::throw_exception(d[a] >= 1, "Conv3d Transpose dilation cannot be less than 1");

@@ -9,9 +9,12 @@
 //   nt::layers::Linear                              nt/nn/layers/Linear.h:10-20
 //   gradient GEMM selection of TensorGrad linear/matmult   nt/nn/functional/matmult.cpp:37-62, 253-275
 //   nt::utils::throw_exception                      nt/utils/utils.h:178-202
-// nt::Tensor is reduced to what the path needs: dtype + shape + strides over ref-counted host
-// storage (contiguous tensors and transposed views).  All arithmetic is done by libntgemm.so
-// through the host-pointer C ABI (include/ntgemm.h); there is no CPU fallback.
+// nt::Tensor is reduced to what the path needs: dtype + shape + strides over ref-counted storage
+// (contiguous tensors and transposed views), in host memory or -- DeviceType::HIP -- in the GPU's HBM.
+// All arithmetic is done by libntgemm.so: host tensors go through the host-pointer C ABI
+// (include/ntgemm.h; every call pays the PCIe copies), tensors moved to the device with
+// Tensor::to(DeviceType::HIP) through the `_dev` entry points, so a chain of operations
+// (Linear -> Linear, forward -> backward) never leaves HBM.  There is no CPU fallback.
 #pragma once
 #include <array>
 #include <cstdint>
@@ -44,10 +47,15 @@ template <size_t N> using my_n_tuple = std::array<int64_t, N>;
 using SizeRef = std::vector<int64_t>;
 std::string shape_str(const SizeRef& s);
 
+// nt/memory/DeviceEnum.h:6-10 with the device this backend adds
+enum class DeviceType : int8_t { META = -1, CPU = 0, CPUShared = 1, HIP = 2 };
+constexpr DeviceType dCPU = DeviceType::CPU;
+constexpr DeviceType dHIP = DeviceType::HIP;
+
 class Tensor {
 public:
     Tensor() = default;                                           // null tensor
-    Tensor(SizeRef shape, DType dt);                              // uninitialised contiguous tensor
+    Tensor(SizeRef shape, DType dt, DeviceType dev = DeviceType::CPU);   // uninitialised contiguous tensor
     static Tensor Null() { return Tensor(); }
 
     bool is_null() const { return !storage_; }
@@ -56,6 +64,12 @@ public:
     int64_t dims() const { return (int64_t)shape_.size(); }
     int64_t numel() const;
     DType dtype() const { return dtype_; }
+    DeviceType device() const { return device_; }
+    bool is_device() const { return device_ == DeviceType::HIP; }
+    // copy to the other memory (contiguous result); the tensor itself when it already lives there.  Operands of one
+    // operation must share a device; results live where the operands do.  data_ptr() of a device tensor is a device pointer.
+    Tensor to(DeviceType dev) const;
+    Tensor cpu() const { return to(DeviceType::CPU); }
     void* data_ptr() { return storage_.get() + offset_; }
     const void* data_ptr() const { return storage_.get() + offset_; }
     bool is_contiguous() const;
@@ -77,11 +91,12 @@ private:
     int64_t offset_ = 0;        // bytes
     SizeRef shape_, strides_;   // strides in elements
     DType dtype_ = DType::Float32;
+    DeviceType device_ = DeviceType::CPU;
     bool mutable_ = true;
 };
 
 namespace functional {
-Tensor zeros(SizeRef shape, DType dt = DType::Float32);
+Tensor zeros(SizeRef shape, DType dt = DType::Float32, DeviceType dev = DeviceType::CPU);
 Tensor randn(SizeRef shape, DType dt = DType::Float32, uint64_t seed = 0);   // seeded N(0,1) (the reference's randn is unseeded)
 Tensor from_numpy(const std::string& path);                                   // .npy, C order, f2/f4/f8/i1/i2/i4/i8/u1
 bool allclose(const Tensor& a, const Tensor& b, double rtol = 1e-5, double atol = 1e-8);   // compare.h:34
@@ -178,6 +193,7 @@ namespace layers {
 class Linear {
 public:
     Linear(int64_t in_channels, int64_t out_channels, bool use_bias = true, DType dt = DType::Float32, uint64_t seed = 1);
+    Linear& to(DeviceType dev) { Weight = Weight.to(dev); if (use_bias) Bias = Bias.to(dev); return *this; }
     Tensor forward(const Tensor& x) const;
     functional::LinearGrads backward(const Tensor& x, const Tensor& grad) const;
     bool use_bias;

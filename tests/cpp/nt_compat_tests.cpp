@@ -7,6 +7,7 @@
 // (argument validation must fail BEFORE any device work).  Usage: nt_compat_tests <golden dir> [--host-only]
 #include "../../neurotensor_amd/nt_compat/nt_compat.h"
 
+#include <chrono>
 #include <cmath>
 #include <cstdio>
 #include <cstring>
@@ -320,11 +321,139 @@ static void device_cases(const std::string& g) {
     });
 }
 
+// Tensors moved to the GPU with to(DeviceType::HIP): every operation stays in HBM and must give what the same
+// operation gives on host tensors (the same kernels run either way; only the copies differ).
+static void device_resident_cases(const std::string& g) {
+    using nt::DeviceType;
+    // integers bit for bit; floating results within rounding (strided batches and pointer tables may take different kernels)
+    auto same_bits = [](const Tensor& dev, const Tensor& host, const char* what) {
+        nt::utils::throw_exception(dev.device() == DeviceType::HIP, std::string(what) + ": result left the device");
+        Tensor h = dev.cpu();
+        nt::utils::throw_exception(h.shape() == host.shape() && h.dtype() == host.dtype(), std::string(what) + ": shape / dtype");
+        bool ok;
+        if (host.dtype() == DType::BFloat16) {
+            auto f = [](uint16_t v) { uint32_t u = (uint32_t)v << 16; float x; std::memcpy(&x, &u, 4); return x; };
+            ok = true;
+            for (int64_t i = 0; i < host.numel(); ++i) {
+                const float x = f(h.data<uint16_t>()[i]), y = f(host.data<uint16_t>()[i]);
+                ok = ok && std::fabs(x - y) <= 0.02f * (1.0f + std::fabs(y));
+            }
+        } else if (host.dtype() == DType::Float32 || host.dtype() == DType::Float64) {
+            ok = F::allclose(h, host, 1e-4, 1e-4);
+        } else {
+            ok = std::memcmp(h.data_ptr(), host.data_ptr(), (size_t)(host.numel() * nt::dtype_size(host.dtype()))) == 0;
+        }
+        nt::utils::throw_exception(ok, std::string(what) + ": device and host results differ");
+    };
+    run_test("device tensor round trip, views, clone, zeros", [] {
+        Tensor a = F::randn({3, 7, 5}, DType::Float32, 71);
+        Tensor d = a.to(DeviceType::HIP);
+        nt::utils::throw_exception(d.is_device() && d.to(DeviceType::HIP).data_ptr() == d.data_ptr(), "to(same device) must not copy");
+        nt::utils::throw_exception(F::allclose(d, a, 0, 0), "round trip");
+        nt::utils::throw_exception(F::allclose(d.transpose(-1, -2).cpu(), a.transpose(-1, -2).clone(), 0, 0), "strided view to host");
+        nt::utils::throw_exception(F::allclose(d.transpose(-1, -2).clone(), a.transpose(-1, -2).clone(), 0, 0), "clone of a strided device view");
+        nt::utils::throw_exception(F::allclose(d.item(2).clone(), a.item(2).clone(), 0, 0), "item");
+        nt::utils::throw_exception(F::allclose(F::zeros({4, 3}, DType::Float32, DeviceType::HIP), F::zeros({4, 3}), 0, 0), "zeros");
+        nt::utils::throw_exception(F::allclose(d.sum_leading({5}), a.sum_leading({5}), 1e-5, 1e-5), "sum_as over leading dims");
+        nt::utils::throw_exception(F::allclose(d.sum_leading({7, 1}), a.sum_leading({7, 1}), 1e-5, 1e-5), "sum_as over an inner dim");
+    });
+    expect_throw("matmult of a host and a device tensor", [] {
+        nt::matmult(F::zeros({4, 4}), F::zeros({4, 4}, DType::Float32, DeviceType::HIP));
+    });
+    expect_throw("linear with the bias on the other device", [] {
+        nt::linear(F::zeros({4, 4}, DType::Float32, DeviceType::HIP), F::zeros({4, 4}, DType::Float32, DeviceType::HIP), F::zeros({4}));
+    });
+    for (DType dt : {DType::Float32, DType::Float64, DType::BFloat16, DType::int32}) {
+        run_test((std::string("device matmult / linear == host, ") + nt::dtype_name(dt)).c_str(), [&] {
+            Tensor a = F::randn({5, 2, 33, 20}, dt, 81), b = F::randn({2, 20, 17}, dt, 82), a2 = F::randn({2, 20, 33}, dt, 83);
+            Tensor bb = F::randn({5, 2, 20, 17}, dt, 87);
+            Tensor da = a.to(DeviceType::HIP), db = b.to(DeviceType::HIP), da2 = a2.to(DeviceType::HIP), dbb = bb.to(DeviceType::HIP);
+            same_bits(nt::matmult(da, db), nt::matmult(a, b), "bigger A");
+            same_bits(nt::matmult(da2, dbb, true, false), nt::matmult(a2, bb, true, false), "bigger B, transpose_a");
+            same_bits(nt::matmult(da, db.transpose(-1, -2).clone(), false, true), nt::matmult(a, b.transpose(-1, -2).clone(), false, true), "transpose_b");
+            same_bits(nt::matmult(da, db.transpose(-1, -2).clone().transpose(-1, -2)), nt::matmult(a, b), "transposed device view == flag");
+            Tensor c = F::randn({5, 2, 33, 17}, dt, 84), dc = c.to(DeviceType::HIP);
+            nt::matmult(a, b, c);
+            nt::matmult(da, db, dc);
+            same_bits(dc, c, "out= accumulates on the device");
+            if (dt != DType::int32) {
+                Tensor bias = F::randn({17}, dt, 85), bias2 = F::randn({2, 33, 1}, dt, 86);
+                same_bits(nt::linear(da, db, bias.to(DeviceType::HIP)), nt::linear(a, b, bias), "linear, bias [n]");
+                same_bits(nt::linear(da, db, bias2.to(DeviceType::HIP)), nt::linear(a, b, bias2), "linear, bias [2, m, 1]");
+            }
+        });
+    }
+    run_test("Linear -> Linear forward and backward without leaving the device", [] {
+        nt::layers::Linear l1(64, 48, true, DType::Float32, 91), l2(48, 24, true, DType::Float32, 93);
+        Tensor x = F::randn({6, 10, 64}, DType::Float32, 95), gy = F::randn({6, 10, 24}, DType::Float32, 96);
+        Tensor h = l1.forward(x), y = l2.forward(h);
+        F::LinearGrads g2 = l2.backward(h, gy), g1 = l1.backward(x, g2.dx);
+        nt::layers::Linear d1 = l1, d2 = l2;
+        d1.to(DeviceType::HIP); d2.to(DeviceType::HIP);
+        Tensor dx = x.to(DeviceType::HIP), dgy = gy.to(DeviceType::HIP);
+        Tensor dh = d1.forward(dx), dy = d2.forward(dh);
+        F::LinearGrads dg2 = d2.backward(dh, dgy), dg1 = d1.backward(dx, dg2.dx);
+        nt::utils::throw_exception(dy.is_device() && dg1.dx.is_device() && dg1.dw.is_device() && dg1.db.is_device(), "results left the device");
+        nt::utils::throw_exception(F::allclose(dy, y, 1e-4, 1e-4), "forward");
+        nt::utils::throw_exception(F::allclose(dg1.dx, g1.dx, 1e-4, 1e-4) && F::allclose(dg2.dw, g2.dw, 1e-4, 1e-3), "dx / dw of the chain");
+        // dW of a batched input and db are sums over the leading dims: one GEMM with a row of ones on the device
+        nt::utils::throw_exception(F::allclose(dg1.dw, g1.dw, 1e-4, 1e-3) && F::allclose(dg1.db, g1.db, 1e-4, 1e-3) &&
+                                       F::allclose(dg2.db, g2.db, 1e-4, 1e-3), "reduced gradients");
+    });
+    run_test("two Linear layers on 2048 rows: host tensors against device tensors (timing printed)", [] {
+        nt::layers::Linear l1(1024, 1024, true, DType::Float32, 97), l2(1024, 1024, true, DType::Float32, 98);
+        Tensor x = F::randn({2048, 1024}, DType::Float32, 99);
+        auto now = [] { return std::chrono::steady_clock::now(); };
+        auto ms = [](auto a, auto b) { return std::chrono::duration<double, std::milli>(b - a).count(); };
+        Tensor y = l2.forward(l1.forward(x));                       // warm-up (library load, clocks)
+        auto t0 = now();
+        for (int i = 0; i < 5; ++i) y = l2.forward(l1.forward(x));
+        const double host_ms = ms(t0, now()) / 5;
+        nt::layers::Linear d1 = l1, d2 = l2;
+        d1.to(DeviceType::HIP); d2.to(DeviceType::HIP);
+        Tensor dx = x.to(DeviceType::HIP);
+        Tensor dy = d2.forward(d1.forward(dx));
+        Tensor first = dy.cpu();
+        t0 = now();
+        for (int i = 0; i < 50; ++i) dy = d2.forward(d1.forward(dx));
+        Tensor last = dy.cpu();                                      // (waits for the stream)
+        const double dev_ms = ms(t0, now()) / 50;
+        std::printf("       host tensors %.3f ms per chain (PCIe copies in every call), device tensors %.3f ms\n", host_ms, dev_ms);
+        nt::utils::throw_exception(F::allclose(last, y, 1e-4, 1e-3) && F::allclose(first, last, 0, 0), "chain result");
+    });
+    for (const char* sfx : {"", "_grouped_batched"}) {
+        run_test((std::string("device conv2d forward / backward == golden") + sfx).c_str(), [&] {
+            const bool grouped = std::strstr(sfx, "grouped") != nullptr;
+            const int64_t pad = grouped ? 0 : 1, groups = grouped ? 2 : 1;
+            auto fx = [&](const char* part) { return F::from_numpy(g + "/conv2d_" + part + sfx + ".npy"); };
+            Tensor x = fx("input").to(DeviceType::HIP), w = fx("weight").to(DeviceType::HIP);
+            Tensor o = nt::conv2d(x, w, {1, 1}, {pad, pad}, {1, 1}, groups);
+            nt::utils::throw_exception(o.is_device() && F::allclose(o, fx("output"), 1e-4, 1e-4), "conv2d output");
+            F::ConvGrads gr = F::conv2d_backward(x, w, fx("grad").to(DeviceType::HIP), {1, 1}, {pad, pad}, {1, 1}, groups);
+            nt::utils::throw_exception(gr.d_image.is_device() && F::allclose(gr.d_image, fx("xgrad"), 1e-4, 1e-4), "conv2d xgrad");
+            nt::utils::throw_exception(F::allclose(gr.d_kernel, fx("wgrad"), 1e-4, 1e-3), "conv2d wgrad");
+        });
+    }
+    run_test("device conv2d (channels-last path), conv1d, conv_transpose2d, unfold2d, conv3d == host", [&] {
+        Tensor x = F::randn({3, 32, 9, 11}, DType::Float32, 101), w = F::randn({24, 16, 3, 3}, DType::Float32, 102);
+        Tensor dx = x.to(DeviceType::HIP), dw = w.to(DeviceType::HIP);
+        nt::utils::throw_exception(F::allclose(nt::conv2d(dx, dw, {1, 1}, {1, 1}, {1, 1}, 2), nt::conv2d(x, w, {1, 1}, {1, 1}, {1, 1}, 2), 1e-5, 1e-5), "conv2d");
+        Tensor x1 = F::randn({4, 6, 40}, DType::Float32, 103), w1 = F::randn({8, 3, 5}, DType::Float32, 104);
+        same_bits(nt::conv1d(x1.to(DeviceType::HIP), w1.to(DeviceType::HIP), 2, 2, 1, 2), nt::conv1d(x1, w1, 2, 2, 1, 2), "conv1d");
+        Tensor xt = F::randn({2, 6, 7, 5}, DType::Float32, 105), wt = F::randn({6, 4, 3, 3}, DType::Float32, 106);
+        nt::utils::throw_exception(F::allclose(nt::conv_transpose2d(xt.to(DeviceType::HIP), wt.to(DeviceType::HIP), {2, 2}, {1, 1}, {1, 1}, {1, 1}, 2),
+                                               nt::conv_transpose2d(xt, wt, {2, 2}, {1, 1}, {1, 1}, {1, 1}, 2), 1e-5, 1e-5), "conv_transpose2d");
+        same_bits(F::unfold2d(dx, {3, 2}, {1, 2}, {1, 1}, {2, 2}, true), F::unfold2d(x, {3, 2}, {1, 2}, {1, 1}, {2, 2}, true), "unfold2d");
+        Tensor x3 = F::randn({2, 4, 5, 6, 7}, DType::Float32, 107), w3 = F::randn({6, 4, 2, 3, 2}, DType::Float32, 108);
+        same_bits(nt::conv3d(x3.to(DeviceType::HIP), w3.to(DeviceType::HIP)), nt::conv3d(x3, w3), "conv3d");
+    });
+}
+
 int main(int argc, char** argv) {
     if (argc < 2) { std::fprintf(stderr, "usage: %s <golden dir> [--host-only]\n", argv[0]); return 2; }
     const bool host_only = argc > 2 && std::strcmp(argv[2], "--host-only") == 0;
     host_only_cases();
-    if (!host_only) device_cases(argv[1]);
+    if (!host_only) { device_cases(argv[1]); device_resident_cases(argv[1]); }
     std::printf("%d cases, %d failed\n", g_run, g_failed);
     return g_failed ? 1 : 0;
 }

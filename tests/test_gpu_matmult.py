@@ -197,6 +197,32 @@ def test_c_modes(dtype):
     assert_close(got, ref0, to_f64(a, bf), to_f64(b, bf), k, dtype, "overwrite")
 
 
+@pytest.mark.parametrize("tdtype", [torch.float32, torch.float64, torch.bfloat16, torch.float16, torch.int32, torch.int8],
+                         ids=["fp32", "fp64", "bf16", "fp16", "int32", "int8"])
+def test_empty_k_is_an_empty_sum(tdtype):
+    """k = 0: C += nothing leaves C alone, overwrite gives zeros, bias mode gives the broadcast bias -- for a strided
+    batch, without touching A or B (the product kernels themselves assume at least one k)."""
+    lib = _lib.load()
+    st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    batch, m, n = 3, 48, 80
+    c0 = (torch.arange(batch * m * n, device=DEV) % 13 - 6).to(tdtype).reshape(batch, m, n)
+    bias = (torch.arange(batch * n, device=DEV) % 7 - 3).to(tdtype).reshape(batch, 1, n)
+    dummy = torch.zeros(16, dtype=tdtype, device=DEV)
+    for mode, want in ((_lib.C_ACCUMULATE, c0), (_lib.C_OVERWRITE, torch.zeros_like(c0)), (_lib.C_BIAS, bias.expand(batch, m, n))):
+        c = c0.clone()
+        d = _lib.GemmDesc()
+        d.dtype = F.ntg_dtype(c)
+        d.c_mode = mode
+        d.m, d.k, d.n, d.batches = m, 0, n, batch
+        d.stride_c = m * n
+        if mode == _lib.C_BIAS:
+            d.bias = bias.data_ptr()
+            d.bias_batch_stride, d.bias_row_stride, d.bias_col_stride = n, 0, 1
+        _lib.check(lib.ntg_gemm_dev(ctypes.byref(d), dummy.data_ptr(), dummy.data_ptr(), c.data_ptr(), st))
+        torch.cuda.synchronize()
+        assert torch.equal(c, want), mode
+
+
 def test_host_batch_with_repeated_pointers():
     """nt_matmult_batch: uniform shape, entries of A/B may repeat (broadcast by handle)."""
     rng = np.random.default_rng(500)
