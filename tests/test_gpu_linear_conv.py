@@ -322,6 +322,8 @@ IMPLICIT_GEOMS = [
     (4, 64, 15, 15, 40, 3, 3, 1, 1, 1, 1),                 # Ho*Wo = 225
     (3, 64, 14, 14, 48, 3, 3, 2, 1, 1, 2),                 # Ho*Wo = 49, two groups of 32 channels
     (2, 128, 19, 11, 72, 3, 2, 1, (2, 0), (2, 1), 1),               # Ho*Wo = 190
+    (2, 64, 1, 50, 48, 1, 5, 1, (0, 2), 1, 1),                      # one image row: what conv1d lowers to
+    (1, 32, 40, 6, 8, 4, 1, (3, 1), 0, (2, 1), 1),                  # fewer filters than one tile row, one tap column
 ]
 
 
