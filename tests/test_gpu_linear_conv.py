@@ -607,3 +607,35 @@ def test_config5a_conv2d_resnet_block():
         assert np.abs(out[b:b + 1].cpu().numpy() - ref).max() <= tol
     ref_all = torch.nn.functional.conv2d(tx.double(), tw.double(), padding=1)
     assert (out.double() - ref_all).abs().max().item() <= tol
+    # the same block in BFloat16: the first 59 images and the last 5 come from two launches on different tiles
+    xh, wh = tx.bfloat16(), tw.bfloat16()
+    outh = F.conv2d(xh, wh, stride=1, padding=1)
+    refh = torch.nn.functional.conv2d(xh.double(), wh.double(), padding=1)
+    scale = refh.abs().max().item()
+    for lo, hi in ((0, 59), (59, 64)):
+        assert (outh[lo:hi].double() - refh[lo:hi]).abs().max().item() <= HALF_REL * scale
+    del ref_all, refh
+
+
+def test_config5a_conv2d_gradients_full_size():
+    """Both gradients of the config-5a block at full size (channels-last kernels), Float32 against the stated bound
+    and BFloat16 against 2e-2 of the largest gradient; references from torch autograd in double."""
+    rng = np.random.default_rng(1008)
+    x = dev(rng.standard_normal((64, 256, 56, 56)).astype(np.float32))
+    w = dev((rng.standard_normal((256, 256, 3, 3)) / np.sqrt(2304.0)).astype(np.float32))
+    g = dev(rng.standard_normal((64, 256, 56, 56)).astype(np.float32))
+    for half in (False, True):
+        tx, tw, tg = (t.bfloat16() if half else t for t in (x, w, g))
+        rx = tx.double().requires_grad_(True)
+        rw = tw.double().requires_grad_(True)
+        torch.nn.functional.conv2d(rx, rw, padding=1).backward(tg.double())
+        dx, dw = F.conv2d_backward(tx, tw, tg, stride=1, padding=1)
+        ex = (dx.double() - rx.grad).abs().max().item()
+        ew = (dw.double() - rw.grad).abs().max().item()
+        if half:
+            assert ex <= HALF_REL * rx.grad.abs().max().item()
+            assert ew <= HALF_REL * rw.grad.abs().max().item()
+        else:
+            assert ex <= 1e-5 * 2304 * float(tg.abs().max() * tw.abs().max())
+            assert ew <= 1e-5 * 200704 * float(tg.abs().max() * tx.abs().max())
+        del rx, rw, dx, dw
