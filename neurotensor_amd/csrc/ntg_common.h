@@ -156,8 +156,9 @@ hipError_t launch_splitk_reduce(int dtype, const void* part, int splits, const G
 // the gradient-to-image convolution
 hipError_t launch_reduce_batch(int dtype, const void* part, void* out, int64_t batch, int64_t n, int accumulate, hipStream_t s);
 hipError_t launch_nchw_to_nhwc(int64_t elem_size, const void* in, void* out, int64_t batch, int64_t C, int64_t P, hipStream_t s);
-hipError_t launch_weights_channels_last(int64_t elem_size, const void* w, void* wp, int64_t rows, int64_t cg, int64_t taps, hipStream_t s);
-hipError_t launch_flip_weights_channels_last(int64_t es, const void* w, void* wt, int64_t groups, int64_t og, int64_t cg, int64_t taps, hipStream_t s);
+hipError_t launch_weights_channels_last(int64_t es, const void* w, void* wp, int64_t rows, int64_t cg, int64_t cgp, int64_t taps, hipStream_t s);
+hipError_t launch_nchw_to_nhwc_padded(int64_t es, const void* in, void* out, int64_t batch, int64_t groups, int64_t cg, int64_t cgp, int64_t P, hipStream_t s);
+hipError_t launch_flip_weights_channels_last(int64_t es, const void* w, void* wt, int64_t groups, int64_t og, int64_t ogp, int64_t cg, int64_t taps, hipStream_t s);
 // channels-last convolution (image [B][pixel][C], weights [O][(r, q, c)]); F16 / BF16 / F32, two spatial axes
 hipError_t launch_conv_nhwc(int dtype, const GemmParams& p, hipStream_t s);
 hipError_t launch_conv_nhwc_dw(int dtype, const GemmParams& p, hipStream_t s);

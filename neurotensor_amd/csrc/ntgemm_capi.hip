@@ -602,39 +602,50 @@ static bool conv_nhwc_offsets_fit(int64_t channels, int64_t es, const Geo3& g) {
     const int64_t reach = ((pr + g.k[1] * g.d[1]) * g.sz[2] + pc + g.k[2] * g.d[2]) * channels * es;
     return channels * g.vol() * es < (1LL << 30) && reach < (1LL << 30);
 }
+// A K-step of the channels-last kernel is 64 bytes of channels of one tap, so the copy pads the channels of each group
+// with zeros to the next multiple of 64 bytes (and the permuted weights likewise).  The padding is arithmetic spent on
+// zeros: accepted up to 4x for the 16-bit types, whose element-wise gather is bound by the vector ALU (beyond that --
+// RGB input layers -- the gathering kernels are the better choice); Float32 takes whole runs only: its element-wise
+// DMA gather was measured faster than a padded copy (24 -> 32 channels: 48 against 60 us).  0: not accepted.
+static int64_t nhwc_padded_channels(int64_t es, int64_t cg) {
+    const int64_t step = 64 / es, cgp = (cg + step - 1) / step * step;
+    return cg > 0 && cgp <= (es == 2 ? 4 : 1) * cg ? cgp : 0;
+}
 static bool conv_nhwc_ok(int dtype, int64_t channels, int64_t out_channels, int64_t groups, const Geo3& g) {
     if (dtype != ntg::DT_F32 && dtype != ntg::DT_F16 && dtype != ntg::DT_BF16) return false;
     if (g.nd != 2 || !conv_implicit_g(dtype, channels, g)) return false;
-    const int64_t es = ntg::elem_size(dtype), cg = channels / groups;
-    return cg % (64 / es) == 0 && out_channels > 0 && conv_nhwc_offsets_fit(channels, es, g);
+    const int64_t es = ntg::elem_size(dtype), cgp = nhwc_padded_channels(es, channels / groups);
+    return cgp > 0 && out_channels > 0 && conv_nhwc_offsets_fit(groups * cgp, es, g);
 }
 static int64_t conv_nhwc_workspace(int dtype, int64_t batch, int64_t channels, int64_t out_channels, int64_t groups, const Geo3& g) {
-    const int64_t es = ntg::elem_size(dtype);
-    return (int64_t)align_up((size_t)(batch * channels * g.vol() * es), 256) + out_channels * (channels / groups) * g.taps() * es;
+    const int64_t es = ntg::elem_size(dtype), cgp = nhwc_padded_channels(es, channels / groups);
+    return (int64_t)align_up((size_t)(batch * groups * cgp * g.vol() * es), 256) + out_channels * cgp * g.taps() * es;
 }
 static int conv_forward_nhwc(int dtype, const void* image, const void* kernel, void* out, void* ws, int64_t batch, int64_t channels,
                              int64_t out_channels, const Geo3& g, int64_t groups, hipStream_t hs) {
     const int64_t es = ntg::elem_size(dtype), cg = channels / groups, og = out_channels / groups;
-    const int64_t L = g.L(), taps = g.taps(), vol = g.vol(), K = taps * cg;
+    const int64_t cgp = nhwc_padded_channels(es, cg), chp = groups * cgp;      // channels per group / per pixel in the copy
+    const int64_t L = g.L(), taps = g.taps(), vol = g.vol(), K = taps * cgp;
     char* ws_img = static_cast<char*>(ws);
-    char* ws_w = ws_img + align_up((size_t)(batch * channels * vol * es), 256);
-    hipError_t e = ntg::launch_nchw_to_nhwc(es, image, ws_img, batch, channels, vol, hs);
+    char* ws_w = ws_img + align_up((size_t)(batch * chp * vol * es), 256);
+    hipError_t e = cgp == cg ? ntg::launch_nchw_to_nhwc(es, image, ws_img, batch, channels, vol, hs)
+                             : ntg::launch_nchw_to_nhwc_padded(es, image, ws_img, batch, groups, cg, cgp, vol, hs);
     if (e != hipSuccess) return hip_fail(e, "channels-last copy launch");
-    e = ntg::launch_weights_channels_last(es, kernel, ws_w, out_channels, cg, taps, hs);
+    e = ntg::launch_weights_channels_last(es, kernel, ws_w, out_channels, cg, cgp, taps, hs);
     if (e != hipSuccess) return hip_fail(e, "weight permutation launch");
     for (int64_t gi = 0; gi < groups; ++gi) {
         ntg::GemmParams p;
         std::memset(&p, 0, sizeof p);
         p.M = (int)og; p.K = (int)K; p.N = (int)L; p.batch = (int)batch;
         p.A = ws_w + gi * og * K * es;
-        p.B = ws_img + gi * cg * es;
+        p.B = ws_img + gi * cgp * es;
         p.C = static_cast<char*>(out) + gi * og * L * es;
-        p.lda = K; p.ldb = channels; p.ldc = L;
-        p.sA = 0; p.sB = channels * vol; p.sC = out_channels * L;
+        p.lda = K; p.ldb = chp; p.ldc = L;
+        p.sA = 0; p.sB = chp * vol; p.sC = out_channels * L;
         p.cmode = ntg::C_OVERWRITE;
         p.vecA_ok = 1; p.vecB_ok = 1;
-        fill_conv_geom(p.conv, cg, g);
-        p.conv.chan = (int)channels;               // elements from one pixel to the next
+        fill_conv_geom(p.conv, cgp, g);
+        p.conv.chan = (int)chp;                    // elements from one pixel to the next
         e = ntg::launch_conv_nhwc(dtype, p, hs);
         if (e != hipSuccess) return hip_fail(e, "channels-last convolution launch");
     }
@@ -707,12 +718,14 @@ static int64_t conv_dimage_nhwc_workspace(int dtype, int64_t batch, int64_t chan
 static int conv_dimage_nhwc(int dtype, const void* kernel, const void* grad_out, void* d_image, void* ws, int64_t batch,
                             int64_t channels, int64_t out_channels, const Geo3& g, int64_t groups, int accumulate, hipStream_t hs) {
     const int64_t es = ntg::elem_size(dtype), cg = channels / groups, og = out_channels / groups;
-    const int64_t L = g.L(), taps = g.taps(), vol = g.vol(), K = taps * og;
+    const int64_t ogp = nhwc_padded_channels(es, og), ochp = groups * ogp;      // out channels per group / per pixel in the copy
+    const int64_t L = g.L(), taps = g.taps(), vol = g.vol(), K = taps * ogp;
     char* ws_gy = static_cast<char*>(ws);
-    char* ws_w = ws_gy + align_up((size_t)(batch * out_channels * L * es), 256);
-    hipError_t e = ntg::launch_nchw_to_nhwc(es, grad_out, ws_gy, batch, out_channels, L, hs);
+    char* ws_w = ws_gy + align_up((size_t)(batch * ochp * L * es), 256);
+    hipError_t e = ogp == og ? ntg::launch_nchw_to_nhwc(es, grad_out, ws_gy, batch, out_channels, L, hs)
+                             : ntg::launch_nchw_to_nhwc_padded(es, grad_out, ws_gy, batch, groups, og, ogp, L, hs);
     if (e != hipSuccess) return hip_fail(e, "channels-last copy launch");
-    e = ntg::launch_flip_weights_channels_last(es, kernel, ws_w, groups, og, cg, taps, hs);
+    e = ntg::launch_flip_weights_channels_last(es, kernel, ws_w, groups, og, ogp, cg, taps, hs);
     if (e != hipSuccess) return hip_fail(e, "weight flip launch");
     const Geo3 t = geo_dimage(g);
     for (int64_t gi = 0; gi < groups; ++gi) {
@@ -720,14 +733,14 @@ static int conv_dimage_nhwc(int dtype, const void* kernel, const void* grad_out,
         std::memset(&p, 0, sizeof p);
         p.M = (int)cg; p.K = (int)K; p.N = (int)vol; p.batch = (int)batch;
         p.A = ws_w + gi * cg * K * es;
-        p.B = ws_gy + gi * og * es;
+        p.B = ws_gy + gi * ogp * es;
         p.C = static_cast<char*>(d_image) + gi * cg * vol * es;
-        p.lda = K; p.ldb = out_channels; p.ldc = vol;
-        p.sA = 0; p.sB = out_channels * L; p.sC = channels * vol;
+        p.lda = K; p.ldb = ochp; p.ldc = vol;
+        p.sA = 0; p.sB = ochp * L; p.sC = channels * vol;
         p.cmode = accumulate ? ntg::C_ACCUMULATE : ntg::C_OVERWRITE;
         p.vecA_ok = 1; p.vecB_ok = 1;
-        fill_conv_geom(p.conv, og, t);
-        p.conv.chan = (int)out_channels;
+        fill_conv_geom(p.conv, ogp, t);
+        p.conv.chan = (int)ochp;
         e = ntg::launch_conv_nhwc(dtype, p, hs);
         if (e != hipSuccess) return hip_fail(e, "channels-last conv_dimage launch");
     }

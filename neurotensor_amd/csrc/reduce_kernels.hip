@@ -258,58 +258,100 @@ hipError_t launch_nchw_to_nhwc(int64_t es, const void* in, void* out, int64_t ba
     return hipGetLastError();
 }
 
-// wp[o][t][c] = w[o][c][t]: convolution weights with the channel index fastest (the k order of the channels-last gather)
-template <class T>
-__global__ void __launch_bounds__(256) weights_channels_last_kernel(const T* __restrict__ w, T* __restrict__ wp, const int64_t rows,
-                                                                    const int64_t cg, const int64_t taps) {
-    const int64_t total = rows * cg * taps;
-    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-    for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += stride) {
-        const int64_t c = idx % cg;
-        const int64_t t = (idx / cg) % taps;
-        const int64_t o = idx / (cg * taps);
-        wp[idx] = w[(o * cg + c) * taps + t];
-    }
-}
-
 // wt[g][c][t][oc] = w[g*og + oc][c][taps-1-t]: the weights of the convolution that maps the output gradient back to the
-// image (channel axes swapped inside each group, taps reversed), with the out channels of one tap consecutive.
+// image (channel axes swapped inside each group, taps reversed), with the out channels of one tap consecutive and
+// padded with zeros from og to ogp per tap.
 template <class T>
 __global__ void __launch_bounds__(256) flip_weights_channels_last_kernel(const T* __restrict__ w, T* __restrict__ wt, const int64_t groups,
-                                                                         const int64_t og, const int64_t cg, const int64_t taps) {
-    const int64_t total = groups * og * cg * taps;
+                                                                         const int64_t og, const int64_t ogp, const int64_t cg, const int64_t taps) {
+    const int64_t total = groups * ogp * cg * taps;
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
     for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += stride) {
-        const int64_t oc = idx % og;
-        int64_t r = idx / og;
+        const int64_t oc = idx % ogp;
+        int64_t r = idx / ogp;
         const int64_t t = r % taps;
         r /= taps;
         const int64_t c = r % cg;
         const int64_t g = r / cg;
-        wt[idx] = w[((g * og + oc) * cg + c) * taps + (taps - 1 - t)];
+        wt[idx] = oc < og ? w[((g * og + oc) * cg + c) * taps + (taps - 1 - t)] : (T)0;
     }
 }
 
-hipError_t launch_flip_weights_channels_last(int64_t es, const void* w, void* wt, int64_t groups, int64_t og, int64_t cg, int64_t taps, hipStream_t s) {
-    const int64_t total = groups * og * cg * taps;
+hipError_t launch_flip_weights_channels_last(int64_t es, const void* w, void* wt, int64_t groups, int64_t og, int64_t ogp, int64_t cg, int64_t taps, hipStream_t s) {
+    const int64_t total = groups * ogp * cg * taps;
     if (total == 0) return hipSuccess;
     const dim3 g(grid_for(total)), t(256);
     switch (es) {
-    case 2: hipLaunchKernelGGL(flip_weights_channels_last_kernel<uint16_t>, g, t, 0, s, (const uint16_t*)w, (uint16_t*)wt, groups, og, cg, taps); break;
-    case 4: hipLaunchKernelGGL(flip_weights_channels_last_kernel<uint32_t>, g, t, 0, s, (const uint32_t*)w, (uint32_t*)wt, groups, og, cg, taps); break;
+    case 2: hipLaunchKernelGGL(flip_weights_channels_last_kernel<uint16_t>, g, t, 0, s, (const uint16_t*)w, (uint16_t*)wt, groups, og, ogp, cg, taps); break;
+    case 4: hipLaunchKernelGGL(flip_weights_channels_last_kernel<uint32_t>, g, t, 0, s, (const uint32_t*)w, (uint32_t*)wt, groups, og, ogp, cg, taps); break;
     default: return hipErrorInvalidValue;
     }
     return hipGetLastError();
 }
 
-hipError_t launch_weights_channels_last(int64_t es, const void* w, void* wp, int64_t rows, int64_t cg, int64_t taps, hipStream_t s) {
-    const int64_t total = rows * cg * taps;
+// wp[o][t][c] = w[o][c][t]: convolution weights with the channel index fastest (the k order of the channels-last gather),
+// the channels of one tap padded with zeros from cg to cgp
+template <class T>
+__global__ void __launch_bounds__(256) weights_channels_last_kernel(const T* __restrict__ w, T* __restrict__ wp, const int64_t rows,
+                                                                    const int64_t cg, const int64_t cgp, const int64_t taps) {
+    const int64_t total = rows * cgp * taps;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += stride) {
+        const int64_t c = idx % cgp;
+        const int64_t t = (idx / cgp) % taps;
+        const int64_t o = idx / (cgp * taps);
+        wp[idx] = c < cg ? w[(o * cg + c) * taps + t] : (T)0;
+    }
+}
+
+hipError_t launch_weights_channels_last(int64_t es, const void* w, void* wp, int64_t rows, int64_t cg, int64_t cgp, int64_t taps, hipStream_t s) {
+    const int64_t total = rows * cgp * taps;
     if (total == 0) return hipSuccess;
     const dim3 g(grid_for(total)), t(256);
     switch (es) {
-    case 2: hipLaunchKernelGGL(weights_channels_last_kernel<uint16_t>, g, t, 0, s, (const uint16_t*)w, (uint16_t*)wp, rows, cg, taps); break;
-    case 4: hipLaunchKernelGGL(weights_channels_last_kernel<uint32_t>, g, t, 0, s, (const uint32_t*)w, (uint32_t*)wp, rows, cg, taps); break;
+    case 2: hipLaunchKernelGGL(weights_channels_last_kernel<uint16_t>, g, t, 0, s, (const uint16_t*)w, (uint16_t*)wp, rows, cg, cgp, taps); break;
+    case 4: hipLaunchKernelGGL(weights_channels_last_kernel<uint32_t>, g, t, 0, s, (const uint32_t*)w, (uint32_t*)wp, rows, cg, cgp, taps); break;
     default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+
+// out[b][p][g*cgp + c] = in[b][g*cg + c][p] for c < cg, 0 for cg <= c < cgp: the channels-last copy with the channels of
+// every group padded to cgp.  64 x 64 tiles of (channel inside the group, pixel) through LDS, like the plain copy.
+template <class T>
+__global__ void __launch_bounds__(256) nchw_to_nhwc_pad_kernel(const T* __restrict__ in, T* __restrict__ out, const int64_t groups,
+                                                               const int64_t cg, const int64_t cgp, const int64_t P, const int cblocks) {
+    __shared__ T tile[64][65];
+    const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+    const int64_t g = blockIdx.y / cblocks, c0 = (int64_t)(blockIdx.y % cblocks) * 64;
+    const int64_t p0 = (int64_t)blockIdx.x * 64, b = blockIdx.z;
+    const T* src = in + (b * groups + g) * cg * P;
+    T* dst = out + b * P * groups * cgp + g * cgp;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        const int64_t c = c0 + ty + 4 * i, pp = p0 + tx;
+        tile[ty + 4 * i][tx] = (c < cg && pp < P) ? src[c * P + pp] : (T)0;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        const int64_t pp = p0 + ty + 4 * i, c = c0 + tx;
+        if (c < cgp && pp < P) dst[pp * groups * cgp + c] = tile[tx][ty + 4 * i];
+    }
+}
+
+hipError_t launch_nchw_to_nhwc_padded(int64_t es, const void* in, void* out, int64_t batch, int64_t groups, int64_t cg, int64_t cgp, int64_t P, hipStream_t s) {
+    if (batch * groups * cgp * P == 0) return hipSuccess;
+    const int64_t cblocks = (cgp + 63) / 64, gx = (P + 63) / 64, gy = cblocks * groups;
+    if (gx > 0x7fffffffLL || gy > 65535) return hipErrorInvalidValue;
+    for (int64_t b0 = 0; b0 < batch; b0 += 65535) {                    // (grid z limit)
+        const int64_t nb = batch - b0 < 65535 ? batch - b0 : 65535;
+        const dim3 g((unsigned)gx, (unsigned)gy, (unsigned)nb), t(256);
+        const char* src = static_cast<const char*>(in) + b0 * groups * cg * P * es;
+        char* dst = static_cast<char*>(out) + b0 * groups * cgp * P * es;
+        if (es == 2) hipLaunchKernelGGL(nchw_to_nhwc_pad_kernel<uint16_t>, g, t, 0, s, (const uint16_t*)src, (uint16_t*)dst, groups, cg, cgp, P, (int)cblocks);
+        else if (es == 4) hipLaunchKernelGGL(nchw_to_nhwc_pad_kernel<uint32_t>, g, t, 0, s, (const uint32_t*)src, (uint32_t*)dst, groups, cg, cgp, P, (int)cblocks);
+        else return hipErrorInvalidValue;
     }
     return hipGetLastError();
 }

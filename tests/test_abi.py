@@ -78,7 +78,11 @@ def test_argument_errors_do_not_need_a_device():
     fast = lib.ntg_conv2d_fast_workspace_bytes
     assert fast(_lib.BFLOAT16, 2, 64, 7, 7, 48, 3, 3, 1, 1, 1, 1, 1, 1, 2) == 12544 + 48 * 32 * 9 * 2    # 2*64*49*2 = 12544
     assert fast(_lib.FLOAT32, 1, 16, 5, 5, 8, 3, 3, 1, 1, 1, 1, 1, 1, 1) == 1792 + 8 * 16 * 9 * 4        # 1600 -> 1792
-    assert fast(_lib.BFLOAT16, 1, 16, 5, 5, 8, 3, 3, 1, 1, 1, 1, 1, 1, 1) == 0                            # 32 bytes of channels: gathers
+    # 16-bit: channels per group are padded to whole 64-byte runs in the copy (up to 4x); Float32 takes whole runs only
+    assert fast(_lib.BFLOAT16, 1, 16, 5, 5, 8, 3, 3, 1, 1, 1, 1, 1, 1, 1) == 1792 + 8 * 32 * 9 * 2       # 16 -> 32 channels: 1600 -> 1792
+    assert fast(_lib.FLOAT16, 2, 24, 5, 5, 8, 3, 3, 1, 1, 1, 1, 1, 1, 2) == 6400 + 8 * 32 * 9 * 2         # 2 groups of 12 -> 32
+    assert fast(_lib.BFLOAT16, 1, 3, 8, 8, 4, 3, 3, 1, 1, 1, 1, 1, 1, 1) == 0                             # 3 -> 32 would be 10x: gathers
+    assert fast(_lib.FLOAT32, 1, 24, 8, 8, 4, 3, 3, 1, 1, 1, 1, 1, 1, 1) == 0                             # 24 is not a multiple of 16
     assert fast(_lib.FLOAT64, 1, 16, 5, 5, 8, 3, 3, 1, 1, 1, 1, 1, 1, 1) == 0
     assert fast(_lib.INT32, 1, 16, 5, 5, 8, 3, 3, 1, 1, 1, 1, 1, 1, 1) == 16 * 9 * 25 * 4
     assert fast(_lib.FLOAT32, 4, 64, 8, 8, 32, 1, 1, 1, 1, 0, 0, 1, 1, 1) == 0                            # 1x1: product in place
