@@ -45,7 +45,9 @@ hipError_t launch_conv_mfma_f32(bool tb, int nd, const GemmParams& p, hipStream_
 hipError_t launch_conv_nhwc_f32(const GemmParams& p, hipStream_t s) {
     return ring_f32_tile_edge(p) == 128 ? launch_ring_nhwc_cfg<DT_F32, 2>(p, s) : launch_ring_nhwc_cfg<DT_F32, 1>(p, s);
 }
-hipError_t launch_conv_nhwc_dw_f32(const GemmParams& p, hipStream_t s) {
-    return ring_f32_tile_edge(p) == 128 ? launch_ring_nhwc_dw_cfg<DT_F32, 2>(p, s) : launch_ring_nhwc_dw_cfg<DT_F32, 1>(p, s);
+hipError_t launch_conv_nhwc_dw_f32(bool ta, const GemmParams& p, hipStream_t s) {
+    const bool big = ring_f32_tile_edge(p) == 128;
+    if (ta) return big ? launch_ring_nhwc_dw_cfg<DT_F32, 2, true>(p, s) : launch_ring_nhwc_dw_cfg<DT_F32, 1, true>(p, s);
+    return big ? launch_ring_nhwc_dw_cfg<DT_F32, 2>(p, s) : launch_ring_nhwc_dw_cfg<DT_F32, 1>(p, s);
 }
 }  // namespace ntg

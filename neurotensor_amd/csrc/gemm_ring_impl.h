@@ -182,7 +182,7 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
     constexpr int WT = G::WT;
     static_assert(!GATHER4 || (ES == 4 && !TA && RAGGED), "gathered operands: Float32, A stored [m][k], guarded edges");
     static_assert(!GATHER16 || ((ES == 4 || ES == 2) && !TA && RAGGED), "channels-last gather: 16/32-bit floats, A stored [m][k], guarded edges");
-    static_assert(!GATHERW || ((ES == 4 || ES == 2) && !TA && !TB && RAGGED), "channels-last weight gradient: 16/32-bit floats, A stored [m][k], guarded edges");
+    static_assert(!GATHERW || ((ES == 4 || ES == 2) && !TB && RAGGED), "channels-last weight gradient: 16/32-bit floats, guarded edges");
     constexpr int NA = WB, NB = GATHER4 ? 4 * WB : WB;   // DMA instructions per wavefront and K-step for the A / B tile
     // B instructions issued in the first / second half-step (the second also carries the A tile's).  Splitting a gathered
     // tile between the two was measured slower than issuing all of it in the first.
@@ -386,6 +386,8 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
     // WB 16-byte DMA instructions per wavefront; a lane's 16 bytes are channels c .. of ONE tap for the whole K loop
     // (tap reach and byte offset kept per lane), and its k-row moves on by BK output pixels per K-step: the pixel is
     // split into (row, column) with one multiply-shift division per instruction.  Padding and k >= K read zeros.
+    // Several images may share one K loop (p.conv.fold_L = output pixels per image, 0: one image): k then counts the
+    // output pixels of consecutive images, and one more division gives the image, p.conv.fold_stride elements apart.
     int krow4[WB], noff4[WB];
     uint32_t tap4[WB];
     int k4_k = 0;
@@ -412,12 +414,17 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
             const ConvGeom& g = p.conv;
             const char* img = reinterpret_cast<const char*>(B);
             const uint32_t l = (uint32_t)(k4_k + krow4[x]);
-            const uint32_t oh = fast_div(l, g.div_wo), ow = l - oh * (uint32_t)g.Wo;
+            uint32_t li = l, im = 0u;
+            if (g.fold_L) {                                        // (uniform)
+                im = fast_div(l, g.div_fold);
+                li = l - im * (uint32_t)g.fold_L;
+            }
+            const uint32_t oh = fast_div(li, g.div_wo), ow = li - oh * (uint32_t)g.Wo;
             const int ih0 = (int)oh * g.s_r - g.p_r, iw0 = (int)ow * g.s_c - g.p_c;
             const bool ok = (l < (uint32_t)p.K) & ((uint32_t)(ih0 + (int)(tap4[x] & 0xffffu)) < (uint32_t)g.H) &
                             ((uint32_t)(iw0 + (int)(tap4[x] >> 16)) < (uint32_t)g.W);
             const int off = (int)((oh * (uint32_t)g.s_r * (uint32_t)g.W + ow * (uint32_t)g.s_c) * (uint32_t)g.chan * (uint32_t)ES) + noff4[x];
-            const char* src = ok ? img + (int64_t)off : reinterpret_cast<const char*>(ring_zero_word);
+            const char* src = ok ? img + ((int64_t)im * g.fold_stride * ES + (int64_t)off) : reinterpret_cast<const char*>(ring_zero_word);
             asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
                          :: "s"(lds_tile + (uint32_t)(wave_u * WB + x) * 1024u), "v"(src) : "memory");
             if (x == WB - 1) k4_k += BK;
@@ -846,7 +853,7 @@ static hipError_t launch_ring_nhwc_cfg(const GemmParams& pin, hipStream_t s) {
 }
 
 // weight gradient of a convolution with op(B) gathered from a channels-last image (see CONV = 4)
-template <int DT, int WB>
+template <int DT, int WB, bool TA = false>
 static hipError_t launch_ring_nhwc_dw_cfg(const GemmParams& pin, hipStream_t s) {
     constexpr int TE = RingGeom<WB, (int)sizeof(typename Elem<DT>::T)>::BM;
     GemmParams p = pin;
@@ -855,7 +862,7 @@ static hipError_t launch_ring_nhwc_dw_cfg(const GemmParams& pin, hipStream_t s) 
     const int64_t blocks = (int64_t)p.tiles_m * p.tiles_n * p.batch;
     if (blocks <= 0) return hipSuccess;
     if (blocks > 0x7fffffffLL) return hipErrorInvalidValue;
-    hipLaunchKernelGGL((gemm_ring_kernel<DT, false, false, true, WB, 4>), dim3((unsigned)blocks), dim3(256), 0, s, p);
+    hipLaunchKernelGGL((gemm_ring_kernel<DT, TA, false, true, WB, 4>), dim3((unsigned)blocks), dim3(256), 0, s, p);
     return hipGetLastError();
 }
 

@@ -45,6 +45,11 @@ struct ConvGeom {
     int k_d, k_r, k_c, k_rc, k_drc, Wo, HoWo;
     int last;                // index of the last element of the image slice at p.B (loads are clamped to it)
     FastDiv div_kdrc, div_krc, div_kc, div_wo, div_howo;
+    // channels-last weight gradient with several images per K loop: output pixels per image (0: one image per item),
+    // its divider, and the elements from one image to the next
+    int fold_L;
+    FastDiv div_fold;
+    int64_t fold_stride;
 };
 
 struct GemmParams {
@@ -161,7 +166,7 @@ hipError_t launch_nchw_to_nhwc_padded(int64_t es, const void* in, void* out, int
 hipError_t launch_flip_weights_channels_last(int64_t es, const void* w, void* wt, int64_t groups, int64_t og, int64_t ogp, int64_t cg, int64_t taps, hipStream_t s);
 // channels-last convolution (image [B][pixel][C], weights [O][(r, q, c)]); F16 / BF16 / F32, two spatial axes
 hipError_t launch_conv_nhwc(int dtype, const GemmParams& p, hipStream_t s);
-hipError_t launch_conv_nhwc_dw(int dtype, const GemmParams& p, hipStream_t s);
+hipError_t launch_conv_nhwc_dw(int dtype, bool ta, const GemmParams& p, hipStream_t s);   // ta: A (the output gradient) stored [k][m]
 hipError_t launch_reduce_batch_taps_last(int dtype, const void* part, void* out, int64_t batch, int64_t rows, int64_t cg, int64_t taps,
                                          int accumulate, hipStream_t s);
 hipError_t launch_flip_weights(int64_t elem_size, const void* w, void* wt, int64_t groups, int64_t og, int64_t cg, int64_t taps, hipStream_t s);

@@ -36,14 +36,14 @@ hipError_t launch_conv_nhwc(int dtype, const GemmParams& p, hipStream_t s) {
     }
 }
 
-hipError_t launch_conv_nhwc_dw_f32(const GemmParams& p, hipStream_t s);
-hipError_t launch_conv_nhwc_dw_f16(const GemmParams& p, hipStream_t s);
-hipError_t launch_conv_nhwc_dw_bf16(const GemmParams& p, hipStream_t s);
-hipError_t launch_conv_nhwc_dw(int dtype, const GemmParams& p, hipStream_t s) {
+hipError_t launch_conv_nhwc_dw_f32(bool ta, const GemmParams& p, hipStream_t s);
+hipError_t launch_conv_nhwc_dw_f16(bool ta, const GemmParams& p, hipStream_t s);
+hipError_t launch_conv_nhwc_dw_bf16(bool ta, const GemmParams& p, hipStream_t s);
+hipError_t launch_conv_nhwc_dw(int dtype, bool ta, const GemmParams& p, hipStream_t s) {
     switch (dtype) {
-    case DT_F32: return launch_conv_nhwc_dw_f32(p, s);
-    case DT_F16: return launch_conv_nhwc_dw_f16(p, s);
-    case DT_BF16: return launch_conv_nhwc_dw_bf16(p, s);
+    case DT_F32: return launch_conv_nhwc_dw_f32(ta, p, s);
+    case DT_F16: return launch_conv_nhwc_dw_f16(ta, p, s);
+    case DT_BF16: return launch_conv_nhwc_dw_bf16(ta, p, s);
     default: return hipErrorInvalidValue;
     }
 }
@@ -751,44 +751,85 @@ static int conv_dimage_nhwc(int dtype, const void* kernel, const void* grad_out,
 // P_{b,g} [og][(taps, c)] = dY_{b,g} [og, L] . col^T gathered 16 bytes of channels at a time; the per-image results are
 // summed in batch order into the kernel's [O][c][taps] layout.  Needs rows of dY and the channels of a group to be
 // 16-byte multiples.
+// Large output planes with 16-byte rows: dY is read where it lies, one image per K loop (measured faster from about 512
+// pixels: no copy, one LDS read per block instead of the transposing ones).  Otherwise, when the out channels of a group
+// are a 16-byte multiple, dY goes through its own channels-last copy: as a [pixel][out channel] matrix the images follow
+// each other, so several of them can share one K loop.
+static bool conv_dkernel_nhwc_copies_dy(int dtype, int64_t out_channels, int64_t groups, const Geo3& g) {
+    const int64_t es = ntg::elem_size(dtype);
+    if ((g.L() * es) % 16 == 0 && g.L() >= 512) return false;
+    return ((out_channels / groups) * es) % 16 == 0;
+}
+// Images per K loop: the largest divisor of the batch that still leaves two workgroups per CU (128 x 128 tiles), so that
+// fewer per-image results are written and summed (64 images of a 3 x 3 x 256 x 256 layer: 16 partial sums instead of 64;
+// 7 x 7 maps: K = 784 instead of 49).
+static int64_t conv_dkernel_fold(int64_t batch, int64_t og, int64_t n, int64_t groups, int64_t L) {
+    const int64_t tiles = ((og + 127) / 128) * ((n + 127) / 128) * groups;
+    int64_t best = 1;
+    for (int64_t f = 2; f <= batch; ++f) {
+        if (batch % f) continue;
+        if ((batch / f) * tiles < 512 || f * L >= (1LL << 30)) break;
+        best = f;
+    }
+    return best;
+}
 static bool conv_dkernel_nhwc_ok(int dtype, int64_t channels, int64_t out_channels, int64_t groups, const Geo3& g) {
     if (dtype != ntg::DT_F32 && dtype != ntg::DT_F16 && dtype != ntg::DT_BF16) return false;
     if (g.nd != 2 || !conv_implicit_g(dtype, channels, g)) return false;
     const int64_t es = ntg::elem_size(dtype), cg = channels / groups;
     if (g.k[1] * g.d[1] >= 32768 || g.k[2] * g.d[2] >= 32768) return false;      // tap reach packed in 16 bits
-    return (cg * es) % 16 == 0 && (g.L() * es) % 16 == 0 && out_channels > 0 && cg * g.taps() < 0x7fffffffLL &&
+    // rows of dY that are 16-byte multiples are read where they lie; otherwise dY is copied channels-last too and read
+    // as a [pixel][out channel] operand, which needs the out channels of a group to be a 16-byte multiple
+    const bool a_ok = (g.L() * es) % 16 == 0 || conv_dkernel_nhwc_copies_dy(dtype, out_channels, groups, g);
+    return (cg * es) % 16 == 0 && a_ok && out_channels > 0 && cg * g.taps() < 0x7fffffffLL &&
            conv_nhwc_offsets_fit(channels, es, g);
 }
 static int64_t conv_dkernel_nhwc_workspace(int dtype, int64_t batch, int64_t channels, int64_t out_channels, int64_t groups, const Geo3& g) {
     const int64_t es = ntg::elem_size(dtype);
-    return (int64_t)align_up((size_t)(batch * channels * g.vol() * es), 256) + batch * out_channels * (channels / groups) * g.taps() * es;
+    const int64_t gy = conv_dkernel_nhwc_copies_dy(dtype, out_channels, groups, g) ? (int64_t)align_up((size_t)(batch * out_channels * g.L() * es), 256) : 0;
+    return (int64_t)align_up((size_t)(batch * channels * g.vol() * es), 256) + gy + batch * out_channels * (channels / groups) * g.taps() * es;
 }
 static int conv_dkernel_nhwc(int dtype, const void* image, const void* grad_out, void* d_kernel, void* ws, int64_t batch,
                              int64_t channels, int64_t out_channels, const Geo3& g, int64_t groups, int accumulate, hipStream_t hs) {
     const int64_t es = ntg::elem_size(dtype), cg = channels / groups, og = out_channels / groups;
     const int64_t L = g.L(), taps = g.taps(), vol = g.vol(), N = taps * cg;
+    const bool copy_dy = conv_dkernel_nhwc_copies_dy(dtype, out_channels, groups, g);      // dY read as [pixel][out channel] from its own copy
+    const int64_t fold = copy_dy ? conv_dkernel_fold(batch, og, N, groups, L) : 1, items = batch / fold;
     char* ws_img = static_cast<char*>(ws);
-    char* ws_part = ws_img + align_up((size_t)(batch * channels * vol * es), 256);
+    char* ws_gy = ws_img + align_up((size_t)(batch * channels * vol * es), 256);
+    char* ws_part = ws_gy + (copy_dy ? align_up((size_t)(batch * out_channels * L * es), 256) : 0);
     hipError_t e = ntg::launch_nchw_to_nhwc(es, image, ws_img, batch, channels, vol, hs);
+    if (e == hipSuccess && copy_dy) e = ntg::launch_nchw_to_nhwc(es, grad_out, ws_gy, batch, out_channels, L, hs);
     if (e != hipSuccess) return hip_fail(e, "channels-last copy launch");
     for (int64_t gi = 0; gi < groups; ++gi) {
         ntg::GemmParams p;
         std::memset(&p, 0, sizeof p);
-        p.M = (int)og; p.K = (int)L; p.N = (int)N; p.batch = (int)batch;
-        p.A = static_cast<const char*>(grad_out) + gi * og * L * es;
+        p.M = (int)og; p.K = (int)(fold * L); p.N = (int)N; p.batch = (int)items;
+        if (copy_dy) {
+            p.A = ws_gy + gi * og * es;
+            p.lda = out_channels;
+        } else {
+            p.A = static_cast<const char*>(grad_out) + gi * og * L * es;
+            p.lda = L;
+        }
         p.B = ws_img + gi * cg * es;
         p.C = ws_part + gi * og * N * es;
-        p.lda = L; p.ldb = channels; p.ldc = N;
-        p.sA = out_channels * L; p.sB = channels * vol; p.sC = out_channels * N;
+        p.ldb = channels; p.ldc = N;
+        p.sA = fold * out_channels * L; p.sB = fold * channels * vol; p.sC = out_channels * N;
         p.cmode = ntg::C_OVERWRITE;
         p.vecA_ok = 1; p.vecB_ok = 1;
         fill_conv_geom(p.conv, cg, g);
         p.conv.chan = (int)channels;               // elements from one pixel to the next
-        e = ntg::launch_conv_nhwc_dw(dtype, p, hs);
+        if (fold > 1) {
+            p.conv.fold_L = (int)L;
+            p.conv.div_fold = ntg::make_fastdiv((uint32_t)L);
+            p.conv.fold_stride = channels * vol;
+        }
+        e = ntg::launch_conv_nhwc_dw(dtype, copy_dy, p, hs);
         if (e != hipSuccess) return hip_fail(e, "channels-last conv_dkernel launch");
     }
     // (groups are consecutive row blocks of both layouts, so one pass covers them all)
-    e = ntg::launch_reduce_batch_taps_last(dtype, ws_part, d_kernel, batch, out_channels, cg, taps, accumulate, hs);
+    e = ntg::launch_reduce_batch_taps_last(dtype, ws_part, d_kernel, items, out_channels, cg, taps, accumulate, hs);
     if (e != hipSuccess) return hip_fail(e, "weight gradient reduction launch");
     return NTG_OK;
 }

@@ -242,6 +242,9 @@ BACKWARD_GEOMS = [
     (3, 48, 15, 13, 64, 3, 3, 1, 1, 1, 2),                 # channels-last dX with image planes of odd size (195), two groups
     (2, 16, 9, 11, 96, 3, 2, 1, (2, 0), (2, 1), 1),
     (2, 16, 12, 16, 24, 3, 3, (2, 1), (1, 2), (1, 2), 2),  # channels-last dW with stride, dilation and groups (L = 96)
+    (64, 256, 6, 6, 128, 3, 3, 1, 1, 1, 1),                # dW with two images per K loop (36 pixels each: the seam falls inside a K-step)
+    (8, 512, 5, 7, 512, 3, 3, 1, 1, 1, 1),                 # 35 pixels per image, two images per K loop, four tile rows
+    (12, 128, 7, 7, 64, 3, 3, 1, 1, 1, 4),                 # groups; 49 pixels per image (rows of dY not 16-byte multiples)
 ]
 
 
