@@ -166,6 +166,19 @@ hipError_t launch_nchw_to_nhwc_padded(int64_t es, const void* in, void* out, int
 hipError_t launch_flip_weights_channels_last(int64_t es, const void* w, void* wt, int64_t groups, int64_t og, int64_t ogp, int64_t cg, int64_t taps, hipStream_t s);
 // channels-last convolution (image [B][pixel][C], weights [O][(r, q, c)]); F16 / BF16 / F32, two spatial axes
 hipError_t launch_conv_nhwc(int dtype, const GemmParams& p, hipStream_t s);
+// Image gradient of a strided convolution as one stride-1 convolution per phase of the image (see conv_dimage_phases):
+// where the phase planes lie in the temporary buffer (element offsets; -1: the phase has no taps) and how image
+// coordinates map to them.  Strides up to 4.
+struct PhaseLayout {
+    int H, W, p_r, p_c, s_r, s_c;
+    uint32_t total;              // batch * channels * H * W
+    int a0r[4], a0c[4], hp[4], wp[4];
+    int64_t off[16];
+    FastDiv div_w, div_h, div_sr, div_sc;
+};
+hipError_t launch_phase_weights(int64_t es, const void* w, void* wt, int64_t groups, int64_t og, int64_t ogp, int64_t cg, int64_t k_r, int64_t k_c,
+                                int64_t er, int64_t ec, int64_t s_r, int64_t s_c, int64_t Mr, int64_t Mc, hipStream_t s);
+hipError_t launch_phase_interleave(int dtype, const void* tmp, void* im, const PhaseLayout& q, int accumulate, hipStream_t s);
 hipError_t launch_conv_nhwc_dw(int dtype, bool ta, const GemmParams& p, hipStream_t s);   // ta: A (the output gradient) stored [k][m]
 hipError_t launch_reduce_batch_taps_last(int dtype, const void* part, void* out, int64_t batch, int64_t rows, int64_t cg, int64_t taps,
                                          int accumulate, hipStream_t s);

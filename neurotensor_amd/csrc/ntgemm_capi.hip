@@ -747,6 +747,111 @@ static int conv_dimage_nhwc(int dtype, const void* kernel, const void* grad_out,
     return NTG_OK;
 }
 
+// dX of a convolution with strides > 1 (dilation 1), without the col matrix: the image rows y with (y + p) mod s = e
+// form one phase; they receive only the taps i = e + s m (m = 0 .. M_e - 1), and, with a = (y + p) / s,
+//   dX[y] = sum_m dY[a - m] W[e + s m],
+// a stride-1 convolution of dY with the M_e reversed taps.  So every phase (er, ec) is one channels-last convolution
+// (the forward kernel) of the shared channels-last copy of dY with its own small kernel, written to a plane of the
+// phase's rows and columns in the workspace; a last pass interleaves the planes into dX.  Exactly the products of the
+// reference's GEMM + col2im, none wasted on the zeros a dilated gradient would hold.
+struct PhasePlan {
+    bool ok;
+    int64_t Mr[4], Mc[4], a0r[4], a0c[4], hp[4], wp[4];
+    int64_t ogp, gy_bytes, w_bytes, tmp_bytes;
+};
+static Geo3 phase_geo(const Geo3& g, const PhasePlan& pp, int er, int ec) {
+    // image = the dY plane, kernel Mr x Mc, stride 1, padding (M - 1) - a0 (first row of the plane is a0), outputs hp x wp
+    return Geo3{2, {1, g.o[1], g.o[2]}, {1, pp.Mr[er], pp.Mc[ec]}, {1, 1, 1}, {0, pp.Mr[er] - 1 - pp.a0r[er], pp.Mc[ec] - 1 - pp.a0c[ec]},
+                {1, 1, 1}, {1, pp.hp[er], pp.wp[ec]}};
+}
+static PhasePlan plan_dimage_phases(int dtype, int64_t batch, int64_t channels, int64_t out_channels, int64_t groups, const Geo3& g) {
+    PhasePlan pp;
+    std::memset(&pp, 0, sizeof pp);
+    if (dtype != ntg::DT_F32 && dtype != ntg::DT_F16 && dtype != ntg::DT_BF16) return pp;
+    if (g.nd != 2 || g.d[1] != 1 || g.d[2] != 1 || (g.s[1] == 1 && g.s[2] == 1) || g.s[1] > 4 || g.s[2] > 4 || g.p[1] < 0 || g.p[2] < 0) return pp;
+    if (g.k[1] > 8 * g.s[1] || g.k[2] > 8 * g.s[2]) return pp;
+    const int64_t es = ntg::elem_size(dtype), og = out_channels / groups;
+    pp.ogp = nhwc_padded_channels(es, og);
+    if (pp.ogp == 0 || batch * channels * g.vol() >= 0x7fffffffLL) return pp;
+    for (int ax = 1; ax <= 2; ++ax) {
+        int64_t* M = ax == 1 ? pp.Mr : pp.Mc;
+        int64_t* a0 = ax == 1 ? pp.a0r : pp.a0c;
+        int64_t* n = ax == 1 ? pp.hp : pp.wp;
+        for (int64_t e = 0; e < g.s[ax]; ++e) {
+            M[e] = e < g.k[ax] ? (g.k[ax] - e + g.s[ax] - 1) / g.s[ax] : 0;
+            // image positions y = s a + e - p in [0, size): a from a0
+            a0[e] = g.p[ax] > e ? (g.p[ax] - e + g.s[ax] - 1) / g.s[ax] : 0;
+            const int64_t last = g.sz[ax] - 1 + g.p[ax] - e;                      // largest s a
+            n[e] = last >= 0 && last / g.s[ax] >= a0[e] ? last / g.s[ax] - a0[e] + 1 : 0;
+        }
+    }
+    int64_t wmax = 0, tmp = 0;
+    for (int64_t er = 0; er < g.s[1]; ++er)
+        for (int64_t ec = 0; ec < g.s[2]; ++ec) {
+            if (pp.Mr[er] == 0 || pp.Mc[ec] == 0 || pp.hp[er] == 0 || pp.wp[ec] == 0) continue;
+            if (!conv_nhwc_ok(dtype, out_channels, channels, groups, phase_geo(g, pp, (int)er, (int)ec))) return pp;
+            wmax += (int64_t)align_up((size_t)(channels * pp.Mr[er] * pp.Mc[ec] * pp.ogp * es), 256);
+            tmp += (int64_t)align_up((size_t)(batch * channels * pp.hp[er] * pp.wp[ec] * es), 256);
+        }
+    pp.gy_bytes = (int64_t)align_up((size_t)(batch * groups * pp.ogp * g.L() * es), 256);
+    pp.w_bytes = wmax;
+    pp.tmp_bytes = tmp;
+    pp.ok = true;
+    return pp;
+}
+static int conv_dimage_phases(int dtype, const PhasePlan& pp, const void* kernel, const void* grad_out, void* d_image, void* ws, int64_t batch,
+                              int64_t channels, int64_t out_channels, const Geo3& g, int64_t groups, int accumulate, hipStream_t hs) {
+    const int64_t es = ntg::elem_size(dtype), cg = channels / groups, og = out_channels / groups;
+    const int64_t ogp = pp.ogp, ochp = groups * ogp, L = g.L();
+    char* ws_gy = static_cast<char*>(ws);
+    char* ws_w = ws_gy + pp.gy_bytes;
+    char* ws_tmp = ws_w + pp.w_bytes;
+    hipError_t e = ogp == og ? ntg::launch_nchw_to_nhwc(es, grad_out, ws_gy, batch, out_channels, L, hs)
+                             : ntg::launch_nchw_to_nhwc_padded(es, grad_out, ws_gy, batch, groups, og, ogp, L, hs);
+    if (e != hipSuccess) return hip_fail(e, "channels-last copy launch");
+    ntg::PhaseLayout lay;
+    std::memset(&lay, 0, sizeof lay);
+    lay.H = (int)g.sz[1]; lay.W = (int)g.sz[2]; lay.p_r = (int)g.p[1]; lay.p_c = (int)g.p[2]; lay.s_r = (int)g.s[1]; lay.s_c = (int)g.s[2];
+    lay.total = (uint32_t)(batch * channels * g.vol());
+    lay.div_w = ntg::make_fastdiv((uint32_t)lay.W); lay.div_h = ntg::make_fastdiv((uint32_t)lay.H);
+    lay.div_sr = ntg::make_fastdiv((uint32_t)lay.s_r); lay.div_sc = ntg::make_fastdiv((uint32_t)lay.s_c);
+    for (int i = 0; i < 4; ++i) { lay.a0r[i] = (int)pp.a0r[i]; lay.a0c[i] = (int)pp.a0c[i]; lay.hp[i] = (int)pp.hp[i]; lay.wp[i] = (int)pp.wp[i]; }
+    for (int i = 0; i < 16; ++i) lay.off[i] = -1;
+    int64_t w_off = 0, t_off = 0;
+    for (int64_t er = 0; er < g.s[1]; ++er)
+        for (int64_t ec = 0; ec < g.s[2]; ++ec) {
+            if (pp.Mr[er] == 0 || pp.Mc[ec] == 0 || pp.hp[er] == 0 || pp.wp[ec] == 0) continue;
+            const Geo3 t = phase_geo(g, pp, (int)er, (int)ec);
+            const int64_t taps = pp.Mr[er] * pp.Mc[ec], K = taps * ogp, plane = pp.hp[er] * pp.wp[ec];
+            char* wph = ws_w + w_off;
+            char* tph = ws_tmp + t_off;
+            e = ntg::launch_phase_weights(es, kernel, wph, groups, og, ogp, cg, g.k[1], g.k[2], er, ec, g.s[1], g.s[2], pp.Mr[er], pp.Mc[ec], hs);
+            if (e != hipSuccess) return hip_fail(e, "phase weight launch");
+            for (int64_t gi = 0; gi < groups; ++gi) {
+                ntg::GemmParams p;
+                std::memset(&p, 0, sizeof p);
+                p.M = (int)cg; p.K = (int)K; p.N = (int)plane; p.batch = (int)batch;
+                p.A = wph + gi * cg * K * es;
+                p.B = ws_gy + gi * ogp * es;
+                p.C = tph + gi * cg * plane * es;
+                p.lda = K; p.ldb = ochp; p.ldc = plane;
+                p.sA = 0; p.sB = ochp * L; p.sC = channels * plane;
+                p.cmode = ntg::C_OVERWRITE;
+                p.vecA_ok = 1; p.vecB_ok = 1;
+                fill_conv_geom(p.conv, ogp, t);
+                p.conv.chan = (int)ochp;
+                e = ntg::launch_conv_nhwc(dtype, p, hs);
+                if (e != hipSuccess) return hip_fail(e, "phase convolution launch");
+            }
+            lay.off[er * g.s[2] + ec] = t_off / es;
+            w_off += (int64_t)align_up((size_t)(channels * taps * ogp * es), 256);
+            t_off += (int64_t)align_up((size_t)(batch * channels * plane * es), 256);
+        }
+    e = ntg::launch_phase_interleave(dtype, ws_tmp, d_image, lay, accumulate, hs);
+    if (e != hipSuccess) return hip_fail(e, "phase interleave launch");
+    return NTG_OK;
+}
+
 // dW through the channels-last kernel: the image is copied to [B][pixel][C]; per image and group
 // P_{b,g} [og][(taps, c)] = dY_{b,g} [og, L] . col^T gathered 16 bytes of channels at a time; the per-image results are
 // summed in batch order into the kernel's [O][c][taps] layout.  Needs rows of dY and the channels of a group to be
@@ -835,7 +940,7 @@ static int conv_dkernel_nhwc(int dtype, const void* image, const void* grad_out,
 }
 
 // Which backward gradients run as implicit GEMMs, and the workspace the call needs.
-struct ConvBackwardPlan { bool gather_dw, gather_dx, nhwc_dx, nhwc_dw; int64_t need, need_nhwc_dx, need_nhwc_dw; };
+struct ConvBackwardPlan { bool gather_dw, gather_dx, nhwc_dx, nhwc_dw, phase_dx; int64_t need, need_nhwc_dx, need_nhwc_dw, need_phase_dx; PhasePlan phases; };
 static ConvBackwardPlan plan_conv_backward_g(int dtype, bool want_dx, bool want_dw, int64_t batch, int64_t channels, int64_t out_channels,
                                              const Geo3& g, int64_t groups) {
     const int64_t es = ntg::elem_size(dtype);
@@ -853,6 +958,12 @@ static ConvBackwardPlan plan_conv_backward_g(int dtype, bool want_dx, bool want_
     pl.need_nhwc_dx = pl.nhwc_dx ? conv_dimage_nhwc_workspace(dtype, batch, channels, out_channels, groups, g) : 0;
     pl.nhwc_dw = pl.gather_dw && conv_dkernel_nhwc_ok(dtype, channels, out_channels, groups, g);
     pl.need_nhwc_dw = pl.nhwc_dw ? conv_dkernel_nhwc_workspace(dtype, batch, channels, out_channels, groups, g) : 0;
+    // strides > 1: dX phase by phase instead of GEMM + col2im, again when the workspace allows
+    std::memset(&pl.phases, 0, sizeof pl.phases);
+    if (want_dx && !pl.gather_dx && conv_implicit_g(dtype, out_channels, geo_dimage(g)))
+        pl.phases = plan_dimage_phases(dtype, batch, channels, out_channels, groups, g);
+    pl.phase_dx = pl.phases.ok;
+    pl.need_phase_dx = pl.phase_dx ? pl.phases.gy_bytes + pl.phases.w_bytes + pl.phases.tmp_bytes : 0;
     return pl;
 }
 
@@ -1036,7 +1147,7 @@ int64_t ntg_conv2d_backward_workspace_bytes(int dtype, int64_t batch, int64_t ch
     // the larger of what the call needs at least and what lets dX take its channels-last form (copy of dY + flipped weights)
     const ConvBackwardPlan pl = plan_conv_backward(dtype, true, true, batch, channels, height, width, out_channels, k_r, k_c, s_r, s_c, p_r, p_c,
                                                    d_r, d_c, groups, Ho, Wo);
-    return std::max(pl.need, std::max(pl.need_nhwc_dx, pl.need_nhwc_dw));
+    return std::max(std::max(pl.need, pl.need_phase_dx), std::max(pl.need_nhwc_dx, pl.need_nhwc_dw));
 }
 
 int ntg_conv2d_backward_dev(int dtype, const void* image, const void* kernel, const void* grad_out,
@@ -1086,6 +1197,11 @@ int ntg_conv2d_backward_dev(int dtype, const void* image, const void* kernel, co
     }
     if (gather_dw) d_kernel = nullptr;    // done
     if (gather_dx) d_image = nullptr;
+    if (d_image && plan.phase_dx && workspace_bytes >= plan.need_phase_dx && (reinterpret_cast<uintptr_t>(ws) & 15) == 0) {
+        rc = conv_dimage_phases(dtype, plan.phases, kernel, grad_out, d_image, ws, batch, channels, out_channels, geo, groups, accumulate, hs);
+        if (rc) return rc;
+        d_image = nullptr;
+    }
     if (d_kernel) {
         // col = im2col(image); per group g:  dW_g [og, add] (+)= sum_b dY_{b,g} [og, L] . col_{b,g}^T  (col_{b,g} stored [add, L])
         rc = ntg_unfold2d_dev(dtype, image, ws, batch, channels, height, width, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c, stream);
@@ -1156,7 +1272,7 @@ int64_t ntg_conv_transpose2d_workspace_bytes(int dtype, int64_t batch, int64_t i
         unfold_out(oh, ow, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c, Ho, Wo)) return -1;
     const ConvBackwardPlan pl = plan_conv_backward(dtype, true, false, batch, out_channels, oh, ow, in_channels, k_r, k_c, s_r, s_c, p_r, p_c,
                                                    d_r, d_c, groups, Ho, Wo);
-    return std::max(pl.need, pl.need_nhwc_dx);      // (the larger amount lets the stride-1 case run channels-last)
+    return std::max(pl.need, std::max(pl.need_nhwc_dx, pl.need_phase_dx));      // (the larger amount lets it run channels-last)
 }
 
 int ntg_conv_transpose2d_dev(int dtype, const void* input, const void* kernel, void* out, void* workspace, int64_t workspace_bytes,

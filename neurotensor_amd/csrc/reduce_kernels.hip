@@ -289,6 +289,72 @@ hipError_t launch_flip_weights_channels_last(int64_t es, const void* w, void* wt
     return hipGetLastError();
 }
 
+// Weights of one phase of a strided convolution's image gradient: the taps i = er + s_r (Mr-1-mr), j = ec + s_c (Mc-1-mc)
+// of w [g*og + oc][c][k_r][k_c], as wt[g][c][(mr, mc)][oc] with the out channels padded with zeros from og to ogp.
+struct PhaseWeights { int64_t groups, og, ogp, cg, k_r, k_c, er, ec, s_r, s_c, Mr, Mc; };
+template <class T>
+__global__ void __launch_bounds__(256) phase_weights_kernel(const T* __restrict__ w, T* __restrict__ wt, const PhaseWeights q) {
+    const int64_t total = q.groups * q.cg * q.Mr * q.Mc * q.ogp;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += stride) {
+        const int64_t oc = idx % q.ogp;
+        int64_t r = idx / q.ogp;
+        const int64_t mc = r % q.Mc;
+        r /= q.Mc;
+        const int64_t mr = r % q.Mr;
+        r /= q.Mr;
+        const int64_t c = r % q.cg, g = r / q.cg;
+        const int64_t i = q.er + q.s_r * (q.Mr - 1 - mr), j = q.ec + q.s_c * (q.Mc - 1 - mc);
+        wt[idx] = oc < q.og ? w[(((g * q.og + oc) * q.cg + c) * q.k_r + i) * q.k_c + j] : (T)0;
+    }
+}
+
+hipError_t launch_phase_weights(int64_t es, const void* w, void* wt, int64_t groups, int64_t og, int64_t ogp, int64_t cg, int64_t k_r, int64_t k_c,
+                                int64_t er, int64_t ec, int64_t s_r, int64_t s_c, int64_t Mr, int64_t Mc, hipStream_t s) {
+    const PhaseWeights q{groups, og, ogp, cg, k_r, k_c, er, ec, s_r, s_c, Mr, Mc};
+    const int64_t total = groups * cg * Mr * Mc * ogp;
+    if (total == 0) return hipSuccess;
+    const dim3 g(grid_for(total)), t(256);
+    switch (es) {
+    case 2: hipLaunchKernelGGL(phase_weights_kernel<uint16_t>, g, t, 0, s, (const uint16_t*)w, (uint16_t*)wt, q); break;
+    case 4: hipLaunchKernelGGL(phase_weights_kernel<uint32_t>, g, t, 0, s, (const uint32_t*)w, (uint32_t*)wt, q); break;
+    default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+
+// im[b][c][y][x] (+)= the element of the phase plane that holds it: phase (er, ec) = ((y + p_r) % s_r, (x + p_c) % s_c)
+// stores the image rows y = s_r (a0 + a) + er - p_r as its rows a (columns likewise); phases without taps contribute zero.
+template <class T, class Acc>
+__global__ void __launch_bounds__(256) phase_interleave_kernel(const T* __restrict__ tmp, T* __restrict__ im, const PhaseLayout q, const int accumulate) {
+    const uint32_t idx = blockIdx.x * 256u + threadIdx.x;
+    if (idx >= q.total) return;
+    const uint32_t t = fast_div(idx, q.div_w), x = idx - t * (uint32_t)q.W;
+    const uint32_t bc = fast_div(t, q.div_h), y = t - bc * (uint32_t)q.H;
+    const uint32_t Y = y + (uint32_t)q.p_r, X = x + (uint32_t)q.p_c;
+    const uint32_t ar = fast_div(Y, q.div_sr), er = Y - ar * (uint32_t)q.s_r;
+    const uint32_t ac = fast_div(X, q.div_sc), ec = X - ac * (uint32_t)q.s_c;
+    Acc v = accumulate ? (Acc)im[idx] : (Acc)0;
+    const int ph = (int)(er * (uint32_t)q.s_c + ec);
+    if (q.off[ph] >= 0) {
+        const int a = (int)ar - q.a0r[er], b = (int)ac - q.a0c[ec];      // inside the plane by construction
+        v += (Acc)tmp[q.off[ph] + ((int64_t)bc * q.hp[er] + a) * q.wp[ec] + b];
+    }
+    im[idx] = (T)v;
+}
+
+hipError_t launch_phase_interleave(int dtype, const void* tmp, void* im, const PhaseLayout& q, int accumulate, hipStream_t s) {
+    if (q.total == 0) return hipSuccess;
+    const dim3 g((q.total + 255u) / 256u), t(256);
+    switch (dtype) {
+    case DT_F32: hipLaunchKernelGGL((phase_interleave_kernel<float, float>), g, t, 0, s, (const float*)tmp, (float*)im, q, accumulate); break;
+    case DT_F16: hipLaunchKernelGGL((phase_interleave_kernel<_Float16, float>), g, t, 0, s, (const _Float16*)tmp, (_Float16*)im, q, accumulate); break;
+    case DT_BF16: hipLaunchKernelGGL((phase_interleave_kernel<__bf16, float>), g, t, 0, s, (const __bf16*)tmp, (__bf16*)im, q, accumulate); break;
+    default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+
 // wp[o][t][c] = w[o][c][t]: convolution weights with the channel index fastest (the k order of the channels-last gather),
 // the channels of one tap padded with zeros from cg to cgp
 template <class T>

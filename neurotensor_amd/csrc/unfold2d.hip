@@ -111,6 +111,48 @@ __global__ void __launch_bounds__(256) col2im_kernel(const T* __restrict__ col, 
     }
 }
 
+// The same gather in 32-bit arithmetic (every size and the number of image elements below 2^31): the element index is
+// split with multiply-shift divisions, a tap row or column is skipped as soon as it falls before the image (the
+// position only decreases with the tap index), and "divisible by the stride" is one more multiply-shift.  Taps are
+// still visited in ascending (i, j), so the sum has the same order.
+struct Col2imFastParams {
+    int channels, height, width, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c, Ho, Wo;
+    uint32_t total;
+    int64_t L, ccol;
+    FastDiv div_w, div_h, div_c, div_sr, div_sc;
+};
+
+template <class T, class Acc>
+__global__ void __launch_bounds__(256) col2im_fast_kernel(const T* __restrict__ col, T* __restrict__ im, const Col2imFastParams u, const int accumulate) {
+    const uint32_t idx = blockIdx.x * 256u + threadIdx.x;
+    if (idx >= u.total) return;
+    uint32_t t = fast_div(idx, u.div_w);
+    const int x = (int)(idx - t * (uint32_t)u.width);
+    uint32_t t2 = fast_div(t, u.div_h);
+    const int y = (int)(t - t2 * (uint32_t)u.height);
+    const uint32_t b = fast_div(t2, u.div_c), c = t2 - b * (uint32_t)u.channels;
+    Acc acc = accumulate ? (Acc)im[idx] : (Acc)0;
+    const T* colc = col + ((int64_t)b * u.ccol + (int64_t)c * u.k_r * u.k_c) * u.L;      // row (c, 0, 0) of this image's col
+    int hn = y + u.p_r;
+    for (int i = 0; i < u.k_r && hn >= 0; ++i, hn -= u.d_r) {
+        const uint32_t h = fast_div((uint32_t)hn, u.div_sr);
+        if ((int)h * u.s_r != hn || (int)h >= u.Ho) continue;
+        const T* rowp = colc + (int64_t)i * u.k_c * u.L + (int64_t)h * u.Wo;
+        int wn = x + u.p_c;
+        for (int j = 0; j < u.k_c && wn >= 0; ++j, wn -= u.d_c) {
+            const uint32_t w = fast_div((uint32_t)wn, u.div_sc);
+            if ((int)w * u.s_c != wn || (int)w >= u.Wo) continue;
+            acc += (Acc)rowp[(int64_t)j * u.L + w];
+        }
+    }
+    im[idx] = (T)acc;
+}
+
+template <class T, class Acc>
+static void launch_col2im_fast(const void* col, void* im, const Col2imFastParams& q, int accumulate, hipStream_t s) {
+    hipLaunchKernelGGL((col2im_fast_kernel<T, Acc>), dim3((q.total + 255u) / 256u), dim3(256), 0, s, (const T*)col, (T*)im, q, accumulate);
+}
+
 // ---- the same two transforms over up to NTG_MAX_SPATIAL axes (unfold3d / unfoldnd and their adjoints:
 // nt/functional/cpu/unfold3d.cpp:9-80, unfoldnd.cpp, unfold3d_backward.cpp, unfoldnd_backward.cpp).
 // Row index of col: ((c*k0 + t0)*k1 + t1)*... ; column index: (o0*out1 + o1)*... ; last axis fastest.
@@ -226,6 +268,28 @@ hipError_t launch_col2im(int dtype, const void* col, void* im,
     if (e != hipSuccess) return e;
     const int64_t total = batch * channels * height * width;
     if (total == 0) return hipSuccess;
+    const int64_t lim = 1LL << 30;
+    if (total < 0x7fffffffLL && u.k_r * u.d_r < lim && u.k_c * u.d_c < lim && u.p_r < lim && u.p_c < lim && u.p_r > -lim && u.p_c > -lim &&
+        u.Ho * u.s_r < lim && u.Wo * u.s_c < lim && height < lim && width < lim && u.k_r < lim && u.k_c < lim && u.p_r >= 0 && u.p_c >= 0) {
+        Col2imFastParams q;
+        q.channels = (int)channels; q.height = (int)height; q.width = (int)width; q.k_r = (int)u.k_r; q.k_c = (int)u.k_c;
+        q.s_r = (int)u.s_r; q.s_c = (int)u.s_c; q.p_r = (int)u.p_r; q.p_c = (int)u.p_c; q.d_r = (int)u.d_r; q.d_c = (int)u.d_c;
+        q.Ho = (int)u.Ho; q.Wo = (int)u.Wo; q.total = (uint32_t)total; q.L = u.Ho * u.Wo; q.ccol = u.ccol;
+        q.div_w = make_fastdiv((uint32_t)width); q.div_h = make_fastdiv((uint32_t)height); q.div_c = make_fastdiv((uint32_t)channels);
+        q.div_sr = make_fastdiv((uint32_t)u.s_r); q.div_sc = make_fastdiv((uint32_t)u.s_c);
+        switch (dtype) {
+        case DT_F32: launch_col2im_fast<float, float>(col, im, q, accumulate, s); break;
+        case DT_F64: launch_col2im_fast<double, double>(col, im, q, accumulate, s); break;
+        case DT_F16: launch_col2im_fast<_Float16, float>(col, im, q, accumulate, s); break;
+        case DT_BF16: launch_col2im_fast<__bf16, float>(col, im, q, accumulate, s); break;
+        case DT_I8: case DT_U8: launch_col2im_fast<uint8_t, uint8_t>(col, im, q, accumulate, s); break;
+        case DT_I16: case DT_U16: launch_col2im_fast<uint16_t, uint16_t>(col, im, q, accumulate, s); break;
+        case DT_I32: case DT_U32: launch_col2im_fast<uint32_t, uint32_t>(col, im, q, accumulate, s); break;
+        case DT_I64: case DT_U64: launch_col2im_fast<uint64_t, uint64_t>(col, im, q, accumulate, s); break;
+        default: return hipErrorInvalidValue;
+        }
+        return hipGetLastError();
+    }
     int64_t blocks = (total + 255) / 256;
     if (blocks > 256 * 64) blocks = 256 * 64;
     const dim3 g((unsigned)blocks), b(256);

@@ -245,6 +245,12 @@ BACKWARD_GEOMS = [
     (64, 256, 6, 6, 128, 3, 3, 1, 1, 1, 1),                # dW with two images per K loop (36 pixels each: the seam falls inside a K-step)
     (8, 512, 5, 7, 512, 3, 3, 1, 1, 1, 1),                 # 35 pixels per image, two images per K loop, four tile rows
     (12, 128, 7, 7, 64, 3, 3, 1, 1, 1, 4),                 # groups; 49 pixels per image (rows of dY not 16-byte multiples)
+    # strides > 1: dX as one stride-1 convolution per phase of the image
+    (4, 32, 17, 19, 64, 3, 3, 2, 1, 1, 1),
+    (2, 16, 20, 14, 32, 5, 4, (2, 3), (2, 1), 1, 2),       # different strides per axis, groups
+    (3, 8, 9, 9, 16, 2, 2, 4, 0, 1, 1),                    # stride beyond the kernel: phases without taps stay zero
+    (2, 8, 23, 23, 16, 7, 7, 2, 3, 1, 1),
+    (2, 16, 11, 12, 32, 3, 3, (1, 2), (0, 2), 1, 1),       # stride on one axis only, rows left over by the stride
 ]
 
 
