@@ -1179,8 +1179,37 @@ int ntg_conv2d_backward_dev(int dtype, const void* image, const void* kernel, co
     hipStream_t hs = static_cast<hipStream_t>(stream);
     ntg_gemm_desc d;
     // Floating dtypes: neither gradient needs the stored im2col matrix (conv_dkernel_gather, conv_dimage_gather).
-    const bool gather_dw = plan.gather_dw, gather_dx = plan.gather_dx;
+    bool gather_dw = plan.gather_dw, gather_dx = plan.gather_dx;
     const Geo3 geo = geo2(height, width, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c, Ho, Wo);
+    // 1x1 kernel, unit stride, no padding (floating dtypes, 16-byte rows): col is the image itself, so both gradients are
+    // products on the tensors where they lie: dX_b = W_g^T . dY_b, and dW_g = sum_b dY_b . X_b^T through per-image results
+    // in the workspace (the amount the gathering form needs), summed in batch order.
+    if (!is_int_dtype(dtype) && conv_pointwise_ok(dtype, channels, groups, geo) && (og * es) % 16 == 0 &&
+        ((reinterpret_cast<uintptr_t>(image) | reinterpret_cast<uintptr_t>(kernel) | reinterpret_cast<uintptr_t>(grad_out) |
+          reinterpret_cast<uintptr_t>(d_image) | reinterpret_cast<uintptr_t>(d_kernel) | reinterpret_cast<uintptr_t>(ws)) & 15) == 0) {
+        const int64_t cg = channels / groups;
+        for (int64_t g = 0; g < groups && d_image; ++g) {
+            std::memset(&d, 0, sizeof d);
+            d.dtype = dtype; d.transpose_a = 1; d.c_mode = accumulate ? NTG_C_ACCUMULATE : NTG_C_OVERWRITE;
+            d.m = cg; d.k = og; d.n = L; d.batches = batch;
+            d.stride_a = 0; d.stride_b = out_channels * L; d.stride_c = channels * L;
+            rc = ntg_gemm_dev(&d, kern + g * og * cg * es, gy + g * og * L * es, static_cast<char*>(d_image) + g * cg * L * es, stream);
+            if (rc) return rc;
+        }
+        for (int64_t g = 0; g < groups && d_kernel; ++g) {
+            std::memset(&d, 0, sizeof d);
+            d.dtype = dtype; d.transpose_b = 1; d.c_mode = NTG_C_OVERWRITE;
+            d.m = og; d.k = L; d.n = cg; d.batches = batch;
+            d.stride_a = out_channels * L; d.stride_b = channels * L; d.stride_c = out_channels * cg;
+            rc = ntg_gemm_dev(&d, gy + g * og * L * es, static_cast<const char*>(image) + g * cg * L * es, ws + g * og * cg * es, stream);
+            if (rc) return rc;
+        }
+        if (d_kernel) {
+            hipError_t e = ntg::launch_reduce_batch(dtype, ws, d_kernel, batch, out_channels * cg, accumulate, hs);
+            if (e != hipSuccess) return hip_fail(e, "weight gradient reduction launch");
+        }
+        return NTG_OK;
+    }
     if (gather_dw) {
         if (plan.nhwc_dw && workspace_bytes >= plan.need_nhwc_dw && ((reinterpret_cast<uintptr_t>(ws) | reinterpret_cast<uintptr_t>(grad_out)) & 15) == 0)
             rc = conv_dkernel_nhwc(dtype, image, grad_out, d_kernel, ws, batch, channels, out_channels, geo, groups, accumulate, hs);

@@ -245,6 +245,7 @@ BACKWARD_GEOMS = [
     (64, 256, 6, 6, 128, 3, 3, 1, 1, 1, 1),                # dW with two images per K loop (36 pixels each: the seam falls inside a K-step)
     (8, 512, 5, 7, 512, 3, 3, 1, 1, 1, 1),                 # 35 pixels per image, two images per K loop, four tile rows
     (12, 128, 7, 7, 64, 3, 3, 1, 1, 1, 4),                 # groups; 49 pixels per image (rows of dY not 16-byte multiples)
+    (6, 32, 8, 12, 48, 1, 1, 1, 0, 1, 2),                  # 1x1: both gradients are plain batched products
     # strides > 1: dX as one stride-1 convolution per phase of the image
     (4, 32, 17, 19, 64, 3, 3, 2, 1, 1, 1),
     (2, 16, 20, 14, 32, 5, 4, (2, 3), (2, 1), 1, 2),       # different strides per axis, groups
