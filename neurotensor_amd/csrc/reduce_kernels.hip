@@ -35,6 +35,43 @@ __global__ void __launch_bounds__(256) reduce_batch_taps_last_kernel(const T* __
     }
 }
 
+// The same with 16-byte loads: a thread owns VEC consecutive channels of one (row, tap) and keeps four partial-sum
+// loads in flight; the order of the additions per element is unchanged.  Needs cg % VEC == 0 and aligned partial sums.
+template <class T, class Acc>
+__global__ void __launch_bounds__(256) reduce_batch_taps_last_vec_kernel(const T* __restrict__ part, T* __restrict__ out, const int64_t batch,
+                                                                         const int64_t rows, const int64_t cg, const int64_t taps, const int accumulate) {
+    constexpr int VEC = 16 / (int)sizeof(T);
+    typedef T TV __attribute__((ext_vector_type(VEC)));
+    const int64_t n = rows * cg * taps, nv = n / VEC;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t v = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; v < nv; v += stride) {
+        const int64_t i = v * VEC;
+        const int64_t c = i % cg, t = (i / cg) % taps, o = i / (cg * taps);
+        T* dst = out + (o * cg + c) * taps + t;
+        Acc acc[VEC];
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) acc[e] = accumulate ? (Acc)dst[(int64_t)e * taps] : (Acc)0;
+        const T* pp = part + i;
+        int64_t b = 0;
+        for (; b + 4 <= batch; b += 4) {
+            TV x[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) x[u] = *reinterpret_cast<const TV*>(pp + (b + u) * n);
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) acc[e] += (Acc)x[u][e];
+        }
+        for (; b < batch; ++b) {
+            const TV x = *reinterpret_cast<const TV*>(pp + b * n);
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) acc[e] += (Acc)x[e];
+        }
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) dst[(int64_t)e * taps] = (T)acc[e];
+    }
+}
+
 // Split-K epilogue: C (+)= sum over the k ranges of part[s][m][n], s ascending, starting from C0 (the incoming C, the
 // broadcast bias, or zero).  One rounding to T at the end.
 template <class T, class P, class Acc>
@@ -159,6 +196,17 @@ hipError_t launch_reduce_batch_taps_last(int dtype, const void* part, void* out,
                                          int accumulate, hipStream_t s) {
     const int64_t n = rows * cg * taps;
     if (n == 0) return hipSuccess;
+    const int64_t vec = 16 / elem_size(dtype);
+    if (cg % vec == 0 && (reinterpret_cast<uintptr_t>(part) & 15) == 0) {
+        const dim3 g(grid_for(n / vec)), b(256);
+        switch (dtype) {
+        case DT_F32: hipLaunchKernelGGL((reduce_batch_taps_last_vec_kernel<float, float>), g, b, 0, s, (const float*)part, (float*)out, batch, rows, cg, taps, accumulate); break;
+        case DT_F16: hipLaunchKernelGGL((reduce_batch_taps_last_vec_kernel<_Float16, float>), g, b, 0, s, (const _Float16*)part, (_Float16*)out, batch, rows, cg, taps, accumulate); break;
+        case DT_BF16: hipLaunchKernelGGL((reduce_batch_taps_last_vec_kernel<__bf16, float>), g, b, 0, s, (const __bf16*)part, (__bf16*)out, batch, rows, cg, taps, accumulate); break;
+        default: return hipErrorInvalidValue;
+        }
+        return hipGetLastError();
+    }
     const dim3 g(grid_for(n)), b(256);
     switch (dtype) {
     case DT_F32: hipLaunchKernelGGL((reduce_batch_taps_last_kernel<float, float>), g, b, 0, s, (const float*)part, (float*)out, batch, rows, cg, taps, accumulate); break;
