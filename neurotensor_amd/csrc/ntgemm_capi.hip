@@ -773,6 +773,9 @@ static PhasePlan plan_dimage_phases(int dtype, int64_t batch, int64_t channels, 
     const int64_t es = ntg::elem_size(dtype), og = out_channels / groups;
     pp.ogp = nhwc_padded_channels(es, og);
     if (pp.ogp == 0 || batch * channels * g.vol() >= 0x7fffffffLL) return pp;
+    // the image channels of a group are the rows of these products: with a handful of them (an RGB input layer) a 64-row
+    // tile is mostly padding, and the GEMM over (channel, tap) rows followed by col2im is the better form
+    if (channels / groups < 16) return pp;
     for (int ax = 1; ax <= 2; ++ax) {
         int64_t* M = ax == 1 ? pp.Mr : pp.Mc;
         int64_t* a0 = ax == 1 ? pp.a0r : pp.a0c;
