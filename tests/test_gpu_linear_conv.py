@@ -407,6 +407,46 @@ def test_conv2d_pointwise_is_a_product_on_the_image(dtype):
             assert err <= HALF_REL * ref.abs().max().item()
 
 
+@pytest.mark.parametrize("seed,big", [(11, False), (12, False), (13, True)], ids=["small-a", "small-b", "large"])
+def test_conv2d_random_geometries_forward_and_gradients(seed, big):
+    """Seeded random geometries (channels per group from 3 to 256, kernels up to 5x5, strides up to 3, dilation, padding,
+    groups, batches up to 64, Float32 / BFloat16 / Float16) through conv2d and both gradients against torch in double:
+    whichever of the kernels a geometry selects -- channels-last with or without padded channels, phases, several images
+    per K loop, pointwise products, element-wise gathers, GEMM + col2im -- the result must be the convolution."""
+    rng = np.random.default_rng(seed)
+    for it in range(24 if big else 60):
+        dt = [torch.float32, torch.bfloat16, torch.float16][int(rng.integers(0, 3))]
+        groups = int(rng.choice([1, 1, 1, 2, 4]))
+        cg = int(rng.choice([16, 32, 64, 128, 256] if big else [3, 8, 12, 16, 24, 32, 48, 64]))
+        og = int(rng.choice([16, 32, 64, 128, 256] if big else [4, 8, 16, 24, 32, 40, 64, 96]))
+        kh, kw = int(rng.integers(1, 6)), int(rng.integers(1, 6))
+        s = (int(rng.integers(1, 4)), int(rng.integers(1, 4))) if rng.random() < 0.5 else (1, 1)
+        d = (int(rng.integers(1, 3)), int(rng.integers(1, 3))) if rng.random() < 0.3 else (1, 1)
+        p = (int(rng.integers(0, 4)), int(rng.integers(0, 4)))
+        H, W = int(rng.integers(1, 50 if big else 30)), int(rng.integers(1, 50 if big else 30))
+        B = int(rng.choice([1, 2, 16, 64, 24] if big else [1, 2, 3, 8, 33]))
+        if H + 2 * p[0] - d[0] * (kh - 1) - 1 < 0 or W + 2 * p[1] - d[1] * (kw - 1) - 1 < 0:
+            continue
+        case = f"dt={dt} B={B} C={cg * groups} H={H} W={W} O={og * groups} k=({kh},{kw}) s={s} p={p} d={d} groups={groups}"
+        print(case, flush=True)
+        x = torch.randn(B, cg * groups, H, W, device=DEV).to(dt)
+        w = (torch.randn(og * groups, cg, kh, kw, device=DEV) / (cg * kh * kw) ** 0.5).to(dt)
+        xr, wr = x.double().requires_grad_(True), w.double().requires_grad_(True)
+        yr = torch.nn.functional.conv2d(xr, wr, None, s, p, d, groups)
+        g = torch.randn_like(yr).to(dt)
+        yr.backward(g.double())
+        y = F.conv2d(x, w, stride=s, padding=p, dilation=d, groups=groups)
+        dx, dw = F.conv2d_backward(x, w, g, stride=s, padding=p, dilation=d, groups=groups)
+        if dt == torch.float32:
+            L = yr.shape[2] * yr.shape[3]
+            tols = (1e-5 * cg * kh * kw * float(x.abs().max() * w.abs().max()), 1e-5 * og * kh * kw * float(g.abs().max() * w.abs().max()),
+                    1e-5 * B * L * float(g.abs().max() * x.abs().max()))
+        else:
+            tols = tuple(HALF_REL * max(r.abs().max().item(), 1e-30) for r in (yr, xr.grad, wr.grad))
+        for got, ref, tol, what in ((y, yr.detach(), tols[0], "y"), (dx, xr.grad, tols[1], "dx"), (dw, wr.grad, tols[2], "dw")):
+            assert (got.double() - ref).abs().max().item() <= tol, (case, what)
+
+
 def _gpu_family(golden_dir, name, sfx, fwd, bwd, ofwd, obwd, kw):
     x, w, exp, g, xg, wg = (load(golden_dir, f"{name}_{part}{sfx}") for part in ("input", "weight", "output", "grad", "xgrad", "wgrad"))
     out = fwd(dev(x), dev(w), **kw).cpu().numpy()
