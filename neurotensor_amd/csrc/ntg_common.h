@@ -180,8 +180,8 @@ hipError_t launch_phase_weights(int64_t es, const void* w, void* wt, int64_t gro
                                 int64_t er, int64_t ec, int64_t s_r, int64_t s_c, int64_t Mr, int64_t Mc, hipStream_t s);
 hipError_t launch_phase_interleave(int dtype, const void* tmp, void* im, const PhaseLayout& q, int accumulate, hipStream_t s);
 hipError_t launch_conv_nhwc_dw(int dtype, bool ta, const GemmParams& p, hipStream_t s);   // ta: A (the output gradient) stored [k][m]
-hipError_t launch_reduce_batch_taps_last(int dtype, const void* part, void* out, int64_t batch, int64_t rows, int64_t cg, int64_t taps,
-                                         int accumulate, hipStream_t s);
+hipError_t launch_reduce_batch_taps_last(int dtype, const void* part, void* out, int64_t batch, int64_t rows, int64_t cg, int64_t cgp,
+                                         int64_t taps, int accumulate, hipStream_t s);   // part rows hold cgp >= cg channels per tap
 hipError_t launch_flip_weights(int64_t elem_size, const void* w, void* wt, int64_t groups, int64_t og, int64_t cg, int64_t taps, hipStream_t s);
 
 // grid of a grid-stride element-wise kernel (256 lanes per workgroup, at most 64 workgroups per CU)

@@ -881,6 +881,7 @@ static int64_t conv_dkernel_fold(int64_t batch, int64_t og, int64_t n, int64_t g
     }
     return best;
 }
+static int64_t dkernel_padded_channels(int64_t es, int64_t cg) { const int64_t v = 16 / es; return (cg + v - 1) / v * v; }
 static bool conv_dkernel_nhwc_ok(int dtype, int64_t channels, int64_t out_channels, int64_t groups, const Geo3& g) {
     if (dtype != ntg::DT_F32 && dtype != ntg::DT_F16 && dtype != ntg::DT_BF16) return false;
     if (g.nd != 2 || !conv_implicit_g(dtype, channels, g)) return false;
@@ -889,24 +890,28 @@ static bool conv_dkernel_nhwc_ok(int dtype, int64_t channels, int64_t out_channe
     // rows of dY that are 16-byte multiples are read where they lie; otherwise dY is copied channels-last too and read
     // as a [pixel][out channel] operand, which needs the out channels of a group to be a 16-byte multiple
     const bool a_ok = (g.L() * es) % 16 == 0 || conv_dkernel_nhwc_copies_dy(dtype, out_channels, groups, g);
-    return (cg * es) % 16 == 0 && a_ok && out_channels > 0 && cg * g.taps() < 0x7fffffffLL &&
-           conv_nhwc_offsets_fit(channels, es, g);
+    // the channels of a group are gathered in 16-byte runs: the copy pads them to whole runs (RGB: 3 -> 8 or 4)
+    const int64_t cgp = dkernel_padded_channels(es, cg);
+    return a_ok && cgp <= 4 * cg && out_channels > 0 && cgp * g.taps() < 0x7fffffffLL && conv_nhwc_offsets_fit(groups * cgp, es, g);
 }
 static int64_t conv_dkernel_nhwc_workspace(int dtype, int64_t batch, int64_t channels, int64_t out_channels, int64_t groups, const Geo3& g) {
     const int64_t es = ntg::elem_size(dtype);
     const int64_t gy = conv_dkernel_nhwc_copies_dy(dtype, out_channels, groups, g) ? (int64_t)align_up((size_t)(batch * out_channels * g.L() * es), 256) : 0;
-    return (int64_t)align_up((size_t)(batch * channels * g.vol() * es), 256) + gy + batch * out_channels * (channels / groups) * g.taps() * es;
+    const int64_t cgp = dkernel_padded_channels(es, channels / groups);
+    return (int64_t)align_up((size_t)(batch * groups * cgp * g.vol() * es), 256) + gy + batch * out_channels * cgp * g.taps() * es;
 }
 static int conv_dkernel_nhwc(int dtype, const void* image, const void* grad_out, void* d_kernel, void* ws, int64_t batch,
                              int64_t channels, int64_t out_channels, const Geo3& g, int64_t groups, int accumulate, hipStream_t hs) {
     const int64_t es = ntg::elem_size(dtype), cg = channels / groups, og = out_channels / groups;
-    const int64_t L = g.L(), taps = g.taps(), vol = g.vol(), N = taps * cg;
+    const int64_t cgp = dkernel_padded_channels(es, cg), chp = groups * cgp;      // channels per group / per pixel in the copy
+    const int64_t L = g.L(), taps = g.taps(), vol = g.vol(), N = taps * cgp;
     const bool copy_dy = conv_dkernel_nhwc_copies_dy(dtype, out_channels, groups, g);      // dY read as [pixel][out channel] from its own copy
     const int64_t fold = copy_dy ? conv_dkernel_fold(batch, og, N, groups, L) : 1, items = batch / fold;
     char* ws_img = static_cast<char*>(ws);
-    char* ws_gy = ws_img + align_up((size_t)(batch * channels * vol * es), 256);
+    char* ws_gy = ws_img + align_up((size_t)(batch * chp * vol * es), 256);
     char* ws_part = ws_gy + (copy_dy ? align_up((size_t)(batch * out_channels * L * es), 256) : 0);
-    hipError_t e = ntg::launch_nchw_to_nhwc(es, image, ws_img, batch, channels, vol, hs);
+    hipError_t e = cgp == cg ? ntg::launch_nchw_to_nhwc(es, image, ws_img, batch, channels, vol, hs)
+                             : ntg::launch_nchw_to_nhwc_padded(es, image, ws_img, batch, groups, cg, cgp, vol, hs);
     if (e == hipSuccess && copy_dy) e = ntg::launch_nchw_to_nhwc(es, grad_out, ws_gy, batch, out_channels, L, hs);
     if (e != hipSuccess) return hip_fail(e, "channels-last copy launch");
     for (int64_t gi = 0; gi < groups; ++gi) {
@@ -920,24 +925,24 @@ static int conv_dkernel_nhwc(int dtype, const void* image, const void* grad_out,
             p.A = static_cast<const char*>(grad_out) + gi * og * L * es;
             p.lda = L;
         }
-        p.B = ws_img + gi * cg * es;
+        p.B = ws_img + gi * cgp * es;
         p.C = ws_part + gi * og * N * es;
-        p.ldb = channels; p.ldc = N;
-        p.sA = fold * out_channels * L; p.sB = fold * channels * vol; p.sC = out_channels * N;
+        p.ldb = chp; p.ldc = N;
+        p.sA = fold * out_channels * L; p.sB = fold * chp * vol; p.sC = out_channels * N;
         p.cmode = ntg::C_OVERWRITE;
         p.vecA_ok = 1; p.vecB_ok = 1;
-        fill_conv_geom(p.conv, cg, g);
-        p.conv.chan = (int)channels;               // elements from one pixel to the next
+        fill_conv_geom(p.conv, cgp, g);
+        p.conv.chan = (int)chp;                    // elements from one pixel to the next
         if (fold > 1) {
             p.conv.fold_L = (int)L;
             p.conv.div_fold = ntg::make_fastdiv((uint32_t)L);
-            p.conv.fold_stride = channels * vol;
+            p.conv.fold_stride = chp * vol;
         }
         e = ntg::launch_conv_nhwc_dw(dtype, copy_dy, p, hs);
         if (e != hipSuccess) return hip_fail(e, "channels-last conv_dkernel launch");
     }
     // (groups are consecutive row blocks of both layouts, so one pass covers them all)
-    e = ntg::launch_reduce_batch_taps_last(dtype, ws_part, d_kernel, items, out_channels, cg, taps, accumulate, hs);
+    e = ntg::launch_reduce_batch_taps_last(dtype, ws_part, d_kernel, items, out_channels, cg, cgp, taps, accumulate, hs);
     if (e != hipSuccess) return hip_fail(e, "weight gradient reduction launch");
     return NTG_OK;
 }

@@ -23,11 +23,13 @@ __global__ void __launch_bounds__(256) reduce_batch_kernel(const T* __restrict__
 // out[o][c][t]: threads follow the partial sums (coalesced reads of the large side), the small result is written scattered.
 template <class T, class Acc>
 __global__ void __launch_bounds__(256) reduce_batch_taps_last_kernel(const T* __restrict__ part, T* __restrict__ out, const int64_t batch,
-                                                                     const int64_t rows, const int64_t cg, const int64_t taps, const int accumulate) {
-    const int64_t n = rows * cg * taps;
+                                                                     const int64_t rows, const int64_t cg, const int64_t cgp, const int64_t taps,
+                                                                     const int accumulate) {
+    const int64_t n = rows * cgp * taps;                  // (the partial sums hold cgp >= cg channels per tap, the rest padding)
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
-        const int64_t c = i % cg, t = (i / cg) % taps, o = i / (cg * taps);
+        const int64_t c = i % cgp, t = (i / cgp) % taps, o = i / (cgp * taps);
+        if (c >= cg) continue;
         T* dst = out + (o * cg + c) * taps + t;
         Acc acc = accumulate ? (Acc)*dst : (Acc)0;
         for (int64_t b = 0; b < batch; ++b) acc += (Acc)part[b * n + i];
@@ -192,12 +194,12 @@ hipError_t launch_reduce_batch(int dtype, const void* part, void* out, int64_t b
     return hipGetLastError();
 }
 
-hipError_t launch_reduce_batch_taps_last(int dtype, const void* part, void* out, int64_t batch, int64_t rows, int64_t cg, int64_t taps,
-                                         int accumulate, hipStream_t s) {
-    const int64_t n = rows * cg * taps;
+hipError_t launch_reduce_batch_taps_last(int dtype, const void* part, void* out, int64_t batch, int64_t rows, int64_t cg, int64_t cgp,
+                                         int64_t taps, int accumulate, hipStream_t s) {
+    const int64_t n = rows * cgp * taps;
     if (n == 0) return hipSuccess;
     const int64_t vec = 16 / elem_size(dtype);
-    if (cg % vec == 0 && (reinterpret_cast<uintptr_t>(part) & 15) == 0) {
+    if (cgp == cg && cg % vec == 0 && (reinterpret_cast<uintptr_t>(part) & 15) == 0) {
         const dim3 g(grid_for(n / vec)), b(256);
         switch (dtype) {
         case DT_F32: hipLaunchKernelGGL((reduce_batch_taps_last_vec_kernel<float, float>), g, b, 0, s, (const float*)part, (float*)out, batch, rows, cg, taps, accumulate); break;
@@ -209,9 +211,9 @@ hipError_t launch_reduce_batch_taps_last(int dtype, const void* part, void* out,
     }
     const dim3 g(grid_for(n)), b(256);
     switch (dtype) {
-    case DT_F32: hipLaunchKernelGGL((reduce_batch_taps_last_kernel<float, float>), g, b, 0, s, (const float*)part, (float*)out, batch, rows, cg, taps, accumulate); break;
-    case DT_F16: hipLaunchKernelGGL((reduce_batch_taps_last_kernel<_Float16, float>), g, b, 0, s, (const _Float16*)part, (_Float16*)out, batch, rows, cg, taps, accumulate); break;
-    case DT_BF16: hipLaunchKernelGGL((reduce_batch_taps_last_kernel<__bf16, float>), g, b, 0, s, (const __bf16*)part, (__bf16*)out, batch, rows, cg, taps, accumulate); break;
+    case DT_F32: hipLaunchKernelGGL((reduce_batch_taps_last_kernel<float, float>), g, b, 0, s, (const float*)part, (float*)out, batch, rows, cg, cgp, taps, accumulate); break;
+    case DT_F16: hipLaunchKernelGGL((reduce_batch_taps_last_kernel<_Float16, float>), g, b, 0, s, (const _Float16*)part, (_Float16*)out, batch, rows, cg, cgp, taps, accumulate); break;
+    case DT_BF16: hipLaunchKernelGGL((reduce_batch_taps_last_kernel<__bf16, float>), g, b, 0, s, (const __bf16*)part, (__bf16*)out, batch, rows, cg, cgp, taps, accumulate); break;
     default: return hipErrorInvalidValue;
     }
     return hipGetLastError();

@@ -89,7 +89,9 @@ def test_argument_errors_do_not_need_a_device():
     assert fast(_lib.FLOAT32, 4, 64, 7, 7, 32, 1, 1, 1, 1, 0, 0, 1, 1, 1) == 50176 + 32 * 64 * 4   # rows of 196 bytes
     assert fast(_lib.FLOAT32, 1, 16, 2, 2, 8, 3, 3, 1, 1, 0, 0, 1, 1, 1) == -1                            # kernel larger than the image
     # per-image weight gradients [B, O, C/g * taps] instead of the im2col matrix
-    assert lib.ntg_conv2d_backward_workspace_bytes(_lib.FLOAT32, 2, 4, 8, 8, 6, 3, 3, 1, 1, 1, 1, 1, 1, 2) == 2 * 6 * 2 * 9 * 4
+    # (the larger figure: channels-last copy of the image with the 2 channels of each group padded to 4, per-image results)
+    assert lib.ntg_conv2d_backward_workspace_bytes(_lib.FLOAT32, 2, 4, 8, 8, 6, 3, 3, 1, 1, 1, 1, 1, 1, 2) == 2 * 2 * 4 * 64 * 4 + 2 * 6 * 4 * 9 * 4
+    assert lib.ntg_conv2d_backward_workspace_bytes(_lib.FLOAT64, 2, 4, 8, 8, 6, 3, 3, 1, 1, 1, 1, 1, 1, 2) == 2 * 6 * 2 * 9 * 8
     assert lib.ntg_conv2d_backward_workspace_bytes(_lib.FLOAT32, 2, 4, 8, 8, 6, 3, 3, 1, 1, 1, 1, 1, 1, 3) == -1
     # transposed convolution: output_padding must stay below the stride; sizes follow (in-1)*s - 2p + d(k-1) + 1 + op
     assert lib.ntg_conv_transpose2d_workspace_bytes(_lib.FLOAT32, 1, 3, 9, 7, 8, 3, 3, 2, 2, 0, 0, 1, 1, 2, 1, 1) == -1
