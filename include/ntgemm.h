@@ -189,8 +189,9 @@ int64_t ntg_conv2d_forward_workspace_bytes(int dtype, int64_t batch, int64_t cha
                                            int64_t p_r, int64_t p_c, int64_t d_r, int64_t d_c);
 
 /* Bytes of device workspace with which ntg_conv2d_dev runs its fastest form.  For Float32 whose channels per group are a
- * multiple of 16, and Float16 / BFloat16 with at least 8 channels per group (padded with zeros to a multiple of 32 in the
- * copy), that is a channels-last copy of the image plus the weights with the channel index fastest; the convolution
+ * multiple of 16, Float16 / BFloat16 with at least 8 channels per group (padded with zeros to a multiple of 32 in the
+ * copy), and groups of up to 32 bytes of channels in all three (RGB input layers: pixels of 16 or 32 bytes, several taps
+ * per K-step), that is a channels-last copy of the image plus the weights with the channel index fastest; the convolution
  * (conv.cpp:86-118) then gathers its operand in 16-byte pieces.  Otherwise the figure of
  * ntg_conv2d_forward_workspace_bytes.  ntg_conv2d_dev accepts any smaller workspace and falls back to its other forms. */
 int64_t ntg_conv2d_fast_workspace_bytes(int dtype, int64_t batch, int64_t channels, int64_t height, int64_t width,

@@ -332,7 +332,10 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
     // the B tile [pixel row][64 B] is filled by the same WB 16-byte DMA instructions per wavefront as a stored K-major
     // operand, each lane's address being a wave-uniform term of the K-step (tap and first channel, advanced by counters
     // in scalar registers) plus a per-lane term of its output pixel and 16-byte slot; padding taps read zeros.
-    uint32_t lanepart3[WB], cmask3[WB];
+    // Few channels (p.conv.tap_step = T = 2 or 4): a pixel holds 64 / T bytes of channels and a K-step covers T consecutive
+    // taps of one tap row (the row padded to p.conv.kq_pad taps with zero weights): a lane's 16-byte slot then belongs to
+    // tap q + tq3 of the step, which shifts its address and its validity bit.
+    uint32_t lanepart3[WB], cmask3[WB], tq3[WB];
     int k3_c0 = 0, k3_q = 0, k3_r = 0, k3_up = 0, k3_k = 0, k3_cg = 1;
     if constexpr (GATHER16) {
         const ConvGeom& g = p.conv;
@@ -353,7 +356,14 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
             }
             cmask3[x] = n < p.N ? m : 0u;
             const uint32_t kv = (uint32_t)((lane & 3) ^ ((row >> 1) & 3));
-            lanepart3[x] = (oh * (uint32_t)g.s_r * (uint32_t)g.W + ow * (uint32_t)g.s_c) * (uint32_t)g.chan * (uint32_t)ES + kv * 16u;
+            uint32_t tq = 0u, cho = kv * 16u;
+            if (g.tap_step > 1) {
+                const uint32_t cb = 64u / (uint32_t)g.tap_step;        // bytes of channels per pixel: 16 or 32
+                tq = cho / cb;
+                cho -= tq * cb;
+            }
+            tq3[x] = tq;
+            lanepart3[x] = (oh * (uint32_t)g.s_r * (uint32_t)g.W + ow * (uint32_t)g.s_c + tq * (uint32_t)g.d_c) * (uint32_t)g.chan * (uint32_t)ES + cho;
         }
     }
     // instruction x (0 .. WB - 1) of this wavefront's share of the NEXT gathered tile; the K-step's counters move on after the last
@@ -361,22 +371,25 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
         if constexpr (GATHER16) {
             const ConvGeom& g = p.conv;
             const char* img = reinterpret_cast<const char*>(B);
-            const uint32_t sr = k3_k < p.K ? (uint32_t)k3_r : 31u, sq = 8u + (uint32_t)k3_q;
+            const uint32_t sr = k3_k < p.K ? (uint32_t)k3_r : 31u, sq = 8u + (uint32_t)k3_q + tq3[x];
             const bool ok = ((cmask3[x] >> sr) & (cmask3[x] >> sq) & 1u) != 0u;
             const char* src = ok ? img + (int64_t)k3_up + lanepart3[x] : reinterpret_cast<const char*>(ring_zero_word);
             asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
                          :: "s"(lds_tile + (uint32_t)(wave_u * WB + x) * 1024u), "v"(src) : "memory");
             if (x == WB - 1) {
+                // one K-step on: the next 64 bytes of channels of this tap, else the next tap (or the next tap_step taps)
+                const bool merged = g.tap_step > 1;
+                const int qstep = merged ? g.tap_step : 1, qend = merged ? g.kq_pad : g.k_c;
                 int c0 = k3_c0 + BK, up = k3_up + BK * ES, q = k3_q, r = k3_r;
-                const bool w0 = c0 >= k3_cg;
+                const bool w0 = merged || c0 >= k3_cg;
+                up = merged ? k3_up + qstep * g.d_c * g.chan * ES : w0 ? up - k3_cg * ES + g.d_c * g.chan * ES : up;
                 c0 = w0 ? c0 - k3_cg : c0;
-                up = w0 ? up - k3_cg * ES + g.d_c * g.chan * ES : up;
-                q = w0 ? q + 1 : q;
-                const bool w1 = q >= g.k_c;
+                q = w0 ? q + qstep : q;
+                const bool w1 = q >= qend;
                 q = w1 ? 0 : q;
-                up = w1 ? up - g.k_c * g.d_c * g.chan * ES + g.d_r * g.W * g.chan * ES : up;
+                up = w1 ? up - qend * g.d_c * g.chan * ES + g.d_r * g.W * g.chan * ES : up;
                 r = w1 ? r + 1 : r;
-                k3_c0 = c0; k3_up = up; k3_q = q; k3_r = r; k3_k += BK;
+                k3_c0 = merged ? 0 : c0; k3_up = up; k3_q = q; k3_r = r; k3_k += BK;
             }
         }
     };

@@ -50,6 +50,8 @@ struct ConvGeom {
     int fold_L;
     FastDiv div_fold;
     int64_t fold_stride;
+    // channels-last convolution of few channels: taps of one tap row per K-step (0 / 1: one tap) and the padded row length
+    int tap_step, kq_pad;
 };
 
 struct GemmParams {
@@ -162,6 +164,8 @@ hipError_t launch_splitk_reduce(int dtype, const void* part, int splits, const G
 hipError_t launch_reduce_batch(int dtype, const void* part, void* out, int64_t batch, int64_t n, int accumulate, hipStream_t s);
 hipError_t launch_nchw_to_nhwc(int64_t elem_size, const void* in, void* out, int64_t batch, int64_t C, int64_t P, hipStream_t s);
 hipError_t launch_weights_channels_last(int64_t es, const void* w, void* wp, int64_t rows, int64_t cg, int64_t cgp, int64_t taps, hipStream_t s);
+hipError_t launch_weights_channels_last_rows(int64_t es, const void* w, void* wp, int64_t rows, int64_t cg, int64_t cgp, int64_t k_r, int64_t k_c,
+                                             int64_t kq_pad, hipStream_t s);   // tap rows padded from k_c to kq_pad taps
 hipError_t launch_nchw_to_nhwc_padded(int64_t es, const void* in, void* out, int64_t batch, int64_t groups, int64_t cg, int64_t cgp, int64_t P, hipStream_t s);
 hipError_t launch_flip_weights_channels_last(int64_t es, const void* w, void* wt, int64_t groups, int64_t og, int64_t ogp, int64_t cg, int64_t taps, hipStream_t s);
 // channels-last convolution (image [B][pixel][C], weights [O][(r, q, c)]); F16 / BF16 / F32, two spatial axes

@@ -611,6 +611,24 @@ static int64_t nhwc_padded_channels(int64_t es, int64_t cg) {
     const int64_t step = 64 / es, cgp = (cg + step - 1) / step * step;
     return cg > 0 && cgp <= (es == 2 ? 4 : 1) * cg ? cgp : 0;
 }
+// Few channels per group (up to 32 bytes of them): a pixel of the copy holds 16 or 32 bytes and a K-step covers 4 or 2
+// consecutive taps of a tap row, the row padded to a multiple of that with zero weights -- an RGB 7 x 7 input layer in
+// BFloat16 runs on K = 7 * 8 * 8 instead of 49 * 32.  Forward only.
+struct MergedTaps { int64_t cgp, T, kq_pad; };
+static bool conv_nhwc_merged(int dtype, int64_t channels, int64_t out_channels, int64_t groups, const Geo3& g, MergedTaps& mt) {
+    if (dtype != ntg::DT_F32 && dtype != ntg::DT_F16 && dtype != ntg::DT_BF16) return false;
+    if (g.nd != 2 || !conv_implicit_g(dtype, channels, g) || out_channels <= 0) return false;
+    const int64_t es = ntg::elem_size(dtype), cg = channels / groups;
+    if (cg <= 0 || cg * es > 32) return false;
+    const int64_t cb = cg * es <= 16 ? 16 : 32;
+    mt.cgp = cb / es; mt.T = 64 / cb; mt.kq_pad = (g.k[2] + mt.T - 1) / mt.T * mt.T;
+    if (mt.kq_pad > 8 || mt.kq_pad * mt.cgp > 4 * g.k[2] * cg) return false;          // (padding: at most 4x the arithmetic)
+    return conv_nhwc_offsets_fit(groups * mt.cgp, es, g);
+}
+static int64_t conv_nhwc_merged_workspace(int dtype, int64_t batch, int64_t out_channels, int64_t groups, const Geo3& g, const MergedTaps& mt) {
+    const int64_t es = ntg::elem_size(dtype);
+    return (int64_t)align_up((size_t)(batch * groups * mt.cgp * g.vol() * es), 256) + out_channels * g.k[1] * mt.kq_pad * mt.cgp * es;
+}
 static bool conv_nhwc_ok(int dtype, int64_t channels, int64_t out_channels, int64_t groups, const Geo3& g) {
     if (dtype != ntg::DT_F32 && dtype != ntg::DT_F16 && dtype != ntg::DT_BF16) return false;
     if (g.nd != 2 || !conv_implicit_g(dtype, channels, g)) return false;
@@ -622,16 +640,17 @@ static int64_t conv_nhwc_workspace(int dtype, int64_t batch, int64_t channels, i
     return (int64_t)align_up((size_t)(batch * groups * cgp * g.vol() * es), 256) + out_channels * cgp * g.taps() * es;
 }
 static int conv_forward_nhwc(int dtype, const void* image, const void* kernel, void* out, void* ws, int64_t batch, int64_t channels,
-                             int64_t out_channels, const Geo3& g, int64_t groups, hipStream_t hs) {
+                             int64_t out_channels, const Geo3& g, int64_t groups, hipStream_t hs, const MergedTaps* mt = nullptr) {
     const int64_t es = ntg::elem_size(dtype), cg = channels / groups, og = out_channels / groups;
-    const int64_t cgp = nhwc_padded_channels(es, cg), chp = groups * cgp;      // channels per group / per pixel in the copy
-    const int64_t L = g.L(), taps = g.taps(), vol = g.vol(), K = taps * cgp;
+    const int64_t cgp = mt ? mt->cgp : nhwc_padded_channels(es, cg), chp = groups * cgp;      // channels per group / per pixel in the copy
+    const int64_t L = g.L(), taps = g.taps(), vol = g.vol(), K = mt ? g.k[1] * mt->kq_pad * cgp : taps * cgp;
     char* ws_img = static_cast<char*>(ws);
     char* ws_w = ws_img + align_up((size_t)(batch * chp * vol * es), 256);
     hipError_t e = cgp == cg ? ntg::launch_nchw_to_nhwc(es, image, ws_img, batch, channels, vol, hs)
                              : ntg::launch_nchw_to_nhwc_padded(es, image, ws_img, batch, groups, cg, cgp, vol, hs);
     if (e != hipSuccess) return hip_fail(e, "channels-last copy launch");
-    e = ntg::launch_weights_channels_last(es, kernel, ws_w, out_channels, cg, cgp, taps, hs);
+    e = mt ? ntg::launch_weights_channels_last_rows(es, kernel, ws_w, out_channels, cg, cgp, g.k[1], g.k[2], mt->kq_pad, hs)
+           : ntg::launch_weights_channels_last(es, kernel, ws_w, out_channels, cg, cgp, taps, hs);
     if (e != hipSuccess) return hip_fail(e, "weight permutation launch");
     for (int64_t gi = 0; gi < groups; ++gi) {
         ntg::GemmParams p;
@@ -646,6 +665,7 @@ static int conv_forward_nhwc(int dtype, const void* image, const void* kernel, v
         p.vecA_ok = 1; p.vecB_ok = 1;
         fill_conv_geom(p.conv, cgp, g);
         p.conv.chan = (int)chp;                    // elements from one pixel to the next
+        if (mt) { p.conv.tap_step = (int)mt->T; p.conv.kq_pad = (int)mt->kq_pad; }
         e = ntg::launch_conv_nhwc(dtype, p, hs);
         if (e != hipSuccess) return hip_fail(e, "channels-last convolution launch");
     }
@@ -984,6 +1004,8 @@ int64_t ntg_conv2d_fast_workspace_bytes(int dtype, int64_t batch, int64_t channe
     const Geo3 g = geo2(height, width, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c, Ho, Wo);
     const bool groups_ok = groups >= 1 && channels % groups == 0 && out_channels % groups == 0;      // (the call itself reports bad groups)
     if (groups_ok && conv_pointwise_ok(dtype, channels, groups, g)) return 0;
+    MergedTaps mt;
+    if (groups_ok && conv_nhwc_merged(dtype, channels, out_channels, groups, g, mt)) return conv_nhwc_merged_workspace(dtype, batch, out_channels, groups, g, mt);
     if (groups_ok && conv_nhwc_ok(dtype, channels, out_channels, groups, g)) return conv_nhwc_workspace(dtype, batch, channels, out_channels, groups, g);
     return ntg_conv2d_forward_workspace_bytes(dtype, batch, channels, height, width, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c);
 }
@@ -1034,6 +1056,10 @@ int ntg_conv2d_dev(int dtype, const void* image, const void* kernel, void* out,
             (is_int_dtype(dtype) || ((reinterpret_cast<uintptr_t>(image) | reinterpret_cast<uintptr_t>(kernel) | reinterpret_cast<uintptr_t>(out)) & 15) == 0))
             return conv_forward_pointwise(dtype, image, kernel, out, batch, channels, out_channels, g, groups, stream);
         // with the workspace of ntg_conv2d_fast_workspace_bytes: channels-last copy of the image, 16-byte gathers
+        MergedTaps mt;
+        if (conv_nhwc_merged(dtype, channels, out_channels, groups, g, mt) && workspace && (reinterpret_cast<uintptr_t>(workspace) & 15) == 0 &&
+            workspace_bytes >= conv_nhwc_merged_workspace(dtype, batch, out_channels, groups, g, mt))
+            return conv_forward_nhwc(dtype, image, kernel, out, workspace, batch, channels, out_channels, g, groups, static_cast<hipStream_t>(stream), &mt);
         if (conv_nhwc_ok(dtype, channels, out_channels, groups, g) && workspace && (reinterpret_cast<uintptr_t>(workspace) & 15) == 0 &&
             workspace_bytes >= conv_nhwc_workspace(dtype, batch, channels, out_channels, groups, g))
             return conv_forward_nhwc(dtype, image, kernel, out, workspace, batch, channels, out_channels, g, groups, static_cast<hipStream_t>(stream));

@@ -432,6 +432,35 @@ hipError_t launch_weights_channels_last(int64_t es, const void* w, void* wp, int
     return hipGetLastError();
 }
 
+// wp[o][r][q][c] = w[o][c][r][q] with every tap row padded with zeros from k_c to kq_pad taps and the channels from cg to cgp
+template <class T>
+__global__ void __launch_bounds__(256) weights_channels_last_rows_kernel(const T* __restrict__ w, T* __restrict__ wp, const int64_t rows, const int64_t cg,
+                                                                         const int64_t cgp, const int64_t k_r, const int64_t k_c, const int64_t kq_pad) {
+    const int64_t total = rows * k_r * kq_pad * cgp;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += stride) {
+        const int64_t c = idx % cgp;
+        int64_t t = idx / cgp;
+        const int64_t q = t % kq_pad;
+        t /= kq_pad;
+        const int64_t r = t % k_r, o = t / k_r;
+        wp[idx] = (c < cg && q < k_c) ? w[((o * cg + c) * k_r + r) * k_c + q] : (T)0;
+    }
+}
+
+hipError_t launch_weights_channels_last_rows(int64_t es, const void* w, void* wp, int64_t rows, int64_t cg, int64_t cgp, int64_t k_r, int64_t k_c,
+                                             int64_t kq_pad, hipStream_t s) {
+    const int64_t total = rows * k_r * kq_pad * cgp;
+    if (total == 0) return hipSuccess;
+    const dim3 g(grid_for(total)), t(256);
+    switch (es) {
+    case 2: hipLaunchKernelGGL(weights_channels_last_rows_kernel<uint16_t>, g, t, 0, s, (const uint16_t*)w, (uint16_t*)wp, rows, cg, cgp, k_r, k_c, kq_pad); break;
+    case 4: hipLaunchKernelGGL(weights_channels_last_rows_kernel<uint32_t>, g, t, 0, s, (const uint32_t*)w, (uint32_t*)wp, rows, cg, cgp, k_r, k_c, kq_pad); break;
+    default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+
 // out[b][p][g*cgp + c] = in[b][g*cg + c][p] for c < cg, 0 for cg <= c < cgp: the channels-last copy with the channels of
 // every group padded to cgp.  64 x 64 tiles of (channel inside the group, pixel) through LDS, like the plain copy.
 template <class T>
@@ -456,8 +485,41 @@ __global__ void __launch_bounds__(256) nchw_to_nhwc_pad_kernel(const T* __restri
     }
 }
 
+// The same for groups of at most 32 bytes of channels (padded to 16 or 32 bytes): one thread per pixel and group reads its
+// cg channels (each a coalesced stream over the pixels) and stores the padded run with 16-byte stores.
+template <class T, int CP>
+__global__ void __launch_bounds__(256) nchw_to_nhwc_few_kernel(const T* __restrict__ in, T* __restrict__ out, const int64_t total, const int64_t groups,
+                                                               const int64_t cg, const int64_t P) {
+    constexpr int VEC = 16 / (int)sizeof(T);
+    typedef T TV __attribute__((ext_vector_type(VEC)));
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= total) return;
+    const int64_t pp = idx % P, bg = idx / P, b = bg / groups, g = bg - b * groups;
+    const T* src = in + bg * cg * P + pp;
+    TV* dst = reinterpret_cast<TV*>(out + ((b * P + pp) * groups + g) * CP);
+#pragma unroll
+    for (int v = 0; v < CP / VEC; ++v) {
+        TV x;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) x[e] = (v * VEC + e) < cg ? src[(int64_t)(v * VEC + e) * P] : (T)0;
+        dst[v] = x;
+    }
+}
+
 hipError_t launch_nchw_to_nhwc_padded(int64_t es, const void* in, void* out, int64_t batch, int64_t groups, int64_t cg, int64_t cgp, int64_t P, hipStream_t s) {
     if (batch * groups * cgp * P == 0) return hipSuccess;
+    if (cgp * es <= 32 && (cgp * es) % 16 == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0) {
+        const int64_t total = batch * groups * P, blocks = (total + 255) / 256;
+        if (blocks <= 0x7fffffffLL) {
+            const dim3 g((unsigned)blocks), t(256);
+            if (es == 2 && cgp == 8) hipLaunchKernelGGL((nchw_to_nhwc_few_kernel<uint16_t, 8>), g, t, 0, s, (const uint16_t*)in, (uint16_t*)out, total, groups, cg, P);
+            else if (es == 2) hipLaunchKernelGGL((nchw_to_nhwc_few_kernel<uint16_t, 16>), g, t, 0, s, (const uint16_t*)in, (uint16_t*)out, total, groups, cg, P);
+            else if (es == 4 && cgp == 4) hipLaunchKernelGGL((nchw_to_nhwc_few_kernel<uint32_t, 4>), g, t, 0, s, (const uint32_t*)in, (uint32_t*)out, total, groups, cg, P);
+            else if (es == 4) hipLaunchKernelGGL((nchw_to_nhwc_few_kernel<uint32_t, 8>), g, t, 0, s, (const uint32_t*)in, (uint32_t*)out, total, groups, cg, P);
+            else return hipErrorInvalidValue;
+            return hipGetLastError();
+        }
+    }
     const int64_t cblocks = (cgp + 63) / 64, gx = (P + 63) / 64, gy = cblocks * groups;
     if (gx > 0x7fffffffLL || gy > 65535) return hipErrorInvalidValue;
     for (int64_t b0 = 0; b0 < batch; b0 += 65535) {                    // (grid z limit)

@@ -79,10 +79,13 @@ def test_argument_errors_do_not_need_a_device():
     assert fast(_lib.BFLOAT16, 2, 64, 7, 7, 48, 3, 3, 1, 1, 1, 1, 1, 1, 2) == 12544 + 48 * 32 * 9 * 2    # 2*64*49*2 = 12544
     assert fast(_lib.FLOAT32, 1, 16, 5, 5, 8, 3, 3, 1, 1, 1, 1, 1, 1, 1) == 1792 + 8 * 16 * 9 * 4        # 1600 -> 1792
     # 16-bit: channels per group are padded to whole 64-byte runs in the copy (up to 4x); Float32 takes whole runs only
-    assert fast(_lib.BFLOAT16, 1, 16, 5, 5, 8, 3, 3, 1, 1, 1, 1, 1, 1, 1) == 1792 + 8 * 32 * 9 * 2       # 16 -> 32 channels: 1600 -> 1792
-    assert fast(_lib.FLOAT16, 2, 24, 5, 5, 8, 3, 3, 1, 1, 1, 1, 1, 1, 2) == 6400 + 8 * 32 * 9 * 2         # 2 groups of 12 -> 32
-    assert fast(_lib.BFLOAT16, 1, 3, 8, 8, 4, 3, 3, 1, 1, 1, 1, 1, 1, 1) == 0                             # 3 -> 32 would be 10x: gathers
+    assert fast(_lib.BFLOAT16, 2, 40, 5, 5, 8, 3, 3, 1, 1, 1, 1, 1, 1, 1) == 6400 + 8 * 64 * 9 * 2        # 40 -> 64 channels
     assert fast(_lib.FLOAT32, 1, 24, 8, 8, 4, 3, 3, 1, 1, 1, 1, 1, 1, 1) == 0                             # 24 is not a multiple of 16
+    # up to 32 bytes of channels per group: pixels of 16 or 32 bytes, 4 or 2 taps of a tap row per K-step (rows padded to that)
+    assert fast(_lib.BFLOAT16, 1, 16, 5, 5, 8, 3, 3, 1, 1, 1, 1, 1, 1, 1) == 1024 + 8 * 3 * 4 * 16 * 2   # 16 channels, rows of 3 -> 4 taps
+    assert fast(_lib.FLOAT16, 2, 24, 5, 5, 8, 3, 3, 1, 1, 1, 1, 1, 1, 2) == 3328 + 8 * 3 * 4 * 16 * 2     # 2 groups of 12 -> 16
+    assert fast(_lib.BFLOAT16, 1, 3, 8, 8, 4, 3, 3, 1, 1, 1, 1, 1, 1, 1) == 1024 + 4 * 3 * 4 * 8 * 2      # RGB: 3 -> 8 channels
+    assert fast(_lib.FLOAT32, 1, 3, 8, 8, 4, 3, 3, 1, 1, 1, 1, 1, 1, 1) == 1024 + 4 * 3 * 4 * 4 * 4       # RGB: 3 -> 4 channels
     assert fast(_lib.FLOAT64, 1, 16, 5, 5, 8, 3, 3, 1, 1, 1, 1, 1, 1, 1) == 0
     assert fast(_lib.INT32, 1, 16, 5, 5, 8, 3, 3, 1, 1, 1, 1, 1, 1, 1) == 16 * 9 * 25 * 4
     assert fast(_lib.FLOAT32, 4, 64, 8, 8, 32, 1, 1, 1, 1, 0, 0, 1, 1, 1) == 0                            # 1x1: product in place
