@@ -595,7 +595,8 @@ static int conv_forward_pointwise(int dtype, const void* image, const void* kern
 // Channels-last form of the same convolution, for the floating dtypes up to 32 bits: the image is first copied to
 // [B][pixel][C] and the weights to [O][(taps, c)] in the workspace; then one K-step of the product is 64 bytes of consecutive
 // channels of one tap, and the kernel's DMA gathers the operand in 16-byte pieces instead of element by element.
-// byte offsets inside a channels-last image are formed in 32 bits from two terms (the pixel of the window origin, and the
+
+// Byte offsets inside a channels-last image are formed in 32 bits from two terms (the pixel of the window origin, and the
 // tap reach with the padding taken off): both must stay below 2^30
 static bool conv_nhwc_offsets_fit(int64_t channels, int64_t es, const Geo3& g) {
     const int64_t pr = g.p[1] < 0 ? -g.p[1] : g.p[1], pc = g.p[2] < 0 ? -g.p[2] : g.p[2];
@@ -728,7 +729,7 @@ static int conv_dimage_gather(int dtype, const void* kernel, const void* grad_ou
 }
 
 // The same gradient through the channels-last kernel: dY is copied to [B][pixel][O] and the flipped weights to
-// [C][(taps, oc)] in the workspace, when the out channels of a group fill whole 64-byte runs.
+// [C][(taps, oc)] in the workspace (out channels of a group in whole 64-byte runs, padded like the forward copy).
 static bool conv_dimage_nhwc_ok(int dtype, int64_t channels, int64_t out_channels, int64_t groups, const Geo3& g) {
     return conv_nhwc_ok(dtype, out_channels, channels, groups, geo_dimage(g));
 }
@@ -877,8 +878,8 @@ static int conv_dimage_phases(int dtype, const PhasePlan& pp, const void* kernel
 
 // dW through the channels-last kernel: the image is copied to [B][pixel][C]; per image and group
 // P_{b,g} [og][(taps, c)] = dY_{b,g} [og, L] . col^T gathered 16 bytes of channels at a time; the per-image results are
-// summed in batch order into the kernel's [O][c][taps] layout.  Needs rows of dY and the channels of a group to be
-// 16-byte multiples.
+// summed in batch order into the kernel's [O][c][taps] layout.  The copy pads the channels of a group to whole 16-byte
+// runs; dY is read where it lies or from a channels-last copy of its own (below).
 // Large output planes with 16-byte rows: dY is read where it lies, one image per K loop (measured faster from about 512
 // pixels: no copy, one LDS read per block instead of the transposing ones).  Otherwise, when the out channels of a group
 // are a 16-byte multiple, dY goes through its own channels-last copy: as a [pixel][out channel] matrix the images follow
