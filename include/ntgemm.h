@@ -155,13 +155,16 @@ typedef struct ntg_gemm_desc {
     int64_t stride_a, stride_b, stride_c;   /* elements between items; 0 on A/B = broadcast */
     const void* bias;           /* device pointer, NTG_C_BIAS only */
     int64_t bias_batch_stride, bias_row_stride, bias_col_stride;   /* elements; 0 = broadcast */
-    void* workspace;            /* optional device scratch, 16-byte aligned, ntg_gemm_workspace_bytes(desc) bytes: lets a   */
-    int64_t workspace_bytes;    /* single product with few output tiles and a deep k be split along k (deterministic)      */
+    void* workspace;            /* optional device scratch, 256-byte aligned, ntg_gemm_workspace_bytes(desc) bytes: lets a   */
+    int64_t workspace_bytes;    /* single product with few output tiles and a deep k be split along k (deterministic), and  */
+                                /* a large Int32 / UInt32 product run as byte planes on the 8-bit matrix pipe (bit-exact)   */
 } ntg_gemm_desc;
 
-/* Bytes of workspace with which ntg_gemm_dev can split the product along k (0: it would not split).  Without a
- * workspace the same result is computed by one pass over k; only the speed of shapes such as [256, 8192] x [8192, 8192]
- * differs.  The reference has no counterpart: its k loop is always serial (nt_matmult.hpp:196). */
+/* Bytes of workspace with which ntg_gemm_dev runs its faster form (0: there is none for this product): a split along k
+ * for shapes such as [256, 8192] x [8192, 8192], or, for Int32 / UInt32 products of 2^31 multiply-adds or more, the ten
+ * products of balanced byte planes on v_mfma_i32_32x32x32_i8, whose sum modulo 2^32 is the reference's wrapping result
+ * (nt/mp/simde_traits/simde_traits_avx2.h: 32-bit mullo / add).  Without a workspace the same result is computed by the
+ * plain kernels.  The reference has no counterpart: its k loop is always serial (nt_matmult.hpp:196). */
 int64_t ntg_gemm_workspace_bytes(const ntg_gemm_desc* desc);
 
 /* nt_matmult<T> on device buffers: C += op(A).op(B), dense leading dimensions. */

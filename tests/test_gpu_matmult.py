@@ -223,6 +223,54 @@ def test_empty_k_is_an_empty_sum(tdtype):
         assert torch.equal(c, want), mode
 
 
+@pytest.mark.parametrize("code", [_lib.INT32, _lib.UINT32], ids=["int32", "uint32"])
+def test_int32_on_the_8bit_matrix_pipe_bit_exact(code):
+    """Large Int32 / UInt32 products run as ten products of balanced byte planes on v_mfma_i32_32x32x32_i8 when the
+    caller gives the workspace: every result must equal the wrapping 32-bit arithmetic of the reference over the FULL value
+    range -- checked against the vector-ALU kernel (same call without workspace) on all elements and against exact
+    integer arithmetic on sampled rows -- in all four transpose forms, the three C modes, ragged sizes (k and n not
+    multiples of 16), a broadcast operand."""
+    lib = _lib.load()
+    st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    rng = np.random.default_rng(4200)
+    batch, m, k, n = 4, 520, 2057, 522
+    for (ta, tb), mode, bcast_b in zip(TRANS, (_lib.C_OVERWRITE, _lib.C_ACCUMULATE, _lib.C_BIAS, _lib.C_ACCUMULATE), (False, True, False, False)):
+        nb = 1 if bcast_b else batch
+        a = rng.integers(-2**31, 2**31, (batch, m, k), dtype=np.int64).astype(np.int32)
+        b = rng.integers(-2**31, 2**31, (nb, k, n), dtype=np.int64).astype(np.int32)
+        c0 = rng.integers(-2**31, 2**31, (batch, m, n), dtype=np.int64).astype(np.int32)
+        bias = rng.integers(-2**31, 2**31, (n,), dtype=np.int64).astype(np.int32)
+        sa = np.ascontiguousarray(a.transpose(0, 2, 1)) if ta else a
+        sb = np.ascontiguousarray(b.transpose(0, 2, 1)) if tb else b
+        ta_, tb_, tbias = (torch.from_numpy(x).to(DEV) for x in (sa, sb, bias))      # (the two dtypes share their bit patterns)
+        results = []
+        for use_ws in (True, False):
+            c = torch.from_numpy(c0.copy()).to(DEV)
+            d = _lib.GemmDesc()
+            d.dtype = code
+            d.transpose_a, d.transpose_b, d.c_mode = int(ta), int(tb), mode
+            d.m, d.k, d.n, d.batches = m, k, n, batch
+            d.stride_a, d.stride_b, d.stride_c = m * k, (0 if bcast_b else k * n), m * n
+            if mode == _lib.C_BIAS:
+                d.bias = tbias.data_ptr()
+                d.bias_col_stride = 1
+            wsb = lib.ntg_gemm_workspace_bytes(ctypes.byref(d))
+            assert wsb > 0
+            if use_ws:
+                ws = torch.empty(wsb, dtype=torch.uint8, device=DEV)
+                d.workspace, d.workspace_bytes = ws.data_ptr(), wsb
+            _lib.check(lib.ntg_gemm_dev(ctypes.byref(d), ta_.data_ptr(), tb_.data_ptr(), c.data_ptr(), st))
+            torch.cuda.synchronize()
+            results.append(c.cpu().numpy())
+        assert np.array_equal(results[0], results[1]), (ta, tb, mode)
+        # exact arithmetic (int64 wraps modulo 2^64, which keeps the low 32 bits) on a few rows of two items
+        for bi in (0, batch - 1):
+            rows = np.r_[0:3, m - 3:m]
+            exact = a[bi, rows].astype(np.int64) @ b[0 if bcast_b else bi].astype(np.int64)
+            init = c0[bi, rows].astype(np.int64) if mode == _lib.C_ACCUMULATE else bias.astype(np.int64)[None, :] if mode == _lib.C_BIAS else 0
+            assert np.array_equal(results[0][bi, rows], (exact + init).astype(np.int32)), (ta, tb, mode, bi)
+
+
 def test_host_batch_with_repeated_pointers():
     """nt_matmult_batch: uniform shape, entries of A/B may repeat (broadcast by handle)."""
     rng = np.random.default_rng(500)
