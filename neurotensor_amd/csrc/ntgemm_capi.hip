@@ -411,8 +411,21 @@ int ntg_matmult_batch(int dtype, const void* const* A, const void* const* B, voi
     std::memset(&d, 0, sizeof d);
     d.dtype = dtype; d.transpose_a = transpose_a; d.transpose_b = transpose_b; d.c_mode = NTG_C_ACCUMULATE;
     d.m = m; d.k = k; d.n = n; d.batches = batches;
+    // The arena is this function's own: when every item's A (and B) is a new matrix, or all items share one, the slots
+    // lie at a constant stride and the strided kernels (and their workspace forms) serve the batch; any other pattern of
+    // repeated pointers goes through the pointer tables.
+    auto constant_stride = [&](const std::map<const void*, size_t>& slot, const void* const* P, size_t bytes, int64_t& stride) {
+        const size_t step = slot.size() == 1 ? 0 : align_up(bytes, 256);
+        for (int64_t i = 0; i < batches; ++i)
+            if (slot.at(P[i]) != slot.at(P[0]) + (size_t)i * step) return false;
+        stride = (int64_t)(step / (size_t)es);
+        return true;
+    };
+    const bool strided = constant_stride(slotA, A, a_bytes, d.stride_a) && constant_stride(slotB, B, b_bytes, d.stride_b);
+    if (strided) d.stride_c = (int64_t)(align_up(c_bytes, 256) / (size_t)es);
+    else d.stride_a = d.stride_b = 0;
     const size_t ws_off = off;
-    const int64_t ws_bytes = batches == 1 ? ntg_gemm_workspace_bytes(&d) : 0;
+    const int64_t ws_bytes = strided ? ntg_gemm_workspace_bytes(&d) : 0;
     if (ws_bytes > 0) off += (size_t)ws_bytes;
 
     DeviceMem mem;
@@ -433,8 +446,8 @@ int ntg_matmult_batch(int dtype, const void* const* A, const void* const* B, voi
 
     void** dtab = reinterpret_cast<void**>(mem.at(tab_off));
     if (ws_bytes > 0) { d.workspace = mem.at(ws_off); d.workspace_bytes = ws_bytes; }
-    if (batches == 1) {
-        rc = ntg_gemm_dev(&d, tab[0], tab[1], tab[2], nullptr);
+    if (strided) {
+        rc = ntg_gemm_dev(&d, tab[0], tab[(size_t)batches], tab[(size_t)(2 * batches)], nullptr);
     } else {
         rc = ntg_gemm_ptrs_dev(&d, dtab, dtab + batches, dtab + 2 * batches, nullptr);
     }

@@ -69,7 +69,7 @@ static std::shared_ptr<char> device_alloc(size_t bytes) {
     return std::shared_ptr<char>(static_cast<char*>(p), [](char* q) { (void)hipFree(q); });
 }
 
-// Scratch for the `_dev` convolutions: one buffer per thread that only grows.  All device work of this facade is
+// Scratch for the `_dev` convolutions and products: one buffer per thread that only grows.  All device work of this facade is
 // issued on the default stream, so a later call reuses it safely after the earlier one in stream order.
 static void* device_workspace(int64_t bytes) {
     static thread_local std::shared_ptr<char> buf;
@@ -466,6 +466,8 @@ static void device_gemm(int dt, int64_t es, bool ta, bool tb, int mode, int64_t 
             d.bias_row_stride = brow > 1 ? bcol : 0;
             d.bias_col_stride = bcol > 1 ? 1 : 0;
         }
+        const int64_t wsb = ntg_gemm_workspace_bytes(&d);      // > 0: a faster form exists (split along k, byte planes)
+        if (wsb > 0) { d.workspace = device_workspace(wsb); d.workspace_bytes = wsb; }
         check_status(ntg_gemm_dev(&d, A + (na > 1 ? (i0 % na) * m * k * es : 0), B + (nb > 1 ? (i0 % nb) * k * n * es : 0),
                                   C + i0 * m * n * es, nullptr));
     }

@@ -295,6 +295,35 @@ def test_host_batch_with_repeated_pointers():
     assert single.tobytes() == got[0].tobytes()
 
 
+@pytest.mark.parametrize("pattern", ["distinct", "shared_b", "shared_a", "mixed"])
+def test_host_batch_int32_full_range_every_pointer_pattern(pattern):
+    """nt_matmult_batch on host pointers, Int32 wrapping modulo 2^32 with full-range entries: items that are all new
+    matrices or all one matrix take the strided kernels (large enough here for the byte-plane form), any other pattern
+    of repeated pointers the pointer tables; every pattern equals exact integer arithmetic, item by item."""
+    rng = np.random.default_rng(77)
+    nb, m, k, n = 4, 256, 1024, 2304
+    full = lambda shape: rng.integers(-2**31, 2**31, shape, dtype=np.int64).astype(np.int32)
+    As = [full((m, k)) for _ in range(nb)]
+    Bs = [full((k, n)) for _ in range(nb)]
+    if pattern == "shared_b":
+        Bs = [Bs[0]] * nb
+    elif pattern == "shared_a":
+        As = [As[0]] * nb
+    elif pattern == "mixed":
+        As = [As[0], As[1], As[0], As[1]]
+    C0 = [full((m, n)) for _ in range(nb)]
+    got = [c.copy() for c in C0]
+    arr = ctypes.c_void_p * nb
+    lib = _lib.load()
+    _lib.check(lib.ntg_matmult_batch(_lib.INT32, arr(*[x.ctypes.data for x in As]), arr(*[x.ctypes.data for x in Bs]),
+                                     arr(*[x.ctypes.data for x in got]), nb, m, k, k, n, 0, 0))
+    rows = np.array([0, 1, 127, 128, 255])
+    for i in range(nb):
+        # exact: 64-bit wrapping sums of 32 x 32 -> 64-bit products keep the low 32 bits intact
+        exact = As[i][rows].astype(np.int64) @ Bs[i].astype(np.int64) + C0[i][rows].astype(np.int64)
+        assert np.array_equal(got[i][rows], exact.astype(np.int32)), (pattern, i)
+
+
 def test_functional_batch_rules_and_views():
     """N-D x K-D: trailing batch dims must match; lower-rank operand is reused; a transposed
     view is consumed by flipping the flag (no copy); results equal the oracle's."""
