@@ -157,13 +157,13 @@ typedef struct ntg_gemm_desc {
     int64_t bias_batch_stride, bias_row_stride, bias_col_stride;   /* elements; 0 = broadcast */
     void* workspace;            /* optional device scratch, 256-byte aligned, ntg_gemm_workspace_bytes(desc) bytes: lets a   */
     int64_t workspace_bytes;    /* single product with few output tiles and a deep k be split along k (deterministic), and  */
-                                /* a large Int32 / UInt32 product run as byte planes on the 8-bit matrix pipe (bit-exact)   */
+                                /* a large 16/32/64-bit integer product run as byte planes on the 8-bit matrix pipe (bit-exact) */
 } ntg_gemm_desc;
 
 /* Bytes of workspace with which ntg_gemm_dev runs its faster form (0: there is none for this product): a split along k
- * for shapes such as [256, 8192] x [8192, 8192], or, for Int32 / UInt32 products of 2^31 multiply-adds or more, the ten
- * products of balanced byte planes on v_mfma_i32_32x32x32_i8, whose sum modulo 2^32 is the reference's wrapping result
- * (nt/mp/simde_traits/simde_traits_avx2.h: 32-bit mullo / add).  Without a workspace the same result is computed by the
+ * for shapes such as [256, 8192] x [8192, 8192], or, for large Int16 / Int32 / Int64 products and their unsigned forms, the
+ * 3 / 10 / 36 products of balanced byte planes on v_mfma_i32_32x32x32_i8, whose sum modulo 2^W is the reference's wrapping
+ * result (nt/mp/simde_traits/simde_traits_avx2.h:810-812, :444-446, :523-540: multiply and add in the element type).  Without a workspace the same result is computed by the
  * plain kernels.  The reference has no counterpart: its k loop is always serial (nt_matmult.hpp:196). */
 int64_t ntg_gemm_workspace_bytes(const ntg_gemm_desc* desc);
 

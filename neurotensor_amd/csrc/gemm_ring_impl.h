@@ -762,7 +762,7 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
                 const bool hi_ok = !RAGGED || ES != 4 || n + 4 < p.N;
                 if constexpr (CM == C_PARTIAL) {
                     // split-K: the fp32 sums of this k range go to a float matrix; rounding happens after the reduction
-                    // (8-bit operands: the 32-bit integer sums, for the byte-plane form of the Int32 product)
+                    // (8-bit operands: the 32-bit integer sums, for the byte-plane form of the wider integer products)
                     float* wp = static_cast<float*>(p.C) + (int64_t)b * p.sC + (int64_t)m * p.ldc + n;
                     *reinterpret_cast<accx4*>(wp) = lo;
                     if (hi_ok) *reinterpret_cast<accx4*>(wp + 4) = hi;

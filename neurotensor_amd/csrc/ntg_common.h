@@ -183,10 +183,10 @@ struct PhaseLayout {
 hipError_t launch_phase_weights(int64_t es, const void* w, void* wt, int64_t groups, int64_t og, int64_t ogp, int64_t cg, int64_t k_r, int64_t k_c,
                                 int64_t er, int64_t ec, int64_t s_r, int64_t s_c, int64_t Mr, int64_t Mc, hipStream_t s);
 hipError_t launch_phase_interleave(int dtype, const void* tmp, void* im, const PhaseLayout& q, int accumulate, hipStream_t s);
-// Int32 / UInt32 products on the 8-bit matrix pipe (see gemm_mfma_i8.hip)
-struct I32PlanesParams { int M, N, K, Kp, Np, batch; int64_t lda, ldb, sA, sB; int ta, tb; };
-hipError_t launch_i32_split_planes(const void* A, const void* B, void* a_planes, void* b_planes, const I32PlanesParams& q, hipStream_t s);
-hipError_t launch_i32_combine(const void* parts, const GemmParams& p, int Np, hipStream_t s);
+// 16-, 32- and 64-bit integer products on the 8-bit matrix pipe as byte planes (see gemm_mfma_i8.hip); planes = bytes per element
+struct IntPlanesParams { int M, N, K, Kp, Np, batch; int64_t lda, ldb, sA, sB; int ta, tb; };
+hipError_t launch_int_split_planes(int planes, const void* A, const void* B, void* a_planes, void* b_planes, const IntPlanesParams& q, hipStream_t s);
+hipError_t launch_int_combine(int planes, const void* parts, const GemmParams& p, int Np, hipStream_t s);
 hipError_t launch_conv_nhwc_dw(int dtype, bool ta, const GemmParams& p, hipStream_t s);   // ta: A (the output gradient) stored [k][m]
 hipError_t launch_reduce_batch_taps_last(int dtype, const void* part, void* out, int64_t batch, int64_t rows, int64_t cg, int64_t cgp,
                                          int64_t taps, int accumulate, hipStream_t s);   // part rows hold cgp >= cg channels per tap

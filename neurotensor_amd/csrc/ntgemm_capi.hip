@@ -136,52 +136,76 @@ int launch_gemm(ntg::GemmParams p, int dtype, bool ta, bool tb, hipStream_t s) {
 // range order by a second kernel.  Deterministic; applied only when the caller supplies the workspace.
 struct SplitPlan { int splits; int64_t kc; int64_t bytes; };
 
-// Int32 / UInt32 on the 8-bit matrix pipe (byte planes, gemm_mfma_i8.hip): ten 8-bit products at about 2 Pop/s against
-// about 30 Top/s on the vector ALU, plus some 60 us of splitting and recombining: taken from about 2^31 multiply-adds,
-// when the caller supplies the workspace.
-struct I32Plan { bool ok; int Kp, Np; int64_t a_bytes, b_bytes, p_bytes; int64_t bytes() const { return a_bytes + b_bytes + p_bytes; } };
-static I32Plan plan_i32_mfma(const ntg::GemmParams& p, int dtype) {
-    I32Plan pl;
+// 16-, 32- and 64-bit integers on the 8-bit matrix pipe (byte planes, gemm_mfma_i8.hip): P (P + 1) / 2 8-bit products
+// (P bytes per element) instead of the vector ALU's multiply-adds, plus the passes that split the operands and
+// recombine the partial sums.  Taken when the caller supplies the workspace and an estimate of both times favours it.
+// Measured on MI355X: the vector-ALU kernel spends about 0.07 us (16- and 32-bit; 0.13 us 64-bit) per k on each round of
+// 64 x 64 tiles over the 256 CUs, plus as much once; the plane form costs its P + 3 launches (17 / 30 / 55 us for
+// P = 2 / 4 / 8), the 8-bit products at about 10^9 multiply-adds per us, and the partial sums written and read at 4 TB/s.
+struct IntPlanesPlan {
+    bool ok; int planes, Kp, Np; int64_t a_bytes, b_bytes, p_bytes;
+    int64_t bytes() const { return a_bytes + b_bytes + p_bytes; }
+};
+static int int_planes_of(int dtype) {
+    switch (dtype) {
+    case ntg::DT_I16: case ntg::DT_U16: return 2;
+    case ntg::DT_I32: case ntg::DT_U32: return 4;
+    case ntg::DT_I64: case ntg::DT_U64: return 8;
+    default: return 0;
+    }
+}
+static IntPlanesPlan plan_int_planes(const ntg::GemmParams& p, int dtype) {
+    IntPlanesPlan pl;
     std::memset(&pl, 0, sizeof pl);
-    if ((dtype != ntg::DT_I32 && dtype != ntg::DT_U32) || p.Aptr || p.Bptr || p.Cptr) return pl;
-    if (p.M < 128 || p.N < 128 || p.K < 64 || p.K >= 32768) return pl;
-    if ((double)p.M * p.N * p.K * p.batch < 2147483648.0) return pl;
+    const int P = int_planes_of(dtype);
+    if (P == 0 || p.Aptr || p.Bptr || p.Cptr) return pl;
+    if (p.M < 128 || p.N < 128 || p.K < 64) return pl;
+    pl.planes = P;
     pl.Kp = (p.K + 15) / 16 * 16;
     pl.Np = (p.N + 15) / 16 * 16;
-    if (4LL * pl.Kp >= (1 << 23) || pl.Np >= (1 << 23)) return pl;
-    pl.a_bytes = (int64_t)align_up((size_t)((p.sA == 0 ? 1 : p.batch) * (int64_t)p.M * 4 * pl.Kp), 256);
-    pl.b_bytes = (int64_t)align_up((size_t)((p.sB == 0 ? 1 : p.batch) * 4LL * pl.Kp * pl.Np), 256);
-    pl.p_bytes = 4LL * p.batch * p.M * pl.Np * 4;
+    {
+        const double macs = (double)p.M * p.N * p.K * p.batch;
+        const double rounds = (double)(((int64_t)((p.M + 63) / 64) * ((p.N + 63) / 64) * p.batch + 255) / 256);
+        const double valu_us = (double)p.K * (P == 8 ? 0.13 : P == 4 ? 0.07 : 0.055) * (rounds + 1.0);
+        const double planes_us = (P == 8 ? 55.0 : P == 4 ? 30.0 : 17.0) + macs * (P * (P + 1) / 2) / 1.0e9 +
+                                 8.0 * P * p.batch * (double)p.M * pl.Np / 4.0e6;
+        if (planes_us > 0.8 * valu_us) return pl;
+    }
+    if ((int64_t)P * pl.Kp >= (1 << 17) || pl.Np >= (1 << 23)) return pl;     // 32-bit partial sums: P K 2^14 < 2^31
+    pl.a_bytes = (int64_t)align_up((size_t)((p.sA == 0 ? 1 : p.batch) * (int64_t)p.M * P * pl.Kp), 256);
+    pl.b_bytes = (int64_t)align_up((size_t)((p.sB == 0 ? 1 : p.batch) * (int64_t)P * pl.Kp * pl.Np), 256);
+    pl.p_bytes = (int64_t)P * p.batch * p.M * pl.Np * 4;
     pl.ok = true;
     return pl;
 }
-static int run_i32_mfma(const ntg::GemmParams& p, const I32Plan& pl, bool ta, bool tb, void* ws, hipStream_t s) {
+static int run_int_planes(const ntg::GemmParams& p, const IntPlanesPlan& pl, bool ta, bool tb, void* ws, hipStream_t s) {
+    const int P = pl.planes;
     char* a_pl = static_cast<char*>(ws);
     char* b_pl = a_pl + pl.a_bytes;
     char* parts = b_pl + pl.b_bytes;
-    ntg::I32PlanesParams q;
+    ntg::IntPlanesParams q;
     q.M = p.M; q.N = p.N; q.K = p.K; q.Kp = pl.Kp; q.Np = pl.Np; q.batch = p.batch;
     q.lda = p.lda; q.ldb = p.ldb; q.sA = p.sA; q.sB = p.sB; q.ta = ta; q.tb = tb;
-    hipError_t e = ntg::launch_i32_split_planes(p.A, p.B, a_pl, b_pl, q, s);
+    hipError_t e = ntg::launch_int_split_planes(P, p.A, p.B, a_pl, b_pl, q, s);
     if (e != hipSuccess) return hip_fail(e, "byte-plane split launch");
     const int64_t per = (int64_t)p.M * pl.Np;
-    for (int sh = 0; sh < 4; ++sh) {
+    for (int sh = 0; sh < P; ++sh) {
         ntg::GemmParams g;
         std::memset(&g, 0, sizeof g);
         g.M = p.M; g.N = pl.Np; g.K = (sh + 1) * pl.Kp; g.batch = p.batch;
         g.A = a_pl;
-        g.B = b_pl + (int64_t)(3 - sh) * pl.Kp * pl.Np;
+        g.B = b_pl + (int64_t)(P - 1 - sh) * pl.Kp * pl.Np;
         g.C = parts + (int64_t)sh * p.batch * per * 4;
-        g.lda = 4LL * pl.Kp; g.ldb = pl.Np; g.ldc = pl.Np;
-        g.sA = p.sA == 0 ? 0 : (int64_t)p.M * 4 * pl.Kp;
-        g.sB = p.sB == 0 ? 0 : 4LL * pl.Kp * pl.Np;
+        g.lda = (int64_t)P * pl.Kp; g.ldb = pl.Np; g.ldc = pl.Np;
+        g.sA = p.sA == 0 ? 0 : (int64_t)p.M * P * pl.Kp;
+        g.sB = p.sB == 0 ? 0 : (int64_t)P * pl.Kp * pl.Np;
         g.sC = per;
         g.cmode = ntg::C_PARTIAL;
         g.vecA_ok = 1; g.vecB_ok = 1;
         e = ntg::launch_gemm_mfma_i8(ntg::DT_I8, false, false, g, s);
         if (e != hipSuccess) return hip_fail(e, "byte-plane product launch");
     }
-    e = ntg::launch_i32_combine(parts, p, pl.Np, s);
+    e = ntg::launch_int_combine(P, parts, p, pl.Np, s);
     if (e != hipSuccess) return hip_fail(e, "byte-plane combine launch");
     return NTG_OK;
 }
@@ -263,10 +287,10 @@ int run_gemm(ntg::GemmParams p, int dtype, bool ta, bool tb, hipStream_t s, void
         if (e != hipSuccess) return hip_fail(e, "empty-k launch");
         return NTG_OK;
     }
-    if (dtype == ntg::DT_I32 || dtype == ntg::DT_U32) {
-        const I32Plan ip = plan_i32_mfma(p, dtype);
+    if (int_planes_of(dtype)) {
+        const IntPlanesPlan ip = plan_int_planes(p, dtype);
         if (ip.ok && workspace && workspace_bytes >= ip.bytes() && (reinterpret_cast<uintptr_t>(workspace) & 255) == 0)
-            return run_i32_mfma(p, ip, ta, tb, workspace, s);
+            return run_int_planes(p, ip, ta, tb, workspace, s);
     }
     const SplitPlan plan = plan_splitk(p, dtype, ta);
     if (plan.splits > 1 && workspace && workspace_bytes >= plan.bytes && (reinterpret_cast<uintptr_t>(workspace) & 15) == 0) {
@@ -346,8 +370,8 @@ int64_t ntg_gemm_workspace_bytes(const ntg_gemm_desc* d) {
     ntg::GemmParams p;
     if (desc_to_params(d, p)) return -1;
     if (p.M == 0 || p.N == 0 || p.batch == 0) return 0;
-    if (d->dtype == ntg::DT_I32 || d->dtype == ntg::DT_U32) {
-        const I32Plan ip = plan_i32_mfma(p, d->dtype);
+    if (int_planes_of(d->dtype)) {
+        const IntPlanesPlan ip = plan_int_planes(p, d->dtype);
         return ip.ok ? ip.bytes() : 0;
     }
     return plan_splitk(p, d->dtype, d->transpose_a != 0).bytes;      // pointers taken as 16-byte aligned

@@ -223,26 +223,26 @@ def test_empty_k_is_an_empty_sum(tdtype):
         assert torch.equal(c, want), mode
 
 
-@pytest.mark.parametrize("code", [_lib.INT32, _lib.UINT32], ids=["int32", "uint32"])
-def test_int32_on_the_8bit_matrix_pipe_bit_exact(code):
-    """Large Int32 / UInt32 products run as ten products of balanced byte planes on v_mfma_i32_32x32x32_i8 when the
-    caller gives the workspace: every result must equal the wrapping 32-bit arithmetic of the reference over the FULL value
-    range -- checked against the vector-ALU kernel (same call without workspace) on all elements and against exact
-    integer arithmetic on sampled rows -- in all four transpose forms, the three C modes, ragged sizes (k and n not
-    multiples of 16), a broadcast operand."""
+@pytest.mark.parametrize("code,npdt", [(_lib.INT16, np.int16), (_lib.UINT16, np.int16), (_lib.INT32, np.int32), (_lib.UINT32, np.int32),
+                                       (_lib.INT64, np.int64), (_lib.UINT64, np.int64)],
+                         ids=["int16", "uint16", "int32", "uint32", "int64", "uint64"])
+def test_wide_integers_on_the_8bit_matrix_pipe_bit_exact(code, npdt):
+    """Large 16-, 32- and 64-bit integer products run as 3 / 10 / 36 products of balanced byte planes on
+    v_mfma_i32_32x32x32_i8 when the caller gives the workspace: every result must equal the wrapping arithmetic of the
+    reference in the element type over the FULL value range -- checked against the vector-ALU kernel (same call without
+    workspace) on all elements and against exact integer arithmetic on sampled rows -- in all four transpose forms, the
+    three C modes, ragged sizes (k and n not multiples of 16), a broadcast operand."""
     lib = _lib.load()
     st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
     rng = np.random.default_rng(4200)
     batch, m, k, n = 4, 520, 2057, 522
+    full = lambda shape: rng.integers(0, 2**64, shape, dtype=np.uint64).astype(npdt)      # (keeps the low bits)
     for (ta, tb), mode, bcast_b in zip(TRANS, (_lib.C_OVERWRITE, _lib.C_ACCUMULATE, _lib.C_BIAS, _lib.C_ACCUMULATE), (False, True, False, False)):
         nb = 1 if bcast_b else batch
-        a = rng.integers(-2**31, 2**31, (batch, m, k), dtype=np.int64).astype(np.int32)
-        b = rng.integers(-2**31, 2**31, (nb, k, n), dtype=np.int64).astype(np.int32)
-        c0 = rng.integers(-2**31, 2**31, (batch, m, n), dtype=np.int64).astype(np.int32)
-        bias = rng.integers(-2**31, 2**31, (n,), dtype=np.int64).astype(np.int32)
+        a, b, c0, bias = full((batch, m, k)), full((nb, k, n)), full((batch, m, n)), full((n,))
         sa = np.ascontiguousarray(a.transpose(0, 2, 1)) if ta else a
         sb = np.ascontiguousarray(b.transpose(0, 2, 1)) if tb else b
-        ta_, tb_, tbias = (torch.from_numpy(x).to(DEV) for x in (sa, sb, bias))      # (the two dtypes share their bit patterns)
+        ta_, tb_, tbias = (torch.from_numpy(x).to(DEV) for x in (sa, sb, bias))      # (signed and unsigned share their bit patterns)
         results = []
         for use_ws in (True, False):
             c = torch.from_numpy(c0.copy()).to(DEV)
@@ -263,12 +263,12 @@ def test_int32_on_the_8bit_matrix_pipe_bit_exact(code):
             torch.cuda.synchronize()
             results.append(c.cpu().numpy())
         assert np.array_equal(results[0], results[1]), (ta, tb, mode)
-        # exact arithmetic (int64 wraps modulo 2^64, which keeps the low 32 bits) on a few rows of two items
+        # exact arithmetic (uint64 wraps modulo 2^64, which keeps the low bits of every width) on a few rows of two items
         for bi in (0, batch - 1):
             rows = np.r_[0:3, m - 3:m]
-            exact = a[bi, rows].astype(np.int64) @ b[0 if bcast_b else bi].astype(np.int64)
-            init = c0[bi, rows].astype(np.int64) if mode == _lib.C_ACCUMULATE else bias.astype(np.int64)[None, :] if mode == _lib.C_BIAS else 0
-            assert np.array_equal(results[0][bi, rows], (exact + init).astype(np.int32)), (ta, tb, mode, bi)
+            exact = a[bi, rows].astype(np.uint64) @ b[0 if bcast_b else bi].astype(np.uint64)
+            init = c0[bi, rows].astype(np.uint64) if mode == _lib.C_ACCUMULATE else bias.astype(np.uint64)[None, :] if mode == _lib.C_BIAS else np.uint64(0)
+            assert np.array_equal(results[0][bi, rows], (exact + init).astype(npdt)), (ta, tb, mode, bi)
 
 
 def test_host_batch_with_repeated_pointers():
