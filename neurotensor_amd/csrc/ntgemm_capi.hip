@@ -457,9 +457,10 @@ int ntg_matmult_batch(int dtype, const void* const* A, const void* const* B, voi
     for (auto& kv : slotA) HIP_TRY(hipMemcpy(mem.at(kv.second), kv.first, a_bytes, hipMemcpyHostToDevice));
     for (auto& kv : slotB) HIP_TRY(hipMemcpy(mem.at(kv.second), kv.first, b_bytes, hipMemcpyHostToDevice));
     std::vector<void*> tab(3 * (size_t)batches);
+    std::map<const void*, int64_t> seenC;
     for (int64_t i = 0; i < batches; ++i) {
-        for (int64_t j = 0; j < i; ++j)
-            if (C[j] == C[i]) return fail(NTG_ERR_INVALID_ARGUMENT, "output pointers of items %lld and %lld alias", (long long)j, (long long)i);
+        const auto ins = seenC.emplace(C[i], i);
+        if (!ins.second) return fail(NTG_ERR_INVALID_ARGUMENT, "output pointers of items %lld and %lld alias", (long long)ins.first->second, (long long)i);
         char* dc = mem.at(c_off + (size_t)i * align_up(c_bytes, 256));
         HIP_TRY(hipMemcpy(dc, C[i], c_bytes, hipMemcpyHostToDevice));   // accumulate contract: C is an input too
         tab[(size_t)i] = mem.at(slotA[A[i]]);
