@@ -168,30 +168,36 @@ __device__ __forceinline__ uint32_t lds_addr_of(const char* p) {
 // (convolution: the tap (c, r, q) is uniform, the pixel per lane; weight gradient: the other way round).  Padding taps
 // and columns / k-rows past the edge read a zero word instead, so the tile in LDS is exact and the multiply loop is the
 // plain one.  Wavefront w gathers k-rows 4 w .. 4 w + 3 of every K-step.
-template <int DT, bool TA, bool TB, bool RAGGED, int WB, int CONV = 0>
+// WBN_ != 0: a rectangular tile, 64 WB_ rows x 64 WBN_ columns (plain products only).
+template <int DT, bool TA, bool TB, bool RAGGED, int WB_, int CONV = 0, int WBN_ = 0>
 __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
     using E = Elem<DT>;
     using T = typename E::T;
     constexpr int ES = sizeof(T);
-    using G = RingGeom<WB, ES>;
+    constexpr int WBM = WB_, WBN = WBN_ ? WBN_ : WB_;    // 32 x 32 blocks per wavefront along m / along n
+    constexpr int WB = WBN;                              // (the gathered operand is B; gathering kernels have square tiles)
+    static_assert(CONV == 0 || WBM == WBN, "gathering kernels have square tiles");
+    using GA = RingGeom<WBM, ES>;                        // geometry of the A tile
+    using G = RingGeom<WBN, ES>;                         // geometry of the B tile
+    constexpr int A_TILE_BYTES = GA::TILE_BYTES, STAGE_BYTES = GA::TILE_BYTES + G::TILE_BYTES;
+    constexpr int WTM = GA::WT, WTN = G::WT;             // a wavefront's share of the tile: WTM rows x WTN columns
     constexpr bool GATHER4 = CONV == 1 || CONV == 2;     // op(B) gathered element by element from an NCHW image
     constexpr bool GATHER16 = CONV == 3;                 // op(B) = col^T gathered in 16-byte pieces from a channels-last image
     constexpr bool GATHERW = CONV == 4;                  // op(B) = col^T of a channels-last image, 16-byte pieces along the channels (weight gradient)
     constexpr bool A_KC = !TA, B_KC = GATHER4 ? false : GATHER16 ? true : GATHERW ? false : TB;
     constexpr int BK = G::BK;
-    constexpr int WT = G::WT;
     static_assert(!GATHER4 || (ES == 4 && !TA && RAGGED), "gathered operands: Float32, A stored [m][k], guarded edges");
     static_assert(!GATHER16 || ((ES == 4 || ES == 2) && !TA && RAGGED), "channels-last gather: 16/32-bit floats, A stored [m][k], guarded edges");
     static_assert(!GATHERW || ((ES == 4 || ES == 2) && !TB && RAGGED), "channels-last weight gradient: 16/32-bit floats, guarded edges");
-    constexpr int NA = WB, NB = GATHER4 ? 4 * WB : WB;   // DMA instructions per wavefront and K-step for the A / B tile
+    constexpr int NA = WBM, NB = GATHER4 ? 4 * WB : WBN;   // DMA instructions per wavefront and K-step for the A / B tile
     // B instructions issued in the first / second half-step (the second also carries the A tile's).  Splitting a gathered
     // tile between the two was measured slower than issuing all of it in the first.
     constexpr int NB1 = NB, NB2 = NB - NB1;
 
-    __shared__ __attribute__((aligned(1024))) char st0[G::STAGE_BYTES];
-    __shared__ __attribute__((aligned(1024))) char st1[G::STAGE_BYTES];
-    __shared__ __attribute__((aligned(1024))) char st2[G::STAGE_BYTES];
-    __shared__ __attribute__((aligned(1024))) char st3[G::STAGE_BYTES];
+    __shared__ __attribute__((aligned(1024))) char st0[STAGE_BYTES];
+    __shared__ __attribute__((aligned(1024))) char st1[STAGE_BYTES];
+    __shared__ __attribute__((aligned(1024))) char st2[STAGE_BYTES];
+    __shared__ __attribute__((aligned(1024))) char st3[STAGE_BYTES];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -203,7 +209,7 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
     const int b = lid / tiles;
     int tm, tn;
     tile_coords(lid - b * tiles, p.tiles_m, p.tiles_n, 4, tm, tn);
-    const int m0 = tm * G::BM, n0 = tn * G::BN;
+    const int m0 = tm * GA::BM, n0 = tn * G::BN;
 
     const T* A = static_cast<const T*>(p.A) + (int64_t)b * p.sA;
     const T* B = static_cast<const T*>(p.B) + (int64_t)b * p.sB;
@@ -214,14 +220,14 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
     const int KT = (p.K + BK - 1) / BK;
     const int last = KT - 1;
     const int kr = p.K - last * BK;                                  // k that exist in the last K-step (a multiple of one chunk)
-    const int mvalid = p.M - m0 < G::BM ? p.M - m0 : G::BM;
+    const int mvalid = p.M - m0 < GA::BM ? p.M - m0 : GA::BM;
     const int nvalid = p.N - n0 < G::BN ? p.N - n0 : G::BN;
-    uint32_t offA[WB], offB[WB];      // K-steps before the last
-    uint32_t offAt[WB], offBt[WB];    // the last K-step (RAGGED: k clamped to what exists)
-    dma_offsets<A_KC, RAGGED, WB, ES>(offA, p.lda, wave, lane, mvalid, BK);
-    dma_offsets<B_KC, RAGGED, WB, ES>(offB, p.ldb, wave, lane, nvalid, BK);
-    dma_offsets<A_KC, RAGGED, WB, ES>(offAt, p.lda, wave, lane, mvalid, kr);
-    dma_offsets<B_KC, RAGGED, WB, ES>(offBt, p.ldb, wave, lane, nvalid, kr);
+    uint32_t offA[WBM], offB[WBN];      // K-steps before the last
+    uint32_t offAt[WBM], offBt[WBN];    // the last K-step (RAGGED: k clamped to what exists)
+    dma_offsets<A_KC, RAGGED, WBM, ES>(offA, p.lda, wave, lane, mvalid, BK);
+    dma_offsets<B_KC, RAGGED, WBN, ES>(offB, p.ldb, wave, lane, nvalid, BK);
+    dma_offsets<A_KC, RAGGED, WBM, ES>(offAt, p.lda, wave, lane, mvalid, kr);
+    dma_offsets<B_KC, RAGGED, WBN, ES>(offBt, p.ldb, wave, lane, nvalid, kr);
     const char* baseA = reinterpret_cast<const char*>(A) + (A_KC ? (int64_t)m0 * p.lda : (int64_t)m0) * ES;
     const char* baseB = reinterpret_cast<const char*>(B) + (B_KC ? (int64_t)n0 * p.ldb : (int64_t)n0) * ES;
     const int64_t advA = (A_KC ? (int64_t)BK : (int64_t)BK * p.lda) * ES;
@@ -465,67 +471,68 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
         const int slot = (2 * ks + (lane >> 5)) ^ ((lane >> 1) & 3);
         return row * 64 + slot * 16;
     };
-    auto frag_off_mm = [&](int wbase, int blk, int ks, int half) -> int {
+    // (mnrow = bytes of one k-row of the operand's MN-major tile, chunks = 16-byte chunks in it)
+    auto frag_off_mm = [&](int mnrow, int wbase, int blk, int ks, int half) -> int {
         const int bl = lane >> 4, s = lane & 15, e = s >> 2, q = s & 3;
         const int krow = 16 * ks + 8 * (bl >> 1) + 4 * half + e;
         const int mnl = wbase + blk * 32 + 16 * (bl & 1) + 4 * q;
         const int chunk = (mnl >> 3) ^ (2 * e);
-        return krow * G::MN_ROW_BYTES + chunk * 16 + (mnl & 7) * 2;
+        return krow * mnrow + chunk * 16 + (mnl & 7) * 2;
     };
     // 8-bit: ds_read_b64_tr_b8 works on groups of 16 lanes; lane i of a group reads the 8 bytes (mn) 8 (i & 1) .. + 7 of
     // k-row i >> 1 and receives, as lane s, the 8 consecutive k of mn s.  Read t (0, 1) of a block covers
     // k = 32 ks + 16 (lane / 32) + 8 t .. + 7 for mn = 32 blk + lane % 32.
-    auto frag_off_mm8 = [&](int wbase, int blk, int ks, int t) -> int {
+    auto frag_off_mm8 = [&](int mnrow, int wbase, int blk, int ks, int t) -> int {
         const int grp = lane >> 4, i = lane & 15;
         const int krow = 32 * ks + 16 * (grp >> 1) + 8 * t + (i >> 1);
         const int mnl = wbase + blk * 32 + 16 * (grp & 1) + 8 * (i & 1);
-        const int chunk = (mnl >> 4) ^ mn8_swizzle<G::CHUNKS>(krow);
-        return krow * G::MN_ROW_BYTES + chunk * 16 + (mnl & 15);
+        const int chunk = (mnl >> 4) ^ (mnrow / 16 >= 8 ? (krow & 7) : ((krow & 7) >> 1));      // mn8_swizzle of the operand
+        return krow * mnrow + chunk * 16 + (mnl & 15);
     };
-    auto frag_off_mm32 = [&](int wbase, int blk, int ks, int e) -> int {
+    auto frag_off_mm32 = [&](int mnrow, int wbase, int blk, int ks, int e) -> int {
         const int krow = 8 * ks + 4 * (lane >> 5) + e;
         const int mnl = wbase + blk * 32 + (lane & 31);
-        if constexpr (GATHER4) return krow * G::MN_ROW_BYTES + mnl * 4;            // gathered tiles are stored unswizzled
-        return krow * G::MN_ROW_BYTES + ((mnl * 4) ^ (128 * (lane >> 5)));      // (krow >> 2) & 1 == lane / 32
+        if constexpr (GATHER4) return krow * mnrow + mnl * 4;            // gathered tiles are stored unswizzled
+        return krow * mnrow + ((mnl * 4) ^ (128 * (lane >> 5)));      // (krow >> 2) & 1 == lane / 32
     };
 
     // One LDS read instruction of an operand's fragment set for half-step ks.  A K-major
     // operand takes WB reads (one ds_read_b128 per block), an MN-major one 2 WB (two transposing
     // 8-byte reads per block; Float32: 4 WB four-byte reads); read r lands in frag[r / per_block].
-    auto read_op = [&](u32x4 (&frag)[WB], const char* tile, bool kc, int wbase, int ks, int r) {
+    auto read_op = [&](auto& frag, int mnrow, const char* tile, bool kc, int wbase, int ks, int r) {
         if (kc) {
             frag[r] = *reinterpret_cast<const u32x4*>(tile + frag_off_km(wbase, r, ks));
         } else if constexpr (ES == 4) {
-            frag[r >> 2][r & 3] = *reinterpret_cast<const uint32_t*>(tile + frag_off_mm32(wbase, r >> 2, ks, r & 3));
+            frag[r >> 2][r & 3] = *reinterpret_cast<const uint32_t*>(tile + frag_off_mm32(mnrow, wbase, r >> 2, ks, r & 3));
         } else if constexpr (ES == 1) {
             const int blk = r >> 1, t = r & 1;
             const intx2v v = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
-                (__attribute__((address_space(3))) intx2v*)(tile + frag_off_mm8(wbase, blk, ks, t)));
+                (__attribute__((address_space(3))) intx2v*)(tile + frag_off_mm8(mnrow, wbase, blk, ks, t)));
             frag[blk][2 * t] = (uint32_t)v[0];
             frag[blk][2 * t + 1] = (uint32_t)v[1];
         } else {
             const int blk = r >> 1, half = r & 1;
             const shortx4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                (__attribute__((address_space(3))) shortx4*)(tile + frag_off_mm(wbase, blk, ks, half)));
+                (__attribute__((address_space(3))) shortx4*)(tile + frag_off_mm(mnrow, wbase, blk, ks, half)));
             typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
             const u32x2 w = __builtin_bit_cast(u32x2, v);
             frag[blk][2 * half] = w[0];
             frag[blk][2 * half + 1] = w[1];
         }
     };
-    constexpr int MNR = ES == 4 ? 4 * WB : 2 * WB;       // reads of an MN-major operand per half-step
-    constexpr int NRA = A_KC ? WB : MNR, NRB = B_KC ? WB : MNR, NR = NRA + NRB;
+    constexpr int MNRB = ES == 4 ? 4 : 2;                // reads of one block of an MN-major operand per half-step
+    constexpr int NRA = A_KC ? WBM : MNRB * WBM, NRB = B_KC ? WBN : MNRB * WBN, NR = NRA + NRB;
     constexpr int MPP = ES == 4 ? 4 : 1;                 // MFMAs per pair of fragments
-    constexpr int NMMA = WB * WB * MPP;                  // MFMAs per half-step
+    constexpr int NMMA = WBM * WBN * MPP;                // MFMAs per half-step
     constexpr int RPM = (NR + NMMA - 1) / NMMA;          // LDS reads slotted behind each MFMA
 
     using AccV = typename E::AccV;
     using AccS = typename E::AccS;
-    AccV acc[WB][WB];
+    AccV acc[WBM][WBN];
 #pragma unroll
-    for (int i = 0; i < WB; ++i)
+    for (int i = 0; i < WBM; ++i)
 #pragma unroll
-        for (int j = 0; j < WB; ++j)
+        for (int j = 0; j < WBN; ++j)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = (AccS)0;
 
@@ -545,24 +552,24 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
 #pragma unroll
             for (int x = 0; x < WB; ++x) conv4_dma(x, lds_tile);
         }
-        else dma_tile<WB>(srcB(kt), kt >= last ? offBt : offB, lds_tile, wave_u);
+        else dma_tile<WBN>(srcB(kt), kt >= last ? offBt : offB, lds_tile, wave_u);
     };
-    dma_tile<WB>(srcA(0), 0 >= last ? offAt : offA, lds_addr_of(st0), wave_u);
-    b_tile(0, lds_addr_of(st0) + G::TILE_BYTES);
-    dma_tile<WB>(srcA(1), 1 >= last ? offAt : offA, lds_addr_of(st1), wave_u);
-    b_tile(1, lds_addr_of(st1) + G::TILE_BYTES);
-    dma_tile<WB>(srcA(2), 2 >= last ? offAt : offA, lds_addr_of(st2), wave_u);
-    b_tile(2, lds_addr_of(st2) + G::TILE_BYTES);
-    dma_tile<WB>(srcA(3), 3 >= last ? offAt : offA, lds_addr_of(st3), wave_u);
+    dma_tile<WBM>(srcA(0), 0 >= last ? offAt : offA, lds_addr_of(st0), wave_u);
+    b_tile(0, lds_addr_of(st0) + A_TILE_BYTES);
+    dma_tile<WBM>(srcA(1), 1 >= last ? offAt : offA, lds_addr_of(st1), wave_u);
+    b_tile(1, lds_addr_of(st1) + A_TILE_BYTES);
+    dma_tile<WBM>(srcA(2), 2 >= last ? offAt : offA, lds_addr_of(st2), wave_u);
+    b_tile(2, lds_addr_of(st2) + A_TILE_BYTES);
+    dma_tile<WBM>(srcA(3), 3 >= last ? offAt : offA, lds_addr_of(st3), wave_u);
 
-    u32x4 af[2][WB], bf[2][WB];   // fragment double buffer: [half-step parity][block]
+    u32x4 af[2][WBM], bf[2][WBN];   // fragment double buffer: [half-step parity][block]
 
     // all reads of one fragment set, back to back (prologue only)
     auto load_frags = [&](const char* stage, int ks, int buf) {
 #pragma unroll
-        for (int r = 0; r < NRA; ++r) read_op(af[buf], stage, A_KC, wm * WT, ks, r);
+        for (int r = 0; r < NRA; ++r) read_op(af[buf], GA::MN_ROW_BYTES, stage, A_KC, wm * WTM, ks, r);
 #pragma unroll
-        for (int r = 0; r < NRB; ++r) read_op(bf[buf], stage + G::TILE_BYTES, B_KC, wn * WT, ks, r);
+        for (int r = 0; r < NRB; ++r) read_op(bf[buf], G::MN_ROW_BYTES, stage + A_TILE_BYTES, B_KC, wn * WTN, ks, r);
     };
     // The NMMA MFMAs of one half-step on fragment set `cur_buf`, with the NR reads of the next set (stage/ks ->
     // `nxt_buf`) slotted RPM (one; two for the small 16-bit tiles) per MFMA, so LDS latency is
@@ -576,8 +583,8 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
 #pragma unroll
         for (int q = 0; q < NMMA; ++q) {
             // serpentine order: consecutive MFMAs always share one operand fragment
-            const int e = q / (WB * WB), pr = q % (WB * WB);
-            const int i = pr / WB, j = (i & 1) ? WB - 1 - (pr % WB) : (pr % WB);
+            const int e = q / (WBM * WBN), pr = q % (WBM * WBN);
+            const int i = pr / WBN, j = (i & 1) ? WBN - 1 - (pr % WBN) : (pr % WBN);
             if constexpr (ES != 4) {
                 E::mma(acc[i][j], bf[cur_buf][j], af[cur_buf][i]);   // D rows <-> n, cols <-> m
             } else {
@@ -587,8 +594,8 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
             }
 #pragma unroll
             for (int r = q * RPM; r < (q + 1) * RPM; ++r) {
-                if (r < NRA) read_op(af[nxt_buf], stage, A_KC, wm * WT, ks, r);
-                else if (r < NR) read_op(bf[nxt_buf], stage + G::TILE_BYTES, B_KC, wn * WT, ks, r - NRA);
+                if (r < NRA) read_op(af[nxt_buf], GA::MN_ROW_BYTES, stage, A_KC, wm * WTM, ks, r);
+                else if (r < NR) read_op(bf[nxt_buf], G::MN_ROW_BYTES, stage + A_TILE_BYTES, B_KC, wn * WTN, ks, r - NRA);
             }
             constexpr int DGAP = NMMA >= NDMA ? NMMA / NDMA : 1, DPER = NMMA >= NDMA ? 1 : NDMA / NMMA;   // MFMAs between two DMA instructions / DMA instructions per MFMA
             if (q % DGAP == DGAP - 1) {
@@ -633,12 +640,12 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
     auto mask_tail = [&](int buf, int ks) {
         const bool ok = (BK / 2) * ks + (BK / 4) * (lane >> 5) < kr;
 #pragma unroll
-        for (int i = 0; i < WB; ++i)
+        for (int e = 0; e < 4; ++e) {
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                af[buf][i][e] = ok ? af[buf][i][e] : 0u;
-                bf[buf][i][e] = ok ? bf[buf][i][e] : 0u;
-            }
+            for (int i = 0; i < WBM; ++i) af[buf][i][e] = ok ? af[buf][i][e] : 0u;
+#pragma unroll
+            for (int j = 0; j < WBN; ++j) bf[buf][j][e] = ok ? bf[buf][j][e] : 0u;
+        }
     };
 
     // (inlined by force: as a call, the stage pointers would arrive in vector registers and could not feed M0)
@@ -648,7 +655,7 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
             const void* src = nullptr;
             if constexpr (CONV == 0) src = srcB(kt + 3);
             const bool tail = kt + 3 >= last;
-            const uint32_t lds_tile = lds_addr_of(prv) + G::TILE_BYTES;
+            const uint32_t lds_tile = lds_addr_of(prv) + A_TILE_BYTES;
             mma_step_prefetch(0, cur, 1, 1, std::integral_constant<int, NB1>{}, std::integral_constant<int, (CONV ? NB1 : 0)>{},
                               [&](int x) __attribute__((always_inline)) {
                 if constexpr (GATHER4) conv_dma(x, lds_tile);
@@ -667,11 +674,11 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
         {
             const void* src = srcA(kt + 4);
             const bool tail = kt + 4 >= last;
-            const uint32_t lds_tile = lds_addr_of(cur), lds_gather = lds_addr_of(prv) + G::TILE_BYTES;
+            const uint32_t lds_tile = lds_addr_of(cur), lds_gather = lds_addr_of(prv) + A_TILE_BYTES;
             mma_step_prefetch(1, nxt, 0, 0, std::integral_constant<int, NB2 + NA>{}, std::integral_constant<int, NB2>{},
                               [&](int x) __attribute__((always_inline)) {
                 if (x < NB2) conv_dma(NB1 + x, lds_gather);       // rest of B(kt+3)
-                else dma_1k(src, (RAGGED && tail) ? offAt[x - NB2] : offA[x - NB2], lds_tile + (uint32_t)(wave_u * WB + x - NB2) * 1024u);
+                else dma_1k(src, (RAGGED && tail) ? offAt[x - NB2] : offA[x - NB2], lds_tile + (uint32_t)(wave_u * WBM + x - NB2) * 1024u);
             });
         }
     };
@@ -687,14 +694,16 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
     asm volatile("" ::: "memory");
 
     // ---- epilogue: per wavefront, WB 32-row slabs through a private fp32 LDS region ----
-    // 32 rows x SROW bytes (the wavefront's WT columns in fp32) per wavefront; 16-byte slot s of
+    // 32 rows x SROW bytes (the wavefront's WTN columns in fp32) per wavefront; 16-byte slot s of
     // row r lives at s ^ (r & 7).  LPR lanes cover a row (8 columns each), so one step of the
     // read-back moves RPS rows.
-    constexpr int SROW = WT * 4, LPR = WT / 8, RPS = 64 / LPR, NSTEP = 32 / RPS;
-    char* slab = ((wave & 2) ? st1 : st0) + (wave & 1) * (32 * SROW);
+    constexpr int SROW = WTN * 4, LPR = WTN / 8, RPS = 64 / LPR, NSTEP = 32 / RPS;
+    // (two slabs fit into one stage unless the tile is wider than tall: then every wavefront takes a stage of its own)
+    char* slab = WBN > WBM ? (wave == 0 ? st0 : wave == 1 ? st1 : wave == 2 ? st2 : st3)
+                           : ((wave & 2) ? st1 : st0) + (wave & 1) * (32 * SROW);
     char* Cb = reinterpret_cast<char*>(C);
     const int col = 8 * (lane % LPR);              // this lane's 8 consecutive columns in the slab
-    const int n = n0 + wn * WT + col;
+    const int n = n0 + wn * WTN + col;
     constexpr int NV = ES == 4 ? 2 : 1;            // 16-byte vectors of C per lane and row: 8 columns of 1 (half a vector), 2 or 4 bytes
     // (only the channels-last convolution meets rows of C that are not 16-byte multiples; uniform)
     const bool c_rows_16 = !GATHER16 || (p.ldc % G::VEL == 0 && p.sC % G::VEL == 0 && (reinterpret_cast<uintptr_t>(p.C) & 15) == 0);
@@ -704,13 +713,13 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
         constexpr int CM = decltype(cmode_tag)::value;
         const T* bias = static_cast<const T*>(p.bias);
 #pragma unroll
-        for (int i = 0; i < WB; ++i) {
+        for (int i = 0; i < WBM; ++i) {
             // C0 of the whole slab is requested before the LDS round trip
             u32x4 c0[NSTEP][NV];
             if constexpr (CM == C_ACCUMULATE) {
 #pragma unroll
                 for (int t = 0; t < NSTEP && c_rows_16; ++t) {
-                    const int m = m0 + wm * WT + 32 * i + RPS * t + lane / LPR;
+                    const int m = m0 + wm * WTM + 32 * i + RPS * t + lane / LPR;
 #pragma unroll
                     for (int v = 0; v < NV; ++v) {
                         if (!RAGGED || (m < p.M && n + 4 * v < p.N)) {
@@ -726,14 +735,14 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
             }
             // lane holds rows m = 32 i + lane%32, cols 32 j + 8 rq + 4 (lane/32) + (0..3)
 #pragma unroll
-            for (int j = 0; j < WB; ++j)
+            for (int j = 0; j < WBN; ++j)
 #pragma unroll
                 for (int rq = 0; rq < 4; ++rq) {
                     accx4 v = {acc[i][j][4 * rq], acc[i][j][4 * rq + 1], acc[i][j][4 * rq + 2], acc[i][j][4 * rq + 3]};
                     const int slot = 8 * j + 2 * rq + (lane >> 5);
                     *reinterpret_cast<accx4*>(slab + (lane & 31) * SROW + ((slot ^ (lane & 7)) * 16)) = v;
                 }
-            // 32 rows x WT cols: NSTEP steps of RPS rows; a lane owns 8 consecutive columns
+            // 32 rows x WTN cols: NSTEP steps of RPS rows; a lane owns 8 consecutive columns
 #pragma unroll
             for (int t = 0; t < NSTEP; ++t) {
                 const int row = RPS * t + lane / LPR;
@@ -741,7 +750,7 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
                 const accx4 lo = *reinterpret_cast<const accx4*>(slab + row * SROW + ((sl ^ (row & 7)) * 16));
                 const accx4 hi = *reinterpret_cast<const accx4*>(slab + row * SROW + (((sl + 1) ^ (row & 7)) * 16));
                 AccS v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-                const int m = m0 + wm * WT + 32 * i + row;
+                const int m = m0 + wm * WTM + 32 * i + row;
                 // 16-bit: N % 8 == 0, a lane's 8 columns exist or not together; Float32: N % 4 == 0, the halves separately
                 if (RAGGED && (m >= p.M || n >= p.N)) continue;
                 if constexpr (GATHER16) {
@@ -822,18 +831,20 @@ static inline bool ring_eligible(const GemmParams& p, bool ta, int es = 2) {
            ((reinterpret_cast<uintptr_t>(p.C) & 15) == 0);
 }
 
-template <int DT, bool TA, bool TB, int WB>
+// WBN != 0: rectangular tiles of 64 WB rows x 64 WBN columns
+template <int DT, bool TA, bool TB, int WB, int WBN = 0>
 static hipError_t launch_ring_cfg(const GemmParams& pin, hipStream_t s) {
-    constexpr int TE = RingGeom<WB, (int)sizeof(typename Elem<DT>::T)>::BM, BK = RingGeom<WB, (int)sizeof(typename Elem<DT>::T)>::BK;
+    constexpr int ES = (int)sizeof(typename Elem<DT>::T);
+    constexpr int TEM = RingGeom<WB, ES>::BM, TEN = RingGeom<(WBN ? WBN : WB), ES>::BM, BK = RingGeom<WB, ES>::BK;
     GemmParams p = pin;
-    p.tiles_m = (p.M + TE - 1) / TE;
-    p.tiles_n = (p.N + TE - 1) / TE;
+    p.tiles_m = (p.M + TEM - 1) / TEM;
+    p.tiles_n = (p.N + TEN - 1) / TEN;
     const int64_t blocks = (int64_t)p.tiles_m * p.tiles_n * p.batch;
     if (blocks > 0x7fffffffLL) return hipErrorInvalidValue;
-    if (p.M % TE == 0 && p.N % TE == 0 && p.K % BK == 0)
-        hipLaunchKernelGGL((gemm_ring_kernel<DT, TA, TB, false, WB>), dim3((unsigned)blocks), dim3(256), 0, s, p);
+    if (p.M % TEM == 0 && p.N % TEN == 0 && p.K % BK == 0)
+        hipLaunchKernelGGL((gemm_ring_kernel<DT, TA, TB, false, WB, 0, WBN>), dim3((unsigned)blocks), dim3(256), 0, s, p);
     else
-        hipLaunchKernelGGL((gemm_ring_kernel<DT, TA, TB, true, WB>), dim3((unsigned)blocks), dim3(256), 0, s, p);
+        hipLaunchKernelGGL((gemm_ring_kernel<DT, TA, TB, true, WB, 0, WBN>), dim3((unsigned)blocks), dim3(256), 0, s, p);
     return hipGetLastError();
 }
 
@@ -880,10 +891,10 @@ static hipError_t launch_ring_nhwc_dw_cfg(const GemmParams& pin, hipStream_t s) 
     return hipGetLastError();
 }
 
-template <int DT, int WB>
+template <int DT, int WB, int WBN = 0>
 static hipError_t launch_ring_wb(bool ta, bool tb, const GemmParams& p, hipStream_t s) {
-    if (ta) return tb ? launch_ring_cfg<DT, true, true, WB>(p, s) : launch_ring_cfg<DT, true, false, WB>(p, s);
-    return tb ? launch_ring_cfg<DT, false, true, WB>(p, s) : launch_ring_cfg<DT, false, false, WB>(p, s);
+    if (ta) return tb ? launch_ring_cfg<DT, true, true, WB, WBN>(p, s) : launch_ring_cfg<DT, true, false, WB, WBN>(p, s);
+    return tb ? launch_ring_cfg<DT, false, true, WB, WBN>(p, s) : launch_ring_cfg<DT, false, false, WB, WBN>(p, s);
 }
 
 // items [b0, b0 + nb) of a strided batch as a product of their own
@@ -900,8 +911,8 @@ static inline GemmParams ring_batch_range(const GemmParams& p, int64_t es, int b
 // 16-bit products: tile edge from the cost estimate; a batch that leaves a small rest of tiles after whole rounds
 // over the CUs goes out as two launches (see ring16_plan).  launch(edge, params) starts one of them.
 template <class Launch>
-static hipError_t launch_ring16_planned(const GemmParams& p, hipStream_t s, Launch&& launch) {
-    Ring16Plan pl = ring16_plan(p.M, p.N, p.K, p.batch);
+static hipError_t launch_ring16_planned(const GemmParams& p, hipStream_t s, Launch&& launch, bool rect = false) {
+    Ring16Plan pl = ring16_plan(p.M, p.N, p.K, p.batch, rect);
     if (p.cmode == C_PARTIAL || p.Aptr || p.Bptr || p.Cptr) pl.head = p.batch;
     if (pl.head >= p.batch) return launch(pl.edge, p);
     const hipError_t e = launch(pl.edge, ring_batch_range(p, 2, 0, pl.head));
@@ -913,9 +924,10 @@ template <int DT>
 static hipError_t launch_ring16(bool ta, bool tb, const GemmParams& p, hipStream_t s) {
     return launch_ring16_planned(p, s, [&](int te, const GemmParams& q) {
         if (te == 256) return launch_ring_wb<DT, 4>(ta, tb, q, s);
+        if (te == 192) return launch_ring_wb<DT, 2, 4>(ta, tb, q, s);      // 128 rows x 256 columns
         if (te == 64) return launch_ring_wb<DT, 1>(ta, tb, q, s);
         return launch_ring_wb<DT, 2>(ta, tb, q, s);
-    });
+    }, true);
 }
 
 }  // namespace ntg

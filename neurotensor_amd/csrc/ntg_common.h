@@ -74,24 +74,35 @@ struct GemmParams {
     ConvGeom conv;           // used by the implicit-im2col kernels only: B = image, op(B) = col or col^T
 };
 
-// Tile edge (256, 128 or 64) the DMA-fed 16-bit kernel uses for M x N x K x batch.  Larger tiles need less LDS traffic per
-// flop (a CU sustains about 0.5 / 0.4 / 0.25 of its MFMA peak on 256 / 128 / 64-wide tiles at full load, 0.64 on 256-wide
-// tiles while most CUs are idle and the clock is high), smaller ones spread the work over the 256 CUs more evenly,
-// waste less on the padding of M and N, and hide a tile's prologue and epilogue (about 3 / 1.5 / 0.6 us of exposed
-// latency per tile) behind their neighbours on the CU.  Estimated time = tiles per CU x (tile time + exposed latency).
+// Tile the DMA-fed 16-bit kernel uses for M x N x K x batch: square with edge 256, 128 or 64, or (code 192, plain products
+// only) 128 rows x 256 columns.  Larger tiles need less LDS traffic per flop (a CU sustains about 0.5 / 0.5 / 0.4 / 0.25 of
+// its MFMA peak on 256-wide / 128 x 256 / 128-wide / 64-wide tiles at full load, 0.64 / 0.55 on the two largest while
+// most CUs are idle and the clock is high), smaller ones spread the work over the 256 CUs more evenly, waste less on
+// the padding of M and N, and hide a tile's prologue and epilogue (about 3 / 5 / 1.5 / 0.6 us of exposed latency per
+// tile; the 128 x 256 tile has its CU to itself and writes its output in long rows, the 128-wide tiles share a CU in
+// pairs) behind their neighbours on the CU.  Estimated time = tiles per CU x (tile time + exposed latency).
 static inline double ring16_cost_us(int t, int64_t nt, int64_t K) {
     const double cu_flops_per_us = 9.77e6;                      // 2500 TFLOP/s over 256 CUs
-    const double f = t == 256 ? (nt >= 192 ? 0.5 : 0.64) : t == 128 ? 0.4 : 0.25;
-    const double latency = t == 256 ? 3.0 : t == 128 ? 1.5 : 0.6;
-    return (double)((nt + 255) / 256) * (2.0 * t * t * (double)K / (cu_flops_per_us * f) + latency);
+    const double f = t == 256 ? (nt >= 192 ? 0.5 : 0.64) : t == 192 ? (nt >= 192 ? 0.5 : 0.55) : t == 128 ? 0.4 : 0.25;
+    const double latency = t == 256 ? 3.0 : t == 192 ? 5.0 : t == 128 ? 1.5 : 0.6;
+    const double area = t == 192 ? 128.0 * 256.0 : (double)t * t;
+    return (double)((nt + 255) / 256) * (2.0 * area * (double)K / (cu_flops_per_us * f) + latency);
 }
-static inline int64_t ring16_tiles(int t, int64_t M, int64_t N, int64_t batch) { return ((M + t - 1) / t) * ((N + t - 1) / t) * batch; }
-static inline int ring16_tile_edge(int64_t M, int64_t N, int64_t K, int64_t batch) {
+static inline int64_t ring16_tiles(int t, int64_t M, int64_t N, int64_t batch) {
+    if (t == 192) return ((M + 127) / 128) * ((N + 255) / 256) * batch;
+    return ((M + t - 1) / t) * ((N + t - 1) / t) * batch;
+}
+// rect: the 128 x 256 tile is a candidate.  It wins where it fills whole rounds over the CUs and the square tiles do
+// not (2048 x 4096 outputs: 256 tiles against 128 or 512) and K is long enough to carry its latency; over many rounds
+// it was measured slower than the estimate says (2 x 4736 x 5888, K = 8192: 891 us against 816 us on 256-wide tiles),
+// so it has to be 10 % ahead of the 256-wide tile; the smaller tiles then have to beat its estimate as it stands.
+static inline int ring16_tile_edge(int64_t M, int64_t N, int64_t K, int64_t batch, bool rect = false) {
     int best = 256;
     double best_us = 0.0;
-    for (int t = 256; t >= 64; t /= 2) {
+    for (int t : {256, 192, 128, 64}) {
+        if (t == 192 && !rect) continue;
         const double us = ring16_cost_us(t, ring16_tiles(t, M, N, batch), K);
-        if (t == 256 || us < best_us) { best = t; best_us = us; }
+        if (t == 256 || us < (t == 192 ? 0.9 * best_us : best_us)) { best = t; best_us = us; }
     }
     return best;
 }
@@ -101,9 +112,9 @@ static inline int ring16_tile_edge(int64_t M, int64_t N, int64_t K, int64_t batc
 // remaining ones a tile chosen for them alone (usually the next smaller one, spread over all CUs), as two launches; the
 // estimate has to improve by 7 % (the second launch costs a few microseconds).  head == batch: one launch.
 struct Ring16Plan { int edge, head, tail_edge; };
-static inline Ring16Plan ring16_plan(int64_t M, int64_t N, int64_t K, int64_t batch) {
+static inline Ring16Plan ring16_plan(int64_t M, int64_t N, int64_t K, int64_t batch, bool rect = false) {
     Ring16Plan pl;
-    pl.edge = pl.tail_edge = ring16_tile_edge(M, N, K, batch);
+    pl.edge = pl.tail_edge = ring16_tile_edge(M, N, K, batch, rect);
     pl.head = (int)batch;
     if (batch < 2 || pl.edge == 64) return pl;
     const int64_t per_item = ring16_tiles(pl.edge, M, N, 1), total = per_item * batch;
@@ -111,7 +122,7 @@ static inline Ring16Plan ring16_plan(int64_t M, int64_t N, int64_t K, int64_t ba
     if (full < 1 || total % 256 == 0) return pl;
     const int64_t head = full * 256 / per_item;
     if (head < 1 || head >= batch) return pl;
-    const int tail_edge = ring16_tile_edge(M, N, K, batch - head);
+    const int tail_edge = ring16_tile_edge(M, N, K, batch - head, rect);
     const double split_us = ring16_cost_us(pl.edge, per_item * head, K) +
                             ring16_cost_us(tail_edge, ring16_tiles(tail_edge, M, N, batch - head), K) + 2.0;
     if (split_us < 0.93 * ring16_cost_us(pl.edge, total, K)) { pl.head = (int)head; pl.tail_edge = tail_edge; }

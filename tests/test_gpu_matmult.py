@@ -464,9 +464,10 @@ def test_config3_4096_cube(dtype, scale):
                          ids=lambda s: "x".join(map(str, s)))
 def test_ragged_16bit_dma_kernel(dtype, shape):
     """M, N, K that are not multiples of the tile (but keep 16-byte rows) stay on the DMA-fed kernel: edge
-    rows/columns, the k tail (8, 24, none, 8-only) and all three C modes.  The tile edge follows the kernel's cost
-    estimate: 3848 x 4088 (16 x 16 large tiles, one per CU) runs on 256 x 256 tiles, 2056 x 2312 and 2304 x 1928 on
-    128 x 128, the others (short k, or few tiles) on 64 x 64; two shapes are tile-aligned."""
+    rows/columns, the k tail (8, 24, none, 8-only) and all three C modes.  The tile follows the kernel's cost
+    estimate: 3848 x 4088 (16 x 16 large tiles, one per CU) and 4104 x 2056 run on 256 x 256 tiles, 2056 x 2312,
+    1800 x 3080 and 2304 x 1928 on the 128 x 256 tile (one round over the CUs), 3000 x 2056 with k = 40 on 128 x 128,
+    the others (short k, or few tiles) on 64 x 64; two shapes are tile-aligned."""
     m, k, n = shape
     bf = dtype == "bf16"
     rng = np.random.default_rng(1100 + k)
