@@ -533,6 +533,30 @@ def test_batched_16bit_two_launch_plan(dtype, shape):
     assert ((y.float() - refy).abs().max() / refy.abs().max()).item() <= HALF_REL
 
 
+@pytest.mark.parametrize("dtype", ["bf16", np.float16], ids=["bf16", "fp16"])
+@pytest.mark.parametrize("shape", [(2048, 1024, 4096), (2040, 1000, 2312), (1000, 1016, 1720)], ids=lambda s: "x".join(map(str, s)))
+def test_16bit_product_is_the_same_in_every_batch_size(dtype, shape):
+    """A product alone, as every item of a batch of 3 and of a batch of 5: the kernel's cost estimate gives these different
+    tiles (128 x 256 for the single 2048 x 4096 output and for 3 x 1000 x 1720, 256 x 256 or 128 x 128 for the others),
+    and the bits must not depend on that (the reference's batched == per-item rule, tests/src/matmult_test.cpp:108-189).
+    All four transpose forms; the single product also against torch in float."""
+    m, k, n = shape
+    bf = dtype == "bf16"
+    rng = np.random.default_rng(3100 + m)
+    a = to_torch(randn(rng, (m, k), dtype, 0.25), DEV, bf)
+    b = to_torch(randn(rng, (k, n), dtype, 0.25), DEV, bf)
+    ref = torch.matmul(a.float(), b.float())
+    for ta, tb in TRANS:
+        sa = a.t().contiguous() if ta else a
+        sb = b.t().contiguous() if tb else b
+        one = F.matmult(sa, sb, None, ta, tb)
+        assert ((one.float() - ref).abs().max() / ref.abs().max()).item() <= HALF_REL, (shape, ta, tb)
+        for batch in (3, 5):
+            out = F.matmult(sa.expand(batch, *sa.shape).contiguous(), sb.expand(batch, *sb.shape).contiguous(), None, ta, tb)
+            for i in range(batch):
+                assert torch.equal(out[i].view(torch.int16), one.view(torch.int16)), (shape, ta, tb, batch, i)
+
+
 @pytest.mark.parametrize("dtype", [np.float32, np.float64], ids=["fp32", "fp64"])
 @pytest.mark.parametrize("shape", [(1860, 260, 1860), (2052, 1000, 2308), (1028, 132, 516), (68, 20, 4), (132, 16, 260), (130, 22, 66)],
                          ids=lambda s: "x".join(map(str, s)))
