@@ -168,7 +168,7 @@ __device__ __forceinline__ uint32_t lds_addr_of(const char* p) {
 // (convolution: the tap (c, r, q) is uniform, the pixel per lane; weight gradient: the other way round).  Padding taps
 // and columns / k-rows past the edge read a zero word instead, so the tile in LDS is exact and the multiply loop is the
 // plain one.  Wavefront w gathers k-rows 4 w .. 4 w + 3 of every K-step.
-// WBN_ != 0: a rectangular tile, 64 WB_ rows x 64 WBN_ columns (plain products only).
+// WBN_ != 0: a rectangular tile, 64 WB_ rows x 64 WBN_ columns (plain products only; WB_ = 3 only with A stored [m][k]).
 template <int DT, bool TA, bool TB, bool RAGGED, int WB_, int CONV = 0, int WBN_ = 0>
 __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
     using E = Elem<DT>;
@@ -177,6 +177,7 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
     constexpr int WBM = WB_, WBN = WBN_ ? WBN_ : WB_;    // 32 x 32 blocks per wavefront along m / along n
     constexpr int WB = WBN;                              // (the gathered operand is B; gathering kernels have square tiles)
     static_assert(CONV == 0 || WBM == WBN, "gathering kernels have square tiles");
+    static_assert((WBM & (WBM - 1)) == 0 || !TA, "a k-row of a 192-row tile is not a whole number of DMA pieces");
     using GA = RingGeom<WBM, ES>;                        // geometry of the A tile
     using G = RingGeom<WBN, ES>;                         // geometry of the B tile
     constexpr int A_TILE_BYTES = GA::TILE_BYTES, STAGE_BYTES = GA::TILE_BYTES + G::TILE_BYTES;
@@ -911,7 +912,7 @@ static inline GemmParams ring_batch_range(const GemmParams& p, int64_t es, int b
 // 16-bit products: tile edge from the cost estimate; a batch that leaves a small rest of tiles after whole rounds
 // over the CUs goes out as two launches (see ring16_plan).  launch(edge, params) starts one of them.
 template <class Launch>
-static hipError_t launch_ring16_planned(const GemmParams& p, hipStream_t s, Launch&& launch, bool rect = false) {
+static hipError_t launch_ring16_planned(const GemmParams& p, hipStream_t s, Launch&& launch, int rect = RECT_NONE) {
     Ring16Plan pl = ring16_plan(p.M, p.N, p.K, p.batch, rect);
     if (p.cmode == C_PARTIAL || p.Aptr || p.Bptr || p.Cptr) pl.head = p.batch;
     if (pl.head >= p.batch) return launch(pl.edge, p);
@@ -924,10 +925,11 @@ template <int DT>
 static hipError_t launch_ring16(bool ta, bool tb, const GemmParams& p, hipStream_t s) {
     return launch_ring16_planned(p, s, [&](int te, const GemmParams& q) {
         if (te == 256) return launch_ring_wb<DT, 4>(ta, tb, q, s);
+        if (te == 224) return tb ? launch_ring_cfg<DT, false, true, 3, 4>(q, s) : launch_ring_cfg<DT, false, false, 3, 4>(q, s);   // 192 rows x 256 columns
         if (te == 192) return launch_ring_wb<DT, 2, 4>(ta, tb, q, s);      // 128 rows x 256 columns
         if (te == 64) return launch_ring_wb<DT, 1>(ta, tb, q, s);
         return launch_ring_wb<DT, 2>(ta, tb, q, s);
-    }, true);
+    }, ta ? RECT_128 : RECT_128 | RECT_192);
 }
 
 }  // namespace ntg

@@ -74,35 +74,44 @@ struct GemmParams {
     ConvGeom conv;           // used by the implicit-im2col kernels only: B = image, op(B) = col or col^T
 };
 
-// Tile the DMA-fed 16-bit kernel uses for M x N x K x batch: square with edge 256, 128 or 64, or (code 192, plain products
-// only) 128 rows x 256 columns.  Larger tiles need less LDS traffic per flop (a CU sustains about 0.5 / 0.5 / 0.4 / 0.25 of
-// its MFMA peak on 256-wide / 128 x 256 / 128-wide / 64-wide tiles at full load, 0.64 / 0.55 on the two largest while
-// most CUs are idle and the clock is high), smaller ones spread the work over the 256 CUs more evenly, waste less on
-// the padding of M and N, and hide a tile's prologue and epilogue (about 3 / 5 / 1.5 / 0.6 us of exposed latency per
-// tile; the 128 x 256 tile has its CU to itself and writes its output in long rows, the 128-wide tiles share a CU in
-// pairs) behind their neighbours on the CU.  Estimated time = tiles per CU x (tile time + exposed latency).
+// Tile the DMA-fed 16-bit kernel uses for M x N x K x batch: square with edge 256, 128 or 64, or (plain products only)
+// 128 rows x 256 columns (code 192) or 192 rows x 256 columns (code 224; A stored [m][k] only: a k-row of 192 elements is
+// not a whole number of the 1-KiB pieces the DMA writes).  Larger tiles need less LDS traffic per flop (a CU sustains
+// about 0.5 of its MFMA peak on the 256-column tiles, 0.4 / 0.25 on 128-wide / 64-wide ones at full load; 0.64 on
+// 256-wide and 0.55 on the rectangular tiles while most CUs are idle and the clock is high), smaller ones spread the
+// work over the 256 CUs more evenly, waste less on the padding of M and N, and hide a tile's prologue and epilogue
+// (about 3 / 4 / 5 / 1.5 / 0.6 us of exposed latency per tile of 256 x 256 / 192 x 256 / 128 x 256 / 128 x 128 /
+// 64 x 64; the 256-column tiles have their CU to themselves, the 128-wide ones share a CU in pairs) behind their
+// neighbours on the CU.  Estimated time = tiles per CU x (tile time + exposed latency).
+static inline int ring16_tile_rows(int t) { return t == 224 ? 192 : t == 192 ? 128 : t; }
+static inline int ring16_tile_cols(int t) { return t == 224 || t == 192 ? 256 : t; }
 static inline double ring16_cost_us(int t, int64_t nt, int64_t K) {
     const double cu_flops_per_us = 9.77e6;                      // 2500 TFLOP/s over 256 CUs
-    const double f = t == 256 ? (nt >= 192 ? 0.5 : 0.64) : t == 192 ? (nt >= 192 ? 0.5 : 0.55) : t == 128 ? 0.4 : 0.25;
-    const double latency = t == 256 ? 3.0 : t == 192 ? 5.0 : t == 128 ? 1.5 : 0.6;
-    const double area = t == 192 ? 128.0 * 256.0 : (double)t * t;
+    const double f = t == 256 ? (nt >= 192 ? 0.5 : 0.64) : t == 224 || t == 192 ? (nt >= 192 ? 0.5 : 0.55) : t == 128 ? 0.4 : 0.25;
+    const double latency = t == 256 ? 3.0 : t == 224 ? 4.0 : t == 192 ? 5.0 : t == 128 ? 1.5 : 0.6;
+    const double area = (double)ring16_tile_rows(t) * ring16_tile_cols(t);
     return (double)((nt + 255) / 256) * (2.0 * area * (double)K / (cu_flops_per_us * f) + latency);
 }
 static inline int64_t ring16_tiles(int t, int64_t M, int64_t N, int64_t batch) {
-    if (t == 192) return ((M + 127) / 128) * ((N + 255) / 256) * batch;
-    return ((M + t - 1) / t) * ((N + t - 1) / t) * batch;
+    const int r = ring16_tile_rows(t), c = ring16_tile_cols(t);
+    return ((M + r - 1) / r) * ((N + c - 1) / c) * batch;
 }
-// rect: the 128 x 256 tile is a candidate.  It wins where it fills whole rounds over the CUs and the square tiles do
-// not (2048 x 4096 outputs: 256 tiles against 128 or 512) and K is long enough to carry its latency; over many rounds
-// it was measured slower than the estimate says (2 x 4736 x 5888, K = 8192: 891 us against 816 us on 256-wide tiles),
-// so it has to be 10 % ahead of the 256-wide tile; the smaller tiles then have to beat its estimate as it stands.
-static inline int ring16_tile_edge(int64_t M, int64_t N, int64_t K, int64_t batch, bool rect = false) {
+// rect: which rectangular tiles are candidates (RECT_128 | RECT_192).  They win where they fill whole rounds over the
+// CUs better than the square tiles (3072 x 3072 outputs: 192 tiles of 192 x 256 against 144 of 256 x 256; 2048 x 4096:
+// 256 tiles of 128 x 256 against 128 or 512) and K is long enough to carry their latency.  Over many rounds the
+// 128 x 256 tile was measured slower than the estimate says (2 x 4736 x 5888, K = 8192: 891 us against 816 us on
+// 256-wide tiles), so it has to be 10 % ahead of the larger tiles, and the 192 x 256 tile 5 % ahead of the 256-wide one
+// where that one has more than two rounds (12 x 968 x 4136, K = 2048: 244 us against 216 us at estimates of 226 and
+// 232); the smaller tiles then have to beat the chosen estimate as it stands.
+enum { RECT_NONE = 0, RECT_128 = 1, RECT_192 = 2 };
+static inline int ring16_tile_edge(int64_t M, int64_t N, int64_t K, int64_t batch, int rect = RECT_NONE) {
     int best = 256;
     double best_us = 0.0;
-    for (int t : {256, 192, 128, 64}) {
-        if (t == 192 && !rect) continue;
+    for (int t : {256, 224, 192, 128, 64}) {
+        if ((t == 224 && !(rect & RECT_192)) || (t == 192 && !(rect & RECT_128))) continue;
         const double us = ring16_cost_us(t, ring16_tiles(t, M, N, batch), K);
-        if (t == 256 || us < (t == 192 ? 0.9 * best_us : best_us)) { best = t; best_us = us; }
+        const double margin = t == 192 ? 0.9 : t == 224 && ring16_tiles(256, M, N, batch) > 512 ? 0.95 : 1.0;
+        if (t == 256 || us < margin * best_us) { best = t; best_us = us; }
     }
     return best;
 }
@@ -112,7 +121,7 @@ static inline int ring16_tile_edge(int64_t M, int64_t N, int64_t K, int64_t batc
 // remaining ones a tile chosen for them alone (usually the next smaller one, spread over all CUs), as two launches; the
 // estimate has to improve by 7 % (the second launch costs a few microseconds).  head == batch: one launch.
 struct Ring16Plan { int edge, head, tail_edge; };
-static inline Ring16Plan ring16_plan(int64_t M, int64_t N, int64_t K, int64_t batch, bool rect = false) {
+static inline Ring16Plan ring16_plan(int64_t M, int64_t N, int64_t K, int64_t batch, int rect = RECT_NONE) {
     Ring16Plan pl;
     pl.edge = pl.tail_edge = ring16_tile_edge(M, N, K, batch, rect);
     pl.head = (int)batch;
