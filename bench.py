@@ -208,6 +208,8 @@ def main():
         f2k = 2.0 * 2048 ** 3
         run("mid_bf16_2048", make_gemm(torch.bfloat16, 2048, 2048, 2048, scale=0.05, mode=_lib.C_OVERWRITE), f2k, PEAK_TFLOPS["bf16"], st=steps * 4)
         run("mid_fp32_2048", make_gemm(torch.float32, 2048, 2048, 2048, mode=_lib.C_OVERWRITE), f2k, PEAK_TFLOPS["fp32"], st=steps * 2)
+        # 192 tiles of 192 x 256 (144 of 256 x 256)
+        run("mid_bf16_3072", make_gemm(torch.bfloat16, 3072, 3072, 3072, scale=0.05, mode=_lib.C_OVERWRITE), 2.0 * 3072 ** 3, PEAK_TFLOPS["bf16"], st=steps * 2)
         # one round of 256 tiles of 128 x 256 (the square tiles give 128 or 512)
         run("mid_bf16_2048x4096x4096", make_gemm(torch.bfloat16, 2048, 4096, 4096, scale=0.05, mode=_lib.C_OVERWRITE), 2.0 * 2048 * 4096 * 4096,
             PEAK_TFLOPS["bf16"], st=steps * 2)
