@@ -91,7 +91,7 @@ struct RingGeom {
 // WB DMA instructions into one operand tile.  Instruction j = WB*wave + jj fills LDS bytes
 // [1024 j, 1024 j + 1024) of the tile:
 //   K-contiguous operand: rows 16 j + lane/4, 16-byte slot lane%4 holds kv = slot ^ ((row>>1)&3)
-//   MN-contiguous operand (CH chunks per k-row): k-rows (64/CH) j + lane/CH, slot lane%CH holds
+//   MN-contiguous operand (CH chunks per k-row): piece 64 j + lane of the tile = k-row (64 j + lane) / CH, slot (64 j + lane) % CH, holds
 //                          chunk = slot ^ (2*(krow&3)) for 16-bit elements (what the transposing
 //                          reads need), slot ^ mn8_swizzle(krow) for 8-bit elements,
 //                          slot ^ (8*((krow>>2)&1)) for Float32 (the two k-rows that one
@@ -121,8 +121,9 @@ __device__ __forceinline__ void dma_offsets(uint32_t (&off)[WB], int64_t ld, int
             }
             off[jj] = (uint32_t)(((int64_t)row * ld + kv * VEL) * ES);
         } else {
-            int krow = (64 / CH) * j + lane / CH;
-            int chunk = (lane % CH) ^ (ES == 2 ? 2 * (krow & 3) : ES == 4 ? 8 * ((krow >> 2) & 1) : ES == 1 ? mn8_swizzle<CH>(krow) : 0);   // Float64: stored as is
+            // (CH = 24, the 192-row tile: three instructions fill eight k-rows, a k-row may begin inside an instruction)
+            int krow = (64 * j + lane) / CH;
+            int chunk = ((64 * j + lane) % CH) ^ (ES == 2 ? 2 * (krow & 3) : ES == 4 ? 8 * ((krow >> 2) & 1) : ES == 1 ? mn8_swizzle<CH>(krow) : 0);   // Float64: stored as is
             if constexpr (RAGGED) {
                 krow = krow < k_valid ? krow : k_valid - 1;
                 chunk = chunk < mn_valid / VEL ? chunk : mn_valid / VEL - 1;
@@ -168,7 +169,7 @@ __device__ __forceinline__ uint32_t lds_addr_of(const char* p) {
 // (convolution: the tap (c, r, q) is uniform, the pixel per lane; weight gradient: the other way round).  Padding taps
 // and columns / k-rows past the edge read a zero word instead, so the tile in LDS is exact and the multiply loop is the
 // plain one.  Wavefront w gathers k-rows 4 w .. 4 w + 3 of every K-step.
-// WBN_ != 0: a rectangular tile, 64 WB_ rows x 64 WBN_ columns (plain products only; WB_ = 3 only with A stored [m][k]).
+// WBN_ != 0: a rectangular tile, 64 WB_ rows x 64 WBN_ columns (plain products only).
 template <int DT, bool TA, bool TB, bool RAGGED, int WB_, int CONV = 0, int WBN_ = 0>
 __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
     using E = Elem<DT>;
@@ -177,7 +178,6 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
     constexpr int WBM = WB_, WBN = WBN_ ? WBN_ : WB_;    // 32 x 32 blocks per wavefront along m / along n
     constexpr int WB = WBN;                              // (the gathered operand is B; gathering kernels have square tiles)
     static_assert(CONV == 0 || WBM == WBN, "gathering kernels have square tiles");
-    static_assert((WBM & (WBM - 1)) == 0 || !TA, "a k-row of a 192-row tile is not a whole number of DMA pieces");
     using GA = RingGeom<WBM, ES>;                        // geometry of the A tile
     using G = RingGeom<WBN, ES>;                         // geometry of the B tile
     constexpr int A_TILE_BYTES = GA::TILE_BYTES, STAGE_BYTES = GA::TILE_BYTES + G::TILE_BYTES;
@@ -925,11 +925,11 @@ template <int DT>
 static hipError_t launch_ring16(bool ta, bool tb, const GemmParams& p, hipStream_t s) {
     return launch_ring16_planned(p, s, [&](int te, const GemmParams& q) {
         if (te == 256) return launch_ring_wb<DT, 4>(ta, tb, q, s);
-        if (te == 224) return tb ? launch_ring_cfg<DT, false, true, 3, 4>(q, s) : launch_ring_cfg<DT, false, false, 3, 4>(q, s);   // 192 rows x 256 columns
+        if (te == 224) return launch_ring_wb<DT, 3, 4>(ta, tb, q, s);      // 192 rows x 256 columns
         if (te == 192) return launch_ring_wb<DT, 2, 4>(ta, tb, q, s);      // 128 rows x 256 columns
         if (te == 64) return launch_ring_wb<DT, 1>(ta, tb, q, s);
         return launch_ring_wb<DT, 2>(ta, tb, q, s);
-    }, ta ? RECT_128 : RECT_128 | RECT_192);
+    }, RECT_128 | RECT_192);
 }
 
 }  // namespace ntg

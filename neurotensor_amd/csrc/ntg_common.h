@@ -75,8 +75,7 @@ struct GemmParams {
 };
 
 // Tile the DMA-fed 16-bit kernel uses for M x N x K x batch: square with edge 256, 128 or 64, or (plain products only)
-// 128 rows x 256 columns (code 192) or 192 rows x 256 columns (code 224; A stored [m][k] only: a k-row of 192 elements is
-// not a whole number of the 1-KiB pieces the DMA writes).  Larger tiles need less LDS traffic per flop (a CU sustains
+// 128 rows x 256 columns (code 192) or 192 rows x 256 columns (code 224).  Larger tiles need less LDS traffic per flop (a CU sustains
 // about 0.5 of its MFMA peak on the 256-column tiles, 0.4 / 0.25 on 128-wide / 64-wide ones at full load; 0.64 on
 // 256-wide and 0.55 on the rectangular tiles while most CUs are idle and the clock is high), smaller ones spread the
 // work over the 256 CUs more evenly, waste less on the padding of M and N, and hide a tile's prologue and epilogue

@@ -467,8 +467,8 @@ def test_ragged_16bit_dma_kernel(dtype, shape):
     """M, N, K that are not multiples of the tile (but keep 16-byte rows) stay on the DMA-fed kernel: edge
     rows/columns, the k tail (8, 24, none, 8-only) and all three C modes.  The tile follows the kernel's cost
     estimate: 3848 x 4088 (16 x 16 large tiles, one per CU) and 4104 x 2056 run on 256 x 256 tiles, 2056 x 2312,
-    1800 x 3080 and 2304 x 1928 on the 128 x 256 tile (one round over the CUs), 3000 x 4000 on the 192 x 256 tile where
-    A is stored [m][k] (16 x 16 tiles; 128 x 128 otherwise), 3000 x 2056 with k = 40 on 128 x 128, the others (short k,
+    1800 x 3080 and 2304 x 1928 on the 128 x 256 tile (one round over the CUs), 3000 x 4000 on the 192 x 256 tile
+    (16 x 16 tiles), 3000 x 2056 with k = 40 on 128 x 128, the others (short k,
     or few tiles) on 64 x 64; two shapes are tile-aligned."""
     m, k, n = shape
     bf = dtype == "bf16"
@@ -541,7 +541,7 @@ def test_batched_16bit_two_launch_plan(dtype, shape):
 def test_16bit_product_is_the_same_in_every_batch_size(dtype, shape):
     """A product alone, as every item of a batch of 3 and of a batch of 5: the kernel's cost estimate gives these different
     tiles (128 x 256 for the single 2048 x 4096 output and for 3 x 1000 x 1720, 192 x 256 for 3000 x 4000 and for batches of
-    1800 x 3080 where A is stored [m][k], 256 x 256 or 128 x 128 for the others),
+    1800 x 3080, 256 x 256 or 128 x 128 for the others),
     and the bits must not depend on that (the reference's batched == per-item rule, tests/src/matmult_test.cpp:108-189).
     All four transpose forms; the single product also against torch in float."""
     m, k, n = shape
