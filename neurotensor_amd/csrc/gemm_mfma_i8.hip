@@ -10,8 +10,11 @@ hipError_t launch_gemm_mfma_i8(int dtype, bool ta, bool tb, const GemmParams& p,
         if (p.cmode == C_PARTIAL) return hipErrorInvalidValue;      // (only the DMA-fed kernel writes 32-bit sums)
         return launch_gemm_valu(dtype, ta, tb, p, s);
     }
-    const int te = ring16_tile_edge(p.M, p.N, p.K, p.batch);
+    // (an MN-major 192-row tile of bytes has 12 chunks per k-row, which the chunk swizzle of the transposing reads does not fit)
+    const int te = ring16_tile_edge(p.M, p.N, p.K, p.batch, ta ? RECT_128 : RECT_128 | RECT_192);
     if (te == 256) return launch_ring_wb<DT_I8, 4>(ta, tb, p, s);
+    if (te == 224) return tb ? launch_ring_cfg<DT_I8, false, true, 3, 4>(p, s) : launch_ring_cfg<DT_I8, false, false, 3, 4>(p, s);
+    if (te == 192) return launch_ring_wb<DT_I8, 2, 4>(ta, tb, p, s);
     if (te == 64) return launch_ring_wb<DT_I8, 1>(ta, tb, p, s);
     return launch_ring_wb<DT_I8, 2>(ta, tb, p, s);
 }
