@@ -175,6 +175,19 @@ int ntg_matmult_dev(int dtype, const void* dA, const void* dB, void* dC,
  * (matmult_cpu.cpp:863-1005) lower to when the views are affine. */
 int ntg_gemm_dev(const ntg_gemm_desc* desc, const void* dA, const void* dB, void* dC, void* stream);
 
+/* ntg_gemm_dev for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc): it has NO counterpart in the reference.  Same arguments, results bit-identical to
+ * ntg_gemm_dev called with a workspace of ntg_gemm_workspace_bytes(desc) bytes; desc->workspace and desc->workspace_bytes
+ * are ignored.  The split along k and the byte-plane products of the wide integers keep their partial sums in a fixed
+ * array of NTG_NOALLOC_SCRATCH_BYTES bytes that is part of the library's device code (every GPU the library runs on holds
+ * its copy until the process ends); the call itself allocates and frees nothing.  A product whose workspace form needs
+ * more than that is rejected with NTG_ERR_INVALID_ARGUMENT (use ntg_gemm_dev with your own workspace).  All calls on one
+ * GPU share the array: calls that may overlap on one GPU (different streams, different threads) race; calls on one
+ * stream are ordered and safe.  The first call on a device looks the array's address up (hipGetSymbolAddress): make
+ * that call before a stream capture begins. */
+#define NTG_NOALLOC_SCRATCH_BYTES (64ll << 20)
+int ntg_gemm_noalloc_dev(const ntg_gemm_desc* desc, const void* dA, const void* dB, void* dC, void* stream);
+
 /* nt_matmult_batch<T> with the pointer tables themselves in device memory. */
 int ntg_gemm_ptrs_dev(const ntg_gemm_desc* desc, const void* const* dA, const void* const* dB,
                       void* const* dC, void* stream);

@@ -10,6 +10,7 @@
 #include <algorithm>
 #include <cstring>
 #include <map>
+#include <mutex>
 #include <string>
 #include <vector>
 
@@ -58,6 +59,11 @@ hipError_t launch_conv_mfma(int dtype, bool tb, int nd, const GemmParams& p, hip
     }
 }
 }  // namespace ntg
+
+// Scratch memory of ntg_gemm_noalloc_dev: a fixed array in every GPU's copy of this code object, so that the entry point
+// needs no allocator.  Host code never uses the array's name as an address: ntg::noalloc_scratch_of_current_device() asks the runtime
+// for the address of the current device's copy once and keeps it.
+static __device__ __align__(256) unsigned char scratch[NTG_NOALLOC_SCRATCH_BYTES];
 
 namespace {
 
@@ -343,6 +349,29 @@ int desc_to_params(const ntg_gemm_desc* d, ntg::GemmParams& p) {
 
 }  // namespace
 
+// Device address of `scratch` on the current device (each GPU holds its own copy at its own address), looked up on the
+// first call per device.  The function has external linkage on purpose: the compiler gives a file-scope static device
+// variable a symbol the runtime can look up only when a host function with external linkage refers to it.
+namespace ntg {
+int noalloc_scratch_of_current_device(void** out) {
+    constexpr int kMaxDevices = 64;
+    static std::mutex mutex;
+    static void* ptrs[kMaxDevices];
+    int dev = -1;
+    HIP_TRY(hipGetDevice(&dev));
+    if (dev < 0 || dev >= kMaxDevices) return fail(NTG_ERR_DEVICE, "device ordinal %d outside 0..%d", dev, kMaxDevices - 1);
+    std::lock_guard<std::mutex> lock(mutex);
+    if (!ptrs[dev]) {
+        void* ptr = nullptr;
+        HIP_TRY(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+        if (!ptr) return fail(NTG_ERR_DEVICE, "hipGetSymbolAddress returned a null address for the static scratch");
+        ptrs[dev] = ptr;
+    }
+    *out = ptrs[dev];
+    return NTG_OK;
+}
+}  // namespace ntg
+
 extern "C" {
 
 const char* ntg_last_error(void) { return g_last_error.c_str(); }
@@ -375,6 +404,27 @@ int64_t ntg_gemm_workspace_bytes(const ntg_gemm_desc* d) {
         return ip.ok ? ip.bytes() : 0;
     }
     return plan_splitk(p, d->dtype, d->transpose_a != 0).bytes;      // pointers taken as 16-byte aligned
+}
+
+int ntg_gemm_noalloc_dev(const ntg_gemm_desc* d, const void* dA, const void* dB, void* dC, void* stream) {
+    ntg::GemmParams p;
+    int rc = desc_to_params(d, p);
+    if (rc) return rc;
+    if (p.M == 0 || p.N == 0 || p.batch == 0) return NTG_OK;
+    if (!dA || !dB || !dC) return fail(NTG_ERR_INVALID_ARGUMENT, "null matrix pointer");
+    if (p.batch > 1 && p.sC == 0) return fail(NTG_ERR_INVALID_ARGUMENT, "stride_c must be non-zero for a batch (outputs may not alias)");
+    const int64_t need = ntg_gemm_workspace_bytes(d);
+    if (need < 0) return fail(NTG_ERR_INVALID_ARGUMENT, "bad descriptor");
+    if (need > (int64_t)NTG_NOALLOC_SCRATCH_BYTES)
+        return fail(NTG_ERR_INVALID_ARGUMENT, "this product's workspace form needs %lld bytes, the static scratch of ntg_gemm_noalloc_dev holds %lld: "
+                    "call ntg_gemm_dev with a workspace of the caller's", (long long)need, (long long)NTG_NOALLOC_SCRATCH_BYTES);
+    void* ws = nullptr;
+    if (need > 0) {
+        rc = ntg::noalloc_scratch_of_current_device(&ws);
+        if (rc) return rc;
+    }
+    p.A = dA; p.B = dB; p.C = dC;
+    return run_gemm(p, d->dtype, d->transpose_a != 0, d->transpose_b != 0, static_cast<hipStream_t>(stream), ws, need);
 }
 
 int ntg_gemm_ptrs_dev(const ntg_gemm_desc* d, const void* const* dA, const void* const* dB, void* const* dC, void* stream) {
