@@ -107,13 +107,19 @@ def test_config4_linear_training_step(dtype):
     check(y, x, w, False, True, rows, cols, K)                    # Y  = X . W^T
     check(dx, gy, w, False, False, rows, np.r_[0:24, 4072:4096], N)   # dX = dY . W
     check(dw, gy, x, True, False, np.r_[0:24, 10984:11008], np.r_[0:24, 4072:4096], M)   # dW = dY^T . X
-    # whole-matrix cross-check with an independent GEMM
-    if not bf:
-        ref = torch.matmul(tx.double(), tw.double().t())
-        assert (y.double() - ref).abs().max().item() <= 1e-5 * K * tx.abs().max().item() * tw.abs().max().item()
-    else:
-        ref = torch.matmul(tx.float(), tw.float().t())
-        assert ((y.float() - ref).abs().max() / ref.abs().max()).item() <= HALF_REL
+    # whole-matrix cross-check of all three products with an independent GEMM (double for Float32, float for BFloat16)
+    def whole(got, lhs, rhs, kk):
+        if not bf:
+            ref = torch.matmul(lhs.double(), rhs.double())
+            assert (got.double() - ref).abs().max().item() <= 1e-5 * kk * lhs.abs().max().item() * rhs.abs().max().item()
+        else:
+            ref = torch.matmul(lhs.float(), rhs.float())
+            assert ((got.float() - ref).abs().max() / ref.abs().max()).item() <= HALF_REL
+        del ref
+
+    whole(y, tx, tw.t(), K)            # Y  = X . W^T
+    whole(dx, tg, tw, N)               # dX = dY . W
+    whole(dw, tg.t(), tx, M)           # dW = dY^T . X
 
 
 def test_unfold_golden_and_random(golden_dir):

@@ -204,16 +204,40 @@ def test_f16_ktile_rounding_schedule():
 
 
 def test_bf16_definition():
+    """BFloat16 has no counterpart in the reference; this build defines it as: bf16 operands, one float32 fma chain over
+    all of K starting from C0, ONE round-to-nearest-even at the end.  Pinned against RNE_bf16(float64 GEMM): products of
+    two bf16 values are exact in float32, so the chain's only error is the float32 accumulation, and the result must be
+    bit-equal to RNE(exact) wherever the exact value is further from a rounding boundary than that error, and within one
+    bf16 ulp everywhere.  A wrong rounding point (truncation, rounding per k-tile, double rounding through another
+    format) fails this."""
+    from util import assert_one_rounding
     r = rng(11)
-    m, k, n = 7, 100, 9
-    a = oracle.to_bf16_bits(r.standard_normal((m, k)).astype(np.float32))
-    b = oracle.to_bf16_bits(r.standard_normal((k, n)).astype(np.float32))
-    got = oracle.matmult2d(a, b, dt=oracle.BF16)
-    ref = oracle.from_bf16_bits(a).astype(np.float64) @ oracle.from_bf16_bits(b).astype(np.float64)
-    g = oracle.from_bf16_bits(got).astype(np.float64)
-    assert np.abs(g - ref).max() <= 2e-2 * np.abs(ref).max()
-    got_n = oracle.matmult2d(a, b, dt=oracle.BF16, kind="naive")
-    assert got.tobytes() == got_n.tobytes()
+    for (m, k, n, with_c0, ta, tb) in [(7, 100, 9, False, False, False), (33, 257, 40, True, False, True), (16, 1001, 24, True, True, False),
+                                       (5, 8, 3, True, True, True), (64, 515, 17, False, False, False)]:
+        a = oracle.to_bf16_bits(r.standard_normal((m, k)).astype(np.float32))
+        b = oracle.to_bf16_bits(r.standard_normal((k, n)).astype(np.float32))
+        c0 = oracle.to_bf16_bits((r.standard_normal((m, n)) * (4.0 if with_c0 else 0.0)).astype(np.float32))
+        sa = np.ascontiguousarray(a.T) if ta else a
+        sb = np.ascontiguousarray(b.T) if tb else b
+        got = oracle.matmult2d(sa, sb, c0.copy(), ta, tb, dt=oracle.BF16)
+        a64, b64, c64 = (oracle.from_bf16_bits(x).astype(np.float64) for x in (a, b, c0))
+        ref = c64 + a64 @ b64
+        mag = np.abs(c64) + np.sqrt((a64 * a64) @ (b64 * b64))
+        assert_one_rounding(oracle.from_bf16_bits(got).astype(np.float64), ref, mag, k, "bf16", f"bf16 oracle {m}x{k}x{n}")
+        got_n = oracle.matmult2d(sa, sb, c0.copy(), ta, tb, dt=oracle.BF16, kind="naive")
+        assert got.tobytes() == got_n.tobytes()
+    # the check has teeth: truncating instead of rounding, or rounding every 16 k, fails it
+    a64, b64 = oracle.from_bf16_bits(a).astype(np.float64), oracle.from_bf16_bits(b).astype(np.float64)
+    ref = a64 @ b64
+    mag = np.sqrt((a64 * a64) @ (b64 * b64))
+    trunc = ((ref.astype(np.float32).view(np.uint32) >> 16).astype(np.uint16))
+    with pytest.raises(AssertionError):
+        assert_one_rounding(oracle.from_bf16_bits(trunc).astype(np.float64), ref, mag, k, "bf16")
+    acc = np.zeros((m, n), np.float64)
+    for k0 in range(0, k, 16):
+        acc = oracle.from_bf16_bits(oracle.to_bf16_bits((acc + a64[:, k0:k0 + 16] @ b64[k0:k0 + 16]).astype(np.float32))).astype(np.float64)
+    with pytest.raises(AssertionError):
+        assert_one_rounding(acc, ref, mag, k, "bf16")
 
 
 def test_batched_equals_per_item_and_broadcast():
