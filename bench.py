@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the matmult hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-extras] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-extras] [--no-cpu] [--only NAME[,NAME...]]
 
 One "step" is one pass of nt::matmult over the headline workload of BASELINE.json
 (config 3): a 4096 x 4096 x 4096 BFloat16 product, inputs randn*0.02 already resident in
@@ -14,7 +14,12 @@ Besides the headline value the line carries
   roofline      achieved vs. MI355X dense-MFMA peak for the dominant kernel,
   cpu_baseline  the CPU oracle's tiled restatement of the reference's TBB/SIMD GEMM, timed
                 on this host's cores on a bounded sample (reported, not a target),
-  extras        the other dtypes at 4096^3 and the remaining BASELINE configurations.
+  extras        the other dtypes at 4096^3 and the remaining BASELINE configurations; every entry is timed after the
+                same settling load as the headline (see settle()), so the figures do not depend on --warmup.
+
+--only NAME[,NAME...] times just those extras entries (for one rocprofv3 run per workload); the settling load is a
+different kernel instantiation than the workload, so a kernel-trace summary of such a run averages the workload's
+kernels over its --warmup + timed launches only.
 """
 import argparse
 import ctypes
@@ -40,6 +45,7 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--no-extras", action="store_true", help="only the headline workload")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--only", default="", help="comma-separated extras entries to time alone (skips the headline and the CPU leg)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 256 MiB device copy (known HBM traffic) so that counter runs "
                          "(rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE) can be scaled")
@@ -134,113 +140,190 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
-    # ---------------- headline: config 3, BFloat16 4096^3, C += A.B ----------------
     N = 4096
     flops = 2.0 * N * N * N
-    head = make_gemm(torch.bfloat16, N, N, N, scale=0.02)
-    # Coming from idle the GPU runs its first 20-30 ms of work at lower clocks.  A measuring run (20 or more timed steps)
-    # therefore brings the untimed launches ahead of the timed region up to 300, whatever --warmup says; the timed region
-    # itself is exactly --steps launches.  Counter-collection runs (a handful of steps) skip this.
-    settle = max(0, 300 - args.warmup) if args.steps >= 20 else 0
-    for _ in range(settle):
-        head()
-    wall_ms, ev_ms = time_steps(head, args.steps, args.warmup)
-    value = flops / (wall_ms * 1e-3) / 1e12
-    achieved = flops / (ev_ms * 1e-3) / 1e12
+    only = [x for x in args.only.split(",") if x]
 
-    out = {
-        "metric": "matmult TFLOP/s at 4096^3 (BFloat16, fp32 accumulate)",
-        "value": round(value, 2),
-        "unit": "TFLOP/s",
-        "n_gpus": 1,
-        "steps": args.steps,
-        "warmup": args.warmup,
-        "ms_per_step": round(wall_ms, 5),
-        "higher_is_better": True,
-        "scaling": "weak",
-        "vs_baseline": None,
-        "dtype": "bf16",
-        "data": "synthetic",
-        "config": {"workload": "nt::matmult A[4096,4096].B[4096,4096] BFloat16, inputs randn*0.02 resident in HBM, "
-                               "C += A.B (BASELINE config 3)", "m": N, "k": N, "n": N, "c_mode": "accumulate",
-                   "untimed_launches_before_timed_region": settle + args.warmup},
-        "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_TFLOPS["bf16"], "unit": "TFLOP/s",
-                     "frac": round(achieved / PEAK_TFLOPS["bf16"], 4), "traffic": read_traffic_note(),
-                     "kernel": "ntg::gemm_ring_kernel<BFloat16, NN>", "launch_ms": round(ev_ms, 5)},
-    }
+    # Coming from idle the GPU runs its first 20-30 ms of work at lower clocks.  Every measurement (20 or more timed steps)
+    # is therefore preceded by SETTLE_MS of back-to-back 4096^3 16-bit products -- the Float16 instantiation for every
+    # workload but the Float16 one, which gets the BFloat16 instantiation: a load of the same kind under another kernel
+    # name, so that a kernel-trace summary of the run averages the measured kernel over its own launches only.  The
+    # workload's --warmup launches and its timed launches follow without a gap.  Counter-collection runs (a handful of
+    # steps) skip the load.
+    SETTLE_MS = 40.0
+    settle_f16 = make_gemm(torch.float16, N, N, N, scale=0.02, mode=_lib.C_OVERWRITE)
+    settle_bf16 = make_gemm(torch.bfloat16, N, N, N, scale=0.02, mode=_lib.C_OVERWRITE)
+    settled_launches = {}
+
+    def settle(name, load=None):
+        if args.steps < 20:
+            return
+        load = load or settle_f16
+        n = int(SETTLE_MS / 0.105) + 1
+        for _ in range(n):
+            load()
+        settled_launches[name] = n
+
+    out = {}
+    extras = {}
+    if not only:
+        # the driver's protocol from a cold start: what --steps / --warmup alone read, first thing after start-up (the
+        # two launches before the pause load the code object; the pause lets the clocks fall back to idle)
+        head = make_gemm(torch.bfloat16, N, N, N, scale=0.02)
+        head(); head()
+        torch.cuda.synchronize()
+        time.sleep(0.5)
+        _, cold_ms = time_steps(head, args.steps, args.warmup)
+        extras["c3_bf16_4096_cold"] = {"ms": round(cold_ms, 5), "rate": round(flops / (cold_ms * 1e-3) / 1e12, 2), "unit": "TFLOP/s",
+                                       "frac_of_peak": round(flops / (cold_ms * 1e-3) / 1e12 / PEAK_TFLOPS["bf16"], 4),
+                                       "note": f"the headline workload from an idle GPU: {args.warmup} warm-up launches, no settling load"}
+
+        # ---------------- headline: config 3, BFloat16 4096^3, C += A.B ----------------
+        settle("headline")
+        wall_ms, ev_ms = time_steps(head, args.steps, args.warmup)
+        value = flops / (wall_ms * 1e-3) / 1e12
+        achieved = flops / (ev_ms * 1e-3) / 1e12
+
+        out = {
+            "metric": "matmult TFLOP/s at 4096^3 (BFloat16, fp32 accumulate)",
+            "value": round(value, 2),
+            "unit": "TFLOP/s",
+            "n_gpus": 1,
+            "steps": args.steps,
+            "warmup": args.warmup,
+            "ms_per_step": round(wall_ms, 5),
+            "higher_is_better": True,
+            "scaling": "weak",
+            "vs_baseline": None,
+            "dtype": "bf16",
+            "data": "synthetic",
+            "config": {"workload": "nt::matmult A[4096,4096].B[4096,4096] BFloat16, inputs randn*0.02 resident in HBM, "
+                                   "C += A.B (BASELINE config 3)", "m": N, "k": N, "n": N, "c_mode": "accumulate",
+                       "untimed_launches_before_timed_region": settled_launches.get("headline", 0) + args.warmup,
+                       "settling_load": f"{settled_launches.get('headline', 0)} launches of the Float16 4096^3 product (about {SETTLE_MS:.0f} ms) "
+                                        "before the warm-up launches of every timed workload"},
+            "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_TFLOPS["bf16"], "unit": "TFLOP/s",
+                         "frac": round(achieved / PEAK_TFLOPS["bf16"], 4), "traffic": read_traffic_note(),
+                         "traffic_source": "profiles/gemm_ring_bf16_4096_hbm_traffic.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, not measured in this run)",
+                         "kernel": "ntg::gemm_ring_kernel<BFloat16, NN>", "launch_ms": round(ev_ms, 5)},
+        }
+        del head
 
     # ---------------- extras: the other dtypes and configurations ----------------
-    if not args.no_extras:
-        extras = {}
-        steps, warm = max(5, args.steps // 5), max(2, args.warmup // 3)
+    if not args.no_extras or only:
+        steps, warm = max(20, args.steps), max(5, args.warmup)
 
-        def run(name, fn, work, peak=None, unit="TFLOP/s", scale=1e12, st=steps):
+        def run(name, make, work, peak=None, unit="TFLOP/s", scale=1e12, load=None):
+            """make() builds the workload (its buffers live only while it is timed); timed over at least `steps`
+            launches and about 10 ms, after the settling load and `warm` warm-up launches"""
+            if only and name not in only:
+                return
+            fn = make()
+            fn(); fn()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            fn()
+            torch.cuda.synchronize()
+            est_ms = max((time.perf_counter() - t0) * 1e3, 1e-3)
+            st = int(min(max(steps, 10.0 / est_ms), 1000))
+            settle(name, load)
             _, ms = time_steps(fn, st, warm)
             rate = work / (ms * 1e-3) / scale
-            e = {"ms": round(ms, 5), "rate": round(rate, 2), "unit": unit}
+            e = {"ms": round(ms, 5), "rate": round(rate, 2), "unit": unit, "timed_launches": st}
             if peak:
                 e["frac_of_peak"] = round(rate / peak, 4)
             extras[name] = e
+            del fn
 
-        run("c3_fp16_4096", make_gemm(torch.float16, N, N, N, scale=0.02), flops, PEAK_TFLOPS["fp16"])
-        run("c3_bf16_4096_overwrite", make_gemm(torch.bfloat16, N, N, N, scale=0.02, mode=_lib.C_OVERWRITE), flops, PEAK_TFLOPS["bf16"])
-        run("c3_fp32_4096", make_gemm(torch.float32, N, N, N), flops, PEAK_TFLOPS["fp32"])
-        run("c3_fp64_4096", make_gemm(torch.float64, N, N, N), flops, PEAK_TFLOPS["fp64"])
-        run("c1_fp32_512", make_gemm(torch.float32, 512, 512, 512), 2.0 * 512 ** 3, PEAK_TFLOPS["fp32"], st=steps * 4)
+        G = lambda *a, **k: (lambda: make_gemm(*a, **k))
+        run("c3_fp16_4096", G(torch.float16, N, N, N, scale=0.02), flops, PEAK_TFLOPS["fp16"], load=settle_bf16)
+        run("c3_bf16_4096_overwrite", G(torch.bfloat16, N, N, N, scale=0.02, mode=_lib.C_OVERWRITE), flops, PEAK_TFLOPS["bf16"])
+        run("c3_fp32_4096", G(torch.float32, N, N, N), flops, PEAK_TFLOPS["fp32"])
+        run("c3_fp64_4096", G(torch.float64, N, N, N), flops, PEAK_TFLOPS["fp64"])
+        run("c1_fp32_512", G(torch.float32, 512, 512, 512), 2.0 * 512 ** 3, PEAK_TFLOPS["fp32"])
         f2 = 2.0 * 32 * 1024 * 768 * 1024
-        run("c2a_fp32_b32_1024x768x1024", make_gemm(torch.float32, 1024, 768, 1024, batch=32), f2, PEAK_TFLOPS["fp32"])
-        run("c2b_fp32_b32_transpose_b", make_gemm(torch.float32, 1024, 768, 1024, tb=True, batch=32), f2, PEAK_TFLOPS["fp32"])
-        run("c2c_int32_b8_1024", make_gemm(torch.int32, 1024, 1024, 1024, batch=8, ints=True), 2.0 * 8 * 1024 ** 3, None, "Top/s")
-        run("c3_int8_4096", make_gemm(torch.int8, N, N, N, ints=True, mode=_lib.C_OVERWRITE), flops, PEAK_TFLOPS["int8"], "Top/s")
+        run("c2a_fp32_b32_1024x768x1024", G(torch.float32, 1024, 768, 1024, batch=32), f2, PEAK_TFLOPS["fp32"])
+        run("c2b_fp32_b32_transpose_b", G(torch.float32, 1024, 768, 1024, tb=True, batch=32), f2, PEAK_TFLOPS["fp32"])
+        run("c2c_int32_b8_1024", G(torch.int32, 1024, 1024, 1024, batch=8, ints=True), 2.0 * 8 * 1024 ** 3, None, "Top/s")
+        run("c3_int8_4096", G(torch.int8, N, N, N, ints=True, mode=_lib.C_OVERWRITE), flops, PEAK_TFLOPS["int8"], "Top/s")
         f4 = 2.0 * 8192 * 4096 * 11008
         for dt, nm in ((torch.float32, "fp32"), (torch.bfloat16, "bf16")):
             pk = PEAK_TFLOPS[nm]
-            run(f"c4_linear_fwd_{nm}", make_gemm(dt, 8192, 4096, 11008, tb=True, mode=_lib.C_OVERWRITE, scale=0.1), f4, pk)
-            run(f"c4_linear_dx_{nm}", make_gemm(dt, 8192, 11008, 4096, mode=_lib.C_OVERWRITE, scale=0.1), f4, pk)
-            run(f"c4_linear_dw_{nm}", make_gemm(dt, 11008, 8192, 4096, ta=True, mode=_lib.C_OVERWRITE, scale=0.1), f4, pk)
+            run(f"c4_linear_fwd_{nm}", G(dt, 8192, 4096, 11008, tb=True, mode=_lib.C_OVERWRITE, scale=0.1), f4, pk)
+            run(f"c4_linear_dx_{nm}", G(dt, 8192, 11008, 4096, mode=_lib.C_OVERWRITE, scale=0.1), f4, pk)
+            run(f"c4_linear_dw_{nm}", G(dt, 11008, 8192, 4096, ta=True, mode=_lib.C_OVERWRITE, scale=0.1), f4, pk)
         # the same Linear layer on 16 and 256 rows (inference-sized batches): HBM-bound streaming kernel, split along k
         wbytes = 2.0 * 4096 * 11008
-        run("linear_bf16_16_rows_4096x11008", make_gemm(torch.bfloat16, 16, 4096, 11008, mode=_lib.C_OVERWRITE, scale=0.1),
-            wbytes + 2.0 * 16 * (4096 + 11008), PEAK_HBM_GBS, "GB/s", 1e9, st=steps * 4)
-        run("linear_bf16_256_rows_4096x11008", make_gemm(torch.bfloat16, 256, 4096, 11008, mode=_lib.C_OVERWRITE, scale=0.1),
-            2.0 * 256 * 4096 * 11008, PEAK_TFLOPS["bf16"], st=steps * 2)
+        run("linear_bf16_16_rows_4096x11008", G(torch.bfloat16, 16, 4096, 11008, mode=_lib.C_OVERWRITE, scale=0.1),
+            wbytes + 2.0 * 16 * (4096 + 11008), PEAK_HBM_GBS, "GB/s", 1e9)
+        run("linear_bf16_256_rows_4096x11008", G(torch.bfloat16, 256, 4096, 11008, mode=_lib.C_OVERWRITE, scale=0.1),
+            2.0 * 256 * 4096 * 11008, PEAK_TFLOPS["bf16"])
         # mid-sized squares: the 128 x 128 (16-bit) and 64/128 (Float32) tiles of the DMA-fed kernel
         f2k = 2.0 * 2048 ** 3
-        run("mid_bf16_2048", make_gemm(torch.bfloat16, 2048, 2048, 2048, scale=0.05, mode=_lib.C_OVERWRITE), f2k, PEAK_TFLOPS["bf16"], st=steps * 4)
-        run("mid_fp32_2048", make_gemm(torch.float32, 2048, 2048, 2048, mode=_lib.C_OVERWRITE), f2k, PEAK_TFLOPS["fp32"], st=steps * 2)
+        run("mid_bf16_2048", G(torch.bfloat16, 2048, 2048, 2048, scale=0.05, mode=_lib.C_OVERWRITE), f2k, PEAK_TFLOPS["bf16"])
+        run("mid_fp32_2048", G(torch.float32, 2048, 2048, 2048, mode=_lib.C_OVERWRITE), f2k, PEAK_TFLOPS["fp32"])
         # 192 tiles of 192 x 256 (144 of 256 x 256)
-        run("mid_bf16_3072", make_gemm(torch.bfloat16, 3072, 3072, 3072, scale=0.05, mode=_lib.C_OVERWRITE), 2.0 * 3072 ** 3, PEAK_TFLOPS["bf16"], st=steps * 2)
+        run("mid_bf16_3072", G(torch.bfloat16, 3072, 3072, 3072, scale=0.05, mode=_lib.C_OVERWRITE), 2.0 * 3072 ** 3, PEAK_TFLOPS["bf16"])
         # one round of 256 tiles of 128 x 256 (the square tiles give 128 or 512)
-        run("mid_bf16_2048x4096x4096", make_gemm(torch.bfloat16, 2048, 4096, 4096, scale=0.05, mode=_lib.C_OVERWRITE), 2.0 * 2048 * 4096 * 4096,
-            PEAK_TFLOPS["bf16"], st=steps * 2)
-        x = torch.randn(64, 256, 56, 56, device=dev)
-        w = torch.randn(256, 256, 3, 3, device=dev) / 48.0
+        run("mid_bf16_2048x4096x4096", G(torch.bfloat16, 2048, 4096, 4096, scale=0.05, mode=_lib.C_OVERWRITE), 2.0 * 2048 * 4096 * 4096,
+            PEAK_TFLOPS["bf16"])
         fc = 2.0 * 200704 * 2304 * 256
-        run("c5a_conv2d_fp32", lambda: F.conv2d(x, w, padding=1), fc, PEAK_TFLOPS["fp32"])
-        g = torch.randn(64, 256, 56, 56, device=dev)
-        run("c5a_conv2d_backward_fp32", lambda: F.conv2d_backward(x, w, g, padding=1), 2.0 * fc, PEAK_TFLOPS["fp32"])
-        xh, wh, gh = x.bfloat16(), w.bfloat16(), g.bfloat16()
-        run("c5a_conv2d_bf16", lambda: F.conv2d(xh, wh, padding=1), fc, PEAK_TFLOPS["bf16"], st=steps * 2)
-        run("c5a_conv2d_backward_bf16", lambda: F.conv2d_backward(xh, wh, gh, padding=1), 2.0 * fc, PEAK_TFLOPS["bf16"], st=steps * 2)
-        del x, w, g, xh, wh, gh
+
+        def conv_case(half, backward):
+            def make():
+                x = torch.randn(64, 256, 56, 56, device=dev)
+                w = torch.randn(256, 256, 3, 3, device=dev) / 48.0
+                g = torch.randn(64, 256, 56, 56, device=dev) if backward else None
+                if half:
+                    x, w, g = x.bfloat16(), w.bfloat16(), (g.bfloat16() if backward else None)
+                if backward:
+                    return lambda: F.conv2d_backward(x, w, g, padding=1)
+                return lambda: F.conv2d(x, w, padding=1)
+            return make
+
+        run("c5a_conv2d_fp32", conv_case(False, False), fc, PEAK_TFLOPS["fp32"])
+        run("c5a_conv2d_backward_fp32", conv_case(False, True), 2.0 * fc, PEAK_TFLOPS["fp32"])
+        run("c5a_conv2d_bf16", conv_case(True, False), fc, PEAK_TFLOPS["bf16"])
+        run("c5a_conv2d_backward_bf16", conv_case(True, True), 2.0 * fc, PEAK_TFLOPS["bf16"])
         skinny_bytes = 4.0 * (16 * 8192 + 8192 * 8192 + 2 * 16 * 8192)
-        run("c5b_skinny_fp32_16x8192x8192", make_gemm(torch.float32, 16, 8192, 8192), skinny_bytes, PEAK_HBM_GBS, "GB/s", 1e9,
-            st=steps * 4)
-        # the host-pointer drop-in entry point (nt_matmult's signature): H2D of A, B, C + kernel + D2H of C
+        run("c5b_skinny_fp32_16x8192x8192", G(torch.float32, 16, 8192, 8192), skinny_bytes, PEAK_HBM_GBS, "GB/s", 1e9)
+
+        # the host-pointer drop-in entry points (nt_matmult / nt_matmult_batch's signatures, operands in pageable host
+        # memory): H2D of A, B and C (the accumulate contract makes C an input), the kernel, D2H of C -- wall clock
         import numpy as np
-        ha = np.random.default_rng(7).standard_normal((N, N)).astype(np.float32)
-        hb = np.random.default_rng(8).standard_normal((N, N)).astype(np.float32)
-        hc = np.zeros((N, N), np.float32)
         vp = lambda x: x.ctypes.data_as(ctypes.c_void_p)
-        host_call = lambda: _lib.check(lib.ntg_matmult(_lib.FLOAT32, vp(ha), vp(hb), vp(hc), N, N, N, N, 0, 0))
-        host_call()
-        t0 = time.perf_counter()
-        for _ in range(3):
-            host_call()
-        ms = (time.perf_counter() - t0) / 3 * 1e3
-        extras["c3_fp32_4096_host_pointer_entry"] = {"ms": round(ms, 3), "rate": round(flops / (ms * 1e-3) / 1e12, 2), "unit": "TFLOP/s",
-                                                     "note": "includes 192 MiB host->device and 64 MiB device->host over PCIe (pageable memory)"}
+
+        def host_entry(name, m, k, n, batch, note):
+            if only and name not in only:
+                return
+            rng = np.random.default_rng(7)
+            ha = rng.standard_normal((batch, m, k)).astype(np.float32)
+            hb = rng.standard_normal((batch, k, n)).astype(np.float32)
+            hc = np.zeros((batch, m, n), np.float32)
+            if batch == 1:
+                call = lambda: _lib.check(lib.ntg_matmult(_lib.FLOAT32, vp(ha), vp(hb), vp(hc), m, k, k, n, 0, 0))
+            else:
+                arr = lambda x: (ctypes.c_void_p * batch)(*[x[i].ctypes.data for i in range(batch)])
+                pa, pb, pc = arr(ha), arr(hb), arr(hc)
+                call = lambda: _lib.check(lib.ntg_matmult_batch(_lib.FLOAT32, pa, pb, pc, batch, m, k, k, n, 0, 0))
+            call(); call()
+            reps = 0
+            t0 = time.perf_counter()
+            while reps < 3 or (time.perf_counter() - t0 < 0.2 and reps < 200):
+                call()
+                reps += 1
+            ms = (time.perf_counter() - t0) / reps * 1e3
+            extras[name] = {"ms": round(ms, 4), "rate": round(2.0 * batch * m * k * n / (ms * 1e-3) / 1e12, 3), "unit": "TFLOP/s", "calls": reps, "note": note}
+
+        host_entry("c1_fp32_512_host_pointer_entry", 512, 512, 512, 1, "ntg_matmult: 3 MiB host->device, 1 MiB device->host")
+        host_entry("c2a_fp32_b32_host_pointer_entry", 1024, 768, 1024, 32, "ntg_matmult_batch, 32 items: 320 MiB host->device, 128 MiB device->host")
+        host_entry("c3_fp32_4096_host_pointer_entry", N, N, N, 1, "ntg_matmult: 192 MiB host->device, 64 MiB device->host")
+        lib.ntg_release_host_buffers()
+    if extras:
         out["extras"] = extras
+    if only:
+        print(json.dumps(out))
+        return
 
     # ---------------- CPU baseline: the oracle's restatement of the reference loop nest ----------------
     if not args.no_cpu:

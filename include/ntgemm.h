@@ -20,7 +20,8 @@
  *
  * Every entry point returns 0 (NTG_OK) or a non-zero ntg_status and never throws;
  * ntg_last_error() returns a thread-local description of the last failure.
- * Host-pointer entry points are synchronous (results are in C on return) and thread-safe.
+ * Host-pointer entry points are synchronous (results are in C on return) and thread-safe
+ * (concurrent callers take turns on the library's staging buffers).
  * Device-pointer entry points (suffix _dev) enqueue on the given HIP stream and return.
  */
 #ifndef NTGEMM_H
@@ -138,6 +139,13 @@ int ntg_conv2d_backward(int dtype, const void* image, const void* kernel, const 
                         int64_t out_channels, int64_t k_r, int64_t k_c,
                         int64_t s_r, int64_t s_c, int64_t p_r, int64_t p_c, int64_t d_r, int64_t d_c,
                         int64_t groups, int accumulate);
+
+/* The host-pointer entry points stage their operands through buffers the library keeps between calls: a device arena
+ * that only grows, 32 MiB of pinned host memory and a private stream per GPU (so a sequence of calls pays no
+ * hipMalloc / hipFree, and copies run chunk by chunk with the CPU side of one chunk overlapping the DMA of the
+ * previous one).  This call gives all of it back; the next host-pointer call allocates afresh.  No counterpart in the
+ * reference (its pack buffers are static, nt/functional/cpu/matmult/nt_matmult_blocks.h:12-16). */
+int ntg_release_host_buffers(void);
 
 /* ------------------------------------------------------------------------------------ */
 /* Device-pointer entry points (buffers already in HBM; asynchronous on `stream`).        */

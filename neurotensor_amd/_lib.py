@@ -51,6 +51,7 @@ SIGNATURES = {
     "ntg_version": (_ci, []),
     "ntg_dtype_size": (_i64, [_ci]),
     "ntg_device_count": (_ci, []),
+    "ntg_release_host_buffers": (_ci, []),
     "ntg_matmult": (_ci, [_ci, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _ci, _ci]),
     "ntg_matmult_batch": (_ci, [_ci, _pp, _pp, _pp, _i64, _i64, _i64, _i64, _i64, _ci, _ci]),
     "ntg_linear": (_ci, [_ci, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _ci, _ci, _i64, _i64]),

@@ -137,18 +137,20 @@ __device__ __forceinline__ void dma_offsets(uint32_t (&off)[WB], int64_t ld, int
 // to LDS bytes [lds_addr, lds_addr + 1024).  Written as inline assembly so that the only
 // waits on these loads are the explicit s_waitcnt vmcnt(N) of the pipeline: the compiler's
 // own tracking of LDS-DMA writes made every read of one of the four stages wait for all
-// outstanding loads.  The memory clobber keeps LDS reads from being moved across it; m0 is
-// declared clobbered because the statement overwrites it.
+// outstanding loads.  The memory clobber keeps LDS reads from being moved across it.  m0 is not
+// in the clobber list: it is a reserved register to the compiler, which never keeps a value in it
+// across statements (it loads m0 right before each of its own uses) and rejects it in a clobber
+// list with a "reserved register" diagnostic.
 __device__ __forceinline__ void dma_1k(const void* base, uint32_t off, uint32_t lds_addr) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-                 :: "s"(lds_addr), "v"(off), "s"(base) : "memory", "m0");
+                 :: "s"(lds_addr), "v"(off), "s"(base) : "memory");
 }
 
 // One gathering DMA instruction: 64 lanes x 4 bytes, every lane from its own address, to LDS bytes
 // [lds_addr, lds_addr + 256).
 __device__ __forceinline__ void dma_dword(const void* addr, uint32_t lds_addr) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off"
-                 :: "s"(lds_addr), "v"(addr) : "memory", "m0");
+                 :: "s"(lds_addr), "v"(addr) : "memory");
 }
 // what the padding taps of a gathered convolution operand read
 static __device__ __attribute__((aligned(16))) const uint32_t ring_zero_word[4] = {0u, 0u, 0u, 0u};
@@ -383,7 +385,7 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
             const bool ok = ((cmask3[x] >> sr) & (cmask3[x] >> sq) & 1u) != 0u;
             const char* src = ok ? img + (int64_t)k3_up + lanepart3[x] : reinterpret_cast<const char*>(ring_zero_word);
             asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
-                         :: "s"(lds_tile + (uint32_t)(wave_u * WB + x) * 1024u), "v"(src) : "memory", "m0");
+                         :: "s"(lds_tile + (uint32_t)(wave_u * WB + x) * 1024u), "v"(src) : "memory");
             if (x == WB - 1) {
                 // one K-step on: the next 64 bytes of channels of this tap, else the next tap (or the next tap_step taps)
                 const bool merged = g.tap_step > 1;
@@ -447,7 +449,7 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
             const int off = (int)((oh * (uint32_t)g.s_r * (uint32_t)g.W + ow * (uint32_t)g.s_c) * (uint32_t)g.chan * (uint32_t)ES) + noff4[x];
             const char* src = ok ? img + ((int64_t)im * g.fold_stride * ES + (int64_t)off) : reinterpret_cast<const char*>(ring_zero_word);
             asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
-                         :: "s"(lds_tile + (uint32_t)(wave_u * WB + x) * 1024u), "v"(src) : "memory", "m0");
+                         :: "s"(lds_tile + (uint32_t)(wave_u * WB + x) * 1024u), "v"(src) : "memory");
             if (x == WB - 1) k4_k += BK;
         }
     };

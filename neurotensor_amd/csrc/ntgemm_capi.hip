@@ -4,6 +4,7 @@
 // thread-local message.
 #include "../../include/ntgemm.h"
 #include "ntg_common.h"
+#include "host_stage.h"
 
 #include <cstdarg>
 #include <cstdio>
@@ -91,12 +92,6 @@ int hip_fail(hipError_t e, const char* what) {
         if (e__ != hipSuccess) return hip_fail(e__, #expr); \
     } while (0)
 
-struct DeviceMem {
-    void* p = nullptr;
-    ~DeviceMem() { if (p) (void)hipFree(p); }
-    hipError_t alloc(size_t bytes) { return hipMalloc(&p, bytes ? bytes : 1); }
-    char* at(size_t off) const { return static_cast<char*>(p) + off; }
-};
 
 inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
@@ -378,6 +373,11 @@ const char* ntg_last_error(void) { return g_last_error.c_str(); }
 int ntg_version(void) { return 100; }
 int64_t ntg_dtype_size(int dtype) { return ntg::elem_size(dtype); }
 
+int ntg_release_host_buffers(void) {
+    ntg::HostSession::release_all();
+    return NTG_OK;
+}
+
 int ntg_device_count(void) {
     int n = 0;
     if (hipGetDeviceCount(&n) != hipSuccess) return 0;
@@ -502,34 +502,32 @@ int ntg_matmult_batch(int dtype, const void* const* A, const void* const* B, voi
     const int64_t ws_bytes = strided ? ntg_gemm_workspace_bytes(&d) : 0;
     if (ws_bytes > 0) off += (size_t)ws_bytes;
 
-    DeviceMem mem;
-    HIP_TRY(mem.alloc(off));
-    for (auto& kv : slotA) HIP_TRY(hipMemcpy(mem.at(kv.second), kv.first, a_bytes, hipMemcpyHostToDevice));
-    for (auto& kv : slotB) HIP_TRY(hipMemcpy(mem.at(kv.second), kv.first, b_bytes, hipMemcpyHostToDevice));
+    ntg::HostSession mem;
+    HIP_TRY(mem.reserve(off));
+    for (auto& kv : slotA) HIP_TRY(mem.upload(kv.second, kv.first, a_bytes));
+    for (auto& kv : slotB) HIP_TRY(mem.upload(kv.second, kv.first, b_bytes));
     std::vector<void*> tab(3 * (size_t)batches);
     std::map<const void*, int64_t> seenC;
     for (int64_t i = 0; i < batches; ++i) {
         const auto ins = seenC.emplace(C[i], i);
         if (!ins.second) return fail(NTG_ERR_INVALID_ARGUMENT, "output pointers of items %lld and %lld alias", (long long)ins.first->second, (long long)i);
-        char* dc = mem.at(c_off + (size_t)i * align_up(c_bytes, 256));
-        HIP_TRY(hipMemcpy(dc, C[i], c_bytes, hipMemcpyHostToDevice));   // accumulate contract: C is an input too
+        const size_t dc_off = c_off + (size_t)i * align_up(c_bytes, 256);
+        HIP_TRY(mem.upload(dc_off, C[i], c_bytes));   // accumulate contract: C is an input too
         tab[(size_t)i] = mem.at(slotA[A[i]]);
         tab[(size_t)(batches + i)] = mem.at(slotB[B[i]]);
-        tab[(size_t)(2 * batches + i)] = dc;
+        tab[(size_t)(2 * batches + i)] = mem.at(dc_off);
     }
-    HIP_TRY(hipMemcpy(mem.at(tab_off), tab.data(), tab.size() * sizeof(void*), hipMemcpyHostToDevice));
-
     void** dtab = reinterpret_cast<void**>(mem.at(tab_off));
     if (ws_bytes > 0) { d.workspace = mem.at(ws_off); d.workspace_bytes = ws_bytes; }
     if (strided) {
-        rc = ntg_gemm_dev(&d, tab[0], tab[(size_t)batches], tab[(size_t)(2 * batches)], nullptr);
+        rc = ntg_gemm_dev(&d, tab[0], tab[(size_t)batches], tab[(size_t)(2 * batches)], mem.stream());
     } else {
-        rc = ntg_gemm_ptrs_dev(&d, dtab, dtab + batches, dtab + 2 * batches, nullptr);
+        HIP_TRY(mem.upload(tab_off, tab.data(), tab.size() * sizeof(void*)));
+        rc = ntg_gemm_ptrs_dev(&d, dtab, dtab + batches, dtab + 2 * batches, mem.stream());
     }
     if (rc) return rc;
-    HIP_TRY(hipStreamSynchronize(nullptr));
     for (int64_t i = 0; i < batches; ++i)
-        HIP_TRY(hipMemcpy(C[i], tab[(size_t)(2 * batches + i)], c_bytes, hipMemcpyDeviceToHost));
+        HIP_TRY(mem.download(C[i], c_off + (size_t)i * align_up(c_bytes, 256), c_bytes));
     return NTG_OK;
 }
 
@@ -547,12 +545,12 @@ int ntg_linear(int dtype, const void* X, const void* W, const void* bias, void* 
     if (!X || !W || !bias || !Y) return fail(NTG_ERR_INVALID_ARGUMENT, "null pointer");
     const size_t x_bytes = (size_t)(m * k * es), w_bytes = (size_t)(k * n * es), y_bytes = (size_t)(m * n * es);
     const size_t bias_bytes = (size_t)(bias_rows * bias_cols * es);
-    DeviceMem mem;
+    ntg::HostSession mem;
     const size_t ox = 0, ow = align_up(x_bytes, 256), ob = ow + align_up(w_bytes, 256), oy = ob + align_up(bias_bytes, 256);
-    HIP_TRY(mem.alloc(oy + y_bytes));
-    if (x_bytes) HIP_TRY(hipMemcpy(mem.at(ox), X, x_bytes, hipMemcpyHostToDevice));
-    if (w_bytes) HIP_TRY(hipMemcpy(mem.at(ow), W, w_bytes, hipMemcpyHostToDevice));
-    HIP_TRY(hipMemcpy(mem.at(ob), bias, bias_bytes, hipMemcpyHostToDevice));
+    HIP_TRY(mem.reserve(oy + y_bytes));
+    if (x_bytes) HIP_TRY(mem.upload(ox, X, x_bytes));
+    if (w_bytes) HIP_TRY(mem.upload(ow, W, w_bytes));
+    HIP_TRY(mem.upload(ob, bias, bias_bytes));
     ntg_gemm_desc d;
     std::memset(&d, 0, sizeof d);
     d.dtype = dtype; d.transpose_a = transpose_x; d.transpose_b = transpose_w; d.c_mode = NTG_C_BIAS;
@@ -560,10 +558,9 @@ int ntg_linear(int dtype, const void* X, const void* W, const void* bias, void* 
     d.bias = mem.at(ob);
     d.bias_row_stride = (bias_rows == 1) ? 0 : bias_cols;
     d.bias_col_stride = (bias_cols == 1) ? 0 : 1;
-    rc = ntg_gemm_dev(&d, mem.at(ox), mem.at(ow), mem.at(oy), nullptr);
+    rc = ntg_gemm_dev(&d, mem.at(ox), mem.at(ow), mem.at(oy), mem.stream());
     if (rc) return rc;
-    HIP_TRY(hipStreamSynchronize(nullptr));
-    HIP_TRY(hipMemcpy(Y, mem.at(oy), y_bytes, hipMemcpyDeviceToHost));
+    HIP_TRY(mem.download(Y, oy, y_bytes));
     return NTG_OK;
 }
 
@@ -609,14 +606,13 @@ int ntg_unfold2d(int dtype, const void* image, void* col,
     if (!image || !col) return fail(NTG_ERR_INVALID_ARGUMENT, "null pointer");
     const size_t im_bytes = (size_t)(batch * channels * height * width * es);
     const size_t col_bytes = (size_t)(batch * channels * k_r * k_c * Ho * Wo * es);
-    DeviceMem mem;
+    ntg::HostSession mem;
     const size_t oc = align_up(im_bytes, 256);
-    HIP_TRY(mem.alloc(oc + col_bytes));
-    HIP_TRY(hipMemcpy(mem.at(0), image, im_bytes, hipMemcpyHostToDevice));
-    rc = ntg_unfold2d_dev(dtype, mem.at(0), mem.at(oc), batch, channels, height, width, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c, nullptr);
+    HIP_TRY(mem.reserve(oc + col_bytes));
+    HIP_TRY(mem.upload(0, image, im_bytes));
+    rc = ntg_unfold2d_dev(dtype, mem.at(0), mem.at(oc), batch, channels, height, width, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c, mem.stream());
     if (rc) return rc;
-    HIP_TRY(hipStreamSynchronize(nullptr));
-    HIP_TRY(hipMemcpy(col, mem.at(oc), col_bytes, hipMemcpyDeviceToHost));
+    HIP_TRY(mem.download(col, oc, col_bytes));
     return NTG_OK;
 }
 
@@ -1255,16 +1251,15 @@ int ntg_conv2d(int dtype, const void* image, const void* kernel, void* out,
     const size_t k_bytes = (size_t)(out_channels * (channels / groups) * k_r * k_c * es);
     const size_t o_bytes = (size_t)(batch * out_channels * Ho * Wo * es);
     const int64_t ws = ntg_conv2d_fast_workspace_bytes(dtype, batch, channels, height, width, out_channels, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c, groups);
-    DeviceMem mem;
+    ntg::HostSession mem;
     const size_t ok_ = align_up(im_bytes, 256), oo = ok_ + align_up(k_bytes, 256), ow = oo + align_up(o_bytes, 256);
-    HIP_TRY(mem.alloc(ow + (size_t)ws));
-    if (im_bytes) HIP_TRY(hipMemcpy(mem.at(0), image, im_bytes, hipMemcpyHostToDevice));
-    if (k_bytes) HIP_TRY(hipMemcpy(mem.at(ok_), kernel, k_bytes, hipMemcpyHostToDevice));
+    HIP_TRY(mem.reserve(ow + (size_t)ws));
+    if (im_bytes) HIP_TRY(mem.upload(0, image, im_bytes));
+    if (k_bytes) HIP_TRY(mem.upload(ok_, kernel, k_bytes));
     rc = ntg_conv2d_dev(dtype, mem.at(0), mem.at(ok_), mem.at(oo), mem.at(ow), ws, batch, channels, height, width,
-                        out_channels, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c, groups, nullptr);
+                        out_channels, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c, groups, mem.stream());
     if (rc) return rc;
-    HIP_TRY(hipStreamSynchronize(nullptr));
-    HIP_TRY(hipMemcpy(out, mem.at(oo), o_bytes, hipMemcpyDeviceToHost));
+    HIP_TRY(mem.download(out, oo, o_bytes));
     return NTG_OK;
 }
 
@@ -1300,16 +1295,15 @@ int ntg_unfold2d_backward(int dtype, const void* col, void* image,
     if (!col || !image) return fail(NTG_ERR_INVALID_ARGUMENT, "null pointer");
     const size_t im_bytes = (size_t)(batch * channels * height * width * es);
     const size_t col_bytes = (size_t)(batch * channels * k_r * k_c * Ho * Wo * es);
-    DeviceMem mem;
+    ntg::HostSession mem;
     const size_t oc = align_up(im_bytes, 256);
-    HIP_TRY(mem.alloc(oc + col_bytes));
-    if (accumulate) HIP_TRY(hipMemcpy(mem.at(0), image, im_bytes, hipMemcpyHostToDevice));
-    HIP_TRY(hipMemcpy(mem.at(oc), col, col_bytes, hipMemcpyHostToDevice));
+    HIP_TRY(mem.reserve(oc + col_bytes));
+    if (accumulate) HIP_TRY(mem.upload(0, image, im_bytes));
+    HIP_TRY(mem.upload(oc, col, col_bytes));
     rc = ntg_unfold2d_backward_dev(dtype, mem.at(oc), mem.at(0), batch, channels, height, width, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c,
-                                   accumulate, nullptr);
+                                   accumulate, mem.stream());
     if (rc) return rc;
-    HIP_TRY(hipStreamSynchronize(nullptr));
-    HIP_TRY(hipMemcpy(image, mem.at(0), im_bytes, hipMemcpyDeviceToHost));
+    HIP_TRY(mem.download(image, 0, im_bytes));
     return NTG_OK;
 }
 
@@ -1531,16 +1525,15 @@ int ntg_conv_transpose2d(int dtype, const void* input, const void* kernel, void*
     const int64_t wsb = ntg_conv_transpose2d_workspace_bytes(dtype, batch, in_channels, in_h, in_w, out_channels, k_r, k_c, s_r, s_c,
                                                              p_r, p_c, d_r, d_c, op_r, op_c, groups);
     if (wsb < 0) return fail(NTG_ERR_INVALID_ARGUMENT, "invalid geometry");
-    DeviceMem mem;
+    ntg::HostSession mem;
     const size_t o_k = align_up(in_bytes, 256), o_o = o_k + align_up(k_bytes, 256), o_ws = o_o + align_up(o_bytes, 256);
-    HIP_TRY(mem.alloc(o_ws + (size_t)wsb));
-    if (in_bytes) HIP_TRY(hipMemcpy(mem.at(0), input, in_bytes, hipMemcpyHostToDevice));
-    if (k_bytes) HIP_TRY(hipMemcpy(mem.at(o_k), kernel, k_bytes, hipMemcpyHostToDevice));
+    HIP_TRY(mem.reserve(o_ws + (size_t)wsb));
+    if (in_bytes) HIP_TRY(mem.upload(0, input, in_bytes));
+    if (k_bytes) HIP_TRY(mem.upload(o_k, kernel, k_bytes));
     rc = ntg_conv_transpose2d_dev(dtype, mem.at(0), mem.at(o_k), mem.at(o_o), mem.at(o_ws), wsb, batch, in_channels, in_h, in_w, out_channels,
-                                  k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c, op_r, op_c, groups, nullptr);
+                                  k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c, op_r, op_c, groups, mem.stream());
     if (rc) return rc;
-    HIP_TRY(hipStreamSynchronize(nullptr));
-    HIP_TRY(hipMemcpy(out, mem.at(o_o), o_bytes, hipMemcpyDeviceToHost));
+    HIP_TRY(mem.download(out, o_o, o_bytes));
     return NTG_OK;
 }
 
@@ -1566,22 +1559,21 @@ int ntg_conv2d_backward(int dtype, const void* image, const void* kernel, const 
     const size_t g_bytes = (size_t)(batch * out_channels * Ho * Wo * es);
     const int64_t wsb = ntg_conv2d_backward_workspace_bytes(dtype, batch, channels, height, width, out_channels, k_r, k_c, s_r, s_c,
                                                             p_r, p_c, d_r, d_c, groups);
-    DeviceMem mem;
+    ntg::HostSession mem;
     const size_t o_k = align_up(im_bytes, 256), o_g = o_k + align_up(k_bytes, 256), o_di = o_g + align_up(g_bytes, 256);
     const size_t o_dk = o_di + align_up(im_bytes, 256), o_ws = o_dk + align_up(k_bytes, 256);
-    HIP_TRY(mem.alloc(o_ws + (size_t)wsb));
-    HIP_TRY(hipMemcpy(mem.at(0), image, im_bytes, hipMemcpyHostToDevice));
-    HIP_TRY(hipMemcpy(mem.at(o_k), kernel, k_bytes, hipMemcpyHostToDevice));
-    HIP_TRY(hipMemcpy(mem.at(o_g), grad_out, g_bytes, hipMemcpyHostToDevice));
-    if (accumulate && d_image) HIP_TRY(hipMemcpy(mem.at(o_di), d_image, im_bytes, hipMemcpyHostToDevice));
-    if (accumulate && d_kernel) HIP_TRY(hipMemcpy(mem.at(o_dk), d_kernel, k_bytes, hipMemcpyHostToDevice));
+    HIP_TRY(mem.reserve(o_ws + (size_t)wsb));
+    HIP_TRY(mem.upload(0, image, im_bytes));
+    HIP_TRY(mem.upload(o_k, kernel, k_bytes));
+    HIP_TRY(mem.upload(o_g, grad_out, g_bytes));
+    if (accumulate && d_image) HIP_TRY(mem.upload(o_di, d_image, im_bytes));
+    if (accumulate && d_kernel) HIP_TRY(mem.upload(o_dk, d_kernel, k_bytes));
     rc = ntg_conv2d_backward_dev(dtype, mem.at(0), mem.at(o_k), mem.at(o_g), d_image ? mem.at(o_di) : nullptr,
                                  d_kernel ? mem.at(o_dk) : nullptr, mem.at(o_ws), wsb, batch, channels, height, width, out_channels,
-                                 k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c, groups, accumulate, nullptr);
+                                 k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c, groups, accumulate, mem.stream());
     if (rc) return rc;
-    HIP_TRY(hipStreamSynchronize(nullptr));
-    if (d_image) HIP_TRY(hipMemcpy(d_image, mem.at(o_di), im_bytes, hipMemcpyDeviceToHost));
-    if (d_kernel) HIP_TRY(hipMemcpy(d_kernel, mem.at(o_dk), k_bytes, hipMemcpyDeviceToHost));
+    if (d_image) HIP_TRY(mem.download(d_image, o_di, im_bytes));
+    if (d_kernel) HIP_TRY(mem.download(d_kernel, o_dk, k_bytes));
     return NTG_OK;
 }
 
@@ -1868,16 +1860,15 @@ int ntg_convnd(int dtype, const void* image, const void* kernel, void* out, int6
     const size_t im_bytes = (size_t)(batch * channels * u.vol * es), k_bytes = (size_t)(out_channels * (channels / groups) * u.taps * es);
     const size_t o_bytes = (size_t)(batch * out_channels * u.L * es);
     const int64_t wsb = ntg_convnd_workspace_bytes(dtype, batch, channels, out_channels, ndim, size, kernel_size, stride, padding, dilation, groups, 0);
-    DeviceMem mem;
+    ntg::HostSession mem;
     const size_t o_k = align_up(im_bytes, 256), o_o = o_k + align_up(k_bytes, 256), o_ws = o_o + align_up(o_bytes, 256);
-    HIP_TRY(mem.alloc(o_ws + (size_t)wsb));
-    if (im_bytes) HIP_TRY(hipMemcpy(mem.at(0), image, im_bytes, hipMemcpyHostToDevice));
-    if (k_bytes) HIP_TRY(hipMemcpy(mem.at(o_k), kernel, k_bytes, hipMemcpyHostToDevice));
+    HIP_TRY(mem.reserve(o_ws + (size_t)wsb));
+    if (im_bytes) HIP_TRY(mem.upload(0, image, im_bytes));
+    if (k_bytes) HIP_TRY(mem.upload(o_k, kernel, k_bytes));
     rc = ntg_convnd_dev(dtype, mem.at(0), mem.at(o_k), mem.at(o_o), mem.at(o_ws), wsb, batch, channels, out_channels, ndim, size, kernel_size,
-                        stride, padding, dilation, groups, nullptr);
+                        stride, padding, dilation, groups, mem.stream());
     if (rc) return rc;
-    HIP_TRY(hipStreamSynchronize(nullptr));
-    HIP_TRY(hipMemcpy(out, mem.at(o_o), o_bytes, hipMemcpyDeviceToHost));
+    HIP_TRY(mem.download(out, o_o, o_bytes));
     return NTG_OK;
 }
 
@@ -1896,22 +1887,21 @@ int ntg_convnd_backward(int dtype, const void* image, const void* kernel, const 
     const size_t im_bytes = (size_t)(batch * channels * u.vol * es), k_bytes = (size_t)(out_channels * (channels / groups) * u.taps * es);
     const size_t g_bytes = (size_t)(batch * out_channels * u.L * es);
     const int64_t wsb = ntg_convnd_workspace_bytes(dtype, batch, channels, out_channels, ndim, size, kernel_size, stride, padding, dilation, groups, 1);
-    DeviceMem mem;
+    ntg::HostSession mem;
     const size_t o_k = align_up(im_bytes, 256), o_g = o_k + align_up(k_bytes, 256), o_di = o_g + align_up(g_bytes, 256);
     const size_t o_dk = o_di + align_up(im_bytes, 256), o_ws = o_dk + align_up(k_bytes, 256);
-    HIP_TRY(mem.alloc(o_ws + (size_t)wsb));
-    HIP_TRY(hipMemcpy(mem.at(0), image, im_bytes, hipMemcpyHostToDevice));
-    HIP_TRY(hipMemcpy(mem.at(o_k), kernel, k_bytes, hipMemcpyHostToDevice));
-    HIP_TRY(hipMemcpy(mem.at(o_g), grad_out, g_bytes, hipMemcpyHostToDevice));
-    if (accumulate && d_image) HIP_TRY(hipMemcpy(mem.at(o_di), d_image, im_bytes, hipMemcpyHostToDevice));
-    if (accumulate && d_kernel) HIP_TRY(hipMemcpy(mem.at(o_dk), d_kernel, k_bytes, hipMemcpyHostToDevice));
+    HIP_TRY(mem.reserve(o_ws + (size_t)wsb));
+    HIP_TRY(mem.upload(0, image, im_bytes));
+    HIP_TRY(mem.upload(o_k, kernel, k_bytes));
+    HIP_TRY(mem.upload(o_g, grad_out, g_bytes));
+    if (accumulate && d_image) HIP_TRY(mem.upload(o_di, d_image, im_bytes));
+    if (accumulate && d_kernel) HIP_TRY(mem.upload(o_dk, d_kernel, k_bytes));
     rc = ntg_convnd_backward_dev(dtype, mem.at(0), mem.at(o_k), mem.at(o_g), d_image ? mem.at(o_di) : nullptr, d_kernel ? mem.at(o_dk) : nullptr,
                                  mem.at(o_ws), wsb, batch, channels, out_channels, ndim, size, kernel_size, stride, padding, dilation, groups,
-                                 accumulate, nullptr);
+                                 accumulate, mem.stream());
     if (rc) return rc;
-    HIP_TRY(hipStreamSynchronize(nullptr));
-    if (d_image) HIP_TRY(hipMemcpy(d_image, mem.at(o_di), im_bytes, hipMemcpyDeviceToHost));
-    if (d_kernel) HIP_TRY(hipMemcpy(d_kernel, mem.at(o_dk), k_bytes, hipMemcpyDeviceToHost));
+    if (d_image) HIP_TRY(mem.download(d_image, o_di, im_bytes));
+    if (d_kernel) HIP_TRY(mem.download(d_kernel, o_dk, k_bytes));
     return NTG_OK;
 }
 
@@ -1934,16 +1924,15 @@ int ntg_conv_transposend(int dtype, const void* input, const void* kernel, void*
     const int64_t wsb = ntg_conv_transposend_workspace_bytes(dtype, batch, in_channels, out_channels, ndim, in_size, kernel_size, stride, padding,
                                                              dilation, output_padding, groups);
     if (wsb < 0) return fail(NTG_ERR_INVALID_ARGUMENT, "invalid geometry");
-    DeviceMem mem;
+    ntg::HostSession mem;
     const size_t o_k = align_up(in_bytes, 256), o_o = o_k + align_up(k_bytes, 256), o_ws = o_o + align_up(o_bytes, 256);
-    HIP_TRY(mem.alloc(o_ws + (size_t)wsb));
-    if (in_bytes) HIP_TRY(hipMemcpy(mem.at(0), input, in_bytes, hipMemcpyHostToDevice));
-    if (k_bytes) HIP_TRY(hipMemcpy(mem.at(o_k), kernel, k_bytes, hipMemcpyHostToDevice));
+    HIP_TRY(mem.reserve(o_ws + (size_t)wsb));
+    if (in_bytes) HIP_TRY(mem.upload(0, input, in_bytes));
+    if (k_bytes) HIP_TRY(mem.upload(o_k, kernel, k_bytes));
     rc = ntg_conv_transposend_dev(dtype, mem.at(0), mem.at(o_k), mem.at(o_o), mem.at(o_ws), wsb, batch, in_channels, out_channels, ndim, in_size,
-                                  kernel_size, stride, padding, dilation, output_padding, groups, nullptr);
+                                  kernel_size, stride, padding, dilation, output_padding, groups, mem.stream());
     if (rc) return rc;
-    HIP_TRY(hipStreamSynchronize(nullptr));
-    HIP_TRY(hipMemcpy(out, mem.at(o_o), o_bytes, hipMemcpyDeviceToHost));
+    HIP_TRY(mem.download(out, o_o, o_bytes));
     return NTG_OK;
 }
 

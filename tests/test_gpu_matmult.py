@@ -745,3 +745,61 @@ def test_skinny_fp32_config5b():
         ref = oracle.matmult2d(sa, sb, c0.copy(), ta, tb)
         got = dev_matmult(sa, sb, c0, m, k, n, ta, tb, np.float32)
         assert np.abs(got - ref).max() <= float_tol(k, A, B), (m, k, n, ta, tb)
+
+
+def test_host_entry_staging_large_transfers_threads_and_release():
+    """The host-pointer seam stages through a grow-only device arena and a ring of 8 MiB pinned chunks: operands of
+    several chunks (and not a whole number of them), a smaller call after a larger one, a larger one after that (the
+    arena grows), two threads calling at once, and a call after ntg_release_host_buffers -- every result bit-identical
+    to the device entry point on the same operands."""
+    import threading
+    lib = _lib.load()
+    rng = np.random.default_rng(515)
+
+    def case(m, k, n, dtype, ta=False, tb=False):
+        a, b, sa, sb, c0 = make_inputs(rng, m, k, n, dtype, ta, tb, int_range=(-1000, 1000))
+        want = dev_matmult(sa, sb, c0, m, k, n, ta, tb, dtype)
+        return (sa, sb, c0, m, k, n, ta, tb, dtype, want)
+
+    def check_case(cs):
+        sa, sb, c0, m, k, n, ta, tb, dtype, want = cs
+        got = host_matmult(sa, sb, c0.copy(), m, k, n, ta, tb, code_of(dtype))
+        assert got.tobytes() == want.tobytes(), (m, k, n, dtype)
+
+    big = case(2500, 1100, 2300, np.float32)           # A 10.5 MiB, B 9.7 MiB, C 21.9 MiB
+    small = case(70, 90, 50, np.float32, True, True)
+    bigger = case(3000, 2100, 2600, np.int32, False, True)
+    half = case(1111, 1000, 2224, "bf16")
+    for cs in (big, small, bigger, half, big):
+        check_case(cs)
+    errors = []
+
+    def worker(cs):
+        try:
+            for _ in range(3):
+                check_case(cs)
+        except Exception as e:          # noqa: BLE001 (reported below)
+            errors.append(e)
+
+    ts = [threading.Thread(target=worker, args=(cs,)) for cs in (big, half, small)]
+    for t in ts:
+        t.start()
+    for t in ts:
+        t.join()
+    assert not errors, errors
+    assert lib.ntg_release_host_buffers() == 0
+    check_case(small)
+    check_case(big)
+    # batch entry point with repeated inputs, several chunks in total
+    m, k, n = 600, 700, 800
+    As = [rng.standard_normal((m, k)).astype(np.float32) for _ in range(3)]
+    Bm = rng.standard_normal((k, n)).astype(np.float32)
+    Cs = [rng.standard_normal((m, n)).astype(np.float32) for _ in range(5)]
+    want = [c + 0 for c in Cs]
+    idx = [0, 1, 2, 1, 0]
+    for i, c in enumerate(want):
+        host_matmult(As[idx[i]], Bm, c, m, k, n, False, False, _lib.FLOAT32)
+    arr = lambda xs: (ctypes.c_void_p * len(xs))(*[x.ctypes.data for x in xs])
+    _lib.check(lib.ntg_matmult_batch(_lib.FLOAT32, arr([As[i] for i in idx]), arr([Bm] * 5), arr(Cs), 5, m, k, k, n, 0, 0))
+    for i in range(5):
+        assert np.abs(Cs[i] - want[i]).max() <= float_tol(k, As[idx[i]], Bm)
