@@ -37,11 +37,20 @@ extern "C" {
  * nt/dtype/compatible/DTypeDeclareMacros.h:5-33) so a caller can pass
  * static_cast<int>(tensor.dtype()).  BFLOAT16 and UINT64 are extensions: the reference
  * has no BFloat16 DType (nt/types/bfloat16.h:4-5) and instantiates uint64_t only at the
- * kernel level (nt_matmult_uint64.cpp). Complex and 128-bit types are not supported. */
+ * kernel level (nt_matmult_uint64.cpp).  The complex types hold interleaved (re, im) pairs of half / float / double; their
+ * matmult is the reference's: its generic micro kernel multiplies the interleaved lanes element-wise
+ * (nt/mp/simde_traits/simde_traits_avx2.h:928-937, :996-1002), so the result is one real product of the real parts and one
+ * of the imaginary parts (Complex32 rounded to half every 8 k), NOT the complex product.  They are served by the product,
+ * linear, unfold and forward-convolution entry points (up to two spatial axes); the gradient and transposed convolutions
+ * return NTG_ERR_UNSUPPORTED_DTYPE for them.  The 128-bit types (Float128 = 3, int128 = 11, uint128 = 15) stay on the
+ * reference's matmult_naive. */
 typedef enum ntg_dtype {
     NTG_FLOAT16 = 0,
     NTG_FLOAT32 = 1,
     NTG_FLOAT64 = 2,
+    NTG_COMPLEX32 = 4,
+    NTG_COMPLEX64 = 5,
+    NTG_COMPLEX128 = 6,
     NTG_INT8 = 7,
     NTG_INT16 = 8,
     NTG_INT32 = 9,

@@ -10,6 +10,7 @@ LIB_PATH = os.path.join(_HERE, "lib", "libntgemm.so")
 
 # ntg_dtype (== nt::DType values; BF16/U64 are extensions)
 FLOAT16, FLOAT32, FLOAT64 = 0, 1, 2
+COMPLEX32, COMPLEX64, COMPLEX128 = 4, 5, 6      # interleaved (re, im) pairs of half / float / double
 INT8, INT16, INT32, INT64 = 7, 8, 9, 10
 UINT8, UINT16, UINT32 = 12, 13, 14
 BFLOAT16, UINT64 = 100, 101

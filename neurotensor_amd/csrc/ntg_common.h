@@ -8,6 +8,7 @@ namespace ntg {
 // numeric values follow nt::DType (nt/dtype/DType_enum.h:14-20); BF16/U64 are extensions
 enum DType : int {
     DT_F16 = 0, DT_F32 = 1, DT_F64 = 2,
+    DT_C32 = 4, DT_C64 = 5, DT_C128 = 6,      // interleaved (re, im) pairs of half / float / double
     DT_I8 = 7, DT_I16 = 8, DT_I32 = 9, DT_I64 = 10,
     DT_U8 = 12, DT_U16 = 13, DT_U32 = 14,
     DT_BF16 = 100, DT_U64 = 101
@@ -143,6 +144,9 @@ static inline int64_t elem_size(int dt) {
     case DT_F16: case DT_BF16: case DT_I16: case DT_U16: return 2;
     case DT_F32: case DT_I32: case DT_U32: return 4;
     case DT_F64: case DT_I64: case DT_U64: return 8;
+    case DT_C32: return 4;
+    case DT_C64: return 8;
+    case DT_C128: return 16;
     default: return 0;
     }
 }
@@ -151,6 +155,7 @@ static inline int64_t elem_size(int dt) {
 hipError_t launch_gemm_mfma(int dtype, bool ta, bool tb, const GemmParams& p, hipStream_t s);
 hipError_t launch_gemm_valu(int dtype, bool ta, bool tb, const GemmParams& p, hipStream_t s);
 hipError_t launch_gemm_mfma_i8(int dtype, bool ta, bool tb, const GemmParams& p, hipStream_t s);   // Int8 / UInt8: MFMA where rows are 16-byte multiples
+hipError_t launch_gemm_complex(int dtype, bool ta, bool tb, const GemmParams& p, hipStream_t s);   // Complex32 / 64 / 128: lane-wise products on (re, im) pairs
 hipError_t launch_gemm_skinny(int dtype, bool ta, bool tb, const GemmParams& p, hipStream_t s, bool* handled);
 // op(B) is the im2col matrix of the image at p.B (tb: its transpose); floating dtypes only
 hipError_t launch_conv_mfma(int dtype, bool tb, const GemmParams& p, hipStream_t s);

@@ -103,6 +103,17 @@ bool is_int_dtype(int dt) {
     }
 }
 
+bool is_complex_dtype(int dt) { return dt == ntg::DT_C32 || dt == ntg::DT_C64 || dt == ntg::DT_C128; }
+// integers and the complex types: computed lane by lane on the vector ALU, bit-exact; no matrix-pipe or gathering forms
+bool is_valu_dtype(int dt) { return is_int_dtype(dt) || is_complex_dtype(dt); }
+
+// The complex types reach the product, im2col and the forward convolutions (what the reference's tests exercise,
+// tests/src/conv_test.cpp:192-213); col2im and the gradient / transposed convolutions are not built for them.
+int reject_complex(int dtype, const char* what) {
+    if (!is_complex_dtype(dtype)) return NTG_OK;
+    return fail(NTG_ERR_UNSUPPORTED_DTYPE, "%s is not available for the complex dtypes (dtype %d)", what, dtype);
+}
+
 // Fills the derived fields and launches the kernel family for the dtype.
 int launch_gemm(ntg::GemmParams p, int dtype, bool ta, bool tb, hipStream_t s) {
     const int64_t es = ntg::elem_size(dtype);
@@ -114,6 +125,8 @@ int launch_gemm(ntg::GemmParams p, int dtype, bool ta, bool tb, hipStream_t s) {
         e = ntg::launch_gemm_mfma_i8(dtype, ta, tb, p, s);
     } else if (is_int_dtype(dtype)) {
         e = ntg::launch_gemm_valu(dtype, ta, tb, p, s);
+    } else if (is_complex_dtype(dtype)) {
+        e = ntg::launch_gemm_complex(dtype, ta, tb, p, s);
     } else {
         bool handled = false;
         e = ntg::launch_gemm_skinny(dtype, ta, tb, p, s, &handled);
@@ -214,7 +227,7 @@ static int run_int_planes(const ntg::GemmParams& p, const IntPlanesPlan& pl, boo
 SplitPlan plan_splitk(const ntg::GemmParams& p, int dtype, bool ta) {
     SplitPlan none{1, p.K, 0};
     const int64_t es = ntg::elem_size(dtype);
-    if (is_int_dtype(dtype) || es == 0 || p.batch != 1 || p.Aptr || p.Bptr || p.Cptr) return none;
+    if (is_valu_dtype(dtype) || es == 0 || p.batch != 1 || p.Aptr || p.Bptr || p.Cptr) return none;
     if (p.M <= 32 && dtype != ntg::DT_F64) return none;                       // the streaming kernels take these
     const bool half = dtype == ntg::DT_F16 || dtype == ntg::DT_BF16;
     if (half) {
@@ -276,6 +289,8 @@ int run_gemm(ntg::GemmParams p, int dtype, bool ta, bool tb, hipStream_t s, void
         hipError_t e = hipSuccess;
         if (is_int_dtype(dtype)) {
             e = ntg::launch_gemm_valu(dtype, ta, tb, p, s);                 // its k loop runs zero times
+        } else if (is_complex_dtype(dtype)) {
+            e = ntg::launch_gemm_complex(dtype, ta, tb, p, s);              // likewise
         } else {
             for (int b = 0; b < p.batch && e == hipSuccess; ++b) {
                 ntg::GemmParams q = p;
@@ -644,7 +659,7 @@ static Geo3 geo_dimage(const Geo3& g) {
 // The floating dtypes gather the im2col operand inside the GEMM (no col buffer) when every index the kernel forms fits
 // 32 bits with room for its out-of-range sentinels and the kernel has at most 8 taps per axis (one byte of tap mask).
 static bool conv_implicit_g(int dtype, int64_t channels, const Geo3& g) {
-    if (is_int_dtype(dtype)) return false;
+    if (is_valu_dtype(dtype)) return false;
     const int64_t lim = 1 << 24;
     for (int a = 0; a < 3; ++a) {
         if (g.k[a] > 8) return false;
@@ -713,7 +728,7 @@ static bool conv_pointwise(const Geo3& g) {
 }
 static bool conv_pointwise_ok(int dtype, int64_t channels, int64_t groups, const Geo3& g) {
     if (!conv_pointwise(g)) return false;
-    if (is_int_dtype(dtype)) return true;
+    if (is_valu_dtype(dtype)) return true;
     const int64_t es = ntg::elem_size(dtype);
     return (g.L() * es) % 16 == 0 && (channels / groups * es) % 16 == 0;
 }
@@ -1197,7 +1212,7 @@ int ntg_conv2d_dev(int dtype, const void* image, const void* kernel, void* out,
     {
         const Geo3 g = geo2(height, width, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c, Ho, Wo);
         if (conv_pointwise_ok(dtype, channels, groups, g) &&
-            (is_int_dtype(dtype) || ((reinterpret_cast<uintptr_t>(image) | reinterpret_cast<uintptr_t>(kernel) | reinterpret_cast<uintptr_t>(out)) & 15) == 0))
+            (is_valu_dtype(dtype) || ((reinterpret_cast<uintptr_t>(image) | reinterpret_cast<uintptr_t>(kernel) | reinterpret_cast<uintptr_t>(out)) & 15) == 0))
             return conv_forward_pointwise(dtype, image, kernel, out, batch, channels, out_channels, g, groups, stream);
         // with the workspace of ntg_conv2d_fast_workspace_bytes: channels-last copy of the image, 16-byte gathers
         MergedTaps mt;
@@ -1267,6 +1282,7 @@ int ntg_unfold2d_backward_dev(int dtype, const void* col, void* image,
                               int64_t batch, int64_t channels, int64_t height, int64_t width,
                               int64_t k_r, int64_t k_c, int64_t s_r, int64_t s_c,
                               int64_t p_r, int64_t p_c, int64_t d_r, int64_t d_c, int accumulate, void* stream) {
+    if (int rcx = reject_complex(dtype, "ntg_unfold2d_backward_dev")) return rcx;
     const int64_t es = ntg::elem_size(dtype);
     if (es == 0) return fail(NTG_ERR_UNSUPPORTED_DTYPE, "dtype %d is not supported", dtype);
     if (batch < 0 || channels < 0 || height < 0 || width < 0) return fail(NTG_ERR_INVALID_ARGUMENT, "negative size");
@@ -1285,6 +1301,7 @@ int ntg_unfold2d_backward(int dtype, const void* col, void* image,
                           int64_t batch, int64_t channels, int64_t height, int64_t width,
                           int64_t k_r, int64_t k_c, int64_t s_r, int64_t s_c,
                           int64_t p_r, int64_t p_c, int64_t d_r, int64_t d_c, int accumulate) {
+    if (int rcx = reject_complex(dtype, "ntg_unfold2d_backward")) return rcx;
     const int64_t es = ntg::elem_size(dtype);
     if (es == 0) return fail(NTG_ERR_UNSUPPORTED_DTYPE, "dtype %d is not supported", dtype);
     if (batch < 0 || channels < 0 || height < 0 || width < 0) return fail(NTG_ERR_INVALID_ARGUMENT, "negative size");
@@ -1332,6 +1349,7 @@ int ntg_conv2d_backward_dev(int dtype, const void* image, const void* kernel, co
                             int64_t out_channels, int64_t k_r, int64_t k_c,
                             int64_t s_r, int64_t s_c, int64_t p_r, int64_t p_c, int64_t d_r, int64_t d_c,
                             int64_t groups, int accumulate, void* stream) {
+    if (int rcx = reject_complex(dtype, "ntg_conv2d_backward_dev")) return rcx;
     const int64_t es = ntg::elem_size(dtype);
     if (es == 0) return fail(NTG_ERR_UNSUPPORTED_DTYPE, "dtype %d is not supported", dtype);
     if (batch < 0 || channels < 0 || out_channels < 0 || height < 0 || width < 0) return fail(NTG_ERR_INVALID_ARGUMENT, "negative size");
@@ -1360,7 +1378,7 @@ int ntg_conv2d_backward_dev(int dtype, const void* image, const void* kernel, co
     // 1x1 kernel, unit stride, no padding (floating dtypes, 16-byte rows): col is the image itself, so both gradients are
     // products on the tensors where they lie: dX_b = W_g^T . dY_b, and dW_g = sum_b dY_b . X_b^T through per-image results
     // in the workspace (the amount the gathering form needs), summed in batch order.
-    if (!is_int_dtype(dtype) && conv_pointwise_ok(dtype, channels, groups, geo) && (og * es) % 16 == 0 &&
+    if (!is_valu_dtype(dtype) && conv_pointwise_ok(dtype, channels, groups, geo) && (og * es) % 16 == 0 &&
         ((reinterpret_cast<uintptr_t>(image) | reinterpret_cast<uintptr_t>(kernel) | reinterpret_cast<uintptr_t>(grad_out) |
           reinterpret_cast<uintptr_t>(d_image) | reinterpret_cast<uintptr_t>(d_kernel) | reinterpret_cast<uintptr_t>(ws)) & 15) == 0) {
         const int64_t cg = channels / groups;
@@ -1484,6 +1502,7 @@ int ntg_conv_transpose2d_dev(int dtype, const void* input, const void* kernel, v
                              int64_t batch, int64_t in_channels, int64_t in_h, int64_t in_w, int64_t out_channels,
                              int64_t k_r, int64_t k_c, int64_t s_r, int64_t s_c, int64_t p_r, int64_t p_c, int64_t d_r, int64_t d_c,
                              int64_t op_r, int64_t op_c, int64_t groups, void* stream) {
+    if (int rcx = reject_complex(dtype, "ntg_conv_transpose2d_dev")) return rcx;
     if (ntg::elem_size(dtype) == 0) return fail(NTG_ERR_UNSUPPORTED_DTYPE, "dtype %d is not supported", dtype);
     if (batch < 0 || in_channels < 0 || out_channels < 0) return fail(NTG_ERR_INVALID_ARGUMENT, "negative size");
     if (groups < 1) return fail(NTG_ERR_INVALID_ARGUMENT, "groups must be >= 1");
@@ -1508,6 +1527,7 @@ int ntg_conv_transpose2d(int dtype, const void* input, const void* kernel, void*
                          int64_t batch, int64_t in_channels, int64_t in_h, int64_t in_w, int64_t out_channels,
                          int64_t k_r, int64_t k_c, int64_t s_r, int64_t s_c, int64_t p_r, int64_t p_c, int64_t d_r, int64_t d_c,
                          int64_t op_r, int64_t op_c, int64_t groups) {
+    if (int rcx = reject_complex(dtype, "ntg_conv_transpose2d")) return rcx;
     const int64_t es = ntg::elem_size(dtype);
     if (es == 0) return fail(NTG_ERR_UNSUPPORTED_DTYPE, "dtype %d is not supported", dtype);
     if (batch < 0 || in_channels < 0 || out_channels < 0) return fail(NTG_ERR_INVALID_ARGUMENT, "negative size");
@@ -1543,6 +1563,7 @@ int ntg_conv2d_backward(int dtype, const void* image, const void* kernel, const 
                         int64_t out_channels, int64_t k_r, int64_t k_c,
                         int64_t s_r, int64_t s_c, int64_t p_r, int64_t p_c, int64_t d_r, int64_t d_c,
                         int64_t groups, int accumulate) {
+    if (int rcx = reject_complex(dtype, "ntg_conv2d_backward")) return rcx;
     const int64_t es = ntg::elem_size(dtype);
     if (es == 0) return fail(NTG_ERR_UNSUPPORTED_DTYPE, "dtype %d is not supported", dtype);
     if (batch < 0 || channels < 0 || out_channels < 0 || height < 0 || width < 0) return fail(NTG_ERR_INVALID_ARGUMENT, "negative size");
@@ -1634,6 +1655,7 @@ int ntg_unfoldnd_dev(int dtype, const void* image, void* col, int64_t batch, int
 int ntg_unfoldnd_backward_dev(int dtype, const void* col, void* image, int64_t batch, int64_t channels, int ndim, const int64_t* size,
                               const int64_t* kernel_size, const int64_t* stride, const int64_t* padding, const int64_t* dilation,
                               int accumulate, void* stream) {
+    if (int rcx = reject_complex(dtype, "ntg_unfoldnd_backward_dev")) return rcx;
     if (ntg::elem_size(dtype) == 0) return fail(NTG_ERR_UNSUPPORTED_DTYPE, "dtype %d is not supported", dtype);
     ntg::UnfoldNdParams u;
     int rc = fill_nd(u, batch, channels, ndim, size, kernel_size, stride, padding, dilation);
@@ -1687,6 +1709,7 @@ int ntg_convnd_dev(int dtype, const void* image, const void* kernel, void* out, 
         return ntg_conv2d_dev(dtype, image, kernel, out, workspace, workspace_bytes, batch, channels, g.h, g.w, out_channels, g.kr, g.kc,
                               g.sr, g.sc, g.pr, g.pc, g.dr, g.dc, groups, stream);
     }
+    if (int rcx = reject_complex(dtype, "a convolution over three or more axes")) return rcx;
     if (batch == 0 || out_channels == 0) return NTG_OK;
     if (!image || !kernel || !out) return fail(NTG_ERR_INVALID_ARGUMENT, "null pointer");
     if (ndim == 3) {
@@ -1720,6 +1743,7 @@ int ntg_convnd_backward_dev(int dtype, const void* image, const void* kernel, co
                             void* workspace, int64_t workspace_bytes, int64_t batch, int64_t channels, int64_t out_channels, int ndim,
                             const int64_t* size, const int64_t* kernel_size, const int64_t* stride, const int64_t* padding,
                             const int64_t* dilation, int64_t groups, int accumulate, void* stream) {
+    if (int rcx = reject_complex(dtype, "ntg_convnd_backward_dev")) return rcx;
     const int64_t es = ntg::elem_size(dtype);
     if (es == 0) return fail(NTG_ERR_UNSUPPORTED_DTYPE, "dtype %d is not supported", dtype);
     int rc = check_groups(channels, out_channels, groups);
@@ -1827,6 +1851,7 @@ int ntg_conv_transposend_dev(int dtype, const void* input, const void* kernel, v
                              int64_t batch, int64_t in_channels, int64_t out_channels, int ndim, const int64_t* in_size,
                              const int64_t* kernel_size, const int64_t* stride, const int64_t* padding, const int64_t* dilation,
                              const int64_t* output_padding, int64_t groups, void* stream) {
+    if (int rcx = reject_complex(dtype, "ntg_conv_transposend_dev")) return rcx;
     if (ntg::elem_size(dtype) == 0) return fail(NTG_ERR_UNSUPPORTED_DTYPE, "dtype %d is not supported", dtype);
     int rc = check_groups(in_channels, out_channels, groups);
     if (rc) return rc;
@@ -1875,6 +1900,7 @@ int ntg_convnd(int dtype, const void* image, const void* kernel, void* out, int6
 int ntg_convnd_backward(int dtype, const void* image, const void* kernel, const void* grad_out, void* d_image, void* d_kernel,
                         int64_t batch, int64_t channels, int64_t out_channels, int ndim, const int64_t* size, const int64_t* kernel_size,
                         const int64_t* stride, const int64_t* padding, const int64_t* dilation, int64_t groups, int accumulate) {
+    if (int rcx = reject_complex(dtype, "ntg_convnd_backward")) return rcx;
     const int64_t es = ntg::elem_size(dtype);
     if (es == 0) return fail(NTG_ERR_UNSUPPORTED_DTYPE, "dtype %d is not supported", dtype);
     int rc = check_groups(channels, out_channels, groups);
@@ -1908,6 +1934,7 @@ int ntg_convnd_backward(int dtype, const void* image, const void* kernel, const 
 int ntg_conv_transposend(int dtype, const void* input, const void* kernel, void* out, int64_t batch, int64_t in_channels, int64_t out_channels,
                          int ndim, const int64_t* in_size, const int64_t* kernel_size, const int64_t* stride, const int64_t* padding,
                          const int64_t* dilation, const int64_t* output_padding, int64_t groups) {
+    if (int rcx = reject_complex(dtype, "ntg_conv_transposend")) return rcx;
     const int64_t es = ntg::elem_size(dtype);
     if (es == 0) return fail(NTG_ERR_UNSUPPORTED_DTYPE, "dtype %d is not supported", dtype);
     int rc = check_groups(in_channels, out_channels, groups);

@@ -8,6 +8,13 @@
 
 namespace ntg {
 
+// a 16-byte element that is only moved (Complex128)
+struct alignas(16) Bytes16 {
+    uint64_t lo, hi;
+    __host__ __device__ Bytes16() = default;
+    __host__ __device__ Bytes16(int) : lo(0), hi(0) {}
+};
+
 struct UnfoldParams {
     int64_t batch, channels, height, width;
     int64_t k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c;
@@ -224,6 +231,7 @@ hipError_t launch_unfoldnd(int64_t es, const void* im, void* col, const UnfoldNd
     case 2: hipLaunchKernelGGL(unfoldnd_kernel<uint16_t>, g, b, 0, s, (const uint16_t*)im, (uint16_t*)col, u); break;
     case 4: hipLaunchKernelGGL(unfoldnd_kernel<uint32_t>, g, b, 0, s, (const uint32_t*)im, (uint32_t*)col, u); break;
     case 8: hipLaunchKernelGGL(unfoldnd_kernel<uint64_t>, g, b, 0, s, (const uint64_t*)im, (uint64_t*)col, u); break;
+    case 16: hipLaunchKernelGGL(unfoldnd_kernel<Bytes16>, g, b, 0, s, (const Bytes16*)im, (Bytes16*)col, u); break;
     default: return hipErrorInvalidValue;
     }
     return hipGetLastError();
@@ -324,7 +332,7 @@ hipError_t launch_unfold2d(int64_t es, const void* im, void* col,
         // 16-byte stores when every row of col is a whole number of vectors and all sizes fit 32-bit arithmetic
         const int64_t L = u.Ho * u.Wo, V = 16 / es, rows = batch * u.ccol;
         const int64_t lim = 1 << 24;
-        if (L % V == 0 && (reinterpret_cast<uintptr_t>(col) & 15) == 0 && L < 0x7fffffffLL && rows < 0x7fffffffLL &&
+        if (es < 16 && L % V == 0 && (reinterpret_cast<uintptr_t>(col) & 15) == 0 && L < 0x7fffffffLL && rows < 0x7fffffffLL &&
             height < lim && width < lim && k_r * d_r < lim && k_c * d_c < lim && u.Ho * s_r < lim && u.Wo * s_c < lim && p_r < lim && p_c < lim &&
             p_r > -lim && p_c > -lim && u.ccol < 0x7fffffffLL) {
             UnfoldVecParams q;
@@ -356,6 +364,7 @@ hipError_t launch_unfold2d(int64_t es, const void* im, void* col,
     case 2: hipLaunchKernelGGL(unfold2d_kernel<uint16_t>, dim3((unsigned)blocks), dim3(256), 0, s, (const uint16_t*)im, (uint16_t*)col, u); break;
     case 4: hipLaunchKernelGGL(unfold2d_kernel<uint32_t>, dim3((unsigned)blocks), dim3(256), 0, s, (const uint32_t*)im, (uint32_t*)col, u); break;
     case 8: hipLaunchKernelGGL(unfold2d_kernel<uint64_t>, dim3((unsigned)blocks), dim3(256), 0, s, (const uint64_t*)im, (uint64_t*)col, u); break;
+    case 16: hipLaunchKernelGGL(unfold2d_kernel<Bytes16>, dim3((unsigned)blocks), dim3(256), 0, s, (const Bytes16*)im, (Bytes16*)col, u); break;
     default: return hipErrorInvalidValue;
     }
     return hipGetLastError();

@@ -25,6 +25,7 @@ const char* dtype_name(DType dt) {
     case DType::BFloat16: return "BFloat16"; case DType::int8: return "int8"; case DType::int16: return "int16";
     case DType::int32: return "int32"; case DType::int64: return "int64"; case DType::uint8: return "uint8";
     case DType::uint16: return "uint16"; case DType::uint32: return "uint32"; case DType::uint64: return "uint64";
+    case DType::Complex32: return "Complex32"; case DType::Complex64: return "Complex64"; case DType::Complex128: return "Complex128";
     case DType::Bool: return "Bool"; case DType::TensorObj: return "TensorObj";
     default: return "unsupported";
     }
@@ -201,6 +202,21 @@ Tensor Tensor::item(int64_t i) const {
     return out;
 }
 
+TensorList Tensor::split_axis(int64_t axis) const {
+    utils::throw_exception(!is_null() && is_contiguous() && dims() >= 2, "split_axis needs a contiguous tensor of two or more dimensions");
+    utils::throw_exception(axis == 0, "nt_compat splits along axis 0 only");
+    TensorList out;
+    const int64_t per = numel() / std::max<int64_t>(shape_[0], 1);
+    for (int64_t i = 0; i < shape_[0]; ++i) {
+        Tensor t = *this;
+        t.offset_ = offset_ + i * per * dtype_size(dtype_);
+        t.shape_.assign(shape_.begin() + 1, shape_.end());
+        t.strides_ = dense_strides(t.shape_);
+        out.push_back(std::move(t));
+    }
+    return out;
+}
+
 template <class T>
 static void sum_as_t(const Tensor& src, Tensor& dst, const SizeRef& tgt_padded) {
     // src contiguous with shape S; dst contiguous with shape tgt_padded (same rank, dims equal or 1)
@@ -290,6 +306,23 @@ static uint16_t f32_to_bf16(float f) {
     return (uint16_t)(x >> 16);
 }
 
+// binary16 <- binary32, round to nearest even
+static uint16_t f32_to_f16(float f) {
+    uint32_t x;
+    std::memcpy(&x, &f, 4);
+    const uint32_t sign = (x >> 16) & 0x8000u, ax = x & 0x7fffffffu;
+    if (ax >= 0x7f800000u) return (uint16_t)(sign | (ax > 0x7f800000u ? 0x7e00u : 0x7c00u));
+    if (ax >= 0x477ff000u) return (uint16_t)(sign | 0x7c00u);
+    if (ax < 0x33000001u) return (uint16_t)sign;
+    const int32_t e = (int32_t)(ax >> 23) - 127;
+    const uint32_t man = (ax & 0x7fffffu) | 0x800000u;
+    const uint32_t shift = e < -14 ? (uint32_t)(13 + (-14 - e)) : 13u, half_exp = e < -14 ? 0u : (uint32_t)(e + 15);
+    uint32_t q = man >> shift;
+    const uint32_t rem = man & ((1u << shift) - 1u), halfway = 1u << (shift - 1);
+    if (rem > halfway || (rem == halfway && (q & 1u))) ++q;
+    return (uint16_t)(sign | (half_exp == 0 ? q : ((half_exp - 1) << 10) + q));
+}
+
 Tensor randn(SizeRef shape, DType dt, uint64_t seed) {
     Tensor t(std::move(shape), dt);
     std::mt19937_64 gen(seed ? seed : 0x9e3779b97f4a7c15ull);
@@ -299,6 +332,10 @@ Tensor randn(SizeRef shape, DType dt, uint64_t seed) {
     case DType::Float32: for (int64_t i = 0; i < n; ++i) t.data<float>()[i] = (float)nd(gen); break;
     case DType::Float64: for (int64_t i = 0; i < n; ++i) t.data<double>()[i] = nd(gen); break;
     case DType::BFloat16: for (int64_t i = 0; i < n; ++i) t.data<uint16_t>()[i] = f32_to_bf16((float)nd(gen)); break;
+    case DType::Float16: for (int64_t i = 0; i < n; ++i) t.data<uint16_t>()[i] = f32_to_f16((float)nd(gen)); break;
+    case DType::Complex32: for (int64_t i = 0; i < 2 * n; ++i) t.data<uint16_t>()[i] = f32_to_f16((float)nd(gen)); break;
+    case DType::Complex64: for (int64_t i = 0; i < 2 * n; ++i) t.data<float>()[i] = (float)nd(gen); break;
+    case DType::Complex128: for (int64_t i = 0; i < 2 * n; ++i) t.data<double>()[i] = nd(gen); break;
     case DType::int32: for (int64_t i = 0; i < n; ++i) t.data<int32_t>()[i] = (int32_t)std::lround(nd(gen) * 4.0); break;
     case DType::int64: for (int64_t i = 0; i < n; ++i) t.data<int64_t>()[i] = (int64_t)std::lround(nd(gen) * 4.0); break;
     default: utils::throw_exception(false, std::string("randn is not available for ") + dtype_name(dt));
@@ -532,6 +569,79 @@ Tensor& matmult(const Tensor& a, const Tensor& b, Tensor& c, bool trans_a, bool 
 }
 
 Tensor matmult_cT(const Tensor& a, const Tensor& b) { return functional::matmult(a, b, false, true); }   // tensor_files/matmult.cpp:38
+
+// Tensors of tensors: subT_check (matmult_cpu.cpp:1556-1566), handle_dim_{n_n,n_k,k_n}_subT_matmult_std (:1240-1485).
+// Every pair (a[i], b[i]) follows the N-D x K-D rule; all matrices of all pairs go out as one nt_matmult_batch, the
+// lower-rank side's matrices repeated by handle (return_split_tensor_of_tensors_repeat).
+Tensor matmult(const TensorList& a, const TensorList& b, bool trans_a, bool trans_b) {
+    utils::throw_exception(a.size() == b.size(), "Expected both tensors to have the same number of sub-tensors, going to have these multiplied in a "
+                                                 "list-like fashion, but got " + std::to_string(a.size()) + " and " + std::to_string(b.size()) + " tensors");
+    utils::throw_exception(!a.empty(), "Cannot perform operation matmult on an empty list of tensors");
+    const int64_t L = (int64_t)a.size();
+    // the first pair fixes the shapes, the flags and every check; the others must look the same (nt_matmult_batch is uniform)
+    const MatmultPlan p0 = plan_matmult(a[0], b[0], trans_a, trans_b, false);
+    std::vector<const Tensor*> all;
+    for (const Tensor& t : a) all.push_back(&t);
+    for (const Tensor& t : b) all.push_back(&t);
+    DeviceType dev = a[0].device();
+    for (const Tensor* t : all) {
+        utils::throw_exception(!t->is_null(), "Cannot perform operation matmult on a null tensor");
+        utils::throw_exception(t->device() == dev, "Expected all tensors of matmult to be on the same device");
+    }
+    std::vector<Tensor> as, bs;
+    for (int64_t i = 0; i < L; ++i) {
+        utils::throw_exception(a[(size_t)i].shape() == a[0].shape() && b[(size_t)i].shape() == b[0].shape() && a[(size_t)i].dtype() == a[0].dtype() &&
+                                   b[(size_t)i].dtype() == b[0].dtype(),
+                               "Expected the sub-tensors of one list to share one shape and dtype, item " + std::to_string(i) + " differs");
+        bool ta = trans_a, tb = trans_b;
+        Tensor sa = matrix_storage(a[(size_t)i], ta), sb = matrix_storage(b[(size_t)i], tb);
+        utils::throw_exception(ta == p0.ta && tb == p0.tb,
+                               "Expected the sub-tensors of one list to share one memory layout (all contiguous or all transposed views)");
+        as.push_back(sa);
+        bs.push_back(sb);
+    }
+    SizeRef out_shape = p0.out_shape;                              // the higher-rank item's batch dims + [m, n]
+    out_shape[0] *= L;                                             // bigger_shape_vec[0] *= a.numel() (:1264, :1363); pairs of plain
+                                                                   // matrices: the L results stacked along the rows
+    const int64_t es = dtype_size(a[0].dtype()), total = L * p0.nbig;
+    const int dt = static_cast<int>(a[0].dtype());
+    if (dev == DeviceType::HIP) {
+        Tensor c(out_shape, a[0].dtype(), DeviceType::HIP);
+        if (total == 0 || p0.m == 0 || p0.n == 0) return c;
+        if (p0.k == 0) return zeros(out_shape, a[0].dtype(), DeviceType::HIP);
+        std::vector<const void*> tab((size_t)(3 * total));
+        for (int64_t i = 0; i < L; ++i)
+            for (int64_t j = 0; j < p0.nbig; ++j) {
+                const int64_t t = i * p0.nbig + j;
+                tab[(size_t)t] = static_cast<const char*>(as[(size_t)i].data_ptr()) + (j % p0.na) * p0.m * p0.k * es;
+                tab[(size_t)(total + t)] = static_cast<const char*>(bs[(size_t)i].data_ptr()) + (j % p0.nb) * p0.k * p0.n * es;
+                tab[(size_t)(2 * total + t)] = static_cast<char*>(c.data_ptr()) + t * p0.m * p0.n * es;
+            }
+        std::shared_ptr<char> dtab = device_alloc(tab.size() * sizeof(void*));
+        hip_check(hipMemcpy(dtab.get(), tab.data(), tab.size() * sizeof(void*), hipMemcpyHostToDevice), "hipMemcpy (pointer tables)");
+        ntg_gemm_desc d;
+        std::memset(&d, 0, sizeof d);
+        d.dtype = dt; d.transpose_a = p0.ta; d.transpose_b = p0.tb; d.c_mode = NTG_C_OVERWRITE;
+        d.m = p0.m; d.k = p0.k; d.n = p0.n; d.batches = total;
+        void** T = reinterpret_cast<void**>(dtab.get());
+        check_status(ntg_gemm_ptrs_dev(&d, T, T + total, T + 2 * total, nullptr));
+        hip_check(hipStreamSynchronize(nullptr), "hipStreamSynchronize");      // the table is freed on return
+        return c;
+    }
+    Tensor c = zeros(out_shape, a[0].dtype());
+    if (total == 0 || p0.m == 0 || p0.n == 0 || p0.k == 0) return c;
+    std::vector<const void*> pa((size_t)total), pb((size_t)total);
+    std::vector<void*> pc((size_t)total);
+    for (int64_t i = 0; i < L; ++i)
+        for (int64_t j = 0; j < p0.nbig; ++j) {
+            const int64_t t = i * p0.nbig + j;
+            pa[(size_t)t] = static_cast<const char*>(as[(size_t)i].data_ptr()) + (j % p0.na) * p0.m * p0.k * es;
+            pb[(size_t)t] = static_cast<const char*>(bs[(size_t)i].data_ptr()) + (j % p0.nb) * p0.k * p0.n * es;
+            pc[(size_t)t] = static_cast<char*>(c.data_ptr()) + t * p0.m * p0.n * es;
+        }
+    check_status(ntg_matmult_batch(dt, pa.data(), pb.data(), pc.data(), total, p0.m, p0.k, p0.k, p0.n, p0.ta, p0.tb));
+    return c;
+}
 
 Tensor linear(const Tensor& x_in, const Tensor& w_in, const Tensor& b_in, bool trans_a, bool trans_b) {
     utils::throw_exception(!x_in.is_null() && !w_in.is_null() && !b_in.is_null(), "Cannot perform operation linear on a null tensor");

@@ -45,6 +45,10 @@ template <size_t N> using my_n_tuple = std::array<int64_t, N>;
 }  // namespace utils
 
 using SizeRef = std::vector<int64_t>;
+class Tensor;
+// A list of tensors: what the reference holds as a 1-D tensor of DType::TensorObj (Tensor::split_axis,
+// nt/functional/cpu/matmult_cpu.cpp:1240-1485 multiply two of them item by item)
+using TensorList = std::vector<Tensor>;
 std::string shape_str(const SizeRef& s);
 
 // nt/memory/DeviceEnum.h:6-10 with the device this backend adds
@@ -82,6 +86,7 @@ public:
     Tensor transpose(int64_t a, int64_t b) const;                 // strided view, no copy
     Tensor unsqueeze_front(int64_t n) const;                      // prepend n dims of 1
     Tensor item(int64_t batch_index) const;                       // i-th matrix of a contiguous [.., r, c] tensor
+    TensorList split_axis(int64_t axis) const;                    // axis 0 of a contiguous tensor: its shape[0] slices, as views
     Tensor sum_leading(const SizeRef& target_shape) const;        // reduce broadcast dims back (sum_as)
     template <class T> T* data() { return reinterpret_cast<T*>(data_ptr()); }
     template <class T> const T* data() const { return reinterpret_cast<const T*>(data_ptr()); }
@@ -97,13 +102,18 @@ private:
 
 namespace functional {
 Tensor zeros(SizeRef shape, DType dt = DType::Float32, DeviceType dev = DeviceType::CPU);
-Tensor randn(SizeRef shape, DType dt = DType::Float32, uint64_t seed = 0);   // seeded N(0,1) (the reference's randn is unseeded)
+Tensor randn(SizeRef shape, DType dt = DType::Float32, uint64_t seed = 0);   // seeded N(0,1) (the reference's randn is unseeded); complex: both parts
 Tensor from_numpy(const std::string& path);                                   // .npy, C order, f2/f4/f8/i1/i2/i4/i8/u1
 bool allclose(const Tensor& a, const Tensor& b, double rtol = 1e-5, double atol = 1e-8);   // compare.h:34
 
 Tensor matmult(const Tensor& a, const Tensor& b, bool trans_a = false, bool trans_b = false);
 Tensor& matmult(const Tensor& a, const Tensor& b, Tensor& c, bool trans_a = false, bool trans_b = false);
 Tensor matmult_cT(const Tensor& a, const Tensor& b);
+// Tensors of tensors (matmult_cpu.cpp:1240-1485, dispatched at :1576-1580): two lists of equal length are multiplied item by
+// item in ONE nt_matmult_batch over all their matrices; items of one list share shape and dtype, the lower-rank side's
+// matrices repeat under the higher-rank side's (the N-D x K-D rule inside every pair).  The result is one tensor: the
+// higher-rank item's shape with its first dimension multiplied by the list length and the last two replaced by [m, n].
+Tensor matmult(const TensorList& a, const TensorList& b, bool trans_a = false, bool trans_b = false);
 Tensor linear(const Tensor& input, const Tensor& weight, const Tensor& bias, bool trans_input = false, bool trans_weight = false);
 Tensor unfold2d(const Tensor& x, utils::my_tuple kernel_size, utils::my_tuple dilation = {1, 1}, utils::my_tuple padding = {0, 0},
                 utils::my_tuple stride = {1, 1}, bool transpose_out = true);
@@ -157,6 +167,9 @@ inline Tensor matmult(const Tensor& input, const Tensor& other, bool transpose_a
 }
 inline Tensor& matmult(const Tensor& input, const Tensor& other, Tensor& out, bool transpose_a = false, bool transpose_b = false) {
     return functional::matmult(input, other, out, transpose_a, transpose_b);
+}
+inline Tensor matmult(const TensorList& input, const TensorList& other, bool transpose_a = false, bool transpose_b = false) {
+    return functional::matmult(input, other, transpose_a, transpose_b);
 }
 inline Tensor linear(const Tensor& input, const Tensor& weight, const Tensor& bias, bool transpose_a = false, bool transpose_b = false) {
     return functional::linear(input, weight, bias, transpose_a, transpose_b);

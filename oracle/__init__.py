@@ -28,6 +28,8 @@ F16, F32, F64 = 0, 1, 2
 I8, I16, I32, I64 = 7, 8, 9, 10
 U8, U16, U32 = 12, 13, 14
 BF16, U64 = 100, 101
+C32, C64, C128 = 4, 5, 6          # interleaved (re, im) pairs; numpy carries them as real arrays with a trailing axis of 2
+_COMPLEX_REAL = {C32: np.dtype(np.float16), C64: np.dtype(np.float32), C128: np.dtype(np.float64)}
 
 _NP_TO_DT = {
     np.dtype(np.float16): F16, np.dtype(np.float32): F32, np.dtype(np.float64): F64,
@@ -130,6 +132,25 @@ def matmult2d(a, b, c=None, ta=False, tb=False, dt=None, kind="closed", threads=
         raise ValueError(kind)
     if rc:
         raise RuntimeError(f"oracle matmult failed rc={rc}")
+    return c
+
+
+def matmult2d_complex(a, b, c=None, ta=False, tb=False, dt=C64, kind="closed"):
+    """The reference's complex matmult (lane-wise on interleaved re / im, see closed_c64 in nt_oracle.c) on arrays
+    [rows, cols, 2] of the real type (float16 for C32, float32 for C64, float64 for C128)."""
+    real = _COMPLEX_REAL[dt]
+    a = np.ascontiguousarray(a, dtype=real)
+    b = np.ascontiguousarray(b, dtype=real)
+    assert a.ndim == 3 and b.ndim == 3 and a.shape[2] == 2 and b.shape[2] == 2
+    m, k, n = _mkn(a.shape[:2], b.shape[:2], ta, tb)
+    if c is None:
+        c = np.zeros((m, n, 2), dtype=real)
+    assert c.flags["C_CONTIGUOUS"] and c.shape == (m, n, 2) and c.dtype == real
+    L = lib()
+    fn = L.oracle_matmult if kind == "closed" else L.oracle_matmult_naive
+    rc = fn(dt, _ptr(a), _ptr(b), _ptr(c), m, k, n, int(ta), int(tb))
+    if rc:
+        raise RuntimeError(f"oracle complex matmult failed rc={rc}")
     return c
 
 

@@ -91,6 +91,9 @@ int64_t oracle_elem_size(int dt) {
     case OR_F16: case OR_BF16: case OR_I16: case OR_U16: return 2;
     case OR_F32: case OR_I32: case OR_U32: return 4;
     case OR_F64: case OR_I64: case OR_U64: return 8;
+    case OR_C32: return 4;
+    case OR_C64: return 8;
+    case OR_C128: return 16;
     default: return 0;
     }
 }
@@ -206,6 +209,63 @@ CLOSED_INT(closed_u16, uint16_t)
 CLOSED_INT(closed_u32, uint32_t)
 CLOSED_INT(closed_u64, uint64_t)
 
+/* Complex types.  The reference runs them through the SAME generic micro kernel
+ * (nt_matmult_simde.hpp:301-350): a C tile row is two vectors of interleaved
+ * (re, im) lanes; broadcast(A + kk) = set1(a) fills a vector with (a.re, a.im,
+ * a.re, a.im, ...) (simde_traits_avx2.h:928-937 complex_64, :1037-1044
+ * complex_128, :1285-1294 and :1365 complex_32 -- set_ps lists lanes from the
+ * highest down, so lane 2t holds re and lane 2t+1 im, the memory order of
+ * my_complex {re, im}, nt/types/complex.h:109); fmadd is the plain lane-wise
+ * _mm256_fmadd_ps / _pd (:996-1002, :1106-1112, :1367-1373).  Hence per element
+ *     c.re = fma(a.re, b.re, c.re);   c.im = fma(a.im, b.im, c.im)
+ * for kk ascending: two independent real products, one on the real parts and
+ * one on the imaginary parts -- NOT the complex product.  complex_32 keeps
+ * float lanes inside a k tile of 2 * pack_size = 8 (pack_size 4, :1275) and
+ * converts half <-> float at the tile's load / store (:1276-1303), so it rounds
+ * to half every 8 k.  No test of the reference pins a complex matmult value:
+ * parity unpinned by any reference fixture; the restatement follows the code. */
+static void closed_c64(const float* A, const float* Bkn, float* C, int64_t m, int64_t k, int64_t n, int ta) {
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < m; ++i) {
+        float* c = C + 2 * i * n;
+        for (int64_t kk = 0; kk < k; ++kk) {
+            const float* a = A + 2 * A_IDX(i, kk);
+            const float* b = Bkn + 2 * kk * n;
+            for (int64_t j = 0; j < 2 * n; ++j) c[j] = fmaf(a[j & 1], b[j], c[j]);
+        }
+    }
+}
+static void closed_c128(const double* A, const double* Bkn, double* C, int64_t m, int64_t k, int64_t n, int ta) {
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < m; ++i) {
+        double* c = C + 2 * i * n;
+        for (int64_t kk = 0; kk < k; ++kk) {
+            const double* a = A + 2 * A_IDX(i, kk);
+            const double* b = Bkn + 2 * kk * n;
+            for (int64_t j = 0; j < 2 * n; ++j) c[j] = fma(a[j & 1], b[j], c[j]);
+        }
+    }
+}
+static void closed_c32(const uint16_t* A, const uint16_t* Bkn, uint16_t* C, int64_t m, int64_t k, int64_t n, int ta) {
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < m; ++i) {
+        float* acc = (float*)malloc((size_t)(2 * n) * sizeof(float));
+        uint16_t* c = C + 2 * i * n;
+        for (int64_t k0 = 0; k0 < k; k0 += 8) {
+            const int64_t k1 = (k0 + 8 < k) ? k0 + 8 : k;
+            for (int64_t j = 0; j < 2 * n; ++j) acc[j] = oracle_f16_to_f32(c[j]);
+            for (int64_t kk = k0; kk < k1; ++kk) {
+                const uint16_t* a = A + 2 * A_IDX(i, kk);
+                const float av[2] = {oracle_f16_to_f32(a[0]), oracle_f16_to_f32(a[1])};
+                const uint16_t* b = Bkn + 2 * kk * n;
+                for (int64_t j = 0; j < 2 * n; ++j) acc[j] = fmaf(av[j & 1], oracle_f16_to_f32(b[j]), acc[j]);
+            }
+            for (int64_t j = 0; j < 2 * n; ++j) c[j] = oracle_f32_to_f16(acc[j]);
+        }
+        free(acc);
+    }
+}
+
 int oracle_matmult(int dt, const void* A, const void* B, void* C,
                    int64_t m, int64_t k, int64_t n, int ta, int tb) {
     const int64_t es = oracle_elem_size(dt);
@@ -221,6 +281,9 @@ int oracle_matmult(int dt, const void* A, const void* B, void* C,
     case OR_I16: case OR_U16: closed_u16((const uint16_t*)A, (const uint16_t*)Bkn, (uint16_t*)C, m, k, n, ta); break;
     case OR_I32: case OR_U32: closed_u32((const uint32_t*)A, (const uint32_t*)Bkn, (uint32_t*)C, m, k, n, ta); break;
     case OR_I64: case OR_U64: closed_u64((const uint64_t*)A, (const uint64_t*)Bkn, (uint64_t*)C, m, k, n, ta); break;
+    case OR_C64: closed_c64((const float*)A, (const float*)Bkn, (float*)C, m, k, n, ta); break;
+    case OR_C128: closed_c128((const double*)A, (const double*)Bkn, (double*)C, m, k, n, ta); break;
+    case OR_C32: closed_c32((const uint16_t*)A, (const uint16_t*)Bkn, (uint16_t*)C, m, k, n, ta); break;
     default: if (tb) free(Bkn); return -1;
     }
     if (tb) free(Bkn);
@@ -290,6 +353,35 @@ int oracle_matmult_naive(int dt, const void* A, const void* B, void* C,
                 }
                 c_[i * n + j] = oracle_f32_to_bf16(acc);
             }
+        return 0;
+    }
+    case OR_C64: case OR_C128: case OR_C32: {
+        /* the literal loop on (re, im) pairs; complex_32 in k tiles of 8 */
+        for (int64_t i = 0; i < m; ++i)
+            for (int64_t j = 0; j < n; ++j)
+                for (int c = 0; c < 2; ++c) {
+                    const int64_t ci = 2 * (i * n + j) + c;
+                    if (dt == OR_C64) {
+                        float acc = ((float*)C)[ci];
+                        for (int64_t kk = 0; kk < k; ++kk)
+                            acc = fmaf(((const float*)A)[2 * (ta ? kk * m + i : i * k + kk) + c], ((const float*)B)[2 * (tb ? j * k + kk : kk * n + j) + c], acc);
+                        ((float*)C)[ci] = acc;
+                    } else if (dt == OR_C128) {
+                        double acc = ((double*)C)[ci];
+                        for (int64_t kk = 0; kk < k; ++kk)
+                            acc = fma(((const double*)A)[2 * (ta ? kk * m + i : i * k + kk) + c], ((const double*)B)[2 * (tb ? j * k + kk : kk * n + j) + c], acc);
+                        ((double*)C)[ci] = acc;
+                    } else {
+                        uint16_t* c_ = (uint16_t*)C;
+                        for (int64_t k0 = 0; k0 < k; k0 += 8) {
+                            float acc = oracle_f16_to_f32(c_[ci]);
+                            for (int64_t kk = k0; kk < k0 + 8 && kk < k; ++kk)
+                                acc = fmaf(oracle_f16_to_f32(((const uint16_t*)A)[2 * (ta ? kk * m + i : i * k + kk) + c]),
+                                           oracle_f16_to_f32(((const uint16_t*)B)[2 * (tb ? j * k + kk : kk * n + j) + c]), acc);
+                            c_[ci] = oracle_f32_to_f16(acc);
+                        }
+                    }
+                }
         return 0;
     }
     default: return -1;

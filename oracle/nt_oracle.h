@@ -28,6 +28,14 @@
  *   fp16 GEMM       <- numpy float16 rounding of an independently computed
  *       chunked sum (16-wide k tiles), software half conversion checked
  *       against numpy for all 65536 bit patterns.
+ *   complex GEMM    <- parity unpinned by any reference fixture (none holds a complex
+ *       matmult value).  The reference's generic micro kernel multiplies the
+ *       interleaved (re, im) lanes element-wise (simde_traits_avx2.h:928-937,
+ *       :996-1002): the result is one real product of the real parts and one
+ *       of the imaginary parts, not the complex product.  Pinned by that
+ *       reduction (bitwise equal to the real oracle on the two planes), by a
+ *       literal vector-lane walk of the micro kernel on tiny inputs, and, for
+ *       complex_32, by an independent numpy restatement of the 8-wide k tiles.
  *   bf16 GEMM       <- parity unpinned: the reference has no BFloat16 DType
  *       (nt/types/bfloat16.h:4-5); this build defines it (fp32 accumulate over
  *       all K, one round-to-nearest-even at the end).
@@ -44,6 +52,7 @@ extern "C" {
  * nt/dtype/compatible/DTypeDeclareMacros.h:5-33); BF16/U64 are extensions. */
 enum oracle_dtype {
     OR_F16 = 0, OR_F32 = 1, OR_F64 = 2,
+    OR_C32 = 4, OR_C64 = 5, OR_C128 = 6,      /* interleaved (re, im) pairs of half / float / double */
     OR_I8 = 7, OR_I16 = 8, OR_I32 = 9, OR_I64 = 10,
     OR_U8 = 12, OR_U16 = 13, OR_U32 = 14,
     OR_BF16 = 100, OR_U64 = 101

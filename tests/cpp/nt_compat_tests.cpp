@@ -99,7 +99,7 @@ static void host_only_cases() {
     expect_throw("matmult dtype mismatch", [] { nt::matmult(F::zeros({4, 4}), F::zeros({4, 4}, DType::Float64)); });
     expect_throw("matmult batch dims do not line up", [] { nt::matmult(F::zeros({2, 3, 4, 4}), F::zeros({2, 4, 4})); });
     expect_throw("matmult null operand", [] { nt::matmult(Tensor::Null(), F::zeros({4, 4})); });
-    expect_throw("matmult unsupported dtype", [] { Tensor t; nt::matmult(Tensor({2, 2}, DType::Complex64), Tensor({2, 2}, DType::Complex64)); });
+    expect_throw("matmult unsupported dtype", [] { Tensor t; nt::matmult(Tensor({2, 2}, DType::Float128), Tensor({2, 2}, DType::Float128)); });
     expect_throw("matmult out wrong shape", [] { Tensor c = F::zeros({4, 5}); nt::matmult(F::zeros({4, 4}), F::zeros({4, 4}), c); });
     expect_throw("matmult out wrong dtype", [] { Tensor c = F::zeros({4, 4}, DType::Float64); nt::matmult(F::zeros({4, 4}), F::zeros({4, 4}), c); });
     expect_throw("matmult out immutable", [] { Tensor c = F::zeros({4, 4}); c.set_mutability(false); nt::matmult(F::zeros({4, 4}), F::zeros({4, 4}), c); });
@@ -156,6 +156,69 @@ static void device_cases(const std::string& g) {
             Tensor oi = nt::matmult(a.item(i).clone(), b.item(i).clone());
             nt::utils::throw_exception(std::memcmp(oi.data_ptr(), o.item(i).data_ptr(), 9 * sizeof(float)) == 0, "item differs");
         }
+    });
+    // tests/src/matmult_test.cpp:108-189: two lists of tensors multiplied item by item in one batch == per-item products, bit for bit
+    struct ListCase { const char* name; SizeRef as, bs; bool ta, tb; SizeRef view; };
+    for (const ListCase& lc : {ListCase{"matmult tensors (no bigger)", {5, 2, 3, 4}, {5, 2, 4, 3}, false, false, {5, 2, 3, 3}},
+                               ListCase{"matmult tensors Ta", {5, 2, 4, 3}, {5, 2, 4, 3}, true, false, {5, 2, 3, 3}},
+                               ListCase{"matmult tensors Tb", {5, 2, 4, 3}, {5, 2, 4, 3}, false, true, {5, 2, 4, 4}},
+                               ListCase{"matmult tensors Ta (bigger a)", {5, 2, 4, 3}, {5, 4, 3}, true, false, {5, 2, 3, 3}},
+                               ListCase{"matmult tensors Tb (bigger a)", {5, 2, 4, 3}, {5, 4, 3}, false, true, {5, 2, 4, 4}},
+                               ListCase{"matmult tensors T(a, b) (bigger b)", {5, 4, 3}, {5, 2, 6, 4}, true, true, {5, 2, 3, 6}}}) {
+        run_test(lc.name, [&] {
+            nt::TensorList a = F::randn(lc.as, DType::Float32, 51).split_axis(0), b = F::randn(lc.bs, DType::Float32, 52).split_axis(0);
+            Tensor o = nt::matmult(a, b, lc.ta, lc.tb);
+            SizeRef flat = lc.view;
+            flat.erase(flat.begin());
+            flat[0] *= 5;
+            nt::utils::throw_exception(o.shape() == flat, "Error: Got unexpected shape (" + nt::shape_str(o.shape()) + ")");
+            Tensor ov = o.view(lc.view);
+            const int64_t per = ov.numel() / 5;
+            for (int64_t i = 0; i < 5; ++i) {
+                Tensor o1 = nt::matmult(a[(size_t)i], b[(size_t)i], lc.ta, lc.tb);
+                nt::utils::throw_exception(o1.numel() == per && std::memcmp(o1.data_ptr(), static_cast<const char*>(ov.data_ptr()) + i * per * 4, (size_t)per * 4) == 0,
+                                           "Error tensors did not match at index " + std::to_string(i));
+            }
+        });
+    }
+    run_test("matmult tensors: list errors", [] {
+        nt::TensorList a = F::randn({3, 4, 5}, DType::Float32, 53).split_axis(0), b = F::randn({2, 5, 4}, DType::Float32, 54).split_axis(0);
+        bool threw = false;
+        try { nt::matmult(a, b); } catch (const nt::utils::nt_error&) { threw = true; }
+        nt::utils::throw_exception(threw, "lists of different lengths must be rejected");
+        nt::TensorList c = F::randn({3, 6, 4}, DType::Float32, 55).split_axis(0);
+        threw = false;
+        try { nt::matmult(a, c); } catch (const nt::utils::nt_error&) { threw = true; }
+        nt::utils::throw_exception(threw, "inner sizes that differ must be rejected");
+    });
+    // tests/src/conv_test.cpp:192-213: conv2d over every floating and complex dtype
+    run_test("conv2d dtype sweep (floating and complex)", [] {
+        for (DType dt : {DType::Float32, DType::Float64, DType::Float16, DType::BFloat16, DType::Complex32, DType::Complex64, DType::Complex128}) {
+            Tensor x = F::randn({1, 3, 16, 16}, dt, 61), w = F::randn({4, 3, 3, 3}, dt, 62);
+            Tensor y = nt::conv2d(x, w, {1, 1}, {1, 1});
+            nt::utils::throw_exception(!x.is_null() && !y.is_null() && y.shape() == SizeRef({1, 4, 16, 16}) && y.dtype() == dt,
+                                       std::string("Error x was made null after conv2d call for ") + nt::dtype_name(dt));
+        }
+        // Complex64: the reference's lane-wise product = a real convolution of the real parts and one of the imaginary parts
+        Tensor x = F::randn({2, 3, 9, 8}, DType::Complex64, 63), w = F::randn({4, 3, 3, 3}, DType::Complex64, 64);
+        Tensor y = nt::conv2d(x, w, {1, 1}, {1, 1});
+        for (int part = 0; part < 2; ++part) {
+            Tensor xr({2, 3, 9, 8}, DType::Float32), wr({4, 3, 3, 3}, DType::Float32);
+            for (int64_t i = 0; i < xr.numel(); ++i) xr.data<float>()[i] = x.data<float>()[2 * i + part];
+            for (int64_t i = 0; i < wr.numel(); ++i) wr.data<float>()[i] = w.data<float>()[2 * i + part];
+            Tensor yr = nt::conv2d(xr, wr, {1, 1}, {1, 1});
+            for (int64_t i = 0; i < yr.numel(); ++i)
+                nt::utils::throw_exception(std::fabs(yr.data<float>()[i] - y.data<float>()[2 * i + part]) <= 1e-4, "complex conv2d plane differs from the real convolution");
+        }
+        Tensor a = F::randn({7, 9}, DType::Complex128, 65), b = F::randn({9, 5}, DType::Complex128, 66);
+        Tensor o = nt::matmult(a, b);
+        for (int64_t i = 0; i < 7; ++i)
+            for (int64_t j = 0; j < 5; ++j)
+                for (int part = 0; part < 2; ++part) {
+                    double sum = 0;
+                    for (int64_t t = 0; t < 9; ++t) sum = std::fma(a.data<double>()[2 * (i * 9 + t) + part], b.data<double>()[2 * (t * 5 + j) + part], sum);
+                    nt::utils::throw_exception(o.data<double>()[2 * (i * 5 + j) + part] == sum, "Complex128 matmult is the lane-wise fused chain, bit for bit");
+                }
     });
     run_test("matmult transposed view == flag (no copy)", [] {
         Tensor a = F::randn({6, 40, 30}, DType::Float32, 33), b = F::randn({6, 20, 30}, DType::Float32, 34);
@@ -434,6 +497,14 @@ static void device_resident_cases(const std::string& g) {
             nt::utils::throw_exception(F::allclose(gr.d_kernel, fx("wgrad"), 1e-4, 1e-3), "conv2d wgrad");
         });
     }
+    run_test("device tensors of tensors == host, bit for bit", [&] {
+        Tensor A = F::randn({5, 2, 40, 30}, DType::Float32, 111), B = F::randn({5, 40, 24}, DType::Float32, 112);
+        nt::TensorList a = A.split_axis(0), b = B.split_axis(0);
+        nt::TensorList da = A.to(DeviceType::HIP).split_axis(0), db = B.to(DeviceType::HIP).split_axis(0);
+        Tensor o = nt::matmult(a, b, true, false), dout = nt::matmult(da, db, true, false);
+        nt::utils::throw_exception(dout.is_device() && dout.shape() == SizeRef({10, 30, 24}), "shape of the device result");
+        same_bits(dout, o, "list product");
+    });
     run_test("device conv2d (channels-last path), conv1d, conv_transpose2d, unfold2d, conv3d == host", [&] {
         Tensor x = F::randn({3, 32, 9, 11}, DType::Float32, 101), w = F::randn({24, 16, 3, 3}, DType::Float32, 102);
         Tensor dx = x.to(DeviceType::HIP), dw = w.to(DeviceType::HIP);

@@ -31,11 +31,12 @@ def test_header_symbols_all_exported_and_bound():
 def test_dtype_sizes_follow_nt_dtype_values():
     lib = _lib.load()
     sizes = {_lib.FLOAT16: 2, _lib.FLOAT32: 4, _lib.FLOAT64: 8, _lib.INT8: 1, _lib.INT16: 2, _lib.INT32: 4,
-             _lib.INT64: 8, _lib.UINT8: 1, _lib.UINT16: 2, _lib.UINT32: 4, _lib.BFLOAT16: 2, _lib.UINT64: 8}
+             _lib.INT64: 8, _lib.UINT8: 1, _lib.UINT16: 2, _lib.UINT32: 4, _lib.BFLOAT16: 2, _lib.UINT64: 8,
+             _lib.COMPLEX32: 4, _lib.COMPLEX64: 8, _lib.COMPLEX128: 16}
     for dt, sz in sizes.items():
         assert lib.ntg_dtype_size(dt) == sz
-    # Float128=3, complex 4..6, int128=11, uint128=15, Bool=16, TensorObj=17 are not served
-    for dt in (3, 4, 5, 6, 11, 15, 16, 17, 55):
+    # Float128=3, int128=11, uint128=15, Bool=16, TensorObj=17 are not served
+    for dt in (3, 11, 15, 16, 17, 55):
         assert lib.ntg_dtype_size(dt) == 0
     assert lib.ntg_version() >= 100
 
@@ -51,9 +52,12 @@ def test_argument_errors_do_not_need_a_device():
     # inner sizes differ
     rc = lib.ntg_matmult(_lib.FLOAT32, p, p, p, 4, 4, 3, 4, 0, 0)
     assert rc == 1 and b"inner sizes" in lib.ntg_last_error()
-    # unsupported dtype (Complex64 = 5)
-    rc = lib.ntg_matmult(5, p, p, p, 4, 4, 4, 4, 0, 0)
+    # unsupported dtype (Float128 = 3)
+    rc = lib.ntg_matmult(3, p, p, p, 4, 4, 4, 4, 0, 0)
     assert rc == 2
+    # the complex dtypes have no gradient / transposed convolutions
+    rc = lib.ntg_conv2d_backward(_lib.COMPLEX64, p, p, p, p, p, 1, 1, 2, 2, 1, 1, 1, 1, 1, 0, 0, 1, 1, 1, 0)
+    assert rc == 2 and b"complex" in lib.ntg_last_error()
     # negative size
     rc = lib.ntg_matmult(_lib.FLOAT32, p, p, p, -1, 4, 4, 4, 0, 0)
     assert rc == 1
