@@ -238,6 +238,9 @@ def main():
         G = lambda *a, **k: (lambda: make_gemm(*a, **k))
         run("c3_fp16_4096", G(torch.float16, N, N, N, scale=0.02), flops, PEAK_TFLOPS["fp16"], load=settle_bf16)
         run("c3_bf16_4096_overwrite", G(torch.bfloat16, N, N, N, scale=0.02, mode=_lib.C_OVERWRITE), flops, PEAK_TFLOPS["bf16"])
+        # diagnostic: the same kernel on all-zero operands (no operand toggling: the clock stays higher) -- the difference to the
+        # line above is what the power manager takes, not what the instruction stream costs
+        run("c3_bf16_4096_zero_operands", G(torch.bfloat16, N, N, N, scale=0.0, mode=_lib.C_OVERWRITE), flops, PEAK_TFLOPS["bf16"])
         run("c3_fp32_4096", G(torch.float32, N, N, N), flops, PEAK_TFLOPS["fp32"])
         run("c3_fp64_4096", G(torch.float64, N, N, N), flops, PEAK_TFLOPS["fp64"])
         run("c1_fp32_512", G(torch.float32, 512, 512, 512), 2.0 * 512 ** 3, PEAK_TFLOPS["fp32"])
