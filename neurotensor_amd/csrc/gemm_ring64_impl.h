@@ -49,9 +49,9 @@ __global__ void __launch_bounds__(256) gemm_ring64_kernel(const GemmParams p) {
     tile_coords(lid - b * tiles, p.tiles_m, p.tiles_n, 8, tm, tn);
     const int m0 = tm * G::BM, n0 = tn * G::BN;
 
-    const double* A = static_cast<const double*>(p.A) + (int64_t)b * p.sA;
-    const double* B = static_cast<const double*>(p.B) + (int64_t)b * p.sB;
-    double* C = static_cast<double*>(p.C) + (int64_t)b * p.sC;
+    const double* A = p.Aptr ? static_cast<const double*>(p.Aptr[b]) : static_cast<const double*>(p.A) + (int64_t)b * p.sA;
+    const double* B = p.Bptr ? static_cast<const double*>(p.Bptr[b]) : static_cast<const double*>(p.B) + (int64_t)b * p.sB;
+    double* C = p.Cptr ? static_cast<double*>(p.Cptr[b]) : static_cast<double*>(p.C) + (int64_t)b * p.sC;
 
     const int wave_u = __builtin_amdgcn_readfirstlane(wave);
     const int KT = (p.K + BK - 1) / BK;
@@ -196,7 +196,7 @@ __global__ void __launch_bounds__(256) gemm_ring64_kernel(const GemmParams p) {
 // 16-byte aligned rows everywhere; per-lane DMA offsets are 32-bit (128 rows of lda doubles below 4 GiB)
 static inline bool ring64_eligible(const GemmParams& p, bool ta) {
     return p.K >= 2 && p.K % 2 == 0 && p.N % 2 == 0 && (!ta || p.M % 2 == 0) &&
-           !p.Aptr && !p.Bptr && !p.Cptr && p.vecA_ok && p.vecB_ok && p.lda < (1 << 21) && p.ldb < (1 << 21) &&
+           ((!p.Aptr && !p.Bptr && !p.Cptr) || (p.ptrs_aligned && p.Aptr && p.Bptr && p.Cptr)) && p.vecA_ok && p.vecB_ok && p.lda < (1 << 21) && p.ldb < (1 << 21) &&
            ((reinterpret_cast<uintptr_t>(p.A) & 15) == 0) && ((reinterpret_cast<uintptr_t>(p.B) & 15) == 0) &&
            ((reinterpret_cast<uintptr_t>(p.C) & 7) == 0);
 }

@@ -215,9 +215,10 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
     tile_coords(lid - b * tiles, p.tiles_m, p.tiles_n, 4, tm, tn);
     const int m0 = tm * GA::BM, n0 = tn * G::BN;
 
-    const T* A = static_cast<const T*>(p.A) + (int64_t)b * p.sA;
-    const T* B = static_cast<const T*>(p.B) + (int64_t)b * p.sB;
-    T* C = static_cast<T*>(p.C) + (int64_t)b * p.sC;
+    // (pointer tables: one uniform load per operand; everything below is base + offset either way)
+    const T* A = p.Aptr ? static_cast<const T*>(p.Aptr[b]) : static_cast<const T*>(p.A) + (int64_t)b * p.sA;
+    const T* B = p.Bptr ? static_cast<const T*>(p.Bptr[b]) : static_cast<const T*>(p.B) + (int64_t)b * p.sB;
+    T* C = p.Cptr ? static_cast<T*>(p.Cptr[b]) : static_cast<T*>(p.C) + (int64_t)b * p.sC;
 
     // ---- DMA sources: uniform tile base (advances by adv bytes per K-step) + per-lane offsets ----
     const int wave_u = __builtin_amdgcn_readfirstlane(wave);
@@ -825,12 +826,13 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
 // dimensions, batch strides, base pointers) and every contiguous extent a multiple of one 16-byte
 // chunk (es = element size: 8 or 4 elements).  M, N and K themselves may be ragged with respect
 // to the tile.  Per-lane DMA offsets are 32-bit: 256 rows of lda elements must stay below 4 GiB.
+// Pointer tables qualify when the caller vouches for the entries' alignment (p.ptrs_aligned).
 static inline bool ring_eligible(const GemmParams& p, bool ta, int es = 2) {
     const int vel = 16 / es;
     const int64_t ldmax = (int64_t)(1 << 23) / es;
     return p.K >= vel && p.K % vel == 0 && p.N % vel == 0 && (!ta || p.M % vel == 0) &&
-           !p.Aptr && !p.Bptr && !p.Cptr && p.vecA_ok && p.vecB_ok &&
-           p.ldc % vel == 0 && p.sC % vel == 0 && p.lda < ldmax && p.ldb < ldmax &&
+           ((!p.Aptr && !p.Bptr && !p.Cptr) || (p.ptrs_aligned && p.Aptr && p.Bptr && p.Cptr && p.cmode != C_PARTIAL)) && p.vecA_ok && p.vecB_ok &&
+           p.ldc % vel == 0 && (p.Cptr || p.sC % vel == 0) && p.lda < ldmax && p.ldb < ldmax &&
            ((reinterpret_cast<uintptr_t>(p.A) & 15) == 0) && ((reinterpret_cast<uintptr_t>(p.B) & 15) == 0) &&
            ((reinterpret_cast<uintptr_t>(p.C) & 15) == 0);
 }

@@ -72,6 +72,8 @@ struct GemmParams {
     int cmode;
     int tiles_m, tiles_n;
     int vecA_ok, vecB_ok;    // 16-byte vector loads are legal for every row of A / B
+    int ptrs_aligned;        // pointer tables only: the caller vouches that every entry is a multiple of 16 bytes (the tables
+                             // live in device memory, the host cannot look); lets table batches onto the DMA-fed kernels
     ConvGeom conv;           // used by the implicit-im2col kernels only: B = image, op(B) = col or col^T
 };
 
@@ -215,6 +217,14 @@ hipError_t launch_conv_nhwc_dw(int dtype, bool ta, const GemmParams& p, hipStrea
 hipError_t launch_reduce_batch_taps_last(int dtype, const void* part, void* out, int64_t batch, int64_t rows, int64_t cg, int64_t cgp,
                                          int64_t taps, int accumulate, hipStream_t s);   // part rows hold cgp >= cg channels per tap
 hipError_t launch_flip_weights(int64_t elem_size, const void* w, void* wt, int64_t groups, int64_t og, int64_t cg, int64_t taps, hipStream_t s);
+
+// padded copies of operands whose rows are not 16-byte multiples (pad_copy.hip); es = 1 or 2 bytes per element, sizes in elements
+hipError_t launch_pad_copy(int64_t es, const void* src, int64_t ld_src, int64_t s_src, void* dst, int64_t ld_dst, int64_t s_dst,
+                           int64_t rows, int64_t cols, int64_t rows_dst, int64_t batch, hipStream_t s);
+hipError_t launch_unpad_copy(int64_t es, const void* src, int64_t ld_src, int64_t s_src, void* dst, int64_t ld_dst, int64_t s_dst,
+                             int64_t rows, int64_t cols, int64_t batch, hipStream_t s);
+hipError_t launch_bias_fill(int64_t es, const void* bias, int64_t bs, int64_t rs, int64_t cs, void* dst, int64_t ld_dst, int64_t s_dst,
+                            int64_t rows, int64_t cols, int64_t rows_dst, int64_t batch, hipStream_t s);
 
 // grid of a grid-stride element-wise kernel (256 lanes per workgroup, at most 64 workgroups per CU)
 static inline unsigned grid_for(int64_t total) {

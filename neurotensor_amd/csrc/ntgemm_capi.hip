@@ -224,6 +224,86 @@ static int run_int_planes(const ntg::GemmParams& p, const IntPlanesPlan& pl, boo
     return NTG_OK;
 }
 
+// Padded copies.  The DMA-fed kernels need 16-byte rows (leading dimensions, batch strides, base pointers, and K, N -- M
+// under transpose_a -- multiples of one 16-byte chunk); an 8- or 16-bit product that misses this falls to the vector ALU
+// (8-bit: 40 x slower) or the register-staged kernel (16-bit: half the rate).  With a workspace the operands that need it
+// are copied into rows padded with zeros to whole chunks (zero products add nothing: bit-identical integers, the same
+// single rounding for the 16-bit floats), the product runs on the DMA-fed kernel, and a result whose own rows are not
+// 16-byte multiples is computed into a padded copy and copied back.  Taken for products large enough to repay the copies.
+struct PadPlan {
+    bool ok, padA, padB, padC;
+    int Mp, Kp, Np;
+    int64_t lda2, ldb2, rowsA2, rowsB2, a_bytes, b_bytes, c_bytes;
+    int64_t bytes() const { return a_bytes + b_bytes + c_bytes; }
+};
+static PadPlan plan_pad(const ntg::GemmParams& p, int dtype, bool ta, bool tb) {
+    PadPlan pl;
+    std::memset(&pl, 0, sizeof pl);
+    const bool half = dtype == ntg::DT_F16 || dtype == ntg::DT_BF16, byte = dtype == ntg::DT_I8 || dtype == ntg::DT_U8;
+    if ((!half && !byte) || p.Aptr || p.Bptr || p.Cptr || p.M <= 32) return pl;
+    const int64_t es = half ? 2 : 1, ve = 16 / es;
+    const double macs = (double)p.M * p.N * p.K * p.batch;
+    if (macs < (half ? 2147483648.0 : 268435456.0)) return pl;
+    auto up = [&](int64_t v) { return (v + ve - 1) / ve * ve; };
+    pl.Kp = (int)up(p.K); pl.Np = (int)up(p.N); pl.Mp = ta ? (int)up(p.M) : p.M;
+    auto misaligned = [&](const void* ptr, int64_t ld, int64_t stride) {
+        return ld % ve != 0 || (p.batch > 1 && stride % ve != 0) || (reinterpret_cast<uintptr_t>(ptr) & 15) != 0;
+    };
+    pl.padA = misaligned(p.A, p.lda, p.sA) || pl.Kp != p.K || pl.Mp != p.M;
+    pl.padB = misaligned(p.B, p.ldb, p.sB) || pl.Kp != p.K || pl.Np != p.N;
+    pl.padC = misaligned(p.C, p.ldc, p.sC) || pl.Np != p.N || pl.Mp != p.M;
+    if (!pl.padA && !pl.padB && !pl.padC) return pl;                       // nothing that padding would fix
+    pl.lda2 = ta ? pl.Mp : pl.Kp; pl.rowsA2 = ta ? pl.Kp : p.M;
+    pl.ldb2 = tb ? pl.Kp : pl.Np; pl.rowsB2 = tb ? pl.Np : pl.Kp;
+    const int64_t ldmax = (int64_t)(1 << 23) / es;                         // (the kernels' 32-bit lane offsets)
+    if ((pl.padA ? pl.lda2 : p.lda) >= ldmax || (pl.padB ? pl.ldb2 : p.ldb) >= ldmax) return pl;
+    if (pl.padA) pl.a_bytes = (int64_t)align_up((size_t)((p.sA == 0 ? 1 : p.batch) * pl.rowsA2 * pl.lda2 * es), 256);
+    if (pl.padB) pl.b_bytes = (int64_t)align_up((size_t)((p.sB == 0 ? 1 : p.batch) * pl.rowsB2 * pl.ldb2 * es), 256);
+    if (pl.padC) pl.c_bytes = (int64_t)align_up((size_t)((int64_t)p.batch * pl.Mp * pl.Np * es), 256);
+    pl.ok = true;
+    return pl;
+}
+static int run_padded(const ntg::GemmParams& p, const PadPlan& pl, int dtype, bool ta, bool tb, void* ws, hipStream_t s) {
+    const int64_t es = ntg::elem_size(dtype);
+    char* a2 = static_cast<char*>(ws);
+    char* b2 = a2 + pl.a_bytes;
+    char* c2 = b2 + pl.b_bytes;
+    ntg::GemmParams q = p;
+    q.M = pl.Mp; q.K = pl.Kp; q.N = pl.Np;
+    hipError_t e;
+    if (pl.padA) {
+        e = ntg::launch_pad_copy(es, p.A, p.lda, p.sA, a2, pl.lda2, pl.rowsA2 * pl.lda2, ta ? p.K : p.M, ta ? p.M : p.K, pl.rowsA2, p.sA == 0 ? 1 : p.batch, s);
+        if (e != hipSuccess) return hip_fail(e, "padded copy of A");
+        q.A = a2; q.lda = pl.lda2; q.sA = p.sA == 0 ? 0 : pl.rowsA2 * pl.lda2;
+    }
+    if (pl.padB) {
+        e = ntg::launch_pad_copy(es, p.B, p.ldb, p.sB, b2, pl.ldb2, pl.rowsB2 * pl.ldb2, tb ? p.N : p.K, tb ? p.K : p.N, pl.rowsB2, p.sB == 0 ? 1 : p.batch, s);
+        if (e != hipSuccess) return hip_fail(e, "padded copy of B");
+        q.B = b2; q.ldb = pl.ldb2; q.sB = p.sB == 0 ? 0 : pl.rowsB2 * pl.ldb2;
+    }
+    if (pl.padC) {
+        const int64_t sc2 = (int64_t)pl.Mp * pl.Np;
+        if (p.cmode == ntg::C_ACCUMULATE) {
+            e = ntg::launch_pad_copy(es, p.C, p.ldc, p.sC, c2, pl.Np, sc2, p.M, p.N, pl.Mp, p.batch, s);
+            if (e != hipSuccess) return hip_fail(e, "padded copy of C");
+        } else if (p.cmode == ntg::C_BIAS) {
+            // the bias becomes the initial accumulator in the padded layout (reading it at padded indices would leave its array)
+            e = ntg::launch_bias_fill(es, p.bias, p.bias_bs, p.bias_rs, p.bias_cs, c2, pl.Np, sc2, p.M, p.N, pl.Mp, p.batch, s);
+            if (e != hipSuccess) return hip_fail(e, "bias fill");
+            q.cmode = ntg::C_ACCUMULATE;
+            q.bias = nullptr;
+        }
+        q.C = c2; q.ldc = pl.Np; q.sC = sc2;
+    }
+    const int rc = launch_gemm(q, dtype, ta, tb, s);
+    if (rc) return rc;
+    if (pl.padC) {
+        e = ntg::launch_unpad_copy(es, c2, pl.Np, (int64_t)pl.Mp * pl.Np, p.C, p.ldc, p.sC, p.M, p.N, p.batch, s);
+        if (e != hipSuccess) return hip_fail(e, "copy of the padded result");
+    }
+    return NTG_OK;
+}
+
 SplitPlan plan_splitk(const ntg::GemmParams& p, int dtype, bool ta) {
     SplitPlan none{1, p.K, 0};
     const int64_t es = ntg::elem_size(dtype);
@@ -307,6 +387,11 @@ int run_gemm(ntg::GemmParams p, int dtype, bool ta, bool tb, hipStream_t s, void
         const IntPlanesPlan ip = plan_int_planes(p, dtype);
         if (ip.ok && workspace && workspace_bytes >= ip.bytes() && (reinterpret_cast<uintptr_t>(workspace) & 255) == 0)
             return run_int_planes(p, ip, ta, tb, workspace, s);
+    }
+    {
+        const PadPlan pp = plan_pad(p, dtype, ta, tb);
+        if (pp.ok && workspace && workspace_bytes >= pp.bytes() && (reinterpret_cast<uintptr_t>(workspace) & 255) == 0)
+            return run_padded(p, pp, dtype, ta, tb, workspace, s);
     }
     const SplitPlan plan = plan_splitk(p, dtype, ta);
     if (plan.splits > 1 && workspace && workspace_bytes >= plan.bytes && (reinterpret_cast<uintptr_t>(workspace) & 15) == 0) {
@@ -418,6 +503,10 @@ int64_t ntg_gemm_workspace_bytes(const ntg_gemm_desc* d) {
         const IntPlanesPlan ip = plan_int_planes(p, d->dtype);
         return ip.ok ? ip.bytes() : 0;
     }
+    {
+        const PadPlan pp = plan_pad(p, d->dtype, d->transpose_a != 0, d->transpose_b != 0);      // pointers taken as 16-byte aligned
+        if (pp.ok) return pp.bytes();
+    }
     return plan_splitk(p, d->dtype, d->transpose_a != 0).bytes;      // pointers taken as 16-byte aligned
 }
 
@@ -442,14 +531,20 @@ int ntg_gemm_noalloc_dev(const ntg_gemm_desc* d, const void* dA, const void* dB,
     return run_gemm(p, d->dtype, d->transpose_a != 0, d->transpose_b != 0, static_cast<hipStream_t>(stream), ws, need);
 }
 
-int ntg_gemm_ptrs_dev(const ntg_gemm_desc* d, const void* const* dA, const void* const* dB, void* const* dC, void* stream) {
+// aligned: the caller vouches that every table entry is a multiple of 16 bytes (true for the host entry points' own arena)
+static int gemm_ptrs(const ntg_gemm_desc* d, const void* const* dA, const void* const* dB, void* const* dC, void* stream, bool aligned) {
     ntg::GemmParams p;
     int rc = desc_to_params(d, p);
     if (rc) return rc;
     if (p.M == 0 || p.N == 0 || p.batch == 0) return NTG_OK;
     if (!dA || !dB || !dC) return fail(NTG_ERR_INVALID_ARGUMENT, "null pointer table");
     p.Aptr = dA; p.Bptr = dB; p.Cptr = dC;
+    p.ptrs_aligned = aligned ? 1 : 0;
     return run_gemm(p, d->dtype, d->transpose_a != 0, d->transpose_b != 0, static_cast<hipStream_t>(stream));
+}
+
+int ntg_gemm_ptrs_dev(const ntg_gemm_desc* d, const void* const* dA, const void* const* dB, void* const* dC, void* stream) {
+    return gemm_ptrs(d, dA, dB, dC, stream, false);     // (the tables are in device memory: their entries' alignment is unknown here)
 }
 
 int ntg_matmult_dev(int dtype, const void* dA, const void* dB, void* dC, int64_t m, int64_t k, int64_t n,
@@ -538,7 +633,7 @@ int ntg_matmult_batch(int dtype, const void* const* A, const void* const* B, voi
         rc = ntg_gemm_dev(&d, tab[0], tab[(size_t)batches], tab[(size_t)(2 * batches)], mem.stream());
     } else {
         HIP_TRY(mem.upload(tab_off, tab.data(), tab.size() * sizeof(void*)));
-        rc = ntg_gemm_ptrs_dev(&d, dtab, dtab + batches, dtab + 2 * batches, mem.stream());
+        rc = gemm_ptrs(&d, dtab, dtab + batches, dtab + 2 * batches, mem.stream(), true);     // (every slot of the arena is 256-byte aligned)
     }
     if (rc) return rc;
     for (int64_t i = 0; i < batches; ++i)

@@ -151,8 +151,13 @@ def test_split_k_planner_needs_no_device():
     # a short k does not pay for the second pass; a product that already has a tile for most CUs does not either
     assert ws(_lib.BFLOAT16, 1024, 1024, 1024) == 0
     assert ws(_lib.BFLOAT16, 1536, 4096, 1536) == 0
-    # rows that are not 16-byte multiples cannot use the kernel that writes fp32 partial sums
-    assert ws(_lib.BFLOAT16, 128, 8192, 8190) == 0 and ws(_lib.BFLOAT16, 128, 8192, 8192, lda=8196) == 0
+    # rows that are not 16-byte multiples cannot use the kernel that writes fp32 partial sums; products this large are
+    # offered padded copies of the operands that need them instead (B and C for n = 8190, A for a pitch of 8196)
+    assert ws(_lib.BFLOAT16, 128, 8192, 8190) == 8192 * 8192 * 2 + 128 * 8192 * 2 and ws(_lib.BFLOAT16, 128, 8192, 8192, lda=8196) == 128 * 8192 * 2
+    assert ws(_lib.BFLOAT16, 128, 1024, 1022) == 0 and ws(_lib.BFLOAT16, 128, 1024, 1024, lda=1028) == 0      # too small to repay the copies
+    # 8-bit integers: the alternative is the vector ALU, so the padded form starts earlier
+    assert ws(_lib.INT8, 520, 1001, 530) == 520 * 1008 + 1008 * 544 + 520 * 544 + (256 - 520 * 1008 % 256) % 256 + (256 - 1008 * 544 % 256) % 256 + (256 - 520 * 544 % 256) % 256
+    assert ws(_lib.INT8, 100, 101, 103) == 0 and ws(_lib.INT32, 100, 101, 103) == 0
     # fp32 / fp64, 64 x 64 tiles: 16 tiles and k = 1024 -> eight ranges of 128; 256 or more tiles -> none
     assert ranges(_lib.FLOAT32, 256, 1024, 256, 4) == 8
     assert ranges(_lib.FLOAT64, 256, 1024, 256, 8) == 8

@@ -81,6 +81,8 @@ def run_case(rng, name, m, k, n, ta, tb, pads, mode, batches=1, gap=0, base=0, b
     ws = None
     if workspace:
         need = lib.ntg_gemm_workspace_bytes(ctypes.byref(d))
+        if workspace is not True:
+            need = max(need, int(workspace))          # explicit size: the query knows sizes and pitches, not the base pointers
         assert need > 0, (name, m, k, n, "expected a workspace form")
         ws = torch.empty(need, dtype=torch.uint8, device=DEV)
         d.workspace, d.workspace_bytes = ws.data_ptr(), need
@@ -179,3 +181,20 @@ def test_16bit_results_are_rounded_once_on_ragged_k(name):
         run_case(rng, name, 8, 8, 8, ta, tb, (0, 0, 0), _lib.C_ACCUMULATE, one_rounding=True)
     run_case(rng, name, 128, 2080, 264, False, True, (0, 0, 0), _lib.C_ACCUMULATE, workspace=True, one_rounding=True)
     run_case(rng, name, 520, 1544, 776, False, False, (0, 0, 0), _lib.C_ACCUMULATE, one_rounding=True)      # 256-wide tiles, ragged everywhere
+
+
+@pytest.mark.parametrize("name", ["bf16", "f16", "i8", "u8"])
+def test_rows_that_are_not_16_byte_multiples_through_padded_copies(name):
+    """Large 8- and 16-bit products whose pitches, sizes or base pointers miss the 16-byte rule are offered a workspace
+    (ntg_gemm_workspace_bytes) with which the operands are copied into zero-padded rows and the DMA-fed kernel runs:
+    every flag pair, the three C modes, batches with a broadcast operand, odd k / n / m and odd base pointers;
+    integers bit-exact against the oracle, 16-bit floats held to one rounding."""
+    rng = np.random.default_rng(8100 + list(DTYPES).index(name))
+    half = name in FLOATS
+    m, k, n = (1304, 1001, 1702) if half else (520, 1001, 530)
+    modes = (_lib.C_ACCUMULATE, _lib.C_BIAS, _lib.C_OVERWRITE, _lib.C_ACCUMULATE)
+    for (ta, tb), mode in zip(TRANS, modes):
+        run_case(rng, name, m, k, n, ta, tb, (0, 0, 0), mode, workspace=True, one_rounding=half)             # odd k: A and B padded, C as it lies
+    run_case(rng, name, m + 3, k + 7, n + 1, True, False, ODD, _lib.C_BIAS, base=1, workspace=True, one_rounding=half)   # everything odd, C padded too
+    run_case(rng, name, m, k + 7, n - 6, False, True, (0, 8, 5), _lib.C_ACCUMULATE, batches=2, gap=3, workspace=True, one_rounding=half)
+    run_case(rng, name, m, 1008, n - 6, False, False, (0, 0, 0), _lib.C_OVERWRITE, batches=2, bcast_b=True, base=3, workspace=64 << 20, one_rounding=half)   # only the base pointers are odd
