@@ -6,7 +6,8 @@ import ctypes
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "lib", "libntgemm.so")
+# NTG_LIB_PATH points the loader at another build of the same library (the host-sanitizer build, lib/asan/libntgemm.so)
+LIB_PATH = os.environ.get("NTG_LIB_PATH") or os.path.join(_HERE, "lib", "libntgemm.so")
 
 # ntg_dtype (== nt::DType values; BF16/U64 are extensions)
 FLOAT16, FLOAT32, FLOAT64 = 0, 1, 2

@@ -965,8 +965,7 @@ static Vol3 vol3(const Tensor& t, bool is_kernel, const char* what) {
 Tensor conv3d(const Tensor& image, const Tensor& kernel, utils::my_n_tuple<3> s, utils::my_n_tuple<3> p, utils::my_n_tuple<3> d, int64_t groups) {
     utils::throw_exception(!image.is_null() && !kernel.is_null(), "Cannot perform operation conv3d on a null tensor");
     utils::throw_exception(image.dtype() == kernel.dtype(), "Expected both kernel and image to have the same dtype for conv3d");
-    if (common_device({&image, &kernel}, "conv3d") == DeviceType::HIP)      // the three-axis forms take device tensors through host memory
-        return functional::conv3d(image.cpu(), kernel.cpu(), s, p, d, groups).to(DeviceType::HIP);
+    const DeviceType dev = common_device({&image, &kernel}, "conv3d");
     for (int a = 0; a < 3; ++a) {   // conv.cpp:129-131
         utils::throw_exception(s[a] >= 1, "Conv3d stride cannot be less than 1");
         utils::throw_exception(d[a] >= 1, "Conv3d dilation cannot be less than 1");
@@ -982,26 +981,38 @@ Tensor conv3d(const Tensor& image, const Tensor& kernel, utils::my_n_tuple<3> s,
         out[a] = (xv.size[a] + 2 * p[a] - d[a] * (wv.size[a] - 1) - 1) / s[a] + 1;
         utils::throw_exception(out[a] > 0, "conv3d output would be empty");
     }
-    Tensor y({xv.B, O, out[0], out[1], out[2]}, x.dtype());
-    check_status(ntg_convnd(static_cast<int>(x.dtype()), x.data_ptr(), w.data_ptr(), y.data_ptr(), xv.B, xv.C, O, 3, xv.size, wv.size, s.data(),
-                            p.data(), d.data(), groups));
+    Tensor y({xv.B, O, out[0], out[1], out[2]}, x.dtype(), dev);
+    const int dt = static_cast<int>(x.dtype());
+    if (dev == DeviceType::HIP) {
+        const int64_t wsb = ntg_convnd_workspace_bytes(dt, xv.B, xv.C, O, 3, xv.size, wv.size, s.data(), p.data(), d.data(), groups, 0);
+        utils::throw_exception(wsb >= 0, "conv3d output would be empty");
+        check_status(ntg_convnd_dev(dt, x.data_ptr(), w.data_ptr(), y.data_ptr(), device_workspace(wsb), wsb, xv.B, xv.C, O, 3, xv.size, wv.size,
+                                    s.data(), p.data(), d.data(), groups, nullptr));
+        return y;
+    }
+    check_status(ntg_convnd(dt, x.data_ptr(), w.data_ptr(), y.data_ptr(), xv.B, xv.C, O, 3, xv.size, wv.size, s.data(), p.data(), d.data(), groups));
     return y;
 }
 
 ConvGrads conv3d_backward(const Tensor& image, const Tensor& kernel, const Tensor& grad, utils::my_n_tuple<3> s, utils::my_n_tuple<3> p,
                           utils::my_n_tuple<3> d, int64_t groups) {
     utils::throw_exception(!image.is_null() && !kernel.is_null() && !grad.is_null(), "Cannot perform operation conv3d backward on a null tensor");
-    if (common_device({&image, &kernel, &grad}, "conv3d backward") == DeviceType::HIP) {
-        ConvGrads h = functional::conv3d_backward(image.cpu(), kernel.cpu(), grad.cpu(), s, p, d, groups);
-        return {h.d_image.to(DeviceType::HIP), h.d_kernel.to(DeviceType::HIP)};
-    }
+    const DeviceType dev = common_device({&image, &kernel, &grad}, "conv3d backward");
     Tensor x = image.contiguous(), w = kernel.contiguous(), g = grad.contiguous();
     const Vol3 xv = vol3(x, false, "conv3d backward"), wv = vol3(w, true, "conv3d backward");
     int64_t L = 1;
     for (int a = 0; a < 3; ++a) L *= (xv.size[a] + 2 * p[a] - d[a] * (wv.size[a] - 1) - 1) / s[a] + 1;
     utils::throw_exception(g.numel() == xv.B * wv.B * L, "grad does not have the shape of the convolution output");
-    ConvGrads out{Tensor(image.shape(), x.dtype()), Tensor(kernel.shape(), x.dtype())};
-    check_status(ntg_convnd_backward(static_cast<int>(x.dtype()), x.data_ptr(), w.data_ptr(), g.data_ptr(), out.d_image.data_ptr(),
+    ConvGrads out{Tensor(image.shape(), x.dtype(), dev), Tensor(kernel.shape(), x.dtype(), dev)};
+    const int dt = static_cast<int>(x.dtype());
+    if (dev == DeviceType::HIP) {
+        const int64_t wsb = ntg_convnd_workspace_bytes(dt, xv.B, xv.C, wv.B, 3, xv.size, wv.size, s.data(), p.data(), d.data(), groups, 1);
+        utils::throw_exception(wsb >= 0, "conv3d backward: geometry has no output");
+        check_status(ntg_convnd_backward_dev(dt, x.data_ptr(), w.data_ptr(), g.data_ptr(), out.d_image.data_ptr(), out.d_kernel.data_ptr(),
+                                             device_workspace(wsb), wsb, xv.B, xv.C, wv.B, 3, xv.size, wv.size, s.data(), p.data(), d.data(), groups, 0, nullptr));
+        return out;
+    }
+    check_status(ntg_convnd_backward(dt, x.data_ptr(), w.data_ptr(), g.data_ptr(), out.d_image.data_ptr(),
                                      out.d_kernel.data_ptr(), xv.B, xv.C, wv.B, 3, xv.size, wv.size, s.data(), p.data(), d.data(), groups, 0));
     return out;
 }
@@ -1010,8 +1021,7 @@ Tensor conv_transpose3d(const Tensor& image, const Tensor& kernel, utils::my_n_t
                         utils::my_n_tuple<3> d, int64_t groups) {
     utils::throw_exception(!image.is_null() && !kernel.is_null(), "Cannot perform operation conv_transpose3d on a null tensor");
     utils::throw_exception(image.dtype() == kernel.dtype(), "Expected both kernel and image to have the same dtype for conv3d transpose");
-    if (common_device({&image, &kernel}, "conv_transpose3d") == DeviceType::HIP)
-        return functional::conv_transpose3d(image.cpu(), kernel.cpu(), s, p, op, d, groups).to(DeviceType::HIP);
+    const DeviceType dev = common_device({&image, &kernel}, "conv_transpose3d");
     for (int a = 0; a < 3; ++a) {   // conv.cpp:687-691
         utils::throw_exception(s[a] >= 1, "Conv3d Transpose stride cannot be less than 1");
         utils::throw_exception(d[a] >= 1, "Conv3d Transpose dilation cannot be less than 1");
@@ -1026,8 +1036,16 @@ Tensor conv_transpose3d(const Tensor& image, const Tensor& kernel, utils::my_n_t
     utils::throw_exception(xv.C % groups == 0, "Expected image channels to be divisible by groups in Conv3d Transpose");
     int64_t out[3];
     for (int a = 0; a < 3; ++a) out[a] = (xv.size[a] - 1) * s[a] - 2 * p[a] + d[a] * (wv.size[a] - 1) + 1 + op[a];
-    Tensor y({xv.B, wv.C * groups, out[0], out[1], out[2]}, x.dtype());
-    check_status(ntg_conv_transposend(static_cast<int>(x.dtype()), x.data_ptr(), w.data_ptr(), y.data_ptr(), xv.B, xv.C, wv.C * groups, 3, xv.size,
+    Tensor y({xv.B, wv.C * groups, out[0], out[1], out[2]}, x.dtype(), dev);
+    const int dt = static_cast<int>(x.dtype());
+    if (dev == DeviceType::HIP) {
+        const int64_t wsb = ntg_conv_transposend_workspace_bytes(dt, xv.B, xv.C, wv.C * groups, 3, xv.size, wv.size, s.data(), p.data(), d.data(), op.data(), groups);
+        utils::throw_exception(wsb >= 0, "conv_transpose3d output would be empty");
+        check_status(ntg_conv_transposend_dev(dt, x.data_ptr(), w.data_ptr(), y.data_ptr(), device_workspace(wsb), wsb, xv.B, xv.C, wv.C * groups, 3,
+                                              xv.size, wv.size, s.data(), p.data(), d.data(), op.data(), groups, nullptr));
+        return y;
+    }
+    check_status(ntg_conv_transposend(dt, x.data_ptr(), w.data_ptr(), y.data_ptr(), xv.B, xv.C, wv.C * groups, 3, xv.size,
                                       wv.size, s.data(), p.data(), d.data(), op.data(), groups));
     return y;
 }

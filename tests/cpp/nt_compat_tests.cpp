@@ -518,6 +518,21 @@ static void device_resident_cases(const std::string& g) {
         Tensor x3 = F::randn({2, 4, 5, 6, 7}, DType::Float32, 107), w3 = F::randn({6, 4, 2, 3, 2}, DType::Float32, 108);
         same_bits(nt::conv3d(x3.to(DeviceType::HIP), w3.to(DeviceType::HIP)), nt::conv3d(x3, w3), "conv3d");
     });
+    run_test("device conv3d family stays in HBM: forward, gradients, transposed == host", [&] {
+        Tensor x3 = F::randn({2, 4, 5, 6, 7}, DType::Float32, 121), w3 = F::randn({6, 2, 2, 3, 2}, DType::Float32, 122);
+        Tensor dx3 = x3.to(DeviceType::HIP), dw3 = w3.to(DeviceType::HIP);
+        Tensor y = nt::conv3d(x3, w3, {1, 2, 1}, {1, 0, 1}, {1, 1, 2}, 2), dy = nt::conv3d(dx3, dw3, {1, 2, 1}, {1, 0, 1}, {1, 1, 2}, 2);
+        nt::utils::throw_exception(dy.is_device() && F::allclose(dy, y, 1e-5, 1e-5), "conv3d (strided, dilated, grouped)");
+        Tensor g = F::randn(y.shape(), DType::Float32, 123);
+        F::ConvGrads hg = F::conv3d_backward(x3, w3, g, {1, 2, 1}, {1, 0, 1}, {1, 1, 2}, 2);
+        F::ConvGrads dg = F::conv3d_backward(dx3, dw3, g.to(DeviceType::HIP), {1, 2, 1}, {1, 0, 1}, {1, 1, 2}, 2);
+        nt::utils::throw_exception(dg.d_image.is_device() && dg.d_kernel.is_device() && F::allclose(dg.d_image, hg.d_image, 1e-4, 1e-4) &&
+                                       F::allclose(dg.d_kernel, hg.d_kernel, 1e-4, 1e-3), "conv3d gradients");
+        Tensor xt = F::randn({2, 6, 3, 4, 5}, DType::Float32, 124), wt = F::randn({6, 2, 2, 3, 3}, DType::Float32, 125);
+        Tensor yt = nt::conv_transpose3d(xt, wt, {2, 1, 2}, {0, 1, 1}, {1, 0, 1}, {1, 1, 1}, 2);
+        Tensor dyt = nt::conv_transpose3d(xt.to(DeviceType::HIP), wt.to(DeviceType::HIP), {2, 1, 2}, {0, 1, 1}, {1, 0, 1}, {1, 1, 1}, 2);
+        nt::utils::throw_exception(dyt.is_device() && F::allclose(dyt, yt, 1e-5, 1e-5), "conv_transpose3d");
+    });
 }
 
 int main(int argc, char** argv) {
