@@ -11,12 +11,26 @@ hipError_t launch_gemm_mfma_i8(int dtype, bool ta, bool tb, const GemmParams& p,
         return launch_gemm_valu(dtype, ta, tb, p, s);
     }
     // (an MN-major 192-row tile of bytes has 12 chunks per k-row, which the chunk swizzle of the transposing reads does not fit)
-    const int te = ring16_tile_edge(p.M, p.N, p.K, p.batch, ta ? RECT_128 : RECT_128 | RECT_192);
-    if (te == 256) return launch_ring_wb<DT_I8, 4>(ta, tb, p, s);
-    if (te == 224) return tb ? launch_ring_cfg<DT_I8, false, true, 3, 4>(p, s) : launch_ring_cfg<DT_I8, false, false, 3, 4>(p, s);
-    if (te == 192) return launch_ring_wb<DT_I8, 2, 4>(ta, tb, p, s);
-    if (te == 64) return launch_ring_wb<DT_I8, 1>(ta, tb, p, s);
-    return launch_ring_wb<DT_I8, 2>(ta, tb, p, s);
+    const int rect = ta ? RECT_128 : RECT_128 | RECT_192;
+    auto launch = [&](int te, const GemmParams& q) {
+        if (te == 256) return launch_ring_wb<DT_I8, 4>(ta, tb, q, s);
+        if (te == 224) return tb ? launch_ring_cfg<DT_I8, false, true, 3, 4>(q, s) : launch_ring_cfg<DT_I8, false, false, 3, 4>(q, s);
+        if (te == 192) return launch_ring_wb<DT_I8, 2, 4>(ta, tb, q, s);
+        if (te == 64) return launch_ring_wb<DT_I8, 1>(ta, tb, q, s);
+        return launch_ring_wb<DT_I8, 2>(ta, tb, q, s);
+    };
+    if (p.batch == 1 && p.cmode != C_PARTIAL) {
+        // (the estimate of the 16-bit kernel: a K-step of 64 bytes per row is 64 k here, so the same tile takes half the steps)
+        const Ring16Split sp = ring16_split(p.M, p.N, p.K, rect);
+        if (sp.axis) {
+            GemmParams head, tail;
+            ring_split_params(p, ta, tb, 1, sp, head, tail);
+            const hipError_t e = launch(sp.head_edge, head);
+            if (e != hipSuccess) return e;
+            return launch(sp.tail_edge, tail);
+        }
+    }
+    return launch(ring16_tile_edge(p.M, p.N, p.K, p.batch, rect), p);
 }
 
 // ---- 16-, 32- and 64-bit integer products on the same pipe --------------------------------------------------------

@@ -926,15 +926,49 @@ static hipError_t launch_ring16_planned(const GemmParams& p, hipStream_t s, Laun
     return launch(pl.tail_edge, ring_batch_range(p, 2, pl.head, p.batch - pl.head));
 }
 
+// the two sub-products of a split single product (see ring16_split): leading columns / rows, then the remaining strip
+static inline void ring_split_params(const GemmParams& p, bool ta, bool tb, int64_t es, const Ring16Split& sp, GemmParams& head, GemmParams& tail) {
+    head = p;
+    tail = p;
+    const char* A = static_cast<const char*>(p.A);
+    const char* B = static_cast<const char*>(p.B);
+    char* C = static_cast<char*>(p.C);
+    const char* bias = static_cast<const char*>(p.bias);
+    if (sp.axis == 1) {                          // columns [0, head) | [head, N)
+        head.N = (int)sp.head;
+        tail.N = p.N - (int)sp.head;
+        tail.B = B + (tb ? sp.head * p.ldb : sp.head) * es;
+        tail.C = C + sp.head * es;
+        if (bias) tail.bias = bias + sp.head * p.bias_cs * es;
+    } else {                                     // rows [0, head) | [head, M)
+        head.M = (int)sp.head;
+        tail.M = p.M - (int)sp.head;
+        tail.A = A + (ta ? sp.head : sp.head * p.lda) * es;
+        tail.C = C + sp.head * p.ldc * es;
+        if (bias) tail.bias = bias + sp.head * p.bias_rs * es;
+    }
+}
+
 template <int DT>
 static hipError_t launch_ring16(bool ta, bool tb, const GemmParams& p, hipStream_t s) {
-    return launch_ring16_planned(p, s, [&](int te, const GemmParams& q) {
+    auto launch = [&](int te, const GemmParams& q) {
         if (te == 256) return launch_ring_wb<DT, 4>(ta, tb, q, s);
         if (te == 224) return launch_ring_wb<DT, 3, 4>(ta, tb, q, s);      // 192 rows x 256 columns
         if (te == 192) return launch_ring_wb<DT, 2, 4>(ta, tb, q, s);      // 128 rows x 256 columns
         if (te == 64) return launch_ring_wb<DT, 1>(ta, tb, q, s);
         return launch_ring_wb<DT, 2>(ta, tb, q, s);
-    }, RECT_128 | RECT_192);
+    };
+    if (p.batch == 1 && p.cmode != C_PARTIAL && !p.Aptr && !p.Bptr && !p.Cptr) {
+        const Ring16Split sp = ring16_split(p.M, p.N, p.K, RECT_128 | RECT_192);
+        if (sp.axis) {
+            GemmParams head, tail;
+            ring_split_params(p, ta, tb, 2, sp, head, tail);
+            const hipError_t e = launch(sp.head_edge, head);
+            if (e != hipSuccess) return e;
+            return launch(sp.tail_edge, tail);
+        }
+    }
+    return launch_ring16_planned(p, s, launch, RECT_128 | RECT_192);
 }
 
 }  // namespace ntg

@@ -140,6 +140,34 @@ static inline Ring16Plan ring16_plan(int64_t M, int64_t N, int64_t K, int64_t ba
     return pl;
 }
 
+// A single large product whose tiles fill the 256 CUs a whole number of times plus a rest spends a full tile time on that
+// rest (8192 x 11008 on 256 x 256 tiles: 1376 tiles = 5.4 rounds, the sixth round a third full).  The split gives the
+// leading tile columns (axis 1) or tile rows (axis 2) to the chosen tile -- as many as make whole rounds, or nearly -- and
+// the remaining strip to a tile chosen for it alone (usually 128 x 256: twice the tiles, each half as long), as two
+// launches on sub-matrices of the same operands.  `head` = elements of the split axis in the first launch; axis 0: no split.
+// The estimate has to improve by 5 % (the second launch costs a few microseconds).
+struct Ring16Split { int axis; int64_t head; int head_edge, tail_edge; };
+static inline Ring16Split ring16_split(int64_t M, int64_t N, int64_t K, int rect = RECT_NONE) {
+    Ring16Split sp = {0, 0, 0, 0};
+    const int edge = ring16_tile_edge(M, N, K, 1, rect);
+    if (edge == 64) return sp;
+    const int64_t tr = ring16_tile_rows(edge), tc = ring16_tile_cols(edge);
+    const int64_t tm = (M + tr - 1) / tr, tn = (N + tc - 1) / tc, T = tm * tn;
+    if (T <= 256 || T % 256 == 0) return sp;
+    double best = 0.95 * ring16_cost_us(edge, T, K);
+    for (int axis = 1; axis <= 2; ++axis) {
+        const int64_t count = axis == 1 ? tn : tm, other = axis == 1 ? tm : tn, step = axis == 1 ? tc : tr;
+        for (int64_t c = 1; c < count; ++c) {
+            const int64_t rest = (axis == 1 ? N : M) - c * step;
+            const int64_t Mt = axis == 1 ? M : rest, Nt = axis == 1 ? rest : N;
+            const int te = ring16_tile_edge(Mt, Nt, K, 1, rect);
+            const double us = ring16_cost_us(edge, other * c, K) + ring16_cost_us(te, ring16_tiles(te, Mt, Nt, 1), K) + 2.0;
+            if (us < best) { best = us; sp.axis = axis; sp.head = c * step; sp.head_edge = edge; sp.tail_edge = te; }
+        }
+    }
+    return sp;
+}
+
 static inline int64_t elem_size(int dt) {
     switch (dt) {
     case DT_I8: case DT_U8: return 1;

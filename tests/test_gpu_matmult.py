@@ -803,3 +803,47 @@ def test_host_entry_staging_large_transfers_threads_and_release():
     _lib.check(lib.ntg_matmult_batch(_lib.FLOAT32, arr([As[i] for i in idx]), arr([Bm] * 5), arr(Cs), 5, m, k, k, n, 0, 0))
     for i in range(5):
         assert np.abs(Cs[i] - want[i]).max() <= float_tol(k, As[idx[i]], Bm)
+
+
+@pytest.mark.parametrize("kind", ["bf16", "int8"])
+def test_single_large_products_split_into_two_launches(kind):
+    """A single product whose tiles make whole rounds over the CUs plus a rest goes out as two launches on sub-matrices
+    (leading tile columns or rows on the chosen tile, the remaining strip on another): the seam must not show -- bias
+    and C0 follow the strip, both transpose layouts, ragged edges.  Checked whole against float64 products on the GPU:
+    Int8 bit-exact (wrapping), BFloat16 within one ulp of the correctly rounded result and equal to it almost everywhere."""
+    lib = _lib.load()
+    st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    gen = torch.Generator(device=DEV).manual_seed(77)
+    cases = [(8192, 1024, 11008, False, True, _lib.C_BIAS), (11008, 1024, 4096, True, False, _lib.C_ACCUMULATE),
+             (5000, 1024, 5000, False, False, _lib.C_ACCUMULATE), (8192, 1024, 11008, False, False, _lib.C_OVERWRITE)]
+    for (m, k, n, ta, tb, mode) in cases:
+        if kind == "bf16":
+            mk = lambda *shape: (torch.randn(*shape, device=DEV, generator=gen) * 0.25).bfloat16()
+        else:
+            mk = lambda *shape: torch.randint(-128, 128, shape, device=DEV, generator=gen, dtype=torch.int8)
+        a, b, c0, bias = mk(m, k), mk(k, n), mk(m, n), mk(n)
+        sa = a.t().contiguous() if ta else a
+        sb = b.t().contiguous() if tb else b
+        c = c0.clone()
+        d = _lib.GemmDesc()
+        d.dtype, d.transpose_a, d.transpose_b, d.c_mode = F.ntg_dtype(a), int(ta), int(tb), mode
+        d.m, d.k, d.n, d.batches = m, k, n, 1
+        if mode == _lib.C_BIAS:
+            d.bias, d.bias_col_stride = bias.data_ptr(), 1
+        _lib.check(lib.ntg_gemm_dev(ctypes.byref(d), sa.data_ptr(), sb.data_ptr(), c.data_ptr(), st))
+        torch.cuda.synchronize()
+        ref = a.double() @ b.double()
+        if mode == _lib.C_ACCUMULATE:
+            ref += c0.double()
+        elif mode == _lib.C_BIAS:
+            ref += bias.double()
+        if kind == "int8":
+            want = (ref.to(torch.int64) & 0xff).to(torch.uint8)
+            assert torch.equal(c.view(torch.uint8), want), (m, k, n, ta, tb, mode)
+        else:
+            want = ref.to(torch.bfloat16)                      # correctly rounded (float64 holds the sum exactly enough)
+            ulp = torch.maximum(ref.abs(), torch.tensor(1e-30, device=DEV, dtype=torch.float64)).log2().floor().exp2() * 2.0 ** -7
+            err = (c.double() - want.double()).abs()
+            assert bool((err <= 1.5 * ulp + 1e-4).all()), (m, k, n, ta, tb, mode, float((err / ulp).max()))
+            assert float((c == want).double().mean()) > 0.97, (m, k, n, ta, tb, mode)
+        del ref
