@@ -14,7 +14,7 @@ hipError_t launch_conv_mfma_bf16(bool tb, int nd, const GemmParams& p, hipStream
     return tb ? launch_conv_cfg<DT_BF16, true, 2, 2, 2, 64>(p, s) : launch_conv_cfg<DT_BF16, false, 2, 2, 2, 64>(p, s);
 }
 hipError_t launch_conv_nhwc_bf16(const GemmParams& p, hipStream_t s) {
-    return launch_ring16_planned(p, s, [&](int te, const GemmParams& q) {
+    return launch_conv_nhwc16_planned(p, s, [&](int te, const GemmParams& q) {
         if (te == 256) return launch_ring_nhwc_cfg<DT_BF16, 4>(q, s);
         if (te == 64) return launch_ring_nhwc_cfg<DT_BF16, 1>(q, s);
         return launch_ring_nhwc_cfg<DT_BF16, 2>(q, s);

@@ -14,7 +14,7 @@ hipError_t launch_conv_mfma_f16(bool tb, int nd, const GemmParams& p, hipStream_
     return tb ? launch_conv_cfg<DT_F16, true, 2, 2, 2, 64>(p, s) : launch_conv_cfg<DT_F16, false, 2, 2, 2, 64>(p, s);
 }
 hipError_t launch_conv_nhwc_f16(const GemmParams& p, hipStream_t s) {
-    return launch_ring16_planned(p, s, [&](int te, const GemmParams& q) {
+    return launch_conv_nhwc16_planned(p, s, [&](int te, const GemmParams& q) {
         if (te == 256) return launch_ring_nhwc_cfg<DT_F16, 4>(q, s);
         if (te == 64) return launch_ring_nhwc_cfg<DT_F16, 1>(q, s);
         return launch_ring_nhwc_cfg<DT_F16, 2>(q, s);

@@ -186,7 +186,8 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
     constexpr int A_TILE_BYTES = GA::TILE_BYTES, STAGE_BYTES = GA::TILE_BYTES + G::TILE_BYTES;
     constexpr int WTM = GA::WT, WTN = G::WT;             // a wavefront's share of the tile: WTM rows x WTN columns
     constexpr bool GATHER4 = CONV == 1 || CONV == 2;     // op(B) gathered element by element from an NCHW image
-    constexpr bool GATHER16 = CONV == 3;                 // op(B) = col^T gathered in 16-byte pieces from a channels-last image
+    constexpr bool GATHER16 = CONV == 3 || CONV == 5;    // op(B) = col^T gathered in 16-byte pieces from a channels-last image
+    constexpr bool HALO = CONV == 5;                     // ... whose copy carries the padding as pixels of zeros: every tap of every window exists
     constexpr bool GATHERW = CONV == 4;                  // op(B) = col^T of a channels-last image, 16-byte pieces along the channels (weight gradient)
     constexpr bool A_KC = !TA, B_KC = GATHER4 ? false : GATHER16 ? true : GATHERW ? false : TB;
     constexpr int BK = G::BK;
@@ -356,7 +357,7 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
         for (int x = 0; x < WB; ++x) {
             const int row = 16 * (wave * WB + x) + (lane >> 2);
             const int n = n0 + row;
-            const uint32_t l = n < p.N ? (uint32_t)n : 0u;
+            const uint32_t l = (n < p.N ? (uint32_t)n : 0u) + (uint32_t)g.n_base;
             const uint32_t oh = fast_div(l, g.div_wo), ow = l - oh * (uint32_t)g.Wo;
             const int ih0 = (int)oh * g.s_r - g.p_r, iw0 = (int)ow * g.s_c - g.p_c;
             uint32_t m = 0;
@@ -382,11 +383,19 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
         if constexpr (GATHER16) {
             const ConvGeom& g = p.conv;
             const char* img = reinterpret_cast<const char*>(B);
+            if constexpr (HALO) {
+                // the image carries its padding (p.conv describes the padded image, padding 0): no tap is ever outside, the
+                // address is a uniform base plus the lane's constant offset, exactly the DMA of a stored operand
+                // (K-steps past the end re-read tap 0: their stage is never multiplied)
+                const int64_t up = k3_k < p.K ? (int64_t)k3_up : 0;
+                dma_1k(img + up, lanepart3[x], lds_tile + (uint32_t)(wave_u * WB + x) * 1024u);
+            } else {
             const uint32_t sr = k3_k < p.K ? (uint32_t)k3_r : 31u, sq = 8u + (uint32_t)k3_q + tq3[x];
             const bool ok = ((cmask3[x] >> sr) & (cmask3[x] >> sq) & 1u) != 0u;
             const char* src = ok ? img + (int64_t)k3_up + lanepart3[x] : reinterpret_cast<const char*>(ring_zero_word);
             asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
                          :: "s"(lds_tile + (uint32_t)(wave_u * WB + x) * 1024u), "v"(src) : "memory");
+            }
             if (x == WB - 1) {
                 // one K-step on: the next 64 bytes of channels of this tap, else the next tap (or the next tap_step taps)
                 const bool merged = g.tap_step > 1;
@@ -869,9 +878,24 @@ static hipError_t launch_ring_conv_cfg(bool tb, const GemmParams& pin, hipStream
     return hipGetLastError();
 }
 
+// ... from a channels-last image that carries its padding as zero pixels (CONV = 5)
+template <int DT, int WB>
+static hipError_t launch_ring_nhwc_halo_cfg(const GemmParams& pin, hipStream_t s) {
+    constexpr int TE = RingGeom<WB, (int)sizeof(typename Elem<DT>::T)>::BM;
+    GemmParams p = pin;
+    p.tiles_m = (p.M + TE - 1) / TE;
+    p.tiles_n = (p.N + TE - 1) / TE;
+    const int64_t blocks = (int64_t)p.tiles_m * p.tiles_n * p.batch;
+    if (blocks <= 0) return hipSuccess;
+    if (blocks > 0x7fffffffLL) return hipErrorInvalidValue;
+    hipLaunchKernelGGL((gemm_ring_kernel<DT, false, true, true, WB, 5>), dim3((unsigned)blocks), dim3(256), 0, s, p);
+    return hipGetLastError();
+}
+
 // convolution with op(B) gathered in 16-byte pieces from a channels-last image (see CONV = 3)
 template <int DT, int WB>
 static hipError_t launch_ring_nhwc_cfg(const GemmParams& pin, hipStream_t s) {
+    if (pin.conv.halo) return launch_ring_nhwc_halo_cfg<DT, WB>(pin, s);
     constexpr int TE = RingGeom<WB, (int)sizeof(typename Elem<DT>::T)>::BM;
     GemmParams p = pin;
     p.tiles_m = (p.M + TE - 1) / TE;
@@ -924,6 +948,23 @@ static hipError_t launch_ring16_planned(const GemmParams& p, hipStream_t s, Laun
     const hipError_t e = launch(pl.edge, ring_batch_range(p, 2, 0, pl.head));
     if (e != hipSuccess) return e;
     return launch(pl.tail_edge, ring_batch_range(p, 2, pl.head, p.batch - pl.head));
+}
+
+// channels-last convolution, 16-bit: the whole tile columns of every image, then the narrow rest of every image on a tile
+// of its own (see ring16_column_split); each part planned over the batch like any other
+template <class Launch>
+static hipError_t launch_conv_nhwc16_planned(const GemmParams& p, hipStream_t s, Launch&& launch) {
+    const int64_t head_cols = p.cmode == C_PARTIAL ? 0 : ring16_column_split(p.M, p.N, p.K, p.batch);
+    if (head_cols == 0) return launch_ring16_planned(p, s, launch);
+    GemmParams head = p, tail = p;
+    head.N = (int)head_cols;
+    tail.N = p.N - (int)head_cols;
+    tail.conv.n_base = p.conv.n_base + (int)head_cols;
+    tail.C = static_cast<char*>(p.C) + head_cols * 2;
+    if (p.bias) tail.bias = static_cast<const char*>(p.bias) + head_cols * p.bias_cs * 2;
+    const hipError_t e = launch_ring16_planned(head, s, launch);
+    if (e != hipSuccess) return e;
+    return launch_ring16_planned(tail, s, launch);
 }
 
 // the two sub-products of a split single product (see ring16_split): leading columns / rows, then the remaining strip

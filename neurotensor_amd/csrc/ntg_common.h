@@ -53,6 +53,11 @@ struct ConvGeom {
     int64_t fold_stride;
     // channels-last convolution of few channels: taps of one tap row per K-step (0 / 1: one tap) and the padded row length
     int tap_step, kq_pad;
+    // channels-last convolution: the copy of the image carries the padding as pixels of zeros (H, W, chan describe the padded
+    // image, p_r = p_c = 0), so the gather needs no validity test
+    int halo;
+    // channels-last convolution: column n of this launch is output pixel n + n_base (a launch on the trailing columns)
+    int n_base;
 };
 
 struct GemmParams {
@@ -140,6 +145,26 @@ static inline Ring16Plan ring16_plan(int64_t M, int64_t N, int64_t K, int64_t ba
     return pl;
 }
 
+static inline double ring16_plan_cost_us(const Ring16Plan& pl, int64_t M, int64_t N, int64_t K, int64_t batch) {
+    if (pl.head >= batch) return ring16_cost_us(pl.edge, ring16_tiles(pl.edge, M, N, batch), K);
+    return ring16_cost_us(pl.edge, ring16_tiles(pl.edge, M, N, pl.head), K) +
+           ring16_cost_us(pl.tail_edge, ring16_tiles(pl.tail_edge, M, N, batch - pl.head), K) + 2.0;
+}
+// A batch of products whose columns are whole tiles plus a narrow rest (a convolution of 56 x 56 images: 3136 output
+// pixels = 12 tiles of 256 and 64 more) spends a whole tile on that rest in every item.  The column split gives the
+// whole tiles of every item to the chosen tile and the rest of every item to a tile chosen for it alone, as two
+// (planned) launches.  head_cols = columns of the first launch; 0: no split.  It has to be 5 % ahead of the batch plan.
+static inline int64_t ring16_column_split(int64_t M, int64_t N, int64_t K, int64_t batch) {
+    const int edge = ring16_tile_edge(M, N, K, batch);
+    if (edge == 64) return 0;
+    const int64_t head_cols = N / edge * edge, rest = N - head_cols;
+    if (head_cols == 0 || rest == 0) return 0;
+    const double whole = ring16_plan_cost_us(ring16_plan(M, N, K, batch), M, N, K, batch);
+    const double split = ring16_plan_cost_us(ring16_plan(M, head_cols, K, batch), M, head_cols, K, batch) +
+                         ring16_plan_cost_us(ring16_plan(M, rest, K, batch), M, rest, K, batch) + 2.0;
+    return split < 0.95 * whole ? head_cols : 0;
+}
+
 // A single large product whose tiles fill the 256 CUs a whole number of times plus a rest spends a full tile time on that
 // rest (8192 x 11008 on 256 x 256 tiles: 1376 tiles = 5.4 rounds, the sixth round a third full).  The split gives the
 // leading tile columns (axis 1) or tile rows (axis 2) to the chosen tile -- as many as make whole rounds, or nearly -- and
@@ -216,11 +241,16 @@ hipError_t launch_splitk_reduce(int dtype, const void* part, int splits, const G
 // conv2d backward helpers (unfold2d.hip): ordered sum of per-image weight gradients; weights of
 // the gradient-to-image convolution
 hipError_t launch_reduce_batch(int dtype, const void* part, void* out, int64_t batch, int64_t n, int accumulate, hipStream_t s);
-hipError_t launch_nchw_to_nhwc(int64_t elem_size, const void* in, void* out, int64_t batch, int64_t C, int64_t P, hipStream_t s);
+// Where the pixels of a channels-last copy go when the copy carries a border of zero pixels: pixel (h, w) of a W-wide image is
+// pixel (h + top) * Wp + (w + left) of a padded image of Hp x Wp pixels.  nullptr / Wp == 0: no border.
+struct HaloMap { int64_t W, H, Wp, Hp, top, left; };
+hipError_t launch_nchw_to_nhwc(int64_t elem_size, const void* in, void* out, int64_t batch, int64_t C, int64_t P, hipStream_t s, const HaloMap* halo = nullptr);
+hipError_t launch_halo_zero(int64_t elem_size, void* out, int64_t batch, int64_t C, const HaloMap& halo, hipStream_t s);   // zeros the border pixels
 hipError_t launch_weights_channels_last(int64_t es, const void* w, void* wp, int64_t rows, int64_t cg, int64_t cgp, int64_t taps, hipStream_t s);
 hipError_t launch_weights_channels_last_rows(int64_t es, const void* w, void* wp, int64_t rows, int64_t cg, int64_t cgp, int64_t k_r, int64_t k_c,
                                              int64_t kq_pad, hipStream_t s);   // tap rows padded from k_c to kq_pad taps
-hipError_t launch_nchw_to_nhwc_padded(int64_t es, const void* in, void* out, int64_t batch, int64_t groups, int64_t cg, int64_t cgp, int64_t P, hipStream_t s);
+hipError_t launch_nchw_to_nhwc_padded(int64_t es, const void* in, void* out, int64_t batch, int64_t groups, int64_t cg, int64_t cgp, int64_t P, hipStream_t s,
+                                      const HaloMap* halo = nullptr);
 hipError_t launch_flip_weights_channels_last(int64_t es, const void* w, void* wt, int64_t groups, int64_t og, int64_t ogp, int64_t cg, int64_t taps, hipStream_t s);
 // channels-last convolution (image [B][pixel][C], weights [O][(r, q, c)]); F16 / BF16 / F32, two spatial axes
 hipError_t launch_conv_nhwc(int dtype, const GemmParams& p, hipStream_t s);

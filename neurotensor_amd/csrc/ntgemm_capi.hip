@@ -865,6 +865,26 @@ static int64_t nhwc_padded_channels(int64_t es, int64_t cg) {
     const int64_t step = 64 / es, cgp = (cg + step - 1) / step * step;
     return cg > 0 && cgp <= (es == 2 ? 4 : 1) * cg ? cgp : 0;
 }
+// The channels-last copy carries the convolution's padding as a border of zero pixels (two axes, non-negative padding):
+// the padded image is as large as the windows reach, every tap of every window then exists, and the kernel's gather needs
+// neither a validity test nor a per-lane address select -- its DMA is that of a stored operand.  gp describes the padded
+// image with padding 0 (what the kernel is told); hm where the copy puts the pixels.
+struct HaloPlan { bool on; ntg::HaloMap hm; Geo3 gp; int64_t vol; };
+static HaloPlan conv_halo(const Geo3& g) {
+    HaloPlan h;
+    std::memset(&h.hm, 0, sizeof h.hm);
+    h.on = false; h.gp = g; h.vol = g.vol();
+    if (g.nd != 2 || g.p[1] < 0 || g.p[2] < 0) return h;
+    const int64_t need_h = (g.o[1] - 1) * g.s[1] + (g.k[1] - 1) * g.d[1] + 1, need_w = (g.o[2] - 1) * g.s[2] + (g.k[2] - 1) * g.d[2] + 1;
+    const int64_t Hp = std::max(need_h, g.p[1] + g.sz[1]), Wp = std::max(need_w, g.p[2] + g.sz[2]);
+    if (Hp * Wp > 2 * g.sz[1] * g.sz[2] + 64) return h;               // (a border larger than the image: not worth the copy)
+    h.hm.W = g.sz[2]; h.hm.H = g.sz[1]; h.hm.Wp = Wp; h.hm.Hp = Hp; h.hm.top = g.p[1]; h.hm.left = g.p[2];
+    h.gp.sz[1] = Hp; h.gp.sz[2] = Wp; h.gp.p[1] = 0; h.gp.p[2] = 0;
+    h.vol = Hp * Wp;
+    h.on = true;
+    return h;
+}
+
 // Few channels per group (up to 32 bytes of them): a pixel of the copy holds 16 or 32 bytes and a K-step covers 4 or 2
 // consecutive taps of a tap row, the row padded to a multiple of that with zero weights -- an RGB 7 x 7 input layer in
 // BFloat16 runs on K = 7 * 8 * 8 instead of 49 * 32.  Forward only.
@@ -887,22 +907,30 @@ static bool conv_nhwc_ok(int dtype, int64_t channels, int64_t out_channels, int6
     if (dtype != ntg::DT_F32 && dtype != ntg::DT_F16 && dtype != ntg::DT_BF16) return false;
     if (g.nd != 2 || !conv_implicit_g(dtype, channels, g)) return false;
     const int64_t es = ntg::elem_size(dtype), cgp = nhwc_padded_channels(es, channels / groups);
-    return cgp > 0 && out_channels > 0 && conv_nhwc_offsets_fit(groups * cgp, es, g);
+    return cgp > 0 && out_channels > 0 && conv_nhwc_offsets_fit(groups * cgp, es, g) && conv_nhwc_offsets_fit(groups * cgp, es, conv_halo(g).gp);
 }
 static int64_t conv_nhwc_workspace(int dtype, int64_t batch, int64_t channels, int64_t out_channels, int64_t groups, const Geo3& g) {
     const int64_t es = ntg::elem_size(dtype), cgp = nhwc_padded_channels(es, channels / groups);
-    return (int64_t)align_up((size_t)(batch * groups * cgp * g.vol() * es), 256) + out_channels * cgp * g.taps() * es;
+    return (int64_t)align_up((size_t)(batch * groups * cgp * conv_halo(g).vol * es), 256) + out_channels * cgp * g.taps() * es;
 }
 static int conv_forward_nhwc(int dtype, const void* image, const void* kernel, void* out, void* ws, int64_t batch, int64_t channels,
                              int64_t out_channels, const Geo3& g, int64_t groups, hipStream_t hs, const MergedTaps* mt = nullptr) {
     const int64_t es = ntg::elem_size(dtype), cg = channels / groups, og = out_channels / groups;
     const int64_t cgp = mt ? mt->cgp : nhwc_padded_channels(es, cg), chp = groups * cgp;      // channels per group / per pixel in the copy
     const int64_t L = g.L(), taps = g.taps(), vol = g.vol(), K = mt ? g.k[1] * mt->kq_pad * cgp : taps * cgp;
+    HaloPlan halo = conv_halo(g);
+    if (mt) { halo.on = false; halo.vol = vol; halo.gp = g; }                    // (the merged-tap form keeps its validity bits)
+    const int64_t volp = halo.vol;                                               // pixels per image of the copy
     char* ws_img = static_cast<char*>(ws);
-    char* ws_w = ws_img + align_up((size_t)(batch * chp * vol * es), 256);
-    hipError_t e = cgp == cg ? ntg::launch_nchw_to_nhwc(es, image, ws_img, batch, channels, vol, hs)
-                             : ntg::launch_nchw_to_nhwc_padded(es, image, ws_img, batch, groups, cg, cgp, vol, hs);
+    char* ws_w = ws_img + align_up((size_t)(batch * chp * volp * es), 256);
+    const ntg::HaloMap* hm = halo.on ? &halo.hm : nullptr;
+    hipError_t e = cgp == cg ? ntg::launch_nchw_to_nhwc(es, image, ws_img, batch, channels, vol, hs, hm)
+                             : ntg::launch_nchw_to_nhwc_padded(es, image, ws_img, batch, groups, cg, cgp, vol, hs, hm);
     if (e != hipSuccess) return hip_fail(e, "channels-last copy launch");
+    if (halo.on && volp != vol) {
+        e = ntg::launch_halo_zero(es, ws_img, batch, chp, halo.hm, hs);
+        if (e != hipSuccess) return hip_fail(e, "border fill launch");
+    }
     e = mt ? ntg::launch_weights_channels_last_rows(es, kernel, ws_w, out_channels, cg, cgp, g.k[1], g.k[2], mt->kq_pad, hs)
            : ntg::launch_weights_channels_last(es, kernel, ws_w, out_channels, cg, cgp, taps, hs);
     if (e != hipSuccess) return hip_fail(e, "weight permutation launch");
@@ -914,11 +942,12 @@ static int conv_forward_nhwc(int dtype, const void* image, const void* kernel, v
         p.B = ws_img + gi * cgp * es;
         p.C = static_cast<char*>(out) + gi * og * L * es;
         p.lda = K; p.ldb = chp; p.ldc = L;
-        p.sA = 0; p.sB = chp * vol; p.sC = out_channels * L;
+        p.sA = 0; p.sB = chp * volp; p.sC = out_channels * L;
         p.cmode = ntg::C_OVERWRITE;
         p.vecA_ok = 1; p.vecB_ok = 1;
-        fill_conv_geom(p.conv, cgp, g);
+        fill_conv_geom(p.conv, cgp, halo.gp);
         p.conv.chan = (int)chp;                    // elements from one pixel to the next
+        p.conv.halo = halo.on ? 1 : 0;
         if (mt) { p.conv.tap_step = (int)mt->T; p.conv.kq_pad = (int)mt->kq_pad; }
         e = ntg::launch_conv_nhwc(dtype, p, hs);
         if (e != hipSuccess) return hip_fail(e, "channels-last convolution launch");
@@ -994,14 +1023,21 @@ static int conv_dimage_nhwc(int dtype, const void* kernel, const void* grad_out,
     const int64_t es = ntg::elem_size(dtype), cg = channels / groups, og = out_channels / groups;
     const int64_t ogp = nhwc_padded_channels(es, og), ochp = groups * ogp;      // out channels per group / per pixel in the copy
     const int64_t L = g.L(), taps = g.taps(), vol = g.vol(), K = taps * ogp;
+    const Geo3 t = geo_dimage(g);
+    const HaloPlan halo = conv_halo(t);                                         // (the "image" of this convolution is dY)
+    const int64_t Lp = halo.vol;
     char* ws_gy = static_cast<char*>(ws);
-    char* ws_w = ws_gy + align_up((size_t)(batch * ochp * L * es), 256);
-    hipError_t e = ogp == og ? ntg::launch_nchw_to_nhwc(es, grad_out, ws_gy, batch, out_channels, L, hs)
-                             : ntg::launch_nchw_to_nhwc_padded(es, grad_out, ws_gy, batch, groups, og, ogp, L, hs);
+    char* ws_w = ws_gy + align_up((size_t)(batch * ochp * Lp * es), 256);
+    const ntg::HaloMap* hm = halo.on ? &halo.hm : nullptr;
+    hipError_t e = ogp == og ? ntg::launch_nchw_to_nhwc(es, grad_out, ws_gy, batch, out_channels, L, hs, hm)
+                             : ntg::launch_nchw_to_nhwc_padded(es, grad_out, ws_gy, batch, groups, og, ogp, L, hs, hm);
     if (e != hipSuccess) return hip_fail(e, "channels-last copy launch");
+    if (halo.on && Lp != L) {
+        e = ntg::launch_halo_zero(es, ws_gy, batch, ochp, halo.hm, hs);
+        if (e != hipSuccess) return hip_fail(e, "border fill launch");
+    }
     e = ntg::launch_flip_weights_channels_last(es, kernel, ws_w, groups, og, ogp, cg, taps, hs);
     if (e != hipSuccess) return hip_fail(e, "weight flip launch");
-    const Geo3 t = geo_dimage(g);
     for (int64_t gi = 0; gi < groups; ++gi) {
         ntg::GemmParams p;
         std::memset(&p, 0, sizeof p);
@@ -1010,11 +1046,12 @@ static int conv_dimage_nhwc(int dtype, const void* kernel, const void* grad_out,
         p.B = ws_gy + gi * ogp * es;
         p.C = static_cast<char*>(d_image) + gi * cg * vol * es;
         p.lda = K; p.ldb = ochp; p.ldc = vol;
-        p.sA = 0; p.sB = ochp * L; p.sC = channels * vol;
+        p.sA = 0; p.sB = ochp * Lp; p.sC = channels * vol;
         p.cmode = accumulate ? ntg::C_ACCUMULATE : ntg::C_OVERWRITE;
         p.vecA_ok = 1; p.vecB_ok = 1;
-        fill_conv_geom(p.conv, ogp, t);
+        fill_conv_geom(p.conv, ogp, halo.gp);
         p.conv.chan = (int)ochp;
+        p.conv.halo = halo.on ? 1 : 0;
         e = ntg::launch_conv_nhwc(dtype, p, hs);
         if (e != hipSuccess) return hip_fail(e, "channels-last conv_dimage launch");
     }

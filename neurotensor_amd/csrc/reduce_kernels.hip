@@ -3,6 +3,8 @@
 // All are HBM bound, deterministic (fixed summation order, no atomics) and launched on the caller's stream.
 #include "ntg_common.h"
 
+#include <algorithm>
+
 namespace ntg {
 
 // out[i] (+)= sum over b of part[b*n + i], b ascending: the order in which per-image weight
@@ -234,13 +236,58 @@ hipError_t launch_flip_weights(int64_t es, const void* w, void* wt, int64_t grou
 
 // out[b][p][c] = in[b][c][p]: an image batch from channel planes to channels-last, 64 x 64 tiles through LDS so that
 // both the loads (along p) and the stores (along c) are coalesced.
+// Where pixel p of the source image goes in a copy that carries a border of zero pixels (Wp == 0: no border, Pp == P)
+struct PixRemap { int64_t Pp; uint32_t W, Wp, off0; };
+__device__ __forceinline__ int64_t remap_pixel(const PixRemap& r, int64_t p) {
+    return r.Wp ? p + (int64_t)((uint32_t)p / r.W) * (r.Wp - r.W) + r.off0 : p;
+}
+static PixRemap make_remap(const HaloMap* h, int64_t P) {
+    PixRemap r;
+    r.Pp = P; r.W = 1; r.Wp = 0; r.off0 = 0;
+    if (h && h->Wp) { r.Pp = h->Hp * h->Wp; r.W = (uint32_t)h->W; r.Wp = (uint32_t)h->Wp; r.off0 = (uint32_t)(h->top * h->Wp + h->left); }
+    return r;
+}
+
+// zeros the border pixels of a channels-last copy [B][Hp * Wp][C] (16-byte pieces; C * sizeof(T) a multiple of 16).
+// Only the border is visited: its pixels are numbered top rows, bottom rows, then the left and right pieces of the
+// image's rows.
+__global__ void __launch_bounds__(256) halo_zero_kernel(uint4* __restrict__ out, const uint32_t per_image, const uint32_t vec_per_pixel, const HaloMap h) {
+    const uint32_t top_n = (uint32_t)(h.top * h.Wp), bot_n = (uint32_t)((h.Hp - h.top - h.H) * h.Wp), side = (uint32_t)(h.Wp - h.W);
+    uint4* img = out + (int64_t)blockIdx.y * (h.Hp * h.Wp) * vec_per_pixel;
+    for (uint32_t i = blockIdx.x * 256u + threadIdx.x; i < per_image; i += gridDim.x * 256u) {
+        uint32_t j = i / vec_per_pixel, pix;
+        const uint32_t v = i - j * vec_per_pixel;
+        if (j < top_n) pix = j;
+        else if (j < top_n + bot_n) pix = (uint32_t)((h.top + h.H) * h.Wp) + (j - top_n);
+        else {
+            j -= top_n + bot_n;
+            const uint32_t row = j / side, c = j - row * side;
+            pix = (uint32_t)((h.top + row) * h.Wp) + (c < (uint32_t)h.left ? c : (uint32_t)h.W + c);
+        }
+        img[(int64_t)pix * vec_per_pixel + v] = make_uint4(0u, 0u, 0u, 0u);
+    }
+}
+hipError_t launch_halo_zero(int64_t es, void* out, int64_t batch, int64_t C, const HaloMap& h, hipStream_t s) {
+    if ((C * es) % 16 != 0 || (reinterpret_cast<uintptr_t>(out) & 15) != 0) return hipErrorInvalidValue;
+    const int64_t vpp = C * es / 16, border = h.Hp * h.Wp - h.H * h.W, per_image = border * vpp;
+    if (batch <= 0 || per_image <= 0) return hipSuccess;
+    if (per_image > 0x7fffffffLL || h.Hp * h.Wp > 0x7fffffffLL) return hipErrorInvalidValue;
+    const int64_t gx = std::min<int64_t>((per_image + 255) / 256, 64);
+    for (int64_t b0 = 0; b0 < batch; b0 += 65535) {
+        const int64_t nb = std::min<int64_t>(batch - b0, 65535);
+        hipLaunchKernelGGL(halo_zero_kernel, dim3((unsigned)gx, (unsigned)nb), dim3(256), 0, s,
+                           (uint4*)out + b0 * h.Hp * h.Wp * vpp, (uint32_t)per_image, (uint32_t)vpp, h);
+    }
+    return hipGetLastError();
+}
+
 template <class T>
-__global__ void __launch_bounds__(256) nchw_to_nhwc_kernel(const T* __restrict__ in, T* __restrict__ out, const int64_t C, const int64_t P) {
+__global__ void __launch_bounds__(256) nchw_to_nhwc_kernel(const T* __restrict__ in, T* __restrict__ out, const int64_t C, const int64_t P, const PixRemap r) {
     __shared__ T tile[64][65];
     const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
     const int64_t p0 = (int64_t)blockIdx.x * 64, c0 = (int64_t)blockIdx.y * 64, b = blockIdx.z;
     const T* src = in + b * C * P;
-    T* dst = out + b * C * P;
+    T* dst = out + b * C * r.Pp;
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
         const int64_t c = c0 + ty + 4 * i, pp = p0 + tx;
@@ -250,7 +297,7 @@ __global__ void __launch_bounds__(256) nchw_to_nhwc_kernel(const T* __restrict__
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
         const int64_t pp = p0 + ty + 4 * i, c = c0 + tx;
-        if (c < C && pp < P) dst[pp * C + c] = tile[tx][ty + 4 * i];
+        if (c < C && pp < P) dst[remap_pixel(r, pp) * C + c] = tile[tx][ty + 4 * i];
     }
 }
 
@@ -258,14 +305,14 @@ __global__ void __launch_bounds__(256) nchw_to_nhwc_kernel(const T* __restrict__
 // thread loads VEC pixels of one channel, the tile goes through LDS as single elements (row pitch chosen so that the
 // column-wise read-back spreads over the banks), and a thread stores VEC channels of one pixel.
 template <class T>
-__global__ void __launch_bounds__(256) nchw_to_nhwc_vec_kernel(const T* __restrict__ in, T* __restrict__ out, const int64_t C, const int64_t P) {
+__global__ void __launch_bounds__(256) nchw_to_nhwc_vec_kernel(const T* __restrict__ in, T* __restrict__ out, const int64_t C, const int64_t P, const PixRemap r) {
     constexpr int VEC = 16 / (int)sizeof(T), VPR = 64 / VEC;            // elements per vector, vectors per tile row
     constexpr int PITCH = sizeof(T) == 2 ? 66 : 65;                     // elements: 33 / 65 words
     typedef T TV __attribute__((ext_vector_type(VEC)));
     __shared__ T tile[64 * PITCH];
     const int64_t p0 = (int64_t)blockIdx.x * 64, c0 = (int64_t)blockIdx.y * 64, b = blockIdx.z;
     const T* src = in + b * C * P;
-    T* dst = out + b * C * P;
+    T* dst = out + b * C * r.Pp;
 #pragma unroll
     for (int i = 0; i < 64 * VPR / 256; ++i) {
         const int v = threadIdx.x + 256 * i, c = v / VPR, pv = v % VPR;
@@ -283,13 +330,14 @@ __global__ void __launch_bounds__(256) nchw_to_nhwc_vec_kernel(const T* __restri
             TV x;
 #pragma unroll
             for (int e = 0; e < VEC; ++e) x[e] = tile[(cv * VEC + e) * PITCH + pp];
-            *reinterpret_cast<TV*>(dst + (p0 + pp) * C + c0 + cv * VEC) = x;
+            *reinterpret_cast<TV*>(dst + remap_pixel(r, p0 + pp) * C + c0 + cv * VEC) = x;
         }
     }
 }
 
-hipError_t launch_nchw_to_nhwc(int64_t es, const void* in, void* out, int64_t batch, int64_t C, int64_t P, hipStream_t s) {
+hipError_t launch_nchw_to_nhwc(int64_t es, const void* in, void* out, int64_t batch, int64_t C, int64_t P, hipStream_t s, const HaloMap* halo) {
     if (batch * C * P == 0) return hipSuccess;
+    const PixRemap r = make_remap(halo, P);
     const int64_t gx = (P + 63) / 64, gy = (C + 63) / 64;
     if (gx > 0x7fffffffLL || gy > 65535) return hipErrorInvalidValue;
     const int64_t vec = 16 / es;
@@ -298,11 +346,11 @@ hipError_t launch_nchw_to_nhwc(int64_t es, const void* in, void* out, int64_t ba
         const int64_t nb = batch - b0 < 65535 ? batch - b0 : 65535;
         const dim3 g((unsigned)gx, (unsigned)gy, (unsigned)nb), t(256);
         const char* src = static_cast<const char*>(in) + b0 * C * P * es;
-        char* dst = static_cast<char*>(out) + b0 * C * P * es;
-        if (es == 2 && vec_ok) hipLaunchKernelGGL(nchw_to_nhwc_vec_kernel<uint16_t>, g, t, 0, s, (const uint16_t*)src, (uint16_t*)dst, C, P);
-        else if (es == 4 && vec_ok) hipLaunchKernelGGL(nchw_to_nhwc_vec_kernel<uint32_t>, g, t, 0, s, (const uint32_t*)src, (uint32_t*)dst, C, P);
-        else if (es == 2) hipLaunchKernelGGL(nchw_to_nhwc_kernel<uint16_t>, g, t, 0, s, (const uint16_t*)src, (uint16_t*)dst, C, P);
-        else if (es == 4) hipLaunchKernelGGL(nchw_to_nhwc_kernel<uint32_t>, g, t, 0, s, (const uint32_t*)src, (uint32_t*)dst, C, P);
+        char* dst = static_cast<char*>(out) + b0 * C * r.Pp * es;
+        if (es == 2 && vec_ok) hipLaunchKernelGGL(nchw_to_nhwc_vec_kernel<uint16_t>, g, t, 0, s, (const uint16_t*)src, (uint16_t*)dst, C, P, r);
+        else if (es == 4 && vec_ok) hipLaunchKernelGGL(nchw_to_nhwc_vec_kernel<uint32_t>, g, t, 0, s, (const uint32_t*)src, (uint32_t*)dst, C, P, r);
+        else if (es == 2) hipLaunchKernelGGL(nchw_to_nhwc_kernel<uint16_t>, g, t, 0, s, (const uint16_t*)src, (uint16_t*)dst, C, P, r);
+        else if (es == 4) hipLaunchKernelGGL(nchw_to_nhwc_kernel<uint32_t>, g, t, 0, s, (const uint32_t*)src, (uint32_t*)dst, C, P, r);
         else return hipErrorInvalidValue;
     }
     return hipGetLastError();
@@ -465,13 +513,13 @@ hipError_t launch_weights_channels_last_rows(int64_t es, const void* w, void* wp
 // every group padded to cgp.  64 x 64 tiles of (channel inside the group, pixel) through LDS, like the plain copy.
 template <class T>
 __global__ void __launch_bounds__(256) nchw_to_nhwc_pad_kernel(const T* __restrict__ in, T* __restrict__ out, const int64_t groups,
-                                                               const int64_t cg, const int64_t cgp, const int64_t P, const int cblocks) {
+                                                               const int64_t cg, const int64_t cgp, const int64_t P, const int cblocks, const PixRemap r) {
     __shared__ T tile[64][65];
     const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
     const int64_t g = blockIdx.y / cblocks, c0 = (int64_t)(blockIdx.y % cblocks) * 64;
     const int64_t p0 = (int64_t)blockIdx.x * 64, b = blockIdx.z;
     const T* src = in + (b * groups + g) * cg * P;
-    T* dst = out + b * P * groups * cgp + g * cgp;
+    T* dst = out + b * r.Pp * groups * cgp + g * cgp;
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
         const int64_t c = c0 + ty + 4 * i, pp = p0 + tx;
@@ -481,7 +529,7 @@ __global__ void __launch_bounds__(256) nchw_to_nhwc_pad_kernel(const T* __restri
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
         const int64_t pp = p0 + ty + 4 * i, c = c0 + tx;
-        if (c < cgp && pp < P) dst[pp * groups * cgp + c] = tile[tx][ty + 4 * i];
+        if (c < cgp && pp < P) dst[remap_pixel(r, pp) * groups * cgp + c] = tile[tx][ty + 4 * i];
     }
 }
 
@@ -489,14 +537,14 @@ __global__ void __launch_bounds__(256) nchw_to_nhwc_pad_kernel(const T* __restri
 // cg channels (each a coalesced stream over the pixels) and stores the padded run with 16-byte stores.
 template <class T, int CP>
 __global__ void __launch_bounds__(256) nchw_to_nhwc_few_kernel(const T* __restrict__ in, T* __restrict__ out, const int64_t total, const int64_t groups,
-                                                               const int64_t cg, const int64_t P) {
+                                                               const int64_t cg, const int64_t P, const PixRemap r) {
     constexpr int VEC = 16 / (int)sizeof(T);
     typedef T TV __attribute__((ext_vector_type(VEC)));
     const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (idx >= total) return;
     const int64_t pp = idx % P, bg = idx / P, b = bg / groups, g = bg - b * groups;
     const T* src = in + bg * cg * P + pp;
-    TV* dst = reinterpret_cast<TV*>(out + ((b * P + pp) * groups + g) * CP);
+    TV* dst = reinterpret_cast<TV*>(out + ((b * r.Pp + remap_pixel(r, pp)) * groups + g) * CP);
 #pragma unroll
     for (int v = 0; v < CP / VEC; ++v) {
         TV x;
@@ -506,16 +554,18 @@ __global__ void __launch_bounds__(256) nchw_to_nhwc_few_kernel(const T* __restri
     }
 }
 
-hipError_t launch_nchw_to_nhwc_padded(int64_t es, const void* in, void* out, int64_t batch, int64_t groups, int64_t cg, int64_t cgp, int64_t P, hipStream_t s) {
+hipError_t launch_nchw_to_nhwc_padded(int64_t es, const void* in, void* out, int64_t batch, int64_t groups, int64_t cg, int64_t cgp, int64_t P, hipStream_t s,
+                                      const HaloMap* halo) {
     if (batch * groups * cgp * P == 0) return hipSuccess;
+    const PixRemap r = make_remap(halo, P);
     if (cgp * es <= 32 && (cgp * es) % 16 == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0) {
         const int64_t total = batch * groups * P, blocks = (total + 255) / 256;
         if (blocks <= 0x7fffffffLL) {
             const dim3 g((unsigned)blocks), t(256);
-            if (es == 2 && cgp == 8) hipLaunchKernelGGL((nchw_to_nhwc_few_kernel<uint16_t, 8>), g, t, 0, s, (const uint16_t*)in, (uint16_t*)out, total, groups, cg, P);
-            else if (es == 2) hipLaunchKernelGGL((nchw_to_nhwc_few_kernel<uint16_t, 16>), g, t, 0, s, (const uint16_t*)in, (uint16_t*)out, total, groups, cg, P);
-            else if (es == 4 && cgp == 4) hipLaunchKernelGGL((nchw_to_nhwc_few_kernel<uint32_t, 4>), g, t, 0, s, (const uint32_t*)in, (uint32_t*)out, total, groups, cg, P);
-            else if (es == 4) hipLaunchKernelGGL((nchw_to_nhwc_few_kernel<uint32_t, 8>), g, t, 0, s, (const uint32_t*)in, (uint32_t*)out, total, groups, cg, P);
+            if (es == 2 && cgp == 8) hipLaunchKernelGGL((nchw_to_nhwc_few_kernel<uint16_t, 8>), g, t, 0, s, (const uint16_t*)in, (uint16_t*)out, total, groups, cg, P, r);
+            else if (es == 2) hipLaunchKernelGGL((nchw_to_nhwc_few_kernel<uint16_t, 16>), g, t, 0, s, (const uint16_t*)in, (uint16_t*)out, total, groups, cg, P, r);
+            else if (es == 4 && cgp == 4) hipLaunchKernelGGL((nchw_to_nhwc_few_kernel<uint32_t, 4>), g, t, 0, s, (const uint32_t*)in, (uint32_t*)out, total, groups, cg, P, r);
+            else if (es == 4) hipLaunchKernelGGL((nchw_to_nhwc_few_kernel<uint32_t, 8>), g, t, 0, s, (const uint32_t*)in, (uint32_t*)out, total, groups, cg, P, r);
             else return hipErrorInvalidValue;
             return hipGetLastError();
         }
@@ -526,9 +576,9 @@ hipError_t launch_nchw_to_nhwc_padded(int64_t es, const void* in, void* out, int
         const int64_t nb = batch - b0 < 65535 ? batch - b0 : 65535;
         const dim3 g((unsigned)gx, (unsigned)gy, (unsigned)nb), t(256);
         const char* src = static_cast<const char*>(in) + b0 * groups * cg * P * es;
-        char* dst = static_cast<char*>(out) + b0 * groups * cgp * P * es;
-        if (es == 2) hipLaunchKernelGGL(nchw_to_nhwc_pad_kernel<uint16_t>, g, t, 0, s, (const uint16_t*)src, (uint16_t*)dst, groups, cg, cgp, P, (int)cblocks);
-        else if (es == 4) hipLaunchKernelGGL(nchw_to_nhwc_pad_kernel<uint32_t>, g, t, 0, s, (const uint32_t*)src, (uint32_t*)dst, groups, cg, cgp, P, (int)cblocks);
+        char* dst = static_cast<char*>(out) + b0 * groups * cgp * r.Pp * es;
+        if (es == 2) hipLaunchKernelGGL(nchw_to_nhwc_pad_kernel<uint16_t>, g, t, 0, s, (const uint16_t*)src, (uint16_t*)dst, groups, cg, cgp, P, (int)cblocks, r);
+        else if (es == 4) hipLaunchKernelGGL(nchw_to_nhwc_pad_kernel<uint32_t>, g, t, 0, s, (const uint32_t*)src, (uint32_t*)dst, groups, cg, cgp, P, (int)cblocks, r);
         else return hipErrorInvalidValue;
     }
     return hipGetLastError();

@@ -77,13 +77,14 @@ def test_argument_errors_do_not_need_a_device():
     # a 1x1 kernel with unit stride and no padding is a product on the image where it lies: no buffer for any dtype
     assert lib.ntg_conv2d_forward_workspace_bytes(_lib.INT32, 2, 3, 8, 8, 1, 1, 1, 1, 0, 0, 1, 1) == 0
     assert lib.ntg_conv2d_forward_workspace_bytes(_lib.INT32, 2, 3, 8, 8, 1, 1, 2, 1, 0, 0, 1, 1) == 2 * 3 * 4 * 8 * 4
-    # the faster forward form: channels-last copy of the image (256-byte aligned) + permuted weights, when the channels of
-    # a group fill whole 64-byte runs; else what the plain query says
+    # the faster forward form: channels-last copy of the image with its zero border (the padding made real: 7x7 -> 9x9;
+    # 256-byte aligned) + permuted weights, when the channels of a group fill whole 64-byte runs; else what the plain query says
     fast = lib.ntg_conv2d_fast_workspace_bytes
-    assert fast(_lib.BFLOAT16, 2, 64, 7, 7, 48, 3, 3, 1, 1, 1, 1, 1, 1, 2) == 12544 + 48 * 32 * 9 * 2    # 2*64*49*2 = 12544
-    assert fast(_lib.FLOAT32, 1, 16, 5, 5, 8, 3, 3, 1, 1, 1, 1, 1, 1, 1) == 1792 + 8 * 16 * 9 * 4        # 1600 -> 1792
+    assert fast(_lib.BFLOAT16, 2, 64, 7, 7, 48, 3, 3, 1, 1, 1, 1, 1, 1, 2) == 20736 + 48 * 32 * 9 * 2    # 2*64*81*2 = 20736
+    assert fast(_lib.FLOAT32, 1, 16, 5, 5, 8, 3, 3, 1, 1, 1, 1, 1, 1, 1) == 3328 + 8 * 16 * 9 * 4        # 16*49*4 = 3136 -> 3328
     # 16-bit: channels per group are padded to whole 64-byte runs in the copy (up to 4x); Float32 takes whole runs only
-    assert fast(_lib.BFLOAT16, 2, 40, 5, 5, 8, 3, 3, 1, 1, 1, 1, 1, 1, 1) == 6400 + 8 * 64 * 9 * 2        # 40 -> 64 channels
+    assert fast(_lib.BFLOAT16, 2, 40, 5, 5, 8, 3, 3, 1, 1, 1, 1, 1, 1, 1) == 12544 + 8 * 64 * 9 * 2       # 40 -> 64 channels, 5x5 -> 7x7
+    assert fast(_lib.BFLOAT16, 2, 64, 5, 5, 8, 3, 3, 2, 2, 0, 0, 1, 1, 1) == 6400 + 8 * 64 * 9 * 2        # no padding: no border
     assert fast(_lib.FLOAT32, 1, 24, 8, 8, 4, 3, 3, 1, 1, 1, 1, 1, 1, 1) == 0                             # 24 is not a multiple of 16
     # up to 32 bytes of channels per group: pixels of 16 or 32 bytes, 4 or 2 taps of a tap row per K-step (rows padded to that)
     assert fast(_lib.BFLOAT16, 1, 16, 5, 5, 8, 3, 3, 1, 1, 1, 1, 1, 1, 1) == 1024 + 8 * 3 * 4 * 16 * 2   # 16 channels, rows of 3 -> 4 taps

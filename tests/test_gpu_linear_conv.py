@@ -10,7 +10,7 @@ import torch
 import oracle
 from neurotensor_amd import _lib
 from neurotensor_amd import functional as F
-from util import HALF_REL, float_tol, from_torch, randn, to_f64, to_torch
+from util import HALF_REL, assert_one_rounding, float_tol, from_torch, randn, to_f64, to_torch
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
@@ -663,13 +663,19 @@ def test_config5a_conv2d_resnet_block():
         assert np.abs(out[b:b + 1].cpu().numpy() - ref).max() <= tol
     ref_all = torch.nn.functional.conv2d(tx.double(), tw.double(), padding=1)
     assert (out.double() - ref_all).abs().max().item() <= tol
-    # the same block in BFloat16: the first 59 images and the last 5 come from two launches on different tiles
+    # the same block in BFloat16: output pixels 0 .. 3071 of every image (12 tiles of 256) and pixels 3072 .. 3135 come from
+    # two launches on different tiles, both gathering from a channels-last copy that carries the padding as a zero border
     xh, wh = tx.bfloat16(), tw.bfloat16()
     outh = F.conv2d(xh, wh, stride=1, padding=1)
     refh = torch.nn.functional.conv2d(xh.double(), wh.double(), padding=1)
     scale = refh.abs().max().item()
-    for lo, hi in ((0, 59), (59, 64)):
-        assert (outh[lo:hi].double() - refh[lo:hi]).abs().max().item() <= HALF_REL * scale
+    flat, flat_ref = outh.double().reshape(64, 256, 3136), refh.reshape(64, 256, 3136)
+    for lo, hi in ((0, 3072), (3072, 3136)):
+        assert (flat[:, :, lo:hi] - flat_ref[:, :, lo:hi]).abs().max().item() <= HALF_REL * scale
+    # and one rounding of the exact sum: two whole images, element by element
+    for b in (0, 63):
+        spread = torch.nn.functional.conv2d(xh[b:b + 1].double() ** 2, wh.double() ** 2, padding=1).sqrt()
+        assert_one_rounding(outh[b:b + 1].double().cpu().numpy(), refh[b:b + 1].cpu().numpy(), spread.cpu().numpy(), 2304, "bf16", f"conv image {b}")
     del ref_all, refh
 
 
@@ -691,6 +697,10 @@ def test_config5a_conv2d_gradients_full_size():
         if half:
             assert ex <= HALF_REL * rx.grad.abs().max().item()
             assert ew <= HALF_REL * rw.grad.abs().max().item()
+            # dX is one rounding of the exact sum (whole tile columns and the narrow rest come from two launches)
+            for b in (0, 63):
+                spread = torch.nn.functional.conv_transpose2d(tg[b:b + 1].double() ** 2, tw.double() ** 2, padding=1).sqrt()
+                assert_one_rounding(dx[b:b + 1].double().cpu().numpy(), rx.grad[b:b + 1].cpu().numpy(), spread.cpu().numpy(), 2304, "bf16", f"dX image {b}")
         else:
             assert ex <= 1e-5 * 2304 * float(tg.abs().max() * tw.abs().max())
             assert ew <= 1e-5 * 200704 * float(tg.abs().max() * tx.abs().max())
