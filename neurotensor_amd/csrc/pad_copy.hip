@@ -13,36 +13,45 @@ typedef uint32_t padx4 __attribute__((ext_vector_type(4)));
 template <class T>
 __global__ void __launch_bounds__(256) pad_copy_kernel(const T* __restrict__ src, const int64_t ld_src, const int64_t s_src,
                                                        T* __restrict__ dst, const int64_t ld_dst, const int64_t s_dst,
-                                                       const int64_t rows, const int64_t cols, const int64_t rows_dst, const int64_t batch) {
+                                                       const int64_t rows, const int64_t cols, const int64_t rows_dst, const int64_t batch, const int sh) {
     constexpr int V = 16 / (int)sizeof(T);
-    const int64_t vpr = ld_dst / V, total = batch * rows_dst * vpr;
-    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
-        const int64_t v = i % vpr, r = (i / vpr) % rows_dst, b = i / (vpr * rows_dst);
+    // a block covers 256 >> sh consecutive rows (of all items, counted through) x 1 << sh chunks of 16 bytes; blockIdx.y
+    // counts the pieces of rows longer than 256 chunks (sh = 8)
+    const int64_t vpr = ld_dst / V, v = (int64_t)blockIdx.y * 256 + (threadIdx.x & ((1u << sh) - 1u));
+    const int64_t gr = (int64_t)blockIdx.x * (256 >> sh) + (threadIdx.x >> sh);
+    if (v >= vpr || gr >= batch * rows_dst) return;
+    const int64_t b = batch == 1 ? 0 : gr / rows_dst, r = gr - b * rows_dst;
+    const T* s = src + b * s_src + r * ld_src + v * V;
+    padx4 w;
+    if (r < rows && v * V + V <= cols) {
+        // 16 bytes inside the row: one load, whatever the address (global memory takes unaligned vector accesses)
+        __builtin_memcpy(&w, s, 16);
+    } else {
         T tmp[V];
-        const T* s = src + b * s_src + r * ld_src + v * V;
 #pragma unroll
         for (int e = 0; e < V; ++e) tmp[e] = (r < rows && v * V + e < cols) ? s[e] : (T)0;
-        padx4 w;
         __builtin_memcpy(&w, tmp, 16);
-        *reinterpret_cast<padx4*>(dst + b * s_dst + r * ld_dst + v * V) = w;
     }
+    *reinterpret_cast<padx4*>(dst + b * s_dst + r * ld_dst + v * V) = w;
 }
 
 // dst[b][r][0 .. cols) = src[b][r][0 .. cols): src rows are 16-byte aligned with pitch ld_src, dst has any pitch and alignment
 template <class T>
 __global__ void __launch_bounds__(256) unpad_copy_kernel(const T* __restrict__ src, const int64_t ld_src, const int64_t s_src,
                                                          T* __restrict__ dst, const int64_t ld_dst, const int64_t s_dst,
-                                                         const int64_t rows, const int64_t cols, const int64_t batch) {
+                                                         const int64_t rows, const int64_t cols, const int64_t batch, const int sh) {
     constexpr int V = 16 / (int)sizeof(T);
-    const int64_t vpr = (cols + V - 1) / V, total = batch * rows * vpr;
-    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
-        const int64_t v = i % vpr, r = (i / vpr) % rows, b = i / (vpr * rows);
-        const padx4 w = *reinterpret_cast<const padx4*>(src + b * s_src + r * ld_src + v * V);
+    const int64_t vpr = (cols + V - 1) / V, v = (int64_t)blockIdx.y * 256 + (threadIdx.x & ((1u << sh) - 1u));
+    const int64_t gr = (int64_t)blockIdx.x * (256 >> sh) + (threadIdx.x >> sh);
+    if (v >= vpr || gr >= batch * rows) return;
+    const int64_t b = batch == 1 ? 0 : gr / rows, r = gr - b * rows;
+    const padx4 w = *reinterpret_cast<const padx4*>(src + b * s_src + r * ld_src + v * V);
+    T* d = dst + b * s_dst + r * ld_dst + v * V;
+    if (v * V + V <= cols) {
+        __builtin_memcpy(d, &w, 16);                 // (one store, aligned or not)
+    } else {
         T tmp[V];
         __builtin_memcpy(tmp, &w, 16);
-        T* d = dst + b * s_dst + r * ld_dst + v * V;
 #pragma unroll
         for (int e = 0; e < V; ++e)
             if (v * V + e < cols) d[e] = tmp[e];
@@ -63,24 +72,37 @@ __global__ void __launch_bounds__(256) bias_fill_kernel(const T* __restrict__ bi
     }
 }
 
+// log2 of the lanes a block gives to one row: rows of up to 256 chunks share a block with their neighbours
+static int row_shift(int64_t vpr) {
+    int sh = 0;
+    while (sh < 8 && (1 << sh) < vpr) ++sh;
+    return sh;
+}
+
 hipError_t launch_pad_copy(int64_t es, const void* src, int64_t ld_src, int64_t s_src, void* dst, int64_t ld_dst, int64_t s_dst,
                            int64_t rows, int64_t cols, int64_t rows_dst, int64_t batch, hipStream_t s) {
-    const int64_t total = batch * rows_dst * (ld_dst * es / 16);
-    if (total <= 0) return hipSuccess;
-    const dim3 g(grid_for(total)), t(256);
-    if (es == 1) hipLaunchKernelGGL(pad_copy_kernel<uint8_t>, g, t, 0, s, (const uint8_t*)src, ld_src, s_src, (uint8_t*)dst, ld_dst, s_dst, rows, cols, rows_dst, batch);
-    else if (es == 2) hipLaunchKernelGGL(pad_copy_kernel<uint16_t>, g, t, 0, s, (const uint16_t*)src, ld_src, s_src, (uint16_t*)dst, ld_dst, s_dst, rows, cols, rows_dst, batch);
+    const int64_t vpr = ld_dst * es / 16;
+    const int sh = row_shift(vpr);
+    const int64_t gx = (batch * rows_dst + (256 >> sh) - 1) / (256 >> sh), gy = (vpr + 255) / 256;
+    if (gx <= 0 || gy <= 0) return hipSuccess;
+    if (gx > 0x7fffffffLL || gy > 65535) return hipErrorInvalidValue;
+    const dim3 g((unsigned)gx, (unsigned)gy), t(256);
+    if (es == 1) hipLaunchKernelGGL(pad_copy_kernel<uint8_t>, g, t, 0, s, (const uint8_t*)src, ld_src, s_src, (uint8_t*)dst, ld_dst, s_dst, rows, cols, rows_dst, batch, sh);
+    else if (es == 2) hipLaunchKernelGGL(pad_copy_kernel<uint16_t>, g, t, 0, s, (const uint16_t*)src, ld_src, s_src, (uint16_t*)dst, ld_dst, s_dst, rows, cols, rows_dst, batch, sh);
     else return hipErrorInvalidValue;
     return hipGetLastError();
 }
 
 hipError_t launch_unpad_copy(int64_t es, const void* src, int64_t ld_src, int64_t s_src, void* dst, int64_t ld_dst, int64_t s_dst,
                              int64_t rows, int64_t cols, int64_t batch, hipStream_t s) {
-    const int64_t total = batch * rows * ((cols * es + 15) / 16);
-    if (total <= 0) return hipSuccess;
-    const dim3 g(grid_for(total)), t(256);
-    if (es == 1) hipLaunchKernelGGL(unpad_copy_kernel<uint8_t>, g, t, 0, s, (const uint8_t*)src, ld_src, s_src, (uint8_t*)dst, ld_dst, s_dst, rows, cols, batch);
-    else if (es == 2) hipLaunchKernelGGL(unpad_copy_kernel<uint16_t>, g, t, 0, s, (const uint16_t*)src, ld_src, s_src, (uint16_t*)dst, ld_dst, s_dst, rows, cols, batch);
+    const int64_t vpr = (cols * es + 15) / 16;
+    const int sh = row_shift(vpr);
+    const int64_t gx = (batch * rows + (256 >> sh) - 1) / (256 >> sh), gy = (vpr + 255) / 256;
+    if (gx <= 0 || gy <= 0) return hipSuccess;
+    if (gx > 0x7fffffffLL || gy > 65535) return hipErrorInvalidValue;
+    const dim3 g((unsigned)gx, (unsigned)gy), t(256);
+    if (es == 1) hipLaunchKernelGGL(unpad_copy_kernel<uint8_t>, g, t, 0, s, (const uint8_t*)src, ld_src, s_src, (uint8_t*)dst, ld_dst, s_dst, rows, cols, batch, sh);
+    else if (es == 2) hipLaunchKernelGGL(unpad_copy_kernel<uint16_t>, g, t, 0, s, (const uint16_t*)src, ld_src, s_src, (uint16_t*)dst, ld_dst, s_dst, rows, cols, batch, sh);
     else return hipErrorInvalidValue;
     return hipGetLastError();
 }
