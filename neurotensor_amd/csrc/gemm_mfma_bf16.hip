@@ -21,7 +21,7 @@ hipError_t launch_conv_nhwc_bf16(const GemmParams& p, hipStream_t s) {
     });
 }
 hipError_t launch_conv_nhwc_dw_bf16(bool ta, const GemmParams& p, hipStream_t s) {
-    return launch_ring16_planned(p, s, [&](int te, const GemmParams& q) {
+    return launch_conv_nhwc16_planned(p, s, [&](int te, const GemmParams& q) {
         if (ta) {
             if (te == 256) return launch_ring_nhwc_dw_cfg<DT_BF16, 4, true>(q, s);
             if (te == 64) return launch_ring_nhwc_dw_cfg<DT_BF16, 1, true>(q, s);

@@ -427,14 +427,14 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
     if constexpr (GATHERW) {
         const ConvGeom& g = p.conv;
         constexpr int CH = G::CHUNKS;
-        const uint32_t cgc = (uint32_t)p.N / (uint32_t)g.k_rc;               // channels of the slice: N = taps * channels
+        const uint32_t cgc = (uint32_t)(g.n_total ? g.n_total : p.N) / (uint32_t)g.k_rc;   // channels of the slice: N = taps * channels
 #pragma unroll
         for (int x = 0; x < WB; ++x) {
             const int j = wave * WB + x;
             const int krow = (64 / CH) * j + lane / CH;
             const int chunk = (lane % CH) ^ (ES == 2 ? 2 * (krow & 3) : 8 * ((krow >> 2) & 1));
             const int n = n0 + chunk * G::VEL;
-            const uint32_t nn = n < p.N ? (uint32_t)n : 0u;
+            const uint32_t nn = (n < p.N ? (uint32_t)n : 0u) + (uint32_t)g.n_base;
             const uint32_t t = nn / cgc, c = nn - t * cgc;
             const uint32_t r = fast_div(t, g.div_kc), q = t - r * (uint32_t)g.k_c;
             krow4[x] = n < p.N ? krow : 0x40000000;                       // columns past the edge: never inside
@@ -950,8 +950,8 @@ static hipError_t launch_ring16_planned(const GemmParams& p, hipStream_t s, Laun
     return launch(pl.tail_edge, ring_batch_range(p, 2, pl.head, p.batch - pl.head));
 }
 
-// channels-last convolution, 16-bit: the whole tile columns of every image, then the narrow rest of every image on a tile
-// of its own (see ring16_column_split); each part planned over the batch like any other
+// channels-last convolution and weight gradient, 16-bit: the leading columns of every item, then the remaining ones on a tile
+// of their own (see ring16_column_split); each part planned over the batch like any other
 template <class Launch>
 static hipError_t launch_conv_nhwc16_planned(const GemmParams& p, hipStream_t s, Launch&& launch) {
     const int64_t head_cols = p.cmode == C_PARTIAL ? 0 : ring16_column_split(p.M, p.N, p.K, p.batch);
@@ -960,6 +960,7 @@ static hipError_t launch_conv_nhwc16_planned(const GemmParams& p, hipStream_t s,
     head.N = (int)head_cols;
     tail.N = p.N - (int)head_cols;
     tail.conv.n_base = p.conv.n_base + (int)head_cols;
+    head.conv.n_total = tail.conv.n_total = p.conv.n_total ? p.conv.n_total : p.N;
     tail.C = static_cast<char*>(p.C) + head_cols * 2;
     if (p.bias) tail.bias = static_cast<const char*>(p.bias) + head_cols * p.bias_cs * 2;
     const hipError_t e = launch_ring16_planned(head, s, launch);

@@ -56,8 +56,9 @@ struct ConvGeom {
     // channels-last convolution: the copy of the image carries the padding as pixels of zeros (H, W, chan describe the padded
     // image, p_r = p_c = 0), so the gather needs no validity test
     int halo;
-    // channels-last convolution: column n of this launch is output pixel n + n_base (a launch on the trailing columns)
-    int n_base;
+    // channels-last convolution and weight gradient: column n of this launch is column n + n_base of the whole product
+    // (a launch on the trailing columns); n_total = columns of the whole product (0: this launch has them all)
+    int n_base, n_total;
 };
 
 struct GemmParams {
@@ -150,19 +151,23 @@ static inline double ring16_plan_cost_us(const Ring16Plan& pl, int64_t M, int64_
     return ring16_cost_us(pl.edge, ring16_tiles(pl.edge, M, N, pl.head), K) +
            ring16_cost_us(pl.tail_edge, ring16_tiles(pl.tail_edge, M, N, batch - pl.head), K) + 2.0;
 }
-// A batch of products whose columns are whole tiles plus a narrow rest (a convolution of 56 x 56 images: 3136 output
-// pixels = 12 tiles of 256 and 64 more) spends a whole tile on that rest in every item.  The column split gives the
-// whole tiles of every item to the chosen tile and the rest of every item to a tile chosen for it alone, as two
-// (planned) launches.  head_cols = columns of the first launch; 0: no split.  It has to be 5 % ahead of the batch plan.
+// A batch of products can leave the CUs badly filled in two ways that a split along the columns mends: columns that are
+// whole tiles plus a narrow rest (a convolution of 56 x 56 images: 3136 output pixels = 12 tiles of 256 and 64 more spend a
+// whole tile on that rest in every item), and tile counts that are whole rounds over the CUs plus a fraction (the weight
+// gradient of the same layer: 9 tiles of 256 x 256 per image, 576 = 2.25 rounds; columns 0 .. 2047 of every image are 512
+// tiles = two rounds, the last 256 columns go to 128 x 128 tiles).  The split gives the leading head_cols columns of every
+// item to one (planned) launch and the remaining columns to another, each on the tile chosen for it alone.
+// head_cols = columns of the first launch, a multiple of 128; 0: no split.  It has to be 5 % ahead of the batch plan.
 static inline int64_t ring16_column_split(int64_t M, int64_t N, int64_t K, int64_t batch) {
-    const int edge = ring16_tile_edge(M, N, K, batch);
-    if (edge == 64) return 0;
-    const int64_t head_cols = N / edge * edge, rest = N - head_cols;
-    if (head_cols == 0 || rest == 0) return 0;
-    const double whole = ring16_plan_cost_us(ring16_plan(M, N, K, batch), M, N, K, batch);
-    const double split = ring16_plan_cost_us(ring16_plan(M, head_cols, K, batch), M, head_cols, K, batch) +
-                         ring16_plan_cost_us(ring16_plan(M, rest, K, batch), M, rest, K, batch) + 2.0;
-    return split < 0.95 * whole ? head_cols : 0;
+    if (N < 256 || N / 128 > 2048) return 0;
+    double best = 0.95 * ring16_plan_cost_us(ring16_plan(M, N, K, batch), M, N, K, batch);
+    int64_t best_cols = 0;
+    for (int64_t c = 128; c < N; c += 128) {
+        const double us = ring16_plan_cost_us(ring16_plan(M, c, K, batch), M, c, K, batch) +
+                          ring16_plan_cost_us(ring16_plan(M, N - c, K, batch), M, N - c, K, batch) + 2.0;
+        if (us < best) { best = us; best_cols = c; }
+    }
+    return best_cols;
 }
 
 // A single large product whose tiles fill the 256 CUs a whole number of times plus a rest spends a full tile time on that
