@@ -224,8 +224,9 @@ int64_t ntg_conv2d_forward_workspace_bytes(int dtype, int64_t batch, int64_t cha
 /* Bytes of device workspace with which ntg_conv2d_dev runs its fastest form.  For Float32 whose channels per group are a
  * multiple of 16, Float16 / BFloat16 with at least 8 channels per group (padded with zeros to a multiple of 32 in the
  * copy), and groups of up to 32 bytes of channels in all three (RGB input layers: pixels of 16 or 32 bytes, several taps
- * per K-step), that is a channels-last copy of the image plus the weights with the channel index fastest; the convolution
- * (conv.cpp:86-118) then gathers its operand in 16-byte pieces.  Otherwise the figure of
+ * per K-step), that is a channels-last copy of the image (with the padding as a border of zero pixels where the channels
+ * of a group fill whole 64-byte runs) plus the weights with the channel index fastest; the convolution (conv.cpp:86-118)
+ * then gathers its operand in 16-byte pieces.  Otherwise the figure of
  * ntg_conv2d_forward_workspace_bytes.  ntg_conv2d_dev accepts any smaller workspace and falls back to its other forms. */
 int64_t ntg_conv2d_fast_workspace_bytes(int dtype, int64_t batch, int64_t channels, int64_t height, int64_t width,
                                         int64_t out_channels, int64_t k_r, int64_t k_c, int64_t s_r, int64_t s_c,
