@@ -85,7 +85,7 @@ def main():
     torch.manual_seed(1003)
     stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
 
-    def make_gemm(dtype, m, k, n, ta=False, tb=False, batch=1, scale=1.0, mode=_lib.C_ACCUMULATE, ints=False):
+    def make_gemm(dtype, m, k, n, ta=False, tb=False, batch=1, scale=1.0, mode=_lib.C_ACCUMULATE, ints=False, bias_relu=False):
         ashape = (batch, k, m) if ta else (batch, m, k)
         bshape = (batch, n, k) if tb else (batch, k, n)
         if ints:
@@ -106,10 +106,16 @@ def main():
         if ws is not None:
             d.workspace, d.workspace_bytes = ws.data_ptr(), ws_bytes
 
-        def launch():
-            _lib.check(lib.ntg_gemm_dev(ctypes.byref(d), a.data_ptr(), b.data_ptr(), c.data_ptr(), stream))
+        bias = None
+        if bias_relu:                       # Linear -> ReLU in one launch: bias row as starting value, clamp in the epilogue
+            bias = (torch.randn((n,), device=dev) * scale).to(dtype)
+            d.c_mode, d.bias, d.bias_col_stride = _lib.C_BIAS, bias.data_ptr(), 1
+        entry = lib.ntg_gemm_relu_dev if bias_relu else lib.ntg_gemm_dev
 
-        launch.keep = (a, b, c, d, ws)
+        def launch():
+            _lib.check(entry(ctypes.byref(d), a.data_ptr(), b.data_ptr(), c.data_ptr(), stream))
+
+        launch.keep = (a, b, c, d, ws, bias)
         return launch
 
     def time_steps(fn, steps, warmup):
@@ -256,6 +262,7 @@ def main():
         for dt, nm in ((torch.float32, "fp32"), (torch.bfloat16, "bf16")):
             pk = PEAK_TFLOPS[nm]
             run(f"c4_linear_fwd_{nm}", G(dt, 8192, 4096, 11008, tb=True, mode=_lib.C_OVERWRITE, scale=0.1), f4, pk)
+            run(f"c4_linear_fwd_bias_relu_{nm}", G(dt, 8192, 4096, 11008, tb=True, scale=0.1, bias_relu=True), f4, pk)
             run(f"c4_linear_dx_{nm}", G(dt, 8192, 11008, 4096, mode=_lib.C_OVERWRITE, scale=0.1), f4, pk)
             run(f"c4_linear_dw_{nm}", G(dt, 11008, 8192, 4096, ta=True, mode=_lib.C_OVERWRITE, scale=0.1), f4, pk)
         # the same Linear layer on 16 and 256 rows (inference-sized batches): HBM-bound streaming kernel, split along k

@@ -192,6 +192,17 @@ int ntg_matmult_dev(int dtype, const void* dA, const void* dB, void* dC,
  * (matmult_cpu.cpp:863-1005) lower to when the views are affine. */
 int ntg_gemm_dev(const ntg_gemm_desc* desc, const void* dA, const void* dB, void* dC, void* stream);
 
+/* ntg_gemm_dev followed by relu_ on the result, in one pass: C = max(result, 0), where result is what ntg_gemm_dev would
+ * have stored (so Linear -> ReLU, nt::functional::relu_(linear(x, w, b)), is one launch with c_mode = NTG_C_BIAS).  relu_ is
+ * clamp_(x, 0) (nt/functional/tensor_files/activation_functions.cpp:141-143), i.e. max(x, 0) with 0 returned for NaN and
+ * for -0 (nt/functional/cpu/min_max.cpp:45-63, :115-121); rounding is monotonic and keeps the sign, so clamping the sum
+ * before its one rounding gives the bits of clamping the stored value.  Float16, BFloat16, Float32, Float64.  The DMA-fed
+ * kernels and the split-K reduction clamp in their epilogue; where another kernel serves the product a second small
+ * kernel clamps C in place.  With k = 0 and NTG_C_ACCUMULATE the call is relu_ itself on the matrix at dC (dA, dB may be
+ * null).  The reference's other activations (sigmoid, silu, gelu: SVML exp / tanh / pow) are not offered
+ * as epilogues: their bits are those of its vector maths library, which this library cannot reproduce. */
+int ntg_gemm_relu_dev(const ntg_gemm_desc* desc, const void* dA, const void* dB, void* dC, void* stream);
+
 /* ntg_gemm_dev for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
  * harnesses that forbid hipMalloc): it has NO counterpart in the reference.  Same arguments, results bit-identical to
  * ntg_gemm_dev called with a workspace of ntg_gemm_workspace_bytes(desc) bytes; desc->workspace and desc->workspace_bytes

@@ -61,6 +61,7 @@ SIGNATURES = {
     "ntg_conv2d": (_ci, [_ci, _vp, _vp, _vp] + [_i64] * 14),
     "ntg_matmult_dev": (_ci, [_ci, _vp, _vp, _vp, _i64, _i64, _i64, _ci, _ci, _vp]),
     "ntg_gemm_dev": (_ci, [ctypes.POINTER(GemmDesc), _vp, _vp, _vp, _vp]),
+    "ntg_gemm_relu_dev": (_ci, [ctypes.POINTER(GemmDesc), _vp, _vp, _vp, _vp]),
     "ntg_gemm_noalloc_dev": (_ci, [ctypes.POINTER(GemmDesc), _vp, _vp, _vp, _vp]),
     "ntg_gemm_workspace_bytes": (_i64, [ctypes.POINTER(GemmDesc)]),
     "ntg_gemm_ptrs_dev": (_ci, [ctypes.POINTER(GemmDesc), _vp, _vp, _vp, _vp]),

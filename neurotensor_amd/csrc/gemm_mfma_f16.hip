@@ -7,6 +7,10 @@ hipError_t launch_gemm_mfma_f16(bool ta, bool tb, const GemmParams& p, hipStream
     if (big_tiles >= 256) return launch_trans<DT_F16, 4, 4, 64>(ta, tb, p, s);   // 256 x 256 x 64
     return launch_trans<DT_F16, 2, 2, 64>(ta, tb, p, s);                          // 128 x 128 x 64
 }
+hipError_t launch_gemm_ring_only_f16(bool ta, bool tb, const GemmParams& p, hipStream_t s, bool* taken) {
+    *taken = ring_eligible(p, ta);
+    return *taken ? launch_ring16<DT_F16>(ta, tb, p, s) : hipSuccess;
+}
 // convolution / conv_dkernel with op(B) gathered from the image (tb: col^T), nd = 2 or 3 spatial axes.  128 x 128 x 64 tiles,
 // two workgroups per CU: the gather's registers do not fit beside a 256 x 256 accumulator.
 hipError_t launch_conv_mfma_f16(bool tb, int nd, const GemmParams& p, hipStream_t s) {

@@ -22,6 +22,11 @@ hipError_t launch_gemm_mfma_f32(bool ta, bool tb, const GemmParams& p, hipStream
     if (big_tiles >= 192 && p.M > 64 && p.N > 64) return launch_trans<DT_F32, 2, 2, 32>(ta, tb, p, s);   // a 128-wide tile would be half empty
     return launch_trans<DT_F32, 1, 1, 32>(ta, tb, p, s);
 }
+hipError_t launch_gemm_ring_only_f32(bool ta, bool tb, const GemmParams& p, hipStream_t s, bool* taken) {
+    *taken = ring_eligible(p, ta, 4);
+    if (!*taken) return hipSuccess;
+    return ring_f32_tile_edge(p) == 64 ? launch_ring_wb<DT_F32, 1>(ta, tb, p, s) : launch_ring_wb<DT_F32, 2>(ta, tb, p, s);
+}
 // convolution / conv_dkernel with op(B) gathered from the image (tb: col^T), nd = 2 or 3 spatial axes
 template <int ND>
 static hipError_t launch_conv_nd_f32(bool tb, const GemmParams& p, hipStream_t s) {

@@ -723,9 +723,29 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
     const bool c_rows_16 = !GATHER16 || (p.ldc % G::VEL == 0 && p.sC % G::VEL == 0 && (reinterpret_cast<uintptr_t>(p.C) & 15) == 0);
     typedef AccS accx4 __attribute__((ext_vector_type(4)));
     typedef uint32_t u32x2v __attribute__((ext_vector_type(2)));
+    // (uniform) the bias is contiguous along the columns and every lane's 8 values start on a 16-byte boundary
+    const bool bias_rows_16 = ES != 1 && p.bias && p.bias_cs == 1 && p.bias_rs % G::VEL == 0 && p.bias_bs % G::VEL == 0 &&
+                              (reinterpret_cast<uintptr_t>(p.bias) & 15) == 0;
     auto epilogue = [&](auto cmode_tag) {
         constexpr int CM = decltype(cmode_tag)::value;
         const T* bias = static_cast<const T*>(p.bias);
+        // one bias row for every row of C (cpu::linear's [n] vector): the lane's 8 columns never change, one load for the whole tile
+        AccS bias_row[8] = {};
+        const bool bias_row_const = CM == C_BIAS && bias_rows_16 && p.bias_rs == 0 && (!RAGGED || n + 8 <= p.N);
+        if constexpr (CM == C_BIAS && ES != 1) {
+            if (bias_row_const) {
+                const T* bp = bias + (int64_t)b * p.bias_bs + (int64_t)n;
+                if constexpr (ES == 2) {
+                    const u32x4 bv = *reinterpret_cast<const u32x4*>(bp);
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) bias_row[e] = Cvt16<DT>::up((uint16_t)(bv[e >> 1] >> (16 * (e & 1))));
+                } else {
+                    const accx4 b0 = *reinterpret_cast<const accx4*>(bp), b1 = *reinterpret_cast<const accx4*>(bp + 4);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) { bias_row[e] = b0[e]; bias_row[4 + e] = b1[e]; }
+                }
+            }
+        }
 #pragma unroll
         for (int i = 0; i < WBM; ++i) {
             // C0 of the whole slab is requested before the LDS round trip
@@ -799,10 +819,32 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
                         else { const uint32_t cu = c0[t][e >> 2][e & 3]; v[e] += __builtin_bit_cast(float, cu); }
                     }
                 } else if constexpr (CM == C_BIAS) {
+                    const T* bp = bias + (int64_t)b * p.bias_bs + (int64_t)m * p.bias_rs + (int64_t)n * p.bias_cs;
+                    if (bias_row_const) {
 #pragma unroll
-                    for (int e = 0; e < 8; ++e)
-                        if (ES != 4 || e < 4 || hi_ok)
-                            v[e] += (AccS)bias[(int64_t)b * p.bias_bs + (int64_t)m * p.bias_rs + (int64_t)(n + e) * p.bias_cs];
+                        for (int e = 0; e < 8; ++e) v[e] += bias_row[e];
+                    } else if (bias_rows_16 && (ES != 4 || hi_ok)) {
+                        // a bias that runs along the columns (cpu::linear's [n] vector): the lane's 8 values in 16-byte loads
+                        if constexpr (ES == 2) {
+                            const u32x4 bv = *reinterpret_cast<const u32x4*>(bp);
+#pragma unroll
+                            for (int e = 0; e < 8; ++e) v[e] += Cvt16<DT>::up((uint16_t)(bv[e >> 1] >> (16 * (e & 1))));
+                        } else if constexpr (ES == 4) {
+                            const accx4 b0 = *reinterpret_cast<const accx4*>(bp), b1 = *reinterpret_cast<const accx4*>(bp + 4);
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) { v[e] += b0[e]; v[4 + e] += b1[e]; }
+                        }
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 8; ++e)
+                            if (ES != 4 || e < 4 || hi_ok) v[e] += (AccS)bp[(int64_t)e * p.bias_cs];
+                    }
+                }
+                if constexpr (ES != 1) {
+                    if (p.act == ACT_RELU) {                   // (uniform) relu_ on the result before its one rounding: the same bits
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) v[e] = v[e] > (AccS)0 ? v[e] : (AccS)0;
+                    }
                 }
                 char* cp = Cb + ((int64_t)m * p.ldc + n) * ES;
                 if constexpr (ES == 2) {

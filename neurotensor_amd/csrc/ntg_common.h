@@ -80,8 +80,11 @@ struct GemmParams {
     int vecA_ok, vecB_ok;    // 16-byte vector loads are legal for every row of A / B
     int ptrs_aligned;        // pointer tables only: the caller vouches that every entry is a multiple of 16 bytes (the tables
                              // live in device memory, the host cannot look); lets table batches onto the DMA-fed kernels
+    int act;                 // ACT_RELU: the stored result is max(result, 0) (relu_ of the reference = clamp_(x, 0): NaN and -0 become +0);
+                             // honoured by the DMA-fed Float16 / BFloat16 / Float32 kernels and the split-K reduction only
     ConvGeom conv;           // used by the implicit-im2col kernels only: B = image, op(B) = col or col^T
 };
+enum { ACT_NONE = 0, ACT_RELU = 1 };
 
 // Tile the DMA-fed 16-bit kernel uses for M x N x K x batch: square with edge 256, 128 or 64, or (plain products only)
 // 128 rows x 256 columns (code 192) or 192 rows x 256 columns (code 224).  Larger tiles need less LDS traffic per flop (a CU sustains
@@ -213,6 +216,11 @@ static inline int64_t elem_size(int dt) {
 
 // launchers implemented in the .hip files; all return a hipError_t
 hipError_t launch_gemm_mfma(int dtype, bool ta, bool tb, const GemmParams& p, hipStream_t s);
+// Float16 / BFloat16 / Float32 on the DMA-fed kernel or not at all (*taken = false, nothing launched): the kernel whose
+// epilogue applies GemmParams::act
+hipError_t launch_gemm_ring_only(int dtype, bool ta, bool tb, const GemmParams& p, hipStream_t s, bool* taken);
+// C[b][m][n] = max(C[b][m][n], 0) in place (floating dtypes)
+hipError_t launch_relu_inplace(int dtype, void* C, int64_t ldc, int64_t sC, int64_t M, int64_t N, int64_t batch, hipStream_t s);
 hipError_t launch_gemm_valu(int dtype, bool ta, bool tb, const GemmParams& p, hipStream_t s);
 hipError_t launch_gemm_mfma_i8(int dtype, bool ta, bool tb, const GemmParams& p, hipStream_t s);   // Int8 / UInt8: MFMA where rows are 16-byte multiples
 hipError_t launch_gemm_complex(int dtype, bool ta, bool tb, const GemmParams& p, hipStream_t s);   // Complex32 / 64 / 128: lane-wise products on (re, im) pairs

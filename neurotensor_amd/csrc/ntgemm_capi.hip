@@ -21,6 +21,18 @@ hipError_t launch_gemm_mfma_f64(bool ta, bool tb, const GemmParams& p, hipStream
 hipError_t launch_gemm_mfma_f16(bool ta, bool tb, const GemmParams& p, hipStream_t s);
 hipError_t launch_gemm_mfma_bf16(bool ta, bool tb, const GemmParams& p, hipStream_t s);
 hipError_t launch_gemm_skinny(int dtype, bool ta, bool tb, const GemmParams& p, hipStream_t s, bool* handled);
+hipError_t launch_gemm_ring_only_f32(bool ta, bool tb, const GemmParams& p, hipStream_t s, bool* taken);
+hipError_t launch_gemm_ring_only_f16(bool ta, bool tb, const GemmParams& p, hipStream_t s, bool* taken);
+hipError_t launch_gemm_ring_only_bf16(bool ta, bool tb, const GemmParams& p, hipStream_t s, bool* taken);
+hipError_t launch_gemm_ring_only(int dtype, bool ta, bool tb, const GemmParams& p, hipStream_t s, bool* taken) {
+    *taken = false;
+    switch (dtype) {
+    case DT_F32: return launch_gemm_ring_only_f32(ta, tb, p, s, taken);
+    case DT_F16: return launch_gemm_ring_only_f16(ta, tb, p, s, taken);
+    case DT_BF16: return launch_gemm_ring_only_bf16(ta, tb, p, s, taken);
+    default: return hipSuccess;
+    }
+}
 hipError_t launch_conv_mfma_f32(bool tb, int nd, const GemmParams& p, hipStream_t s);
 hipError_t launch_conv_mfma_f64(bool tb, int nd, const GemmParams& p, hipStream_t s);
 hipError_t launch_conv_mfma_f16(bool tb, int nd, const GemmParams& p, hipStream_t s);
@@ -121,6 +133,27 @@ int launch_gemm(ntg::GemmParams p, int dtype, bool ta, bool tb, hipStream_t s) {
     p.vecA_ok = (p.lda % ve == 0) && (p.Aptr || p.sA % ve == 0);
     p.vecB_ok = (p.ldb % ve == 0) && (p.Bptr || p.sB % ve == 0);
     hipError_t e;
+    // relu_ on the result: inside the DMA-fed kernel's epilogue where that kernel serves the product (more than 32 rows: the
+    // streaming kernels take the others), else as a pass over C after whichever kernel runs
+    const int act = p.act;
+    p.act = ntg::ACT_NONE;
+    if (act != ntg::ACT_NONE) {
+        if (p.Cptr || !(dtype == ntg::DT_F32 || dtype == ntg::DT_F64 || dtype == ntg::DT_F16 || dtype == ntg::DT_BF16))
+            return fail(NTG_ERR_INVALID_ARGUMENT, "the relu epilogue takes strided floating-point results");
+        if (p.M > 32 && p.cmode != ntg::C_PARTIAL) {
+            ntg::GemmParams q = p;
+            q.act = act;
+            bool taken = false;
+            e = ntg::launch_gemm_ring_only(dtype, ta, tb, q, s, &taken);
+            if (e != hipSuccess) return hip_fail(e, "gemm launch");
+            if (taken) return NTG_OK;
+        }
+    }
+    const auto finish = [&]() -> int {
+        if (act == ntg::ACT_NONE) return NTG_OK;
+        const hipError_t ea = ntg::launch_relu_inplace(dtype, p.C, p.ldc, p.sC, p.M, p.N, p.batch, s);
+        return ea == hipSuccess ? NTG_OK : hip_fail(ea, "relu launch");
+    };
     if (dtype == ntg::DT_I8 || dtype == ntg::DT_U8) {
         e = ntg::launch_gemm_mfma_i8(dtype, ta, tb, p, s);
     } else if (is_int_dtype(dtype)) {
@@ -131,7 +164,7 @@ int launch_gemm(ntg::GemmParams p, int dtype, bool ta, bool tb, hipStream_t s) {
         bool handled = false;
         e = ntg::launch_gemm_skinny(dtype, ta, tb, p, s, &handled);
         if (e != hipSuccess) return hip_fail(e, "skinny gemm launch");
-        if (handled) return NTG_OK;
+        if (handled) return finish();
         switch (dtype) {
         case ntg::DT_F32: e = ntg::launch_gemm_mfma_f32(ta, tb, p, s); break;
         case ntg::DT_F64: e = ntg::launch_gemm_mfma_f64(ta, tb, p, s); break;
@@ -141,7 +174,7 @@ int launch_gemm(ntg::GemmParams p, int dtype, bool ta, bool tb, hipStream_t s) {
         }
     }
     if (e != hipSuccess) return hip_fail(e, "gemm launch");
-    return NTG_OK;
+    return finish();
 }
 
 // Split-K.  A single product whose output tiles cannot occupy the 256 CUs but whose K is deep (a Linear layer on a few
@@ -364,7 +397,7 @@ int run_gemm(ntg::GemmParams p, int dtype, bool ta, bool tb, hipStream_t s, void
     if (p.M == 0 || p.N == 0 || p.batch == 0) return NTG_OK;
     if (p.K == 0) {
         // empty sum: C keeps what it holds, or becomes the bias / zero.  The product kernels assume at least one k.
-        if (p.cmode == ntg::C_ACCUMULATE) return NTG_OK;
+        if (p.cmode == ntg::C_ACCUMULATE && p.act == ntg::ACT_NONE) return NTG_OK;      // (with relu: C = relu_(C), below)
         if (p.Cptr) return fail(NTG_ERR_INVALID_ARGUMENT, "k = 0 with a C mode other than accumulate needs strided operands");
         hipError_t e = hipSuccess;
         if (is_int_dtype(dtype)) {
@@ -405,6 +438,7 @@ int run_gemm(ntg::GemmParams p, int dtype, bool ta, bool tb, hipStream_t s, void
         q.sC = (int64_t)p.M * p.N;
         q.cmode = (dtype == ntg::DT_F16 || dtype == ntg::DT_BF16) ? ntg::C_PARTIAL : ntg::C_OVERWRITE;
         q.bias = nullptr;
+        q.act = ntg::ACT_NONE;                     // (the reduction applies it, after the last k range)
         int rc = launch_gemm(q, dtype, ta, tb, s);
         if (rc) return rc;
         hipError_t e = ntg::launch_splitk_reduce(dtype, workspace, plan.splits, p, s);
@@ -492,6 +526,20 @@ int ntg_gemm_dev(const ntg_gemm_desc* d, const void* dA, const void* dB, void* d
     if (!dA || !dB || !dC) return fail(NTG_ERR_INVALID_ARGUMENT, "null matrix pointer");
     if (p.batch > 1 && p.sC == 0) return fail(NTG_ERR_INVALID_ARGUMENT, "stride_c must be non-zero for a batch (outputs may not alias)");
     p.A = dA; p.B = dB; p.C = dC;
+    return run_gemm(p, d->dtype, d->transpose_a != 0, d->transpose_b != 0, static_cast<hipStream_t>(stream), d->workspace, d->workspace_bytes);
+}
+
+int ntg_gemm_relu_dev(const ntg_gemm_desc* d, const void* dA, const void* dB, void* dC, void* stream) {
+    ntg::GemmParams p;
+    int rc = desc_to_params(d, p);
+    if (rc) return rc;
+    if (!(d->dtype == ntg::DT_F32 || d->dtype == ntg::DT_F64 || d->dtype == ntg::DT_F16 || d->dtype == ntg::DT_BF16))
+        return fail(NTG_ERR_UNSUPPORTED_DTYPE, "ntg_gemm_relu_dev takes Float16, BFloat16, Float32 and Float64 (dtype %d)", d->dtype);
+    if (p.M == 0 || p.N == 0 || p.batch == 0) return NTG_OK;
+    if (!dC || (p.K > 0 && (!dA || !dB))) return fail(NTG_ERR_INVALID_ARGUMENT, "null matrix pointer");      // (k = 0: C = relu_(C0), no operands)
+    if (p.batch > 1 && p.sC == 0) return fail(NTG_ERR_INVALID_ARGUMENT, "stride_c must be non-zero for a batch (outputs may not alias)");
+    p.A = dA; p.B = dB; p.C = dC;
+    p.act = ntg::ACT_RELU;
     return run_gemm(p, d->dtype, d->transpose_a != 0, d->transpose_b != 0, static_cast<hipStream_t>(stream), d->workspace, d->workspace_bytes);
 }
 

@@ -91,6 +91,7 @@ __global__ void __launch_bounds__(256) splitk_reduce_kernel(const P* __restrict_
         if (p.cmode == C_ACCUMULATE) acc = (Acc)*cp;
         else if (p.cmode == C_BIAS) acc = (Acc)bias[m * p.bias_rs + n * p.bias_cs];
         for (int s = 0; s < splits; ++s) acc += (Acc)part[(int64_t)s * total + idx];
+        if (p.act == ACT_RELU) acc = acc > (Acc)0 ? acc : (Acc)0;
         *cp = (T)acc;
     }
 }
@@ -135,7 +136,7 @@ __global__ void __launch_bounds__(256) splitk_reduce_vec_kernel(const P* __restr
         }
         TV o;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) o[e] = (T)acc[e];
+        for (int e = 0; e < 4; ++e) o[e] = (T)((p.act == ACT_RELU && !(acc[e] > (Acc)0)) ? (Acc)0 : acc[e]);
         *cp = o;
     }
 }
@@ -147,6 +148,45 @@ static void launch_splitk_reduce_t(const void* part, int splits, const GemmParam
                      (reinterpret_cast<uintptr_t>(part) % (4 * sizeof(P))) == 0;
     if (vec) hipLaunchKernelGGL((splitk_reduce_vec_kernel<T, P, Acc>), dim3(grid_for(total / 4)), dim3(256), 0, s, (const P*)part, splits, p);
     else hipLaunchKernelGGL((splitk_reduce_kernel<T, P, Acc>), dim3(grid_for(total)), dim3(256), 0, s, (const P*)part, splits, p);
+}
+
+// C[b][m][n] = C[b][m][n] > 0 ? C[b][m][n] : 0 -- relu_ = clamp_(x, 0) of the reference (activation_functions.cpp:143,
+// min_max.cpp:115-121: max(x, 0) with the second operand returned for NaN and for -0)
+template <class T>
+__global__ void __launch_bounds__(256) relu_inplace_kernel(T* __restrict__ C, const int64_t ldc, const int64_t sC, const int64_t M, const int64_t N,
+                                                           const int64_t batch) {
+    const int64_t total = batch * M * N;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+        const int64_t n = i % N, m = (i / N) % M, b = i / (N * M);
+        T* cp = C + b * sC + m * ldc + n;
+        const T v = *cp;
+        if (!((float)v > 0.0f) || v != v) *cp = (T)0.0f;
+    }
+}
+template <>
+__global__ void __launch_bounds__(256) relu_inplace_kernel<double>(double* __restrict__ C, const int64_t ldc, const int64_t sC, const int64_t M,
+                                                                   const int64_t N, const int64_t batch) {
+    const int64_t total = batch * M * N;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+        const int64_t n = i % N, m = (i / N) % M, b = i / (N * M);
+        double* cp = C + b * sC + m * ldc + n;
+        if (!(*cp > 0.0)) *cp = 0.0;
+    }
+}
+hipError_t launch_relu_inplace(int dtype, void* C, int64_t ldc, int64_t sC, int64_t M, int64_t N, int64_t batch, hipStream_t s) {
+    const int64_t total = batch * M * N;
+    if (total <= 0) return hipSuccess;
+    const dim3 g(grid_for(total)), t(256);
+    switch (dtype) {
+    case DT_F32: hipLaunchKernelGGL(relu_inplace_kernel<float>, g, t, 0, s, (float*)C, ldc, sC, M, N, batch); break;
+    case DT_F64: hipLaunchKernelGGL(relu_inplace_kernel<double>, g, t, 0, s, (double*)C, ldc, sC, M, N, batch); break;
+    case DT_F16: hipLaunchKernelGGL(relu_inplace_kernel<_Float16>, g, t, 0, s, (_Float16*)C, ldc, sC, M, N, batch); break;
+    case DT_BF16: hipLaunchKernelGGL(relu_inplace_kernel<__bf16>, g, t, 0, s, (__bf16*)C, ldc, sC, M, N, batch); break;
+    default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
 }
 
 hipError_t launch_splitk_reduce(int dtype, const void* part, int splits, const GemmParams& p, hipStream_t s) {

@@ -485,7 +485,7 @@ static DeviceType common_device(std::initializer_list<const Tensor*> ts, const c
 // in nbig / chunk consecutive chunks inside which every operand is either strided or one matrix.
 static void device_gemm(int dt, int64_t es, bool ta, bool tb, int mode, int64_t m, int64_t k, int64_t n, int64_t nbig,
                         const char* A, int64_t na, const char* B, int64_t nb, char* C,
-                        const char* bias = nullptr, int64_t nbias = 1, int64_t brow = 1, int64_t bcol = 1) {
+                        const char* bias = nullptr, int64_t nbias = 1, int64_t brow = 1, int64_t bcol = 1, bool relu = false) {
     int64_t chunk = nbig;
     for (int64_t cnt : {na, nb, nbias})
         if (cnt > 1 && cnt < chunk) chunk = cnt;
@@ -505,8 +505,9 @@ static void device_gemm(int dt, int64_t es, bool ta, bool tb, int mode, int64_t 
         }
         const int64_t wsb = ntg_gemm_workspace_bytes(&d);      // > 0: a faster form exists (split along k, byte planes)
         if (wsb > 0) { d.workspace = device_workspace(wsb); d.workspace_bytes = wsb; }
-        check_status(ntg_gemm_dev(&d, A + (na > 1 ? (i0 % na) * m * k * es : 0), B + (nb > 1 ? (i0 % nb) * k * n * es : 0),
-                                  C + i0 * m * n * es, nullptr));
+        const char* a_i = A + (na > 1 ? (i0 % na) * m * k * es : 0);
+        const char* b_i = B + (nb > 1 ? (i0 % nb) * k * n * es : 0);
+        check_status(relu ? ntg_gemm_relu_dev(&d, a_i, b_i, C + i0 * m * n * es, nullptr) : ntg_gemm_dev(&d, a_i, b_i, C + i0 * m * n * es, nullptr));
     }
 }
 
@@ -643,7 +644,7 @@ Tensor matmult(const TensorList& a, const TensorList& b, bool trans_a, bool tran
     return c;
 }
 
-Tensor linear(const Tensor& x_in, const Tensor& w_in, const Tensor& b_in, bool trans_a, bool trans_b) {
+static Tensor linear_impl(const Tensor& x_in, const Tensor& w_in, const Tensor& b_in, bool trans_a, bool trans_b, bool with_relu) {
     utils::throw_exception(!x_in.is_null() && !w_in.is_null() && !b_in.is_null(), "Cannot perform operation linear on a null tensor");
     utils::throw_exception(x_in.dtype() == w_in.dtype() && x_in.dtype() == b_in.dtype(), "linear expects input, weight and bias of one dtype");
     const int64_t nd = std::max({x_in.dims(), w_in.dims(), b_in.dims()});
@@ -686,7 +687,7 @@ Tensor linear(const Tensor& x_in, const Tensor& w_in, const Tensor& b_in, bool t
     if (dev == DeviceType::HIP) {
         device_gemm(dt, es, p.ta, p.tb, NTG_C_BIAS, p.m, p.k, p.n, p.nbig, static_cast<const char*>(p.a.data_ptr()), p.na,
                     static_cast<const char*>(p.b.data_ptr()), p.nb, static_cast<char*>(c.data_ptr()),
-                    static_cast<const char*>(b.data_ptr()), nbias, brow, bcol);
+                    static_cast<const char*>(b.data_ptr()), nbias, brow, bcol, with_relu);
         return c;
     }
     // bias broadcast to the output is the initial accumulator (:1637-1647); fused on the device
@@ -696,7 +697,60 @@ Tensor linear(const Tensor& x_in, const Tensor& w_in, const Tensor& b_in, bool t
                                 static_cast<const char*>(b.data_ptr()) + (i % nbias) * brow * bcol * es,
                                 static_cast<char*>(c.data_ptr()) + i * p.m * p.n * es, p.m, p.k, p.n, p.ta, p.tb, brow, bcol));
     }
+    if (with_relu) relu_(c);
     return c;
+}
+
+Tensor linear(const Tensor& x, const Tensor& w, const Tensor& b, bool trans_a, bool trans_b) { return linear_impl(x, w, b, trans_a, trans_b, false); }
+Tensor linear_relu(const Tensor& x, const Tensor& w, const Tensor& b, bool trans_a, bool trans_b) { return linear_impl(x, w, b, trans_a, trans_b, true); }
+
+template <class T>
+static void relu_host(void* data, int64_t n) {
+    T* p = static_cast<T*>(data);
+    for (int64_t i = 0; i < n; ++i) p[i] = p[i] > T(0) ? p[i] : T(0);
+}
+static void relu_host_16(void* data, int64_t n, bool bf) {
+    // sign and NaN are visible in the bit pattern: negative (sign bit set, -0 included) or NaN -> +0
+    uint16_t* p = static_cast<uint16_t*>(data);
+    const uint16_t exp_mask = bf ? 0x7f80 : 0x7c00, man_mask = bf ? 0x007f : 0x03ff;
+    for (int64_t i = 0; i < n; ++i) {
+        const uint16_t v = p[i];
+        const bool nan = (v & exp_mask) == exp_mask && (v & man_mask) != 0;
+        if ((v & 0x8000) || nan) p[i] = 0;
+    }
+}
+
+Tensor& relu_(Tensor& x) {
+    utils::throw_exception(!x.is_null(), "Cannot perform operation relu_ on a null tensor");
+    const DType dt = x.dtype();
+    utils::throw_exception(dt == DType::Float16 || dt == DType::BFloat16 || dt == DType::Float32 || dt == DType::Float64,
+                           "relu_ expects a floating dtype");
+    utils::throw_exception(x.is_contiguous(), "relu_ expects a contiguous tensor");
+    const int64_t n = x.numel();
+    if (n == 0) return x;
+    if (x.is_device()) {
+        // relu_ on device memory = the product entry point with an empty k: C = max(C, 0)
+        const SizeRef& sh = x.shape();
+        const int64_t cols = sh.empty() ? 1 : sh.back();
+        ntg_gemm_desc d;
+        std::memset(&d, 0, sizeof d);
+        d.dtype = static_cast<int>(dt); d.c_mode = NTG_C_ACCUMULATE;
+        d.m = n / cols; d.k = 0; d.n = cols; d.batches = 1;
+        check_status(ntg_gemm_relu_dev(&d, nullptr, nullptr, x.data_ptr(), nullptr));
+        return x;
+    }
+    switch (dt) {
+    case DType::Float32: relu_host<float>(x.data_ptr(), n); break;
+    case DType::Float64: relu_host<double>(x.data_ptr(), n); break;
+    case DType::Float16: relu_host_16(x.data_ptr(), n, false); break;
+    default: relu_host_16(x.data_ptr(), n, true); break;
+    }
+    return x;
+}
+
+Tensor relu(const Tensor& x) {
+    Tensor out = x.contiguous().clone();
+    return relu_(out);
 }
 
 MatmultGrads matmult_backward(const Tensor& a, const Tensor& b, const Tensor& grad, bool trans_a, bool trans_b) {

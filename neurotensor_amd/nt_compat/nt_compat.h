@@ -115,6 +115,12 @@ Tensor matmult_cT(const Tensor& a, const Tensor& b);
 // higher-rank item's shape with its first dimension multiplied by the list length and the last two replaced by [m, n].
 Tensor matmult(const TensorList& a, const TensorList& b, bool trans_a = false, bool trans_b = false);
 Tensor linear(const Tensor& input, const Tensor& weight, const Tensor& bias, bool trans_input = false, bool trans_weight = false);
+// relu = clamp(x, 0), relu_ in place (activation_functions.cpp:141-143; min_max.cpp:115-121: max(x, 0), 0 for NaN and -0);
+// floating dtypes.  linear_relu(x, w, b) == relu_(linear(x, w, b)) bit for bit; on device tensors it is one launch (the
+// clamp runs in the product's epilogue) -- the reference has no fused form, its layers call the two in a row.
+Tensor relu(const Tensor& x);
+Tensor& relu_(Tensor& x);
+Tensor linear_relu(const Tensor& input, const Tensor& weight, const Tensor& bias, bool trans_input = false, bool trans_weight = false);
 Tensor unfold2d(const Tensor& x, utils::my_tuple kernel_size, utils::my_tuple dilation = {1, 1}, utils::my_tuple padding = {0, 0},
                 utils::my_tuple stride = {1, 1}, bool transpose_out = true);
 Tensor conv2d(const Tensor& image, const Tensor& kernel, utils::my_tuple stride = {1, 1}, utils::my_tuple padding = {0, 0},

@@ -94,6 +94,7 @@ static void linear_shape_case(const char* name, SizeRef as, SizeRef bs, SizeRef 
 
 static void host_only_cases() {
     expect_throw("matmult inner sizes differ", [] { nt::matmult(F::zeros({4, 5}), F::zeros({4, 5})); });
+    expect_throw("relu of an integer tensor", [] { Tensor i32 = F::randn({4, 4}, DType::int32, 207); F::relu(i32); });
     expect_throw("matmult inner sizes differ with flags", [] { nt::matmult(F::zeros({4, 5}), F::zeros({4, 6}), true, true); });
     expect_throw("matmult 1-D operand", [] { nt::matmult(F::zeros({5}), F::zeros({5, 5})); });
     expect_throw("matmult dtype mismatch", [] { nt::matmult(F::zeros({4, 4}), F::zeros({4, 4}, DType::Float64)); });
@@ -462,6 +463,36 @@ static void device_resident_cases(const std::string& g) {
         // dW of a batched input and db are sums over the leading dims: one GEMM with a row of ones on the device
         nt::utils::throw_exception(F::allclose(dg1.dw, g1.dw, 1e-4, 1e-3) && F::allclose(dg1.db, g1.db, 1e-4, 1e-3) &&
                                        F::allclose(dg2.db, g2.db, 1e-4, 1e-3), "reduced gradients");
+    });
+    run_test("Linear -> ReLU -> Linear: relu_(linear) in one launch == the two in a row, bit for bit, four dtypes", [&] {
+        for (DType dt : {DType::Float32, DType::Float64, DType::Float16, DType::BFloat16}) {
+            Tensor x = F::randn({3, 40, 64}, dt, 201), w = F::randn({64, 72}, dt, 202), b = F::randn({72}, dt, 203);
+            Tensor w2 = F::randn({72, 24}, dt, 204), b2 = F::randn({24}, dt, 205);
+            // host: the reference's order of calls
+            Tensor h = nt::linear(x, w, b);
+            Tensor hr = F::relu(h);
+            Tensor y = nt::linear(hr, w2, b2);
+            nt::utils::throw_exception(!F::allclose(h, hr, 0, 0), "relu changed nothing");
+            nt::utils::throw_exception(F::allclose(F::linear_relu(x, w, b), hr, 0, 0), "host linear_relu");
+            // device: fused epilogue, relu_ in place on device memory, and the chain
+            Tensor dx = x.to(DeviceType::HIP), dw = w.to(DeviceType::HIP), db = b.to(DeviceType::HIP);
+            Tensor dfused = F::linear_relu(dx, dw, db);
+            nt::utils::throw_exception(dfused.is_device(), "result left the device");
+            same_bits(dfused, hr, "device linear_relu == relu(linear) on the host");
+            Tensor dh = nt::linear(dx, dw, db);
+            same_bits(F::relu_(dh), hr, "device relu_ in place");
+            same_bits(nt::linear(dfused, w2.to(DeviceType::HIP), b2.to(DeviceType::HIP)), y, "second layer on the clamped activations");
+        }
+        // NaN and -0 become +0 (max(x, 0) returns its second operand for both)
+        Tensor t = F::randn({2, 8}, DType::Float32, 206);
+        float* p = static_cast<float*>(t.data_ptr());
+        p[0] = std::nanf(""); p[1] = -0.0f; p[2] = -3.5f; p[3] = 2.25f;
+        Tensor r = F::relu(t), dr = F::relu(t.to(DeviceType::HIP));
+        const float* q = static_cast<const float*>(r.data_ptr());
+        uint32_t b0, b1;
+        std::memcpy(&b0, q, 4); std::memcpy(&b1, q + 1, 4);
+        nt::utils::throw_exception(b0 == 0 && b1 == 0 && q[2] == 0.0f && q[3] == 2.25f, "relu of NaN / -0 / negative / positive");
+        same_bits(dr, r, "device relu of NaN and -0");
     });
     run_test("two Linear layers on 2048 rows: host tensors against device tensors (timing printed)", [] {
         nt::layers::Linear l1(1024, 1024, true, DType::Float32, 97), l2(1024, 1024, true, DType::Float32, 98);
