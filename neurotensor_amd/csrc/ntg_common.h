@@ -225,6 +225,10 @@ hipError_t launch_gemm_valu(int dtype, bool ta, bool tb, const GemmParams& p, hi
 hipError_t launch_gemm_mfma_i8(int dtype, bool ta, bool tb, const GemmParams& p, hipStream_t s);   // Int8 / UInt8: MFMA where rows are 16-byte multiples
 hipError_t launch_gemm_complex(int dtype, bool ta, bool tb, const GemmParams& p, hipStream_t s);   // Complex32 / 64 / 128: lane-wise products on (re, im) pairs
 hipError_t launch_gemm_skinny(int dtype, bool ta, bool tb, const GemmParams& p, hipStream_t s, bool* handled);
+// Float32 products with so few output elements that 64 x 64 tiles leave most CUs idle: 32 x 32 tiles, k split over the
+// four wavefronts of a workgroup (gemm_small.hip)
+bool small32_f32_wins(const GemmParams& p);
+hipError_t launch_gemm_small32_f32(bool ta, bool tb, const GemmParams& p, hipStream_t s);
 // op(B) is the im2col matrix of the image at p.B (tb: its transpose); floating dtypes only
 hipError_t launch_conv_mfma(int dtype, bool tb, const GemmParams& p, hipStream_t s);
 hipError_t launch_unfold2d(int64_t elem_size, const void* im, void* col,

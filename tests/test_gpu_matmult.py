@@ -847,3 +847,55 @@ def test_single_large_products_split_into_two_launches(kind):
             assert bool((err <= 1.5 * ulp + 1e-4).all()), (m, k, n, ta, tb, mode, float((err / ulp).max()))
             assert float((c == want).double().mean()) > 0.97, (m, k, n, ta, tb, mode)
         del ref
+
+
+def test_small_fp32_products_on_32_wide_tiles():
+    """Float32 products with too few output elements for 64 x 64 tiles run on 32 x 32 tiles whose four or eight wavefronts split
+    k (config 1 is one of them): every transpose pair and C mode, ragged edges in m, n and k, padded rows, batches,
+    against float64 products within the stated bound; two runs are bit-identical (fixed order of the partial sums)."""
+    lib = _lib.load()
+    st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    gen = torch.Generator(device=DEV).manual_seed(4242)
+    modes = (_lib.C_OVERWRITE, _lib.C_ACCUMULATE, _lib.C_BIAS)
+    i = 0
+    for (m, k, n, batch) in [(512, 512, 512, 1), (100, 300, 70, 1), (33, 64, 33, 1), (40, 1003, 50, 2), (256, 130, 250, 3), (65, 77, 129, 4)]:
+        for ta, tb in TRANS:
+            mode = modes[i % 3]
+            i += 1
+            lda, ldb, ldc = (m if ta else k) + 3, (k if tb else n) + 5, n + 2
+            a = torch.randn(batch, k if ta else m, lda, device=DEV, generator=gen)
+            b = torch.randn(batch, n if tb else k, ldb, device=DEV, generator=gen)
+            c0 = torch.randn(batch, m, ldc, device=DEV, generator=gen)
+            bias = torch.randn(n, device=DEV, generator=gen)
+            la = a[:, :, :m].transpose(1, 2) if ta else a[:, :, :k]
+            lb = b[:, :, :k].transpose(1, 2) if tb else b[:, :, :n]
+            d = _lib.GemmDesc()
+            d.dtype, d.transpose_a, d.transpose_b, d.c_mode = _lib.FLOAT32, int(ta), int(tb), mode
+            d.m, d.k, d.n, d.batches = m, k, n, batch
+            d.lda, d.ldb, d.ldc = lda, ldb, ldc
+            d.stride_a, d.stride_b, d.stride_c = a.shape[1] * lda, b.shape[1] * ldb, m * ldc
+            if mode == _lib.C_BIAS:
+                d.bias, d.bias_col_stride = bias.data_ptr(), 1
+            assert lib.ntg_gemm_workspace_bytes(ctypes.byref(d)) == 0
+            outs = []
+            for rep in range(2):
+                c = c0.clone()
+                _lib.check(lib.ntg_gemm_dev(ctypes.byref(d), a.data_ptr(), b.data_ptr(), c.data_ptr(), st))
+                torch.cuda.synchronize()
+                outs.append(c)
+            assert torch.equal(outs[0], outs[1])
+            ref = la.double() @ lb.double()
+            if mode == _lib.C_ACCUMULATE:
+                ref += c0[:, :, :n].double()
+            elif mode == _lib.C_BIAS:
+                ref += bias.double()
+            tol = 1e-5 * k * float(la.abs().max() * lb.abs().max())
+            assert (outs[0][:, :, :n].double() - ref).abs().max().item() <= tol, (m, k, n, batch, ta, tb, mode)
+            assert torch.equal(outs[0][:, :, n:], c0[:, :, n:])                 # padding of C untouched
+            # relu_ in the same launch == clamp of the plain result
+            c = c0.clone()
+            _lib.check(lib.ntg_gemm_relu_dev(ctypes.byref(d), a.data_ptr(), b.data_ptr(), c.data_ptr(), st))
+            torch.cuda.synchronize()
+            want = outs[0].clone()
+            want[:, :, :n] = torch.where(outs[0][:, :, :n] > 0, outs[0][:, :, :n], torch.zeros_like(outs[0][:, :, :n]))
+            assert torch.equal(c, want)
