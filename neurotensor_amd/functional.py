@@ -62,7 +62,7 @@ def _logical(a_shape, b_shape, ta, tb):
 
 
 def _launch(a, b, c, m, k, n, ta, tb, batches, sa, sb, sc, c_mode, bias=None, bias_strides=(0, 0, 0),
-            a_off=0, b_off=0, c_off=0, bias_off=0):
+            a_off=0, b_off=0, c_off=0, bias_off=0, relu=False):
     es = a.element_size()
     d = GemmDesc()
     d.dtype = ntg_dtype(a)
@@ -79,8 +79,8 @@ def _launch(a, b, c, m, k, n, ta, tb, batches, sa, sb, sc, c_mode, bias=None, bi
     if ws_bytes > 0:
         ws = torch.empty((ws_bytes,), dtype=torch.uint8, device=a.device)
         d.workspace, d.workspace_bytes = ws.data_ptr(), ws_bytes
-    check(L.ntg_gemm_dev(ctypes.byref(d), a.data_ptr() + a_off * es, b.data_ptr() + b_off * es,
-                         c.data_ptr() + c_off * es, _stream()))
+    entry = L.ntg_gemm_relu_dev if relu else L.ntg_gemm_dev
+    check(entry(ctypes.byref(d), a.data_ptr() + a_off * es, b.data_ptr() + b_off * es, c.data_ptr() + c_off * es, _stream()))
 
 
 def matmult(a, b, out=None, transpose_a=False, transpose_b=False, accumulate=None):
@@ -154,7 +154,24 @@ def matmult_cT(a, b):
     return matmult(a, b, None, False, True)
 
 
-def linear(x, w, bias, transpose_a=False, transpose_b=False):
+def linear_relu(x, w, bias, transpose_a=False, transpose_b=False):
+    """relu_(linear(x, w, bias)) in one launch (activation_functions.cpp:141-143: relu = clamp(x, 0)); the clamp runs in
+    the product's epilogue and gives the bits of the two calls in a row."""
+    return linear(x, w, bias, transpose_a, transpose_b, _relu=True)
+
+
+def relu_(x):
+    """relu_ on a contiguous floating tensor in HBM: the product entry point with an empty k (C = max(C, 0))."""
+    _require_device(x)
+    if not x.is_contiguous():
+        raise ValueError("relu_ expects a contiguous tensor")
+    if x.numel():
+        cols = x.shape[-1] if x.dim() else 1
+        _launch(x, x, x, x.numel() // cols, 0, cols, False, False, 1, 0, 0, 0, _lib.C_ACCUMULATE, relu=True)
+    return x
+
+
+def linear(x, w, bias, transpose_a=False, transpose_b=False, _relu=False):
     """functional::linear -> cpu::linear (matmult_cpu.cpp:1624-1714): the bias, broadcast to the
     output shape, is the initial accumulator of the GEMM.  Done here in one pass (C_BIAS)."""
     _require_device(x, w, bias)
@@ -209,13 +226,13 @@ def linear(x, w, bias, transpose_a=False, transpose_b=False):
     if all(v in (1, nbig) for v in (nx, nw, nb)):
         _launch(x_st, w_st, out, m, k, n, ta, tb, nbig,
                 m * k if nx == nbig else 0, k * n if nw == nbig else 0, m * n, _lib.C_BIAS,
-                bias=bias_c, bias_strides=(bmat if nb == nbig else 0, brs, bcs))
+                bias=bias_c, bias_strides=(bmat if nb == nbig else 0, brs, bcs), relu=_relu)
     else:
         # mixed ranks: item i uses item i mod count of each lower-rank operand
         for i in range(nbig):
             _launch(x_st, w_st, out, m, k, n, ta, tb, 1, 0, 0, 0, _lib.C_BIAS,
                     bias=bias_c, bias_strides=(0, brs, bcs),
-                    a_off=(i % nx) * m * k, b_off=(i % nw) * k * n, c_off=i * m * n, bias_off=(i % nb) * bmat)
+                    a_off=(i % nx) * m * k, b_off=(i % nw) * k * n, c_off=i * m * n, bias_off=(i % nb) * bmat, relu=_relu)
     return out
 
 

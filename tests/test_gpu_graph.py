@@ -19,14 +19,16 @@ def setup_module(module):
 
 def _chain(x16, w16, b16, x32, w32, img, ker, xs):
     """A small model step touching every kernel family: DMA-fed 16-bit GEMM with bias, fp32 MFMA GEMM, the streaming
-    (m <= 32) kernel, split-K, implicit-GEMM convolution and its gradients."""
+    (m <= 32) kernel, split-K, implicit-GEMM convolution and its gradients, the clamp epilogue and relu_ in place."""
     y16 = F.linear(x16, w16, b16)                                   # [512, 1024] x [1024, 2048] + bias, bf16
-    y32 = F.matmult(x32, w32, None, False, True)                    # fp32, transpose_b
+    y32 = F.matmult(x32, w32, None, False, True)                    # fp32, transpose_b: 32-wide tiles, k split over the wavefronts
+    yr = F.linear_relu(x16, w16, b16)                               # Linear -> ReLU in one launch
+    y32r = F.relu_(F.matmult(x32, w32, None, False, True))          # relu_ on device memory
     ysk = F.matmult(xs, w16)                                        # 8 rows: streaming kernel
     ysp = F.matmult(y16[:256].contiguous(), w16, None, False, True)  # [256, 2048] x [2048, 1024]: split along k
     conv = F.conv2d(img, ker, padding=1)
     dimg, dker = F.conv2d_backward(img, ker, conv, padding=1)
-    return y16, y32, ysk, ysp, conv, dimg, dker
+    return y16, y32, ysk, ysp, conv, dimg, dker, yr, y32r
 
 
 def test_capture_and_replay():
