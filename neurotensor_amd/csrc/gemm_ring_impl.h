@@ -396,7 +396,22 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
             asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
                          :: "s"(lds_tile + (uint32_t)(wave_u * WB + x) * 1024u), "v"(src) : "memory");
             }
-            if (x == WB - 1) {
+            if (HALO && g.tap_inner && x == WB - 1) {
+                // one K-step on, taps inside a run of 64 bytes of channels: the next tap of this run, else the next run.  The
+                // taps of one run reach the same few pixels of the copy again and again while they are still in the XCD's L2;
+                // with the taps outermost every tap streamed the whole panel of the image through it again.
+                int q = k3_q + 1, r = k3_r, c0 = k3_c0, up = k3_up + g.d_c * g.chan * ES;
+                const bool w0 = q >= g.k_c;
+                q = w0 ? 0 : q;
+                r = w0 ? r + 1 : r;
+                up = w0 ? up - g.k_c * g.d_c * g.chan * ES + g.d_r * g.W * g.chan * ES : up;
+                const bool w1 = r >= g.k_r;
+                r = w1 ? 0 : r;
+                c0 = w1 ? c0 + BK : c0;
+                up = w1 ? up - g.k_r * g.d_r * g.W * g.chan * ES + BK * ES : up;
+                k3_c0 = c0; k3_up = up; k3_q = q; k3_r = r; k3_k += BK;
+            }
+            if (!(HALO && g.tap_inner) && x == WB - 1) {
                 // one K-step on: the next 64 bytes of channels of this tap, else the next tap (or the next tap_step taps)
                 const bool merged = g.tap_step > 1;
                 const int qstep = merged ? g.tap_step : 1, qend = merged ? g.kq_pad : g.k_c;

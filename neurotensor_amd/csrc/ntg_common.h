@@ -56,6 +56,9 @@ struct ConvGeom {
     // channels-last convolution: the copy of the image carries the padding as pixels of zeros (H, W, chan describe the padded
     // image, p_r = p_c = 0), so the gather needs no validity test
     int halo;
+    // ... and k runs (64-byte run of channels, tap, channel inside the run) instead of (tap, channel): the taps of a run reach
+    // the same pixels while they are in L2 (unit strides; the weights are permuted to match)
+    int tap_inner;
     // channels-last convolution and weight gradient: column n of this launch is column n + n_base of the whole product
     // (a launch on the trailing columns); n_total = columns of the whole product (0: this launch has them all)
     int n_base, n_total;
@@ -263,12 +266,12 @@ hipError_t launch_reduce_batch(int dtype, const void* part, void* out, int64_t b
 struct HaloMap { int64_t W, H, Wp, Hp, top, left; };
 hipError_t launch_nchw_to_nhwc(int64_t elem_size, const void* in, void* out, int64_t batch, int64_t C, int64_t P, hipStream_t s, const HaloMap* halo = nullptr);
 hipError_t launch_halo_zero(int64_t elem_size, void* out, int64_t batch, int64_t C, const HaloMap& halo, hipStream_t s);   // zeros the border pixels
-hipError_t launch_weights_channels_last(int64_t es, const void* w, void* wp, int64_t rows, int64_t cg, int64_t cgp, int64_t taps, hipStream_t s);
+hipError_t launch_weights_channels_last(int64_t es, const void* w, void* wp, int64_t rows, int64_t cg, int64_t cgp, int64_t taps, hipStream_t s, int64_t chunk = 0);
 hipError_t launch_weights_channels_last_rows(int64_t es, const void* w, void* wp, int64_t rows, int64_t cg, int64_t cgp, int64_t k_r, int64_t k_c,
                                              int64_t kq_pad, hipStream_t s);   // tap rows padded from k_c to kq_pad taps
 hipError_t launch_nchw_to_nhwc_padded(int64_t es, const void* in, void* out, int64_t batch, int64_t groups, int64_t cg, int64_t cgp, int64_t P, hipStream_t s,
                                       const HaloMap* halo = nullptr);
-hipError_t launch_flip_weights_channels_last(int64_t es, const void* w, void* wt, int64_t groups, int64_t og, int64_t ogp, int64_t cg, int64_t taps, hipStream_t s);
+hipError_t launch_flip_weights_channels_last(int64_t es, const void* w, void* wt, int64_t groups, int64_t og, int64_t ogp, int64_t cg, int64_t taps, hipStream_t s, int64_t chunk = 0);
 // channels-last convolution (image [B][pixel][C], weights [O][(r, q, c)]); F16 / BF16 / F32, two spatial axes
 hipError_t launch_conv_nhwc(int dtype, const GemmParams& p, hipStream_t s);
 // Image gradient of a strided convolution as one stride-1 convolution per phase of the image (see conv_dimage_phases):

@@ -969,6 +969,7 @@ static int conv_forward_nhwc(int dtype, const void* image, const void* kernel, v
     HaloPlan halo = conv_halo(g);
     if (mt) { halo.on = false; halo.vol = vol; halo.gp = g; }                    // (the merged-tap form keeps its validity bits)
     const int64_t volp = halo.vol;                                               // pixels per image of the copy
+    const bool tap_inner = halo.on && g.s[1] == 1 && g.s[2] == 1;                // (neighbouring taps share pixels only at unit strides)
     char* ws_img = static_cast<char*>(ws);
     char* ws_w = ws_img + align_up((size_t)(batch * chp * volp * es), 256);
     const ntg::HaloMap* hm = halo.on ? &halo.hm : nullptr;
@@ -980,7 +981,7 @@ static int conv_forward_nhwc(int dtype, const void* image, const void* kernel, v
         if (e != hipSuccess) return hip_fail(e, "border fill launch");
     }
     e = mt ? ntg::launch_weights_channels_last_rows(es, kernel, ws_w, out_channels, cg, cgp, g.k[1], g.k[2], mt->kq_pad, hs)
-           : ntg::launch_weights_channels_last(es, kernel, ws_w, out_channels, cg, cgp, taps, hs);
+           : ntg::launch_weights_channels_last(es, kernel, ws_w, out_channels, cg, cgp, taps, hs, tap_inner ? 64 / es : 0);      // (taps inside a 64-byte run of channels)
     if (e != hipSuccess) return hip_fail(e, "weight permutation launch");
     for (int64_t gi = 0; gi < groups; ++gi) {
         ntg::GemmParams p;
@@ -996,6 +997,7 @@ static int conv_forward_nhwc(int dtype, const void* image, const void* kernel, v
         fill_conv_geom(p.conv, cgp, halo.gp);
         p.conv.chan = (int)chp;                    // elements from one pixel to the next
         p.conv.halo = halo.on ? 1 : 0;
+        p.conv.tap_inner = tap_inner ? 1 : 0;
         if (mt) { p.conv.tap_step = (int)mt->T; p.conv.kq_pad = (int)mt->kq_pad; }
         e = ntg::launch_conv_nhwc(dtype, p, hs);
         if (e != hipSuccess) return hip_fail(e, "channels-last convolution launch");
@@ -1074,6 +1076,7 @@ static int conv_dimage_nhwc(int dtype, const void* kernel, const void* grad_out,
     const Geo3 t = geo_dimage(g);
     const HaloPlan halo = conv_halo(t);                                         // (the "image" of this convolution is dY)
     const int64_t Lp = halo.vol;
+    const bool tap_inner = halo.on && t.s[1] == 1 && t.s[2] == 1;
     char* ws_gy = static_cast<char*>(ws);
     char* ws_w = ws_gy + align_up((size_t)(batch * ochp * Lp * es), 256);
     const ntg::HaloMap* hm = halo.on ? &halo.hm : nullptr;
@@ -1084,7 +1087,7 @@ static int conv_dimage_nhwc(int dtype, const void* kernel, const void* grad_out,
         e = ntg::launch_halo_zero(es, ws_gy, batch, ochp, halo.hm, hs);
         if (e != hipSuccess) return hip_fail(e, "border fill launch");
     }
-    e = ntg::launch_flip_weights_channels_last(es, kernel, ws_w, groups, og, ogp, cg, taps, hs);
+    e = ntg::launch_flip_weights_channels_last(es, kernel, ws_w, groups, og, ogp, cg, taps, hs, tap_inner ? 64 / es : 0);
     if (e != hipSuccess) return hip_fail(e, "weight flip launch");
     for (int64_t gi = 0; gi < groups; ++gi) {
         ntg::GemmParams p;
@@ -1100,6 +1103,7 @@ static int conv_dimage_nhwc(int dtype, const void* kernel, const void* grad_out,
         fill_conv_geom(p.conv, ogp, halo.gp);
         p.conv.chan = (int)ochp;
         p.conv.halo = halo.on ? 1 : 0;
+        p.conv.tap_inner = tap_inner ? 1 : 0;
         e = ntg::launch_conv_nhwc(dtype, p, hs);
         if (e != hipSuccess) return hip_fail(e, "channels-last conv_dimage launch");
     }

@@ -401,7 +401,8 @@ hipError_t launch_nchw_to_nhwc(int64_t es, const void* in, void* out, int64_t ba
 // padded with zeros from og to ogp per tap.
 template <class T>
 __global__ void __launch_bounds__(256) flip_weights_channels_last_kernel(const T* __restrict__ w, T* __restrict__ wt, const int64_t groups,
-                                                                         const int64_t og, const int64_t ogp, const int64_t cg, const int64_t taps) {
+                                                                         const int64_t og, const int64_t ogp, const int64_t cg, const int64_t taps,
+                                                                         const int64_t chunk) {
     const int64_t total = groups * ogp * cg * taps;
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
     for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += stride) {
@@ -411,17 +412,20 @@ __global__ void __launch_bounds__(256) flip_weights_channels_last_kernel(const T
         r /= taps;
         const int64_t c = r % cg;
         const int64_t g = r / cg;
-        wt[idx] = oc < og ? w[((g * og + oc) * cg + c) * taps + (taps - 1 - t)] : (T)0;
+        // chunk != 0: the k order (run of `chunk` out channels, tap, out channel inside the run) instead of (tap, out channel)
+        const int64_t dst = chunk ? r * taps * ogp + ((oc / chunk) * taps + t) * chunk + oc % chunk : idx;
+        wt[dst] = oc < og ? w[((g * og + oc) * cg + c) * taps + (taps - 1 - t)] : (T)0;
     }
 }
 
-hipError_t launch_flip_weights_channels_last(int64_t es, const void* w, void* wt, int64_t groups, int64_t og, int64_t ogp, int64_t cg, int64_t taps, hipStream_t s) {
+hipError_t launch_flip_weights_channels_last(int64_t es, const void* w, void* wt, int64_t groups, int64_t og, int64_t ogp, int64_t cg, int64_t taps, hipStream_t s,
+                                             int64_t chunk) {
     const int64_t total = groups * ogp * cg * taps;
     if (total == 0) return hipSuccess;
     const dim3 g(grid_for(total)), t(256);
     switch (es) {
-    case 2: hipLaunchKernelGGL(flip_weights_channels_last_kernel<uint16_t>, g, t, 0, s, (const uint16_t*)w, (uint16_t*)wt, groups, og, ogp, cg, taps); break;
-    case 4: hipLaunchKernelGGL(flip_weights_channels_last_kernel<uint32_t>, g, t, 0, s, (const uint32_t*)w, (uint32_t*)wt, groups, og, ogp, cg, taps); break;
+    case 2: hipLaunchKernelGGL(flip_weights_channels_last_kernel<uint16_t>, g, t, 0, s, (const uint16_t*)w, (uint16_t*)wt, groups, og, ogp, cg, taps, chunk); break;
+    case 4: hipLaunchKernelGGL(flip_weights_channels_last_kernel<uint32_t>, g, t, 0, s, (const uint32_t*)w, (uint32_t*)wt, groups, og, ogp, cg, taps, chunk); break;
     default: return hipErrorInvalidValue;
     }
     return hipGetLastError();
@@ -497,24 +501,26 @@ hipError_t launch_phase_interleave(int dtype, const void* tmp, void* im, const P
 // the channels of one tap padded with zeros from cg to cgp
 template <class T>
 __global__ void __launch_bounds__(256) weights_channels_last_kernel(const T* __restrict__ w, T* __restrict__ wp, const int64_t rows,
-                                                                    const int64_t cg, const int64_t cgp, const int64_t taps) {
+                                                                    const int64_t cg, const int64_t cgp, const int64_t taps, const int64_t chunk) {
     const int64_t total = rows * cgp * taps;
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
     for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += stride) {
         const int64_t c = idx % cgp;
         const int64_t t = (idx / cgp) % taps;
         const int64_t o = idx / (cgp * taps);
-        wp[idx] = c < cg ? w[(o * cg + c) * taps + t] : (T)0;
+        // chunk != 0: the k order (run of `chunk` channels, tap, channel inside the run) instead of (tap, channel)
+        const int64_t dst = chunk ? o * taps * cgp + ((c / chunk) * taps + t) * chunk + c % chunk : idx;
+        wp[dst] = c < cg ? w[(o * cg + c) * taps + t] : (T)0;
     }
 }
 
-hipError_t launch_weights_channels_last(int64_t es, const void* w, void* wp, int64_t rows, int64_t cg, int64_t cgp, int64_t taps, hipStream_t s) {
+hipError_t launch_weights_channels_last(int64_t es, const void* w, void* wp, int64_t rows, int64_t cg, int64_t cgp, int64_t taps, hipStream_t s, int64_t chunk) {
     const int64_t total = rows * cgp * taps;
     if (total == 0) return hipSuccess;
     const dim3 g(grid_for(total)), t(256);
     switch (es) {
-    case 2: hipLaunchKernelGGL(weights_channels_last_kernel<uint16_t>, g, t, 0, s, (const uint16_t*)w, (uint16_t*)wp, rows, cg, cgp, taps); break;
-    case 4: hipLaunchKernelGGL(weights_channels_last_kernel<uint32_t>, g, t, 0, s, (const uint32_t*)w, (uint32_t*)wp, rows, cg, cgp, taps); break;
+    case 2: hipLaunchKernelGGL(weights_channels_last_kernel<uint16_t>, g, t, 0, s, (const uint16_t*)w, (uint16_t*)wp, rows, cg, cgp, taps, chunk); break;
+    case 4: hipLaunchKernelGGL(weights_channels_last_kernel<uint32_t>, g, t, 0, s, (const uint32_t*)w, (uint32_t*)wp, rows, cg, cgp, taps, chunk); break;
     default: return hipErrorInvalidValue;
     }
     return hipGetLastError();
