@@ -1067,6 +1067,22 @@ static hipError_t launch_ring16(bool ta, bool tb, const GemmParams& p, hipStream
             return launch(sp.tail_edge, tail);
         }
     }
+    if (p.batch > 1 && p.cmode != C_PARTIAL && !p.Aptr && !p.Bptr && !p.Cptr) {
+        // a batch whose tiles are whole rounds over the CUs plus a fraction: leading columns of every item, then the rest
+        // (see ring16_column_split; the same products, tiled differently)
+        const int64_t head_cols = ring16_column_split(p.M, p.N, p.K, p.batch);
+        if (head_cols) {
+            GemmParams head = p, tail = p;
+            head.N = (int)head_cols;
+            tail.N = p.N - (int)head_cols;
+            tail.B = static_cast<const char*>(p.B) + head_cols * (tb ? p.ldb : 1) * 2;
+            tail.C = static_cast<char*>(p.C) + head_cols * 2;
+            if (p.bias) tail.bias = static_cast<const char*>(p.bias) + head_cols * p.bias_cs * 2;
+            const hipError_t e = launch_ring16_planned(head, s, launch, RECT_128 | RECT_192);
+            if (e != hipSuccess) return e;
+            return launch_ring16_planned(tail, s, launch, RECT_128 | RECT_192);
+        }
+    }
     return launch_ring16_planned(p, s, launch, RECT_128 | RECT_192);
 }
 

@@ -101,7 +101,9 @@ static inline int ring16_tile_rows(int t) { return t == 224 ? 192 : t == 192 ? 1
 static inline int ring16_tile_cols(int t) { return t == 224 || t == 192 ? 256 : t; }
 static inline double ring16_cost_us(int t, int64_t nt, int64_t K) {
     const double cu_flops_per_us = 9.77e6;                      // 2500 TFLOP/s over 256 CUs
-    const double f = t == 256 ? (nt >= 192 ? 0.5 : 0.64) : t == 224 || t == 192 ? (nt >= 192 ? 0.5 : 0.55) : t == 128 ? 0.4 : 0.25;
+    // (128 x 128 tiles are bound by the LDS of their CU whether one or two workgroups share it: 0.3 of the peak once every CU has
+    //  more than one tile to work through -- 64 x [256 x 3136] . [3136 x 2304] took 376 us on them, 280 us on 256-wide tiles)
+    const double f = t == 256 ? (nt >= 192 ? 0.5 : 0.64) : t == 224 || t == 192 ? (nt >= 192 ? 0.5 : 0.55) : t == 128 ? (nt > 256 ? 0.3 : 0.4) : 0.25;
     const double latency = t == 256 ? 3.0 : t == 224 ? 4.0 : t == 192 ? 5.0 : t == 128 ? 1.5 : 0.6;
     const double area = (double)ring16_tile_rows(t) * ring16_tile_cols(t);
     return (double)((nt + 255) / 256) * (2.0 * area * (double)K / (cu_flops_per_us * f) + latency);

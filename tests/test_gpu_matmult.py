@@ -899,3 +899,41 @@ def test_small_fp32_products_on_32_wide_tiles():
             want = outs[0].clone()
             want[:, :, :n] = torch.where(outs[0][:, :, :n] > 0, outs[0][:, :, :n], torch.zeros_like(outs[0][:, :, :n]))
             assert torch.equal(c, want)
+
+
+@pytest.mark.parametrize("dtype", ["bf16", np.float16], ids=["bf16", "fp16"])
+def test_batched_16bit_products_split_along_the_columns(dtype):
+    """A batch whose 256-wide tiles make whole rounds over the CUs plus a fraction (64 x [256 x 2304] outputs: 576 tiles)
+    goes out as two launches, the leading 2048 columns of every item and the last 256 on other tiles.  Items must equal
+    the same product computed alone, bit for bit (bias and C0 follow the columns), for both layouts of B."""
+    bf = dtype == "bf16"
+    lib = _lib.load()
+    st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    rng = np.random.default_rng(5151)
+    batch, m, k, n = 64, 256, 1024, 2304
+    a = to_torch(randn(rng, (batch, m, k), dtype, 0.25), DEV, bf)
+    c0 = to_torch(randn(rng, (batch, m, n), dtype), DEV, bf)
+    bias = to_torch(randn(rng, (n,), dtype), DEV, bf)
+    for tb, mode in ((False, _lib.C_BIAS), (True, _lib.C_ACCUMULATE)):
+        b = to_torch(randn(rng, (batch, n, k) if tb else (batch, k, n), dtype, 0.25), DEV, bf)
+        d = _lib.GemmDesc()
+        d.dtype, d.transpose_b, d.c_mode = F.ntg_dtype(a), int(tb), mode
+        d.m, d.k, d.n, d.batches = m, k, n, batch
+        d.stride_a, d.stride_b, d.stride_c = m * k, k * n, m * n
+        if mode == _lib.C_BIAS:
+            d.bias, d.bias_col_stride = bias.data_ptr(), 1
+        c = c0.clone()
+        _lib.check(lib.ntg_gemm_dev(ctypes.byref(d), a.data_ptr(), b.data_ptr(), c.data_ptr(), st))
+        for i in (0, 17, 63):
+            one = c0[i].clone()
+            d1 = _lib.GemmDesc()
+            d1.dtype, d1.transpose_b, d1.c_mode = d.dtype, int(tb), mode
+            d1.m, d1.k, d1.n, d1.batches = m, k, n, 1
+            if mode == _lib.C_BIAS:
+                d1.bias, d1.bias_col_stride = bias.data_ptr(), 1
+            _lib.check(lib.ntg_gemm_dev(ctypes.byref(d1), a[i].data_ptr(), b[i].data_ptr(), one.data_ptr(), st))
+            torch.cuda.synchronize()
+            assert torch.equal(c[i].view(torch.int16), one.view(torch.int16)), (tb, mode, i)
+            bi = b[i].t() if tb else b[i]
+            ref = a[i].double() @ bi.double() + (c0[i].double() if mode == _lib.C_ACCUMULATE else bias.double())
+            assert (one.double() - ref).abs().max().item() <= HALF_REL * ref.abs().max().item()
