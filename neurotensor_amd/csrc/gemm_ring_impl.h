@@ -1070,7 +1070,7 @@ static hipError_t launch_ring16(bool ta, bool tb, const GemmParams& p, hipStream
     if (p.batch > 1 && p.cmode != C_PARTIAL && !p.Aptr && !p.Bptr && !p.Cptr) {
         // a batch whose tiles are whole rounds over the CUs plus a fraction: leading columns of every item, then the rest
         // (see ring16_column_split; the same products, tiled differently)
-        const int64_t head_cols = ring16_column_split(p.M, p.N, p.K, p.batch);
+        const int64_t head_cols = ring16_column_split(p.M, p.N, p.K, p.batch, RECT_128 | RECT_192);
         if (head_cols) {
             GemmParams head = p, tail = p;
             head.N = (int)head_cols;

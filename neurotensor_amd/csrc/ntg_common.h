@@ -166,13 +166,13 @@ static inline double ring16_plan_cost_us(const Ring16Plan& pl, int64_t M, int64_
 // tiles = two rounds, the last 256 columns go to 128 x 128 tiles).  The split gives the leading head_cols columns of every
 // item to one (planned) launch and the remaining columns to another, each on the tile chosen for it alone.
 // head_cols = columns of the first launch, a multiple of 128; 0: no split.  It has to be 5 % ahead of the batch plan.
-static inline int64_t ring16_column_split(int64_t M, int64_t N, int64_t K, int64_t batch) {
+static inline int64_t ring16_column_split(int64_t M, int64_t N, int64_t K, int64_t batch, int rect = RECT_NONE) {
     if (N < 256 || N / 128 > 2048) return 0;
-    double best = 0.95 * ring16_plan_cost_us(ring16_plan(M, N, K, batch), M, N, K, batch);
+    double best = 0.95 * ring16_plan_cost_us(ring16_plan(M, N, K, batch, rect), M, N, K, batch);
     int64_t best_cols = 0;
     for (int64_t c = 128; c < N; c += 128) {
-        const double us = ring16_plan_cost_us(ring16_plan(M, c, K, batch), M, c, K, batch) +
-                          ring16_plan_cost_us(ring16_plan(M, N - c, K, batch), M, N - c, K, batch) + 2.0;
+        const double us = ring16_plan_cost_us(ring16_plan(M, c, K, batch, rect), M, c, K, batch) +
+                          ring16_plan_cost_us(ring16_plan(M, N - c, K, batch, rect), M, N - c, K, batch) + 2.0;
         if (us < best) { best = us; best_cols = c; }
     }
     return best_cols;
