@@ -167,10 +167,31 @@ static inline double ring16_plan_cost_us(const Ring16Plan& pl, int64_t M, int64_
 // item to one (planned) launch and the remaining columns to another, each on the tile chosen for it alone.
 // head_cols = columns of the first launch, a multiple of 128; 0: no split.  It has to be 5 % ahead of the batch plan.
 static inline int64_t ring16_column_split(int64_t M, int64_t N, int64_t K, int64_t batch, int rect = RECT_NONE) {
-    if (N < 256 || N / 128 > 2048) return 0;
+    if (N < 256) return 0;
+    // candidates (a handful, so that planning stays a few microseconds on the launch path): for 256- and 128-wide tile
+    // columns, the whole tile columns before a narrow rest, and the largest count of tile columns whose tiles over the whole
+    // batch are whole rounds of the 256 CUs -- as head and, mirrored, as tail
+    int64_t cand[8];
+    int nc = 0;
+    auto add = [&](int64_t c) {
+        if (c <= 0 || c >= N || c % 128 != 0) return;
+        for (int i = 0; i < nc; ++i)
+            if (cand[i] == c) return;
+        cand[nc++] = c;
+    };
+    for (int64_t tc : {(int64_t)256, (int64_t)128}) {
+        add(N / tc * tc);
+        const int64_t per_col = ((M + tc - 1) / tc) * batch;             // tiles of one tile column over the batch (square tiles)
+        int64_t g = per_col, h = 256;
+        while (h) { const int64_t r = g % h; g = h; h = r; }              // gcd(per_col, 256)
+        const int64_t q0 = 256 / g, q = (N / tc) / q0 * q0;
+        add(q * tc);
+        add(N - q * tc);
+    }
     double best = 0.95 * ring16_plan_cost_us(ring16_plan(M, N, K, batch, rect), M, N, K, batch);
     int64_t best_cols = 0;
-    for (int64_t c = 128; c < N; c += 128) {
+    for (int i = 0; i < nc; ++i) {
+        const int64_t c = cand[i];
         const double us = ring16_plan_cost_us(ring16_plan(M, c, K, batch, rect), M, c, K, batch) +
                           ring16_plan_cost_us(ring16_plan(M, N - c, K, batch, rect), M, N - c, K, batch) + 2.0;
         if (us < best) { best = us; best_cols = c; }
@@ -195,7 +216,15 @@ static inline Ring16Split ring16_split(int64_t M, int64_t N, int64_t K, int rect
     double best = 0.95 * ring16_cost_us(edge, T, K);
     for (int axis = 1; axis <= 2; ++axis) {
         const int64_t count = axis == 1 ? tn : tm, other = axis == 1 ? tm : tn, step = axis == 1 ? tc : tr;
-        for (int64_t c = 1; c < count; ++c) {
+        // candidates: the counts of leading tile columns / rows that make whole rounds over the CUs (the largest two), and all
+        // but the last one or two -- a handful, so that planning stays on the order of a microsecond
+        int64_t g = other, h = 256;
+        while (h) { const int64_t r = g % h; g = h; h = r; }              // gcd(other, 256)
+        const int64_t q0 = 256 / g, qmax = (count - 1) / q0 * q0;
+        const int64_t cands[4] = {qmax, qmax - q0, count - 1, count - 2};
+        for (int ci = 0; ci < 4; ++ci) {
+            const int64_t c = cands[ci];
+            if (c < 1 || c >= count) continue;
             const int64_t rest = (axis == 1 ? N : M) - c * step;
             const int64_t Mt = axis == 1 ? M : rest, Nt = axis == 1 ? rest : N;
             const int te = ring16_tile_edge(Mt, Nt, K, 1, rect);
