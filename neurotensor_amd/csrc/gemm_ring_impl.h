@@ -75,12 +75,15 @@ template <> struct Cvt16<DT_BF16> {
 // WB = 32 x 32 blocks per wavefront along each of m and n: 4 -> 256 x 256 tile, 2 -> 128 x 128 tile
 // ES = bytes per element (2: Float16 / BFloat16, 4: Float32).  A K-step is 64 bytes of k for every row (32 or 16
 // elements), so the byte geometry of tiles, stages and DMA instructions is the same for both element sizes.
-template <int WB, int ES>
+// KD = 64-byte runs of k per row and K-step: 1, or 2 for the deep K-step of the small 16-bit tiles (see gemm_ring_kernel)
+template <int WB, int ES, int KD = 1>
 struct RingGeom {
-    static constexpr int BM = 64 * WB, BN = 64 * WB, BK = 64 / ES, NST = 4;
+    static constexpr int KB = 64 * KD;                   // bytes of k per row and K-step
+    static constexpr int BM = 64 * WB, BN = 64 * WB, BK = KB / ES, NST = 4;
     static constexpr int VEL = 16 / ES;                  // elements per 16-byte chunk
     static constexpr int WT = 32 * WB;                   // edge of a wavefront's share of the tile
-    static constexpr int TILE_BYTES = BM * 64;           // one operand tile, 16 / 8 KiB
+    static constexpr int TILE_BYTES = BM * KB;           // one operand tile, 16 / 8 KiB (twice that with KD = 2)
+    static constexpr int NI = WB * KD;                   // DMA instructions per wavefront and operand tile
     static constexpr int STAGE_BYTES = 2 * TILE_BYTES;   // 32 / 16 KiB
     static constexpr int MN_ROW_BYTES = BM * ES;         // one k-row of an MN-contiguous operand tile
     static constexpr int CHUNKS = MN_ROW_BYTES / 16;     // 16-byte chunks in such a row (16 .. 64)
@@ -106,15 +109,21 @@ struct RingGeom {
 template <int CH>
 __device__ __forceinline__ int mn8_swizzle(int krow) { return CH >= 8 ? (krow & 7) : ((krow & 7) >> 1); }
 
-template <bool KC, bool RAGGED, int WB, int ES>
-__device__ __forceinline__ void dma_offsets(uint32_t (&off)[WB], int64_t ld, int wave, int lane, int mn_valid, int k_valid) {
+// 128-byte rows (KD = 2): 16-byte slot kv of row r is stored at kv ^ swz8(r).  Eight consecutive rows get eight different
+// values, and so do the eight rows of either parity among sixteen consecutive ones: whichever way the banks repeat
+// (every 128 or every 256 bytes), the lanes that one pass of a ds_read_b128 serves hit different banks.
+__device__ __forceinline__ int swz8(int row) { return (row & 7) ^ ((row >> 3) & 1); }
+
+template <bool KC, bool RAGGED, int WB, int ES, int KD = 1>
+__device__ __forceinline__ void dma_offsets(uint32_t (&off)[WB * KD], int64_t ld, int wave, int lane, int mn_valid, int k_valid) {
     constexpr int CH = RingGeom<WB, ES>::CHUNKS, VEL = RingGeom<WB, ES>::VEL;
 #pragma unroll
-    for (int jj = 0; jj < WB; ++jj) {
-        const int j = wave * WB + jj;
+    for (int jj = 0; jj < WB * KD; ++jj) {
+        const int j = wave * WB * KD + jj;
         if constexpr (KC) {
-            int row = 16 * j + (lane >> 2);
-            int kv = (lane & 3) ^ ((row >> 1) & 3);
+            // (KD = 2: an instruction covers 8 rows of 128 bytes, whole cache lines)
+            int row = KD == 2 ? 8 * j + (lane >> 3) : 16 * j + (lane >> 2);
+            int kv = KD == 2 ? (lane & 7) ^ swz8(row) : (lane & 3) ^ ((row >> 1) & 3);
             if constexpr (RAGGED) {
                 row = row < mn_valid ? row : mn_valid - 1;
                 kv = kv < k_valid / VEL ? kv : k_valid / VEL - 1;
@@ -155,7 +164,7 @@ __device__ __forceinline__ void dma_dword(const void* addr, uint32_t lds_addr) {
 // what the padding taps of a gathered convolution operand read
 static __device__ __attribute__((aligned(16))) const uint32_t ring_zero_word[4] = {0u, 0u, 0u, 0u};
 
-template <int WB>
+template <int WB>   // (WB = instructions per wavefront)
 __device__ __forceinline__ void dma_tile(const void* sbase, const uint32_t (&off)[WB], uint32_t lds_tile, int wave_u) {
 #pragma unroll
     for (int jj = 0; jj < WB; ++jj) dma_1k(sbase, off[jj], lds_tile + (uint32_t)(wave_u * WB + jj) * 1024u);
@@ -173,7 +182,11 @@ __device__ __forceinline__ uint32_t lds_addr_of(const char* p) {
 // and columns / k-rows past the edge read a zero word instead, so the tile in LDS is exact and the multiply loop is the
 // plain one.  Wavefront w gathers k-rows 4 w .. 4 w + 3 of every K-step.
 // WBN_ != 0: a rectangular tile, 64 WB_ rows x 64 WBN_ columns (plain products only).
-template <int DT, bool TA, bool TB, bool RAGGED, int WB_, int CONV = 0, int WBN_ = 0>
+// KD_ = 2 (16-bit plain products on 128 x 128 tiles): a K-step is 128 bytes of k per row, so a K-contiguous operand is
+// fetched in whole 128-byte cache lines (half the requests to L2 of the 64-byte K-step) and the one barrier of a K-step
+// comes every sixteen MFMAs instead of every eight; the four stages are 32 KiB each (one workgroup per CU).  Fragments
+// are read two quarter-steps ahead (four sets in registers), the whole of tile kt + 3 is fetched during K-step kt.
+template <int DT, bool TA, bool TB, bool RAGGED, int WB_, int CONV = 0, int WBN_ = 0, int KD_ = 1>
 __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
     using E = Elem<DT>;
     using T = typename E::T;
@@ -181,8 +194,10 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
     constexpr int WBM = WB_, WBN = WBN_ ? WBN_ : WB_;    // 32 x 32 blocks per wavefront along m / along n
     constexpr int WB = WBN;                              // (the gathered operand is B; gathering kernels have square tiles)
     static_assert(CONV == 0 || WBM == WBN, "gathering kernels have square tiles");
-    using GA = RingGeom<WBM, ES>;                        // geometry of the A tile
-    using G = RingGeom<WBN, ES>;                         // geometry of the B tile
+    constexpr int KD = KD_;
+    static_assert(KD == 1 || (KD == 2 && CONV == 0 && ES == 2 && WB_ == 2 && WBN_ == 0), "deep K-steps: 16-bit plain products on 128 x 128 tiles");
+    using GA = RingGeom<WBM, ES, KD>;                    // geometry of the A tile
+    using G = RingGeom<WBN, ES, KD>;                     // geometry of the B tile
     constexpr int A_TILE_BYTES = GA::TILE_BYTES, STAGE_BYTES = GA::TILE_BYTES + G::TILE_BYTES;
     constexpr int WTM = GA::WT, WTN = G::WT;             // a wavefront's share of the tile: WTM rows x WTN columns
     constexpr bool GATHER4 = CONV == 1 || CONV == 2;     // op(B) gathered element by element from an NCHW image
@@ -194,7 +209,7 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
     static_assert(!GATHER4 || (ES == 4 && !TA && RAGGED), "gathered operands: Float32, A stored [m][k], guarded edges");
     static_assert(!GATHER16 || ((ES == 4 || ES == 2) && !TA && RAGGED), "channels-last gather: 16/32-bit floats, A stored [m][k], guarded edges");
     static_assert(!GATHERW || ((ES == 4 || ES == 2) && !TB && RAGGED), "channels-last weight gradient: 16/32-bit floats, guarded edges");
-    constexpr int NA = WBM, NB = GATHER4 ? 4 * WB : WBN;   // DMA instructions per wavefront and K-step for the A / B tile
+    constexpr int NA = WBM * KD, NB = GATHER4 ? 4 * WB : WBN * KD;   // DMA instructions per wavefront and K-step for the A / B tile
     // B instructions issued in the first / second half-step (the second also carries the A tile's).  Splitting a gathered
     // tile between the two was measured slower than issuing all of it in the first.
     constexpr int NB1 = NB, NB2 = NB - NB1;
@@ -228,12 +243,12 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
     const int kr = p.K - last * BK;                                  // k that exist in the last K-step (a multiple of one chunk)
     const int mvalid = p.M - m0 < GA::BM ? p.M - m0 : GA::BM;
     const int nvalid = p.N - n0 < G::BN ? p.N - n0 : G::BN;
-    uint32_t offA[WBM], offB[WBN];      // K-steps before the last
-    uint32_t offAt[WBM], offBt[WBN];    // the last K-step (RAGGED: k clamped to what exists)
-    dma_offsets<A_KC, RAGGED, WBM, ES>(offA, p.lda, wave, lane, mvalid, BK);
-    dma_offsets<B_KC, RAGGED, WBN, ES>(offB, p.ldb, wave, lane, nvalid, BK);
-    dma_offsets<A_KC, RAGGED, WBM, ES>(offAt, p.lda, wave, lane, mvalid, kr);
-    dma_offsets<B_KC, RAGGED, WBN, ES>(offBt, p.ldb, wave, lane, nvalid, kr);
+    uint32_t offA[WBM * KD], offB[WBN * KD];      // K-steps before the last
+    uint32_t offAt[WBM * KD], offBt[WBN * KD];    // the last K-step (RAGGED: k clamped to what exists)
+    dma_offsets<A_KC, RAGGED, WBM, ES, KD>(offA, p.lda, wave, lane, mvalid, BK);
+    dma_offsets<B_KC, RAGGED, WBN, ES, KD>(offB, p.ldb, wave, lane, nvalid, BK);
+    dma_offsets<A_KC, RAGGED, WBM, ES, KD>(offAt, p.lda, wave, lane, mvalid, kr);
+    dma_offsets<B_KC, RAGGED, WBN, ES, KD>(offBt, p.ldb, wave, lane, nvalid, kr);
     const char* baseA = reinterpret_cast<const char*>(A) + (A_KC ? (int64_t)m0 * p.lda : (int64_t)m0) * ES;
     const char* baseB = reinterpret_cast<const char*>(B) + (B_KC ? (int64_t)n0 * p.ldb : (int64_t)n0) * ES;
     const int64_t advA = (A_KC ? (int64_t)BK : (int64_t)BK * p.lda) * ES;
@@ -497,6 +512,7 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
     // MN-major, Float32: four ds_read_b32 per block, element e from k-row 8 ks + 4 (lane/32) + e
     auto frag_off_km = [&](int wbase, int blk, int ks) -> int {
         const int row = wbase + blk * 32 + (lane & 31);
+        if constexpr (KD == 2) return row * 128 + (((2 * ks + (lane >> 5)) ^ swz8(lane & 31)) * 16);   // (wbase + 32 blk is a multiple of 16)
         const int slot = (2 * ks + (lane >> 5)) ^ ((lane >> 1) & 3);
         return row * 64 + slot * 16;
     };
@@ -581,17 +597,18 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
 #pragma unroll
             for (int x = 0; x < WB; ++x) conv4_dma(x, lds_tile);
         }
-        else dma_tile<WBN>(srcB(kt), kt >= last ? offBt : offB, lds_tile, wave_u);
+        else dma_tile<WBN * KD>(srcB(kt), kt >= last ? offBt : offB, lds_tile, wave_u);
     };
-    dma_tile<WBM>(srcA(0), 0 >= last ? offAt : offA, lds_addr_of(st0), wave_u);
+    dma_tile<NA>(srcA(0), 0 >= last ? offAt : offA, lds_addr_of(st0), wave_u);
     b_tile(0, lds_addr_of(st0) + A_TILE_BYTES);
-    dma_tile<WBM>(srcA(1), 1 >= last ? offAt : offA, lds_addr_of(st1), wave_u);
+    dma_tile<NA>(srcA(1), 1 >= last ? offAt : offA, lds_addr_of(st1), wave_u);
     b_tile(1, lds_addr_of(st1) + A_TILE_BYTES);
-    dma_tile<WBM>(srcA(2), 2 >= last ? offAt : offA, lds_addr_of(st2), wave_u);
+    dma_tile<NA>(srcA(2), 2 >= last ? offAt : offA, lds_addr_of(st2), wave_u);
     b_tile(2, lds_addr_of(st2) + A_TILE_BYTES);
-    dma_tile<WBM>(srcA(3), 3 >= last ? offAt : offA, lds_addr_of(st3), wave_u);
+    if constexpr (KD == 1) dma_tile<NA>(srcA(3), 3 >= last ? offAt : offA, lds_addr_of(st3), wave_u);
 
-    u32x4 af[2][WBM], bf[2][WBN];   // fragment double buffer: [half-step parity][block]
+    constexpr int NBUF = 2 * KD;
+    u32x4 af[NBUF][WBM], bf[NBUF][WBN];   // fragment sets: [half-step parity][block]; deep K-steps: [quarter-step][block]
 
     // all reads of one fragment set, back to back (prologue only)
     auto load_frags = [&](const char* stage, int ks, int buf) {
@@ -651,10 +668,11 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
     };
 
     // tile 0 must have landed before its first fragments are read
-    NTG_WAIT_VMCNT(2 * (NA + NB) + NA);
+    NTG_WAIT_VMCNT(2 * (NA + NB) + (KD == 1 ? NA : 0));
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
     load_frags(st0, 0, 0);
+    if constexpr (KD == 2) load_frags(st0, 1, 1);
 
     // One K-step.  `cur` holds tile kt (its half-step 0 fragments are already in registers),
     // `nxt` holds tile kt+1, `prv` held tile kt-1.  The single barrier sits between the two
@@ -663,11 +681,11 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
     // second half-step, its B half during the first half-step of the next K-step.  Tile kt+1,
     // first touched in the second half, has had three K-steps to arrive.
     // RAGGED: zero the k >= K part of a fragment set of the last K-step.  Every lane's fragment
-    // covers one chunk of consecutive k (8 or 4) starting at (BK/2) ks + (BK/4) (lane / 32) in both
+    // covers one chunk of consecutive k (8 or 4) starting at (32 bytes) ks + (16 bytes) (lane / 32) in both
     // LDS layouts, and K is a multiple of the chunk, so a lane's fragment is either entirely real or
     // entirely past the end.
     auto mask_tail = [&](int buf, int ks) {
-        const bool ok = (BK / 2) * ks + (BK / 4) * (lane >> 5) < kr;
+        const bool ok = (32 / ES) * ks + (16 / ES) * (lane >> 5) < kr;
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
 #pragma unroll
@@ -712,11 +730,54 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
         }
     };
 
+    // One deep K-step (KD = 2): four quarter-steps, fragment set q holding quarter-step q.  Sets 0 and 1 of tile kt are in
+    // registers on entry; quarter-steps 0 and 1 read sets 2 and 3 from `cur`, then the barrier (every wavefront is done
+    // with `cur`, which the next K-step refills, and tile kt + 1 has landed), and quarter-steps 2 and 3 read sets 0 and 1 of
+    // `nxt`.  `prv` went back to the DMA at the previous K-step's barrier: the whole of tile kt + 3 is fetched into it, a
+    // quarter of the instructions per quarter-step.
+    auto iteration_deep = [&](int kt, char* cur, const char* nxt, char* prv) __attribute__((always_inline)) {
+      if constexpr (KD == 2) {
+        static_assert((NA + NB) % 4 == 0, "a quarter of the tile's DMA instructions per quarter-step");
+        constexpr int PER = (NA + NB) / 4;
+        const bool lastk = RAGGED && kt == last && kr < BK;
+        const void* sa = srcA(kt + 3);
+        const void* sb = srcB(kt + 3);
+        const bool tail = kt + 3 >= last;
+        const uint32_t lds_a = lds_addr_of(prv), lds_b = lds_addr_of(prv) + A_TILE_BYTES;
+        auto issue_at = [&](int y) __attribute__((always_inline)) {
+            if (y < NA) dma_1k(sa, (RAGGED && tail) ? offAt[y] : offA[y], lds_a + (uint32_t)(wave_u * NA + y) * 1024u);
+            else dma_1k(sb, (RAGGED && tail) ? offBt[y - NA] : offB[y - NA], lds_b + (uint32_t)(wave_u * NB + y - NA) * 1024u);
+        };
+        using NP = std::integral_constant<int, PER>;
+        using N0 = std::integral_constant<int, 0>;
+        if (lastk) mask_tail(0, 0);
+        mma_step_prefetch(0, cur, 2, 2, NP{}, N0{}, [&](int x) __attribute__((always_inline)) { issue_at(x); });
+        if (lastk) mask_tail(1, 1);
+        mma_step_prefetch(1, cur, 3, 3, NP{}, N0{}, [&](int x) __attribute__((always_inline)) { issue_at(PER + x); });
+        // issued since the last instruction of tile kt+1: tile kt+2 and half of tile kt+3
+        NTG_WAIT_VMCNT((NA + NB) + 2 * PER);
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // my reads of `cur` are complete
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        if (lastk) mask_tail(2, 2);
+        mma_step_prefetch(2, nxt, 0, 0, NP{}, N0{}, [&](int x) __attribute__((always_inline)) { issue_at(2 * PER + x); });
+        if (lastk) mask_tail(3, 3);
+        mma_step_prefetch(3, nxt, 1, 1, NP{}, N0{}, [&](int x) __attribute__((always_inline)) { issue_at(3 * PER + x); });
+      }
+    };
+
     for (int kt = 0; kt < KT; kt += 4) {
-        iteration(kt, st0, st1, st3);
-        if (kt + 1 < KT) iteration(kt + 1, st1, st2, st0);
-        if (kt + 2 < KT) iteration(kt + 2, st2, st3, st1);
-        if (kt + 3 < KT) iteration(kt + 3, st3, st0, st2);
+        if constexpr (KD == 2) {
+            iteration_deep(kt, st0, st1, st3);
+            if (kt + 1 < KT) iteration_deep(kt + 1, st1, st2, st0);
+            if (kt + 2 < KT) iteration_deep(kt + 2, st2, st3, st1);
+            if (kt + 3 < KT) iteration_deep(kt + 3, st3, st0, st2);
+        } else {
+            iteration(kt, st0, st1, st3);
+            if (kt + 1 < KT) iteration(kt + 1, st1, st2, st0);
+            if (kt + 2 < KT) iteration(kt + 2, st2, st3, st1);
+            if (kt + 3 < KT) iteration(kt + 3, st3, st0, st2);
+        }
     }
     NTG_WAIT_VMCNT(0);              // clamped tail DMAs have landed
     __builtin_amdgcn_s_barrier();   // all fragment reads done: LDS is free for the epilogue
@@ -904,19 +965,19 @@ static inline bool ring_eligible(const GemmParams& p, bool ta, int es = 2) {
 }
 
 // WBN != 0: rectangular tiles of 64 WB rows x 64 WBN columns
-template <int DT, bool TA, bool TB, int WB, int WBN = 0>
+template <int DT, bool TA, bool TB, int WB, int WBN = 0, int KD = 1>
 static hipError_t launch_ring_cfg(const GemmParams& pin, hipStream_t s) {
     constexpr int ES = (int)sizeof(typename Elem<DT>::T);
-    constexpr int TEM = RingGeom<WB, ES>::BM, TEN = RingGeom<(WBN ? WBN : WB), ES>::BM, BK = RingGeom<WB, ES>::BK;
+    constexpr int TEM = RingGeom<WB, ES>::BM, TEN = RingGeom<(WBN ? WBN : WB), ES>::BM, BK = RingGeom<WB, ES, KD>::BK;
     GemmParams p = pin;
     p.tiles_m = (p.M + TEM - 1) / TEM;
     p.tiles_n = (p.N + TEN - 1) / TEN;
     const int64_t blocks = (int64_t)p.tiles_m * p.tiles_n * p.batch;
     if (blocks > 0x7fffffffLL) return hipErrorInvalidValue;
     if (p.M % TEM == 0 && p.N % TEN == 0 && p.K % BK == 0)
-        hipLaunchKernelGGL((gemm_ring_kernel<DT, TA, TB, false, WB, 0, WBN>), dim3((unsigned)blocks), dim3(256), 0, s, p);
+        hipLaunchKernelGGL((gemm_ring_kernel<DT, TA, TB, false, WB, 0, WBN, KD>), dim3((unsigned)blocks), dim3(256), 0, s, p);
     else
-        hipLaunchKernelGGL((gemm_ring_kernel<DT, TA, TB, true, WB, 0, WBN>), dim3((unsigned)blocks), dim3(256), 0, s, p);
+        hipLaunchKernelGGL((gemm_ring_kernel<DT, TA, TB, true, WB, 0, WBN, KD>), dim3((unsigned)blocks), dim3(256), 0, s, p);
     return hipGetLastError();
 }
 
@@ -978,10 +1039,10 @@ static hipError_t launch_ring_nhwc_dw_cfg(const GemmParams& pin, hipStream_t s) 
     return hipGetLastError();
 }
 
-template <int DT, int WB, int WBN = 0>
+template <int DT, int WB, int WBN = 0, int KD = 1>
 static hipError_t launch_ring_wb(bool ta, bool tb, const GemmParams& p, hipStream_t s) {
-    if (ta) return tb ? launch_ring_cfg<DT, true, true, WB, WBN>(p, s) : launch_ring_cfg<DT, true, false, WB, WBN>(p, s);
-    return tb ? launch_ring_cfg<DT, false, true, WB, WBN>(p, s) : launch_ring_cfg<DT, false, false, WB, WBN>(p, s);
+    if (ta) return tb ? launch_ring_cfg<DT, true, true, WB, WBN, KD>(p, s) : launch_ring_cfg<DT, true, false, WB, WBN, KD>(p, s);
+    return tb ? launch_ring_cfg<DT, false, true, WB, WBN, KD>(p, s) : launch_ring_cfg<DT, false, false, WB, WBN, KD>(p, s);
 }
 
 // items [b0, b0 + nb) of a strided batch as a product of their own
@@ -1055,6 +1116,8 @@ static hipError_t launch_ring16(bool ta, bool tb, const GemmParams& p, hipStream
         if (te == 224) return launch_ring_wb<DT, 3, 4>(ta, tb, q, s);      // 192 rows x 256 columns
         if (te == 192) return launch_ring_wb<DT, 2, 4>(ta, tb, q, s);      // 128 rows x 256 columns
         if (te == 64) return launch_ring_wb<DT, 1>(ta, tb, q, s);
+        // 128 x 128: the deep K-step unless many tiles with a short k queue up on every CU (see ring16_deep128)
+        if (ring16_deep128(ring16_tiles(128, q.M, q.N, q.batch), q.K)) return launch_ring_wb<DT, 2, 0, 2>(ta, tb, q, s);
         return launch_ring_wb<DT, 2>(ta, tb, q, s);
     };
     if (p.batch == 1 && p.cmode != C_PARTIAL && !p.Aptr && !p.Bptr && !p.Cptr) {

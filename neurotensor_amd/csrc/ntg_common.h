@@ -99,12 +99,19 @@ enum { ACT_NONE = 0, ACT_RELU = 1 };
 // neighbours on the CU.  Estimated time = tiles per CU x (tile time + exposed latency).
 static inline int ring16_tile_rows(int t) { return t == 224 ? 192 : t == 192 ? 128 : t; }
 static inline int ring16_tile_cols(int t) { return t == 224 || t == 192 ? 256 : t; }
+// 128 x 128 tiles come in two forms: the deep K-step (128 bytes of k per row: whole cache lines of a K-contiguous operand,
+// half as many barriers; 128 KiB of LDS, one workgroup per CU) and the 64-byte K-step with two workgroups per CU, which
+// is ahead only where many tiles with a short k queue up on every CU (the second workgroup hides the first one's prologue
+// and epilogue): 1024 tiles at k = 1024 took 40.6 us against 44.6, 1024 tiles at k = 4096 145 against 134.
+static inline bool ring16_deep128(int64_t nt, int64_t K) { return nt <= 256 || K >= 2048; }
 static inline double ring16_cost_us(int t, int64_t nt, int64_t K) {
     const double cu_flops_per_us = 9.77e6;                      // 2500 TFLOP/s over 256 CUs
-    // (128 x 128 tiles are bound by the LDS of their CU whether one or two workgroups share it: 0.3 of the peak once every CU has
-    //  more than one tile to work through -- 64 x [256 x 3136] . [3136 x 2304] took 376 us on them, 280 us on 256-wide tiles)
-    const double f = t == 256 ? (nt >= 192 ? 0.5 : 0.64) : t == 224 || t == 192 ? (nt >= 192 ? 0.5 : 0.55) : t == 128 ? (nt > 256 ? 0.3 : 0.4) : 0.25;
-    const double latency = t == 256 ? 3.0 : t == 224 ? 4.0 : t == 192 ? 5.0 : t == 128 ? 1.5 : 0.6;
+    // (measured per-tile figures: fraction of the CU's MFMA peak in the K loop, and microseconds of prologue + epilogue;
+    //  the 64-byte K-step on 128 x 128 tiles is bound by the LDS of its CU whether one or two workgroups share it)
+    const bool deep = t == 128 && ring16_deep128(nt, K);
+    const double f = t == 256 ? (nt >= 192 ? 0.5 : 0.64) : t == 224 || t == 192 ? (nt >= 192 ? 0.5 : 0.55)
+                   : t == 128 ? (deep ? (nt > 256 ? 0.45 : nt >= 192 ? 0.5 : 0.565) : 0.3) : 0.25;
+    const double latency = t == 256 ? 3.0 : t == 224 ? 4.0 : t == 192 ? 5.0 : t == 128 ? (deep ? (nt >= 192 ? 7.0 : 4.0) : 1.5) : 0.6;
     const double area = (double)ring16_tile_rows(t) * ring16_tile_cols(t);
     return (double)((nt + 255) / 256) * (2.0 * area * (double)K / (cu_flops_per_us * f) + latency);
 }

@@ -937,3 +937,51 @@ def test_batched_16bit_products_split_along_the_columns(dtype):
             bi = b[i].t() if tb else b[i]
             ref = a[i].double() @ bi.double() + (c0[i].double() if mode == _lib.C_ACCUMULATE else bias.double())
             assert (one.double() - ref).abs().max().item() <= HALF_REL * ref.abs().max().item()
+
+
+@pytest.mark.parametrize("dtype", ["bf16", np.float16], ids=["bf16", "fp16"])
+def test_16bit_products_on_deep_k_steps(dtype):
+    """Mid-sized 16-bit products (up to 256 tiles of 128 x 128, or a deep k) run on the kernel whose K-step is 128 bytes of
+    k per row.  All four storage forms, edges that are not multiples of the tile, k that is not a multiple of the 64-element
+    K-step (tails of 8 and 40), overwrite / accumulate / bias: every element is the once-rounded exact result (within the
+    float32 accumulation bound), and a strip of 64 columns computed as a product of its own -- on 64 x 64 tiles, 64-byte
+    K-steps -- has the same bits: the order of summation over k does not depend on the kernel."""
+    from util import assert_one_rounding
+    bf = dtype == "bf16"
+    fmt = "bf16" if bf else "f16"
+    lib = _lib.load()
+    st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    rng = np.random.default_rng(6464)
+    cases = [(1536, 4136, 1528, _lib.C_ACCUMULATE), (776, 3080, 4040, _lib.C_BIAS), (2048, 2048, 2048, _lib.C_OVERWRITE),
+             (264, 4104, 5000, _lib.C_ACCUMULATE)]
+    for m, k, n, mode in cases:
+        for ta in (False, True):
+            for tb in (False, True):
+                a = to_torch(randn(rng, (k, m) if ta else (m, k), dtype, 0.25), DEV, bf)
+                b = to_torch(randn(rng, (n, k) if tb else (k, n), dtype, 0.25), DEV, bf)
+                c0 = to_torch(randn(rng, (m, n), dtype), DEV, bf)
+                bias = to_torch(randn(rng, (n,), dtype), DEV, bf)
+
+                def run(ncols, out, ldc):
+                    d = _lib.GemmDesc()
+                    d.dtype, d.transpose_a, d.transpose_b, d.c_mode = F.ntg_dtype(a), int(ta), int(tb), mode
+                    d.m, d.k, d.n, d.batches = m, k, ncols, 1
+                    d.lda, d.ldb, d.ldc = (m if ta else k), (k if tb else n), ldc
+                    if mode == _lib.C_BIAS:
+                        d.bias, d.bias_col_stride = bias.data_ptr(), 1
+                    _lib.check(lib.ntg_gemm_dev(ctypes.byref(d), a.data_ptr(), b.data_ptr(), out.data_ptr(), st))
+
+                c = c0.clone()
+                run(n, c, n)
+                strip = c0[:, :64].contiguous()
+                run(64, strip, 64)
+                torch.cuda.synchronize()
+                what = f"{fmt} {m}x{k}x{n} ta={ta} tb={tb} mode={mode}"
+                assert torch.equal(c[:, :64].contiguous().view(torch.int16), strip.view(torch.int16)), what
+                al = (a.t() if ta else a).double()
+                bl = (b.t() if tb else b).double()
+                add = c0.double() if mode == _lib.C_ACCUMULATE else bias.double().expand(m, n) if mode == _lib.C_BIAS else torch.zeros(m, n, device=DEV, dtype=torch.float64)
+                ref = al @ bl + add
+                spread = add.abs() + ((al * al) @ (bl * bl)).sqrt()
+                # (Float16 at k = 4000: the float32 accumulation bound is a good part of an ulp, so fewer elements are clear of a boundary)
+                assert_one_rounding(c.double().cpu().numpy(), ref.cpu().numpy(), spread.cpu().numpy(), k, fmt, what, min_exact=0.75 if bf else 0.2)
