@@ -186,6 +186,8 @@ __device__ __forceinline__ uint32_t lds_addr_of(const char* p) {
 // fetched in whole 128-byte cache lines (half the requests to L2 of the 64-byte K-step) and the one barrier of a K-step
 // comes every sixteen MFMAs instead of every eight; the four stages are 32 KiB each (one workgroup per CU).  Fragments
 // are read two quarter-steps ahead (four sets in registers), the whole of tile kt + 3 is fetched during K-step kt.
+// With WBN_ = 4 (128 x 256 tiles) the stages are 48 KiB and there are three of them: tile kt + 2 is fetched from the
+// barrier of K-step kt - 1 (which frees its stage) to the barrier of K-step kt.
 template <int DT, bool TA, bool TB, bool RAGGED, int WB_, int CONV = 0, int WBN_ = 0, int KD_ = 1>
 __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
     using E = Elem<DT>;
@@ -195,7 +197,8 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
     constexpr int WB = WBN;                              // (the gathered operand is B; gathering kernels have square tiles)
     static_assert(CONV == 0 || WBM == WBN, "gathering kernels have square tiles");
     constexpr int KD = KD_;
-    static_assert(KD == 1 || (KD == 2 && CONV == 0 && ES == 2 && WB_ == 2 && WBN_ == 0), "deep K-steps: 16-bit plain products on 128 x 128 tiles");
+    static_assert(KD == 1 || (KD == 2 && CONV == 0 && ES == 2 && WB_ == 2 && (WBN_ == 0 || WBN_ == 4)), "deep K-steps: 16-bit plain products on 128 x 128 and 128 x 256 tiles");
+    constexpr bool RING3 = KD == 2 && WBN_ == 4;         // three stages of 48 KiB
     using GA = RingGeom<WBM, ES, KD>;                    // geometry of the A tile
     using G = RingGeom<WBN, ES, KD>;                     // geometry of the B tile
     constexpr int A_TILE_BYTES = GA::TILE_BYTES, STAGE_BYTES = GA::TILE_BYTES + G::TILE_BYTES;
@@ -217,7 +220,7 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
     __shared__ __attribute__((aligned(1024))) char st0[STAGE_BYTES];
     __shared__ __attribute__((aligned(1024))) char st1[STAGE_BYTES];
     __shared__ __attribute__((aligned(1024))) char st2[STAGE_BYTES];
-    __shared__ __attribute__((aligned(1024))) char st3[STAGE_BYTES];
+    __shared__ __attribute__((aligned(1024))) char st3[RING3 ? 1024 : STAGE_BYTES];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -603,9 +606,20 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
     b_tile(0, lds_addr_of(st0) + A_TILE_BYTES);
     dma_tile<NA>(srcA(1), 1 >= last ? offAt : offA, lds_addr_of(st1), wave_u);
     b_tile(1, lds_addr_of(st1) + A_TILE_BYTES);
-    dma_tile<NA>(srcA(2), 2 >= last ? offAt : offA, lds_addr_of(st2), wave_u);
-    b_tile(2, lds_addr_of(st2) + A_TILE_BYTES);
-    if constexpr (KD == 1) dma_tile<NA>(srcA(3), 3 >= last ? offAt : offA, lds_addr_of(st3), wave_u);
+    // instruction y (A's first, then B's) of this wavefront's share of tile kt, into the stage at lds_stage
+    auto tile_dma = [&](int y, int kt, uint32_t lds_stage) __attribute__((always_inline)) {
+        const bool tail = RAGGED && kt >= last;
+        if (y < NA) dma_1k(srcA(kt), tail ? offAt[y] : offA[y], lds_stage + (uint32_t)(wave_u * NA + y) * 1024u);
+        else dma_1k(srcB(kt), tail ? offBt[y - NA] : offB[y - NA], lds_stage + A_TILE_BYTES + (uint32_t)(wave_u * NB + y - NA) * 1024u);
+    };
+    if constexpr (RING3) {
+#pragma unroll
+        for (int y = 0; y < (NA + NB) / 2; ++y) tile_dma(y, 2, lds_addr_of(st2));     // first half of tile 2
+    } else {
+        dma_tile<NA>(srcA(2), 2 >= last ? offAt : offA, lds_addr_of(st2), wave_u);
+        b_tile(2, lds_addr_of(st2) + A_TILE_BYTES);
+        if constexpr (KD == 1) dma_tile<NA>(srcA(3), 3 >= last ? offAt : offA, lds_addr_of(st3), wave_u);
+    }
 
     constexpr int NBUF = 2 * KD;
     u32x4 af[NBUF][WBM], bf[NBUF][WBN];   // fragment sets: [half-step parity][block]; deep K-steps: [quarter-step][block]
@@ -668,7 +682,7 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
     };
 
     // tile 0 must have landed before its first fragments are read
-    NTG_WAIT_VMCNT(2 * (NA + NB) + (KD == 1 ? NA : 0));
+    NTG_WAIT_VMCNT(RING3 ? (NA + NB) + (NA + NB) / 2 : 2 * (NA + NB) + (KD == 1 ? NA : 0));
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
     load_frags(st0, 0, 0);
@@ -766,6 +780,39 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
       }
     };
 
+    // ... with three stages: `prv` (tile kt - 1's) takes the second half of tile kt + 2 during quarter-steps 0 and 1, `cur` the
+    // first half of tile kt + 3 after the barrier.  Tile kt + 1 has landed at the barrier when at most the instructions of
+    // tile kt + 2 are outstanding.
+    auto iteration_deep3 = [&](int kt, char* cur, const char* nxt, char* prv) __attribute__((always_inline)) {
+      if constexpr (RING3) {
+        static_assert((NA + NB) % 4 == 0, "a quarter of the tile's DMA instructions per quarter-step");
+        constexpr int PER = (NA + NB) / 4;
+        const bool lastk = RAGGED && kt == last && kr < BK;
+        const uint32_t lds_prv = lds_addr_of(prv), lds_cur = lds_addr_of(cur);
+        using NP = std::integral_constant<int, PER>;
+        using N0 = std::integral_constant<int, 0>;
+        if (lastk) mask_tail(0, 0);
+        mma_step_prefetch(0, cur, 2, 2, NP{}, N0{}, [&](int x) __attribute__((always_inline)) { tile_dma(2 * PER + x, kt + 2, lds_prv); });
+        if (lastk) mask_tail(1, 1);
+        mma_step_prefetch(1, cur, 3, 3, NP{}, N0{}, [&](int x) __attribute__((always_inline)) { tile_dma(3 * PER + x, kt + 2, lds_prv); });
+        NTG_WAIT_VMCNT(NA + NB);
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // my reads of `cur` are complete
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        if (lastk) mask_tail(2, 2);
+        mma_step_prefetch(2, nxt, 0, 0, NP{}, N0{}, [&](int x) __attribute__((always_inline)) { tile_dma(x, kt + 3, lds_cur); });
+        if (lastk) mask_tail(3, 3);
+        mma_step_prefetch(3, nxt, 1, 1, NP{}, N0{}, [&](int x) __attribute__((always_inline)) { tile_dma(PER + x, kt + 3, lds_cur); });
+      }
+    };
+
+    if constexpr (RING3) {
+        for (int kt = 0; kt < KT; kt += 3) {
+            iteration_deep3(kt, st0, st1, st2);
+            if (kt + 1 < KT) iteration_deep3(kt + 1, st1, st2, st0);
+            if (kt + 2 < KT) iteration_deep3(kt + 2, st2, st0, st1);
+        }
+    } else
     for (int kt = 0; kt < KT; kt += 4) {
         if constexpr (KD == 2) {
             iteration_deep(kt, st0, st1, st3);
@@ -789,7 +836,9 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
     // read-back moves RPS rows.
     constexpr int SROW = WTN * 4, LPR = WTN / 8, RPS = 64 / LPR, NSTEP = 32 / RPS;
     // (two slabs fit into one stage unless the tile is wider than tall: then every wavefront takes a stage of its own)
-    char* slab = WBN > WBM ? (wave == 0 ? st0 : wave == 1 ? st1 : wave == 2 ? st2 : st3)
+    // (three stages of 48 KiB: three 16-KiB slabs in the first, the fourth in the second)
+    char* slab = RING3 ? (wave == 3 ? st1 : st0 + wave * (32 * SROW))
+               : WBN > WBM ? (wave == 0 ? st0 : wave == 1 ? st1 : wave == 2 ? st2 : st3)
                            : ((wave & 2) ? st1 : st0) + (wave & 1) * (32 * SROW);
     char* Cb = reinterpret_cast<char*>(C);
     const int col = 8 * (lane % LPR);              // this lane's 8 consecutive columns in the slab
@@ -1114,7 +1163,7 @@ static hipError_t launch_ring16(bool ta, bool tb, const GemmParams& p, hipStream
     auto launch = [&](int te, const GemmParams& q) {
         if (te == 256) return launch_ring_wb<DT, 4>(ta, tb, q, s);
         if (te == 224) return launch_ring_wb<DT, 3, 4>(ta, tb, q, s);      // 192 rows x 256 columns
-        if (te == 192) return launch_ring_wb<DT, 2, 4>(ta, tb, q, s);      // 128 rows x 256 columns
+        if (te == 192) return launch_ring_wb<DT, 2, 4, 2>(ta, tb, q, s);   // 128 rows x 256 columns, deep K-steps
         if (te == 64) return launch_ring_wb<DT, 1>(ta, tb, q, s);
         // 128 x 128: the deep K-step unless many tiles with a short k queue up on every CU (see ring16_deep128)
         if (ring16_deep128(ring16_tiles(128, q.M, q.N, q.batch), q.K)) return launch_ring_wb<DT, 2, 0, 2>(ta, tb, q, s);

@@ -941,7 +941,7 @@ def test_batched_16bit_products_split_along_the_columns(dtype):
 
 @pytest.mark.parametrize("dtype", ["bf16", np.float16], ids=["bf16", "fp16"])
 def test_16bit_products_on_deep_k_steps(dtype):
-    """Mid-sized 16-bit products (up to 256 tiles of 128 x 128, or a deep k) run on the kernel whose K-step is 128 bytes of
+    """Mid-sized 16-bit products (128 x 128 and 128 x 256 tiles) run on the kernels whose K-step is 128 bytes of
     k per row.  All four storage forms, edges that are not multiples of the tile, k that is not a multiple of the 64-element
     K-step (tails of 8 and 40), overwrite / accumulate / bias: every element is the once-rounded exact result (within the
     float32 accumulation bound), and a strip of 64 columns computed as a product of its own -- on 64 x 64 tiles, 64-byte
@@ -952,8 +952,9 @@ def test_16bit_products_on_deep_k_steps(dtype):
     lib = _lib.load()
     st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
     rng = np.random.default_rng(6464)
+    # (the last two take 128 x 256 tiles: three stages of 48 KiB)
     cases = [(1536, 4136, 1528, _lib.C_ACCUMULATE), (776, 3080, 4040, _lib.C_BIAS), (2048, 2048, 2048, _lib.C_OVERWRITE),
-             (264, 4104, 5000, _lib.C_ACCUMULATE)]
+             (264, 4104, 5000, _lib.C_ACCUMULATE), (2304, 2312, 2296, _lib.C_BIAS), (520, 4104, 11000, _lib.C_ACCUMULATE)]
     for m, k, n, mode in cases:
         for ta in (False, True):
             for tb in (False, True):
