@@ -15,8 +15,10 @@ hipError_t launch_gemm_mfma_i8(int dtype, bool ta, bool tb, const GemmParams& p,
     auto launch = [&](int te, const GemmParams& q) {
         if (te == 256) return launch_ring_wb<DT_I8, 4>(ta, tb, q, s);
         if (te == 224) return tb ? launch_ring_cfg<DT_I8, false, true, 3, 4>(q, s) : launch_ring_cfg<DT_I8, false, false, 3, 4>(q, s);
-        if (te == 192) return launch_ring_wb<DT_I8, 2, 4>(ta, tb, q, s);
+        if (te == 192) return launch_ring_wb<DT_I8, 2, 4, 2>(ta, tb, q, s);     // (128-byte K-steps, as for the 16-bit products)
         if (te == 64) return launch_ring_wb<DT_I8, 1>(ta, tb, q, s);
+        // (k in 16-bit elements: the same number of K-steps)
+        if (ring16_deep128(ring16_tiles(128, q.M, q.N, q.batch), q.K / 2)) return launch_ring_wb<DT_I8, 2, 0, 2>(ta, tb, q, s);
         return launch_ring_wb<DT_I8, 2>(ta, tb, q, s);
     };
     if (p.batch == 1 && p.cmode != C_PARTIAL) {

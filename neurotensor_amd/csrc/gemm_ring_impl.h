@@ -197,7 +197,7 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
     constexpr int WB = WBN;                              // (the gathered operand is B; gathering kernels have square tiles)
     static_assert(CONV == 0 || WBM == WBN, "gathering kernels have square tiles");
     constexpr int KD = KD_;
-    static_assert(KD == 1 || (KD == 2 && CONV == 0 && ES == 2 && WB_ == 2 && (WBN_ == 0 || WBN_ == 4)), "deep K-steps: 16-bit plain products on 128 x 128 and 128 x 256 tiles");
+    static_assert(KD == 1 || (KD == 2 && CONV == 0 && (ES == 2 || ES == 1) && WB_ == 2 && (WBN_ == 0 || WBN_ == 4)), "deep K-steps: 16- and 8-bit plain products on 128 x 128 and 128 x 256 tiles");
     constexpr bool RING3 = KD == 2 && WBN_ == 4;         // three stages of 48 KiB
     using GA = RingGeom<WBM, ES, KD>;                    // geometry of the A tile
     using G = RingGeom<WBN, ES, KD>;                     // geometry of the B tile
