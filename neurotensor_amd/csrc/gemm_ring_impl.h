@@ -20,6 +20,9 @@
 //     per K-step, placed between its two halves; the DMA instructions and the LDS
 //     fragment reads are slotted between the MFMAs one at a time, so neither the CU's single
 //     address unit nor LDS latency ever holds up the matrix pipe.
+//   * 16- and 8-bit plain products on 128 x 128 and 128 x 256 tiles take K-steps of 128 bytes of k per row instead (KD = 2
+//     of the kernel template: whole cache lines of a K-contiguous operand, one barrier per sixteen MFMAs, fragments read
+//     two quarter-steps ahead; four stages of 32 KiB or three of 48 KiB, one workgroup per CU).  Same order of summation.
 //   * LDS layouts are conflict free for the reads the MFMA operands need:
 //       operand stored K-contiguous  -> [row][64 B of k], 16-byte slot kv stored at
 //                                        kv ^ ((row >> 1) & 3); one ds_read_b128 per block;
