@@ -302,7 +302,14 @@ hipError_t launch_reduce_batch(int dtype, const void* part, void* out, int64_t b
 // Where the pixels of a channels-last copy go when the copy carries a border of zero pixels: pixel (h, w) of a W-wide image is
 // pixel (h + top) * Wp + (w + left) of a padded image of Hp x Wp pixels.  nullptr / Wp == 0: no border.
 struct HaloMap { int64_t W, H, Wp, Hp, top, left; };
-hipError_t launch_nchw_to_nhwc(int64_t elem_size, const void* in, void* out, int64_t batch, int64_t C, int64_t P, hipStream_t s, const HaloMap* halo = nullptr);
+// A weight permutation that the launch of a channels-last copy can take along (its blocks share the elements after
+// their tiles): kind 1 = launch_weights_channels_last(w, wp, rows = a, cg, cgp, taps, chunk), kind 2 =
+// launch_flip_weights_channels_last(w, wp, groups = a, og, ogp, cg, taps, chunk).
+struct WeightsJob { int kind; const void* w; void* wp; int64_t a, og, ogp, cg, cgp, taps, chunk; };
+// With `halo`, pixels go to their places inside the bordered copy.  When the 16-byte kernel serves the copy it also zeroes
+// the border and runs `job` in the same launch and sets *took_along; otherwise the caller launches those two itself.
+hipError_t launch_nchw_to_nhwc(int64_t elem_size, const void* in, void* out, int64_t batch, int64_t C, int64_t P, hipStream_t s, const HaloMap* halo = nullptr,
+                               const WeightsJob* job = nullptr, bool* took_along = nullptr);
 hipError_t launch_halo_zero(int64_t elem_size, void* out, int64_t batch, int64_t C, const HaloMap& halo, hipStream_t s);   // zeros the border pixels
 hipError_t launch_weights_channels_last(int64_t es, const void* w, void* wp, int64_t rows, int64_t cg, int64_t cgp, int64_t taps, hipStream_t s, int64_t chunk = 0);
 hipError_t launch_weights_channels_last_rows(int64_t es, const void* w, void* wp, int64_t rows, int64_t cg, int64_t cgp, int64_t k_r, int64_t k_c,

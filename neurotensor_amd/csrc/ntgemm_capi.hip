@@ -973,15 +973,19 @@ static int conv_forward_nhwc(int dtype, const void* image, const void* kernel, v
     char* ws_img = static_cast<char*>(ws);
     char* ws_w = ws_img + align_up((size_t)(batch * chp * volp * es), 256);
     const ntg::HaloMap* hm = halo.on ? &halo.hm : nullptr;
-    hipError_t e = cgp == cg ? ntg::launch_nchw_to_nhwc(es, image, ws_img, batch, channels, vol, hs, hm)
+    // (the 16-byte copy kernel zeroes the border and permutes the weights in the same launch)
+    const int64_t wchunk = tap_inner ? 64 / es : 0;                              // (taps inside a 64-byte run of channels)
+    const ntg::WeightsJob wjob = {mt ? 0 : 1, kernel, ws_w, out_channels, 0, 0, cg, cgp, taps, wchunk};
+    bool took_along = false;
+    hipError_t e = cgp == cg ? ntg::launch_nchw_to_nhwc(es, image, ws_img, batch, channels, vol, hs, hm, &wjob, &took_along)
                              : ntg::launch_nchw_to_nhwc_padded(es, image, ws_img, batch, groups, cg, cgp, vol, hs, hm);
     if (e != hipSuccess) return hip_fail(e, "channels-last copy launch");
-    if (halo.on && volp != vol) {
+    if (halo.on && volp != vol && !took_along) {
         e = ntg::launch_halo_zero(es, ws_img, batch, chp, halo.hm, hs);
         if (e != hipSuccess) return hip_fail(e, "border fill launch");
     }
-    e = mt ? ntg::launch_weights_channels_last_rows(es, kernel, ws_w, out_channels, cg, cgp, g.k[1], g.k[2], mt->kq_pad, hs)
-           : ntg::launch_weights_channels_last(es, kernel, ws_w, out_channels, cg, cgp, taps, hs, tap_inner ? 64 / es : 0);      // (taps inside a 64-byte run of channels)
+    if (mt) e = ntg::launch_weights_channels_last_rows(es, kernel, ws_w, out_channels, cg, cgp, g.k[1], g.k[2], mt->kq_pad, hs);
+    else if (!took_along) e = ntg::launch_weights_channels_last(es, kernel, ws_w, out_channels, cg, cgp, taps, hs, wchunk);
     if (e != hipSuccess) return hip_fail(e, "weight permutation launch");
     for (int64_t gi = 0; gi < groups; ++gi) {
         ntg::GemmParams p;
@@ -1080,14 +1084,17 @@ static int conv_dimage_nhwc(int dtype, const void* kernel, const void* grad_out,
     char* ws_gy = static_cast<char*>(ws);
     char* ws_w = ws_gy + align_up((size_t)(batch * ochp * Lp * es), 256);
     const ntg::HaloMap* hm = halo.on ? &halo.hm : nullptr;
-    hipError_t e = ogp == og ? ntg::launch_nchw_to_nhwc(es, grad_out, ws_gy, batch, out_channels, L, hs, hm)
+    const int64_t wchunk = tap_inner ? 64 / es : 0;
+    const ntg::WeightsJob wjob = {2, kernel, ws_w, groups, og, ogp, cg, 0, taps, wchunk};
+    bool took_along = false;                                                    // (border and weight flip inside the copy's launch)
+    hipError_t e = ogp == og ? ntg::launch_nchw_to_nhwc(es, grad_out, ws_gy, batch, out_channels, L, hs, hm, &wjob, &took_along)
                              : ntg::launch_nchw_to_nhwc_padded(es, grad_out, ws_gy, batch, groups, og, ogp, L, hs, hm);
     if (e != hipSuccess) return hip_fail(e, "channels-last copy launch");
-    if (halo.on && Lp != L) {
+    if (halo.on && Lp != L && !took_along) {
         e = ntg::launch_halo_zero(es, ws_gy, batch, ochp, halo.hm, hs);
         if (e != hipSuccess) return hip_fail(e, "border fill launch");
     }
-    e = ntg::launch_flip_weights_channels_last(es, kernel, ws_w, groups, og, ogp, cg, taps, hs, tap_inner ? 64 / es : 0);
+    if (!took_along) e = ntg::launch_flip_weights_channels_last(es, kernel, ws_w, groups, og, ogp, cg, taps, hs, wchunk);
     if (e != hipSuccess) return hip_fail(e, "weight flip launch");
     for (int64_t gi = 0; gi < groups; ++gi) {
         ntg::GemmParams p;

@@ -4,6 +4,7 @@
 #include "ntg_common.h"
 
 #include <algorithm>
+#include <cstring>
 
 namespace ntg {
 
@@ -291,10 +292,11 @@ static PixRemap make_remap(const HaloMap* h, int64_t P) {
 // zeros the border pixels of a channels-last copy [B][Hp * Wp][C] (16-byte pieces; C * sizeof(T) a multiple of 16).
 // Only the border is visited: its pixels are numbered top rows, bottom rows, then the left and right pieces of the
 // image's rows.
-__global__ void __launch_bounds__(256) halo_zero_kernel(uint4* __restrict__ out, const uint32_t per_image, const uint32_t vec_per_pixel, const HaloMap h) {
+// (vectors first, first + step, ... of the per_image 16-byte vectors of one image's border)
+__device__ __forceinline__ void zero_border_vectors(uint4* __restrict__ img, const uint32_t per_image, const uint32_t vec_per_pixel, const HaloMap& h,
+                                                    const uint32_t first, const uint32_t step) {
     const uint32_t top_n = (uint32_t)(h.top * h.Wp), bot_n = (uint32_t)((h.Hp - h.top - h.H) * h.Wp), side = (uint32_t)(h.Wp - h.W);
-    uint4* img = out + (int64_t)blockIdx.y * (h.Hp * h.Wp) * vec_per_pixel;
-    for (uint32_t i = blockIdx.x * 256u + threadIdx.x; i < per_image; i += gridDim.x * 256u) {
+    for (uint32_t i = first; i < per_image; i += step) {
         uint32_t j = i / vec_per_pixel, pix;
         const uint32_t v = i - j * vec_per_pixel;
         if (j < top_n) pix = j;
@@ -306,6 +308,9 @@ __global__ void __launch_bounds__(256) halo_zero_kernel(uint4* __restrict__ out,
         }
         img[(int64_t)pix * vec_per_pixel + v] = make_uint4(0u, 0u, 0u, 0u);
     }
+}
+__global__ void __launch_bounds__(256) halo_zero_kernel(uint4* __restrict__ out, const uint32_t per_image, const uint32_t vec_per_pixel, const HaloMap h) {
+    zero_border_vectors(out + (int64_t)blockIdx.y * (h.Hp * h.Wp) * vec_per_pixel, per_image, vec_per_pixel, h, blockIdx.x * 256u + threadIdx.x, gridDim.x * 256u);
 }
 hipError_t launch_halo_zero(int64_t es, void* out, int64_t batch, int64_t C, const HaloMap& h, hipStream_t s) {
     if ((C * es) % 16 != 0 || (reinterpret_cast<uintptr_t>(out) & 15) != 0) return hipErrorInvalidValue;
@@ -341,11 +346,39 @@ __global__ void __launch_bounds__(256) nchw_to_nhwc_kernel(const T* __restrict__
     }
 }
 
+// element idx of the two weight permutations (see weights_channels_last_kernel, flip_weights_channels_last_kernel)
+template <class T>
+__device__ __forceinline__ void weights_channels_last_elem(const T* __restrict__ w, T* __restrict__ wp, const int64_t idx, const int64_t cg, const int64_t cgp,
+                                                           const int64_t taps, const int64_t chunk) {
+    const int64_t c = idx % cgp;
+    const int64_t t = (idx / cgp) % taps;
+    const int64_t o = idx / (cgp * taps);
+    // chunk != 0: the k order (run of `chunk` channels, tap, channel inside the run) instead of (tap, channel)
+    const int64_t dst = chunk ? o * taps * cgp + ((c / chunk) * taps + t) * chunk + c % chunk : idx;
+    wp[dst] = c < cg ? w[(o * cg + c) * taps + t] : (T)0;
+}
+template <class T>
+__device__ __forceinline__ void flip_weights_channels_last_elem(const T* __restrict__ w, T* __restrict__ wt, const int64_t idx, const int64_t og, const int64_t ogp,
+                                                                const int64_t cg, const int64_t taps, const int64_t chunk) {
+    const int64_t oc = idx % ogp;
+    int64_t r = idx / ogp;
+    const int64_t t = r % taps;
+    r /= taps;
+    const int64_t c = r % cg;
+    const int64_t g = r / cg;
+    // chunk != 0: the k order (run of `chunk` out channels, tap, out channel inside the run) instead of (tap, out channel)
+    const int64_t dst = chunk ? r * taps * ogp + ((oc / chunk) * taps + t) * chunk + oc % chunk : idx;
+    wt[dst] = oc < og ? w[((g * og + oc) * cg + c) * taps + (taps - 1 - t)] : (T)0;
+}
+// what a channels-last copy takes along: the border of zero pixels of its own output and a weight permutation
+struct CopyExtras { HaloMap h; uint32_t border_vecs, vpp; WeightsJob job; int64_t job_total; };
+
 // The same copy with 16-byte accesses on both sides (C and P multiples of one 16-byte vector, aligned pointers): a
 // thread loads VEC pixels of one channel, the tile goes through LDS as single elements (row pitch chosen so that the
 // column-wise read-back spreads over the banks), and a thread stores VEC channels of one pixel.
 template <class T>
-__global__ void __launch_bounds__(256) nchw_to_nhwc_vec_kernel(const T* __restrict__ in, T* __restrict__ out, const int64_t C, const int64_t P, const PixRemap r) {
+__global__ void __launch_bounds__(256) nchw_to_nhwc_vec_kernel(const T* __restrict__ in, T* __restrict__ out, const int64_t C, const int64_t P, const PixRemap r,
+                                                               const CopyExtras ex) {
     constexpr int VEC = 16 / (int)sizeof(T), VPR = 64 / VEC;            // elements per vector, vectors per tile row
     constexpr int PITCH = sizeof(T) == 2 ? 66 : 65;                     // elements: 33 / 65 words
     typedef T TV __attribute__((ext_vector_type(VEC)));
@@ -373,25 +406,53 @@ __global__ void __launch_bounds__(256) nchw_to_nhwc_vec_kernel(const T* __restri
             *reinterpret_cast<TV*>(dst + remap_pixel(r, p0 + pp) * C + c0 + cv * VEC) = x;
         }
     }
+    // the blocks of an image share its border, all blocks of the launch the weight permutation (a few elements each)
+    const uint32_t per_image = gridDim.x * gridDim.y, bid = blockIdx.y * gridDim.x + blockIdx.x;
+    if (ex.border_vecs)
+        zero_border_vectors(reinterpret_cast<uint4*>(dst), ex.border_vecs, ex.vpp, ex.h, bid * 256u + threadIdx.x, per_image * 256u);
+    if (ex.job.kind) {
+        const int64_t step = (int64_t)gridDim.z * per_image * 256;
+        for (int64_t idx = ((int64_t)blockIdx.z * per_image + bid) * 256 + threadIdx.x; idx < ex.job_total; idx += step) {
+            if (ex.job.kind == 1) weights_channels_last_elem<T>((const T*)ex.job.w, (T*)ex.job.wp, idx, ex.job.cg, ex.job.cgp, ex.job.taps, ex.job.chunk);
+            else flip_weights_channels_last_elem<T>((const T*)ex.job.w, (T*)ex.job.wp, idx, ex.job.og, ex.job.ogp, ex.job.cg, ex.job.taps, ex.job.chunk);
+        }
+    }
 }
 
-hipError_t launch_nchw_to_nhwc(int64_t es, const void* in, void* out, int64_t batch, int64_t C, int64_t P, hipStream_t s, const HaloMap* halo) {
+hipError_t launch_nchw_to_nhwc(int64_t es, const void* in, void* out, int64_t batch, int64_t C, int64_t P, hipStream_t s, const HaloMap* halo,
+                               const WeightsJob* job, bool* took_along) {
+    if (took_along) *took_along = false;
     if (batch * C * P == 0) return hipSuccess;
     const PixRemap r = make_remap(halo, P);
     const int64_t gx = (P + 63) / 64, gy = (C + 63) / 64;
     if (gx > 0x7fffffffLL || gy > 65535) return hipErrorInvalidValue;
     const int64_t vec = 16 / es;
     const bool vec_ok = C % vec == 0 && P % vec == 0 && ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) & 15) == 0;
+    CopyExtras ex;
+    std::memset(&ex, 0, sizeof ex);
+    if (vec_ok && (es == 2 || es == 4) && took_along) {
+        // (the caller acts on *took_along: without it the copy stays what it was)
+        const int64_t vpp = C * es / 16, border = halo && halo->Wp ? halo->Hp * halo->Wp - halo->H * halo->W : 0;
+        if (border * vpp <= 0x7fffffffLL && (!halo || halo->Hp * halo->Wp <= 0x7fffffffLL)) {
+            if (border > 0) { ex.h = *halo; ex.border_vecs = (uint32_t)(border * vpp); ex.vpp = (uint32_t)vpp; }
+            if (job && job->kind) {
+                ex.job = *job;
+                ex.job_total = job->kind == 1 ? job->a * job->cgp * job->taps : job->a * job->ogp * job->cg * job->taps;
+            }
+            *took_along = true;
+        }
+    }
     for (int64_t b0 = 0; b0 < batch; b0 += 65535) {                    // (grid z limit)
         const int64_t nb = batch - b0 < 65535 ? batch - b0 : 65535;
         const dim3 g((unsigned)gx, (unsigned)gy, (unsigned)nb), t(256);
         const char* src = static_cast<const char*>(in) + b0 * C * P * es;
         char* dst = static_cast<char*>(out) + b0 * C * r.Pp * es;
-        if (es == 2 && vec_ok) hipLaunchKernelGGL(nchw_to_nhwc_vec_kernel<uint16_t>, g, t, 0, s, (const uint16_t*)src, (uint16_t*)dst, C, P, r);
-        else if (es == 4 && vec_ok) hipLaunchKernelGGL(nchw_to_nhwc_vec_kernel<uint32_t>, g, t, 0, s, (const uint32_t*)src, (uint32_t*)dst, C, P, r);
+        if (es == 2 && vec_ok) hipLaunchKernelGGL(nchw_to_nhwc_vec_kernel<uint16_t>, g, t, 0, s, (const uint16_t*)src, (uint16_t*)dst, C, P, r, ex);
+        else if (es == 4 && vec_ok) hipLaunchKernelGGL(nchw_to_nhwc_vec_kernel<uint32_t>, g, t, 0, s, (const uint32_t*)src, (uint32_t*)dst, C, P, r, ex);
         else if (es == 2) hipLaunchKernelGGL(nchw_to_nhwc_kernel<uint16_t>, g, t, 0, s, (const uint16_t*)src, (uint16_t*)dst, C, P, r);
         else if (es == 4) hipLaunchKernelGGL(nchw_to_nhwc_kernel<uint32_t>, g, t, 0, s, (const uint32_t*)src, (uint32_t*)dst, C, P, r);
         else return hipErrorInvalidValue;
+        ex.job.kind = 0;                                               // (the first launch has done the weights)
     }
     return hipGetLastError();
 }
@@ -405,17 +466,8 @@ __global__ void __launch_bounds__(256) flip_weights_channels_last_kernel(const T
                                                                          const int64_t chunk) {
     const int64_t total = groups * ogp * cg * taps;
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-    for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += stride) {
-        const int64_t oc = idx % ogp;
-        int64_t r = idx / ogp;
-        const int64_t t = r % taps;
-        r /= taps;
-        const int64_t c = r % cg;
-        const int64_t g = r / cg;
-        // chunk != 0: the k order (run of `chunk` out channels, tap, out channel inside the run) instead of (tap, out channel)
-        const int64_t dst = chunk ? r * taps * ogp + ((oc / chunk) * taps + t) * chunk + oc % chunk : idx;
-        wt[dst] = oc < og ? w[((g * og + oc) * cg + c) * taps + (taps - 1 - t)] : (T)0;
-    }
+    for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += stride)
+        flip_weights_channels_last_elem<T>(w, wt, idx, og, ogp, cg, taps, chunk);
 }
 
 hipError_t launch_flip_weights_channels_last(int64_t es, const void* w, void* wt, int64_t groups, int64_t og, int64_t ogp, int64_t cg, int64_t taps, hipStream_t s,
@@ -504,14 +556,8 @@ __global__ void __launch_bounds__(256) weights_channels_last_kernel(const T* __r
                                                                     const int64_t cg, const int64_t cgp, const int64_t taps, const int64_t chunk) {
     const int64_t total = rows * cgp * taps;
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-    for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += stride) {
-        const int64_t c = idx % cgp;
-        const int64_t t = (idx / cgp) % taps;
-        const int64_t o = idx / (cgp * taps);
-        // chunk != 0: the k order (run of `chunk` channels, tap, channel inside the run) instead of (tap, channel)
-        const int64_t dst = chunk ? o * taps * cgp + ((c / chunk) * taps + t) * chunk + c % chunk : idx;
-        wp[dst] = c < cg ? w[(o * cg + c) * taps + t] : (T)0;
-    }
+    for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += stride)
+        weights_channels_last_elem<T>(w, wp, idx, cg, cgp, taps, chunk);
 }
 
 hipError_t launch_weights_channels_last(int64_t es, const void* w, void* wp, int64_t rows, int64_t cg, int64_t cgp, int64_t taps, hipStream_t s, int64_t chunk) {
