@@ -986,3 +986,58 @@ def test_16bit_products_on_deep_k_steps(dtype):
                 spread = add.abs() + ((al * al) @ (bl * bl)).sqrt()
                 # (Float16 at k = 4000: the float32 accumulation bound is a good part of an ulp, so fewer elements are clear of a boundary)
                 assert_one_rounding(c.double().cpu().numpy(), ref.cpu().numpy(), spread.cpu().numpy(), k, fmt, what, min_exact=0.75 if bf else 0.2)
+
+
+def test_deep_k_steps_at_their_shortest_k():
+    """The tile choice puts products on the 128-byte K-step kernels from k = 304 on (128 x 256 tiles, a batch of two
+    2112 x 3840 outputs) and k = 536 (128 x 128 tiles): five to nine K-steps, so the loops end inside their first rounds
+    over the stages, with a k tail (304 = 4 x 64 + 48, 536 = 8 x 64 + 24).  BFloat16 against the once-rounded exact result
+    and, bit for bit, against a strip of 64 columns computed on 64 x 64 tiles; Int8 (k = 304 is two K-steps of 128 and a tail
+    of 48) against exact integer arithmetic."""
+    from util import assert_one_rounding
+    lib = _lib.load()
+    st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    rng = np.random.default_rng(304)
+    for batch, m, k, n in ((2, 2112, 304, 3840), (1, 576, 536, 3648)):
+        for ta, tb in ((False, False), (False, True), (True, False)):
+            a = to_torch(randn(rng, (batch, k, m) if ta else (batch, m, k), "bf16", 0.25), DEV, True)
+            b = to_torch(randn(rng, (batch, n, k) if tb else (batch, k, n), "bf16", 0.25), DEV, True)
+            c0 = to_torch(randn(rng, (batch, m, n), "bf16"), DEV, True)
+
+            def run(ncols, out, ldc):
+                d = _lib.GemmDesc()
+                d.dtype, d.transpose_a, d.transpose_b, d.c_mode = F.ntg_dtype(a), int(ta), int(tb), _lib.C_ACCUMULATE
+                d.m, d.k, d.n, d.batches = m, k, ncols, batch
+                d.lda, d.ldb, d.ldc = (m if ta else k), (k if tb else n), ldc
+                d.stride_a, d.stride_b, d.stride_c = m * k, k * n, m * ldc
+                _lib.check(lib.ntg_gemm_dev(ctypes.byref(d), a.data_ptr(), b.data_ptr(), out.data_ptr(), st))
+
+            c = c0.clone()
+            run(n, c, n)
+            strip = c0[:, :, :64].contiguous()
+            run(64, strip, 64)
+            torch.cuda.synchronize()
+            what = f"bf16 {batch}x{m}x{k}x{n} ta={ta} tb={tb}"
+            assert torch.equal(c[:, :, :64].contiguous().view(torch.int16), strip.view(torch.int16)), what
+            al = (a.transpose(1, 2) if ta else a).double()
+            bl = (b.transpose(1, 2) if tb else b).double()
+            ref = al @ bl + c0.double()
+            spread = c0.double().abs() + ((al * al) @ (bl * bl)).sqrt()
+            assert_one_rounding(c.double().cpu().numpy(), ref.cpu().numpy(), spread.cpu().numpy(), k, "bf16", what)
+    # Int8: the same batch, every value of the range, wrapping sums
+    batch, m, k, n = 2, 2112, 304, 3840
+    for tb in (False, True):
+        a = torch.randint(-128, 128, (batch, m, k), device=DEV, dtype=torch.int8)
+        b = torch.randint(-128, 128, (batch, n, k) if tb else (batch, k, n), device=DEV, dtype=torch.int8)
+        c0 = torch.randint(-128, 128, (batch, m, n), device=DEV, dtype=torch.int8)
+        c = c0.clone()
+        d = _lib.GemmDesc()
+        d.dtype, d.transpose_b, d.c_mode = F.ntg_dtype(a), int(tb), _lib.C_ACCUMULATE
+        d.m, d.k, d.n, d.batches = m, k, n, batch
+        d.stride_a, d.stride_b, d.stride_c = m * k, k * n, m * n
+        _lib.check(lib.ntg_gemm_dev(ctypes.byref(d), a.data_ptr(), b.data_ptr(), c.data_ptr(), st))
+        torch.cuda.synchronize()
+        bl = (b.transpose(1, 2) if tb else b).double()
+        exact = (a.double() @ bl + c0.double()).to(torch.int64)          # |sum| < 2^23: exact in float64
+        want = ((exact + 128) % 256 - 128).to(torch.int8)
+        assert torch.equal(c, want), ("int8", tb)
