@@ -107,10 +107,11 @@ static inline bool ring16_deep128(int64_t nt, int64_t K) { return nt <= 256 || K
 static inline double ring16_cost_us(int t, int64_t nt, int64_t K) {
     const double cu_flops_per_us = 9.77e6;                      // 2500 TFLOP/s over 256 CUs
     // (measured per-tile figures: fraction of the CU's MFMA peak in the K loop, and microseconds of prologue + epilogue;
-    //  the 64-byte K-step on 128 x 128 tiles is bound by the LDS of its CU whether one or two workgroups share it)
+    //  the 64-byte K-step on 128 x 128 tiles is bound by the LDS of its CU whether one or two workgroups share it; 64 x 64
+    //  tiles with a deep k on many CUs run at 0.15 - 0.19: 256 tiles at k = 4096 took 21 us)
     const bool deep = t == 128 && ring16_deep128(nt, K);
     const double f = t == 256 ? (nt >= 192 ? 0.5 : 0.64) : t == 224 || t == 192 ? (nt >= 192 ? 0.5 : 0.55)
-                   : t == 128 ? (deep ? (nt > 256 ? 0.45 : nt >= 192 ? 0.5 : 0.565) : 0.3) : 0.25;
+                   : t == 128 ? (deep ? (nt > 256 ? 0.45 : nt >= 192 ? 0.5 : 0.565) : 0.3) : (nt >= 96 && K >= 1536 ? 0.18 : 0.25);
     const double latency = t == 256 ? 3.0 : t == 224 ? 4.0 : t == 192 ? 5.0 : t == 128 ? (deep ? (nt >= 192 ? 7.0 : 4.0) : 1.5) : 0.6;
     const double area = (double)ring16_tile_rows(t) * ring16_tile_cols(t);
     return (double)((nt + 255) / 256) * (2.0 * area * (double)K / (cu_flops_per_us * f) + latency);

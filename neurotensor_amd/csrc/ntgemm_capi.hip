@@ -347,24 +347,23 @@ SplitPlan plan_splitk(const ntg::GemmParams& p, int dtype, bool ta) {
         // only the DMA-fed kernel writes fp32 partial sums: 16-byte rows everywhere
         if (p.K % 8 || p.N % 8 || (ta && p.M % 8) || p.lda % 8 || p.ldb % 8 || p.lda >= (1 << 22) || p.ldb >= (1 << 22)) return none;
         if ((reinterpret_cast<uintptr_t>(p.A) & 15) || (reinterpret_cast<uintptr_t>(p.B) & 15)) return none;
-        // The DMA-fed kernel at its 128 x 128 tile (larger problems fill the chip by themselves).  Measured on MI355X:
-        // a workgroup alone on its CU takes about 0.215 us per 32-wide K-step, n >= 2 sharing a CU about 0.26 n us;
-        // launching the reduction and writing/reading the fp32 partial sums costs about 6 us + 8 S M N bytes at 4 TB/s.
-        // Pick the S with the smallest estimate (S = 1: no split).
-        if (ntg::ring16_tile_edge(p.M, p.N, p.K, 1) == 256) return none;
-        const int64_t tiles = ((p.M + 127) / 128) * ((p.N + 127) / 128);
-        auto estimate_us = [&](int64_t sp) {
-            const int64_t per_cu = (tiles * sp + 255) / 256;
-            const double step = per_cu == 1 ? 0.215 : 0.26 * (double)per_cu;
-            const double second_pass = sp == 1 ? 0.0 : 6.0 + 8.0 * (double)sp * (double)p.M * (double)p.N / 4.0e6;
-            return (double)(p.K / sp / 32) * step + second_pass;
-        };
+        // Both sides from the tile estimate of the 16-bit kernels (ring16_cost_us): the product as it is, against S batched
+        // products over K / S (the tiles that the batched launch picks) plus the second pass, measured at about 4 us + the
+        // fp32 partial sums written and read (8 S M N bytes) at 4 TB/s.  A split has to win by 5 %.  On a sweep of 23
+        // shapes (64 .. 1024 rows, k 2048 .. 16384) the choice is the best measured S in 20 and within 5 % in two more
+        // (1024 x 4096 x 1024: no split, 20.9 us against 24.5; 64 x 8192 x 8192: two ranges, 26.9 us against 38.3).
+        const int rect = ntg::RECT_128 | ntg::RECT_192;
+        const int edge1 = ntg::ring16_tile_edge(p.M, p.N, p.K, 1, rect);
+        if (edge1 == 256) return none;                                // (larger problems fill the chip by themselves)
+        const double whole_us = ntg::ring16_cost_us(edge1, ntg::ring16_tiles(edge1, p.M, p.N, 1), p.K);
         int64_t best = 1;
-        double best_us = estimate_us(1);
+        double best_us = whole_us;
         for (int64_t sp = 2; sp <= 16; ++sp) {
             if (p.K % (sp * 32) != 0 || p.K / sp < 256) continue;
-            const double us = estimate_us(sp);
-            if (us < 0.9 * best_us) { best = sp; best_us = us; }      // a split must win clearly
+            const int edge = ntg::ring16_tile_edge(p.M, p.N, p.K / sp, sp, rect);
+            const double us = ntg::ring16_cost_us(edge, ntg::ring16_tiles(edge, p.M, p.N, sp), p.K / sp) + 4.0 +
+                              8.0 * (double)sp * (double)p.M * (double)p.N / 4.0e6;
+            if (us < 0.95 * whole_us && us < best_us) { best = sp; best_us = us; }
         }
         if (best == 1) return none;
         return SplitPlan{(int)best, p.K / best, best * (int64_t)p.M * p.N * 4};
