@@ -874,10 +874,11 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
                 }
             }
         }
-#pragma unroll
-        for (int i = 0; i < WBM; ++i) {
-            // C0 of the whole slab is requested before the LDS round trip
-            u32x4 c0[NSTEP][NV];
+        // C0 of a whole slab is requested one slab ahead: the loads of slab i + 1 are in flight while slab i goes through LDS
+        // and out to memory (the rows of two slabs are different rows of C, but the compiler cannot know that and would
+        // keep every load behind the stores before it).
+        u32x4 c0s[2][NSTEP][NV];
+        auto load_c0 = [&](int i, u32x4 (&c0)[NSTEP][NV]) __attribute__((always_inline)) {
             if constexpr (CM == C_ACCUMULATE) {
 #pragma unroll
                 for (int t = 0; t < NSTEP && c_rows_16; ++t) {
@@ -895,6 +896,12 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
                     }
                 }
             }
+        };
+        load_c0(0, c0s[0]);
+#pragma unroll
+        for (int i = 0; i < WBM; ++i) {
+            u32x4 (&c0)[NSTEP][NV] = c0s[i & 1];
+            if (i + 1 < WBM) load_c0(i + 1, c0s[(i + 1) & 1]);
             // lane holds rows m = 32 i + lane%32, cols 32 j + 8 rq + 4 (lane/32) + (0..3)
 #pragma unroll
             for (int j = 0; j < WBN; ++j)
