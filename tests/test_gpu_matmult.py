@@ -1041,3 +1041,27 @@ def test_deep_k_steps_at_their_shortest_k():
         exact = (a.double() @ bl + c0.double()).to(torch.int64)          # |sum| < 2^23: exact in float64
         want = ((exact + 128) % 256 - 128).to(torch.int8)
         assert torch.equal(c, want), ("int8", tb)
+
+
+def test_host_batch_bf16_pointer_tables_on_deep_k_steps():
+    """nt_matmult_batch with a mixed pattern of repeated pointers (pointer tables) at a size that takes the 128-byte
+    K-step kernels: every item has the bits of the same product run alone through nt_matmult (the reference's
+    batched == per-item invariant), and is the once-rounded exact result on a sample of rows."""
+    from util import assert_one_rounding
+    rng = np.random.default_rng(4242)
+    nb, m, k, n = 3, 1536, 4104, 1528
+    a = [randn(rng, (m, k), "bf16", 0.25) for _ in range(2)]
+    b = [randn(rng, (k, n), "bf16", 0.25) for _ in range(2)]
+    As, Bs = [a[0], a[1], a[0]], [b[0], b[0], b[1]]
+    C0 = [randn(rng, (m, n), "bf16") for _ in range(nb)]
+    got = [c.copy() for c in C0]
+    arr = ctypes.c_void_p * nb
+    lib = _lib.load()
+    _lib.check(lib.ntg_matmult_batch(_lib.BFLOAT16, arr(*[x.ctypes.data for x in As]), arr(*[x.ctypes.data for x in Bs]),
+                                     arr(*[x.ctypes.data for x in got]), nb, m, k, k, n, 0, 0))
+    rows = np.arange(0, m, 37)
+    for i in range(nb):
+        single = host_matmult(As[i], Bs[i], C0[i].copy(), m, k, n, False, False, _lib.BFLOAT16)
+        assert single.tobytes() == got[i].tobytes(), i
+        al, bl, cl = to_f64(As[i][rows], True), to_f64(Bs[i], True), to_f64(C0[i][rows], True)
+        assert_one_rounding(to_f64(got[i][rows], True), al @ bl + cl, np.abs(cl) + np.sqrt((al * al) @ (bl * bl)), k, "bf16", f"item {i}")
