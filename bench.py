@@ -46,6 +46,9 @@ def parse_args():
     ap.add_argument("--no-extras", action="store_true", help="only the headline workload")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only", default="", help="comma-separated extras entries to time alone (skips the headline and the CPU leg)")
+    ap.add_argument("--power", default="", help="comma-separated extras entries that are ALSO run back to back for --power-seconds while amd-smi is "
+                                                "sampled (average socket power, clocks): what the power manager does under each workload")
+    ap.add_argument("--power-seconds", type=float, default=2.5)
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 256 MiB device copy (known HBM traffic) so that counter runs "
                          "(rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE) can be scaled")
@@ -149,6 +152,76 @@ def main():
     N = 4096
     flops = 2.0 * N * N * N
     only = [x for x in args.only.split(",") if x]
+    power = [x for x in args.power.split(",") if x]
+
+    def smi_sample():
+        """One reading of amd-smi: socket power in W and the graphics clock in MHz averaged over the XCDs (None without the tool)."""
+        import subprocess
+        try:
+            txt = subprocess.run(["amd-smi", "metric", "--power", "--clock", "--json"], capture_output=True, text=True, timeout=10).stdout
+            data = json.loads(txt)
+            gpu = (data["gpu_data"] if isinstance(data, dict) else data)[0]
+        except Exception:
+            return None
+        out = {}
+        try:
+            out["power_w"] = float(gpu["power"]["socket_power"]["value"])
+        except (KeyError, TypeError, ValueError):
+            pass
+        clks = []
+        for key, val in gpu.get("clock", {}).items():
+            try:
+                if key.startswith("gfx_"):
+                    clks.append(float(val["clk"]["value"]))
+                elif key.startswith("mem_") and "mclk_mhz" not in out:
+                    out["mclk_mhz"] = float(val["clk"]["value"])
+            except (KeyError, TypeError, ValueError):
+                pass
+        if clks:
+            out["sclk_mhz"] = sum(clks) / len(clks)
+        return out or None
+
+    def power_run(fn, seconds):
+        """fn() back to back for `seconds` (launches queued a few milliseconds ahead) while a thread samples amd-smi;
+        the first 0.5 s of samples are dropped (clocks and the power average settling)."""
+        import threading
+        samples, stop = [], threading.Event()
+
+        def sampler():
+            t0 = time.perf_counter()
+            while not stop.is_set():
+                smp = smi_sample()
+                if smp and time.perf_counter() - t0 > 0.5:
+                    samples.append(smp)
+
+        th = threading.Thread(target=sampler, daemon=True)
+        fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        fn()
+        torch.cuda.synchronize()
+        per = max(time.perf_counter() - t0, 2e-5)
+        chunk = max(1, int(0.004 / per))
+        th.start()
+        n, t0 = 0, time.perf_counter()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        while time.perf_counter() - t0 < seconds:
+            for _ in range(chunk):
+                fn()
+            n += chunk
+            torch.cuda.synchronize()
+        e1.record()
+        torch.cuda.synchronize()
+        stop.set()
+        th.join(timeout=15)
+        res = {"launches": n, "ms_per_launch": round(e0.elapsed_time(e1) / n, 5), "smi_samples": len(samples)}
+        for key in ("power_w", "sclk_mhz", "mclk_mhz"):
+            vals = [smp[key] for smp in samples if key in smp]
+            if vals:
+                res[key + "_avg"] = round(sum(vals) / len(vals), 1)
+                res[key + "_max"] = round(max(vals), 1)
+        return res
 
     # Coming from idle the GPU runs its first 20-30 ms of work at lower clocks.  Every measurement (20 or more timed steps)
     # is therefore preceded by SETTLE_MS of back-to-back 4096^3 16-bit products -- the Float16 instantiation for every
@@ -239,6 +312,10 @@ def main():
             e = {"ms": round(ms, 5), "rate": round(rate, 2), "unit": unit, "timed_launches": st}
             if peak:
                 e["frac_of_peak"] = round(rate / peak, 4)
+            if name in power:
+                pw = power_run(fn, args.power_seconds)
+                pw["rate"] = round(work / (pw["ms_per_launch"] * 1e-3) / scale, 2)
+                e["sustained"] = pw
             extras[name] = e
             del fn
 
@@ -250,6 +327,21 @@ def main():
         # diagnostic: the same kernel on all-zero operands (no operand toggling: the clock stays higher) -- the difference to the
         # line above is what the power manager takes, not what the instruction stream costs
         run("c3_bf16_4096_zero_operands", G(torch.bfloat16, N, N, N, scale=0.0, mode=_lib.C_OVERWRITE), flops, PEAK_TFLOPS["bf16"])
+
+        # the same matrix instruction on operands that stay in registers (no LDS, no global memory in the loop; 256 workgroups
+        # of four wavefronts with the 256 x 256 tile's accumulator blocks): what the matrix pipes sustain on these operand
+        # values before any data movement -- the ceiling of a product kernel on such data
+        def mfma_only(scale):
+            def make():
+                ops = (torch.randn(_lib.DIAG_MFMA_OPERAND_BYTES // 2, device=dev) * scale).bfloat16()
+                sink = torch.empty(256 * 256, device=dev, dtype=torch.float32)
+                call = lambda: _lib.check(lib.ntg_diag_mfma_rate_dev(_lib.BFLOAT16, ops.data_ptr(), 100, 256, sink.data_ptr(), stream))
+                call.keep = (ops, sink)
+                return call
+            return make
+        mf = 256 * 100 * float(_lib.DIAG_MFMA_FLOPS_PER_PASS)
+        run("mfma_registers_only_bf16_random_operands", mfma_only(0.02), mf, PEAK_TFLOPS["bf16"])
+        run("mfma_registers_only_bf16_zero_operands", mfma_only(0.0), mf, PEAK_TFLOPS["bf16"])
         run("c3_fp32_4096", G(torch.float32, N, N, N), flops, PEAK_TFLOPS["fp32"])
         run("c3_fp64_4096", G(torch.float64, N, N, N), flops, PEAK_TFLOPS["fp64"])
         run("c1_fp32_512", G(torch.float32, 512, 512, 512), 2.0 * 512 ** 3, PEAK_TFLOPS["fp32"])

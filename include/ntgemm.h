@@ -216,6 +216,17 @@ int ntg_gemm_relu_dev(const ntg_gemm_desc* desc, const void* dA, const void* dB,
 #define NTG_NOALLOC_SCRATCH_BYTES (64ll << 20)
 int ntg_gemm_noalloc_dev(const ntg_gemm_desc* desc, const void* dA, const void* dB, void* dC, void* stream);
 
+/* Measurement aid with NO counterpart in the reference (bench.py reports it beside the headline): `iters` passes of the
+ * 16-bit product kernels' matrix instruction (v_mfma_f32_32x32x16, Float16 or BFloat16) on operand fragments that stay in
+ * registers -- no LDS and no global memory in the loop -- on `workgroups` workgroups of four wavefronts with the 4 x 4
+ * accumulator blocks of the 256 x 256 tile.  `operands`: NTG_DIAG_MFMA_OPERAND_BYTES bytes of 16-bit values in device memory
+ * (16-byte aligned), loaded once; `sink`: 256 floats per workgroup.  One pass of one workgroup is
+ * NTG_DIAG_MFMA_FLOPS_PER_PASS floating-point operations.  The rate depends on the operand VALUES (the clock falls as
+ * operand bits toggle): random against all-zero operands is what the figure is for. */
+#define NTG_DIAG_MFMA_OPERAND_BYTES (128 << 10)
+#define NTG_DIAG_MFMA_FLOPS_PER_PASS 8388608ll
+int ntg_diag_mfma_rate_dev(int dtype, const void* operands, int64_t iters, int64_t workgroups, float* sink, void* stream);
+
 /* nt_matmult_batch<T> with the pointer tables themselves in device memory. */
 int ntg_gemm_ptrs_dev(const ntg_gemm_desc* desc, const void* const* dA, const void* const* dB,
                       void* const* dC, void* stream);

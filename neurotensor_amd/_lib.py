@@ -18,6 +18,8 @@ BFLOAT16, UINT64 = 100, 101
 
 C_OVERWRITE, C_ACCUMULATE, C_BIAS = 0, 1, 2
 NOALLOC_SCRATCH_BYTES = 64 << 20      # NTG_NOALLOC_SCRATCH_BYTES
+DIAG_MFMA_OPERAND_BYTES = 128 << 10   # NTG_DIAG_MFMA_OPERAND_BYTES
+DIAG_MFMA_FLOPS_PER_PASS = 8388608    # NTG_DIAG_MFMA_FLOPS_PER_PASS
 
 STATUS_NAMES = {0: "NTG_OK", 1: "NTG_ERR_INVALID_ARGUMENT", 2: "NTG_ERR_UNSUPPORTED_DTYPE",
                 3: "NTG_ERR_DEVICE", 4: "NTG_ERR_OUT_OF_MEMORY", 5: "NTG_ERR_NO_DEVICE"}
@@ -65,6 +67,7 @@ SIGNATURES = {
     "ntg_gemm_noalloc_dev": (_ci, [ctypes.POINTER(GemmDesc), _vp, _vp, _vp, _vp]),
     "ntg_gemm_workspace_bytes": (_i64, [ctypes.POINTER(GemmDesc)]),
     "ntg_gemm_ptrs_dev": (_ci, [ctypes.POINTER(GemmDesc), _vp, _vp, _vp, _vp]),
+    "ntg_diag_mfma_rate_dev": (_ci, [_ci, _vp, _i64, _i64, _vp, _vp]),
     "ntg_unfold2d_dev": (_ci, [_ci, _vp, _vp] + [_i64] * 12 + [_vp]),
     "ntg_conv2d_workspace_bytes": (_i64, [_ci] + [_i64] * 12),
     "ntg_conv2d_forward_workspace_bytes": (_i64, [_ci] + [_i64] * 12),
