@@ -175,7 +175,14 @@ typedef struct ntg_gemm_desc {
     void* workspace;            /* optional device scratch, 256-byte aligned, ntg_gemm_workspace_bytes(desc) bytes: lets a   */
     int64_t workspace_bytes;    /* single product with few output tiles and a deep k be split along k (deterministic), and  */
                                 /* a large 16/32/64-bit integer product run as byte planes on the 8-bit matrix pipe (bit-exact) */
+    int64_t flags;              /* NTG_GEMM_* bits below; 0 for none */
 } ntg_gemm_desc;
+
+/* ntg_gemm_ptrs_dev only: the caller vouches that EVERY entry of the three pointer tables is a multiple of 16 bytes.  The
+ * tables live in device memory, so the library cannot look; with the vouch (and rows that are 16-byte multiples) a table
+ * batch runs on the DMA-fed kernels like its strided twin, without it on the register-staged ones.  An entry that breaks
+ * the promise makes the kernel read from a misaligned address (wrong results, not a fault). */
+#define NTG_GEMM_PTRS_ALIGNED16 1
 
 /* Bytes of workspace with which ntg_gemm_dev runs its faster form (0: there is none for this product): a split along k
  * for shapes such as [256, 8192] x [8192, 8192], or, for large Int16 / Int32 / Int64 products and their unsigned forms, the
@@ -206,13 +213,18 @@ int ntg_gemm_relu_dev(const ntg_gemm_desc* desc, const void* dA, const void* dB,
 /* ntg_gemm_dev for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
  * harnesses that forbid hipMalloc): it has NO counterpart in the reference.  Same arguments, results bit-identical to
  * ntg_gemm_dev called with a workspace of ntg_gemm_workspace_bytes(desc) bytes; desc->workspace and desc->workspace_bytes
- * are ignored.  The split along k and the byte-plane products of the wide integers keep their partial sums in a fixed
- * array of NTG_NOALLOC_SCRATCH_BYTES bytes that is part of the library's device code (every GPU the library runs on holds
- * its copy until the process ends); the call itself allocates and frees nothing.  A product whose workspace form needs
- * more than that is rejected with NTG_ERR_INVALID_ARGUMENT (use ntg_gemm_dev with your own workspace).  All calls on one
- * GPU share the array: calls that may overlap on one GPU (different streams, different threads) race; calls on one
- * stream are ordered and safe.  The first call on a device looks the array's address up (hipGetSymbolAddress): make
- * that call before a stream capture begins. */
+ * are ignored.  The split along k, the byte-plane products of the wide integers and the padded copies of unaligned 8- and
+ * 16-bit operands keep their intermediate data in a fixed array of NTG_NOALLOC_SCRATCH_BYTES bytes that is part of the
+ * library's device code (every GPU the library runs on holds its copy until the process ends); the call itself allocates and
+ * frees no memory.  A product whose workspace form needs more than that is rejected with NTG_ERR_INVALID_ARGUMENT: use
+ * ntg_gemm_dev with your own workspace, or -- it allocates nothing either -- ntg_gemm_dev with workspace = NULL, which runs
+ * the plain kernels (same integer results; a floating product that would have been split along k is then summed in one
+ * range, so its last bits may differ).  All calls on one GPU share the array.  Calls on one stream are ordered by the
+ * stream.  Calls on different streams or from different threads are ordered by the library: a call is enqueued as a whole
+ * (a mutex per GPU) and makes its stream wait for an event recorded behind the previous user's last kernel.  A stream under
+ * capture takes no part in that ordering (an event recorded inside a capture cannot be waited for from outside): graphs
+ * that contain such calls must not run while other users of the array are in flight.  The first call on a device looks the
+ * array's address up (hipGetSymbolAddress) and creates the event: make that call before a stream capture begins. */
 #define NTG_NOALLOC_SCRATCH_BYTES (64ll << 20)
 int ntg_gemm_noalloc_dev(const ntg_gemm_desc* desc, const void* dA, const void* dB, void* dC, void* stream);
 
@@ -227,7 +239,10 @@ int ntg_gemm_noalloc_dev(const ntg_gemm_desc* desc, const void* dA, const void* 
 #define NTG_DIAG_MFMA_FLOPS_PER_PASS 8388608ll
 int ntg_diag_mfma_rate_dev(int dtype, const void* operands, int64_t iters, int64_t workgroups, float* sink, void* stream);
 
-/* nt_matmult_batch<T> with the pointer tables themselves in device memory. */
+/* nt_matmult_batch<T> with the pointer tables themselves in device memory.  desc->workspace is not used: a table batch is
+ * never split along k, so an item whose single-product form ntg_gemm_workspace_bytes offers a split (the order of summation
+ * over k then differs) is, for bit-identical results alone and in a batch, better sent through ntg_gemm_dev item by item --
+ * what ntg_matmult_batch and the C++ facade do with such lists. */
 int ntg_gemm_ptrs_dev(const ntg_gemm_desc* desc, const void* const* dA, const void* const* dB,
                       void* const* dC, void* stream);
 

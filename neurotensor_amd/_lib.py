@@ -17,6 +17,7 @@ UINT8, UINT16, UINT32 = 12, 13, 14
 BFLOAT16, UINT64 = 100, 101
 
 C_OVERWRITE, C_ACCUMULATE, C_BIAS = 0, 1, 2
+GEMM_PTRS_ALIGNED16 = 1               # NTG_GEMM_PTRS_ALIGNED16
 NOALLOC_SCRATCH_BYTES = 64 << 20      # NTG_NOALLOC_SCRATCH_BYTES
 DIAG_MFMA_OPERAND_BYTES = 128 << 10   # NTG_DIAG_MFMA_OPERAND_BYTES
 DIAG_MFMA_FLOPS_PER_PASS = 8388608    # NTG_DIAG_MFMA_FLOPS_PER_PASS
@@ -35,6 +36,7 @@ class GemmDesc(ctypes.Structure):
         ("bias", ctypes.c_void_p),
         ("bias_batch_stride", ctypes.c_int64), ("bias_row_stride", ctypes.c_int64), ("bias_col_stride", ctypes.c_int64),
         ("workspace", ctypes.c_void_p), ("workspace_bytes", ctypes.c_int64),
+        ("flags", ctypes.c_int64),
     ]
 
 

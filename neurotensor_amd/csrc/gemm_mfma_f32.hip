@@ -14,7 +14,6 @@ static int ring_f32_tile_edge(const GemmParams& p) {
 }
 
 hipError_t launch_gemm_mfma_f32(bool ta, bool tb, const GemmParams& p, hipStream_t s) {
-    if (small32_f32_wins(p)) return launch_gemm_small32_f32(ta, tb, p, s);
     if (ring_eligible(p, ta, 4))
         return ring_f32_tile_edge(p) == 64 ? launch_ring_wb<DT_F32, 1>(ta, tb, p, s) : launch_ring_wb<DT_F32, 2>(ta, tb, p, s);
     // rows that are not 16-byte aligned (or pointer tables): register-staged kernel, 128 x 128 x 32 tiles unless that
@@ -24,10 +23,6 @@ hipError_t launch_gemm_mfma_f32(bool ta, bool tb, const GemmParams& p, hipStream
     return launch_trans<DT_F32, 1, 1, 32>(ta, tb, p, s);
 }
 hipError_t launch_gemm_ring_only_f32(bool ta, bool tb, const GemmParams& p, hipStream_t s, bool* taken) {
-    if (small32_f32_wins(p)) {             // (its epilogue applies GemmParams::act too)
-        *taken = true;
-        return launch_gemm_small32_f32(ta, tb, p, s);
-    }
     *taken = ring_eligible(p, ta, 4);
     if (!*taken) return hipSuccess;
     return ring_f32_tile_edge(p) == 64 ? launch_ring_wb<DT_F32, 1>(ta, tb, p, s) : launch_ring_wb<DT_F32, 2>(ta, tb, p, s);

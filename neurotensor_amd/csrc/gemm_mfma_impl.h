@@ -440,8 +440,8 @@ __global__ void __launch_bounds__(256) gemm_mfma_kernel(const GemmParams p) {
     tile_coords(lid - b * tiles, p.tiles_m, p.tiles_n, SH::GROUP_M, tm, tn);
     const int m0 = tm * BM, n0 = tn * BN;
 
-    const gptr<T> A = (gptr<T>)(p.Aptr ? static_cast<const T*>(((gptr<const void*>)p.Aptr)[b]) : static_cast<const T*>(p.A) + (int64_t)b * p.sA);
-    const gptr<T> B = (gptr<T>)(p.Bptr ? static_cast<const T*>(((gptr<const void*>)p.Bptr)[b]) : static_cast<const T*>(p.B) + (int64_t)b * p.sB);
+    const gptr<T> A = (gptr<T>)(p.Aptr ? static_cast<const T*>(((gptr<const void*>)p.Aptr)[b]) : static_cast<const T*>(p.A) + operand_offset(p, b, p.sA, p.sAk));
+    const gptr<T> B = (gptr<T>)(p.Bptr ? static_cast<const T*>(((gptr<const void*>)p.Bptr)[b]) : static_cast<const T*>(p.B) + operand_offset(p, b, p.sB, p.sBk));
     const gptr_mut<T> C = (gptr_mut<T>)(p.Cptr ? static_cast<T*>(((gptr<void*>)p.Cptr)[b]) : static_cast<T*>(p.C) + (int64_t)b * p.sC);
     const bool vecA = p.vecA_ok && ((reinterpret_cast<uintptr_t>(A) & 15) == 0);
     const bool vecB = p.vecB_ok && ((reinterpret_cast<uintptr_t>(B) & 15) == 0);

@@ -49,8 +49,8 @@ __global__ void __launch_bounds__(256) gemm_ring64_kernel(const GemmParams p) {
     tile_coords(lid - b * tiles, p.tiles_m, p.tiles_n, 8, tm, tn);
     const int m0 = tm * G::BM, n0 = tn * G::BN;
 
-    const double* A = p.Aptr ? static_cast<const double*>(p.Aptr[b]) : static_cast<const double*>(p.A) + (int64_t)b * p.sA;
-    const double* B = p.Bptr ? static_cast<const double*>(p.Bptr[b]) : static_cast<const double*>(p.B) + (int64_t)b * p.sB;
+    const double* A = p.Aptr ? static_cast<const double*>(p.Aptr[b]) : static_cast<const double*>(p.A) + operand_offset(p, b, p.sA, p.sAk);
+    const double* B = p.Bptr ? static_cast<const double*>(p.Bptr[b]) : static_cast<const double*>(p.B) + operand_offset(p, b, p.sB, p.sBk);
     double* C = p.Cptr ? static_cast<double*>(p.Cptr[b]) : static_cast<double*>(p.C) + (int64_t)b * p.sC;
 
     const int wave_u = __builtin_amdgcn_readfirstlane(wave);

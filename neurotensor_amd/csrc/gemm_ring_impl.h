@@ -238,8 +238,8 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
     const int m0 = tm * GA::BM, n0 = tn * G::BN;
 
     // (pointer tables: one uniform load per operand; everything below is base + offset either way)
-    const T* A = p.Aptr ? static_cast<const T*>(p.Aptr[b]) : static_cast<const T*>(p.A) + (int64_t)b * p.sA;
-    const T* B = p.Bptr ? static_cast<const T*>(p.Bptr[b]) : static_cast<const T*>(p.B) + (int64_t)b * p.sB;
+    const T* A = p.Aptr ? static_cast<const T*>(p.Aptr[b]) : static_cast<const T*>(p.A) + operand_offset(p, b, p.sA, p.sAk);
+    const T* B = p.Bptr ? static_cast<const T*>(p.Bptr[b]) : static_cast<const T*>(p.B) + operand_offset(p, b, p.sB, p.sBk);
     T* C = p.Cptr ? static_cast<T*>(p.Cptr[b]) : static_cast<T*>(p.C) + (int64_t)b * p.sC;
 
     // ---- DMA sources: uniform tile base (advances by adv bytes per K-step) + per-lane offsets ----

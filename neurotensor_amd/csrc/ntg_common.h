@@ -77,6 +77,10 @@ struct GemmParams {
     int64_t bias_bs, bias_rs, bias_cs;
     int64_t lda, ldb, ldc;   // row length of the stored matrices, in elements
     int64_t sA, sB, sC;      // batch strides in elements, 0 = the same matrix for every item
+    // A batch whose items are each split into k ranges (split-K of a batch): launch index b = range * krange_items + item,
+    // A and B of it lie at item * sA + range * sAk (sB, sBk); C (the partial sums) at b * sC.  0: a plain batch.
+    int krange_items;
+    int64_t sAk, sBk;
     int M, N, K, batch;      // logical sizes (after the transpose flags)
     int cmode;
     int tiles_m, tiles_n;
@@ -267,10 +271,6 @@ hipError_t launch_gemm_valu(int dtype, bool ta, bool tb, const GemmParams& p, hi
 hipError_t launch_gemm_mfma_i8(int dtype, bool ta, bool tb, const GemmParams& p, hipStream_t s);   // Int8 / UInt8: MFMA where rows are 16-byte multiples
 hipError_t launch_gemm_complex(int dtype, bool ta, bool tb, const GemmParams& p, hipStream_t s);   // Complex32 / 64 / 128: lane-wise products on (re, im) pairs
 hipError_t launch_gemm_skinny(int dtype, bool ta, bool tb, const GemmParams& p, hipStream_t s, bool* handled);
-// Float32 products with so few output elements that 64 x 64 tiles leave most CUs idle: 32 x 32 tiles, k split over the
-// four wavefronts of a workgroup (gemm_small.hip)
-bool small32_f32_wins(const GemmParams& p);
-hipError_t launch_gemm_small32_f32(bool ta, bool tb, const GemmParams& p, hipStream_t s);
 // op(B) is the im2col matrix of the image at p.B (tb: its transpose); floating dtypes only
 hipError_t launch_conv_mfma(int dtype, bool tb, const GemmParams& p, hipStream_t s);
 hipError_t launch_unfold2d(int64_t elem_size, const void* im, void* col,
@@ -358,6 +358,13 @@ static inline unsigned grid_for(int64_t total) {
 }
 
 #ifdef __HIPCC__
+// element offset of launch index b's A (stride = p.sA, kstride = p.sAk) or B operand
+__device__ __forceinline__ int64_t operand_offset(const GemmParams& p, int b, int64_t stride, int64_t kstride) {
+    if (p.krange_items == 0) return (int64_t)b * stride;
+    const int range = b / p.krange_items, item = b - range * p.krange_items;
+    return (int64_t)item * stride + (int64_t)range * kstride;
+}
+
 __device__ __forceinline__ uint32_t fast_div(uint32_t n, const FastDiv& f) {
     const uint32_t t = __umulhi(f.m, n);
     return (t + ((n - t) >> f.s1)) >> f.s2;

@@ -130,8 +130,8 @@ int reject_complex(int dtype, const char* what) {
 int launch_gemm(ntg::GemmParams p, int dtype, bool ta, bool tb, hipStream_t s) {
     const int64_t es = ntg::elem_size(dtype);
     const int64_t ve = 16 / es;
-    p.vecA_ok = (p.lda % ve == 0) && (p.Aptr || p.sA % ve == 0);
-    p.vecB_ok = (p.ldb % ve == 0) && (p.Bptr || p.sB % ve == 0);
+    p.vecA_ok = (p.lda % ve == 0) && (p.Aptr || p.sA % ve == 0) && (p.krange_items == 0 || p.sAk % ve == 0);
+    p.vecB_ok = (p.ldb % ve == 0) && (p.Bptr || p.sB % ve == 0) && (p.krange_items == 0 || p.sBk % ve == 0);
     hipError_t e;
     // relu_ on the result: inside the DMA-fed kernel's epilogue where that kernel serves the product (more than 32 rows: the
     // streaming kernels take the others), else as a pass over C after whichever kernel runs
@@ -177,10 +177,14 @@ int launch_gemm(ntg::GemmParams p, int dtype, bool ta, bool tb, hipStream_t s) {
     return finish();
 }
 
-// Split-K.  A single product whose output tiles cannot occupy the 256 CUs but whose K is deep (a Linear layer on a few
+// Split-K.  A product whose output tiles cannot occupy the 256 CUs but whose K is deep (a Linear layer on a few
 // hundred rows) is cut into `splits` equal k ranges, computed as one batched launch of the ordinary kernels into a
 // workspace [splits][M][N] (fp32 sums for the 16-bit dtypes, so nothing is rounded early), and added up in ascending
 // range order by a second kernel.  Deterministic; applied only when the caller supplies the workspace.
+// The plan is a function of ONE item's M, N, K (and dtype, flags, alignment) only, never of the batch count: a split
+// changes the order of summation over k, and an item must come out bit for bit the same alone and inside a batch
+// (the reference's batched == per-item rule, tests/src/matmult_test.cpp:108-189).  A batch whose items are split runs one
+// batched launch per k range into [splits][batch][M][N] and one reduction over all items.
 struct SplitPlan { int splits; int64_t kc; int64_t bytes; };
 
 // 16-, 32- and 64-bit integers on the 8-bit matrix pipe (byte planes, gemm_mfma_i8.hip): P (P + 1) / 2 8-bit products
@@ -340,13 +344,14 @@ static int run_padded(const ntg::GemmParams& p, const PadPlan& pl, int dtype, bo
 SplitPlan plan_splitk(const ntg::GemmParams& p, int dtype, bool ta) {
     SplitPlan none{1, p.K, 0};
     const int64_t es = ntg::elem_size(dtype);
-    if (is_valu_dtype(dtype) || es == 0 || p.batch != 1 || p.Aptr || p.Bptr || p.Cptr) return none;
+    if (is_valu_dtype(dtype) || es == 0 || p.batch < 1 || p.batch > 65535 || p.Aptr || p.Bptr || p.Cptr) return none;
     if (p.M <= 32 && dtype != ntg::DT_F64) return none;                       // the streaming kernels take these
     const bool half = dtype == ntg::DT_F16 || dtype == ntg::DT_BF16;
     if (half) {
         // only the DMA-fed kernel writes fp32 partial sums: 16-byte rows everywhere
         if (p.K % 8 || p.N % 8 || (ta && p.M % 8) || p.lda % 8 || p.ldb % 8 || p.lda >= (1 << 22) || p.ldb >= (1 << 22)) return none;
         if ((reinterpret_cast<uintptr_t>(p.A) & 15) || (reinterpret_cast<uintptr_t>(p.B) & 15)) return none;
+        if (p.batch > 1 && (p.sA % 8 || p.sB % 8)) return none;
         // Both sides from the tile estimate of the 16-bit kernels (ring16_cost_us): the product as it is, against S batched
         // products over K / S (the tiles that the batched launch picks) plus the second pass, measured at about 4 us + the
         // fp32 partial sums written and read (8 S M N bytes) at 4 TB/s.  A split has to win by 5 %.  On a sweep of 23
@@ -366,7 +371,7 @@ SplitPlan plan_splitk(const ntg::GemmParams& p, int dtype, bool ta) {
             if (us < 0.95 * whole_us && us < best_us) { best = sp; best_us = us; }
         }
         if (best == 1) return none;
-        return SplitPlan{(int)best, p.K / best, best * (int64_t)p.M * p.N * 4};
+        return SplitPlan{(int)best, p.K / best, best * (int64_t)p.batch * p.M * p.N * 4};
     }
     // fp32 / fp64: their kernels go down to 64 x 64 tiles by themselves; a split pays only when those leave CUs without a
     // tile.  Same kind of estimate: a CU spends about 14.4 ns (fp32) / 28.8 ns (fp64) per k on each 64 x 64 tile it is
@@ -386,7 +391,7 @@ SplitPlan plan_splitk(const ntg::GemmParams& p, int dtype, bool ta) {
         const double us = estimate_us(sp);
         if (us < 0.9 * best_us) { best = sp; best_us = us; }
     }
-    if (best > 1) return SplitPlan{(int)best, p.K / best, best * (int64_t)p.M * p.N * es};
+    if (best > 1) return SplitPlan{(int)best, p.K / best, best * (int64_t)p.batch * p.M * p.N * es};
     return none;
 }
 
@@ -429,17 +434,28 @@ int run_gemm(ntg::GemmParams p, int dtype, bool ta, bool tb, hipStream_t s, void
     if (plan.splits > 1 && workspace && workspace_bytes >= plan.bytes && (reinterpret_cast<uintptr_t>(workspace) & 15) == 0) {
         ntg::GemmParams q = p;
         q.K = (int)plan.kc;
-        q.batch = plan.splits;
-        q.sA = ta ? plan.kc * p.lda : plan.kc;
-        q.sB = tb ? plan.kc : plan.kc * p.ldb;
-        q.C = workspace;
         q.ldc = p.N;
         q.sC = (int64_t)p.M * p.N;
         q.cmode = (dtype == ntg::DT_F16 || dtype == ntg::DT_BF16) ? ntg::C_PARTIAL : ntg::C_OVERWRITE;
         q.bias = nullptr;
         q.act = ntg::ACT_NONE;                     // (the reduction applies it, after the last k range)
-        int rc = launch_gemm(q, dtype, ta, tb, s);
-        if (rc) return rc;
+        const int64_t step_a = (ta ? plan.kc * p.lda : plan.kc), step_b = (tb ? plan.kc : plan.kc * p.ldb);   // elements from one k range to the next
+        q.C = workspace;
+        q.batch = plan.splits * p.batch;
+        if (p.batch == 1) {
+            // the k ranges are the items of one batched launch
+            q.sA = step_a;
+            q.sB = step_b;
+        } else {
+            // ... range r of item i is launch index r * batch + i
+            q.krange_items = p.batch;
+            q.sAk = step_a;
+            q.sBk = step_b;
+        }
+        {
+            int rc = launch_gemm(q, dtype, ta, tb, s);
+            if (rc) return rc;
+        }
         hipError_t e = ntg::launch_splitk_reduce(dtype, workspace, plan.splits, p, s);
         if (e != hipSuccess) return hip_fail(e, "split-K reduction launch");
         return NTG_OK;
@@ -481,21 +497,34 @@ int desc_to_params(const ntg_gemm_desc* d, ntg::GemmParams& p) {
 // first call per device.  The function has external linkage on purpose: the compiler gives a file-scope static device
 // variable a symbol the runtime can look up only when a host function with external linkage refers to it.
 namespace ntg {
-int noalloc_scratch_of_current_device(void** out) {
+// One per GPU: the address of its copy of `scratch`, and what orders the users of that copy.  Calls that use the array are
+// enqueued one at a time (the mutex spans a call's whole sequence of launches); a call on another stream than the previous
+// user's first makes its stream wait for the event recorded behind that user's last kernel.  Streams under capture take no
+// part in this (an event recorded inside a capture cannot be waited for from outside): their callers order such calls themselves.
+struct NoallocState {
+    std::mutex mutex;
+    void* ptr = nullptr;
+    hipEvent_t done = nullptr;
+    hipStream_t last_stream = nullptr;
+    bool used = false;
+};
+int noalloc_state_of_current_device(NoallocState** out) {
     constexpr int kMaxDevices = 64;
-    static std::mutex mutex;
-    static void* ptrs[kMaxDevices];
+    static std::mutex setup_mutex;
+    static NoallocState states[kMaxDevices];
     int dev = -1;
     HIP_TRY(hipGetDevice(&dev));
     if (dev < 0 || dev >= kMaxDevices) return fail(NTG_ERR_DEVICE, "device ordinal %d outside 0..%d", dev, kMaxDevices - 1);
-    std::lock_guard<std::mutex> lock(mutex);
-    if (!ptrs[dev]) {
+    NoallocState& st = states[dev];
+    std::lock_guard<std::mutex> lock(setup_mutex);
+    if (!st.ptr) {
         void* ptr = nullptr;
         HIP_TRY(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
         if (!ptr) return fail(NTG_ERR_DEVICE, "hipGetSymbolAddress returned a null address for the static scratch");
-        ptrs[dev] = ptr;
+        HIP_TRY(hipEventCreateWithFlags(&st.done, hipEventDisableTiming));
+        st.ptr = ptr;
     }
-    *out = ptrs[dev];
+    *out = &st;
     return NTG_OK;
 }
 }  // namespace ntg
@@ -568,14 +597,30 @@ int ntg_gemm_noalloc_dev(const ntg_gemm_desc* d, const void* dA, const void* dB,
     if (need < 0) return fail(NTG_ERR_INVALID_ARGUMENT, "bad descriptor");
     if (need > (int64_t)NTG_NOALLOC_SCRATCH_BYTES)
         return fail(NTG_ERR_INVALID_ARGUMENT, "this product's workspace form needs %lld bytes, the static scratch of ntg_gemm_noalloc_dev holds %lld: "
-                    "call ntg_gemm_dev with a workspace of the caller's", (long long)need, (long long)NTG_NOALLOC_SCRATCH_BYTES);
-    void* ws = nullptr;
-    if (need > 0) {
-        rc = ntg::noalloc_scratch_of_current_device(&ws);
-        if (rc) return rc;
-    }
+                    "call ntg_gemm_dev with a workspace of the caller's, or ntg_gemm_dev without a workspace (the plain kernels: they allocate "
+                    "nothing either, but a split along k is then not taken and floating-point sums may differ in their last bits)",
+                    (long long)need, (long long)NTG_NOALLOC_SCRATCH_BYTES);
     p.A = dA; p.B = dB; p.C = dC;
-    return run_gemm(p, d->dtype, d->transpose_a != 0, d->transpose_b != 0, static_cast<hipStream_t>(stream), ws, need);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (need == 0) return run_gemm(p, d->dtype, d->transpose_a != 0, d->transpose_b != 0, s);      // the plain kernels: the array is not used
+    ntg::NoallocState* st = nullptr;
+    rc = ntg::noalloc_state_of_current_device(&st);
+    if (rc) return rc;
+    std::lock_guard<std::mutex> lock(st->mutex);
+    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(s, &capture) != hipSuccess) {      // (e.g. the default stream while another stream captures)
+        (void)hipGetLastError();
+        capture = hipStreamCaptureStatusActive;
+    }
+    const bool ordered = capture == hipStreamCaptureStatusNone;
+    if (ordered && st->used && st->last_stream != s) HIP_TRY(hipStreamWaitEvent(s, st->done, 0));     // the previous user of the array finishes first
+    rc = run_gemm(p, d->dtype, d->transpose_a != 0, d->transpose_b != 0, s, st->ptr, need);
+    if (ordered) {
+        HIP_TRY(hipEventRecord(st->done, s));
+        st->last_stream = s;
+        st->used = true;
+    }
+    return rc;
 }
 
 // aligned: the caller vouches that every table entry is a multiple of 16 bytes (true for the host entry points' own arena)
@@ -591,7 +636,8 @@ static int gemm_ptrs(const ntg_gemm_desc* d, const void* const* dA, const void* 
 }
 
 int ntg_gemm_ptrs_dev(const ntg_gemm_desc* d, const void* const* dA, const void* const* dB, void* const* dC, void* stream) {
-    return gemm_ptrs(d, dA, dB, dC, stream, false);     // (the tables are in device memory: their entries' alignment is unknown here)
+    // (the tables are in device memory: their entries' alignment is what the caller says it is)
+    return gemm_ptrs(d, dA, dB, dC, stream, d && (d->flags & NTG_GEMM_PTRS_ALIGNED16) != 0);
 }
 
 int ntg_matmult_dev(int dtype, const void* dA, const void* dB, void* dC, int64_t m, int64_t k, int64_t n,
@@ -656,7 +702,17 @@ int ntg_matmult_batch(int dtype, const void* const* A, const void* const* B, voi
     if (strided) d.stride_c = (int64_t)(align_up(c_bytes, 256) / (size_t)es);
     else d.stride_a = d.stride_b = 0;
     const size_t ws_off = off;
-    const int64_t ws_bytes = strided ? ntg_gemm_workspace_bytes(&d) : 0;
+    int64_t ws_bytes = strided ? ntg_gemm_workspace_bytes(&d) : 0;
+    // A pattern of repeated pointers runs as ONE table batch, which has no workspace form.  Where an item on its own would
+    // be given one that changes the order of summation over k (a split), the items go out one by one in that form instead,
+    // so that an item comes out bit for bit the same alone and in any batch (tests/src/matmult_test.cpp:108-189).
+    bool per_item = false;
+    if (!strided) {
+        ntg_gemm_desc one = d;
+        one.batches = 1;
+        const int64_t wb = ntg_gemm_workspace_bytes(&one);
+        if (wb > 0) { per_item = true; ws_bytes = wb; }
+    }
     if (ws_bytes > 0) off += (size_t)ws_bytes;
 
     ntg::HostSession mem;
@@ -678,6 +734,10 @@ int ntg_matmult_batch(int dtype, const void* const* A, const void* const* B, voi
     if (ws_bytes > 0) { d.workspace = mem.at(ws_off); d.workspace_bytes = ws_bytes; }
     if (strided) {
         rc = ntg_gemm_dev(&d, tab[0], tab[(size_t)batches], tab[(size_t)(2 * batches)], mem.stream());
+    } else if (per_item) {
+        d.batches = 1;
+        for (int64_t i = 0; i < batches && rc == NTG_OK; ++i)
+            rc = ntg_gemm_dev(&d, tab[(size_t)i], tab[(size_t)(batches + i)], tab[(size_t)(2 * batches + i)], mem.stream());
     } else {
         HIP_TRY(mem.upload(tab_off, tab.data(), tab.size() * sizeof(void*)));
         rc = gemm_ptrs(&d, dtab, dtab + batches, dtab + 2 * batches, mem.stream(), true);     // (every slot of the arena is 256-byte aligned)

@@ -80,18 +80,20 @@ __global__ void __launch_bounds__(256) reduce_batch_taps_last_vec_kernel(const T
 // Split-K epilogue: C (+)= sum over the k ranges of part[s][m][n], s ascending, starting from C0 (the incoming C, the
 // broadcast bias, or zero).  One rounding to T at the end.
 template <class T, class P, class Acc>
-__global__ void __launch_bounds__(256) splitk_reduce_kernel(const P* __restrict__ part, const int splits, const GemmParams p) {
+__global__ void __launch_bounds__(256) splitk_reduce_kernel(const P* __restrict__ part, const int splits, const int64_t split_stride, const GemmParams p) {
     const int64_t total = (int64_t)p.M * p.N;
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-    T* C = static_cast<T*>(p.C);
-    const T* bias = static_cast<const T*>(p.bias);
+    const int64_t b = blockIdx.y;                                      // item of the batch: its partial sums follow the previous item's
+    T* C = static_cast<T*>(p.C) + b * p.sC;
+    const T* bias = static_cast<const T*>(p.bias) + b * p.bias_bs;
+    part += b * total;
     for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += stride) {
         const int64_t m = idx / p.N, n = idx - m * p.N;
         T* cp = C + m * p.ldc + n;
         Acc acc = (Acc)0;
         if (p.cmode == C_ACCUMULATE) acc = (Acc)*cp;
         else if (p.cmode == C_BIAS) acc = (Acc)bias[m * p.bias_rs + n * p.bias_cs];
-        for (int s = 0; s < splits; ++s) acc += (Acc)part[(int64_t)s * total + idx];
+        for (int s = 0; s < splits; ++s) acc += (Acc)part[(int64_t)s * split_stride + idx];
         if (p.act == ACT_RELU) acc = acc > (Acc)0 ? acc : (Acc)0;
         *cp = (T)acc;
     }
@@ -100,13 +102,15 @@ __global__ void __launch_bounds__(256) splitk_reduce_kernel(const P* __restrict_
 // The same sum, four consecutive columns per thread with 16-byte accesses to the partial sums (rows of C and of the
 // partial matrices must start on a multiple of four elements); the partial loads of four k ranges are in flight together.
 template <class T, class P, class Acc>
-__global__ void __launch_bounds__(256) splitk_reduce_vec_kernel(const P* __restrict__ part, const int splits, const GemmParams p) {
+__global__ void __launch_bounds__(256) splitk_reduce_vec_kernel(const P* __restrict__ part, const int splits, const int64_t split_stride, const GemmParams p) {
     typedef T TV __attribute__((ext_vector_type(4)));
     typedef P PV __attribute__((ext_vector_type(4)));
     const int64_t nq = p.N / 4, total = (int64_t)p.M * p.N, quads = (int64_t)p.M * nq;
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-    T* C = static_cast<T*>(p.C);
-    const T* bias = static_cast<const T*>(p.bias);
+    const int64_t b = blockIdx.y;
+    T* C = static_cast<T*>(p.C) + b * p.sC;
+    const T* bias = static_cast<const T*>(p.bias) + b * p.bias_bs;
+    part += b * total;
     for (int64_t q = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; q < quads; q += stride) {
         const int64_t m = q / nq, n = (q - m * nq) * 4;
         TV* cp = reinterpret_cast<TV*>(C + m * p.ldc + n);
@@ -124,14 +128,14 @@ __global__ void __launch_bounds__(256) splitk_reduce_vec_kernel(const P* __restr
         for (; s + 4 <= splits; s += 4) {
             PV v[4];
 #pragma unroll
-            for (int u = 0; u < 4; ++u) v[u] = *reinterpret_cast<const PV*>(pp + (int64_t)(s + u) * total);
+            for (int u = 0; u < 4; ++u) v[u] = *reinterpret_cast<const PV*>(pp + (int64_t)(s + u) * split_stride);
 #pragma unroll
             for (int u = 0; u < 4; ++u)
 #pragma unroll
                 for (int e = 0; e < 4; ++e) acc[e] += (Acc)v[u][e];
         }
         for (; s < splits; ++s) {
-            const PV v = *reinterpret_cast<const PV*>(pp + (int64_t)s * total);
+            const PV v = *reinterpret_cast<const PV*>(pp + (int64_t)s * split_stride);
 #pragma unroll
             for (int e = 0; e < 4; ++e) acc[e] += (Acc)v[e];
         }
@@ -142,13 +146,15 @@ __global__ void __launch_bounds__(256) splitk_reduce_vec_kernel(const P* __restr
     }
 }
 
+// p.batch items (at most 65535 per call): item b's partial sums start b * M * N elements into every k range's block, the
+// ranges' blocks lie p.batch * M * N elements apart
 template <class T, class P, class Acc>
 static void launch_splitk_reduce_t(const void* part, int splits, const GemmParams& p, hipStream_t s) {
-    const int64_t total = (int64_t)p.M * p.N;
-    const bool vec = p.N % 4 == 0 && p.ldc % 4 == 0 && (reinterpret_cast<uintptr_t>(p.C) % (4 * sizeof(T))) == 0 &&
+    const int64_t total = (int64_t)p.M * p.N, split_stride = total * p.batch;
+    const bool vec = p.N % 4 == 0 && p.ldc % 4 == 0 && p.sC % 4 == 0 && (reinterpret_cast<uintptr_t>(p.C) % (4 * sizeof(T))) == 0 &&
                      (reinterpret_cast<uintptr_t>(part) % (4 * sizeof(P))) == 0;
-    if (vec) hipLaunchKernelGGL((splitk_reduce_vec_kernel<T, P, Acc>), dim3(grid_for(total / 4)), dim3(256), 0, s, (const P*)part, splits, p);
-    else hipLaunchKernelGGL((splitk_reduce_kernel<T, P, Acc>), dim3(grid_for(total)), dim3(256), 0, s, (const P*)part, splits, p);
+    if (vec) hipLaunchKernelGGL((splitk_reduce_vec_kernel<T, P, Acc>), dim3(grid_for(total / 4), (unsigned)p.batch), dim3(256), 0, s, (const P*)part, splits, split_stride, p);
+    else hipLaunchKernelGGL((splitk_reduce_kernel<T, P, Acc>), dim3(grid_for(total), (unsigned)p.batch), dim3(256), 0, s, (const P*)part, splits, split_stride, p);
 }
 
 // C[b][m][n] = C[b][m][n] > 0 ? C[b][m][n] : 0 -- relu_ = clamp_(x, 0) of the reference (activation_functions.cpp:143,
@@ -192,7 +198,8 @@ hipError_t launch_relu_inplace(int dtype, void* C, int64_t ldc, int64_t sC, int6
 
 hipError_t launch_splitk_reduce(int dtype, const void* part, int splits, const GemmParams& p, hipStream_t s) {
     const int64_t total = (int64_t)p.M * p.N;
-    if (total == 0) return hipSuccess;
+    if (total == 0 || p.batch < 1) return hipSuccess;
+    if (p.batch > 65535) return hipErrorInvalidValue;
     switch (dtype) {
     case DT_F32: launch_splitk_reduce_t<float, float, float>(part, splits, p, s); break;
     case DT_F64: launch_splitk_reduce_t<double, double, double>(part, splits, p, s); break;

@@ -85,6 +85,43 @@ static void* device_workspace(int64_t bytes) {
     return buf.get();
 }
 
+// Pointer tables of a list product: copied to a device buffer this thread keeps (it only grows), through a pinned host buffer, on
+// the default stream.  The copy is ordered behind the kernels of the previous call that still read the device buffer; the
+// event says when the pinned buffer may be overwritten.  Nothing is allocated, freed or waited for in the steady state.
+namespace {
+struct TableBuffers {
+    std::shared_ptr<char> dev;
+    char* pinned = nullptr;
+    int64_t cap = 0;
+    hipEvent_t copied = nullptr;
+    ~TableBuffers() {
+        if (pinned) (void)hipHostFree(pinned);
+        if (copied) (void)hipEventDestroy(copied);
+    }
+};
+}  // namespace
+static void* upload_table(const void* src, int64_t bytes) {
+    static thread_local TableBuffers tb;
+    if (bytes > tb.cap) {
+        hip_check(hipDeviceSynchronize(), "hipDeviceSynchronize");     // kernels may still read the smaller table
+        if (tb.pinned) { (void)hipHostFree(tb.pinned); tb.pinned = nullptr; }
+        tb.dev.reset();
+        tb.cap = 0;
+        tb.dev = device_alloc((size_t)bytes);
+        void* h = nullptr;
+        hip_check(hipHostMalloc(&h, (size_t)bytes, hipHostMallocDefault), "hipHostMalloc");
+        tb.pinned = static_cast<char*>(h);
+        tb.cap = bytes;
+        if (!tb.copied) hip_check(hipEventCreateWithFlags(&tb.copied, hipEventDisableTiming), "hipEventCreate");
+    } else {
+        hip_check(hipEventSynchronize(tb.copied), "hipEventSynchronize");   // the previous copy has left the pinned buffer
+    }
+    std::memcpy(tb.pinned, src, (size_t)bytes);
+    hip_check(hipMemcpyAsync(tb.dev.get(), tb.pinned, (size_t)bytes, hipMemcpyHostToDevice, nullptr), "hipMemcpyAsync (pointer tables)");
+    hip_check(hipEventRecord(tb.copied, nullptr), "hipEventRecord");
+    return tb.dev.get();
+}
+
 Tensor::Tensor(SizeRef shape, DType dt, DeviceType dev) : shape_(std::move(shape)), dtype_(dt), device_(dev) {
     const int64_t es = dtype_size(dt);
     utils::throw_exception(es > 0, std::string("dtype ") + dtype_name(dt) + " has no storage in nt_compat");
@@ -618,15 +655,52 @@ Tensor matmult(const TensorList& a, const TensorList& b, bool trans_a, bool tran
                 tab[(size_t)(total + t)] = static_cast<const char*>(bs[(size_t)i].data_ptr()) + (j % p0.nb) * p0.k * p0.n * es;
                 tab[(size_t)(2 * total + t)] = static_cast<char*>(c.data_ptr()) + t * p0.m * p0.n * es;
             }
-        std::shared_ptr<char> dtab = device_alloc(tab.size() * sizeof(void*));
-        hip_check(hipMemcpy(dtab.get(), tab.data(), tab.size() * sizeof(void*), hipMemcpyHostToDevice), "hipMemcpy (pointer tables)");
         ntg_gemm_desc d;
         std::memset(&d, 0, sizeof d);
         d.dtype = dt; d.transpose_a = p0.ta; d.transpose_b = p0.tb; d.c_mode = NTG_C_OVERWRITE;
         d.m = p0.m; d.k = p0.k; d.n = p0.n; d.batches = total;
-        void** T = reinterpret_cast<void**>(dtab.get());
+        // (1) Lists made by split_axis are slices of one allocation: the matrices of an operand then lie at a constant stride
+        // (or are all the same matrix) and the list is an ordinary strided batch, workspace forms included.
+        auto affine = [&](const void* const* P, int64_t& stride) {
+            const char* p0c = static_cast<const char*>(P[0]);
+            const int64_t step = total > 1 ? static_cast<const char*>(P[1]) - p0c : 0;
+            if (step < 0 || step % es != 0) return false;
+            for (int64_t t = 0; t < total; ++t)
+                if (static_cast<const char*>(P[t]) != p0c + t * step) return false;
+            stride = step / es;
+            return true;
+        };
+        auto with_workspace = [&](ntg_gemm_desc& q) {
+            const int64_t wsb = ntg_gemm_workspace_bytes(&q);
+            if (wsb > 0) { q.workspace = device_workspace(wsb); q.workspace_bytes = wsb; }
+            return wsb;
+        };
+        if (affine(tab.data(), d.stride_a) && affine(tab.data() + total, d.stride_b)) {
+            d.stride_c = p0.m * p0.n;
+            with_workspace(d);
+            check_status(ntg_gemm_dev(&d, tab[0], tab[(size_t)total], const_cast<void*>(tab[(size_t)(2 * total)]), nullptr));
+            return c;
+        }
+        // (2) Any other list: where one item on its own would be given a workspace form (a split along k changes the order of
+        // summation), the items go out one by one in that form, so that an item comes out bit for bit the same alone and in a
+        // list (tests/src/matmult_test.cpp:108-189) ...
+        {
+            ntg_gemm_desc one = d;
+            one.batches = 1;
+            if (with_workspace(one) > 0) {
+                for (int64_t t = 0; t < total; ++t)
+                    check_status(ntg_gemm_dev(&one, tab[(size_t)t], tab[(size_t)(total + t)], const_cast<void*>(tab[(size_t)(2 * total + t)]), nullptr));
+                return c;
+            }
+        }
+        // (3) ... else one table batch.  The tables go to this thread's cached device buffer (upload_table), so nothing is
+        // allocated, freed or waited for here; the host can see every entry, so it vouches for their alignment where that
+        // holds (the facade's own allocations are 256-byte aligned).
+        bool aligned = true;
+        for (const void* q : tab) aligned = aligned && (reinterpret_cast<uintptr_t>(q) & 15) == 0;
+        if (aligned) d.flags |= NTG_GEMM_PTRS_ALIGNED16;
+        void** T = static_cast<void**>(upload_table(tab.data(), (int64_t)(tab.size() * sizeof(void*))));
         check_status(ntg_gemm_ptrs_dev(&d, T, T + total, T + 2 * total, nullptr));
-        hip_check(hipStreamSynchronize(nullptr), "hipStreamSynchronize");      // the table is freed on return
         return c;
     }
     Tensor c = zeros(out_shape, a[0].dtype());

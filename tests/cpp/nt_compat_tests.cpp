@@ -536,6 +536,30 @@ static void device_resident_cases(const std::string& g) {
         nt::utils::throw_exception(dout.is_device() && dout.shape() == SizeRef({10, 30, 24}), "shape of the device result");
         same_bits(dout, o, "list product");
     });
+    run_test("device lists of separately allocated tensors: every item == the pair alone, bit for bit", [&] {
+        // the reference's list test (tests/src/matmult_test.cpp:108-189) on lists that are NOT slices of one allocation, at
+        // sizes where an item alone is split along k (64 x 4096 x 64: its items then go out one by one) and where it is not
+        // (a pointer-table batch); two rounds, so the cached tables are reused
+        for (int round = 0; round < 2; ++round)
+            for (const SizeRef& mkn : {SizeRef{64, 4096, 64}, SizeRef{96, 200, 72}, SizeRef{16, 512, 128}}) {
+                nt::TensorList da, db;
+                for (int i = 0; i < 4; ++i) {
+                    da.push_back(F::randn({mkn[0], mkn[1]}, DType::Float32, 300 + i + 10 * round).to(DeviceType::HIP));
+                    db.push_back(F::randn({mkn[1], mkn[2]}, DType::Float32, 400 + i + 10 * round).to(DeviceType::HIP));
+                }
+                nt::TensorList shuffled_a = {da[2], da[0], da[3], da[0]}, shuffled_b = {db[2], db[1], db[3], db[0]};
+                Tensor o = nt::matmult(shuffled_a, shuffled_b);
+                nt::utils::throw_exception(o.is_device() && o.shape() == SizeRef({4 * mkn[0], mkn[2]}), "shape of the list result");
+                Tensor oh = o.cpu();
+                const int ia[4] = {2, 0, 3, 0}, ib[4] = {2, 1, 3, 0};
+                for (int i = 0; i < 4; ++i) {
+                    Tensor one = nt::matmult(da[(size_t)ia[i]], db[(size_t)ib[i]]).cpu();
+                    const size_t bytes = (size_t)(mkn[0] * mkn[2]) * sizeof(float);
+                    nt::utils::throw_exception(std::memcmp(static_cast<const char*>(oh.data_ptr()) + (size_t)i * bytes, one.data_ptr(), bytes) == 0,
+                                               "item " + std::to_string(i) + " of the list differs from the pair alone");
+                }
+            }
+    });
     run_test("device conv2d (channels-last path), conv1d, conv_transpose2d, unfold2d, conv3d == host", [&] {
         Tensor x = F::randn({3, 32, 9, 11}, DType::Float32, 101), w = F::randn({24, 16, 3, 3}, DType::Float32, 102);
         Tensor dx = x.to(DeviceType::HIP), dw = w.to(DeviceType::HIP);

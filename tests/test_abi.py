@@ -42,7 +42,8 @@ def test_dtype_sizes_follow_nt_dtype_values():
 
 
 def test_desc_struct_layout():
-    assert ctypes.sizeof(_lib.GemmDesc) == 16 + 8 * 3 + 8 * 3 + 8 + 8 * 3 + 8 + 8 * 3 + 8 + 8
+    assert ctypes.sizeof(_lib.GemmDesc) == 16 + 8 * 3 + 8 * 3 + 8 + 8 * 3 + 8 + 8 * 3 + 8 + 8 + 8
+    assert _lib.GemmDesc.flags.offset == ctypes.sizeof(_lib.GemmDesc) - 8 and _lib.GemmDesc.workspace_bytes.offset == _lib.GemmDesc.flags.offset - 8
 
 
 def test_argument_errors_do_not_need_a_device():
@@ -140,10 +141,14 @@ def test_split_k_planner_needs_no_device():
         assert b % (m * n * es) == 0
         return b // (m * n * es)
 
-    # full-chip products are never split; integers, batches and the streaming (m <= 32) shapes neither
+    # full-chip products are never split; integers and the streaming (m <= 32) shapes neither.  The plan looks at one item
+    # only -- a split changes the order of summation over k, and an item must come out the same alone and in a batch -- so a
+    # batch is offered its item's split, with the partial sums of every item
     for dt in (_lib.BFLOAT16, _lib.FLOAT16, _lib.FLOAT32, _lib.FLOAT64):
         assert ws(dt, 4096, 4096, 4096) == 0
-        assert ws(dt, 256, 8192, 2048, batches=2) == 0
+        assert ws(dt, 4096, 4096, 4096, batches=3) == 0
+        one = ws(dt, 256, 8192, 2048)
+        assert one > 0 and ws(dt, 256, 8192, 2048, batches=2) == 2 * one and ws(dt, 256, 8192, 2048, batches=7) == 7 * one
     assert ws(_lib.INT32, 64, 8192, 64) == 0
     assert ws(_lib.FLOAT32, 16, 8192, 8192) == 0 and ws(_lib.BFLOAT16, 32, 8192, 8192) == 0
     # 16-bit, 128 x 128 tiles: 64 tiles and k = 8192 -> four ranges; one tile and k = 16384 -> sixteen

@@ -445,6 +445,22 @@ def test_config3_4096_cube(dtype, scale):
     else:
         ref = torch.matmul(ta_.float(), tb_.float())
         assert ((out.float() - ref).abs().max() / ref.abs().max()).item() <= HALF_REL
+        # 384 whole rows (from the first, a middle and the last tile row, each crossing a block boundary of the tile) against the
+        # exact result: every element is the once-rounded float64 product wherever that is clear of a rounding boundary
+        from util import assert_one_rounding
+        fmt = "bf16" if bf else "f16"
+        rsel = torch.as_tensor(np.r_[0:128, 1984:2112, 3968:4096], device=DEV)
+        ar, bd = ta_[rsel].double(), tb_.double()
+        ref64 = ar @ bd
+        spread = ((ar * ar) @ (bd * bd)).sqrt()
+        assert_one_rounding(out[rsel].double().cpu().numpy(), ref64.cpu().numpy(), spread.cpu().numpy(), n, fmt, f"{fmt} 4096^3 overwrite",
+                            min_exact=0.75 if bf else 0.2)
+        c0r = to_torch(randn(rng, (n, n), dtype, 0.5), DEV, bf)
+        accr = c0r.clone()
+        F.matmult(ta_, tb_, accr)                                    # the headline's own mode: C += A.B
+        assert_one_rounding(accr[rsel].double().cpu().numpy(), (ref64 + c0r[rsel].double()).cpu().numpy(),
+                            (spread + c0r[rsel].double().abs()).cpu().numpy(), n, fmt, f"{fmt} 4096^3 accumulate", min_exact=0.75 if bf else 0.2)
+        del ar, bd, ref64, spread, c0r, accr
     # linearity, a size-independent property: (2A).B == 2(A.B) exactly in binary floating point
     out2 = F.matmult(ta_ * 2, tb_)
     if dtype is np.float16:      # half subnormals (|c| < 6.1e-5) round on a fixed 2^-24 grid
@@ -719,8 +735,8 @@ def test_split_k_medium_rows(dtype):
         y = F.linear(to_torch(a, DEV, bf), to_torch(b, DEV, bf), bias)
         refy = to_torch(a, DEV, bf).double() @ to_torch(b, DEV, bf).double() + bias.double()
         assert (y.double() - refy).abs().max().item() <= tol + (HALF_REL * scale if half else 0)
-    # no split where it does not apply: many tiles, shallow k, batches
-    for (m, k, n, bt) in [(4096, 4096, 4096, 1), (256, 128, 256, 1), (256, 4096, 2048, 2)]:
+    # no split where it does not apply: many tiles, shallow k (a batch is offered what its item is offered)
+    for (m, k, n, bt) in [(4096, 4096, 4096, 1), (256, 128, 256, 1), (4096, 4096, 4096, 2)]:
         d = _lib.GemmDesc()
         d.dtype, d.m, d.k, d.n, d.batches = F.ntg_dtype(ta_), m, k, n, bt
         d.stride_a, d.stride_b, d.stride_c = m * k, k * n, m * n
@@ -1065,3 +1081,84 @@ def test_host_batch_bf16_pointer_tables_on_deep_k_steps():
         assert single.tobytes() == got[i].tobytes(), i
         al, bl, cl = to_f64(As[i][rows], True), to_f64(Bs[i], True), to_f64(C0[i][rows], True)
         assert_one_rounding(to_f64(got[i][rows], True), al @ bl + cl, np.abs(cl) + np.sqrt((al * al) @ (bl * bl)), k, "bf16", f"item {i}")
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64, "bf16", np.float16], ids=["fp32", "fp64", "bf16", "fp16"])
+@pytest.mark.parametrize("shape", [(256, 256, 256), (64, 8192, 64), (48, 300, 100), (16, 512, 256), (256, 1024, 256), (256, 8192, 512),
+                                   (512, 512, 512)], ids=lambda s: "x".join(map(str, s)))
+def test_item_is_the_same_alone_and_in_every_batch_form(dtype, shape):
+    """The reference's batched == per-item rule (tests/src/matmult_test.cpp:108-189: every item of a list product equals the
+    product of the pair alone, element for element) at sizes where this library has kernels that sum over k in different
+    orders: products with few output tiles and a deep k are split along k when a workspace is offered (64 x 8192 x 64,
+    256 x 1024 x 256, 256 x 8192 x 512), 16 rows take the streaming kernel, the others the tile kernels.  Which order an item
+    gets may depend on the item's own sizes only: alone, as every item of strided batches of 3 and 8 (distinct items), in a
+    device pointer table (with and without the caller's vouch for the entries' alignment), through the host entry points
+    with distinct and with repeated pointers -- the bits are the same."""
+    m, k, n = shape
+    bf = dtype == "bf16"
+    rng = np.random.default_rng(9100 + m + k)
+    nb = 8
+    a = to_torch(randn(rng, (nb, m, k), dtype, 0.5), DEV, bf)
+    b = to_torch(randn(rng, (nb, k, n), dtype, 0.5), DEV, bf)
+    bits = lambda t: t.contiguous().view(torch.int16 if t.element_size() == 2 else torch.int32 if t.element_size() == 4 else torch.int64)
+    lib = _lib.load()
+    st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    for ta, tb in ((False, False), (False, True), (True, False)):
+        sa = a.transpose(1, 2).contiguous() if ta else a
+        sb = b.transpose(1, 2).contiguous() if tb else b
+        alone = [F.matmult(sa[i], sb[i], None, ta, tb) for i in range(nb)]
+        ref = torch.matmul(a[0].double(), b[0].double())
+        tol = 1e-5 * k * float(a[0].abs().max() * b[0].abs().max()) if dtype in (np.float32, np.float64) else HALF_REL * float(ref.abs().max())
+        assert (alone[0].double() - ref).abs().max().item() <= tol
+        for batch in (3, 8):
+            out = F.matmult(sa[:batch].contiguous(), sb[:batch].contiguous(), None, ta, tb)
+            for i in range(batch):
+                assert torch.equal(bits(out[i]), bits(alone[i])), (shape, ta, tb, "strided batch", batch, i)
+        # one matrix against every item (stride 0 on B): still the item's own result
+        out = F.matmult(sa[:3].contiguous(), sb[1], None, ta, tb)
+        assert torch.equal(bits(out[1]), bits(alone[1])), (shape, ta, tb, "broadcast b")
+        # device pointer tables: never split along k, so they stand for the items only where an item alone is not split either
+        d = _lib.GemmDesc()
+        d.dtype = code_of(dtype)
+        d.transpose_a, d.transpose_b, d.c_mode = int(ta), int(tb), _lib.C_OVERWRITE
+        d.m, d.k, d.n, d.batches = m, k, n, 1
+        if lib.ntg_gemm_workspace_bytes(ctypes.byref(d)) == 0:
+            d.batches = 5
+            order = [4, 0, 2, 2, 7]
+            for flags in (_lib.GEMM_PTRS_ALIGNED16, 0):
+                d.flags = flags
+                c = torch.zeros((5, m, n), dtype=a.dtype, device=DEV)
+                tab = torch.tensor([sa[i].data_ptr() for i in order] + [sb[i].data_ptr() for i in order] + [c[j].data_ptr() for j in range(5)],
+                                   dtype=torch.int64, device=DEV)
+                _lib.check(lib.ntg_gemm_ptrs_dev(ctypes.byref(d), tab.data_ptr(), tab.data_ptr() + 40, tab.data_ptr() + 80, st))
+                torch.cuda.synchronize()
+                for j, i in enumerate(order):
+                    assert torch.equal(bits(c[j]), bits(alone[i])), (shape, ta, tb, "pointer table", flags, j)
+    # the host entry points (the drop-in seam): nt_matmult against nt_matmult_batch with distinct and with repeated pointers
+    if dtype == "bf16":
+        return
+    ha = [a[i].cpu().numpy() for i in range(4)]
+    hb = [b[i].cpu().numpy() for i in range(4)]
+    code = code_of(dtype)
+    single = []
+    for i in range(4):
+        c = np.zeros((m, n), ha[0].dtype)
+        host_matmult(ha[i], hb[i], c, m, k, n, False, False, code)
+        single.append(c)
+        assert np.array_equal(c.view(np.uint8), alone_np(a[i], b[i]).view(np.uint8)), (shape, "host alone == device alone", i)
+    arr = ctypes.c_void_p * 4
+    for name, ia, ib in (("distinct", [0, 1, 2, 3], [0, 1, 2, 3]), ("shared b", [0, 1, 2, 3], [1, 1, 1, 1]), ("mixed", [0, 1, 0, 1], [2, 2, 3, 3])):
+        got = [np.zeros((m, n), ha[0].dtype) for _ in range(4)]
+        _lib.check(lib.ntg_matmult_batch(code, arr(*[ha[i].ctypes.data for i in ia]), arr(*[hb[i].ctypes.data for i in ib]),
+                                         arr(*[g.ctypes.data for g in got]), 4, m, k, k, n, 0, 0))
+        for j in range(4):
+            want = single[ia[j]] if ia[j] == ib[j] else None
+            if want is None:
+                want = np.zeros((m, n), ha[0].dtype)
+                host_matmult(ha[ia[j]], hb[ib[j]], want, m, k, n, False, False, code)
+            assert np.array_equal(got[j].view(np.uint8), want.view(np.uint8)), (shape, "host batch", name, j)
+
+
+def alone_np(a, b):
+    """one product on device tensors through the functional face, as a numpy array"""
+    return from_torch(F.matmult(a, b))

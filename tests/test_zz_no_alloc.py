@@ -1,5 +1,5 @@
-"""ntg_gemm_noalloc_dev (the entry point that allocates nothing: its split-K partial sums and integer byte planes live
-in a fixed array inside the library's device code) against ntg_gemm_dev with a caller-owned workspace, through the C ABI.
+"""ntg_gemm_noalloc_dev (the entry point that allocates nothing: its split-K partial sums, integer byte planes and padded
+copies live in a fixed array inside the library's device code) against ntg_gemm_dev with a caller-owned workspace, through the C ABI.
 
 Both run the same kernels in the same order, so every result must be bit-identical -- for the floating dtypes too.
 Calls follow each other on one stream, a smaller product after a larger one, so stale contents of the shared array
@@ -97,6 +97,16 @@ def test_noalloc_entry_point_matches_the_workspace_entry_point():
     _both(lib, rng, "bf16", 256, 4096, 2048, False, False, OV)
     # a batch of integer products (planes of every item in the array)
     _both(lib, rng, np.int16, 256, 256, 256, False, False, ACC, batches=3)
+    # padded copies (rows that are not 16-byte multiples: A, B and C copied into the array, the bias written as the padded
+    # C's starting value, the result copied back), a larger product before a smaller one, then the 8-bit form
+    big = _both(lib, rng, "bf16", 2048, 1001, 2044, False, False, BIAS)
+    small = _both(lib, rng, "bf16", 1032, 2001, 1048, False, True, ACC)
+    assert small < big, (small, big)
+    _both(lib, rng, np.float16, 2048, 1001, 2044, True, False, ACC)
+    _both(lib, rng, np.int8, 520, 1001, 530, False, False, ACC)
+    # a batch whose items are split along k (the partial sums of every item and k range in the array)
+    _both(lib, rng, "bf16", 256, 4096, 512, False, False, ACC, batches=3)
+    _both(lib, rng, np.float32, 64, 4096, 256, False, True, BIAS, batches=5)
     # products that have no workspace form run on the plain kernels
     _both(lib, rng, np.float32, 512, 512, 512, False, False, ACC, expect_workspace=False)
     _both(lib, rng, "bf16", 100, 72, 48, False, True, OV, expect_workspace=False)
@@ -115,9 +125,43 @@ def test_noalloc_entry_point_rejects_what_does_not_fit():
     assert rc == 1
     msg = lib.ntg_last_error().decode()
     assert str(need) in msg and str(_lib.NOALLOC_SCRATCH_BYTES) in msg, msg
+    assert "ntg_gemm_dev" in msg and "without a workspace" in msg, msg         # (the message names the allocation-free fallback)
     torch.cuda.synchronize()
     assert int(c.abs().max()) == 0                                            # nothing was launched
     # argument errors as in ntg_gemm_dev
     assert lib.ntg_gemm_noalloc_dev(ctypes.byref(d), None, a.data_ptr(), c.data_ptr(), st) == 1
     d.stride_c = 0
     assert lib.ntg_gemm_noalloc_dev(ctypes.byref(d), a.data_ptr(), a.data_ptr(), c.data_ptr(), st) == 1
+
+
+def test_noalloc_calls_on_two_streams_are_ordered_by_the_library():
+    """Two streams use the one array without any synchronisation by the caller: a long split product on one stream, a short
+    one on the other right behind it, several rounds.  The library orders them (an event behind each user's last kernel),
+    so both results are those of caller-owned workspaces."""
+    lib = _lib.load()
+    rng = np.random.default_rng(99)
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    a1, b1, c1, _ = _operands(rng, "bf16", 256, 8192, 2048, False, False)
+    a2, b2, c2, _ = _operands(rng, "bf16", 64, 4096, 512, False, True)
+    d1 = _desc(a1, 256, 8192, 2048, False, False, _lib.C_OVERWRITE)
+    d2 = _desc(a2, 64, 4096, 512, False, True, _lib.C_OVERWRITE)
+    want = []
+    for (d, a, b, c) in ((d1, a1, b1, c1), (d2, a2, b2, c2)):
+        need = lib.ntg_gemm_workspace_bytes(ctypes.byref(d))
+        assert 0 < need <= _lib.NOALLOC_SCRATCH_BYTES
+        ws = torch.empty(need, dtype=torch.uint8, device=DEV)
+        w = torch.empty_like(c)
+        d.workspace, d.workspace_bytes = ws.data_ptr(), need
+        _lib.check(lib.ntg_gemm_dev(ctypes.byref(d), a.data_ptr(), b.data_ptr(), w.data_ptr(), ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)))
+        d.workspace, d.workspace_bytes = None, 0
+        want.append(w)
+    torch.cuda.synchronize()
+    for rnd in range(6):
+        g1, g2 = torch.zeros_like(c1), torch.zeros_like(c2)
+        torch.cuda.synchronize()
+        _lib.check(lib.ntg_gemm_noalloc_dev(ctypes.byref(d1), a1.data_ptr(), b1.data_ptr(), g1.data_ptr(), ctypes.c_void_p(s1.cuda_stream)))
+        _lib.check(lib.ntg_gemm_noalloc_dev(ctypes.byref(d2), a2.data_ptr(), b2.data_ptr(), g2.data_ptr(), ctypes.c_void_p(s2.cuda_stream)))
+        _lib.check(lib.ntg_gemm_noalloc_dev(ctypes.byref(d1), a1.data_ptr(), b1.data_ptr(), g1.data_ptr(), ctypes.c_void_p(s1.cuda_stream)))
+        torch.cuda.synchronize()
+        assert torch.equal(g1.view(torch.int16), want[0].view(torch.int16)), rnd
+        assert torch.equal(g2.view(torch.int16), want[1].view(torch.int16)), rnd
