@@ -40,10 +40,11 @@ extern "C" {
  * kernel level (nt_matmult_uint64.cpp).  The complex types hold interleaved (re, im) pairs of half / float / double; their
  * matmult is the reference's: its generic micro kernel multiplies the interleaved lanes element-wise
  * (nt/mp/simde_traits/simde_traits_avx2.h:928-937, :996-1002), so the result is one real product of the real parts and one
- * of the imaginary parts (Complex32 rounded to half every 8 k), NOT the complex product.  They are served by the product,
- * linear, unfold and forward-convolution entry points (up to two spatial axes); the gradient and transposed convolutions
- * return NTG_ERR_UNSUPPORTED_DTYPE for them.  The 128-bit types (Float128 = 3, int128 = 11, uint128 = 15) stay on the
- * reference's matmult_naive. */
+ * of the imaginary parts (Complex32 rounded to half every 8 k), NOT the complex product.  Every entry point serves them:
+ * the convolutions over one to four axes, their gradients and the transposed convolutions unfold into the workspace and
+ * run that product like the reference (nt/functional/tensor_files/conv.cpp:69-175, :318-535, :538-745; the unfold adjoint
+ * adds taps lane by lane in the lane's type, the weight gradient adds the per-image products in batch order in that type).
+ * The 128-bit types (Float128 = 3, int128 = 11, uint128 = 15) stay on the reference's matmult_naive. */
 typedef enum ntg_dtype {
     NTG_FLOAT16 = 0,
     NTG_FLOAT32 = 1,

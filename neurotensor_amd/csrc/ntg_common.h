@@ -358,6 +358,20 @@ static inline unsigned grid_for(int64_t total) {
 }
 
 #ifdef __HIPCC__
+// One element of the complex dtypes as the reference's element-wise code treats it: two lanes (re, im) of the real type,
+// added lane by lane in that type (my_complex<T>::operator+=; complex_32 adds in half, rounding every sum).
+template <class R>
+struct LanePair {
+    R re, im;
+    LanePair() = default;
+    __device__ __forceinline__ LanePair(int z) : re((R)z), im((R)z) {}      // (Acc)0
+    __device__ __forceinline__ LanePair& operator+=(const LanePair& o) {
+        re = re + o.re;
+        im = im + o.im;
+        return *this;
+    }
+};
+
 // element offset of launch index b's A (stride = p.sA, kstride = p.sAk) or B operand
 __device__ __forceinline__ int64_t operand_offset(const GemmParams& p, int b, int64_t stride, int64_t kstride) {
     if (p.krange_items == 0) return (int64_t)b * stride;

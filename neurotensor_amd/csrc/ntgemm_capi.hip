@@ -119,13 +119,6 @@ bool is_complex_dtype(int dt) { return dt == ntg::DT_C32 || dt == ntg::DT_C64 ||
 // integers and the complex types: computed lane by lane on the vector ALU, bit-exact; no matrix-pipe or gathering forms
 bool is_valu_dtype(int dt) { return is_int_dtype(dt) || is_complex_dtype(dt); }
 
-// The complex types reach the product, im2col and the forward convolutions (what the reference's tests exercise,
-// tests/src/conv_test.cpp:192-213); col2im and the gradient / transposed convolutions are not built for them.
-int reject_complex(int dtype, const char* what) {
-    if (!is_complex_dtype(dtype)) return NTG_OK;
-    return fail(NTG_ERR_UNSUPPORTED_DTYPE, "%s is not available for the complex dtypes (dtype %d)", what, dtype);
-}
-
 // Fills the derived fields and launches the kernel family for the dtype.
 int launch_gemm(ntg::GemmParams p, int dtype, bool ta, bool tb, hipStream_t s) {
     const int64_t es = ntg::elem_size(dtype);
@@ -1376,6 +1369,50 @@ static int conv_dkernel_nhwc(int dtype, const void* image, const void* grad_out,
     return NTG_OK;
 }
 
+// The weight gradient from a stored col matrix (integers, complex types, four spatial axes): per group g
+//   dW_g [og, add] (+)= sum over the images b of dY_{b,g} [og, L] . col_{b,g}^T   (col_{b,g} stored [add, L]).
+// Integers: one accumulating product per (group, image) straight into dW (exact in any order).  Complex types: the
+// reference's order, which the results are checked against bit for bit -- every image's product on its own from zero, the
+// products added up in batch order in the element type, that sum added to dW last (conv.cpp:444-471: matmult(grad, image,
+// false, true).sum(0), then d_kernel +=); the per-image products [B][O][add] lie behind the col matrix in the workspace.
+static int64_t complex_dkernel_extra(int dtype, int64_t batch, int64_t out_channels, int64_t add, int64_t col_bytes) {
+    if (!is_complex_dtype(dtype)) return 0;
+    return (int64_t)(align_up((size_t)col_bytes, 256) - (size_t)col_bytes) + batch * out_channels * add * ntg::elem_size(dtype);
+}
+static int conv_dkernel_from_col(int dtype, const char* gy, char* col, void* d_kernel, int64_t batch, int64_t out_channels, int64_t ccol,
+                                 int64_t groups, int64_t L, int accumulate, void* stream) {
+    const int64_t es = ntg::elem_size(dtype), add = ccol / groups, og = out_channels / groups;
+    ntg_gemm_desc d;
+    int rc = NTG_OK;
+    if (is_complex_dtype(dtype)) {
+        char* per = col + align_up((size_t)(batch * ccol * L * es), 256);
+        for (int64_t g = 0; g < groups && rc == NTG_OK; ++g) {
+            std::memset(&d, 0, sizeof d);
+            d.dtype = dtype; d.transpose_b = 1; d.c_mode = NTG_C_OVERWRITE;
+            d.m = og; d.k = L; d.n = add;
+            d.lda = L; d.ldb = L; d.ldc = add; d.batches = batch;
+            d.stride_a = out_channels * L; d.stride_b = ccol * L; d.stride_c = out_channels * add;
+            rc = ntg_gemm_dev(&d, gy + g * og * L * es, col + g * add * L * es, per + g * og * add * es, stream);
+        }
+        if (rc) return rc;
+        hipError_t e = ntg::launch_reduce_batch(dtype, per, d_kernel, batch, out_channels * add, accumulate, static_cast<hipStream_t>(stream));
+        if (e != hipSuccess) return hip_fail(e, "weight gradient reduction launch");
+        return NTG_OK;
+    }
+    for (int64_t g = 0; g < groups; ++g)
+        for (int64_t b = 0; b < batch; ++b) {
+            std::memset(&d, 0, sizeof d);
+            d.dtype = dtype; d.transpose_b = 1;
+            d.c_mode = (b == 0 && !accumulate) ? NTG_C_OVERWRITE : NTG_C_ACCUMULATE;
+            d.m = og; d.k = L; d.n = add;
+            d.lda = L; d.ldb = L; d.ldc = add; d.batches = 1;
+            rc = ntg_gemm_dev(&d, gy + ((b * out_channels + g * og) * L) * es, col + ((b * ccol + g * add) * L) * es,
+                              static_cast<char*>(d_kernel) + g * og * add * es, stream);
+            if (rc) return rc;
+        }
+    return NTG_OK;
+}
+
 // Which backward gradients run as implicit GEMMs, and the workspace the call needs.
 struct ConvBackwardPlan { bool gather_dw, gather_dx, nhwc_dx, nhwc_dw, phase_dx; int64_t need, need_nhwc_dx, need_nhwc_dw, need_phase_dx; PhasePlan phases; };
 static ConvBackwardPlan plan_conv_backward_g(int dtype, bool want_dx, bool want_dw, int64_t batch, int64_t channels, int64_t out_channels,
@@ -1387,7 +1424,7 @@ static ConvBackwardPlan plan_conv_backward_g(int dtype, bool want_dx, bool want_
     pl.gather_dx = want_dx && g.s[0] == 1 && g.s[1] == 1 && g.s[2] == 1 && conv_implicit_g(dtype, out_channels, geo_dimage(g));
     const int64_t col = batch * channels * taps * g.L() * es;
     int64_t need = 0;
-    if (want_dw) need = std::max(need, pl.gather_dw ? batch * out_channels * cg * taps * es : col);
+    if (want_dw) need = std::max(need, pl.gather_dw ? batch * out_channels * cg * taps * es : col + complex_dkernel_extra(dtype, batch, out_channels, cg * taps, col));
     if (want_dx) need = std::max(need, pl.gather_dx ? out_channels * cg * taps * es : col);
     pl.need = need;
     // the channels-last form of dX is taken when the caller's workspace also holds the copy of dY
@@ -1532,7 +1569,6 @@ int ntg_unfold2d_backward_dev(int dtype, const void* col, void* image,
                               int64_t batch, int64_t channels, int64_t height, int64_t width,
                               int64_t k_r, int64_t k_c, int64_t s_r, int64_t s_c,
                               int64_t p_r, int64_t p_c, int64_t d_r, int64_t d_c, int accumulate, void* stream) {
-    if (int rcx = reject_complex(dtype, "ntg_unfold2d_backward_dev")) return rcx;
     const int64_t es = ntg::elem_size(dtype);
     if (es == 0) return fail(NTG_ERR_UNSUPPORTED_DTYPE, "dtype %d is not supported", dtype);
     if (batch < 0 || channels < 0 || height < 0 || width < 0) return fail(NTG_ERR_INVALID_ARGUMENT, "negative size");
@@ -1551,7 +1587,6 @@ int ntg_unfold2d_backward(int dtype, const void* col, void* image,
                           int64_t batch, int64_t channels, int64_t height, int64_t width,
                           int64_t k_r, int64_t k_c, int64_t s_r, int64_t s_c,
                           int64_t p_r, int64_t p_c, int64_t d_r, int64_t d_c, int accumulate) {
-    if (int rcx = reject_complex(dtype, "ntg_unfold2d_backward")) return rcx;
     const int64_t es = ntg::elem_size(dtype);
     if (es == 0) return fail(NTG_ERR_UNSUPPORTED_DTYPE, "dtype %d is not supported", dtype);
     if (batch < 0 || channels < 0 || height < 0 || width < 0) return fail(NTG_ERR_INVALID_ARGUMENT, "negative size");
@@ -1599,7 +1634,6 @@ int ntg_conv2d_backward_dev(int dtype, const void* image, const void* kernel, co
                             int64_t out_channels, int64_t k_r, int64_t k_c,
                             int64_t s_r, int64_t s_c, int64_t p_r, int64_t p_c, int64_t d_r, int64_t d_c,
                             int64_t groups, int accumulate, void* stream) {
-    if (int rcx = reject_complex(dtype, "ntg_conv2d_backward_dev")) return rcx;
     const int64_t es = ntg::elem_size(dtype);
     if (es == 0) return fail(NTG_ERR_UNSUPPORTED_DTYPE, "dtype %d is not supported", dtype);
     if (batch < 0 || channels < 0 || out_channels < 0 || height < 0 || width < 0) return fail(NTG_ERR_INVALID_ARGUMENT, "negative size");
@@ -1679,17 +1713,8 @@ int ntg_conv2d_backward_dev(int dtype, const void* image, const void* kernel, co
         // col = im2col(image); per group g:  dW_g [og, add] (+)= sum_b dY_{b,g} [og, L] . col_{b,g}^T  (col_{b,g} stored [add, L])
         rc = ntg_unfold2d_dev(dtype, image, ws, batch, channels, height, width, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c, stream);
         if (rc) return rc;
-        for (int64_t g = 0; g < groups; ++g)
-            for (int64_t b = 0; b < batch; ++b) {
-                std::memset(&d, 0, sizeof d);
-                d.dtype = dtype; d.transpose_b = 1;
-                d.c_mode = (b == 0 && !accumulate) ? NTG_C_OVERWRITE : NTG_C_ACCUMULATE;
-                d.m = og; d.k = L; d.n = add;
-                d.lda = L; d.ldb = L; d.ldc = add; d.batches = 1;
-                rc = ntg_gemm_dev(&d, gy + ((b * out_channels + g * og) * L) * es, ws + ((b * ckk + g * add) * L) * es,
-                                  static_cast<char*>(d_kernel) + g * og * add * es, stream);
-                if (rc) return rc;
-            }
+        rc = conv_dkernel_from_col(dtype, gy, ws, d_kernel, batch, out_channels, ckk, groups, L, accumulate, stream);
+        if (rc) return rc;
     }
     if (d_image) {
         // d_col_{b,g} [add, L] = W_g^T . dY_{b,g}   (W_g stored [og, add] -> transpose_a), then col2im
@@ -1752,7 +1777,6 @@ int ntg_conv_transpose2d_dev(int dtype, const void* input, const void* kernel, v
                              int64_t batch, int64_t in_channels, int64_t in_h, int64_t in_w, int64_t out_channels,
                              int64_t k_r, int64_t k_c, int64_t s_r, int64_t s_c, int64_t p_r, int64_t p_c, int64_t d_r, int64_t d_c,
                              int64_t op_r, int64_t op_c, int64_t groups, void* stream) {
-    if (int rcx = reject_complex(dtype, "ntg_conv_transpose2d_dev")) return rcx;
     if (ntg::elem_size(dtype) == 0) return fail(NTG_ERR_UNSUPPORTED_DTYPE, "dtype %d is not supported", dtype);
     if (batch < 0 || in_channels < 0 || out_channels < 0) return fail(NTG_ERR_INVALID_ARGUMENT, "negative size");
     if (groups < 1) return fail(NTG_ERR_INVALID_ARGUMENT, "groups must be >= 1");
@@ -1777,7 +1801,6 @@ int ntg_conv_transpose2d(int dtype, const void* input, const void* kernel, void*
                          int64_t batch, int64_t in_channels, int64_t in_h, int64_t in_w, int64_t out_channels,
                          int64_t k_r, int64_t k_c, int64_t s_r, int64_t s_c, int64_t p_r, int64_t p_c, int64_t d_r, int64_t d_c,
                          int64_t op_r, int64_t op_c, int64_t groups) {
-    if (int rcx = reject_complex(dtype, "ntg_conv_transpose2d")) return rcx;
     const int64_t es = ntg::elem_size(dtype);
     if (es == 0) return fail(NTG_ERR_UNSUPPORTED_DTYPE, "dtype %d is not supported", dtype);
     if (batch < 0 || in_channels < 0 || out_channels < 0) return fail(NTG_ERR_INVALID_ARGUMENT, "negative size");
@@ -1813,7 +1836,6 @@ int ntg_conv2d_backward(int dtype, const void* image, const void* kernel, const 
                         int64_t out_channels, int64_t k_r, int64_t k_c,
                         int64_t s_r, int64_t s_c, int64_t p_r, int64_t p_c, int64_t d_r, int64_t d_c,
                         int64_t groups, int accumulate) {
-    if (int rcx = reject_complex(dtype, "ntg_conv2d_backward")) return rcx;
     const int64_t es = ntg::elem_size(dtype);
     if (es == 0) return fail(NTG_ERR_UNSUPPORTED_DTYPE, "dtype %d is not supported", dtype);
     if (batch < 0 || channels < 0 || out_channels < 0 || height < 0 || width < 0) return fail(NTG_ERR_INVALID_ARGUMENT, "negative size");
@@ -1905,7 +1927,6 @@ int ntg_unfoldnd_dev(int dtype, const void* image, void* col, int64_t batch, int
 int ntg_unfoldnd_backward_dev(int dtype, const void* col, void* image, int64_t batch, int64_t channels, int ndim, const int64_t* size,
                               const int64_t* kernel_size, const int64_t* stride, const int64_t* padding, const int64_t* dilation,
                               int accumulate, void* stream) {
-    if (int rcx = reject_complex(dtype, "ntg_unfoldnd_backward_dev")) return rcx;
     if (ntg::elem_size(dtype) == 0) return fail(NTG_ERR_UNSUPPORTED_DTYPE, "dtype %d is not supported", dtype);
     ntg::UnfoldNdParams u;
     int rc = fill_nd(u, batch, channels, ndim, size, kernel_size, stride, padding, dilation);
@@ -1941,7 +1962,7 @@ int64_t ntg_convnd_workspace_bytes(int dtype, int64_t batch, int64_t channels, i
         if (backward) return plan_conv_backward_g(dtype, true, true, batch, channels, out_channels, g, groups).need;
         if (conv_implicit_g(dtype, channels, g)) return 0;
     }
-    return u.total * es;
+    return u.total * es + (backward ? complex_dkernel_extra(dtype, batch, out_channels, (channels / groups) * u.taps, u.total * es) : 0);
 }
 
 int ntg_convnd_dev(int dtype, const void* image, const void* kernel, void* out, void* workspace, int64_t workspace_bytes,
@@ -1959,7 +1980,6 @@ int ntg_convnd_dev(int dtype, const void* image, const void* kernel, void* out, 
         return ntg_conv2d_dev(dtype, image, kernel, out, workspace, workspace_bytes, batch, channels, g.h, g.w, out_channels, g.kr, g.kc,
                               g.sr, g.sc, g.pr, g.pc, g.dr, g.dc, groups, stream);
     }
-    if (int rcx = reject_complex(dtype, "a convolution over three or more axes")) return rcx;
     if (batch == 0 || out_channels == 0) return NTG_OK;
     if (!image || !kernel || !out) return fail(NTG_ERR_INVALID_ARGUMENT, "null pointer");
     if (ndim == 3) {
@@ -1993,7 +2013,6 @@ int ntg_convnd_backward_dev(int dtype, const void* image, const void* kernel, co
                             void* workspace, int64_t workspace_bytes, int64_t batch, int64_t channels, int64_t out_channels, int ndim,
                             const int64_t* size, const int64_t* kernel_size, const int64_t* stride, const int64_t* padding,
                             const int64_t* dilation, int64_t groups, int accumulate, void* stream) {
-    if (int rcx = reject_complex(dtype, "ntg_convnd_backward_dev")) return rcx;
     const int64_t es = ntg::elem_size(dtype);
     if (es == 0) return fail(NTG_ERR_UNSUPPORTED_DTYPE, "dtype %d is not supported", dtype);
     int rc = check_groups(channels, out_channels, groups);
@@ -2008,7 +2027,7 @@ int ntg_convnd_backward_dev(int dtype, const void* image, const void* kernel, co
     }
     if (batch == 0 || out_channels == 0 || channels == 0) return NTG_OK;
     if (!kernel || !grad_out || (d_kernel && !image)) return fail(NTG_ERR_INVALID_ARGUMENT, "null pointer");
-    int64_t need = u.total * es;
+    int64_t need = u.total * es + (d_kernel ? complex_dkernel_extra(dtype, batch, out_channels, (channels / groups) * u.taps, u.total * es) : 0);
     if (ndim == 3) {
         const Geo3 g = geo_from(u);
         const ConvBackwardPlan plan = plan_conv_backward_g(dtype, d_image != nullptr, d_kernel != nullptr, batch, channels, out_channels, g, groups);
@@ -2039,17 +2058,8 @@ int ntg_convnd_backward_dev(int dtype, const void* image, const void* kernel, co
     if (d_kernel) {
         hipError_t e = ntg::launch_unfoldnd(es, image, ws, u, static_cast<hipStream_t>(stream));
         if (e != hipSuccess) return hip_fail(e, "unfoldnd launch");
-        for (int64_t g = 0; g < groups; ++g)
-            for (int64_t b = 0; b < batch; ++b) {
-                std::memset(&d, 0, sizeof d);
-                d.dtype = dtype; d.transpose_b = 1;
-                d.c_mode = (b == 0 && !accumulate) ? NTG_C_OVERWRITE : NTG_C_ACCUMULATE;
-                d.m = og; d.k = L; d.n = add;
-                d.lda = L; d.ldb = L; d.ldc = add; d.batches = 1;
-                rc = ntg_gemm_dev(&d, gy + ((b * out_channels + g * og) * L) * es, ws + ((b * u.ccol + g * add) * L) * es,
-                                  static_cast<char*>(d_kernel) + g * og * add * es, stream);
-                if (rc) return rc;
-            }
+        rc = conv_dkernel_from_col(dtype, gy, ws, d_kernel, batch, out_channels, u.ccol, groups, L, accumulate, stream);
+        if (rc) return rc;
     }
     if (d_image) {
         for (int64_t g = 0; g < groups; ++g) {
@@ -2101,7 +2111,6 @@ int ntg_conv_transposend_dev(int dtype, const void* input, const void* kernel, v
                              int64_t batch, int64_t in_channels, int64_t out_channels, int ndim, const int64_t* in_size,
                              const int64_t* kernel_size, const int64_t* stride, const int64_t* padding, const int64_t* dilation,
                              const int64_t* output_padding, int64_t groups, void* stream) {
-    if (int rcx = reject_complex(dtype, "ntg_conv_transposend_dev")) return rcx;
     if (ntg::elem_size(dtype) == 0) return fail(NTG_ERR_UNSUPPORTED_DTYPE, "dtype %d is not supported", dtype);
     int rc = check_groups(in_channels, out_channels, groups);
     if (rc) return rc;
@@ -2150,7 +2159,6 @@ int ntg_convnd(int dtype, const void* image, const void* kernel, void* out, int6
 int ntg_convnd_backward(int dtype, const void* image, const void* kernel, const void* grad_out, void* d_image, void* d_kernel,
                         int64_t batch, int64_t channels, int64_t out_channels, int ndim, const int64_t* size, const int64_t* kernel_size,
                         const int64_t* stride, const int64_t* padding, const int64_t* dilation, int64_t groups, int accumulate) {
-    if (int rcx = reject_complex(dtype, "ntg_convnd_backward")) return rcx;
     const int64_t es = ntg::elem_size(dtype);
     if (es == 0) return fail(NTG_ERR_UNSUPPORTED_DTYPE, "dtype %d is not supported", dtype);
     int rc = check_groups(channels, out_channels, groups);
@@ -2184,7 +2192,6 @@ int ntg_convnd_backward(int dtype, const void* image, const void* kernel, const 
 int ntg_conv_transposend(int dtype, const void* input, const void* kernel, void* out, int64_t batch, int64_t in_channels, int64_t out_channels,
                          int ndim, const int64_t* in_size, const int64_t* kernel_size, const int64_t* stride, const int64_t* padding,
                          const int64_t* dilation, const int64_t* output_padding, int64_t groups) {
-    if (int rcx = reject_complex(dtype, "ntg_conv_transposend")) return rcx;
     const int64_t es = ntg::elem_size(dtype);
     if (es == 0) return fail(NTG_ERR_UNSUPPORTED_DTYPE, "dtype %d is not supported", dtype);
     int rc = check_groups(in_channels, out_channels, groups);

@@ -22,6 +22,25 @@ __global__ void __launch_bounds__(256) reduce_batch_kernel(const T* __restrict__
 }
 
 
+// The reference's own order for the element types whose sums are checked bit for bit (the complex types):
+// conv_dkernel forms sum(0) of the per-image products first -- item 0, then += item 1, ... in the element type
+// (tensor_files/sum_exp_log.cpp:112-124) -- and adds that sum to d_kernel last (conv.cpp:466-469).
+template <class T>
+__global__ void __launch_bounds__(256) reduce_batch_sum_first_kernel(const T* __restrict__ part, T* __restrict__ out, const int64_t batch,
+                                                                     const int64_t n, const int accumulate) {
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+        T acc = part[i];
+        for (int64_t b = 1; b < batch; ++b) acc += part[b * n + i];
+        if (accumulate) {
+            T o = out[i];
+            o += acc;
+            acc = o;
+        }
+        out[i] = acc;
+    }
+}
+
 // The same ordered sum for per-image weight gradients held channels-last, part[b][o][t][c], into the kernel's own layout
 // out[o][c][t]: threads follow the partial sums (coalesced reads of the large side), the small result is written scattered.
 template <class T, class Acc>
@@ -239,6 +258,9 @@ hipError_t launch_reduce_batch(int dtype, const void* part, void* out, int64_t b
     case DT_F64: hipLaunchKernelGGL((reduce_batch_kernel<double, double>), g, b, 0, s, (const double*)part, (double*)out, batch, n, accumulate); break;
     case DT_F16: hipLaunchKernelGGL((reduce_batch_kernel<_Float16, float>), g, b, 0, s, (const _Float16*)part, (_Float16*)out, batch, n, accumulate); break;
     case DT_BF16: hipLaunchKernelGGL((reduce_batch_kernel<__bf16, float>), g, b, 0, s, (const __bf16*)part, (__bf16*)out, batch, n, accumulate); break;
+    case DT_C32: hipLaunchKernelGGL((reduce_batch_sum_first_kernel<LanePair<_Float16>>), g, b, 0, s, (const LanePair<_Float16>*)part, (LanePair<_Float16>*)out, batch, n, accumulate); break;
+    case DT_C64: hipLaunchKernelGGL((reduce_batch_sum_first_kernel<LanePair<float>>), g, b, 0, s, (const LanePair<float>*)part, (LanePair<float>*)out, batch, n, accumulate); break;
+    case DT_C128: hipLaunchKernelGGL((reduce_batch_sum_first_kernel<LanePair<double>>), g, b, 0, s, (const LanePair<double>*)part, (LanePair<double>*)out, batch, n, accumulate); break;
     default: return hipErrorInvalidValue;
     }
     return hipGetLastError();

@@ -250,6 +250,10 @@ hipError_t launch_col2imnd(int dtype, const void* col, void* im, const UnfoldNdP
     case DT_I16: case DT_U16: hipLaunchKernelGGL((col2imnd_kernel<uint16_t, uint16_t>), g, b, 0, s, (const uint16_t*)col, (uint16_t*)im, u, accumulate); break;
     case DT_I32: case DT_U32: hipLaunchKernelGGL((col2imnd_kernel<uint32_t, uint32_t>), g, b, 0, s, (const uint32_t*)col, (uint32_t*)im, u, accumulate); break;
     case DT_I64: case DT_U64: hipLaunchKernelGGL((col2imnd_kernel<uint64_t, uint64_t>), g, b, 0, s, (const uint64_t*)col, (uint64_t*)im, u, accumulate); break;
+    // complex: the two lanes of an element are added separately in the lane's type, taps in the same ascending order
+    case DT_C32: hipLaunchKernelGGL((col2imnd_kernel<LanePair<_Float16>, LanePair<_Float16>>), g, b, 0, s, (const LanePair<_Float16>*)col, (LanePair<_Float16>*)im, u, accumulate); break;
+    case DT_C64: hipLaunchKernelGGL((col2imnd_kernel<LanePair<float>, LanePair<float>>), g, b, 0, s, (const LanePair<float>*)col, (LanePair<float>*)im, u, accumulate); break;
+    case DT_C128: hipLaunchKernelGGL((col2imnd_kernel<LanePair<double>, LanePair<double>>), g, b, 0, s, (const LanePair<double>*)col, (LanePair<double>*)im, u, accumulate); break;
     default: return hipErrorInvalidValue;
     }
     return hipGetLastError();
@@ -294,6 +298,9 @@ hipError_t launch_col2im(int dtype, const void* col, void* im,
         case DT_I16: case DT_U16: launch_col2im_fast<uint16_t, uint16_t>(col, im, q, accumulate, s); break;
         case DT_I32: case DT_U32: launch_col2im_fast<uint32_t, uint32_t>(col, im, q, accumulate, s); break;
         case DT_I64: case DT_U64: launch_col2im_fast<uint64_t, uint64_t>(col, im, q, accumulate, s); break;
+        case DT_C32: launch_col2im_fast<LanePair<_Float16>, LanePair<_Float16>>(col, im, q, accumulate, s); break;
+        case DT_C64: launch_col2im_fast<LanePair<float>, LanePair<float>>(col, im, q, accumulate, s); break;
+        case DT_C128: launch_col2im_fast<LanePair<double>, LanePair<double>>(col, im, q, accumulate, s); break;
         default: return hipErrorInvalidValue;
         }
         return hipGetLastError();
@@ -310,6 +317,9 @@ hipError_t launch_col2im(int dtype, const void* col, void* im,
     case DT_I16: case DT_U16: hipLaunchKernelGGL((col2im_kernel<uint16_t, uint16_t>), g, b, 0, s, (const uint16_t*)col, (uint16_t*)im, u, accumulate); break;
     case DT_I32: case DT_U32: hipLaunchKernelGGL((col2im_kernel<uint32_t, uint32_t>), g, b, 0, s, (const uint32_t*)col, (uint32_t*)im, u, accumulate); break;
     case DT_I64: case DT_U64: hipLaunchKernelGGL((col2im_kernel<uint64_t, uint64_t>), g, b, 0, s, (const uint64_t*)col, (uint64_t*)im, u, accumulate); break;
+    case DT_C32: hipLaunchKernelGGL((col2im_kernel<LanePair<_Float16>, LanePair<_Float16>>), g, b, 0, s, (const LanePair<_Float16>*)col, (LanePair<_Float16>*)im, u, accumulate); break;
+    case DT_C64: hipLaunchKernelGGL((col2im_kernel<LanePair<float>, LanePair<float>>), g, b, 0, s, (const LanePair<float>*)col, (LanePair<float>*)im, u, accumulate); break;
+    case DT_C128: hipLaunchKernelGGL((col2im_kernel<LanePair<double>, LanePair<double>>), g, b, 0, s, (const LanePair<double>*)col, (LanePair<double>*)im, u, accumulate); break;
     default: return hipErrorInvalidValue;
     }
     return hipGetLastError();

@@ -29,6 +29,7 @@ I8, I16, I32, I64 = 7, 8, 9, 10
 U8, U16, U32 = 12, 13, 14
 BF16, U64 = 100, 101
 C32, C64, C128 = 4, 5, 6          # interleaved (re, im) pairs; numpy carries them as real arrays with a trailing axis of 2
+F16_LANE8 = 200                   # closed form only: float16 values with k tiles of 8 -- one lane of a Complex32 product
 _COMPLEX_REAL = {C32: np.dtype(np.float16), C64: np.dtype(np.float32), C128: np.dtype(np.float64)}
 
 _NP_TO_DT = {
@@ -93,9 +94,14 @@ def from_bf16_bits(b):
     return (np.ascontiguousarray(b, dtype=np.uint16).astype(np.uint32) << 16).view(np.float32)
 
 
+_HALF_AS_COMPLEX32_LANE = [False]
+
+
 def dtype_code(arr, dt=None):
     if dt is not None:
         return dt
+    if _HALF_AS_COMPLEX32_LANE[0] and arr.dtype == np.float16:
+        return F16_LANE8
     return _NP_TO_DT[arr.dtype]
 
 
@@ -256,6 +262,39 @@ def linear_backward(x, w, bias_shape, grad, ta=False, tb=False, dt=None, kind="c
     return dx, dw, db
 
 
+def _batch_ordered_sum(per_item):
+    """sum(0) as the reference forms it (tensor_files/sum_exp_log.cpp:112-124): item 0, then += item 1, ... in the element
+    type (float16 sums round after every addition)."""
+    acc = per_item[0].copy()
+    for b in range(1, per_item.shape[0]):
+        acc = acc + per_item[b]
+    return acc
+
+
+def complex_lanes(fn, dt, *arrays, **kw):
+    """A convolution of the complex dtypes, restated plane by plane.  The reference's complex matmult works lane-wise on
+    interleaved (re, im) pairs -- one real product of the real parts, one of the imaginary parts, see matmult2d_complex --
+    and unfold / its adjoint / element-wise sums move or add whole elements lane by lane, so the whole unfold -> matmult
+    pipeline on complex tensors is the same pipeline on the plane of real parts and on the plane of imaginary parts, each in
+    the lane's real type: float32 chains for Complex64, float64 for Complex128, and for Complex32 half values with float
+    chains rounded to half every 8 k (the complex_32 tile, not Float16's 16).  `arrays`: complex tensors as real arrays with
+    a trailing axis of 2; fn(*planes, **kw) is one of this module's real convolution functions; its result (an array or a
+    tuple of arrays) comes back with the lanes stacked on a new trailing axis."""
+    real = _COMPLEX_REAL[dt]
+    outs = []
+    prev = _HALF_AS_COMPLEX32_LANE[0]
+    _HALF_AS_COMPLEX32_LANE[0] = dt == C32
+    try:
+        for lane in (0, 1):
+            planes = [np.ascontiguousarray(np.asarray(a, dtype=real)[..., lane]) for a in arrays]
+            outs.append(fn(*planes, **kw))
+    finally:
+        _HALF_AS_COMPLEX32_LANE[0] = prev
+    if isinstance(outs[0], tuple):
+        return tuple(np.stack([outs[0][i], outs[1][i]], axis=-1) for i in range(len(outs[0])))
+    return np.stack(outs, axis=-1)
+
+
 def out_hw(h, w, k, s, p, d):
     return ((h + 2 * p[0] - d[0] * (k[0] - 1) - 1) // s[0] + 1,
             (w + 2 * p[1] - d[1] * (k[1] - 1) - 1) // s[1] + 1)
@@ -288,8 +327,11 @@ def unfold2d_backward(col, output_size, kernel_size, dilation=1, padding=0, stri
     B = col.shape[0]
     C = col.shape[1] // (k[0] * k[1]) if channels is None else channels
     H, W = output_size
+    if col.dtype not in (np.float32, np.float64):
+        # the same scatter-add, taps in ascending order, in the element type (float16 sums round after every addition)
+        return unfoldnd_backward(col.reshape(B, -1, col.shape[-1]), (H, W), k, d, p, s)
     im = np.zeros((B, C, H, W), dtype=col.dtype)
-    rc = lib().oracle_unfold2d_backward(dtype_code(col), _ptr(col), _ptr(im), B, C, H, W,
+    rc = lib().oracle_unfold2d_backward(_NP_TO_DT[col.dtype], _ptr(col), _ptr(im), B, C, H, W,
                                         k[0], k[1], s[0], s[1], p[0], p[1], d[0], d[1])
     if rc:
         raise RuntimeError("oracle unfold2d_backward failed")
@@ -344,7 +386,7 @@ def conv2d_backward(image, kernel, grad, stride=1, padding=0, dilation=1, groups
         dcol[:, g * add:(g + 1) * add, :] = matmult(wg, gg, None, True, False, kind=kind)
         colg = np.ascontiguousarray(col[:, g * add:(g + 1) * add, :])
         per_item = matmult(gg, colg, None, False, True, kind=kind)   # [B, og, add]
-        dk[g * og:(g + 1) * og] = per_item.sum(axis=0)
+        dk[g * og:(g + 1) * og] = _batch_ordered_sum(per_item)
     dimg = unfold2d_backward(dcol, (H, W), (kh, kw), d, p, s, channels=C)
     return dimg, dk.reshape(kernel.shape)
 
@@ -501,7 +543,7 @@ def convnd_backward(image, kernel, grad, stride=1, padding=0, dilation=1, groups
         gg = np.ascontiguousarray(g3[:, g * og:(g + 1) * og, :])
         dcol[:, g * add:(g + 1) * add, :] = matmult(wg, gg, None, True, False, kind=kind)
         colg = np.ascontiguousarray(col[:, g * add:(g + 1) * add, :])
-        dk[g * og:(g + 1) * og] = matmult(gg, colg, None, False, True, kind=kind).sum(axis=0)
+        dk[g * og:(g + 1) * og] = _batch_ordered_sum(matmult(gg, colg, None, False, True, kind=kind))
     dimg = unfoldnd_backward(dcol, x.shape[2:], w.shape[2:], dilation, padding, stride)
     return dimg, dk.reshape(w.shape)
 

@@ -88,7 +88,7 @@ float oracle_bf16_to_f32(uint16_t h) { return bits_f32((uint32_t)h << 16); }
 int64_t oracle_elem_size(int dt) {
     switch (dt) {
     case OR_I8: case OR_U8: return 1;
-    case OR_F16: case OR_BF16: case OR_I16: case OR_U16: return 2;
+    case OR_F16: case OR_F16_LANE8: case OR_BF16: case OR_I16: case OR_U16: return 2;
     case OR_F32: case OR_I32: case OR_U32: return 4;
     case OR_F64: case OR_I64: case OR_U64: return 8;
     case OR_C32: return 4;
@@ -152,13 +152,13 @@ static void closed_f64(const double* A, const double* Bkn, double* C, int64_t m,
 /* Float16: lanes are fp32 inside a 16-wide k tile; C is widened on load and
  * narrowed (RNE) on store once per k tile (nt_matmult_simde.hpp:316-349 with
  * tile_size 16 = 2*pack 8, simde_traits_avx2.h:1130-1132). */
-static void closed_f16(const uint16_t* A, const uint16_t* Bkn, uint16_t* C, int64_t m, int64_t k, int64_t n, int ta) {
+static void closed_f16_tile(const uint16_t* A, const uint16_t* Bkn, uint16_t* C, int64_t m, int64_t k, int64_t n, int ta, int64_t tile) {
 #pragma omp parallel for schedule(static)
     for (int64_t i = 0; i < m; ++i) {
         float* acc = (float*)malloc((size_t)n * sizeof(float));
         uint16_t* c = C + i * n;
-        for (int64_t k0 = 0; k0 < k; k0 += 16) {
-            const int64_t k1 = (k0 + 16 < k) ? k0 + 16 : k;
+        for (int64_t k0 = 0; k0 < k; k0 += tile) {
+            const int64_t k1 = (k0 + tile < k) ? k0 + tile : k;
             for (int64_t j = 0; j < n; ++j) acc[j] = oracle_f16_to_f32(c[j]);
             for (int64_t kk = k0; kk < k1; ++kk) {
                 const float a = oracle_f16_to_f32(A[A_IDX(i, kk)]);
@@ -169,6 +169,15 @@ static void closed_f16(const uint16_t* A, const uint16_t* Bkn, uint16_t* C, int6
         }
         free(acc);
     }
+}
+
+static void closed_f16(const uint16_t* A, const uint16_t* Bkn, uint16_t* C, int64_t m, int64_t k, int64_t n, int ta) {
+    closed_f16_tile(A, Bkn, C, m, k, n, ta, 16);
+}
+/* One lane (the real parts, or the imaginary parts) of a complex_32 product on its own: the same half values and float
+ * chains as closed_c32 below, k tiles of 8 (OR_F16_LANE8; used to restate the complex convolutions plane by plane). */
+static void closed_f16_lane8(const uint16_t* A, const uint16_t* Bkn, uint16_t* C, int64_t m, int64_t k, int64_t n, int ta) {
+    closed_f16_tile(A, Bkn, C, m, k, n, ta, 8);
 }
 
 /* BFloat16 (this build's extension, no reference function): fp32 chain over
@@ -276,6 +285,7 @@ int oracle_matmult(int dt, const void* A, const void* B, void* C,
     case OR_F32: closed_f32((const float*)A, (const float*)Bkn, (float*)C, m, k, n, ta); break;
     case OR_F64: closed_f64((const double*)A, (const double*)Bkn, (double*)C, m, k, n, ta); break;
     case OR_F16: closed_f16((const uint16_t*)A, (const uint16_t*)Bkn, (uint16_t*)C, m, k, n, ta); break;
+    case OR_F16_LANE8: closed_f16_lane8((const uint16_t*)A, (const uint16_t*)Bkn, (uint16_t*)C, m, k, n, ta); break;
     case OR_BF16: closed_bf16((const uint16_t*)A, (const uint16_t*)Bkn, (uint16_t*)C, m, k, n, ta); break;
     case OR_I8: case OR_U8: closed_u8((const uint8_t*)A, (const uint8_t*)Bkn, (uint8_t*)C, m, k, n, ta); break;
     case OR_I16: case OR_U16: closed_u16((const uint16_t*)A, (const uint16_t*)Bkn, (uint16_t*)C, m, k, n, ta); break;

@@ -55,7 +55,8 @@ enum oracle_dtype {
     OR_C32 = 4, OR_C64 = 5, OR_C128 = 6,      /* interleaved (re, im) pairs of half / float / double */
     OR_I8 = 7, OR_I16 = 8, OR_I32 = 9, OR_I64 = 10,
     OR_U8 = 12, OR_U16 = 13, OR_U32 = 14,
-    OR_BF16 = 100, OR_U64 = 101
+    OR_BF16 = 100, OR_U64 = 101,
+    OR_F16_LANE8 = 200                        /* oracle_matmult only: half values, float chains rounded to half every 8 k (one lane of complex_32) */
 };
 
 int64_t oracle_elem_size(int dtype);

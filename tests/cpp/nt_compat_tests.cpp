@@ -221,6 +221,45 @@ static void device_cases(const std::string& g) {
                     nt::utils::throw_exception(o.data<double>()[2 * (i * 5 + j) + part] == sum, "Complex128 matmult is the lane-wise fused chain, bit for bit");
                 }
     });
+    // tests/src/conv_test.cpp:175-189, :216-279: conv1d, conv3d and the transposed convolutions over every floating and complex dtype
+    run_test("conv1d / conv3d / conv_transpose1d / 2d / 3d dtype sweep (floating and complex)", [] {
+        for (DType dt : {DType::Float32, DType::Float64, DType::Float16, DType::BFloat16, DType::Complex32, DType::Complex64, DType::Complex128}) {
+            const std::string name = nt::dtype_name(dt);
+            Tensor x1 = F::randn({1, 3, 10}, dt, 71), w1 = F::randn({2, 3, 3}, dt, 72);
+            Tensor y1 = nt::conv1d(x1, w1, 1, 1);
+            nt::utils::throw_exception(!x1.is_null() && y1.shape() == SizeRef({1, 2, 10}) && y1.dtype() == dt, "conv1d for " + name);
+            Tensor x3 = F::randn({1, 3, 8, 8, 8}, dt, 73), w3 = F::randn({4, 3, 3, 3, 3}, dt, 74);
+            Tensor y3 = nt::conv3d(x3, w3, {1, 1, 1}, {1, 1, 1});
+            nt::utils::throw_exception(!x3.is_null() && y3.shape() == SizeRef({1, 4, 8, 8, 8}) && y3.dtype() == dt, "conv3d for " + name);
+            Tensor xt1 = F::randn({1, 3, 10}, dt, 75), wt1 = F::randn({3, 2, 3}, dt, 76);
+            Tensor yt1 = nt::conv_transpose1d(xt1, wt1, 1, 1);
+            nt::utils::throw_exception(!xt1.is_null() && yt1.shape() == SizeRef({1, 2, 10}) && yt1.dtype() == dt, "conv_transpose1d for " + name);
+            Tensor xt2 = F::randn({1, 3, 16, 16}, dt, 77), wt2 = F::randn({3, 4, 3, 3}, dt, 78);
+            Tensor yt2 = nt::conv_transpose2d(xt2, wt2, {1, 1}, {1, 1});
+            nt::utils::throw_exception(!xt2.is_null() && yt2.shape() == SizeRef({1, 4, 16, 16}) && yt2.dtype() == dt, "conv_transpose2d for " + name);
+            Tensor xt3 = F::randn({1, 3, 8, 8, 8}, dt, 79), wt3 = F::randn({3, 4, 3, 3, 3}, dt, 80);
+            Tensor yt3 = nt::conv_transpose3d(xt3, wt3, {1, 1, 1}, {1, 1, 1});
+            nt::utils::throw_exception(!xt3.is_null() && yt3.shape() == SizeRef({1, 4, 8, 8, 8}) && yt3.dtype() == dt, "conv_transpose3d for " + name);
+        }
+        // Complex64 conv3d and conv_transpose2d: every plane is the real operation on that plane (the reference's lane-wise product)
+        Tensor x = F::randn({2, 4, 4, 5, 6}, DType::Complex64, 81), w = F::randn({6, 2, 2, 3, 2}, DType::Complex64, 82);
+        Tensor y = nt::conv3d(x, w, {1, 2, 1}, {1, 0, 1}, {1, 1, 1}, 2);
+        Tensor xt = F::randn({2, 4, 5, 6}, DType::Complex64, 83), wt = F::randn({4, 3, 3, 2}, DType::Complex64, 84);
+        Tensor yt = nt::conv_transpose2d(xt, wt, {2, 2}, {1, 1}, {1, 1}, {1, 1}, 2);
+        auto plane = [](const Tensor& t, int part) {
+            Tensor r(t.shape(), DType::Float32);
+            for (int64_t i = 0; i < r.numel(); ++i) r.data<float>()[i] = t.data<float>()[2 * i + part];
+            return r;
+        };
+        for (int part = 0; part < 2; ++part) {
+            Tensor yr = nt::conv3d(plane(x, part), plane(w, part), {1, 2, 1}, {1, 0, 1}, {1, 1, 1}, 2);
+            for (int64_t i = 0; i < yr.numel(); ++i)
+                nt::utils::throw_exception(std::fabs(yr.data<float>()[i] - y.data<float>()[2 * i + part]) <= 1e-4, "complex conv3d plane differs from the real convolution");
+            Tensor ytr = nt::conv_transpose2d(plane(xt, part), plane(wt, part), {2, 2}, {1, 1}, {1, 1}, {1, 1}, 2);
+            for (int64_t i = 0; i < ytr.numel(); ++i)
+                nt::utils::throw_exception(std::fabs(ytr.data<float>()[i] - yt.data<float>()[2 * i + part]) <= 1e-4, "complex conv_transpose2d plane differs from the real one");
+        }
+    });
     run_test("matmult transposed view == flag (no copy)", [] {
         Tensor a = F::randn({6, 40, 30}, DType::Float32, 33), b = F::randn({6, 20, 30}, DType::Float32, 34);
         Tensor o1 = nt::matmult(a, b, false, true);

@@ -108,3 +108,64 @@ def test_complex32_rounds_to_half_every_8_k():
         g = oracle.matmult2d_complex(stored(a, ta), stored(b, tb), c0.copy(), ta, tb, oracle.C32)
         assert g.tobytes() == got.tobytes()
         assert oracle.matmult2d_complex(stored(a, ta), stored(b, tb), c0.copy(), ta, tb, oracle.C32, kind="naive").tobytes() == got.tobytes()
+
+
+def test_one_lane_of_a_complex32_product_is_the_half_product_with_k_tiles_of_8():
+    """F16_LANE8 (half values, float chains rounded to half every 8 k) on the plane of real parts and on the plane of
+    imaginary parts == the two lanes of the Complex32 product, bit for bit, with C0 and every flag pair: what lets the
+    complex convolutions be restated plane by plane (oracle.complex_lanes)."""
+    rng = np.random.default_rng(77)
+    for (m, k, n) in [(3, 5, 4), (9, 8, 7), (17, 41, 12), (6, 64, 10)]:
+        for ta, tb in TRANS:
+            a = rng.standard_normal((m, k, 2)).astype(np.float16)
+            b = rng.standard_normal((k, n, 2)).astype(np.float16)
+            c0 = rng.standard_normal((m, n, 2)).astype(np.float16)
+            sa, sb = stored(a, ta), stored(b, tb)
+            want = oracle.matmult2d_complex(sa, sb, c0.copy(), ta, tb, oracle.C32)
+            for lane in (0, 1):
+                got = oracle.matmult2d(np.ascontiguousarray(sa[..., lane]), np.ascontiguousarray(sb[..., lane]),
+                                       np.ascontiguousarray(c0[..., lane]), ta, tb, dt=oracle.F16_LANE8)
+                assert got.tobytes() == np.ascontiguousarray(want[..., lane]).tobytes(), (m, k, n, ta, tb, lane)
+            # ... and it is not Float16's own schedule (tiles of 16) once k passes 8
+            if k > 8:
+                f16 = oracle.matmult2d(np.ascontiguousarray(sa[..., 0]), np.ascontiguousarray(sb[..., 0]), np.ascontiguousarray(c0[..., 0]), ta, tb)
+                assert f16.tobytes() != np.ascontiguousarray(want[..., 0]).tobytes() or k <= 16
+
+
+@pytest.mark.parametrize("dt", list(CODES))
+def test_complex_convolutions_plane_by_plane_equal_unfold_then_complex_matmult(dt):
+    """oracle.complex_lanes(oracle.conv2d / convnd) against the direct statement of the reference's lowering: unfold the
+    complex image (whole elements move), then the complex matmult per group (conv.cpp:69-118, :134-174)."""
+    real = CODES[dt]
+    rng = np.random.default_rng(5)
+    for (B, C, H, W, O, kr, kc, s, p, dil, groups) in [(2, 4, 7, 6, 6, 3, 2, 1, 1, 1, 2), (1, 3, 9, 9, 4, 3, 3, 2, 1, 1, 1)]:
+        x = (rng.standard_normal((B, C, H, W, 2)) * 0.5).astype(real)
+        w = (rng.standard_normal((O, C // groups, kr, kc, 2)) * 0.5).astype(real)
+        got = oracle.complex_lanes(oracle.conv2d, dt, x, w, stride=s, padding=p, dilation=dil, groups=groups)
+        col = np.stack([oracle.unfold2d(np.ascontiguousarray(x[..., q]), (kr, kc), dilation=dil, padding=p, stride=s) for q in (0, 1)], axis=-1)
+        cg, og, taps = C // groups, O // groups, kr * kc
+        want = np.empty((B, O, col.shape[2], 2), real)
+        for bi in range(B):
+            for g in range(groups):
+                w2d = np.ascontiguousarray(w[g * og:(g + 1) * og].reshape(og, cg * taps, 2))
+                want[bi, g * og:(g + 1) * og] = oracle.matmult2d_complex(w2d, np.ascontiguousarray(col[bi, g * cg * taps:(g + 1) * cg * taps]), dt=dt)
+        assert got.reshape(want.shape).tobytes() == want.tobytes(), (dt, B, C, H, W)
+    # three spatial axes
+    x = (rng.standard_normal((2, 4, 4, 5, 6, 2)) * 0.5).astype(real)
+    w = (rng.standard_normal((6, 2, 2, 3, 2, 2)) * 0.5).astype(real)
+    got = oracle.complex_lanes(oracle.convnd, dt, x, w, stride=(1, 2, 1), padding=(1, 0, 1), dilation=1, groups=2)
+    cols = [oracle.unfoldnd(np.ascontiguousarray(x[..., q]), (2, 3, 2), 1, (1, 0, 1), (1, 2, 1))[0] for q in (0, 1)]
+    col = np.stack(cols, axis=-1)
+    want = np.empty((2, 6, col.shape[2], 2), real)
+    for bi in range(2):
+        for g in range(2):
+            w2d = np.ascontiguousarray(w[g * 3:(g + 1) * 3].reshape(3, 24, 2))
+            want[bi, g * 3:(g + 1) * 3] = oracle.matmult2d_complex(w2d, np.ascontiguousarray(col[bi, g * 24:(g + 1) * 24]), dt=dt)
+    assert got.reshape(want.shape).tobytes() == want.tobytes()
+
+
+def test_batch_ordered_sum_rounds_after_every_addition_in_half():
+    """the weight gradient adds the per-image products item by item in the element type (sum_exp_log.cpp:112-124)"""
+    per = np.array([[2048.0], [1.0], [1.0], [1.0]], np.float16)        # 2048 + 1 rounds back to 2048 in half, three times over
+    assert float(oracle._batch_ordered_sum(per)[0]) == 2048.0
+    assert float(per.astype(np.float32).sum()) == 2051.0
