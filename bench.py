@@ -398,7 +398,9 @@ def main():
         import numpy as np
         vp = lambda x: x.ctypes.data_as(ctypes.c_void_p)
 
-        def host_entry(name, m, k, n, batch, note):
+        def host_entry(name, m, k, n, batch, note, zero_c=False):
+            """zero_c: C is zeroed before every call (outside the timed span) -- what functional::matmult hands to nt_matmult
+            (zeros, then accumulate); otherwise every call accumulates onto the previous result, so C is uploaded too"""
             if only and name not in only:
                 return
             rng = np.random.default_rng(7)
@@ -412,17 +414,24 @@ def main():
                 pa, pb, pc = arr(ha), arr(hb), arr(hc)
                 call = lambda: _lib.check(lib.ntg_matmult_batch(_lib.FLOAT32, pa, pb, pc, batch, m, k, k, n, 0, 0))
             call(); call()
-            reps = 0
-            t0 = time.perf_counter()
-            while reps < 3 or (time.perf_counter() - t0 < 0.2 and reps < 200):
+            reps, spent, t_begin = 0, 0.0, time.perf_counter()
+            while reps < 3 or (time.perf_counter() - t_begin < 0.3 and reps < 200):
+                if zero_c:
+                    hc.fill(0.0)
+                t0 = time.perf_counter()
                 call()
+                spent += time.perf_counter() - t0
                 reps += 1
-            ms = (time.perf_counter() - t0) / reps * 1e3
+            ms = spent / reps * 1e3
             extras[name] = {"ms": round(ms, 4), "rate": round(2.0 * batch * m * k * n / (ms * 1e-3) / 1e12, 3), "unit": "TFLOP/s", "calls": reps, "note": note}
 
         host_entry("c1_fp32_512_host_pointer_entry", 512, 512, 512, 1, "ntg_matmult: 3 MiB host->device, 1 MiB device->host")
-        host_entry("c2a_fp32_b32_host_pointer_entry", 1024, 768, 1024, 32, "ntg_matmult_batch, 32 items: 320 MiB host->device, 128 MiB device->host")
         host_entry("c3_fp32_4096_host_pointer_entry", N, N, N, 1, "ntg_matmult: 192 MiB host->device, 64 MiB device->host")
+        host_entry("c3_fp32_4096_host_pointer_entry_zero_c", N, N, N, 1, "ntg_matmult on a zeroed C (functional::matmult's call): C is found to be zeros "
+                   "and not uploaded, 128 MiB host->device, 64 MiB device->host", zero_c=True)
+        host_entry("c2a_fp32_b32_host_pointer_entry", 1024, 768, 1024, 32, "ntg_matmult_batch, 32 items: 320 MiB host->device, 128 MiB device->host")
+        host_entry("c2a_fp32_b32_host_pointer_entry_zero_c", 1024, 768, 1024, 32, "ntg_matmult_batch, 32 items, zeroed C: 192 MiB host->device, "
+                   "128 MiB device->host", zero_c=True)
         lib.ntg_release_host_buffers()
     if extras:
         out["extras"] = extras

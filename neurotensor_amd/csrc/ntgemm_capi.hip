@@ -651,6 +651,134 @@ int ntg_matmult(int dtype, const void* A, const void* B, void* C,
     return ntg_matmult_batch(dtype, As, Bs, Cs, 1, a_rows, a_cols, b_rows, b_cols, transpose_a, transpose_b);
 }
 
+// The host-pointer seam, pipelined: large operands cross the link in panels so that uploads, products and downloads
+// overlap (the link is full duplex and the kernel is short beside the transfers).
+//   one product:  B first (and A whole when it is stored [k][m]), then panels of rows: A's rows and C's rows up, the
+//                 panel's product on a second stream, its rows of C down on a third while the next panels go up;
+//   a batch of distinct matrices (or one shared A or B): the same with groups of items as panels.
+// A C that is all zeros in the caller's memory (what functional::matmult hands over: zeros, then accumulate,
+// matmult_cpu.cpp:110, :707) is not uploaded; the products overwrite instead, which gives the same bits (the sums start
+// from +0 either way).  Panels are products of their own, so this form is taken only where that cannot change a bit: no
+// workspace form exists for the whole product (a split along k would depend on the panel's rows), more than 32 rows.
+// Returns -1 when the call is not one for this form (nothing has been done then).
+static int matmult_host_pipelined(int dtype, const void* const* A, const void* const* B, void* const* C, int64_t batches,
+                                  int64_t m, int64_t k, int64_t n, int ta, int tb) {
+    const int64_t es = ntg::elem_size(dtype);
+    const size_t a_bytes = (size_t)(m * k * es), b_bytes = (size_t)(k * n * es), c_bytes = (size_t)(m * n * es);
+    if ((a_bytes + b_bytes + c_bytes) * (size_t)batches < ((size_t)48 << 20)) return -1;
+    ntg_gemm_desc d;
+    std::memset(&d, 0, sizeof d);
+    d.dtype = dtype; d.transpose_a = ta; d.transpose_b = tb;
+    d.m = m; d.k = k; d.n = n; d.batches = 1;
+    const size_t a_slot = align_up(a_bytes, 256), b_slot = align_up(b_bytes, 256), c_slot = align_up(c_bytes, 256);
+    std::vector<ntg::HostSession::Range> up;
+    if (batches == 1) {
+        if (m < 1024 || ntg_gemm_workspace_bytes(&d) != 0) return -1;
+        // rows per panel: multiples of 256, about 16 MiB of A and C rows together, at least four panels
+        int64_t rows = (int64_t)(((size_t)16 << 20) / (size_t)((k + n) * es)) / 256 * 256;
+        rows = std::max<int64_t>(256, std::min<int64_t>(rows, (m / 4) / 256 * 256));
+        // (the rows that are left over join the last panel: a panel of 32 rows or fewer would run on the streaming kernel,
+        //  whose sums over k have another order)
+        const int panels = (int)std::max<int64_t>(1, m / rows);
+        auto panel_rows = [&](int p) { return p == panels - 1 ? m - (int64_t)p * rows : rows; };
+        ntg::HostSession mem;
+        HIP_TRY(mem.reserve(a_slot + b_slot + c_slot));
+
+        const size_t oa = 0, ob = a_slot, oc = a_slot + b_slot;
+        // B (and an A stored [k][m]: a panel of rows of op(A) is a column block of the stored matrix) go first; C is looked
+        // at while the stagers are busy with them
+        up.push_back({ob, B[0], b_bytes, 0});
+        if (ta) up.push_back({oa, A[0], a_bytes, 0});
+        HIP_TRY(mem.begin_uploads(up.data(), up.size(), 1));
+        const bool zero = ntg::HostSession::all_zero(C[0], c_bytes);
+        HIP_TRY(mem.end_uploads());
+        up.clear();
+        for (int p = 0; p < panels; ++p) {
+            const int64_t m0 = p * rows, mr = panel_rows(p);
+            if (!ta) up.push_back({oa + (size_t)(m0 * k * es), static_cast<const char*>(A[0]) + m0 * k * es, (size_t)(mr * k * es), p});
+            if (!zero) up.push_back({oc + (size_t)(m0 * n * es), static_cast<const char*>(C[0]) + m0 * n * es, (size_t)(mr * n * es), p});
+        }
+        HIP_TRY(mem.begin_uploads(up.data(), up.size(), panels));
+        d.lda = ta ? m : k;
+        d.c_mode = zero ? NTG_C_OVERWRITE : NTG_C_ACCUMULATE;
+        for (int p = 0; p < panels; ++p) {
+            const int64_t m0 = p * rows, mr = panel_rows(p);
+            const size_t c_off = (size_t)(m0 * n * es);
+            HIP_TRY(mem.uploaded_through(p));
+            d.m = mr;
+            const int rc = ntg_gemm_dev(&d, mem.at(oa + (size_t)((ta ? m0 : m0 * k) * es)), mem.at(ob), mem.at(oc + c_off), mem.compute_stream());
+            if (rc) return rc;
+            HIP_TRY(mem.download_async(static_cast<char*>(C[0]) + c_off, oc + c_off, (size_t)(mr * n * es), mem.compute_stream()));
+        }
+        HIP_TRY(mem.end_uploads());
+        HIP_TRY(mem.finish_downloads());
+        return NTG_OK;
+    }
+    // a batch: distinct A, B, C per item, or one B (or one A) for all
+    if (m <= 32) return -1;
+    bool a_same = true, b_same = true;
+    for (int64_t i = 1; i < batches; ++i) { a_same = a_same && A[i] == A[0]; b_same = b_same && B[i] == B[0]; }
+    {
+        std::map<const void*, int64_t> seen;
+        for (int64_t i = 0; i < batches && !a_same; ++i)
+            if (!seen.emplace(A[i], i).second) return -1;
+        seen.clear();
+        for (int64_t i = 0; i < batches && !b_same; ++i)
+            if (!seen.emplace(B[i], i).second) return -1;
+        seen.clear();
+        for (int64_t i = 0; i < batches; ++i)
+            if (!seen.emplace(C[i], i).second) return -1;          // (aliasing outputs: the general path reports it)
+    }
+    const size_t per_item = (a_same ? 0 : a_bytes) + (b_same ? 0 : b_bytes) + c_bytes;
+    int64_t group = std::max<int64_t>(1, (int64_t)(((size_t)24 << 20) / per_item));
+    group = std::min(group, std::max<int64_t>(1, batches / 4));
+    const int panels = (int)((batches + group - 1) / group);
+    d.batches = group;
+    d.stride_a = a_same ? 0 : (int64_t)(a_slot / (size_t)es);
+    d.stride_b = b_same ? 0 : (int64_t)(b_slot / (size_t)es);
+    d.stride_c = (int64_t)(c_slot / (size_t)es);
+    if (a_slot % (size_t)es || b_slot % (size_t)es || c_slot % (size_t)es) return -1;
+    const int64_t ws_bytes = ntg_gemm_workspace_bytes(&d);          // (planned per item: the same form for any group size)
+    if (ws_bytes < 0) return -1;
+    const size_t na = a_same ? 1 : (size_t)batches, nb = b_same ? 1 : (size_t)batches;
+    const size_t oa = 0, ob = na * a_slot, oc = ob + nb * b_slot, ow = oc + (size_t)batches * c_slot;
+    ntg::HostSession mem;
+    HIP_TRY(mem.reserve(ow + (size_t)ws_bytes));
+    // the shared operand and the first group's A and B go first; the outputs are looked at while the stagers are busy with them
+    if (a_same) up.push_back({oa, A[0], a_bytes, 0});
+    if (b_same) up.push_back({ob, B[0], b_bytes, 0});
+    for (int64_t i = 0; i < std::min(group, batches); ++i) {
+        if (!a_same) up.push_back({oa + (size_t)i * a_slot, A[i], a_bytes, 0});
+        if (!b_same) up.push_back({ob + (size_t)i * b_slot, B[i], b_bytes, 0});
+    }
+    HIP_TRY(mem.begin_uploads(up.data(), up.size(), 1));
+    bool zero = true;
+    for (int64_t i = 0; i < batches && zero; ++i) zero = ntg::HostSession::all_zero(C[i], c_bytes);
+    HIP_TRY(mem.end_uploads());
+    up.clear();
+    for (int64_t i = 0; i < batches; ++i) {
+        const int p = (int)(i / group);
+        if (!a_same && p > 0) up.push_back({oa + (size_t)i * a_slot, A[i], a_bytes, p});
+        if (!b_same && p > 0) up.push_back({ob + (size_t)i * b_slot, B[i], b_bytes, p});
+        if (!zero) up.push_back({oc + (size_t)i * c_slot, C[i], c_bytes, p});
+    }
+    HIP_TRY(mem.begin_uploads(up.data(), up.size(), panels));
+    if (ws_bytes > 0) { d.workspace = mem.at(ow); d.workspace_bytes = ws_bytes; }
+    d.c_mode = zero ? NTG_C_OVERWRITE : NTG_C_ACCUMULATE;
+    for (int p = 0; p < panels; ++p) {
+        const int64_t i0 = p * group, cnt = std::min(group, batches - i0);
+        HIP_TRY(mem.uploaded_through(p));
+        d.batches = cnt;
+        const int rc = ntg_gemm_dev(&d, mem.at(oa + (a_same ? 0 : (size_t)i0 * a_slot)), mem.at(ob + (b_same ? 0 : (size_t)i0 * b_slot)),
+                                    mem.at(oc + (size_t)i0 * c_slot), mem.compute_stream());
+        if (rc) return rc;
+        for (int64_t i = i0; i < i0 + cnt; ++i) HIP_TRY(mem.download_async(C[i], oc + (size_t)i * c_slot, c_bytes, mem.compute_stream()));
+    }
+    HIP_TRY(mem.end_uploads());
+    HIP_TRY(mem.finish_downloads());
+    return NTG_OK;
+}
+
 int ntg_matmult_batch(int dtype, const void* const* A, const void* const* B, void* const* C,
                       int64_t batches, int64_t a_rows, int64_t a_cols, int64_t b_rows, int64_t b_cols,
                       int transpose_a, int transpose_b) {
@@ -664,6 +792,9 @@ int ntg_matmult_batch(int dtype, const void* const* A, const void* const* B, voi
     if (!A || !B || !C) return fail(NTG_ERR_INVALID_ARGUMENT, "null pointer array");
     for (int64_t i = 0; i < batches; ++i)
         if (!A[i] || !B[i] || !C[i]) return fail(NTG_ERR_INVALID_ARGUMENT, "null matrix pointer in item %lld", (long long)i);
+    rc = matmult_host_pipelined(dtype, A, B, C, batches, m, k, n, transpose_a, transpose_b);
+    if (rc >= 0) return rc;
+    rc = NTG_OK;
 
     const size_t a_bytes = (size_t)(m * k * es), b_bytes = (size_t)(k * n * es), c_bytes = (size_t)(m * n * es);
     // every distinct input matrix gets one slot in a single device arena

@@ -1162,3 +1162,48 @@ def test_item_is_the_same_alone_and_in_every_batch_form(dtype, shape):
 def alone_np(a, b):
     """one product on device tensors through the functional face, as a numpy array"""
     return from_torch(F.matmult(a, b))
+
+
+def test_host_entry_pipelined_panels_and_groups_bit_identical_to_the_device_entry():
+    """Host-pointer calls of 48 MiB and more cross the link in panels (rows of one product, groups of items of a batch):
+    uploads on one stream, the panels' products on a second, downloads on a third.  Every storage form, a C that is
+    zeros (not uploaded: the products overwrite) and one that is not (uploaded, accumulated), 16-bit operands, a last panel
+    that is not whole, a batch with distinct matrices and one with a shared B -- each bit-identical to the device entry
+    point on the whole product / batch."""
+    lib = _lib.load()
+    rng = np.random.default_rng(616)
+    st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    for (m, k, n, dtype, ta, tb) in [(3100, 2000, 2600, np.float32, False, False), (2900, 2100, 2500, np.float32, True, False),
+                                      (3000, 2056, 2504, np.float32, False, True), (5000, 3000, 4104, "bf16", False, False),
+                                      (2600, 1500, 2200, np.float64, True, True)]:
+        a, b, sa, sb, c0 = make_inputs(rng, m, k, n, dtype, ta, tb)
+        for zero in (False, True):
+            start = np.zeros_like(c0) if zero else c0
+            want = dev_matmult(sa, sb, start, m, k, n, ta, tb, dtype)
+            got = host_matmult(sa, sb, start.copy(), m, k, n, ta, tb, code_of(dtype))
+            assert got.tobytes() == want.tobytes(), (m, k, n, dtype, ta, tb, zero)
+    # batches: 9 items of 1000 x 1100 x 1200 (groups of two; the last group has one), distinct and with one B for all
+    nb, m, k, n = 9, 1000, 1100, 1200
+    As = [rng.standard_normal((m, k)).astype(np.float32) for _ in range(nb)]
+    Bs = [rng.standard_normal((k, n)).astype(np.float32) for _ in range(nb)]
+    arr = lambda xs: (ctypes.c_void_p * len(xs))(*[x.ctypes.data for x in xs])
+    for shared_b in (False, True):
+        for zero in (False, True):
+            C0 = [np.zeros((m, n), np.float32) if zero else rng.standard_normal((m, n)).astype(np.float32) for _ in range(nb)]
+            Bl = [Bs[0]] * nb if shared_b else Bs
+            got = [c.copy() for c in C0]
+            _lib.check(lib.ntg_matmult_batch(_lib.FLOAT32, arr(As), arr(Bl), arr(got), nb, m, k, k, n, 0, 0))
+            # the device entry on the whole batch
+            da = torch.from_numpy(np.stack(As)).to(DEV)
+            db = torch.from_numpy(Bs[0] if shared_b else np.stack(Bs)).to(DEV)
+            dc = torch.from_numpy(np.stack(C0)).to(DEV)
+            d = _lib.GemmDesc()
+            d.dtype, d.c_mode = _lib.FLOAT32, _lib.C_ACCUMULATE
+            d.m, d.k, d.n, d.batches = m, k, n, nb
+            d.stride_a, d.stride_b, d.stride_c = m * k, 0 if shared_b else k * n, m * n
+            _lib.check(lib.ntg_gemm_dev(ctypes.byref(d), da.data_ptr(), db.data_ptr(), dc.data_ptr(), st))
+            torch.cuda.synchronize()
+            want = dc.cpu().numpy()
+            for i in range(nb):
+                assert got[i].tobytes() == want[i].tobytes(), ("batch", shared_b, zero, i)
+    assert lib.ntg_release_host_buffers() == 0
