@@ -372,6 +372,28 @@ def main():
         # one round of 256 tiles of 128 x 256 (the square tiles give 128 or 512)
         run("mid_bf16_2048x4096x4096", G(torch.bfloat16, 2048, 4096, 4096, scale=0.05, mode=_lib.C_OVERWRITE), 2.0 * 2048 * 4096 * 4096,
             PEAK_TFLOPS["bf16"])
+        # a batch as a strided launch and as device pointer tables whose entries the caller vouches for (ntg_gemm_ptrs_dev with
+        # NTG_GEMM_PTRS_ALIGNED16: the same DMA-fed kernels; without the vouch the register-staged ones)
+        fb = 2.0 * 32 * 1024 ** 3
+        run("batch_bf16_32x1024_strided", G(torch.bfloat16, 1024, 1024, 1024, batch=32, scale=0.05, mode=_lib.C_OVERWRITE), fb, PEAK_TFLOPS["bf16"])
+
+        def ptr_tables(vouch):
+            def make():
+                a = (torch.randn(32, 1024, 1024, device=dev) * 0.05).bfloat16()
+                b = (torch.randn(32, 1024, 1024, device=dev) * 0.05).bfloat16()
+                c = torch.zeros(32, 1024, 1024, device=dev, dtype=torch.bfloat16)
+                tab = torch.tensor([x[i].data_ptr() for x in (a, b, c) for i in range(32)], dtype=torch.int64, device=dev)
+                d = _lib.GemmDesc()
+                d.dtype, d.c_mode, d.m, d.k, d.n, d.batches = _lib.BFLOAT16, _lib.C_OVERWRITE, 1024, 1024, 1024, 32
+                d.flags = _lib.GEMM_PTRS_ALIGNED16 if vouch else 0
+                call = lambda: _lib.check(lib.ntg_gemm_ptrs_dev(ctypes.byref(d), tab.data_ptr(), tab.data_ptr() + 256, tab.data_ptr() + 512, stream))
+                call.keep = (a, b, c, tab, d)
+                return call
+            return make
+        run("batch_bf16_32x1024_pointer_tables_vouched", ptr_tables(True), fb, PEAK_TFLOPS["bf16"])
+        run("batch_bf16_32x1024_pointer_tables", ptr_tables(False), fb, PEAK_TFLOPS["bf16"])
+        # rows that are not 16-byte multiples: operands copied into zero-padded rows in the workspace, then the DMA-fed kernel
+        run("c3_fp32_4096x4001x4096_padded_copies", G(torch.float32, N, 4001, N, mode=_lib.C_OVERWRITE), 2.0 * N * 4001 * N, PEAK_TFLOPS["fp32"])
         fc = 2.0 * 200704 * 2304 * 256
 
         def conv_case(half, backward):

@@ -186,7 +186,10 @@ typedef struct ntg_gemm_desc {
 #define NTG_GEMM_PTRS_ALIGNED16 1
 
 /* Bytes of workspace with which ntg_gemm_dev runs its faster form (0: there is none for this product): a split along k
- * for shapes such as [256, 8192] x [8192, 8192], or, for large Int16 / Int32 / Int64 products and their unsigned forms, the
+ * for shapes such as [256, 8192] x [8192, 8192] (planned from one item's sizes, so a batch is offered its item's split with
+ * the partial sums of every item); zero-padded copies of large 8-bit, 16-bit, Float32 and Float64 operands whose rows, pitches
+ * or base pointers are not 16-byte multiples, so that they run on the DMA-fed kernels (same results: zeros add nothing);
+ * or, for large Int16 / Int32 / Int64 products and their unsigned forms, the
  * 3 / 10 / 36 products of balanced byte planes on v_mfma_i32_32x32x32_i8, whose sum modulo 2^W is the reference's wrapping
  * result (nt/mp/simde_traits/simde_traits_avx2.h:810-812, :444-446, :523-540: multiply and add in the element type).  Without a workspace the same result is computed by the
  * plain kernels.  The reference has no counterpart: its k loop is always serial (nt_matmult.hpp:196). */

@@ -342,7 +342,7 @@ hipError_t launch_reduce_batch_taps_last(int dtype, const void* part, void* out,
                                          int64_t taps, int accumulate, hipStream_t s);   // part rows hold cgp >= cg channels per tap
 hipError_t launch_flip_weights(int64_t elem_size, const void* w, void* wt, int64_t groups, int64_t og, int64_t cg, int64_t taps, hipStream_t s);
 
-// padded copies of operands whose rows are not 16-byte multiples (pad_copy.hip); es = 1 or 2 bytes per element, sizes in elements
+// padded copies of operands whose rows are not 16-byte multiples (pad_copy.hip); es = 1, 2, 4 or 8 bytes per element, sizes in elements
 hipError_t launch_pad_copy(int64_t es, const void* src, int64_t ld_src, int64_t s_src, void* dst, int64_t ld_dst, int64_t s_dst,
                            int64_t rows, int64_t cols, int64_t rows_dst, int64_t batch, hipStream_t s);
 hipError_t launch_unpad_copy(int64_t es, const void* src, int64_t ld_src, int64_t s_src, void* dst, int64_t ld_dst, int64_t s_dst,

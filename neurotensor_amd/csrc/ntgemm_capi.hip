@@ -255,8 +255,8 @@ static int run_int_planes(const ntg::GemmParams& p, const IntPlanesPlan& pl, boo
 }
 
 // Padded copies.  The DMA-fed kernels need 16-byte rows (leading dimensions, batch strides, base pointers, and K, N -- M
-// under transpose_a -- multiples of one 16-byte chunk); an 8- or 16-bit product that misses this falls to the vector ALU
-// (8-bit: 40 x slower) or the register-staged kernel (16-bit: half the rate).  With a workspace the operands that need it
+// under transpose_a -- multiples of one 16-byte chunk); a product that misses this falls to the vector ALU
+// (8-bit: 40 x slower) or the register-staged kernel (16-bit: half the rate; Float32 / Float64: 0.8 - 0.85 of it).  With a workspace the operands that need it
 // are copied into rows padded with zeros to whole chunks (zero products add nothing: bit-identical integers, the same
 // single rounding for the 16-bit floats), the product runs on the DMA-fed kernel, and a result whose own rows are not
 // 16-byte multiples is computed into a padded copy and copied back.  Taken for products large enough to repay the copies.
@@ -270,10 +270,13 @@ static PadPlan plan_pad(const ntg::GemmParams& p, int dtype, bool ta, bool tb) {
     PadPlan pl;
     std::memset(&pl, 0, sizeof pl);
     const bool half = dtype == ntg::DT_F16 || dtype == ntg::DT_BF16, byte = dtype == ntg::DT_I8 || dtype == ntg::DT_U8;
-    if ((!half && !byte) || p.Aptr || p.Bptr || p.Cptr || p.M <= 32) return pl;
-    const int64_t es = half ? 2 : 1, ve = 16 / es;
+    const bool wide = dtype == ntg::DT_F32 || dtype == ntg::DT_F64;
+    if ((!half && !byte && !wide) || p.Aptr || p.Bptr || p.Cptr || p.M <= 32) return pl;
+    const int64_t es = ntg::elem_size(dtype), ve = 16 / es;
+    // from where the faster kernel repays the copies: 8-bit against the vector ALU (40 x), 16-bit against the register-staged
+    // kernel at half the rate, Float32 / Float64 against the register-staged kernel at 0.8 - 0.85 of the DMA-fed one
     const double macs = (double)p.M * p.N * p.K * p.batch;
-    if (macs < (half ? 2147483648.0 : 268435456.0)) return pl;
+    if (macs < (byte ? 268435456.0 : half ? 2147483648.0 : dtype == ntg::DT_F32 ? 4294967296.0 : 8589934592.0)) return pl;
     auto up = [&](int64_t v) { return (v + ve - 1) / ve * ve; };
     pl.Kp = (int)up(p.K); pl.Np = (int)up(p.N); pl.Mp = ta ? (int)up(p.M) : p.M;
     auto misaligned = [&](const void* ptr, int64_t ld, int64_t stride) {

@@ -1,4 +1,4 @@
-// Copies that bring operands with rows that are not 16-byte multiples onto the DMA-fed kernels: the matrix is copied into
+// Copies that bring operands (1, 2, 4 or 8 bytes per element) with rows that are not 16-byte multiples onto the DMA-fed kernels: the matrix is copied into
 // a workspace with its rows padded to whole 16-byte chunks (zeros in the padding, which add nothing to any sum), the
 // product runs on the copies, and a result whose own rows are not 16-byte multiples is copied back.  HBM bound; one lane
 // per 16 bytes of the padded side.
@@ -89,6 +89,8 @@ hipError_t launch_pad_copy(int64_t es, const void* src, int64_t ld_src, int64_t 
     const dim3 g((unsigned)gx, (unsigned)gy), t(256);
     if (es == 1) hipLaunchKernelGGL(pad_copy_kernel<uint8_t>, g, t, 0, s, (const uint8_t*)src, ld_src, s_src, (uint8_t*)dst, ld_dst, s_dst, rows, cols, rows_dst, batch, sh);
     else if (es == 2) hipLaunchKernelGGL(pad_copy_kernel<uint16_t>, g, t, 0, s, (const uint16_t*)src, ld_src, s_src, (uint16_t*)dst, ld_dst, s_dst, rows, cols, rows_dst, batch, sh);
+    else if (es == 4) hipLaunchKernelGGL(pad_copy_kernel<uint32_t>, g, t, 0, s, (const uint32_t*)src, ld_src, s_src, (uint32_t*)dst, ld_dst, s_dst, rows, cols, rows_dst, batch, sh);
+    else if (es == 8) hipLaunchKernelGGL(pad_copy_kernel<uint64_t>, g, t, 0, s, (const uint64_t*)src, ld_src, s_src, (uint64_t*)dst, ld_dst, s_dst, rows, cols, rows_dst, batch, sh);
     else return hipErrorInvalidValue;
     return hipGetLastError();
 }
@@ -103,6 +105,8 @@ hipError_t launch_unpad_copy(int64_t es, const void* src, int64_t ld_src, int64_
     const dim3 g((unsigned)gx, (unsigned)gy), t(256);
     if (es == 1) hipLaunchKernelGGL(unpad_copy_kernel<uint8_t>, g, t, 0, s, (const uint8_t*)src, ld_src, s_src, (uint8_t*)dst, ld_dst, s_dst, rows, cols, batch, sh);
     else if (es == 2) hipLaunchKernelGGL(unpad_copy_kernel<uint16_t>, g, t, 0, s, (const uint16_t*)src, ld_src, s_src, (uint16_t*)dst, ld_dst, s_dst, rows, cols, batch, sh);
+    else if (es == 4) hipLaunchKernelGGL(unpad_copy_kernel<uint32_t>, g, t, 0, s, (const uint32_t*)src, ld_src, s_src, (uint32_t*)dst, ld_dst, s_dst, rows, cols, batch, sh);
+    else if (es == 8) hipLaunchKernelGGL(unpad_copy_kernel<uint64_t>, g, t, 0, s, (const uint64_t*)src, ld_src, s_src, (uint64_t*)dst, ld_dst, s_dst, rows, cols, batch, sh);
     else return hipErrorInvalidValue;
     return hipGetLastError();
 }
@@ -114,6 +118,8 @@ hipError_t launch_bias_fill(int64_t es, const void* bias, int64_t bs, int64_t rs
     const dim3 g(grid_for(total)), t(256);
     if (es == 1) hipLaunchKernelGGL(bias_fill_kernel<uint8_t>, g, t, 0, s, (const uint8_t*)bias, bs, rs, cs, (uint8_t*)dst, ld_dst, s_dst, rows, cols, rows_dst, batch);
     else if (es == 2) hipLaunchKernelGGL(bias_fill_kernel<uint16_t>, g, t, 0, s, (const uint16_t*)bias, bs, rs, cs, (uint16_t*)dst, ld_dst, s_dst, rows, cols, rows_dst, batch);
+    else if (es == 4) hipLaunchKernelGGL(bias_fill_kernel<uint32_t>, g, t, 0, s, (const uint32_t*)bias, bs, rs, cs, (uint32_t*)dst, ld_dst, s_dst, rows, cols, rows_dst, batch);
+    else if (es == 8) hipLaunchKernelGGL(bias_fill_kernel<uint64_t>, g, t, 0, s, (const uint64_t*)bias, bs, rs, cs, (uint64_t*)dst, ld_dst, s_dst, rows, cols, rows_dst, batch);
     else return hipErrorInvalidValue;
     return hipGetLastError();
 }

@@ -183,15 +183,15 @@ def test_16bit_results_are_rounded_once_on_ragged_k(name):
     run_case(rng, name, 520, 1544, 776, False, False, (0, 0, 0), _lib.C_ACCUMULATE, one_rounding=True)      # 256-wide tiles, ragged everywhere
 
 
-@pytest.mark.parametrize("name", ["bf16", "f16", "i8", "u8"])
+@pytest.mark.parametrize("name", ["bf16", "f16", "i8", "u8", "f32", "f64"])
 def test_rows_that_are_not_16_byte_multiples_through_padded_copies(name):
-    """Large 8- and 16-bit products whose pitches, sizes or base pointers miss the 16-byte rule are offered a workspace
-    (ntg_gemm_workspace_bytes) with which the operands are copied into zero-padded rows and the DMA-fed kernel runs:
+    """Large 8-bit, 16-bit, Float32 and Float64 products whose pitches, sizes or base pointers miss the 16-byte rule are offered
+    a workspace (ntg_gemm_workspace_bytes) with which the operands are copied into zero-padded rows and the DMA-fed kernel runs:
     every flag pair, the three C modes, batches with a broadcast operand, odd k / n / m and odd base pointers;
-    integers bit-exact against the oracle, 16-bit floats held to one rounding."""
+    integers bit-exact against the oracle, 16-bit floats held to one rounding, Float32 / Float64 within their bound."""
     rng = np.random.default_rng(8100 + list(DTYPES).index(name))
-    half = name in FLOATS
-    m, k, n = (1304, 1001, 1702) if half else (520, 1001, 530)
+    half = name in ("bf16", "f16")
+    m, k, n = (1304, 1001, 1702) if half else (1700, 1501, 1702) if name == "f32" else (2100, 2001, 2053) if name == "f64" else (520, 1001, 530)
     modes = (_lib.C_ACCUMULATE, _lib.C_BIAS, _lib.C_OVERWRITE, _lib.C_ACCUMULATE)
     for (ta, tb), mode in zip(TRANS, modes):
         run_case(rng, name, m, k, n, ta, tb, (0, 0, 0), mode, workspace=True, one_rounding=half)             # odd k: A and B padded, C as it lies
