@@ -43,6 +43,7 @@
 #include "gemm_mfma_impl.h"
 
 #include <type_traits>
+#include <cstdlib>
 
 namespace ntg {
 
@@ -230,11 +231,11 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
     const int wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
 
-    const int lid = xcd_contiguous_id(blockIdx.x, gridDim.x);
+    const int lid = p.group_m < 0 ? (int)blockIdx.x : xcd_contiguous_id(blockIdx.x, gridDim.x);      // (group_m != 0: measurement only, see ring_tile_order_override)
     const int tiles = p.tiles_m * p.tiles_n;
     const int b = lid / tiles;
     int tm, tn;
-    tile_coords(lid - b * tiles, p.tiles_m, p.tiles_n, 4, tm, tn);
+    tile_coords(lid - b * tiles, p.tiles_m, p.tiles_n, p.group_m > 0 ? p.group_m : p.group_m < 0 ? -p.group_m : 4, tm, tn);
     const int m0 = tm * GA::BM, n0 = tn * G::BN;
 
     // (pointer tables: one uniform load per operand; everything below is base + offset either way)
@@ -1023,6 +1024,14 @@ static inline bool ring_eligible(const GemmParams& p, bool ta, int es = 2) {
            ((reinterpret_cast<uintptr_t>(p.C) & 15) == 0);
 }
 
+// Measurement knob (read once): NTG_TILE_GROUP_M = g makes groups of g tile rows instead of 4 in the tile order of the plain
+// products (with 32 CUs per XCD: 4 -> every XCD works on 4 x 8 tiles at a time, 2 -> 2 x 16, 8 -> 8 x 4 ...); a negative
+// value also deals the workgroups to the XCDs round-robin as the hardware numbers them.  Results do not depend on it.
+static inline int ring_tile_order_override() {
+    static const int v = [] { const char* e = getenv("NTG_TILE_GROUP_M"); return e ? atoi(e) : 0; }();
+    return v;
+}
+
 // WBN != 0: rectangular tiles of 64 WB rows x 64 WBN columns
 template <int DT, bool TA, bool TB, int WB, int WBN = 0, int KD = 1>
 static hipError_t launch_ring_cfg(const GemmParams& pin, hipStream_t s) {
@@ -1031,6 +1040,7 @@ static hipError_t launch_ring_cfg(const GemmParams& pin, hipStream_t s) {
     GemmParams p = pin;
     p.tiles_m = (p.M + TEM - 1) / TEM;
     p.tiles_n = (p.N + TEN - 1) / TEN;
+    p.group_m = ring_tile_order_override();
     const int64_t blocks = (int64_t)p.tiles_m * p.tiles_n * p.batch;
     if (blocks > 0x7fffffffLL) return hipErrorInvalidValue;
     if (p.M % TEM == 0 && p.N % TEN == 0 && p.K % BK == 0)

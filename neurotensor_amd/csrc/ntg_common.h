@@ -87,6 +87,7 @@ struct GemmParams {
     int vecA_ok, vecB_ok;    // 16-byte vector loads are legal for every row of A / B
     int ptrs_aligned;        // pointer tables only: the caller vouches that every entry is a multiple of 16 bytes (the tables
                              // live in device memory, the host cannot look); lets table batches onto the DMA-fed kernels
+    int group_m;             // DMA-fed kernels: tile rows per group of the tile order (0: the default, 4; see tile_coords)
     int act;                 // ACT_RELU: the stored result is max(result, 0) (relu_ of the reference = clamp_(x, 0): NaN and -0 become +0);
                              // honoured by the DMA-fed Float16 / BFloat16 / Float32 kernels and the split-K reduction only
     ConvGeom conv;           // used by the implicit-im2col kernels only: B = image, op(B) = col or col^T
