@@ -460,10 +460,11 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
     // output pixels of consecutive images, and one more division gives the image, p.conv.fold_stride elements apart.
     int krow4[WB], noff4[WB];
     uint32_t tap4[WB];
-    int k4_k = 0;
+    int k4_k = 0, k4_base = 0;
     if constexpr (GATHERW) {
         const ConvGeom& g = p.conv;
         constexpr int CH = G::CHUNKS;
+        if (g.k_ranges) k4_base = b * p.K;                         // this item's first output pixel, counted through the images
         const uint32_t cgc = (uint32_t)(g.n_total ? g.n_total : p.N) / (uint32_t)g.k_rc;   // channels of the slice: N = taps * channels
 #pragma unroll
         for (int x = 0; x < WB; ++x) {
@@ -483,7 +484,7 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
         if constexpr (GATHERW) {
             const ConvGeom& g = p.conv;
             const char* img = reinterpret_cast<const char*>(B);
-            const uint32_t l = (uint32_t)(k4_k + krow4[x]);
+            const uint32_t lk = (uint32_t)(k4_k + krow4[x]), l = lk + (uint32_t)k4_base;
             uint32_t li = l, im = 0u;
             if (g.fold_L) {                                        // (uniform)
                 im = fast_div(l, g.div_fold);
@@ -491,7 +492,7 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
             }
             const uint32_t oh = fast_div(li, g.div_wo), ow = li - oh * (uint32_t)g.Wo;
             const int ih0 = (int)oh * g.s_r - g.p_r, iw0 = (int)ow * g.s_c - g.p_c;
-            const bool ok = (l < (uint32_t)p.K) & ((uint32_t)(ih0 + (int)(tap4[x] & 0xffffu)) < (uint32_t)g.H) &
+            const bool ok = (lk < (uint32_t)p.K) & ((uint32_t)(ih0 + (int)(tap4[x] & 0xffffu)) < (uint32_t)g.H) &
                             ((uint32_t)(iw0 + (int)(tap4[x] >> 16)) < (uint32_t)g.W);
             const int off = (int)((oh * (uint32_t)g.s_r * (uint32_t)g.W + ow * (uint32_t)g.s_c) * (uint32_t)g.chan * (uint32_t)ES) + noff4[x];
             const char* src = ok ? img + ((int64_t)im * g.fold_stride * ES + (int64_t)off) : reinterpret_cast<const char*>(ring_zero_word);
@@ -591,7 +592,16 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
     // K-steps past the end are clamped to the last one: the tail iterations then issue the
     // same DMA traffic as the steady state (into stages nobody reads any more), which keeps
     // the loop body free of branches and the vmcnt bookkeeping uniform.
-    auto srcA = [&](int kt) { return tile_src(baseA + (int64_t)(kt < last ? kt : last) * advA); };
+    auto srcA = [&](int kt) {
+        const int kc = kt < last ? kt : last;
+        if constexpr (GATHERW && A_KC) {
+            if (p.conv.a_steps) {                                  // (uniform) K-step counted through the images -> image, step inside it
+                const uint32_t gs = (uint32_t)(b * KT + kc), im = fast_div(gs, p.conv.div_a_steps);
+                return tile_src(baseA + ((int64_t)im * p.conv.a_image_stride * ES + (int64_t)(gs - im * (uint32_t)p.conv.a_steps) * advA));
+            }
+        }
+        return tile_src(baseA + (int64_t)kc * advA);
+    };
     auto srcB = [&](int kt) { return tile_src(baseB + (int64_t)(kt < last ? kt : last) * advB); };
 
     // prologue: tiles 0..2 and the A half of tile 3 in flight (3 (NA + NB) + NA instructions)
@@ -1141,6 +1151,7 @@ static hipError_t launch_ring16_planned(const GemmParams& p, hipStream_t s, Laun
 // of their own (see ring16_column_split); each part planned over the batch like any other
 template <class Launch>
 static hipError_t launch_conv_nhwc16_planned(const GemmParams& p, hipStream_t s, Launch&& launch) {
+    if (p.conv.k_ranges) return launch(ring16_tile_edge(p.M, p.N, p.K, p.batch), p);     // items are k ranges: one launch, planned by the caller
     const int64_t head_cols = p.cmode == C_PARTIAL ? 0 : ring16_column_split(p.M, p.N, p.K, p.batch);
     if (head_cols == 0) return launch_ring16_planned(p, s, launch);
     GemmParams head = p, tail = p;

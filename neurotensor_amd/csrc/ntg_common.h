@@ -62,6 +62,13 @@ struct ConvGeom {
     // channels-last convolution and weight gradient: column n of this launch is column n + n_base of the whole product
     // (a launch on the trailing columns); n_total = columns of the whole product (0: this launch has them all)
     int n_base, n_total;
+    // channels-last weight gradient, items = k ranges: the k axis is the output pixels of ALL images counted through, item b
+    // covers pixels [b K, (b + 1) K) of it (K a whole number of K-steps, and so is an image: a K-step never straddles two).
+    // The gathered operand finds image and pixel by division (fold_L, fold_stride as above); dY, read where it lies as
+    // [image][out channel][pixel], jumps a_image_stride elements after every a_steps K-steps.  0: off.
+    int k_ranges, a_steps;
+    FastDiv div_a_steps;
+    int64_t a_image_stride;
 };
 
 struct GemmParams {

@@ -8,6 +8,7 @@
 
 #include <cstdarg>
 #include <cstdio>
+#include <cstdlib>
 #include <algorithm>
 #include <cstring>
 #include <map>
@@ -1437,6 +1438,52 @@ static int64_t conv_dkernel_fold(int64_t batch, int64_t og, int64_t n, int64_t g
     }
     return best;
 }
+// 16-bit, dY read where it lies: instead of one product per image, the output pixels of all images counted through are cut
+// into `ranges` equal k ranges (whole K-steps; an image is whole K-steps too) so that tiles x ranges fill whole rounds
+// over the CUs: 64 images of a 3 x 3 x 256 x 256 layer on 56 x 56 maps are 9 tiles x 28 ranges = 252 tiles of 7168 pixels
+// in one round (270 us + 10 us for adding 28 partial sums), against 512 + 256 tiles in three rounds (236 + 50 us, + 18 us
+// for 64 partial sums).  Returns the number of ranges, 0: one product per image.
+// The estimate prices the gathering kernel as measured on that layer: 0.37 of a CU's MFMA peak on 256 x 256 tiles, 0.30 on
+// 128 x 128 tiles when two workgroups share a CU and 0.21 when one has it alone; it has to be 5 % ahead.
+static double dkernel16_cost_us(int edge, int64_t tiles, int64_t K) {
+    const double cu_flops_per_us = 9.77e6, area = (double)edge * edge;
+    if (edge == 256) return (double)((tiles + 255) / 256) * (2.0 * area * (double)K / (cu_flops_per_us * 0.37) + 6.0);
+    if (edge == 128) {
+        if (tiles <= 256) return 2.0 * area * (double)K / (cu_flops_per_us * 0.21) + 3.0;
+        return (double)((tiles + 511) / 512) * (4.0 * area * (double)K / (cu_flops_per_us * 0.30) + 3.0);
+    }
+    return (double)((tiles + 1023) / 1024) * (8.0 * area * (double)K / (cu_flops_per_us * 0.2) + 2.0);
+}
+static double dkernel16_plan_cost_us(int64_t M, int64_t N, int64_t K, int64_t batch) {
+    const ntg::Ring16Plan pl = ntg::ring16_plan(M, N, K, batch);
+    if (pl.head >= batch) return dkernel16_cost_us(pl.edge, ntg::ring16_tiles(pl.edge, M, N, batch), K);
+    return dkernel16_cost_us(pl.edge, ntg::ring16_tiles(pl.edge, M, N, pl.head), K) +
+           dkernel16_cost_us(pl.tail_edge, ntg::ring16_tiles(pl.tail_edge, M, N, batch - pl.head), K) + 2.0;
+}
+static int64_t conv_dkernel_ranges(int dtype, int64_t batch, int64_t og, int64_t out_channels, int64_t N, int64_t L) {
+    const int64_t es = ntg::elem_size(dtype), bk = 64 / es;
+    if (es != 2 || batch < 2 || L % bk != 0 || batch * L >= (1LL << 30)) return 0;
+    auto reduce_us = [&](int64_t items) { return 3.0 + (double)items * (double)(out_channels * N * es) / 4.0e6; };
+    const int64_t hc = ntg::ring16_column_split(og, N, L, batch);
+    const double cur = (hc ? dkernel16_plan_cost_us(og, hc, L, batch) + dkernel16_plan_cost_us(og, N - hc, L, batch) + 2.0
+                           : dkernel16_plan_cost_us(og, N, L, batch)) + reduce_us(batch);
+    const int64_t steps = batch * L / bk;
+    // measurement and test knob: NTG_DW_RANGES=r forces r ranges where r is admissible, 0 forces one product per image
+    if (const char* env = std::getenv("NTG_DW_RANGES")) {
+        const int64_t r = std::atoll(env);
+        return r > 0 && r <= batch && steps % r == 0 ? r : 0;
+    }
+    int64_t best = 0;
+    double best_us = 0.95 * cur;
+    for (int64_t r = 1; r <= batch; ++r) {
+        if (steps % r != 0 || steps / r < 16) continue;
+        const int64_t kr = steps / r * bk;
+        const int edge = ntg::ring16_tile_edge(og, N, kr, r);
+        const double us = dkernel16_cost_us(edge, ntg::ring16_tiles(edge, og, N, r), kr) + reduce_us(r);
+        if (us < best_us) { best_us = us; best = r; }
+    }
+    return best;
+}
 static int64_t dkernel_padded_channels(int64_t es, int64_t cg) { const int64_t v = 16 / es; return (cg + v - 1) / v * v; }
 static bool conv_dkernel_nhwc_ok(int dtype, int64_t channels, int64_t out_channels, int64_t groups, const Geo3& g) {
     if (dtype != ntg::DT_F32 && dtype != ntg::DT_F16 && dtype != ntg::DT_BF16) return false;
@@ -1462,7 +1509,8 @@ static int conv_dkernel_nhwc(int dtype, const void* image, const void* grad_out,
     const int64_t cgp = dkernel_padded_channels(es, cg), chp = groups * cgp;      // channels per group / per pixel in the copy
     const int64_t L = g.L(), taps = g.taps(), vol = g.vol(), N = taps * cgp;
     const bool copy_dy = conv_dkernel_nhwc_copies_dy(dtype, out_channels, groups, g);      // dY read as [pixel][out channel] from its own copy
-    const int64_t fold = copy_dy ? conv_dkernel_fold(batch, og, N, groups, L) : 1, items = batch / fold;
+    const int64_t ranges = copy_dy ? 0 : conv_dkernel_ranges(dtype, batch, og, out_channels, N, L);
+    const int64_t fold = copy_dy ? conv_dkernel_fold(batch, og, N, groups, L) : 1, items = ranges ? ranges : batch / fold;
     char* ws_img = static_cast<char*>(ws);
     char* ws_gy = ws_img + align_up((size_t)(batch * chp * vol * es), 256);
     char* ws_part = ws_gy + (copy_dy ? align_up((size_t)(batch * out_channels * L * es), 256) : 0);
@@ -1489,10 +1537,19 @@ static int conv_dkernel_nhwc(int dtype, const void* image, const void* grad_out,
         p.vecA_ok = 1; p.vecB_ok = 1;
         fill_conv_geom(p.conv, cgp, g);
         p.conv.chan = (int)chp;                    // elements from one pixel to the next
-        if (fold > 1) {
+        if (fold > 1 || ranges) {
             p.conv.fold_L = (int)L;
             p.conv.div_fold = ntg::make_fastdiv((uint32_t)L);
             p.conv.fold_stride = chp * vol;
+        }
+        if (ranges) {
+            const int64_t bk = 64 / es;
+            p.K = (int)(batch * L / ranges);
+            p.sA = 0; p.sB = 0;
+            p.conv.k_ranges = 1;
+            p.conv.a_steps = (int)(L / bk);
+            p.conv.div_a_steps = ntg::make_fastdiv((uint32_t)(L / bk));
+            p.conv.a_image_stride = out_channels * L;
         }
         e = ntg::launch_conv_nhwc_dw(dtype, copy_dy, p, hs);
         if (e != hipSuccess) return hip_fail(e, "channels-last conv_dkernel launch");

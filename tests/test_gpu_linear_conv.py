@@ -705,3 +705,29 @@ def test_config5a_conv2d_gradients_full_size():
             assert ex <= 1e-5 * 2304 * float(tg.abs().max() * tw.abs().max())
             assert ew <= 1e-5 * 200704 * float(tg.abs().max() * tx.abs().max())
         del rx, rw, dx, dw
+
+
+@pytest.mark.parametrize("ranges", [1, 3, 4, 6])
+def test_conv2d_weight_gradient_k_ranges_across_images(ranges, monkeypatch):
+    """The 16-bit weight gradient with the output pixels of all images cut into k ranges (forced through the library's
+    NTG_DW_RANGES knob): ranges that end inside an image (4 ranges over 6 images), pairs of images (3), whole images (6) and
+    everything in one (1), against torch autograd in double and against the per-image form; grouped as well."""
+    rng = np.random.default_rng(77 + ranges)
+    for groups, dt in ((1, torch.bfloat16), (2, torch.float16)):
+        x = dev(rng.standard_normal((6, 16, 32, 32)).astype(np.float32)).to(dt)
+        w = dev((rng.standard_normal((32, 16 // groups, 3, 3)) / 12.0).astype(np.float32)).to(dt)
+        g = dev(rng.standard_normal((6, 32, 32, 32)).astype(np.float32)).to(dt)
+        rx = x.double().requires_grad_(True)
+        rw = w.double().requires_grad_(True)
+        torch.nn.functional.conv2d(rx, rw, padding=1, groups=groups).backward(g.double())
+        monkeypatch.setenv("NTG_DW_RANGES", "0")
+        _, dw_images = F.conv2d_backward(x, w, g, stride=1, padding=1, groups=groups)
+        monkeypatch.setenv("NTG_DW_RANGES", str(ranges))
+        _, dw = F.conv2d_backward(x, w, g, stride=1, padding=1, groups=groups)
+        monkeypatch.delenv("NTG_DW_RANGES")
+        tol = HALF_REL * rw.grad.abs().max().item()
+        assert (dw.double() - rw.grad).abs().max().item() <= tol, (groups, ranges)
+        assert (dw.double() - dw_images.double()).abs().max().item() <= tol, (groups, ranges)
+        if ranges == 6:
+            # whole images per range: the same products and the same order of adding them up
+            assert torch.equal(dw, dw_images)
