@@ -192,6 +192,10 @@ __device__ __forceinline__ uint32_t lds_addr_of(const char* p) {
 // are read two quarter-steps ahead (four sets in registers), the whole of tile kt + 3 is fetched during K-step kt.
 // With WBN_ = 4 (128 x 256 tiles) the stages are 48 KiB and there are three of them: tile kt + 2 is fetched from the
 // barrier of K-step kt - 1 (which frees its stage) to the barrier of K-step kt.
+// entries of the weight gradient's LDS table of window origins (16 + 128 KiB beside the 256 x 256 tile's ring; 14 + 64 KiB
+// on the smaller tiles, so that two workgroups still share a CU)
+constexpr int dw_table_entries(int wb) { return wb == 4 ? 6144 : 3584; }
+
 template <int DT, bool TA, bool TB, bool RAGGED, int WB_, int CONV = 0, int WBN_ = 0, int KD_ = 1>
 __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
     using E = Elem<DT>;
@@ -225,6 +229,9 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
     __shared__ __attribute__((aligned(1024))) char st1[STAGE_BYTES];
     __shared__ __attribute__((aligned(1024))) char st2[STAGE_BYTES];
     __shared__ __attribute__((aligned(1024))) char st3[RING3 ? 1024 : STAGE_BYTES];
+    // channels-last weight gradient: byte offset of every output pixel's window origin inside one (bordered) image
+    constexpr int DW_TABLE = CONV == 4 ? dw_table_entries(WB) : 1;
+    __shared__ int dw_tab[DW_TABLE];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -480,10 +487,54 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
             noff4[x] = (((int)(r * (uint32_t)g.d_r) - g.p_r) * g.W + ((int)(q * (uint32_t)g.d_c) - g.p_c)) * g.chan * ES + (int)c * ES;
         }
     }
+    // Table form (p.conv.pix_table = output pixels per image, at most DW_TABLE - BK; the copy of the image carries its padding
+    // as pixels of zeros, so every tap of every window exists): the window origin's byte offset of each output pixel is
+    // computed once per workgroup into LDS, BK entries of zeros behind them.  A K-step then lies inside ONE image (per-image
+    // items, or k ranges whose images are whole K-steps): image and first pixel are wave-uniform counters, a lane reads its
+    // pixel's entry one K-step ahead, and the per-instruction work is two additions instead of two divisions and the tests.
+    int pre4[WB];
+    int t4_pix = 0, t4_pixn = 0;
+    int64_t t4_img = 0, t4_imgn = 0;
+    if constexpr (GATHERW) {
+        const ConvGeom& g = p.conv;
+        if (g.pix_table) {                                        // (uniform)
+            const int Lp = g.pix_table;
+            for (int i = tid; i < Lp + BK; i += 256) {
+                const uint32_t oh = fast_div((uint32_t)i, g.div_wo), ow = (uint32_t)i - oh * (uint32_t)g.Wo;
+                dw_tab[i] = i < Lp ? (int)((oh * (uint32_t)g.s_r * (uint32_t)g.W + ow * (uint32_t)g.s_c) * (uint32_t)g.chan * (uint32_t)ES) : 0;
+            }
+            __syncthreads();
+            if (g.k_ranges) {
+                const uint32_t im0 = fast_div((uint32_t)k4_base, g.div_fold);
+                t4_pix = k4_base - (int)im0 * Lp;
+                t4_img = (int64_t)im0 * g.fold_stride * ES;
+            }
+            t4_pixn = t4_pix + BK;
+            t4_imgn = t4_img;
+            if (g.k_ranges && t4_pixn >= Lp) { t4_pixn -= Lp; t4_imgn += g.fold_stride * ES; }
+#pragma unroll
+            for (int x = 0; x < WB; ++x) pre4[x] = dw_tab[t4_pix + (krow4[x] & 63)];
+        }
+    }
     auto conv4_dma = [&](int x, uint32_t lds_tile) __attribute__((always_inline)) {
         if constexpr (GATHERW) {
             const ConvGeom& g = p.conv;
             const char* img = reinterpret_cast<const char*>(B);
+            if (g.pix_table) {                                     // (uniform)
+                const uint32_t lk = (uint32_t)(k4_k + krow4[x]);
+                const char* src = lk < (uint32_t)p.K ? img + (t4_img + (int64_t)(pre4[x] + noff4[x])) : reinterpret_cast<const char*>(ring_zero_word);
+                asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+                             :: "s"(lds_tile + (uint32_t)(wave_u * WB + x) * 1024u), "v"(src) : "memory");
+                const int pn = t4_pixn < g.pix_table ? t4_pixn : g.pix_table;      // (K-steps past the end: the zeros behind the table)
+                pre4[x] = dw_tab[pn + (krow4[x] & 63)];
+                if (x == WB - 1) {
+                    k4_k += BK;
+                    t4_pix = t4_pixn; t4_img = t4_imgn;
+                    t4_pixn += BK;
+                    if (g.k_ranges && t4_pixn >= g.pix_table) { t4_pixn -= g.pix_table; t4_imgn += g.fold_stride * ES; }
+                }
+                return;
+            }
             const uint32_t lk = (uint32_t)(k4_k + krow4[x]), l = lk + (uint32_t)k4_base;
             uint32_t li = l, im = 0u;
             if (g.fold_L) {                                        // (uniform)
@@ -1114,6 +1165,8 @@ static hipError_t launch_ring_nhwc_dw_cfg(const GemmParams& pin, hipStream_t s) 
     const int64_t blocks = (int64_t)p.tiles_m * p.tiles_n * p.batch;
     if (blocks <= 0) return hipSuccess;
     if (blocks > 0x7fffffffLL) return hipErrorInvalidValue;
+    // (more output pixels per image than the table holds: the divisions per instruction, which serve a bordered copy as well)
+    if (p.conv.pix_table + 64 > dw_table_entries(WB)) p.conv.pix_table = 0;
     hipLaunchKernelGGL((gemm_ring_kernel<DT, TA, false, true, WB, 4>), dim3((unsigned)blocks), dim3(256), 0, s, p);
     return hipGetLastError();
 }

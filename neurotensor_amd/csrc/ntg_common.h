@@ -69,6 +69,9 @@ struct ConvGeom {
     int k_ranges, a_steps;
     FastDiv div_a_steps;
     int64_t a_image_stride;
+    // channels-last weight gradient on a copy that carries the padding as pixels of zeros (H, W describe the padded image,
+    // p_r = p_c = 0): output pixels per image when the kernel keeps their window origins in an LDS table, 0: off
+    int pix_table;
 };
 
 struct GemmParams {

@@ -1441,16 +1441,16 @@ static int64_t conv_dkernel_fold(int64_t batch, int64_t og, int64_t n, int64_t g
 // 16-bit, dY read where it lies: instead of one product per image, the output pixels of all images counted through are cut
 // into `ranges` equal k ranges (whole K-steps; an image is whole K-steps too) so that tiles x ranges fill whole rounds
 // over the CUs: 64 images of a 3 x 3 x 256 x 256 layer on 56 x 56 maps are 9 tiles x 28 ranges = 252 tiles of 7168 pixels
-// in one round (270 us + 10 us for adding 28 partial sums), against 512 + 256 tiles in three rounds (236 + 50 us, + 18 us
+// in one round (235 us + 10 us for adding 28 partial sums), against 512 + 256 tiles in three rounds (217 + 46 us, + 18 us
 // for 64 partial sums).  Returns the number of ranges, 0: one product per image.
-// The estimate prices the gathering kernel as measured on that layer: 0.37 of a CU's MFMA peak on 256 x 256 tiles, 0.30 on
-// 128 x 128 tiles when two workgroups share a CU and 0.21 when one has it alone; it has to be 5 % ahead.
+// The estimate prices the gathering kernel as measured on that layer: 0.41 of a CU's MFMA peak on 256 x 256 tiles, 0.35 on
+// 128 x 128 tiles when two workgroups share a CU and 0.245 when one has it alone; it has to be 5 % ahead.
 static double dkernel16_cost_us(int edge, int64_t tiles, int64_t K) {
     const double cu_flops_per_us = 9.77e6, area = (double)edge * edge;
-    if (edge == 256) return (double)((tiles + 255) / 256) * (2.0 * area * (double)K / (cu_flops_per_us * 0.37) + 6.0);
+    if (edge == 256) return (double)((tiles + 255) / 256) * (2.0 * area * (double)K / (cu_flops_per_us * 0.41) + 6.0);
     if (edge == 128) {
-        if (tiles <= 256) return 2.0 * area * (double)K / (cu_flops_per_us * 0.21) + 3.0;
-        return (double)((tiles + 511) / 512) * (4.0 * area * (double)K / (cu_flops_per_us * 0.30) + 3.0);
+        if (tiles <= 256) return 2.0 * area * (double)K / (cu_flops_per_us * 0.245) + 3.0;
+        return (double)((tiles + 511) / 512) * (4.0 * area * (double)K / (cu_flops_per_us * 0.35) + 3.0);
     }
     return (double)((tiles + 1023) / 1024) * (8.0 * area * (double)K / (cu_flops_per_us * 0.2) + 2.0);
 }
@@ -1485,6 +1485,15 @@ static int64_t conv_dkernel_ranges(int dtype, int64_t batch, int64_t og, int64_t
     return best;
 }
 static int64_t dkernel_padded_channels(int64_t es, int64_t cg) { const int64_t v = 16 / es; return (cg + v - 1) / v * v; }
+// The copy of the image carries the padding as a border of zero pixels where the plain 16-byte copy serves it (whole
+// 16-byte runs of channels): the gather then needs no validity test, and keeps the window origins in a table.
+static HaloPlan dkernel_halo(int64_t es, int64_t cg, int64_t groups, const Geo3& g) {
+    HaloPlan h = conv_halo(g);
+    if (h.on && (dkernel_padded_channels(es, cg) != cg || !conv_nhwc_offsets_fit(groups * cg, es, h.gp))) {
+        h.on = false; h.gp = g; h.vol = g.vol();
+    }
+    return h;
+}
 static bool conv_dkernel_nhwc_ok(int dtype, int64_t channels, int64_t out_channels, int64_t groups, const Geo3& g) {
     if (dtype != ntg::DT_F32 && dtype != ntg::DT_F16 && dtype != ntg::DT_BF16) return false;
     if (g.nd != 2 || !conv_implicit_g(dtype, channels, g)) return false;
@@ -1501,21 +1510,26 @@ static int64_t conv_dkernel_nhwc_workspace(int dtype, int64_t batch, int64_t cha
     const int64_t es = ntg::elem_size(dtype);
     const int64_t gy = conv_dkernel_nhwc_copies_dy(dtype, out_channels, groups, g) ? (int64_t)align_up((size_t)(batch * out_channels * g.L() * es), 256) : 0;
     const int64_t cgp = dkernel_padded_channels(es, channels / groups);
-    return (int64_t)align_up((size_t)(batch * groups * cgp * g.vol() * es), 256) + gy + batch * out_channels * cgp * g.taps() * es;
+    return (int64_t)align_up((size_t)(batch * groups * cgp * dkernel_halo(es, channels / groups, groups, g).vol * es), 256) + gy +
+           batch * out_channels * cgp * g.taps() * es;
 }
 static int conv_dkernel_nhwc(int dtype, const void* image, const void* grad_out, void* d_kernel, void* ws, int64_t batch,
                              int64_t channels, int64_t out_channels, const Geo3& g, int64_t groups, int accumulate, hipStream_t hs) {
     const int64_t es = ntg::elem_size(dtype), cg = channels / groups, og = out_channels / groups;
     const int64_t cgp = dkernel_padded_channels(es, cg), chp = groups * cgp;      // channels per group / per pixel in the copy
     const int64_t L = g.L(), taps = g.taps(), vol = g.vol(), N = taps * cgp;
+    const HaloPlan halo = dkernel_halo(es, cg, groups, g);
+    const int64_t volp = halo.vol;                                                         // pixels per image of the copy
     const bool copy_dy = conv_dkernel_nhwc_copies_dy(dtype, out_channels, groups, g);      // dY read as [pixel][out channel] from its own copy
     const int64_t ranges = copy_dy ? 0 : conv_dkernel_ranges(dtype, batch, og, out_channels, N, L);
     const int64_t fold = copy_dy ? conv_dkernel_fold(batch, og, N, groups, L) : 1, items = ranges ? ranges : batch / fold;
     char* ws_img = static_cast<char*>(ws);
-    char* ws_gy = ws_img + align_up((size_t)(batch * chp * vol * es), 256);
+    char* ws_gy = ws_img + align_up((size_t)(batch * chp * volp * es), 256);
     char* ws_part = ws_gy + (copy_dy ? align_up((size_t)(batch * out_channels * L * es), 256) : 0);
-    hipError_t e = cgp == cg ? ntg::launch_nchw_to_nhwc(es, image, ws_img, batch, channels, vol, hs)
+    bool took_along = false;
+    hipError_t e = cgp == cg ? ntg::launch_nchw_to_nhwc(es, image, ws_img, batch, channels, vol, hs, halo.on ? &halo.hm : nullptr, nullptr, &took_along)
                              : ntg::launch_nchw_to_nhwc_padded(es, image, ws_img, batch, groups, cg, cgp, vol, hs);
+    if (e == hipSuccess && halo.on && volp != vol && !took_along) e = ntg::launch_halo_zero(es, ws_img, batch, chp, halo.hm, hs);
     if (e == hipSuccess && copy_dy) e = ntg::launch_nchw_to_nhwc(es, grad_out, ws_gy, batch, out_channels, L, hs);
     if (e != hipSuccess) return hip_fail(e, "channels-last copy launch");
     for (int64_t gi = 0; gi < groups; ++gi) {
@@ -1532,16 +1546,17 @@ static int conv_dkernel_nhwc(int dtype, const void* image, const void* grad_out,
         p.B = ws_img + gi * cgp * es;
         p.C = ws_part + gi * og * N * es;
         p.ldb = chp; p.ldc = N;
-        p.sA = fold * out_channels * L; p.sB = fold * chp * vol; p.sC = out_channels * N;
+        p.sA = fold * out_channels * L; p.sB = fold * chp * volp; p.sC = out_channels * N;
         p.cmode = ntg::C_OVERWRITE;
         p.vecA_ok = 1; p.vecB_ok = 1;
-        fill_conv_geom(p.conv, cgp, g);
+        fill_conv_geom(p.conv, cgp, halo.gp);
         p.conv.chan = (int)chp;                    // elements from one pixel to the next
         if (fold > 1 || ranges) {
             p.conv.fold_L = (int)L;
             p.conv.div_fold = ntg::make_fastdiv((uint32_t)L);
-            p.conv.fold_stride = chp * vol;
+            p.conv.fold_stride = chp * volp;
         }
+        if (halo.on && fold == 1 && L < (1 << 20)) p.conv.pix_table = (int)L;     // (a K-step inside one image: see the kernel)
         if (ranges) {
             const int64_t bk = 64 / es;
             p.K = (int)(batch * L / ranges);
