@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the matmult hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-extras] [--no-cpu] [--only NAME[,NAME...]]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-extras] [--no-cpu] [--only NAME[,NAME...]] [--context]
 
 One "step" is one pass of nt::matmult over the headline workload of BASELINE.json
 (config 3): a 4096 x 4096 x 4096 BFloat16 product, inputs randn*0.02 already resident in
@@ -49,10 +49,95 @@ def parse_args():
     ap.add_argument("--power", default="", help="comma-separated extras entries that are ALSO run back to back for --power-seconds while amd-smi is "
                                                 "sampled (average socket power, clocks): what the power manager does under each workload")
     ap.add_argument("--power-seconds", type=float, default=2.5)
+    ap.add_argument("--context", action="store_true",
+                    help="also time torch's own operators (hipBLASLt / MIOpen behind torch.matmul, bmm, _int_mm, conv2d) on the same "
+                         "operands, alternating with this library in one process: context for the figures, never part of `value`")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 256 MiB device copy (known HBM traffic) so that counter runs "
                          "(rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE) can be scaled")
     return ap.parse_args()
+
+
+def context_table(torch, F, _lib, lib, dev, stream, make_gemm, settle):
+    """torch's operators on the same operands as this library, same process, alternating: five blocks of back-to-back
+    launches per side after one settling load, the median block's microseconds per launch.  What torch dispatches to
+    (hipBLASLt, rocBLAS, MIOpen) is torch's choice; its outputs are not compared here (the parity tests do that against the
+    oracle)."""
+    table = {}
+
+    def block(fn, n):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(n):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e3 / n
+
+    def compare(name, ours, theirs, op):
+        for fn in (ours, theirs):
+            for _ in range(3):
+                fn()
+        torch.cuda.synchronize()
+        settle("context_" + name)
+        est = max(block(ours, 3), 1.0)
+        n = int(min(max(20, 4000.0 / est), 400))
+        a, b = [], []
+        for _ in range(5):
+            a.append(block(ours, n))
+            b.append(block(theirs, n))
+        a.sort()
+        b.sort()
+        table[name] = {"this_library_us": round(a[2], 2), "torch_us": round(b[2], 2), "torch_op": op, "launches_per_block": n}
+
+    def gemm(name, dtype, m, k, n, tb=False, batch=1, scale=0.05):
+        ours = make_gemm(dtype, m, k, n, tb=tb, batch=batch, scale=scale, mode=_lib.C_OVERWRITE)
+        a, b, c = ours.keep[0], ours.keep[1], ours.keep[2]
+        if batch == 1:
+            a2, b2, c2 = a[0], b[0], torch.empty_like(c[0])
+            theirs = (lambda: torch.matmul(a2, b2.t(), out=c2)) if tb else (lambda: torch.matmul(a2, b2, out=c2))
+            op = "torch.matmul(out=)"
+        else:
+            c2 = torch.empty_like(c)
+            theirs = (lambda: torch.bmm(a, b.transpose(1, 2), out=c2)) if tb else (lambda: torch.bmm(a, b, out=c2))
+            op = "torch.bmm(out=)"
+        compare(name, ours, theirs, op)
+
+    bf, hf, f32, f64 = torch.bfloat16, torch.float16, torch.float32, torch.float64
+    gemm("bf16_4096", bf, 4096, 4096, 4096, scale=0.02)
+    gemm("fp16_4096", hf, 4096, 4096, 4096, scale=0.02)
+    gemm("fp32_4096", f32, 4096, 4096, 4096)
+    gemm("fp64_4096", f64, 4096, 4096, 4096)
+    gemm("fp32_512", f32, 512, 512, 512)
+    gemm("fp32_b32_1024x768x1024", f32, 1024, 768, 1024, batch=32)
+    gemm("bf16_2048", bf, 2048, 2048, 2048)
+    gemm("bf16_3072", bf, 3072, 3072, 3072)
+    gemm("bf16_2048x4096x4096", bf, 2048, 4096, 4096)
+    gemm("bf16_256x4096x11008", bf, 256, 4096, 11008, scale=0.1)
+    gemm("bf16_linear_8192x4096x11008_x_wT", bf, 8192, 4096, 11008, tb=True, scale=0.1)
+    gemm("fp32_linear_8192x4096x11008_x_wT", f32, 8192, 4096, 11008, tb=True, scale=0.1)
+    gemm("bf16_b32_1024", bf, 1024, 1024, 1024, batch=32)
+    gemm("bf16_16x8192x8192", bf, 16, 8192, 8192)
+    gemm("fp32_16x8192x8192", f32, 16, 8192, 8192)
+    if hasattr(torch, "_int_mm"):
+        a = torch.randint(-128, 128, (4096, 4096), device=dev, dtype=torch.int8)
+        b = torch.randint(-128, 128, (4096, 4096), device=dev, dtype=torch.int8)
+        ours = make_gemm(torch.int8, 4096, 4096, 4096, ints=True, mode=_lib.C_OVERWRITE)
+        compare("int8_4096", ours, lambda: torch._int_mm(a, b), "torch._int_mm (int32 result; this library stores the wrapped int8)")
+    for half in (True, False):
+        x = torch.randn(64, 256, 56, 56, device=dev)
+        w = torch.randn(256, 256, 3, 3, device=dev) / 48.0
+        g = torch.randn(64, 256, 56, 56, device=dev)
+        if half:
+            x, w, g = x.bfloat16(), w.bfloat16(), g.bfloat16()
+        tag = "bf16" if half else "fp32"
+        compare("conv2d_64x256x56x56_3x3_" + tag, lambda: F.conv2d(x, w, padding=1), lambda: torch.nn.functional.conv2d(x, w, padding=1),
+                "torch.nn.functional.conv2d")
+        compare("conv2d_backward_64x256x56x56_3x3_" + tag, lambda: F.conv2d_backward(x, w, g, padding=1),
+                lambda: torch.ops.aten.convolution_backward(g, x, w, None, [1, 1], [1, 1], [1, 1], False, [0, 0], 1, [True, True, False]),
+                "aten.convolution_backward (input and weight gradients)")
+        del x, w, g
+    return table
 
 
 def read_traffic_note():
@@ -458,6 +543,8 @@ def main():
         lib.ntg_release_host_buffers()
     if extras:
         out["extras"] = extras
+    if args.context:
+        out["context"] = context_table(torch, F, _lib, lib, dev, stream, make_gemm, settle)
     if only:
         print(json.dumps(out))
         return
