@@ -453,6 +453,28 @@ __global__ void __launch_bounds__(256) gemm_mfma_kernel(const GemmParams p) {
         for (int j = 0; j < WBN; ++j)
 #pragma unroll
             for (int r = 0; r < E::ACCN; ++r) acc[i][j][r] = (AccS)0;
+    // Float32: the accumulators start from C0 (C itself, or the bias): every output element is then the reference's chain
+    // c = C0; c = fma(a_k, b_k, c) in ascending k, bit for bit, as in the DMA-fed kernel; the epilogue only stores.
+    constexpr bool CHAIN_FROM_C0 = std::is_same<T, float>::value;
+    if constexpr (CHAIN_FROM_C0) {
+        if (p.cmode == C_ACCUMULATE || p.cmode == C_BIAS) {            // (uniform)
+            const gptr<T> bias0 = (gptr<T>)static_cast<const T*>(p.bias);
+#pragma unroll
+            for (int i = 0; i < WBM; ++i)
+#pragma unroll
+                for (int j = 0; j < WBN; ++j) {
+                    const int n = n0 + (B_KM ? (wn * WBN + j) * R + lr : (wn * R + lr) * WBN + j);
+#pragma unroll
+                    for (int r = 0; r < E::ACCN; ++r) {
+                        const int lrow = acc_row<R>(r, lane);
+                        const int m = m0 + (A_KM ? (wm * WBM + i) * R + lrow : (wm * R + lrow) * WBM + i);
+                        if (m < p.M && n < p.N)
+                            acc[i][j][r] = p.cmode == C_ACCUMULATE ? (AccS)C[(int64_t)m * p.ldc + n]
+                                                                   : (AccS)bias0[(int64_t)b * p.bias_bs + (int64_t)m * p.bias_rs + (int64_t)n * p.bias_cs];
+                    }
+                }
+        }
+    }
 
     LA la;
     LB lb;
@@ -518,17 +540,32 @@ __global__ void __launch_bounds__(256) gemm_mfma_kernel(const GemmParams p) {
 #pragma unroll
             for (int kq = 0; kq < KQ; ++kq) {
                 T af[WBM][VE], bf[WBN][VE];
+                // Float32: MFMA e of the group multiplies k = 2 e (lanes 0..31) and 2 e + 1 (lanes 32..63), two fused
+                // multiply-adds in that order per output element, so that every element is the chain c = fma(a_k, b_k, c) in
+                // ascending k -- the order of the DMA-fed kernel and of the reference.  A K-major fragment arrives as
+                // k 0..3 | k 4..7 and is rearranged with two v_permlane32_swap; an MN-major one is read that way.
+                constexpr bool ASC = sizeof(T) == 4;
+                auto ascend = [](T (&f)[VE]) {
+                    if constexpr (ASC) {
+                        typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+                        const u32x2 a = __builtin_amdgcn_permlane32_swap(__builtin_bit_cast(uint32_t, f[0]), __builtin_bit_cast(uint32_t, f[1]), false, false);
+                        const u32x2 c = __builtin_amdgcn_permlane32_swap(__builtin_bit_cast(uint32_t, f[2]), __builtin_bit_cast(uint32_t, f[3]), false, false);
+                        const uint32_t a0 = a[0], a1 = a[1], c0 = c[0], c1 = c[1];
+                        f[0] = __builtin_bit_cast(T, a0); f[1] = __builtin_bit_cast(T, c0); f[2] = __builtin_bit_cast(T, a1); f[3] = __builtin_bit_cast(T, c1);
+                    }
+                };
                 if constexpr (A_KM) {
 #pragma unroll
                     for (int i = 0; i < WBM; ++i) {
                         const TVE t = *reinterpret_cast<const TVE*>(sA + (((wm * WBM + i) * R + lr) * SA + kq * G + lg) * 16);
 #pragma unroll
                         for (int e = 0; e < VE; ++e) af[i][e] = t[e];
+                        ascend(af[i]);
                     }
                 } else {
 #pragma unroll
                     for (int e = 0; e < VE; ++e) {
-                        const int krow = (kq * G + lg) * VE + e;
+                        const int krow = ASC ? kq * G * VE + e * G + lg : (kq * G + lg) * VE + e;
                         const TVA t = *reinterpret_cast<const TVA*>(sA + ((int)sizeof(T)) * (krow * BM + (wm * R + lr) * WBM));
 #pragma unroll
                         for (int i = 0; i < WBM; ++i) af[i][e] = t[i];
@@ -540,11 +577,12 @@ __global__ void __launch_bounds__(256) gemm_mfma_kernel(const GemmParams p) {
                         const TVE t = *reinterpret_cast<const TVE*>(sB + (((wn * WBN + j) * R + lr) * SB + kq * G + lg) * 16);
 #pragma unroll
                         for (int e = 0; e < VE; ++e) bf[j][e] = t[e];
+                        ascend(bf[j]);
                     }
                 } else {
 #pragma unroll
                     for (int e = 0; e < VE; ++e) {
-                        const int krow = (kq * G + lg) * VE + e;
+                        const int krow = ASC ? kq * G * VE + e * G + lg : (kq * G + lg) * VE + e;
                         const TVB t = *reinterpret_cast<const TVB*>(sB + ((int)sizeof(T)) * (krow * BN + (wn * R + lr) * WBN));
 #pragma unroll
                         for (int j = 0; j < WBN; ++j) bf[j][e] = t[j];
@@ -589,8 +627,10 @@ __global__ void __launch_bounds__(256) gemm_mfma_kernel(const GemmParams p) {
                 if ((ALIGNED && CONV == 0) || (m < p.M && n < p.N)) {
                     const gptr_mut<T> cp = C + (int64_t)m * p.ldc + n;
                     AccS val = acc[i][j][r];
-                    if (cmode == C_ACCUMULATE) val += (AccS)(*cp);
-                    else if (cmode == C_BIAS) val += (AccS)bias[(int64_t)b * p.bias_bs + (int64_t)m * p.bias_rs + (int64_t)n * p.bias_cs];
+                    if constexpr (!CHAIN_FROM_C0) {
+                        if (cmode == C_ACCUMULATE) val += (AccS)(*cp);
+                        else if (cmode == C_BIAS) val += (AccS)bias[(int64_t)b * p.bias_bs + (int64_t)m * p.bias_rs + (int64_t)n * p.bias_cs];
+                    }
                     *cp = (T)val;
                 }
             }

@@ -97,11 +97,11 @@ struct RingGeom {
 // Per-lane BYTE offsets (relative to the tile's first element at K-step 0) of this wavefront's
 // WB DMA instructions into one operand tile.  Instruction j = WB*wave + jj fills LDS bytes
 // [1024 j, 1024 j + 1024) of the tile:
-//   K-contiguous operand: rows 16 j + lane/4, 16-byte slot lane%4 holds kv = slot ^ ((row>>1)&3)
+//   K-contiguous operand: rows 16 j + lane/4, 16-byte slot lane%4 holds kv = slot ^ km_swz(row)
 //   MN-contiguous operand (CH chunks per k-row): piece 64 j + lane of the tile = k-row (64 j + lane) / CH, slot (64 j + lane) % CH, holds
 //                          chunk = slot ^ (2*(krow&3)) for 16-bit elements (what the transposing
 //                          reads need), slot ^ mn8_swizzle(krow) for 8-bit elements,
-//                          slot ^ (8*((krow>>2)&1)) for Float32 (the two k-rows that one
+//                          slot ^ (8*(krow&1)) for Float32 (the two consecutive k-rows that one
 //                          ds_read_b32 touches land in different halves of the 64 banks)
 // With RAGGED, mn_valid (1..BM rows/columns of the tile that exist) and k_valid (k of the
 // K-step that exist, a multiple of one chunk) clamp the SOURCE address into the matrix: lanes
@@ -118,6 +118,12 @@ __device__ __forceinline__ int mn8_swizzle(int krow) { return CH >= 8 ? (krow & 
 // (every 128 or every 256 bytes), the lanes that one pass of a ds_read_b128 serves hit different banks.
 __device__ __forceinline__ int swz8(int row) { return (row & 7) ^ ((row >> 3) & 1); }
 
+// 64-byte rows (K-major tiles, KD = 1): 16-byte slot kv of row r is stored at kv ^ km_swz(r): read 16 bytes per lane, eight
+// lanes to a pass, rows r .. r + 7 hit eight different 16-byte bank groups.  (Float32 plain products read such rows one dword
+// per lane; taking bits 2 and 3 of the row for them instead was measured and changed nothing.)
+template <int ES>
+__device__ __forceinline__ int km_swz(int row) { return (row >> 1) & 3; }
+
 template <bool KC, bool RAGGED, int WB, int ES, int KD = 1>
 __device__ __forceinline__ void dma_offsets(uint32_t (&off)[WB * KD], int64_t ld, int wave, int lane, int mn_valid, int k_valid) {
     constexpr int CH = RingGeom<WB, ES>::CHUNKS, VEL = RingGeom<WB, ES>::VEL;
@@ -127,7 +133,7 @@ __device__ __forceinline__ void dma_offsets(uint32_t (&off)[WB * KD], int64_t ld
         if constexpr (KC) {
             // (KD = 2: an instruction covers 8 rows of 128 bytes, whole cache lines)
             int row = KD == 2 ? 8 * j + (lane >> 3) : 16 * j + (lane >> 2);
-            int kv = KD == 2 ? (lane & 7) ^ swz8(row) : (lane & 3) ^ ((row >> 1) & 3);
+            int kv = KD == 2 ? (lane & 7) ^ swz8(row) : (lane & 3) ^ km_swz<ES>(row);
             if constexpr (RAGGED) {
                 row = row < mn_valid ? row : mn_valid - 1;
                 kv = kv < k_valid / VEL ? kv : k_valid / VEL - 1;
@@ -136,7 +142,7 @@ __device__ __forceinline__ void dma_offsets(uint32_t (&off)[WB * KD], int64_t ld
         } else {
             // (CH = 24, the 192-row tile: three instructions fill eight k-rows, a k-row may begin inside an instruction)
             int krow = (64 * j + lane) / CH;
-            int chunk = ((64 * j + lane) % CH) ^ (ES == 2 ? 2 * (krow & 3) : ES == 4 ? 8 * ((krow >> 2) & 1) : ES == 1 ? mn8_swizzle<CH>(krow) : 0);   // Float64: stored as is
+            int chunk = ((64 * j + lane) % CH) ^ (ES == 2 ? 2 * (krow & 3) : ES == 4 ? 8 * (krow & 1) : ES == 1 ? mn8_swizzle<CH>(krow) : 0);   // Float64: stored as is
             if constexpr (RAGGED) {
                 krow = krow < k_valid ? krow : k_valid - 1;
                 chunk = chunk < mn_valid / VEL ? chunk : mn_valid / VEL - 1;
@@ -249,6 +255,53 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
     const T* A = p.Aptr ? static_cast<const T*>(p.Aptr[b]) : static_cast<const T*>(p.A) + operand_offset(p, b, p.sA, p.sAk);
     const T* B = p.Bptr ? static_cast<const T*>(p.Bptr[b]) : static_cast<const T*>(p.B) + operand_offset(p, b, p.sB, p.sBk);
     T* C = p.Cptr ? static_cast<T*>(p.Cptr[b]) : static_cast<T*>(p.C) + (int64_t)b * p.sC;
+
+    using AccV = typename E::AccV;
+    using AccS = typename E::AccS;
+    AccV acc[WBM][WBN];
+#pragma unroll
+    for (int i = 0; i < WBM; ++i)
+#pragma unroll
+        for (int j = 0; j < WBN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = (AccS)0;
+    // Float32: the accumulators start from C0 (C itself, or the bias), so that every output element is the reference's chain
+    // c = C0; c = fma(a_k, b_k, c) for ascending k, bit for bit, and the epilogue only stores.  A lane holds rows
+    // 32 i + lane % 32 and columns 32 j + 8 rq + 4 (lane / 32) + (0..3) of its wavefront's part of the tile.
+    if constexpr (ES == 4 && std::is_same<AccS, float>::value) {
+        if (p.cmode == C_ACCUMULATE || p.cmode == C_BIAS) {            // (uniform)
+            const bool from_c = p.cmode == C_ACCUMULATE;
+            const float* bias = static_cast<const float*>(p.bias);
+            const bool vec_ok = from_c ? (p.ldc % 4 == 0 && (reinterpret_cast<uintptr_t>(C) & 15) == 0)
+                                       : (p.bias_cs == 1 && p.bias_rs % 4 == 0 && p.bias_bs % 4 == 0 && (reinterpret_cast<uintptr_t>(bias) & 15) == 0);
+            const int64_t cstep = from_c ? 1 : p.bias_cs;
+            typedef float f32x4 __attribute__((ext_vector_type(4)));
+#pragma unroll
+            for (int i = 0; i < WBM; ++i) {
+                const int m = m0 + wm * WTM + 32 * i + (lane & 31);
+#pragma unroll
+                for (int j = 0; j < WBN; ++j)
+#pragma unroll
+                    for (int rq = 0; rq < 4; ++rq) {
+                        const int nn = n0 + wn * WTN + 32 * j + 8 * rq + 4 * (lane >> 5);
+                        f32x4 v = {0.0f, 0.0f, 0.0f, 0.0f};
+                        if (m < p.M && nn < p.N) {
+                            const float* src = from_c ? reinterpret_cast<const float*>(C) + (int64_t)m * p.ldc + nn
+                                                      : bias + (int64_t)b * p.bias_bs + (int64_t)m * p.bias_rs + (int64_t)nn * p.bias_cs;
+                            if (vec_ok && nn + 4 <= p.N) v = *reinterpret_cast<const f32x4*>(src);
+                            else {
+#pragma unroll
+                                for (int e = 0; e < 4; ++e)
+                                    if (nn + e < p.N) v[e] = src[(int64_t)e * cstep];
+                            }
+                        }
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) acc[i][j][4 * rq + e] = v[e];
+                    }
+            }
+        }
+    }
+
 
     // ---- DMA sources: uniform tile base (advances by adv bytes per K-step) + per-lane offsets ----
     const int wave_u = __builtin_amdgcn_readfirstlane(wave);
@@ -396,7 +449,7 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
                 if (t < g.k_c && (unsigned)(iw0 + t * g.d_c) < (unsigned)g.W) m |= 256u << t;
             }
             cmask3[x] = n < p.N ? m : 0u;
-            const uint32_t kv = (uint32_t)((lane & 3) ^ ((row >> 1) & 3));
+            const uint32_t kv = (uint32_t)((lane & 3) ^ km_swz<ES>(row));
             uint32_t tq = 0u, cho = kv * 16u;
             if (g.tap_step > 1) {
                 const uint32_t cb = 64u / (uint32_t)g.tap_step;        // bytes of channels per pixel: 16 or 32
@@ -477,7 +530,7 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
         for (int x = 0; x < WB; ++x) {
             const int j = wave * WB + x;
             const int krow = (64 / CH) * j + lane / CH;
-            const int chunk = (lane % CH) ^ (ES == 2 ? 2 * (krow & 3) : 8 * ((krow >> 2) & 1));
+            const int chunk = (lane % CH) ^ (ES == 2 ? 2 * (krow & 3) : 8 * (krow & 1));
             const int n = n0 + chunk * G::VEL;
             const uint32_t nn = (n < p.N ? (uint32_t)n : 0u) + (uint32_t)g.n_base;
             const uint32_t t = nn / cgc, c = nn - t * cgc;
@@ -563,12 +616,18 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
 
     // ---- per-lane LDS read offsets (bytes inside an operand tile), for half-step ks (0, 1) of a K-step ----
     // A lane's fragment of one block is 16 bytes of k: lanes 0..31 hold the first 16 bytes of the half-step of
-    // their row, lanes 32..63 the second (8 + 8 consecutive k of 16-bit elements for one 32x32x16 MFMA; 4 + 4 of
-    // Float32, element e of both halves feeding the e-th of four 32x32x2 MFMAs -- the order of k inside a half-step
-    // is the same permutation for A and B).
+    // their row, lanes 32..63 the second (8 + 8 consecutive k of 16-bit elements for one 32x32x16 MFMA).
+    // Float32: a v_mfma_f32_32x32x2 is, per output element, two fused multiply-adds in a row -- first the k of lanes 0..31,
+    // then the k of lanes 32..63 (checked against fmaf chains on the host, bit for bit) -- so the four MFMAs of a half-step
+    // multiply k = (0, 1), (2, 3), (4, 5), (6, 7) in that order and every output element is the reference's own chain
+    // c = fma(a_k, b_k, c) in ascending k.  Both layouts are therefore read one dword per element, element e = k 2 e + lane / 32
+    // (a 16-byte read of a K-major row would hand a lane four consecutive k, and rearranging them with cross-lane moves in the
+    // MFMA stream was measured 4 % slower per K-major operand).  The channels-last convolution (CONV = 3 / 5: both operands
+    // K-major), whose k runs taps-outermost and so cannot be the reference's order anyway, keeps the 16-byte reads: element e
+    // of both operands is k = e (lanes 0..31) | 4 + e (lanes 32..63), the same pairs on both sides.
     // K-major: block b of the wavefront, row = wbase + 32 b + lane%32, slot (2 ks + lane/32) ^ ((row>>1)&3)
     // MN-major, 16-bit: two transposing reads per block; see the header comment
-    // MN-major, Float32: four ds_read_b32 per block, element e from k-row 8 ks + 4 (lane/32) + e
+    // MN-major, Float32: four ds_read_b32 per block, element e from k-row 8 ks + 2 e + lane/32
     auto frag_off_km = [&](int wbase, int blk, int ks) -> int {
         const int row = wbase + blk * 32 + (lane & 31);
         if constexpr (KD == 2) return row * 128 + (((2 * ks + (lane >> 5)) ^ swz8(lane & 31)) * 16);   // (wbase + 32 blk is a multiple of 16)
@@ -594,10 +653,10 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
         return krow * mnrow + chunk * 16 + (mnl & 15);
     };
     auto frag_off_mm32 = [&](int mnrow, int wbase, int blk, int ks, int e) -> int {
-        const int krow = 8 * ks + 4 * (lane >> 5) + e;
+        const int krow = 8 * ks + 2 * e + (lane >> 5);                    // MFMA e of the half-step multiplies k = 2 e (lanes 0..31) and 2 e + 1
         const int mnl = wbase + blk * 32 + (lane & 31);
         if constexpr (GATHER4) return krow * mnrow + mnl * 4;            // gathered tiles are stored unswizzled
-        return krow * mnrow + ((mnl * 4) ^ (128 * (lane >> 5)));      // (krow >> 2) & 1 == lane / 32
+        return krow * mnrow + ((mnl * 4) ^ (128 * (lane >> 5)));      // krow & 1 == lane / 32
     };
 
     // One LDS read instruction of an operand's fragment set for half-step ks.  A K-major
@@ -605,6 +664,13 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
     // 8-byte reads per block; Float32: 4 WB four-byte reads); read r lands in frag[r / per_block].
     auto read_op = [&](auto& frag, int mnrow, const char* tile, bool kc, int wbase, int ks, int r) {
         if (kc) {
+            if constexpr (ES == 4 && !GATHER16) {
+                // Float32 (read r = block r / 4, element e = r % 4): element e is k = 2 e + lane / 32 of the half-step (see above),
+                // dword (2 e + lane / 32) % 4 of the 16-byte slot 2 ks + e / 2 of the row
+                const int blk = r >> 2, e = r & 3;
+                const int row = wbase + blk * 32 + (lane & 31), sw = km_swz<4>(lane & 31);
+                frag[blk][e] = *reinterpret_cast<const uint32_t*>(tile + row * 64 + (((2 * ks + (e >> 1)) ^ sw) * 16) + 8 * (e & 1) + 4 * (lane >> 5));
+            } else
             frag[r] = *reinterpret_cast<const u32x4*>(tile + frag_off_km(wbase, r, ks));
         } else if constexpr (ES == 4) {
             frag[r >> 2][r & 3] = *reinterpret_cast<const uint32_t*>(tile + frag_off_mm32(mnrow, wbase, r >> 2, ks, r & 3));
@@ -625,20 +691,11 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
         }
     };
     constexpr int MNRB = ES == 4 ? 4 : 2;                // reads of one block of an MN-major operand per half-step
-    constexpr int NRA = A_KC ? WBM : MNRB * WBM, NRB = B_KC ? WBN : MNRB * WBN, NR = NRA + NRB;
+    constexpr bool KM128 = ES != 4 || GATHER16;          // K-major fragments come in one 16-byte read
+    constexpr int NRA = A_KC && KM128 ? WBM : MNRB * WBM, NRB = B_KC && KM128 ? WBN : MNRB * WBN, NR = NRA + NRB;
     constexpr int MPP = ES == 4 ? 4 : 1;                 // MFMAs per pair of fragments
     constexpr int NMMA = WBM * WBN * MPP;                // MFMAs per half-step
     constexpr int RPM = (NR + NMMA - 1) / NMMA;          // LDS reads slotted behind each MFMA
-
-    using AccV = typename E::AccV;
-    using AccS = typename E::AccS;
-    AccV acc[WBM][WBN];
-#pragma unroll
-    for (int i = 0; i < WBM; ++i)
-#pragma unroll
-        for (int j = 0; j < WBN; ++j)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[i][j][r] = (AccS)0;
 
     // K-steps past the end are clamped to the last one: the tail iterations then issue the
     // same DMA traffic as the steady state (into stages nobody reads any more), which keeps
@@ -667,6 +724,17 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
         }
         else dma_tile<WBN * KD>(srcB(kt), kt >= last ? offBt : offB, lds_tile, wave_u);
     };
+    if constexpr (ES == 4 && std::is_same<AccS, float>::value) {
+        if (p.cmode == C_ACCUMULATE || p.cmode == C_BIAS) {
+            // The starting values (requested first thing, their latency behind the set-up above) are taken here, before the first
+            // DMA instruction is issued: the compiler counts only its own loads, so its wait for them would otherwise stand in
+            // front of the first MFMA and cover every DMA load issued since -- the whole fill of the ring instead of the first tile.
+#pragma unroll
+            for (int i = 0; i < WBM; ++i)
+#pragma unroll
+                for (int j = 0; j < WBN; ++j) asm volatile("" : "+v"(acc[i][j]));
+        }
+    }
     dma_tile<NA>(srcA(0), 0 >= last ? offAt : offA, lds_addr_of(st0), wave_u);
     b_tile(0, lds_addr_of(st0) + A_TILE_BYTES);
     dma_tile<NA>(srcA(1), 1 >= last ? offAt : offA, lds_addr_of(st1), wave_u);
@@ -763,14 +831,18 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
     // covers one chunk of consecutive k (8 or 4) starting at (32 bytes) ks + (16 bytes) (lane / 32) in both
     // LDS layouts, and K is a multiple of the chunk, so a lane's fragment is either entirely real or
     // entirely past the end.
+    // (Float32: element e of a fragment is k = 2 e + lane / 32 of the half-step in both layouts; the channels-last convolution keeps
+    //  the 16-byte fragments: k 0..3 | k 4..7)
     auto mask_tail = [&](int buf, int ks) {
         const bool ok = (32 / ES) * ks + (16 / ES) * (lane >> 5) < kr;
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
+            const bool oke = 8 * ks + 2 * e + (lane >> 5) < kr;
+            const bool oka = ES == 4 && !GATHER16 ? oke : ok, okb = ES == 4 && !GATHER16 ? oke : ok;
 #pragma unroll
-            for (int i = 0; i < WBM; ++i) af[buf][i][e] = ok ? af[buf][i][e] : 0u;
+            for (int i = 0; i < WBM; ++i) af[buf][i][e] = oka ? af[buf][i][e] : 0u;
 #pragma unroll
-            for (int j = 0; j < WBN; ++j) bf[buf][j][e] = ok ? bf[buf][j][e] : 0u;
+            for (int j = 0; j < WBN; ++j) bf[buf][j][e] = okb ? bf[buf][j][e] : 0u;
         }
     };
 
@@ -1064,10 +1136,16 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
             }
         }
     };
-    if (p.cmode == C_ACCUMULATE) epilogue(std::integral_constant<int, C_ACCUMULATE>{});
-    else if (p.cmode == C_PARTIAL) epilogue(std::integral_constant<int, C_PARTIAL>{});
-    else if (p.cmode == C_BIAS) epilogue(std::integral_constant<int, C_BIAS>{});
-    else epilogue(std::integral_constant<int, C_OVERWRITE>{});
+    if constexpr (ES == 4 && std::is_same<AccS, float>::value) {
+        // (C0 or the bias went into the accumulators before the K loop)
+        if (p.cmode == C_PARTIAL) epilogue(std::integral_constant<int, C_PARTIAL>{});
+        else epilogue(std::integral_constant<int, C_OVERWRITE>{});
+    } else {
+        if (p.cmode == C_ACCUMULATE) epilogue(std::integral_constant<int, C_ACCUMULATE>{});
+        else if (p.cmode == C_PARTIAL) epilogue(std::integral_constant<int, C_PARTIAL>{});
+        else if (p.cmode == C_BIAS) epilogue(std::integral_constant<int, C_BIAS>{});
+        else epilogue(std::integral_constant<int, C_OVERWRITE>{});
+    }
 }
 
 // true when the fast kernel can serve the problem: 16-byte aligned rows everywhere (leading

@@ -471,7 +471,8 @@ def test_config3_4096_cube(dtype, scale):
     acc = out.clone()
     F.matmult(ta_, tb_, acc)
     if dtype in (np.float32, np.float64):
-        assert torch.allclose(acc, 2 * out, rtol=1e-5, atol=1e-4)
+        # (Float32 starts every chain from C0, as the reference does: C0 + A.B is not the rounded sum of two rounded terms)
+        assert (acc.double() - 2 * out.double()).abs().max().item() <= 1e-5 * n * float(ta_.abs().max() * tb_.abs().max())
     else:
         assert ((acc.float() - 2 * out.float()).abs().max() / out.float().abs().max()).item() <= HALF_REL
 
@@ -1207,3 +1208,46 @@ def test_host_entry_pipelined_panels_and_groups_bit_identical_to_the_device_entr
             for i in range(nb):
                 assert got[i].tobytes() == want[i].tobytes(), ("batch", shared_b, zero, i)
     assert lib.ntg_release_host_buffers() == 0
+
+
+@pytest.mark.parametrize("shape", [(128, 256, 128), (512, 512, 512), (300, 1000, 260), (130, 22, 66), (33, 77, 35), (1860, 36, 132), (96, 4100, 64)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_fp32_product_is_the_reference_chain_bit_for_bit(shape):
+    """Float32 on the matrix pipe, bit for bit the reference's own sum: every output element is c = 0; for k ascending:
+    c = fma(a[i, k], b[k, j], c) (the closed form of the oracle, which the reference's k-outer loop nest computes).  Holds
+    because one v_mfma_f32_32x32x2 is two fused multiply-adds in a row per element and the kernels feed it k in ascending
+    order.  All four storage forms; shapes on 128- and 64-wide tiles of the DMA-fed kernel, with k tails and ragged edges, and
+    shapes whose rows are not 16-byte multiples (the register-staged kernel); no workspace, so nothing is split along k."""
+    m, k, n = shape
+    rng = np.random.default_rng(4242 + m + k + n)
+    a = randn(rng, (m, k), np.float32)
+    b = randn(rng, (k, n), np.float32)
+    if k >= 64:       # wide dynamic range: rounding differences could not hide
+        a[:, ::7] *= 1000.0
+        b[5::11, :] *= 1e-3
+    for ta, tb in TRANS:
+        sa = np.ascontiguousarray(a.T) if ta else a
+        sb = np.ascontiguousarray(b.T) if tb else b
+        want = oracle.matmult2d(sa, sb, None, ta, tb)
+        got = dev_matmult(sa, sb, np.zeros((m, n), np.float32), m, k, n, ta, tb, np.float32, mode=_lib.C_OVERWRITE)
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), (shape, ta, tb, int((got != want).sum()))
+        # the accumulate contract: the chain starts from what C holds (nt_matmult's C += ...)
+        c0 = randn(rng, (m, n), np.float32) * 50.0
+        want = oracle.matmult2d(sa, sb, c0.copy(), ta, tb)
+        got = dev_matmult(sa, sb, c0, m, k, n, ta, tb, np.float32, mode=_lib.C_ACCUMULATE)
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), (shape, ta, tb, "accumulate", int((got != want).sum()))
+    # cpu::linear: the bias row is the starting value of every row's chains (matmult_cpu.cpp:1637-1647)
+    bias = randn(rng, (n,), np.float32) * 20.0
+    w_nk = np.ascontiguousarray(b.T)
+    want = oracle.linear(a, w_nk, bias, False, True)
+    tx, tw, tbias = to_torch(a, DEV, False), to_torch(w_nk, DEV, False), to_torch(bias, DEV, False)
+    ty = torch.empty((m, n), dtype=torch.float32, device=DEV)
+    d = _lib.GemmDesc()
+    d.dtype, d.transpose_b, d.c_mode = _lib.FLOAT32, 1, _lib.C_BIAS
+    d.m, d.k, d.n, d.batches = m, k, n, 1
+    d.bias, d.bias_col_stride = tbias.data_ptr(), 1
+    _lib.check(_lib.load().ntg_gemm_dev(ctypes.byref(d), tx.data_ptr(), tw.data_ptr(), ty.data_ptr(),
+                                        ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)))
+    torch.cuda.synchronize()
+    got = ty.cpu().numpy()
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), (shape, "linear", int((got != want).sum()))
