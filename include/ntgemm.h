@@ -184,6 +184,13 @@ typedef struct ntg_gemm_desc {
  * batch runs on the DMA-fed kernels like its strided twin, without it on the register-staged ones.  An entry that breaks
  * the promise makes the kernel read from a misaligned address (wrong results, not a fault). */
 #define NTG_GEMM_PTRS_ALIGNED16 1
+/* Keep the reference's order of summation: never split this product along k (workspace or not), and run products of up to 32
+ * rows on the tile kernels instead of the streaming ones (which share k out between wavefronts).  A Float32 product is then
+ * the reference's own sum bit for bit -- every element is c = C0; c = fma(a[i,k], b[k,j], c) for ascending k, what the
+ * k-outer loop nest of nt_matmult.hpp:196 computes.  Without the flag that also holds for every Float32 product of more than
+ * 32 rows that is given no workspace.  The host-pointer entry points set it for Float32 themselves (the transfers hide what
+ * the faster forms would gain); ntg_gemm_workspace_bytes honours it. */
+#define NTG_GEMM_KEEP_K_ORDER 2
 
 /* Bytes of workspace with which ntg_gemm_dev runs its faster form (0: there is none for this product): a split along k
  * for shapes such as [256, 8192] x [8192, 8192] (planned from one item's sizes, so a batch is offered its item's split with

@@ -18,6 +18,7 @@ BFLOAT16, UINT64 = 100, 101
 
 C_OVERWRITE, C_ACCUMULATE, C_BIAS = 0, 1, 2
 GEMM_PTRS_ALIGNED16 = 1               # NTG_GEMM_PTRS_ALIGNED16
+GEMM_KEEP_K_ORDER = 2                 # NTG_GEMM_KEEP_K_ORDER
 NOALLOC_SCRATCH_BYTES = 64 << 20      # NTG_NOALLOC_SCRATCH_BYTES
 DIAG_MFMA_OPERAND_BYTES = 128 << 10   # NTG_DIAG_MFMA_OPERAND_BYTES
 DIAG_MFMA_FLOPS_PER_PASS = 8388608    # NTG_DIAG_MFMA_FLOPS_PER_PASS

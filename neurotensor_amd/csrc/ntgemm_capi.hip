@@ -156,7 +156,8 @@ int launch_gemm(ntg::GemmParams p, int dtype, bool ta, bool tb, hipStream_t s) {
         e = ntg::launch_gemm_complex(dtype, ta, tb, p, s);
     } else {
         bool handled = false;
-        e = ntg::launch_gemm_skinny(dtype, ta, tb, p, s, &handled);
+        // (the streaming kernels for up to 32 rows split k over their wavefronts: not for a caller who wants the one chain)
+        if (!(p.keep_k_order && dtype == ntg::DT_F32)) e = ntg::launch_gemm_skinny(dtype, ta, tb, p, s, &handled);
         if (e != hipSuccess) return hip_fail(e, "skinny gemm launch");
         if (handled) return finish();
         switch (dtype) {
@@ -341,7 +342,7 @@ static int run_padded(const ntg::GemmParams& p, const PadPlan& pl, int dtype, bo
 SplitPlan plan_splitk(const ntg::GemmParams& p, int dtype, bool ta) {
     SplitPlan none{1, p.K, 0};
     const int64_t es = ntg::elem_size(dtype);
-    if (is_valu_dtype(dtype) || es == 0 || p.batch < 1 || p.batch > 65535 || p.Aptr || p.Bptr || p.Cptr) return none;
+    if (is_valu_dtype(dtype) || es == 0 || p.batch < 1 || p.batch > 65535 || p.Aptr || p.Bptr || p.Cptr || p.keep_k_order) return none;
     if (p.M <= 32 && dtype != ntg::DT_F64) return none;                       // the streaming kernels take these
     const bool half = dtype == ntg::DT_F16 || dtype == ntg::DT_BF16;
     if (half) {
@@ -485,6 +486,7 @@ int desc_to_params(const ntg_gemm_desc* d, ntg::GemmParams& p) {
     p.bias = d->bias;
     p.bias_bs = d->bias_batch_stride; p.bias_rs = d->bias_row_stride; p.bias_cs = d->bias_col_stride;
     if (p.cmode == NTG_C_BIAS && !p.bias) return fail(NTG_ERR_INVALID_ARGUMENT, "c_mode is bias but bias is null");
+    p.keep_k_order = (d->flags & NTG_GEMM_KEEP_K_ORDER) != 0;
     return NTG_OK;
 }
 
@@ -637,6 +639,10 @@ int ntg_gemm_ptrs_dev(const ntg_gemm_desc* d, const void* const* dA, const void*
     return gemm_ptrs(d, dA, dB, dC, stream, d && (d->flags & NTG_GEMM_PTRS_ALIGNED16) != 0);
 }
 
+// The host-pointer entry points are the reference's own seam (nt_matmult / nt_matmult_batch / cpu::linear on host memory): there a
+// Float32 product keeps the reference's order of summation -- no split along k, whose gain the transfers would hide anyway.
+static int64_t host_entry_flags(int dtype) { return dtype == ntg::DT_F32 ? NTG_GEMM_KEEP_K_ORDER : 0; }
+
 int ntg_matmult_dev(int dtype, const void* dA, const void* dB, void* dC, int64_t m, int64_t k, int64_t n,
                     int transpose_a, int transpose_b, void* stream) {
     ntg_gemm_desc d;
@@ -674,6 +680,7 @@ static int matmult_host_pipelined(int dtype, const void* const* A, const void* c
     std::memset(&d, 0, sizeof d);
     d.dtype = dtype; d.transpose_a = ta; d.transpose_b = tb;
     d.m = m; d.k = k; d.n = n; d.batches = 1;
+    d.flags = host_entry_flags(dtype);
     const size_t a_slot = align_up(a_bytes, 256), b_slot = align_up(b_bytes, 256), c_slot = align_up(c_bytes, 256);
     std::vector<ntg::HostSession::Range> up;
     if (batches == 1) {
@@ -816,6 +823,7 @@ int ntg_matmult_batch(int dtype, const void* const* A, const void* const* B, voi
     std::memset(&d, 0, sizeof d);
     d.dtype = dtype; d.transpose_a = transpose_a; d.transpose_b = transpose_b; d.c_mode = NTG_C_ACCUMULATE;
     d.m = m; d.k = k; d.n = n; d.batches = batches;
+    d.flags = host_entry_flags(dtype);
     // The arena is this function's own: when every item's A (and B) is a new matrix, or all items share one, the slots
     // lie at a constant stride and the strided kernels (and their workspace forms) serve the batch; any other pattern of
     // repeated pointers goes through the pointer tables.
@@ -900,6 +908,7 @@ int ntg_linear(int dtype, const void* X, const void* W, const void* bias, void* 
     std::memset(&d, 0, sizeof d);
     d.dtype = dtype; d.transpose_a = transpose_x; d.transpose_b = transpose_w; d.c_mode = NTG_C_BIAS;
     d.m = m; d.k = k; d.n = n; d.batches = 1;
+    d.flags = host_entry_flags(dtype);
     d.bias = mem.at(ob);
     d.bias_row_stride = (bias_rows == 1) ? 0 : bias_cols;
     d.bias_col_stride = (bias_cols == 1) ? 0 : 1;

@@ -731,3 +731,31 @@ def test_conv2d_weight_gradient_k_ranges_across_images(ranges, monkeypatch):
         if ranges == 6:
             # whole images per range: the same products and the same order of adding them up
             assert torch.equal(dw, dw_images)
+
+
+@pytest.mark.parametrize("geom", [
+    # (B, C, H, W, O, kh, kw, stride, padding, dilation, groups)
+    (2, 8, 18, 18, 16, 3, 3, 1, 1, 1, 1),       # rows of the weights and of the output plane are 16-byte multiples: the DMA-fed gather
+    (3, 16, 20, 12, 24, 3, 3, 2, 1, 1, 2),      # grouped, strided
+    (2, 5, 9, 11, 7, 3, 2, 1, 0, 1, 1),         # nothing aligned: the register-staged gather
+    (1, 12, 15, 15, 8, 5, 5, 1, 2, 2, 1),       # dilated
+], ids=lambda g: "x".join(map(str, g)))
+def test_conv2d_fp32_without_workspace_is_the_reference_chain_bit_for_bit(geom):
+    """Float32 conv2d on the gathering kernels (no workspace): the k axis is the reference's own (channel, tap row, tap column)
+    order of im2col, every output element is the chain c = 0; c = fma(w[o, kk], col[kk, l], c) in ascending kk -- the bits of
+    unfold + matmult (conv.cpp:86-95), which the oracle restates."""
+    B, C, H, W, O, kh, kw, st, pd, dl, groups = geom
+    rng = np.random.default_rng(31 + B + C + O)
+    x = rng.standard_normal((B, C, H, W)).astype(np.float32)
+    w = (rng.standard_normal((O, C // groups, kh, kw)) * 3.0).astype(np.float32)
+    want = oracle.conv2d(x, w, st, pd, dl, groups)
+    tx, tw = dev(x), dev(w)
+    out = torch.empty(want.shape, dtype=torch.float32, device=DEV)
+    lib = _lib.load()
+    need = lib.ntg_conv2d_forward_workspace_bytes(_lib.FLOAT32, B, C, H, W, kh, kw, st, st, pd, pd, dl, dl)
+    assert need == 0
+    _lib.check(lib.ntg_conv2d_dev(_lib.FLOAT32, tx.data_ptr(), tw.data_ptr(), out.data_ptr(), None, 0, B, C, H, W, O, kh, kw,
+                                  st, st, pd, pd, dl, dl, groups, ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)))
+    torch.cuda.synchronize()
+    got = out.cpu().numpy()
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), (geom, int((got != want).sum()))

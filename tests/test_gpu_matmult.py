@@ -1251,3 +1251,43 @@ def test_fp32_product_is_the_reference_chain_bit_for_bit(shape):
     torch.cuda.synchronize()
     got = ty.cpu().numpy()
     assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), (shape, "linear", int((got != want).sum()))
+
+
+@pytest.mark.parametrize("shape", [(16, 1024, 640), (64, 8192, 64), (300, 257, 123), (2048, 3000, 2048)], ids=lambda s: "x".join(map(str, s)))
+def test_host_entry_points_fp32_are_the_reference_chain_bit_for_bit(shape):
+    """The drop-in seam in Float32: nt_matmult / nt_matmult_batch / linear on host memory give the bits of the reference's
+    own loop nest (the oracle's tiled restatement == its closed form): 16 rows (the streaming kernel is bypassed), few tiles
+    with a deep k (no split along k at the seam), ragged sizes on the register-staged kernel, and a product large enough to
+    cross the link in panels; C0 random (the accumulate contract), two storage forms."""
+    m, k, n = shape
+    rng = np.random.default_rng(777 + m)
+    lib = _lib.load()
+    a = randn(rng, (m, k), np.float32)
+    b = randn(rng, (k, n), np.float32)
+    for ta, tb in ((False, False), (True, True)) if m < 2048 else ((False, True),):
+        sa = np.ascontiguousarray(a.T) if ta else a
+        sb = np.ascontiguousarray(b.T) if tb else b
+        c0 = randn(rng, (m, n), np.float32) * 10.0
+        want = oracle.matmult2d(sa, sb, c0.copy(), ta, tb, kind="tiled", threads=8)
+        got = host_matmult(sa, sb, c0.copy(), m, k, n, ta, tb, _lib.FLOAT32)
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), (shape, ta, tb, int((got != want).sum()))
+    if m >= 2048:
+        return
+    # a batch with a repeated operand, and linear with its bias row
+    items = 3
+    As = [randn(rng, (m, k), np.float32) for _ in range(items)]
+    Cs = [randn(rng, (m, n), np.float32) for _ in range(items)]
+    want = [oracle.matmult2d(As[i], b, Cs[i].copy(), False, False, kind="tiled", threads=8) for i in range(items)]
+    pa = (ctypes.c_void_p * items)(*[x.ctypes.data for x in As])
+    pb = (ctypes.c_void_p * items)(*[b.ctypes.data] * items)
+    pc = (ctypes.c_void_p * items)(*[x.ctypes.data for x in Cs])
+    _lib.check(lib.ntg_matmult_batch(_lib.FLOAT32, pa, pb, pc, items, m, k, k, n, 0, 0))
+    for i in range(items):
+        assert np.array_equal(Cs[i].view(np.uint32), want[i].view(np.uint32)), (shape, "batch item", i)
+    bias = randn(rng, (n,), np.float32) * 5.0
+    w_nk = np.ascontiguousarray(b.T)
+    want = oracle.linear(a, w_nk, bias, False, True)
+    y = np.empty((m, n), np.float32)
+    vp = lambda x: x.ctypes.data_as(ctypes.c_void_p)
+    _lib.check(lib.ntg_linear(_lib.FLOAT32, vp(a), vp(w_nk), vp(bias), vp(y), m, k, n, 0, 1, 1, n))
+    assert np.array_equal(y.view(np.uint32), want.view(np.uint32)), (shape, "linear")
