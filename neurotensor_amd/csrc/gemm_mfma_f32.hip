@@ -13,7 +13,156 @@ static int ring_f32_tile_edge(const GemmParams& p) {
     return cost64 < cost128 ? 64 : 128;
 }
 
+// Products with so few output elements that 64 x 64 tiles reach fewer than half of the CUs (config 1, 512^3: 64 tiles, each a
+// chain of k / 2 MFMAs of 64 cycles on one wavefront per block): one workgroup per 32 x 32 tile of C, four wavefronts with one
+// 16 x 16 block each on v_mfma_f32_16x16x4, whose four lane groups are multiplied in a row -- per output element four fused
+// multiply-adds in ascending k, the same chain c = C0; c = fma(a_k, b_k, c) that the 32x32x2 kernels compute (both checked
+// against fmaf chains on the host), so the results are bit-identical to theirs and the choice between the kernels is free.
+// The chain of a block is k / 4 instructions of 32 cycles: four times shorter, on four times as many workgroups.
+// Operands go through LDS in stages of 128 k (four 16-byte loads of A and four of B per thread and stage, the loads of the
+// next two stages in flight behind the multiplies): a K-contiguous operand is stored [row][132 floats], an M/N-contiguous
+// one [k][48 floats], both free of bank conflicts for the one-dword-per-lane reads of the MFMA operands.
+// Needs what the DMA-fed kernel needs (16-byte rows and pointers); C0 / bias start the chain, relu clamps in the epilogue.
+template <bool TA, bool TB>
+__global__ void __launch_bounds__(256) gemm_small16_f32_kernel(const GemmParams p) {
+    constexpr int KB = 128, LDK = KB + 4, LDM = 48, NP = KB / 32;       // NP 16-byte pieces of each operand per thread and stage
+    constexpr int A_STAGE = TA ? KB * LDM : 32 * LDK, B_STAGE = TB ? 32 * LDK : KB * LDM;
+    __shared__ __attribute__((aligned(16))) float sA[2][A_STAGE];
+    __shared__ __attribute__((aligned(16))) float sB[2][B_STAGE];
+    typedef float f32x4 __attribute__((ext_vector_type(4)));
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int bi = wave >> 1, bj = wave & 1, li = lane & 15, lg = lane >> 4;
+    const int tiles = p.tiles_m * p.tiles_n;
+    const int b = (int)blockIdx.x / tiles, t = (int)blockIdx.x - b * tiles;
+    const int m0 = (t / p.tiles_n) * 32, n0 = (t % p.tiles_n) * 32;
+    const float* A = p.Aptr ? static_cast<const float*>(p.Aptr[b]) : static_cast<const float*>(p.A) + operand_offset(p, b, p.sA, p.sAk);
+    const float* B = p.Bptr ? static_cast<const float*>(p.Bptr[b]) : static_cast<const float*>(p.B) + operand_offset(p, b, p.sB, p.sBk);
+    float* C = p.Cptr ? static_cast<float*>(p.Cptr[b]) : static_cast<float*>(p.C) + (int64_t)b * p.sC;
+
+    // this lane's four results: row m, columns n .. n + 3 (the operands are handed to the MFMA the other way round, so that
+    // a lane's four accumulator registers are consecutive columns of one row)
+    const int m = m0 + bi * 16 + li, n = n0 + bj * 16 + 4 * lg;
+    const bool c_ok = m < p.M && n < p.N;                        // (N is a multiple of 4: the four columns exist together)
+    f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (c_ok) {
+        if (p.cmode == C_ACCUMULATE) acc = *reinterpret_cast<const f32x4*>(C + (int64_t)m * p.ldc + n);
+        else if (p.cmode == C_BIAS) {
+            const float* bias = static_cast<const float*>(p.bias) + (int64_t)b * p.bias_bs + (int64_t)m * p.bias_rs + (int64_t)n * p.bias_cs;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) acc[e] = bias[(int64_t)e * p.bias_cs];
+        }
+    }
+
+    // Piece u of this thread: a K-contiguous operand has 32 pieces (128 k) per row, rows tid / 32 + 8 u; an M/N-contiguous one
+    // 8 pieces (32 rows or columns of C) per k-row, k-rows tid / 8 + 32 u.  The sizes along the contiguous axis are multiples
+    // of 4, so a piece lies inside the matrix or outside as a whole; outside pieces are zeros (their rows / columns of C are
+    // not stored, their k are not multiplied).
+    const f32x4 zero4 = {0.0f, 0.0f, 0.0f, 0.0f};
+    auto load_a = [&](int k0, f32x4 (&v)[NP]) {
+#pragma unroll
+        for (int u = 0; u < NP; ++u) {
+            if constexpr (TA) {
+                const int k = k0 + (tid >> 3) + 32 * u, mm = m0 + (tid & 7) * 4;
+                v[u] = (k < p.K && mm < p.M) ? *reinterpret_cast<const f32x4*>(A + (int64_t)k * p.lda + mm) : zero4;
+            } else {
+                const int mm = m0 + (tid >> 5) + 8 * u, k = k0 + (tid & 31) * 4;
+                v[u] = (mm < p.M && k < p.K) ? *reinterpret_cast<const f32x4*>(A + (int64_t)mm * p.lda + k) : zero4;
+            }
+        }
+    };
+    auto load_b = [&](int k0, f32x4 (&v)[NP]) {
+#pragma unroll
+        for (int u = 0; u < NP; ++u) {
+            if constexpr (TB) {
+                const int nn = n0 + (tid >> 5) + 8 * u, k = k0 + (tid & 31) * 4;
+                v[u] = (nn < p.N && k < p.K) ? *reinterpret_cast<const f32x4*>(B + (int64_t)nn * p.ldb + k) : zero4;
+            } else {
+                const int k = k0 + (tid >> 3) + 32 * u, nn = n0 + (tid & 7) * 4;
+                v[u] = (k < p.K && nn < p.N) ? *reinterpret_cast<const f32x4*>(B + (int64_t)k * p.ldb + nn) : zero4;
+            }
+        }
+    };
+    auto store = [&](int buf, const f32x4 (&va)[NP], const f32x4 (&vb)[NP]) {
+#pragma unroll
+        for (int u = 0; u < NP; ++u) {
+            if constexpr (TA) *reinterpret_cast<f32x4*>(&sA[buf][((tid >> 3) + 32 * u) * LDM + (tid & 7) * 4]) = va[u];
+            else *reinterpret_cast<f32x4*>(&sA[buf][((tid >> 5) + 8 * u) * LDK + (tid & 31) * 4]) = va[u];
+            if constexpr (TB) *reinterpret_cast<f32x4*>(&sB[buf][((tid >> 5) + 8 * u) * LDK + (tid & 31) * 4]) = vb[u];
+            else *reinterpret_cast<f32x4*>(&sB[buf][((tid >> 3) + 32 * u) * LDM + (tid & 7) * 4]) = vb[u];
+        }
+    };
+    // two stages of loads in flight: stage kt + 2 is requested before stage kt is multiplied
+    const int KT = (p.K + KB - 1) / KB;
+    f32x4 va[2][NP], vb[2][NP];
+    load_a(0, va[0]); load_b(0, vb[0]);
+    if (KT > 1) { load_a(KB, va[1]); load_b(KB, vb[1]); }
+    store(0, va[0], vb[0]);
+    __syncthreads();
+    for (int kt = 0; kt < KT; ++kt) {
+        const int buf = kt & 1;
+        if (kt + 2 < KT) { load_a((kt + 2) * KB, va[buf]); load_b((kt + 2) * KB, vb[buf]); }     // (stage kt's registers are in LDS already)
+        const float* a_s = sA[buf];
+        const float* b_s = sB[buf];
+        const int steps = p.K - kt * KB < KB ? (p.K - kt * KB) / 4 : KB / 4;      // (K is a multiple of 4: whole instructions)
+        // (groups of eight instructions; the sixteen operand reads of the next group are issued before the instructions of this
+        //  one, so that the chain never waits for LDS)
+        auto read_group = [&](int q0, float (&av)[8], float (&bv)[8]) __attribute__((always_inline)) {
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const int k = 4 * (q0 + u) + lg;
+                av[u] = TA ? a_s[k * LDM + bi * 16 + li] : a_s[(bi * 16 + li) * LDK + k];
+                bv[u] = TB ? b_s[(bj * 16 + li) * LDK + k] : b_s[k * LDM + bj * 16 + li];
+            }
+        };
+        if (steps == KB / 4) {
+            float av[2][8], bv[2][8];
+            read_group(0, av[0], bv[0]);
+#pragma unroll
+            for (int g = 0; g < KB / 32; ++g) {
+                if (g + 1 < KB / 32) read_group(8 * (g + 1), av[(g + 1) & 1], bv[(g + 1) & 1]);
+#pragma unroll
+                for (int u = 0; u < 8; ++u) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(bv[g & 1][u], av[g & 1][u], acc, 0, 0, 0);
+            }
+        } else {
+            for (int q = 0; q < steps; ++q) {                                     // (the last stage of a k that is not a multiple of 128)
+                const int k = 4 * q + lg;
+                const float av = TA ? a_s[k * LDM + bi * 16 + li] : a_s[(bi * 16 + li) * LDK + k];
+                const float bv = TB ? b_s[(bj * 16 + li) * LDK + k] : b_s[k * LDM + bj * 16 + li];
+                acc = __builtin_amdgcn_mfma_f32_16x16x4f32(bv, av, acc, 0, 0, 0);
+            }
+        }
+        if (kt + 1 < KT) store(buf ^ 1, va[buf ^ 1], vb[buf ^ 1]);
+        __syncthreads();
+    }
+    if (c_ok) {
+        if (p.act == ACT_RELU) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) acc[e] = acc[e] > 0.0f ? acc[e] : 0.0f;
+        }
+        *reinterpret_cast<f32x4*>(C + (int64_t)m * p.ldc + n) = acc;
+    }
+}
+
+// where the kernel above is ahead of the 64 x 64 tiles: those would reach fewer than half of the CUs, and k is deep enough for
+// the shorter chain to matter.  The results do not depend on the choice.
+static bool small16_f32_wins(const GemmParams& p) {
+    const int64_t t64 = (int64_t)((p.M + 63) / 64) * ((p.N + 63) / 64) * p.batch;
+    return t64 <= 128 && p.K >= 64 && p.M > 32 && p.cmode != C_PARTIAL && p.krange_items == 0;
+}
+static hipError_t launch_small16_f32(bool ta, bool tb, const GemmParams& pin, hipStream_t s) {
+    GemmParams p = pin;
+    p.tiles_m = (p.M + 31) / 32;
+    p.tiles_n = (p.N + 31) / 32;
+    const int64_t blocks = (int64_t)p.tiles_m * p.tiles_n * p.batch;
+    if (blocks <= 0) return hipSuccess;
+    const dim3 g((unsigned)blocks), t(256);
+    if (ta) { if (tb) hipLaunchKernelGGL((gemm_small16_f32_kernel<true, true>), g, t, 0, s, p); else hipLaunchKernelGGL((gemm_small16_f32_kernel<true, false>), g, t, 0, s, p); }
+    else { if (tb) hipLaunchKernelGGL((gemm_small16_f32_kernel<false, true>), g, t, 0, s, p); else hipLaunchKernelGGL((gemm_small16_f32_kernel<false, false>), g, t, 0, s, p); }
+    return hipGetLastError();
+}
+
 hipError_t launch_gemm_mfma_f32(bool ta, bool tb, const GemmParams& p, hipStream_t s) {
+    if (ring_eligible(p, ta, 4) && small16_f32_wins(p)) return launch_small16_f32(ta, tb, p, s);
     if (ring_eligible(p, ta, 4))
         return ring_f32_tile_edge(p) == 64 ? launch_ring_wb<DT_F32, 1>(ta, tb, p, s) : launch_ring_wb<DT_F32, 2>(ta, tb, p, s);
     // rows that are not 16-byte aligned (or pointer tables): register-staged kernel, 128 x 128 x 32 tiles unless that
@@ -25,6 +174,7 @@ hipError_t launch_gemm_mfma_f32(bool ta, bool tb, const GemmParams& p, hipStream
 hipError_t launch_gemm_ring_only_f32(bool ta, bool tb, const GemmParams& p, hipStream_t s, bool* taken) {
     *taken = ring_eligible(p, ta, 4);
     if (!*taken) return hipSuccess;
+    if (small16_f32_wins(p)) return launch_small16_f32(ta, tb, p, s);
     return ring_f32_tile_edge(p) == 64 ? launch_ring_wb<DT_F32, 1>(ta, tb, p, s) : launch_ring_wb<DT_F32, 2>(ta, tb, p, s);
 }
 // convolution / conv_dkernel with op(B) gathered from the image (tb: col^T), nd = 2 or 3 spatial axes

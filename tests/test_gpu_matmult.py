@@ -71,7 +71,7 @@ def host_matmult(sa, sb, c, m, k, n, ta, tb, dt):
     return c
 
 
-def dev_matmult(sa, sb, c0, m, k, n, ta, tb, dtype, mode=_lib.C_ACCUMULATE):
+def dev_matmult(sa, sb, c0, m, k, n, ta, tb, dtype, mode=_lib.C_ACCUMULATE, flags=0):
     bf = dtype == "bf16"
     ta_, tb_ = to_torch(sa, DEV, bf), to_torch(sb, DEV, bf)
     tc = to_torch(c0.copy(), DEV, bf)
@@ -80,6 +80,7 @@ def dev_matmult(sa, sb, c0, m, k, n, ta, tb, dtype, mode=_lib.C_ACCUMULATE):
     d.dtype = code_of(dtype)
     d.transpose_a, d.transpose_b, d.c_mode = int(ta), int(tb), mode
     d.m, d.k, d.n, d.batches = m, k, n, 1
+    d.flags = flags
     _lib.check(lib.ntg_gemm_dev(ctypes.byref(d), ta_.data_ptr(), tb_.data_ptr(), tc.data_ptr(),
                                 ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)))
     torch.cuda.synchronize()
@@ -1146,7 +1147,11 @@ def test_item_is_the_same_alone_and_in_every_batch_form(dtype, shape):
         c = np.zeros((m, n), ha[0].dtype)
         host_matmult(ha[i], hb[i], c, m, k, n, False, False, code)
         single.append(c)
-        assert np.array_equal(c.view(np.uint8), alone_np(a[i], b[i]).view(np.uint8)), (shape, "host alone == device alone", i)
+        # (Float32: the seam keeps the reference's order of summation -- NTG_GEMM_KEEP_K_ORDER -- so it stands beside the device
+        #  entry under the same flag; the other dtypes beside the functional face, workspace forms included)
+        dev_alone = dev_matmult(ha[i], hb[i], np.zeros((m, n), ha[0].dtype), m, k, n, False, False, dtype, mode=_lib.C_OVERWRITE,
+                                flags=_lib.GEMM_KEEP_K_ORDER) if dtype is np.float32 else alone_np(a[i], b[i])
+        assert np.array_equal(c.view(np.uint8), dev_alone.view(np.uint8)), (shape, "host alone == device alone", i)
     arr = ctypes.c_void_p * 4
     for name, ia, ib in (("distinct", [0, 1, 2, 3], [0, 1, 2, 3]), ("shared b", [0, 1, 2, 3], [1, 1, 1, 1]), ("mixed", [0, 1, 0, 1], [2, 2, 3, 3])):
         got = [np.zeros((m, n), ha[0].dtype) for _ in range(4)]
