@@ -18,6 +18,13 @@
  *   - the GEMM ACCUMULATES: C[m, n] += op(A) . op(B); the caller initialises C;
  *   - A and B are read-only and may alias each other; C must not alias an input.
  *
+ * Results against the reference's: the integer and complex types are bit-identical.  Float32 products are bit-identical too --
+ * every element is the reference's chain c = C0; c = fma(a[i,k], b[k,j], c) in ascending k (nt_matmult.hpp:196: k tiles
+ * outermost and ascending) -- through the host-pointer entry points always, through the device entry points unless a
+ * workspace lets the product be split along k or it has at most 32 rows (NTG_GEMM_KEEP_K_ORDER switches both off), and so is
+ * the Float32 convolution on the gathering kernels (no workspace: unfold + matmult, conv.cpp:86-95).  Float64, Float16 and
+ * BFloat16 results agree to the bounds stated with the tests (their matrix instructions do not sum k in a chain).
+ *
  * Every entry point returns 0 (NTG_OK) or a non-zero ntg_status and never throws;
  * ntg_last_error() returns a thread-local description of the last failure.
  * Host-pointer entry points are synchronous (results are in C on return) and thread-safe

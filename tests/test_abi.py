@@ -169,6 +169,13 @@ def test_split_k_planner_needs_no_device():
     assert ranges(_lib.FLOAT64, 256, 1024, 256, 8) == 8
     assert ws(_lib.FLOAT32, 1024, 4096, 1024) == 0 and ws(_lib.FLOAT64, 1024, 4096, 1024) == 0
     assert ws(_lib.FLOAT32, 768, 768, 768) == 0
+    # NTG_GEMM_KEEP_K_ORDER: no split along k is offered (padded copies and byte planes keep the order and stay on offer)
+    d = _lib.GemmDesc()
+    d.dtype, d.c_mode, d.flags = _lib.FLOAT32, _lib.C_OVERWRITE, _lib.GEMM_KEEP_K_ORDER
+    d.m, d.k, d.n, d.batches = 256, 1024, 256, 1
+    assert lib.ntg_gemm_workspace_bytes(ctypes.byref(d)) == 0
+    d.dtype, d.m, d.k, d.n = _lib.BFLOAT16, 128, 8192, 8190
+    assert lib.ntg_gemm_workspace_bytes(ctypes.byref(d)) == 8192 * 8192 * 2 + 128 * 8192 * 2
 
 
 def test_missing_library_fails_loudly(monkeypatch, tmp_path):
