@@ -1767,7 +1767,13 @@ int ntg_conv2d(int dtype, const void* image, const void* kernel, void* out,
     const size_t im_bytes = (size_t)(batch * channels * height * width * es);
     const size_t k_bytes = (size_t)(out_channels * (channels / groups) * k_r * k_c * es);
     const size_t o_bytes = (size_t)(batch * out_channels * Ho * Wo * es);
-    const int64_t ws = ntg_conv2d_fast_workspace_bytes(dtype, batch, channels, height, width, out_channels, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c, groups);
+    // Float32 at the reference's seam: the gathering kernels (no workspace), whose k axis is im2col's own -- the result is
+    // unfold + matmult bit for bit (conv.cpp:86-95); the channels-last kernels sum the same products taps-outermost, and what
+    // they would gain is small beside the transfers of this call.  The other dtypes take the faster form.
+    const int64_t ws = dtype == ntg::DT_F32
+        ? ntg_conv2d_forward_workspace_bytes(dtype, batch, channels, height, width, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c)
+        : ntg_conv2d_fast_workspace_bytes(dtype, batch, channels, height, width, out_channels, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c, groups);
+    if (ws < 0) return fail(NTG_ERR_INVALID_ARGUMENT, "the array of sliding blocks would be empty");
     ntg::HostSession mem;
     const size_t ok_ = align_up(im_bytes, 256), oo = ok_ + align_up(k_bytes, 256), ow = oo + align_up(o_bytes, 256);
     HIP_TRY(mem.reserve(ow + (size_t)ws));
