@@ -1630,13 +1630,17 @@ static int conv_dkernel_from_col(int dtype, const char* gy, char* col, void* d_k
 
 // Which backward gradients run as implicit GEMMs, and the workspace the call needs.
 struct ConvBackwardPlan { bool gather_dw, gather_dx, nhwc_dx, nhwc_dw, phase_dx; int64_t need, need_nhwc_dx, need_nhwc_dw, need_phase_dx; PhasePlan phases; };
+// reference_order (Float32 through the host entry points): the forms whose sums are the reference's own, bit for bit -- the
+// image gradient as W^T . dY into the col matrix + col2im (conv.cpp:318-346; the implicit forms run one chain over out
+// channels and taps where the reference rounds in between), the weight gradient per image with k = the output pixels +
+// the sum over the batch (conv.cpp:444-471; not the channels-last kernels, whose partial sums may span images).
 static ConvBackwardPlan plan_conv_backward_g(int dtype, bool want_dx, bool want_dw, int64_t batch, int64_t channels, int64_t out_channels,
-                                             const Geo3& g, int64_t groups) {
+                                             const Geo3& g, int64_t groups, bool reference_order = false) {
     const int64_t es = ntg::elem_size(dtype);
     const int64_t cg = channels / groups, taps = g.taps();
     ConvBackwardPlan pl;
     pl.gather_dw = want_dw && conv_implicit_g(dtype, channels, g);
-    pl.gather_dx = want_dx && g.s[0] == 1 && g.s[1] == 1 && g.s[2] == 1 && conv_implicit_g(dtype, out_channels, geo_dimage(g));
+    pl.gather_dx = want_dx && !reference_order && g.s[0] == 1 && g.s[1] == 1 && g.s[2] == 1 && conv_implicit_g(dtype, out_channels, geo_dimage(g));
     const int64_t col = batch * channels * taps * g.L() * es;
     int64_t need = 0;
     if (want_dw) need = std::max(need, pl.gather_dw ? batch * out_channels * cg * taps * es : col + complex_dkernel_extra(dtype, batch, out_channels, cg * taps, col));
@@ -1645,11 +1649,11 @@ static ConvBackwardPlan plan_conv_backward_g(int dtype, bool want_dx, bool want_
     // the channels-last form of dX is taken when the caller's workspace also holds the copy of dY
     pl.nhwc_dx = pl.gather_dx && g.nd == 2 && conv_dimage_nhwc_ok(dtype, channels, out_channels, groups, g);
     pl.need_nhwc_dx = pl.nhwc_dx ? conv_dimage_nhwc_workspace(dtype, batch, channels, out_channels, groups, g) : 0;
-    pl.nhwc_dw = pl.gather_dw && conv_dkernel_nhwc_ok(dtype, channels, out_channels, groups, g);
+    pl.nhwc_dw = pl.gather_dw && !reference_order && conv_dkernel_nhwc_ok(dtype, channels, out_channels, groups, g);
     pl.need_nhwc_dw = pl.nhwc_dw ? conv_dkernel_nhwc_workspace(dtype, batch, channels, out_channels, groups, g) : 0;
     // strides > 1: dX phase by phase instead of GEMM + col2im, again when the workspace allows
     std::memset(&pl.phases, 0, sizeof pl.phases);
-    if (want_dx && !pl.gather_dx && conv_implicit_g(dtype, out_channels, geo_dimage(g)))
+    if (want_dx && !pl.gather_dx && !reference_order && conv_implicit_g(dtype, out_channels, geo_dimage(g)))
         pl.phases = plan_dimage_phases(dtype, batch, channels, out_channels, groups, g);
     pl.phase_dx = pl.phases.ok;
     pl.need_phase_dx = pl.phase_dx ? pl.phases.gy_bytes + pl.phases.w_bytes + pl.phases.tmp_bytes : 0;
@@ -1832,9 +1836,9 @@ int ntg_unfold2d_backward(int dtype, const void* col, void* image,
 
 static ConvBackwardPlan plan_conv_backward(int dtype, bool want_dx, bool want_dw, int64_t batch, int64_t channels, int64_t height, int64_t width,
                                            int64_t out_channels, int64_t k_r, int64_t k_c, int64_t s_r, int64_t s_c, int64_t p_r, int64_t p_c,
-                                           int64_t d_r, int64_t d_c, int64_t groups, int64_t Ho, int64_t Wo) {
+                                           int64_t d_r, int64_t d_c, int64_t groups, int64_t Ho, int64_t Wo, bool reference_order = false) {
     return plan_conv_backward_g(dtype, want_dx, want_dw, batch, channels, out_channels,
-                                geo2(height, width, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c, Ho, Wo), groups);
+                                geo2(height, width, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c, Ho, Wo), groups, reference_order);
 }
 
 int64_t ntg_conv2d_backward_workspace_bytes(int dtype, int64_t batch, int64_t channels, int64_t height, int64_t width,
@@ -1849,12 +1853,12 @@ int64_t ntg_conv2d_backward_workspace_bytes(int dtype, int64_t batch, int64_t ch
     return std::max(std::max(pl.need, pl.need_phase_dx), std::max(pl.need_nhwc_dx, pl.need_nhwc_dw));
 }
 
-int ntg_conv2d_backward_dev(int dtype, const void* image, const void* kernel, const void* grad_out,
-                            void* d_image, void* d_kernel, void* workspace, int64_t workspace_bytes,
-                            int64_t batch, int64_t channels, int64_t height, int64_t width,
-                            int64_t out_channels, int64_t k_r, int64_t k_c,
-                            int64_t s_r, int64_t s_c, int64_t p_r, int64_t p_c, int64_t d_r, int64_t d_c,
-                            int64_t groups, int accumulate, void* stream) {
+static int conv2d_backward_dev_impl(int dtype, const void* image, const void* kernel, const void* grad_out,
+                                    void* d_image, void* d_kernel, void* workspace, int64_t workspace_bytes,
+                                    int64_t batch, int64_t channels, int64_t height, int64_t width,
+                                    int64_t out_channels, int64_t k_r, int64_t k_c,
+                                    int64_t s_r, int64_t s_c, int64_t p_r, int64_t p_c, int64_t d_r, int64_t d_c,
+                                    int64_t groups, int accumulate, void* stream, bool reference_order) {
     const int64_t es = ntg::elem_size(dtype);
     if (es == 0) return fail(NTG_ERR_UNSUPPORTED_DTYPE, "dtype %d is not supported", dtype);
     if (batch < 0 || channels < 0 || out_channels < 0 || height < 0 || width < 0) return fail(NTG_ERR_INVALID_ARGUMENT, "negative size");
@@ -1869,7 +1873,7 @@ int ntg_conv2d_backward_dev(int dtype, const void* image, const void* kernel, co
     const int64_t L = Ho * Wo, ckk = channels * k_r * k_c;
     const int64_t add = (channels / groups) * k_r * k_c, og = out_channels / groups;
     const ConvBackwardPlan plan = plan_conv_backward(dtype, d_image != nullptr, d_kernel != nullptr, batch, channels, height, width,
-                                                     out_channels, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c, groups, Ho, Wo);
+                                                     out_channels, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c, groups, Ho, Wo, reference_order);
     if (plan.need > 0 && (!workspace || workspace_bytes < plan.need))
         return fail(NTG_ERR_INVALID_ARGUMENT, "workspace of %lld bytes needed, %lld given", (long long)plan.need, (long long)workspace_bytes);
     const char* kern = static_cast<const char*>(kernel);
@@ -1883,7 +1887,7 @@ int ntg_conv2d_backward_dev(int dtype, const void* image, const void* kernel, co
     // 1x1 kernel, unit stride, no padding (floating dtypes, 16-byte rows): col is the image itself, so both gradients are
     // products on the tensors where they lie: dX_b = W_g^T . dY_b, and dW_g = sum_b dY_b . X_b^T through per-image results
     // in the workspace (the amount the gathering form needs), summed in batch order.
-    if (!is_valu_dtype(dtype) && conv_pointwise_ok(dtype, channels, groups, geo) && (og * es) % 16 == 0 &&
+    if (!is_valu_dtype(dtype) && !(reference_order && accumulate) && conv_pointwise_ok(dtype, channels, groups, geo) && (og * es) % 16 == 0 &&
         ((reinterpret_cast<uintptr_t>(image) | reinterpret_cast<uintptr_t>(kernel) | reinterpret_cast<uintptr_t>(grad_out) |
           reinterpret_cast<uintptr_t>(d_image) | reinterpret_cast<uintptr_t>(d_kernel) | reinterpret_cast<uintptr_t>(ws)) & 15) == 0) {
         const int64_t cg = channels / groups;
@@ -1953,6 +1957,16 @@ int ntg_conv2d_backward_dev(int dtype, const void* image, const void* kernel, co
         if (rc) return rc;
     }
     return NTG_OK;
+}
+
+int ntg_conv2d_backward_dev(int dtype, const void* image, const void* kernel, const void* grad_out,
+                            void* d_image, void* d_kernel, void* workspace, int64_t workspace_bytes,
+                            int64_t batch, int64_t channels, int64_t height, int64_t width,
+                            int64_t out_channels, int64_t k_r, int64_t k_c,
+                            int64_t s_r, int64_t s_c, int64_t p_r, int64_t p_c, int64_t d_r, int64_t d_c,
+                            int64_t groups, int accumulate, void* stream) {
+    return conv2d_backward_dev_impl(dtype, image, kernel, grad_out, d_image, d_kernel, workspace, workspace_bytes, batch, channels, height, width,
+                                    out_channels, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c, groups, accumulate, stream, false);
 }
 
 // conv_transpose2d = the image gradient of the convolution whose output is `input`: per group
@@ -2071,8 +2085,13 @@ int ntg_conv2d_backward(int dtype, const void* image, const void* kernel, const 
     const size_t im_bytes = (size_t)(batch * channels * height * width * es);
     const size_t k_bytes = (size_t)(out_channels * (channels / groups) * k_r * k_c * es);
     const size_t g_bytes = (size_t)(batch * out_channels * Ho * Wo * es);
-    const int64_t wsb = ntg_conv2d_backward_workspace_bytes(dtype, batch, channels, height, width, out_channels, k_r, k_c, s_r, s_c,
-                                                            p_r, p_c, d_r, d_c, groups);
+    // Float32 at the reference's seam: its own two algorithms (see plan_conv_backward_g), whose results are conv_dimage's and
+    // conv_dkernel's bit for bit; what the faster forms would gain is small beside the transfers of this call
+    const bool reference_order = dtype == ntg::DT_F32;
+    const int64_t wsb = reference_order
+        ? plan_conv_backward(dtype, d_image != nullptr, d_kernel != nullptr, batch, channels, height, width, out_channels, k_r, k_c, s_r, s_c,
+                             p_r, p_c, d_r, d_c, groups, Ho, Wo, true).need
+        : ntg_conv2d_backward_workspace_bytes(dtype, batch, channels, height, width, out_channels, k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c, groups);
     ntg::HostSession mem;
     const size_t o_k = align_up(im_bytes, 256), o_g = o_k + align_up(k_bytes, 256), o_di = o_g + align_up(g_bytes, 256);
     const size_t o_dk = o_di + align_up(im_bytes, 256), o_ws = o_dk + align_up(k_bytes, 256);
@@ -2082,9 +2101,9 @@ int ntg_conv2d_backward(int dtype, const void* image, const void* kernel, const 
     HIP_TRY(mem.upload(o_g, grad_out, g_bytes));
     if (accumulate && d_image) HIP_TRY(mem.upload(o_di, d_image, im_bytes));
     if (accumulate && d_kernel) HIP_TRY(mem.upload(o_dk, d_kernel, k_bytes));
-    rc = ntg_conv2d_backward_dev(dtype, mem.at(0), mem.at(o_k), mem.at(o_g), d_image ? mem.at(o_di) : nullptr,
-                                 d_kernel ? mem.at(o_dk) : nullptr, mem.at(o_ws), wsb, batch, channels, height, width, out_channels,
-                                 k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c, groups, accumulate, mem.stream());
+    rc = conv2d_backward_dev_impl(dtype, mem.at(0), mem.at(o_k), mem.at(o_g), d_image ? mem.at(o_di) : nullptr,
+                                  d_kernel ? mem.at(o_dk) : nullptr, mem.at(o_ws), wsb, batch, channels, height, width, out_channels,
+                                  k_r, k_c, s_r, s_c, p_r, p_c, d_r, d_c, groups, accumulate, mem.stream(), reference_order);
     if (rc) return rc;
     if (d_image) HIP_TRY(mem.download(d_image, o_di, im_bytes));
     if (d_kernel) HIP_TRY(mem.download(d_kernel, o_dk, k_bytes));

@@ -22,7 +22,7 @@ __global__ void __launch_bounds__(256) reduce_batch_kernel(const T* __restrict__
 }
 
 
-// The reference's own order for the element types whose sums are checked bit for bit (the complex types):
+// The reference's own order for the element types whose sums are checked bit for bit (Float32, Float64, the complex types):
 // conv_dkernel forms sum(0) of the per-image products first -- item 0, then += item 1, ... in the element type
 // (tensor_files/sum_exp_log.cpp:112-124) -- and adds that sum to d_kernel last (conv.cpp:466-469).
 template <class T>
@@ -254,8 +254,8 @@ hipError_t launch_reduce_batch(int dtype, const void* part, void* out, int64_t b
     if (n == 0) return hipSuccess;
     const dim3 g(grid_for(n)), b(256);
     switch (dtype) {
-    case DT_F32: hipLaunchKernelGGL((reduce_batch_kernel<float, float>), g, b, 0, s, (const float*)part, (float*)out, batch, n, accumulate); break;
-    case DT_F64: hipLaunchKernelGGL((reduce_batch_kernel<double, double>), g, b, 0, s, (const double*)part, (double*)out, batch, n, accumulate); break;
+    case DT_F32: hipLaunchKernelGGL((reduce_batch_sum_first_kernel<float>), g, b, 0, s, (const float*)part, (float*)out, batch, n, accumulate); break;
+    case DT_F64: hipLaunchKernelGGL((reduce_batch_sum_first_kernel<double>), g, b, 0, s, (const double*)part, (double*)out, batch, n, accumulate); break;
     case DT_F16: hipLaunchKernelGGL((reduce_batch_kernel<_Float16, float>), g, b, 0, s, (const _Float16*)part, (_Float16*)out, batch, n, accumulate); break;
     case DT_BF16: hipLaunchKernelGGL((reduce_batch_kernel<__bf16, float>), g, b, 0, s, (const __bf16*)part, (__bf16*)out, batch, n, accumulate); break;
     case DT_C32: hipLaunchKernelGGL((reduce_batch_sum_first_kernel<LanePair<_Float16>>), g, b, 0, s, (const LanePair<_Float16>*)part, (LanePair<_Float16>*)out, batch, n, accumulate); break;

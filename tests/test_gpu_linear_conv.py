@@ -195,7 +195,10 @@ def test_conv2d_backward_golden(golden_dir, sfx, pad, groups):
     p = lambda a: np.ascontiguousarray(a).ctypes.data_as(ctypes.c_void_p)
     _lib.check(lib.ntg_conv2d_backward(_lib.FLOAT32, p(x), p(w), p(g), hx.ctypes.data_as(ctypes.c_void_p),
                                        hw.ctypes.data_as(ctypes.c_void_p), B, C, H, W, O, kh, kw, 1, 1, pad, pad, 1, 1, groups, 0))
-    assert np.array_equal(hx, dx) and np.array_equal(hw, dw)
+    # (Float32 at the host seam: the reference's own two algorithms, the oracle's bits; the functional face above may take the
+    #  implicit and channels-last forms, which sum the same products in another order)
+    assert np.array_equal(hx.view(np.uint32), odx.view(np.uint32)) and np.array_equal(hw.view(np.uint32), odw.view(np.uint32))
+    assert np.abs(hx - dx).max() <= 1e-5 * max(1.0, np.abs(dx).max()) and np.abs(hw - dw).max() <= 1e-4 * max(1.0, np.abs(dw).max())
     # accumulate != 0 adds to the incoming gradients, like the reference's += (conv.cpp:466-469)
     hx2, hw2 = hx.copy(), hw.copy()
     _lib.check(lib.ntg_conv2d_backward(_lib.FLOAT32, p(x), p(w), p(g), hx2.ctypes.data_as(ctypes.c_void_p),
@@ -767,3 +770,43 @@ def test_conv2d_fp32_without_workspace_is_the_reference_chain_bit_for_bit(geom):
     vp = lambda a: a.ctypes.data_as(ctypes.c_void_p)
     _lib.check(lib.ntg_conv2d(_lib.FLOAT32, vp(x), vp(w), vp(host), B, C, H, W, O, kh, kw, st, st, pd, pd, dl, dl, groups))
     assert np.array_equal(host.view(np.uint32), want.view(np.uint32)), (geom, "host entry")
+
+
+@pytest.mark.parametrize("geom", [
+    (2, 8, 18, 18, 16, 3, 3, 1, 1, 1, 1),
+    (3, 16, 20, 12, 24, 3, 3, 2, 1, 1, 2),
+    (2, 5, 9, 11, 7, 3, 2, 1, 0, 1, 1),
+    (1, 12, 15, 15, 8, 5, 5, 1, 2, 2, 1),
+    (4, 6, 10, 10, 6, 1, 1, 1, 0, 1, 1),        # 1 x 1: products on the tensors where they lie
+], ids=lambda g: "x".join(map(str, g)))
+def test_conv2d_backward_fp32_host_entry_is_the_reference_bit_for_bit(geom):
+    """ntg_conv2d_backward on host memory in Float32 runs the reference's own two algorithms -- conv_dimage as W^T . dY into the
+    col matrix + col2im (conv.cpp:318-346), conv_dkernel as one product per image over the output pixels + the sum over the batch
+    (conv.cpp:444-471) -- and returns the oracle's bits, also when it adds to gradients that are already there (square geometries here: one stride,
+    padding and dilation for both axes)."""
+    B, C, H, W, O, kh, kw, st, pd, dl, groups = geom
+    rng = np.random.default_rng(97 + B + C + O)
+    x = rng.standard_normal((B, C, H, W)).astype(np.float32)
+    w = (rng.standard_normal((O, C // groups, kh, kw)) * 2.0).astype(np.float32)
+    Ho = (H + 2 * pd - dl * (kh - 1) - 1) // st + 1
+    Wo = (W + 2 * pd - dl * (kw - 1) - 1) // st + 1
+    g = rng.standard_normal((B, O, Ho, Wo)).astype(np.float32)
+    odx, odw = oracle.conv2d_backward(x, w, g, st, pd, dl, groups)
+    lib = _lib.load()
+    vp = lambda a: a.ctypes.data_as(ctypes.c_void_p)
+    dx = np.full(x.shape, np.nan, np.float32)
+    dw = np.full(w.shape, np.nan, np.float32)
+    _lib.check(lib.ntg_conv2d_backward(_lib.FLOAT32, vp(x), vp(w), vp(g), vp(dx), vp(dw), B, C, H, W, O, kh, kw, st, st, pd, pd, dl, dl, groups, 0))
+    assert np.array_equal(dx.view(np.uint32), odx.view(np.uint32)), (geom, "d_image", int((dx != odx).sum()))
+    assert np.array_equal(dw.view(np.uint32), odw.view(np.uint32)), (geom, "d_kernel", int((dw != odw).sum()))
+    dx0 = rng.standard_normal(x.shape).astype(np.float32)
+    dw0 = rng.standard_normal(w.shape).astype(np.float32)
+    dx, dw = dx0.copy(), dw0.copy()
+    _lib.check(lib.ntg_conv2d_backward(_lib.FLOAT32, vp(x), vp(w), vp(g), vp(dx), vp(dw), B, C, H, W, O, kh, kw, st, st, pd, pd, dl, dl, groups, 1))
+    # d_kernel: the summed per-image products are added in one addition (sum(0), then +=); d_image: unfold2d_backward scatters
+    # onto the tensor it is handed, so the taps land on the old values one by one (conv.cpp:343-345)
+    assert np.array_equal(dw.view(np.uint32), (dw0 + odw).view(np.uint32)), (geom, "d_kernel +=")
+    from test_gpu_complex import _col2im_onto, _dcol_plane
+    dcol = _dcol_plane(oracle, w, g, B, C, O, kh, kw, groups, None)
+    want = _col2im_onto(dx0, dcol, (H, W), (kh, kw), dl, pd, st)
+    assert np.array_equal(dx.view(np.uint32), np.ascontiguousarray(want).view(np.uint32)), (geom, "d_image +=")
