@@ -2408,6 +2408,11 @@ int ntg_convnd_backward(int dtype, const void* image, const void* kernel, const 
     if (rc) return rc;
     if (batch == 0 || out_channels == 0 || channels == 0) return NTG_OK;
     if (!image || !kernel || !grad_out) return fail(NTG_ERR_INVALID_ARGUMENT, "null pointer");
+    if (ndim <= 2) {        // (the two-axis host entry point: it keeps the reference's order of summation for Float32)
+        const Geo2 g = as_2d(ndim, size, kernel_size, stride, padding, dilation);
+        return ntg_conv2d_backward(dtype, image, kernel, grad_out, d_image, d_kernel, batch, channels, g.h, g.w, out_channels, g.kr, g.kc,
+                                   g.sr, g.sc, g.pr, g.pc, g.dr, g.dc, groups, accumulate);
+    }
     const size_t im_bytes = (size_t)(batch * channels * u.vol * es), k_bytes = (size_t)(out_channels * (channels / groups) * u.taps * es);
     const size_t g_bytes = (size_t)(batch * out_channels * u.L * es);
     const int64_t wsb = ntg_convnd_workspace_bytes(dtype, batch, channels, out_channels, ndim, size, kernel_size, stride, padding, dilation, groups, 1);
