@@ -30,6 +30,7 @@ __global__ void __launch_bounds__(256) gemm_small16_f32_kernel(const GemmParams 
     __shared__ __attribute__((aligned(16))) float sA[2][A_STAGE];
     __shared__ __attribute__((aligned(16))) float sB[2][B_STAGE];
     typedef float f32x4 __attribute__((ext_vector_type(4)));
+    if (p.gate && *p.gate != p.gate_want) return;       // (uniform: the other kernel of a gated pair does this product)
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int bi = wave >> 1, bj = wave & 1, li = lane & 15, lg = lane >> 4;
     const int tiles = p.tiles_m * p.tiles_n;

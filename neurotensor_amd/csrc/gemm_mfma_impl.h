@@ -427,6 +427,7 @@ __global__ void __launch_bounds__(256) gemm_mfma_kernel(const GemmParams p) {
 
     extern __shared__ __attribute__((aligned(16))) char smem[];
 
+    if (p.gate && *p.gate != p.gate_want) return;       // (uniform: the other kernel of a gated pair does this product)
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;

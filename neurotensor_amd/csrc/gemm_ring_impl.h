@@ -239,6 +239,7 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
     constexpr int DW_TABLE = CONV == 4 ? dw_table_entries(WB) : 1;
     __shared__ int dw_tab[DW_TABLE];
 
+    if (p.gate && *p.gate != p.gate_want) return;       // (uniform: the other kernel of a gated pair does this product)
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;

@@ -96,6 +96,10 @@ struct GemmParams {
     int tiles_m, tiles_n;
     int vecA_ok, vecB_ok;    // 16-byte vector loads are legal for every row of A / B
     int keep_k_order;        // never split along k (the caller wants the one chain per element in ascending k)
+    // Pointer tables whose entries' alignment the library found out on the device (see gemm_ptrs): the product is launched on
+    // the DMA-fed kernel AND on the register-staged one; a kernel whose gate_want differs from *gate returns at once.
+    const int* gate;
+    int gate_want;
     int ptrs_aligned;        // pointer tables only: the caller vouches that every entry is a multiple of 16 bytes (the tables
                              // live in device memory, the host cannot look); lets table batches onto the DMA-fed kernels
     int group_m;             // DMA-fed kernels: tile rows per group of the tile order (0: the default, 4; see tile_coords)

@@ -79,6 +79,25 @@ hipError_t launch_conv_mfma(int dtype, bool tb, int nd, const GemmParams& p, hip
 // for the address of the current device's copy once and keeps it.
 static __device__ __align__(256) unsigned char scratch[NTG_NOALLOC_SCRATCH_BYTES];
 
+// Flags of ntg_gemm_ptrs_dev's alignment check (one word per call, handed out round-robin), in the same kind of array and
+// for the same reason: the device entry points allocate nothing.
+#define NTG_GATE_SLOTS 1024
+static __device__ __align__(256) int gate_flags[NTG_GATE_SLOTS];
+namespace ntg {
+// *flag = 1 when every entry of the three pointer tables is a multiple of 16 bytes, else 0
+__global__ void __launch_bounds__(256) ptr_tables_aligned_kernel(const void* const* a, const void* const* b, void* const* c, const int batch, int* flag) {
+    __shared__ unsigned bits;
+    if (threadIdx.x == 0) bits = 0u;
+    __syncthreads();
+    unsigned mine = 0u;
+    for (int i = threadIdx.x; i < batch; i += 256)
+        mine |= (unsigned)(reinterpret_cast<uintptr_t>(a[i]) | reinterpret_cast<uintptr_t>(b[i]) | reinterpret_cast<uintptr_t>(c[i])) & 15u;
+    if (mine) atomicOr(&bits, mine);
+    __syncthreads();
+    if (threadIdx.x == 0) *flag = bits == 0u ? 1 : 0;
+}
+}  // namespace ntg
+
 namespace {
 
 thread_local std::string g_last_error;
@@ -622,6 +641,56 @@ int ntg_gemm_noalloc_dev(const ntg_gemm_desc* d, const void* dA, const void* dB,
     return rc;
 }
 
+// Address of the current device's copy of gate_flags (looked up once per device) and the next slot of it.
+static int next_gate_slot(int** out) {
+    constexpr int kMaxDevices = 64;
+    static std::mutex mutex;
+    static int* base[kMaxDevices];
+    static unsigned next[kMaxDevices];
+    int dev = -1;
+    HIP_TRY(hipGetDevice(&dev));
+    if (dev < 0 || dev >= kMaxDevices) return fail(NTG_ERR_DEVICE, "device ordinal %d outside 0..%d", dev, kMaxDevices - 1);
+    std::lock_guard<std::mutex> lock(mutex);
+    if (!base[dev]) {
+        void* ptr = nullptr;
+        HIP_TRY(hipGetSymbolAddress(&ptr, HIP_SYMBOL(gate_flags)));
+        if (!ptr) return fail(NTG_ERR_DEVICE, "hipGetSymbolAddress returned a null address for the gate flags");
+        base[dev] = static_cast<int*>(ptr);
+    }
+    *out = base[dev] + (next[dev]++ % NTG_GATE_SLOTS);
+    return NTG_OK;
+}
+
+// Pointer tables without the caller's vouch: the entries' alignment is a fact of device memory, so it is found out there.  A
+// one-workgroup kernel ORs the low bits of all entries into a flag; then the product is launched twice, on the DMA-fed
+// kernel (which needs 16-byte entries) and on the register-staged one (which does not), each returning at once unless the
+// flag names it.  The two kernels give the same bits, so nothing depends on which one runs.  Worth two extra launches
+// (about 4 us) only for products that take a few times that; the floating types that have both kernels, more than 32 rows.
+static bool gated_tables_pay(const ntg::GemmParams& p, int dtype) {
+    if (dtype != ntg::DT_F32 && dtype != ntg::DT_F16 && dtype != ntg::DT_BF16) return false;
+    if (p.M <= 32 || p.K <= 0 || p.act != ntg::ACT_NONE) return false;
+    const double flops = 2.0 * (double)p.M * (double)p.N * (double)p.K * (double)p.batch;
+    return flops >= (dtype == ntg::DT_F32 ? 3.2e10 : 8.0e9);
+}
+static int launch_gemm_tables_gated(ntg::GemmParams p, int dtype, bool ta, bool tb, hipStream_t s) {
+    int* flag = nullptr;
+    int rc = next_gate_slot(&flag);
+    if (rc) return rc;
+    hipLaunchKernelGGL(ntg::ptr_tables_aligned_kernel, dim3(1), dim3(256), 0, s, p.Aptr, p.Bptr, p.Cptr, p.batch, flag);
+    HIP_TRY(hipGetLastError());
+    const int64_t ve = 16 / ntg::elem_size(dtype);
+    ntg::GemmParams q = p;
+    q.vecA_ok = p.lda % ve == 0;
+    q.vecB_ok = p.ldb % ve == 0;
+    q.ptrs_aligned = 1; q.gate = flag; q.gate_want = 1;
+    bool taken = false;
+    hipError_t e = ntg::launch_gemm_ring_only(dtype, ta, tb, q, s, &taken);
+    if (e != hipSuccess) return hip_fail(e, "gemm launch");
+    p.ptrs_aligned = 0;
+    if (taken) { p.gate = flag; p.gate_want = 0; }        // (not taken: sizes or pitches rule the DMA-fed kernel out anyway)
+    return launch_gemm(p, dtype, ta, tb, s);
+}
+
 // aligned: the caller vouches that every table entry is a multiple of 16 bytes (true for the host entry points' own arena)
 static int gemm_ptrs(const ntg_gemm_desc* d, const void* const* dA, const void* const* dB, void* const* dC, void* stream, bool aligned) {
     ntg::GemmParams p;
@@ -631,6 +700,8 @@ static int gemm_ptrs(const ntg_gemm_desc* d, const void* const* dA, const void* 
     if (!dA || !dB || !dC) return fail(NTG_ERR_INVALID_ARGUMENT, "null pointer table");
     p.Aptr = dA; p.Bptr = dB; p.Cptr = dC;
     p.ptrs_aligned = aligned ? 1 : 0;
+    if (!aligned && gated_tables_pay(p, d->dtype))
+        return launch_gemm_tables_gated(p, d->dtype, d->transpose_a != 0, d->transpose_b != 0, static_cast<hipStream_t>(stream));
     return run_gemm(p, d->dtype, d->transpose_a != 0, d->transpose_b != 0, static_cast<hipStream_t>(stream));
 }
 

@@ -1296,3 +1296,36 @@ def test_host_entry_points_fp32_are_the_reference_chain_bit_for_bit(shape):
     vp = lambda x: x.ctypes.data_as(ctypes.c_void_p)
     _lib.check(lib.ntg_linear(_lib.FLOAT32, vp(a), vp(w_nk), vp(bias), vp(y), m, k, n, 0, 1, 1, n))
     assert np.array_equal(y.view(np.uint32), want.view(np.uint32)), (shape, "linear")
+
+
+@pytest.mark.parametrize("dtype", ["bf16", np.float32], ids=["bf16", "fp32"])
+def test_pointer_tables_without_a_vouch_find_their_alignment_on_the_device(dtype):
+    """ntg_gemm_ptrs_dev without NTG_GEMM_PTRS_ALIGNED16 on products large enough to pay for it: a small kernel looks at the
+    tables' entries, and the product runs on the DMA-fed kernel when all of them are 16-byte multiples, on the register-staged
+    one otherwise (both are launched, one of them returns at once).  Aligned tables, then tables with one entry moved by one
+    element: in both cases every item has the bits of the item alone."""
+    bf = dtype == "bf16"
+    m, k, n, nb = (1024, 1024, 1024, 6) if bf else (2048, 1024, 2048, 5)
+    rng = np.random.default_rng(60606)
+    lib = _lib.load()
+    st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    # operands inside larger buffers, so that an entry can be moved by one element without leaving its allocation
+    abuf = to_torch(randn(rng, (nb, m * k + 8), dtype, 0.5), DEV, bf)
+    bbuf = to_torch(randn(rng, (nb, k * n + 8), dtype, 0.5), DEV, bf)
+    bits = lambda t: t.contiguous().view(torch.int16 if t.element_size() == 2 else torch.int32)
+    for shift in (0, 1):
+        offs = [0] * nb
+        offs[2] = shift                                   # one misaligned A, and below one misaligned B
+        a = [abuf[i, offs[i]:offs[i] + m * k].view(m, k) for i in range(nb)]
+        b = [bbuf[i, (shift if i == 4 else 0):(shift if i == 4 else 0) + k * n].view(k, n) for i in range(nb)]
+        alone = [F.matmult(a[i].clone(), b[i].clone()) for i in range(nb)]
+        c = torch.zeros((nb, m, n), dtype=abuf.dtype, device=DEV)
+        d = _lib.GemmDesc()
+        d.dtype = code_of(dtype)
+        d.c_mode = _lib.C_OVERWRITE
+        d.m, d.k, d.n, d.batches = m, k, n, nb
+        tab = torch.tensor([x.data_ptr() for x in a] + [x.data_ptr() for x in b] + [c[j].data_ptr() for j in range(nb)], dtype=torch.int64, device=DEV)
+        _lib.check(lib.ntg_gemm_ptrs_dev(ctypes.byref(d), tab.data_ptr(), tab.data_ptr() + 8 * nb, tab.data_ptr() + 16 * nb, st))
+        torch.cuda.synchronize()
+        for i in range(nb):
+            assert torch.equal(bits(c[i]), bits(alone[i])), (dtype, "shift", shift, "item", i)
