@@ -58,7 +58,7 @@ def sub(buf, off, rows, cols, ld):
     return np.lib.stride_tricks.as_strided(buf[off:], (rows, cols), (ld * buf.itemsize, buf.itemsize))
 
 
-def run_case(rng, name, m, k, n, ta, tb, pads, mode, batches=1, gap=0, base=0, bcast_b=False, workspace=False, one_rounding=False):
+def run_case(rng, name, m, k, n, ta, tb, pads, mode, batches=1, gap=0, base=0, bcast_b=False, workspace=False, one_rounding=False, flags=0, f32_bits=False):
     npdt, code, ocode = DTYPES[name]
     es = np.dtype(npdt).itemsize
     ra, ca = (k, m) if ta else (m, k)
@@ -79,6 +79,9 @@ def run_case(rng, name, m, k, n, ta, tb, pads, mode, batches=1, gap=0, base=0, b
         d.bias, d.bias_col_stride = dbias.data_ptr(), 1
     lib = _lib.load()
     ws = None
+    d.flags = flags
+    if workspace == "offered":                        # whatever form the query offers for this descriptor, if any
+        workspace = lib.ntg_gemm_workspace_bytes(ctypes.byref(d)) > 0
     if workspace:
         need = lib.ntg_gemm_workspace_bytes(ctypes.byref(d))
         if workspace is not True:
@@ -91,7 +94,7 @@ def run_case(rng, name, m, k, n, ta, tb, pads, mode, batches=1, gap=0, base=0, b
     torch.cuda.synchronize()
     got = dC.cpu().numpy().view(npdt)
     want = bufC.copy()                     # bytes outside the C sub-views must survive
-    what = f"{name} {m}x{k}x{n} ta={ta} tb={tb} pads={pads} mode={mode} batches={batches} base={base} ws={workspace}"
+    what = f"{name} {m}x{k}x{n} ta={ta} tb={tb} pads={pads} mode={mode} batches={batches} gap={gap} base={base} bcast_b={bcast_b} ws={workspace} flags={flags}"
     for bi in range(batches):
         sa = np.ascontiguousarray(sub(bufA, base + bi * sA, ra, ca, lda))
         sb = np.ascontiguousarray(sub(bufB, base + bi * sB, rb, cb, ldb))
@@ -110,6 +113,8 @@ def run_case(rng, name, m, k, n, ta, tb, pads, mode, batches=1, gap=0, base=0, b
             if name in ("f32", "f64"):
                 err = np.abs(g.astype(np.float64) - ref.astype(np.float64)).max()
                 assert err <= float_tol(k, al, bl), f"{what} item {bi}: max|d| = {err}"
+                if f32_bits:       # the reference's chain of fused multiply-adds in ascending k, starting from C0: the same bits
+                    assert np.array_equal(g.view(np.uint32), ref.view(np.uint32)), f"{what} item {bi}: {int((g != ref).sum())} elements differ from the chain"
             else:
                 r64 = widen(name, ref)
                 assert np.abs(widen(name, g) - r64).max() <= HALF_REL * max(np.abs(r64).max(), 1e-30), f"{what} item {bi}"
@@ -198,3 +203,47 @@ def test_rows_that_are_not_16_byte_multiples_through_padded_copies(name):
     run_case(rng, name, m + 3, k + 7, n + 1, True, False, ODD, _lib.C_BIAS, base=1, workspace=True, one_rounding=half)   # everything odd, C padded too
     run_case(rng, name, m, k + 7, n - 6, False, True, (0, 8, 5), _lib.C_ACCUMULATE, batches=2, gap=3, workspace=True, one_rounding=half)
     run_case(rng, name, m, 1008, n - 6, False, False, (0, 0, 0), _lib.C_OVERWRITE, batches=2, bcast_b=True, base=3, workspace=64 << 20, one_rounding=half)   # only the base pointers are odd
+
+
+def _random_dim(rng, hi):
+    """sizes that sit on, just below and just above the tile edges, tiny ones, multiples of 8 and anything else"""
+    kind = int(rng.integers(0, 4))
+    if kind == 0:
+        return int(rng.integers(1, 40))
+    if kind == 1:
+        d = int(rng.choice([32, 64, 128, 256, 512])) * int(rng.integers(1, 4)) + int(rng.choice([-8, -1, 0, 0, 1, 4, 8]))
+        return max(1, min(d, hi))
+    if kind == 2:
+        return 8 * int(rng.integers(1, hi // 8 + 1))
+    return int(rng.integers(1, hi + 1))
+
+
+@pytest.mark.parametrize("name", list(DTYPES))
+def test_seeded_random_shapes(name):
+    """A seeded sweep over what the fixed cases above pick by hand: sizes around every tile edge, the four storage forms, the
+    three C modes, pitches that keep or miss the 16-byte rule, batches with gaps, odd base pointers and a broadcast B, with
+    and without the workspace form that the query offers.  Integers bit-exact, 16-bit floats within 2e-2 of max|C|,
+    Float32 / Float64 within 1e-5 K max|A| max|B|; Float32 without a split along k (no workspace, or NTG_GEMM_KEEP_K_ORDER)
+    and above the streaming kernel's 32 rows, or with the flag at any size, must be the reference's chain bit for bit."""
+    import os
+    rounds = int(os.environ.get("NTG_TEST_SWEEP_ROUNDS", "1"))     # (more of the same from further seeds, for a longer run by hand)
+    rng = np.random.default_rng(9100 + list(DTYPES).index(name))
+    modes = (_lib.C_ACCUMULATE, _lib.C_BIAS, _lib.C_OVERWRITE)
+    done = 0
+    while done < 40 * rounds:
+        m, k, n = _random_dim(rng, 700), _random_dim(rng, 1400), _random_dim(rng, 700)
+        batches = int(rng.choice([1, 1, 1, 2, 5]))
+        if m * k * n * batches > 1.2e8:
+            continue
+        ta, tb = bool(rng.integers(0, 2)), bool(rng.integers(0, 2))
+        pads = ALIGNED if rng.integers(0, 3) == 0 else ODD if rng.integers(0, 2) == 0 else (0, 0, 0)
+        gap = int(rng.choice([0, 0, 16, 7])) if batches > 1 else 0
+        base = int(rng.choice([0, 0, 0, 16, 3]))
+        bcast_b = batches > 1 and bool(rng.integers(0, 3) == 0)
+        keep = name == "f32" and bool(rng.integers(0, 2))
+        ws = "offered" if rng.integers(0, 2) else False
+        # (the chain is kept by the flag; without it only where neither a split along k nor the streaming kernel is in reach)
+        bits = name == "f32" and (keep or (ws is False and m > 32))
+        run_case(rng, name, m, k, n, ta, tb, pads, modes[int(rng.integers(0, 3))], batches=batches, gap=gap, base=base, bcast_b=bcast_b,
+                 workspace=ws, flags=_lib.GEMM_KEEP_K_ORDER if keep else 0, f32_bits=bits)
+        done += 1
