@@ -20,10 +20,10 @@ static int ring_f32_tile_edge(const GemmParams& p) {
 // against fmaf chains on the host), so the results are bit-identical to theirs and the choice between the kernels is free.
 // The chain of a block is k / 4 instructions of 32 cycles: four times shorter, on four times as many workgroups.
 // Operands go through LDS in stages of 128 k (four 16-byte loads of A and four of B per thread and stage, the loads of the
-// next two stages in flight behind the multiplies): a K-contiguous operand is stored [row][132 floats], an M/N-contiguous
+// next four stages in flight behind the multiplies): a K-contiguous operand is stored [row][132 floats], an M/N-contiguous
 // one [k][48 floats], both free of bank conflicts for the one-dword-per-lane reads of the MFMA operands.
 // Needs what the DMA-fed kernel needs (16-byte rows and pointers); C0 / bias start the chain, relu clamps in the epilogue.
-template <bool TA, bool TB>
+template <bool TA, bool TB, bool SHORTK>
 __global__ void __launch_bounds__(256) gemm_small16_f32_kernel(const GemmParams p) {
     constexpr int KB = 128, LDK = KB + 4, LDM = 48, NP = KB / 32;       // NP 16-byte pieces of each operand per thread and stage
     constexpr int A_STAGE = TA ? KB * LDM : 32 * LDK, B_STAGE = TB ? 32 * LDK : KB * LDM;
@@ -36,9 +36,13 @@ __global__ void __launch_bounds__(256) gemm_small16_f32_kernel(const GemmParams 
     const int tiles = p.tiles_m * p.tiles_n;
     const int b = (int)blockIdx.x / tiles, t = (int)blockIdx.x - b * tiles;
     const int m0 = (t / p.tiles_n) * 32, n0 = (t % p.tiles_n) * 32;
-    const float* A = p.Aptr ? static_cast<const float*>(p.Aptr[b]) : static_cast<const float*>(p.A) + operand_offset(p, b, p.sA, p.sAk);
-    const float* B = p.Bptr ? static_cast<const float*>(p.Bptr[b]) : static_cast<const float*>(p.B) + operand_offset(p, b, p.sB, p.sBk);
-    float* C = p.Cptr ? static_cast<float*>(p.Cptr[b]) : static_cast<float*>(p.C) + (int64_t)b * p.sC;
+    // (pointers into global memory, said so: loads through a generic pointer count as LDS operations as well, and every wait
+    //  for an operand read from LDS would then wait for the stages in flight too)
+    typedef __attribute__((address_space(1))) const float* gcfp;
+    typedef __attribute__((address_space(1))) float* gfp;
+    const gcfp A = (gcfp)(p.Aptr ? static_cast<const float*>(p.Aptr[b]) : static_cast<const float*>(p.A) + operand_offset(p, b, p.sA, p.sAk));
+    const gcfp B = (gcfp)(p.Bptr ? static_cast<const float*>(p.Bptr[b]) : static_cast<const float*>(p.B) + operand_offset(p, b, p.sB, p.sBk));
+    const gfp C = (gfp)(p.Cptr ? static_cast<float*>(p.Cptr[b]) : static_cast<float*>(p.C) + (int64_t)b * p.sC);
 
     // this lane's four results: row m, columns n .. n + 3 (the operands are handed to the MFMA the other way round, so that
     // a lane's four accumulator registers are consecutive columns of one row)
@@ -46,9 +50,9 @@ __global__ void __launch_bounds__(256) gemm_small16_f32_kernel(const GemmParams 
     const bool c_ok = m < p.M && n < p.N;                        // (N is a multiple of 4: the four columns exist together)
     f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
     if (c_ok) {
-        if (p.cmode == C_ACCUMULATE) acc = *reinterpret_cast<const f32x4*>(C + (int64_t)m * p.ldc + n);
+        if (p.cmode == C_ACCUMULATE) acc = *(__attribute__((address_space(1))) const f32x4*)(C + (int64_t)m * p.ldc + n);
         else if (p.cmode == C_BIAS) {
-            const float* bias = static_cast<const float*>(p.bias) + (int64_t)b * p.bias_bs + (int64_t)m * p.bias_rs + (int64_t)n * p.bias_cs;
+            const gcfp bias = (gcfp)(static_cast<const float*>(p.bias) + (int64_t)b * p.bias_bs + (int64_t)m * p.bias_rs + (int64_t)n * p.bias_cs);
 #pragma unroll
             for (int e = 0; e < 4; ++e) acc[e] = bias[(int64_t)e * p.bias_cs];
         }
@@ -56,18 +60,23 @@ __global__ void __launch_bounds__(256) gemm_small16_f32_kernel(const GemmParams 
 
     // Piece u of this thread: a K-contiguous operand has 32 pieces (128 k) per row, rows tid / 32 + 8 u; an M/N-contiguous one
     // 8 pieces (32 rows or columns of C) per k-row, k-rows tid / 8 + 32 u.  The sizes along the contiguous axis are multiples
-    // of 4, so a piece lies inside the matrix or outside as a whole; outside pieces are zeros (their rows / columns of C are
-    // not stored, their k are not multiplied).
-    const f32x4 zero4 = {0.0f, 0.0f, 0.0f, 0.0f};
+    // of 4, so a piece lies inside the matrix or outside as a whole.  A piece outside is fetched from the last piece inside
+    // instead (no branch, so the loads of several stages stay in flight and are waited for one stage at a time): rows of A
+    // and columns of B past the edge only reach elements of C that are not stored, and k past the end is never multiplied.
+    const int k_last = p.K - 4, m_last = TA ? p.M - 4 : p.M - 1, n_last = TB ? p.N - 1 : p.N - 4;
     auto load_a = [&](int k0, f32x4 (&v)[NP]) {
 #pragma unroll
         for (int u = 0; u < NP; ++u) {
             if constexpr (TA) {
-                const int k = k0 + (tid >> 3) + 32 * u, mm = m0 + (tid & 7) * 4;
-                v[u] = (k < p.K && mm < p.M) ? *reinterpret_cast<const f32x4*>(A + (int64_t)k * p.lda + mm) : zero4;
+                int k = k0 + (tid >> 3) + 32 * u, mm = m0 + (tid & 7) * 4;
+                k = k < p.K ? k : p.K - 1;
+                mm = mm < m_last ? mm : m_last;
+                v[u] = *(__attribute__((address_space(1))) const f32x4*)(A + (int64_t)k * p.lda + mm);
             } else {
-                const int mm = m0 + (tid >> 5) + 8 * u, k = k0 + (tid & 31) * 4;
-                v[u] = (mm < p.M && k < p.K) ? *reinterpret_cast<const f32x4*>(A + (int64_t)mm * p.lda + k) : zero4;
+                int mm = m0 + (tid >> 5) + 8 * u, k = k0 + (tid & 31) * 4;
+                mm = mm < m_last ? mm : m_last;
+                k = k < k_last ? k : k_last;
+                v[u] = *(__attribute__((address_space(1))) const f32x4*)(A + (int64_t)mm * p.lda + k);
             }
         }
     };
@@ -75,33 +84,54 @@ __global__ void __launch_bounds__(256) gemm_small16_f32_kernel(const GemmParams 
 #pragma unroll
         for (int u = 0; u < NP; ++u) {
             if constexpr (TB) {
-                const int nn = n0 + (tid >> 5) + 8 * u, k = k0 + (tid & 31) * 4;
-                v[u] = (nn < p.N && k < p.K) ? *reinterpret_cast<const f32x4*>(B + (int64_t)nn * p.ldb + k) : zero4;
+                int nn = n0 + (tid >> 5) + 8 * u, k = k0 + (tid & 31) * 4;
+                nn = nn < n_last ? nn : n_last;
+                k = k < k_last ? k : k_last;
+                v[u] = *(__attribute__((address_space(1))) const f32x4*)(B + (int64_t)nn * p.ldb + k);
             } else {
-                const int k = k0 + (tid >> 3) + 32 * u, nn = n0 + (tid & 7) * 4;
-                v[u] = (k < p.K && nn < p.N) ? *reinterpret_cast<const f32x4*>(B + (int64_t)k * p.ldb + nn) : zero4;
+                int k = k0 + (tid >> 3) + 32 * u, nn = n0 + (tid & 7) * 4;
+                k = k < p.K ? k : p.K - 1;
+                nn = nn < n_last ? nn : n_last;
+                v[u] = *(__attribute__((address_space(1))) const f32x4*)(B + (int64_t)k * p.ldb + nn);
             }
         }
     };
-    auto store = [&](int buf, const f32x4 (&va)[NP], const f32x4 (&vb)[NP]) {
-#pragma unroll
-        for (int u = 0; u < NP; ++u) {
-            if constexpr (TA) *reinterpret_cast<f32x4*>(&sA[buf][((tid >> 3) + 32 * u) * LDM + (tid & 7) * 4]) = va[u];
-            else *reinterpret_cast<f32x4*>(&sA[buf][((tid >> 5) + 8 * u) * LDK + (tid & 31) * 4]) = va[u];
-            if constexpr (TB) *reinterpret_cast<f32x4*>(&sB[buf][((tid >> 5) + 8 * u) * LDK + (tid & 31) * 4]) = vb[u];
-            else *reinterpret_cast<f32x4*>(&sB[buf][((tid >> 3) + 32 * u) * LDM + (tid & 7) * 4]) = vb[u];
-        }
+    // piece u of both operands of one stage, from registers to LDS buffer `buf`
+    auto store_piece = [&](int buf, int u, const f32x4 (&va)[NP], const f32x4 (&vb)[NP]) __attribute__((always_inline)) {
+        if constexpr (TA) *reinterpret_cast<f32x4*>(&sA[buf][((tid >> 3) + 32 * u) * LDM + (tid & 7) * 4]) = va[u];
+        else *reinterpret_cast<f32x4*>(&sA[buf][((tid >> 5) + 8 * u) * LDK + (tid & 31) * 4]) = va[u];
+        if constexpr (TB) *reinterpret_cast<f32x4*>(&sB[buf][((tid >> 5) + 8 * u) * LDK + (tid & 31) * 4]) = vb[u];
+        else *reinterpret_cast<f32x4*>(&sB[buf][((tid >> 3) + 32 * u) * LDM + (tid & 7) * 4]) = vb[u];
     };
-    // two stages of loads in flight: stage kt + 2 is requested before stage kt is multiplied
+    // DEPTH stages of loads in flight (stage kt + DEPTH is requested before stage kt is multiplied): every workgroup walks
+    // through k in step with all the others, so each stage is the first touch of its cache lines and comes at the latency of
+    // memory, not of the L2 cache -- with four stages of 128 k a product of k <= 512 asks for everything at once.
+    // Control flow is laid out so that the number of loads in flight is the same on every path to each wait (the compiler
+    // counts them; where paths with different counts meet it waits for everything): no branch inside a stage, a main loop
+    // of whole rounds of DEPTH stages that always request (past the end: the last pieces again), and the last one to DEPTH
+    // stages as straight-line code without requests.
+    constexpr int DEPTH = 4;
+    static_assert(KB / 32 == NP, "one piece of each operand goes to LDS per group of eight instructions");
     const int KT = (p.K + KB - 1) / KB;
-    f32x4 va[2][NP], vb[2][NP];
+    f32x4 va[DEPTH][NP], vb[DEPTH][NP];
     load_a(0, va[0]); load_b(0, vb[0]);
-    if (KT > 1) { load_a(KB, va[1]); load_b(KB, vb[1]); }
-    store(0, va[0], vb[0]);
+#pragma unroll
+    for (int sg = 1; sg < DEPTH; ++sg) {
+        // SHORTK (fewer than DEPTH stages): a short k asks for nothing it does not use, at the price of inexact waits
+        if (!SHORTK || sg < KT) { load_a(sg * KB, va[sg]); load_b(sg * KB, vb[sg]); }
+    }
+#pragma unroll
+    for (int u = 0; u < NP; ++u) store_piece(0, u, va[0], vb[0]);
     __syncthreads();
-    for (int kt = 0; kt < KT; ++kt) {
-        const int buf = kt & 1;
-        if (kt + 2 < KT) { load_a((kt + 2) * KB, va[buf]); load_b((kt + 2) * KB, vb[buf]); }     // (stage kt's registers are in LDS already)
+    // Stage kt (in LDS buffer SLOT % 2, its registers free again): request stage kt + DEPTH (REQUEST), multiply, and hand
+    // stage kt + 1 (which arrived long ago) to the other LDS buffer a piece at a time between the groups of instructions, so
+    // that only the barrier and the first operand reads of the next stage are left outside the chain's shadow.
+    auto stage = [&](int kt, auto slot_tag, auto request_tag) __attribute__((always_inline)) {
+        constexpr int SLOT = decltype(slot_tag)::value, NEXT = (SLOT + 1) % DEPTH, buf = SLOT & 1;
+        if constexpr (decltype(request_tag)::value) {
+            load_a((kt + DEPTH) * KB, va[SLOT]);
+            load_b((kt + DEPTH) * KB, vb[SLOT]);
+        }
         const float* a_s = sA[buf];
         const float* b_s = sB[buf];
         const int steps = p.K - kt * KB < KB ? (p.K - kt * KB) / 4 : KB / 4;      // (K is a multiple of 4: whole instructions)
@@ -121,8 +151,13 @@ __global__ void __launch_bounds__(256) gemm_small16_f32_kernel(const GemmParams 
 #pragma unroll
             for (int g = 0; g < KB / 32; ++g) {
                 if (g + 1 < KB / 32) read_group(8 * (g + 1), av[(g + 1) & 1], bv[(g + 1) & 1]);
+                store_piece(buf ^ 1, g, va[NEXT], vb[NEXT]);
+                // (nothing moves across: left alone, the scheduler sinks every read to just before its instruction, and the
+                //  chain then waits for LDS once per pair of instructions)
+                __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int u = 0; u < 8; ++u) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(bv[g & 1][u], av[g & 1][u], acc, 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
             }
         } else {
             for (int q = 0; q < steps; ++q) {                                     // (the last stage of a k that is not a multiple of 128)
@@ -131,16 +166,34 @@ __global__ void __launch_bounds__(256) gemm_small16_f32_kernel(const GemmParams 
                 const float bv = TB ? b_s[(bj * 16 + li) * LDK + k] : b_s[k * LDM + bj * 16 + li];
                 acc = __builtin_amdgcn_mfma_f32_16x16x4f32(bv, av, acc, 0, 0, 0);
             }
+#pragma unroll
+            for (int u = 0; u < NP; ++u) store_piece(buf ^ 1, u, va[NEXT], vb[NEXT]);
         }
-        if (kt + 1 < KT) store(buf ^ 1, va[buf ^ 1], vb[buf ^ 1]);
         __syncthreads();
+    };
+    using S0 = std::integral_constant<int, 0>; using S1 = std::integral_constant<int, 1>;
+    using S2 = std::integral_constant<int, 2>; using S3 = std::integral_constant<int, 3>;
+    int kt = 0;
+    for (; kt + DEPTH < KT; kt += DEPTH) {
+        stage(kt, S0{}, std::true_type{});
+        stage(kt + 1, S1{}, std::true_type{});
+        stage(kt + 2, S2{}, std::true_type{});
+        stage(kt + 3, S3{}, std::true_type{});
+    }
+    stage(kt, S0{}, std::false_type{});                  // (K >= 64: at least one stage)
+    if (kt + 1 < KT) {
+        stage(kt + 1, S1{}, std::false_type{});
+        if (kt + 2 < KT) {
+            stage(kt + 2, S2{}, std::false_type{});
+            if (kt + 3 < KT) stage(kt + 3, S3{}, std::false_type{});
+        }
     }
     if (c_ok) {
         if (p.act == ACT_RELU) {
 #pragma unroll
             for (int e = 0; e < 4; ++e) acc[e] = acc[e] > 0.0f ? acc[e] : 0.0f;
         }
-        *reinterpret_cast<f32x4*>(C + (int64_t)m * p.ldc + n) = acc;
+        *(__attribute__((address_space(1))) f32x4*)(C + (int64_t)m * p.ldc + n) = acc;
     }
 }
 
@@ -157,8 +210,13 @@ static hipError_t launch_small16_f32(bool ta, bool tb, const GemmParams& pin, hi
     const int64_t blocks = (int64_t)p.tiles_m * p.tiles_n * p.batch;
     if (blocks <= 0) return hipSuccess;
     const dim3 g((unsigned)blocks), t(256);
-    if (ta) { if (tb) hipLaunchKernelGGL((gemm_small16_f32_kernel<true, true>), g, t, 0, s, p); else hipLaunchKernelGGL((gemm_small16_f32_kernel<true, false>), g, t, 0, s, p); }
-    else { if (tb) hipLaunchKernelGGL((gemm_small16_f32_kernel<false, true>), g, t, 0, s, p); else hipLaunchKernelGGL((gemm_small16_f32_kernel<false, false>), g, t, 0, s, p); }
+    const bool short_k = p.K <= 3 * 128;                 // fewer stages than the kernel keeps in flight
+#define NTG_SMALL16(TA_, TB_) \
+    do { if (short_k) hipLaunchKernelGGL((gemm_small16_f32_kernel<TA_, TB_, true>), g, t, 0, s, p); \
+         else hipLaunchKernelGGL((gemm_small16_f32_kernel<TA_, TB_, false>), g, t, 0, s, p); } while (0)
+    if (ta) { if (tb) NTG_SMALL16(true, true); else NTG_SMALL16(true, false); }
+    else { if (tb) NTG_SMALL16(false, true); else NTG_SMALL16(false, false); }
+#undef NTG_SMALL16
     return hipGetLastError();
 }
 

@@ -28,9 +28,10 @@ __global__ void __launch_bounds__(512) gemm_skinny_f32_kernel(const GemmParams p
     const int b = blockIdx.y;
     const int n0 = blockIdx.x * SW;
 
-    const float* A = p.Aptr ? static_cast<const float*>(p.Aptr[b]) : static_cast<const float*>(p.A) + (int64_t)b * p.sA;
-    const float* B = p.Bptr ? static_cast<const float*>(p.Bptr[b]) : static_cast<const float*>(p.B) + (int64_t)b * p.sB;
-    float* C = p.Cptr ? static_cast<float*>(p.Cptr[b]) : static_cast<float*>(p.C) + (int64_t)b * p.sC;
+    // (global pointers: the waits of the register ring below are per k-step only if the loads are not FLAT instructions)
+    const NTG_GLOBAL float* A = (const NTG_GLOBAL float*)(p.Aptr ? static_cast<const float*>(p.Aptr[b]) : static_cast<const float*>(p.A) + (int64_t)b * p.sA);
+    const NTG_GLOBAL float* B = (const NTG_GLOBAL float*)(p.Bptr ? static_cast<const float*>(p.Bptr[b]) : static_cast<const float*>(p.B) + (int64_t)b * p.sB);
+    NTG_GLOBAL float* C = (NTG_GLOBAL float*)(p.Cptr ? static_cast<float*>(p.Cptr[b]) : static_cast<float*>(p.C) + (int64_t)b * p.sC);
 
     floatx4 acc[MB][CPL];
 #pragma unroll
@@ -51,7 +52,7 @@ __global__ void __launch_bounds__(512) gemm_skinny_f32_kernel(const GemmParams p
         for (int i = 0; i < MB; ++i) {
             const int row = i * 16 + c;
             if constexpr (FAST && !TA) {
-                const floatx4 t = (row < p.M) ? *reinterpret_cast<const floatx4*>(A + (int64_t)row * p.lda + kl) : floatx4{0.f, 0.f, 0.f, 0.f};
+                const floatx4 t = (row < p.M) ? *(const NTG_GLOBAL floatx4*)(A + (int64_t)row * p.lda + kl) : floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int e = 0; e < 4; ++e) a[d][i][e] = t[e];
             } else {
@@ -70,7 +71,7 @@ __global__ void __launch_bounds__(512) gemm_skinny_f32_kernel(const GemmParams p
             for (int e = 0; e < 4; ++e) {
                 const int k = kl + e;
                 if constexpr (FAST) {
-                    const fv t = *reinterpret_cast<const fv*>(B + (int64_t)k * p.ldb + n0 + CPL * c);
+                    const fv t = *(const NTG_GLOBAL fv*)(B + (int64_t)k * p.ldb + n0 + CPL * c);
 #pragma unroll
                     for (int j = 0; j < CPL; ++j) bv[d][e][j] = t[j];
                 } else {
@@ -86,7 +87,7 @@ __global__ void __launch_bounds__(512) gemm_skinny_f32_kernel(const GemmParams p
             for (int j = 0; j < CPL; ++j) {
                 const int n = n0 + CPL * c + j;
                 if constexpr (FAST) {
-                    const floatx4 t = *reinterpret_cast<const floatx4*>(B + (int64_t)n * p.ldb + kl);
+                    const floatx4 t = *(const NTG_GLOBAL floatx4*)(B + (int64_t)n * p.ldb + kl);
 #pragma unroll
                     for (int e = 0; e < 4; ++e) bv[d][e][j] = t[e];
                 } else {
@@ -100,22 +101,41 @@ __global__ void __launch_bounds__(512) gemm_skinny_f32_kernel(const GemmParams p
         }
     };
 
+    auto compute = [&](int d) __attribute__((always_inline)) {
 #pragma unroll
-    for (int d = 0; d < D; ++d)
-        if (wave + d * NW < steps) load_step(d, wave + d * NW);
-
-    for (int base = wave; base < steps; base += D * NW) {
+        for (int e = 0; e < 4; ++e)
+#pragma unroll
+            for (int i = 0; i < MB; ++i)
+#pragma unroll
+                for (int j = 0; j < CPL; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[d][i][e], bv[d][e][j], acc[i][j], 0, 0, 0);
+    };
+    // Rounds of D k-steps.  While a whole further round exists, a round runs without a branch (multiply step d, request the
+    // step that takes its registers): the number of loads in flight is then the same at every wait, and the compiler waits
+    // for one step's loads and leaves the other D - 1 steps in flight.  (Where paths with different counts meet it waits
+    // for everything; the guarded rounds at the end, and the whole loop for a short k, are of that kind.)
+    int base = wave;
+    if (wave + (2 * D - 1) * NW < steps) {               // (uniform per wavefront)
+#pragma unroll
+        for (int d = 0; d < D; ++d) load_step(d, wave + d * NW);
+        for (; base + (2 * D - 1) * NW < steps; base += D * NW) {
+#pragma unroll
+            for (int d = 0; d < D; ++d) {
+                compute(d);
+                load_step(d, base + (d + D) * NW);
+            }
+        }
+    } else {
+#pragma unroll
+        for (int d = 0; d < D; ++d)
+            if (wave + d * NW < steps) load_step(d, wave + d * NW);
+    }
+    for (; base < steps; base += D * NW) {
 #pragma unroll
         for (int d = 0; d < D; ++d) {
             const int s = base + d * NW;
             if (s < steps) {
-#pragma unroll
-                for (int e = 0; e < 4; ++e)
-#pragma unroll
-                    for (int i = 0; i < MB; ++i)
-#pragma unroll
-                        for (int j = 0; j < CPL; ++j)
-                            acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[d][i][e], bv[d][e][j], acc[i][j], 0, 0, 0);
+                compute(d);
                 if (s + D * NW < steps) load_step(d, s + D * NW);
             }
         }
@@ -130,7 +150,7 @@ __global__ void __launch_bounds__(512) gemm_skinny_f32_kernel(const GemmParams p
     __syncthreads();
 
     constexpr int TOTAL = MB * CPL * 4 * 64;
-    const float* bias = static_cast<const float*>(p.bias);
+    const NTG_GLOBAL float* bias = (const NTG_GLOBAL float*)static_cast<const float*>(p.bias);
     for (int idx = tid; idx < TOTAL; idx += 512) {
         const int l = idx & 63, q = idx >> 6;
         float sum = 0.f;
@@ -140,7 +160,7 @@ __global__ void __launch_bounds__(512) gemm_skinny_f32_kernel(const GemmParams p
         const int m = i * 16 + 4 * (l >> 4) + r;
         const int n = n0 + CPL * (l & 15) + j;
         if (m < p.M && n < p.N) {
-            float* cp = C + (int64_t)m * p.ldc + n;
+            NTG_GLOBAL float* cp = C + (int64_t)m * p.ldc + n;
             if (p.cmode == C_ACCUMULATE) sum += *cp;
             else if (p.cmode == C_BIAS) sum += bias[(int64_t)b * p.bias_bs + (int64_t)m * p.bias_rs + (int64_t)n * p.bias_cs];
             *cp = sum;
@@ -209,9 +229,9 @@ __global__ void __launch_bounds__(512) gemm_skinny16_kernel(const GemmParams p) 
     const int b = blockIdx.y;
     const int n0 = blockIdx.x * SW;
 
-    const T* A = p.Aptr ? static_cast<const T*>(p.Aptr[b]) : static_cast<const T*>(p.A) + (int64_t)b * p.sA;
-    const T* B = p.Bptr ? static_cast<const T*>(p.Bptr[b]) : static_cast<const T*>(p.B) + (int64_t)b * p.sB;
-    T* C = p.Cptr ? static_cast<T*>(p.Cptr[b]) : static_cast<T*>(p.C) + (int64_t)b * p.sC;
+    const NTG_GLOBAL T* A = (const NTG_GLOBAL T*)(p.Aptr ? static_cast<const T*>(p.Aptr[b]) : static_cast<const T*>(p.A) + (int64_t)b * p.sA);
+    const NTG_GLOBAL T* B = (const NTG_GLOBAL T*)(p.Bptr ? static_cast<const T*>(p.Bptr[b]) : static_cast<const T*>(p.B) + (int64_t)b * p.sB);
+    NTG_GLOBAL T* C = (NTG_GLOBAL T*)(p.Cptr ? static_cast<T*>(p.Cptr[b]) : static_cast<T*>(p.C) + (int64_t)b * p.sC);
 
     floatx4 acc[MB][CPL];
 #pragma unroll
@@ -239,7 +259,7 @@ __global__ void __launch_bounds__(512) gemm_skinny16_kernel(const GemmParams p) 
         for (int i = 0; i < MB; ++i) {
             const int row = i * 16 + c;
             if constexpr (FAST && !TA) {
-                a[d][i] = (row < p.M) ? *reinterpret_cast<const su32x4*>(A + (int64_t)row * p.lda + kl) : su32x4{0u, 0u, 0u, 0u};
+                a[d][i] = (row < p.M) ? *(const NTG_GLOBAL su32x4*)(A + (int64_t)row * p.lda + kl) : su32x4{0u, 0u, 0u, 0u};
             } else {
                 a[d][i] = gather8([&](int e) -> T {
                     const int k = kl + e;
@@ -254,7 +274,7 @@ __global__ void __launch_bounds__(512) gemm_skinny16_kernel(const GemmParams p) 
                 const int n = n0 + c + 16 * j;
                 su32x4 t;
                 if constexpr (FAST) {
-                    t = *reinterpret_cast<const su32x4*>(B + (int64_t)n * p.ldb + kl);
+                    t = *(const NTG_GLOBAL su32x4*)(B + (int64_t)n * p.ldb + kl);
                 } else {
                     t = gather8([&](int e) -> T { return (n < p.N && kl + e < p.K) ? B[(int64_t)n * p.ldb + kl + e] : (T)0.0f; });
                 }
@@ -268,16 +288,16 @@ __global__ void __launch_bounds__(512) gemm_skinny16_kernel(const GemmParams p) 
                 const int n = n0 + CPL * c;
                 if constexpr (FAST) {
                     if constexpr (CPL == 8) {
-                        const su32x4 t = *reinterpret_cast<const su32x4*>(B + (int64_t)k * p.ldb + n);
+                        const su32x4 t = *(const NTG_GLOBAL su32x4*)(B + (int64_t)k * p.ldb + n);
 #pragma unroll
                         for (int w = 0; w < 4; ++w) bv[d][e][w] = t[w];
                     } else if constexpr (CPL == 4) {
                         typedef uint32_t u2 __attribute__((ext_vector_type(2)));
-                        const u2 t = *reinterpret_cast<const u2*>(B + (int64_t)k * p.ldb + n);
+                        const u2 t = *(const NTG_GLOBAL u2*)(B + (int64_t)k * p.ldb + n);
                         bv[d][e][0] = t[0];
                         bv[d][e][1] = t[1];
                     } else {
-                        bv[d][e][0] = *reinterpret_cast<const uint32_t*>(B + (int64_t)k * p.ldb + n);
+                        bv[d][e][0] = *(const NTG_GLOBAL uint32_t*)(B + (int64_t)k * p.ldb + n);
                     }
                 } else {
                     T tmp[2 * BW];
@@ -309,11 +329,24 @@ __global__ void __launch_bounds__(512) gemm_skinny16_kernel(const GemmParams p) 
         }
     };
 
+    // (rounds without a branch while a whole further round exists: see the Float32 kernel above)
+    int base = wave;
+    if (wave + (2 * D - 1) * NW < steps) {               // (uniform per wavefront)
 #pragma unroll
-    for (int d = 0; d < D; ++d)
-        if (wave + d * NW < steps) load_step(d, wave + d * NW);
-
-    for (int base = wave; base < steps; base += D * NW) {
+        for (int d = 0; d < D; ++d) load_step(d, wave + d * NW);
+        for (; base + (2 * D - 1) * NW < steps; base += D * NW) {
+#pragma unroll
+            for (int d = 0; d < D; ++d) {
+                compute(d);
+                load_step(d, base + (d + D) * NW);
+            }
+        }
+    } else {
+#pragma unroll
+        for (int d = 0; d < D; ++d)
+            if (wave + d * NW < steps) load_step(d, wave + d * NW);
+    }
+    for (; base < steps; base += D * NW) {
 #pragma unroll
         for (int d = 0; d < D; ++d) {
             const int s = base + d * NW;
@@ -333,7 +366,7 @@ __global__ void __launch_bounds__(512) gemm_skinny16_kernel(const GemmParams p) 
     __syncthreads();
 
     constexpr int TOTAL = MB * CPL * 4 * 64;
-    const T* bias = static_cast<const T*>(p.bias);
+    const NTG_GLOBAL T* bias = (const NTG_GLOBAL T*)static_cast<const T*>(p.bias);
     for (int idx = tid; idx < TOTAL; idx += 512) {
         const int l = idx & 63, q = idx >> 6;
         float sum = 0.f;
@@ -343,7 +376,7 @@ __global__ void __launch_bounds__(512) gemm_skinny16_kernel(const GemmParams p) 
         const int m = i * 16 + 4 * (l >> 4) + r;
         const int n = n0 + (TB ? (l & 15) + 16 * j : CPL * (l & 15) + j);
         if (m < p.M && n < p.N) {
-            T* cp = C + (int64_t)m * p.ldc + n;
+            NTG_GLOBAL T* cp = C + (int64_t)m * p.ldc + n;
             if (p.cmode == C_ACCUMULATE) sum += (float)*cp;
             else if (p.cmode == C_BIAS) sum += (float)bias[(int64_t)b * p.bias_bs + (int64_t)m * p.bias_rs + (int64_t)n * p.bias_cs];
             *cp = (T)sum;

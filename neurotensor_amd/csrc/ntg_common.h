@@ -3,6 +3,12 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+// A pointer known to point into global memory.  The pointers of GemmParams are generic; a load through a generic pointer is a
+// FLAT instruction, which counts as an LDS operation as well and may return out of order with the global ones, so the
+// compiler can only wait for ALL outstanding loads at once: kernels that keep several steps of loads in flight cast their
+// operand pointers with this first.
+#define NTG_GLOBAL __attribute__((address_space(1)))
+
 namespace ntg {
 
 // numeric values follow nt::DType (nt/dtype/DType_enum.h:14-20); BF16/U64 are extensions
