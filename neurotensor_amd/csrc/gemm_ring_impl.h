@@ -272,9 +272,9 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
     if constexpr (ES == 4 && std::is_same<AccS, float>::value) {
         if (p.cmode == C_ACCUMULATE || p.cmode == C_BIAS) {            // (uniform)
             const bool from_c = p.cmode == C_ACCUMULATE;
-            const float* bias = static_cast<const float*>(p.bias);
+            const NTG_GLOBAL float* bias = (const NTG_GLOBAL float*)static_cast<const float*>(p.bias);
             const bool vec_ok = from_c ? (p.ldc % 4 == 0 && (reinterpret_cast<uintptr_t>(C) & 15) == 0)
-                                       : (p.bias_cs == 1 && p.bias_rs % 4 == 0 && p.bias_bs % 4 == 0 && (reinterpret_cast<uintptr_t>(bias) & 15) == 0);
+                                       : (p.bias_cs == 1 && p.bias_rs % 4 == 0 && p.bias_bs % 4 == 0 && (reinterpret_cast<uintptr_t>(p.bias) & 15) == 0);
             const int64_t cstep = from_c ? 1 : p.bias_cs;
             typedef float f32x4 __attribute__((ext_vector_type(4)));
 #pragma unroll
@@ -287,9 +287,9 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
                         const int nn = n0 + wn * WTN + 32 * j + 8 * rq + 4 * (lane >> 5);
                         f32x4 v = {0.0f, 0.0f, 0.0f, 0.0f};
                         if (m < p.M && nn < p.N) {
-                            const float* src = from_c ? reinterpret_cast<const float*>(C) + (int64_t)m * p.ldc + nn
+                            const NTG_GLOBAL float* src = from_c ? (const NTG_GLOBAL float*)reinterpret_cast<const float*>(C) + (int64_t)m * p.ldc + nn
                                                       : bias + (int64_t)b * p.bias_bs + (int64_t)m * p.bias_rs + (int64_t)nn * p.bias_cs;
-                            if (vec_ok && nn + 4 <= p.N) v = *reinterpret_cast<const f32x4*>(src);
+                            if (vec_ok && nn + 4 <= p.N) v = *(const NTG_GLOBAL f32x4*)src;
                             else {
 #pragma unroll
                                 for (int e = 0; e < 4; ++e)
@@ -978,7 +978,9 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
     char* slab = RING3 ? (wave == 3 ? st1 : st0 + wave * (32 * SROW))
                : WBN > WBM ? (wave == 0 ? st0 : wave == 1 ? st1 : wave == 2 ? st2 : st3)
                            : ((wave & 2) ? st1 : st0) + (wave & 1) * (32 * SROW);
-    char* Cb = reinterpret_cast<char*>(C);
+    // (C and the bias through pointers into global memory: as FLAT instructions their loads and stores would count as LDS
+    //  operations too, and every wait for a slab read would wait for the stores of the slab before it)
+    NTG_GLOBAL char* Cb = (NTG_GLOBAL char*)reinterpret_cast<char*>(C);
     const int col = 8 * (lane % LPR);              // this lane's 8 consecutive columns in the slab
     const int n = n0 + wn * WTN + col;
     constexpr int NV = ES == 4 ? 2 : 1;            // 16-byte vectors of C per lane and row: 8 columns of 1 (half a vector), 2 or 4 bytes
@@ -991,19 +993,19 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
                               (reinterpret_cast<uintptr_t>(p.bias) & 15) == 0;
     auto epilogue = [&](auto cmode_tag) {
         constexpr int CM = decltype(cmode_tag)::value;
-        const T* bias = static_cast<const T*>(p.bias);
+        const NTG_GLOBAL T* bias = (const NTG_GLOBAL T*)static_cast<const T*>(p.bias);
         // one bias row for every row of C (cpu::linear's [n] vector): the lane's 8 columns never change, one load for the whole tile
         AccS bias_row[8] = {};
         const bool bias_row_const = CM == C_BIAS && bias_rows_16 && p.bias_rs == 0 && (!RAGGED || n + 8 <= p.N);
         if constexpr (CM == C_BIAS && ES != 1) {
             if (bias_row_const) {
-                const T* bp = bias + (int64_t)b * p.bias_bs + (int64_t)n;
+                const NTG_GLOBAL T* bp = bias + (int64_t)b * p.bias_bs + (int64_t)n;
                 if constexpr (ES == 2) {
-                    const u32x4 bv = *reinterpret_cast<const u32x4*>(bp);
+                    const u32x4 bv = *(const NTG_GLOBAL u32x4*)bp;
 #pragma unroll
                     for (int e = 0; e < 8; ++e) bias_row[e] = Cvt16<DT>::up((uint16_t)(bv[e >> 1] >> (16 * (e & 1))));
                 } else {
-                    const accx4 b0 = *reinterpret_cast<const accx4*>(bp), b1 = *reinterpret_cast<const accx4*>(bp + 4);
+                    const accx4 b0 = *(const NTG_GLOBAL accx4*)bp, b1 = *(const NTG_GLOBAL accx4*)(bp + 4);
 #pragma unroll
                     for (int e = 0; e < 4; ++e) { bias_row[e] = b0[e]; bias_row[4 + e] = b1[e]; }
                 }
@@ -1022,10 +1024,10 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
                     for (int v = 0; v < NV; ++v) {
                         if (!RAGGED || (m < p.M && n + 4 * v < p.N)) {
                             if constexpr (ES == 1) {
-                                const u32x2v c8 = *reinterpret_cast<const u32x2v*>(Cb + (int64_t)m * p.ldc + n);
+                                const u32x2v c8 = *(const NTG_GLOBAL u32x2v*)(Cb + (int64_t)m * p.ldc + n);
                                 c0[t][v] = u32x4{c8[0], c8[1], 0u, 0u};
                             } else {
-                                c0[t][v] = *reinterpret_cast<const u32x4*>(Cb + ((int64_t)m * p.ldc + n) * ES + 16 * v);
+                                c0[t][v] = *(const NTG_GLOBAL u32x4*)(Cb + ((int64_t)m * p.ldc + n) * ES + 16 * v);
                             }
                         } else c0[t][v] = u32x4{0u, 0u, 0u, 0u};
                     }
@@ -1060,7 +1062,7 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
                 if constexpr (GATHER16) {
                     // output planes whose rows are not 16-byte multiples (Ho*Wo = 49, 900, ...): element-wise stores
                     if (!c_rows_16) {
-                        T* ce = reinterpret_cast<T*>(Cb) + (int64_t)m * p.ldc + n;
+                        NTG_GLOBAL T* ce = (NTG_GLOBAL T*)Cb + (int64_t)m * p.ldc + n;
 #pragma unroll
                         for (int e = 0; e < 8; ++e) {
                             if (n + e >= p.N) break;
@@ -1076,9 +1078,9 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
                 if constexpr (CM == C_PARTIAL) {
                     // split-K: the fp32 sums of this k range go to a float matrix; rounding happens after the reduction
                     // (8-bit operands: the 32-bit integer sums, for the byte-plane form of the wider integer products)
-                    float* wp = static_cast<float*>(p.C) + (int64_t)b * p.sC + (int64_t)m * p.ldc + n;
-                    *reinterpret_cast<accx4*>(wp) = lo;
-                    if (hi_ok) *reinterpret_cast<accx4*>(wp + 4) = hi;
+                    NTG_GLOBAL float* wp = (NTG_GLOBAL float*)static_cast<float*>(p.C) + (int64_t)b * p.sC + (int64_t)m * p.ldc + n;
+                    *(NTG_GLOBAL accx4*)wp = lo;
+                    if (hi_ok) *(NTG_GLOBAL accx4*)(wp + 4) = hi;
                     continue;
                 }
                 if constexpr (CM == C_ACCUMULATE) {
@@ -1089,18 +1091,18 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
                         else { const uint32_t cu = c0[t][e >> 2][e & 3]; v[e] += __builtin_bit_cast(float, cu); }
                     }
                 } else if constexpr (CM == C_BIAS) {
-                    const T* bp = bias + (int64_t)b * p.bias_bs + (int64_t)m * p.bias_rs + (int64_t)n * p.bias_cs;
+                    const NTG_GLOBAL T* bp = bias + (int64_t)b * p.bias_bs + (int64_t)m * p.bias_rs + (int64_t)n * p.bias_cs;
                     if (bias_row_const) {
 #pragma unroll
                         for (int e = 0; e < 8; ++e) v[e] += bias_row[e];
                     } else if (bias_rows_16 && (ES != 4 || hi_ok)) {
                         // a bias that runs along the columns (cpu::linear's [n] vector): the lane's 8 values in 16-byte loads
                         if constexpr (ES == 2) {
-                            const u32x4 bv = *reinterpret_cast<const u32x4*>(bp);
+                            const u32x4 bv = *(const NTG_GLOBAL u32x4*)bp;
 #pragma unroll
                             for (int e = 0; e < 8; ++e) v[e] += Cvt16<DT>::up((uint16_t)(bv[e >> 1] >> (16 * (e & 1))));
                         } else if constexpr (ES == 4) {
-                            const accx4 b0 = *reinterpret_cast<const accx4*>(bp), b1 = *reinterpret_cast<const accx4*>(bp + 4);
+                            const accx4 b0 = *(const NTG_GLOBAL accx4*)bp, b1 = *(const NTG_GLOBAL accx4*)(bp + 4);
 #pragma unroll
                             for (int e = 0; e < 4; ++e) { v[e] += b0[e]; v[4 + e] += b1[e]; }
                         }
@@ -1116,23 +1118,23 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
                         for (int e = 0; e < 8; ++e) v[e] = v[e] > (AccS)0 ? v[e] : (AccS)0;
                     }
                 }
-                char* cp = Cb + ((int64_t)m * p.ldc + n) * ES;
+                NTG_GLOBAL char* cp = Cb + ((int64_t)m * p.ldc + n) * ES;
                 if constexpr (ES == 2) {
                     u32x4 o;
 #pragma unroll
                     for (int e = 0; e < 4; ++e)
                         o[e] = (uint32_t)Cvt16<DT>::down(v[2 * e]) | ((uint32_t)Cvt16<DT>::down(v[2 * e + 1]) << 16);
-                    *reinterpret_cast<u32x4*>(cp) = o;
+                    *(NTG_GLOBAL u32x4*)cp = o;
                 } else if constexpr (ES == 1) {
                     u32x2v o;                       // the low 8 bits of each sum: wrapping arithmetic in the element type
 #pragma unroll
                     for (int h = 0; h < 2; ++h)
                         o[h] = ((uint32_t)v[4 * h] & 0xffu) | (((uint32_t)v[4 * h + 1] & 0xffu) << 8) |
                                (((uint32_t)v[4 * h + 2] & 0xffu) << 16) | ((uint32_t)v[4 * h + 3] << 24);
-                    *reinterpret_cast<u32x2v*>(cp) = o;
+                    *(NTG_GLOBAL u32x2v*)cp = o;
                 } else {
-                    *reinterpret_cast<accx4*>(cp) = accx4{v[0], v[1], v[2], v[3]};
-                    if (hi_ok) *reinterpret_cast<accx4*>(cp + 16) = accx4{v[4], v[5], v[6], v[7]};
+                    *(NTG_GLOBAL accx4*)cp = accx4{v[0], v[1], v[2], v[3]};
+                    if (hi_ok) *(NTG_GLOBAL accx4*)(cp + 16) = accx4{v[4], v[5], v[6], v[7]};
                 }
             }
         }
