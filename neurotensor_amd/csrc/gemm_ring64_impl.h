@@ -51,7 +51,7 @@ __global__ void __launch_bounds__(256) gemm_ring64_kernel(const GemmParams p) {
 
     const double* A = p.Aptr ? static_cast<const double*>(p.Aptr[b]) : static_cast<const double*>(p.A) + operand_offset(p, b, p.sA, p.sAk);
     const double* B = p.Bptr ? static_cast<const double*>(p.Bptr[b]) : static_cast<const double*>(p.B) + operand_offset(p, b, p.sB, p.sBk);
-    double* C = p.Cptr ? static_cast<double*>(p.Cptr[b]) : static_cast<double*>(p.C) + (int64_t)b * p.sC;
+    NTG_GLOBAL double* C = (NTG_GLOBAL double*)(p.Cptr ? static_cast<double*>(p.Cptr[b]) : static_cast<double*>(p.C) + (int64_t)b * p.sC);   // (global memory: no FLAT instructions)
 
     const int wave_u = __builtin_amdgcn_readfirstlane(wave);
     const int KT = (p.K + BK - 1) / BK;
@@ -173,7 +173,7 @@ __global__ void __launch_bounds__(256) gemm_ring64_kernel(const GemmParams p) {
     NTG_WAIT_VMCNT(0);                        // the clamped tail DMAs have landed before the workgroup's LDS is released
 
     // ---- epilogue: straight from the accumulators; the 16 lanes of a group cover 128 consecutive bytes of a row ----
-    const double* bias = static_cast<const double*>(p.bias);
+    const NTG_GLOBAL double* bias = (const NTG_GLOBAL double*)static_cast<const double*>(p.bias);
     const int cmode = p.cmode;
 #pragma unroll
     for (int i = 0; i < NBL; ++i)
@@ -184,7 +184,7 @@ __global__ void __launch_bounds__(256) gemm_ring64_kernel(const GemmParams p) {
             for (int r = 0; r < 4; ++r) {
                 const int m = m0 + wm * WT + 16 * i + 4 * r + lg;
                 if (RAGGED && (m >= p.M || n >= p.N)) continue;
-                double* cp = C + (int64_t)m * p.ldc + n;
+                NTG_GLOBAL double* cp = C + (int64_t)m * p.ldc + n;
                 double v = acc[i][j][r];
                 if (cmode == C_ACCUMULATE) v += *cp;
                 else if (cmode == C_BIAS) v += bias[(int64_t)b * p.bias_bs + (int64_t)m * p.bias_rs + (int64_t)n * p.bias_cs];
