@@ -64,37 +64,39 @@ __global__ void __launch_bounds__(256) gemm_small16_f32_kernel(const GemmParams 
     // instead (no branch, so the loads of several stages stay in flight and are waited for one stage at a time): rows of A
     // and columns of B past the edge only reach elements of C that are not stored, and k past the end is never multiplied.
     const int k_last = p.K - 4, m_last = TA ? p.M - 4 : p.M - 1, n_last = TB ? p.N - 1 : p.N - 4;
-    auto load_a = [&](int k0, f32x4 (&v)[NP]) {
-#pragma unroll
-        for (int u = 0; u < NP; ++u) {
-            if constexpr (TA) {
-                int k = k0 + (tid >> 3) + 32 * u, mm = m0 + (tid & 7) * 4;
-                k = k < p.K ? k : p.K - 1;
-                mm = mm < m_last ? mm : m_last;
-                v[u] = *(__attribute__((address_space(1))) const f32x4*)(A + (int64_t)k * p.lda + mm);
-            } else {
-                int mm = m0 + (tid >> 5) + 8 * u, k = k0 + (tid & 31) * 4;
-                mm = mm < m_last ? mm : m_last;
-                k = k < k_last ? k : k_last;
-                v[u] = *(__attribute__((address_space(1))) const f32x4*)(A + (int64_t)mm * p.lda + k);
-            }
+    auto load_a_piece = [&](int k0, int u, f32x4 (&v)[NP]) __attribute__((always_inline)) {
+        if constexpr (TA) {
+            int k = k0 + (tid >> 3) + 32 * u, mm = m0 + (tid & 7) * 4;
+            k = k < p.K ? k : p.K - 1;
+            mm = mm < m_last ? mm : m_last;
+            v[u] = *(__attribute__((address_space(1))) const f32x4*)(A + (int64_t)k * p.lda + mm);
+        } else {
+            int mm = m0 + (tid >> 5) + 8 * u, k = k0 + (tid & 31) * 4;
+            mm = mm < m_last ? mm : m_last;
+            k = k < k_last ? k : k_last;
+            v[u] = *(__attribute__((address_space(1))) const f32x4*)(A + (int64_t)mm * p.lda + k);
         }
     };
-    auto load_b = [&](int k0, f32x4 (&v)[NP]) {
-#pragma unroll
-        for (int u = 0; u < NP; ++u) {
-            if constexpr (TB) {
-                int nn = n0 + (tid >> 5) + 8 * u, k = k0 + (tid & 31) * 4;
-                nn = nn < n_last ? nn : n_last;
-                k = k < k_last ? k : k_last;
-                v[u] = *(__attribute__((address_space(1))) const f32x4*)(B + (int64_t)nn * p.ldb + k);
-            } else {
-                int k = k0 + (tid >> 3) + 32 * u, nn = n0 + (tid & 7) * 4;
-                k = k < p.K ? k : p.K - 1;
-                nn = nn < n_last ? nn : n_last;
-                v[u] = *(__attribute__((address_space(1))) const f32x4*)(B + (int64_t)k * p.ldb + nn);
-            }
+    auto load_b_piece = [&](int k0, int u, f32x4 (&v)[NP]) __attribute__((always_inline)) {
+        if constexpr (TB) {
+            int nn = n0 + (tid >> 5) + 8 * u, k = k0 + (tid & 31) * 4;
+            nn = nn < n_last ? nn : n_last;
+            k = k < k_last ? k : k_last;
+            v[u] = *(__attribute__((address_space(1))) const f32x4*)(B + (int64_t)nn * p.ldb + k);
+        } else {
+            int k = k0 + (tid >> 3) + 32 * u, nn = n0 + (tid & 7) * 4;
+            k = k < p.K ? k : p.K - 1;
+            nn = nn < n_last ? nn : n_last;
+            v[u] = *(__attribute__((address_space(1))) const f32x4*)(B + (int64_t)k * p.ldb + nn);
         }
+    };
+    auto load_a = [&](int k0, f32x4 (&v)[NP]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int u = 0; u < NP; ++u) load_a_piece(k0, u, v);
+    };
+    auto load_b = [&](int k0, f32x4 (&v)[NP]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int u = 0; u < NP; ++u) load_b_piece(k0, u, v);
     };
     // piece u of both operands of one stage, from registers to LDS buffer `buf`
     auto store_piece = [&](int buf, int u, const f32x4 (&va)[NP], const f32x4 (&vb)[NP]) __attribute__((always_inline)) {
@@ -128,10 +130,7 @@ __global__ void __launch_bounds__(256) gemm_small16_f32_kernel(const GemmParams 
     // that only the barrier and the first operand reads of the next stage are left outside the chain's shadow.
     auto stage = [&](int kt, auto slot_tag, auto request_tag) __attribute__((always_inline)) {
         constexpr int SLOT = decltype(slot_tag)::value, NEXT = (SLOT + 1) % DEPTH, buf = SLOT & 1;
-        if constexpr (decltype(request_tag)::value) {
-            load_a((kt + DEPTH) * KB, va[SLOT]);
-            load_b((kt + DEPTH) * KB, vb[SLOT]);
-        }
+        constexpr bool REQUEST = decltype(request_tag)::value;
         const float* a_s = sA[buf];
         const float* b_s = sB[buf];
         const int steps = p.K - kt * KB < KB ? (p.K - kt * KB) / 4 : KB / 4;      // (K is a multiple of 4: whole instructions)
@@ -150,17 +149,32 @@ __global__ void __launch_bounds__(256) gemm_small16_f32_kernel(const GemmParams 
             read_group(0, av[0], bv[0]);
 #pragma unroll
             for (int g = 0; g < KB / 32; ++g) {
+                // One group: its eight instructions (a dependent chain: 40 cycles each, the issue slots between them free), and
+                // in their shadow the operand reads of the next group, one piece of stage kt + 1 on its way to LDS and one piece
+                // of each operand of stage kt + DEPTH requested.  Left alone the scheduler puts all of that between two groups
+                // (the chain idle meanwhile) and sinks every read to just before its instruction; the recipe below deals the
+                // other instructions out behind the MFMAs, and nothing crosses the end of the group.
                 if (g + 1 < KB / 32) read_group(8 * (g + 1), av[(g + 1) & 1], bv[(g + 1) & 1]);
                 store_piece(buf ^ 1, g, va[NEXT], vb[NEXT]);
-                // (nothing moves across: left alone, the scheduler sinks every read to just before its instruction, and the
-                //  chain then waits for LDS once per pair of instructions)
-                __builtin_amdgcn_sched_barrier(0);
+                if constexpr (REQUEST) {
+                    load_a_piece((kt + DEPTH) * KB, g, va[SLOT]);
+                    load_b_piece((kt + DEPTH) * KB, g, vb[SLOT]);
+                }
 #pragma unroll
                 for (int u = 0; u < 8; ++u) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(bv[g & 1][u], av[g & 1][u], acc, 0, 0, 0);
+#pragma unroll
+                for (int u = 0; u < 8; ++u) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                // one MFMA
+                    __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);                // LDS reads of the next group
+                    if (u == 2 || u == 5) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);     // LDS writes of the hand-over
+                    __builtin_amdgcn_sched_group_barrier(0x002, 6, 0);                // address arithmetic
+                    if (REQUEST && (u == 3 || u == 6)) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);   // the requests
+                }
                 __builtin_amdgcn_sched_barrier(0);
             }
         } else {
-            for (int q = 0; q < steps; ++q) {                                     // (the last stage of a k that is not a multiple of 128)
+            // (the last stage of a k that is not a multiple of 128: never a stage that requests, kt + DEPTH < KT there)
+            for (int q = 0; q < steps; ++q) {
                 const int k = 4 * q + lg;
                 const float av = TA ? a_s[k * LDM + bi * 16 + li] : a_s[(bi * 16 + li) * LDK + k];
                 const float bv = TB ? b_s[(bj * 16 + li) * LDK + k] : b_s[k * LDM + bj * 16 + li];
