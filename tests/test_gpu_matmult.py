@@ -868,19 +868,25 @@ def test_single_large_products_split_into_two_launches(kind):
 
 
 def test_small_fp32_products_on_32_wide_tiles():
-    """Float32 products with too few output elements for 64 x 64 tiles run on 32 x 32 tiles whose four or eight wavefronts split
-    k (config 1 is one of them): every transpose pair and C mode, ragged edges in m, n and k, padded rows, batches,
-    against float64 products within the stated bound; two runs are bit-identical (fixed order of the partial sums)."""
+    """Float32 products with too few output elements for 64 x 64 tiles (config 1 is one of them): every transpose pair and C
+    mode, ragged edges in m, n and k, padded rows, batches, against float64 products within the stated bound; two runs are
+    bit-identical.  Rows that keep the 16-byte rule (pitches +4 / +8 / +4, sizes that are multiples of 4) take the 32 x 32-tile
+    kernel on v_mfma_f32_16x16x4 -- k tails that are not whole 128-k stages, one to nine stages, edge tiles whose loads are
+    clamped -- the odd pitches the register-staged kernel."""
     lib = _lib.load()
     st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
     gen = torch.Generator(device=DEV).manual_seed(4242)
     modes = (_lib.C_OVERWRITE, _lib.C_ACCUMULATE, _lib.C_BIAS)
     i = 0
-    for (m, k, n, batch) in [(512, 512, 512, 1), (100, 300, 70, 1), (33, 64, 33, 1), (40, 1003, 50, 2), (256, 130, 250, 3), (65, 77, 129, 4)]:
+    cases = [(512, 512, 512, 1, (3, 5, 2)), (100, 300, 70, 1, (3, 5, 2)), (33, 64, 33, 1, (3, 5, 2)), (40, 1003, 50, 2, (3, 5, 2)),
+             (256, 130, 250, 3, (3, 5, 2)), (65, 77, 129, 4, (3, 5, 2)),
+             (512, 512, 512, 1, (4, 8, 4)), (100, 300, 72, 1, (4, 8, 4)), (36, 64, 36, 1, (0, 0, 0)), (40, 1004, 52, 2, (4, 8, 4)),
+             (256, 132, 248, 3, (0, 4, 8)), (68, 76, 128, 4, (4, 8, 4)), (132, 1156, 60, 1, (0, 0, 0)), (48, 640, 36, 5, (8, 4, 4))]
+    for (m, k, n, batch, pads) in cases:
         for ta, tb in TRANS:
             mode = modes[i % 3]
             i += 1
-            lda, ldb, ldc = (m if ta else k) + 3, (k if tb else n) + 5, n + 2
+            lda, ldb, ldc = (m if ta else k) + pads[0], (k if tb else n) + pads[1], n + pads[2]
             a = torch.randn(batch, k if ta else m, lda, device=DEV, generator=gen)
             b = torch.randn(batch, n if tb else k, ldb, device=DEV, generator=gen)
             c0 = torch.randn(batch, m, ldc, device=DEV, generator=gen)
@@ -894,7 +900,7 @@ def test_small_fp32_products_on_32_wide_tiles():
             d.stride_a, d.stride_b, d.stride_c = a.shape[1] * lda, b.shape[1] * ldb, m * ldc
             if mode == _lib.C_BIAS:
                 d.bias, d.bias_col_stride = bias.data_ptr(), 1
-            assert lib.ntg_gemm_workspace_bytes(ctypes.byref(d)) == 0
+            # (a deep k on few tiles may be offered a split along k; no workspace is passed here, so the plain kernels run)
             outs = []
             for rep in range(2):
                 c = c0.clone()
