@@ -215,7 +215,7 @@ __global__ void __launch_bounds__(256) gemm_small16_f32_kernel(const GemmParams 
 // the shorter chain to matter.  The results do not depend on the choice.
 static bool small16_f32_wins(const GemmParams& p) {
     const int64_t t64 = (int64_t)((p.M + 63) / 64) * ((p.N + 63) / 64) * p.batch;
-    return t64 <= 128 && p.K >= 64 && p.M > 32 && p.cmode != C_PARTIAL && p.krange_items == 0;
+    return t64 <= 128 && p.K >= 64 && p.M > 32 && p.cmode != C_PARTIAL && p.krange_items == 0 && !p.tailA && !p.tailB;
 }
 static hipError_t launch_small16_f32(bool ta, bool tb, const GemmParams& pin, hipStream_t s) {
     GemmParams p = pin;
@@ -235,6 +235,7 @@ static hipError_t launch_small16_f32(bool ta, bool tb, const GemmParams& pin, hi
 }
 
 hipError_t launch_gemm_mfma_f32(bool ta, bool tb, const GemmParams& p, hipStream_t s) {
+    if ((p.tailA || p.tailB) && !ring_eligible(p, ta, 4)) return hipErrorInvalidValue;       // (only the DMA-fed kernel reads copied tail rows)
     if (ring_eligible(p, ta, 4) && small16_f32_wins(p)) return launch_small16_f32(ta, tb, p, s);
     if (ring_eligible(p, ta, 4))
         return ring_f32_tile_edge(p) == 64 ? launch_ring_wb<DT_F32, 1>(ta, tb, p, s) : launch_ring_wb<DT_F32, 2>(ta, tb, p, s);

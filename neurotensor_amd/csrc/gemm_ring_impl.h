@@ -608,7 +608,7 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
     };
 
     // uniform (scalar) source pointer of one operand tile
-    auto tile_src = [&](const char* base) -> const void* {
+    auto tile_src = [&](const char* base) __attribute__((always_inline)) -> const void* {
         const uint64_t bu = reinterpret_cast<uint64_t>(base);
         const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)bu);
         const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(bu >> 32));
@@ -701,8 +701,14 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
     // K-steps past the end are clamped to the last one: the tail iterations then issue the
     // same DMA traffic as the steady state (into stages nobody reads any more), which keeps
     // the loop body free of branches and the vmcnt bookkeeping uniform.
-    auto srcA = [&](int kt) {
+    // (Float32, guarded instantiation: the last k-rows of an operand that is read in place may come from a zero-padded copy)
+    constexpr bool TAIL_ROWS = RAGGED && CONV == 0 && ES == 4;
+    auto srcA = [&](int kt) __attribute__((always_inline)) {
         const int kc = kt < last ? kt : last;
+        if constexpr (TAIL_ROWS && !A_KC) {
+            if (p.tailA && kc * BK >= p.tail_k0)                   // (uniform)
+                return tile_src(static_cast<const char*>(p.tailA) + ((int64_t)b * p.s_tailA + (int64_t)(kc * BK - p.tail_k0) * p.lda + m0) * ES);
+        }
         if constexpr (GATHERW && A_KC) {
             if (p.conv.a_steps) {                                  // (uniform) K-step counted through the images -> image, step inside it
                 const uint32_t gs = (uint32_t)(b * KT + kc), im = fast_div(gs, p.conv.div_a_steps);
@@ -711,7 +717,14 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
         }
         return tile_src(baseA + (int64_t)kc * advA);
     };
-    auto srcB = [&](int kt) { return tile_src(baseB + (int64_t)(kt < last ? kt : last) * advB); };
+    auto srcB = [&](int kt) __attribute__((always_inline)) {
+        const int kc = kt < last ? kt : last;
+        if constexpr (TAIL_ROWS && !B_KC) {
+            if (p.tailB && kc * BK >= p.tail_k0)                   // (uniform)
+                return tile_src(static_cast<const char*>(p.tailB) + ((int64_t)b * p.s_tailB + (int64_t)(kc * BK - p.tail_k0) * p.ldb + n0) * ES);
+        }
+        return tile_src(baseB + (int64_t)kc * advB);
+    };
 
     // prologue: tiles 0..2 and the A half of tile 3 in flight (3 (NA + NB) + NA instructions)
     auto b_tile = [&](int kt, uint32_t lds_tile) __attribute__((always_inline)) {
@@ -1185,7 +1198,7 @@ static hipError_t launch_ring_cfg(const GemmParams& pin, hipStream_t s) {
     p.group_m = ring_tile_order_override();
     const int64_t blocks = (int64_t)p.tiles_m * p.tiles_n * p.batch;
     if (blocks > 0x7fffffffLL) return hipErrorInvalidValue;
-    if (p.M % TEM == 0 && p.N % TEN == 0 && p.K % BK == 0)
+    if (p.M % TEM == 0 && p.N % TEN == 0 && p.K % BK == 0 && !p.tailA && !p.tailB)      // (copied tail rows: the guarded instantiation reads them)
         hipLaunchKernelGGL((gemm_ring_kernel<DT, TA, TB, false, WB, 0, WBN, KD>), dim3((unsigned)blocks), dim3(256), 0, s, p);
     else
         hipLaunchKernelGGL((gemm_ring_kernel<DT, TA, TB, true, WB, 0, WBN, KD>), dim3((unsigned)blocks), dim3(256), 0, s, p);

@@ -283,6 +283,8 @@ static int run_int_planes(const ntg::GemmParams& p, const IntPlanesPlan& pl, boo
 // 16-byte multiples is computed into a padded copy and copied back.  Taken for products large enough to repay the copies.
 struct PadPlan {
     bool ok, padA, padB, padC;
+    bool stripA, stripB;            // Float32: the operand stays where it is, only its last k-rows are copied (and continued with zeros)
+    int strip_k0, strip_rows;
     int Mp, Kp, Np;
     int64_t lda2, ldb2, rowsA2, rowsB2, a_bytes, b_bytes, c_bytes;
     int64_t bytes() const { return a_bytes + b_bytes + c_bytes; }
@@ -311,6 +313,16 @@ static PadPlan plan_pad(const ntg::GemmParams& p, int dtype, bool ta, bool tb) {
     pl.ldb2 = tb ? pl.Kp : pl.Np; pl.rowsB2 = tb ? pl.Np : pl.Kp;
     const int64_t ldmax = (int64_t)(1 << 23) / es;                         // (the kernels' 32-bit lane offsets)
     if ((pl.padA ? pl.lda2 : p.lda) >= ldmax || (pl.padB ? pl.ldb2 : p.ldb) >= ldmax) return pl;
+    // Float32, an operand stored [k][m] / [k][n] that only lacks k-rows up to a whole chunk: its rows keep the 16-byte rule, so the
+    // kernel reads it in place and takes the last K-step's rows from a copy of at most 16 rows instead of a copy of everything
+    if (dtype == ntg::DT_F32 && pl.Kp != p.K && p.K > 16) {
+        pl.strip_k0 = (pl.Kp - 1) / 16 * 16;
+        pl.strip_rows = pl.Kp - pl.strip_k0;
+        pl.stripA = pl.padA && ta && !misaligned(p.A, p.lda, p.sA) && pl.Mp == p.M;
+        pl.stripB = pl.padB && !tb && !misaligned(p.B, p.ldb, p.sB) && pl.Np == p.N;
+        if (pl.stripA) { pl.padA = false; pl.a_bytes = (int64_t)align_up((size_t)((p.sA == 0 ? 1 : p.batch) * pl.strip_rows * p.lda * es), 256); }
+        if (pl.stripB) { pl.padB = false; pl.b_bytes = (int64_t)align_up((size_t)((p.sB == 0 ? 1 : p.batch) * pl.strip_rows * p.ldb * es), 256); }
+    }
     if (pl.padA) pl.a_bytes = (int64_t)align_up((size_t)((p.sA == 0 ? 1 : p.batch) * pl.rowsA2 * pl.lda2 * es), 256);
     if (pl.padB) pl.b_bytes = (int64_t)align_up((size_t)((p.sB == 0 ? 1 : p.batch) * pl.rowsB2 * pl.ldb2 * es), 256);
     if (pl.padC) pl.c_bytes = (int64_t)align_up((size_t)((int64_t)p.batch * pl.Mp * pl.Np * es), 256);
@@ -334,6 +346,18 @@ static int run_padded(const ntg::GemmParams& p, const PadPlan& pl, int dtype, bo
         e = ntg::launch_pad_copy(es, p.B, p.ldb, p.sB, b2, pl.ldb2, pl.rowsB2 * pl.ldb2, tb ? p.N : p.K, tb ? p.K : p.N, pl.rowsB2, p.sB == 0 ? 1 : p.batch, s);
         if (e != hipSuccess) return hip_fail(e, "padded copy of B");
         q.B = b2; q.ldb = pl.ldb2; q.sB = p.sB == 0 ? 0 : pl.rowsB2 * pl.ldb2;
+    }
+    if (pl.stripA) {
+        e = ntg::launch_pad_copy(es, static_cast<const char*>(p.A) + (int64_t)pl.strip_k0 * p.lda * es, p.lda, p.sA, a2, p.lda, (int64_t)pl.strip_rows * p.lda,
+                                 p.K - pl.strip_k0, p.M, pl.strip_rows, p.sA == 0 ? 1 : p.batch, s);
+        if (e != hipSuccess) return hip_fail(e, "copy of A's last k-rows");
+        q.tailA = a2; q.s_tailA = p.sA == 0 ? 0 : (int64_t)pl.strip_rows * p.lda; q.tail_k0 = pl.strip_k0;
+    }
+    if (pl.stripB) {
+        e = ntg::launch_pad_copy(es, static_cast<const char*>(p.B) + (int64_t)pl.strip_k0 * p.ldb * es, p.ldb, p.sB, b2, p.ldb, (int64_t)pl.strip_rows * p.ldb,
+                                 p.K - pl.strip_k0, p.N, pl.strip_rows, p.sB == 0 ? 1 : p.batch, s);
+        if (e != hipSuccess) return hip_fail(e, "copy of B's last k-rows");
+        q.tailB = b2; q.s_tailB = p.sB == 0 ? 0 : (int64_t)pl.strip_rows * p.ldb; q.tail_k0 = pl.strip_k0;
     }
     if (pl.padC) {
         const int64_t sc2 = (int64_t)pl.Mp * pl.Np;

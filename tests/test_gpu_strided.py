@@ -203,6 +203,14 @@ def test_rows_that_are_not_16_byte_multiples_through_padded_copies(name):
     run_case(rng, name, m + 3, k + 7, n + 1, True, False, ODD, _lib.C_BIAS, base=1, workspace=True, one_rounding=half)   # everything odd, C padded too
     run_case(rng, name, m, k + 7, n - 6, False, True, (0, 8, 5), _lib.C_ACCUMULATE, batches=2, gap=3, workspace=True, one_rounding=half)
     run_case(rng, name, m, 1008, n - 6, False, False, (0, 0, 0), _lib.C_OVERWRITE, batches=2, bcast_b=True, base=3, workspace=64 << 20, one_rounding=half)   # only the base pointers are odd
+    if name == "f32":
+        # only k misses the chunk and an operand stored [k][m] / [k][n] keeps the 16-byte rule: it is read where it lies and only
+        # its last k-rows are copied (k = 4 j + 1, + 2, + 3, and a k whose padded size is a whole K-step); the reference's bits
+        for (ta, tb), mode, k2 in zip(TRANS, modes, (1501, 1502, 1503, 1535)):
+            run_case(rng, name, 1700, k2, 1704, ta, tb, (0, 0, 0), mode, workspace=True, flags=_lib.GEMM_KEEP_K_ORDER, f32_bits=True)
+        run_case(rng, name, 1700, 1501, 1704, False, False, (0, 8, 4), _lib.C_ACCUMULATE, batches=2, gap=8, workspace=True)
+        run_case(rng, name, 1700, 1509, 1704, True, False, (4, 0, 0), _lib.C_BIAS, batches=3, bcast_b=True, workspace=True)
+        run_case(rng, name, 520, 16385, 512, False, False, (0, 0, 0), _lib.C_OVERWRITE, workspace=True)          # few tiles, a deep k
 
 
 def _random_dim(rng, hi):
