@@ -2,6 +2,7 @@
 #include "gemm_ring_impl.h"
 namespace ntg {
 hipError_t launch_gemm_mfma_f16(bool ta, bool tb, const GemmParams& p, hipStream_t s) {
+    if ((p.tailA || p.tailB) && !ring_eligible(p, ta)) return hipErrorInvalidValue;       // (only the DMA-fed kernel reads copied tail rows)
     if (ring_eligible(p, ta)) return launch_ring16<DT_F16>(ta, tb, p, s);   // DMA-fed LDS ring; the tile (256 x 256 .. 64 x 64, 192 x 256, 128 x 256) follows ring16_tile_edge
     const int64_t big_tiles = (int64_t)((p.M + 255) / 256) * ((p.N + 255) / 256) * p.batch;
     if (big_tiles >= 256) return launch_trans<DT_F16, 4, 4, 64>(ta, tb, p, s);   // 256 x 256 x 64

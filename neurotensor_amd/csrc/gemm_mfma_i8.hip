@@ -6,6 +6,7 @@
 #include "gemm_ring_impl.h"
 namespace ntg {
 hipError_t launch_gemm_mfma_i8(int dtype, bool ta, bool tb, const GemmParams& p, hipStream_t s) {
+    if ((p.tailA || p.tailB) && !ring_eligible(p, ta, 1)) return hipErrorInvalidValue;     // (only the DMA-fed kernel reads copied tail rows)
     if (!ring_eligible(p, ta, 1)) {
         if (p.cmode == C_PARTIAL) return hipErrorInvalidValue;      // (only the DMA-fed kernel writes 32-bit sums)
         return launch_gemm_valu(dtype, ta, tb, p, s);

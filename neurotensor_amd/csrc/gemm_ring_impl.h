@@ -701,8 +701,8 @@ __global__ void __launch_bounds__(256) gemm_ring_kernel(const GemmParams p) {
     // K-steps past the end are clamped to the last one: the tail iterations then issue the
     // same DMA traffic as the steady state (into stages nobody reads any more), which keeps
     // the loop body free of branches and the vmcnt bookkeeping uniform.
-    // (Float32, guarded instantiation: the last k-rows of an operand that is read in place may come from a zero-padded copy)
-    constexpr bool TAIL_ROWS = RAGGED && CONV == 0 && ES == 4;
+    // (guarded instantiation: the last k-rows of an M/N-contiguous operand that is read in place may come from a zero-padded copy)
+    constexpr bool TAIL_ROWS = RAGGED && CONV == 0;
     auto srcA = [&](int kt) __attribute__((always_inline)) {
         const int kc = kt < last ? kt : last;
         if constexpr (TAIL_ROWS && !A_KC) {
@@ -1278,6 +1278,8 @@ static inline GemmParams ring_batch_range(const GemmParams& p, int64_t es, int b
     q.B = static_cast<const char*>(p.B) + (int64_t)b0 * p.sB * es;
     q.C = static_cast<char*>(p.C) + (int64_t)b0 * p.sC * es;
     if (p.bias) q.bias = static_cast<const char*>(p.bias) + (int64_t)b0 * p.bias_bs * es;
+    if (p.tailA) q.tailA = static_cast<const char*>(p.tailA) + (int64_t)b0 * p.s_tailA * es;
+    if (p.tailB) q.tailB = static_cast<const char*>(p.tailB) + (int64_t)b0 * p.s_tailB * es;
     q.batch = nb;
     return q;
 }
@@ -1325,12 +1327,14 @@ static inline void ring_split_params(const GemmParams& p, bool ta, bool tb, int6
         head.N = (int)sp.head;
         tail.N = p.N - (int)sp.head;
         tail.B = B + (tb ? sp.head * p.ldb : sp.head) * es;
+        if (p.tailB) tail.tailB = static_cast<const char*>(p.tailB) + sp.head * es;       // (copied k-rows exist for B stored [k][n] only)
         tail.C = C + sp.head * es;
         if (bias) tail.bias = bias + sp.head * p.bias_cs * es;
     } else {                                     // rows [0, head) | [head, M)
         head.M = (int)sp.head;
         tail.M = p.M - (int)sp.head;
         tail.A = A + (ta ? sp.head : sp.head * p.lda) * es;
+        if (p.tailA) tail.tailA = static_cast<const char*>(p.tailA) + sp.head * es;       // (... for A stored [k][m] only)
         tail.C = C + sp.head * p.ldc * es;
         if (bias) tail.bias = bias + sp.head * p.bias_rs * es;
     }
@@ -1366,6 +1370,7 @@ static hipError_t launch_ring16(bool ta, bool tb, const GemmParams& p, hipStream
             head.N = (int)head_cols;
             tail.N = p.N - (int)head_cols;
             tail.B = static_cast<const char*>(p.B) + head_cols * (tb ? p.ldb : 1) * 2;
+            if (p.tailB) tail.tailB = static_cast<const char*>(p.tailB) + head_cols * 2;
             tail.C = static_cast<char*>(p.C) + head_cols * 2;
             if (p.bias) tail.bias = static_cast<const char*>(p.bias) + head_cols * p.bias_cs * 2;
             const hipError_t e = launch_ring16_planned(head, s, launch, RECT_128 | RECT_192);

@@ -283,7 +283,7 @@ static int run_int_planes(const ntg::GemmParams& p, const IntPlanesPlan& pl, boo
 // 16-byte multiples is computed into a padded copy and copied back.  Taken for products large enough to repay the copies.
 struct PadPlan {
     bool ok, padA, padB, padC;
-    bool stripA, stripB;            // Float32: the operand stays where it is, only its last k-rows are copied (and continued with zeros)
+    bool stripA, stripB;            // the operand stays where it is, only its last k-rows are copied (and continued with zeros)
     int strip_k0, strip_rows;
     int Mp, Kp, Np;
     int64_t lda2, ldb2, rowsA2, rowsB2, a_bytes, b_bytes, c_bytes;
@@ -313,10 +313,11 @@ static PadPlan plan_pad(const ntg::GemmParams& p, int dtype, bool ta, bool tb) {
     pl.ldb2 = tb ? pl.Kp : pl.Np; pl.rowsB2 = tb ? pl.Np : pl.Kp;
     const int64_t ldmax = (int64_t)(1 << 23) / es;                         // (the kernels' 32-bit lane offsets)
     if ((pl.padA ? pl.lda2 : p.lda) >= ldmax || (pl.padB ? pl.ldb2 : p.ldb) >= ldmax) return pl;
-    // Float32, an operand stored [k][m] / [k][n] that only lacks k-rows up to a whole chunk: its rows keep the 16-byte rule, so the
-    // kernel reads it in place and takes the last K-step's rows from a copy of at most 16 rows instead of a copy of everything
-    if (dtype == ntg::DT_F32 && pl.Kp != p.K && p.K > 16) {
-        pl.strip_k0 = (pl.Kp - 1) / 16 * 16;
+    // An operand stored [k][m] / [k][n] that only lacks k-rows up to a whole chunk: its rows keep the 16-byte rule, so the kernel
+    // reads it in place and takes its last k-rows (from a multiple of 128, which every kernel's K-step divides) from a copy of at
+    // most 128 rows that continues with rows of zeros, instead of a copy of everything.  (Not Float64: its kernel has no such source.)
+    if (dtype != ntg::DT_F64 && pl.Kp != p.K && p.K > 128) {
+        pl.strip_k0 = (pl.Kp - 1) / 128 * 128;
         pl.strip_rows = pl.Kp - pl.strip_k0;
         pl.stripA = pl.padA && ta && !misaligned(p.A, p.lda, p.sA) && pl.Mp == p.M;
         pl.stripB = pl.padB && !tb && !misaligned(p.B, p.ldb, p.sB) && pl.Np == p.N;

@@ -203,15 +203,25 @@ def test_rows_that_are_not_16_byte_multiples_through_padded_copies(name):
     run_case(rng, name, m + 3, k + 7, n + 1, True, False, ODD, _lib.C_BIAS, base=1, workspace=True, one_rounding=half)   # everything odd, C padded too
     run_case(rng, name, m, k + 7, n - 6, False, True, (0, 8, 5), _lib.C_ACCUMULATE, batches=2, gap=3, workspace=True, one_rounding=half)
     run_case(rng, name, m, 1008, n - 6, False, False, (0, 0, 0), _lib.C_OVERWRITE, batches=2, bcast_b=True, base=3, workspace=64 << 20, one_rounding=half)   # only the base pointers are odd
-    if name == "f32":
+    if name != "f64":
         # only k misses the chunk and an operand stored [k][m] / [k][n] keeps the 16-byte rule: it is read where it lies and only
-        # its last k-rows are copied (k = 4 j + 1, + 2, + 3, and a k whose padded size is a whole K-step); the reference's bits
-        for (ta, tb), mode, k2 in zip(TRANS, modes, (1501, 1502, 1503, 1535)):
-            run_case(rng, name, 1700, k2, 1704, ta, tb, (0, 0, 0), mode, workspace=True, flags=_lib.GEMM_KEEP_K_ORDER, f32_bits=True)
-        run_case(rng, name, 1700, 1501, 1704, False, False, (0, 8, 4), _lib.C_ACCUMULATE, batches=2, gap=8, workspace=True)
-        run_case(rng, name, 1700, 1509, 1704, True, False, (4, 0, 0), _lib.C_BIAS, batches=3, bcast_b=True, workspace=True)
-        run_case(rng, name, 520, 16385, 512, False, False, (0, 0, 0), _lib.C_OVERWRITE, workspace=True)          # few tiles, a deep k
-
+        # its last k-rows are copied (several k tails, among them one whose padded size is a whole K-step); Float32 must be
+        # the reference's bits
+        f32 = name == "f32"
+        m2, n2 = (1700, 1704) if f32 else (1304, 1712) if half else (528, 544)
+        ks = (1501, 1502, 1503, 1535) if f32 else (1001, 1003, 1017, 1087) if half else (1001, 1009, 1023, 1090)
+        for (ta, tb), mode, k2 in zip(TRANS, modes, ks):
+            run_case(rng, name, m2, k2, n2, ta, tb, (0, 0, 0), mode, workspace=True, one_rounding=half,
+                     flags=_lib.GEMM_KEEP_K_ORDER if f32 else 0, f32_bits=f32)
+        run_case(rng, name, m2, ks[0], n2, False, False, (0, 16, 16), _lib.C_ACCUMULATE, batches=2, gap=16, workspace=True, one_rounding=half)
+        run_case(rng, name, m2, ks[1] + 8, n2, True, False, (16, 0, 0), _lib.C_BIAS, batches=3, bcast_b=True, workspace=True, one_rounding=half)
+        if f32:
+            run_case(rng, name, 520, 16385, 512, False, False, (0, 0, 0), _lib.C_OVERWRITE, workspace=True)          # few tiles, a deep k
+        if half:
+            # products that go out as two launches with shifted operand pointers (rows / columns split, a batch in two parts)
+            run_case(rng, name, 2056, 1001, 2320, False, False, (0, 0, 0), _lib.C_ACCUMULATE, workspace=True, one_rounding=True)
+            run_case(rng, name, 2320, 1001, 2056, True, False, (0, 0, 0), _lib.C_OVERWRITE, workspace=True, one_rounding=True)
+            run_case(rng, name, 264, 1001, 2304, False, False, (0, 0, 0), _lib.C_ACCUMULATE, batches=33, workspace=True, one_rounding=True)
 
 def _random_dim(rng, hi):
     """sizes that sit on, just below and just above the tile edges, tiny ones, multiples of 8 and anything else"""
