@@ -11,6 +11,7 @@ static int ring64_tile_edge(const GemmParams& p) {
     return cost64 < cost128 ? 64 : 128;
 }
 hipError_t launch_gemm_mfma_f64(bool ta, bool tb, const GemmParams& p, hipStream_t s) {
+    if ((p.tailA || p.tailB) && !ring64_eligible(p, ta)) return hipErrorInvalidValue;       // (only the DMA-fed kernel reads copied tail rows)
     if (ring64_eligible(p, ta))
         return ring64_tile_edge(p) == 64 ? launch_ring64_wb<1>(ta, tb, p, s) : launch_ring64_wb<2>(ta, tb, p, s);
     // rows that are not 16-byte aligned (or pointer tables): register-staged kernel

@@ -68,15 +68,30 @@ __global__ void __launch_bounds__(256) gemm_ring64_kernel(const GemmParams p) {
     const char* baseB = reinterpret_cast<const char*>(B) + (B_KC ? (int64_t)n0 * p.ldb : (int64_t)n0) * 8;
     const int64_t advA = (A_KC ? (int64_t)BK : (int64_t)BK * p.lda) * 8;
     const int64_t advB = (B_KC ? (int64_t)BK : (int64_t)BK * p.ldb) * 8;
-    auto tile_src = [&](const char* base) -> const void* {
+    auto tile_src = [&](const char* base) __attribute__((always_inline)) -> const void* {
         const uint64_t bu = reinterpret_cast<uint64_t>(base);
         const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)bu);
         const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(bu >> 32));
         return reinterpret_cast<const void*>(((uint64_t)hi << 32) | lo);
     };
     // K-steps past the end re-fetch the last one (into stages nobody reads any more): the loop body stays branch free
-    auto srcA = [&](int kt) { return tile_src(baseA + (int64_t)(kt < last ? kt : last) * advA); };
-    auto srcB = [&](int kt) { return tile_src(baseB + (int64_t)(kt < last ? kt : last) * advB); };
+    // (guarded instantiation: the last k-rows of an M/N-contiguous operand that is read in place may come from a zero-padded copy)
+    auto srcA = [&](int kt) __attribute__((always_inline)) {
+        const int kc = kt < last ? kt : last;
+        if constexpr (RAGGED && !A_KC) {
+            if (p.tailA && kc * BK >= p.tail_k0)                   // (uniform)
+                return tile_src(static_cast<const char*>(p.tailA) + ((int64_t)b * p.s_tailA + (int64_t)(kc * BK - p.tail_k0) * p.lda + m0) * 8);
+        }
+        return tile_src(baseA + (int64_t)kc * advA);
+    };
+    auto srcB = [&](int kt) __attribute__((always_inline)) {
+        const int kc = kt < last ? kt : last;
+        if constexpr (RAGGED && !B_KC) {
+            if (p.tailB && kc * BK >= p.tail_k0)                   // (uniform)
+                return tile_src(static_cast<const char*>(p.tailB) + ((int64_t)b * p.s_tailB + (int64_t)(kc * BK - p.tail_k0) * p.ldb + n0) * 8);
+        }
+        return tile_src(baseB + (int64_t)kc * advB);
+    };
 
     // fragment read r of an operand: K-major r = block; MN-major r = 2 * block + k parity
     constexpr int NRA = A_KC ? NBL : 2 * NBL, NRB = B_KC ? NBL : 2 * NBL, NR = NRA + NRB;
@@ -210,7 +225,7 @@ static hipError_t launch_ring64_cfg(const GemmParams& pin, hipStream_t s) {
     const int64_t blocks = (int64_t)p.tiles_m * p.tiles_n * p.batch;
     if (blocks <= 0) return hipSuccess;
     if (blocks > 0x7fffffffLL) return hipErrorInvalidValue;
-    if (p.M % TE == 0 && p.N % TE == 0 && p.K % 8 == 0)
+    if (p.M % TE == 0 && p.N % TE == 0 && p.K % 8 == 0 && !p.tailA && !p.tailB)      // (copied tail rows: the guarded instantiation reads them)
         hipLaunchKernelGGL((gemm_ring64_kernel<TA, TB, false, WB>), dim3((unsigned)blocks), dim3(256), 0, s, p);
     else
         hipLaunchKernelGGL((gemm_ring64_kernel<TA, TB, true, WB>), dim3((unsigned)blocks), dim3(256), 0, s, p);

@@ -101,7 +101,7 @@ struct GemmParams {
     int cmode;
     int tiles_m, tiles_n;
     int vecA_ok, vecB_ok;    // 16-byte vector loads are legal for every row of A / B
-    // Padded-copy form (DMA-fed kernels, not Float64): an operand stored [k][m] / [k][n] whose rows keep the 16-byte rule is read where it lies, and only
+    // Padded-copy form (DMA-fed kernels): an operand stored [k][m] / [k][n] whose rows keep the 16-byte rule is read where it lies, and only
     // its k-rows from tail_k0 (a multiple of the K-step) on come from a small copy that continues with rows of zeros up to the padded K
     // (same row pitch as the operand; s_tail = elements between the items' copies, 0 = one for all).  Null: none.
     const void* tailA;

@@ -315,8 +315,8 @@ static PadPlan plan_pad(const ntg::GemmParams& p, int dtype, bool ta, bool tb) {
     if ((pl.padA ? pl.lda2 : p.lda) >= ldmax || (pl.padB ? pl.ldb2 : p.ldb) >= ldmax) return pl;
     // An operand stored [k][m] / [k][n] that only lacks k-rows up to a whole chunk: its rows keep the 16-byte rule, so the kernel
     // reads it in place and takes its last k-rows (from a multiple of 128, which every kernel's K-step divides) from a copy of at
-    // most 128 rows that continues with rows of zeros, instead of a copy of everything.  (Not Float64: its kernel has no such source.)
-    if (dtype != ntg::DT_F64 && pl.Kp != p.K && p.K > 128) {
+    // most 128 rows that continues with rows of zeros, instead of a copy of everything.
+    if (pl.Kp != p.K && p.K > 128) {
         pl.strip_k0 = (pl.Kp - 1) / 128 * 128;
         pl.strip_rows = pl.Kp - pl.strip_k0;
         pl.stripA = pl.padA && ta && !misaligned(p.A, p.lda, p.sA) && pl.Mp == p.M;
