@@ -478,7 +478,9 @@ def main():
         run("batch_bf16_32x1024_pointer_tables_vouched", ptr_tables(True), fb, PEAK_TFLOPS["bf16"])
         run("batch_bf16_32x1024_pointer_tables", ptr_tables(False), fb, PEAK_TFLOPS["bf16"])
         # rows that are not 16-byte multiples: operands copied into zero-padded rows in the workspace, then the DMA-fed kernel
+        # (A, whose rows of 4001 elements miss the rule, is copied; B, stored [k][n], is read where it lies and only its last k-rows are copied)
         run("c3_fp32_4096x4001x4096_padded_copies", G(torch.float32, N, 4001, N, mode=_lib.C_OVERWRITE), 2.0 * N * 4001 * N, PEAK_TFLOPS["fp32"])
+        run("c3_bf16_4096x4001x4096_padded_copies", G(torch.bfloat16, N, 4001, N, scale=0.02, mode=_lib.C_OVERWRITE), 2.0 * N * 4001 * N, PEAK_TFLOPS["bf16"])
         fc = 2.0 * 200704 * 2304 * 256
 
         def conv_case(half, backward):
