@@ -162,7 +162,8 @@ def test_split_k_planner_needs_no_device():
     assert ws(_lib.BFLOAT16, 128, 8192, 8190) == 8192 * 8192 * 2 + 128 * 8192 * 2 and ws(_lib.BFLOAT16, 128, 8192, 8192, lda=8196) == 128 * 8192 * 2
     assert ws(_lib.BFLOAT16, 128, 1024, 1022) == 0 and ws(_lib.BFLOAT16, 128, 1024, 1024, lda=1028) == 0      # too small to repay the copies
     # 8-bit integers: the alternative is the vector ALU, so the padded form starts earlier
-    assert ws(_lib.INT8, 520, 1001, 530) == 520 * 1008 + 1008 * 544 + 520 * 544 + (256 - 520 * 1008 % 256) % 256 + (256 - 1008 * 544 % 256) % 256 + (256 - 520 * 544 % 256) % 256
+    # (k 1001 -> 1008, n 530 -> 544; the copies of A and B have rows of whole 128-byte lines: 1024 and 640 bytes)
+    assert ws(_lib.INT8, 520, 1001, 530) == 520 * 1024 + 1008 * 640 + 520 * 544 + (256 - 520 * 1024 % 256) % 256 + (256 - 1008 * 640 % 256) % 256 + (256 - 520 * 544 % 256) % 256
     assert ws(_lib.INT8, 100, 101, 103) == 0 and ws(_lib.INT32, 100, 101, 103) == 0
     # fp32 / fp64, 64 x 64 tiles: 16 tiles and k = 1024 -> eight ranges of 128; 256 or more tiles -> none
     assert ranges(_lib.FLOAT32, 256, 1024, 256, 4) == 8
