@@ -121,6 +121,10 @@ __global__ void __launch_bounds__(256) gemm_small16_f32_kernel(const GemmParams 
     for (int sg = 1; sg < DEPTH; ++sg) {
         // SHORTK (fewer than DEPTH stages): a short k asks for nothing it does not use, at the price of inexact waits
         if (!SHORTK || sg < KT) { load_a(sg * KB, va[sg]); load_b(sg * KB, vb[sg]); }
+        else {                          // (never multiplied, but handed to LDS like any stage: defined values)
+#pragma unroll
+            for (int u = 0; u < NP; ++u) va[sg][u] = vb[sg][u] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+        }
     }
 #pragma unroll
     for (int u = 0; u < NP; ++u) store_piece(0, u, va[0], vb[0]);
