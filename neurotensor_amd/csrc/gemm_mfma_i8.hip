@@ -35,6 +35,11 @@ hipError_t launch_gemm_mfma_i8(int dtype, bool ta, bool tb, const GemmParams& p,
     }
     return launch(ring16_tile_edge(p.M, p.N, p.K, p.batch, rect), p);
 }
+// the DMA-fed kernel or nothing (the gated pair of an unvouched pointer-table batch)
+hipError_t launch_gemm_ring_only_i8(int dtype, bool ta, bool tb, const GemmParams& p, hipStream_t s, bool* taken) {
+    *taken = ring_eligible(p, ta, 1);
+    return *taken ? launch_gemm_mfma_i8(dtype, ta, tb, p, s) : hipSuccess;
+}
 
 // ---- 16-, 32- and 64-bit integer products on the same pipe --------------------------------------------------------
 // The reference's integer product wraps in the element type (nt/mp/simde_traits/simde_traits_avx2.h:810-812 16-bit,

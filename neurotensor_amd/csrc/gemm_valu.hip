@@ -16,6 +16,7 @@ __global__ void __launch_bounds__(256) gemm_valu_kernel(const GemmParams p, cons
     __shared__ T sA[BK][BM + PAD];
     __shared__ T sB[BK][BN + PAD];
 
+    if (p.gate && *p.gate != p.gate_want) return;       // (uniform: the other kernel of a gated pair does this product)
     const int tid = threadIdx.x;
     const int lid = xcd_contiguous_id(blockIdx.x, gridDim.x);
     const int tiles = p.tiles_m * p.tiles_n;
