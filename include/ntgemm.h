@@ -189,8 +189,8 @@ typedef struct ntg_gemm_desc {
 /* ntg_gemm_ptrs_dev only: the caller vouches that EVERY entry of the three pointer tables is a multiple of 16 bytes.  The
  * tables live in device memory, so the host side of the library cannot look; with the vouch (and rows that are 16-byte
  * multiples) a table batch runs on the DMA-fed kernels like its strided twin.  An entry that breaks the promise makes the
- * kernel read from a misaligned address (wrong results, not a fault).  Without the vouch, Float32 / Float16 / BFloat16 / 8-bit
- * batches of some size (from 8 GFLOP; Float32 from 32, 8-bit integers from 1) have their entries looked at on the device: one small kernel sets a
+ * kernel read from a misaligned address (wrong results, not a fault).  Without the vouch, floating-point and 8-bit
+ * batches of some size (from 8 GFLOP; Float32 and Float64 from 32, 8-bit integers from 1) have their entries looked at on the device: one small kernel sets a
  * flag, then the product is launched on both kernel families and the one the flag does not name returns at once -- two
  * extra launches (about 4 us), the same bits; smaller batches run on the register-staged kernels.  The flags live in a static
  * array of the library's device code: make the first such call on a device outside a stream capture. */

@@ -19,6 +19,12 @@ hipError_t launch_gemm_mfma_f64(bool ta, bool tb, const GemmParams& p, hipStream
     if (big_tiles >= 192 && p.M > 64 && p.N > 64) return launch_trans<DT_F64, 4, 4, 16>(ta, tb, p, s);   // a 128-wide tile would be half empty   // 128 x 128 x 16 tile
     return launch_trans<DT_F64, 2, 2, 16>(ta, tb, p, s);                          // 64 x 64 x 16 tile
 }
+// the DMA-fed kernel or nothing (the gated pair of an unvouched pointer-table batch)
+hipError_t launch_gemm_ring_only_f64(bool ta, bool tb, const GemmParams& p, hipStream_t s, bool* taken) {
+    *taken = ring64_eligible(p, ta) && p.act == ACT_NONE;        // (this kernel's epilogue has no clamp)
+    if (!*taken) return hipSuccess;
+    return ring64_tile_edge(p) == 64 ? launch_ring64_wb<1>(ta, tb, p, s) : launch_ring64_wb<2>(ta, tb, p, s);
+}
 // convolution / conv_dkernel with op(B) gathered from the image (tb: col^T), nd = 2 or 3 spatial axes
 template <int ND>
 static hipError_t launch_conv_nd_f64(bool tb, const GemmParams& p, hipStream_t s) {

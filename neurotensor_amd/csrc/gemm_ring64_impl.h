@@ -42,6 +42,7 @@ __global__ void __launch_bounds__(256) gemm_ring64_kernel(const GemmParams p) {
     const int wm = wave >> 1, wn = wave & 1;
     const int lr = lane & 15, lg = lane >> 4;
 
+    if (p.gate && *p.gate != p.gate_want) return;       // (uniform: the other kernel of a gated pair does this product)
     const int lid = xcd_contiguous_id(blockIdx.x, gridDim.x);
     const int tiles = p.tiles_m * p.tiles_n;
     const int b = lid / tiles;

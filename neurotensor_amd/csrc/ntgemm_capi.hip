@@ -26,11 +26,13 @@ hipError_t launch_gemm_ring_only_f32(bool ta, bool tb, const GemmParams& p, hipS
 hipError_t launch_gemm_ring_only_f16(bool ta, bool tb, const GemmParams& p, hipStream_t s, bool* taken);
 hipError_t launch_gemm_ring_only_bf16(bool ta, bool tb, const GemmParams& p, hipStream_t s, bool* taken);
 hipError_t launch_gemm_ring_only_i8(int dtype, bool ta, bool tb, const GemmParams& p, hipStream_t s, bool* taken);
+hipError_t launch_gemm_ring_only_f64(bool ta, bool tb, const GemmParams& p, hipStream_t s, bool* taken);
 hipError_t launch_gemm_ring_only(int dtype, bool ta, bool tb, const GemmParams& p, hipStream_t s, bool* taken) {
     *taken = false;
     switch (dtype) {
     case DT_I8: case DT_U8: return launch_gemm_ring_only_i8(dtype, ta, tb, p, s, taken);
     case DT_F32: return launch_gemm_ring_only_f32(ta, tb, p, s, taken);
+    case DT_F64: return launch_gemm_ring_only_f64(ta, tb, p, s, taken);
     case DT_F16: return launch_gemm_ring_only_f16(ta, tb, p, s, taken);
     case DT_BF16: return launch_gemm_ring_only_bf16(ta, tb, p, s, taken);
     default: return hipSuccess;
@@ -698,11 +700,11 @@ static int next_gate_slot(int** out) {
 // (about 4 us) only for products that take a few times that; the floating types that have both kernels, more than 32 rows.
 static bool gated_tables_pay(const ntg::GemmParams& p, int dtype) {
     const bool byte = dtype == ntg::DT_I8 || dtype == ntg::DT_U8;
-    if (dtype != ntg::DT_F32 && dtype != ntg::DT_F16 && dtype != ntg::DT_BF16 && !byte) return false;
+    if (dtype != ntg::DT_F32 && dtype != ntg::DT_F64 && dtype != ntg::DT_F16 && dtype != ntg::DT_BF16 && !byte) return false;
     if (p.M <= 32 || p.K <= 0 || p.act != ntg::ACT_NONE) return false;
     const double flops = 2.0 * (double)p.M * (double)p.N * (double)p.K * (double)p.batch;
     // (8-bit: the kernel that needs no alignment is the vector ALU's, 40 x slower: the check pays almost at once)
-    return flops >= (byte ? 1.0e9 : dtype == ntg::DT_F32 ? 3.2e10 : 8.0e9);
+    return flops >= (byte ? 1.0e9 : dtype == ntg::DT_F32 || dtype == ntg::DT_F64 ? 3.2e10 : 8.0e9);
 }
 static int launch_gemm_tables_gated(ntg::GemmParams p, int dtype, bool ta, bool tb, hipStream_t s) {
     int* flag = nullptr;

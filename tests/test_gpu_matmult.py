@@ -1304,14 +1304,14 @@ def test_host_entry_points_fp32_are_the_reference_chain_bit_for_bit(shape):
     assert np.array_equal(y.view(np.uint32), want.view(np.uint32)), (shape, "linear")
 
 
-@pytest.mark.parametrize("dtype", ["bf16", np.float32, np.int8], ids=["bf16", "fp32", "int8"])
+@pytest.mark.parametrize("dtype", ["bf16", np.float32, np.int8, np.float64], ids=["bf16", "fp32", "int8", "fp64"])
 def test_pointer_tables_without_a_vouch_find_their_alignment_on_the_device(dtype):
     """ntg_gemm_ptrs_dev without NTG_GEMM_PTRS_ALIGNED16 on products large enough to pay for it: a small kernel looks at the
     tables' entries, and the product runs on the DMA-fed kernel when all of them are 16-byte multiples, on the register-staged
     one otherwise (8-bit integers: the vector ALU's; both are launched, one of them returns at once).  Aligned tables, then
     tables with one entry moved by one element: in both cases every item has the bits of the item alone."""
     bf = dtype == "bf16"
-    m, k, n, nb = (2048, 1024, 2048, 5) if dtype == np.float32 else (1024, 1024, 1024, 6)
+    m, k, n, nb = (2048, 1024, 2048, 5) if dtype in (np.float32, np.float64) else (1024, 1024, 1024, 6)
     rng = np.random.default_rng(60606)
     lib = _lib.load()
     st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
@@ -1322,7 +1322,7 @@ def test_pointer_tables_without_a_vouch_find_their_alignment_on_the_device(dtype
     else:
         abuf = to_torch(randn(rng, (nb, m * k + 8), dtype, 0.5), DEV, bf)
         bbuf = to_torch(randn(rng, (nb, k * n + 8), dtype, 0.5), DEV, bf)
-    bits = lambda t: t.contiguous().view({1: torch.int8, 2: torch.int16, 4: torch.int32}[t.element_size()])
+    bits = lambda t: t.contiguous().view({1: torch.int8, 2: torch.int16, 4: torch.int32, 8: torch.int64}[t.element_size()])
     for shift in (0, 1):
         offs = [0] * nb
         offs[2] = shift                                   # one misaligned A, and below one misaligned B
