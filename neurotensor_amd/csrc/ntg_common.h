@@ -1,6 +1,7 @@
 // Shared declarations of the gfx950 matmult backend (device + host side).
 #pragma once
 #include <hip/hip_runtime.h>
+#include <cstdlib>
 #include <stdint.h>
 
 // A pointer known to point into global memory.  The pointers of GemmParams are generic; a load through a generic pointer is a
@@ -162,6 +163,9 @@ static inline int64_t ring16_tiles(int t, int64_t M, int64_t N, int64_t batch) {
 // 232); the smaller tiles then have to beat the chosen estimate as it stands.
 enum { RECT_NONE = 0, RECT_128 = 1, RECT_192 = 2 };
 static inline int ring16_tile_edge(int64_t M, int64_t N, int64_t K, int64_t batch, int rect = RECT_NONE) {
+    // (measurement knob, read once: NTG_TILE_EDGE = 256 / 224 / 192 / 128 / 64 forces the tile; results do not depend on it)
+    static const int forced = [] { const char* e = getenv("NTG_TILE_EDGE"); return e ? atoi(e) : 0; }();
+    if (forced == 256 || forced == 128 || forced == 64 || (forced == 224 && (rect & RECT_192)) || (forced == 192 && (rect & RECT_128))) return forced;
     int best = 256;
     double best_us = 0.0;
     for (int t : {256, 224, 192, 128, 64}) {
