@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the matmult hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-extras] [--no-cpu] [--only NAME[,NAME...]] [--context]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-extras] [--no-cpu] [--only NAME[,NAME...]] [--context] [--shapes SPEC[,SPEC...]]
 
 One "step" is one pass of nt::matmult over the headline workload of BASELINE.json
 (config 3): a 4096 x 4096 x 4096 BFloat16 product, inputs randn*0.02 already resident in
@@ -49,6 +49,9 @@ def parse_args():
     ap.add_argument("--power", default="", help="comma-separated extras entries that are ALSO run back to back for --power-seconds while amd-smi is "
                                                 "sampled (average socket power, clocks): what the power manager does under each workload")
     ap.add_argument("--power-seconds", type=float, default=2.5)
+    ap.add_argument("--shapes", default="",
+                    help="comma-separated extra products DTYPE:MxKxN[:nn|nt|tn|tt] (bf16, fp16, fp32, fp64; results overwritten) to time "
+                         "like the extras entries; with --only none just these are run (planner studies, e.g. under NTG_TILE_EDGE)")
     ap.add_argument("--context", action="store_true",
                     help="also time torch's own operators (hipBLASLt / MIOpen behind torch.matmul, bmm, _int_mm, conv2d) on the same "
                          "operands, alternating with this library in one process: context for the figures, never part of `value`")
@@ -547,6 +550,21 @@ def main():
         out["extras"] = extras
     if args.context:
         out["context"] = context_table(torch, F, _lib, lib, dev, stream, make_gemm, settle)
+    if args.shapes:
+        dts = {"bf16": torch.bfloat16, "fp16": torch.float16, "fp32": torch.float32, "fp64": torch.float64}
+        res = {}
+        for spec in [x for x in args.shapes.split(",") if x]:
+            parts = spec.split(":")
+            m, k, n = (int(v) for v in parts[1].split("x"))
+            form = parts[2] if len(parts) > 2 else "nn"
+            fn = make_gemm(dts[parts[0]], m, k, n, ta=form[0] == "t", tb=form[1] == "t", scale=0.02 if parts[0] in ("bf16", "fp16") else 1.0,
+                           mode=_lib.C_OVERWRITE)
+            settle(spec)
+            steps = max(args.steps, int(0.01 / max(2.0 * m * k * n / 1.0e15, 1e-6)))       # about 10 ms of launches
+            _, ev_ms = time_steps(fn, steps, args.warmup)
+            res[spec] = {"us": round(ev_ms * 1e3, 2), "TFLOP/s": round(2.0 * m * k * n / (ev_ms * 1e-3) / 1e12, 1), "timed_launches": steps}
+            del fn
+        out["shapes"] = res
     if only:
         print(json.dumps(out))
         return

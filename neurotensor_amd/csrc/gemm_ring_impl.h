@@ -1351,8 +1351,9 @@ static hipError_t launch_ring16(bool ta, bool tb, const GemmParams& p, hipStream
         if (ring16_deep128(ring16_tiles(128, q.M, q.N, q.batch), q.K)) return launch_ring_wb<DT, 2, 0, 2>(ta, tb, q, s);
         return launch_ring_wb<DT, 2>(ta, tb, q, s);
     };
+    const int rect = RECT_128 | RECT_192 | (!ta && tb ? RECT_BOTH_K : 0);
     if (p.batch == 1 && p.cmode != C_PARTIAL && !p.Aptr && !p.Bptr && !p.Cptr) {
-        const Ring16Split sp = ring16_split(p.M, p.N, p.K, RECT_128 | RECT_192);
+        const Ring16Split sp = ring16_split(p.M, p.N, p.K, rect);
         if (sp.axis) {
             GemmParams head, tail;
             ring_split_params(p, ta, tb, 2, sp, head, tail);
@@ -1364,7 +1365,7 @@ static hipError_t launch_ring16(bool ta, bool tb, const GemmParams& p, hipStream
     if (p.batch > 1 && p.cmode != C_PARTIAL && !p.Aptr && !p.Bptr && !p.Cptr) {
         // a batch whose tiles are whole rounds over the CUs plus a fraction: leading columns of every item, then the rest
         // (see ring16_column_split; the same products, tiled differently)
-        const int64_t head_cols = ring16_column_split(p.M, p.N, p.K, p.batch, RECT_128 | RECT_192);
+        const int64_t head_cols = ring16_column_split(p.M, p.N, p.K, p.batch, rect);
         if (head_cols) {
             GemmParams head = p, tail = p;
             head.N = (int)head_cols;
@@ -1373,12 +1374,12 @@ static hipError_t launch_ring16(bool ta, bool tb, const GemmParams& p, hipStream
             if (p.tailB) tail.tailB = static_cast<const char*>(p.tailB) + head_cols * 2;
             tail.C = static_cast<char*>(p.C) + head_cols * 2;
             if (p.bias) tail.bias = static_cast<const char*>(p.bias) + head_cols * p.bias_cs * 2;
-            const hipError_t e = launch_ring16_planned(head, s, launch, RECT_128 | RECT_192);
+            const hipError_t e = launch_ring16_planned(head, s, launch, rect);
             if (e != hipSuccess) return e;
-            return launch_ring16_planned(tail, s, launch, RECT_128 | RECT_192);
+            return launch_ring16_planned(tail, s, launch, rect);
         }
     }
-    return launch_ring16_planned(p, s, launch, RECT_128 | RECT_192);
+    return launch_ring16_planned(p, s, launch, rect);
 }
 
 }  // namespace ntg
