@@ -415,6 +415,9 @@ def main():
         # diagnostic: the same kernel on all-zero operands (no operand toggling: the clock stays higher) -- the difference to the
         # line above is what the power manager takes, not what the instruction stream costs
         run("c3_bf16_4096_zero_operands", G(torch.bfloat16, N, N, N, scale=0.0, mode=_lib.C_OVERWRITE), flops, PEAK_TFLOPS["bf16"])
+        # (Float16 runs the same instruction stream: equal to BFloat16 on zeros, slower on random operands by what its wider mantissa draws)
+        run("c3_fp16_4096_zero_operands", G(torch.float16, N, N, N, scale=0.0, mode=_lib.C_OVERWRITE), flops, PEAK_TFLOPS["fp16"], load=settle_bf16)
+        run("c3_fp16_4096_overwrite", G(torch.float16, N, N, N, scale=0.02, mode=_lib.C_OVERWRITE), flops, PEAK_TFLOPS["fp16"], load=settle_bf16)
 
         # the same matrix instruction on operands that stay in registers (no LDS, no global memory in the loop; 256 workgroups
         # of four wavefronts with the 256 x 256 tile's accumulator blocks): what the matrix pipes sustain on these operand
